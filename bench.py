@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the device-op hot path on one MI355X.
+
+Headline workload: the wide-MLP train step (BASELINE.json configs[4]: 4096 -> 4096 -> 4096 -> 1024,
+batch 4096, fp32, forward + backward + Adam), issued op by op through the C ABI exactly as the reference's
+training loop reaches its device.  `value` is train steps per second with every operand resident in HBM.
+
+The same JSON line also carries:
+  roofline      the dominant kernel (the fp32 MFMA GEMM): algorithmic FLOPs of the step's eight GEMM launches
+                divided by their summed duration, measured with HIP events on the stream they run on
+  cpu_baseline  the CPU oracle (C restatement of HostDevice + the box's BLAS) running the same step
+  ops           the op microbenchmark suite of configs[1] (GEMM variants, bmm, broadcast add, axis
+                reductions, fused softmax cross-entropy), each with its own roofline fraction
+  mlp_b64       the batch-64 MLP of configs[0] (latency-bound): steps per second
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+WIDE_DIMS = [4096, 4096, 4096, 1024]
+WIDE_BATCH = 4096
+
+
+def gemm_flops_per_step(dims, batch):
+    """2*m*n*k over the GEMMs of one train step: forward per layer, dX for layers > 0, dW per layer."""
+    total = 0
+    for l, (fi, fo) in enumerate(zip(dims[:-1], dims[1:])):
+        total += 2 * batch * fo * fi  # forward
+        total += 2 * fo * fi * batch  # dW
+        if l > 0:
+            total += 2 * batch * fi * fo  # dX
+    return total
+
+
+class GemmTimer:
+    """Brackets every bmm_acc dispatch with HIP events on the device's own stream."""
+
+    def __init__(self, dev):
+        self.dev = dev
+        self.pairs = []
+        self._orig = dev._op_bmm_acc
+        self.on = False
+
+    def install(self):
+        def wrapped(**p):
+            if not self.on:
+                return self._orig(**p)
+            e0 = self.dev.event().record()
+            self._orig(**p)
+            e1 = self.dev.event().record()
+            self.pairs.append((e0, e1))
+
+        self.dev._op_bmm_acc = wrapped
+
+    def total_ms(self):
+        return sum(a.elapsed_ms(b) for a, b in self.pairs)
+
+
+def time_op(dev, fn, iters, warmup=3):
+    for _ in range(warmup):
+        fn()
+    dev.sync()
+    e0 = dev.event().record()
+    for _ in range(iters):
+        fn()
+    e1 = dev.event().record()
+    return e0.elapsed_ms(e1) / iters
+
+
+def op_suite(dev, quick=False):
+    """configs[1]: per-op time, achieved TFLOP/s or GB/s from the algorithmic work, fraction of roofline."""
+    from zigrad_amd.device import F32, U64
+
+    out = {}
+    r = np.random.default_rng(0)
+    iters = 5 if quick else 20
+
+    def dev_normal(n):
+        b = dev.mem_alloc(F32, n)
+        dev.mem_random(b, "normal", seed=int(r.integers(1 << 30)))
+        return b
+
+    # GEMM 4096^3: NN, TN (A transposed), NT (B transposed)
+    n = 4096
+    A, B, C = dev_normal(n * n), dev_normal(n * n), dev_normal(n * n)
+    for tag, ta, tb in (("matmul_4096_nn", False, False), ("matmul_4096_tn", True, False), ("matmul_4096_nt", False, True)):
+        ms = time_op(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=n, n=n, k=n, trans_a=ta, trans_b=tb, lda=n, ldb=n,
+                                                ldc=n, alpha=1.0, beta=0.0), iters)
+        tf = 2 * n ** 3 / (ms * 1e-3) / 1e12
+        out[tag] = {"ms": ms, "tflops": tf, "frac_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+    # bmm 32 x 512^3
+    nb, s = 32, 512
+    ms = time_op(dev, lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, s, s], B_shape=[nb, s, s], C_shape=[nb, s, s],
+                                            trans_a=False, trans_b=False, lda=s, ldb=s, ldc=s, alpha=1.0, beta=0.0), iters)
+    tf = 2 * nb * s ** 3 / (ms * 1e-3) / 1e12
+    out["bmm_32x512"] = {"ms": ms, "tflops": tf, "frac_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+    for b in (A, B, C):
+        dev.mem_free(b)
+
+    # memory-bound ops on [8192, 4096]
+    rows, cols = 8192, 4096
+    X, bias, Z = dev_normal(rows * cols), dev_normal(cols), dev.mem_alloc(F32, rows * cols)
+    yrow = dev.mem_alloc(F32, rows)
+
+    def gbs(nbytes, ms):
+        g = nbytes / (ms * 1e-3) / 1e9
+        return {"ms": ms, "gbs": g, "frac_hbm": g / PEAK_HBM_GBS}
+
+    ms = time_op(dev, lambda: dev.dispatch("add", x=X, y=bias, z=Z), iters * 5)
+    out["add_bcast_8192x4096"] = gbs((2 * rows * cols + cols) * 4, ms)
+    ms = time_op(dev, lambda: dev.dispatch("sum_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
+    out["sum_axis1_8192x4096"] = gbs((rows * cols + rows) * 4, ms)
+    ms = time_op(dev, lambda: dev.dispatch("max_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
+    out["max_axis1_8192x4096"] = gbs((rows * cols + rows) * 4, ms)
+    for b in (X, bias, Z, yrow):
+        dev.mem_free(b)
+
+    # fused softmax cross-entropy, integer labels, logits [8192, 32000]
+    M, N = 8192, 32000
+    logits, grad = dev_normal(M * N), dev.mem_alloc(F32, M * N)
+    labels = dev.from_numpy(r.integers(0, N, M).astype(np.uint64))
+    lse, loss = dev.mem_alloc(F32, M), dev.mem_alloc(F32, 1)
+    ms = time_op(dev, lambda: dev.dispatch("smce_label_fwd", logits=logits, labels=labels, lse=lse, loss=loss, rows=M, cols=N),
+                 iters)
+    out["smce_fwd_8192x32000"] = gbs(4 * M * N + 8 * M + 4, ms)
+    ms = time_op(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
+                                            accumulate=False), iters)
+    out["smce_bwd_8192x32000"] = gbs(2 * 4 * M * N, ms)
+    ms = time_op(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
+                                            accumulate=True), iters)
+    out["smce_bwd_accumulate_8192x32000"] = gbs(3 * 4 * M * N, ms)
+    for b in (logits, grad, labels, lse, loss):
+        dev.mem_free(b)
+    return out
+
+
+def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3):
+    from zigrad_amd.trainers import MLPTrainer, mlp_inputs
+
+    params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data=data)
+    tr = MLPTrainer(dev, dims, batch, optimizer=optimizer, lr=lr, clip=True, loss_mode=loss_mode)
+    tr.load_params(params)
+    tr.set_batch(x, onehot, labels)
+    for _ in range(warmup):
+        tr.step()
+    dev.sync()
+    if timer is not None:
+        timer.on = True
+    t0 = time.perf_counter()
+    loss = None
+    for _ in range(steps):
+        loss = tr.step()
+    dev.sync()
+    dt = time.perf_counter() - t0
+    if timer is not None:
+        timer.on = False
+    return dt, loss
+
+
+def cpu_baseline(dims, batch, budget_steps=2):
+    """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share."""
+    from oracle.oracle_device import OracleDevice
+
+    odev = OracleDevice()
+    cores = min(16, os.cpu_count() or 1)
+    cores = odev.set_threads(cores)
+    dt, _ = run_mlp(odev, dims, batch, "adam", steps=budget_steps, warmup=1, data="normal")
+    return {
+        "value": budget_steps / dt,
+        "unit": "steps/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{budget_steps} timed steps (+1 warm-up) of the same batch-{batch} wide-MLP train step; "
+                  f"C restatement of HostDevice with BLAS={odev.blas_name()}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ops", action="store_true", help="skip the op microbenchmark suite")
+    ap.add_argument("--loss-mode", default="onehot", choices=["onehot", "label"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the hot path is single-device and this build uses no second GPU "
+                 "(run with --gpus 1)")
+
+    from zigrad_amd import HipDevice
+
+    dev = HipDevice(0)
+    timer = GemmTimer(dev)
+    timer.install()
+    dt, loss = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", timer, args.loss_mode)
+    ms_per_step = dt / args.steps * 1e3
+    gemm_ms = timer.total_ms()
+    n_launch = len(timer.pairs)
+    flops = gemm_flops_per_step(WIDE_DIMS, WIDE_BATCH) * args.steps
+    achieved = flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
+
+    result = {
+        "metric": "MLP train steps/sec @ batch 4096 (wide MLP 4096-4096-4096-1024, fwd+bwd+Adam)",
+        "value": args.steps / dt,
+        "unit": "steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "wide MLP train step: 4096->4096->4096->1024, batch 4096, softmax-CE "
+                               f"({args.loss_mode}), Adam lr 1e-3, per-tensor grad clip on", "final_loss": loss},
+        "roofline": {
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+            "traffic": None,
+            "kernel": "gemm_kernel (fp32 MFMA 32x32x2), 8 launches per step",
+            "gemm_ms_per_step": gemm_ms / args.steps,
+            "launches_timed": n_launch,
+        },
+    }
+    # batch-64 MLP of configs[0]: latency-bound
+    dt64, _ = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01)
+    result["mlp_b64"] = {"steps_per_s": 200 / dt64, "ms_per_step": dt64 / 200 * 1e3,
+                         "workload": "784-128-64-10, batch 64, SGD lr 0.01, clip on, loss read every step"}
+    if not args.no_ops:
+        result["ops"] = op_suite(dev)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH)
+    else:
+        result["cpu_baseline"] = None
+    dev.deinit()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,246 @@
+/*
+ * zg_hip.h -- C ABI of the MI355X (gfx950) device backend for Zigrad.
+ *
+ * One entry point per device op that Zigrad reaches through
+ * DeviceReference.dispatch (reference: src/device/device_reference.zig:15-27,
+ * parameter structs in src/device/opspec.zig) plus the memory API of
+ * src/device/device_reference.zig:29-131.  A Zig `HipDevice` struct binds these
+ * one-to-one (see zig/hip_device.zig); the structural precedent on the reference
+ * side is src/cuda/{cuda_utils,blas_conflux,nn_conflux}.h.
+ *
+ * Conventions
+ *   - element type is fp32 throughout (every configuration of the reference's
+ *     examples is fp32); `usize` of the reference is uint64_t here;
+ *   - a reference slice `[]T` becomes (pointer, length); all data pointers are
+ *     DEVICE pointers unless a parameter is documented as host memory;
+ *     index arrays may live in device memory or in pinned host memory obtained
+ *     from zg_hip_host_alloc (both are readable by the kernels);
+ *   - shapes (x_shape, A_shape, ...) are HOST arrays, as in the reference where
+ *     they are stack slices (src/ndarray.zig:884-888);
+ *   - every call is asynchronous on the context's single stream, in order,
+ *     except where stated (d2h copies block, as NDTensor.get needs:
+ *     src/ndtensor.zig:524-528);
+ *   - every function returns 0 on success and a ZG_HIP_E* code otherwise;
+ *     zg_hip_last_error() gives the message.  The reference's ops return void
+ *     and panic on failure (src/device/device_reference.zig:20-22); the Zig
+ *     binding turns a non-zero return into @panic.
+ *   - argument checks happen on the host before any launch; a rejected call
+ *     launches nothing.
+ */
+#ifndef ZG_HIP_H
+#define ZG_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct zg_hip_ctx zg_hip_ctx;
+typedef struct zg_hip_event zg_hip_event;
+
+enum {
+    ZG_HIP_OK = 0,
+    ZG_HIP_EINVAL = 1,   /* argument/shape check failed; nothing was launched */
+    ZG_HIP_EOOM = 2,     /* device allocation failed (reference: Error.DeviceOOM, src/allocators/device_data.zig:44) */
+    ZG_HIP_ERUNTIME = 3, /* a HIP runtime call failed */
+};
+
+/* kinds for zg_hip_mem_random (reference: RandType, src/device/device_common.zig:3) */
+enum { ZG_RAND_UNIFORM = 0, ZG_RAND_NORMAL = 1, ZG_RAND_KAIMING = 2 };
+
+/* ---------------------------------------------------------------------------------------------
+ * context (replaces HostDevice.init/deinit/sync: src/device/host_device.zig:183-196, :960;
+ * shape precedent: src/device/cuda_device.zig:126-160)
+ * ------------------------------------------------------------------------------------------- */
+const char *zg_hip_last_error(void);
+int zg_hip_device_count(int *count);
+int zg_hip_init(int device_id, zg_hip_ctx **out);
+int zg_hip_deinit(zg_hip_ctx *ctx);
+int zg_hip_sync(zg_hip_ctx *ctx);
+int zg_hip_total_memory(zg_hip_ctx *ctx, size_t *bytes);
+/* the HIP stream every op is enqueued on, as an opaque pointer (hipStream_t) */
+void *zg_hip_stream(zg_hip_ctx *ctx);
+
+/* timing helpers on the context's stream (hipEvent_t underneath) */
+int zg_hip_event_create(zg_hip_ctx *ctx, zg_hip_event **out);
+int zg_hip_event_record(zg_hip_ctx *ctx, zg_hip_event *ev);
+int zg_hip_event_elapsed_ms(zg_hip_event *start, zg_hip_event *stop, float *ms); /* blocks until `stop` completed */
+int zg_hip_event_destroy(zg_hip_event *ev);
+
+/* ---------------------------------------------------------------------------------------------
+ * DataHandler primitives for src/allocators/caching_allocator.zig (contract: map/unmap/alloc/free/
+ * page_size; host version src/device/host_device.zig:50-110, cuda version src/device/cuda_device.zig:21-81)
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_page_size(zg_hip_ctx *ctx, size_t *bytes);
+int zg_hip_pool_map(zg_hip_ctx *ctx, size_t bytes, void **out);  /* one contiguous device region for a block pool */
+int zg_hip_pool_unmap(zg_hip_ctx *ctx, void *ptr);
+int zg_hip_alloc(zg_hip_ctx *ctx, size_t bytes, void **out);    /* mem_alloc: src/device/host_device.zig:890-898 */
+int zg_hip_free(zg_hip_ctx *ctx, void *ptr);                    /* mem_free:  src/device/host_device.zig:900-903 */
+int zg_hip_host_alloc(zg_hip_ctx *ctx, size_t bytes, void **out); /* pinned, device-readable host memory */
+int zg_hip_host_free(zg_hip_ctx *ctx, void *ptr);
+
+/* The library's own caching allocator (block pools over two mapped regions + grow-only scratch),
+ * the C++ counterpart of CachingAllocator(DataHandler) (src/allocators/caching_allocator.zig:15-162)
+ * for callers that do not bring Zigrad's.  `block` is the DeviceData.ctx of the reference
+ * (src/allocators/device_data.zig:32-40). A zero-byte request yields (NULL, 0). */
+int zg_hip_cache_configure(zg_hip_ctx *ctx, size_t small_pool_bytes, size_t large_pool_bytes);
+int zg_hip_mem_cache_alloc(zg_hip_ctx *ctx, size_t bytes, void **out, uint64_t *block);
+int zg_hip_mem_cache_free(zg_hip_ctx *ctx, void *ptr, uint64_t block);
+int zg_hip_mem_scratch(zg_hip_ctx *ctx, size_t bytes, void **out); /* src/allocators/caching_allocator.zig:133-156 */
+int zg_hip_clear_cache(zg_hip_ctx *ctx);
+int zg_hip_cache_stats(zg_hip_ctx *ctx, size_t *bytes_in_use, size_t *bytes_mapped, uint64_t *n_device_allocs);
+
+/* ---------------------------------------------------------------------------------------------
+ * memory ops (src/device/host_device.zig:919-958)
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_memcpy_h2d(zg_hip_ctx *ctx, void *dst, const void *src_host, size_t bytes); /* mem_transfer .HtoD */
+int zg_hip_memcpy_d2h(zg_hip_ctx *ctx, void *dst_host, const void *src, size_t bytes); /* .DtoH, blocking */
+int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes);      /* mem_copy / .DtoD */
+int zg_hip_mem_fill(zg_hip_ctx *ctx, float *x, size_t n, float value);
+int zg_hip_mem_fill_u8(zg_hip_ctx *ctx, void *x, size_t n, uint8_t value);
+int zg_hip_mem_fill_u64(zg_hip_ctx *ctx, uint64_t *x, size_t n, uint64_t value);
+int zg_hip_mem_sequence(zg_hip_ctx *ctx, float *x, size_t n, float initial, float step);
+int zg_hip_mem_take(zg_hip_ctx *ctx, const float *src, size_t src_len, const uint64_t *idxs, size_t n, float *dst);
+/* values are generated on the host (the reference hands mem_random a host std.Random,
+ * src/device/host_device.zig:931-945) and copied up; `seed` stands in for that generator */
+int zg_hip_mem_random(zg_hip_ctx *ctx, float *x, size_t n, int kind, uint64_t fan, uint64_t seed);
+
+/* ---------------------------------------------------------------------------------------------
+ * elementwise binary (src/device/host_device.zig:205-219, :975-1019; opspec.zig:19-57)
+ * requires max(xl,yl) % min(xl,yl) == 0 and zl == max(xl,yl); z may alias x or y
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_add(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
+int zg_hip_sub(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
+int zg_hip_mul(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
+int zg_hip_div(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
+
+/* ---------------------------------------------------------------------------------------------
+ * linear algebra (src/device/host_device.zig:224-346)
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_dot(zg_hip_ctx *ctx, const float *x, const float *y, size_t n, float *z);
+int zg_hip_matvec(zg_hip_ctx *ctx, const float *A, const float *x, float *y, size_t m, size_t n, int trans_a,
+                  float alpha, float beta);
+/* row-major C = alpha*op(A)*op(B) + beta*C; C is not read when beta == 0 */
+int zg_hip_matmul(zg_hip_ctx *ctx, const float *A, const float *B, float *C, size_t m, size_t n, size_t k,
+                  int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta);
+/* shapes are host arrays of 3: {batches, rows, cols} of the logical (post-transpose) operands */
+int zg_hip_bmm_acc(zg_hip_ctx *ctx, const float *A, const uint64_t *A_shape, const float *B,
+                   const uint64_t *B_shape, float *C, const uint64_t *C_shape, int trans_a, int trans_b, size_t lda,
+                   size_t ldb, size_t ldc, float alpha, float beta);
+int zg_hip_outer(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *A, float alpha);
+/* B = A^T + alpha*B; B is not read when alpha == 0 (the reference hands in uninitialised B then:
+ * src/ndarray.zig:794-802) */
+int zg_hip_transpose(zg_hip_ctx *ctx, const float *A, float *B, size_t m, size_t n, float alpha);
+/* alpha is read through the pointer: a host pointer when alpha_on_device == 0 (SGD, src/nn/optim.zig:114-118),
+ * a device pointer otherwise (dot backward, src/ndtensor.zig:1146-1150) */
+int zg_hip_axpy(zg_hip_ctx *ctx, const float *x, float *y, size_t n, const float *alpha, int alpha_on_device);
+int zg_hip_sum(zg_hip_ctx *ctx, const float *x, size_t n, float *y); /* sum of |x|, as cblas_sasum */
+int zg_hip_scale(zg_hip_ctx *ctx, float *x, size_t n, float alpha);
+int zg_hip_nrm2(zg_hip_ctx *ctx, const float *x, size_t n, float *y);
+int zg_hip_clip_nrm2(zg_hip_ctx *ctx, float *x, size_t n, float max_norm, float delta);
+
+/* ---------------------------------------------------------------------------------------------
+ * unary forward/backward (src/device/host_device.zig:353-598); y may alias x in the *_fwd ops
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_pow_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n, float e);
+int zg_hip_pow_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, const float *y_g, size_t n, float e, float eps);
+int zg_hip_sqrt_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n);
+int zg_hip_sqrt_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, const float *y_g, size_t n, float eps);
+int zg_hip_rsqrt_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n, float eps);
+int zg_hip_rsqrt_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, const float *y_g, size_t n, float eps);
+int zg_hip_exp_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n);
+int zg_hip_exp_bwd(zg_hip_ctx *ctx, float *x_g, const float *y, const float *y_g, size_t n);
+int zg_hip_relu_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n);
+int zg_hip_relu_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, const float *y_g, size_t n);
+int zg_hip_relu_inplace_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, size_t n);
+int zg_hip_tanh_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n);
+int zg_hip_tanh_bwd(zg_hip_ctx *ctx, float *x_g, const float *y, const float *y_g, size_t n);
+int zg_hip_tanh_inplace_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, size_t n);
+int zg_hip_sigm_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n);
+int zg_hip_sigm_bwd(zg_hip_ctx *ctx, float *x_g, const float *y, const float *y_g, size_t n);
+int zg_hip_sigm_inplace_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, size_t n);
+int zg_hip_clamp_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n, float lo, float hi);
+int zg_hip_clamp_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, const float *y_g, size_t n, float lo, float hi);
+int zg_hip_max_fwd(zg_hip_ctx *ctx, const float *x, size_t n, float *y); /* x[isamax(x)]: largest |x|, first on ties */
+int zg_hip_max_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, size_t n, const float *y, const float *y_g);
+
+/* ---------------------------------------------------------------------------------------------
+ * reductions (src/device/host_device.zig:709-874, src/device/reduce.zig)
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_sum_along(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape, size_t x_rank, float *y, size_t y_len,
+                     size_t dim, float alpha, float beta);
+int zg_hip_max_along(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape, size_t x_rank, float *y, size_t y_len,
+                     size_t dim);
+/* no reference op: first index of the maximum along dim (std.mem.indexOfMax per slice,
+ * examples/mnist/src/main-simple.zig:124-125) */
+int zg_hip_argmax_along(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape, size_t x_rank, uint64_t *y,
+                        size_t y_len, size_t dim);
+/* scratch sizing rule of NDArray.unbroadcast_ (src/ndarray.zig:701-719), in floats */
+size_t zg_hip_unbroadcast_scratch_len(const uint64_t *x_shape, size_t x_rank, const uint64_t *y_shape,
+                                      size_t y_rank);
+int zg_hip_unbroadcast(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape, size_t x_rank, float *y,
+                       const uint64_t *y_shape, size_t y_rank, float *scratch, size_t scratch_len, float alpha,
+                       float beta);
+int zg_hip_broadcast(zg_hip_ctx *ctx, const float *x, size_t xl, float *y, size_t yl, float alpha, float beta);
+
+/* ---------------------------------------------------------------------------------------------
+ * indexing (src/device/host_device.zig:1039-1087, :1356-1403; src/ndarray.zig:593-633;
+ * src/ndtensor.zig:1437-1513).  All accumulating ops add contributions to one destination element
+ * in the order of the input index array, so results do not depend on scheduling.
+ * ------------------------------------------------------------------------------------------- */
+/* offsets of NDArray.gather computed on the device; shapes are host arrays of `rank`; `indices`, `offsets`
+ * device-readable.  Out-of-range indices are reported through *status (host, optional, blocking when given):
+ * 0 ok, 1 InvalidIndexShape, 2 IndexOutOfBounds */
+int zg_hip_gather_offsets(zg_hip_ctx *ctx, const uint64_t *src_shape, const uint64_t *idx_shape, size_t rank,
+                          const uint64_t *indices, size_t dim, uint64_t *offsets, int *status);
+int zg_hip_scatter_add(zg_hip_ctx *ctx, const float *src, const uint64_t *offsets, size_t n, float *dst,
+                       size_t dst_len);
+int zg_hip_index_select_fwd(zg_hip_ctx *ctx, const float *src, size_t src_len, const uint64_t *indices, size_t n_idx,
+                            size_t stride, float *dst);
+int zg_hip_index_select_bwd(zg_hip_ctx *ctx, const float *y_grad, const uint64_t *indices, size_t n_idx,
+                            size_t stride, float *x_grad, size_t x_len);
+/* n_nodes = number of rows of dst/h (the reference derives it from the slices' lengths) */
+int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx *ctx, float *dst, const float *h, const float *deg,
+                                  const uint64_t *src_indices, const uint64_t *tgt_indices, size_t stride,
+                                  size_t n_edge, size_t n_nodes);
+int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx *ctx, const float *grad_output, const float *h, const float *deg,
+                                      const uint64_t *src_indices, const uint64_t *tgt_indices, float *grad_h,
+                                      float *grad_deg, size_t stride, size_t n_edge, size_t n_nodes);
+
+/* ---------------------------------------------------------------------------------------------
+ * losses: the host loops of src/nn/loss.zig:94-305 as device ops (new op names; the reference
+ * dereferences .raw on the host and has no opspec for them)
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_smce_fwd(zg_hip_ctx *ctx, const float *logits, const float *target, float *probs, float *loss,
+                    size_t rows, size_t cols);
+int zg_hip_smce_bwd(zg_hip_ctx *ctx, const float *probs, const float *target, float *grad, size_t rows, size_t cols);
+/* integer-label form: one pass over the logits forward (online softmax), lse[rows] kept for backward */
+int zg_hip_smce_label_fwd(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, float *lse, float *loss,
+                          size_t rows, size_t cols);
+/* accumulate != 0: grad += (p - onehot)/rows (the reference's `+=`, src/nn/loss.zig:157);
+ * accumulate == 0: grad is overwritten (valid when the caller knows grad is a fresh zero buffer) */
+int zg_hip_smce_label_bwd(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, const float *lse,
+                          float *grad, size_t rows, size_t cols, int accumulate);
+int zg_hip_softmax_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t rows, size_t cols);
+int zg_hip_softmax_bwd(zg_hip_ctx *ctx, const float *y, const float *y_g, float *x_g, size_t rows, size_t cols);
+int zg_hip_smooth_l1_fwd(zg_hip_ctx *ctx, const float *pred, const float *target, size_t n, float beta, float *loss);
+int zg_hip_smooth_l1_bwd(zg_hip_ctx *ctx, const float *pred, const float *target, float *grad, size_t n, float beta);
+int zg_hip_mse_fwd(zg_hip_ctx *ctx, const float *pred, const float *target, size_t n, float *loss);
+int zg_hip_mse_bwd(zg_hip_ctx *ctx, const float *pred, const float *target, float *grad, size_t n);
+
+/* ---------------------------------------------------------------------------------------------
+ * optimizers: src/nn/optim.zig:100-122 (SGD.update) and :177-234 (Adam.update) as one op per
+ * parameter tensor.  `clip` != 0 applies the reference's per-tensor clip_nrm2 to grad first
+ * (grad is modified in place, as in the reference).
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_sgd_step(zg_hip_ctx *ctx, float *param, float *grad, size_t n, float lr, int clip, float max_norm,
+                    float delta);
+/* t: the per-tensor-update counter AFTER the reference's `self.t += 1` (src/nn/optim.zig:189) */
+int zg_hip_adam_step(zg_hip_ctx *ctx, float *param, float *grad, float *m, float *v, size_t n, uint64_t t, float lr,
+                     float beta1, float beta2, float epsilon, int clip, float max_norm, float delta);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

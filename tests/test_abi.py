@@ -1,0 +1,38 @@
+"""The shared library loads and exports every entry point include/zg_hip.h declares (no GPU calls)."""
+import ctypes
+
+from zigrad_amd._lib import LIB_PATH, Library, parse_header
+
+
+def test_header_declares_expected_surface():
+    protos = parse_header()
+    # every DeviceReference op of the hot path has an entry point
+    for op in ["add", "sub", "mul", "div", "dot", "matvec", "matmul", "bmm_acc", "outer", "transpose", "axpy", "sum",
+               "scale", "nrm2", "clip_nrm2", "pow_fwd", "pow_bwd", "sqrt_fwd", "sqrt_bwd", "rsqrt_fwd", "rsqrt_bwd",
+               "exp_fwd", "exp_bwd", "relu_fwd", "relu_bwd", "relu_inplace_bwd", "tanh_fwd", "tanh_bwd",
+               "tanh_inplace_bwd", "sigm_fwd", "sigm_bwd", "sigm_inplace_bwd", "max_fwd", "max_bwd", "clamp_fwd",
+               "clamp_bwd", "unbroadcast", "broadcast", "sum_along", "max_along", "argmax_along", "scatter_add",
+               "scatter_gcn_deg_scaled", "scatter_gcn_deg_scaled_bwd", "index_select_fwd", "index_select_bwd",
+               "smce_fwd", "smce_bwd", "smce_label_fwd", "smce_label_bwd", "smooth_l1_fwd", "smooth_l1_bwd", "mse_fwd",
+               "mse_bwd", "sgd_step", "adam_step", "mem_fill", "mem_sequence", "mem_take", "mem_random",
+               "mem_cache_alloc", "mem_cache_free", "mem_scratch", "memcpy_h2d", "memcpy_d2h", "memcpy_d2d", "sync"]:
+        assert "zg_hip_" + op in protos, op
+    assert len(protos) >= 90
+
+
+def test_library_exports_every_declared_symbol():
+    assert LIB_PATH.exists(), "build the library first: python -m zigrad_amd.build"
+    lib = Library()
+    for name in lib.protos:
+        assert hasattr(lib.cdll, name), name
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = Library()
+    # a null context is rejected on the host before anything touches a device
+    rc = lib.cdll.zg_hip_sync(None)
+    assert rc == 1
+    assert b"null context" in lib.cdll.zg_hip_last_error()
+    n = ctypes.c_int(-1)
+    assert lib.cdll.zg_hip_device_count(ctypes.byref(n)) == 0
+    assert n.value >= 0

@@ -1,0 +1,282 @@
+"""Losses, optimizers and indexing ops of the HIP device against the CPU oracle, through the C ABI."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+from scipy.special import logsumexp, softmax
+
+from conftest import rel_fro, run_op
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def both(oracle, hip, name, params, outputs):
+    a = run_op(oracle, name, {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in params.items()}, outputs)
+    b = run_op(hip, name, params, outputs)
+    return a, b
+
+
+# ----------------------------------------------------------------------------------------------
+# softmax / cross-entropy
+# ----------------------------------------------------------------------------------------------
+SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001)]
+
+
+@pytest.mark.parametrize("rows,cols", SMCE_SHAPES)
+def test_smce_onehot_and_label(oracle, hip, rows, cols):
+    r = rng(rows * 7 + cols)
+    x = (r.standard_normal((rows, cols)) * 3).astype(np.float32)
+    lab = r.integers(0, cols, rows).astype(np.uint64)
+    t = np.zeros((rows, cols), np.float32)
+    t[np.arange(rows), lab] = 1.0
+    one = np.zeros(1, np.float32)
+    a, b = both(oracle, hip, "smce_fwd", {"logits": x, "target": t, "probs": np.zeros_like(x), "loss": one, "rows": rows,
+                                          "cols": cols}, ["probs", "loss"])
+    x64 = x.astype(np.float64)
+    sm = softmax(x64, axis=1)
+    loss = float(np.mean(logsumexp(x64, axis=1) - x64[np.arange(rows), lab]))
+    assert rel_fro(b["probs"], sm) <= TOL and rel_fro(a["probs"], sm) <= TOL
+    assert abs(b["loss"][0] - loss) <= 1e-5 * max(1.0, abs(loss))
+    assert abs(b["loss"][0] - a["loss"][0]) <= 1e-5 * max(1.0, abs(loss))
+    g0 = (r.standard_normal((rows, cols)) * 0.01).astype(np.float32)
+    ga, gb = both(oracle, hip, "smce_bwd", {"probs": b["probs"], "target": t, "grad": g0, "rows": rows, "cols": cols}, ["grad"])
+    np.testing.assert_array_equal(ga["grad"], gb["grad"])  # pure sub/div/add on identical inputs
+    # integer labels
+    a2, b2 = both(oracle, hip, "smce_label_fwd", {"logits": x, "labels": lab, "lse": np.zeros(rows, np.float32), "loss": one,
+                                                  "rows": rows, "cols": cols}, ["lse", "loss"])
+    assert rel_fro(b2["lse"], logsumexp(x64, axis=1)) <= 1e-6
+    assert abs(b2["loss"][0] - loss) <= 1e-5 * max(1.0, abs(loss))
+    assert abs(b2["loss"][0] - a2["loss"][0]) <= 1e-5 * max(1.0, abs(loss))
+    want = g0 + (sm - t) / rows
+    for acc in (True, False):
+        g = run_op(hip, "smce_label_bwd", {"logits": x, "labels": lab, "lse": b2["lse"], "grad": g0.copy(), "rows": rows,
+                                           "cols": cols, "accumulate": acc}, ["grad"])["grad"]
+        assert rel_fro(g, want if acc else (sm - t) / rows) <= TOL
+        # every row of the un-accumulated gradient sums to zero
+        if not acc:
+            assert np.abs(g.astype(np.float64).sum(axis=1)).max() <= 1e-6
+    go = run_op(oracle, "smce_label_bwd", {"logits": x, "labels": lab, "lse": a2["lse"], "grad": g0.copy(), "rows": rows,
+                                           "cols": cols}, ["grad"])["grad"]
+    assert rel_fro(go, want) <= TOL
+
+
+def test_smce_clamp_edge(oracle, hip):
+    """A vanishing probability is clamped to 1e-7 in the loss only (src/nn/loss.zig:143)."""
+    x = np.asarray([[100.0, 0.0, 0.0], [0.0, 0.0, 50.0]], np.float32)
+    lab = np.asarray([1, 0], np.uint64)
+    t = np.zeros((2, 3), np.float32)
+    t[[0, 1], [1, 0]] = 1
+    one = np.zeros(1, np.float32)
+    a, b = both(oracle, hip, "smce_fwd", {"logits": x, "target": t, "probs": np.zeros_like(x), "loss": one, "rows": 2, "cols": 3},
+                ["loss"])
+    want = -np.log(np.float32(1e-7))
+    assert abs(b["loss"][0] - want) <= 1e-5 * want and abs(a["loss"][0] - want) <= 1e-5 * want
+    a, b = both(oracle, hip, "smce_label_fwd", {"logits": x, "labels": lab, "lse": np.zeros(2, np.float32), "loss": one,
+                                                "rows": 2, "cols": 3}, ["loss"])
+    assert abs(b["loss"][0] - want) <= 1e-5 * want and abs(a["loss"][0] - want) <= 1e-5 * want
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 10), (5, 3000), (1, 7)])
+def test_softmax_fwd_bwd(oracle, hip, rows, cols):
+    r = rng(rows + cols)
+    x = r.standard_normal((rows, cols)).astype(np.float32)
+    a, b = both(oracle, hip, "softmax_fwd", {"x": x, "y": np.zeros_like(x), "rows": rows, "cols": cols}, ["y"])
+    assert rel_fro(b["y"], softmax(x.astype(np.float64), axis=1)) <= TOL
+    yg = r.standard_normal((rows, cols)).astype(np.float32)
+    g0 = r.standard_normal((rows, cols)).astype(np.float32)
+    a, b = both(oracle, hip, "softmax_bwd", {"y": b["y"], "y_g": yg, "x_g": g0, "rows": rows, "cols": cols}, ["x_g"])
+    assert rel_fro(b["x_g"], a["x_g"]) <= TOL
+
+
+@pytest.mark.parametrize("n", [6, 64, 100001])
+def test_smooth_l1_and_mse(oracle, hip, n):
+    r = rng(n)
+    p, t = r.standard_normal(n).astype(np.float32) * 2, r.standard_normal(n).astype(np.float32)
+    one = np.zeros(1, np.float32)
+    g0 = r.standard_normal(n).astype(np.float32)
+    a, b = both(oracle, hip, "smooth_l1_fwd", {"pred": p, "target": t, "beta": 1.0, "loss": one}, ["loss"])
+    assert abs(a["loss"][0] - b["loss"][0]) <= 1e-5 * abs(a["loss"][0])
+    a, b = both(oracle, hip, "smooth_l1_bwd", {"pred": p, "target": t, "grad": g0, "beta": 1.0}, ["grad"])
+    np.testing.assert_array_equal(a["grad"], b["grad"])
+    a, b = both(oracle, hip, "mse_fwd", {"pred": p, "target": t, "loss": one}, ["loss"])
+    assert abs(a["loss"][0] - b["loss"][0]) <= 1e-5 * abs(a["loss"][0])
+    a, b = both(oracle, hip, "mse_bwd", {"pred": p, "target": t, "grad": g0}, ["grad"])
+    np.testing.assert_array_equal(a["grad"], b["grad"])
+
+
+# ----------------------------------------------------------------------------------------------
+# optimizers
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [10, 640, 8192, 100352, (1 << 21) + 3])
+@pytest.mark.parametrize("clip", [False, True])
+def test_sgd_and_adam_steps(oracle, hip, n, clip):
+    r = rng(n + clip)
+    p0 = r.standard_normal(n).astype(np.float32)
+    # with clip on, one gradient is large enough to be clipped (norm > 10) and one is not
+    for gscale in ((5.0, 1e-3) if clip else (1.0,)):
+        g0 = (r.standard_normal(n) * gscale).astype(np.float32)
+        a, b = both(oracle, hip, "sgd_step", {"param": p0, "grad": g0, "lr": 0.01, "clip": clip, "max_norm": 10.0, "delta": 1e-6},
+                    ["param", "grad"])
+        if clip:
+            assert rel_fro(b["param"], a["param"]) <= 1e-6 and rel_fro(b["grad"], a["grad"]) <= 1e-6
+        else:
+            np.testing.assert_array_equal(a["param"], b["param"])
+            np.testing.assert_array_equal(a["grad"], b["grad"])
+        # Adam: two consecutive steps with the per-tensor counter t
+        state = {}
+        for name, dev in (("o", oracle), ("h", hip)):
+            P, G, M, V = (dev.from_numpy(x) for x in (p0, g0, np.zeros(n, np.float32), np.zeros(n, np.float32)))
+            for t in (1, 2):
+                dev.dispatch("adam_step", param=P, grad=G, m=M, v=V, t=t, lr=1e-3, beta1=0.9, beta2=0.999, epsilon=1e-8,
+                             clip=clip, max_norm=10.0, delta=1e-6)
+            dev.sync()
+            state[name] = [dev.to_numpy(x) for x in (P, G, M, V)]
+        for xo, xh in zip(state["o"], state["h"]):
+            if clip:
+                assert rel_fro(xh, xo) <= 1e-6
+            else:
+                np.testing.assert_array_equal(xo, xh)
+
+
+def test_adam_closed_form(hip):
+    """Two hand-traced steps: t increments per update, lr_t in fp32 (src/nn/optim.zig:189-191, 226-229)."""
+    p, g = np.asarray([1.0, -2.0], np.float32), np.asarray([0.5, -0.25], np.float32)
+    P, G, M, V = (hip.from_numpy(x) for x in (p, g, np.zeros(2, np.float32), np.zeros(2, np.float32)))
+    m = v = np.zeros(2)
+    want = p.astype(np.float64)
+    for t in (1, 2):
+        hip.dispatch("adam_step", param=P, grad=G, m=M, v=V, t=t, lr=0.01, beta1=0.9, beta2=0.999, epsilon=1e-8, clip=False,
+                     max_norm=10.0, delta=1e-6)
+        m = 0.9 * m + 0.1 * g
+        v = 0.999 * v + 0.001 * g * g
+        lr_t = 0.01 * np.sqrt(1 - 0.999 ** t) / (1 - 0.9 ** t)
+        want = want - lr_t * m / (np.sqrt(v) + 1e-8)
+    np.testing.assert_allclose(hip.to_numpy(P), want, rtol=1e-5)
+
+
+# ----------------------------------------------------------------------------------------------
+# indexing: gather offsets, scatter_add, index_select, GCN scatter
+# ----------------------------------------------------------------------------------------------
+def test_gather_offsets_bit_exact(oracle, hip):
+    r = rng(1)
+    for src_shape, idx_shape, dim in [([64, 2], [64, 1], 1), ([5, 6, 7], [5, 4, 7], 1), ([5, 6, 7], [3, 6, 2], 0), ([9], [4], 0)]:
+        n = int(np.prod(idx_shape))
+        idx = r.integers(0, src_shape[dim], n).astype(np.uint64)
+        res = []
+        for dev in (oracle, hip):
+            I, O = dev.from_numpy(idx), dev.from_numpy(np.zeros(n, np.uint64))
+            assert dev.gather_offsets(src_shape, idx_shape, I, dim, O) == 0
+            dev.sync()
+            res.append(dev.to_numpy(O))
+        np.testing.assert_array_equal(res[0], res[1])
+        # brute force: numpy take_along_axis over a tensor of flat positions
+        pos = np.arange(int(np.prod(src_shape))).reshape(src_shape)
+        sl = tuple(slice(0, s) for s in idx_shape)
+        want = np.take_along_axis(pos[tuple(s if i != dim else slice(None) for i, s in enumerate(sl))],
+                                  idx.reshape(idx_shape).astype(np.int64), axis=dim)
+        np.testing.assert_array_equal(res[1], want.ravel().astype(np.uint64))
+
+
+@pytest.mark.parametrize("n,dst_len", [(64, 128), (13264, 2708), (100000, 17), (5000, 300000), (1, 1), (40000, 5000)])
+def test_scatter_add_bit_exact(oracle, hip, n, dst_len):
+    """Order of accumulation per destination equals the host loop's, so the floats agree bit for bit."""
+    r = rng(n + dst_len)
+    src = r.standard_normal(n).astype(np.float32)
+    off = r.integers(0, dst_len, n).astype(np.uint64)
+    if n > 100:
+        off[: n // 4] = np.sort(off[: n // 4])  # runs of consecutive / repeated offsets
+    dst0 = r.standard_normal(dst_len).astype(np.float32)
+    a, b = both(oracle, hip, "scatter_add", {"src": src, "offsets": off, "dst": dst0}, ["dst"])
+    np.testing.assert_array_equal(a["dst"], b["dst"])
+    # invariant: total mass is conserved
+    assert abs(b["dst"].astype(np.float64).sum() - (dst0.astype(np.float64).sum() + src.astype(np.float64).sum())) <= 1e-3 * (1 + np.abs(src).sum())
+
+
+def test_scatter_add_heavy_hitter_is_deterministic(hip):
+    r = rng(6)
+    n = 200000
+    src = r.standard_normal(n).astype(np.float32)
+    off = np.where(r.random(n) < 0.5, 3, r.integers(0, 1000, n)).astype(np.uint64)
+    outs = [run_op(hip, "scatter_add", {"src": src, "offsets": off, "dst": np.zeros(1000, np.float32)}, ["dst"])["dst"]
+            for _ in range(3)]
+    np.testing.assert_array_equal(outs[0], outs[1])
+    np.testing.assert_array_equal(outs[0], outs[2])
+    want = np.zeros(1000, np.float32)
+    for i in range(n):
+        want[off[i]] += src[i]
+    np.testing.assert_array_equal(outs[0], want)
+
+
+@pytest.mark.parametrize("rows,stride,n_idx", [(100, 16, 37), (2708, 7, 5000), (50, 300, 200), (10, 1, 10)])
+def test_index_select(oracle, hip, rows, stride, n_idx):
+    r = rng(rows + stride)
+    src = r.standard_normal(rows * stride).astype(np.float32)
+    idx = r.integers(0, rows, n_idx).astype(np.uint64)
+    a, b = both(oracle, hip, "index_select_fwd", {"src": src, "indices": idx, "stride": stride,
+                                                  "dst": np.zeros(n_idx * stride, np.float32)}, ["dst"])
+    np.testing.assert_array_equal(a["dst"], b["dst"])
+    np.testing.assert_array_equal(b["dst"], src.reshape(rows, stride)[idx.astype(np.int64)].ravel())
+    yg = r.standard_normal(n_idx * stride).astype(np.float32)
+    xg = r.standard_normal(rows * stride).astype(np.float32)
+    a, b = both(oracle, hip, "index_select_bwd", {"y_grad": yg, "indices": idx, "stride": stride, "x_grad": xg}, ["x_grad"])
+    np.testing.assert_array_equal(a["x_grad"], b["x_grad"])
+
+
+def random_graph(r, n_nodes, n_pairs):
+    """Symmetrised random pairs plus self loops, [2, E] layout (src row then tgt row)."""
+    u, v = r.integers(0, n_nodes, n_pairs), r.integers(0, n_nodes, n_pairs)
+    loops = np.arange(n_nodes)
+    src = np.concatenate([u, v, loops]).astype(np.uint64)
+    tgt = np.concatenate([v, u, loops]).astype(np.uint64)
+    return src, tgt
+
+
+@pytest.mark.parametrize("n_nodes,n_pairs,stride", [(2708, 5278, 16), (2708, 5278, 7), (50, 400, 3), (300, 100, 70), (10, 0, 4)])
+def test_scatter_gcn_fwd_bwd_bit_exact(oracle, hip, n_nodes, n_pairs, stride):
+    r = rng(n_nodes + stride)
+    src, tgt = random_graph(r, n_nodes, n_pairs)
+    E = src.size
+    h = r.standard_normal(n_nodes * stride).astype(np.float32)
+    indeg = np.bincount(tgt.astype(np.int64), minlength=n_nodes).astype(np.float32)
+    deg = (1.0 / np.sqrt(1.0 + indeg)).astype(np.float32)
+    dst0 = np.zeros(n_nodes * stride, np.float32)
+    a, b = both(oracle, hip, "scatter_gcn_deg_scaled", {"dst": dst0, "h": h, "deg": deg, "src_indices": src, "tgt_indices": tgt,
+                                                        "stride": stride, "n_edge": E}, ["dst"])
+    np.testing.assert_array_equal(a["dst"], b["dst"])
+    # textbook cross-check: dense D^-1/2 A D^-1/2 H
+    Aw = np.zeros((n_nodes, n_nodes))
+    np.add.at(Aw, (tgt.astype(np.int64), src.astype(np.int64)), 1.0)
+    dense = (deg[:, None].astype(np.float64) * Aw * deg[None, :].astype(np.float64)) @ h.reshape(n_nodes, stride).astype(np.float64)
+    assert rel_fro(b["dst"], dense.ravel()) <= TOL
+    go = r.standard_normal(n_nodes * stride).astype(np.float32)
+    gh0 = r.standard_normal(n_nodes * stride).astype(np.float32)
+    gd0 = r.standard_normal(n_nodes).astype(np.float32)
+    a, b = both(oracle, hip, "scatter_gcn_deg_scaled_bwd", {"grad_output": go, "h": h, "deg": deg, "src_indices": src,
+                                                            "tgt_indices": tgt, "grad_h": gh0, "grad_deg": gd0, "stride": stride,
+                                                            "n_edge": E}, ["grad_h", "grad_deg"])
+    np.testing.assert_array_equal(a["grad_h"], b["grad_h"])
+    np.testing.assert_array_equal(a["grad_deg"], b["grad_deg"])
+
+
+def test_scatter_gcn_indices_in_pinned_host_memory(oracle, hip):
+    """The reference hands the device op index slices that live in host memory (examples/gcn/src/model.zig:204-205)."""
+    r = rng(21)
+    n_nodes, stride = 200, 16
+    src, tgt = random_graph(r, n_nodes, 600)
+    h = r.standard_normal(n_nodes * stride).astype(np.float32)
+    deg = (r.random(n_nodes) + 0.5).astype(np.float32)
+    want = run_op(oracle, "scatter_gcn_deg_scaled", {"dst": np.zeros(n_nodes * stride, np.float32), "h": h, "deg": deg,
+                                                     "src_indices": src, "tgt_indices": tgt, "stride": stride, "n_edge": src.size},
+                  ["dst"])["dst"]
+    S, T = hip.mem_alloc_host(np.uint64, src.size), hip.mem_alloc_host(np.uint64, tgt.size)
+    hip.mem_transfer(src, S, "HtoD")
+    hip.mem_transfer(tgt, T, "HtoD")
+    D, H, G = hip.from_numpy(np.zeros(n_nodes * stride, np.float32)), hip.from_numpy(h), hip.from_numpy(deg)
+    hip.dispatch("scatter_gcn_deg_scaled", dst=D, h=H, deg=G, src_indices=S, tgt_indices=T, stride=stride, n_edge=src.size)
+    hip.sync()
+    np.testing.assert_array_equal(hip.to_numpy(D), want)

@@ -1,0 +1,106 @@
+// Shared declarations of the gfx950 backend: context, error reporting, launch helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/zg_hip.h"
+
+#define ZG_API extern "C" __attribute__((visibility("default")))
+
+namespace zg {
+
+constexpr int kWave = 64;          // CDNA wavefront width
+constexpr int kBlock = 256;        // default workgroup: 4 waves, one per SIMD
+constexpr size_t kPoolAlign = 256; // min split size of the block pools, bytes
+
+void set_error(const char* fmt, ...);
+
+struct BlockPool;  // allocator.cpp
+
+}  // namespace zg
+
+struct zg_hip_event {
+    hipEvent_t ev;
+};
+
+struct zg_hip_ctx {
+    int device = 0;
+    int n_cu = 256;
+    size_t total_mem = 0;
+    hipStream_t stream = nullptr;
+
+    // Internal workspace for multi-stage reductions and sort plans. Grow-only; growth synchronises the stream.
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+
+    // small device slots for scalars: [0] staged host scalar (axpy alpha), [1] clip factor
+    float* scalar_slot = nullptr;
+    // fixed buffer for the per-workgroup partials of flat reductions (64 KiB)
+    void* partials = nullptr;
+
+    // caching allocator state (allocator.cpp)
+    zg::BlockPool* small_pool = nullptr;
+    zg::BlockPool* large_pool = nullptr;
+    size_t small_pool_bytes = 0;
+    size_t large_pool_bytes = 0;
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    uint64_t n_device_allocs = 0;
+
+    // regions handed out by pool_map/alloc, for ownership checks at free time
+    std::map<void*, size_t> raw_allocs;
+    std::map<void*, size_t> host_allocs;
+};
+
+namespace zg {
+
+// Returns a workspace of at least `bytes` bytes (256-byte aligned), or nullptr with the error set.
+void* workspace(zg_hip_ctx* ctx, size_t bytes);
+
+inline int ceil_div(size_t a, size_t b) {
+    return (int)((a + b - 1) / b);
+}
+inline size_t ceil_div_sz(size_t a, size_t b) {
+    return (a + b - 1) / b;
+}
+inline bool aligned16(const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+}  // namespace zg
+
+#define ZG_REQUIRE(cond, ...)             \
+    do {                                  \
+        if (!(cond)) {                    \
+            zg::set_error(__VA_ARGS__);   \
+            return ZG_HIP_EINVAL;         \
+        }                                 \
+    } while (0)
+
+#define ZG_HIP_TRY(expr)                                                                         \
+    do {                                                                                         \
+        hipError_t _e = (expr);                                                                  \
+        if (_e != hipSuccess) {                                                                  \
+            zg::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+            return (_e == hipErrorOutOfMemory) ? ZG_HIP_EOOM : ZG_HIP_ERUNTIME;                  \
+        }                                                                                        \
+    } while (0)
+
+// After a kernel launch: report launch-configuration errors without synchronising.
+#define ZG_LAUNCH_CHECK()                                                                        \
+    do {                                                                                         \
+        hipError_t _e = hipGetLastError();                                                       \
+        if (_e != hipSuccess) {                                                                  \
+            zg::set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(_e), __FILE__, __LINE__); \
+            return ZG_HIP_ERUNTIME;                                                              \
+        }                                                                                        \
+    } while (0)
+
+#define ZG_CTX(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")

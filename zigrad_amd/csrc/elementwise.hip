@@ -1,0 +1,418 @@
+// Elementwise binary (broadcasting) and unary forward/backward ops.
+//
+// All of these are HBM-bound streams.  The kernels move 128 bits per lane per access, keep four
+// independent accesses in flight per thread and never re-read an operand; the broadcasting form
+// holds the short operand in registers while it walks down the rows of the long one.
+// Arithmetic is kept as separate fp32 multiplies and adds (no contraction) so each element rounds
+// exactly like the host loop it replaces.
+#include "common.h"
+
+namespace zg {
+
+// ------------------------------------------------------------------------------------------------
+// generic map kernel: out[i] = Op::f(a[i], b[i], c[i], p0, p1)
+// ------------------------------------------------------------------------------------------------
+constexpr int kUnroll = 4;
+
+template <class Op, int NIN>
+__global__ __launch_bounds__(kBlock) void map_vec4_kernel(float* out, const float* a, const float* b,
+                                                           const float* c, size_t n, float p0, float p1) {
+    const size_t n4 = n >> 2;
+    const float4* a4 = reinterpret_cast<const float4*>(a);
+    const float4* b4 = reinterpret_cast<const float4*>(b);
+    const float4* c4 = reinterpret_cast<const float4*>(c);
+    float4* o4 = reinterpret_cast<float4*>(out);
+    size_t base = (size_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * (kBlock * kUnroll);
+    for (; base < n4; base += stride) {
+        float4 va[kUnroll], vb[kUnroll], vc[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            size_t i = base + (size_t)u * kBlock;
+            if (i < n4) {
+                va[u] = a4[i];
+                if (NIN > 1) vb[u] = b4[i];
+                if (NIN > 2) vc[u] = c4[i];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            size_t i = base + (size_t)u * kBlock;
+            if (i < n4) {
+                float4 r;
+                r.x = Op::f(va[u].x, NIN > 1 ? vb[u].x : 0.f, NIN > 2 ? vc[u].x : 0.f, p0, p1);
+                r.y = Op::f(va[u].y, NIN > 1 ? vb[u].y : 0.f, NIN > 2 ? vc[u].y : 0.f, p0, p1);
+                r.z = Op::f(va[u].z, NIN > 1 ? vb[u].z : 0.f, NIN > 2 ? vc[u].z : 0.f, p0, p1);
+                r.w = Op::f(va[u].w, NIN > 1 ? vb[u].w : 0.f, NIN > 2 ? vc[u].w : 0.f, p0, p1);
+                o4[i] = r;
+            }
+        }
+    }
+    // tail (n % 4 elements), handled by the first threads of block 0
+    const size_t tail0 = n4 << 2;
+    if (blockIdx.x == 0) {
+        size_t i = tail0 + threadIdx.x;
+        if (i < n) out[i] = Op::f(a[i], NIN > 1 ? b[i] : 0.f, NIN > 2 ? c[i] : 0.f, p0, p1);
+    }
+}
+
+template <class Op, int NIN>
+__global__ __launch_bounds__(kBlock) void map_scalar_kernel(float* out, const float* a, const float* b,
+                                                             const float* c, size_t n, float p0, float p1) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) out[i] = Op::f(a[i], NIN > 1 ? b[i] : 0.f, NIN > 2 ? c[i] : 0.f, p0, p1);
+}
+
+static int map_grid(zg_hip_ctx* ctx, size_t items, int per_block) {
+    size_t blocks = ceil_div_sz(items, (size_t)per_block);
+    size_t cap = (size_t)ctx->n_cu * 32;
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+template <class Op, int NIN>
+static int launch_map(zg_hip_ctx* ctx, float* out, const float* a, const float* b, const float* c, size_t n,
+                      float p0 = 0.f, float p1 = 0.f) {
+    if (n == 0) return ZG_HIP_OK;
+    bool vec = aligned16(out) && aligned16(a) && (NIN < 2 || aligned16(b)) && (NIN < 3 || aligned16(c)) && n >= 4;
+    if (vec) {
+        int grid = map_grid(ctx, n >> 2, kBlock * kUnroll);
+        hipLaunchKernelGGL((map_vec4_kernel<Op, NIN>), dim3(grid), dim3(kBlock), 0, ctx->stream, out, a, b, c, n, p0,
+                           p1);
+    } else {
+        int grid = map_grid(ctx, n, kBlock);
+        hipLaunchKernelGGL((map_scalar_kernel<Op, NIN>), dim3(grid), dim3(kBlock), 0, ctx->stream, out, a, b, c, n, p0,
+                           p1);
+    }
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// binary ops with the reference's broadcasting regimes
+// ------------------------------------------------------------------------------------------------
+struct AddOp { static __device__ __forceinline__ float f(float a, float b) { return __fadd_rn(a, b); } };
+struct SubOp { static __device__ __forceinline__ float f(float a, float b) { return __fsub_rn(a, b); } };
+struct MulOp { static __device__ __forceinline__ float f(float a, float b) { return __fmul_rn(a, b); } };
+struct DivOp { static __device__ __forceinline__ float f(float a, float b) { return __fdiv_rn(a, b); } };
+
+// adapters to the map kernel
+template <class B> struct Bin2 { static __device__ __forceinline__ float f(float a, float b, float, float, float) { return B::f(a, b); } };
+// scalar operand broadcast from device memory: p is read once per thread
+template <class B, bool SCALAR_LHS>
+__global__ __launch_bounds__(kBlock) void bin_scalar_kernel(float* out, const float* vec, const float* scalar,
+                                                             size_t n) {
+    const float s = scalar[0];
+    const bool v4ok = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(vec)) & 15u) == 0;
+    if (v4ok) {
+        const size_t n4 = n >> 2;
+        const float4* v4 = reinterpret_cast<const float4*>(vec);
+        float4* o4 = reinterpret_cast<float4*>(out);
+        size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+        const size_t stride = (size_t)gridDim.x * kBlock;
+        for (; i < n4; i += stride) {
+            float4 v = v4[i], r;
+            r.x = SCALAR_LHS ? B::f(s, v.x) : B::f(v.x, s);
+            r.y = SCALAR_LHS ? B::f(s, v.y) : B::f(v.y, s);
+            r.z = SCALAR_LHS ? B::f(s, v.z) : B::f(v.z, s);
+            r.w = SCALAR_LHS ? B::f(s, v.w) : B::f(v.w, s);
+            o4[i] = r;
+        }
+        if (blockIdx.x == 0) {
+            size_t t = (n4 << 2) + threadIdx.x;
+            if (t < n) out[t] = SCALAR_LHS ? B::f(s, vec[t]) : B::f(vec[t], s);
+        }
+    } else {
+        size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+        const size_t stride = (size_t)gridDim.x * kBlock;
+        for (; i < n; i += stride) out[i] = SCALAR_LHS ? B::f(s, vec[i]) : B::f(vec[i], s);
+    }
+}
+
+// Row broadcast: `lng` is [rows, period], `sht` is [period]; period % 4 == 0, all 16-byte aligned.
+// Thread (tx, ty): tx walks float4 columns, ty walks rows; the short operand stays in registers.
+constexpr int kRbX = 64, kRbY = 4, kRbRows = 4;
+template <class B, bool SHORT_LHS>
+__global__ __launch_bounds__(kRbX * kRbY) void bin_rowbcast_kernel(float* out, const float* lng, const float* sht,
+                                                                    size_t rows, size_t p4) {
+    const size_t col = (size_t)blockIdx.x * kRbX + threadIdx.x;
+    if (col >= p4) return;
+    const float4 s = reinterpret_cast<const float4*>(sht)[col];
+    const float4* l4 = reinterpret_cast<const float4*>(lng);
+    float4* o4 = reinterpret_cast<float4*>(out);
+    const size_t row_step = (size_t)gridDim.y * kRbY;
+    // each thread handles kRbRows rows per trip: rows r, r+row_step, ...
+    size_t r = (size_t)blockIdx.y * kRbY + threadIdx.y;
+    for (; r < rows; r += row_step * kRbRows) {
+        float4 v[kRbRows];
+#pragma unroll
+        for (int u = 0; u < kRbRows; u++) {
+            size_t rr = r + (size_t)u * row_step;
+            if (rr < rows) v[u] = l4[rr * p4 + col];
+        }
+#pragma unroll
+        for (int u = 0; u < kRbRows; u++) {
+            size_t rr = r + (size_t)u * row_step;
+            if (rr < rows) {
+                float4 q;
+                q.x = SHORT_LHS ? B::f(s.x, v[u].x) : B::f(v[u].x, s.x);
+                q.y = SHORT_LHS ? B::f(s.y, v[u].y) : B::f(v[u].y, s.y);
+                q.z = SHORT_LHS ? B::f(s.z, v[u].z) : B::f(v[u].z, s.z);
+                q.w = SHORT_LHS ? B::f(s.w, v[u].w) : B::f(v[u].w, s.w);
+                o4[rr * p4 + col] = q;
+            }
+        }
+    }
+}
+
+// Fallback for any period/alignment: z[i] = x[i % xl] o y[i % yl] (one of the two is the identity map)
+template <class B>
+__global__ __launch_bounds__(kBlock) void bin_modulo_kernel(float* out, const float* x, size_t xl, const float* y,
+                                                             size_t yl, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) {
+        size_t xi = (xl == n) ? i : i % xl;
+        size_t yi = (yl == n) ? i : i % yl;
+        out[i] = B::f(x[xi], y[yi]);
+    }
+}
+
+__global__ void broadcast_modulo_kernel(float* y, const float* x, size_t xl, size_t yl, float alpha, float beta) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < yl; i += stride) y[i] = __fadd_rn(__fmul_rn(alpha, x[i % xl]), __fmul_rn(beta, y[i]));
+}
+
+template <class B>
+static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t xl, const float* y, size_t yl, float* z,
+                     size_t zl) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(xl > 0 && yl > 0 && zl > 0, "%s: empty operand", name);
+    ZG_REQUIRE(x && y && z, "%s: null pointer", name);
+    const size_t mx = xl > yl ? xl : yl, mn = xl < yl ? xl : yl;
+    // src/device/opspec.zig:1-11: the longer length is a multiple of the shorter and z has the longer length
+    ZG_REQUIRE(mx % mn == 0, "%s: lengths %zu and %zu do not broadcast", name, xl, yl);
+    ZG_REQUIRE(zl == mx, "%s: z.len %zu != max(x.len, y.len) %zu", name, zl, mx);
+
+    if (xl == yl) return launch_map<Bin2<B>, 2>(ctx, z, x, y, nullptr, zl);
+    if (mn == 1) {
+        int grid = map_grid(ctx, (zl + 3) / 4, kBlock);
+        if (xl == 1)
+            hipLaunchKernelGGL((bin_scalar_kernel<B, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, y, x, zl);
+        else
+            hipLaunchKernelGGL((bin_scalar_kernel<B, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, x, y, zl);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    const bool short_lhs = xl < yl;
+    const float* lng = short_lhs ? y : x;
+    const float* sht = short_lhs ? x : y;
+    if (mn % 4 == 0 && aligned16(lng) && aligned16(sht) && aligned16(z)) {
+        size_t p4 = mn / 4, rows = mx / mn;
+        unsigned gx = (unsigned)ceil_div_sz(p4, kRbX);
+        // enough row groups to fill the machine, each thread then loops over the rest
+        size_t want_blocks = (size_t)ctx->n_cu * 16;
+        size_t gy = ceil_div_sz(want_blocks, gx);
+        size_t max_gy = ceil_div_sz(rows, (size_t)kRbY * kRbRows);
+        if (gy > max_gy) gy = max_gy;
+        if (gy < 1) gy = 1;
+        if (gy > 65535) gy = 65535;
+        dim3 grid(gx, (unsigned)gy), block(kRbX, kRbY);
+        if (short_lhs)
+            hipLaunchKernelGGL((bin_rowbcast_kernel<B, true>), grid, block, 0, ctx->stream, z, lng, sht, rows, p4);
+        else
+            hipLaunchKernelGGL((bin_rowbcast_kernel<B, false>), grid, block, 0, ctx->stream, z, lng, sht, rows, p4);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    int grid = map_grid(ctx, zl, kBlock);
+    hipLaunchKernelGGL((bin_modulo_kernel<B>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, x, xl, y, yl, zl);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// unary forward/backward functors.  Argument order of f() is the order the launcher passes arrays.
+// ------------------------------------------------------------------------------------------------
+#define ZG_OP(NAME, BODY)                                                                        \
+    struct NAME {                                                                                \
+        static __device__ __forceinline__ float f(float a, float b, float c, float p0, float p1) { \
+            (void)a; (void)b; (void)c; (void)p0; (void)p1;                                       \
+            BODY                                                                                 \
+        }                                                                                        \
+    };
+
+// forward ops: a = x
+ZG_OP(PowFwd, return powf(a, p0);)
+ZG_OP(SqrtFwd, return __fsqrt_rn(a);)
+ZG_OP(RsqrtFwd, return __fdiv_rn(1.0f, __fsqrt_rn(fmaxf(a, p0)));)
+ZG_OP(ExpFwd, return expf(a);)
+ZG_OP(ReluFwd, return a > 0.f ? a : 0.f;)
+ZG_OP(TanhFwd, return tanhf(a);)
+ZG_OP(SigmFwd, return __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-a)));)
+ZG_OP(ClampFwd, return fminf(p1, fmaxf(p0, a));)
+// backward ops: a = x (or y), b = x_g (accumulated into), c = y_g
+ZG_OP(PowBwd, if (a < p1) return __fadd_rn(b, 0.0f);
+      return __fadd_rn(b, __fmul_rn(__fmul_rn(p0, powf(a, __fsub_rn(p0, 1.0f))), c));)
+ZG_OP(SqrtBwd, if (a < p0) return __fadd_rn(b, 0.0f);
+      return __fadd_rn(b, __fmul_rn(__fdiv_rn(0.5f, __fsqrt_rn(a)), c));)
+ZG_OP(RsqrtBwd, if (a < p0) return __fadd_rn(b, 0.0f);
+      float s = __fsqrt_rn(a); float inv = __fdiv_rn(1.0f, __fmul_rn(a, s));
+      return __fadd_rn(b, __fmul_rn(__fmul_rn(-0.5f, inv), c));)
+// exp_bwd: a = y, b = x_g, c = y_g
+ZG_OP(ExpBwd, return __fadd_rn(b, __fmul_rn(a, c));)
+ZG_OP(ReluBwd, return __fadd_rn(b, (a > 0.f) ? c : 0.f);)
+// relu_inplace_bwd: a = x, b = x_g
+ZG_OP(ReluInplaceBwd, return (a <= 0.f) ? 0.f : b;)
+// tanh_bwd: a = y, b = x_g, c = y_g
+ZG_OP(TanhBwd, return __fadd_rn(b, __fmul_rn(__fsub_rn(1.0f, __fmul_rn(a, a)), c));)
+ZG_OP(TanhInplaceBwd, return __fmul_rn(b, __fsub_rn(1.0f, __fmul_rn(a, a)));)
+ZG_OP(SigmBwd, return __fadd_rn(b, __fmul_rn(__fmul_rn(a, __fsub_rn(1.0f, a)), c));)
+ZG_OP(SigmInplaceBwd, return __fmul_rn(b, __fmul_rn(a, __fsub_rn(1.0f, a)));)
+ZG_OP(ClampBwd, return (p0 < a && a < p1) ? __fadd_rn(b, c) : b;)
+// scale: a = x
+ZG_OP(ScaleOp, return __fmul_rn(a, p0);)
+// broadcast / scaled copy: a = x, b = y -> alpha*x + beta*y
+ZG_OP(ScaledCopy, return __fadd_rn(__fmul_rn(p0, a), __fmul_rn(p1, b));)
+ZG_OP(ScaledCopyNoRead, return __fmul_rn(p0, a);)
+// smooth-l1 / mse backward: a = pred, b = target, c = grad; p0 = beta or scale, p1 = n
+ZG_OP(SmoothL1Bwd, float d = __fsub_rn(a, b);
+      if (fabsf(d) < p0) return __fadd_rn(c, __fdiv_rn(d, __fmul_rn(p0, p1)));
+      float sg = (d > 0.f) ? 1.f : ((d < 0.f) ? -1.f : 0.f); return __fadd_rn(c, __fdiv_rn(sg, p1));)
+ZG_OP(MseBwd, return __fadd_rn(c, __fmul_rn(p0, __fsub_rn(a, b)));)
+
+}  // namespace zg
+
+using namespace zg;
+
+#define ZG_CHECK_N(name, n, ...)                                         \
+    ZG_CTX(ctx);                                                         \
+    if ((n) == 0) return ZG_HIP_OK;                                      \
+    {                                                                    \
+        const void* _ptrs[] = {__VA_ARGS__};                             \
+        for (const void* _p : _ptrs) ZG_REQUIRE(_p != nullptr, "%s: null pointer", name); \
+    }
+
+ZG_API int zg_hip_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
+    return binary_op<AddOp>(ctx, "add", x, xl, y, yl, z, zl);
+}
+ZG_API int zg_hip_sub(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
+    return binary_op<SubOp>(ctx, "sub", x, xl, y, yl, z, zl);
+}
+ZG_API int zg_hip_mul(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
+    return binary_op<MulOp>(ctx, "mul", x, xl, y, yl, z, zl);
+}
+ZG_API int zg_hip_div(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
+    return binary_op<DivOp>(ctx, "div", x, xl, y, yl, z, zl);
+}
+
+ZG_API int zg_hip_pow_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n, float e) {
+    ZG_CHECK_N("pow_fwd", n, x, y);
+    return launch_map<PowFwd, 1>(ctx, y, x, nullptr, nullptr, n, e);
+}
+ZG_API int zg_hip_pow_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, const float* y_g, size_t n, float e, float eps) {
+    ZG_CHECK_N("pow_bwd", n, x, x_g, y_g);
+    return launch_map<PowBwd, 3>(ctx, x_g, x, x_g, y_g, n, e, eps);
+}
+ZG_API int zg_hip_sqrt_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) {
+    ZG_CHECK_N("sqrt_fwd", n, x, y);
+    return launch_map<SqrtFwd, 1>(ctx, y, x, nullptr, nullptr, n);
+}
+ZG_API int zg_hip_sqrt_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, const float* y_g, size_t n, float eps) {
+    ZG_CHECK_N("sqrt_bwd", n, x, x_g, y_g);
+    return launch_map<SqrtBwd, 3>(ctx, x_g, x, x_g, y_g, n, eps);
+}
+ZG_API int zg_hip_rsqrt_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n, float eps) {
+    ZG_CHECK_N("rsqrt_fwd", n, x, y);
+    return launch_map<RsqrtFwd, 1>(ctx, y, x, nullptr, nullptr, n, eps);
+}
+ZG_API int zg_hip_rsqrt_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, const float* y_g, size_t n, float eps) {
+    ZG_CHECK_N("rsqrt_bwd", n, x, x_g, y_g);
+    return launch_map<RsqrtBwd, 3>(ctx, x_g, x, x_g, y_g, n, eps);
+}
+ZG_API int zg_hip_exp_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) {
+    ZG_CHECK_N("exp_fwd", n, x, y);
+    return launch_map<ExpFwd, 1>(ctx, y, x, nullptr, nullptr, n);
+}
+ZG_API int zg_hip_exp_bwd(zg_hip_ctx* ctx, float* x_g, const float* y, const float* y_g, size_t n) {
+    ZG_CHECK_N("exp_bwd", n, x_g, y, y_g);
+    return launch_map<ExpBwd, 3>(ctx, x_g, y, x_g, y_g, n);
+}
+ZG_API int zg_hip_relu_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) {
+    ZG_CHECK_N("relu_fwd", n, x, y);
+    return launch_map<ReluFwd, 1>(ctx, y, x, nullptr, nullptr, n);
+}
+ZG_API int zg_hip_relu_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, const float* y_g, size_t n) {
+    ZG_CHECK_N("relu_bwd", n, x, x_g, y_g);
+    return launch_map<ReluBwd, 3>(ctx, x_g, x, x_g, y_g, n);
+}
+ZG_API int zg_hip_relu_inplace_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, size_t n) {
+    ZG_CHECK_N("relu_inplace_bwd", n, x, x_g);
+    return launch_map<ReluInplaceBwd, 2>(ctx, x_g, x, x_g, nullptr, n);
+}
+ZG_API int zg_hip_tanh_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) {
+    ZG_CHECK_N("tanh_fwd", n, x, y);
+    return launch_map<TanhFwd, 1>(ctx, y, x, nullptr, nullptr, n);
+}
+ZG_API int zg_hip_tanh_bwd(zg_hip_ctx* ctx, float* x_g, const float* y, const float* y_g, size_t n) {
+    ZG_CHECK_N("tanh_bwd", n, x_g, y, y_g);
+    return launch_map<TanhBwd, 3>(ctx, x_g, y, x_g, y_g, n);
+}
+ZG_API int zg_hip_tanh_inplace_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, size_t n) {
+    ZG_CHECK_N("tanh_inplace_bwd", n, x, x_g);
+    return launch_map<TanhInplaceBwd, 2>(ctx, x_g, x, x_g, nullptr, n);
+}
+ZG_API int zg_hip_sigm_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) {
+    ZG_CHECK_N("sigm_fwd", n, x, y);
+    return launch_map<SigmFwd, 1>(ctx, y, x, nullptr, nullptr, n);
+}
+ZG_API int zg_hip_sigm_bwd(zg_hip_ctx* ctx, float* x_g, const float* y, const float* y_g, size_t n) {
+    ZG_CHECK_N("sigm_bwd", n, x_g, y, y_g);
+    return launch_map<SigmBwd, 3>(ctx, x_g, y, x_g, y_g, n);
+}
+ZG_API int zg_hip_sigm_inplace_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, size_t n) {
+    ZG_CHECK_N("sigm_inplace_bwd", n, x, x_g);
+    return launch_map<SigmInplaceBwd, 2>(ctx, x_g, x, x_g, nullptr, n);
+}
+ZG_API int zg_hip_clamp_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n, float lo, float hi) {
+    ZG_CHECK_N("clamp_fwd", n, x, y);
+    return launch_map<ClampFwd, 1>(ctx, y, x, nullptr, nullptr, n, lo, hi);
+}
+ZG_API int zg_hip_clamp_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, const float* y_g, size_t n, float lo,
+                            float hi) {
+    ZG_CHECK_N("clamp_bwd", n, x, x_g, y_g);
+    return launch_map<ClampBwd, 3>(ctx, x_g, x, x_g, y_g, n, lo, hi);
+}
+ZG_API int zg_hip_scale(zg_hip_ctx* ctx, float* x, size_t n, float alpha) {
+    ZG_CHECK_N("scale", n, x);
+    return launch_map<ScaleOp, 1>(ctx, x, x, nullptr, nullptr, n, alpha);
+}
+
+// src/device/host_device.zig:782-795 (see the oracle for the double application when lengths are equal)
+ZG_API int zg_hip_broadcast(zg_hip_ctx* ctx, const float* x, size_t xl, float* y, size_t yl, float alpha, float beta) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(xl > 0 && yl > 0 && x && y, "broadcast: empty or null operand");
+    ZG_REQUIRE(yl % xl == 0, "broadcast: y.len %zu is not a multiple of x.len %zu", yl, xl);
+    if (xl == yl) {
+        int rc = launch_map<ScaledCopy, 2>(ctx, y, x, y, nullptr, yl, alpha, beta);
+        if (rc) return rc;
+        return launch_map<ScaledCopy, 2>(ctx, y, x, y, nullptr, yl, alpha, beta);
+    }
+    int grid = map_grid(ctx, yl, kBlock);
+    hipLaunchKernelGGL(broadcast_modulo_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, y, x, xl, yl, alpha, beta);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_smooth_l1_bwd(zg_hip_ctx* ctx, const float* pred, const float* target, float* grad, size_t n,
+                                float beta) {
+    ZG_CHECK_N("smooth_l1_bwd", n, pred, target, grad);
+    return launch_map<SmoothL1Bwd, 3>(ctx, grad, pred, target, grad, n, beta, (float)n);
+}
+
+ZG_API int zg_hip_mse_bwd(zg_hip_ctx* ctx, const float* pred, const float* target, float* grad, size_t n) {
+    ZG_CHECK_N("mse_bwd", n, pred, target, grad);
+    return launch_map<MseBwd, 3>(ctx, grad, pred, target, grad, n, 2.0f / (float)n);
+}

@@ -1,0 +1,528 @@
+// Indexing ops: gather offsets, scatter_add, index_select fwd/bwd and the GCN degree-scaled
+// message-passing scatter with its backward.
+//
+// Every accumulating op here is a destination-sorted segmented reduction: the input indices are
+// bucketed by destination (integer histogram + scan + placement), each bucket is put back into input
+// order, and one thread group then adds a destination's contributions one after the other in that
+// order.  That is the order of the sequential host loops (src/device/host_device.zig:1039-1087,
+// :1356-1403), so results are deterministic and round like the host's; there are no floating-point
+// atomics.  The work is latency/HBM bound: indices and rows are read once, destinations written once.
+#include "common.h"
+
+namespace zg {
+
+// ------------------------------------------------------------------------------------------------
+// segment plan: row_ptr[nb + 1], perm[n] (input positions grouped by bucket, ascending inside a bucket)
+// ------------------------------------------------------------------------------------------------
+struct Plan {
+    uint32_t* row_ptr;   // nb + 1
+    uint32_t* cursor;    // nb
+    uint32_t* perm_tmp;  // n
+    uint32_t* perm;      // n
+    uint32_t* tile_sums; // scan scratch
+    size_t n, nb;
+};
+
+constexpr int kScanTile = 2048;  // elements per workgroup of the scan (256 threads x 8)
+
+static size_t align_up(size_t v, size_t a) {
+    return (v + a - 1) / a * a;
+}
+
+static size_t plan_bytes(size_t n, size_t nb) {
+    size_t tiles = ceil_div_sz(nb + 1, kScanTile);
+    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 2 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256);
+}
+
+static Plan carve_plan(void* mem, size_t n, size_t nb) {
+    char* p = (char*)mem;
+    Plan pl;
+    pl.n = n;
+    pl.nb = nb;
+    pl.row_ptr = (uint32_t*)p;
+    p += align_up((nb + 1) * 4, 256);
+    pl.cursor = (uint32_t*)p;
+    p += align_up(nb * 4, 256);
+    pl.perm_tmp = (uint32_t*)p;
+    p += align_up(n * 4, 256);
+    pl.perm = (uint32_t*)p;
+    p += align_up(n * 4, 256);
+    pl.tile_sums = (uint32_t*)p;
+    return pl;
+}
+
+__global__ void zero_u32_kernel(uint32_t* a, size_t na, uint32_t* b, size_t nb) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (size_t k = i; k < na; k += nt) a[k] = 0;
+    for (size_t k = i; k < nb; k += nt) b[k] = 0;
+}
+
+// key = idx[e] / divisor (divisor 1 for plain indices)
+__global__ void histogram_kernel(const uint64_t* keys, size_t n, size_t nb, uint32_t* counts) {
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (; e < n; e += nt) {
+        uint64_t k = keys[e];
+        if (k < nb) atomicAdd(&counts[k], 1u);
+    }
+}
+
+// exclusive scan, three launches: per-tile scan + tile sums, scan of tile sums (one workgroup), add back
+__global__ __launch_bounds__(256) void scan_tiles_kernel(uint32_t* data, size_t n, uint32_t* tile_sums) {
+    __shared__ uint32_t wave_tot[4];
+    const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * 8;
+    uint32_t v[8], s = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        v[k] = (base + k < n) ? data[base + k] : 0;
+        s += v[k];
+    }
+    // inclusive scan of s across the workgroup
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = s;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        uint32_t t = __shfl_up(inc, d, 64);
+        if (lane >= d) inc += t;
+    }
+    if (lane == 63) wave_tot[wave] = inc;
+    __syncthreads();
+    uint32_t wave_off = 0;
+    for (int w = 0; w < wave; w++) wave_off += wave_tot[w];
+    uint32_t run = wave_off + inc - s;  // exclusive prefix of this thread's first element
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        if (base + k < n) data[base + k] = run;
+        run += v[k];
+    }
+    if (threadIdx.x == 255) tile_sums[blockIdx.x] = wave_off + inc;
+}
+
+__global__ __launch_bounds__(256) void scan_sums_kernel(uint32_t* tile_sums, size_t tiles) {
+    // one workgroup walks the tile sums in chunks of 256, carrying the running total
+    __shared__ uint32_t wave_tot[4];
+    __shared__ uint32_t carry_s;
+    if (threadIdx.x == 0) carry_s = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (size_t c = 0; c < tiles; c += 256) {
+        size_t i = c + threadIdx.x;
+        uint32_t s = (i < tiles) ? tile_sums[i] : 0;
+        uint32_t inc = s;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            uint32_t t = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += t;
+        }
+        if (lane == 63) wave_tot[wave] = inc;
+        __syncthreads();
+        uint32_t off = carry_s;
+        for (int w = 0; w < wave; w++) off += wave_tot[w];
+        if (i < tiles) tile_sums[i] = off + inc - s;
+        __syncthreads();
+        if (threadIdx.x == 255) carry_s = off + inc;
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void scan_add_kernel(uint32_t* data, size_t n, const uint32_t* tile_sums) {
+    const uint32_t off = tile_sums[blockIdx.x];
+    const size_t base = (size_t)blockIdx.x * kScanTile;
+    for (int k = threadIdx.x; k < kScanTile; k += 256)
+        if (base + k < n) data[base + k] += off;
+}
+
+__global__ void place_kernel(const uint64_t* keys, size_t n, size_t nb, const uint32_t* row_ptr, uint32_t* cursor,
+                             uint32_t* perm_tmp) {
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (; e < n; e += nt) {
+        uint64_t k = keys[e];
+        if (k < nb) {
+            uint32_t pos = row_ptr[k] + atomicAdd(&cursor[k], 1u);
+            perm_tmp[pos] = (uint32_t)e;
+        }
+    }
+}
+
+// Put each bucket back into ascending input position: rank of an entry = number of smaller entries
+// in its bucket.  One wave per bucket.
+__global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
+                                                              uint32_t* perm) {
+    const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= nb) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t s = row_ptr[b], len = row_ptr[b + 1] - s;
+    for (uint32_t i = lane; i < len; i += 64) {
+        const uint32_t id = perm_tmp[s + i];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < len; j++) rank += (perm_tmp[s + j] < id) ? 1u : 0u;
+        perm[s + rank] = id;
+    }
+}
+
+static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl) {
+    hipStream_t st = ctx->stream;
+    const size_t n = pl.n, nb = pl.nb;
+    const int g_n = (int)(ceil_div_sz(n ? n : 1, 256) > 4096 ? 4096 : ceil_div_sz(n ? n : 1, 256));
+    const int g_b = (int)(ceil_div_sz(nb + 1, 256) > 4096 ? 4096 : ceil_div_sz(nb + 1, 256));
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(g_b), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.cursor, nb);
+    ZG_LAUNCH_CHECK();
+    if (n) {
+        hipLaunchKernelGGL(histogram_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr);
+        ZG_LAUNCH_CHECK();
+    }
+    const size_t tiles = ceil_div_sz(nb + 1, kScanTile);
+    hipLaunchKernelGGL(scan_tiles_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
+    ZG_LAUNCH_CHECK();
+    if (tiles > 1) {
+        hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, pl.tile_sums, tiles);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_add_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
+        ZG_LAUNCH_CHECK();
+    }
+    if (n) {
+        hipLaunchKernelGGL(place_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr, pl.cursor, pl.perm_tmp);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(nb, 4)), dim3(256), 0, st, pl.row_ptr, nb,
+                           pl.perm_tmp, pl.perm);
+        ZG_LAUNCH_CHECK();
+    }
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// apply kernels
+// ------------------------------------------------------------------------------------------------
+
+// dst[b] += src[e] for the bucket's entries in input order; one thread per destination
+__global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_ptr, const uint32_t* perm, float* dst,
+                                         size_t nb) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nb) return;
+    const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
+    if (s == e) return;
+    float acc = dst[b];
+    for (uint32_t k = s; k < e; k++) acc = __fadd_rn(acc, src[perm[k]]);
+    dst[b] = acc;
+}
+
+// rows of `stride` elements: dst[b, :] = src_row(e) + dst[b, :] in input order.  G threads per destination row.
+// MODE 0: index_select backward  (x_grad[row] = y_grad[e] + x_grad[row], src/ndtensor.zig:1461-1465)
+template <int G>
+__global__ __launch_bounds__(256) void row_scatter_apply_kernel(const float* src, const uint32_t* row_ptr,
+                                                                 const uint32_t* perm, float* dst, size_t nb,
+                                                                 size_t stride) {
+    const size_t b = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
+    if (b >= nb) return;
+    const int lane = threadIdx.x % G;
+    const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
+    if (s == e) return;
+    for (size_t j = lane; j < stride; j += G) {
+        float acc = dst[b * stride + j];
+        for (uint32_t k = s; k < e; k++) acc = __fadd_rn(src[(size_t)perm[k] * stride + j], acc);
+        dst[b * stride + j] = acc;
+    }
+}
+
+// dst[t, :] += (deg[s] * deg[t]) * h[s, :] over the edges into t, in edge order
+template <int G>
+__global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const float* h, const float* deg,
+                                                             const uint64_t* src_idx, const uint32_t* row_ptr,
+                                                             const uint32_t* perm, size_t n_nodes, size_t stride) {
+    const size_t t = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
+    if (t >= n_nodes) return;
+    const int lane = threadIdx.x % G;
+    const uint32_t s0 = row_ptr[t], s1 = row_ptr[t + 1];
+    if (s0 == s1) return;
+    const float dt = deg[t];
+    for (size_t j = lane; j < stride; j += G) {
+        float acc = dst[t * stride + j];
+        for (uint32_t k = s0; k < s1; k++) {
+            const uint64_t s = src_idx[perm[k]];
+            if (s >= n_nodes) continue;
+            const float w = __fmul_rn(deg[s], dt);
+            acc = __fadd_rn(acc, __fmul_rn(w, h[s * stride + j]));
+        }
+        dst[t * stride + j] = acc;
+    }
+}
+
+// grad_h[s, :] += (go[t, :] * deg[s]) * deg[t] over the edges out of s, in edge order
+template <int G>
+__global__ __launch_bounds__(256) void gcn_bwd_gradh_kernel(float* grad_h, const float* go, const float* deg,
+                                                             const uint64_t* tgt_idx, const uint32_t* row_ptr,
+                                                             const uint32_t* perm, size_t n_nodes, size_t stride) {
+    const size_t s = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
+    if (s >= n_nodes) return;
+    const int lane = threadIdx.x % G;
+    const uint32_t s0 = row_ptr[s], s1 = row_ptr[s + 1];
+    if (s0 == s1) return;
+    const float ds = deg[s];
+    for (size_t j = lane; j < stride; j += G) {
+        float acc = grad_h[s * stride + j];
+        for (uint32_t k = s0; k < s1; k++) {
+            const uint64_t t = tgt_idx[perm[k]];
+            if (t >= n_nodes) continue;
+            acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(go[t * stride + j], ds), deg[t]));
+        }
+        grad_h[s * stride + j] = acc;
+    }
+}
+
+// per-edge degree-gradient terms, each summed over the feature dim in index order (one thread per edge)
+__global__ void gcn_bwd_edge_terms_kernel(const float* go, const float* h, const float* deg, const uint64_t* src_idx,
+                                          const uint64_t* tgt_idx, size_t n_edge, size_t n_nodes, size_t stride,
+                                          float* term_src, float* term_tgt) {
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_edge) return;
+    const uint64_t s = src_idx[e], t = tgt_idx[e];
+    float gs = 0.f, gt = 0.f;
+    if (s < n_nodes && t < n_nodes) {
+        const float ds = deg[s], dt = deg[t];
+        for (size_t j = 0; j < stride; j++) {
+            const float g = go[t * stride + j], hv = h[s * stride + j];
+            gs = __fadd_rn(gs, __fmul_rn(__fmul_rn(g, dt), hv));
+            gt = __fadd_rn(gt, __fmul_rn(__fmul_rn(g, ds), hv));
+        }
+    }
+    term_src[e] = gs;
+    term_tgt[e] = gt;
+}
+
+// grad_deg[v] += terms of the edges touching v, merged in edge order (an edge v->v adds its source term first)
+__global__ void gcn_bwd_graddeg_kernel(float* grad_deg, const float* term_src, const float* term_tgt,
+                                       const uint32_t* rp_src, const uint32_t* perm_src, const uint32_t* rp_tgt,
+                                       const uint32_t* perm_tgt, size_t n_nodes) {
+    size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= n_nodes) return;
+    uint32_t a = rp_src[v], a1 = rp_src[v + 1], b = rp_tgt[v], b1 = rp_tgt[v + 1];
+    if (a == a1 && b == b1) return;
+    float acc = grad_deg[v];
+    while (a < a1 || b < b1) {
+        const uint32_t ea = (a < a1) ? perm_src[a] : 0xffffffffu;
+        const uint32_t eb = (b < b1) ? perm_tgt[b] : 0xffffffffu;
+        if (ea <= eb) {
+            acc = __fadd_rn(acc, term_src[ea]);
+            a++;
+        } else {
+            acc = __fadd_rn(acc, term_tgt[eb]);
+            b++;
+        }
+    }
+    grad_deg[v] = acc;
+}
+
+// src/ndarray.zig:614-624
+struct GatherMeta {
+    uint64_t v[24];  // [idx_strides(8) | src_strides(8) | src_shape(8)]
+};
+__global__ void gather_offsets_kernel(const uint64_t* indices, size_t n, int rank, size_t dim, GatherMeta gm,
+                                      uint64_t* offsets, int* status) {
+    const uint64_t* meta = gm.v;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t rem = i, off = 0;
+    bool bad = false;
+    for (int d = 0; d < rank; d++) {
+        uint64_t c = rem / meta[d];
+        rem = rem % meta[d];
+        if ((size_t)d == dim) {
+            c = indices[i];
+            if (c >= meta[16 + d]) bad = true;
+        }
+        off += c * meta[8 + d];
+    }
+    if (bad) {
+        *status = 2;
+        offsets[i] = 0;
+    } else {
+        offsets[i] = off;
+    }
+}
+
+__global__ void index_select_fwd_kernel(const float* src, size_t src_len, const uint64_t* indices, size_t n_idx,
+                                        size_t stride, float* dst) {
+    size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    const size_t total = n_idx * stride;
+    for (; o < total; o += nt) {
+        const size_t d = o / stride, j = o % stride;
+        const uint64_t r = indices[d];
+        if ((r + 1) * stride <= src_len) dst[o] = src[r * stride + j];
+    }
+}
+
+static int group_for(size_t stride) {
+    if (stride <= 4) return 4;
+    if (stride <= 8) return 8;
+    if (stride <= 16) return 16;
+    if (stride <= 32) return 32;
+    return 64;
+}
+
+#define ZG_G_DISPATCH(g, CALL)                          \
+    switch (g) {                                        \
+        case 4: { constexpr int G = 4; CALL; } break;   \
+        case 8: { constexpr int G = 8; CALL; } break;   \
+        case 16: { constexpr int G = 16; CALL; } break; \
+        case 32: { constexpr int G = 32; CALL; } break; \
+        default: { constexpr int G = 64; CALL; } break; \
+    }
+
+}  // namespace zg
+
+using namespace zg;
+
+ZG_API int zg_hip_gather_offsets(zg_hip_ctx* ctx, const uint64_t* src_shape, const uint64_t* idx_shape, size_t rank,
+                                 const uint64_t* indices, size_t dim, uint64_t* offsets, int* status) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(src_shape && idx_shape && indices && offsets, "gather_offsets: null pointer");
+    ZG_REQUIRE(rank >= 1 && rank <= 8 && dim < rank, "gather_offsets: bad rank %zu / dim %zu", rank, dim);
+    if (status) *status = 0;
+    for (size_t i = 0; i < rank; i++) {
+        if (i != dim && idx_shape[i] > src_shape[i]) {  // src/ndarray.zig:602-604
+            if (status) *status = 1;
+            set_error("gather_offsets: InvalidIndexShape at dim %zu", i);
+            return ZG_HIP_EINVAL;
+        }
+    }
+    GatherMeta gm;
+    uint64_t* meta = gm.v;
+    for (int i = 0; i < 24; i++) meta[i] = 0;
+    uint64_t a = 1, b = 1;
+    for (size_t i = rank; i-- > 0;) {
+        meta[i] = a;
+        a *= idx_shape[i];
+        meta[8 + i] = b;
+        b *= src_shape[i];
+        meta[16 + i] = src_shape[i];
+    }
+    const size_t n = (size_t)a;
+    if (n == 0) return ZG_HIP_OK;
+    int* d_status = (int*)(ctx->scalar_slot + 2);
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(64), 0, ctx->stream, (uint32_t*)d_status, (size_t)1,
+                       (uint32_t*)nullptr, (size_t)0);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gather_offsets_kernel, dim3((unsigned)ceil_div_sz(n, 256)), dim3(256), 0, ctx->stream, indices, n,
+                       (int)rank, dim, gm, offsets, d_status);
+    ZG_LAUNCH_CHECK();
+    if (status) {
+        int h = 0;
+        ZG_HIP_TRY(hipMemcpyAsync(&h, d_status, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+        ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        *status = h;
+        if (h) {
+            set_error("gather_offsets: IndexOutOfBounds");
+            return ZG_HIP_EINVAL;
+        }
+    }
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t* offsets, size_t n, float* dst,
+                              size_t dst_len) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(src && offsets && dst, "scatter_add: null pointer");
+    ZG_REQUIRE(dst_len > 0, "scatter_add: empty destination");
+    ZG_REQUIRE(n < 0xffffffffull && dst_len < 0xffffffffull, "scatter_add: sizes beyond 2^32-1");
+    void* mem = workspace(ctx, plan_bytes(n, dst_len));
+    if (!mem) return ZG_HIP_EOOM;
+    Plan pl = carve_plan(mem, n, dst_len);
+    if (int rc = build_plan(ctx, offsets, pl)) return rc;
+    hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(dst_len, 256)), dim3(256), 0, ctx->stream,
+                       src, pl.row_ptr, pl.perm, dst, dst_len);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src_len, const uint64_t* indices,
+                                   size_t n_idx, size_t stride, float* dst) {
+    ZG_CTX(ctx);
+    if (n_idx == 0 || stride == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(src && indices && dst, "index_select_fwd: null pointer");
+    ZG_REQUIRE(src_len >= stride, "index_select_fwd: source shorter than one row");
+    const size_t total = n_idx * stride;
+    size_t blocks = ceil_div_sz(total, 256);
+    if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
+    hipLaunchKernelGGL(index_select_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, src, src_len, indices,
+                       n_idx, stride, dst);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_index_select_bwd(zg_hip_ctx* ctx, const float* y_grad, const uint64_t* indices, size_t n_idx,
+                                   size_t stride, float* x_grad, size_t x_len) {
+    ZG_CTX(ctx);
+    if (n_idx == 0 || stride == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(y_grad && indices && x_grad, "index_select_bwd: null pointer");
+    ZG_REQUIRE(x_len >= stride, "index_select_bwd: gradient shorter than one row");
+    const size_t nb = x_len / stride;
+    ZG_REQUIRE(n_idx < 0xffffffffull && nb < 0xffffffffull, "index_select_bwd: sizes beyond 2^32-1");
+    void* mem = workspace(ctx, plan_bytes(n_idx, nb));
+    if (!mem) return ZG_HIP_EOOM;
+    Plan pl = carve_plan(mem, n_idx, nb);
+    if (int rc = build_plan(ctx, indices, pl)) return rc;
+    const int g = group_for(stride);
+    const unsigned grid = (unsigned)ceil_div_sz(nb, 256 / g);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((row_scatter_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, y_grad,
+                                        pl.row_ptr, pl.perm, x_grad, nb, stride));
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+static int check_gcn(const char* name, size_t stride, size_t n_edge, size_t n_nodes) {
+    ZG_REQUIRE(stride > 0 && n_nodes > 0, "%s: stride and n_nodes must be positive", name);
+    ZG_REQUIRE(n_edge < 0xffffffffull && n_nodes < 0xffffffffull, "%s: sizes beyond 2^32-1", name);
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,
+                                         const uint64_t* src_indices, const uint64_t* tgt_indices, size_t stride,
+                                         size_t n_edge, size_t n_nodes) {
+    ZG_CTX(ctx);
+    if (n_edge == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(dst && h && deg && src_indices && tgt_indices, "scatter_gcn_deg_scaled: null pointer");
+    if (int rc = check_gcn("scatter_gcn_deg_scaled", stride, n_edge, n_nodes)) return rc;
+    void* mem = workspace(ctx, plan_bytes(n_edge, n_nodes));
+    if (!mem) return ZG_HIP_EOOM;
+    Plan pl = carve_plan(mem, n_edge, n_nodes);
+    if (int rc = build_plan(ctx, tgt_indices, pl)) return rc;
+    const int g = group_for(stride);
+    const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
+                                        src_indices, pl.row_ptr, pl.perm, n_nodes, stride));
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_output, const float* h,
+                                             const float* deg, const uint64_t* src_indices,
+                                             const uint64_t* tgt_indices, float* grad_h, float* grad_deg, size_t stride,
+                                             size_t n_edge, size_t n_nodes) {
+    ZG_CTX(ctx);
+    if (n_edge == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(grad_output && h && deg && src_indices && tgt_indices && grad_h && grad_deg,
+               "scatter_gcn_deg_scaled_bwd: null pointer");
+    if (int rc = check_gcn("scatter_gcn_deg_scaled_bwd", stride, n_edge, n_nodes)) return rc;
+    const size_t pb = align_up(plan_bytes(n_edge, n_nodes), 256);
+    const size_t tb = align_up(n_edge * sizeof(float), 256);
+    char* mem = (char*)workspace(ctx, 2 * pb + 2 * tb);
+    if (!mem) return ZG_HIP_EOOM;
+    Plan by_src = carve_plan(mem, n_edge, n_nodes);
+    Plan by_tgt = carve_plan(mem + pb, n_edge, n_nodes);
+    float* term_src = (float*)(mem + 2 * pb);
+    float* term_tgt = (float*)(mem + 2 * pb + tb);
+    if (int rc = build_plan(ctx, src_indices, by_src)) return rc;
+    if (int rc = build_plan(ctx, tgt_indices, by_tgt)) return rc;
+    const int g = group_for(stride);
+    const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
+                                        grad_output, deg, tgt_indices, by_src.row_ptr, by_src.perm, n_nodes, stride));
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
+                       grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride, term_src, term_tgt);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
+                       grad_deg, term_src, term_tgt, by_src.row_ptr, by_src.perm, by_tgt.row_ptr, by_tgt.perm, n_nodes);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}

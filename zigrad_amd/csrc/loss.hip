@@ -1,0 +1,361 @@
+// Softmax / cross-entropy kernels: the host loops of src/nn/loss.zig:130-257 as device ops.
+//
+// Every kernel streams each logit row once per pass with 128-bit accesses.  The integer-label forward
+// needs a single pass (online max / sum-of-exponentials); the one-hot forward needs two (it must write
+// the probabilities the reference keeps for backward).  Row losses are written to a buffer and summed
+// by a fixed-order reduction, so the loss value does not depend on scheduling.
+#include "reduce.cuh"
+
+namespace zg {
+
+// running (max, sum of exp(x - max))
+struct OnlineAccT {
+    float m, s;
+};
+struct OnlineAcc {
+    using Acc = OnlineAccT;
+    static __device__ __forceinline__ Acc init() { return Acc{-INFINITY, 0.f}; }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b) {
+        float m = fmaxf(a.m, b.m);
+        if (m == -INFINITY) return Acc{m, 0.f};
+        float s = __fadd_rn(__fmul_rn(a.s, expf(__fsub_rn(a.m, m))), __fmul_rn(b.s, expf(__fsub_rn(b.m, m))));
+        return Acc{m, s};
+    }
+    static __device__ __forceinline__ Acc shfl_xor(Acc a, int msk) {
+        return Acc{__shfl_xor(a.m, msk, kWave), __shfl_xor(a.s, msk, kWave)};
+    }
+};
+
+__device__ __forceinline__ void online_push(OnlineAccT& a, float x) {
+    if (x > a.m) {
+        a.s = __fmul_rn(a.s, expf(__fsub_rn(a.m, x)));  // exp(-inf) = 0 on the first element
+        a.m = x;
+    }
+    a.s = __fadd_rn(a.s, expf(__fsub_rn(x, a.m)));
+}
+
+// one pass over a row: per-thread online accumulation, then a group reduction
+template <int TPR>
+__device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, int lane) {
+    OnlineAccT acc = OnlineAcc::init();
+    const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15u) == 0) && (cols % 4 == 0);
+    if (vec) {
+        const float4* x4 = reinterpret_cast<const float4*>(xr);
+        const size_t c4 = cols >> 2;
+        size_t j = lane;
+        for (; j + 3 * TPR < c4; j += 4 * TPR) {
+            float4 v0 = x4[j], v1 = x4[j + TPR], v2 = x4[j + 2 * TPR], v3 = x4[j + 3 * TPR];
+            // one rescale per 16 elements: fold the 16 into the running max first
+            float mx = fmaxf(fmaxf(fmaxf(v0.x, v0.y), fmaxf(v0.z, v0.w)), fmaxf(fmaxf(v1.x, v1.y), fmaxf(v1.z, v1.w)));
+            mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(v2.x, v2.y), fmaxf(v2.z, v2.w)), fmaxf(fmaxf(v3.x, v3.y), fmaxf(v3.z, v3.w))));
+            if (mx > acc.m) {
+                acc.s = __fmul_rn(acc.s, expf(__fsub_rn(acc.m, mx)));
+                acc.m = mx;
+            }
+            float s = 0.f;
+            s += expf(v0.x - acc.m) + expf(v0.y - acc.m) + expf(v0.z - acc.m) + expf(v0.w - acc.m);
+            s += expf(v1.x - acc.m) + expf(v1.y - acc.m) + expf(v1.z - acc.m) + expf(v1.w - acc.m);
+            s += expf(v2.x - acc.m) + expf(v2.y - acc.m) + expf(v2.z - acc.m) + expf(v2.w - acc.m);
+            s += expf(v3.x - acc.m) + expf(v3.y - acc.m) + expf(v3.z - acc.m) + expf(v3.w - acc.m);
+            acc.s += s;
+        }
+        for (; j < c4; j += TPR) {
+            float4 v = x4[j];
+            online_push(acc, v.x);
+            online_push(acc, v.y);
+            online_push(acc, v.z);
+            online_push(acc, v.w);
+        }
+    } else {
+        for (size_t j = lane; j < cols; j += TPR) online_push(acc, xr[j]);
+    }
+    return acc;
+}
+
+template <int TPR>
+__device__ __forceinline__ OnlineAccT row_group_reduce(OnlineAccT acc, OnlineAccT* smem) {
+    if (TPR <= kWave) return group_reduce<OnlineAcc, (TPR <= kWave ? TPR : kWave)>(acc);
+    acc = block_reduce<OnlineAcc>(acc, smem);
+    // broadcast wave 0's result to the whole workgroup
+    __syncthreads();
+    if (threadIdx.x == 0) smem[0] = acc;
+    __syncthreads();
+    return smem[0];
+}
+
+// integer labels: lse[row] and the row's loss term  -log(clamp(p_label, 1e-7, 1 - 1e-7))
+template <int TPR>
+__global__ __launch_bounds__(kBlock) void smce_label_fwd_kernel(const float* logits, const uint64_t* labels,
+                                                                 float* lse, float* row_loss, size_t rows,
+                                                                 size_t cols) {
+    __shared__ OnlineAccT smem[kBlock / kWave];
+    constexpr int kRows = kBlock / TPR;
+    const int lane = threadIdx.x % TPR;
+    const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
+    const bool live = row < rows;
+    OnlineAccT acc = OnlineAcc::init();
+    if (live) acc = row_online<TPR>(logits + row * cols, cols, lane);
+    acc = row_group_reduce<TPR>(acc, smem);
+    if (live && lane == 0) {
+        const float l = __fadd_rn(acc.m, logf(acc.s));
+        lse[row] = l;
+        const uint64_t lab = labels[row];
+        float term = 0.f;
+        if (lab < cols) {
+            float p = expf(__fsub_rn(logits[row * cols + lab], l));
+            float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
+            term = -logf(safe);
+        }
+        row_loss[row] = term;
+    }
+}
+
+// grad (+)= (exp(x - lse[row]) - onehot) / rows, elementwise over the whole matrix
+template <bool ACC>
+__global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* logits, const uint64_t* labels,
+                                                                 const float* lse, float* grad, size_t rows,
+                                                                 size_t cols,
+                                                                 float denom) {
+    // grid: x over float4 columns of one row, y over rows (looped)
+    const bool vec = (((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(grad)) & 15u) == 0) &&
+                     (cols % 4 == 0);
+    for (size_t row = blockIdx.y; row < rows; row += gridDim.y) {
+        const float l = lse[row];
+        const uint64_t lab = labels[row];
+        const float* xr = logits + row * cols;
+        float* gr = grad + row * cols;
+        if (vec) {
+            const size_t c4 = cols >> 2;
+            const float4* x4 = reinterpret_cast<const float4*>(xr);
+            float4* g4 = reinterpret_cast<float4*>(gr);
+            for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < c4; j += (size_t)gridDim.x * kBlock) {
+                float4 v = x4[j];
+                float4 g = ACC ? g4[j] : make_float4(0, 0, 0, 0);
+                const size_t c = 4 * j;
+                float d0 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.x, l)), (c + 0 == lab) ? 1.f : 0.f), denom);
+                float d1 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.y, l)), (c + 1 == lab) ? 1.f : 0.f), denom);
+                float d2 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.z, l)), (c + 2 == lab) ? 1.f : 0.f), denom);
+                float d3 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.w, l)), (c + 3 == lab) ? 1.f : 0.f), denom);
+                g.x = ACC ? __fadd_rn(g.x, d0) : d0;
+                g.y = ACC ? __fadd_rn(g.y, d1) : d1;
+                g.z = ACC ? __fadd_rn(g.z, d2) : d2;
+                g.w = ACC ? __fadd_rn(g.w, d3) : d3;
+                g4[j] = g;
+            }
+        } else {
+            for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += (size_t)gridDim.x * kBlock) {
+                float d = __fdiv_rn(__fsub_rn(expf(__fsub_rn(xr[j], l)), (j == lab) ? 1.f : 0.f), denom);
+                gr[j] = ACC ? __fadd_rn(gr[j], d) : d;
+            }
+        }
+    }
+}
+
+// one-hot targets (the reference's form): probabilities are written out; the row's loss term is
+// sum_j -t_j * log(clamp(p_j)).  MODE 0: softmax only (no target, no loss).
+template <int TPR, int MODE>
+__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* logits, const float* target, float* probs,
+                                                               float* row_loss, size_t rows, size_t cols) {
+    __shared__ OnlineAccT smem[kBlock / kWave];
+    __shared__ float lsum[kBlock / kWave];
+    constexpr int kRows = kBlock / TPR;
+    const int lane = threadIdx.x % TPR;
+    const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
+    const bool live = row < rows;
+    OnlineAccT acc = OnlineAcc::init();
+    if (live) acc = row_online<TPR>(logits + row * cols, cols, lane);
+    acc = row_group_reduce<TPR>(acc, smem);
+    float part = 0.f;
+    if (live) {
+        const float l = __fadd_rn(acc.m, logf(acc.s));
+        const float* xr = logits + row * cols;
+        const float* tr = MODE ? target + row * cols : nullptr;
+        float* pr = probs + row * cols;
+        for (size_t j = lane; j < cols; j += TPR) {
+            float p = expf(__fsub_rn(xr[j], l));
+            pr[j] = p;
+            if (MODE) {
+                float t = tr[j];
+                float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
+                part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
+            }
+        }
+    }
+    if (MODE) {
+        if (TPR <= kWave) {
+            part = group_reduce<SumAcc, (TPR <= kWave ? TPR : kWave)>(part);
+        } else {
+            part = block_reduce<SumAcc>(part, lsum);
+        }
+        if (live && lane == 0) row_loss[row] = part;
+    }
+}
+
+// src/nn/loss.zig:150-159
+__global__ __launch_bounds__(kBlock) void smce_bwd_kernel(const float* probs, const float* target, float* grad, size_t n,
+                                                           float denom) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    const bool vec = ((reinterpret_cast<uintptr_t>(probs) | reinterpret_cast<uintptr_t>(target) |
+                       reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
+    if (vec) {
+        const size_t n4 = n >> 2;
+        const float4* p4 = reinterpret_cast<const float4*>(probs);
+        const float4* t4 = reinterpret_cast<const float4*>(target);
+        float4* g4 = reinterpret_cast<float4*>(grad);
+        for (size_t j = i; j < n4; j += nt) {
+            float4 p = p4[j], t = t4[j], g = g4[j];
+            g.x = __fadd_rn(g.x, __fdiv_rn(__fsub_rn(p.x, t.x), denom));
+            g.y = __fadd_rn(g.y, __fdiv_rn(__fsub_rn(p.y, t.y), denom));
+            g.z = __fadd_rn(g.z, __fdiv_rn(__fsub_rn(p.z, t.z), denom));
+            g.w = __fadd_rn(g.w, __fdiv_rn(__fsub_rn(p.w, t.w), denom));
+            g4[j] = g;
+        }
+        for (size_t j = (n4 << 2) + i; j < n; j += nt)
+            grad[j] = __fadd_rn(grad[j], __fdiv_rn(__fsub_rn(probs[j], target[j]), denom));
+    } else {
+        for (; i < n; i += nt) grad[i] = __fadd_rn(grad[i], __fdiv_rn(__fsub_rn(probs[i], target[i]), denom));
+    }
+}
+
+// src/nn/loss.zig:232-245: x_g += y * (y_g - sum_j y_j * y_g_j) per row
+template <int TPR>
+__global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, const float* y_g, float* x_g, size_t rows,
+                                                              size_t cols) {
+    __shared__ float smem[kBlock / kWave];
+    __shared__ float bcast;
+    constexpr int kRows = kBlock / TPR;
+    const int lane = threadIdx.x % TPR;
+    const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
+    const bool live = row < rows;
+    float part = 0.f;
+    if (live)
+        for (size_t j = lane; j < cols; j += TPR) part = __fadd_rn(part, __fmul_rn(y[row * cols + j], y_g[row * cols + j]));
+    if (TPR <= kWave) {
+        part = group_reduce<SumAcc, (TPR <= kWave ? TPR : kWave)>(part);
+    } else {
+        part = block_reduce<SumAcc>(part, smem);
+        __syncthreads();
+        if (threadIdx.x == 0) bcast = part;
+        __syncthreads();
+        part = bcast;
+    }
+    if (live)
+        for (size_t j = lane; j < cols; j += TPR) {
+            size_t k = row * cols + j;
+            x_g[k] = __fadd_rn(x_g[k], __fmul_rn(y[k], __fsub_rn(y_g[k], part)));
+        }
+}
+
+static int pick_tpr(size_t cols) {
+    if (cols <= 32) return 4;
+    if (cols <= 256) return 16;
+    if (cols <= 4096) return 64;
+    return 256;
+}
+
+#define ZG_TPR_DISPATCH(tpr, CALL) \
+    switch (tpr) {                 \
+        case 4: { constexpr int T = 4; CALL; } break;     \
+        case 16: { constexpr int T = 16; CALL; } break;   \
+        case 64: { constexpr int T = 64; CALL; } break;   \
+        default: { constexpr int T = 256; CALL; } break;  \
+    }
+
+static int check_rows(const char* name, size_t rows, size_t cols) {
+    ZG_REQUIRE(rows > 0 && cols > 0, "%s: empty matrix (%zu x %zu)", name, rows, cols);
+    ZG_REQUIRE(rows <= 0x7fffffffull * 64, "%s: too many rows", name);
+    return ZG_HIP_OK;
+}
+
+}  // namespace zg
+
+using namespace zg;
+
+ZG_API int zg_hip_smce_label_fwd(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, float* lse, float* loss,
+                                 size_t rows, size_t cols) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(logits && labels && lse && loss, "smce_label_fwd: null pointer");
+    if (int rc = check_rows("smce_label_fwd", rows, cols)) return rc;
+    float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
+    if (!row_loss) return ZG_HIP_EOOM;
+    const int tpr = pick_tpr(cols);
+    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
+                                            labels, lse, row_loss, rows, cols));
+    ZG_LAUNCH_CHECK();
+    return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows});
+}
+
+ZG_API int zg_hip_smce_label_bwd(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, const float* lse,
+                                 float* grad, size_t rows, size_t cols, int accumulate) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(logits && labels && lse && grad, "smce_label_bwd: null pointer");
+    if (int rc = check_rows("smce_label_bwd", rows, cols)) return rc;
+    size_t gx = ceil_div_sz((cols + 3) / 4, kBlock);
+    if (gx > 64) gx = 64;
+    size_t gy = ceil_div_sz((size_t)ctx->n_cu * 16, gx);
+    if (gy > rows) gy = rows;
+    if (gy > 65535) gy = 65535;
+    dim3 grid((unsigned)gx, (unsigned)gy);
+    if (accumulate)
+        hipLaunchKernelGGL((smce_label_bwd_kernel<true>), grid, dim3(kBlock), 0, ctx->stream, logits, labels, lse, grad,
+                           rows, cols, (float)rows);
+    else
+        hipLaunchKernelGGL((smce_label_bwd_kernel<false>), grid, dim3(kBlock), 0, ctx->stream, logits, labels, lse,
+                           grad, rows, cols, (float)rows);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* target, float* probs, float* loss,
+                           size_t rows, size_t cols) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(logits && target && probs && loss, "smce_fwd: null pointer");
+    if (int rc = check_rows("smce_fwd", rows, cols)) return rc;
+    float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
+    if (!row_loss) return ZG_HIP_EOOM;
+    const int tpr = pick_tpr(cols);
+    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_rows_kernel<T, 1>), dim3(grid), dim3(kBlock), 0, ctx->stream,
+                                            logits, target, probs, row_loss, rows, cols));
+    ZG_LAUNCH_CHECK();
+    return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows});
+}
+
+ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* target, float* grad, size_t rows,
+                           size_t cols) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(probs && target && grad, "smce_bwd: null pointer");
+    if (int rc = check_rows("smce_bwd", rows, cols)) return rc;
+    const size_t n = rows * cols;
+    size_t blocks = ceil_div_sz(n, (size_t)kBlock * 8);
+    if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
+    hipLaunchKernelGGL(smce_bwd_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad, n,
+                       (float)rows);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t rows, size_t cols) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(x && y, "softmax_fwd: null pointer");
+    if (int rc = check_rows("softmax_fwd", rows, cols)) return rc;
+    const int tpr = pick_tpr(cols);
+    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_rows_kernel<T, 0>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                                            (const float*)nullptr, y, (float*)nullptr, rows, cols));
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_softmax_bwd(zg_hip_ctx* ctx, const float* y, const float* y_g, float* x_g, size_t rows, size_t cols) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(y && y_g && x_g, "softmax_bwd: null pointer");
+    if (int rc = check_rows("softmax_bwd", rows, cols)) return rc;
+    const int tpr = pick_tpr(cols);
+    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, y, y_g,
+                                            x_g, rows, cols));
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}

@@ -1,0 +1,147 @@
+// Fused optimizer updates: src/nn/optim.zig:100-122 (SGD.update) and :177-234 (Adam.update), one op
+// per parameter tensor.  The per-tensor gradient clip never synchronises with the host: a reduction
+// leaves the clip factor in a device slot and the update kernel reads it.
+//
+// HBM traffic per element: SGD reads p,g and writes p (12 B; +4 B when the clip changes g);
+// Adam reads p,g,m,v and writes p,m,v (28 B; +4 B when the clip changes g).
+#include "reduce.cuh"
+
+namespace zg {
+
+template <bool CLIP>
+__global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, size_t n, float nlr, const float* factor) {
+    const float f = CLIP ? factor[0] : 1.0f;
+    const bool scale = CLIP && (f != 1.0f);
+    const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g)) & 15u) == 0;
+    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    if (vec) {
+        float4* p4 = reinterpret_cast<float4*>(p);
+        float4* g4 = reinterpret_cast<float4*>(g);
+        const size_t n4 = n >> 2;
+        for (size_t i = tid; i < n4; i += nt) {
+            float4 pv = p4[i], gv = g4[i];
+            if (scale) {
+                gv.x = __fmul_rn(gv.x, f);
+                gv.y = __fmul_rn(gv.y, f);
+                gv.z = __fmul_rn(gv.z, f);
+                gv.w = __fmul_rn(gv.w, f);
+                g4[i] = gv;
+            }
+            pv.x = __fadd_rn(pv.x, __fmul_rn(nlr, gv.x));
+            pv.y = __fadd_rn(pv.y, __fmul_rn(nlr, gv.y));
+            pv.z = __fadd_rn(pv.z, __fmul_rn(nlr, gv.z));
+            pv.w = __fadd_rn(pv.w, __fmul_rn(nlr, gv.w));
+            p4[i] = pv;
+        }
+        tid += n4 << 2;
+    }
+    for (size_t i = vec ? tid : tid; i < n; i += nt) {
+        float gv = g[i];
+        if (scale) {
+            gv = __fmul_rn(gv, f);
+            g[i] = gv;
+        }
+        p[i] = __fadd_rn(p[i], __fmul_rn(nlr, gv));
+    }
+}
+
+__device__ __forceinline__ void adam_elem(float& p, float& g, float& m, float& v, bool scale, float f, float lr_t,
+                                          float b1, float b2, float omb1, float omb2, float eps) {
+    if (scale) g = __fmul_rn(g, f);
+    // src/nn/optim.zig:226-229, evaluated left to right in fp32
+    m = __fadd_rn(__fmul_rn(b1, m), __fmul_rn(omb1, g));
+    v = __fadd_rn(__fmul_rn(b2, v), __fmul_rn(__fmul_rn(omb2, g), g));
+    p = __fsub_rn(p, __fdiv_rn(__fmul_rn(lr_t, m), __fadd_rn(__fsqrt_rn(v), eps)));
+}
+
+template <bool CLIP>
+__global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float* m, float* v, size_t n, float lr_t,
+                                                       float b1, float b2, float omb1, float omb2, float eps,
+                                                       const float* factor) {
+    const float f = CLIP ? factor[0] : 1.0f;
+    const bool scale = CLIP && (f != 1.0f);
+    const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
+                       reinterpret_cast<uintptr_t>(v)) & 15u) == 0;
+    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    if (vec) {
+        float4* p4 = reinterpret_cast<float4*>(p);
+        float4* g4 = reinterpret_cast<float4*>(g);
+        float4* m4 = reinterpret_cast<float4*>(m);
+        float4* v4 = reinterpret_cast<float4*>(v);
+        const size_t n4 = n >> 2;
+        for (size_t i = tid; i < n4; i += nt) {
+            float4 pv = p4[i], gv = g4[i], mv = m4[i], vv = v4[i];
+            adam_elem(pv.x, gv.x, mv.x, vv.x, scale, f, lr_t, b1, b2, omb1, omb2, eps);
+            adam_elem(pv.y, gv.y, mv.y, vv.y, scale, f, lr_t, b1, b2, omb1, omb2, eps);
+            adam_elem(pv.z, gv.z, mv.z, vv.z, scale, f, lr_t, b1, b2, omb1, omb2, eps);
+            adam_elem(pv.w, gv.w, mv.w, vv.w, scale, f, lr_t, b1, b2, omb1, omb2, eps);
+            if (scale) g4[i] = gv;
+            m4[i] = mv;
+            v4[i] = vv;
+            p4[i] = pv;
+        }
+        tid += n4 << 2;
+    }
+    for (size_t i = tid; i < n; i += nt) {
+        float pv = p[i], gv = g[i], mv = m[i], vv = v[i];
+        adam_elem(pv, gv, mv, vv, scale, f, lr_t, b1, b2, omb1, omb2, eps);
+        if (scale) g[i] = gv;
+        m[i] = mv;
+        v[i] = vv;
+        p[i] = pv;
+    }
+}
+
+static int update_grid(zg_hip_ctx* ctx, size_t n) {
+    size_t blocks = ceil_div_sz(n, (size_t)kBlock * 4);
+    size_t cap = (size_t)ctx->n_cu * 16;
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+}  // namespace zg
+
+using namespace zg;
+
+ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n, float lr, int clip, float max_norm,
+                           float delta) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(param && grad, "sgd_step: null pointer");
+    float* factor = ctx->scalar_slot + 1;
+    if (clip) {
+        int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
+        if (rc) return rc;
+        hipLaunchKernelGGL((sgd_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, n,
+                           -lr, factor);
+    } else {
+        hipLaunchKernelGGL((sgd_kernel<false>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad,
+                           n, -lr, factor);
+    }
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_adam_step(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n, uint64_t t,
+                            float lr, float beta1, float beta2, float epsilon, int clip, float max_norm, float delta) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(param && grad && m && v, "adam_step: null pointer");
+    ZG_REQUIRE(t >= 1, "adam_step: t must be >= 1");
+    // src/nn/optim.zig:190-191, fp32 throughout
+    const float tf = (float)t;
+    const float lr_t = lr * sqrtf(1.0f - powf(beta2, tf)) / (1.0f - powf(beta1, tf));
+    const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2;
+    float* factor = ctx->scalar_slot + 1;
+    if (clip) {
+        int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
+        if (rc) return rc;
+        hipLaunchKernelGGL((adam_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, m,
+                           v, n, lr_t, beta1, beta2, omb1, omb2, epsilon, factor);
+    } else {
+        hipLaunchKernelGGL((adam_kernel<false>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad,
+                           m, v, n, lr_t, beta1, beta2, omb1, omb2, epsilon, factor);
+    }
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}

@@ -1,0 +1,304 @@
+// Wavefront / workgroup reduction building blocks shared by the reduction, loss and optimizer kernels.
+#pragma once
+#include "common.h"
+
+namespace zg {
+
+// ---- accumulator policies -------------------------------------------------------------------
+// combine(a, b) must give the same result for (a, b) and (b, a): the butterfly shuffles below apply
+// it with the operands in either order on the two lanes of a pair.
+
+struct SumAcc {
+    using Acc = float;
+    static __device__ __forceinline__ Acc init() { return 0.f; }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return __fadd_rn(a, b); }
+    static __device__ __forceinline__ Acc shfl_xor(Acc a, int m) { return __shfl_xor(a, m, kWave); }
+};
+
+// strict '>' running max from -inf (src/device/host_device.zig:862-873); NaNs never win
+struct MaxAcc {
+    using Acc = float;
+    static __device__ __forceinline__ Acc init() { return -INFINITY; }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return (b > a) ? b : a; }
+    static __device__ __forceinline__ Acc shfl_xor(Acc a, int m) { return __shfl_xor(a, m, kWave); }
+};
+
+// value + position; larger value wins, equal values keep the smaller position (first occurrence)
+struct ArgAccT {
+    float v;
+    uint32_t i;
+};
+struct ArgmaxAcc {
+    using Acc = ArgAccT;
+    static __device__ __forceinline__ Acc init() { return Acc{-INFINITY, 0xffffffffu}; }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b) {
+        bool take_b = (b.v > a.v) || (b.v == a.v && b.i < a.i);
+        return take_b ? b : a;
+    }
+    static __device__ __forceinline__ Acc shfl_xor(Acc a, int m) {
+        Acc r;
+        r.v = __shfl_xor(a.v, m, kWave);
+        r.i = (uint32_t)__shfl_xor((int)a.i, m, kWave);
+        return r;
+    }
+};
+
+// |value| + position + signed value: the element cblas_isamax picks (first index of the largest |x|)
+struct AbsArgAccT {
+    float a;
+    uint32_t i;
+    float v;
+};
+struct AbsArgmaxAcc {
+    using Acc = AbsArgAccT;
+    static __device__ __forceinline__ Acc init() { return Acc{-1.0f, 0xffffffffu, 0.f}; }
+    static __device__ __forceinline__ Acc combine(Acc x, Acc y) {
+        bool take_y = (y.a > x.a) || (y.a == x.a && y.i < x.i);
+        return take_y ? y : x;
+    }
+    static __device__ __forceinline__ Acc shfl_xor(Acc x, int m) {
+        Acc r;
+        r.a = __shfl_xor(x.a, m, kWave);
+        r.i = (uint32_t)__shfl_xor((int)x.i, m, kWave);
+        r.v = __shfl_xor(x.v, m, kWave);
+        return r;
+    }
+};
+
+// two running sums (used by the online softmax: see loss.hip) are handled there.
+
+// ---- wave and block reductions ---------------------------------------------------------------
+template <class P, int WIDTH = kWave>
+__device__ __forceinline__ typename P::Acc group_reduce(typename P::Acc v) {
+#pragma unroll
+    for (int m = WIDTH / 2; m >= 1; m >>= 1) v = P::combine(v, P::shfl_xor(v, m));
+    return v;
+}
+
+// Result valid in every thread of wave 0 (in particular thread 0). `smem` holds >= blockDim.x/64 entries.
+// All threads of the block must call it.
+template <class P>
+__device__ __forceinline__ typename P::Acc block_reduce(typename P::Acc v, typename P::Acc* smem) {
+    v = group_reduce<P>(v);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int nw = (blockDim.x + kWave - 1) / kWave;
+    __syncthreads();  // smem may still be read from a previous call
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    if (wave == 0) {
+        v = (lane < nw) ? smem[lane] : P::init();
+        v = group_reduce<P>(v);
+    }
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// flat reductions
+// ------------------------------------------------------------------------------------------------
+struct TermId {
+    using P = SumAcc;
+    static __device__ __forceinline__ float term(float a, float, size_t, float) { return a; }
+};
+struct TermAbs {
+    using P = SumAcc;
+    static __device__ __forceinline__ float term(float a, float, size_t, float) { return fabsf(a); }
+};
+struct TermSq {
+    using P = SumAcc;
+    static __device__ __forceinline__ float term(float a, float, size_t, float) { return __fmul_rn(a, a); }
+};
+struct TermDot {
+    using P = SumAcc;
+    static __device__ __forceinline__ float term(float a, float b, size_t, float) { return __fmul_rn(a, b); }
+};
+// src/nn/loss.zig:266-274
+struct TermSmoothL1 {
+    using P = SumAcc;
+    static __device__ __forceinline__ float term(float a, float b, size_t, float beta) {
+        float d = __fsub_rn(a, b), ad = fabsf(d);
+        if (ad < beta) return __fdiv_rn(__fmul_rn(0.5f, __fmul_rn(d, d)), beta);
+        return __fsub_rn(ad, __fmul_rn(0.5f, beta));
+    }
+};
+// src/nn/loss.zig:99-102
+struct TermSqDiff {
+    using P = SumAcc;
+    static __device__ __forceinline__ float term(float a, float b, size_t, float) {
+        float d = __fsub_rn(a, b);
+        return __fmul_rn(d, d);
+    }
+};
+struct TermAbsArg {
+    using P = AbsArgmaxAcc;
+    static __device__ __forceinline__ AbsArgAccT term(float a, float, size_t i, float) {
+        return AbsArgAccT{fabsf(a), (uint32_t)i, a};
+    }
+};
+
+struct FinStore {
+    float* y;
+    __device__ void operator()(float s) const { y[0] = s; }
+};
+struct FinAxpby {  // src/device/reduce.zig:45
+    float* y;
+    float alpha, beta;
+    __device__ void operator()(float s) const {
+        float r = __fmul_rn(alpha, s);
+        y[0] = (beta == 0.f) ? r : __fadd_rn(r, __fmul_rn(beta, y[0]));
+    }
+};
+struct FinSqrt {
+    float* y;
+    __device__ void operator()(float s) const { y[0] = __fsqrt_rn(s); }
+};
+struct FinDivN {
+    float* y;
+    float n;
+    __device__ void operator()(float s) const { y[0] = __fdiv_rn(s, n); }
+};
+// src/device/host_device.zig:339-346: the factor clip_nrm2 multiplies by, 1 when no clipping happens
+struct FinClipFactor {
+    float* factor;
+    float max_norm, delta;
+    __device__ void operator()(float s) const {
+        float norm = __fsqrt_rn(s);
+        factor[0] = (norm > max_norm) ? __fdiv_rn(max_norm, __fadd_rn(norm, delta)) : 1.0f;
+    }
+};
+struct FinAbsArg {
+    float* y;
+    __device__ void operator()(AbsArgAccT a) const { y[0] = a.v; }
+};
+
+constexpr int kFlatBlock = 256;
+constexpr int kFlatSingle = 1024;       // block size of the single-workgroup path
+constexpr size_t kFlatSingleMax = 65536;  // up to this many elements one workgroup does everything
+constexpr int kMaxPartials = 2048;
+
+template <class T, int NIN>
+__device__ __forceinline__ typename T::P::Acc flat_accumulate(const float* a, const float* b, size_t n, float p0,
+                                                               size_t tid, size_t nthreads) {
+    using P = typename T::P;
+    typename P::Acc acc = P::init();
+    const bool vec = ((reinterpret_cast<uintptr_t>(a) | (NIN > 1 ? reinterpret_cast<uintptr_t>(b) : 0)) & 15u) == 0;
+    if (vec) {
+        const size_t n4 = n >> 2;
+        const float4* a4 = reinterpret_cast<const float4*>(a);
+        const float4* b4 = reinterpret_cast<const float4*>(b);
+        size_t i = tid;
+        // two independent loads in flight per trip
+        for (; i + nthreads < n4; i += 2 * nthreads) {
+            float4 u0 = a4[i], u1 = a4[i + nthreads];
+            float4 w0 = make_float4(0, 0, 0, 0), w1 = w0;
+            if (NIN > 1) {
+                w0 = b4[i];
+                w1 = b4[i + nthreads];
+            }
+            acc = P::combine(acc, T::term(u0.x, w0.x, 4 * i + 0, p0));
+            acc = P::combine(acc, T::term(u0.y, w0.y, 4 * i + 1, p0));
+            acc = P::combine(acc, T::term(u0.z, w0.z, 4 * i + 2, p0));
+            acc = P::combine(acc, T::term(u0.w, w0.w, 4 * i + 3, p0));
+            const size_t j = i + nthreads;
+            acc = P::combine(acc, T::term(u1.x, w1.x, 4 * j + 0, p0));
+            acc = P::combine(acc, T::term(u1.y, w1.y, 4 * j + 1, p0));
+            acc = P::combine(acc, T::term(u1.z, w1.z, 4 * j + 2, p0));
+            acc = P::combine(acc, T::term(u1.w, w1.w, 4 * j + 3, p0));
+        }
+        for (; i < n4; i += nthreads) {
+            float4 u0 = a4[i];
+            float4 w0 = make_float4(0, 0, 0, 0);
+            if (NIN > 1) w0 = b4[i];
+            acc = P::combine(acc, T::term(u0.x, w0.x, 4 * i + 0, p0));
+            acc = P::combine(acc, T::term(u0.y, w0.y, 4 * i + 1, p0));
+            acc = P::combine(acc, T::term(u0.z, w0.z, 4 * i + 2, p0));
+            acc = P::combine(acc, T::term(u0.w, w0.w, 4 * i + 3, p0));
+        }
+        for (size_t t = (n4 << 2) + tid; t < n; t += nthreads)
+            acc = P::combine(acc, T::term(a[t], NIN > 1 ? b[t] : 0.f, t, p0));
+    } else {
+        for (size_t i = tid; i < n; i += nthreads) acc = P::combine(acc, T::term(a[i], NIN > 1 ? b[i] : 0.f, i, p0));
+    }
+    return acc;
+}
+
+// one workgroup reduces everything and finalises
+template <class T, int NIN, class Fin>
+__global__ __launch_bounds__(kFlatSingle) void flat_single_kernel(const float* a, const float* b, size_t n, float p0,
+                                                                  Fin fin) {
+    using P = typename T::P;
+    __shared__ typename P::Acc smem[kFlatSingle / kWave];
+    typename P::Acc acc = flat_accumulate<T, NIN>(a, b, n, p0, threadIdx.x, blockDim.x);
+    acc = block_reduce<P>(acc, smem);
+    if (threadIdx.x == 0) fin(acc);
+}
+
+template <class T, int NIN>
+__global__ __launch_bounds__(kFlatBlock) void flat_partial_kernel(const float* a, const float* b, size_t n, float p0,
+                                                                   typename T::P::Acc* partials) {
+    using P = typename T::P;
+    __shared__ typename P::Acc smem[kFlatBlock / kWave];
+    typename P::Acc acc = flat_accumulate<T, NIN>(a, b, n, p0, (size_t)blockIdx.x * kFlatBlock + threadIdx.x,
+                                                  (size_t)gridDim.x * kFlatBlock);
+    acc = block_reduce<P>(acc, smem);
+    if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+}
+
+template <class P, class Fin>
+__global__ __launch_bounds__(kFlatBlock) void flat_final_kernel(const typename P::Acc* partials, int n_partials,
+                                                                 Fin fin) {
+    __shared__ typename P::Acc smem[kFlatBlock / kWave];
+    typename P::Acc acc = P::init();
+    for (int i = threadIdx.x; i < n_partials; i += kFlatBlock) acc = P::combine(acc, partials[i]);
+    acc = block_reduce<P>(acc, smem);
+    if (threadIdx.x == 0) fin(acc);
+}
+
+template <class T, int NIN, class Fin>
+static int flat_reduce(zg_hip_ctx* ctx, const float* a, const float* b, size_t n, float p0, Fin fin) {
+    using P = typename T::P;
+    if (n <= kFlatSingleMax) {
+        hipLaunchKernelGGL((flat_single_kernel<T, NIN, Fin>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, a, b, n, p0,
+                           fin);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    size_t blocks = ceil_div_sz(n, (size_t)kFlatBlock * 16);
+    size_t cap = (size_t)ctx->n_cu * 8;
+    if (cap > (size_t)kMaxPartials) cap = kMaxPartials;
+    if (blocks > cap) blocks = cap;
+    static_assert(kMaxPartials * sizeof(typename P::Acc) <= (64 << 10), "partials buffer too small");
+    auto* partials = (typename P::Acc*)ctx->partials;
+    hipLaunchKernelGGL((flat_partial_kernel<T, NIN>), dim3((unsigned)blocks), dim3(kFlatBlock), 0, ctx->stream, a, b, n,
+                       p0, partials);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL((flat_final_kernel<P, Fin>), dim3(1), dim3(kFlatBlock), 0, ctx->stream, partials, (int)blocks,
+                       fin);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// x *= factor[0], skipped entirely when the factor is exactly 1
+static __global__ __launch_bounds__(kBlock) void scale_by_device_factor_kernel(float* x, size_t n, const float* factor) {
+    const float f = factor[0];
+    if (f == 1.0f) return;
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    if (vec) {
+        float4* x4 = reinterpret_cast<float4*>(x);
+        const size_t n4 = n >> 2;
+        for (size_t i = tid; i < n4; i += nt) {
+            float4 v = x4[i];
+            v.x = __fmul_rn(v.x, f);
+            v.y = __fmul_rn(v.y, f);
+            v.z = __fmul_rn(v.z, f);
+            v.w = __fmul_rn(v.w, f);
+            x4[i] = v;
+        }
+        for (size_t t = (n4 << 2) + tid; t < n; t += nt) x[t] = __fmul_rn(x[t], f);
+    } else {
+        for (size_t i = tid; i < n; i += nt) x[i] = __fmul_rn(x[i], f);
+    }
+}
+
+
+}  // namespace zg

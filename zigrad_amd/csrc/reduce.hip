@@ -1,0 +1,525 @@
+// Reductions: flat (sum|x|, sum, nrm2, dot, isamax-style max, clip), along an axis (sum / max /
+// argmax over the last, the first or a middle axis), and unbroadcast.
+//
+// All of them are HBM-bound single passes.  Flat and column reductions with many rows are two
+// launches (per-block partials, then one block that combines the partials in a fixed order); there is
+// no cross-workgroup communication inside a kernel and no floating-point atomics, so results do not
+// depend on scheduling.
+#include "reduce.cuh"
+
+namespace zg {
+
+// max_bwd: x_g[i] += y_g[0] where x[i] == y[0]   (src/device/host_device.zig:582-588)
+__global__ __launch_bounds__(kBlock) void max_bwd_kernel(const float* x, float* x_g, size_t n, const float* y,
+                                                          const float* y_g) {
+    const float val = y[0], grd = y_g[0];
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    for (; i < n; i += nt)
+        if (val == x[i]) x_g[i] = __fadd_rn(x_g[i], grd);
+}
+
+// y += alpha[0] * x with alpha in device memory (src/device/host_device.zig:269-275)
+__global__ __launch_bounds__(kBlock) void axpy_kernel(const float* x, float* y, size_t n, const float* alpha_ptr) {
+    const float al = alpha_ptr[0];
+    const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    if (vec) {
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+        float4* y4 = reinterpret_cast<float4*>(y);
+        const size_t n4 = n >> 2;
+        for (size_t i = tid; i < n4; i += nt) {
+            float4 u = x4[i], v = y4[i];
+            v.x = __fadd_rn(v.x, __fmul_rn(al, u.x));
+            v.y = __fadd_rn(v.y, __fmul_rn(al, u.y));
+            v.z = __fadd_rn(v.z, __fmul_rn(al, u.z));
+            v.w = __fadd_rn(v.w, __fmul_rn(al, u.w));
+            y4[i] = v;
+        }
+        for (size_t t = (n4 << 2) + tid; t < n; t += nt) y[t] = __fadd_rn(y[t], __fmul_rn(al, x[t]));
+    } else {
+        for (size_t i = tid; i < n; i += nt) y[i] = __fadd_rn(y[i], __fmul_rn(al, x[i]));
+    }
+}
+
+static int stream_grid(zg_hip_ctx* ctx, size_t n, size_t per_thread) {
+    size_t blocks = ceil_div_sz(n, (size_t)kBlock * per_thread);
+    size_t cap = (size_t)ctx->n_cu * 16;
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// ------------------------------------------------------------------------------------------------
+// reductions along an axis.  x is viewed as [outer, R, inner]; R is reduced.
+// ------------------------------------------------------------------------------------------------
+struct AxisSum {
+    using P = SumAcc;
+    using Out = float;
+    static __device__ __forceinline__ float term(float v, uint32_t) { return v; }
+    static __device__ __forceinline__ void store(Out* y, size_t o, float s, float alpha, float beta) {
+        float r = __fmul_rn(alpha, s);
+        y[o] = (beta == 0.f) ? r : __fadd_rn(r, __fmul_rn(beta, y[o]));
+    }
+};
+struct AxisMax {
+    using P = MaxAcc;
+    using Out = float;
+    static __device__ __forceinline__ float term(float v, uint32_t) { return v; }
+    static __device__ __forceinline__ void store(Out* y, size_t o, float s, float, float) { y[o] = s; }
+};
+struct AxisArgmax {
+    using P = ArgmaxAcc;
+    using Out = uint64_t;
+    static __device__ __forceinline__ ArgAccT term(float v, uint32_t r) { return ArgAccT{v, r}; }
+    // an all -inf / NaN slice keeps the sentinel; the host loop would answer 0 there
+    static __device__ __forceinline__ void store(Out* y, size_t o, ArgAccT s, float, float) {
+        y[o] = (s.i == 0xffffffffu) ? 0 : (uint64_t)s.i;
+    }
+};
+
+// inner == 1: rows of `cols` contiguous elements, TPR threads per row, 256/TPR rows per workgroup
+template <class A, int TPR>
+__global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, typename A::Out* y, size_t rows, size_t cols,
+                                                             float alpha, float beta) {
+    using P = typename A::P;
+    constexpr int kRows = kBlock / TPR;
+    const int lane = threadIdx.x % TPR;
+    const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
+    typename P::Acc acc = P::init();
+    if (row < rows) {
+        const float* xr = x + row * cols;
+        const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15u) == 0) && (cols % 4 == 0);
+        if (vec) {
+            const float4* x4 = reinterpret_cast<const float4*>(xr);
+            const size_t c4 = cols >> 2;
+            size_t j = lane;
+            for (; j + 3 * TPR < c4; j += 4 * TPR) {
+                float4 v0 = x4[j], v1 = x4[j + TPR], v2 = x4[j + 2 * TPR], v3 = x4[j + 3 * TPR];
+                const float4 vs[4] = {v0, v1, v2, v3};
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    uint32_t c = (uint32_t)(4 * (j + (size_t)u * TPR));
+                    acc = P::combine(acc, A::term(vs[u].x, c + 0));
+                    acc = P::combine(acc, A::term(vs[u].y, c + 1));
+                    acc = P::combine(acc, A::term(vs[u].z, c + 2));
+                    acc = P::combine(acc, A::term(vs[u].w, c + 3));
+                }
+            }
+            for (; j < c4; j += TPR) {
+                float4 v = x4[j];
+                uint32_t c = (uint32_t)(4 * j);
+                acc = P::combine(acc, A::term(v.x, c + 0));
+                acc = P::combine(acc, A::term(v.y, c + 1));
+                acc = P::combine(acc, A::term(v.z, c + 2));
+                acc = P::combine(acc, A::term(v.w, c + 3));
+            }
+        } else {
+            for (size_t j = lane; j < cols; j += TPR) acc = P::combine(acc, A::term(xr[j], (uint32_t)j));
+        }
+    }
+    if (TPR <= kWave) {
+        acc = group_reduce<P, (TPR <= kWave ? TPR : kWave)>(acc);
+    } else {
+        __shared__ typename P::Acc smem[kBlock / kWave];
+        acc = block_reduce<P>(acc, smem);
+    }
+    if (lane == 0 && row < rows) A::store(y, row, acc, alpha, beta);
+}
+
+// inner > 1: column-style.  Workgroup = cx column-threads x ry row-threads (cx*ry = 256), each thread owns V
+// adjacent columns and walks rows ty, ty+ry, ... of its row chunk.  grid = (column groups, row chunks, outer).
+// With one row chunk the result is stored directly; otherwise per-chunk partials go to `partials`
+// laid out [outer, chunks, inner] and col_final_kernel combines them in chunk order.
+template <class A, int V>
+__global__ __launch_bounds__(kBlock) void col_reduce_kernel(const float* x, typename A::Out* y,
+                                                             typename A::P::Acc* partials, size_t R, size_t inner,
+                                                             int log2_cx, size_t rows_per_chunk, float alpha,
+                                                             float beta) {
+    using P = typename A::P;
+    using Acc = typename P::Acc;
+    __shared__ Acc smem[kBlock * V];
+    const int cx = 1 << log2_cx, ry = kBlock >> log2_cx;
+    const int tx = threadIdx.x & (cx - 1), ty = threadIdx.x >> log2_cx;
+    const size_t colv = (size_t)blockIdx.x * cx + tx;  // in units of V columns
+    const size_t col0 = colv * V;
+    const size_t outer = blockIdx.z;
+    const size_t r_begin = (size_t)blockIdx.y * rows_per_chunk;
+    size_t r_end = r_begin + rows_per_chunk;
+    if (r_end > R) r_end = R;
+    Acc acc[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) acc[v] = P::init();
+    const bool active = col0 < inner;
+    if (active) {
+        const float* xb = x + outer * R * inner + col0;
+        size_t r = r_begin + ty;
+        if constexpr (V == 4) {
+            for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
+                float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
+                float4 v1 = *reinterpret_cast<const float4*>(xb + (r + ry) * inner);
+                float4 v2 = *reinterpret_cast<const float4*>(xb + (r + 2 * (size_t)ry) * inner);
+                float4 v3 = *reinterpret_cast<const float4*>(xb + (r + 3 * (size_t)ry) * inner);
+                const float4 vs[4] = {v0, v1, v2, v3};
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    uint32_t rr = (uint32_t)(r + (size_t)u * ry);
+                    acc[0] = P::combine(acc[0], A::term(vs[u].x, rr));
+                    acc[1 % V] = P::combine(acc[1 % V], A::term(vs[u].y, rr));
+                    acc[2 % V] = P::combine(acc[2 % V], A::term(vs[u].z, rr));
+                    acc[3 % V] = P::combine(acc[3 % V], A::term(vs[u].w, rr));
+                }
+            }
+            for (; r < r_end; r += ry) {
+                float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
+                uint32_t rr = (uint32_t)r;
+                acc[0] = P::combine(acc[0], A::term(v0.x, rr));
+                acc[1 % V] = P::combine(acc[1 % V], A::term(v0.y, rr));
+                acc[2 % V] = P::combine(acc[2 % V], A::term(v0.z, rr));
+                acc[3 % V] = P::combine(acc[3 % V], A::term(v0.w, rr));
+            }
+        } else {
+            for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
+                float v0 = xb[r * inner], v1 = xb[(r + ry) * inner], v2 = xb[(r + 2 * (size_t)ry) * inner],
+                      v3 = xb[(r + 3 * (size_t)ry) * inner];
+                acc[0] = P::combine(acc[0], A::term(v0, (uint32_t)r));
+                acc[0] = P::combine(acc[0], A::term(v1, (uint32_t)(r + ry)));
+                acc[0] = P::combine(acc[0], A::term(v2, (uint32_t)(r + 2 * (size_t)ry)));
+                acc[0] = P::combine(acc[0], A::term(v3, (uint32_t)(r + 3 * (size_t)ry)));
+            }
+            for (; r < r_end; r += ry) acc[0] = P::combine(acc[0], A::term(xb[r * inner], (uint32_t)r));
+        }
+    }
+    // combine the ry row-threads of each column in ty order
+#pragma unroll
+    for (int v = 0; v < V; v++) smem[threadIdx.x * V + v] = acc[v];
+    __syncthreads();
+    if (ty == 0 && active) {
+        for (int t = 1; t < ry; t++) {
+#pragma unroll
+            for (int v = 0; v < V; v++) acc[v] = P::combine(acc[v], smem[((t << log2_cx) + tx) * V + v]);
+        }
+#pragma unroll
+        for (int v = 0; v < V; v++) {
+            size_t c = col0 + v;
+            if (c < inner) {
+                if (gridDim.y == 1)
+                    A::store(y, outer * inner + c, acc[v], alpha, beta);
+                else
+                    partials[(outer * gridDim.y + blockIdx.y) * inner + c] = acc[v];
+            }
+        }
+    }
+}
+
+template <class A>
+__global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::Acc* partials, typename A::Out* y,
+                                                            size_t n_out, size_t inner, int chunks, float alpha,
+                                                            float beta) {
+    using P = typename A::P;
+    size_t o = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (o >= n_out) return;
+    const size_t outer = o / inner, c = o % inner;
+    typename P::Acc acc = partials[(outer * chunks) * inner + c];
+    for (int k = 1; k < chunks; k++) acc = P::combine(acc, partials[(outer * chunks + k) * inner + c]);
+    A::store(y, o, acc, alpha, beta);
+}
+
+template <class A>
+static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size_t outer, size_t R, size_t inner,
+                       float alpha, float beta) {
+    using Acc = typename A::P::Acc;
+    if (outer == 0 || R == 0 || inner == 0) return ZG_HIP_OK;
+    if (inner == 1) {
+        const size_t rows = outer, cols = R;
+#define ZG_ROW(TPR)                                                                                          \
+    hipLaunchKernelGGL((row_reduce_kernel<A, TPR>), dim3((unsigned)ceil_div_sz(rows, kBlock / TPR)), dim3(kBlock), 0, \
+                       ctx->stream, x, y, rows, cols, alpha, beta)
+        if (cols <= 32) ZG_ROW(4);
+        else if (cols <= 256) ZG_ROW(16);
+        else if (cols <= 16384 || rows >= (size_t)ctx->n_cu * 8) ZG_ROW(64);
+        else ZG_ROW(256);
+#undef ZG_ROW
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    const bool v4 = (inner % 4 == 0) && aligned16(x);
+    const int V = v4 ? 4 : 1;
+    const size_t colv = inner / V;
+    int log2_cx = 0;
+    while ((1u << log2_cx) < colv && log2_cx < 8) log2_cx++;
+    const int cx = 1 << log2_cx, ry = kBlock >> log2_cx;
+    const size_t gx = ceil_div_sz(colv, cx);
+    // row chunks: enough workgroups to cover the machine several times, but at least 4 trips of ry rows each
+    size_t want = (size_t)ctx->n_cu * 8;
+    size_t chunks = ceil_div_sz(want, gx * outer);
+    size_t max_chunks = ceil_div_sz(R, (size_t)ry * 4);
+    if (chunks > max_chunks) chunks = max_chunks;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 1024) chunks = 1024;
+    const size_t rows_per_chunk = ceil_div_sz(R, chunks);
+    chunks = ceil_div_sz(R, rows_per_chunk);
+    ZG_REQUIRE(outer <= 65535, "axis reduction: %zu leading slices exceed the grid limit", outer);
+    Acc* partials = nullptr;
+    if (chunks > 1) {
+        partials = (Acc*)workspace(ctx, outer * chunks * inner * sizeof(Acc));
+        if (!partials) return ZG_HIP_EOOM;
+    }
+    dim3 grid((unsigned)gx, (unsigned)chunks, (unsigned)outer);
+    if (v4)
+        hipLaunchKernelGGL((col_reduce_kernel<A, 4>), grid, dim3(kBlock), 0, ctx->stream, x, y, partials, R, inner,
+                           log2_cx, rows_per_chunk, alpha, beta);
+    else
+        hipLaunchKernelGGL((col_reduce_kernel<A, 1>), grid, dim3(kBlock), 0, ctx->stream, x, y, partials, R, inner,
+                           log2_cx, rows_per_chunk, alpha, beta);
+    ZG_LAUNCH_CHECK();
+    if (chunks > 1) {
+        const size_t n_out = outer * inner;
+        hipLaunchKernelGGL((col_final_kernel<A>), dim3((unsigned)ceil_div_sz(n_out, kBlock)), dim3(kBlock), 0,
+                           ctx->stream, partials, y, n_out, inner, (int)chunks, alpha, beta);
+        ZG_LAUNCH_CHECK();
+    }
+    return ZG_HIP_OK;
+}
+
+static size_t prod(const uint64_t* s, size_t from, size_t to) {
+    size_t n = 1;
+    for (size_t i = from; i < to; i++) n *= (size_t)s[i];
+    return n;
+}
+
+static int check_axis_args(const char* name, const void* x, const uint64_t* x_shape, size_t x_rank, const void* y,
+                           size_t y_len, size_t dim) {
+    ZG_REQUIRE(x && y && x_shape, "%s: null pointer", name);
+    ZG_REQUIRE(x_rank >= 1 && x_rank <= 8, "%s: rank %zu not in 1..8", name, x_rank);
+    ZG_REQUIRE(dim < x_rank, "%s: dim %zu out of range for rank %zu", name, dim, x_rank);
+    for (size_t i = 0; i < x_rank; i++) ZG_REQUIRE(x_shape[i] > 0, "%s: zero-sized dim %zu", name, i);
+    const size_t total = prod(x_shape, 0, x_rank);
+    ZG_REQUIRE(x_shape[dim] < 0xffffffffull, "%s: reduced dim too large", name);
+    ZG_REQUIRE(y_len == total / x_shape[dim] || y_len == 1, "%s: y.len %zu does not match the reduced shape (%zu)", name,
+               y_len, total / (size_t)x_shape[dim]);
+    return ZG_HIP_OK;
+}
+
+// sum_along with the case split of src/device/host_device.zig:798-847
+static int sum_along_impl(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, float* y,
+                          size_t y_len, size_t dim, float alpha, float beta) {
+    const size_t total = prod(x_shape, 0, x_rank);
+    if (y_len == 1) return flat_reduce<TermId, 1>(ctx, x, nullptr, total, 0.f, FinAxpby{y, alpha, beta});
+    const size_t outer = prod(x_shape, 0, dim), R = x_shape[dim], inner = prod(x_shape, dim + 1, x_rank);
+    ZG_REQUIRE(y_len >= outer * inner, "sum_along: y.len %zu too small for %zu outputs", y_len, outer * inner);
+    return axis_reduce<AxisSum>(ctx, x, y, outer, R, inner, alpha, beta);
+}
+
+}  // namespace zg
+
+using namespace zg;
+
+ZG_API int zg_hip_sum(zg_hip_ctx* ctx, const float* x, size_t n, float* y) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(x && y && n > 0, "sum: null or empty operand");
+    return flat_reduce<TermAbs, 1>(ctx, x, nullptr, n, 0.f, FinStore{y});
+}
+
+ZG_API int zg_hip_nrm2(zg_hip_ctx* ctx, const float* x, size_t n, float* y) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(x && y && n > 0, "nrm2: null or empty operand");
+    return flat_reduce<TermSq, 1>(ctx, x, nullptr, n, 0.f, FinSqrt{y});
+}
+
+ZG_API int zg_hip_dot(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, float* z) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(x && y && z && n > 0, "dot: null or empty operand");
+    return flat_reduce<TermDot, 2>(ctx, x, y, n, 0.f, FinStore{z});
+}
+
+ZG_API int zg_hip_max_fwd(zg_hip_ctx* ctx, const float* x, size_t n, float* y) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(x && y && n > 0, "max_fwd: null or empty operand");
+    ZG_REQUIRE(n < 0xffffffffull, "max_fwd: more than 2^32-1 elements");
+    return flat_reduce<TermAbsArg, 1>(ctx, x, nullptr, n, 0.f, FinAbsArg{y});
+}
+
+ZG_API int zg_hip_max_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, size_t n, const float* y, const float* y_g) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(x && x_g && y && y_g, "max_bwd: null pointer");
+    hipLaunchKernelGGL(max_bwd_kernel, dim3(stream_grid(ctx, n, 4)), dim3(kBlock), 0, ctx->stream, x, x_g, n, y, y_g);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// The norm never leaves the device: a reduction writes the clip factor to a device slot and the
+// scaling kernel reads it (and returns immediately when the factor is 1).
+ZG_API int zg_hip_clip_nrm2(zg_hip_ctx* ctx, float* x, size_t n, float max_norm, float delta) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(x != nullptr, "clip_nrm2: null pointer");
+    float* factor = ctx->scalar_slot + 1;
+    int rc = flat_reduce<TermSq, 1>(ctx, x, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
+    if (rc) return rc;
+    hipLaunchKernelGGL(scale_by_device_factor_kernel, dim3(stream_grid(ctx, n, 8)), dim3(kBlock), 0, ctx->stream, x, n,
+                       factor);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_axpy(zg_hip_ctx* ctx, const float* x, float* y, size_t n, const float* alpha, int alpha_on_device) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(x && y && alpha, "axpy: null pointer");
+    const float* dev_alpha = alpha;
+    if (!alpha_on_device) {
+        // stage the host scalar; the slot is reused only by later work on the same stream
+        ZG_HIP_TRY(hipMemcpyAsync(ctx->scalar_slot, alpha, sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+        dev_alpha = ctx->scalar_slot;
+    }
+    hipLaunchKernelGGL(axpy_kernel, dim3(stream_grid(ctx, n, 8)), dim3(kBlock), 0, ctx->stream, x, y, n, dev_alpha);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_smooth_l1_fwd(zg_hip_ctx* ctx, const float* pred, const float* target, size_t n, float beta,
+                                float* loss) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(pred && target && loss && n > 0, "smooth_l1_fwd: null or empty operand");
+    return flat_reduce<TermSmoothL1, 2>(ctx, pred, target, n, beta, FinDivN{loss, (float)n});
+}
+
+ZG_API int zg_hip_mse_fwd(zg_hip_ctx* ctx, const float* pred, const float* target, size_t n, float* loss) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(pred && target && loss && n > 0, "mse_fwd: null or empty operand");
+    return flat_reduce<TermSqDiff, 2>(ctx, pred, target, n, 0.f, FinDivN{loss, (float)n});
+}
+
+ZG_API int zg_hip_sum_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, float* y,
+                            size_t y_len, size_t dim, float alpha, float beta) {
+    ZG_CTX(ctx);
+    int rc = check_axis_args("sum_along", x, x_shape, x_rank, y, y_len, dim);
+    if (rc) return rc;
+    return sum_along_impl(ctx, x, x_shape, x_rank, y, y_len, dim, alpha, beta);
+}
+
+ZG_API int zg_hip_max_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, float* y,
+                            size_t y_len, size_t dim) {
+    ZG_CTX(ctx);
+    int rc = check_axis_args("max_along", x, x_shape, x_rank, y, y_len, dim);
+    if (rc) return rc;
+    const size_t outer = prod(x_shape, 0, dim), R = x_shape[dim], inner = prod(x_shape, dim + 1, x_rank);
+    ZG_REQUIRE(y_len == outer * inner, "max_along: y.len %zu != %zu", y_len, outer * inner);
+    return axis_reduce<AxisMax>(ctx, x, y, outer, R, inner, 1.f, 0.f);
+}
+
+ZG_API int zg_hip_argmax_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, uint64_t* y,
+                               size_t y_len, size_t dim) {
+    ZG_CTX(ctx);
+    int rc = check_axis_args("argmax_along", x, x_shape, x_rank, y, y_len, dim);
+    if (rc) return rc;
+    const size_t outer = prod(x_shape, 0, dim), R = x_shape[dim], inner = prod(x_shape, dim + 1, x_rank);
+    ZG_REQUIRE(y_len == outer * inner, "argmax_along: y.len %zu != %zu", y_len, outer * inner);
+    return axis_reduce<AxisArgmax>(ctx, x, y, outer, R, inner, 1.f, 0.f);
+}
+
+// src/ndarray.zig:701-719
+ZG_API size_t zg_hip_unbroadcast_scratch_len(const uint64_t* x_shape, size_t x_rank, const uint64_t* y_shape,
+                                             size_t y_rank) {
+    if (!x_shape || !y_shape || x_rank < y_rank) return 0;
+    const size_t x_size = prod(x_shape, 0, x_rank), y_size = prod(y_shape, 0, y_rank);
+    const size_t delta = x_rank - y_rank;
+    size_t coef;
+    if (delta > 0) {
+        coef = prod(x_shape, 0, delta);
+    } else {
+        size_t mm = x_rank;
+        for (size_t i = 0; i < x_rank; i++)
+            if (x_shape[i] != y_shape[i]) {
+                mm = i;
+                break;
+            }
+        if (mm == x_rank) return 0;
+        coef = x_shape[mm];
+    }
+    const size_t n = y_size * coef;
+    return n == x_size ? 0 : n;
+}
+
+namespace zg {
+__global__ __launch_bounds__(kBlock) void scaled_copy_kernel(const float* x, float* y, size_t n, float alpha, float beta) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
+    for (; i < n; i += nt) {
+        float r = __fmul_rn(alpha, x[i]);
+        y[i] = (beta == 0.f) ? r : __fadd_rn(r, __fmul_rn(beta, y[i]));
+    }
+}
+}  // namespace zg
+
+// The staging of src/device/host_device.zig:709-780: one fold over the leading extra dims, then one
+// sum_along per interior 1-dim, alpha/beta applied at every stage exactly as the reference does.
+ZG_API int zg_hip_unbroadcast(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape_in, size_t x_rank_in, float* y,
+                              const uint64_t* y_shape_in, size_t y_rank_in, float* scratch, size_t scratch_len,
+                              float alpha, float beta) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(x && y && x_shape_in && y_shape_in, "unbroadcast: null pointer");
+    ZG_REQUIRE(x_rank_in >= 1 && x_rank_in <= 8 && y_rank_in >= 1 && y_rank_in <= 8, "unbroadcast: rank not in 1..8");
+    ZG_REQUIRE(x_rank_in >= y_rank_in, "unbroadcast: x rank %zu < y rank %zu", x_rank_in, y_rank_in);
+    const size_t x_len = prod(x_shape_in, 0, x_rank_in), y_len = prod(y_shape_in, 0, y_rank_in);
+    ZG_REQUIRE(x_len > 0 && y_len > 0 && x_len % y_len == 0, "unbroadcast: sizes %zu and %zu are incompatible", x_len,
+               y_len);
+    ZG_REQUIRE(x != y, "unbroadcast: input and output alias");
+    if (x_len == y_len) {
+        hipLaunchKernelGGL(scaled_copy_kernel, dim3(stream_grid(ctx, x_len, 4)), dim3(kBlock), 0, ctx->stream, x, y,
+                           x_len, alpha, beta);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    uint64_t xs[8], ys[8];
+    size_t xr = 0, yr = 0;
+    {
+        size_t s = 0;
+        while (s < x_rank_in && x_shape_in[s] == 1) s++;
+        for (size_t i = s; i < x_rank_in; i++) xs[xr++] = x_shape_in[i];
+        size_t b = 0, e = y_rank_in;
+        while (b < e && y_shape_in[b] == 1) b++;
+        while (e > b && y_shape_in[e - 1] == 1) e--;
+        for (size_t i = b; i < e; i++) ys[yr++] = y_shape_in[i];
+    }
+    size_t ones = 0;
+    for (size_t i = 0; i < yr; i++) ones += (ys[i] == 1);
+
+    // every stage is validated before the first launch
+    if (xr > yr) {
+        const size_t dif = xr - yr;
+        const size_t col = prod(xs, dif, xr);
+        if (ones == 0) ZG_REQUIRE(col <= y_len, "unbroadcast: fold writes %zu elements into y of %zu", col, y_len);
+        else ZG_REQUIRE(scratch && col <= scratch_len, "unbroadcast: scratch of %zu floats needed, %zu given", col, scratch_len);
+    }
+    if (xr > yr) {
+        const size_t dif = xr - yr;
+        const size_t row = prod(xs, 0, dif), col = prod(xs, dif, xr);
+        int rc = axis_reduce<AxisSum>(ctx, x, ones == 0 ? y : scratch, 1, row, col, alpha, beta);
+        if (rc) return rc;
+        if (ones == 0) return ZG_HIP_OK;
+        for (size_t i = dif; i < xr; i++) xs[i - dif] = xs[i];
+        xr -= dif;
+    }
+    size_t i = 0;
+    while (ones > 0 && i < xr) {
+        if (i < yr && ys[i] == 1 && xs[i] != 1) {
+            const float* xd = (xr == x_rank_in) ? x : scratch;
+            float* yd = (ones == 1) ? y : scratch;
+            const size_t yl = (ones == 1) ? y_len : scratch_len;
+            const size_t need = prod(xs, 0, xr) / xs[i];
+            ZG_REQUIRE(xd != nullptr && yd != nullptr, "unbroadcast: scratch required but null");
+            ZG_REQUIRE(yl == 1 || yl >= need, "unbroadcast: stage output of %zu elements does not fit %zu", need, yl);
+            ZG_REQUIRE(xd != yd, "unbroadcast: a stage would read and write the scratch buffer at once");
+            int rc = sum_along_impl(ctx, xd, xs, xr, yd, yl, i, alpha, beta);
+            if (rc) return rc;
+            for (size_t j = i + 1; j < xr; j++) xs[j - 1] = xs[j];
+            for (size_t j = i + 1; j < yr; j++) ys[j - 1] = ys[j];
+            xr--;
+            yr--;
+            ones--;
+            continue;
+        }
+        i++;
+    }
+    return ZG_HIP_OK;
+}

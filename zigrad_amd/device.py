@@ -1,0 +1,412 @@
+"""HipDevice: the host-side face of the gfx950 backend.
+
+It mirrors the device interface Zigrad's upper layers program against
+(reference: src/device/device_reference.zig:15-131): `dispatch(name, **params)` takes the op name and
+the field names of the matching parameter struct in src/device/opspec.zig, and the `mem_*` methods
+keep the names and meaning of the reference's memory API.  Every call goes through the C ABI in
+include/zg_hip.h; nothing is computed in Python and nothing falls back to the CPU.
+
+Slices of the reference (`[]T`) are `DevBuf` objects here: a device pointer, an element count and a
+dtype.  `DevBuf.sub(offset, n)` is the pointer-arithmetic sub-slice the reference takes freely
+(src/ndtensor.zig:581, :1462-1464).
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import numpy as np
+
+from ._lib import ZgHipError, lib
+
+F32 = np.dtype(np.float32)
+U64 = np.dtype(np.uint64)
+
+
+@dataclass
+class DevBuf:
+    ptr: int
+    n: int
+    dtype: np.dtype = F32
+    block: int = 0  # DeviceData.ctx of the reference: 0 for views / raw allocations
+    kind: str = "raw"  # "raw" (mem_alloc), "cache" (mem_cache_alloc), "view", "host" (pinned host)
+
+    def __len__(self) -> int:
+        return self.n
+
+    @property
+    def nbytes(self) -> int:
+        return self.n * self.dtype.itemsize
+
+    def sub(self, offset: int, n: int) -> "DevBuf":
+        if offset < 0 or n < 0 or offset + n > self.n:
+            raise IndexError(f"sub-slice [{offset}:{offset + n}] outside a buffer of {self.n} elements")
+        return DevBuf(self.ptr + offset * self.dtype.itemsize, n, self.dtype, 0, "view")
+
+
+def _shape(shape) -> tuple[ctypes.Array, int]:
+    arr = (ctypes.c_uint64 * len(shape))(*[int(s) for s in shape])
+    return arr, len(shape)
+
+
+class HipDevice:
+    """One MI355X device context: a single in-order stream plus the caching allocator."""
+
+    def __init__(self, device_id: int = 0):
+        self._lib = lib()
+        ctx = ctypes.c_void_p()
+        self._lib.call("zg_hip_init", int(device_id), ctypes.byref(ctx))
+        self._ctx = ctx
+        self.device_id = device_id
+
+    # -- lifecycle ---------------------------------------------------------------------------
+    def deinit(self) -> None:
+        if self._ctx is not None:
+            self._lib.call("zg_hip_deinit", self._ctx)
+            self._ctx = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.deinit()
+
+    def is_host(self) -> bool:
+        return False
+
+    def is_compatible(self, other) -> bool:
+        return isinstance(other, HipDevice) and other.device_id == self.device_id
+
+    def sync(self) -> None:
+        self._call("zg_hip_sync")
+
+    def _call(self, name: str, *args) -> None:
+        self._lib.call(name, self._ctx, *args)
+
+    # -- timing ------------------------------------------------------------------------------
+    def event(self) -> "Event":
+        return Event(self)
+
+    # -- memory API (src/device/device_reference.zig:29-123) -----------------------------------
+    def mem_alloc(self, dtype, n: int) -> DevBuf:
+        dtype = np.dtype(dtype)
+        p = ctypes.c_void_p()
+        self._call("zg_hip_alloc", n * dtype.itemsize, ctypes.byref(p))
+        return DevBuf(p.value or 0, n, dtype, 0, "raw")
+
+    def mem_free(self, buf: DevBuf) -> None:
+        if buf.n == 0 or buf.ptr == 0:
+            return
+        if buf.kind == "host":
+            self._call("zg_hip_host_free", buf.ptr)
+        else:
+            self._call("zg_hip_free", buf.ptr)
+        buf.ptr, buf.n = 0, 0
+
+    def mem_alloc_host(self, dtype, n: int) -> DevBuf:
+        """Pinned host memory the kernels can read: for index arrays the caller fills on the host."""
+        dtype = np.dtype(dtype)
+        p = ctypes.c_void_p()
+        self._call("zg_hip_host_alloc", n * dtype.itemsize, ctypes.byref(p))
+        return DevBuf(p.value or 0, n, dtype, 0, "host")
+
+    def mem_alloc_byte_mask(self, n: int) -> DevBuf:
+        return self.mem_alloc(np.uint8, (n - 1) // 8 + 1)
+
+    def mem_cache_alloc(self, dtype, n: int) -> DevBuf:
+        dtype = np.dtype(dtype)
+        p, blk = ctypes.c_void_p(), ctypes.c_uint64()
+        self._call("zg_hip_mem_cache_alloc", n * dtype.itemsize, ctypes.byref(p), ctypes.byref(blk))
+        return DevBuf(p.value or 0, n, dtype, blk.value, "cache")
+
+    def mem_cache_free(self, buf: DevBuf) -> None:
+        if buf.block == 0:
+            return
+        self._call("zg_hip_mem_cache_free", buf.ptr, buf.block)
+        buf.ptr, buf.n, buf.block = 0, 0, 0
+
+    def mem_cache_dupe(self, src: DevBuf) -> DevBuf:
+        dst = self.mem_cache_alloc(src.dtype, src.n)
+        self.mem_copy(src, dst)
+        return dst
+
+    def mem_dupe(self, src: DevBuf) -> DevBuf:
+        dst = self.mem_alloc(src.dtype, src.n)
+        self.mem_copy(src, dst)
+        return dst
+
+    def mem_scratch(self, dtype, n: int) -> DevBuf:
+        dtype = np.dtype(dtype)
+        p = ctypes.c_void_p()
+        self._call("zg_hip_mem_scratch", n * dtype.itemsize, ctypes.byref(p))
+        return DevBuf(p.value or 0, n, dtype, 0, "view")
+
+    def clear_cache(self) -> None:
+        self._call("zg_hip_clear_cache")
+
+    def cache_stats(self) -> dict:
+        u, m, a = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_uint64()
+        self._call("zg_hip_cache_stats", ctypes.byref(u), ctypes.byref(m), ctypes.byref(a))
+        return {"bytes_in_use": u.value, "bytes_mapped": m.value, "n_device_allocs": a.value}
+
+    def mem_fill(self, buf: DevBuf, value) -> None:
+        if buf.dtype == F32:
+            self._call("zg_hip_mem_fill", buf.ptr, buf.n, float(value))
+        elif buf.dtype == U64:
+            self._call("zg_hip_mem_fill_u64", buf.ptr, buf.n, int(value))
+        elif buf.dtype.itemsize == 1:
+            self._call("zg_hip_mem_fill_u8", buf.ptr, buf.n, int(value))
+        else:
+            raise TypeError(f"mem_fill: unsupported dtype {buf.dtype}")
+
+    def mem_copy(self, src: DevBuf, dst: DevBuf) -> None:
+        if dst.n < src.n:
+            raise ValueError("mem_copy: destination shorter than source")
+        self._call("zg_hip_memcpy_d2d", dst.ptr, src.ptr, src.nbytes)
+
+    def mem_sequence(self, buf: DevBuf, initial: float, step: float) -> None:
+        self._call("zg_hip_mem_sequence", buf.ptr, buf.n, float(initial), float(step))
+
+    def mem_random(self, buf: DevBuf, kind: str, seed: int, fan: int = 0) -> None:
+        code = {"uniform": 0, "normal": 1, "kaiming": 2}[kind]
+        self._call("zg_hip_mem_random", buf.ptr, buf.n, code, int(fan), int(seed))
+
+    def mem_take(self, src: DevBuf, idxs: DevBuf, dst: DevBuf) -> None:
+        if dst.n < idxs.n:
+            raise ValueError("mem_take: dst.len < idxs.len")
+        self._call("zg_hip_mem_take", src.ptr, src.n, idxs.ptr, idxs.n, dst.ptr)
+
+    def mem_transfer(self, src, dst, direction: str) -> None:
+        """direction: 'HtoD' (src numpy array), 'DtoH' (dst numpy array, blocking), 'DtoD'."""
+        if direction == "HtoD":
+            a = np.ascontiguousarray(src, dtype=dst.dtype)
+            if a.size > dst.n:
+                raise ValueError("mem_transfer: destination too small")
+            self._call("zg_hip_memcpy_h2d", dst.ptr, a.ctypes.data, a.nbytes)
+        elif direction == "DtoH":
+            if not (isinstance(dst, np.ndarray) and dst.flags.c_contiguous and dst.dtype == src.dtype):
+                raise ValueError("mem_transfer: DtoH needs a contiguous numpy array of the buffer's dtype")
+            if dst.size < src.n:
+                raise ValueError("mem_transfer: destination too small")
+            self._call("zg_hip_memcpy_d2h", dst.ctypes.data, src.ptr, src.nbytes)
+        elif direction == "DtoD":
+            self.mem_copy(src, dst)
+        else:
+            raise ValueError(f"unknown transfer direction {direction!r}")
+
+    # conveniences built on the above (not part of the reference interface)
+    def from_numpy(self, a: np.ndarray, cached: bool = False) -> DevBuf:
+        a = np.ascontiguousarray(a)
+        buf = (self.mem_cache_alloc if cached else self.mem_alloc)(a.dtype, a.size)
+        if a.size:
+            self._call("zg_hip_memcpy_h2d", buf.ptr, a.ctypes.data, a.nbytes)
+        return buf
+
+    def to_numpy(self, buf: DevBuf, shape=None) -> np.ndarray:
+        out = np.empty(buf.n, dtype=buf.dtype)
+        if buf.n:
+            self._call("zg_hip_memcpy_d2h", out.ctypes.data, buf.ptr, buf.nbytes)
+        return out.reshape(shape) if shape is not None else out
+
+    # -- op dispatch (src/device/device_reference.zig:15-27) -----------------------------------
+    def dispatch(self, name: str, **p) -> None:
+        """Run device op `name` with the field names of opspec.<name>; unknown names raise like the
+        reference's @panic("Unimplemented")."""
+        fn = getattr(self, "_op_" + name, None)
+        if fn is None:
+            raise NotImplementedError(f"Unimplemented: {name} for HipDevice")
+        fn(**p)
+
+    # elementwise binary
+    def _bin(self, cname, x, y, z):
+        self._call(cname, x.ptr, x.n, y.ptr, y.n, z.ptr, z.n)
+
+    def _op_add(self, x, y, z): self._bin("zg_hip_add", x, y, z)
+    def _op_sub(self, x, y, z): self._bin("zg_hip_sub", x, y, z)
+    def _op_mul(self, x, y, z): self._bin("zg_hip_mul", x, y, z)
+    def _op_div(self, x, y, z): self._bin("zg_hip_div", x, y, z)
+
+    # linear algebra
+    def _op_dot(self, x, y, z):
+        if x.n != y.n:
+            raise ValueError("dot: length mismatch")
+        self._call("zg_hip_dot", x.ptr, y.ptr, x.n, z.ptr)
+
+    def _op_matvec(self, A, x, y, m, n, trans_a, alpha, beta):
+        self._call("zg_hip_matvec", A.ptr, x.ptr, y.ptr, m, n, int(trans_a), alpha, beta)
+
+    def _op_matmul(self, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta):
+        self._call("zg_hip_matmul", A.ptr, B.ptr, C.ptr, m, n, k, int(trans_a), int(trans_b), lda, ldb, ldc,
+                   alpha, beta)
+
+    def _op_bmm_acc(self, A, B, C, A_shape, B_shape, C_shape, trans_a, trans_b, lda, ldb, ldc, alpha, beta):
+        a, _ = _shape(A_shape)
+        b, _ = _shape(B_shape)
+        c, _ = _shape(C_shape)
+        self._call("zg_hip_bmm_acc", A.ptr, a, B.ptr, b, C.ptr, c, int(trans_a), int(trans_b), lda, ldb, ldc,
+                   alpha, beta)
+
+    def _op_outer(self, x, y, A, alpha):
+        self._call("zg_hip_outer", x.ptr, x.n, y.ptr, y.n, A.ptr, alpha)
+
+    def _op_transpose(self, A, B, m, n, alpha):
+        self._call("zg_hip_transpose", A.ptr, B.ptr, m, n, alpha)
+
+    def _op_axpy(self, x, y, alpha):
+        """alpha: a Python float (the host pointer of SGD) or a 1-element DevBuf (dot backward)."""
+        if isinstance(alpha, DevBuf):
+            self._call("zg_hip_axpy", x.ptr, y.ptr, x.n, alpha.ptr, 1)
+        else:
+            a = ctypes.c_float(alpha)
+            self._call("zg_hip_axpy", x.ptr, y.ptr, x.n, ctypes.byref(a), 0)
+
+    def _op_sum(self, x, y): self._call("zg_hip_sum", x.ptr, x.n, y.ptr)
+    def _op_scale(self, x, alpha): self._call("zg_hip_scale", x.ptr, x.n, alpha)
+    def _op_nrm2(self, x, y): self._call("zg_hip_nrm2", x.ptr, x.n, y.ptr)
+    def _op_clip_nrm2(self, x, max_norm, delta): self._call("zg_hip_clip_nrm2", x.ptr, x.n, max_norm, delta)
+
+    # unary
+    def _op_pow_fwd(self, x, exp, y): self._call("zg_hip_pow_fwd", x.ptr, y.ptr, x.n, exp)
+    def _op_pow_fwd_(self, x, exp): self._call("zg_hip_pow_fwd", x.ptr, x.ptr, x.n, exp)
+    def _op_pow_bwd(self, x, x_g, exp, y_g, eps): self._call("zg_hip_pow_bwd", x.ptr, x_g.ptr, y_g.ptr, x.n, exp, eps)
+    def _op_sqrt_fwd(self, x, y): self._call("zg_hip_sqrt_fwd", x.ptr, y.ptr, x.n)
+    def _op_sqrt_fwd_(self, x): self._call("zg_hip_sqrt_fwd", x.ptr, x.ptr, x.n)
+    def _op_sqrt_bwd(self, x, x_g, y_g, eps): self._call("zg_hip_sqrt_bwd", x.ptr, x_g.ptr, y_g.ptr, x.n, eps)
+    def _op_rsqrt_fwd(self, x, y, eps): self._call("zg_hip_rsqrt_fwd", x.ptr, y.ptr, x.n, eps)
+    def _op_rsqrt_bwd(self, x, x_g, y_g, eps): self._call("zg_hip_rsqrt_bwd", x.ptr, x_g.ptr, y_g.ptr, x.n, eps)
+    def _op_exp_fwd(self, x, y): self._call("zg_hip_exp_fwd", x.ptr, y.ptr, x.n)
+    def _op_exp_bwd(self, x_g, y, y_g): self._call("zg_hip_exp_bwd", x_g.ptr, y.ptr, y_g.ptr, x_g.n)
+    def _op_relu_fwd(self, x, y): self._call("zg_hip_relu_fwd", x.ptr, y.ptr, x.n)
+    def _op_relu_bwd(self, x, x_g, y_g): self._call("zg_hip_relu_bwd", x.ptr, x_g.ptr, y_g.ptr, x.n)
+    def _op_relu_inplace_bwd(self, x, x_g): self._call("zg_hip_relu_inplace_bwd", x.ptr, x_g.ptr, x.n)
+    def _op_tanh_fwd(self, x, y): self._call("zg_hip_tanh_fwd", x.ptr, y.ptr, x.n)
+    def _op_tanh_bwd(self, x_g, y, y_g): self._call("zg_hip_tanh_bwd", x_g.ptr, y.ptr, y_g.ptr, x_g.n)
+    def _op_tanh_inplace_bwd(self, x, x_g): self._call("zg_hip_tanh_inplace_bwd", x.ptr, x_g.ptr, x.n)
+    def _op_sigm_fwd(self, x, y): self._call("zg_hip_sigm_fwd", x.ptr, y.ptr, x.n)
+    def _op_sigm_bwd(self, x_g, y, y_g): self._call("zg_hip_sigm_bwd", x_g.ptr, y.ptr, y_g.ptr, x_g.n)
+    def _op_sigm_inplace_bwd(self, x, x_g): self._call("zg_hip_sigm_inplace_bwd", x.ptr, x_g.ptr, x.n)
+    def _op_clamp_fwd(self, x, y, min, max): self._call("zg_hip_clamp_fwd", x.ptr, y.ptr, x.n, min, max)
+    def _op_clamp_bwd(self, x, x_g, y_g, min, max): self._call("zg_hip_clamp_bwd", x.ptr, x_g.ptr, y_g.ptr, x.n, min, max)
+    def _op_max_fwd(self, x, y): self._call("zg_hip_max_fwd", x.ptr, x.n, y.ptr)
+    def _op_max_bwd(self, x, x_g, y, y_g): self._call("zg_hip_max_bwd", x.ptr, x_g.ptr, x.n, y.ptr, y_g.ptr)
+
+    # reductions
+    def _op_sum_along(self, x, x_shape, y, y_shape=None, dim=0, alpha=1.0, beta=0.0):
+        s, r = _shape(x_shape)
+        self._call("zg_hip_sum_along", x.ptr, s, r, y.ptr, y.n, dim, alpha, beta)
+
+    def _op_max_along(self, x, x_shape, y, y_shape=None, dim=0, alpha=1.0, beta=0.0):
+        s, r = _shape(x_shape)
+        self._call("zg_hip_max_along", x.ptr, s, r, y.ptr, y.n, dim)
+
+    def _op_argmax_along(self, x, x_shape, y, dim):
+        s, r = _shape(x_shape)
+        self._call("zg_hip_argmax_along", x.ptr, s, r, y.ptr, y.n, dim)
+
+    def unbroadcast_scratch_len(self, x_shape, y_shape) -> int:
+        xs, xr = _shape(x_shape)
+        ys, yr = _shape(y_shape)
+        return int(self._lib.cdll.zg_hip_unbroadcast_scratch_len(xs, xr, ys, yr))
+
+    def _op_unbroadcast(self, x, x_shape, y, y_shape, scratch=None, alpha=1.0, beta=0.0):
+        xs, xr = _shape(x_shape)
+        ys, yr = _shape(y_shape)
+        sp, sn = (scratch.ptr, scratch.n) if scratch is not None else (None, 0)
+        self._call("zg_hip_unbroadcast", x.ptr, xs, xr, y.ptr, ys, yr, sp, sn, alpha, beta)
+
+    def _op_broadcast(self, x, y, x_shape=None, y_shape=None, alpha=1.0, beta=0.0):
+        self._call("zg_hip_broadcast", x.ptr, x.n, y.ptr, y.n, alpha, beta)
+
+    # indexing
+    def gather_offsets(self, src_shape, idx_shape, indices: DevBuf, dim: int, offsets: DevBuf, check: bool = True) -> int:
+        ss, r = _shape(src_shape)
+        ish, _ = _shape(idx_shape)
+        st = ctypes.c_int(0)
+        try:
+            self._call("zg_hip_gather_offsets", ss, ish, r, indices.ptr, dim, offsets.ptr,
+                       ctypes.byref(st) if check else None)
+        except ZgHipError:
+            if st.value:
+                return st.value
+            raise
+        return st.value
+
+    def _op_scatter_add(self, src, offsets, dst):
+        if offsets.n != src.n:
+            raise ValueError("scatter_add: offsets.len != src.len")
+        self._call("zg_hip_scatter_add", src.ptr, offsets.ptr, src.n, dst.ptr, dst.n)
+
+    def _op_index_select_fwd(self, src, indices, stride, dst):
+        self._call("zg_hip_index_select_fwd", src.ptr, src.n, indices.ptr, indices.n, stride, dst.ptr)
+
+    def _op_index_select_bwd(self, y_grad, indices, stride, x_grad):
+        self._call("zg_hip_index_select_bwd", y_grad.ptr, indices.ptr, indices.n, stride, x_grad.ptr, x_grad.n)
+
+    def _op_scatter_gcn_deg_scaled(self, dst, h, deg, src_indices, tgt_indices, stride, n_edge):
+        self._call("zg_hip_scatter_gcn_deg_scaled", dst.ptr, h.ptr, deg.ptr, src_indices.ptr, tgt_indices.ptr,
+                   stride, n_edge, deg.n)
+
+    def _op_scatter_gcn_deg_scaled_bwd(self, grad_output, h, deg, src_indices, tgt_indices, grad_h, grad_deg, stride,
+                                       n_edge):
+        self._call("zg_hip_scatter_gcn_deg_scaled_bwd", grad_output.ptr, h.ptr, deg.ptr, src_indices.ptr,
+                   tgt_indices.ptr, grad_h.ptr, grad_deg.ptr, stride, n_edge, deg.n)
+
+    # losses
+    def _op_smce_fwd(self, logits, target, probs, loss, rows, cols):
+        self._call("zg_hip_smce_fwd", logits.ptr, target.ptr, probs.ptr, loss.ptr, rows, cols)
+
+    def _op_smce_bwd(self, probs, target, grad, rows, cols):
+        self._call("zg_hip_smce_bwd", probs.ptr, target.ptr, grad.ptr, rows, cols)
+
+    def _op_smce_label_fwd(self, logits, labels, lse, loss, rows, cols):
+        self._call("zg_hip_smce_label_fwd", logits.ptr, labels.ptr, lse.ptr, loss.ptr, rows, cols)
+
+    def _op_smce_label_bwd(self, logits, labels, lse, grad, rows, cols, accumulate=True):
+        self._call("zg_hip_smce_label_bwd", logits.ptr, labels.ptr, lse.ptr, grad.ptr, rows, cols, int(accumulate))
+
+    def _op_softmax_fwd(self, x, y, rows, cols): self._call("zg_hip_softmax_fwd", x.ptr, y.ptr, rows, cols)
+    def _op_softmax_bwd(self, y, y_g, x_g, rows, cols): self._call("zg_hip_softmax_bwd", y.ptr, y_g.ptr, x_g.ptr, rows, cols)
+
+    def _op_smooth_l1_fwd(self, pred, target, beta, loss):
+        self._call("zg_hip_smooth_l1_fwd", pred.ptr, target.ptr, pred.n, beta, loss.ptr)
+
+    def _op_smooth_l1_bwd(self, pred, target, grad, beta):
+        self._call("zg_hip_smooth_l1_bwd", pred.ptr, target.ptr, grad.ptr, pred.n, beta)
+
+    def _op_mse_fwd(self, pred, target, loss): self._call("zg_hip_mse_fwd", pred.ptr, target.ptr, pred.n, loss.ptr)
+    def _op_mse_bwd(self, pred, target, grad): self._call("zg_hip_mse_bwd", pred.ptr, target.ptr, grad.ptr, pred.n)
+
+    # optimizers
+    def _op_sgd_step(self, param, grad, lr, clip, max_norm, delta):
+        self._call("zg_hip_sgd_step", param.ptr, grad.ptr, param.n, lr, int(clip), max_norm, delta)
+
+    def _op_adam_step(self, param, grad, m, v, t, lr, beta1, beta2, epsilon, clip, max_norm, delta):
+        self._call("zg_hip_adam_step", param.ptr, grad.ptr, m.ptr, v.ptr, param.n, int(t), lr, beta1, beta2, epsilon,
+                   int(clip), max_norm, delta)
+
+
+class Event:
+    """A HIP event on the device's stream (timing only)."""
+
+    def __init__(self, dev: HipDevice):
+        self._dev = dev
+        h = ctypes.c_void_p()
+        dev._call("zg_hip_event_create", ctypes.byref(h))
+        self._h = h
+
+    def record(self) -> "Event":
+        self._dev._call("zg_hip_event_record", self._h)
+        return self
+
+    def elapsed_ms(self, later: "Event") -> float:
+        ms = ctypes.c_float()
+        self._dev._lib.call("zg_hip_event_elapsed_ms", self._h, later._h, ctypes.byref(ms))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self._h is not None:
+                self._dev._lib.cdll.zg_hip_event_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass

@@ -1,0 +1,134 @@
+"""Host-side shape logic that sits between Zigrad's tensors and the device ops.
+
+These functions restate, for `DevBuf` operands, what the reference's NDArray / NDTensor layers do on
+the host before they dispatch to a device: work out batch shapes and leading dimensions for bmm,
+size the scratch for unbroadcast, turn gather indices into flat offsets, and issue the device GEMMs a
+matmul's backward needs.  They run unchanged on any device object with `dispatch` and the `mem_*` API.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+from .device import DevBuf, F32, U64
+
+
+def _prod(xs) -> int:
+    return int(math.prod(int(x) for x in xs))
+
+
+def _broadcast_batch(a: list[int], b: list[int]) -> list[int]:
+    """Right-aligned broadcast of two batch-dim lists (reference: src/ndarray/shape.zig:247-264)."""
+    n = max(len(a), len(b))
+    a = [1] * (n - len(a)) + list(a)
+    b = [1] * (n - len(b)) + list(b)
+    out = []
+    for x, y in zip(a, b):
+        if x != y and x != 1 and y != 1:
+            raise ValueError(f"batch dims {a} and {b} do not broadcast")
+        out.append(max(x, y))
+    return out
+
+
+def bmm_out_shape(a_shape, b_shape, trans_a: bool, trans_b: bool) -> list[int]:
+    a_shape, b_shape = list(a_shape), list(b_shape)
+    if len(a_shape) < 2:
+        a_shape = [1] + a_shape
+    if len(b_shape) < 2:
+        b_shape = [1] + b_shape
+    a_batch = a_shape[:-2] if len(a_shape) > 2 else [1]
+    b_batch = b_shape[:-2] if len(b_shape) > 2 else [1]
+    batch = [] if (len(a_shape) == 2 and len(b_shape) == 2) else _broadcast_batch(a_batch, b_batch)
+    a_rows, a_cols = a_shape[-2:]
+    b_rows, b_cols = b_shape[-2:]
+    M = a_cols if trans_a else a_rows
+    N = b_rows if trans_b else b_cols
+    return batch + [M, N]
+
+
+def bmm_acc_(dev, A: DevBuf, a_shape, B: DevBuf, b_shape, C: DevBuf, trans_a=False, trans_b=False, alpha=1.0,
+             beta=0.0) -> list[int]:
+    """C = alpha * op(A) op(B) + beta * C with batch broadcasting.  Reference: bmm_acc_impl,
+    src/ndarray.zig:817-899 (shape logic, lda/ldb/ldc = physical column counts)."""
+    a_shape, b_shape = list(a_shape), list(b_shape)
+    if len(a_shape) < 2:
+        a_shape = [1] + a_shape
+    if len(b_shape) < 2:
+        b_shape = [1] + b_shape
+    a_batch = a_shape[:-2] if len(a_shape) > 2 else [1]
+    b_batch = b_shape[:-2] if len(b_shape) > 2 else [1]
+    batch = [] if (len(a_shape) == 2 and len(b_shape) == 2) else _broadcast_batch(a_batch, b_batch)
+    a_rows, a_cols = a_shape[-2:]
+    b_rows, b_cols = b_shape[-2:]
+    M = a_cols if trans_a else a_rows
+    K = a_rows if trans_a else a_cols
+    N = b_rows if trans_b else b_cols
+    if K != (b_cols if trans_b else b_rows):
+        raise ValueError(f"incompatible matrix dimensions {a_rows}x{a_cols} and {b_rows}x{b_cols}")
+    c_shape = batch + [M, N]
+    if C.n < _prod(c_shape):
+        raise ValueError("bmm_acc_: output buffer too small")
+    dev.dispatch(
+        "bmm_acc", A=A, B=B, C=C,
+        A_shape=[_prod(a_batch), M, K], B_shape=[_prod(b_batch), K, N], C_shape=[_prod(batch), M, N],
+        trans_a=trans_a, trans_b=trans_b, lda=a_cols, ldb=b_cols, ldc=N, alpha=alpha, beta=beta,
+    )
+    return c_shape
+
+
+def bmm_acc_backward(dev, trans_a: bool, trans_b: bool, A: DevBuf, a_shape, B: DevBuf, b_shape, C_grad: DevBuf, c_shape,
+                     A_grad: DevBuf | None, B_grad: DevBuf | None) -> None:
+    """The device GEMMs BmmAccBwd issues (src/ndtensor.zig:1092-1136); grads are accumulated (beta = 1)."""
+    if A_grad is not None:
+        if not trans_a and not trans_b:      # MATMUL_AB:   dA += dC . B^T
+            bmm_acc_(dev, C_grad, c_shape, B, b_shape, A_grad, False, True, 1.0, 1.0)
+        elif trans_a and not trans_b:        # MATMUL_AtB:  dA += B . dC^T
+            bmm_acc_(dev, B, b_shape, C_grad, c_shape, A_grad, False, True, 1.0, 1.0)
+        elif not trans_a and trans_b:        # MATMUL_ABt:  dA += dC . B
+            bmm_acc_(dev, C_grad, c_shape, B, b_shape, A_grad, False, False, 1.0, 1.0)
+        else:                                # MATMUL_AtBt: dA += B^T . dC^T
+            bmm_acc_(dev, B, b_shape, C_grad, c_shape, A_grad, True, True, 1.0, 1.0)
+    if B_grad is not None:
+        if not trans_a and not trans_b:      # dB += A^T . dC
+            bmm_acc_(dev, A, a_shape, C_grad, c_shape, B_grad, True, False, 1.0, 1.0)
+        elif trans_a and not trans_b:        # dB += A . dC
+            bmm_acc_(dev, A, a_shape, C_grad, c_shape, B_grad, False, False, 1.0, 1.0)
+        elif not trans_a and trans_b:        # dB += dC^T . A
+            bmm_acc_(dev, C_grad, c_shape, A, a_shape, B_grad, True, False, 1.0, 1.0)
+        else:                                # dB += dC^T . A^T
+            bmm_acc_(dev, C_grad, c_shape, A, a_shape, B_grad, True, True, 1.0, 1.0)
+
+
+def unbroadcast_(dev, x: DevBuf, x_shape, out: DevBuf, out_shape, alpha=1.0, beta=0.0) -> None:
+    """Reduce a broadcast gradient back to an operand's shape.  Reference: NDArray.unbroadcast_,
+    src/ndarray.zig:687-730 (scratch sizing) + the device op."""
+    x_shape, out_shape = list(x_shape), list(out_shape)
+    if len(x_shape) < len(out_shape) or _prod(x_shape) % _prod(out_shape) != 0:
+        raise ValueError(f"cannot unbroadcast {x_shape} to {out_shape}")
+    n = dev.unbroadcast_scratch_len(x_shape, out_shape)
+    scratch = dev.mem_scratch(F32, n) if n else None
+    dev.dispatch("unbroadcast", x=x, x_shape=x_shape, y=out, y_shape=out_shape, scratch=scratch, alpha=alpha, beta=beta)
+
+
+def gather(dev, src: DevBuf, src_shape, indices: DevBuf, idx_shape, dim: int, return_offsets: bool = False):
+    """values[i] = src[coord(i) with coord[dim] := indices[i]].  Reference: NDArray.gather,
+    src/ndarray.zig:593-633; the offsets are computed by a device op instead of a host loop."""
+    src_shape, idx_shape = list(src_shape), list(idx_shape)
+    if len(src_shape) != len(idx_shape):
+        raise ValueError("gather: rank mismatch")
+    n = _prod(idx_shape)
+    offsets = dev.mem_alloc(U64, n)
+    status = dev.gather_offsets(src_shape, idx_shape, indices, dim, offsets)
+    if status == 1:
+        dev.mem_free(offsets)
+        raise ValueError("InvalidIndexShape")
+    if status == 2:
+        dev.mem_free(offsets)
+        raise IndexError("IndexOutOfBounds")
+    values = dev.mem_cache_alloc(F32, n)
+    dev.mem_take(src, offsets, values)
+    if return_offsets:
+        return values, offsets
+    dev.mem_free(offsets)
+    return values, None

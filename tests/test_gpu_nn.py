@@ -39,10 +39,17 @@ def test_smce_onehot_and_label(oracle, hip, rows, cols):
                                           "cols": cols}, ["probs", "loss"])
     x64 = x.astype(np.float64)
     sm = softmax(x64, axis=1)
-    loss = float(np.mean(logsumexp(x64, axis=1) - x64[np.arange(rows), lab]))
-    assert rel_fro(b["probs"], sm) <= TOL and rel_fro(a["probs"], sm) <= TOL
+    # the loss clamps the label's probability to [1e-7, 1 - 1e-7] (src/nn/loss.zig:143)
+    p_lab = np.exp(x64[np.arange(rows), lab] - logsumexp(x64, axis=1))
+    loss = float(np.mean(-np.log(np.clip(p_lab, np.float32(1e-7), np.float32(1.0) - np.float32(1e-7)))))
+    # The host loop adds the exponentials of a row one after the other in fp32; for rows of tens of thousands
+    # of columns that alone drifts past 1e-5 from the exact value.  The device result is held to 1e-5 against
+    # fp64; the oracle is held to 1e-5 where its own summation error allows it and to 2e-4 beyond.
+    oracle_tol = TOL if cols <= 4096 else 2e-4
+    assert rel_fro(b["probs"], sm) <= TOL and rel_fro(a["probs"], sm) <= oracle_tol
+    assert rel_fro(b["probs"], a["probs"]) <= max(TOL, 1.1 * rel_fro(a["probs"], sm) + 1e-6)
     assert abs(b["loss"][0] - loss) <= 1e-5 * max(1.0, abs(loss))
-    assert abs(b["loss"][0] - a["loss"][0]) <= 1e-5 * max(1.0, abs(loss))
+    assert abs(b["loss"][0] - a["loss"][0]) <= oracle_tol * max(1.0, abs(loss))
     g0 = (r.standard_normal((rows, cols)) * 0.01).astype(np.float32)
     ga, gb = both(oracle, hip, "smce_bwd", {"probs": b["probs"], "target": t, "grad": g0, "rows": rows, "cols": cols}, ["grad"])
     np.testing.assert_array_equal(ga["grad"], gb["grad"])  # pure sub/div/add on identical inputs
@@ -51,7 +58,7 @@ def test_smce_onehot_and_label(oracle, hip, rows, cols):
                                                   "rows": rows, "cols": cols}, ["lse", "loss"])
     assert rel_fro(b2["lse"], logsumexp(x64, axis=1)) <= 1e-6
     assert abs(b2["loss"][0] - loss) <= 1e-5 * max(1.0, abs(loss))
-    assert abs(b2["loss"][0] - a2["loss"][0]) <= 1e-5 * max(1.0, abs(loss))
+    assert abs(b2["loss"][0] - a2["loss"][0]) <= oracle_tol * max(1.0, abs(loss))
     want = g0 + (sm - t) / rows
     for acc in (True, False):
         g = run_op(hip, "smce_label_bwd", {"logits": x, "labels": lab, "lse": b2["lse"], "grad": g0.copy(), "rows": rows,
@@ -62,7 +69,7 @@ def test_smce_onehot_and_label(oracle, hip, rows, cols):
             assert np.abs(g.astype(np.float64).sum(axis=1)).max() <= 1e-6
     go = run_op(oracle, "smce_label_bwd", {"logits": x, "labels": lab, "lse": a2["lse"], "grad": g0.copy(), "rows": rows,
                                            "cols": cols}, ["grad"])["grad"]
-    assert rel_fro(go, want) <= TOL
+    assert rel_fro(go, want) <= oracle_tol
 
 
 def test_smce_clamp_edge(oracle, hip):
@@ -99,12 +106,18 @@ def test_smooth_l1_and_mse(oracle, hip, n):
     p, t = r.standard_normal(n).astype(np.float32) * 2, r.standard_normal(n).astype(np.float32)
     one = np.zeros(1, np.float32)
     g0 = r.standard_normal(n).astype(np.float32)
+    # the host loops add n terms one after the other in fp32; both sides are held against the fp64 value, the
+    # device (tree sum) to 1e-5 and the oracle to what a sequential fp32 sum of n terms allows
+    d64 = p.astype(np.float64) - t
+    sl1 = np.where(np.abs(d64) < 1.0, 0.5 * d64 * d64, np.abs(d64) - 0.5).mean()
+    seq_tol = max(1e-5, 2e-9 * n)
     a, b = both(oracle, hip, "smooth_l1_fwd", {"pred": p, "target": t, "beta": 1.0, "loss": one}, ["loss"])
-    assert abs(a["loss"][0] - b["loss"][0]) <= 1e-5 * abs(a["loss"][0])
+    assert abs(b["loss"][0] - sl1) <= 1e-5 * sl1 and abs(a["loss"][0] - sl1) <= seq_tol * sl1
     a, b = both(oracle, hip, "smooth_l1_bwd", {"pred": p, "target": t, "grad": g0, "beta": 1.0}, ["grad"])
     np.testing.assert_array_equal(a["grad"], b["grad"])
     a, b = both(oracle, hip, "mse_fwd", {"pred": p, "target": t, "loss": one}, ["loss"])
-    assert abs(a["loss"][0] - b["loss"][0]) <= 1e-5 * abs(a["loss"][0])
+    mse = (d64 * d64).mean()
+    assert abs(b["loss"][0] - mse) <= 1e-5 * mse and abs(a["loss"][0] - mse) <= seq_tol * mse
     a, b = both(oracle, hip, "mse_bwd", {"pred": p, "target": t, "grad": g0}, ["grad"])
     np.testing.assert_array_equal(a["grad"], b["grad"])
 

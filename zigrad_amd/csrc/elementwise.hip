@@ -246,8 +246,8 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
 
 // forward ops: a = x
 ZG_OP(PowFwd, return powf(a, p0);)
-ZG_OP(SqrtFwd, return __fsqrt_rn(a);)
-ZG_OP(RsqrtFwd, return __fdiv_rn(1.0f, __fsqrt_rn(fmaxf(a, p0)));)
+ZG_OP(SqrtFwd, return sqrtf(a);)
+ZG_OP(RsqrtFwd, return __fdiv_rn(1.0f, sqrtf(fmaxf(a, p0)));)
 ZG_OP(ExpFwd, return expf(a);)
 ZG_OP(ReluFwd, return a > 0.f ? a : 0.f;)
 ZG_OP(TanhFwd, return tanhf(a);)
@@ -257,9 +257,9 @@ ZG_OP(ClampFwd, return fminf(p1, fmaxf(p0, a));)
 ZG_OP(PowBwd, if (a < p1) return __fadd_rn(b, 0.0f);
       return __fadd_rn(b, __fmul_rn(__fmul_rn(p0, powf(a, __fsub_rn(p0, 1.0f))), c));)
 ZG_OP(SqrtBwd, if (a < p0) return __fadd_rn(b, 0.0f);
-      return __fadd_rn(b, __fmul_rn(__fdiv_rn(0.5f, __fsqrt_rn(a)), c));)
+      return __fadd_rn(b, __fmul_rn(__fdiv_rn(0.5f, sqrtf(a)), c));)
 ZG_OP(RsqrtBwd, if (a < p0) return __fadd_rn(b, 0.0f);
-      float s = __fsqrt_rn(a); float inv = __fdiv_rn(1.0f, __fmul_rn(a, s));
+      float s = sqrtf(a); float inv = __fdiv_rn(1.0f, __fmul_rn(a, s));
       return __fadd_rn(b, __fmul_rn(__fmul_rn(-0.5f, inv), c));)
 // exp_bwd: a = y, b = x_g, c = y_g
 ZG_OP(ExpBwd, return __fadd_rn(b, __fmul_rn(a, c));)

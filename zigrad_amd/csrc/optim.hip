@@ -51,7 +51,7 @@ __device__ __forceinline__ void adam_elem(float& p, float& g, float& m, float& v
     // src/nn/optim.zig:226-229, evaluated left to right in fp32
     m = __fadd_rn(__fmul_rn(b1, m), __fmul_rn(omb1, g));
     v = __fadd_rn(__fmul_rn(b2, v), __fmul_rn(__fmul_rn(omb2, g), g));
-    p = __fsub_rn(p, __fdiv_rn(__fmul_rn(lr_t, m), __fadd_rn(__fsqrt_rn(v), eps)));
+    p = __fsub_rn(p, __fdiv_rn(__fmul_rn(lr_t, m), __fadd_rn(sqrtf(v), eps)));
 }
 
 template <bool CLIP>

@@ -149,7 +149,7 @@ struct FinAxpby {  // src/device/reduce.zig:45
 };
 struct FinSqrt {
     float* y;
-    __device__ void operator()(float s) const { y[0] = __fsqrt_rn(s); }
+    __device__ void operator()(float s) const { y[0] = sqrtf(s); }
 };
 struct FinDivN {
     float* y;
@@ -161,7 +161,7 @@ struct FinClipFactor {
     float* factor;
     float max_norm, delta;
     __device__ void operator()(float s) const {
-        float norm = __fsqrt_rn(s);
+        float norm = sqrtf(s);
         factor[0] = (norm > max_norm) ? __fdiv_rn(max_norm, __fadd_rn(norm, delta)) : 1.0f;
     }
 };

@@ -14,12 +14,20 @@
 // A rows / B columns in that XCD's L2.
 #include "common.h"
 
+#include <type_traits>
+
 namespace zg {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));  // first-class vector: stays in registers
 
 constexpr int BK = 16;
 constexpr int kGemmThreads = 256;
+
+#ifndef ZG_GEMM_MNMAP
+#define ZG_GEMM_MNMAP 0
+#endif
+
 
 // One operand tile: `BMN` rows in the m (or n) direction by BK along k.
 // KMAJOR: element (mn, k) lives at ptr[mn * ld + k]   (A not transposed, B transposed)
@@ -29,33 +37,47 @@ template <int BMN, bool KMAJOR>
 struct Tile {
     static constexpr int LD = BMN + 4;
     static constexpr int NV = BMN * BK / 4 / kGemmThreads;
-    float4 r[NV];
+    floatx4 r[NV];
+
+    // which float4 of the tile thread `threadIdx.x` handles in its i-th access: (mn, k) of its first element
+    static __device__ __forceinline__ void coords(int i, int& mn, int& k) {
+        const int f = threadIdx.x + i * kGemmThreads;
+        if (KMAJOR) {
+            mn = f / (BK / 4);
+            k = (f % (BK / 4)) * 4;
+        } else {
+#if ZG_GEMM_MNMAP
+            constexpr int L = BMN / 32;  // 128-byte lines per k-row of the tile
+            constexpr int NL = BK * L;   // lines in the tile
+            const int hl = f >> 2, sub = f & 3;
+            const int line = hl % NL, pass = hl / NL;
+            const int half = (pass + line) & 1;
+            k = line / L;
+            mn = ((line % L) * 8 + half * 4 + sub) * 4;
+#else
+            k = f / (BMN / 4);
+            mn = (f % (BMN / 4)) * 4;
+#endif
+        }
+    }
 
     template <bool SAFE>
     __device__ __forceinline__ void load(const float* __restrict__ p, size_t ld, size_t mn0, size_t k0, size_t MN,
                                          size_t K, bool vec_ok) {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int f = threadIdx.x + i * kGemmThreads;
-            size_t mn, k;
-            const float* q;
-            if (KMAJOR) {
-                mn = mn0 + f / (BK / 4);
-                k = k0 + (f % (BK / 4)) * 4;
-                q = p + mn * ld + k;
-            } else {
-                k = k0 + f / (BMN / 4);
-                mn = mn0 + (f % (BMN / 4)) * 4;
-                q = p + k * ld + mn;
-            }
+            int tmn, tk;
+            coords(i, tmn, tk);
+            const size_t mn = mn0 + tmn, k = k0 + tk;
+            const float* q = KMAJOR ? p + mn * ld + k : p + k * ld + mn;
             if (!SAFE) {
-                r[i] = *reinterpret_cast<const float4*>(q);
+                r[i] = *reinterpret_cast<const floatx4*>(q);
             } else {
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
                 if (KMAJOR) {
                     if (mn < MN) {
                         if (vec_ok && k + 4 <= K) {
-                            v = *reinterpret_cast<const float4*>(q);
+                            v = *reinterpret_cast<const floatx4*>(q);
                         } else {
                             if (k + 0 < K) v.x = q[0];
                             if (k + 1 < K) v.y = q[1];
@@ -66,7 +88,7 @@ struct Tile {
                 } else {
                     if (k < K) {
                         if (vec_ok && mn + 4 <= MN) {
-                            v = *reinterpret_cast<const float4*>(q);
+                            v = *reinterpret_cast<const floatx4*>(q);
                         } else {
                             if (mn + 0 < MN) v.x = q[0];
                             if (mn + 1 < MN) v.y = q[1];
@@ -80,19 +102,35 @@ struct Tile {
         }
     }
 
+    // LDS write instructions this thread issues per tile: 4 scalar writes per float4 for a k-major operand
+    // (the transposing store), one 128-bit write otherwise
+    static constexpr int NW = NV * (KMAJOR ? 4 : 1);
+
+    // the op-th of those writes
+    __device__ __forceinline__ void store_op(float* __restrict__ lds, int op) const {
+        const int i = KMAJOR ? op / 4 : op;
+        int mn, k;
+        coords(i, mn, k);
+        if (KMAJOR) {
+            const int c = op % 4;
+            lds[(k + c) * LD + mn] = r[i][c];
+        } else {
+            *reinterpret_cast<floatx4*>(lds + k * LD + mn) = r[i];
+        }
+    }
+
     __device__ __forceinline__ void store(float* __restrict__ lds) const {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int f = threadIdx.x + i * kGemmThreads;
+            int mn, k;
+            coords(i, mn, k);
             if (KMAJOR) {
-                const int mn = f / (BK / 4), k = (f % (BK / 4)) * 4;
                 lds[(k + 0) * LD + mn] = r[i].x;
                 lds[(k + 1) * LD + mn] = r[i].y;
                 lds[(k + 2) * LD + mn] = r[i].z;
                 lds[(k + 3) * LD + mn] = r[i].w;
             } else {
-                const int k = f / (BMN / 4), mn = (f % (BMN / 4)) * 4;
-                *reinterpret_cast<float4*>(lds + k * LD + mn) = r[i];
+                *reinterpret_cast<floatx4*>(lds + k * LD + mn) = r[i];
             }
         }
     }
@@ -160,43 +198,71 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+    const size_t KT = (g.K + BK - 1) / BK;
+    constexpr int NP = BK / 2;   // k-pairs (one MFMA step each) per tile
+    constexpr int NM = TM * TN;  // MFMAs per k-pair
+    constexpr int NW = TA::NW + TB::NW;
+    constexpr int WPM = (NW + NM - 1) / NM;  // LDS writes placed in front of each MFMA of the last pair
+
+    // A wave issues in order and one fp32 MFMA keeps the matrix pipe busy for 64 cycles, so whatever has to
+    // overlap with it must sit between MFMAs in the instruction stream.  The schedule is written out by hand
+    // and pinned with sched_barrier (left alone, the scheduler sinks every load next to its use and exposes
+    // the LDS and L2 latencies):
+    //   tile start : read the fragments of pair 0, issue the global loads of the next tile
+    //   pair p     : read the fragments of pair p+1 (second register set), then the MFMAs of pair p
+    //   last pair  : the LDS writes of the next tile are dealt out in front of its MFMAs
+    float fa[2][TM], fb[2][TN];
+    auto read_frag = [&](int set, const float* As, const float* Bs, int kk) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[set][i] = As[(kk + lk) * TA::LD + wm0 + i * 32 + l32];
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[set][j] = Bs[(kk + lk) * TB::LD + wn0 + j * 32 + l32];
+    };
     TA ta;
     TB tb;
-    const size_t KT = (g.K + BK - 1) / BK;
+    auto tile_step = [&](size_t kt, auto more_tag) {
+        constexpr bool MORE = decltype(more_tag)::value;
+        const int cur = (int)(kt & 1);
+        const float* As = As0 + cur * A_ELEMS;
+        const float* Bs = Bs0 + cur * B_ELEMS;
+        float* As_next = As0 + (cur ^ 1) * A_ELEMS;
+        float* Bs_next = Bs0 + (cur ^ 1) * B_ELEMS;
+        read_frag(0, As, Bs, 0);
+        if (MORE) {
+            ta.template load<SAFE>(A, g.lda, m0, (kt + 1) * BK, g.M, g.K, g.a_vec != 0);
+            tb.template load<SAFE>(B, g.ldb, n0, (kt + 1) * BK, g.N, g.K, g.b_vec != 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            if (p + 1 < NP) read_frag((p + 1) & 1, As, Bs, 2 * (p + 1));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < NM; q++) {
+                if (MORE && p == NP - 1) {
+#pragma unroll
+                    for (int w = q * WPM; w < (q + 1) * WPM && w < NW; w++) {
+                        if (w < TA::NW) ta.store_op(As_next, w);
+                        else tb.store_op(Bs_next, w - TA::NW);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                const int i = q / TN, j = q % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[p & 1][i], fb[p & 1][j], acc[i][j], 0, 0, 0);
+                if (MORE && p == NP - 1) __builtin_amdgcn_sched_barrier(0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    };
+
     ta.template load<SAFE>(A, g.lda, m0, 0, g.M, g.K, g.a_vec != 0);
     tb.template load<SAFE>(B, g.ldb, n0, 0, g.N, g.K, g.b_vec != 0);
     ta.store(As0);
     tb.store(Bs0);
     __syncthreads();
-
-    for (size_t kt = 0; kt < KT; kt++) {
-        const int cur = (int)(kt & 1);
-        const float* As = As0 + cur * A_ELEMS;
-        const float* Bs = Bs0 + cur * B_ELEMS;
-        const bool more = kt + 1 < KT;
-        if (more) {
-            ta.template load<SAFE>(A, g.lda, m0, (kt + 1) * BK, g.M, g.K, g.a_vec != 0);
-            tb.template load<SAFE>(B, g.ldb, n0, (kt + 1) * BK, g.N, g.K, g.b_vec != 0);
-        }
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float a[TM], b[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++) a[i] = As[(kk + lk) * TA::LD + wm0 + i * 32 + l32];
-#pragma unroll
-            for (int j = 0; j < TN; j++) b[j] = Bs[(kk + lk) * TB::LD + wn0 + j * 32 + l32];
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-        if (more) {
-            ta.store(As0 + (cur ^ 1) * A_ELEMS);
-            tb.store(Bs0 + (cur ^ 1) * B_ELEMS);
-        }
-        __syncthreads();
-    }
+    for (size_t kt = 0; kt + 1 < KT; kt++) tile_step(kt, std::true_type{});
+    tile_step(KT - 1, std::false_type{});
 
     // epilogue: accumulator register r of lane l holds C[(r/4)*8 + (l/32)*4 + r%4][l%32] of its 32x32 block
     const float alpha = g.alpha, beta = g.beta;

@@ -56,3 +56,48 @@ def test_no_device_allocation_in_steady_state(hip):
     for _ in range(20):
         tr.step()
     assert hip.cache_stats()["n_device_allocs"] == n0
+
+
+def test_gcn_steps_match_oracle(oracle, hip):
+    """Config 3 at its real size: 2708 nodes, 1433 features, 13264 edges, 140 labelled nodes, Adam."""
+    from zigrad_amd.trainers import GCNTrainer, gcn_inputs
+
+    inp = gcn_inputs(seed=0)
+    runs = {}
+    for name, dev in (("oracle", oracle), ("hip", hip)):
+        tr = GCNTrainer(dev, inp, lr=0.01, clip=True)
+        losses = [tr.step(keep_grads=(s == 0)) for s in range(5)]
+        dev.sync()
+        runs[name] = (losses, tr.last_grads, [dev.to_numpy(p) for p in tr.param_buffers()])
+    (lo, go, po), (lh, gh, ph) = runs["oracle"], runs["hip"]
+    for a, b in zip(lo, lh):
+        assert abs(a - b) <= STEP_TOL * max(1.0, abs(a)), (lo, lh)
+    for a, b in zip(go, gh):
+        assert rel_fro(b, a) <= STEP_TOL
+    for a, b in zip(po, ph):
+        assert rel_fro(b, a) <= STEP_TOL
+    assert lh[-1] < lh[0]
+
+
+def test_dqn_steps_match_oracle(oracle, hip):
+    """Config 4: 4 -> 128 -> 128 -> 2, batch 64, frozen target network, gather, smooth-L1, Adam lr 1e-3."""
+    from zigrad_amd.trainers import DQNTrainer, dqn_inputs
+
+    dims, batch = [4, 128, 128, 2], 64
+    params, _, _, _ = mlp_inputs(dims, batch)
+    b = dqn_inputs(batch=batch)
+    runs = {}
+    for name, dev in (("oracle", oracle), ("hip", hip)):
+        tr = DQNTrainer(dev, dims, batch, lr=1e-3, gamma=0.99, clip=True)
+        tr.load_params(params)
+        tr.set_batch(b)
+        losses = [tr.step(keep_grads=(s == 0)) for s in range(10)]
+        dev.sync()
+        runs[name] = (losses, tr.last_grads, [dev.to_numpy(p) for p in tr.param_buffers()])
+    (lo, go, po), (lh, gh, ph) = runs["oracle"], runs["hip"]
+    for a, b2 in zip(lo, lh):
+        assert abs(a - b2) <= STEP_TOL * max(1.0, abs(a)), (lo, lh)
+    for a, b2 in zip(go, gh):
+        assert rel_fro(b2, a) <= STEP_TOL
+    for a, b2 in zip(po, ph):
+        assert rel_fro(b2, a) <= STEP_TOL

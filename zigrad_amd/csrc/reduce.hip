@@ -218,8 +218,18 @@ __global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::
     size_t o = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (o >= n_out) return;
     const size_t outer = o / inner, c = o % inner;
-    typename P::Acc acc = partials[(outer * chunks) * inner + c];
-    for (int k = 1; k < chunks; k++) acc = P::combine(acc, partials[(outer * chunks + k) * inner + c]);
+    const typename P::Acc* pp = partials + (outer * chunks) * inner + c;
+    typename P::Acc acc = pp[0];
+    int k = 1;
+    // loads of eight chunks in flight, combined in chunk order
+    for (; k + 8 <= chunks; k += 8) {
+        typename P::Acc t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) t[u] = pp[(size_t)(k + u) * inner];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc = P::combine(acc, t[u]);
+    }
+    for (; k < chunks; k++) acc = P::combine(acc, pp[(size_t)k * inner]);
     A::store(y, o, acc, alpha, beta);
 }
 
@@ -245,7 +255,8 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     const int V = v4 ? 4 : 1;
     const size_t colv = inner / V;
     int log2_cx = 0;
-    while ((1u << log2_cx) < colv && log2_cx < 8) log2_cx++;
+    // at most 64 column threads (1 KiB of a row per workgroup with V = 4): more workgroups, fewer partials
+    while ((1u << log2_cx) < colv && log2_cx < 6) log2_cx++;
     const int cx = 1 << log2_cx, ry = kBlock >> log2_cx;
     const size_t gx = ceil_div_sz(colv, cx);
     // row chunks: enough workgroups to cover the machine several times, but at least 4 trips of ry rows each
@@ -254,7 +265,7 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     size_t max_chunks = ceil_div_sz(R, (size_t)ry * 4);
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks < 1) chunks = 1;
-    if (chunks > 1024) chunks = 1024;
+    if (chunks > 64) chunks = 64;  // keeps the partials buffer and the serial tail of the final stage small
     const size_t rows_per_chunk = ceil_div_sz(R, chunks);
     chunks = ceil_div_sz(R, rows_per_chunk);
     ZG_REQUIRE(outer <= 65535, "axis reduction: %zu leading slices exceed the grid limit", outer);

@@ -111,24 +111,28 @@ def unbroadcast_(dev, x: DevBuf, x_shape, out: DevBuf, out_shape, alpha=1.0, bet
     dev.dispatch("unbroadcast", x=x, x_shape=x_shape, y=out, y_shape=out_shape, scratch=scratch, alpha=alpha, beta=beta)
 
 
-def gather(dev, src: DevBuf, src_shape, indices: DevBuf, idx_shape, dim: int, return_offsets: bool = False):
+def gather(dev, src: DevBuf, src_shape, indices: DevBuf, idx_shape, dim: int, return_offsets: bool = False,
+           check: bool = True):
     """values[i] = src[coord(i) with coord[dim] := indices[i]].  Reference: NDArray.gather,
-    src/ndarray.zig:593-633; the offsets are computed by a device op instead of a host loop."""
+    src/ndarray.zig:593-633; the offsets are computed by a device op instead of a host loop.  `check` reads the
+    out-of-bounds status back (one blocking 4-byte copy); without it out-of-range indices are skipped silently."""
     src_shape, idx_shape = list(src_shape), list(idx_shape)
     if len(src_shape) != len(idx_shape):
         raise ValueError("gather: rank mismatch")
     n = _prod(idx_shape)
-    offsets = dev.mem_alloc(U64, n)
-    status = dev.gather_offsets(src_shape, idx_shape, indices, dim, offsets)
+    # the reference takes the offsets from the raw allocator (its own "TODO: cache?"); on a GPU that would be a
+    # hipMalloc/hipFree pair per call, so they come from the caching allocator (free with mem_cache_free)
+    offsets = dev.mem_cache_alloc(U64, n)
+    status = dev.gather_offsets(src_shape, idx_shape, indices, dim, offsets, check=check)
     if status == 1:
-        dev.mem_free(offsets)
+        dev.mem_cache_free(offsets)
         raise ValueError("InvalidIndexShape")
     if status == 2:
-        dev.mem_free(offsets)
+        dev.mem_cache_free(offsets)
         raise IndexError("IndexOutOfBounds")
     values = dev.mem_cache_alloc(F32, n)
     dev.mem_take(src, offsets, values)
     if return_offsets:
         return values, offsets
-    dev.mem_free(offsets)
+    dev.mem_cache_free(offsets)
     return values, None

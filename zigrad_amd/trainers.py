@@ -81,18 +81,14 @@ class Optimizer:
                            epsilon=self.epsilon, clip=self.clip, max_norm=self.max_norm, delta=self.delta)
 
 
-class MLPTrainer:
-    """Linear -> ReLU -> ... -> Linear -> softmax cross-entropy, one train step per `step()` call.
+class MLP:
+    """Parameters, gradients and the forward/backward op sequences of a ReLU multi-layer perceptron whose
+    Linear layers follow examples/mnist/src/model.zig:64-110 (weights [out, in], forward x . W^T + bias)."""
 
-    loss_mode "onehot" is the reference's loss (float one-hot targets, probabilities kept for backward);
-    "label" is the fused integer-label form (same values, one pass over the logits).
-    """
-
-    def __init__(self, dev, dims, batch, optimizer="sgd", lr=0.01, clip=True, loss_mode="onehot"):
-        self.dev, self.dims, self.batch, self.loss_mode = dev, list(dims), batch, loss_mode
+    def __init__(self, dev, dims, optim: Optimizer | None = None):
+        self.dev, self.dims = dev, list(dims)
         self.n_layers = len(dims) - 1
         self.W, self.b, self.Wg, self.bg = [], [], [], []
-        self.optim = Optimizer(dev, optimizer, lr, clip)
         for fan_in, fan_out in zip(dims[:-1], dims[1:]):
             w, wg = dev.mem_alloc(F32, fan_in * fan_out), dev.mem_alloc(F32, fan_in * fan_out)
             b, bg = dev.mem_alloc(F32, fan_out), dev.mem_alloc(F32, fan_out)
@@ -102,31 +98,95 @@ class MLPTrainer:
             self.b.append(b)
             self.Wg.append(wg)
             self.bg.append(bg)
-            self.optim.attach(w, wg)  # attach order of LinearLayer.init: weights, then bias
-            self.optim.attach(b, bg)
+            if optim is not None:
+                optim.attach(w, wg)  # attach order of LinearLayer.init: weights, then bias
+                optim.attach(b, bg)
+
+    def load_params(self, params) -> None:
+        for l in range(self.n_layers):
+            self.dev.mem_transfer(params[2 * l], self.W[l], "HtoD")
+            self.dev.mem_transfer(params[2 * l + 1], self.b[l], "HtoD")
+
+    def copy_params_from(self, other: "MLP") -> None:
+        for l in range(self.n_layers):
+            self.dev.mem_copy(other.W[l], self.W[l])
+            self.dev.mem_copy(other.b[l], self.b[l])
+
+    def param_buffers(self):
+        return [buf for l in range(self.n_layers) for buf in (self.W[l], self.b[l])]
+
+    def grad_buffers(self):
+        return [buf for l in range(self.n_layers) for buf in (self.Wg[l], self.bg[l])]
+
+    def zero_grad(self) -> None:
+        for gb in self.grad_buffers():
+            self.dev.mem_fill(gb, 0.0)
+
+    def forward(self, x: DevBuf, batch: int):
+        """Returns the activations [x, y_1, ..., y_L]; y_l are cache allocations owned by the caller."""
+        d = self.dev
+        acts = [x]
+        for l in range(self.n_layers):
+            fan_in, fan_out = self.dims[l], self.dims[l + 1]
+            y = d.mem_cache_alloc(F32, batch * fan_out)
+            host.bmm_acc_(d, acts[-1], [batch, fan_in], self.W[l], [fan_out, fan_in], y, trans_a=False, trans_b=True)
+            d.dispatch("add", x=self.b[l], y=y, z=y)  # bias.add_(y): shorter operand first
+            if l + 1 < self.n_layers:
+                d.dispatch("relu_fwd", x=y, y=y)
+            acts.append(y)
+        return acts
+
+    def free_activations(self, acts) -> None:
+        for y in acts[1:]:
+            self.dev.mem_cache_free(y)
+
+    def backward(self, acts, g: DevBuf, batch: int) -> None:
+        """g is the gradient of the last activation (a cache allocation; consumed).  Every activation and
+        intermediate gradient goes back to the allocator as soon as its backward ran (eager teardown)."""
+        d = self.dev
+        for l in reversed(range(self.n_layers)):
+            fan_in, fan_out = self.dims[l], self.dims[l + 1]
+            y = acts[l + 1]
+            if l + 1 < self.n_layers:
+                d.dispatch("relu_inplace_bwd", x=y, x_g=g)
+            host.unbroadcast_(d, g, [batch, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
+            g_prev = None
+            if l > 0:  # the network input does not require a gradient
+                g_prev = d.mem_cache_alloc(F32, batch * fan_in)
+                d.mem_fill(g_prev, 0.0)
+            host.bmm_acc_backward(d, False, True, acts[l], [batch, fan_in], self.W[l], [fan_out, fan_in], g,
+                                  [batch, fan_out], g_prev, self.Wg[l])
+            d.mem_cache_free(y)
+            d.mem_cache_free(g)
+            g = g_prev
+
+
+class MLPTrainer:
+    """Linear -> ReLU -> ... -> Linear -> softmax cross-entropy, one train step per `step()` call.
+
+    loss_mode "onehot" is the reference's loss (float one-hot targets, probabilities kept for backward);
+    "label" is the fused integer-label form (same values, one pass over the logits).
+    """
+
+    def __init__(self, dev, dims, batch, optimizer="sgd", lr=0.01, clip=True, loss_mode="onehot"):
+        self.dev, self.dims, self.batch, self.loss_mode = dev, list(dims), batch, loss_mode
+        self.optim = Optimizer(dev, optimizer, lr, clip)
+        self.net = MLP(dev, dims, self.optim)
+        self.n_layers = self.net.n_layers
         self.x = dev.mem_alloc(F32, batch * dims[0])
         self.onehot = dev.mem_alloc(F32, batch * dims[-1])
         self.labels = dev.mem_alloc(U64, batch)
         self.loss_host = np.zeros(1, np.float32)
         self.last_grads = None
 
-    # -- data ----------------------------------------------------------------------------------
     def load_params(self, params) -> None:
-        for l in range(self.n_layers):
-            self.dev.mem_transfer(params[2 * l], self.W[l], "HtoD")
-            self.dev.mem_transfer(params[2 * l + 1], self.b[l], "HtoD")
+        self.net.load_params(params)
 
     def param_buffers(self):
-        out = []
-        for l in range(self.n_layers):
-            out += [self.W[l], self.b[l]]
-        return out
+        return self.net.param_buffers()
 
     def grad_buffers(self):
-        out = []
-        for l in range(self.n_layers):
-            out += [self.Wg[l], self.bg[l]]
-        return out
+        return self.net.grad_buffers()
 
     def set_batch(self, x, onehot, labels=None) -> None:
         self.dev.mem_transfer(x, self.x, "HtoD")
@@ -135,23 +195,9 @@ class MLPTrainer:
             labels = np.argmax(onehot, axis=1).astype(np.uint64)
         self.dev.mem_transfer(labels, self.labels, "HtoD")
 
-    # -- one step --------------------------------------------------------------------------------
-    def forward(self):
-        d, B = self.dev, self.batch
-        acts = [self.x]
-        for l in range(self.n_layers):
-            fan_in, fan_out = self.dims[l], self.dims[l + 1]
-            y = d.mem_cache_alloc(F32, B * fan_out)
-            host.bmm_acc_(d, acts[-1], [B, fan_in], self.W[l], [fan_out, fan_in], y, trans_a=False, trans_b=True)
-            d.dispatch("add", x=self.b[l], y=y, z=y)  # bias.add_(y): shorter operand first
-            if l + 1 < self.n_layers:
-                d.dispatch("relu_fwd", x=y, y=y)
-            acts.append(y)
-        return acts
-
     def step(self, read_loss: bool = True, keep_grads: bool = False):
         d, B, C = self.dev, self.batch, self.dims[-1]
-        acts = self.forward()
+        acts = self.net.forward(self.x, B)
         logits = acts[-1]
         loss = d.mem_cache_alloc(F32, 1)
         if self.loss_mode == "onehot":
@@ -177,24 +223,244 @@ class MLPTrainer:
         d.mem_cache_free(saved)
         d.mem_cache_free(loss_grad)
         d.mem_cache_free(loss)
-        for l in reversed(range(self.n_layers)):
-            fan_in, fan_out = self.dims[l], self.dims[l + 1]
-            y = acts[l + 1]
-            if l + 1 < self.n_layers:
-                d.dispatch("relu_inplace_bwd", x=y, x_g=g)
-            host.unbroadcast_(d, g, [B, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
-            g_prev = None
-            if l > 0:  # the network input does not require a gradient
-                g_prev = d.mem_cache_alloc(F32, B * fan_in)
-                d.mem_fill(g_prev, 0.0)
-            host.bmm_acc_backward(d, False, True, acts[l], [B, fan_in], self.W[l], [fan_out, fan_in], g, [B, fan_out],
-                                  g_prev, self.Wg[l])
-            d.mem_cache_free(y)
-            d.mem_cache_free(g)
-            g = g_prev
+        self.net.backward(acts, g, B)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
         self.optim.step()
-        for gb in self.grad_buffers():  # model.zero_grad()
-            d.mem_fill(gb, 0.0)
+        self.net.zero_grad()  # model.zero_grad()
         return loss_val
+
+
+def dqn_inputs(batch=64, state_dim=4, n_actions=2, seed=0):
+    """Synthetic replay batch: states / next states N(0,1), actions uniform, rewards U[0,1), done = 0."""
+    r = np.random.default_rng(seed)
+    return {
+        "states": r.standard_normal((batch, state_dim), dtype=np.float32),
+        "next_states": r.standard_normal((batch, state_dim), dtype=np.float32),
+        "actions": r.integers(0, n_actions, (batch, 1)).astype(np.uint64),
+        "rewards": r.random(batch, dtype=np.float32),
+        "dones": np.zeros(batch, np.float32),
+    }
+
+
+class DQNTrainer:
+    """One DQN update per `step()`: TD target from a frozen copy of the network, Q(s,a) through gather,
+    smooth-L1 loss, Adam.  Op order follows DQNAgent.train (examples/dqn/src/dqn_agent.zig:125-228) without
+    its host-side clamps, on the network 4 -> 128 -> 128 -> 2."""
+
+    def __init__(self, dev, dims=(4, 128, 128, 2), batch=64, lr=1e-3, gamma=0.99, clip=True):
+        self.dev, self.dims, self.batch, self.gamma = dev, list(dims), batch, gamma
+        self.optim = Optimizer(dev, "adam", lr, clip)
+        self.policy = MLP(dev, dims, self.optim)
+        self.target = MLP(dev, dims, None)
+        B, S, A = batch, dims[0], dims[-1]
+        self.states, self.next_states = dev.mem_alloc(F32, B * S), dev.mem_alloc(F32, B * S)
+        self.actions = dev.mem_alloc(U64, B)
+        self.rewards, self.dones = dev.mem_alloc(F32, B), dev.mem_alloc(F32, B)
+        self.gamma_t = dev.from_numpy(np.asarray([gamma], np.float32))
+        self.one_t = dev.from_numpy(np.asarray([1.0], np.float32))
+        self.loss_host = np.zeros(1, np.float32)
+        self.last_grads = None
+
+    def load_params(self, params) -> None:
+        self.policy.load_params(params)
+        self.target.copy_params_from(self.policy)
+
+    def set_batch(self, b) -> None:
+        d = self.dev
+        d.mem_transfer(b["states"], self.states, "HtoD")
+        d.mem_transfer(b["next_states"], self.next_states, "HtoD")
+        d.mem_transfer(b["actions"].ravel(), self.actions, "HtoD")
+        d.mem_transfer(b["rewards"], self.rewards, "HtoD")
+        d.mem_transfer(b["dones"], self.dones, "HtoD")
+
+    def param_buffers(self):
+        return self.policy.param_buffers()
+
+    def step(self, keep_grads: bool = False) -> float:
+        d, B, A = self.dev, self.batch, self.dims[-1]
+        # TD target, no gradient
+        acts_t = self.target.forward(self.next_states, B)
+        max_next = d.mem_cache_alloc(F32, B)
+        d.mem_fill(max_next, 0.0)  # NDArray.max_along writes into a zero-filled output (src/ndarray.zig:567)
+        d.dispatch("max_along", x=acts_t[-1], x_shape=[B, A], y=max_next, y_shape=[B], dim=1)
+        self.target.free_activations(acts_t)
+        disc = d.mem_cache_alloc(F32, B)
+        d.dispatch("mul", x=max_next, y=self.gamma_t, z=disc)
+        not_done = d.mem_cache_alloc(F32, B)
+        d.dispatch("sub", x=self.one_t, y=self.dones, z=not_done)
+        masked = d.mem_cache_alloc(F32, B)
+        d.dispatch("mul", x=disc, y=not_done, z=masked)
+        targets = d.mem_cache_alloc(F32, B)
+        d.dispatch("add", x=self.rewards, y=masked, z=targets)
+        for t in (max_next, disc, not_done, masked):
+            d.mem_cache_free(t)
+        # Q(s, a)
+        acts = self.policy.forward(self.states, B)
+        q_all = acts[-1]
+        q, offsets = host.gather(d, q_all, [B, A], self.actions, [B, 1], 1, return_offsets=True, check=False)
+        loss = d.mem_cache_alloc(F32, 1)
+        d.dispatch("smooth_l1_fwd", pred=q, target=targets, beta=1.0, loss=loss)
+        self.policy.zero_grad()
+        # backward
+        loss_grad = d.mem_cache_alloc(F32, 1)
+        d.mem_fill(loss_grad, 1.0)
+        g_q = d.mem_cache_alloc(F32, B)
+        d.mem_fill(g_q, 0.0)
+        d.dispatch("smooth_l1_bwd", pred=q, target=targets, grad=g_q, beta=1.0)
+        g_all = d.mem_cache_alloc(F32, B * A)
+        d.mem_fill(g_all, 0.0)
+        d.dispatch("scatter_add", src=g_q, offsets=offsets, dst=g_all)  # GatherBwd, src/ndtensor.zig:1367-1380
+        d.mem_cache_free(offsets)
+        for t in (g_q, loss_grad, q, targets):
+            d.mem_cache_free(t)
+        self.policy.backward(acts, g_all, B)
+        if keep_grads:
+            self.last_grads = [d.to_numpy(b) for b in self.policy.grad_buffers()]
+        self.optim.step()
+        d.mem_transfer(loss, self.loss_host, "DtoH")
+        d.mem_cache_free(loss)
+        return float(self.loss_host[0])
+
+
+def gcn_inputs(n_nodes=2708, n_features=1433, n_pairs=5278, n_classes=7, n_train=140, hidden=16, seed=0):
+    """Synthetic Cora-shaped graph: Bernoulli(0.0127) features, symmetrised uniform random pairs plus self
+    loops in [2, E] layout (source row, then target row), uniform labels, the first n_train nodes labelled."""
+    r = np.random.default_rng(seed)
+    x = (r.random((n_nodes, n_features)) < 0.0127).astype(np.float32)
+    u, v = r.integers(0, n_nodes, n_pairs), r.integers(0, n_nodes, n_pairs)
+    loops = np.arange(n_nodes)
+    src = np.concatenate([u, v, loops]).astype(np.uint64)
+    tgt = np.concatenate([v, u, loops]).astype(np.uint64)
+    labels = r.integers(0, n_classes, n_nodes)
+    onehot = np.zeros((n_nodes, n_classes), np.float32)
+    onehot[np.arange(n_nodes), labels] = 1.0
+    params = []
+    for fan_in, fan_out in ((n_features, hidden), (hidden, n_classes)):
+        params.append((r.standard_normal((fan_out, fan_in)) * np.sqrt(2.0 / fan_in)).astype(np.float32))
+        params.append(np.zeros(fan_out, np.float32))
+    return {"x": x, "src": src, "tgt": tgt, "onehot": onehot, "n_train": n_train, "params": params,
+            "dims": [n_features, hidden, n_classes]}
+
+
+class GCNTrainer:
+    """Two GraphConv layers (GEMM, degree-scaled scatter, bias) with ReLU between, masked softmax
+    cross-entropy, Adam: the op sequence of examples/gcn/src/model.zig:27-36, 100-224 and main.zig:68-84.
+    The labelled nodes are the first `n_train` rows (MaskLayer.backward indexes the masked gradient by node
+    id, examples/gcn/src/model.zig:343-348, which is only meaningful for a prefix mask)."""
+
+    EPS = 1e-12  # Settings.eps, src/zigrad.zig:72
+
+    def __init__(self, dev, inp, lr=0.01, clip=True):
+        d = self.dev = dev
+        self.N = inp["x"].shape[0]
+        self.dims = inp["dims"]
+        self.E = inp["src"].size
+        self.n_train = inp["n_train"]
+        self.optim = Optimizer(dev, "adam", lr, clip)
+        self.W, self.b, self.Wg, self.bg = [], [], [], []
+        for fan_in, fan_out in zip(self.dims[:-1], self.dims[1:]):
+            w, wg = d.mem_alloc(F32, fan_in * fan_out), d.mem_alloc(F32, fan_in * fan_out)
+            b, bg = d.mem_alloc(F32, fan_out), d.mem_alloc(F32, fan_out)
+            for g in (wg, bg):
+                d.mem_fill(g, 0.0)
+            self.W.append(w); self.b.append(b); self.Wg.append(wg); self.bg.append(bg)
+            self.optim.attach(w, wg)
+            self.optim.attach(b, bg)
+        for l in range(2):
+            d.mem_transfer(inp["params"][2 * l], self.W[l], "HtoD")
+            d.mem_transfer(inp["params"][2 * l + 1], self.b[l], "HtoD")
+        self.x = d.from_numpy(inp["x"])
+        # the edge list lives where the host can write it and the kernels can read it
+        self.edge_index = d.mem_alloc_host(U64, 2 * self.E)
+        d.mem_transfer(np.concatenate([inp["src"], inp["tgt"]]), self.edge_index, "HtoD")
+        self.src, self.tgt = self.edge_index.sub(0, self.E), self.edge_index.sub(self.E, self.E)
+        self.label_m = d.from_numpy(inp["onehot"][: self.n_train])
+        self.loss_host = np.zeros(1, np.float32)
+        self.last_grads = None
+
+    def param_buffers(self):
+        return [self.W[0], self.b[0], self.W[1], self.b[1]]
+
+    def grad_buffers(self):
+        return [self.Wg[0], self.bg[0], self.Wg[1], self.bg[1]]
+
+    def _conv_forward(self, l, x_in):
+        d, N, E = self.dev, self.N, self.E
+        fan_in, fan_out = self.dims[l], self.dims[l + 1]
+        h = d.mem_cache_alloc(F32, N * fan_out)
+        host.bmm_acc_(d, x_in, [N, fan_in], self.W[l], [fan_out, fan_in], h, trans_a=False, trans_b=True)
+        deg = d.mem_cache_alloc(F32, N)
+        d.mem_fill(deg, 1.0)
+        ones_edges = d.mem_cache_alloc(F32, E)
+        d.mem_fill(ones_edges, 1.0)
+        contrib = d.mem_cache_alloc(F32, N)
+        d.mem_fill(contrib, 0.0)
+        d.dispatch("scatter_add", src=ones_edges, offsets=self.tgt, dst=contrib)
+        d.mem_cache_free(ones_edges)
+        d.dispatch("add", x=contrib, y=deg, z=deg)  # deg._add(deg_contrib)
+        d.mem_cache_free(contrib)
+        deg_norm = d.mem_cache_alloc(F32, N)
+        d.dispatch("rsqrt_fwd", x=deg, y=deg_norm, eps=self.EPS)
+        d.mem_cache_free(deg)
+        y = d.mem_cache_alloc(F32, N * fan_out)
+        d.mem_fill(y, 0.0)
+        d.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg_norm, src_indices=self.src, tgt_indices=self.tgt,
+                   stride=fan_out, n_edge=E)
+        d.dispatch("add", x=self.b[l], y=y, z=y)  # y._add(bias)
+        return {"x": x_in, "h": h, "deg": deg_norm, "y": y}
+
+    def _conv_backward(self, l, saved, g_y, need_input_grad):
+        d, N, E = self.dev, self.N, self.E
+        fan_in, fan_out = self.dims[l], self.dims[l + 1]
+        host.unbroadcast_(d, g_y, [N, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
+        g_h = d.mem_cache_alloc(F32, N * fan_out)
+        d.mem_fill(g_h, 0.0)
+        g_deg = d.mem_cache_alloc(F32, N)
+        d.mem_fill(g_deg, 0.0)
+        d.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=g_y, h=saved["h"], deg=saved["deg"], src_indices=self.src,
+                   tgt_indices=self.tgt, grad_h=g_h, grad_deg=g_deg, stride=fan_out, n_edge=E)
+        d.mem_cache_free(g_y)
+        d.mem_cache_free(saved["y"])
+        d.mem_cache_free(g_deg)  # deg itself needs no gradient: the chain stops at rsqrt (src/ndtensor.zig:1009)
+        d.mem_cache_free(saved["deg"])
+        g_x = None
+        if need_input_grad:
+            g_x = d.mem_cache_alloc(F32, N * fan_in)
+            d.mem_fill(g_x, 0.0)
+        host.bmm_acc_backward(d, False, True, saved["x"], [N, fan_in], self.W[l], [fan_out, fan_in], g_h, [N, fan_out],
+                              g_x, self.Wg[l])
+        d.mem_cache_free(g_h)
+        d.mem_cache_free(saved["h"])
+        return g_x
+
+    def step(self, keep_grads: bool = False) -> float:
+        d, N, C, M = self.dev, self.N, self.dims[-1], self.n_train
+        s1 = self._conv_forward(0, self.x)
+        d.dispatch("relu_fwd", x=s1["y"], y=s1["y"])
+        s2 = self._conv_forward(1, s1["y"])
+        out_m = d.mem_cache_alloc(F32, M * C)  # MaskLayer.forward: the labelled rows, here one contiguous prefix
+        d.mem_copy(s2["y"].sub(0, M * C), out_m)
+        probs, loss = d.mem_cache_alloc(F32, M * C), d.mem_cache_alloc(F32, 1)
+        d.dispatch("smce_fwd", logits=out_m, target=self.label_m, probs=probs, loss=loss, rows=M, cols=C)
+        d.mem_transfer(loss, self.loss_host, "DtoH")
+        # backward
+        loss_grad = d.mem_cache_alloc(F32, 1)
+        d.mem_fill(loss_grad, 1.0)
+        g_m = d.mem_cache_alloc(F32, M * C)
+        d.mem_fill(g_m, 0.0)
+        d.dispatch("smce_bwd", probs=probs, target=self.label_m, grad=g_m, rows=M, cols=C)
+        g2 = d.mem_cache_alloc(F32, N * C)
+        d.mem_fill(g2, 0.0)
+        d.mem_copy(g_m, g2.sub(0, M * C))  # MaskLayer.backward
+        for t in (probs, loss, loss_grad, g_m, out_m):
+            d.mem_cache_free(t)
+        g1 = self._conv_backward(1, s2, g2, need_input_grad=True)
+        d.dispatch("relu_inplace_bwd", x=s1["y"], x_g=g1)
+        self._conv_backward(0, s1, g1, need_input_grad=False)
+        if keep_grads:
+            self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
+        self.optim.step()
+        for gb in self.grad_buffers():
+            d.mem_fill(gb, 0.0)
+        return float(self.loss_host[0])

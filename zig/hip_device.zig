@@ -1,0 +1,459 @@
+//! HipDevice: Zigrad's second device, backed by libzg_hip.so (include/zg_hip.h).
+//!
+//! Drop this file into src/device/ next to host_device.zig, add the union field shown in
+//! INTEGRATION.md to enabled_devices.zig, link libzg_hip.so, and every NDArray / NDTensor / Graph / nn
+//! call that goes through DeviceReference.dispatch runs on the MI355X unchanged.
+//!
+//! The struct follows the reference's duck-typed device contract (src/device/device_reference.zig:15-131):
+//! one method per opspec `__name__` with the signature `fn (self, T: type, p: opspec.<name>(T)) void`, the
+//! mem_* API, `reference()`, `sync()`.  Ops cannot return errors in that contract, so a non-zero return
+//! code from the C ABI becomes @panic with the library's message, as the CUDA C layer exits on error
+//! (src/cuda/cuda_helpers.cu:21-28).
+//!
+//! This file cannot be compiled in the build container (no Zig toolchain); it is written against Zig 0.14
+//! and the reference's tree layout and is exercised by the steps in INTEGRATION.md.
+const std = @import("std");
+const c = @cImport(@cInclude("zg_hip.h"));
+const opspec = @import("opspec.zig");
+const RandType = @import("device_common.zig").RandType;
+const TransferDirection = @import("device_common.zig").TransferDirection;
+const CachingAllocator = @import("../allocators.zig").CachingAllocator(DataHandler);
+const DeviceData = @import("../allocators.zig").DeviceData;
+const Error = @import("../allocators.zig").Error;
+const adjust_map_size = @import("../allocators.zig").adjust_map_size;
+
+pub const DeviceReference = @import("device_reference.zig");
+const Self = @This();
+
+fn check(rc: c_int) void {
+    if (rc != 0) std.debug.panic("zg_hip: {s}", .{std.mem.span(c.zg_hip_last_error())});
+}
+
+/// The per-device handler src/allocators/caching_allocator.zig is generic over.
+/// `map` hands the block pool one contiguous device region; `map_alloc` is left out on purpose
+/// (src/allocators/block_pool.zig:115 makes it optional): the region is physically backed when mapped.
+const DataHandler = struct {
+    pub const min_split_size = 256; // bytes; every block is then 256-byte aligned, enough for 128-bit accesses
+
+    ctx: *c.zg_hip_ctx,
+
+    pub fn map(self: DataHandler, size: ?usize) Error![]u8 {
+        var total: usize = 0;
+        check(c.zg_hip_total_memory(self.ctx, &total));
+        // default: a quarter of the device per pool instead of over-subscribing all of it
+        const want = adjust_map_size(size orelse total / 4, self.page_size(), total);
+        var ptr: ?*anyopaque = null;
+        if (c.zg_hip_pool_map(self.ctx, want, &ptr) != 0) return Error.DeviceOOM;
+        const bytes: [*]u8 = @ptrCast(ptr.?);
+        return bytes[0..want];
+    }
+    pub fn unmap(self: DataHandler, buf: []u8) void {
+        check(c.zg_hip_pool_unmap(self.ctx, buf.ptr));
+    }
+    pub fn alloc(self: DataHandler, n: usize) ?[*]u8 {
+        var ptr: ?*anyopaque = null;
+        if (c.zg_hip_alloc(self.ctx, n, &ptr) != 0) return null;
+        return @ptrCast(ptr.?);
+    }
+    pub fn free(self: DataHandler, buf: []u8) void {
+        check(c.zg_hip_free(self.ctx, buf.ptr));
+    }
+    pub fn page_size(self: DataHandler) usize {
+        var n: usize = 0;
+        check(c.zg_hip_page_size(self.ctx, &n));
+        return n;
+    }
+    pub inline fn reset(_: DataHandler) void {}
+    pub fn deinit(self: *DataHandler) void {
+        self.* = undefined;
+    }
+};
+
+ctx: *c.zg_hip_ctx,
+cache: CachingAllocator,
+/// one device float that host-side scalar operands are staged through (see `dev_scalar`)
+scalar_slot: [*]f32,
+
+pub fn device_count() u32 {
+    var n: c_int = 0;
+    check(c.zg_hip_device_count(&n));
+    return @intCast(n);
+}
+
+pub fn init(device_number: u32) Self {
+    return init_advanced(device_number, .{});
+}
+
+pub fn init_advanced(device_number: u32, opts: CachingAllocator.Options) Self {
+    var ctx: ?*c.zg_hip_ctx = null;
+    check(c.zg_hip_init(@intCast(device_number), &ctx));
+    var slot: ?*anyopaque = null;
+    check(c.zg_hip_alloc(ctx.?, 256, &slot));
+    return .{
+        .ctx = ctx.?,
+        .cache = CachingAllocator.init(.{ .ctx = ctx.? }, opts),
+        .scalar_slot = @ptrCast(@alignCast(slot.?)),
+    };
+}
+
+pub fn deinit(self: *Self) void {
+    self.sync();
+    self.cache.deinit();
+    check(c.zg_hip_deinit(self.ctx));
+    self.* = undefined;
+}
+
+pub fn reference(self: *Self) DeviceReference {
+    return .{ .ptrs = .{ .hip = self } };
+}
+
+pub fn is_compatible(self: *const Self, other: *const Self) bool {
+    return self.ctx == other.ctx;
+}
+
+pub fn sync(self: *const Self) void {
+    check(c.zg_hip_sync(self.ctx));
+}
+
+pub fn clear_cache(self: *Self) void {
+    self.cache.clear();
+}
+
+// --------------------------------------------------------------------------------------------------
+// Host-pointer hazards.  Callers that grew up on the host device hand over host memory in three places:
+// the scalar operand of add_scalar & co (src/ndarray.zig:251), axpy's alpha (src/nn/optim.zig:117) and index
+// slices filled by host loops (examples/gcn/src/model.zig:204-205).  Index slices must be allocated with
+// `mem_alloc_indices` (pinned, device-readable); scalars are staged here.
+// --------------------------------------------------------------------------------------------------
+fn is_device_ptr(self: *const Self, p: *const anyopaque) bool {
+    const a = @intFromPtr(p);
+    return self.cache.owns(a); // two contiguous pool mappings: an O(1) range test (src/allocators/block_pool.zig:118)
+}
+
+fn dev_scalar(self: *const Self, T: type, s: []const T) [*]const T {
+    if (s.len != 1 or self.is_device_ptr(s.ptr)) return s.ptr;
+    check(c.zg_hip_memcpy_h2d(self.ctx, self.scalar_slot, s.ptr, @sizeOf(T)));
+    return @ptrCast(self.scalar_slot);
+}
+
+/// usize buffers the host may write and the kernels may read (edge lists, gather indices).
+pub fn mem_alloc_indices(self: *Self, n: usize) ![]usize {
+    var ptr: ?*anyopaque = null;
+    if (c.zg_hip_host_alloc(self.ctx, n * @sizeOf(usize), &ptr) != 0) return Error.DeviceOOM;
+    const p: [*]usize = @ptrCast(@alignCast(ptr.?));
+    return p[0..n];
+}
+
+// --------------------------------------------------------------------------------------------------
+// memory API (src/device/device_reference.zig:29-123)
+// --------------------------------------------------------------------------------------------------
+pub fn mem_cache_alloc(self: *Self, T: type, n: usize) !DeviceData(T) {
+    return self.cache.alloc(T, n);
+}
+pub fn mem_cache_free(self: *Self, data: anytype) void {
+    self.cache.free(data);
+}
+pub fn mem_cache_dupe(self: *Self, T: type, src: []const T) !DeviceData(T) {
+    const dst = try self.cache.alloc(T, src.len);
+    // callers pass host stack values here (src/nn/loss.zig:163), so pick the direction by where src lives
+    if (self.is_device_ptr(src.ptr)) self.mem_copy(T, src, dst.raw) else self.mem_transfer(T, src, dst.raw, .HtoD);
+    return dst;
+}
+pub fn mem_alloc(self: *Self, T: type, n: usize) ![]T {
+    if (n == 0) return &.{};
+    var ptr: ?*anyopaque = null;
+    if (c.zg_hip_alloc(self.ctx, n * @sizeOf(T), &ptr) != 0) return Error.DeviceOOM;
+    const p: [*]T = @ptrCast(@alignCast(ptr.?));
+    return p[0..n];
+}
+pub fn mem_alloc_byte_mask(self: *Self, n: usize) ![]u8 {
+    return self.mem_alloc(u8, @divFloor(n - 1, 8) + 1);
+}
+pub fn mem_free(self: *Self, slice: anytype) void {
+    if (slice.len == 0) return;
+    check(c.zg_hip_free(self.ctx, @constCast(@ptrCast(slice.ptr))));
+}
+pub fn mem_dupe(self: *Self, T: type, src: []const T) ![]T {
+    const dst = try self.mem_alloc(T, src.len);
+    self.mem_copy(T, src, dst);
+    return dst;
+}
+pub fn mem_scratch(self: *Self, T: type, n: usize) []T {
+    return self.cache.alloc_scratch(T, n);
+}
+pub fn mem_fill(self: *const Self, T: type, slice: []T, value: T) void {
+    switch (T) {
+        f32 => check(c.zg_hip_mem_fill(self.ctx, slice.ptr, slice.len, value)),
+        u8 => check(c.zg_hip_mem_fill_u8(self.ctx, slice.ptr, slice.len, value)),
+        usize => check(c.zg_hip_mem_fill_u64(self.ctx, @ptrCast(slice.ptr), slice.len, value)),
+        else => @compileError("HipDevice.mem_fill: unsupported element type " ++ @typeName(T)),
+    }
+}
+pub fn mem_copy(self: *const Self, T: type, src: []const T, dst: []T) void {
+    check(c.zg_hip_memcpy_d2d(self.ctx, dst.ptr, src.ptr, src.len * @sizeOf(T)));
+}
+pub fn mem_transfer(self: *const Self, T: type, src: []const T, dst: []T, dir: TransferDirection) void {
+    const n = src.len * @sizeOf(T);
+    switch (dir) {
+        .HtoD => check(c.zg_hip_memcpy_h2d(self.ctx, dst.ptr, src.ptr, n)),
+        .DtoH => check(c.zg_hip_memcpy_d2h(self.ctx, dst.ptr, src.ptr, n)), // blocks: NDTensor.get reads right after
+        .DtoD => check(c.zg_hip_memcpy_d2d(self.ctx, dst.ptr, src.ptr, n)),
+    }
+}
+pub fn mem_sequence(self: *const Self, T: type, slice: []T, initial: T, step: T) void {
+    comptime std.debug.assert(T == f32);
+    check(c.zg_hip_mem_sequence(self.ctx, slice.ptr, slice.len, initial, step));
+}
+pub fn mem_random(self: *const Self, T: type, slice: []T, op: RandType, rand: std.Random) void {
+    // Generate on the host with the caller's generator, exactly as HostDevice does
+    // (src/device/host_device.zig:931-945), then copy up: bit-identical initial weights on both devices.
+    comptime std.debug.assert(T == f32);
+    const tmp = std.heap.page_allocator.alloc(T, slice.len) catch @panic("mem_random: host OOM");
+    defer std.heap.page_allocator.free(tmp);
+    switch (op) {
+        .uniform => for (tmp) |*e| {
+            e.* = rand.float(T);
+        },
+        .normal => for (tmp) |*e| {
+            e.* = rand.floatNorm(T);
+        },
+        .kaiming => |fan| {
+            const std_dev = @sqrt(2.0 / @as(T, @floatFromInt(fan)));
+            for (tmp) |*e| e.* = rand.floatNorm(T) * std_dev;
+        },
+    }
+    self.mem_transfer(T, tmp, slice, .HtoD);
+}
+pub fn mem_take(self: *const Self, T: type, src: []const T, idxs: []const usize, dst: []T) void {
+    comptime std.debug.assert(T == f32);
+    check(c.zg_hip_mem_take(self.ctx, src.ptr, src.len, @ptrCast(idxs.ptr), idxs.len, dst.ptr));
+}
+
+// --------------------------------------------------------------------------------------------------
+// ops: one method per opspec name.  f32 only; any other T is a compile error at the call site.
+// --------------------------------------------------------------------------------------------------
+fn only_f32(T: type) void {
+    if (T != f32) @compileError("HipDevice implements f32 ops; got " ++ @typeName(T));
+}
+
+pub fn add(self: *const Self, T: type, p: opspec.add(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_add(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+}
+pub fn sub(self: *const Self, T: type, p: opspec.sub(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sub(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+}
+pub fn mul(self: *const Self, T: type, p: opspec.mul(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_mul(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+}
+pub fn div(self: *const Self, T: type, p: opspec.div(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_div(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+}
+pub fn dot(self: *const Self, T: type, p: opspec.dot(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_dot(self.ctx, p.x.ptr, p.y.ptr, p.x.len, p.z.ptr));
+}
+pub fn matvec(self: *const Self, T: type, p: opspec.matvec(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_matvec(self.ctx, p.A.ptr, p.x.ptr, p.y.ptr, p.m, p.n, @intFromBool(p.trans_a), p.alpha, p.beta));
+}
+pub fn matmul(self: *const Self, T: type, p: opspec.matmul(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_matmul(self.ctx, p.A.ptr, p.B.ptr, p.C.ptr, p.m, p.n, p.k, @intFromBool(p.trans_a), @intFromBool(p.trans_b), p.lda, p.ldb, p.ldc, p.alpha, p.beta));
+}
+pub fn bmm_acc(self: *const Self, T: type, p: opspec.bmm_acc(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_bmm_acc(self.ctx, p.A.ptr, @ptrCast(p.A_shape.ptr), p.B.ptr, @ptrCast(p.B_shape.ptr), p.C.ptr, @ptrCast(p.C_shape.ptr), @intFromBool(p.trans_a), @intFromBool(p.trans_b), p.lda, p.ldb, p.ldc, p.alpha, p.beta));
+}
+pub fn outer(self: *const Self, T: type, p: opspec.outer(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_outer(self.ctx, p.x.ptr, p.x.len, p.y.ptr, p.y.len, p.A.ptr, p.alpha));
+}
+pub fn transpose(self: *const Self, T: type, p: opspec.transpose(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_transpose(self.ctx, p.A.ptr, p.B.ptr, p.m, p.n, p.alpha));
+}
+pub fn axpy(self: *const Self, T: type, p: opspec.axpy(T)) void {
+    comptime only_f32(T);
+    const on_device = self.is_device_ptr(p.alpha);
+    check(c.zg_hip_axpy(self.ctx, p.x.ptr, p.y.ptr, p.x.len, p.alpha, @intFromBool(on_device)));
+}
+pub fn sum(self: *const Self, T: type, p: opspec.sum(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sum(self.ctx, p.x.ptr, p.x.len, p.y.ptr));
+}
+pub fn scale(self: *const Self, T: type, p: opspec.scale(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scale(self.ctx, p.x.ptr, p.x.len, p.alpha));
+}
+pub fn nrm2(self: *const Self, T: type, p: opspec.nrm2(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_nrm2(self.ctx, p.x.ptr, p.x.len, p.y.ptr));
+}
+pub fn clip_nrm2(self: *const Self, T: type, p: opspec.clip_nrm2(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_clip_nrm2(self.ctx, p.x.ptr, p.x.len, p.max_norm, p.delta));
+}
+pub fn pow_fwd(self: *const Self, T: type, p: opspec.pow_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_pow_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len, p.exp));
+}
+pub fn pow_fwd_(self: *const Self, T: type, p: opspec.pow_fwd_(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_pow_fwd(self.ctx, p.x.ptr, p.x.ptr, p.x.len, p.exp));
+}
+pub fn pow_bwd(self: *const Self, T: type, p: opspec.pow_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_pow_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.y_g.ptr, p.x.len, p.exp, p.eps));
+}
+pub fn sqrt_fwd(self: *const Self, T: type, p: opspec.sqrt_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sqrt_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len));
+}
+pub fn sqrt_fwd_(self: *const Self, T: type, p: opspec.sqrt_fwd_(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sqrt_fwd(self.ctx, p.x.ptr, p.x.ptr, p.x.len));
+}
+pub fn sqrt_bwd(self: *const Self, T: type, p: opspec.sqrt_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sqrt_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.y_g.ptr, p.x.len, p.eps));
+}
+pub fn rsqrt_fwd(self: *const Self, T: type, p: opspec.rsqrt_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_rsqrt_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len, p.eps));
+}
+pub fn rsqrt_bwd(self: *const Self, T: type, p: opspec.rsqrt_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_rsqrt_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.y_g.ptr, p.x.len, p.eps));
+}
+pub fn exp_fwd(self: *const Self, T: type, p: opspec.exp_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_exp_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len));
+}
+pub fn exp_bwd(self: *const Self, T: type, p: opspec.exp_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_exp_bwd(self.ctx, p.x_g.ptr, p.y.ptr, p.y_g.ptr, p.x_g.len));
+}
+pub fn relu_fwd(self: *const Self, T: type, p: opspec.relu_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_relu_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len));
+}
+pub fn relu_bwd(self: *const Self, T: type, p: opspec.relu_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_relu_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.y_g.ptr, p.x.len));
+}
+pub fn relu_inplace_bwd(self: *const Self, T: type, p: opspec.relu_inplace_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_relu_inplace_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.x.len));
+}
+pub fn tanh_fwd(self: *const Self, T: type, p: opspec.tanh_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_tanh_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len));
+}
+pub fn tanh_bwd(self: *const Self, T: type, p: opspec.tanh_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_tanh_bwd(self.ctx, p.x_g.ptr, p.y.ptr, p.y_g.ptr, p.x_g.len));
+}
+pub fn tanh_inplace_bwd(self: *const Self, T: type, p: opspec.tanh_inplace_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_tanh_inplace_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.x.len));
+}
+pub fn sigm_fwd(self: *const Self, T: type, p: opspec.sigm_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sigm_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len));
+}
+pub fn sigm_bwd(self: *const Self, T: type, p: opspec.sigm_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sigm_bwd(self.ctx, p.x_g.ptr, p.y.ptr, p.y_g.ptr, p.x_g.len));
+}
+pub fn sigm_inplace_bwd(self: *const Self, T: type, p: opspec.sigm_inplace_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sigm_inplace_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.x.len));
+}
+pub fn max_fwd(self: *const Self, T: type, p: opspec.max_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_max_fwd(self.ctx, p.x.ptr, p.x.len, p.y.ptr));
+}
+pub fn max_bwd(self: *const Self, T: type, p: opspec.max_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_max_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.x.len, p.y.ptr, p.y_g.ptr));
+}
+pub fn clamp_fwd(self: *const Self, T: type, p: opspec.clamp_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_clamp_fwd(self.ctx, p.x.ptr, p.y.ptr, p.x.len, p.min, p.max));
+}
+pub fn clamp_bwd(self: *const Self, T: type, p: opspec.clamp_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_clamp_bwd(self.ctx, p.x.ptr, p.x_g.ptr, p.y_g.ptr, p.x.len, p.min, p.max));
+}
+pub fn unbroadcast(self: *Self, T: type, p: opspec.unbroadcast(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_unbroadcast(self.ctx, p.x.ptr, @ptrCast(p.x_shape.ptr), p.x_shape.len, p.y.ptr, @ptrCast(p.y_shape.ptr), p.y_shape.len, p.scratch.ptr, p.scratch.len, p.alpha, p.beta));
+}
+pub fn broadcast(self: *const Self, T: type, p: opspec.broadcast(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_broadcast(self.ctx, p.x.ptr, p.x.len, p.y.ptr, p.y.len, p.alpha, p.beta));
+}
+pub fn sum_along(self: *const Self, T: type, p: opspec.sum_along(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sum_along(self.ctx, p.x.ptr, @ptrCast(p.x_shape.ptr), p.x_shape.len, p.y.ptr, p.y.len, p.dim, p.alpha, p.beta));
+}
+pub fn max_along(self: *const Self, T: type, p: opspec.max_along(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_max_along(self.ctx, p.x.ptr, @ptrCast(p.x_shape.ptr), p.x_shape.len, p.y.ptr, p.y.len, p.dim));
+}
+pub fn scatter_add(self: *const Self, T: type, p: opspec.scatter_add(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_add(self.ctx, p.src.ptr, @ptrCast(p.offsets.ptr), p.src.len, p.dst.ptr, p.dst.len));
+}
+pub fn scatter_gcn_deg_scaled(self: *const Self, T: type, p: opspec.scatter_gcn_deg_scaled(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_gcn_deg_scaled(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, @ptrCast(p.src_indices.ptr), @ptrCast(p.tgt_indices.ptr), p.stride, p.n_edge, p.deg.len));
+}
+pub fn scatter_gcn_deg_scaled_bwd(self: *const Self, T: type, p: opspec.scatter_gcn_deg_scaled_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_gcn_deg_scaled_bwd(self.ctx, p.grad_output.ptr, p.h.ptr, p.deg.ptr, @ptrCast(p.src_indices.ptr), @ptrCast(p.tgt_indices.ptr), p.grad_h.ptr, p.grad_deg.ptr, p.stride, p.n_edge, p.deg.len));
+}
+
+// New op names for what the reference computes with host loops over `.raw` (they need the matching
+// parameter structs added to opspec.zig and the call sites switched to dispatch; see INTEGRATION.md):
+//   smce_fwd / smce_bwd / smce_label_fwd / smce_label_bwd   src/nn/loss.zig:130-215
+//   smooth_l1_fwd / smooth_l1_bwd / mse_fwd / mse_bwd        src/nn/loss.zig:94-127, 259-305
+//   sgd_step / adam_step                                     src/nn/optim.zig:100-122, 177-234
+//   argmax_along, gather_offsets, index_select_fwd / _bwd    examples/mnist/src/main-simple.zig:124, src/ndarray.zig:607-624,
+//                                                            src/ndtensor.zig:1437-1513
+pub fn smce_fwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smce_fwd(self.ctx, p.logits.ptr, p.target.ptr, p.probs.ptr, p.loss.ptr, p.rows, p.cols));
+}
+pub fn smce_bwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smce_bwd(self.ctx, p.probs.ptr, p.target.ptr, p.grad.ptr, p.rows, p.cols));
+}
+pub fn smooth_l1_fwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smooth_l1_fwd(self.ctx, p.pred.ptr, p.target.ptr, p.pred.len, p.beta, p.loss.ptr));
+}
+pub fn smooth_l1_bwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smooth_l1_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len, p.beta));
+}
+pub fn mse_fwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_mse_fwd(self.ctx, p.pred.ptr, p.target.ptr, p.pred.len, p.loss.ptr));
+}
+pub fn mse_bwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_mse_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len));
+}
+pub fn sgd_step(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sgd_step(self.ctx, p.param.ptr, p.grad.ptr, p.param.len, p.lr, @intFromBool(p.clip), p.max_norm, p.delta));
+}
+pub fn adam_step(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_adam_step(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.t, p.lr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
+}

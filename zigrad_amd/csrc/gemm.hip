@@ -6,12 +6,20 @@
 //
 // Kernel shape: a workgroup of 4 waves (2 x 2) owns a BM x BN tile of C.  Each wave owns a
 // (BM/2) x (BN/2) sub-tile as a grid of 32x32 accumulator blocks fed by v_mfma_f32_32x32x2_f32.
-// Operand tiles of BK = 16 along k are staged through LDS in a k-major layout ([k][m] and [k][n]), so
-// a wave's fragment read (32 consecutive m or n for one k) is one conflict-free row segment, whatever
-// the operand's layout in HBM.  LDS is double buffered: the global loads of tile t+1 are in flight
-// while the MFMAs of tile t run, with one barrier per tile.  Workgroup ids are remapped so that the
-// workgroups resident on one XCD (ids congruent modulo 8) cover a compact patch of C and share their
-// A rows / B columns in that XCD's L2.
+// Operand tiles of BK = 16 along k are staged through LDS, double buffered, one barrier per tile.
+//
+// A wave cannot overlap its own non-MFMA instructions with its MFMAs to any useful degree (measured: every
+// LDS or global instruction in the loop costs about its issue time), so the loop is built to need few of them:
+//   * LDS keeps each operand tile in the orientation it has in HBM ([mn][k] for a k-contiguous operand,
+//     [k][mn] otherwise), so a tile moves HBM -> registers -> LDS with 16-byte loads and 16-byte LDS writes only.
+//   * An MFMA sums over two k values, one per lane half, and it does not matter which two as long as A and B
+//     agree.  Lane half h takes k = 8g + 4h + c in step c of k-group g.  A lane of a k-contiguous operand then
+//     reads its 4 steps of one 32-row block with one ds_read_b128; a lane of the other kind reads, per step,
+//     its T consecutive rows (block row b <-> tile rows b*T .. b*T+T-1) with one ds_read_b128 / b64.
+//   * All LDS addresses are a per-thread base plus immediates; global addresses are a scalar base plus a
+//     per-thread 32-bit offset.
+// Workgroup ids are remapped so that the workgroups resident on one XCD (ids congruent modulo 8) cover a
+// compact patch of C and share their A rows / B columns in that XCD's L2.
 #include "common.h"
 
 #include <type_traits>
@@ -21,119 +29,130 @@ namespace zg {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));  // first-class vector: stays in registers
 
-constexpr int BK = 16;
 constexpr int kGemmThreads = 256;
 
-#ifndef ZG_GEMM_MNMAP
-#define ZG_GEMM_MNMAP 0
-#endif
+constexpr int kBK = 16;  // tile depth along k: two k-groups of 8
 
+template <int T>
+struct VecOf;
+template <>
+struct VecOf<1> {
+    typedef float type;
+};
+template <>
+struct VecOf<2> {
+    typedef float type __attribute__((ext_vector_type(2)));
+};
+template <>
+struct VecOf<4> {
+    typedef floatx4 type;
+};
 
-// One operand tile: `BMN` rows in the m (or n) direction by BK along k.
-// KMAJOR: element (mn, k) lives at ptr[mn * ld + k]   (A not transposed, B transposed)
-// else  : element (mn, k) lives at ptr[k * ld + mn]   (A transposed, B not transposed)
-// LDS layout is always [k][mn] with row stride LD floats.
+// One operand tile: `BMN` rows in the m (or n) direction by kBK along k.
+// KMAJOR: element (mn, k) lives at ptr[mn * ld + k]   (A not transposed, B transposed); LDS holds [mn][k]
+// else  : element (mn, k) lives at ptr[k * ld + mn]   (A transposed, B not transposed); LDS holds [k][mn]
+// The 4-float row padding makes the 16-byte fragment reads of 16 consecutive lanes hit 64 distinct banks.
 template <int BMN, bool KMAJOR>
 struct Tile {
-    static constexpr int LD = BMN + 4;
-    static constexpr int NV = BMN * BK / 4 / kGemmThreads;
+    static constexpr int LD = KMAJOR ? kBK + 4 : BMN + 4;            // LDS row stride in floats
+    static constexpr int ELEMS = KMAJOR ? BMN * LD : kBK * LD;       // floats per LDS buffer
+    static constexpr int NV = BMN * kBK / 4 / kGemmThreads;          // 16-byte pieces per thread
     floatx4 r[NV];
 
-    // which float4 of the tile thread `threadIdx.x` handles in its i-th access: (mn, k) of its first element
+    // (mn, k) of the first element of the i-th piece of thread `threadIdx.x`
     static __device__ __forceinline__ void coords(int i, int& mn, int& k) {
         const int f = threadIdx.x + i * kGemmThreads;
         if (KMAJOR) {
-            mn = f / (BK / 4);
-            k = (f % (BK / 4)) * 4;
+            mn = f / (kBK / 4);
+            k = (f % (kBK / 4)) * 4;
         } else {
-#if ZG_GEMM_MNMAP
-            constexpr int L = BMN / 32;  // 128-byte lines per k-row of the tile
-            constexpr int NL = BK * L;   // lines in the tile
-            const int hl = f >> 2, sub = f & 3;
-            const int line = hl % NL, pass = hl / NL;
-            const int half = (pass + line) & 1;
-            k = line / L;
-            mn = ((line % L) * 8 + half * 4 + sub) * 4;
-#else
             k = f / (BMN / 4);
             mn = (f % (BMN / 4)) * 4;
-#endif
         }
     }
-
-    template <bool SAFE>
-    __device__ __forceinline__ void load(const float* __restrict__ p, size_t ld, size_t mn0, size_t k0, size_t MN,
-                                         size_t K, bool vec_ok) {
-#pragma unroll
-        for (int i = 0; i < NV; i++) {
-            int tmn, tk;
-            coords(i, tmn, tk);
-            const size_t mn = mn0 + tmn, k = k0 + tk;
-            const float* q = KMAJOR ? p + mn * ld + k : p + k * ld + mn;
-            if (!SAFE) {
-                r[i] = *reinterpret_cast<const floatx4*>(q);
-            } else {
-                floatx4 v = {0.f, 0.f, 0.f, 0.f};
-                if (KMAJOR) {
-                    if (mn < MN) {
-                        if (vec_ok && k + 4 <= K) {
-                            v = *reinterpret_cast<const floatx4*>(q);
-                        } else {
-                            if (k + 0 < K) v.x = q[0];
-                            if (k + 1 < K) v.y = q[1];
-                            if (k + 2 < K) v.z = q[2];
-                            if (k + 3 < K) v.w = q[3];
-                        }
-                    }
-                } else {
-                    if (k < K) {
-                        if (vec_ok && mn + 4 <= MN) {
-                            v = *reinterpret_cast<const floatx4*>(q);
-                        } else {
-                            if (mn + 0 < MN) v.x = q[0];
-                            if (mn + 1 < MN) v.y = q[1];
-                            if (mn + 2 < MN) v.z = q[2];
-                            if (mn + 3 < MN) v.w = q[3];
-                        }
-                    }
-                }
-                r[i] = v;
-            }
-        }
-    }
-
-    // LDS write instructions this thread issues per tile: 4 scalar writes per float4 for a k-major operand
-    // (the transposing store), one 128-bit write otherwise
-    static constexpr int NW = NV * (KMAJOR ? 4 : 1);
-
-    // the op-th of those writes
-    __device__ __forceinline__ void store_op(float* __restrict__ lds, int op) const {
-        const int i = KMAJOR ? op / 4 : op;
+    // element offset of piece i from the tile origin in HBM / in LDS
+    static __device__ __forceinline__ size_t gmem_offset(int i, size_t ld) {
         int mn, k;
         coords(i, mn, k);
-        if (KMAJOR) {
-            const int c = op % 4;
-            lds[(k + c) * LD + mn] = r[i][c];
-        } else {
-            *reinterpret_cast<floatx4*>(lds + k * LD + mn) = r[i];
-        }
+        return KMAJOR ? mn * ld + k : k * ld + mn;
+    }
+    static __device__ __forceinline__ int lds_offset(int i) {
+        int mn, k;
+        coords(i, mn, k);
+        return KMAJOR ? mn * LD + k : k * LD + mn;
     }
 
-    __device__ __forceinline__ void store(float* __restrict__ lds) const {
-#pragma unroll
-        for (int i = 0; i < NV; i++) {
-            int mn, k;
-            coords(i, mn, k);
-            if (KMAJOR) {
-                lds[(k + 0) * LD + mn] = r[i].x;
-                lds[(k + 1) * LD + mn] = r[i].y;
-                lds[(k + 2) * LD + mn] = r[i].z;
-                lds[(k + 3) * LD + mn] = r[i].w;
-            } else {
-                *reinterpret_cast<floatx4*>(lds + k * LD + mn) = r[i];
+    // fast path: `base` is the tile origin (uniform), `off` this thread's byte offset of piece i
+    __device__ __forceinline__ void load_fast(int i, const float* __restrict__ base, unsigned off) {
+        r[i] = *reinterpret_cast<const floatx4*>(reinterpret_cast<const char*>(base) + off);
+    }
+
+    // checked path: zero fill outside [0, MN) x [0, K), scalar loads where 16-byte loads are not legal
+    __device__ __forceinline__ void load_safe(int i, const float* __restrict__ p, size_t ld, size_t mn0, size_t k0,
+                                              size_t MN, size_t K, bool vec_ok) {
+        int tmn, tk;
+        coords(i, tmn, tk);
+        const size_t mn = mn0 + tmn, k = k0 + tk;
+        const float* q = KMAJOR ? p + mn * ld + k : p + k * ld + mn;
+        floatx4 v = {0.f, 0.f, 0.f, 0.f};
+        if (KMAJOR) {
+            if (mn < MN) {
+                if (vec_ok && k + 4 <= K) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+                    if (k + 0 < K) v.x = q[0];
+                    if (k + 1 < K) v.y = q[1];
+                    if (k + 2 < K) v.z = q[2];
+                    if (k + 3 < K) v.w = q[3];
+                }
+            }
+        } else {
+            if (k < K) {
+                if (vec_ok && mn + 4 <= MN) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+                    if (mn + 0 < MN) v.x = q[0];
+                    if (mn + 1 < MN) v.y = q[1];
+                    if (mn + 2 < MN) v.z = q[2];
+                    if (mn + 3 < MN) v.w = q[3];
+                }
             }
         }
+        r[i] = v;
     }
+
+    __device__ __forceinline__ void store_op(float* __restrict__ lds_thread_base, int i) const {
+        // lds_thread_base = buffer + lds_offset(0); the further pieces sit at compile-time distances
+        constexpr int STEP = KMAJOR ? (kGemmThreads / (kBK / 4)) * LD : (kGemmThreads / (BMN / 4)) * LD;
+        *reinterpret_cast<floatx4*>(lds_thread_base + i * STEP) = r[i];
+    }
+};
+
+// The fragments one lane feeds to the MFMAs of one k-group (4 steps) for its T blocks of 32 rows.
+template <int BMN, bool KMAJOR, int T>
+struct Frag {
+    using Tl = Tile<BMN, KMAJOR>;
+    using V = std::conditional_t<KMAJOR, floatx4, typename VecOf<T>::type>;
+    static constexpr int N = KMAJOR ? T : 4;  // LDS reads per k-group
+    V v[N];
+
+    // this lane's read base inside an LDS buffer: w0 = first row of the wave's slab
+    static __device__ __forceinline__ int lane_base(int w0, int l32, int lk) {
+        return KMAJOR ? (w0 + l32) * Tl::LD + lk * 4 : (lk * 4) * Tl::LD + w0 + l32 * T;
+    }
+    // n-th read of k-group g
+    __device__ __forceinline__ void read_op(int n, const float* __restrict__ lane_ptr, int g) {
+        if (KMAJOR) v[n] = *reinterpret_cast<const V*>(lane_ptr + n * 32 * Tl::LD + g * 8);
+        else v[n] = *reinterpret_cast<const V*>(lane_ptr + (g * 8 + n) * Tl::LD);
+    }
+    // operand of block t in step c
+    __device__ __forceinline__ float get(int t, int c) const {
+        if constexpr (KMAJOR) return v[t][c];
+        else if constexpr (T == 1) return v[c];
+        else return v[c][t];
+    }
+    // tile row (or column) that block t, block-row b stands for
+    static __device__ __forceinline__ int index_of(int t, int b) { return KMAJOR ? t * 32 + b : b * T + t; }
 };
 
 struct GemmArgs {
@@ -169,14 +188,16 @@ __device__ __forceinline__ void tile_coords(unsigned pid, unsigned tiles_m, unsi
 
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, bool SAFE>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
+    constexpr int BK = kBK;
     using TA = Tile<BM, A_KMAJOR>;
     using TB = Tile<BN, B_KMAJOR>;
     constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
     constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int A_ELEMS = BK * TA::LD, B_ELEMS = BK * TB::LD;
-    __shared__ __attribute__((aligned(16))) float lds[2 * (A_ELEMS + B_ELEMS)];
-    float* As0 = lds;
-    float* Bs0 = lds + 2 * A_ELEMS;
+    using FA = Frag<BM, A_KMAJOR, TM>;
+    using FB = Frag<BN, B_KMAJOR, TN>;
+    extern __shared__ __attribute__((aligned(16))) float lds[];  // A buffers 0/1, then B buffers 0/1
+    float* const As0 = lds;
+    float* const Bs0 = lds + 2 * TA::ELEMS;
 
     unsigned tm, tn;
     tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
@@ -199,89 +220,190 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     const size_t KT = (g.K + BK - 1) / BK;
-    constexpr int NP = BK / 2;   // k-pairs (one MFMA step each) per tile
-    constexpr int NM = TM * TN;  // MFMAs per k-pair
-    constexpr int NW = TA::NW + TB::NW;
-    constexpr int WPM = (NW + NM - 1) / NM;  // LDS writes placed in front of each MFMA of the last pair
+    constexpr int NM = TM * TN;         // MFMAs per step
+    constexpr int NMF = 4 * NM;         // MFMAs per k-group
+    constexpr int NR = FA::N + FB::N;   // fragment reads per k-group
+    constexpr int NL = TA::NV + TB::NV; // 16-byte global loads (and LDS writes) per thread per tile
 
-    // A wave issues in order and one fp32 MFMA keeps the matrix pipe busy for 64 cycles, so whatever has to
-    // overlap with it must sit between MFMAs in the instruction stream.  The schedule is written out by hand
-    // and pinned with sched_barrier (left alone, the scheduler sinks every load next to its use and exposes
-    // the LDS and L2 latencies):
-    //   tile start : read the fragments of pair 0, issue the global loads of the next tile
-    //   pair p     : read the fragments of pair p+1 (second register set), then the MFMAs of pair p
-    //   last pair  : the LDS writes of the next tile are dealt out in front of its MFMAs
-    float fa[2][TM], fb[2][TN];
-    auto read_frag = [&](int set, const float* As, const float* Bs, int kk) {
+    // per-thread constants: where this thread's pieces go in LDS, where its lane reads fragments, and (fast
+    // path) the byte offsets of its pieces from the tile origin in HBM
+    float* const a_wr = As0 + TA::lds_offset(0);
+    float* const b_wr = Bs0 + TB::lds_offset(0);
+    const float* const a_rd = As0 + FA::lane_base(wm0, l32, lk);
+    const float* const b_rd = Bs0 + FB::lane_base(wn0, l32, lk);
+    unsigned a_off[TA::NV], b_off[TB::NV];
 #pragma unroll
-        for (int i = 0; i < TM; i++) fa[set][i] = As[(kk + lk) * TA::LD + wm0 + i * 32 + l32];
+    for (int i = 0; i < TA::NV; i++) a_off[i] = (unsigned)(TA::gmem_offset(i, g.lda) * sizeof(float));
 #pragma unroll
-        for (int j = 0; j < TN; j++) fb[set][j] = Bs[(kk + lk) * TB::LD + wn0 + j * 32 + l32];
-    };
-    TA ta;
-    TB tb;
-    auto tile_step = [&](size_t kt, auto more_tag) {
-        constexpr bool MORE = decltype(more_tag)::value;
-        const int cur = (int)(kt & 1);
-        const float* As = As0 + cur * A_ELEMS;
-        const float* Bs = Bs0 + cur * B_ELEMS;
-        float* As_next = As0 + (cur ^ 1) * A_ELEMS;
-        float* Bs_next = Bs0 + (cur ^ 1) * B_ELEMS;
-        read_frag(0, As, Bs, 0);
-        if (MORE) {
-            ta.template load<SAFE>(A, g.lda, m0, (kt + 1) * BK, g.M, g.K, g.a_vec != 0);
-            tb.template load<SAFE>(B, g.ldb, n0, (kt + 1) * BK, g.N, g.K, g.b_vec != 0);
+    for (int i = 0; i < TB::NV; i++) b_off[i] = (unsigned)(TB::gmem_offset(i, g.ldb) * sizeof(float));
+    const float* const a_org = A_KMAJOR ? A + m0 * g.lda : A + m0;  // tile origin at k = 0
+    const float* const b_org = B_KMAJOR ? B + n0 * g.ldb : B + n0;
+
+    // Tiles wait in registers for two tile times between their global loads and their LDS writes (slot t % 2),
+    // which covers the HBM latency also when a workgroup has a CU to itself.
+    TA ta[2];
+    TB tb[2];
+    auto load_op = [&](auto slot_tag, int v, size_t k0) {
+        constexpr int S = decltype(slot_tag)::value;
+        if (v < TA::NV) {
+            if (!SAFE) ta[S].load_fast(v, a_org + (A_KMAJOR ? k0 : k0 * g.lda), a_off[v]);
+            else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, g.K, g.a_vec != 0);
+        } else {
+            if (!SAFE) tb[S].load_fast(v - TA::NV, b_org + (B_KMAJOR ? k0 : k0 * g.ldb), b_off[v - TA::NV]);
+            else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, g.K, g.b_vec != 0);
         }
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto store_op = [&](auto slot_tag, int w, int buf) {
+        constexpr int S = decltype(slot_tag)::value;
+        if (w < TA::NV) ta[S].store_op(a_wr + buf * TA::ELEMS, w);
+        else tb[S].store_op(b_wr + buf * TB::ELEMS, w - TA::NV);
+    };
+    // fragment register sets: k-group 0 of a tile lives in set 0, k-group 1 in set 1
+    FA fa[2];
+    FB fb[2];
+    auto read_op = [&](int set, int n, int buf, int grp) {
+        if (n < FA::N) fa[set].read_op(n, a_rd + buf * TA::ELEMS, grp);
+        else fb[set].read_op(n - FA::N, b_rd + buf * TB::ELEMS, grp);
+    };
+
+    // One tile = two k-groups of 4 steps of NM MFMAs.  The other instructions are dealt out behind the MFMAs,
+    // pinned with sched_barrier (left alone, the scheduler sinks every load next to its use):
+    //   group 0: global loads of tile t+2, fragment reads of group 1, LDS writes of tile t+1; then the barrier
+    //   group 1: fragment reads of group 0 of tile t+1
+    // Every tile runs the same code, the last ones included: past the end of k the fast kernels repeat the loads
+    // of the last tile (in bounds, never consumed), the checked kernels load zeros, and the LDS writes and the
+    // barrier still happen.  One loop body without peeled
+    // tails keeps the accumulators in one place.  The tile's parity is a template argument, so all LDS
+    // addresses are immediates.
+    constexpr int E0 = NL + NR + NL;
+    constexpr int PER0 = (E0 + NMF - 1) / NMF;
+    constexpr int PER1 = (NR + (NMF + 1) / 2 - 1) / ((NMF + 1) / 2);  // reads land in the first half of group 1
+    auto tile_step = [&](size_t kt, auto parity_tag) {
+        constexpr int S = decltype(parity_tag)::value;  // kt % 2: LDS buffer and register slot of this tile
+        using SCur = std::integral_constant<int, S>;
+        using SNext = std::integral_constant<int, S ^ 1>;
+        const size_t k_load = (SAFE || kt + 2 < KT) ? (kt + 2) * BK : (KT - 1) * BK;
 #pragma unroll
-        for (int p = 0; p < NP; p++) {
-            if (p + 1 < NP) read_frag((p + 1) & 1, As, Bs, 2 * (p + 1));
-            __builtin_amdgcn_sched_barrier(0);
+        for (int grp = 0; grp < 2; grp++) {
 #pragma unroll
-            for (int q = 0; q < NM; q++) {
-                if (MORE && p == NP - 1) {
-#pragma unroll
-                    for (int w = q * WPM; w < (q + 1) * WPM && w < NW; w++) {
-                        if (w < TA::NW) ta.store_op(As_next, w);
-                        else tb.store_op(Bs_next, w - TA::NW);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+            for (int n = 0; n < NMF; n++) {
+                const int c = n / NM, q = n % NM;
                 const int i = q / TN, j = q % TN;
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[p & 1][i], fb[p & 1][j], acc[i][j], 0, 0, 0);
-                if (MORE && p == NP - 1) __builtin_amdgcn_sched_barrier(0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[grp].get(i, c), fb[grp].get(j, c), acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (grp == 0) {
+#pragma unroll
+                    for (int e = n * PER0; e < (n + 1) * PER0 && e < E0; e++) {
+                        if (e < NL) load_op(SCur{}, e, k_load);              // slot S is free: tile kt is in LDS
+                        else if (e < NL + NR) read_op(1, e - NL, S, 1);
+                        else store_op(SNext{}, e - NL - NR, S ^ 1);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = n * PER1; e < (n + 1) * PER1 && e < NR; e++) read_op(0, e, S ^ 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            if (grp == 0) {
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        __syncthreads();
     };
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
 
-    ta.template load<SAFE>(A, g.lda, m0, 0, g.M, g.K, g.a_vec != 0);
-    tb.template load<SAFE>(B, g.ldb, n0, 0, g.N, g.K, g.b_vec != 0);
-    ta.store(As0);
-    tb.store(Bs0);
+    // prologue: tile 0 goes straight to LDS buffer 0, tile 1 starts its flight in slot 1
+#pragma unroll
+    for (int v = 0; v < NL; v++) load_op(P0{}, v, 0);
+#pragma unroll
+    for (int v = 0; v < NL; v++) load_op(P1{}, v, (SAFE || KT > 1) ? BK : 0);
+#pragma unroll
+    for (int w = 0; w < NL; w++) store_op(P0{}, w, 0);
     __syncthreads();
-    for (size_t kt = 0; kt + 1 < KT; kt++) tile_step(kt, std::true_type{});
-    tile_step(KT - 1, std::false_type{});
+#pragma unroll
+    for (int n = 0; n < NR; n++) read_op(0, n, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
 
-    // epilogue: accumulator register r of lane l holds C[(r/4)*8 + (l/32)*4 + r%4][l%32] of its 32x32 block
+    // Tiles go in pairs so that the loop body is one straight run of MFMAs.  The fast kernels are only used for
+    // an even number of tiles; in the checked kernels a tile past the end of k loads as zeros and adds nothing.
+    for (size_t kt = 0; kt < KT; kt += 2) {
+        tile_step(kt, P0{});
+        tile_step(kt + 1, P1{});
+    }
+
+    // epilogue.  Accumulator register r of lane l belongs to block row (r/4)*8 + (l/32)*4 + r%4 and block
+    // column l%32; Frag::index_of turns those into tile rows and columns.  With B k-contiguous a store
+    // instruction writes two 128-byte row segments; otherwise a lane owns TN adjacent columns and stores them as
+    // one vector.  With beta != 0 the old values of a row of blocks are read together before any is used; C is
+    // not read at all when beta == 0.
     const float alpha = g.alpha, beta = g.beta;
+    const bool use_c = beta != 0.f;
+    // The accumulators are taken out of their AGPRs one row of blocks at a time through an explicit
+    // v_accvgpr_read (the "a" constraint pins the value in an AGPR up to that point).  Left to itself the
+    // register allocator copies all of them to VGPRs at the loop exit, which doubles the kernel's register
+    // count and halves its occupancy.  The instruction is opaque to the hazard recogniser, so the wait states an
+    // AGPR read needs after the MFMA that wrote it are spent explicitly first.
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    constexpr bool VEC_C = !SAFE && !B_KMAJOR && TN > 1;
+    using VC = typename VecOf<VEC_C ? TN : 1>::type;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+        float res[TN][16], old[TN][16];
+        float* cptr[TN];
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const size_t col = n0 + wn0 + j * 32 + l32;
+        for (int j = 0; j < TN; j++)
+            cptr[j] = C + (m0 + wm0 + FA::index_of(i, lk * 4)) * g.ldc + n0 + wn0 + FB::index_of(j, l32);
+        constexpr int RSTEP = A_KMAJOR ? 1 : TM;  // tile rows between consecutive block rows
+        auto row_of = [&](int r) { return ((r >> 2) * 8 + (r & 3)) * RSTEP; };  // relative to block row lk*4
+        auto in_range = [&](int j, int r) {
+            if (!SAFE) return true;
+            const size_t row = m0 + wm0 + FA::index_of(i, lk * 4 + (r >> 2) * 8 + (r & 3));
+            const size_t col = n0 + wn0 + FB::index_of(j, l32);
+            return row < g.M && col < g.N;
+        };
+        if (use_c) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const size_t row = m0 + wm0 + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
-                if (!SAFE || (row < g.M && col < g.N)) {
-                    float* c = C + row * g.ldc + col;
-                    float v = alpha * acc[i][j][r];
-                    if (beta != 0.f) v += beta * (*c);  // C is not read when beta == 0
-                    *c = v;
+                if (VEC_C) {
+                    const VC o = *reinterpret_cast<const VC*>(cptr[0] + (size_t)row_of(r) * g.ldc);
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        if constexpr (VEC_C) old[j][r] = o[j];
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < TN; j++) old[j][r] = in_range(j, r) ? cptr[j][(size_t)row_of(r) * g.ldc] : 0.f;
                 }
             }
         }
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(res[j][r]) : "a"(acc[i][j][r]));
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float v[TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                v[j] = alpha * res[j][r];
+                if (use_c) v[j] += beta * old[j][r];
+            }
+            if (VEC_C) {
+                VC o;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    if constexpr (VEC_C) o[j] = v[j];
+                }
+                *reinterpret_cast<VC*>(cptr[0] + (size_t)row_of(r) * g.ldc) = o;
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    if (in_range(j, r)) cptr[j][(size_t)row_of(r) * g.ldc] = v[j];
+            }
+        }
+        // one row of blocks at a time
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -290,8 +412,12 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
     g.tiles_m = (unsigned)ceil_div_sz(g.M, BM);
     g.tiles_n = (unsigned)ceil_div_sz(g.N, BN);
     dim3 grid(g.tiles_m * g.tiles_n, 1, (unsigned)batches), block(kGemmThreads);
-#define ZG_GEMM(AK, BKM, SF) \
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, SF>), grid, block, 0, ctx->stream, g)
+#define ZG_GEMM(AK, BKM, SF)                                                                                  \
+    do {                                                                                                      \
+        constexpr size_t lds_bytes = 2 * (size_t)(Tile<BM, AK>::ELEMS + Tile<BN, BKM>::ELEMS) * sizeof(float); \
+        static_assert(lds_bytes <= 64 * 1024, "tile buffers exceed the default dynamic LDS limit");           \
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, SF>), grid, block, lds_bytes, ctx->stream, g);       \
+    } while (0)
     if (safe) {
         if (a_kmajor && b_kmajor) ZG_GEMM(true, true, true);
         else if (a_kmajor && !b_kmajor) ZG_GEMM(true, false, true);
@@ -359,21 +485,26 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.a_vec = aligned16(A) && lda % 4 == 0 && a_chunk % 4 == 0;
     g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
 
-    // tile choice: the largest tile that still gives every CU a workgroup
-    const size_t t128 = ceil_div_sz(m, 128) * ceil_div_sz(n, 128) * batches;
-    const size_t t256 = ceil_div_sz(m, 256) * ceil_div_sz(n, 128) * batches;
-    const bool big = t256 >= (size_t)ctx->n_cu * 2;
-    (void)t128;
-    if (big) {
-        const bool safe = !(g.a_vec && g.b_vec && m % 256 == 0 && n % 128 == 0 && k % BK == 0);
-        return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, safe, batches);
-    }
-    if (m > 64 && n > 64) {
-        const bool safe = !(g.a_vec && g.b_vec && m % 128 == 0 && n % 128 == 0 && k % BK == 0);
-        return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, safe, batches);
-    }
-    const bool safe = !(g.a_vec && g.b_vec && m % 64 == 0 && n % 64 == 0 && k % BK == 0);
-    return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, safe, batches);
+    // Fast kernels assume whole tiles, 16-byte alignment of all three matrices and 32-bit byte offsets inside
+    // an operand tile; everything else takes the checked variants.
+    const bool c_vec = aligned16(C) && ldc % 4 == 0 && c_chunk % 4 == 0;
+    const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
+    auto tiles = [&](size_t bm, size_t bn) { return ceil_div_sz(m, bm) * ceil_div_sz(n, bn) * batches; };
+    auto fast = [&](size_t bm, size_t bn) {
+        return g.a_vec && g.b_vec && c_vec && small_ld && m % bm == 0 && n % bn == 0 && k % (2 * kBK) == 0;
+    };
+    // Tile choice by estimated time.  A CU works through its workgroups at a rate that depends on the tile shape
+    // but hardly on how many of them share the CU (measured fraction of a CU's MFMA peak: 0.92 / 0.89 / 0.79),
+    // so the time is the number of rounds the grid needs times the padded work of one tile over that rate.
+    const size_t n_cu = (size_t)ctx->n_cu;
+    auto cost = [&](size_t bm, size_t bn, double eff) {
+        return (double)ceil_div_sz(tiles(bm, bn), n_cu) * (double)(bm * bn) / eff;
+    };
+    const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
+    if (c_large <= c_mid && c_large <= c_small)
+        return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, !fast(256, 128), batches);
+    if (c_mid <= c_small) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, !fast(128, 128), batches);
+    return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, !fast(64, 64), batches);
 }
 
 // ------------------------------------------------------------------------------------------------

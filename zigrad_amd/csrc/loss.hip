@@ -8,6 +8,13 @@
 
 namespace zg {
 
+// exp for the streaming passes of the integer-label kernels: the hardware exponential (v_exp_f32 on x*log2 e).
+// Its relative error grows with |x| (about |x| * 1e-7), far below the 1e-5 bound for softmax terms, and it
+// keeps these passes HBM-bound: the full-precision routine costs about as many VALU cycles as the load takes.
+__device__ __forceinline__ float fexp(float x) {
+    return __expf(x);
+}
+
 // running (max, sum of exp(x - max))
 struct OnlineAccT {
     float m, s;
@@ -49,14 +56,14 @@ __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, i
             float mx = fmaxf(fmaxf(fmaxf(v0.x, v0.y), fmaxf(v0.z, v0.w)), fmaxf(fmaxf(v1.x, v1.y), fmaxf(v1.z, v1.w)));
             mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(v2.x, v2.y), fmaxf(v2.z, v2.w)), fmaxf(fmaxf(v3.x, v3.y), fmaxf(v3.z, v3.w))));
             if (mx > acc.m) {
-                acc.s = __fmul_rn(acc.s, expf(__fsub_rn(acc.m, mx)));
+                acc.s = __fmul_rn(acc.s, fexp(__fsub_rn(acc.m, mx)));
                 acc.m = mx;
             }
             float s = 0.f;
-            s += expf(v0.x - acc.m) + expf(v0.y - acc.m) + expf(v0.z - acc.m) + expf(v0.w - acc.m);
-            s += expf(v1.x - acc.m) + expf(v1.y - acc.m) + expf(v1.z - acc.m) + expf(v1.w - acc.m);
-            s += expf(v2.x - acc.m) + expf(v2.y - acc.m) + expf(v2.z - acc.m) + expf(v2.w - acc.m);
-            s += expf(v3.x - acc.m) + expf(v3.y - acc.m) + expf(v3.z - acc.m) + expf(v3.w - acc.m);
+            s += fexp(v0.x - acc.m) + fexp(v0.y - acc.m) + fexp(v0.z - acc.m) + fexp(v0.w - acc.m);
+            s += fexp(v1.x - acc.m) + fexp(v1.y - acc.m) + fexp(v1.z - acc.m) + fexp(v1.w - acc.m);
+            s += fexp(v2.x - acc.m) + fexp(v2.y - acc.m) + fexp(v2.z - acc.m) + fexp(v2.w - acc.m);
+            s += fexp(v3.x - acc.m) + fexp(v3.y - acc.m) + fexp(v3.z - acc.m) + fexp(v3.w - acc.m);
             acc.s += s;
         }
         for (; j < c4; j += TPR) {
@@ -114,9 +121,9 @@ __global__ __launch_bounds__(kBlock) void smce_label_fwd_kernel(const float* log
 template <bool ACC>
 __global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* logits, const uint64_t* labels,
                                                                  const float* lse, float* grad, size_t rows,
-                                                                 size_t cols,
-                                                                 float denom) {
+                                                                 size_t cols, float denom) {
     // grid: x over float4 columns of one row, y over rows (looped)
+    const float inv_denom = __fdiv_rn(1.0f, denom);  // exact for power-of-two batch sizes, else within 1 ulp of x/denom
     const bool vec = (((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(grad)) & 15u) == 0) &&
                      (cols % 4 == 0);
     for (size_t row = blockIdx.y; row < rows; row += gridDim.y) {
@@ -132,10 +139,10 @@ __global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* log
                 float4 v = x4[j];
                 float4 g = ACC ? g4[j] : make_float4(0, 0, 0, 0);
                 const size_t c = 4 * j;
-                float d0 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.x, l)), (c + 0 == lab) ? 1.f : 0.f), denom);
-                float d1 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.y, l)), (c + 1 == lab) ? 1.f : 0.f), denom);
-                float d2 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.z, l)), (c + 2 == lab) ? 1.f : 0.f), denom);
-                float d3 = __fdiv_rn(__fsub_rn(expf(__fsub_rn(v.w, l)), (c + 3 == lab) ? 1.f : 0.f), denom);
+                float d0 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.x, l)), (c + 0 == lab) ? 1.f : 0.f), inv_denom);
+                float d1 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.y, l)), (c + 1 == lab) ? 1.f : 0.f), inv_denom);
+                float d2 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.z, l)), (c + 2 == lab) ? 1.f : 0.f), inv_denom);
+                float d3 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.w, l)), (c + 3 == lab) ? 1.f : 0.f), inv_denom);
                 g.x = ACC ? __fadd_rn(g.x, d0) : d0;
                 g.y = ACC ? __fadd_rn(g.y, d1) : d1;
                 g.z = ACC ? __fadd_rn(g.z, d2) : d2;
@@ -144,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* log
             }
         } else {
             for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += (size_t)gridDim.x * kBlock) {
-                float d = __fdiv_rn(__fsub_rn(expf(__fsub_rn(xr[j], l)), (j == lab) ? 1.f : 0.f), denom);
+                float d = __fmul_rn(__fsub_rn(fexp(__fsub_rn(xr[j], l)), (j == lab) ? 1.f : 0.f), inv_denom);
                 gr[j] = ACC ? __fadd_rn(gr[j], d) : d;
             }
         }

@@ -11,7 +11,7 @@ The same JSON line also carries:
   cpu_baseline  the CPU oracle (C restatement of HostDevice + the box's BLAS) running the same step
   ops           the op microbenchmark suite of configs[1] (GEMM variants, bmm, broadcast add, axis
                 reductions, fused softmax cross-entropy), each with its own roofline fraction
-  mlp_b64       the batch-64 MLP of configs[0] (latency-bound): steps per second
+  mlp_b64, gcn, dqn   the latency-bound configurations (configs[0], [2], [3]): step time, loss read every step
 """
 from __future__ import annotations
 
@@ -45,6 +45,23 @@ def gemm_flops_per_step(dims, batch):
     return total
 
 
+def gemm_bytes_per_step(dims, batch):
+    """Algorithmic bytes of the same launches: both operands read once, C written, C also read where the
+    reference accumulates (beta = 1 for every gradient GEMM, src/ndtensor.zig:1092-1136)."""
+    total = 0
+    for l, (fi, fo) in enumerate(zip(dims[:-1], dims[1:])):
+        total += 4 * (batch * fi + fo * fi + batch * fo)          # forward: X, W -> Y
+        total += 4 * (batch * fo + batch * fi + 2 * fo * fi)      # dW += dY^T X
+        if l > 0:
+            total += 4 * (batch * fo + fo * fi + 2 * batch * fi)  # dX += dY W
+    return total
+
+
+# HBM-side bytes per GEMM launch (average over the step's 8 launches), from two rocprofv3 counter runs of this
+# script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the copy_calibration kernel.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 732.8e6
+
+
 class GemmTimer:
     """Brackets every bmm_acc dispatch with HIP events on the device's own stream."""
 
@@ -69,15 +86,45 @@ class GemmTimer:
         return sum(a.elapsed_ms(b) for a, b in self.pairs)
 
 
-def time_op(dev, fn, iters, warmup=3):
-    for _ in range(warmup):
-        fn()
+def time_op(dev, fn, iters, warm_ms=60.0, batches=10):
+    """Median (and p10/p90) per-call time in ms over `batches` event-bracketed runs of `iters` back-to-back calls.
+
+    The warm-up runs for at least `warm_ms` of wall time: the GPU raises its clock only under sustained load, and a
+    kernel timed in the first tens of milliseconds after idle reads 10 % slower than in a training loop.
+    """
+    t0 = time.perf_counter()
+    while True:
+        for _ in range(iters):
+            fn()
+        dev.sync()
+        if (time.perf_counter() - t0) * 1e3 >= warm_ms:
+            break
+    pairs = []
+    for _ in range(batches):
+        e0 = dev.event().record()
+        for _ in range(iters):
+            fn()
+        pairs.append((e0, dev.event().record()))
     dev.sync()
-    e0 = dev.event().record()
-    for _ in range(iters):
-        fn()
-    e1 = dev.event().record()
-    return e0.elapsed_ms(e1) / iters
+    ms = sorted(a.elapsed_ms(b) / iters for a, b in pairs)
+    pick = lambda q: ms[min(len(ms) - 1, int(q * len(ms)))]
+    return {"ms": pick(0.5), "ms_p10": pick(0.1), "ms_p90": pick(0.9)}
+
+
+def copy_calibration(dev):
+    """Three launches of a plain streaming kernel of known size (relu_fwd over 2^26 floats: 256 MiB read, 256 MiB
+    written, grid found in a counter trace by its 64 Mi-element size).  HBM byte counters of other kernels are
+    scaled by what they read for this one."""
+    from zigrad_amd.device import F32
+
+    n = 1 << 26
+    x, y = dev.mem_alloc(F32, n), dev.mem_alloc(F32, n)
+    dev.mem_fill(x, 1.0)
+    for _ in range(3):
+        dev.dispatch("relu_fwd", x=x, y=y)
+    dev.sync()
+    dev.mem_free(x)
+    dev.mem_free(y)
 
 
 def op_suite(dev, quick=False):
@@ -88,6 +135,10 @@ def op_suite(dev, quick=False):
     r = np.random.default_rng(0)
     iters = 5 if quick else 20
 
+    def tfl(flops, t):
+        tf = flops / (t["ms"] * 1e-3) / 1e12
+        return {**t, "tflops": tf, "frac_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+
     def dev_normal(n):
         b = dev.mem_alloc(F32, n)
         dev.mem_random(b, "normal", seed=int(r.integers(1 << 30)))
@@ -97,16 +148,14 @@ def op_suite(dev, quick=False):
     n = 4096
     A, B, C = dev_normal(n * n), dev_normal(n * n), dev_normal(n * n)
     for tag, ta, tb in (("matmul_4096_nn", False, False), ("matmul_4096_tn", True, False), ("matmul_4096_nt", False, True)):
-        ms = time_op(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=n, n=n, k=n, trans_a=ta, trans_b=tb, lda=n, ldb=n,
-                                                ldc=n, alpha=1.0, beta=0.0), iters)
-        tf = 2 * n ** 3 / (ms * 1e-3) / 1e12
-        out[tag] = {"ms": ms, "tflops": tf, "frac_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+        t = time_op(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=n, n=n, k=n, trans_a=ta, trans_b=tb, lda=n, ldb=n,
+                                               ldc=n, alpha=1.0, beta=0.0), iters)
+        out[tag] = tfl(2 * n ** 3, t)
     # bmm 32 x 512^3
     nb, s = 32, 512
-    ms = time_op(dev, lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, s, s], B_shape=[nb, s, s], C_shape=[nb, s, s],
-                                            trans_a=False, trans_b=False, lda=s, ldb=s, ldc=s, alpha=1.0, beta=0.0), iters)
-    tf = 2 * nb * s ** 3 / (ms * 1e-3) / 1e12
-    out["bmm_32x512"] = {"ms": ms, "tflops": tf, "frac_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+    t = time_op(dev, lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, s, s], B_shape=[nb, s, s], C_shape=[nb, s, s],
+                                           trans_a=False, trans_b=False, lda=s, ldb=s, ldc=s, alpha=1.0, beta=0.0), iters * 5)
+    out["bmm_32x512"] = tfl(2 * nb * s ** 3, t)
     for b in (A, B, C):
         dev.mem_free(b)
 
@@ -115,9 +164,9 @@ def op_suite(dev, quick=False):
     X, bias, Z = dev_normal(rows * cols), dev_normal(cols), dev.mem_alloc(F32, rows * cols)
     yrow = dev.mem_alloc(F32, rows)
 
-    def gbs(nbytes, ms):
-        g = nbytes / (ms * 1e-3) / 1e9
-        return {"ms": ms, "gbs": g, "frac_hbm": g / PEAK_HBM_GBS}
+    def gbs(nbytes, t):
+        g = nbytes / (t["ms"] * 1e-3) / 1e9
+        return {**t, "gbs": g, "frac_hbm": g / PEAK_HBM_GBS}
 
     ms = time_op(dev, lambda: dev.dispatch("add", x=X, y=bias, z=Z), iters * 5)
     out["add_bcast_8192x4096"] = gbs((2 * rows * cols + cols) * 4, ms)
@@ -170,6 +219,32 @@ def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_m
     return dt, loss
 
 
+def run_small(dev, kind, steps):
+    """Step time of the GCN (2708 nodes, 1433 features, 13264 edges, 140 labelled, Adam) or DQN (4-128-128-2, batch
+    64, Adam) train step; the loss is read back every step, as the reference's loops do."""
+    from zigrad_amd.trainers import DQNTrainer, GCNTrainer, dqn_inputs, gcn_inputs, mlp_inputs
+
+    if kind == "gcn":
+        tr = GCNTrainer(dev, gcn_inputs(seed=0), lr=0.01, clip=True)
+        what = "2-layer GCN 1433-16-7, 2708 nodes, 13264 edges, 140 labelled nodes, Adam lr 0.01"
+    else:
+        dims, batch = [4, 128, 128, 2], 64
+        params, _, _, _ = mlp_inputs(dims, batch)
+        tr = DQNTrainer(dev, dims, batch, lr=1e-3, gamma=0.99, clip=True)
+        tr.load_params(params)
+        tr.set_batch(dqn_inputs(batch=batch))
+        what = "DQN update 4-128-128-2, batch 64, frozen target net, gather, smooth-L1, Adam lr 1e-3"
+    for _ in range(10):
+        tr.step()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tr.step()
+    dev.sync()
+    dt = time.perf_counter() - t0
+    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "workload": what}
+
+
 def cpu_baseline(dims, batch, budget_steps=2):
     """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share."""
     from oracle.oracle_device import OracleDevice
@@ -204,6 +279,7 @@ def main():
     from zigrad_amd import HipDevice
 
     dev = HipDevice(0)
+    copy_calibration(dev)
     timer = GemmTimer(dev)
     timer.install()
     dt, loss = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", timer, args.loss_mode)
@@ -234,16 +310,20 @@ def main():
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic_unit": "bytes per launch (L2 misses to the fabric, rocprofv3 FETCH_SIZE + WRITE_SIZE)",
+            "algorithmic_bytes_per_launch": gemm_bytes_per_step(WIDE_DIMS, WIDE_BATCH) / 8,
             "kernel": "gemm_kernel (fp32 MFMA 32x32x2), 8 launches per step",
             "gemm_ms_per_step": gemm_ms / args.steps,
             "launches_timed": n_launch,
         },
     }
-    # batch-64 MLP of configs[0]: latency-bound
+    # the latency-bound configurations: batch-64 MLP (configs[0]), GCN (configs[2]), DQN update (configs[3])
     dt64, _ = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01)
     result["mlp_b64"] = {"steps_per_s": 200 / dt64, "ms_per_step": dt64 / 200 * 1e3,
                          "workload": "784-128-64-10, batch 64, SGD lr 0.01, clip on, loss read every step"}
+    result["gcn"] = run_small(dev, "gcn", 100)
+    result["dqn"] = run_small(dev, "dqn", 200)
     if not args.no_ops:
         result["ops"] = op_suite(dev)
     if not args.no_cpu:

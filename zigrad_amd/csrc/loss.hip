@@ -49,9 +49,14 @@ __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, i
     if (vec) {
         const float4* x4 = reinterpret_cast<const float4*>(xr);
         const size_t c4 = cols >> 2;
-        size_t j = lane;
-        for (; j + 3 * TPR < c4; j += 4 * TPR) {
-            float4 v0 = x4[j], v1 = x4[j + TPR], v2 = x4[j + 2 * TPR], v3 = x4[j + 3 * TPR];
+        // four 16-byte loads in flight per thread; past the end of the row they are replaced by -inf, which adds
+        // exp(-inf) = 0, so the last partial round takes the same path as the others
+        const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        for (size_t j = lane; j < c4; j += 4 * TPR) {
+            const float4 v0 = nt_load(x4 + j);
+            const float4 v1 = (j + TPR < c4) ? nt_load(x4 + j + TPR) : ninf;
+            const float4 v2 = (j + 2 * TPR < c4) ? nt_load(x4 + j + 2 * TPR) : ninf;
+            const float4 v3 = (j + 3 * TPR < c4) ? nt_load(x4 + j + 3 * TPR) : ninf;
             // one rescale per 16 elements: fold the 16 into the running max first
             float mx = fmaxf(fmaxf(fmaxf(v0.x, v0.y), fmaxf(v0.z, v0.w)), fmaxf(fmaxf(v1.x, v1.y), fmaxf(v1.z, v1.w)));
             mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(v2.x, v2.y), fmaxf(v2.z, v2.w)), fmaxf(fmaxf(v3.x, v3.y), fmaxf(v3.z, v3.w))));
@@ -59,19 +64,13 @@ __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, i
                 acc.s = __fmul_rn(acc.s, fexp(__fsub_rn(acc.m, mx)));
                 acc.m = mx;
             }
+            if (acc.m == -INFINITY) continue;  // nothing but -inf so far: exp(-inf - -inf) must not be formed
             float s = 0.f;
             s += fexp(v0.x - acc.m) + fexp(v0.y - acc.m) + fexp(v0.z - acc.m) + fexp(v0.w - acc.m);
             s += fexp(v1.x - acc.m) + fexp(v1.y - acc.m) + fexp(v1.z - acc.m) + fexp(v1.w - acc.m);
             s += fexp(v2.x - acc.m) + fexp(v2.y - acc.m) + fexp(v2.z - acc.m) + fexp(v2.w - acc.m);
             s += fexp(v3.x - acc.m) + fexp(v3.y - acc.m) + fexp(v3.z - acc.m) + fexp(v3.w - acc.m);
             acc.s += s;
-        }
-        for (; j < c4; j += TPR) {
-            float4 v = x4[j];
-            online_push(acc, v.x);
-            online_push(acc, v.y);
-            online_push(acc, v.z);
-            online_push(acc, v.w);
         }
     } else {
         for (size_t j = lane; j < cols; j += TPR) online_push(acc, xr[j]);
@@ -117,15 +116,17 @@ __global__ __launch_bounds__(kBlock) void smce_label_fwd_kernel(const float* log
     }
 }
 
-// grad (+)= (exp(x - lse[row]) - onehot) / rows, elementwise over the whole matrix
+// grad (+)= (exp(x - lse[row]) - onehot) / rows, elementwise over the whole matrix.
+// grid: x over chunks of 4 * kBlock float4 columns of one row, y over rows (looped).  A thread has four 16-byte
+// loads (eight when accumulating) in flight: with one, the resident waves cannot cover the HBM latency.
 template <bool ACC>
 __global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* logits, const uint64_t* labels,
                                                                  const float* lse, float* grad, size_t rows,
                                                                  size_t cols, float denom) {
-    // grid: x over float4 columns of one row, y over rows (looped)
     const float inv_denom = __fdiv_rn(1.0f, denom);  // exact for power-of-two batch sizes, else within 1 ulp of x/denom
     const bool vec = (((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(grad)) & 15u) == 0) &&
                      (cols % 4 == 0);
+    constexpr int U = 4;
     for (size_t row = blockIdx.y; row < rows; row += gridDim.y) {
         const float l = lse[row];
         const uint64_t lab = labels[row];
@@ -135,19 +136,33 @@ __global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* log
             const size_t c4 = cols >> 2;
             const float4* x4 = reinterpret_cast<const float4*>(xr);
             float4* g4 = reinterpret_cast<float4*>(gr);
-            for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < c4; j += (size_t)gridDim.x * kBlock) {
-                float4 v = x4[j];
-                float4 g = ACC ? g4[j] : make_float4(0, 0, 0, 0);
-                const size_t c = 4 * j;
-                float d0 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.x, l)), (c + 0 == lab) ? 1.f : 0.f), inv_denom);
-                float d1 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.y, l)), (c + 1 == lab) ? 1.f : 0.f), inv_denom);
-                float d2 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.z, l)), (c + 2 == lab) ? 1.f : 0.f), inv_denom);
-                float d3 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v.w, l)), (c + 3 == lab) ? 1.f : 0.f), inv_denom);
-                g.x = ACC ? __fadd_rn(g.x, d0) : d0;
-                g.y = ACC ? __fadd_rn(g.y, d1) : d1;
-                g.z = ACC ? __fadd_rn(g.z, d2) : d2;
-                g.w = ACC ? __fadd_rn(g.w, d3) : d3;
-                g4[j] = g;
+            for (size_t j0 = (size_t)blockIdx.x * (kBlock * U) + threadIdx.x; j0 < c4; j0 += (size_t)gridDim.x * (kBlock * U)) {
+                float4 v[U], g[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const size_t j = j0 + (size_t)u * kBlock;
+                    if (j < c4) {
+                        v[u] = nt_load(x4 + j);
+                        if (ACC) g[u] = nt_load(g4 + j);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const size_t j = j0 + (size_t)u * kBlock;
+                    if (j < c4) {
+                        const size_t c = 4 * j;
+                        float d0 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].x, l)), (c + 0 == lab) ? 1.f : 0.f), inv_denom);
+                        float d1 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].y, l)), (c + 1 == lab) ? 1.f : 0.f), inv_denom);
+                        float d2 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].z, l)), (c + 2 == lab) ? 1.f : 0.f), inv_denom);
+                        float d3 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].w, l)), (c + 3 == lab) ? 1.f : 0.f), inv_denom);
+                        float4 o;
+                        o.x = ACC ? __fadd_rn(g[u].x, d0) : d0;
+                        o.y = ACC ? __fadd_rn(g[u].y, d1) : d1;
+                        o.z = ACC ? __fadd_rn(g[u].z, d2) : d2;
+                        o.w = ACC ? __fadd_rn(g[u].w, d3) : d3;
+                        nt_store(o, g4 + j);
+                    }
+                }
             }
         } else {
             for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += (size_t)gridDim.x * kBlock) {
@@ -157,6 +172,7 @@ __global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* log
         }
     }
 }
+
 
 // one-hot targets (the reference's form): probabilities are written out; the row's loss term is
 // sum_j -t_j * log(clamp(p_j)).  MODE 0: softmax only (no target, no loss).
@@ -298,11 +314,10 @@ ZG_API int zg_hip_smce_label_bwd(zg_hip_ctx* ctx, const float* logits, const uin
     ZG_CTX(ctx);
     ZG_REQUIRE(logits && labels && lse && grad, "smce_label_bwd: null pointer");
     if (int rc = check_rows("smce_label_bwd", rows, cols)) return rc;
-    size_t gx = ceil_div_sz((cols + 3) / 4, kBlock);
-    if (gx > 64) gx = 64;
-    size_t gy = ceil_div_sz((size_t)ctx->n_cu * 16, gx);
-    if (gy > rows) gy = rows;
-    if (gy > 65535) gy = 65535;
+    // one workgroup per (row, chunk of 4 * kBlock float4 columns); rows beyond the grid limit are looped over
+    size_t gx = ceil_div_sz((cols + 3) / 4, (size_t)kBlock * 4);
+    if (gx > 1024) gx = 1024;
+    size_t gy = rows < 65535 ? rows : 65535;
     dim3 grid((unsigned)gx, (unsigned)gy);
     if (accumulate)
         hipLaunchKernelGGL((smce_label_bwd_kernel<true>), grid, dim3(kBlock), 0, ctx->stream, logits, labels, lse, grad,

@@ -4,6 +4,18 @@
 
 namespace zg {
 
+// 16-byte loads and stores with the non-temporal hint, for data a kernel touches exactly once
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 nt_load(const float4* p) {
+    const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void nt_store(float4 v, float4* p) {
+    const f32x4_t o = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t*>(p));
+}
+
+
 // ---- accumulator policies -------------------------------------------------------------------
 // combine(a, b) must give the same result for (a, b) and (b, a): the butterfly shuffles below apply
 // it with the operands in either order on the two lanes of a pair.

@@ -210,27 +210,40 @@ __global__ __launch_bounds__(kBlock) void col_reduce_kernel(const float* x, type
     }
 }
 
+// Workgroup = 64 adjacent outputs x 4 waves; wave w combines chunks w, w+4, w+8, ... of its outputs with all its
+// loads in flight at once (chunks <= 64, so at most 16 per thread), then the four wave results are combined in
+// wave order.  The order is fixed, so the result does not depend on scheduling.
 template <class A>
 __global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::Acc* partials, typename A::Out* y,
                                                             size_t n_out, size_t inner, int chunks, float alpha,
                                                             float beta) {
     using P = typename A::P;
-    size_t o = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (o >= n_out) return;
-    const size_t outer = o / inner, c = o % inner;
-    const typename P::Acc* pp = partials + (outer * chunks) * inner + c;
-    typename P::Acc acc = pp[0];
-    int k = 1;
-    // loads of eight chunks in flight, combined in chunk order
-    for (; k + 8 <= chunks; k += 8) {
-        typename P::Acc t[8];
+    using Acc = typename P::Acc;
+    __shared__ Acc smem[kBlock];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const size_t o = (size_t)blockIdx.x * 64 + lane;
+    Acc acc = P::init();
+    if (o < n_out) {
+        const size_t outer = o / inner, c = o % inner;
+        const Acc* pp = partials + (outer * chunks) * inner + c;
+        Acc t[16];
 #pragma unroll
-        for (int u = 0; u < 8; u++) t[u] = pp[(size_t)(k + u) * inner];
+        for (int u = 0; u < 16; u++) {
+            const int k = w + 4 * u;
+            if (k < chunks) t[u] = pp[(size_t)k * inner];
+        }
 #pragma unroll
-        for (int u = 0; u < 8; u++) acc = P::combine(acc, t[u]);
+        for (int u = 0; u < 16; u++) {
+            const int k = w + 4 * u;
+            if (k < chunks) acc = P::combine(acc, t[u]);
+        }
     }
-    for (; k < chunks; k++) acc = P::combine(acc, pp[(size_t)k * inner]);
-    A::store(y, o, acc, alpha, beta);
+    smem[threadIdx.x] = acc;
+    __syncthreads();
+    if (w == 0 && o < n_out) {
+        for (int t = 1; t < 4; t++) acc = P::combine(acc, smem[t * 64 + lane]);
+        A::store(y, o, acc, alpha, beta);
+    }
 }
 
 template <class A>
@@ -284,7 +297,7 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     ZG_LAUNCH_CHECK();
     if (chunks > 1) {
         const size_t n_out = outer * inner;
-        hipLaunchKernelGGL((col_final_kernel<A>), dim3((unsigned)ceil_div_sz(n_out, kBlock)), dim3(kBlock), 0,
+        hipLaunchKernelGGL((col_final_kernel<A>), dim3((unsigned)ceil_div_sz(n_out, 64)), dim3(kBlock), 0,
                            ctx->stream, partials, y, n_out, inner, (int)chunks, alpha, beta);
         ZG_LAUNCH_CHECK();
     }

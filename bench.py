@@ -196,7 +196,19 @@ def op_suite(dev, quick=False):
     return out
 
 
-def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3):
+def timed_steps(dev, step_fn, steps):
+    dev.sync()
+    t0 = time.perf_counter()
+    loss = None
+    for _ in range(steps):
+        loss = step_fn()
+    dev.sync()
+    return time.perf_counter() - t0, loss
+
+
+def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3, graph=False):
+    """Returns (seconds, last loss) for `steps` eager steps; with graph=True also the same for `steps` replays of
+    the step recorded as an execution graph (the loss is read back every step in both modes)."""
     from zigrad_amd.trainers import MLPTrainer, mlp_inputs
 
     params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data=data)
@@ -205,18 +217,19 @@ def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_m
     tr.set_batch(x, onehot, labels)
     for _ in range(warmup):
         tr.step()
-    dev.sync()
     if timer is not None:
         timer.on = True
-    t0 = time.perf_counter()
-    loss = None
-    for _ in range(steps):
-        loss = tr.step()
-    dev.sync()
-    dt = time.perf_counter() - t0
+    dt, loss = timed_steps(dev, tr.step, steps)
     if timer is not None:
         timer.on = False
-    return dt, loss
+    if not graph:
+        return dt, loss
+    tr.capture()
+    for _ in range(warmup):
+        tr.step_graph()
+    dt_g, loss_g = timed_steps(dev, tr.step_graph, steps)
+    tr.free_graph()
+    return dt, loss, dt_g, loss_g
 
 
 def run_small(dev, kind, steps):
@@ -236,13 +249,16 @@ def run_small(dev, kind, steps):
         what = "DQN update 4-128-128-2, batch 64, frozen target net, gather, smooth-L1, Adam lr 1e-3"
     for _ in range(10):
         tr.step()
-    dev.sync()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        tr.step()
-    dev.sync()
-    dt = time.perf_counter() - t0
-    return {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "workload": what}
+    dt, _ = timed_steps(dev, tr.step, steps)
+    out = {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "workload": what}
+    if hasattr(tr, "capture"):
+        tr.capture()
+        for _ in range(10):
+            tr.step_graph()
+        dt_g, _ = timed_steps(dev, tr.step_graph, steps)
+        tr.free_graph()
+        out["graph_replay"] = {"steps_per_s": steps / dt_g, "ms_per_step": dt_g / steps * 1e3}
+    return out
 
 
 def cpu_baseline(dims, batch, budget_steps=2):
@@ -319,9 +335,11 @@ def main():
         },
     }
     # the latency-bound configurations: batch-64 MLP (configs[0]), GCN (configs[2]), DQN update (configs[3])
-    dt64, _ = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01)
+    dt64, _, dt64g, _ = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=True)
     result["mlp_b64"] = {"steps_per_s": 200 / dt64, "ms_per_step": dt64 / 200 * 1e3,
-                         "workload": "784-128-64-10, batch 64, SGD lr 0.01, clip on, loss read every step"}
+                         "graph_replay": {"steps_per_s": 200 / dt64g, "ms_per_step": dt64g / 200 * 1e3},
+                         "workload": "784-128-64-10, batch 64, SGD lr 0.01, clip on, loss read every step; "
+                                     "graph_replay = the same step recorded once as an execution graph"}
     result["gcn"] = run_small(dev, "gcn", 100)
     result["dqn"] = run_small(dev, "dqn", 200)
     if not args.no_ops:

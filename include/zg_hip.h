@@ -38,12 +38,15 @@ extern "C" {
 
 typedef struct zg_hip_ctx zg_hip_ctx;
 typedef struct zg_hip_event zg_hip_event;
+typedef struct zg_hip_graph zg_hip_graph;
 
 enum {
     ZG_HIP_OK = 0,
     ZG_HIP_EINVAL = 1,   /* argument/shape check failed; nothing was launched */
     ZG_HIP_EOOM = 2,     /* device allocation failed (reference: Error.DeviceOOM, src/allocators/device_data.zig:44) */
     ZG_HIP_ERUNTIME = 3, /* a HIP runtime call failed */
+    ZG_HIP_ECAPTURE = 4, /* the call synchronises, allocates from the driver or touches host memory and was made
+                            while an execution graph was being captured (or a graph call was made out of order) */
 };
 
 /* kinds for zg_hip_mem_random (reference: RandType, src/device/device_common.zig:3) */
@@ -239,6 +242,30 @@ int zg_hip_sgd_step(zg_hip_ctx *ctx, float *param, float *grad, size_t n, float 
 /* t: the per-tensor-update counter AFTER the reference's `self.t += 1` (src/nn/optim.zig:189) */
 int zg_hip_adam_step(zg_hip_ctx *ctx, float *param, float *grad, float *m, float *v, size_t n, uint64_t t, float lr,
                      float beta1, float beta2, float epsilon, int clip, float max_norm, float delta);
+
+/* lr_t of Adam for counter value t, computed in fp32 exactly as zg_hip_adam_step does on the host
+ * (src/nn/optim.zig:190-191). */
+int zg_hip_adam_lr_t(float lr, float beta1, float beta2, uint64_t t, float *lr_t);
+/* zg_hip_adam_step with lr_t read from memory when the kernel executes.  `lr_t` points to device memory or to
+ * zg_hip_host_alloc memory; the host may rewrite it between replays of a captured graph (not while a replay that
+ * reads it is still running).  This is what lets one captured step serve every later step. */
+int zg_hip_adam_step_at(zg_hip_ctx *ctx, float *param, float *grad, float *m, float *v, size_t n, const float *lr_t,
+                        float beta1, float beta2, float epsilon, int clip, float max_norm, float delta);
+
+/* ---------------------------------------------------------------------------------------------
+ * execution graphs: the ExecutionGraph of the reference's second device, src/device/cuda_device.zig:558-611
+ * (open = begin stream capture, save = end capture and instantiate, run = launch, free).
+ * Between open and save every op call is recorded instead of executed.  Calls that synchronise, allocate
+ * from the driver or copy to/from host memory return ZG_HIP_ECAPTURE (run one eager step first so the
+ * caching allocator and the internal workspace have their final size).  zg_hip_mem_cache_free inside a
+ * capture parks the block with the graph instead of returning it to the pool, so the addresses recorded in
+ * the graph stay private to it until zg_hip_graph_free.  Launch-bound steps (tens of 2-microsecond kernels)
+ * replay without per-op host work.
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_graph_open(zg_hip_ctx *ctx);
+int zg_hip_graph_save(zg_hip_ctx *ctx, zg_hip_graph **out);
+int zg_hip_graph_run(zg_hip_ctx *ctx, zg_hip_graph *graph);
+int zg_hip_graph_free(zg_hip_ctx *ctx, zg_hip_graph *graph);
 
 #ifdef __cplusplus
 }

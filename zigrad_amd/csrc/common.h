@@ -54,6 +54,13 @@ struct zg_hip_ctx {
     size_t scratch_bytes = 0;
     uint64_t n_device_allocs = 0;
 
+    // execution-graph capture (runtime.hip): while `capturing`, cache blocks that are freed are parked here
+    // instead of going back to the pool, so a replay never meets another owner at those addresses
+    bool capturing = false;
+    std::vector<std::pair<void*, uint64_t>> capture_parked;
+    int live_graphs = 0;
+    std::vector<void*> retired_ws;  // outgrown workspaces that an instantiated graph may still name
+
     // regions handed out by pool_map/alloc, for ownership checks at free time
     std::map<void*, size_t> raw_allocs;
     std::map<void*, size_t> host_allocs;
@@ -104,3 +111,12 @@ inline bool aligned16(const void* p) {
     } while (0)
 
 #define ZG_CTX(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
+
+// Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.
+#define ZG_NOT_CAPTURING(ctx, who)                                                                       \
+    do {                                                                                                 \
+        if ((ctx)->capturing) {                                                                          \
+            zg::set_error("%s: not allowed while an execution graph is being captured", who);            \
+            return ZG_HIP_ECAPTURE;                                                                      \
+        }                                                                                                \
+    } while (0)

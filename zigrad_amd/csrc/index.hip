@@ -405,6 +405,7 @@ ZG_API int zg_hip_gather_offsets(zg_hip_ctx* ctx, const uint64_t* src_shape, con
                        (int)rank, dim, gm, offsets, d_status);
     ZG_LAUNCH_CHECK();
     if (status) {
+        ZG_NOT_CAPTURING(ctx, "gather_offsets with a status read-back");
         int h = 0;
         ZG_HIP_TRY(hipMemcpyAsync(&h, d_status, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));

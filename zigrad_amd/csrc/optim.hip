@@ -55,9 +55,10 @@ __device__ __forceinline__ void adam_elem(float& p, float& g, float& m, float& v
 }
 
 template <bool CLIP>
-__global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float* m, float* v, size_t n, float lr_t,
-                                                       float b1, float b2, float omb1, float omb2, float eps,
-                                                       const float* factor) {
+__global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float* m, float* v, size_t n,
+                                                       float lr_t_value, const float* lr_t_ptr, float b1, float b2,
+                                                       float omb1, float omb2, float eps, const float* factor) {
+    const float lr_t = lr_t_ptr ? lr_t_ptr[0] : lr_t_value;
     const float f = CLIP ? factor[0] : 1.0f;
     const bool scale = CLIP && (f != 1.0f);
     const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
@@ -122,26 +123,51 @@ ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n,
     return ZG_HIP_OK;
 }
 
-ZG_API int zg_hip_adam_step(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n, uint64_t t,
-                            float lr, float beta1, float beta2, float epsilon, int clip, float max_norm, float delta) {
-    ZG_CTX(ctx);
-    if (n == 0) return ZG_HIP_OK;
-    ZG_REQUIRE(param && grad && m && v, "adam_step: null pointer");
-    ZG_REQUIRE(t >= 1, "adam_step: t must be >= 1");
-    // src/nn/optim.zig:190-191, fp32 throughout
+// src/nn/optim.zig:190-191, fp32 throughout
+static float adam_lr_t(float lr, float beta1, float beta2, uint64_t t) {
     const float tf = (float)t;
-    const float lr_t = lr * sqrtf(1.0f - powf(beta2, tf)) / (1.0f - powf(beta1, tf));
+    return lr * sqrtf(1.0f - powf(beta2, tf)) / (1.0f - powf(beta1, tf));
+}
+
+static int adam_launch(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n, float lr_t,
+                       const float* lr_t_ptr, float beta1, float beta2, float epsilon, int clip, float max_norm,
+                       float delta) {
     const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2;
     float* factor = ctx->scalar_slot + 1;
     if (clip) {
         int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
         if (rc) return rc;
         hipLaunchKernelGGL((adam_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, m,
-                           v, n, lr_t, beta1, beta2, omb1, omb2, epsilon, factor);
+                           v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, factor);
     } else {
         hipLaunchKernelGGL((adam_kernel<false>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad,
-                           m, v, n, lr_t, beta1, beta2, omb1, omb2, epsilon, factor);
+                           m, v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, factor);
     }
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_adam_step(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n, uint64_t t,
+                            float lr, float beta1, float beta2, float epsilon, int clip, float max_norm, float delta) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(param && grad && m && v, "adam_step: null pointer");
+    ZG_REQUIRE(t >= 1, "adam_step: t must be >= 1");
+    return adam_launch(ctx, param, grad, m, v, n, adam_lr_t(lr, beta1, beta2, t), nullptr, beta1, beta2, epsilon, clip,
+                       max_norm, delta);
+}
+
+ZG_API int zg_hip_adam_lr_t(float lr, float beta1, float beta2, uint64_t t, float* lr_t) {
+    ZG_REQUIRE(lr_t != nullptr && t >= 1, "adam_lr_t: null output or t < 1");
+    *lr_t = adam_lr_t(lr, beta1, beta2, t);
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n,
+                               const float* lr_t, float beta1, float beta2, float epsilon, int clip, float max_norm,
+                               float delta) {
+    ZG_CTX(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(param && grad && m && v && lr_t, "adam_step_at: null pointer");
+    return adam_launch(ctx, param, grad, m, v, n, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);
 }

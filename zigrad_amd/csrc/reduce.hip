@@ -19,8 +19,9 @@ __global__ __launch_bounds__(kBlock) void max_bwd_kernel(const float* x, float* 
 }
 
 // y += alpha[0] * x with alpha in device memory (src/device/host_device.zig:269-275)
-__global__ __launch_bounds__(kBlock) void axpy_kernel(const float* x, float* y, size_t n, const float* alpha_ptr) {
-    const float al = alpha_ptr[0];
+__global__ __launch_bounds__(kBlock) void axpy_kernel(const float* x, float* y, size_t n, const float* alpha_ptr,
+                                                       float alpha_value) {
+    const float al = alpha_ptr ? alpha_ptr[0] : alpha_value;
     const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
     size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
     if (vec) {
@@ -390,13 +391,9 @@ ZG_API int zg_hip_axpy(zg_hip_ctx* ctx, const float* x, float* y, size_t n, cons
     ZG_CTX(ctx);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x && y && alpha, "axpy: null pointer");
-    const float* dev_alpha = alpha;
-    if (!alpha_on_device) {
-        // stage the host scalar; the slot is reused only by later work on the same stream
-        ZG_HIP_TRY(hipMemcpyAsync(ctx->scalar_slot, alpha, sizeof(float), hipMemcpyHostToDevice, ctx->stream));
-        dev_alpha = ctx->scalar_slot;
-    }
-    hipLaunchKernelGGL(axpy_kernel, dim3(stream_grid(ctx, n, 8)), dim3(kBlock), 0, ctx->stream, x, y, n, dev_alpha);
+    // a host scalar travels as a kernel argument; a device scalar is read by the kernel
+    hipLaunchKernelGGL(axpy_kernel, dim3(stream_grid(ctx, n, 8)), dim3(kBlock), 0, ctx->stream, x, y, n,
+                       alpha_on_device ? alpha : (const float*)nullptr, alpha_on_device ? 0.f : alpha[0]);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

@@ -21,6 +21,11 @@ void set_error(const char* fmt, ...) {
 
 void* workspace(zg_hip_ctx* ctx, size_t bytes) {
     if (bytes <= ctx->ws_bytes) return ctx->ws;
+    if (ctx->capturing) {
+        set_error("workspace: needs to grow to %zu bytes while an execution graph is being captured; run the same "
+                  "ops once eagerly first", bytes);
+        return nullptr;
+    }
     // grow: nothing may still be reading the old buffer
     if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
         set_error("workspace: stream synchronize failed");
@@ -35,7 +40,11 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes) {
         return nullptr;
     }
     ctx->n_device_allocs++;
-    if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->ws) {
+        // an instantiated graph may have recorded the old address: keep it alive until the context goes
+        if (ctx->live_graphs > 0) ctx->retired_ws.push_back(ctx->ws);
+        else (void)hipFree(ctx->ws);
+    }
     ctx->ws = p;
     ctx->ws_bytes = want;
     return p;
@@ -74,6 +83,7 @@ struct BlockPool {
     }
 
     bool add_segment(zg_hip_ctx* ctx, size_t at_least) {
+        if (ctx->capturing) return false;  // no driver allocation inside a graph capture
         size_t bytes = segment_bytes;
         while (bytes < at_least) bytes *= 2;
         void* p = nullptr;
@@ -149,6 +159,10 @@ struct BlockPool {
     bool owns(void* ptr) const {
         return blocks.find((char*)ptr) != blocks.end();
     }
+    bool owns_live(void* ptr) const {
+        auto it = blocks.find((char*)ptr);
+        return it != blocks.end() && !it->second.free;
+    }
 
     void destroy() {
         for (void* s : segments) (void)hipFree(s);
@@ -171,6 +185,12 @@ static BlockPool* make_pool(size_t segment_bytes) {
 // ------------------------------------------------------------------------------------------------
 // small device kernels of the memory API
 // ------------------------------------------------------------------------------------------------
+template <class T>
+__global__ void copy_kernel(T* __restrict__ dst, const T* __restrict__ src, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += nt) dst[i] = src[i];
+}
+
 template <typename T>
 __global__ void fill_kernel(T* __restrict__ x, size_t n, T v) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -302,6 +322,7 @@ ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
     }
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    for (void* w : ctx->retired_ws) (void)hipFree(w);
     if (ctx->scalar_slot) (void)hipFree(ctx->scalar_slot);
     if (ctx->partials) (void)hipFree(ctx->partials);
     for (auto& kv : ctx->raw_allocs) (void)hipFree(kv.first);
@@ -313,7 +334,90 @@ ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
 
 ZG_API int zg_hip_sync(zg_hip_ctx* ctx) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "sync");
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// execution graphs (src/device/cuda_device.zig:558-611: open / save / run / free)
+// ------------------------------------------------------------------------------------------------
+struct zg_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<std::pair<void*, uint64_t>> parked;  // cache blocks freed inside the capture
+};
+
+static void unpark(zg_hip_ctx* ctx, std::vector<std::pair<void*, uint64_t>>& parked) {
+    for (auto& pb : parked) {
+        BlockPool* pool = pb.second == 2 ? ctx->large_pool : ctx->small_pool;
+        if (pool) (void)pool->release(pb.first);
+    }
+    parked.clear();
+}
+
+ZG_API int zg_hip_graph_open(zg_hip_ctx* ctx) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "graph_open");
+    ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    ZG_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_graph_save(zg_hip_ctx* ctx, zg_hip_graph** out) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(out != nullptr, "graph_save: null output");
+    *out = nullptr;
+    if (!ctx->capturing) {
+        set_error("graph_save: no capture in progress");
+        return ZG_HIP_ECAPTURE;
+    }
+    ctx->capturing = false;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+    if (e != hipSuccess || g == nullptr) {
+        (void)hipGetLastError();
+        unpark(ctx, ctx->capture_parked);
+        set_error("graph_save: hipStreamEndCapture failed: %s", hipGetErrorString(e));
+        return ZG_HIP_ERUNTIME;
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipGraphDestroy(g);
+        unpark(ctx, ctx->capture_parked);
+        set_error("graph_save: hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        return ZG_HIP_ERUNTIME;
+    }
+    zg_hip_graph* gr = new zg_hip_graph();
+    gr->graph = g;
+    gr->exec = exec;
+    gr->parked.swap(ctx->capture_parked);
+    ctx->live_graphs++;
+    *out = gr;
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_graph_run(zg_hip_ctx* ctx, zg_hip_graph* graph) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "graph_run");
+    ZG_REQUIRE(graph != nullptr && graph->exec != nullptr, "graph_run: null or unsaved graph");
+    ZG_HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_graph_free(zg_hip_ctx* ctx, zg_hip_graph* graph) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "graph_free");
+    if (!graph) return ZG_HIP_OK;
+    ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));  // a replay may still be running
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    unpark(ctx, graph->parked);
+    ctx->live_graphs--;
+    delete graph;
     return ZG_HIP_OK;
 }
 
@@ -344,6 +448,7 @@ ZG_API int zg_hip_event_create(zg_hip_ctx* ctx, zg_hip_event** out) {
 
 ZG_API int zg_hip_event_record(zg_hip_ctx* ctx, zg_hip_event* ev) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "event_record");
     ZG_REQUIRE(ev != nullptr, "event_record: null event");
     ZG_HIP_TRY(hipEventRecord(ev->ev, ctx->stream));
     return ZG_HIP_OK;
@@ -375,6 +480,7 @@ ZG_API int zg_hip_page_size(zg_hip_ctx* ctx, size_t* bytes) {
 
 static int raw_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, const char* who) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "alloc");
     ZG_REQUIRE(out != nullptr, "%s: null output", who);
     *out = nullptr;
     if (bytes == 0) return ZG_HIP_OK;
@@ -393,6 +499,7 @@ static int raw_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, const char* who)
 
 static int raw_free(zg_hip_ctx* ctx, void* ptr, const char* who) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "free");
     if (!ptr) return ZG_HIP_OK;
     auto it = ctx->raw_allocs.find(ptr);
     ZG_REQUIRE(it != ctx->raw_allocs.end(), "%s: pointer %p was not allocated by this context", who, ptr);
@@ -418,6 +525,7 @@ ZG_API int zg_hip_free(zg_hip_ctx* ctx, void* ptr) {
 
 ZG_API int zg_hip_host_alloc(zg_hip_ctx* ctx, size_t bytes, void** out) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "host_alloc");
     ZG_REQUIRE(out != nullptr, "host_alloc: null output");
     *out = nullptr;
     if (bytes == 0) return ZG_HIP_OK;
@@ -435,6 +543,7 @@ ZG_API int zg_hip_host_alloc(zg_hip_ctx* ctx, size_t bytes, void** out) {
 
 ZG_API int zg_hip_host_free(zg_hip_ctx* ctx, void* ptr) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "host_free");
     if (!ptr) return ZG_HIP_OK;
     auto it = ctx->host_allocs.find(ptr);
     ZG_REQUIRE(it != ctx->host_allocs.end(), "host_free: pointer %p was not allocated by this context", ptr);
@@ -468,6 +577,11 @@ ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uin
     if (!pool) pool = make_pool(large ? ctx->large_pool_bytes : ctx->small_pool_bytes);
     void* p = pool->alloc(ctx, bytes);
     if (!p) {
+        if (ctx->capturing) {
+            set_error("mem_cache_alloc: the pool would have to grow for %zu bytes while an execution graph is being "
+                      "captured; run the same ops once eagerly first", bytes);
+            return ZG_HIP_ECAPTURE;
+        }
         set_error("mem_cache_alloc: out of device memory for %zu bytes", bytes);
         return ZG_HIP_EOOM;
     }
@@ -481,6 +595,12 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     if (!ptr || block == 0) return ZG_HIP_OK;  // views and empty data: src/allocators/caching_allocator.zig:111-112
     ZG_REQUIRE(block == 1 || block == 2, "mem_cache_free: bad block handle %llu", (unsigned long long)block);
     BlockPool* pool = block == 2 ? ctx->large_pool : ctx->small_pool;
+    if (ctx->capturing) {
+        // the graph being recorded names this address: the block stays out of the pool until the graph is freed
+        ZG_REQUIRE(pool && pool->owns_live(ptr), "mem_cache_free: %p is not a live block of this pool", ptr);
+        ctx->capture_parked.push_back({ptr, block});
+        return ZG_HIP_OK;
+    }
     // Stream order makes reuse safe: a later op that receives this block runs after every op
     // already enqueued on the same stream.
     ZG_REQUIRE(pool && pool->release(ptr), "mem_cache_free: %p is not a live block of this pool", ptr);
@@ -491,6 +611,8 @@ ZG_API int zg_hip_mem_scratch(zg_hip_ctx* ctx, size_t bytes, void** out) {
     ZG_CTX(ctx);
     ZG_REQUIRE(out != nullptr, "mem_scratch: null output");
     if (bytes > ctx->scratch_bytes) {
+        ZG_NOT_CAPTURING(ctx, "mem_scratch (growing)");
+        ZG_REQUIRE(ctx->live_graphs == 0, "mem_scratch: cannot grow while an execution graph may name the old buffer");
         ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
         if (ctx->scratch) ZG_HIP_TRY(hipFree(ctx->scratch));
         ctx->scratch = nullptr;
@@ -511,6 +633,7 @@ ZG_API int zg_hip_mem_scratch(zg_hip_ctx* ctx, size_t bytes, void** out) {
 
 ZG_API int zg_hip_clear_cache(zg_hip_ctx* ctx) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "clear_cache");
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
     for (BlockPool** pp : {&ctx->small_pool, &ctx->large_pool}) {
         if (*pp) {
@@ -548,6 +671,7 @@ ZG_API int zg_hip_cache_stats(zg_hip_ctx* ctx, size_t* bytes_in_use, size_t* byt
 // ------------------------------------------------------------------------------------------------
 ZG_API int zg_hip_memcpy_h2d(zg_hip_ctx* ctx, void* dst, const void* src_host, size_t bytes) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "memcpy_h2d");
     if (bytes == 0) return ZG_HIP_OK;
     ZG_REQUIRE(dst && src_host, "memcpy_h2d: null pointer");
     // The caller may reuse or free a pageable source right after the call, so wait for the copy.
@@ -559,6 +683,7 @@ ZG_API int zg_hip_memcpy_h2d(zg_hip_ctx* ctx, void* dst, const void* src_host, s
 
 ZG_API int zg_hip_memcpy_d2h(zg_hip_ctx* ctx, void* dst_host, const void* src, size_t bytes) {
     ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "memcpy_d2h");
     if (bytes == 0) return ZG_HIP_OK;
     ZG_REQUIRE(dst_host && src, "memcpy_d2h: null pointer");
     ZG_HIP_TRY(hipMemcpyAsync(dst_host, src, bytes, hipMemcpyDefault, ctx->stream));
@@ -570,6 +695,19 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
     ZG_CTX(ctx);
     if (bytes == 0) return ZG_HIP_OK;
     ZG_REQUIRE(dst && src, "memcpy_d2d: null pointer");
+    if (ctx->capturing) {
+        // recorded as a kernel node like everything else in the graph
+        const bool v16 = aligned16(dst) && aligned16(src) && bytes % 16 == 0;
+        const size_t units = v16 ? bytes / 16 : bytes;
+        if (v16)
+            hipLaunchKernelGGL(copy_kernel<uint4>, dim3(grid_for(ctx, units, kBlock)), dim3(kBlock), 0, ctx->stream,
+                               (uint4*)dst, (const uint4*)src, units);
+        else
+            hipLaunchKernelGGL(copy_kernel<uint8_t>, dim3(grid_for(ctx, units, kBlock)), dim3(kBlock), 0, ctx->stream,
+                               (uint8_t*)dst, (const uint8_t*)src, units);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     ZG_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, ctx->stream));
     return ZG_HIP_OK;
 }

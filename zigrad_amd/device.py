@@ -87,6 +87,16 @@ class HipDevice:
     def event(self) -> "Event":
         return Event(self)
 
+    # -- execution graphs (src/device/cuda_device.zig:558-611: open / save / run / free) -----------
+    def graph_open(self) -> None:
+        """Start recording: until graph_save() every op call is captured instead of executed."""
+        self._call("zg_hip_graph_open")
+
+    def graph_save(self) -> "Graph":
+        h = ctypes.c_void_p()
+        self._call("zg_hip_graph_save", ctypes.byref(h))
+        return Graph(self, h)
+
     # -- memory API (src/device/device_reference.zig:29-123) -----------------------------------
     def mem_alloc(self, dtype, n: int) -> DevBuf:
         dtype = np.dtype(dtype)
@@ -383,6 +393,31 @@ class HipDevice:
     def _op_adam_step(self, param, grad, m, v, t, lr, beta1, beta2, epsilon, clip, max_norm, delta):
         self._call("zg_hip_adam_step", param.ptr, grad.ptr, m.ptr, v.ptr, param.n, int(t), lr, beta1, beta2, epsilon,
                    int(clip), max_norm, delta)
+
+    def _op_adam_step_at(self, param, grad, m, v, lr_t, beta1, beta2, epsilon, clip, max_norm, delta):
+        """Adam update whose lr_t is read from `lr_t` (a one-float buffer) when the kernel runs."""
+        self._call("zg_hip_adam_step_at", param.ptr, grad.ptr, m.ptr, v.ptr, param.n, lr_t.ptr, beta1, beta2, epsilon,
+                   int(clip), max_norm, delta)
+
+    def adam_lr_t(self, lr, beta1, beta2, t) -> float:
+        out = ctypes.c_float()
+        self._lib.call("zg_hip_adam_lr_t", lr, beta1, beta2, int(t), ctypes.byref(out))
+        return out.value
+
+
+class Graph:
+    """A captured op sequence; run() replays it on the device's stream."""
+
+    def __init__(self, dev: HipDevice, handle):
+        self._dev, self._h = dev, handle
+
+    def run(self) -> None:
+        self._dev._call("zg_hip_graph_run", self._h)
+
+    def free(self) -> None:
+        if self._h is not None:
+            self._dev._call("zg_hip_graph_free", self._h)
+            self._h = None
 
 
 class Event:

@@ -13,6 +13,8 @@ src/nn/loss.zig:130-171 (softmax cross-entropy), src/nn/optim.zig:46-58, 100-122
 """
 from __future__ import annotations
 
+import ctypes
+
 import numpy as np
 
 from . import host
@@ -60,6 +62,9 @@ class Optimizer:
         self.params: list[tuple[DevBuf, DevBuf]] = []
         self.state: list[tuple[DevBuf, DevBuf]] = []
         self.t = 0  # Adam's counter: incremented once per parameter tensor update (src/nn/optim.zig:189)
+        self.capturing = False  # set while a trainer records its step into an execution graph
+        self.lr_slots = None    # Adam under replay: one lr_t per tensor in pinned host memory the kernels read
+        self._lr_view = None
 
     def attach(self, param: DevBuf, grad: DevBuf) -> None:
         self.params.append((param, grad))
@@ -69,16 +74,79 @@ class Optimizer:
             self.dev.mem_fill(v, 0.0)
             self.state.append((m, v))
 
+    def begin_capture(self) -> None:
+        """Before recording a step: Adam's lr_t changes every step, so the recorded kernels read it from memory."""
+        if self.kind == "adam" and self.lr_slots is None:
+            n = len(self.params)
+            self.lr_slots = self.dev.mem_alloc_host(F32, n)
+            self._lr_view = np.ctypeslib.as_array((ctypes.c_float * n).from_address(self.lr_slots.ptr))
+        self.capturing = True
+
+    def prepare_replay(self) -> None:
+        """Host part of one replayed step: advance the per-tensor counter and publish each tensor's lr_t.
+        The previous replay must have finished (the trainers read the loss back every step)."""
+        if self.kind != "adam":
+            return
+        for i in range(len(self.params)):
+            self.t += 1
+            self._lr_view[i] = self.dev.adam_lr_t(self.lr, self.beta1, self.beta2, self.t)
+
     def step(self) -> None:
         d = self.dev
         for i, (p, g) in enumerate(self.params):
             if self.kind == "sgd":
                 d.dispatch("sgd_step", param=p, grad=g, lr=self.lr, clip=self.clip, max_norm=self.max_norm, delta=self.delta)
+            elif self.capturing:
+                m, v = self.state[i]
+                d.dispatch("adam_step_at", param=p, grad=g, m=m, v=v, lr_t=self.lr_slots.sub(i, 1), beta1=self.beta1,
+                           beta2=self.beta2, epsilon=self.epsilon, clip=self.clip, max_norm=self.max_norm, delta=self.delta)
             else:
                 self.t += 1
                 m, v = self.state[i]
                 d.dispatch("adam_step", param=p, grad=g, m=m, v=v, t=self.t, lr=self.lr, beta1=self.beta1, beta2=self.beta2,
                            epsilon=self.epsilon, clip=self.clip, max_norm=self.max_norm, delta=self.delta)
+
+
+class GraphSteps:
+    """capture() / step_graph() for trainers whose step() touches the host only to read the loss: the step is
+    recorded once as an execution graph (src/device/cuda_device.zig:558-611) and replayed with one launch."""
+
+    graph = None
+    graph_loss = None
+    _capturing = False
+
+    def _read_loss(self, loss: DevBuf):
+        if self._capturing:  # nothing executes while recording: remember where the loss will be
+            self.graph_loss = DevBuf(loss.ptr, 1, loss.dtype, 0, "view")
+            return None
+        self.dev.mem_transfer(loss, self.loss_host, "DtoH")
+        return float(self.loss_host[0])
+
+    def capture(self) -> None:
+        """Record one step.  Run at least one eager step first, so that the allocator and the library's internal
+        workspace have reached their final size (growing either is refused while recording)."""
+        self.optim.begin_capture()
+        self.dev.graph_open()
+        self._capturing = True
+        try:
+            self.step()
+        finally:
+            self._capturing = False
+            self.optim.capturing = False
+            self.graph = self.dev.graph_save()
+
+    def step_graph(self, read_loss: bool = True):
+        self.optim.prepare_replay()
+        self.graph.run()
+        if not read_loss:
+            return None
+        self.dev.mem_transfer(self.graph_loss, self.loss_host, "DtoH")
+        return float(self.loss_host[0])
+
+    def free_graph(self) -> None:
+        if self.graph is not None:
+            self.graph.free()
+            self.graph = None
 
 
 class MLP:
@@ -161,7 +229,7 @@ class MLP:
             g = g_prev
 
 
-class MLPTrainer:
+class MLPTrainer(GraphSteps):
     """Linear -> ReLU -> ... -> Linear -> softmax cross-entropy, one train step per `step()` call.
 
     loss_mode "onehot" is the reference's loss (float one-hot targets, probabilities kept for backward);
@@ -206,10 +274,7 @@ class MLPTrainer:
         else:
             saved = d.mem_cache_alloc(F32, B)  # per-row log-sum-exp
             d.dispatch("smce_label_fwd", logits=logits, labels=self.labels, lse=saved, loss=loss, rows=B, cols=C)
-        loss_val = None
-        if read_loss:
-            d.mem_transfer(loss, self.loss_host, "DtoH")  # loss.get(0): a blocking read before backward
-            loss_val = float(self.loss_host[0])
+        loss_val = self._read_loss(loss) if read_loss else None  # loss.get(0): a blocking read before backward
 
         # backward
         loss_grad = d.mem_cache_alloc(F32, 1)
@@ -243,7 +308,7 @@ def dqn_inputs(batch=64, state_dim=4, n_actions=2, seed=0):
     }
 
 
-class DQNTrainer:
+class DQNTrainer(GraphSteps):
     """One DQN update per `step()`: TD target from a frozen copy of the network, Q(s,a) through gather,
     smooth-L1 loss, Adam.  Op order follows DQNAgent.train (examples/dqn/src/dqn_agent.zig:125-228) without
     its host-side clamps, on the network 4 -> 128 -> 128 -> 2."""
@@ -318,9 +383,9 @@ class DQNTrainer:
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.policy.grad_buffers()]
         self.optim.step()
-        d.mem_transfer(loss, self.loss_host, "DtoH")
+        loss_val = self._read_loss(loss)
         d.mem_cache_free(loss)
-        return float(self.loss_host[0])
+        return loss_val
 
 
 def gcn_inputs(n_nodes=2708, n_features=1433, n_pairs=5278, n_classes=7, n_train=140, hidden=16, seed=0):

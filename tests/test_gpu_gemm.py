@@ -41,6 +41,8 @@ SHAPES = [
     (64, 128, 784), (64, 64, 128), (64, 10, 64), (64, 128, 4), (64, 2, 128), (128, 784, 64), (10, 64, 64),
     (2708, 16, 1433), (2708, 7, 16), (16, 1433, 2708), (1, 1, 1), (33, 65, 17), (129, 257, 31), (256, 128, 16),
     (512, 384, 160), (300, 500, 70), (1024, 1024, 256),
+    # few C tiles and a deep k: the split-k path, whole tiles (fast kernels) and ragged
+    (128, 64, 2048), (64, 64, 4096), (70, 50, 1000),
 ]
 
 
@@ -141,6 +143,25 @@ def test_bmm_acc_batches(oracle, hip, nba, nbb, nbc):
     assert rel_fro(res[1], res[0]) <= TOL
     truth = np.stack([A[i % nba].astype(np.float64) @ B[i % nbb].astype(np.float64) for i in range(nbc)]) + C0
     assert rel_fro(res[1], truth) <= TOL
+
+
+def test_bmm_acc_split_k_batches(oracle, hip):
+    """Batched products with few C tiles and a deep k take the split-k path: partial products per batch and split."""
+    nb, m, n, k = 3, 64, 48, 1536
+    r = rng(7)
+    A = r.standard_normal((nb, m, k)).astype(np.float32)
+    B = r.standard_normal((1, n, k)).astype(np.float32)  # one B shared by all batches, stored transposed
+    C0 = r.standard_normal((nb, m, n)).astype(np.float32)
+    res = []
+    for dev in (oracle, hip):
+        a, b, c = dev.from_numpy(A), dev.from_numpy(B), dev.from_numpy(C0)
+        dev.dispatch("bmm_acc", A=a, B=b, C=c, A_shape=[nb, m, k], B_shape=[1, k, n], C_shape=[nb, m, n], trans_a=False,
+                     trans_b=True, lda=k, ldb=k, ldc=n, alpha=0.5, beta=1.0)
+        dev.sync()
+        res.append(dev.to_numpy(c).reshape(nb, m, n))
+    truth = 0.5 * np.stack([A[i].astype(np.float64) @ B[0].astype(np.float64).T for i in range(nb)]) + C0
+    assert rel_fro(res[1], truth) <= TOL
+    assert rel_fro(res[1], res[0]) <= TOL
 
 
 def test_bmm_32x512_cubed(oracle, hip):

@@ -166,6 +166,9 @@ struct GemmArgs {
     size_t nba, nbb;
     size_t a_chunk, b_chunk, c_chunk;
     unsigned tiles_m, tiles_n;
+    // split-K: workgroup y handles k-tiles [y * split_tiles, (y + 1) * split_tiles) and writes its C tile at
+    // C + y * split_stride (the launcher points C at a buffer of partial products); one split = the whole of k
+    size_t split_tiles, split_stride;
     int a_vec, b_vec;  // 16-byte vector loads are legal for this operand
 };
 
@@ -204,7 +207,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     const size_t z = blockIdx.z;
     const float* A = g.A + (z % g.nba) * g.a_chunk;
     const float* B = g.B + (z % g.nbb) * g.b_chunk;
-    float* C = g.C + z * g.c_chunk;
+    float* C = g.C + z * g.c_chunk + (size_t)blockIdx.y * g.split_stride;
     const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -219,7 +222,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    const size_t KT = (g.K + BK - 1) / BK;
+    // this workgroup's range of k
+    const size_t k_begin = (size_t)blockIdx.y * g.split_tiles * BK;
+    const size_t k_end = (k_begin + g.split_tiles * BK < g.K) ? k_begin + g.split_tiles * BK : g.K;
+    const size_t KT = (k_end - k_begin + BK - 1) / BK;
     constexpr int NM = TM * TN;         // MFMAs per step
     constexpr int NMF = 4 * NM;         // MFMAs per k-group
     constexpr int NR = FA::N + FB::N;   // fragment reads per k-group
@@ -247,10 +253,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         constexpr int S = decltype(slot_tag)::value;
         if (v < TA::NV) {
             if (!SAFE) ta[S].load_fast(v, a_org + (A_KMAJOR ? k0 : k0 * g.lda), a_off[v]);
-            else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, g.K, g.a_vec != 0);
+            else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
         } else {
             if (!SAFE) tb[S].load_fast(v - TA::NV, b_org + (B_KMAJOR ? k0 : k0 * g.ldb), b_off[v - TA::NV]);
-            else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, g.K, g.b_vec != 0);
+            else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
         }
     };
     auto store_op = [&](auto slot_tag, int w, int buf) {
@@ -282,7 +288,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         constexpr int S = decltype(parity_tag)::value;  // kt % 2: LDS buffer and register slot of this tile
         using SCur = std::integral_constant<int, S>;
         using SNext = std::integral_constant<int, S ^ 1>;
-        const size_t k_load = (SAFE || kt + 2 < KT) ? (kt + 2) * BK : (KT - 1) * BK;
+        const size_t k_load = k_begin + ((SAFE || kt + 2 < KT) ? (kt + 2) * BK : (KT - 1) * BK);
 #pragma unroll
         for (int grp = 0; grp < 2; grp++) {
 #pragma unroll
@@ -315,9 +321,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 
     // prologue: tile 0 goes straight to LDS buffer 0, tile 1 starts its flight in slot 1
 #pragma unroll
-    for (int v = 0; v < NL; v++) load_op(P0{}, v, 0);
+    for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin);
 #pragma unroll
-    for (int v = 0; v < NL; v++) load_op(P1{}, v, (SAFE || KT > 1) ? BK : 0);
+    for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0));
 #pragma unroll
     for (int w = 0; w < NL; w++) store_op(P0{}, w, 0);
     __syncthreads();
@@ -411,7 +417,8 @@ template <int BM, int BN>
 static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, bool safe, size_t batches) {
     g.tiles_m = (unsigned)ceil_div_sz(g.M, BM);
     g.tiles_n = (unsigned)ceil_div_sz(g.N, BN);
-    dim3 grid(g.tiles_m * g.tiles_n, 1, (unsigned)batches), block(kGemmThreads);
+    const size_t kt_total = ceil_div_sz(g.K, kBK);
+    dim3 grid(g.tiles_m * g.tiles_n, (unsigned)ceil_div_sz(kt_total, g.split_tiles), (unsigned)batches), block(kGemmThreads);
 #define ZG_GEMM(AK, BKM, SF)                                                                                  \
     do {                                                                                                      \
         constexpr size_t lds_bytes = 2 * (size_t)(Tile<BM, AK>::ELEMS + Tile<BN, BKM>::ELEMS) * sizeof(float); \
@@ -432,6 +439,23 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
 #undef ZG_GEMM
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
+}
+
+// C = alpha * (sum of the split-K partial products, in split order) + beta * C.  P is [batch][split][M][N] dense.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, float* C, size_t M, size_t N, size_t ldc,
+                                                            int splits, float alpha, float beta, size_t c_chunk) {
+    const size_t z = blockIdx.z;
+    const float* p = P + z * (size_t)splits * M * N;
+    float* c = C + z * c_chunk;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (; i < M * N; i += nt) {
+        float acc = p[i];
+        for (int s = 1; s < splits; s++) acc += p[(size_t)s * M * N + i];
+        const size_t r = i / N, col = i % N;
+        float v = alpha * acc;
+        if (beta != 0.f) v += beta * c[r * ldc + col];
+        c[r * ldc + col] = v;
+    }
 }
 
 // C *= beta (or 0) when k == 0 or alpha == 0: BLAS leaves beta*C
@@ -500,10 +524,48 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     auto cost = [&](size_t bm, size_t bn, double eff) {
         return (double)ceil_div_sz(tiles(bm, bn), n_cu) * (double)(bm * bn) / eff;
     };
+    const size_t kt_total = ceil_div_sz(k, kBK);
+    g.split_tiles = kt_total;
+    g.split_stride = 0;
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
     if (c_large <= c_mid && c_large <= c_small)
         return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, !fast(256, 128), batches);
     if (c_mid <= c_small) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, !fast(128, 128), batches);
+    // A deep product with too few C tiles to give every CU a workgroup: split k over several workgroups per tile
+    // (an even number of k-tiles each), let each write its partial tile to the workspace, and add the partials in
+    // split order in a second kernel.  The order is fixed, so the result does not depend on scheduling.
+    const size_t t64 = tiles(64, 64);
+    if (t64 < n_cu && kt_total >= 16) {
+        size_t splits = ceil_div_sz(2 * n_cu, t64);
+        if (splits > kt_total / 4) splits = kt_total / 4;
+        if (splits > 64) splits = 64;
+        size_t per = ceil_div_sz(kt_total, splits);
+        per += per & 1;
+        splits = ceil_div_sz(kt_total, per);
+        if (splits >= 2) {
+            float* part = (float*)workspace(ctx, batches * splits * m * n * sizeof(float));
+            if (!part) return ZG_HIP_EOOM;
+            GemmArgs gs = g;
+            gs.C = part;
+            gs.ldc = n;
+            gs.c_chunk = splits * m * n;
+            gs.split_tiles = per;
+            gs.split_stride = m * n;
+            gs.alpha = 1.f;
+            gs.beta = 0.f;
+            const bool part_vec = n % 4 == 0 && (m * n) % 4 == 0;  // the workspace itself is 256-byte aligned
+            const bool fast_split = g.a_vec && g.b_vec && part_vec && small_ld && m % 64 == 0 && n % 64 == 0 &&
+                                    k % (2 * kBK) == 0;
+            int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, !fast_split, batches);
+            if (rc) return rc;
+            size_t blocks = ceil_div_sz(m * n, 256);
+            if (blocks > 2048) blocks = 2048;
+            hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks, 1, (unsigned)batches), dim3(256), 0,
+                               ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk);
+            ZG_LAUNCH_CHECK();
+            return ZG_HIP_OK;
+        }
+    }
     return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, !fast(64, 64), batches);
 }
 

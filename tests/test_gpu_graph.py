@@ -82,6 +82,24 @@ def test_dqn_replays_equal_eager_steps(hip):
     tr.free_graph()
 
 
+def test_gcn_replays_equal_eager_steps(hip):
+    from zigrad_amd.trainers import GCNTrainer, gcn_inputs
+
+    inp = gcn_inputs(n_nodes=600, n_features=200, n_pairs=1500, n_classes=7, n_train=60, hidden=16, seed=1)
+    eager = GCNTrainer(hip, inp, lr=0.01, clip=True)
+    want = [eager.step() for _ in range(8)]
+    tr = GCNTrainer(hip, inp, lr=0.01, clip=True)
+    got = [tr.step() for _ in range(2)]
+    tr.capture()
+    for _ in range(6):
+        got.append(tr.step_graph())
+        _eager_noise(hip)
+    assert got == want
+    for p, q in zip(eager.param_buffers(), tr.param_buffers()):
+        assert np.array_equal(hip.to_numpy(p), hip.to_numpy(q))
+    tr.free_graph()
+
+
 def test_calls_that_cannot_be_recorded_are_refused(hip):
     a = hip.from_numpy(np.ones(16, np.float32), cached=True)
     hip.graph_open()

@@ -19,6 +19,7 @@ struct Plan {
     uint32_t* cursor;    // nb
     uint32_t* perm_tmp;  // n
     uint32_t* perm;      // n
+    uint32_t* peer;      // n: optional payload (the other endpoint of an edge) in the order of perm
     uint32_t* tile_sums; // scan scratch
     size_t n, nb;
 };
@@ -31,7 +32,7 @@ static size_t align_up(size_t v, size_t a) {
 
 static size_t plan_bytes(size_t n, size_t nb) {
     size_t tiles = ceil_div_sz(nb + 1, kScanTile);
-    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 2 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256);
+    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 3 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256);
 }
 
 static Plan carve_plan(void* mem, size_t n, size_t nb) {
@@ -46,6 +47,8 @@ static Plan carve_plan(void* mem, size_t n, size_t nb) {
     pl.perm_tmp = (uint32_t*)p;
     p += align_up(n * 4, 256);
     pl.perm = (uint32_t*)p;
+    p += align_up(n * 4, 256);
+    pl.peer = (uint32_t*)p;
     p += align_up(n * 4, 256);
     pl.tile_sums = (uint32_t*)p;
     return pl;
@@ -97,6 +100,40 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(uint32_t* data, size_t 
     if (threadIdx.x == 255) tile_sums[blockIdx.x] = wave_off + inc;
 }
 
+// exclusive scan of a short array by one workgroup, 2048 elements per round with a running carry
+__global__ __launch_bounds__(256) void scan_single_kernel(uint32_t* data, size_t n) {
+    __shared__ uint32_t wave_tot[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t carry = 0;
+    for (size_t c = 0; c < n; c += kScanTile) {
+        const size_t base = c + (size_t)threadIdx.x * 8;
+        uint32_t v[8], s = 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = (base + k < n) ? data[base + k] : 0;
+            s += v[k];
+        }
+        uint32_t inc = s;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            uint32_t t = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += t;
+        }
+        __syncthreads();  // wave_tot of the previous round has been read by everyone
+        if (lane == 63) wave_tot[wave] = inc;
+        __syncthreads();
+        uint32_t wave_off = carry;
+        for (int w = 0; w < wave; w++) wave_off += wave_tot[w];
+        uint32_t run = wave_off + inc - s;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            if (base + k < n) data[base + k] = run;
+            run += v[k];
+        }
+        carry += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+    }
+}
+
 __global__ __launch_bounds__(256) void scan_sums_kernel(uint32_t* tile_sums, size_t tiles) {
     // one workgroup walks the tile sums in chunks of 256, carrying the running total
     __shared__ uint32_t wave_tot[4];
@@ -145,8 +182,10 @@ __global__ void place_kernel(const uint64_t* keys, size_t n, size_t nb, const ui
 
 // Put each bucket back into ascending input position: rank of an entry = number of smaller entries
 // in its bucket.  One wave per bucket.
+// With `payload` (the other index array of an edge list, possibly in host memory) the kernel also lays the payload
+// out in the same order, so that the apply kernels read it from device memory next to perm.
 __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
-                                                              uint32_t* perm) {
+                                                              uint32_t* perm, const uint64_t* payload, uint32_t* peer) {
     const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= nb) return;
     const int lane = threadIdx.x & 63;
@@ -156,10 +195,14 @@ __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row
         uint32_t rank = 0;
         for (uint32_t j = 0; j < len; j++) rank += (perm_tmp[s + j] < id) ? 1u : 0u;
         perm[s + rank] = id;
+        if (payload) {
+            const uint64_t v = payload[id];
+            peer[s + rank] = v < 0xffffffffull ? (uint32_t)v : 0xffffffffu;
+        }
     }
 }
 
-static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl) {
+static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, const uint64_t* payload = nullptr) {
     hipStream_t st = ctx->stream;
     const size_t n = pl.n, nb = pl.nb;
     const int g_n = (int)(ceil_div_sz(n ? n : 1, 256) > 4096 ? 4096 : ceil_div_sz(n ? n : 1, 256));
@@ -171,9 +214,12 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl) {
         ZG_LAUNCH_CHECK();
     }
     const size_t tiles = ceil_div_sz(nb + 1, kScanTile);
-    hipLaunchKernelGGL(scan_tiles_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
-    ZG_LAUNCH_CHECK();
-    if (tiles > 1) {
+    if (tiles <= 8) {
+        hipLaunchKernelGGL(scan_single_kernel, dim3(1), dim3(256), 0, st, pl.row_ptr, nb + 1);
+        ZG_LAUNCH_CHECK();
+    } else {
+        hipLaunchKernelGGL(scan_tiles_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
+        ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, pl.tile_sums, tiles);
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(scan_add_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
@@ -183,7 +229,7 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl) {
         hipLaunchKernelGGL(place_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr, pl.cursor, pl.perm_tmp);
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(nb, 4)), dim3(256), 0, st, pl.row_ptr, nb,
-                           pl.perm_tmp, pl.perm);
+                           pl.perm_tmp, pl.perm, payload, pl.peer);
         ZG_LAUNCH_CHECK();
     }
     return ZG_HIP_OK;
@@ -223,11 +269,13 @@ __global__ __launch_bounds__(256) void row_scatter_apply_kernel(const float* src
     }
 }
 
-// dst[t, :] += (deg[s] * deg[t]) * h[s, :] over the edges into t, in edge order
+// dst[t, :] += (deg[s] * deg[t]) * h[s, :] over the edges into t, in edge order.  `peer` holds the source of each
+// edge in that order; four edges are loaded at a time (the loads do not depend on the running sum) and then added
+// one after the other.
 template <int G>
 __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const float* h, const float* deg,
-                                                             const uint64_t* src_idx, const uint32_t* row_ptr,
-                                                             const uint32_t* perm, size_t n_nodes, size_t stride) {
+                                                             const uint32_t* row_ptr, const uint32_t* peer,
+                                                             size_t n_nodes, size_t stride) {
     const size_t t = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     if (t >= n_nodes) return;
     const int lane = threadIdx.x % G;
@@ -236,21 +284,30 @@ __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const fl
     const float dt = deg[t];
     for (size_t j = lane; j < stride; j += G) {
         float acc = dst[t * stride + j];
-        for (uint32_t k = s0; k < s1; k++) {
-            const uint64_t s = src_idx[perm[k]];
-            if (s >= n_nodes) continue;
-            const float w = __fmul_rn(deg[s], dt);
-            acc = __fadd_rn(acc, __fmul_rn(w, h[s * stride + j]));
+        for (uint32_t k = s0; k < s1; k += 4) {
+            uint32_t sv[4];
+            float dv[4], hv[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) sv[u] = (k + u < s1) ? peer[k + u] : 0xffffffffu;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const bool ok = sv[u] < n_nodes;
+                dv[u] = ok ? deg[sv[u]] : 0.f;
+                hv[u] = ok ? h[(size_t)sv[u] * stride + j] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (sv[u] < n_nodes) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(dv[u], dt), hv[u]));
         }
         dst[t * stride + j] = acc;
     }
 }
 
-// grad_h[s, :] += (go[t, :] * deg[s]) * deg[t] over the edges out of s, in edge order
+// grad_h[s, :] += (go[t, :] * deg[s]) * deg[t] over the edges out of s, in edge order; `peer` holds the targets
 template <int G>
 __global__ __launch_bounds__(256) void gcn_bwd_gradh_kernel(float* grad_h, const float* go, const float* deg,
-                                                             const uint64_t* tgt_idx, const uint32_t* row_ptr,
-                                                             const uint32_t* perm, size_t n_nodes, size_t stride) {
+                                                             const uint32_t* row_ptr, const uint32_t* peer,
+                                                             size_t n_nodes, size_t stride) {
     const size_t s = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     if (s >= n_nodes) return;
     const int lane = threadIdx.x % G;
@@ -259,10 +316,20 @@ __global__ __launch_bounds__(256) void gcn_bwd_gradh_kernel(float* grad_h, const
     const float ds = deg[s];
     for (size_t j = lane; j < stride; j += G) {
         float acc = grad_h[s * stride + j];
-        for (uint32_t k = s0; k < s1; k++) {
-            const uint64_t t = tgt_idx[perm[k]];
-            if (t >= n_nodes) continue;
-            acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(go[t * stride + j], ds), deg[t]));
+        for (uint32_t k = s0; k < s1; k += 4) {
+            uint32_t tv[4];
+            float dv[4], gv[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) tv[u] = (k + u < s1) ? peer[k + u] : 0xffffffffu;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const bool ok = tv[u] < n_nodes;
+                dv[u] = ok ? deg[tv[u]] : 0.f;
+                gv[u] = ok ? go[(size_t)tv[u] * stride + j] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (tv[u] < n_nodes) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(gv[u], ds), dv[u]));
         }
         grad_h[s * stride + j] = acc;
     }
@@ -486,11 +553,11 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const floa
     void* mem = workspace(ctx, plan_bytes(n_edge, n_nodes));
     if (!mem) return ZG_HIP_EOOM;
     Plan pl = carve_plan(mem, n_edge, n_nodes);
-    if (int rc = build_plan(ctx, tgt_indices, pl)) return rc;
+    if (int rc = build_plan(ctx, tgt_indices, pl, src_indices)) return rc;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
-                                        src_indices, pl.row_ptr, pl.perm, n_nodes, stride));
+                                        pl.row_ptr, pl.peer, n_nodes, stride));
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
@@ -512,12 +579,12 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     Plan by_tgt = carve_plan(mem + pb, n_edge, n_nodes);
     float* term_src = (float*)(mem + 2 * pb);
     float* term_tgt = (float*)(mem + 2 * pb + tb);
-    if (int rc = build_plan(ctx, src_indices, by_src)) return rc;
+    if (int rc = build_plan(ctx, src_indices, by_src, tgt_indices)) return rc;
     if (int rc = build_plan(ctx, tgt_indices, by_tgt)) return rc;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
-                                        grad_output, deg, tgt_indices, by_src.row_ptr, by_src.perm, n_nodes, stride));
+                                        grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride));
     ZG_LAUNCH_CHECK();
     hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
                        grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride, term_src, term_tgt);

@@ -408,7 +408,7 @@ def gcn_inputs(n_nodes=2708, n_features=1433, n_pairs=5278, n_classes=7, n_train
             "dims": [n_features, hidden, n_classes]}
 
 
-class GCNTrainer:
+class GCNTrainer(GraphSteps):
     """Two GraphConv layers (GEMM, degree-scaled scatter, bias) with ReLU between, masked softmax
     cross-entropy, Adam: the op sequence of examples/gcn/src/model.zig:27-36, 100-224 and main.zig:68-84.
     The labelled nodes are the first `n_train` rows (MaskLayer.backward indexes the masked gradient by node
@@ -508,7 +508,7 @@ class GCNTrainer:
         d.mem_copy(s2["y"].sub(0, M * C), out_m)
         probs, loss = d.mem_cache_alloc(F32, M * C), d.mem_cache_alloc(F32, 1)
         d.dispatch("smce_fwd", logits=out_m, target=self.label_m, probs=probs, loss=loss, rows=M, cols=C)
-        d.mem_transfer(loss, self.loss_host, "DtoH")
+        loss_val = self._read_loss(loss)
         # backward
         loss_grad = d.mem_cache_alloc(F32, 1)
         d.mem_fill(loss_grad, 1.0)
@@ -528,4 +528,4 @@ class GCNTrainer:
         self.optim.step()
         for gb in self.grad_buffers():
             d.mem_fill(gb, 0.0)
-        return float(self.loss_host[0])
+        return loss_val

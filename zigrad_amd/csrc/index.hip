@@ -20,6 +20,7 @@ struct Plan {
     uint32_t* perm_tmp;  // n
     uint32_t* perm;      // n
     uint32_t* peer;      // n: optional payload (the other endpoint of an edge) in the order of perm
+    uint32_t* peer_tmp;  // n: the payload in the order of perm_tmp
     uint32_t* tile_sums; // scan scratch
     size_t n, nb;
 };
@@ -32,7 +33,7 @@ static size_t align_up(size_t v, size_t a) {
 
 static size_t plan_bytes(size_t n, size_t nb) {
     size_t tiles = ceil_div_sz(nb + 1, kScanTile);
-    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 3 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256);
+    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 4 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256);
 }
 
 static Plan carve_plan(void* mem, size_t n, size_t nb) {
@@ -49,6 +50,8 @@ static Plan carve_plan(void* mem, size_t n, size_t nb) {
     pl.perm = (uint32_t*)p;
     p += align_up(n * 4, 256);
     pl.peer = (uint32_t*)p;
+    p += align_up(n * 4, 256);
+    pl.peer_tmp = (uint32_t*)p;
     p += align_up(n * 4, 256);
     pl.tile_sums = (uint32_t*)p;
     return pl;
@@ -168,24 +171,29 @@ __global__ __launch_bounds__(256) void scan_add_kernel(uint32_t* data, size_t n,
         if (base + k < n) data[base + k] += off;
 }
 
+// `payload` (the other index array of an edge list, possibly in host memory) is read here, in input order and
+// coalesced, and travels with its entry from then on in device memory.
 __global__ void place_kernel(const uint64_t* keys, size_t n, size_t nb, const uint32_t* row_ptr, uint32_t* cursor,
-                             uint32_t* perm_tmp) {
+                             uint32_t* perm_tmp, const uint64_t* payload, uint32_t* peer_tmp) {
     size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
     for (; e < n; e += nt) {
         uint64_t k = keys[e];
         if (k < nb) {
             uint32_t pos = row_ptr[k] + atomicAdd(&cursor[k], 1u);
             perm_tmp[pos] = (uint32_t)e;
+            if (payload) {
+                const uint64_t v = payload[e];
+                peer_tmp[pos] = v < 0xffffffffull ? (uint32_t)v : 0xffffffffu;
+            }
         }
     }
 }
 
 // Put each bucket back into ascending input position: rank of an entry = number of smaller entries
 // in its bucket.  One wave per bucket.
-// With `payload` (the other index array of an edge list, possibly in host memory) the kernel also lays the payload
-// out in the same order, so that the apply kernels read it from device memory next to perm.
+// With `peer_tmp` the payload is laid out in the same order, so that the apply kernels read it next to perm.
 __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
-                                                              uint32_t* perm, const uint64_t* payload, uint32_t* peer) {
+                                                              uint32_t* perm, const uint32_t* peer_tmp, uint32_t* peer) {
     const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= nb) return;
     const int lane = threadIdx.x & 63;
@@ -195,10 +203,7 @@ __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row
         uint32_t rank = 0;
         for (uint32_t j = 0; j < len; j++) rank += (perm_tmp[s + j] < id) ? 1u : 0u;
         perm[s + rank] = id;
-        if (payload) {
-            const uint64_t v = payload[id];
-            peer[s + rank] = v < 0xffffffffull ? (uint32_t)v : 0xffffffffu;
-        }
+        if (peer_tmp) peer[s + rank] = peer_tmp[s + i];
     }
 }
 
@@ -226,10 +231,11 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
         ZG_LAUNCH_CHECK();
     }
     if (n) {
-        hipLaunchKernelGGL(place_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr, pl.cursor, pl.perm_tmp);
+        hipLaunchKernelGGL(place_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr, pl.cursor, pl.perm_tmp, payload,
+                           pl.peer_tmp);
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(nb, 4)), dim3(256), 0, st, pl.row_ptr, nb,
-                           pl.perm_tmp, pl.perm, payload, pl.peer);
+                           pl.perm_tmp, pl.perm, payload ? pl.peer_tmp : (const uint32_t*)nullptr, pl.peer);
         ZG_LAUNCH_CHECK();
     }
     return ZG_HIP_OK;

@@ -93,6 +93,48 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float*
     }
 }
 
+// Small tensors with the gradient clip on: one workgroup computes the norm exactly as flat_single_kernel does (same
+// per-thread accumulation and the same combine tree), publishes the clip factor, and goes on to the update.
+// One launch instead of two; the arithmetic per element is that of sgd_kernel / adam_kernel, so the values are
+// the same.  `factor_out` keeps the slot the two-kernel path fills.
+template <bool ADAM>
+__global__ __launch_bounds__(kFlatSingle) void clipped_update_small_kernel(float* p, float* g, float* m, float* v,
+                                                                           size_t n, float step_scale,
+                                                                           const float* lr_t_ptr, float b1, float b2,
+                                                                           float omb1, float omb2, float eps,
+                                                                           float max_norm, float delta,
+                                                                           float* factor_out) {
+    __shared__ float smem[kFlatSingle / kWave];
+    __shared__ float factor_s;
+    float acc = flat_accumulate<TermSq, 1>(g, nullptr, n, 0.f, threadIdx.x, blockDim.x);
+    acc = block_reduce<SumAcc>(acc, smem);
+    if (threadIdx.x == 0) {
+        FinClipFactor{&factor_s, max_norm, delta}(acc);
+        factor_out[0] = factor_s;
+    }
+    __syncthreads();
+    const float f = factor_s;
+    const bool scale = f != 1.0f;
+    const float lr_t = (ADAM && lr_t_ptr) ? lr_t_ptr[0] : step_scale;  // SGD: step_scale = -lr
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float gv = g[i];
+        if (ADAM) {
+            float pv = p[i], mv = m[i], vv = v[i];
+            adam_elem(pv, gv, mv, vv, scale, f, lr_t, b1, b2, omb1, omb2, eps);
+            if (scale) g[i] = gv;
+            m[i] = mv;
+            v[i] = vv;
+            p[i] = pv;
+        } else {
+            if (scale) {
+                gv = __fmul_rn(gv, f);
+                g[i] = gv;
+            }
+            p[i] = __fadd_rn(p[i], __fmul_rn(lr_t, gv));
+        }
+    }
+}
+
 static int update_grid(zg_hip_ctx* ctx, size_t n) {
     size_t blocks = ceil_div_sz(n, (size_t)kBlock * 4);
     size_t cap = (size_t)ctx->n_cu * 16;
@@ -110,7 +152,11 @@ ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n,
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad, "sgd_step: null pointer");
     float* factor = ctx->scalar_slot + 1;
-    if (clip) {
+    if (clip && n <= kFlatSingleMax) {
+        hipLaunchKernelGGL((clipped_update_small_kernel<false>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, param, grad,
+                           (float*)nullptr, (float*)nullptr, n, -lr, (const float*)nullptr, 0.f, 0.f, 0.f, 0.f, 0.f,
+                           max_norm, delta, factor);
+    } else if (clip) {
         int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
         if (rc) return rc;
         hipLaunchKernelGGL((sgd_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, n,
@@ -134,7 +180,10 @@ static int adam_launch(zg_hip_ctx* ctx, float* param, float* grad, float* m, flo
                        float delta) {
     const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2;
     float* factor = ctx->scalar_slot + 1;
-    if (clip) {
+    if (clip && n <= kFlatSingleMax) {
+        hipLaunchKernelGGL((clipped_update_small_kernel<true>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, param, grad,
+                           m, v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, max_norm, delta, factor);
+    } else if (clip) {
         int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
         if (rc) return rc;
         hipLaunchKernelGGL((adam_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, m,

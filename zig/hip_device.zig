@@ -457,3 +457,53 @@ pub fn adam_step(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
     check(c.zg_hip_adam_step(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.t, p.lr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
 }
+
+/// Adam update whose `lr_t` is read from memory when the kernel runs (`p.lr_t` points to device memory or
+/// to `mem_alloc_indices`-style pinned host memory).  A step recorded with `capture.open()` can then be
+/// replayed for every later step: the host only rewrites `lr_t` between replays.
+pub fn adam_step_at(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_adam_step_at(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.lr_t, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
+}
+
+/// The ExecutionGraph of the reference's second device (src/device/cuda_device.zig:558-611), same four calls.
+/// Between `open` and `save` every op is recorded instead of executed; `mem_cache_free` inside a capture parks
+/// the block with the graph, so the recorded addresses stay private to it until `free`.
+pub const ExecutionGraph = struct {
+    ctx: *c.zg_hip_ctx,
+    graph: ?*c.zg_hip_graph = null,
+    open_now: bool = false,
+
+    pub const RunError = error{ CaptureInProgress, UndefinedCapture };
+
+    pub fn run(self: *ExecutionGraph) RunError!void {
+        if (self.open_now) return error.CaptureInProgress;
+        const g = self.graph orelse return error.UndefinedCapture;
+        check(c.zg_hip_graph_run(self.ctx, g));
+    }
+    pub fn open(self: *ExecutionGraph, config: struct {}) void {
+        _ = config;
+        self.free();
+        check(c.zg_hip_graph_open(self.ctx));
+        self.open_now = true;
+    }
+    pub fn save(self: *ExecutionGraph) void {
+        if (!self.open_now) return;
+        var g: ?*c.zg_hip_graph = null;
+        check(c.zg_hip_graph_save(self.ctx, &g));
+        self.graph = g;
+        self.open_now = false;
+    }
+    pub fn free(self: *ExecutionGraph) void {
+        self.save();
+        if (self.graph) |g| check(c.zg_hip_graph_free(self.ctx, g));
+        self.graph = null;
+    }
+    pub fn empty(self: ExecutionGraph) bool {
+        return self.graph == null;
+    }
+};
+
+pub fn execution_graph(self: *const Self) ExecutionGraph {
+    return .{ .ctx = self.ctx };
+}

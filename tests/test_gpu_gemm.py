@@ -43,6 +43,8 @@ SHAPES = [
     (512, 384, 160), (300, 500, 70), (1024, 1024, 256),
     # few C tiles and a deep k: the split-k path, whole tiles (fast kernels) and ragged
     (128, 64, 2048), (64, 64, 4096), (70, 50, 1000),
+    # aligned but ragged in m and n (edge kernels: clamped loads, guarded stores), with and without a k remainder
+    (2072, 1300, 1028), (4100, 2060, 100), (2072, 1300, 1024), (1000, 1000, 512), (100, 68, 64), (4, 4, 32),
 ]
 
 

@@ -189,8 +189,16 @@ __device__ __forceinline__ void tile_coords(unsigned pid, unsigned tiles_m, unsi
     tn = in_group / gsize;
 }
 
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, bool SAFE>
+// MODE 0 (fast): whole tiles, aligned operands, an even number of k-tiles; no bounds checks anywhere.
+// MODE 1 (edge): as fast, but M and N may end inside a tile: the per-thread load offsets are clamped to the last
+//                valid row / 4-column piece once, before the loop (rows and columns past the edge then hold copies
+//                of valid data, which only reach C elements that are never stored), and the epilogue checks bounds.
+//                Needs M % 4 == 0 (N % 4 == 0) when A (B) is not k-contiguous, so that a 16-byte piece is never
+//                half inside.  The loop is the fast loop.
+// MODE 2 (checked): every load checked and zero-filled, scalar loads where 16-byte loads are not legal.
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int MODE>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
+    constexpr bool SAFE = MODE == 2;
     constexpr int BK = kBK;
     using TA = Tile<BM, A_KMAJOR>;
     using TB = Tile<BN, B_KMAJOR>;
@@ -239,9 +247,25 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     const float* const b_rd = Bs0 + FB::lane_base(wn0, l32, lk);
     unsigned a_off[TA::NV], b_off[TB::NV];
 #pragma unroll
-    for (int i = 0; i < TA::NV; i++) a_off[i] = (unsigned)(TA::gmem_offset(i, g.lda) * sizeof(float));
+    for (int i = 0; i < TA::NV; i++) {
+        int tmn, tk;
+        TA::coords(i, tmn, tk);
+        if (MODE == 1) {
+            const size_t last = A_KMAJOR ? g.M - 1 : g.M - 4;
+            if (m0 + tmn > last) tmn = (int)(last - m0);
+        }
+        a_off[i] = (unsigned)((A_KMAJOR ? tmn * g.lda + tk : tk * g.lda + tmn) * sizeof(float));
+    }
 #pragma unroll
-    for (int i = 0; i < TB::NV; i++) b_off[i] = (unsigned)(TB::gmem_offset(i, g.ldb) * sizeof(float));
+    for (int i = 0; i < TB::NV; i++) {
+        int tmn, tk;
+        TB::coords(i, tmn, tk);
+        if (MODE == 1) {
+            const size_t last = B_KMAJOR ? g.N - 1 : g.N - 4;
+            if (n0 + tmn > last) tmn = (int)(last - n0);
+        }
+        b_off[i] = (unsigned)((B_KMAJOR ? tmn * g.ldb + tk : tk * g.ldb + tmn) * sizeof(float));
+    }
     const float* const a_org = A_KMAJOR ? A + m0 * g.lda : A + m0;  // tile origin at k = 0
     const float* const b_org = B_KMAJOR ? B + n0 * g.ldb : B + n0;
 
@@ -363,7 +387,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         constexpr int RSTEP = A_KMAJOR ? 1 : TM;  // tile rows between consecutive block rows
         auto row_of = [&](int r) { return ((r >> 2) * 8 + (r & 3)) * RSTEP; };  // relative to block row lk*4
         auto in_range = [&](int j, int r) {
-            if (!SAFE) return true;
+            if (MODE == 0) return true;
             const size_t row = m0 + wm0 + FA::index_of(i, lk * 4 + (r >> 2) * 8 + (r & 3));
             const size_t col = n0 + wn0 + FB::index_of(j, l32);
             return row < g.M && col < g.N;
@@ -372,7 +396,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 if (VEC_C) {
-                    const VC o = *reinterpret_cast<const VC*>(cptr[0] + (size_t)row_of(r) * g.ldc);
+                    VC o = {};
+                    if (in_range(0, r)) o = *reinterpret_cast<const VC*>(cptr[0] + (size_t)row_of(r) * g.ldc);
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
                         if constexpr (VEC_C) old[j][r] = o[j];
@@ -401,7 +426,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
                 for (int j = 0; j < TN; j++) {
                     if constexpr (VEC_C) o[j] = v[j];
                 }
-                *reinterpret_cast<VC*>(cptr[0] + (size_t)row_of(r) * g.ldc) = o;
+                if (in_range(0, r)) *reinterpret_cast<VC*>(cptr[0] + (size_t)row_of(r) * g.ldc) = o;
             } else {
 #pragma unroll
                 for (int j = 0; j < TN; j++)
@@ -414,28 +439,28 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 }
 
 template <int BM, int BN>
-static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, bool safe, size_t batches) {
+static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, int mode, size_t batches) {
     g.tiles_m = (unsigned)ceil_div_sz(g.M, BM);
     g.tiles_n = (unsigned)ceil_div_sz(g.N, BN);
     const size_t kt_total = ceil_div_sz(g.K, kBK);
     dim3 grid(g.tiles_m * g.tiles_n, (unsigned)ceil_div_sz(kt_total, g.split_tiles), (unsigned)batches), block(kGemmThreads);
-#define ZG_GEMM(AK, BKM, SF)                                                                                  \
+#define ZG_GEMM(AK, BKM, MD)                                                                                  \
     do {                                                                                                      \
         constexpr size_t lds_bytes = 2 * (size_t)(Tile<BM, AK>::ELEMS + Tile<BN, BKM>::ELEMS) * sizeof(float); \
         static_assert(lds_bytes <= 64 * 1024, "tile buffers exceed the default dynamic LDS limit");           \
-        hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, SF>), grid, block, lds_bytes, ctx->stream, g);       \
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, MD>), grid, block, lds_bytes, ctx->stream, g);       \
     } while (0)
-    if (safe) {
-        if (a_kmajor && b_kmajor) ZG_GEMM(true, true, true);
-        else if (a_kmajor && !b_kmajor) ZG_GEMM(true, false, true);
-        else if (!a_kmajor && b_kmajor) ZG_GEMM(false, true, true);
-        else ZG_GEMM(false, false, true);
-    } else {
-        if (a_kmajor && b_kmajor) ZG_GEMM(true, true, false);
-        else if (a_kmajor && !b_kmajor) ZG_GEMM(true, false, false);
-        else if (!a_kmajor && b_kmajor) ZG_GEMM(false, true, false);
-        else ZG_GEMM(false, false, false);
-    }
+#define ZG_GEMM_LAYOUT(MD)                                      \
+    do {                                                        \
+        if (a_kmajor && b_kmajor) ZG_GEMM(true, true, MD);      \
+        else if (a_kmajor && !b_kmajor) ZG_GEMM(true, false, MD); \
+        else if (!a_kmajor && b_kmajor) ZG_GEMM(false, true, MD); \
+        else ZG_GEMM(false, false, MD);                         \
+    } while (0)
+    if (mode == 0) ZG_GEMM_LAYOUT(0);
+    else if (mode == 1) ZG_GEMM_LAYOUT(1);
+    else ZG_GEMM_LAYOUT(2);
+#undef ZG_GEMM_LAYOUT
 #undef ZG_GEMM
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
@@ -470,7 +495,8 @@ __global__ void scale_c_kernel(float* C, size_t M, size_t N, size_t ldc, float b
 
 static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
                          size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta,
-                         size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk) {
+                         size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk,
+                         int depth = 0) {
     if (m == 0 || n == 0 || batches == 0) return ZG_HIP_OK;
     ZG_REQUIRE(A && B && C, "%s: null pointer", name);
     // cblas argument rules for row-major storage
@@ -509,13 +535,16 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.a_vec = aligned16(A) && lda % 4 == 0 && a_chunk % 4 == 0;
     g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
 
-    // Fast kernels assume whole tiles, 16-byte alignment of all three matrices and 32-bit byte offsets inside
-    // an operand tile; everything else takes the checked variants.
+    // Kernel mode per tile shape: fast (whole tiles, aligned, even number of k-tiles), edge (aligned, ragged in m
+    // and n only) or checked (everything else), see gemm_kernel.
     const bool c_vec = aligned16(C) && ldc % 4 == 0 && c_chunk % 4 == 0;
     const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
+    const bool aligned = g.a_vec && g.b_vec && c_vec && small_ld;
+    const bool mn_ok = (a_kmajor || m % 4 == 0) && (b_kmajor || n % 4 == 0);
     auto tiles = [&](size_t bm, size_t bn) { return ceil_div_sz(m, bm) * ceil_div_sz(n, bn) * batches; };
-    auto fast = [&](size_t bm, size_t bn) {
-        return g.a_vec && g.b_vec && c_vec && small_ld && m % bm == 0 && n % bn == 0 && k % (2 * kBK) == 0;
+    auto mode = [&](size_t bm, size_t bn) {
+        if (!aligned || !mn_ok || k % (2 * kBK) != 0) return 2;
+        return (m % bm == 0 && n % bn == 0) ? 0 : 1;
     };
     // Tile choice by estimated time.  A CU works through its workgroups at a rate that depends on the tile shape
     // but hardly on how many of them share the CU (measured fraction of a CU's MFMA peak: 0.92 / 0.89 / 0.79),
@@ -527,10 +556,25 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     const size_t kt_total = ceil_div_sz(k, kBK);
     g.split_tiles = kt_total;
     g.split_stride = 0;
+
+    // A deep, aligned product whose k is not a whole number of tile pairs: the bulk of k goes through the fast /
+    // edge kernels and the remainder (fewer than 32 values of k) is accumulated by a second, checked pass with
+    // beta = 1.  The second pass re-reads and re-writes C, so this only pays when k is long.
+    const size_t k_main = k / (2 * kBK) * (2 * kBK);
+    if (depth == 0 && aligned && mn_ok && k_main < k && k_main >= 16 * kBK && tiles(64, 64) >= n_cu) {
+        const float* a_tail = trans_a ? A + k_main * lda : A + k_main;
+        const float* b_tail = trans_b ? B + k_main : B + k_main * ldb;
+        if (int rc = gemm_dispatch(ctx, name, A, B, C, m, n, k_main, trans_a, trans_b, lda, ldb, ldc, alpha, beta, batches,
+                                   nba, nbb, a_chunk, b_chunk, c_chunk, 1))
+            return rc;
+        return gemm_dispatch(ctx, name, a_tail, b_tail, C, m, n, k - k_main, trans_a, trans_b, lda, ldb, ldc, alpha, 1.f,
+                             batches, nba, nbb, a_chunk, b_chunk, c_chunk, 1);
+    }
+
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
     if (c_large <= c_mid && c_large <= c_small)
-        return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, !fast(256, 128), batches);
-    if (c_mid <= c_small) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, !fast(128, 128), batches);
+        return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, mode(256, 128), batches);
+    if (c_mid <= c_small) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, mode(128, 128), batches);
     // A deep product with too few C tiles to give every CU a workgroup: split k over several workgroups per tile
     // (an even number of k-tiles each), let each write its partial tile to the workspace, and add the partials in
     // split order in a second kernel.  The order is fixed, so the result does not depend on scheduling.
@@ -553,10 +597,9 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
             gs.split_stride = m * n;
             gs.alpha = 1.f;
             gs.beta = 0.f;
-            const bool part_vec = n % 4 == 0 && (m * n) % 4 == 0;  // the workspace itself is 256-byte aligned
-            const bool fast_split = g.a_vec && g.b_vec && part_vec && small_ld && m % 64 == 0 && n % 64 == 0 &&
-                                    k % (2 * kBK) == 0;
-            int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, !fast_split, batches);
+            // the partial-product buffer is 256-byte aligned and dense: its own alignment rule is n % 4 == 0
+            const int split_mode = (mode(64, 64) != 2 && n % 4 == 0 && (m * n) % 4 == 0) ? mode(64, 64) : 2;
+            int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
             if (rc) return rc;
             size_t blocks = ceil_div_sz(m * n, 256);
             if (blocks > 2048) blocks = 2048;
@@ -566,7 +609,7 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
             return ZG_HIP_OK;
         }
     }
-    return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, !fast(64, 64), batches);
+    return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, mode(64, 64), batches);
 }
 
 // ------------------------------------------------------------------------------------------------

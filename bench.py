@@ -11,6 +11,8 @@ The same JSON line also carries:
   cpu_baseline  the CPU oracle (C restatement of HostDevice + the box's BLAS) running the same step
   ops           the op microbenchmark suite of configs[1] (GEMM variants, bmm, broadcast add, axis
                 reductions, fused softmax cross-entropy), each with its own roofline fraction
+  input_pipeline  the same step with a fresh 67 MB batch from pinned host memory every step (PCIe-inclusive rate):
+                blocking upload as the reference does it, and double-buffered on the copy stream
   mlp_b64, gcn, dqn   the latency-bound configurations (configs[0], [2], [3]): step time, loss read every step
 """
 from __future__ import annotations
@@ -232,6 +234,47 @@ def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_m
     return dt, loss, dt_g, loss_g
 
 
+def run_input_pipeline(dev, dims, batch, steps, warmup):
+    """The wide-MLP step with a new batch arriving from host memory every step: uploaded with the reference's
+    blocking transfer before the step, or double-buffered on the copy stream under the previous step.  Both read
+    the batches from pinned host memory that a loader would fill in place."""
+    from zigrad_amd.device import F32, U64
+    from zigrad_amd.trainers import BatchStager, MLPTrainer, mlp_inputs
+
+    params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data="normal")
+    tr = MLPTrainer(dev, dims, batch, optimizer="adam", lr=1e-3, clip=True)
+    tr.load_params(params)
+    own = (tr.x, tr.onehot, tr.labels)
+    st = BatchStager(dev, [(F32, batch * dims[0]), (F32, batch * dims[-1]), (U64, batch)])
+    for slot in range(2):
+        for a, view in zip((x, onehot, labels), st.views[slot]):
+            np.copyto(view, np.asarray(a).ravel())
+    st.upload_first((x, onehot, labels))
+    batch_bytes = sum(b.nbytes for b in st.pinned[0])
+
+    def blocking_step():
+        for src, dst in zip(st.views[0], own):
+            dev.mem_transfer(src, dst, "HtoD")
+        return tr.step()
+
+    def staged_step():
+        tr.use_batch(*st.current())
+        st.prefetch()
+        loss = tr.step()
+        st.advance()
+        return loss
+
+    out = {"batch_bytes": batch_bytes}
+    for name, fn in (("blocking_upload", blocking_step), ("staged_upload", staged_step)):
+        for _ in range(warmup):
+            fn()
+        dt, _ = timed_steps(dev, fn, steps)
+        out[name] = {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3}
+        tr.use_batch(*own)
+    st.free()
+    return out
+
+
 def run_small(dev, kind, steps):
     """Step time of the GCN (2708 nodes, 1433 features, 13264 edges, 140 labelled, Adam) or DQN (4-128-128-2, batch
     64, Adam) train step; the loss is read back every step, as the reference's loops do."""
@@ -340,6 +383,7 @@ def main():
                          "graph_replay": {"steps_per_s": 200 / dt64g, "ms_per_step": dt64g / 200 * 1e3},
                          "workload": "784-128-64-10, batch 64, SGD lr 0.01, clip on, loss read every step; "
                                      "graph_replay = the same step recorded once as an execution graph"}
+    result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
     result["gcn"] = run_small(dev, "gcn", 100)
     result["dqn"] = run_small(dev, "dqn", 200)
     if not args.no_ops:

@@ -253,6 +253,23 @@ int zg_hip_adam_step_at(zg_hip_ctx *ctx, float *param, float *grad, float *m, fl
                         float beta1, float beta2, float epsilon, int clip, float max_norm, float delta);
 
 /* ---------------------------------------------------------------------------------------------
+ * input staging: the step before the hot path.  The reference uploads every batch with a blocking
+ * mem_transfer(.HtoD) (src/device/device_reference.zig:101-105, as used by NDTensor.from_slice in
+ * examples/mnist/src/dataset.zig:51-52).  These three calls let a training loop upload batch k+1 from pinned
+ * host memory on a second stream (default priority) while the kernels of batch k run:
+ *   staged_h2d         asynchronous copy on the copy stream; `src_host` must come from zg_hip_host_alloc and
+ *                      must not be rewritten until zg_hip_staging_wait returned (or a later sync)
+ *   staging_after_compute   copies issued from now on wait for all work issued to the compute stream so far
+ *                      (call it before overwriting a device buffer that earlier ops still read)
+ *   compute_after_staging   ops issued from now on wait for every copy issued so far
+ *   staging_wait       blocks the host until every staged copy has finished (the pinned source may be reused)
+ * ------------------------------------------------------------------------------------------- */
+int zg_hip_staged_h2d(zg_hip_ctx *ctx, void *dst, const void *src_host, size_t bytes);
+int zg_hip_staging_after_compute(zg_hip_ctx *ctx);
+int zg_hip_compute_after_staging(zg_hip_ctx *ctx);
+int zg_hip_staging_wait(zg_hip_ctx *ctx);
+
+/* ---------------------------------------------------------------------------------------------
  * execution graphs: the ExecutionGraph of the reference's second device, src/device/cuda_device.zig:558-611
  * (open = begin stream capture, save = end capture and instantiate, run = launch, free).
  * Between open and save every op call is recorded instead of executed.  Calls that synchronise, allocate

@@ -507,3 +507,20 @@ pub const ExecutionGraph = struct {
 pub fn execution_graph(self: *const Self) ExecutionGraph {
     return .{ .ctx = self.ctx };
 }
+
+// Input staging (no counterpart in the reference, which uploads each batch with a blocking mem_transfer):
+// upload the next batch from `mem_alloc_indices`-style pinned host memory on the copy stream while the current
+// batch computes.  Order per step: compute_after_staging(), staging_after_compute(), staged_h2d(next batch),
+// then the ops of the current step.
+pub fn staged_h2d(self: *const Self, T: type, src_pinned: []const T, dst: []T) void {
+    check(c.zg_hip_staged_h2d(self.ctx, dst.ptr, src_pinned.ptr, src_pinned.len * @sizeOf(T)));
+}
+pub fn staging_after_compute(self: *const Self) void {
+    check(c.zg_hip_staging_after_compute(self.ctx));
+}
+pub fn compute_after_staging(self: *const Self) void {
+    check(c.zg_hip_compute_after_staging(self.ctx));
+}
+pub fn staging_wait(self: *const Self) void {
+    check(c.zg_hip_staging_wait(self.ctx));
+}

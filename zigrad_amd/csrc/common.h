@@ -54,6 +54,10 @@ struct zg_hip_ctx {
     size_t scratch_bytes = 0;
     uint64_t n_device_allocs = 0;
 
+    // input staging (runtime.hip): second stream for host-to-device copies, one event per direction
+    hipStream_t copy_stream = nullptr;
+    hipEvent_t ev_compute = nullptr, ev_copy = nullptr;
+
     // execution-graph capture (runtime.hip): while `capturing`, cache blocks that are freed are parked here
     // instead of going back to the pool, so a replay never meets another owner at those addresses
     bool capturing = false;

@@ -327,6 +327,12 @@ ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
     if (ctx->partials) (void)hipFree(ctx->partials);
     for (auto& kv : ctx->raw_allocs) (void)hipFree(kv.first);
     for (auto& kv : ctx->host_allocs) (void)hipHostFree(kv.first);
+    if (ctx->copy_stream) {
+        (void)hipStreamSynchronize(ctx->copy_stream);
+        (void)hipEventDestroy(ctx->ev_compute);
+        (void)hipEventDestroy(ctx->ev_copy);
+        (void)hipStreamDestroy(ctx->copy_stream);
+    }
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return ZG_HIP_OK;
@@ -336,6 +342,60 @@ ZG_API int zg_hip_sync(zg_hip_ctx* ctx) {
     ZG_CTX(ctx);
     ZG_NOT_CAPTURING(ctx, "sync");
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// input staging: a copy stream beside the compute stream, ordered against it with events
+// ------------------------------------------------------------------------------------------------
+static int ensure_copy_stream(zg_hip_ctx* ctx) {
+    if (ctx->copy_stream) return ZG_HIP_OK;
+    ZG_HIP_TRY(hipStreamCreateWithFlags(&ctx->copy_stream, hipStreamNonBlocking));  // default priority
+    ZG_HIP_TRY(hipEventCreateWithFlags(&ctx->ev_compute, hipEventDisableTiming));
+    ZG_HIP_TRY(hipEventCreateWithFlags(&ctx->ev_copy, hipEventDisableTiming));
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_staged_h2d(zg_hip_ctx* ctx, void* dst, const void* src_host, size_t bytes) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "staged_h2d");
+    if (bytes == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(dst && src_host, "staged_h2d: null pointer");
+    // a pageable source would make the copy synchronous and let the caller reuse it too early
+    bool pinned = false;
+    for (auto& kv : ctx->host_allocs) {
+        const char* lo = (const char*)kv.first;
+        if ((const char*)src_host >= lo && (const char*)src_host + bytes <= lo + kv.second) pinned = true;
+    }
+    ZG_REQUIRE(pinned, "staged_h2d: the source must lie inside a zg_hip_host_alloc allocation");
+    if (int rc = ensure_copy_stream(ctx)) return rc;
+    ZG_HIP_TRY(hipMemcpyAsync(dst, src_host, bytes, hipMemcpyHostToDevice, ctx->copy_stream));
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_staging_after_compute(zg_hip_ctx* ctx) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "staging_after_compute");
+    if (int rc = ensure_copy_stream(ctx)) return rc;
+    ZG_HIP_TRY(hipEventRecord(ctx->ev_compute, ctx->stream));
+    ZG_HIP_TRY(hipStreamWaitEvent(ctx->copy_stream, ctx->ev_compute, 0));
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_compute_after_staging(zg_hip_ctx* ctx) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "compute_after_staging");
+    if (!ctx->copy_stream) return ZG_HIP_OK;  // nothing was ever staged
+    ZG_HIP_TRY(hipEventRecord(ctx->ev_copy, ctx->copy_stream));
+    ZG_HIP_TRY(hipStreamWaitEvent(ctx->stream, ctx->ev_copy, 0));
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_staging_wait(zg_hip_ctx* ctx) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "staging_wait");
+    if (!ctx->copy_stream) return ZG_HIP_OK;
+    ZG_HIP_TRY(hipStreamSynchronize(ctx->copy_stream));
     return ZG_HIP_OK;
 }
 
@@ -548,6 +608,7 @@ ZG_API int zg_hip_host_free(zg_hip_ctx* ctx, void* ptr) {
     auto it = ctx->host_allocs.find(ptr);
     ZG_REQUIRE(it != ctx->host_allocs.end(), "host_free: pointer %p was not allocated by this context", ptr);
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (ctx->copy_stream) ZG_HIP_TRY(hipStreamSynchronize(ctx->copy_stream));
     ZG_HIP_TRY(hipHostFree(ptr));
     ctx->host_allocs.erase(it);
     return ZG_HIP_OK;

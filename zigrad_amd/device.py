@@ -87,6 +87,29 @@ class HipDevice:
     def event(self) -> "Event":
         return Event(self)
 
+    # -- input staging: upload the next batch on a second stream while the current one computes -------
+    def staged_h2d(self, src_host: DevBuf, dst: DevBuf) -> None:
+        """Asynchronous copy from pinned host memory (mem_alloc_host) on the copy stream."""
+        if src_host.kind != "host":
+            raise ValueError("staged_h2d needs a pinned source from mem_alloc_host")
+        self._call("zg_hip_staged_h2d", dst.ptr, src_host.ptr, min(src_host.nbytes, dst.nbytes))
+
+    def staging_after_compute(self) -> None:
+        self._call("zg_hip_staging_after_compute")
+
+    def compute_after_staging(self) -> None:
+        self._call("zg_hip_compute_after_staging")
+
+    def staging_wait(self) -> None:
+        self._call("zg_hip_staging_wait")
+
+    def host_view(self, buf: DevBuf) -> np.ndarray:
+        """numpy view of a pinned host allocation (for the host code that fills it)."""
+        if buf.kind != "host":
+            raise ValueError("host_view needs a buffer from mem_alloc_host")
+        ctype = np.ctypeslib.as_ctypes_type(buf.dtype)
+        return np.ctypeslib.as_array((ctype * buf.n).from_address(buf.ptr))
+
     # -- execution graphs (src/device/cuda_device.zig:558-611: open / save / run / free) -----------
     def graph_open(self) -> None:
         """Start recording: until graph_save() every op call is captured instead of executed."""

@@ -149,6 +149,56 @@ class GraphSteps:
             self.graph = None
 
 
+class BatchStager:
+    """Double-buffered upload of training batches from pinned host memory on the device's copy stream, so the
+    upload of batch k+1 overlaps the kernels of batch k.  (The reference uploads each batch with a blocking
+    NDTensor.from_slice, examples/mnist/src/dataset.zig:51-52.)
+
+    `specs` lists (dtype, element count) of the arrays that make up one batch.  Protocol per step:
+        bufs = stager.current()        # device buffers holding batch k
+        stager.prefetch(arrays_k1)     # start uploading batch k+1 into the other slot
+        ... issue the ops of step k on bufs ...
+        stager.advance()
+    """
+
+    def __init__(self, dev, specs):
+        self.dev = dev
+        self.pinned = [[dev.mem_alloc_host(dt, n) for dt, n in specs] for _ in range(2)]
+        self.views = [[dev.host_view(b) for b in slot] for slot in self.pinned]
+        self.device = [[dev.mem_alloc(dt, n) for dt, n in specs] for _ in range(2)]
+        self.slot = 0
+
+    def upload_first(self, arrays) -> None:
+        for a, dst in zip(arrays, self.device[self.slot]):
+            self.dev.mem_transfer(np.ascontiguousarray(a).ravel(), dst, "HtoD")
+
+    def current(self):
+        return self.device[self.slot]
+
+    def prefetch(self, arrays=None) -> None:
+        """Upload the next batch.  With `arrays` = None the pinned slot is sent as it is (a loader that writes
+        straight into `views[slot ^ 1]` needs no extra host copy)."""
+        d, nxt = self.dev, self.slot ^ 1
+        d.staging_wait()  # the copy that last read pinned[nxt] (two steps ago) has long finished; make it certain
+        if arrays is not None:
+            for a, view in zip(arrays, self.views[nxt]):
+                np.copyto(view, np.asarray(a).ravel())
+        d.compute_after_staging()   # the ops issued next wait for the upload of the current batch
+        d.staging_after_compute()   # the new upload waits for the ops already issued, which read device[nxt]
+        for src, dst in zip(self.pinned[nxt], self.device[nxt]):
+            d.staged_h2d(src, dst)
+
+    def advance(self) -> None:
+        self.slot ^= 1
+
+    def free(self) -> None:
+        self.dev.staging_wait()
+        self.dev.sync()
+        for slot in self.pinned + self.device:
+            for b in slot:
+                self.dev.mem_free(b)
+
+
 class MLP:
     """Parameters, gradients and the forward/backward op sequences of a ReLU multi-layer perceptron whose
     Linear layers follow examples/mnist/src/model.zig:64-110 (weights [out, in], forward x . W^T + bias)."""
@@ -262,6 +312,10 @@ class MLPTrainer(GraphSteps):
         if labels is None:
             labels = np.argmax(onehot, axis=1).astype(np.uint64)
         self.dev.mem_transfer(labels, self.labels, "HtoD")
+
+    def use_batch(self, x: DevBuf, onehot: DevBuf, labels: DevBuf) -> None:
+        """Train on batch buffers owned by the caller (a BatchStager slot) from the next step on."""
+        self.x, self.onehot, self.labels = x, onehot, labels
 
     def step(self, read_loss: bool = True, keep_grads: bool = False):
         d, B, C = self.dev, self.batch, self.dims[-1]

@@ -74,6 +74,15 @@ class Optimizer:
             self.dev.mem_fill(v, 0.0)
             self.state.append((m, v))
 
+    def state_tensors(self, names) -> dict:
+        """{key: (buffer, shape)} of Adam's moments, keyed like the parameters they belong to."""
+        out = {}
+        if self.kind == "adam":
+            for (name, shape), (m, v) in zip(names, self.state):
+                out[f"optim.m.{name}"] = (m, shape)
+                out[f"optim.v.{name}"] = (v, shape)
+        return out
+
     def begin_capture(self) -> None:
         """Before recording a step: Adam's lr_t changes every step, so the recorded kernels read it from memory."""
         if self.kind == "adam" and self.lr_slots is None:
@@ -312,6 +321,32 @@ class MLPTrainer(GraphSteps):
         if labels is None:
             labels = np.argmax(onehot, axis=1).astype(np.uint64)
         self.dev.mem_transfer(labels, self.labels, "HtoD")
+
+    def named_tensors(self) -> dict:
+        """Parameters and optimizer state under dotted keys (the LayerMap convention, src/utils/layer_map.zig)."""
+        names, out = [], {}
+        for l in range(self.n_layers):
+            fan_in, fan_out = self.dims[l], self.dims[l + 1]
+            for key, buf, shape in ((f"layers.{l}.weights", self.net.W[l], [fan_out, fan_in]),
+                                    (f"layers.{l}.bias", self.net.b[l], [fan_out])):
+                out[key] = (buf, shape)
+                names.append((key, shape))
+        out.update(self.optim.state_tensors(names))
+        return out
+
+    def save_checkpoint(self, path) -> None:
+        from .checkpoint import save_tensors
+
+        save_tensors(path, self.dev, self.named_tensors(),
+                     {"optim.kind": self.optim.kind, "optim.t": self.optim.t, "optim.lr": repr(self.optim.lr)})
+
+    def load_checkpoint(self, path) -> None:
+        from .checkpoint import load_tensors
+
+        meta = load_tensors(path, self.dev, self.named_tensors())
+        if meta.get("optim.kind", self.optim.kind) != self.optim.kind:
+            raise ValueError(f"checkpoint was written by {meta['optim.kind']}, this trainer uses {self.optim.kind}")
+        self.optim.t = int(meta.get("optim.t", 0))
 
     def use_batch(self, x: DevBuf, onehot: DevBuf, labels: DevBuf) -> None:
         """Train on batch buffers owned by the caller (a BatchStager slot) from the next step on."""

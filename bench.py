@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the device-op hot path on one MI355X.
 
-Headline workload: the wide-MLP train step (BASELINE.json configs[4]: 4096 -> 4096 -> 4096 -> 1024,
+Headline workload: the wide-MLP train step (configuration 5 of the benchmark definition: 4096 -> 4096 -> 4096 -> 1024,
 batch 4096, fp32, forward + backward + Adam), issued op by op through the C ABI exactly as the reference's
 training loop reaches its device.  `value` is train steps per second with every operand resident in HBM.
 

@@ -1,4 +1,4 @@
-"""The op microbenchmark suite of BASELINE.json configs[1] at its full sizes, checked through properties that do
+"""The op microbenchmark suite (configuration 2 of the benchmark definition) at its full sizes, checked through properties that do
 not need a CPU pass over the whole problem: sampled entries against float64 dot products, exact elementwise
 identities, row invariants of softmax cross-entropy, and doubling under accumulation."""
 from __future__ import annotations

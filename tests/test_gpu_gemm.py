@@ -1,6 +1,6 @@
 """fp32 GEMM family on the matrix cores against the oracle (BLAS sgemm) and an fp64-accumulated GEMM.
 
-Tolerance: relative Frobenius error <= 1e-5 against the fp64-accumulated result (BASELINE.json's per-op
+Tolerance: relative Frobenius error <= 1e-5 against the fp64-accumulated result (the benchmark definition's per-op
 bound); cases built from small integers or permutation matrices are exact in fp32 and compared bit for bit.
 """
 from __future__ import annotations

@@ -2,7 +2,7 @@
 
 Tolerances: bit-exact (array_equal) for index / integer / copy-like work and for elementwise ops built
 only from IEEE add/sub/mul/div/sqrt/compare; relative Frobenius error <= 1e-5 for ops that call
-transcendental functions or change the summation order (the bound BASELINE.json sets per op).
+transcendental functions or change the summation order (the benchmark definition's bound per op).
 """
 from __future__ import annotations
 

@@ -1,5 +1,5 @@
 """Whole train steps on the HIP device against the oracle: relative error <= 1e-4 on loss, gradients and
-updated parameters (the bound BASELINE.json sets for a full step)."""
+updated parameters (the benchmark definition's bound for a full step)."""
 from __future__ import annotations
 
 import numpy as np

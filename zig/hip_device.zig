@@ -1,7 +1,7 @@
 //! HipDevice: Zigrad's second device, backed by libzg_hip.so (include/zg_hip.h).
 //!
-//! Drop this file into src/device/ next to host_device.zig, add the union field shown in
-//! INTEGRATION.md to enabled_devices.zig, link libzg_hip.so, and every NDArray / NDTensor / Graph / nn
+//! Drop this file into src/device/ next to host_device.zig, add a `hip: *HipDevice` field to the device union in
+//! enabled_devices.zig (next to the cuda entry), link libzg_hip.so, and every NDArray / NDTensor / Graph / nn
 //! call that goes through DeviceReference.dispatch runs on the MI355X unchanged.
 //!
 //! The struct follows the reference's duck-typed device contract (src/device/device_reference.zig:15-131):
@@ -11,7 +11,8 @@
 //! (src/cuda/cuda_helpers.cu:21-28).
 //!
 //! This file cannot be compiled in the build container (no Zig toolchain); it is written against Zig 0.14
-//! and the reference's tree layout and is exercised by the steps in INTEGRATION.md.
+//! and the reference's tree layout; the reference's own device-parameterised tests (tests/src/main.zig:21-27)
+//! are what exercises it.
 const std = @import("std");
 const c = @cImport(@cInclude("zg_hip.h"));
 const opspec = @import("opspec.zig");
@@ -419,7 +420,7 @@ pub fn scatter_gcn_deg_scaled_bwd(self: *const Self, T: type, p: opspec.scatter_
 }
 
 // New op names for what the reference computes with host loops over `.raw` (they need the matching
-// parameter structs added to opspec.zig and the call sites switched to dispatch; see INTEGRATION.md):
+// parameter structs added to opspec.zig, field names as used below, and the call sites switched to dispatch):
 //   smce_fwd / smce_bwd / smce_label_fwd / smce_label_bwd   src/nn/loss.zig:130-215
 //   smooth_l1_fwd / smooth_l1_bwd / mse_fwd / mse_bwd        src/nn/loss.zig:94-127, 259-305
 //   sgd_step / adam_step                                     src/nn/optim.zig:100-122, 177-234

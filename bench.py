@@ -193,7 +193,17 @@ def op_suite(dev, quick=False):
     ms = time_op(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
                                             accumulate=True), iters)
     out["smce_bwd_accumulate_8192x32000"] = gbs(3 * 4 * M * N, ms)
-    for b in (logits, grad, labels, lse, loss):
+    # the reference's own form of the loss: float one-hot targets, probabilities saved for backward
+    # (src/nn/loss.zig:130-215): 3 passes of the matrix forward (read logits, read target, write probs), 4 backward
+    target, probs = dev.mem_alloc(F32, M * N), dev.mem_alloc(F32, M * N)
+    dev.mem_fill(target, 0.0)
+    dev.mem_fill(grad, 0.0)
+    ms = time_op(dev, lambda: dev.dispatch("smce_fwd", logits=logits, target=target, probs=probs, loss=loss, rows=M, cols=N),
+                 iters // 2)
+    out["smce_onehot_fwd_8192x32000"] = gbs(3 * 4 * M * N, ms)
+    ms = time_op(dev, lambda: dev.dispatch("smce_bwd", probs=probs, target=target, grad=grad, rows=M, cols=N), iters // 2)
+    out["smce_onehot_bwd_8192x32000"] = gbs(4 * 4 * M * N, ms)
+    for b in (logits, grad, labels, lse, loss, target, probs):
         dev.mem_free(b)
     return out
 

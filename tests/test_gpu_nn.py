@@ -24,7 +24,7 @@ def both(oracle, hip, name, params, outputs):
 # ----------------------------------------------------------------------------------------------
 # softmax / cross-entropy
 # ----------------------------------------------------------------------------------------------
-SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001)]
+SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001), (9, 4100)]
 
 
 @pytest.mark.parametrize("rows,cols", SMCE_SHAPES)
@@ -88,7 +88,7 @@ def test_smce_clamp_edge(oracle, hip):
     assert abs(b["loss"][0] - want) <= 1e-5 * want and abs(a["loss"][0] - want) <= 1e-5 * want
 
 
-@pytest.mark.parametrize("rows,cols", [(64, 10), (5, 3000), (1, 7)])
+@pytest.mark.parametrize("rows,cols", [(64, 10), (5, 3000), (1, 7), (3, 8192), (2, 32768), (2, 32772)])
 def test_softmax_fwd_bwd(oracle, hip, rows, cols):
     r = rng(rows + cols)
     x = r.standard_normal((rows, cols)).astype(np.float32)
@@ -293,3 +293,20 @@ def test_scatter_gcn_indices_in_pinned_host_memory(oracle, hip):
     hip.dispatch("scatter_gcn_deg_scaled", dst=D, h=H, deg=G, src_indices=S, tgt_indices=T, stride=stride, n_edge=src.size)
     hip.sync()
     np.testing.assert_array_equal(hip.to_numpy(D), want)
+
+
+def test_smce_soft_targets_on_long_rows(oracle, hip):
+    """Dense (not one-hot) targets: every column contributes a loss term; rows long enough for the register-cached kernel."""
+    rows, cols = 6, 8192
+    r = rng(77)
+    x = (r.standard_normal((rows, cols)) * 2).astype(np.float32)
+    t = softmax(r.standard_normal((rows, cols)), axis=1).astype(np.float32)
+    one = np.zeros(1, np.float32)
+    a, b = both(oracle, hip, "smce_fwd", {"logits": x, "target": t, "probs": np.zeros_like(x), "loss": one, "rows": rows,
+                                          "cols": cols}, ["probs", "loss"])
+    x64 = x.astype(np.float64)
+    logp = x64 - logsumexp(x64, axis=1, keepdims=True)
+    want = float(-(t.astype(np.float64) * np.log(np.clip(np.exp(logp), 1e-7, 1 - 1e-7))).sum() / rows)
+    assert abs(b["loss"][0] - want) <= 1e-5 * want
+    assert abs(a["loss"][0] - want) <= 1e-4 * want
+    assert rel_fro(b["probs"], softmax(x64, axis=1)) <= TOL

@@ -199,8 +199,10 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* logit
             pr[j] = p;
             if (MODE) {
                 float t = tr[j];
-                float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
-                part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
+                if (t != 0.f) {  // a zero target adds t * log(.) = 0: skipping it changes nothing and saves the log
+                    float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
+                    part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
+                }
             }
         }
     }
@@ -214,6 +216,103 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* logit
     }
 }
 
+// Long rows (up to 32768 columns, 16-byte aligned): one workgroup of 1024 threads per row keeps the whole row in
+// registers (at most 8 float4 per thread), so the logits are read from HBM once: max / sum-of-exponentials over
+// the registers, one workgroup reduction, then the probabilities (and the loss terms) from the same registers.
+// MODE 1 reads the target row as well; its loads are issued before the reduction so they are in flight under it.
+constexpr int kLongRowThreads = 1024;
+constexpr int kLongRowVec = 8;
+template <int MODE>
+__global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(const float* logits, const float* target,
+                                                                            float* probs, float* row_loss,
+                                                                            size_t cols) {
+    __shared__ OnlineAccT smem[kLongRowThreads / kWave];
+    __shared__ float lsum[kLongRowThreads / kWave];
+    __shared__ OnlineAccT total_s;
+    const size_t row = blockIdx.x;
+    const size_t c4 = cols >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
+    const float4* t4 = reinterpret_cast<const float4*>(MODE ? target + row * cols : logits);
+    float4* p4 = reinterpret_cast<float4*>(probs + row * cols);
+    const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    float4 v[kLongRowVec], t[kLongRowVec];
+#pragma unroll
+    for (int u = 0; u < kLongRowVec; u++) {
+        const size_t j = threadIdx.x + (size_t)u * kLongRowThreads;
+        v[u] = (j < c4) ? nt_load(x4 + j) : ninf;
+    }
+    if (MODE) {
+#pragma unroll
+        for (int u = 0; u < kLongRowVec; u++) {
+            const size_t j = threadIdx.x + (size_t)u * kLongRowThreads;
+            t[u] = (j < c4) ? nt_load(t4 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    OnlineAccT acc = OnlineAcc::init();
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < kLongRowVec; u++) mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
+    if (mx != -INFINITY) {
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < kLongRowVec; u++)
+            sum += fexp(v[u].x - mx) + fexp(v[u].y - mx) + fexp(v[u].z - mx) + fexp(v[u].w - mx);
+        acc.m = mx;
+        acc.s = sum;
+    }
+    // workgroup reduction: butterfly inside each wave, then the 16 wave results in wave order by every thread
+    acc = group_reduce<OnlineAcc, kWave>(acc);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) smem[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        OnlineAccT tot = smem[0];
+        for (int w = 1; w < kLongRowThreads / kWave; w++) tot = OnlineAcc::combine(tot, smem[w]);
+        total_s = tot;
+    }
+    __syncthreads();
+    const float l = __fadd_rn(total_s.m, logf(total_s.s));
+    float part = 0.f;
+#pragma unroll
+    for (int u = 0; u < kLongRowVec; u++) {
+        const size_t j = threadIdx.x + (size_t)u * kLongRowThreads;
+        if (j < c4) {
+            float4 p;
+            p.x = fexp(__fsub_rn(v[u].x, l));
+            p.y = fexp(__fsub_rn(v[u].y, l));
+            p.z = fexp(__fsub_rn(v[u].z, l));
+            p.w = fexp(__fsub_rn(v[u].w, l));
+            nt_store(p, p4 + j);
+            if (MODE) {
+                const float pv[4] = {p.x, p.y, p.z, p.w}, tv[4] = {t[u].x, t[u].y, t[u].z, t[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (tv[e] != 0.f) {
+                        const float safe = fminf(fmaxf(pv[e], 1e-7f), 1.0f - 1e-7f);
+                        part = __fsub_rn(part, __fmul_rn(tv[e], logf(safe)));
+                    }
+                }
+            }
+        }
+    }
+    if (MODE) {
+        part = group_reduce<SumAcc, kWave>(part);
+        if (lane == 0) lsum[wave] = part;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float tot = lsum[0];
+            for (int w = 1; w < kLongRowThreads / kWave; w++) tot = __fadd_rn(tot, lsum[w]);
+            row_loss[row] = tot;
+        }
+    }
+}
+
+static bool long_row_ok(const float* a, const float* b, const float* c, size_t rows, size_t cols) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
+    return cols > 4096 && cols % 4 == 0 && cols <= (size_t)kLongRowThreads * kLongRowVec * 4 && (bits & 15u) == 0 &&
+           rows <= 0x7fffffffull;
+}
+
 // src/nn/loss.zig:150-159
 __global__ __launch_bounds__(kBlock) void smce_bwd_kernel(const float* probs, const float* target, float* grad, size_t n,
                                                            float denom) {
@@ -225,13 +324,29 @@ __global__ __launch_bounds__(kBlock) void smce_bwd_kernel(const float* probs, co
         const float4* p4 = reinterpret_cast<const float4*>(probs);
         const float4* t4 = reinterpret_cast<const float4*>(target);
         float4* g4 = reinterpret_cast<float4*>(grad);
-        for (size_t j = i; j < n4; j += nt) {
-            float4 p = p4[j], t = t4[j], g = g4[j];
+        // three streams in, one out: two 16-byte pieces per stream in flight per thread
+        for (size_t j = i; j < n4; j += 2 * nt) {
+            const size_t j2 = j + nt;
+            const bool two = j2 < n4;
+            float4 p = nt_load(p4 + j), t = nt_load(t4 + j), g = nt_load(g4 + j);
+            float4 q = p, u = t, h = g;
+            if (two) {
+                q = nt_load(p4 + j2);
+                u = nt_load(t4 + j2);
+                h = nt_load(g4 + j2);
+            }
             g.x = __fadd_rn(g.x, __fdiv_rn(__fsub_rn(p.x, t.x), denom));
             g.y = __fadd_rn(g.y, __fdiv_rn(__fsub_rn(p.y, t.y), denom));
             g.z = __fadd_rn(g.z, __fdiv_rn(__fsub_rn(p.z, t.z), denom));
             g.w = __fadd_rn(g.w, __fdiv_rn(__fsub_rn(p.w, t.w), denom));
-            g4[j] = g;
+            nt_store(g, g4 + j);
+            if (two) {
+                h.x = __fadd_rn(h.x, __fdiv_rn(__fsub_rn(q.x, u.x), denom));
+                h.y = __fadd_rn(h.y, __fdiv_rn(__fsub_rn(q.y, u.y), denom));
+                h.z = __fadd_rn(h.z, __fdiv_rn(__fsub_rn(q.z, u.z), denom));
+                h.w = __fadd_rn(h.w, __fdiv_rn(__fsub_rn(q.w, u.w), denom));
+                nt_store(h, g4 + j2);
+            }
         }
         for (size_t j = (n4 << 2) + i; j < n; j += nt)
             grad[j] = __fadd_rn(grad[j], __fdiv_rn(__fsub_rn(probs[j], target[j]), denom));
@@ -336,10 +451,15 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
     if (int rc = check_rows("smce_fwd", rows, cols)) return rc;
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
-    const int tpr = pick_tpr(cols);
-    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
-    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_rows_kernel<T, 1>), dim3(grid), dim3(kBlock), 0, ctx->stream,
-                                            logits, target, probs, row_loss, rows, cols));
+    if (long_row_ok(logits, target, probs, rows, cols)) {
+        hipLaunchKernelGGL((softmax_long_rows_kernel<1>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
+                           logits, target, probs, row_loss, cols);
+    } else {
+        const int tpr = pick_tpr(cols);
+        const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+        ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_rows_kernel<T, 1>), dim3(grid), dim3(kBlock), 0, ctx->stream,
+                                                logits, target, probs, row_loss, rows, cols));
+    }
     ZG_LAUNCH_CHECK();
     return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows});
 }
@@ -362,10 +482,15 @@ ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t 
     ZG_CTX(ctx);
     ZG_REQUIRE(x && y, "softmax_fwd: null pointer");
     if (int rc = check_rows("softmax_fwd", rows, cols)) return rc;
-    const int tpr = pick_tpr(cols);
-    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
-    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_rows_kernel<T, 0>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
-                                            (const float*)nullptr, y, (float*)nullptr, rows, cols));
+    if (long_row_ok(x, x, y, rows, cols)) {
+        hipLaunchKernelGGL((softmax_long_rows_kernel<0>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream, x,
+                           (const float*)nullptr, y, (float*)nullptr, cols);
+    } else {
+        const int tpr = pick_tpr(cols);
+        const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+        ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_rows_kernel<T, 0>), dim3(grid), dim3(kBlock), 0, ctx->stream, x,
+                                                (const float*)nullptr, y, (float*)nullptr, rows, cols));
+    }
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

@@ -173,13 +173,18 @@ struct GemmArgs {
 };
 
 // Logical tile id from the hardware workgroup id.  Hardware deals consecutive ids round-robin to the 8
-// XCDs; give each XCD a contiguous run of logical ids, then walk C in column groups of 8 tile-rows.
+// XCDs; give each XCD a contiguous run of logical ids, then walk C in column groups of GM tile-rows.
+// GM = 4: the two workgroups that share a CU do not advance at the same speed (the one placed first wins the
+// arbitration and runs about 17 % ahead), so an XCD's resident workgroups split into an early and a late half
+// that stop sharing L2 lines after a few dozen k-tiles.  Each half is a run of 32 consecutive ids; 4 rows x 8
+// columns is the shape of such a run with the fewest A and B panel bytes for the 256 x 128 tile (8 rows x 4
+// columns fetched 47 % more from the fabric, measured with FETCH_SIZE).
 __device__ __forceinline__ void tile_coords(unsigned pid, unsigned tiles_m, unsigned tiles_n, unsigned& tm,
                                             unsigned& tn) {
     const unsigned total = tiles_m * tiles_n;
     unsigned id = pid;
     if ((total & 7u) == 0) id = (pid & 7u) * (total >> 3) + (pid >> 3);
-    constexpr unsigned GM = 8;
+    constexpr unsigned GM = 4;
     const unsigned per_group = GM * tiles_n;
     const unsigned group = id / per_group;
     const unsigned first_m = group * GM;

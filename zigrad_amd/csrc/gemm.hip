@@ -471,6 +471,101 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
     return ZG_HIP_OK;
 }
 
+// Small products (k <= 256, at most a few hundred 32x32 blocks of C): the staged kernel's fixed costs (two tiles of
+// prologue, LDS round trips, a barrier per tile) dominate there.  Here a workgroup owns one 32x32 block of C and
+// its four waves split k between them in groups of 8 (wave w takes groups w, w+4, ...).  Operands go straight
+// from memory to the MFMA operand registers with the same k assignment as the staged kernel (lane half h, step c
+// of group g: k = 8g + 4h + c), so a k-contiguous operand is one 16-byte load per lane and group; every load is
+// guarded and zero-filled, so any shape and alignment is served.  The four partial blocks are added in wave
+// order through LDS: the result does not depend on scheduling.
+template <bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
+    __shared__ float part[4][16][64];
+    const size_t m0 = (size_t)(blockIdx.x / g.tiles_n) * 32, n0 = (size_t)(blockIdx.x % g.tiles_n) * 32;
+    const size_t z = blockIdx.z;
+    const float* A = g.A + (z % g.nba) * g.a_chunk;
+    const float* B = g.B + (z % g.nbb) * g.b_chunk;
+    float* C = g.C + z * g.c_chunk;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const size_t K = g.K, groups = (K + 7) / 8;
+
+    auto fragment = [&](const float* P, bool kmajor, size_t ld, size_t idx, size_t limit, bool vec_ok, size_t grp) {
+        floatx4 v = {0.f, 0.f, 0.f, 0.f};
+        const size_t k0 = grp * 8 + (size_t)lk * 4;
+        if (idx < limit && k0 < K) {
+            if (kmajor) {
+                const float* q = P + idx * ld + k0;
+                if (vec_ok && k0 + 4 <= K) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        if (k0 + c < K) v[c] = q[c];
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (k0 + c < K) v[c] = P[(k0 + c) * ld + idx];
+            }
+        }
+        return v;
+    };
+    auto frag_a = [&](size_t grp) { return fragment(A, A_KMAJOR, g.lda, m0 + l32, g.M, g.a_vec != 0, grp); };
+    auto frag_b = [&](size_t grp) { return fragment(B, B_KMAJOR, g.ldb, n0 + l32, g.N, g.b_vec != 0, grp); };
+
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    size_t grp = wave;
+    floatx4 a_cur = {0.f, 0.f, 0.f, 0.f}, b_cur = a_cur;
+    if (grp < groups) {
+        a_cur = frag_a(grp);
+        b_cur = frag_b(grp);
+    }
+    for (; grp < groups; grp += 4) {
+        floatx4 a_nxt = {0.f, 0.f, 0.f, 0.f}, b_nxt = a_nxt;
+        if (grp + 4 < groups) {  // the next group's loads are in flight under this group's MFMAs
+            a_nxt = frag_a(grp + 4);
+            b_nxt = frag_b(grp + 4);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[c], b_cur[c], acc, 0, 0, 0);
+        a_cur = a_nxt;
+        b_cur = b_nxt;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) part[wave][r][lane] = acc[r];
+    __syncthreads();
+    const float alpha = g.alpha, beta = g.beta;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int e = threadIdx.x + q * kGemmThreads, r = e >> 6, ln = e & 63;
+        float s = part[0][r][ln];
+        s += part[1][r][ln];
+        s += part[2][r][ln];
+        s += part[3][r][ln];
+        const size_t row = m0 + (r >> 2) * 8 + (ln >> 5) * 4 + (r & 3), col = n0 + (ln & 31);
+        if (row < g.M && col < g.N) {
+            float v = alpha * s;
+            if (beta != 0.f) v += beta * C[row * g.ldc + col];
+            C[row * g.ldc + col] = v;
+        }
+    }
+}
+
+static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, size_t batches) {
+    g.tiles_m = (unsigned)ceil_div_sz(g.M, 32);
+    g.tiles_n = (unsigned)ceil_div_sz(g.N, 32);
+    dim3 grid(g.tiles_m * g.tiles_n, 1, (unsigned)batches), block(kGemmThreads);
+    if (a_kmajor && b_kmajor) hipLaunchKernelGGL((gemm_tiny_kernel<true, true>), grid, block, 0, ctx->stream, g);
+    else if (a_kmajor && !b_kmajor) hipLaunchKernelGGL((gemm_tiny_kernel<true, false>), grid, block, 0, ctx->stream, g);
+    else if (!a_kmajor && b_kmajor) hipLaunchKernelGGL((gemm_tiny_kernel<false, true>), grid, block, 0, ctx->stream, g);
+    else hipLaunchKernelGGL((gemm_tiny_kernel<false, false>), grid, block, 0, ctx->stream, g);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
 // C = alpha * (sum of the split-K partial products, in split order) + beta * C.  P is [batch][split][M][N] dense.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, float* C, size_t M, size_t N, size_t ldc,
                                                             int splits, float alpha, float beta, size_t c_chunk) {
@@ -575,6 +670,8 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         return gemm_dispatch(ctx, name, a_tail, b_tail, C, m, n, k - k_main, trans_a, trans_b, lda, ldb, ldc, alpha, 1.f,
                              batches, nba, nbb, a_chunk, b_chunk, c_chunk, 1);
     }
+
+    if (k <= 256 && tiles(32, 32) <= n_cu) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
 
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
     if (c_large <= c_mid && c_large <= c_small)

@@ -403,6 +403,13 @@ def main():
         result["ops"] = op_suite(dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH)
+        # the same CPU oracle on the batch-64 MLP, the configuration the reference runs today
+        from oracle.oracle_device import OracleDevice
+
+        odev = OracleDevice()
+        threads = odev.set_threads(min(16, os.cpu_count() or 1))
+        dt_cpu, _ = run_mlp(odev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01)
+        result["mlp_b64"]["cpu_oracle"] = {"steps_per_s": 200 / dt_cpu, "ms_per_step": dt_cpu / 200 * 1e3, "cores": threads}
     else:
         result["cpu_baseline"] = None
     dev.deinit()

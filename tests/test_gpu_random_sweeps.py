@@ -1,0 +1,130 @@
+"""Seeded random sweeps over shapes, transposes, leading dimensions and scalars.  Every GEMM path (tiny, split-k,
+fast / edge / checked kernels of each tile size), the broadcasting regimes and the axis reductions are hit many
+times with sizes nobody picked by hand; results are compared with float64 numpy."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from conftest import rel_fro
+from zigrad_amd.device import F32
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def _dim(r, hi):
+    """Sizes biased towards tile edges: multiples of 32/64/128 and their neighbours as well as arbitrary values."""
+    kind = r.integers(0, 4)
+    if kind == 0:
+        return int(r.integers(1, hi + 1))
+    base = int(r.choice([32, 64, 128, 256])) * int(r.integers(1, max(2, hi // 256 + 1)))
+    return max(1, min(hi, base + int(r.choice([-1, 0, 0, 1, 4]))))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_matmul_random_cases(hip, seed):
+    r = np.random.default_rng(1000 + seed)
+    for case in range(30):
+        m, n, k = _dim(r, 700), _dim(r, 700), _dim(r, 1500)
+        ta, tb = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+        pa, pb, pc = (int(r.choice([0, 0, 4, 3])) for _ in range(3))
+        lda, ldb, ldc = (m if ta else k) + pa, (k if tb else n) + pb, n + pc
+        alpha = float(r.choice([1.0, 0.5, -1.25]))
+        beta = float(r.choice([0.0, 1.0, -0.5]))
+        A = np.full((k if ta else m, lda), np.nan, np.float32)
+        B = np.full((n if tb else k, ldb), np.nan, np.float32)
+        C0 = np.full((m, ldc), np.nan, np.float32)
+        A[:, : (m if ta else k)] = r.standard_normal((A.shape[0], m if ta else k))
+        B[:, : (k if tb else n)] = r.standard_normal((B.shape[0], k if tb else n))
+        if beta != 0.0:
+            C0[:, :n] = r.standard_normal((m, n))
+        a, b, c = hip.from_numpy(A), hip.from_numpy(B), hip.from_numpy(C0)
+        hip.dispatch("matmul", A=a, B=b, C=c, m=m, n=n, k=k, trans_a=ta, trans_b=tb, lda=lda, ldb=ldb, ldc=ldc,
+                     alpha=alpha, beta=beta)
+        got = hip.to_numpy(c).reshape(m, ldc)
+        for x in (a, b, c):
+            hip.mem_free(x)
+        A64 = A[:, : (m if ta else k)].astype(np.float64)
+        B64 = B[:, : (k if tb else n)].astype(np.float64)
+        want = alpha * ((A64.T if ta else A64) @ (B64.T if tb else B64))
+        if beta != 0.0:
+            want = want + beta * C0[:, :n].astype(np.float64)
+        what = (seed, case, m, n, k, ta, tb, lda, ldb, ldc, alpha, beta)
+        assert not np.isnan(got[:, :n]).any(), what
+        scale = np.linalg.norm(want) + np.sqrt(m * n) * 1e-3  # products that cancel to nearly nothing stay meaningful
+        assert np.linalg.norm(got[:, :n] - want) <= TOL * scale, what
+        if pc:
+            assert np.isnan(got[:, n:]).all(), what  # padding of C untouched
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_bmm_random_cases(hip, seed):
+    r = np.random.default_rng(2000 + seed)
+    for case in range(10):
+        nbc = int(r.integers(1, 7))
+        nba, nbb = (int(r.choice([1, nbc])) for _ in range(2))
+        m, n, k = _dim(r, 200), _dim(r, 200), _dim(r, 600)
+        ta, tb = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+        A = r.standard_normal((nba, k, m) if ta else (nba, m, k)).astype(np.float32)
+        B = r.standard_normal((nbb, n, k) if tb else (nbb, k, n)).astype(np.float32)
+        C0 = r.standard_normal((nbc, m, n)).astype(np.float32)
+        a, b, c = hip.from_numpy(A), hip.from_numpy(B), hip.from_numpy(C0)
+        hip.dispatch("bmm_acc", A=a, B=b, C=c, A_shape=[nba, m, k], B_shape=[nbb, k, n], C_shape=[nbc, m, n], trans_a=ta,
+                     trans_b=tb, lda=A.shape[2], ldb=B.shape[2], ldc=n, alpha=1.0, beta=1.0)
+        got = hip.to_numpy(c).reshape(nbc, m, n)
+        for x in (a, b, c):
+            hip.mem_free(x)
+        want = np.stack([(A[i % nba].astype(np.float64).T if ta else A[i % nba].astype(np.float64))
+                         @ (B[i % nbb].astype(np.float64).T if tb else B[i % nbb].astype(np.float64)) for i in range(nbc)]) + C0
+        assert rel_fro(got, want) <= TOL, (seed, case, nbc, nba, nbb, m, n, k, ta, tb)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_axis_reductions_random_shapes(hip, seed):
+    r = np.random.default_rng(3000 + seed)
+    for case in range(15):
+        rank = int(r.integers(1, 5))
+        shape = [int(r.integers(1, 40)) for _ in range(rank)]
+        if r.integers(0, 3) == 0:
+            shape[int(r.integers(0, rank))] = int(r.integers(200, 3000))
+        dim = int(r.integers(0, rank))
+        X = r.standard_normal(shape).astype(np.float32)
+        n_out = X.size // shape[dim]
+        x = hip.from_numpy(X)
+        y = hip.mem_alloc(F32, n_out)
+        hip.mem_fill(y, 2.0)
+        alpha, beta = float(r.choice([1.0, 0.5])), float(r.choice([0.0, 1.0]))
+        hip.dispatch("sum_along", x=x, x_shape=shape, y=y, dim=dim, alpha=alpha, beta=beta)
+        want = alpha * X.astype(np.float64).sum(axis=dim).ravel() + beta * 2.0
+        assert np.linalg.norm(hip.to_numpy(y) - want) <= TOL * (np.linalg.norm(want) + 1e-3), (seed, case, shape, dim)
+        hip.mem_fill(y, 0.0)
+        hip.dispatch("max_along", x=x, x_shape=shape, y=y, dim=dim)
+        assert np.array_equal(hip.to_numpy(y), X.max(axis=dim).ravel()), (seed, case, shape, dim)
+        idx = hip.mem_alloc(np.uint64, n_out)
+        hip.dispatch("argmax_along", x=x, x_shape=shape, y=idx, dim=dim)
+        assert np.array_equal(hip.to_numpy(idx), X.argmax(axis=dim).ravel().astype(np.uint64)), (seed, case, shape, dim)
+        for b in (x, y, idx):
+            hip.mem_free(b)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_elementwise_broadcast_random_lengths(hip, seed):
+    """z = x op y with the shorter operand restarting every min(len) elements (src/device/host_device.zig:975-1019)."""
+    r = np.random.default_rng(4000 + seed)
+    ops = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}
+    for case in range(25):
+        short = int(r.choice([1, 3, 4, 7, 64, 100, 128, 1000, 4096]))
+        reps = int(r.integers(1, 60))
+        long_n = short * reps
+        name = str(r.choice(list(ops)))
+        swap = bool(r.integers(0, 2))
+        S = (r.standard_normal(short) + 3.0).astype(np.float32)
+        L = (r.standard_normal(long_n) + 3.0).astype(np.float32)
+        X, Y = (S, L) if swap else (L, S)
+        x, y, z = hip.from_numpy(X), hip.from_numpy(Y), hip.mem_alloc(F32, long_n)
+        hip.dispatch(name, x=x, y=y, z=z)
+        want = ops[name](np.resize(X, long_n), np.resize(Y, long_n))  # one IEEE operation per element: exact
+        assert np.array_equal(hip.to_numpy(z), want), (seed, case, name, short, reps, swap)
+        for b in (x, y, z):
+            hip.mem_free(b)

@@ -128,3 +128,43 @@ def test_elementwise_broadcast_random_lengths(hip, seed):
         assert np.array_equal(hip.to_numpy(z), want), (seed, case, name, short, reps, swap)
         for b in (x, y, z):
             hip.mem_free(b)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_scatter_ops_random_graphs_bit_exact(oracle, hip, seed):
+    """Random edge lists with isolated nodes, hubs and strides that are not powers of two: scatter_add, the GCN
+    scatter and its backward, index_select backward -- bit for bit against the sequential host loops."""
+    from conftest import run_op
+
+    r = np.random.default_rng(5000 + seed)
+    for case in range(6):
+        n_nodes = int(r.integers(1, 4000))
+        n_edge = int(r.integers(0, 6000))
+        stride = int(r.choice([1, 3, 7, 16, 20, 33, 64]))
+        hub = int(r.integers(0, n_nodes))
+        src = r.integers(0, n_nodes, n_edge).astype(np.uint64)
+        tgt = np.where(r.random(n_edge) < 0.2, hub, r.integers(0, n_nodes, n_edge)).astype(np.uint64)
+        what = (seed, case, n_nodes, n_edge, stride)
+        if n_edge:
+            vals = r.standard_normal(n_edge).astype(np.float32)
+            d0 = r.standard_normal(n_nodes).astype(np.float32)
+            p = {"src": vals, "offsets": tgt, "dst": d0}
+            assert np.array_equal(run_op(oracle, "scatter_add", dict(p), ["dst"])["dst"], run_op(hip, "scatter_add", dict(p), ["dst"])["dst"]), what
+        h = r.standard_normal(n_nodes * stride).astype(np.float32)
+        deg = (r.random(n_nodes) + 0.25).astype(np.float32)
+        p = {"dst": r.standard_normal(n_nodes * stride).astype(np.float32), "h": h, "deg": deg, "src_indices": src,
+             "tgt_indices": tgt, "stride": stride, "n_edge": n_edge}
+        assert np.array_equal(run_op(oracle, "scatter_gcn_deg_scaled", dict(p), ["dst"])["dst"],
+                              run_op(hip, "scatter_gcn_deg_scaled", dict(p), ["dst"])["dst"]), what
+        p = {"grad_output": r.standard_normal(n_nodes * stride).astype(np.float32), "h": h, "deg": deg, "src_indices": src,
+             "tgt_indices": tgt, "grad_h": r.standard_normal(n_nodes * stride).astype(np.float32),
+             "grad_deg": r.standard_normal(n_nodes).astype(np.float32), "stride": stride, "n_edge": n_edge}
+        a = run_op(oracle, "scatter_gcn_deg_scaled_bwd", dict(p), ["grad_h", "grad_deg"])
+        b = run_op(hip, "scatter_gcn_deg_scaled_bwd", dict(p), ["grad_h", "grad_deg"])
+        assert np.array_equal(a["grad_h"], b["grad_h"]) and np.array_equal(a["grad_deg"], b["grad_deg"]), what
+        n_idx = int(r.integers(1, 3000))
+        idx = r.integers(0, n_nodes, n_idx).astype(np.uint64)
+        p = {"y_grad": r.standard_normal(n_idx * stride).astype(np.float32), "indices": idx, "stride": stride,
+             "x_grad": r.standard_normal(n_nodes * stride).astype(np.float32)}
+        assert np.array_equal(run_op(oracle, "index_select_bwd", dict(p), ["x_grad"])["x_grad"],
+                              run_op(hip, "index_select_bwd", dict(p), ["x_grad"])["x_grad"]), what

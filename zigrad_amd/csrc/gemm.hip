@@ -82,9 +82,14 @@ struct Tile {
         return KMAJOR ? mn * LD + k : k * LD + mn;
     }
 
-    // fast path: `base` is the tile origin (uniform), `off` this thread's byte offset of piece i
+    // fast path: `base` is the tile origin (uniform), `off` this thread's byte offset of piece i.  A buffer load
+    // takes the base as a scalar resource and the offset as one 32-bit VGPR, so moving along k costs scalar adds
+    // only (a flat global load needs a 64-bit vector add per piece and tile).
     __device__ __forceinline__ void load_fast(int i, const float* __restrict__ base, unsigned off) {
-        r[i] = *reinterpret_cast<const floatx4*>(reinterpret_cast<const char*>(base) + off);
+        typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)0xffffffffu, 0x00020000);
+        r[i] = __builtin_bit_cast(floatx4, (uintx4)__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
     }
 
     // checked path: zero fill outside [0, MN) x [0, K), scalar loads where 16-byte loads are not legal

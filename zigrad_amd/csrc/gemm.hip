@@ -243,7 +243,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // this workgroup's range of k
     const size_t k_begin = (size_t)blockIdx.y * g.split_tiles * BK;
     const size_t k_end = (k_begin + g.split_tiles * BK < g.K) ? k_begin + g.split_tiles * BK : g.K;
-    const size_t KT = (k_end - k_begin + BK - 1) / BK;
+    // 32-bit tile counter: there is no scalar 64-bit ordered compare, and a vector compare in the loop costs MFMA time
+    const unsigned KT = (unsigned)((k_end - k_begin + BK - 1) / BK);
     constexpr int NM = TM * TN;         // MFMAs per step
     constexpr int NMF = 4 * NM;         // MFMAs per k-group
     constexpr int NR = FA::N + FB::N;   // fragment reads per k-group
@@ -318,11 +319,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     constexpr int E0 = NL + NR + NL;
     constexpr int PER0 = (E0 + NMF - 1) / NMF;
     constexpr int PER1 = (NR + (NMF + 1) / 2 - 1) / ((NMF + 1) / 2);  // reads land in the first half of group 1
-    auto tile_step = [&](size_t kt, auto parity_tag) {
+    auto tile_step = [&](unsigned kt, auto parity_tag) {
         constexpr int S = decltype(parity_tag)::value;  // kt % 2: LDS buffer and register slot of this tile
         using SCur = std::integral_constant<int, S>;
         using SNext = std::integral_constant<int, S ^ 1>;
-        const size_t k_load = k_begin + ((SAFE || kt + 2 < KT) ? (kt + 2) * BK : (KT - 1) * BK);
+        const size_t k_load = k_begin + (size_t)((SAFE || kt + 2 < KT) ? kt + 2 : KT - 1) * BK;
 #pragma unroll
         for (int grp = 0; grp < 2; grp++) {
 #pragma unroll
@@ -367,7 +368,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 
     // Tiles go in pairs so that the loop body is one straight run of MFMAs.  The fast kernels are only used for
     // an even number of tiles; in the checked kernels a tile past the end of k loads as zeros and adds nothing.
-    for (size_t kt = 0; kt < KT; kt += 2) {
+    for (unsigned kt = 0; kt < KT; kt += 2) {
         tile_step(kt, P0{});
         tile_step(kt + 1, P1{});
     }

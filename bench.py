@@ -94,6 +94,16 @@ def time_op(dev, fn, iters, warm_ms=60.0, batches=10):
     The warm-up runs for at least `warm_ms` of wall time: the GPU raises its clock only under sustained load, and a
     kernel timed in the first tens of milliseconds after idle reads 10 % slower than in a training loop.
     """
+    if dev.is_host():  # the CPU oracle: wall clock around synchronous calls
+        ms = []
+        for _ in range(batches):
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                fn()
+            ms.append((time.perf_counter() - t0) * 1e3 / iters)
+        ms.sort()
+        pick = lambda q: ms[min(len(ms) - 1, int(q * len(ms)))]
+        return {"ms": pick(0.5), "ms_p10": pick(0.1), "ms_p90": pick(0.9)}
     t0 = time.perf_counter()
     while True:
         for _ in range(iters):
@@ -129,13 +139,17 @@ def copy_calibration(dev):
     dev.mem_free(y)
 
 
-def op_suite(dev, quick=False):
-    """configs[1]: per-op time, achieved TFLOP/s or GB/s from the algorithmic work, fraction of roofline."""
+def op_suite(dev, quick=False, cpu=False):
+    """configs[1]: per-op time, achieved TFLOP/s or GB/s from the algorithmic work, fraction of roofline.
+
+    With cpu=True `dev` is the CPU oracle: the same ops, one call per timing, three timings each, and the loss
+    kernels on the first 1024 of the 8192 rows (rows are independent; the rate is what is reported)."""
     from zigrad_amd.device import F32, U64
 
     out = {}
     r = np.random.default_rng(0)
     iters = 5 if quick else 20
+    timed = (lambda d, fn, it: time_op(d, fn, 1, batches=3)) if cpu else time_op
 
     def tfl(flops, t):
         tf = flops / (t["ms"] * 1e-3) / 1e12
@@ -150,12 +164,12 @@ def op_suite(dev, quick=False):
     n = 4096
     A, B, C = dev_normal(n * n), dev_normal(n * n), dev_normal(n * n)
     for tag, ta, tb in (("matmul_4096_nn", False, False), ("matmul_4096_tn", True, False), ("matmul_4096_nt", False, True)):
-        t = time_op(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=n, n=n, k=n, trans_a=ta, trans_b=tb, lda=n, ldb=n,
+        t = timed(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=n, n=n, k=n, trans_a=ta, trans_b=tb, lda=n, ldb=n,
                                                ldc=n, alpha=1.0, beta=0.0), iters)
         out[tag] = tfl(2 * n ** 3, t)
     # bmm 32 x 512^3
     nb, s = 32, 512
-    t = time_op(dev, lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, s, s], B_shape=[nb, s, s], C_shape=[nb, s, s],
+    t = timed(dev, lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, s, s], B_shape=[nb, s, s], C_shape=[nb, s, s],
                                            trans_a=False, trans_b=False, lda=s, ldb=s, ldc=s, alpha=1.0, beta=0.0), iters * 5)
     out["bmm_32x512"] = tfl(2 * nb * s ** 3, t)
     for b in (A, B, C):
@@ -170,27 +184,27 @@ def op_suite(dev, quick=False):
         g = nbytes / (t["ms"] * 1e-3) / 1e9
         return {**t, "gbs": g, "frac_hbm": g / PEAK_HBM_GBS}
 
-    ms = time_op(dev, lambda: dev.dispatch("add", x=X, y=bias, z=Z), iters * 5)
+    ms = timed(dev, lambda: dev.dispatch("add", x=X, y=bias, z=Z), iters * 5)
     out["add_bcast_8192x4096"] = gbs((2 * rows * cols + cols) * 4, ms)
-    ms = time_op(dev, lambda: dev.dispatch("sum_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
+    ms = timed(dev, lambda: dev.dispatch("sum_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
     out["sum_axis1_8192x4096"] = gbs((rows * cols + rows) * 4, ms)
-    ms = time_op(dev, lambda: dev.dispatch("max_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
+    ms = timed(dev, lambda: dev.dispatch("max_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
     out["max_axis1_8192x4096"] = gbs((rows * cols + rows) * 4, ms)
     for b in (X, bias, Z, yrow):
         dev.mem_free(b)
 
     # fused softmax cross-entropy, integer labels, logits [8192, 32000]
-    M, N = 8192, 32000
+    M, N = (1024 if cpu else 8192), 32000
     logits, grad = dev_normal(M * N), dev.mem_alloc(F32, M * N)
     labels = dev.from_numpy(r.integers(0, N, M).astype(np.uint64))
     lse, loss = dev.mem_alloc(F32, M), dev.mem_alloc(F32, 1)
-    ms = time_op(dev, lambda: dev.dispatch("smce_label_fwd", logits=logits, labels=labels, lse=lse, loss=loss, rows=M, cols=N),
+    ms = timed(dev, lambda: dev.dispatch("smce_label_fwd", logits=logits, labels=labels, lse=lse, loss=loss, rows=M, cols=N),
                  iters)
     out["smce_fwd_8192x32000"] = gbs(4 * M * N + 8 * M + 4, ms)
-    ms = time_op(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
+    ms = timed(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
                                             accumulate=False), iters)
     out["smce_bwd_8192x32000"] = gbs(2 * 4 * M * N, ms)
-    ms = time_op(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
+    ms = timed(dev, lambda: dev.dispatch("smce_label_bwd", logits=logits, labels=labels, lse=lse, grad=grad, rows=M, cols=N,
                                             accumulate=True), iters)
     out["smce_bwd_accumulate_8192x32000"] = gbs(3 * 4 * M * N, ms)
     # the reference's own form of the loss: float one-hot targets, probabilities saved for backward
@@ -198,10 +212,10 @@ def op_suite(dev, quick=False):
     target, probs = dev.mem_alloc(F32, M * N), dev.mem_alloc(F32, M * N)
     dev.mem_fill(target, 0.0)
     dev.mem_fill(grad, 0.0)
-    ms = time_op(dev, lambda: dev.dispatch("smce_fwd", logits=logits, target=target, probs=probs, loss=loss, rows=M, cols=N),
+    ms = timed(dev, lambda: dev.dispatch("smce_fwd", logits=logits, target=target, probs=probs, loss=loss, rows=M, cols=N),
                  iters // 2)
     out["smce_onehot_fwd_8192x32000"] = gbs(3 * 4 * M * N, ms)
-    ms = time_op(dev, lambda: dev.dispatch("smce_bwd", probs=probs, target=target, grad=grad, rows=M, cols=N), iters // 2)
+    ms = timed(dev, lambda: dev.dispatch("smce_bwd", probs=probs, target=target, grad=grad, rows=M, cols=N), iters // 2)
     out["smce_onehot_bwd_8192x32000"] = gbs(4 * 4 * M * N, ms)
     for b in (logits, grad, labels, lse, loss, target, probs):
         dev.mem_free(b)
@@ -218,7 +232,8 @@ def timed_steps(dev, step_fn, steps):
     return time.perf_counter() - t0, loss
 
 
-def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3, graph=False):
+def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3, graph=False,
+            late_read=False):
     """Returns (seconds, last loss) for `steps` eager steps; with graph=True also the same for `steps` replays of
     the step recorded as an execution graph (the loss is read back every step in both modes)."""
     from zigrad_amd.trainers import MLPTrainer, mlp_inputs
@@ -234,6 +249,11 @@ def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_m
     dt, loss = timed_steps(dev, tr.step, steps)
     if timer is not None:
         timer.on = False
+    if late_read:  # the same steps with the loss read moved behind the optimizer step (the queue never drains)
+        late = lambda: tr.step(read_loss="late")
+        late()
+        dt_late, loss_late = timed_steps(dev, late, steps)
+        return dt, loss, dt_late, loss_late
     if not graph:
         return dt, loss
     tr.capture()
@@ -354,7 +374,8 @@ def main():
     copy_calibration(dev)
     timer = GemmTimer(dev)
     timer.install()
-    dt, loss = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", timer, args.loss_mode)
+    dt, loss, dt_late, _ = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", timer, args.loss_mode,
+                                   late_read=True)
     ms_per_step = dt / args.steps * 1e3
     gemm_ms = timer.total_ms()
     n_launch = len(timer.pairs)
@@ -390,6 +411,9 @@ def main():
             "launches_timed": n_launch,
         },
     }
+    # `value` reads the loss where the reference's loop does (before backward: the host blocks and the GPU idles until
+    # the backward launches arrive); the same step with that one read moved behind the optimizer step:
+    result["late_loss_read"] = {"steps_per_s": args.steps / dt_late, "ms_per_step": dt_late / args.steps * 1e3}
     # the latency-bound configurations: batch-64 MLP (configs[0]), GCN (configs[2]), DQN update (configs[3])
     if not args.no_small:
         small = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=not args.no_graph)
@@ -412,6 +436,20 @@ def main():
         threads = odev.set_threads(min(16, os.cpu_count() or 1))
         dt_cpu, _ = run_mlp(odev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01)
         result.setdefault("mlp_b64", {})["cpu_oracle"] = {"steps_per_s": 200 / dt_cpu, "ms_per_step": dt_cpu / 200 * 1e3, "cores": threads}
+        if not args.no_small:
+            for kind in ("gcn", "dqn"):
+                c = run_small(odev, kind, 50, graph=False)
+                result[kind]["cpu_oracle"] = {"steps_per_s": c["steps_per_s"], "ms_per_step": c["ms_per_step"], "cores": threads}
+        if not args.no_ops:
+            # the op suite on the host cores beside the GPU figures (BLAS on `threads` cores, everything else the
+            # oracle's scalar loops on one core)
+            strip = lambda d: {k: v for k, v in d.items() if not k.startswith("frac_")}
+            for name, c in op_suite(odev, cpu=True).items():
+                result["ops"][name]["cpu_oracle"] = strip(c)
+                if name.startswith("smce"):
+                    result["ops"][name]["cpu_oracle"]["rows_timed"] = 1024
+            result["ops_cpu_oracle"] = {"cores_blas": threads, "cores_other": 1, "blas": odev.blas_name(),
+                                        "sample": "one call per timing, median of 3; loss kernels on 1024 of the 8192 rows"}
     else:
         result["cpu_baseline"] = None
     dev.deinit()

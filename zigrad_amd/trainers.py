@@ -352,7 +352,10 @@ class MLPTrainer(GraphSteps):
         """Train on batch buffers owned by the caller (a BatchStager slot) from the next step on."""
         self.x, self.onehot, self.labels = x, onehot, labels
 
-    def step(self, read_loss: bool = True, keep_grads: bool = False):
+    def step(self, read_loss=True, keep_grads: bool = False):
+        """One train step.  read_loss=True reads the loss where the reference's loop does (loss.get(0) before
+        backward, examples/mnist/src/main-simple.zig:67): the host blocks there and the GPU idles until the backward
+        launches arrive.  read_loss="late" moves the same read behind the optimizer step, so the queue never drains."""
         d, B, C = self.dev, self.batch, self.dims[-1]
         acts = self.net.forward(self.x, B)
         logits = acts[-1]
@@ -363,7 +366,7 @@ class MLPTrainer(GraphSteps):
         else:
             saved = d.mem_cache_alloc(F32, B)  # per-row log-sum-exp
             d.dispatch("smce_label_fwd", logits=logits, labels=self.labels, lse=saved, loss=loss, rows=B, cols=C)
-        loss_val = self._read_loss(loss) if read_loss else None  # loss.get(0): a blocking read before backward
+        loss_val = self._read_loss(loss) if read_loss is True else None  # loss.get(0): a blocking read before backward
 
         # backward
         loss_grad = d.mem_cache_alloc(F32, 1)
@@ -376,12 +379,14 @@ class MLPTrainer(GraphSteps):
             d.dispatch("smce_label_bwd", logits=logits, labels=self.labels, lse=saved, grad=g, rows=B, cols=C, accumulate=True)
         d.mem_cache_free(saved)
         d.mem_cache_free(loss_grad)
-        d.mem_cache_free(loss)
         self.net.backward(acts, g, B)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
         self.optim.step()
         self.net.zero_grad()  # model.zero_grad()
+        if read_loss == "late":
+            loss_val = self._read_loss(loss)
+        d.mem_cache_free(loss)
         return loss_val
 
 

@@ -168,3 +168,30 @@ def test_scatter_ops_random_graphs_bit_exact(oracle, hip, seed):
              "x_grad": r.standard_normal(n_nodes * stride).astype(np.float32)}
         assert np.array_equal(run_op(oracle, "index_select_bwd", dict(p), ["x_grad"])["x_grad"],
                               run_op(hip, "index_select_bwd", dict(p), ["x_grad"])["x_grad"]), what
+
+
+@pytest.mark.parametrize("n_nodes,n_edge", [(8191, 16384), (8192, 16384), (8191, 16385), (1, 16384), (300, 16000),
+                                            (20000, 40000), (5, 40000)])
+def test_scatter_ops_large_and_skewed_bit_exact(oracle, hip, n_nodes, n_edge):
+    """Edge lists around powers of two, a single destination, a few very long segments (30 % of all edges on one
+    node) and sizes that need the multi-tile scan: bit for bit against the sequential host loops."""
+    from conftest import run_op
+
+    r = np.random.default_rng(n_nodes * 7 + n_edge)
+    stride = 5
+    src = r.integers(0, n_nodes, n_edge).astype(np.uint64)
+    tgt = np.where(r.random(n_edge) < 0.3, n_nodes // 2, r.integers(0, n_nodes, n_edge)).astype(np.uint64)
+    p = {"src": r.standard_normal(n_edge).astype(np.float32), "offsets": tgt, "dst": r.standard_normal(n_nodes).astype(np.float32)}
+    assert np.array_equal(run_op(oracle, "scatter_add", dict(p), ["dst"])["dst"], run_op(hip, "scatter_add", dict(p), ["dst"])["dst"])
+    h = r.standard_normal(n_nodes * stride).astype(np.float32)
+    deg = (r.random(n_nodes) + 0.25).astype(np.float32)
+    p = {"grad_output": r.standard_normal(n_nodes * stride).astype(np.float32), "h": h, "deg": deg, "src_indices": src,
+         "tgt_indices": tgt, "grad_h": r.standard_normal(n_nodes * stride).astype(np.float32),
+         "grad_deg": r.standard_normal(n_nodes).astype(np.float32), "stride": stride, "n_edge": n_edge}
+    a = run_op(oracle, "scatter_gcn_deg_scaled_bwd", dict(p), ["grad_h", "grad_deg"])
+    b = run_op(hip, "scatter_gcn_deg_scaled_bwd", dict(p), ["grad_h", "grad_deg"])
+    assert np.array_equal(a["grad_h"], b["grad_h"]) and np.array_equal(a["grad_deg"], b["grad_deg"])
+    p = {"dst": r.standard_normal(n_nodes * stride).astype(np.float32), "h": h, "deg": deg, "src_indices": src,
+         "tgt_indices": tgt, "stride": stride, "n_edge": n_edge}
+    assert np.array_equal(run_op(oracle, "scatter_gcn_deg_scaled", dict(p), ["dst"])["dst"],
+                          run_op(hip, "scatter_gcn_deg_scaled", dict(p), ["dst"])["dst"])

@@ -694,7 +694,11 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         size_t per = ceil_div_sz(kt_total, splits);
         per += per & 1;
         splits = ceil_div_sz(kt_total, per);
-        if (splits >= 2) {
+        // Worth it only when the k-tiles saved on the busiest CU outweigh the second launch and the short loops:
+        // a 64x64 k-tile step takes about 0.27 us, the split's fixed costs about 6 us (768-cubed: 15.5 us whole,
+        // 20 us split four ways).
+        const double whole = (double)kt_total, busiest = (double)(ceil_div_sz(t64 * splits, n_cu) * per);
+        if (splits >= 2 && (whole - busiest) * 0.27 > 6.0) {
             float* part = (float*)workspace(ctx, batches * splits * m * n * sizeof(float));
             if (!part) return ZG_HIP_EOOM;
             GemmArgs gs = g;

@@ -36,3 +36,42 @@ def test_argument_errors_are_reported_without_a_gpu():
     n = ctypes.c_int(-1)
     assert lib.cdll.zg_hip_device_count(ctypes.byref(n)) == 0
     assert n.value >= 0
+
+
+def _zig_calls(text):
+    """(name, number of arguments) of every `c.zg_hip_*( ... )` call in Zig source, comments stripped."""
+    import re
+
+    text = re.sub(r"//[^\n]*", "", text)
+    for m in re.finditer(r"\bc\.(zg_hip_\w+)\s*\(", text):
+        depth, args, i, seen = 1, 0, m.end(), False
+        while depth:
+            ch = text[i]
+            if ch in "([{":
+                depth += 1
+            elif ch in ")]}":
+                depth -= 1
+            elif ch == "," and depth == 1:
+                args += 1
+            if depth and not ch.isspace():
+                seen = True
+            i += 1
+        # a trailing comma before the closing parenthesis is Zig's multi-line call style, not another argument
+        body = text[m.end(): i - 1].rstrip()
+        if body.endswith(","):
+            args -= 1
+        yield m.group(1), (args + 1 if seen else 0)
+
+
+def test_zig_veneer_calls_match_the_header():
+    """zig/hip_device.zig binds the library through @cImport of include/zg_hip.h: every entry point it calls must be
+    declared there with the number of arguments the call passes (no Zig toolchain here to compile it)."""
+    from pathlib import Path
+
+    protos = parse_header()
+    text = (Path(__file__).resolve().parents[1] / "zig" / "hip_device.zig").read_text()
+    calls = list(_zig_calls(text))
+    assert len({n for n, _ in calls}) >= 80
+    for name, n_args in calls:
+        assert name in protos, f"{name} is called by the veneer but not declared in zg_hip.h"
+        assert n_args == len(protos[name][1]), f"{name}: veneer passes {n_args} arguments, header declares {len(protos[name][1])}"

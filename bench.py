@@ -233,13 +233,13 @@ def timed_steps(dev, step_fn, steps):
 
 
 def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3, graph=False,
-            late_read=False):
+            late_read=False, fused=False):
     """Returns (seconds, last loss) for `steps` eager steps; with graph=True also the same for `steps` replays of
     the step recorded as an execution graph (the loss is read back every step in both modes)."""
     from zigrad_amd.trainers import MLPTrainer, mlp_inputs
 
     params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data=data)
-    tr = MLPTrainer(dev, dims, batch, optimizer=optimizer, lr=lr, clip=True, loss_mode=loss_mode)
+    tr = MLPTrainer(dev, dims, batch, optimizer=optimizer, lr=lr, clip=True, loss_mode=loss_mode, fused=fused)
     tr.load_params(params)
     tr.set_batch(x, onehot, labels)
     for _ in range(warmup):
@@ -414,6 +414,13 @@ def main():
     # `value` reads the loss where the reference's loop does (before backward: the host blocks and the GPU idles until
     # the backward launches arrive); the same step with that one read moved behind the optimizer step:
     result["late_loss_read"] = {"steps_per_s": args.steps / dt_late, "ms_per_step": dt_late / args.steps * 1e3}
+    # every Linear layer through the fused entry points (bias + ReLU in the GEMM epilogue, ReLU backward in the epilogue
+    # of the input-gradient product; same arithmetic, bit-identical parameters): not the reference's op sequence, so
+    # reported beside `value`, never as it
+    f = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", None, args.loss_mode, late_read=True,
+                fused=True)
+    result["fused_linear"] = {"steps_per_s": args.steps / f[0], "ms_per_step": f[0] / args.steps * 1e3,
+                              "late_loss_read": {"steps_per_s": args.steps / f[2], "ms_per_step": f[2] / args.steps * 1e3}}
     # the latency-bound configurations: batch-64 MLP (configs[0]), GCN (configs[2]), DQN update (configs[3])
     if not args.no_small:
         small = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=not args.no_graph)
@@ -422,6 +429,10 @@ def main():
                                          "graph_replay = the same step recorded once as an execution graph"}
         if not args.no_graph:
             result["mlp_b64"]["graph_replay"] = {"steps_per_s": 200 / small[2], "ms_per_step": small[2] / 200 * 1e3}
+        if not args.no_graph:
+            fs = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=True, fused=True)
+            result["mlp_b64"]["fused_linear"] = {"steps_per_s": 200 / fs[0], "ms_per_step": fs[0] / 200 * 1e3,
+                                                 "graph_replay": {"steps_per_s": 200 / fs[2], "ms_per_step": fs[2] / 200 * 1e3}}
         result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
         result["gcn"] = run_small(dev, "gcn", 100, graph=not args.no_graph)
         result["dqn"] = run_small(dev, "dqn", 200, graph=not args.no_graph)

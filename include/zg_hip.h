@@ -131,6 +131,17 @@ int zg_hip_matmul(zg_hip_ctx *ctx, const float *A, const float *B, float *C, siz
 int zg_hip_bmm_acc(zg_hip_ctx *ctx, const float *A, const uint64_t *A_shape, const float *B,
                    const uint64_t *B_shape, float *C, const uint64_t *C_shape, int trans_a, int trans_b, size_t lda,
                    size_t ldb, size_t ldc, float alpha, float beta);
+/* Fused Linear layer (the epilogue fusion the CUDA backend leaves open): the reference issues bmm_acc(trans_b) +
+ * bias.add_ (examples/mnist/src/model.zig:104-110) + relu_ (:38-46) as three device ops, and in backward
+ * relu_inplace_bwd (src/device/host_device.zig:543-547) + the dA product of BmmAccBwd (src/ndtensor.zig:1092-1136).
+ * These run the same arithmetic in one launch: y[batch, fan_out] = act(x[batch, fan_in] . w[fan_out, fan_in]^T +
+ * bias), bias may be null, relu != 0 applies max(0, .). */
+int zg_hip_linear_fwd(zg_hip_ctx *ctx, const float *x, const float *w, const float *bias, float *y, size_t batch,
+                      size_t fan_in, size_t fan_out, int relu);
+/* gx[batch, fan_in] = (accumulate ? gx : 0) + gy[batch, fan_out] . w, then gx = 0 where act_in <= 0; act_in is the
+ * ReLU output that fed the layer (null: no mask).  With accumulate == 0 gx is not read and needs no zero fill. */
+int zg_hip_linear_bwd_input(zg_hip_ctx *ctx, const float *gy, const float *w, const float *act_in, float *gx,
+                            size_t batch, size_t fan_in, size_t fan_out, int accumulate);
 int zg_hip_outer(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *A, float alpha);
 /* B = A^T + alpha*B; B is not read when alpha == 0 (the reference hands in uninitialised B then:
  * src/ndarray.zig:794-802) */

@@ -177,6 +177,22 @@ class OracleDevice(HipDevice):
         raise NotImplementedError("the oracle is timed with time.perf_counter")
 
     # -- entry points whose oracle signature differs from the C ABI ----------------------------------
+    def _x_zg_hip_linear_fwd(self, x, w, bias, y, batch, fan_in, fan_out, relu):
+        # the three ops the fused entry point stands for (examples/mnist/src/model.zig:104-110, :38-46)
+        c = self._o.cdll
+        c.zo_matmul(x, w, y, batch, fan_out, fan_in, 0, 1, fan_in, fan_in, fan_out, 1.0, 0.0)
+        if bias:
+            c.zo_add(bias, fan_out, y, batch * fan_out, y, batch * fan_out)
+        if relu:
+            c.zo_relu_fwd(y, y, batch * fan_out)
+
+    def _x_zg_hip_linear_bwd_input(self, gy, w, act_in, gx, batch, fan_in, fan_out, accumulate):
+        # dA of BmmAccBwd (src/ndtensor.zig:1092-1136) followed by relu_inplace_bwd (src/device/host_device.zig:543-547)
+        c = self._o.cdll
+        c.zo_matmul(gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in, 1.0, 1.0 if accumulate else 0.0)
+        if act_in:
+            c.zo_relu_inplace_bwd(act_in, gx, batch * fan_in)
+
     def _x_zg_hip_axpy(self, x, y, n, alpha, alpha_on_device):
         return self._o.cdll.zo_axpy(x, y, n, alpha)  # host memory either way
 

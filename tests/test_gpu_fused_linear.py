@@ -1,0 +1,106 @@
+"""The fused Linear entry points against the ops they stand for (examples/mnist/src/model.zig:104-110 forward,
+src/ndtensor.zig:1092-1136 + src/device/host_device.zig:543-547 backward): bit for bit against the separate device
+ops on the same inputs, to 1e-5 against float64, on shapes that reach every GEMM path (tiny, split-k, fast, edge and
+checked kernels of each tile size), and whole train steps with and without fusion."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from conftest import run_op
+from zigrad_amd.trainers import MLPTrainer, mlp_inputs
+
+pytestmark = pytest.mark.gpu
+
+# (batch, fan_in, fan_out)
+SHAPES = [(64, 784, 128), (64, 128, 64), (64, 64, 10), (1, 5, 3), (33, 70, 129), (256, 512, 384), (250, 512, 380),
+          (512, 96, 1024), (1024, 1024, 1024), (2048, 4096, 512), (130, 1433, 16), (300, 260, 7), (2048, 1000, 1024)]
+
+
+def _unfused_fwd(dev, x, w, b, relu):
+    B, I = x.shape
+    O = w.shape[0]
+    y = run_op(dev, "matmul", {"A": x, "B": w, "C": np.zeros((B, O), np.float32), "m": B, "n": O, "k": I, "trans_a": False,
+                               "trans_b": True, "lda": I, "ldb": I, "ldc": O, "alpha": 1.0, "beta": 0.0}, ["C"])["C"]
+    if b is not None:
+        y = run_op(dev, "add", {"x": b, "y": y, "z": np.zeros_like(y)}, ["z"])["z"]
+    if relu:
+        y = run_op(dev, "relu_fwd", {"x": y, "y": np.zeros_like(y)}, ["y"])["y"]
+    return y.reshape(B, O)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("relu,with_bias", [(True, True), (False, True), (True, False)])
+def test_linear_fwd_equals_the_three_ops(oracle, hip, shape, relu, with_bias):
+    B, I, O = shape
+    r = np.random.default_rng(B * 31 + I * 7 + O)
+    x = r.standard_normal((B, I)).astype(np.float32)
+    w = (r.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
+    b = r.standard_normal(O).astype(np.float32) if with_bias else None
+    p = {"x": x, "w": w, "bias": b, "y": np.full((B, O), np.nan, np.float32), "batch": B, "fan_in": I, "fan_out": O,
+         "relu": relu}
+    got = run_op(hip, "linear_fwd", dict(p), ["y"])["y"].reshape(B, O)
+    assert np.array_equal(got, _unfused_fwd(hip, x, w, b, relu)), shape
+    want = x.astype(np.float64) @ w.astype(np.float64).T + (b.astype(np.float64) if with_bias else 0.0)
+    if relu:
+        want = np.maximum(want, 0.0)
+    assert np.linalg.norm(got - want) <= 1e-5 * (np.linalg.norm(want) + 1e-3), shape
+    if B * I * O <= 1 << 22:  # the CPU oracle's composition of the same three ops
+        ref = run_op(oracle, "linear_fwd", dict(p), ["y"])["y"].reshape(B, O)
+        assert np.linalg.norm(got - ref) <= 1e-5 * (np.linalg.norm(ref) + 1e-3), shape
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("accumulate,masked", [(False, True), (True, True), (False, False)])
+def test_linear_bwd_input_equals_product_then_relu_backward(hip, shape, accumulate, masked):
+    B, I, O = shape
+    r = np.random.default_rng(B * 13 + I * 5 + O + 1)
+    gy = r.standard_normal((B, O)).astype(np.float32)
+    w = (r.standard_normal((O, I)) / np.sqrt(O)).astype(np.float32)
+    act = np.maximum(r.standard_normal((B, I)), 0.0).astype(np.float32) if masked else None  # a ReLU output: half zeros
+    gx0 = r.standard_normal((B, I)).astype(np.float32) if accumulate else np.full((B, I), np.nan, np.float32)
+    got = run_op(hip, "linear_bwd_input", {"gy": gy, "w": w, "act_in": act, "gx": gx0.copy(), "batch": B, "fan_in": I,
+                                            "fan_out": O, "accumulate": accumulate}, ["gx"])["gx"].reshape(B, I)
+    base = gx0.copy() if accumulate else np.zeros((B, I), np.float32)
+    ref = run_op(hip, "matmul", {"A": gy, "B": w, "C": base, "m": B, "n": I, "k": O, "trans_a": False, "trans_b": False,
+                                 "lda": O, "ldb": I, "ldc": I, "alpha": 1.0, "beta": 1.0}, ["C"])["C"]
+    if masked:
+        ref = run_op(hip, "relu_inplace_bwd", {"x": act, "x_g": ref}, ["x_g"])["x_g"]
+    assert np.array_equal(got, ref.reshape(B, I)), shape
+    want = gy.astype(np.float64) @ w.astype(np.float64) + (gx0 if accumulate else 0.0)
+    if masked:
+        want = np.where(act > 0, want, 0.0)
+    assert np.linalg.norm(got - want) <= 1e-5 * (np.linalg.norm(want) + 1e-3), shape
+
+
+@pytest.mark.parametrize("dims,batch,optimizer", [([784, 128, 64, 10], 64, "sgd"), ([100, 260, 130, 7], 50, "adam"),
+                                                  ([512, 768, 384, 32], 512, "adam")])
+def test_train_steps_with_and_without_fusion_agree_exactly(hip, dims, batch, optimizer):
+    params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=3, seed_data=4, data="normal")
+    out = []
+    for fused in (False, True):
+        tr = MLPTrainer(hip, dims, batch, optimizer=optimizer, lr=0.01, clip=True, fused=fused)
+        tr.load_params(params)
+        tr.set_batch(x, onehot, labels)
+        losses = [tr.step() for _ in range(4)]
+        out.append((losses, [hip.to_numpy(b) for b in tr.param_buffers()]))
+    assert out[0][0] == out[1][0]
+    for a, b in zip(out[0][1], out[1][1]):
+        assert np.array_equal(a, b)
+
+
+def test_fused_step_replays_from_an_execution_graph(hip):
+    dims, batch = [784, 128, 64, 10], 64
+    params, x, onehot, labels = mlp_inputs(dims, batch, data="uniform")
+    eager = MLPTrainer(hip, dims, batch, optimizer="sgd", lr=0.01, clip=True, fused=True)
+    graph = MLPTrainer(hip, dims, batch, optimizer="sgd", lr=0.01, clip=True, fused=True)
+    for tr in (eager, graph):
+        tr.load_params(params)
+        tr.set_batch(x, onehot, labels)
+    graph.capture()
+    for _ in range(5):
+        assert eager.step() == graph.step_graph()
+        hip.sync()
+    for a, b in zip(eager.param_buffers(), graph.param_buffers()):
+        assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b))
+    graph.free_graph()

@@ -459,6 +459,22 @@ pub fn adam_step(self: *const Self, T: type, p: anytype) void {
     check(c.zg_hip_adam_step(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.t, p.lr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
 }
 
+/// A Linear layer's forward in one launch: y = act(x . w^T + bias), the arithmetic of `bmm_acc(trans_b)` +
+/// `bias.add_` + `relu_` (examples/mnist/src/model.zig:104-110, :38-46).  `p.bias` is an optional slice.
+pub fn linear_fwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    const bias: ?[*]const T = if (p.bias) |b| b.ptr else null;
+    check(c.zg_hip_linear_fwd(self.ctx, p.x.ptr, p.w.ptr, bias, p.y.ptr, p.batch, p.fan_in, p.fan_out, @intFromBool(p.relu)));
+}
+/// The input gradient of a Linear layer with the ReLU backward of the layer before it in one launch:
+/// gx = (accumulate ? gx : 0) + gy . w, zeroed where `p.act_in` (that ReLU's output, optional) is <= 0:
+/// the dA product of BmmAccBwd (src/ndtensor.zig:1092-1136) + relu_inplace_bwd (src/device/host_device.zig:543-547).
+pub fn linear_bwd_input(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    const act: ?[*]const T = if (p.act_in) |a| a.ptr else null;
+    check(c.zg_hip_linear_bwd_input(self.ctx, p.gy.ptr, p.w.ptr, act, p.gx.ptr, p.batch, p.fan_in, p.fan_out, @intFromBool(p.accumulate)));
+}
+
 /// Adam update whose `lr_t` is read from memory when the kernel runs (`p.lr_t` points to device memory or
 /// to `mem_alloc_indices`-style pinned host memory).  A step recorded with `capture.open()` can then be
 /// replayed for every later step: the host only rewrites `lr_t` between replays.

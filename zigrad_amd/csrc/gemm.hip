@@ -175,7 +175,20 @@ struct GemmArgs {
     // C + y * split_stride (the launcher points C at a buffer of partial products); one split = the whole of k
     size_t split_tiles, split_stride;
     int a_vec, b_vec;  // 16-byte vector loads are legal for this operand
+    // Optional epilogue of the fused Linear entry points, applied to v = alpha * acc + beta * C in this order:
+    // v += bias[col]; v = max(v, 0) when relu; v = 0 where gate[row][col] <= 0 (gate laid out like C, only with
+    // beta == 0).  All null / 0 for the plain products.
+    const float* bias;
+    const float* gate;
+    int relu;
 };
+
+// the epilogue extras on one value (the rounding of the separate add / relu / mask kernels: one IEEE add, selects)
+__device__ __forceinline__ float gemm_extras(float v, bool has_bias, float bias, bool relu) {
+    if (has_bias) v = __fadd_rn(v, bias);
+    if (relu) v = v > 0.f ? v : 0.f;
+    return v;
+}
 
 // Logical tile id from the hardware workgroup id.  Hardware deals consecutive ids round-robin to the 8
 // XCDs; give each XCD a contiguous run of logical ids, then walk C in column groups of GM tile-rows.
@@ -380,6 +393,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // not read at all when beta == 0.
     const float alpha = g.alpha, beta = g.beta;
     const bool use_c = beta != 0.f;
+    const bool has_bias = g.bias != nullptr, relu = g.relu != 0, gated = g.gate != nullptr;  // gated implies !use_c
+    // the gate value of a C element sits at the same offset from g.gate as the element from g.C
+    const ptrdiff_t gate_bytes = gated ? reinterpret_cast<const char*>(g.gate) - reinterpret_cast<const char*>(g.C) : 0;
+
+    const bool use_old = use_c || gated;
     // The accumulators are taken out of their AGPRs one row of blocks at a time through an explicit
     // v_accvgpr_read (the "a" constraint pins the value in an AGPR up to that point).  Left to itself the
     // register allocator copies all of them to VGPRs at the loop exit, which doubles the kernel's register
@@ -392,9 +410,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     for (int i = 0; i < TM; i++) {
         float res[TN][16], old[TN][16];
         float* cptr[TN];
+        const float* optr[TN];  // where the old values come from: C itself, or the gate
+        float bias_v[TN];
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-            cptr[j] = C + (m0 + wm0 + FA::index_of(i, lk * 4)) * g.ldc + n0 + wn0 + FB::index_of(j, l32);
+        for (int j = 0; j < TN; j++) {
+            const size_t col = n0 + wn0 + FB::index_of(j, l32);
+            cptr[j] = C + (m0 + wm0 + FA::index_of(i, lk * 4)) * g.ldc + col;
+            optr[j] = reinterpret_cast<const float*>(reinterpret_cast<const char*>(cptr[j]) + gate_bytes);
+            bias_v[j] = (has_bias && (MODE == 0 || col < g.N)) ? g.bias[col] : 0.f;
+        }
         constexpr int RSTEP = A_KMAJOR ? 1 : TM;  // tile rows between consecutive block rows
         auto row_of = [&](int r) { return ((r >> 2) * 8 + (r & 3)) * RSTEP; };  // relative to block row lk*4
         auto in_range = [&](int j, int r) {
@@ -403,19 +427,20 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             const size_t col = n0 + wn0 + FB::index_of(j, l32);
             return row < g.M && col < g.N;
         };
-        if (use_c) {
+        if (use_old) {  // the old C values, or the gate values when gated
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 if (VEC_C) {
                     VC o = {};
-                    if (in_range(0, r)) o = *reinterpret_cast<const VC*>(cptr[0] + (size_t)row_of(r) * g.ldc);
+                    if (in_range(0, r)) o = *reinterpret_cast<const VC*>(optr[0] + (size_t)row_of(r) * g.ldc);
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
                         if constexpr (VEC_C) old[j][r] = o[j];
                     }
                 } else {
 #pragma unroll
-                    for (int j = 0; j < TN; j++) old[j][r] = in_range(j, r) ? cptr[j][(size_t)row_of(r) * g.ldc] : 0.f;
+                    for (int j = 0; j < TN; j++)
+                        old[j][r] = in_range(j, r) ? optr[j][(size_t)row_of(r) * g.ldc] : 0.f;
                 }
             }
         }
@@ -430,6 +455,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             for (int j = 0; j < TN; j++) {
                 v[j] = alpha * res[j][r];
                 if (use_c) v[j] += beta * old[j][r];
+                v[j] = gemm_extras(v[j], has_bias, bias_v[j], relu);
+                if (gated) v[j] = old[j][r] <= 0.f ? 0.f : v[j];
             }
             if (VEC_C) {
                 VC o;
@@ -555,6 +582,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
         if (row < g.M && col < g.N) {
             float v = alpha * s;
             if (beta != 0.f) v += beta * C[row * g.ldc + col];
+            v = gemm_extras(v, g.bias != nullptr, g.bias ? g.bias[col] : 0.f, g.relu != 0);
+            if (g.gate && g.gate[z * g.c_chunk + row * g.ldc + col] <= 0.f) v = 0.f;
             C[row * g.ldc + col] = v;
         }
     }
@@ -574,7 +603,8 @@ static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_
 
 // C = alpha * (sum of the split-K partial products, in split order) + beta * C.  P is [batch][split][M][N] dense.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, float* C, size_t M, size_t N, size_t ldc,
-                                                            int splits, float alpha, float beta, size_t c_chunk) {
+                                                            int splits, float alpha, float beta, size_t c_chunk,
+                                                            const float* bias, const float* gate, int relu) {
     const size_t z = blockIdx.z;
     const float* p = P + z * (size_t)splits * M * N;
     float* c = C + z * c_chunk;
@@ -585,6 +615,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, floa
         const size_t r = i / N, col = i % N;
         float v = alpha * acc;
         if (beta != 0.f) v += beta * c[r * ldc + col];
+        v = gemm_extras(v, bias != nullptr, bias ? bias[col] : 0.f, relu != 0);
+        if (gate && gate[z * c_chunk + r * ldc + col] <= 0.f) v = 0.f;
         c[r * ldc + col] = v;
     }
 }
@@ -599,10 +631,16 @@ __global__ void scale_c_kernel(float* C, size_t M, size_t N, size_t ldc, float b
     }
 }
 
+struct GemmExtras {
+    const float* bias;
+    const float* gate;
+    int relu;
+};
+
 static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
                          size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta,
                          size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk,
-                         int depth = 0) {
+                         int depth = 0, const GemmExtras* extras = nullptr) {
     if (m == 0 || n == 0 || batches == 0) return ZG_HIP_OK;
     ZG_REQUIRE(A && B && C, "%s: null pointer", name);
     // cblas argument rules for row-major storage
@@ -632,6 +670,9 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.ldc = ldc;
     g.alpha = alpha;
     g.beta = beta;
+    g.bias = extras ? extras->bias : nullptr;
+    g.gate = extras ? extras->gate : nullptr;
+    g.relu = extras ? extras->relu : 0;
     g.nba = nba;
     g.nbb = nbb;
     g.a_chunk = a_chunk;
@@ -673,8 +714,18 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         if (int rc = gemm_dispatch(ctx, name, A, B, C, m, n, k_main, trans_a, trans_b, lda, ldb, ldc, alpha, beta, batches,
                                    nba, nbb, a_chunk, b_chunk, c_chunk, 1))
             return rc;
-        return gemm_dispatch(ctx, name, a_tail, b_tail, C, m, n, k - k_main, trans_a, trans_b, lda, ldb, ldc, alpha, 1.f,
-                             batches, nba, nbb, a_chunk, b_chunk, c_chunk, 1);
+        // epilogue extras belong to the finished sum: bias and ReLU ride in the second pass; a gate cannot (it
+        // shares the epilogue's registers with the old C values) and runs as the separate op it replaces
+        const bool gate_after = extras && extras->gate;
+        const GemmExtras tail_extras = {extras ? extras->bias : nullptr, nullptr, extras ? extras->relu : 0};
+        if (int rc = gemm_dispatch(ctx, name, a_tail, b_tail, C, m, n, k - k_main, trans_a, trans_b, lda, ldb, ldc, alpha,
+                                   1.f, batches, nba, nbb, a_chunk, b_chunk, c_chunk, 1, extras ? &tail_extras : nullptr))
+            return rc;
+        if (gate_after) {
+            ZG_REQUIRE(ldc == n && batches == 1, "%s: a gated product needs a dense C", name);
+            return zg_hip_relu_inplace_bwd(ctx, extras->gate, C, m * n);
+        }
+        return ZG_HIP_OK;
     }
 
     if (k <= 256 && tiles(32, 32) <= n_cu) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
@@ -709,6 +760,9 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
             gs.split_stride = m * n;
             gs.alpha = 1.f;
             gs.beta = 0.f;
+            gs.bias = nullptr;  // the extras belong to the sum of the partial products: the reduce kernel applies them
+            gs.gate = nullptr;
+            gs.relu = 0;
             // the partial-product buffer is 256-byte aligned and dense: its own alignment rule is n % 4 == 0
             const int split_mode = (mode(64, 64) != 2 && n % 4 == 0 && (m * n) % 4 == 0) ? mode(64, 64) : 2;
             int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
@@ -716,7 +770,7 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
             size_t blocks = ceil_div_sz(m * n, 256);
             if (blocks > 2048) blocks = 2048;
             hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks, 1, (unsigned)batches), dim3(256), 0,
-                               ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk);
+                               ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk, g.bias, g.gate, g.relu);
             ZG_LAUNCH_CHECK();
             return ZG_HIP_OK;
         }
@@ -791,6 +845,38 @@ ZG_API int zg_hip_matmul(zg_hip_ctx* ctx, const float* A, const float* B, float*
                          int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
     ZG_CTX(ctx);
     return gemm_dispatch(ctx, "matmul", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, 1, 1, 1, 0, 0, 0);
+}
+
+// y = act(x . w^T + bias): one launch where the product is one launch (the bias add and the ReLU ride in the GEMM
+// epilogue or in the split-k reduction), with the arithmetic of the three separate ops.
+ZG_API int zg_hip_linear_fwd(zg_hip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, size_t batch,
+                             size_t fan_in, size_t fan_out, int relu) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(fan_in >= 1, "linear_fwd: fan_in is 0");
+    if (batch == 0 || fan_out == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(x && w && y, "linear_fwd: null pointer");
+    const GemmExtras ex = {bias, nullptr, relu};
+    return gemm_dispatch(ctx, "linear_fwd", x, w, y, batch, fan_out, fan_in, 0, 1, fan_in, fan_in, fan_out, 1.f, 0.f, 1, 1,
+                         1, 0, 0, 0, 0, &ex);
+}
+
+// gx = (accumulate ? gx : 0) + gy . w, then gx = 0 where act_in <= 0 (act_in: the ReLU output that fed this layer,
+// null for none): the input gradient of a Linear layer with the ReLU backward of the layer before it.
+ZG_API int zg_hip_linear_bwd_input(zg_hip_ctx* ctx, const float* gy, const float* w, const float* act_in, float* gx,
+                                   size_t batch, size_t fan_in, size_t fan_out, int accumulate) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(fan_out >= 1, "linear_bwd_input: fan_out is 0");
+    if (batch == 0 || fan_in == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(gy && w && gx, "linear_bwd_input: null pointer");
+    if (accumulate) {  // the mask shares the epilogue registers with the old values of gx: two launches here
+        if (int rc = gemm_dispatch(ctx, "linear_bwd_input", gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in,
+                                   1.f, 1.f, 1, 1, 1, 0, 0, 0))
+            return rc;
+        return act_in ? zg_hip_relu_inplace_bwd(ctx, act_in, gx, batch * fan_in) : ZG_HIP_OK;
+    }
+    const GemmExtras ex = {nullptr, act_in, 0};
+    return gemm_dispatch(ctx, "linear_bwd_input", gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in, 1.f, 0.f,
+                         1, 1, 1, 0, 0, 0, 0, act_in ? &ex : nullptr);
 }
 
 ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_shape, const float* B,

@@ -279,6 +279,16 @@ class HipDevice:
         self._call("zg_hip_bmm_acc", A.ptr, a, B.ptr, b, C.ptr, c, int(trans_a), int(trans_b), lda, ldb, ldc,
                    alpha, beta)
 
+    def _op_linear_fwd(self, x, w, bias, y, batch, fan_in, fan_out, relu):
+        """y = act(x . w^T + bias) in one launch; bias may be None."""
+        self._call("zg_hip_linear_fwd", x.ptr, w.ptr, bias.ptr if bias is not None else None, y.ptr, batch, fan_in,
+                   fan_out, int(relu))
+
+    def _op_linear_bwd_input(self, gy, w, act_in, gx, batch, fan_in, fan_out, accumulate):
+        """gx = (gx if accumulate else 0) + gy . w, zeroed where act_in <= 0 (act_in None: no mask)."""
+        self._call("zg_hip_linear_bwd_input", gy.ptr, w.ptr, act_in.ptr if act_in is not None else None, gx.ptr, batch,
+                   fan_in, fan_out, int(accumulate))
+
     def _op_outer(self, x, y, A, alpha):
         self._call("zg_hip_outer", x.ptr, x.n, y.ptr, y.n, A.ptr, alpha)
 

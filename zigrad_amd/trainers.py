@@ -212,8 +212,8 @@ class MLP:
     """Parameters, gradients and the forward/backward op sequences of a ReLU multi-layer perceptron whose
     Linear layers follow examples/mnist/src/model.zig:64-110 (weights [out, in], forward x . W^T + bias)."""
 
-    def __init__(self, dev, dims, optim: Optimizer | None = None):
-        self.dev, self.dims = dev, list(dims)
+    def __init__(self, dev, dims, optim: Optimizer | None = None, fused: bool = False):
+        self.dev, self.dims, self.fused = dev, list(dims), fused
         self.n_layers = len(dims) - 1
         self.W, self.b, self.Wg, self.bg = [], [], [], []
         for fan_in, fan_out in zip(dims[:-1], dims[1:]):
@@ -256,6 +256,11 @@ class MLP:
         for l in range(self.n_layers):
             fan_in, fan_out = self.dims[l], self.dims[l + 1]
             y = d.mem_cache_alloc(F32, batch * fan_out)
+            if self.fused:  # the same three ops in one launch
+                d.dispatch("linear_fwd", x=acts[-1], w=self.W[l], bias=self.b[l], y=y, batch=batch, fan_in=fan_in,
+                           fan_out=fan_out, relu=l + 1 < self.n_layers)
+                acts.append(y)
+                continue
             host.bmm_acc_(d, acts[-1], [batch, fan_in], self.W[l], [fan_out, fan_in], y, trans_a=False, trans_b=True)
             d.dispatch("add", x=self.b[l], y=y, z=y)  # bias.add_(y): shorter operand first
             if l + 1 < self.n_layers:
@@ -274,6 +279,21 @@ class MLP:
         for l in reversed(range(self.n_layers)):
             fan_in, fan_out = self.dims[l], self.dims[l + 1]
             y = acts[l + 1]
+            if self.fused:
+                # g arrives with this layer's ReLU backward applied (by the product that made it); the input
+                # gradient is written, not accumulated, so it needs no zero fill
+                host.unbroadcast_(d, g, [batch, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
+                g_prev = None
+                if l > 0:
+                    g_prev = d.mem_cache_alloc(F32, batch * fan_in)
+                    d.dispatch("linear_bwd_input", gy=g, w=self.W[l], act_in=acts[l], gx=g_prev, batch=batch,
+                               fan_in=fan_in, fan_out=fan_out, accumulate=False)
+                host.bmm_acc_backward(d, False, True, acts[l], [batch, fan_in], self.W[l], [fan_out, fan_in], g,
+                                      [batch, fan_out], None, self.Wg[l])
+                d.mem_cache_free(y)
+                d.mem_cache_free(g)
+                g = g_prev
+                continue
             if l + 1 < self.n_layers:
                 d.dispatch("relu_inplace_bwd", x=y, x_g=g)
             host.unbroadcast_(d, g, [batch, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
@@ -292,13 +312,15 @@ class MLPTrainer(GraphSteps):
     """Linear -> ReLU -> ... -> Linear -> softmax cross-entropy, one train step per `step()` call.
 
     loss_mode "onehot" is the reference's loss (float one-hot targets, probabilities kept for backward);
-    "label" is the fused integer-label form (same values, one pass over the logits).
+    "label" is the fused integer-label form (same values, one pass over the logits).  fused=True issues every
+    Linear layer through the fused entry points (bias and ReLU in the GEMM epilogue, ReLU backward in the epilogue
+    of the input-gradient product): same arithmetic, fewer launches and passes over the activations.
     """
 
-    def __init__(self, dev, dims, batch, optimizer="sgd", lr=0.01, clip=True, loss_mode="onehot"):
+    def __init__(self, dev, dims, batch, optimizer="sgd", lr=0.01, clip=True, loss_mode="onehot", fused=False):
         self.dev, self.dims, self.batch, self.loss_mode = dev, list(dims), batch, loss_mode
         self.optim = Optimizer(dev, optimizer, lr, clip)
-        self.net = MLP(dev, dims, self.optim)
+        self.net = MLP(dev, dims, self.optim, fused=fused)
         self.n_layers = self.net.n_layers
         self.x = dev.mem_alloc(F32, batch * dims[0])
         self.onehot = dev.mem_alloc(F32, batch * dims[-1])

@@ -305,18 +305,18 @@ def run_input_pipeline(dev, dims, batch, steps, warmup):
     return out
 
 
-def run_small(dev, kind, steps, graph=True):
+def run_small(dev, kind, steps, graph=True, fused=False):
     """Step time of the GCN (2708 nodes, 1433 features, 13264 edges, 140 labelled, Adam) or DQN (4-128-128-2, batch
     64, Adam) train step; the loss is read back every step, as the reference's loops do."""
     from zigrad_amd.trainers import DQNTrainer, GCNTrainer, dqn_inputs, gcn_inputs, mlp_inputs
 
     if kind == "gcn":
-        tr = GCNTrainer(dev, gcn_inputs(seed=0), lr=0.01, clip=True)
+        tr = GCNTrainer(dev, gcn_inputs(seed=0), lr=0.01, clip=True, fused=fused)
         what = "2-layer GCN 1433-16-7, 2708 nodes, 13264 edges, 140 labelled nodes, Adam lr 0.01"
     else:
         dims, batch = [4, 128, 128, 2], 64
         params, _, _, _ = mlp_inputs(dims, batch)
-        tr = DQNTrainer(dev, dims, batch, lr=1e-3, gamma=0.99, clip=True)
+        tr = DQNTrainer(dev, dims, batch, lr=1e-3, gamma=0.99, clip=True, fused=fused)
         tr.load_params(params)
         tr.set_batch(dqn_inputs(batch=batch))
         what = "DQN update 4-128-128-2, batch 64, frozen target net, gather, smooth-L1, Adam lr 1e-3"
@@ -414,12 +414,12 @@ def main():
     # `value` reads the loss where the reference's loop does (before backward: the host blocks and the GPU idles until
     # the backward launches arrive); the same step with that one read moved behind the optimizer step:
     result["late_loss_read"] = {"steps_per_s": args.steps / dt_late, "ms_per_step": dt_late / args.steps * 1e3}
-    # every Linear layer through the fused entry points (bias + ReLU in the GEMM epilogue, ReLU backward in the epilogue
-    # of the input-gradient product; same arithmetic, bit-identical parameters): not the reference's op sequence, so
-    # reported beside `value`, never as it
+    # the fused entry points: every Linear layer with bias + ReLU in the GEMM epilogue and ReLU backward in the epilogue
+    # of the input-gradient product, optimizer step + zero_grad over the whole parameter list (same arithmetic,
+    # bit-identical parameters): not the reference's op sequence, so reported beside `value`, never as it
     f = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", None, args.loss_mode, late_read=True,
                 fused=True)
-    result["fused_linear"] = {"steps_per_s": args.steps / f[0], "ms_per_step": f[0] / args.steps * 1e3,
+    result["fused"] = {"steps_per_s": args.steps / f[0], "ms_per_step": f[0] / args.steps * 1e3,
                               "late_loss_read": {"steps_per_s": args.steps / f[2], "ms_per_step": f[2] / args.steps * 1e3}}
     # the latency-bound configurations: batch-64 MLP (configs[0]), GCN (configs[2]), DQN update (configs[3])
     if not args.no_small:
@@ -431,11 +431,15 @@ def main():
             result["mlp_b64"]["graph_replay"] = {"steps_per_s": 200 / small[2], "ms_per_step": small[2] / 200 * 1e3}
         if not args.no_graph:
             fs = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=True, fused=True)
-            result["mlp_b64"]["fused_linear"] = {"steps_per_s": 200 / fs[0], "ms_per_step": fs[0] / 200 * 1e3,
+            result["mlp_b64"]["fused"] = {"steps_per_s": 200 / fs[0], "ms_per_step": fs[0] / 200 * 1e3,
                                                  "graph_replay": {"steps_per_s": 200 / fs[2], "ms_per_step": fs[2] / 200 * 1e3}}
         result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
         result["gcn"] = run_small(dev, "gcn", 100, graph=not args.no_graph)
         result["dqn"] = run_small(dev, "dqn", 200, graph=not args.no_graph)
+        if not args.no_graph:
+            for kind, n in (("gcn", 100), ("dqn", 200)):
+                f = run_small(dev, kind, n, graph=True, fused=True)
+                result[kind]["fused"] = {k: f[k] for k in ("steps_per_s", "ms_per_step", "graph_replay")}
     if not args.no_ops:
         result["ops"] = op_suite(dev)
     if not args.no_cpu:

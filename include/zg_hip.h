@@ -263,6 +263,21 @@ int zg_hip_adam_lr_t(float lr, float beta1, float beta2, uint64_t t, float *lr_t
 int zg_hip_adam_step_at(zg_hip_ctx *ctx, float *param, float *grad, float *m, float *v, size_t n, const float *lr_t,
                         float beta1, float beta2, float epsilon, int clip, float max_norm, float delta);
 
+/* The optimizer step over a whole parameter list, as Optimizer.step() walks it (src/nn/optim.zig:100-122, :177-234):
+ * tensors of up to 65536 elements share launches (one workgroup per tensor, 16 tensors per launch), larger ones
+ * take the per-tensor kernels; values are those of the per-tensor calls.  The lists are host arrays of n_tensors
+ * entries.  zero_grads != 0 also leaves every gradient zero: optim.step() followed by model.zero_grad()
+ * (examples/mnist/src/main-simple.zig:70-71, examples/mnist/src/model.zig:57-62) without the fills.
+ * Adam: lr_t[i] is tensor i's step size (zg_hip_adam_lr_t with that tensor's counter value); with
+ * lr_t_in_memory != 0 it is an array in device or zg_hip_host_alloc memory that the kernels read when they run
+ * (see zg_hip_adam_step_at), otherwise a host array read during the call. */
+int zg_hip_sgd_step_multi(zg_hip_ctx *ctx, size_t n_tensors, float *const *params, float *const *grads,
+                          const size_t *lens, float lr, int clip, float max_norm, float delta, int zero_grads);
+int zg_hip_adam_step_multi(zg_hip_ctx *ctx, size_t n_tensors, float *const *params, float *const *grads,
+                           float *const *ms, float *const *vs, const size_t *lens, const float *lr_t,
+                           int lr_t_in_memory, float beta1, float beta2, float epsilon, int clip, float max_norm,
+                           float delta, int zero_grads);
+
 /* ---------------------------------------------------------------------------------------------
  * input staging: the step before the hot path.  The reference uploads every batch with a blocking
  * mem_transfer(.HtoD) (src/device/device_reference.zig:101-105, as used by NDTensor.from_slice in

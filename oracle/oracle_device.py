@@ -177,6 +177,22 @@ class OracleDevice(HipDevice):
         raise NotImplementedError("the oracle is timed with time.perf_counter")
 
     # -- entry points whose oracle signature differs from the C ABI ----------------------------------
+    # -- the list entry points are the per-tensor ops in a loop --------------------------------------------
+    def _op_sgd_step_multi(self, params, grads, lr, clip, max_norm, delta, zero_grads):
+        for p, g in zip(params, grads):
+            self.dispatch("sgd_step", param=p, grad=g, lr=lr, clip=clip, max_norm=max_norm, delta=delta)
+            if zero_grads:
+                self.mem_fill(g, 0.0)
+
+    def _op_adam_step_multi(self, params, grads, ms, vs, lr, t_first, beta1, beta2, epsilon, clip, max_norm, delta,
+                            zero_grads, lr_t_mem=None):
+        assert lr_t_mem is None, "the oracle has no recorded steps"
+        for i, (p, g, m, v) in enumerate(zip(params, grads, ms, vs)):
+            self.dispatch("adam_step", param=p, grad=g, m=m, v=v, t=t_first + i, lr=lr, beta1=beta1, beta2=beta2,
+                          epsilon=epsilon, clip=clip, max_norm=max_norm, delta=delta)
+            if zero_grads:
+                self.mem_fill(g, 0.0)
+
     def _x_zg_hip_linear_fwd(self, x, w, bias, y, batch, fan_in, fan_out, relu):
         # the three ops the fused entry point stands for (examples/mnist/src/model.zig:104-110, :38-46)
         c = self._o.cdll

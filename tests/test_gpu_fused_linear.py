@@ -104,3 +104,85 @@ def test_fused_step_replays_from_an_execution_graph(hip):
     for a, b in zip(eager.param_buffers(), graph.param_buffers()):
         assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b))
     graph.free_graph()
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adam"])
+@pytest.mark.parametrize("clip,zero", [(True, True), (True, False), (False, True)])
+def test_optimizer_list_entry_points_equal_the_per_tensor_ops(hip, kind, clip, zero):
+    """Sizes either side of the one-workgroup limit (65536), a list longer than one launch holds (16), gradients
+    large enough that the clip is active for some tensors and not for others."""
+    from zigrad_amd.device import F32
+
+    r = np.random.default_rng(7)
+    sizes = [1, 10, 128, 640, 8192, 65536, 65537, 100352, 3, 64] + [int(r.integers(1, 5000)) for _ in range(14)]
+    host = [(r.standard_normal(n).astype(np.float32), (r.standard_normal(n) * r.choice([0.01, 3.0])).astype(np.float32),
+             (r.standard_normal(n) * 0.1).astype(np.float32), (r.random(n) * 0.1).astype(np.float32)) for n in sizes]
+    beta1, beta2, eps, lr = 0.9, 0.999, 1e-8, 0.01
+    out = []
+    for multi in (False, True):
+        bufs = [[hip.from_numpy(a) for a in t] for t in host]
+        if multi and kind == "sgd":
+            hip.dispatch("sgd_step_multi", params=[b[0] for b in bufs], grads=[b[1] for b in bufs], lr=lr, clip=clip,
+                         max_norm=10.0, delta=1e-6, zero_grads=zero)
+        elif multi:
+            hip.dispatch("adam_step_multi", params=[b[0] for b in bufs], grads=[b[1] for b in bufs], ms=[b[2] for b in bufs],
+                         vs=[b[3] for b in bufs], lr=lr, t_first=5, beta1=beta1, beta2=beta2, epsilon=eps, clip=clip,
+                         max_norm=10.0, delta=1e-6, zero_grads=zero)
+        else:
+            for i, (p, g, m, v) in enumerate(bufs):
+                if kind == "sgd":
+                    hip.dispatch("sgd_step", param=p, grad=g, lr=lr, clip=clip, max_norm=10.0, delta=1e-6)
+                else:
+                    hip.dispatch("adam_step", param=p, grad=g, m=m, v=v, t=5 + i, lr=lr, beta1=beta1, beta2=beta2,
+                                 epsilon=eps, clip=clip, max_norm=10.0, delta=1e-6)
+                if zero:
+                    hip.mem_fill(g, 0.0)
+        out.append([[hip.to_numpy(b) for b in t] for t in bufs])
+        for t in bufs:
+            for b in t:
+                hip.mem_free(b)
+    for i, (a, b) in enumerate(zip(*out)):
+        for which, (x, y) in enumerate(zip(a, b)):
+            if kind == "sgd" and which >= 2:
+                continue
+            assert np.array_equal(x, y), (sizes[i], which)
+
+
+def test_dqn_and_gcn_steps_with_and_without_fusion_agree_exactly(hip):
+    from zigrad_amd.trainers import DQNTrainer, GCNTrainer, dqn_inputs, gcn_inputs
+
+    dims, batch = [4, 128, 128, 2], 64
+    params, _, _, _ = mlp_inputs(dims, batch)
+    inp = gcn_inputs(n_nodes=500, n_features=200, n_pairs=1500, n_train=40, hidden=16, seed=2)
+    for make in (lambda f: DQNTrainer(hip, dims, batch, fused=f), lambda f: GCNTrainer(hip, inp, fused=f)):
+        out = []
+        for fused in (False, True):
+            tr = make(fused)
+            if isinstance(tr, DQNTrainer):
+                tr.load_params(params)
+                tr.set_batch(dqn_inputs(batch=batch))
+            losses = [tr.step() for _ in range(4)]
+            out.append((losses, [hip.to_numpy(b) for b in tr.param_buffers()]))
+        assert out[0][0] == out[1][0]
+        for a, b in zip(out[0][1], out[1][1]):
+            assert np.array_equal(a, b)
+
+
+def test_fused_adam_step_replays_from_an_execution_graph(hip):
+    from zigrad_amd.trainers import DQNTrainer, dqn_inputs
+
+    dims, batch = [4, 128, 128, 2], 64
+    params, _, _, _ = mlp_inputs(dims, batch)
+    eager, graph = DQNTrainer(hip, dims, batch, fused=True), DQNTrainer(hip, dims, batch, fused=True)
+    for tr in (eager, graph):
+        tr.load_params(params)
+        tr.set_batch(dqn_inputs(batch=batch))
+    graph.step()
+    eager.step()
+    graph.capture()
+    for _ in range(5):
+        assert eager.step() == graph.step_graph()
+        hip.sync()
+    for a, b in zip(eager.param_buffers(), graph.param_buffers()):
+        assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b))
+    graph.free_graph()

@@ -459,6 +459,19 @@ pub fn adam_step(self: *const Self, T: type, p: anytype) void {
     check(c.zg_hip_adam_step(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.t, p.lr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
 }
 
+/// Optimizer.step() over a whole parameter list (src/nn/optim.zig:100-122, :177-234), optionally followed by
+/// model.zero_grad(): small tensors share launches.  `p.params`, `p.grads` (and `p.ms`, `p.vs`) are slices of
+/// device pointers, `p.lens` their element counts; Adam's `p.lr_t` holds one step size per tensor
+/// (`adam_lr_t` with that tensor's counter), in host memory unless `p.lr_t_in_memory`.
+pub fn sgd_step_multi(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_sgd_step_multi(self.ctx, p.params.len, p.params.ptr, p.grads.ptr, p.lens.ptr, p.lr, @intFromBool(p.clip), p.max_norm, p.delta, @intFromBool(p.zero_grads)));
+}
+pub fn adam_step_multi(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_adam_step_multi(self.ctx, p.params.len, p.params.ptr, p.grads.ptr, p.ms.ptr, p.vs.ptr, p.lens.ptr, p.lr_t.ptr, @intFromBool(p.lr_t_in_memory), p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta, @intFromBool(p.zero_grads)));
+}
+
 /// A Linear layer's forward in one launch: y = act(x . w^T + bias), the arithmetic of `bmm_acc(trans_b)` +
 /// `bias.add_` + `relu_` (examples/mnist/src/model.zig:104-110, :38-46).  `p.bias` is an optional slice.
 pub fn linear_fwd(self: *const Self, T: type, p: anytype) void {

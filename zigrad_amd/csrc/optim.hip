@@ -135,6 +135,60 @@ __global__ __launch_bounds__(kFlatSingle) void clipped_update_small_kernel(float
     }
 }
 
+// The same update for up to kMultiMax small tensors in one launch: workgroup b does what
+// clipped_update_small_kernel does for tensor b (same accumulation tree for the norm, same arithmetic per element),
+// reads its lr_t from memory when asked to, and with `zero_grads` leaves the gradient zero instead of clipped
+// (optim.step() followed by model.zero_grad(), examples/mnist/src/main-simple.zig:70-71).
+constexpr int kMultiMax = 16;
+struct MultiArgs {
+    float* p[kMultiMax];
+    float* g[kMultiMax];
+    float* m[kMultiMax];
+    float* v[kMultiMax];
+    size_t n[kMultiMax];
+    float lr_t[kMultiMax];       // Adam: lr_t per tensor; SGD: -lr
+    const float* lr_t_mem;       // Adam under replay: lr_t_mem[b] is read when the kernel runs (null: use lr_t[b])
+    float b1, b2, omb1, omb2, eps, max_norm, delta;
+    int clip, zero_grads;
+};
+
+template <bool ADAM>
+__global__ __launch_bounds__(kFlatSingle) void update_multi_kernel(MultiArgs a) {
+    __shared__ float smem[kFlatSingle / kWave];
+    __shared__ float factor_s;
+    const int b = blockIdx.x;
+    float* const p = a.p[b];
+    float* const g = a.g[b];
+    float* const m = a.m[b];
+    float* const v = a.v[b];
+    const size_t n = a.n[b];
+    float f = 1.0f;
+    if (a.clip) {
+        float acc = flat_accumulate<TermSq, 1>(g, nullptr, n, 0.f, threadIdx.x, blockDim.x);
+        acc = block_reduce<SumAcc>(acc, smem);
+        if (threadIdx.x == 0) FinClipFactor{&factor_s, a.max_norm, a.delta}(acc);
+        __syncthreads();
+        f = factor_s;
+    }
+    const bool scale = f != 1.0f;
+    const float lr_t = (ADAM && a.lr_t_mem) ? a.lr_t_mem[b] : a.lr_t[b];
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float gv = g[i];
+        if (ADAM) {
+            float pv = p[i], mv = m[i], vv = v[i];
+            adam_elem(pv, gv, mv, vv, scale, f, lr_t, a.b1, a.b2, a.omb1, a.omb2, a.eps);
+            m[i] = mv;
+            v[i] = vv;
+            p[i] = pv;
+        } else {
+            if (scale) gv = __fmul_rn(gv, f);
+            p[i] = __fadd_rn(p[i], __fmul_rn(lr_t, gv));
+        }
+        if (a.zero_grads) g[i] = 0.f;
+        else if (scale) g[i] = gv;
+    }
+}
+
 static int update_grid(zg_hip_ctx* ctx, size_t n) {
     size_t blocks = ceil_div_sz(n, (size_t)kBlock * 4);
     size_t cap = (size_t)ctx->n_cu * 16;
@@ -219,4 +273,81 @@ ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad && m && v && lr_t, "adam_step_at: null pointer");
     return adam_launch(ctx, param, grad, m, v, n, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);
+}
+
+// Parameter lists: tensors of up to kFlatSingleMax elements share launches, larger ones take the per-tensor path.
+static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_tensors, float* const* params,
+                      float* const* grads, float* const* ms, float* const* vs, const size_t* lens, const float* lr_t,
+                      int lr_t_in_memory, float lr, float beta1, float beta2, float epsilon, int clip, float max_norm,
+                      float delta, int zero_grads) {
+    ZG_REQUIRE(n_tensors == 0 || (params && grads && lens), "%s: null list", name);
+    ZG_REQUIRE(!adam || n_tensors == 0 || (ms && vs && lr_t), "%s: null list", name);
+    MultiArgs a;
+    int filled = 0;
+    size_t first = 0;  // list index of the batch's first tensor (lr_t_mem is indexed by workgroup)
+    auto flush = [&]() -> int {
+        if (!filled) return ZG_HIP_OK;
+        a.lr_t_mem = (adam && lr_t_in_memory) ? lr_t + first : nullptr;
+        if (adam) hipLaunchKernelGGL((update_multi_kernel<true>), dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((update_multi_kernel<false>), dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
+        filled = 0;
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    };
+    a.b1 = beta1;
+    a.b2 = beta2;
+    a.omb1 = 1.0f - beta1;
+    a.omb2 = 1.0f - beta2;
+    a.eps = epsilon;
+    a.max_norm = max_norm;
+    a.delta = delta;
+    a.clip = clip;
+    a.zero_grads = zero_grads;
+    for (size_t i = 0; i < n_tensors; i++) {
+        const size_t n = lens[i];
+        if (n == 0) {  // keeps lr_t_mem's indexing dense: an empty tensor ends the batch
+            if (int rc = flush()) return rc;
+            continue;
+        }
+        ZG_REQUIRE(params[i] && grads[i] && (!adam || (ms[i] && vs[i])), "%s: null pointer in tensor %zu", name, i);
+        if (n <= kFlatSingleMax) {
+            if (filled == 0) first = i;
+            a.p[filled] = params[i];
+            a.g[filled] = grads[i];
+            a.m[filled] = adam ? ms[i] : nullptr;
+            a.v[filled] = adam ? vs[i] : nullptr;
+            a.n[filled] = n;
+            a.lr_t[filled] = adam ? (lr_t_in_memory ? 0.f : lr_t[i]) : -lr;
+            if (++filled == kMultiMax)
+                if (int rc = flush()) return rc;
+            continue;
+        }
+        if (int rc = flush()) return rc;
+        int rc;
+        if (adam)
+            rc = adam_launch(ctx, params[i], grads[i], ms[i], vs[i], n, lr_t_in_memory ? 0.f : lr_t[i],
+                             lr_t_in_memory ? lr_t + i : nullptr, beta1, beta2, epsilon, clip, max_norm, delta);
+        else
+            rc = zg_hip_sgd_step(ctx, params[i], grads[i], n, lr, clip, max_norm, delta);
+        if (rc) return rc;
+        if (zero_grads)
+            if ((rc = zg_hip_mem_fill(ctx, grads[i], n, 0.f))) return rc;
+    }
+    return flush();
+}
+
+ZG_API int zg_hip_sgd_step_multi(zg_hip_ctx* ctx, size_t n_tensors, float* const* params, float* const* grads,
+                                 const size_t* lens, float lr, int clip, float max_norm, float delta, int zero_grads) {
+    ZG_CTX(ctx);
+    return step_multi(ctx, "sgd_step_multi", false, n_tensors, params, grads, nullptr, nullptr, lens, nullptr, 0, lr, 0.f,
+                      0.f, 0.f, clip, max_norm, delta, zero_grads);
+}
+
+ZG_API int zg_hip_adam_step_multi(zg_hip_ctx* ctx, size_t n_tensors, float* const* params, float* const* grads,
+                                  float* const* ms, float* const* vs, const size_t* lens, const float* lr_t,
+                                  int lr_t_in_memory, float beta1, float beta2, float epsilon, int clip, float max_norm,
+                                  float delta, int zero_grads) {
+    ZG_CTX(ctx);
+    return step_multi(ctx, "adam_step_multi", true, n_tensors, params, grads, ms, vs, lens, lr_t, lr_t_in_memory, 0.f,
+                      beta1, beta2, epsilon, clip, max_norm, delta, zero_grads);
 }

@@ -432,6 +432,31 @@ class HipDevice:
         self._call("zg_hip_adam_step_at", param.ptr, grad.ptr, m.ptr, v.ptr, param.n, lr_t.ptr, beta1, beta2, epsilon,
                    int(clip), max_norm, delta)
 
+    @staticmethod
+    def _ptr_list(bufs):
+        return (ctypes.c_void_p * len(bufs))(*[b.ptr for b in bufs])
+
+    def _op_sgd_step_multi(self, params, grads, lr, clip, max_norm, delta, zero_grads):
+        """SGD over a parameter list in as few launches as possible; optionally leaves the gradients zero."""
+        lens = (ctypes.c_size_t * len(params))(*[p.n for p in params])
+        self._call("zg_hip_sgd_step_multi", len(params), self._ptr_list(params), self._ptr_list(grads), lens, lr, int(clip),
+                   max_norm, delta, int(zero_grads))
+
+    def _op_adam_step_multi(self, params, grads, ms, vs, lr, t_first, beta1, beta2, epsilon, clip, max_norm, delta,
+                            zero_grads, lr_t_mem=None):
+        """Adam over a parameter list.  Tensor i is updated with counter value t_first + i (the reference counts
+        once per tensor, src/nn/optim.zig:189); with lr_t_mem (a DevBuf of one float per tensor in device or pinned
+        memory) the kernels read each lr_t from there when they run instead."""
+        lens = (ctypes.c_size_t * len(params))(*[p.n for p in params])
+        if lr_t_mem is not None:
+            lr_arg, in_memory = lr_t_mem.ptr, 1
+        else:
+            lr_arg = (ctypes.c_float * len(params))(*[self.adam_lr_t(lr, beta1, beta2, t_first + i) for i in range(len(params))])
+            in_memory = 0
+        self._call("zg_hip_adam_step_multi", len(params), self._ptr_list(params), self._ptr_list(grads), self._ptr_list(ms),
+                   self._ptr_list(vs), lens, lr_arg, in_memory, beta1, beta2, epsilon, int(clip), max_norm, delta,
+                   int(zero_grads))
+
     def adam_lr_t(self, lr, beta1, beta2, t) -> float:
         out = ctypes.c_float()
         self._lib.call("zg_hip_adam_lr_t", lr, beta1, beta2, int(t), ctypes.byref(out))

@@ -53,10 +53,12 @@ class Optimizer:
     """SGD / Adam over a list of attached parameter tensors, one fused device op per tensor."""
 
     def __init__(self, dev, kind: str, lr: float, clip: bool = True, max_norm: float = GRAD_CLIP_MAX_NORM,
-                 delta: float = GRAD_CLIP_DELTA, beta1: float = 0.9, beta2: float = 0.999, epsilon: float = 1e-8):
+                 delta: float = GRAD_CLIP_DELTA, beta1: float = 0.9, beta2: float = 0.999, epsilon: float = 1e-8,
+                 fused: bool = False):
         if kind not in ("sgd", "adam"):
             raise ValueError(f"unknown optimizer {kind!r}")
         self.dev, self.kind, self.lr, self.clip = dev, kind, lr, clip
+        self.fused = fused  # step_and_zero_grad() through the list entry points: same values, fewer launches
         self.max_norm, self.delta = max_norm, delta
         self.beta1, self.beta2, self.epsilon = beta1, beta2, epsilon
         self.params: list[tuple[DevBuf, DevBuf]] = []
@@ -99,6 +101,24 @@ class Optimizer:
         for i in range(len(self.params)):
             self.t += 1
             self._lr_view[i] = self.dev.adam_lr_t(self.lr, self.beta1, self.beta2, self.t)
+
+    def step_and_zero_grad(self) -> bool:
+        """optim.step() + model.zero_grad() through the list entry points; False when this optimizer is not fused
+        (the caller then issues the two separately)."""
+        if not self.fused:
+            return False
+        d = self.dev
+        params, grads = [p for p, _ in self.params], [g for _, g in self.params]
+        common = dict(clip=self.clip, max_norm=self.max_norm, delta=self.delta, zero_grads=True)
+        if self.kind == "sgd":
+            d.dispatch("sgd_step_multi", params=params, grads=grads, lr=self.lr, **common)
+            return True
+        d.dispatch("adam_step_multi", params=params, grads=grads, ms=[m for m, _ in self.state],
+                   vs=[v for _, v in self.state], lr=self.lr, t_first=self.t + 1, beta1=self.beta1, beta2=self.beta2,
+                   epsilon=self.epsilon, lr_t_mem=self.lr_slots if self.capturing else None, **common)
+        if not self.capturing:
+            self.t += len(params)  # once per tensor (src/nn/optim.zig:189)
+        return True
 
     def step(self) -> None:
         d = self.dev
@@ -319,7 +339,7 @@ class MLPTrainer(GraphSteps):
 
     def __init__(self, dev, dims, batch, optimizer="sgd", lr=0.01, clip=True, loss_mode="onehot", fused=False):
         self.dev, self.dims, self.batch, self.loss_mode = dev, list(dims), batch, loss_mode
-        self.optim = Optimizer(dev, optimizer, lr, clip)
+        self.optim = Optimizer(dev, optimizer, lr, clip, fused=fused)
         self.net = MLP(dev, dims, self.optim, fused=fused)
         self.n_layers = self.net.n_layers
         self.x = dev.mem_alloc(F32, batch * dims[0])
@@ -404,8 +424,9 @@ class MLPTrainer(GraphSteps):
         self.net.backward(acts, g, B)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
-        self.optim.step()
-        self.net.zero_grad()  # model.zero_grad()
+        if not self.optim.step_and_zero_grad():
+            self.optim.step()
+            self.net.zero_grad()  # model.zero_grad()
         if read_loss == "late":
             loss_val = self._read_loss(loss)
         d.mem_cache_free(loss)
@@ -429,11 +450,11 @@ class DQNTrainer(GraphSteps):
     smooth-L1 loss, Adam.  Op order follows DQNAgent.train (examples/dqn/src/dqn_agent.zig:125-228) without
     its host-side clamps, on the network 4 -> 128 -> 128 -> 2."""
 
-    def __init__(self, dev, dims=(4, 128, 128, 2), batch=64, lr=1e-3, gamma=0.99, clip=True):
+    def __init__(self, dev, dims=(4, 128, 128, 2), batch=64, lr=1e-3, gamma=0.99, clip=True, fused=False):
         self.dev, self.dims, self.batch, self.gamma = dev, list(dims), batch, gamma
-        self.optim = Optimizer(dev, "adam", lr, clip)
-        self.policy = MLP(dev, dims, self.optim)
-        self.target = MLP(dev, dims, None)
+        self.optim = Optimizer(dev, "adam", lr, clip, fused=fused)
+        self.policy = MLP(dev, dims, self.optim, fused=fused)
+        self.target = MLP(dev, dims, None, fused=fused)
         B, S, A = batch, dims[0], dims[-1]
         self.states, self.next_states = dev.mem_alloc(F32, B * S), dev.mem_alloc(F32, B * S)
         self.actions = dev.mem_alloc(U64, B)
@@ -482,7 +503,8 @@ class DQNTrainer(GraphSteps):
         q, offsets = host.gather(d, q_all, [B, A], self.actions, [B, 1], 1, return_offsets=True, check=False)
         loss = d.mem_cache_alloc(F32, 1)
         d.dispatch("smooth_l1_fwd", pred=q, target=targets, beta=1.0, loss=loss)
-        self.policy.zero_grad()
+        if not self.optim.fused:  # the fused optimizer step leaves the gradients zero for the next step
+            self.policy.zero_grad()
         # backward
         loss_grad = d.mem_cache_alloc(F32, 1)
         d.mem_fill(loss_grad, 1.0)
@@ -498,7 +520,8 @@ class DQNTrainer(GraphSteps):
         self.policy.backward(acts, g_all, B)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.policy.grad_buffers()]
-        self.optim.step()
+        if not self.optim.step_and_zero_grad():
+            self.optim.step()
         loss_val = self._read_loss(loss)
         d.mem_cache_free(loss)
         return loss_val
@@ -532,13 +555,13 @@ class GCNTrainer(GraphSteps):
 
     EPS = 1e-12  # Settings.eps, src/zigrad.zig:72
 
-    def __init__(self, dev, inp, lr=0.01, clip=True):
+    def __init__(self, dev, inp, lr=0.01, clip=True, fused=False):
         d = self.dev = dev
         self.N = inp["x"].shape[0]
         self.dims = inp["dims"]
         self.E = inp["src"].size
         self.n_train = inp["n_train"]
-        self.optim = Optimizer(dev, "adam", lr, clip)
+        self.optim = Optimizer(dev, "adam", lr, clip, fused=fused)
         self.W, self.b, self.Wg, self.bg = [], [], [], []
         for fan_in, fan_out in zip(self.dims[:-1], self.dims[1:]):
             w, wg = d.mem_alloc(F32, fan_in * fan_out), d.mem_alloc(F32, fan_in * fan_out)
@@ -641,7 +664,8 @@ class GCNTrainer(GraphSteps):
         self._conv_backward(0, s1, g1, need_input_grad=False)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
-        self.optim.step()
-        for gb in self.grad_buffers():
-            d.mem_fill(gb, 0.0)
+        if not self.optim.step_and_zero_grad():
+            self.optim.step()
+            for gb in self.grad_buffers():
+                d.mem_fill(gb, 0.0)
         return loss_val

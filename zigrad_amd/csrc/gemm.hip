@@ -550,22 +550,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
     floatx16 acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    size_t grp = wave;
-    floatx4 a_cur = {0.f, 0.f, 0.f, 0.f}, b_cur = a_cur;
-    if (grp < groups) {
-        a_cur = frag_a(grp);
-        b_cur = frag_b(grp);
-    }
-    for (; grp < groups; grp += 4) {
-        floatx4 a_nxt = {0.f, 0.f, 0.f, 0.f}, b_nxt = a_nxt;
-        if (grp + 4 < groups) {  // the next group's loads are in flight under this group's MFMAs
-            a_nxt = frag_a(grp + 4);
-            b_nxt = frag_b(grp + 4);
-        }
+    // k <= 256 is at most 32 groups, 8 per wave: all of a wave's operand loads are issued before its first MFMA, so
+    // the kernel pays one memory round trip instead of one per group
+    constexpr int kMaxGroups = 8;
+    floatx4 a_frag[kMaxGroups], b_frag[kMaxGroups];
 #pragma unroll
-        for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[c], b_cur[c], acc, 0, 0, 0);
-        a_cur = a_nxt;
-        b_cur = b_nxt;
+    for (int i = 0; i < kMaxGroups; i++) {
+        const size_t grp = (size_t)wave + 4 * (size_t)i;
+        a_frag[i] = frag_a(grp);  // zero beyond k
+        b_frag[i] = frag_b(grp);
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxGroups; i++) {
+        if ((size_t)wave + 4 * (size_t)i < groups) {
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_frag[i][c], b_frag[i][c], acc, 0, 0, 0);
+        }
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) part[wave][r][lane] = acc[r];

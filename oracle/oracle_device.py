@@ -117,6 +117,9 @@ class OracleDevice(HipDevice):
     def mem_alloc_host(self, dtype, n):
         return self._new(dtype, n, "raw")
 
+    def host_view(self, buf):
+        return self._view(buf)  # all of the oracle's memory is host memory
+
     def mem_cache_alloc(self, dtype, n):
         return self._new(dtype, n, "cache")
 

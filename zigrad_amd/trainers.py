@@ -144,12 +144,23 @@ class GraphSteps:
     graph_loss = None
     _capturing = False
 
+    _loss_pinned = None
+    _loss_view = None
+
+    def _init_loss_slot(self) -> None:
+        """One float of pinned host memory the device posts the loss into (allocated with the trainer: driver
+        allocations are refused while a step is being recorded)."""
+        self._loss_pinned = self.dev.mem_alloc_host(F32, 1)
+        self._loss_view = self.dev.host_view(self._loss_pinned)
+
     def _read_loss(self, loss: DevBuf):
-        if self._capturing:  # nothing executes while recording: remember where the loss will be
-            self.graph_loss = DevBuf(loss.ptr, 1, loss.dtype, 0, "view")
+        """loss.get(0): the device posts the value into pinned host memory on its stream (a copy kernel when the step
+        is being recorded) and the host waits for the stream; cheaper than a blocking driver copy of four bytes."""
+        self.dev.mem_copy(loss, self._loss_pinned)
+        if self._capturing:  # nothing executes while recording
             return None
-        self.dev.mem_transfer(loss, self.loss_host, "DtoH")
-        return float(self.loss_host[0])
+        self.dev.sync()
+        return float(self._loss_view[0])
 
     def capture(self) -> None:
         """Record one step.  Run at least one eager step first, so that the allocator and the library's internal
@@ -169,8 +180,8 @@ class GraphSteps:
         self.graph.run()
         if not read_loss:
             return None
-        self.dev.mem_transfer(self.graph_loss, self.loss_host, "DtoH")
-        return float(self.loss_host[0])
+        self.dev.sync()
+        return float(self._loss_view[0])
 
     def free_graph(self) -> None:
         if self.graph is not None:
@@ -345,7 +356,7 @@ class MLPTrainer(GraphSteps):
         self.x = dev.mem_alloc(F32, batch * dims[0])
         self.onehot = dev.mem_alloc(F32, batch * dims[-1])
         self.labels = dev.mem_alloc(U64, batch)
-        self.loss_host = np.zeros(1, np.float32)
+        self._init_loss_slot()
         self.last_grads = None
 
     def load_params(self, params) -> None:
@@ -461,7 +472,7 @@ class DQNTrainer(GraphSteps):
         self.rewards, self.dones = dev.mem_alloc(F32, B), dev.mem_alloc(F32, B)
         self.gamma_t = dev.from_numpy(np.asarray([gamma], np.float32))
         self.one_t = dev.from_numpy(np.asarray([1.0], np.float32))
-        self.loss_host = np.zeros(1, np.float32)
+        self._init_loss_slot()
         self.last_grads = None
 
     def load_params(self, params) -> None:
@@ -580,7 +591,7 @@ class GCNTrainer(GraphSteps):
         d.mem_transfer(np.concatenate([inp["src"], inp["tgt"]]), self.edge_index, "HtoD")
         self.src, self.tgt = self.edge_index.sub(0, self.E), self.edge_index.sub(self.E, self.E)
         self.label_m = d.from_numpy(inp["onehot"][: self.n_train])
-        self.loss_host = np.zeros(1, np.float32)
+        self._init_loss_slot()
         self.last_grads = None
 
     def param_buffers(self):

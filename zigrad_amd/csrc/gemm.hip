@@ -550,22 +550,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
     floatx16 acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    // k <= 256 is at most 32 groups, 8 per wave: all of a wave's operand loads are issued before its first MFMA, so
-    // the kernel pays one memory round trip instead of one per group
+    // 32 groups (k = 256) per round, 8 per wave: all of a wave's operand loads of a round are issued before its first
+    // MFMA, so a round costs one memory round trip instead of one per group.  Most callers need a single round.
     constexpr int kMaxGroups = 8;
-    floatx4 a_frag[kMaxGroups], b_frag[kMaxGroups];
+    for (size_t base = 0; base < groups; base += 4 * kMaxGroups) {
+        floatx4 a_frag[kMaxGroups], b_frag[kMaxGroups];
 #pragma unroll
-    for (int i = 0; i < kMaxGroups; i++) {
-        const size_t grp = (size_t)wave + 4 * (size_t)i;
-        a_frag[i] = frag_a(grp);  // zero beyond k
-        b_frag[i] = frag_b(grp);
-    }
+        for (int i = 0; i < kMaxGroups; i++) {
+            const size_t grp = base + (size_t)wave + 4 * (size_t)i;
+            a_frag[i] = frag_a(grp);  // zero beyond k
+            b_frag[i] = frag_b(grp);
+        }
 #pragma unroll
-    for (int i = 0; i < kMaxGroups; i++) {
-        if ((size_t)wave + 4 * (size_t)i < groups) {
+        for (int i = 0; i < kMaxGroups; i++) {
+            if (base + (size_t)wave + 4 * (size_t)i < groups) {
 #pragma unroll
-            for (int c = 0; c < 4; c++)
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_frag[i][c], b_frag[i][c], acc, 0, 0, 0);
+                for (int c = 0; c < 4; c++)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_frag[i][c], b_frag[i][c], acc, 0, 0, 0);
+            }
         }
     }
 #pragma unroll
@@ -729,7 +731,10 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         return ZG_HIP_OK;
     }
 
-    if (k <= 256 && tiles(32, 32) <= n_cu) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
+    // the unstaged kernel: short k on up to one block per CU, or a longer k when C is only a handful of blocks (the
+    // first layer of the batch-64 MLP, 64 x 128 x 784: 6 us in one launch against 14 us split and reduced)
+    if ((k <= 256 && tiles(32, 32) <= n_cu) || (k <= 2048 && tiles(32, 32) <= 16))
+        return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
 
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
     if (c_large <= c_mid && c_large <= c_small)

@@ -398,6 +398,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     const ptrdiff_t gate_bytes = gated ? reinterpret_cast<const char*>(g.gate) - reinterpret_cast<const char*>(g.C) : 0;
 
     const bool use_old = use_c || gated;
+    const bool any_extras = has_bias || relu || gated;
     // The accumulators are taken out of their AGPRs one row of blocks at a time through an explicit
     // v_accvgpr_read (the "a" constraint pins the value in an AGPR up to that point).  Left to itself the
     // register allocator copies all of them to VGPRs at the loop exit, which doubles the kernel's register
@@ -450,25 +451,37 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             for (int r = 0; r < 16; r++) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(res[j][r]) : "a"(acc[i][j][r]));
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                v[j] = alpha * res[j][r];
-                if (use_c) v[j] += beta * old[j][r];
-                v[j] = gemm_extras(v[j], has_bias, bias_v[j], relu);
-                if (gated) v[j] = old[j][r] <= 0.f ? 0.f : v[j];
+                float v = alpha * res[j][r];
+                if (use_c) v += beta * old[j][r];
+                res[j][r] = v;
             }
+        }
+        if (any_extras) {  // one uniform branch: the plain products skip all of it
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    float v = gemm_extras(res[j][r], has_bias, bias_v[j], relu);
+                    if (gated) v = old[j][r] <= 0.f ? 0.f : v;
+                    res[j][r] = v;
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
             if (VEC_C) {
                 VC o;
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
-                    if constexpr (VEC_C) o[j] = v[j];
+                    if constexpr (VEC_C) o[j] = res[j][r];
                 }
                 if (in_range(0, r)) *reinterpret_cast<VC*>(cptr[0] + (size_t)row_of(r) * g.ldc) = o;
             } else {
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    if (in_range(j, r)) cptr[j][(size_t)row_of(r) * g.ldc] = v[j];
+                    if (in_range(j, r)) cptr[j][(size_t)row_of(r) * g.ldc] = res[j][r];
             }
         }
         // one row of blocks at a time

@@ -75,3 +75,29 @@ def test_zig_veneer_calls_match_the_header():
     for name, n_args in calls:
         assert name in protos, f"{name} is called by the veneer but not declared in zg_hip.h"
         assert n_args == len(protos[name][1]), f"{name}: veneer passes {n_args} arguments, header declares {len(protos[name][1])}"
+
+
+def test_header_is_plain_c_and_links_from_a_c_program(tmp_path):
+    """include/zg_hip.h compiles as C11 with gcc (no C++ in the boundary) and a C program linked against the library
+    can call it: device count and the error string, nothing that needs a GPU."""
+    import subprocess
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    src = tmp_path / "probe.c"
+    src.write_text(
+        '#include <stdio.h>\n#include "zg_hip.h"\n'
+        "int main(void) {\n"
+        "    int n = -1;\n"
+        "    if (zg_hip_device_count(&n) != 0 || n < 0) return 2;\n"
+        "    if (zg_hip_sync(NULL) == 0) return 3; /* a null context must be refused */\n"
+        '    printf("%d %s\\n", n, zg_hip_last_error());\n'
+        "    return 0;\n}\n")
+    exe = tmp_path / "probe"
+    cc = ["gcc", "-std=c11", "-Wall", "-Werror", "-pedantic", f"-I{root / 'include'}", str(src), "-o", str(exe),
+          f"-L{LIB_PATH.parent}", "-lzg_hip", f"-Wl,-rpath,{LIB_PATH.parent}"]
+    built = subprocess.run(cc, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr
+    ran = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert ran.returncode == 0, (ran.returncode, ran.stdout, ran.stderr)
+    assert "null context" in ran.stdout

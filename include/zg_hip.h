@@ -222,6 +222,24 @@ int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx *ctx, const float *grad_output,
                                       const uint64_t *src_indices, const uint64_t *tgt_indices, float *grad_h,
                                       float *grad_deg, size_t stride, size_t n_edge, size_t n_nodes);
 
+/* Edge plans.  The three ops above sort the edge list by destination on every call, because the reference hands
+ * them bare index slices (examples/gcn/src/model.zig:116-224 builds them per forward).  For an edge list that does
+ * not change between calls (the dataset's graph, examples/gcn/src/dataset.zig:110-127) the analysis can be done
+ * once: a plan holds both orderings (by target, by source) and device copies of the two index arrays; the planned
+ * ops launch the same kernels on it and return the same values as zg_hip_scatter_add (offsets = targets),
+ * zg_hip_scatter_gcn_deg_scaled and zg_hip_scatter_gcn_deg_scaled_bwd.  The index arrays may be device or
+ * zg_hip_host_alloc memory and may be reused after create returns.  Create and free are refused while recording. */
+typedef struct zg_hip_edge_plan zg_hip_edge_plan;
+int zg_hip_edge_plan_create(zg_hip_ctx *ctx, const uint64_t *src_indices, const uint64_t *tgt_indices, size_t n_edge,
+                            size_t n_nodes, zg_hip_edge_plan **out);
+int zg_hip_edge_plan_free(zg_hip_ctx *ctx, zg_hip_edge_plan *plan);
+int zg_hip_scatter_add_planned(zg_hip_ctx *ctx, const float *src, const zg_hip_edge_plan *plan, float *dst);
+int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx *ctx, float *dst, const float *h, const float *deg,
+                                          const zg_hip_edge_plan *plan, size_t stride);
+int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx *ctx, const float *grad_output, const float *h,
+                                              const float *deg, const zg_hip_edge_plan *plan, float *grad_h,
+                                              float *grad_deg, size_t stride);
+
 /* ---------------------------------------------------------------------------------------------
  * losses: the host loops of src/nn/loss.zig:94-305 as device ops (new op names; the reference
  * dereferences .raw on the host and has no opspec for them)

@@ -180,6 +180,24 @@ class OracleDevice(HipDevice):
         raise NotImplementedError("the oracle is timed with time.perf_counter")
 
     # -- entry points whose oracle signature differs from the C ABI ----------------------------------
+    # -- planned scatter ops: the plan is just the index arrays, the ops are the sequential host loops ------
+    def edge_plan(self, src_indices, tgt_indices, n_nodes):
+        from zigrad_amd.device import EdgePlan
+
+        return EdgePlan(self, None, src_indices, tgt_indices, n_nodes)
+
+    def _op_scatter_add_planned(self, src, plan, dst):
+        self.dispatch("scatter_add", src=src, offsets=plan.tgt_indices, dst=dst)
+
+    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride):
+        self.dispatch("scatter_gcn_deg_scaled", dst=dst, h=h, deg=deg, src_indices=plan.src_indices,
+                      tgt_indices=plan.tgt_indices, stride=stride, n_edge=plan.src_indices.n)
+
+    def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride):
+        self.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=grad_output, h=h, deg=deg, src_indices=plan.src_indices,
+                      tgt_indices=plan.tgt_indices, grad_h=grad_h, grad_deg=grad_deg, stride=stride,
+                      n_edge=plan.src_indices.n)
+
     # -- the list entry points are the per-tensor ops in a loop --------------------------------------------
     def _op_sgd_step_multi(self, params, grads, lr, clip, max_norm, delta, zero_grads):
         for p, g in zip(params, grads):

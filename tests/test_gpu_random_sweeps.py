@@ -195,3 +195,51 @@ def test_scatter_ops_large_and_skewed_bit_exact(oracle, hip, n_nodes, n_edge):
          "tgt_indices": tgt, "stride": stride, "n_edge": n_edge}
     assert np.array_equal(run_op(oracle, "scatter_gcn_deg_scaled", dict(p), ["dst"])["dst"],
                           run_op(hip, "scatter_gcn_deg_scaled", dict(p), ["dst"])["dst"])
+
+
+@pytest.mark.parametrize("n_nodes,n_edge,where", [(2708, 13264, "host"), (2708, 13264, "device"), (1, 50, "device"),
+                                                  (300, 16000, "host"), (20000, 40000, "device"), (977, 3, "host")])
+def test_planned_scatter_ops_equal_the_unplanned_ones(oracle, hip, n_nodes, n_edge, where):
+    """An edge plan built once from index arrays in pinned host or device memory, used twice: scatter_add,
+    scatter_gcn_deg_scaled and its backward return exactly what the ops that take the bare index arrays return
+    (and what the sequential host loops return)."""
+    from conftest import run_op
+    from zigrad_amd.device import F32, U64
+
+    r = np.random.default_rng(n_nodes + 3 * n_edge)
+    src = r.integers(0, n_nodes, n_edge).astype(np.uint64)
+    tgt = np.where(r.random(n_edge) < 0.2, n_nodes // 3, r.integers(0, n_nodes, n_edge)).astype(np.uint64)
+    if where == "host":
+        s_buf, t_buf = hip.mem_alloc_host(U64, n_edge), hip.mem_alloc_host(U64, n_edge)
+    else:
+        s_buf, t_buf = hip.mem_alloc(U64, n_edge), hip.mem_alloc(U64, n_edge)
+    hip.mem_transfer(src, s_buf, "HtoD")
+    hip.mem_transfer(tgt, t_buf, "HtoD")
+    plan = hip.edge_plan(s_buf, t_buf, n_nodes)
+    hip.mem_transfer(np.zeros(n_edge, np.uint64), s_buf, "HtoD")  # the plan keeps its own copy of the indices
+    for rep, stride in enumerate((5, 16)):
+        vals = r.standard_normal(n_edge).astype(np.float32)
+        d0 = r.standard_normal(n_nodes).astype(np.float32)
+        got = run_op(hip, "scatter_add_planned", {"src": vals, "plan": plan, "dst": d0.copy()}, ["dst"])["dst"]
+        want = run_op(oracle, "scatter_add", {"src": vals, "offsets": tgt, "dst": d0.copy()}, ["dst"])["dst"]
+        assert np.array_equal(got, want), (rep, "scatter_add")
+        h = r.standard_normal(n_nodes * stride).astype(np.float32)
+        deg = (r.random(n_nodes) + 0.25).astype(np.float32)
+        y0 = r.standard_normal(n_nodes * stride).astype(np.float32)
+        got = run_op(hip, "scatter_gcn_deg_scaled_planned", {"dst": y0.copy(), "h": h, "deg": deg, "plan": plan,
+                                                              "stride": stride}, ["dst"])["dst"]
+        want = run_op(oracle, "scatter_gcn_deg_scaled", {"dst": y0.copy(), "h": h, "deg": deg, "src_indices": src,
+                                                         "tgt_indices": tgt, "stride": stride, "n_edge": n_edge}, ["dst"])["dst"]
+        assert np.array_equal(got, want), (rep, "fwd")
+        go = r.standard_normal(n_nodes * stride).astype(np.float32)
+        gh0, gd0 = r.standard_normal(n_nodes * stride).astype(np.float32), r.standard_normal(n_nodes).astype(np.float32)
+        got = run_op(hip, "scatter_gcn_deg_scaled_bwd_planned", {"grad_output": go, "h": h, "deg": deg, "plan": plan,
+                                                                  "grad_h": gh0.copy(), "grad_deg": gd0.copy(),
+                                                                  "stride": stride}, ["grad_h", "grad_deg"])
+        want = run_op(oracle, "scatter_gcn_deg_scaled_bwd", {"grad_output": go, "h": h, "deg": deg, "src_indices": src,
+                                                             "tgt_indices": tgt, "grad_h": gh0.copy(), "grad_deg": gd0.copy(),
+                                                             "stride": stride, "n_edge": n_edge}, ["grad_h", "grad_deg"])
+        assert np.array_equal(got["grad_h"], want["grad_h"]) and np.array_equal(got["grad_deg"], want["grad_deg"]), rep
+    plan.free()
+    hip.mem_free(s_buf)
+    hip.mem_free(t_buf)

@@ -472,6 +472,36 @@ pub fn adam_step_multi(self: *const Self, T: type, p: anytype) void {
     check(c.zg_hip_adam_step_multi(self.ctx, p.params.len, p.params.ptr, p.grads.ptr, p.ms.ptr, p.vs.ptr, p.lens.ptr, p.lr_t.ptr, @intFromBool(p.lr_t_in_memory), p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta, @intFromBool(p.zero_grads)));
 }
 
+/// Both destination orderings of an edge list that does not change between calls (the dataset's graph), built
+/// once; `scatter_add_planned`, `scatter_gcn_deg_scaled_planned` and `scatter_gcn_deg_scaled_bwd_planned` then
+/// return what the ops that take bare index slices return, without sorting the edges again on every call.
+pub const EdgePlan = struct {
+    ctx: *c.zg_hip_ctx,
+    plan: ?*c.zg_hip_edge_plan = null,
+
+    pub fn init(device: *const Self, src_indices: []const usize, tgt_indices: []const usize, n_nodes: usize) EdgePlan {
+        var self = EdgePlan{ .ctx = device.ctx };
+        check(c.zg_hip_edge_plan_create(device.ctx, @ptrCast(src_indices.ptr), @ptrCast(tgt_indices.ptr), src_indices.len, n_nodes, &self.plan));
+        return self;
+    }
+    pub fn deinit(self: *EdgePlan) void {
+        check(c.zg_hip_edge_plan_free(self.ctx, self.plan));
+        self.plan = null;
+    }
+};
+pub fn scatter_add_planned(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_add_planned(self.ctx, p.src.ptr, p.plan.plan, p.dst.ptr));
+}
+pub fn scatter_gcn_deg_scaled_planned(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_gcn_deg_scaled_planned(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.stride));
+}
+pub fn scatter_gcn_deg_scaled_bwd_planned(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_gcn_deg_scaled_bwd_planned(self.ctx, p.grad_output.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.grad_h.ptr, p.grad_deg.ptr, p.stride));
+}
+
 /// A Linear layer's forward in one launch: y = act(x . w^T + bias), the arithmetic of `bmm_acc(trans_b)` +
 /// `bias.add_` + `relu_` (examples/mnist/src/model.zig:104-110, :38-46).  `p.bias` is an optional slice.
 pub fn linear_fwd(self: *const Self, T: type, p: anytype) void {

@@ -600,3 +600,111 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// Edge plans: the segment plans of an edge list that does not change between calls (a dataset's graph), built once.
+// The planned ops launch the same apply kernels on the same plans as the ops above, so their results are identical;
+// what they save is the plan construction (five launches per plan, two plans in the backward op).
+// ------------------------------------------------------------------------------------------------
+struct zg_hip_edge_plan {
+    void* mem;          // one device allocation: both plans, then device copies of the two index arrays
+    zg::Plan by_tgt;    // buckets = targets, peer = source of each edge
+    zg::Plan by_src;    // buckets = sources, peer = target of each edge
+    uint64_t* src_dev;  // the index arrays as the unplanned ops receive them, in device memory
+    uint64_t* tgt_dev;
+    size_t n_edge, n_nodes;
+};
+
+ZG_API int zg_hip_edge_plan_create(zg_hip_ctx* ctx, const uint64_t* src_indices, const uint64_t* tgt_indices,
+                                   size_t n_edge, size_t n_nodes, zg_hip_edge_plan** out) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "edge_plan_create");
+    ZG_REQUIRE(out != nullptr, "edge_plan_create: null output");
+    *out = nullptr;
+    ZG_REQUIRE(src_indices && tgt_indices, "edge_plan_create: null pointer");
+    ZG_REQUIRE(n_edge > 0, "edge_plan_create: empty edge list");
+    if (int rc = check_gcn("edge_plan_create", 1, n_edge, n_nodes)) return rc;
+    const size_t pb = align_up(plan_bytes(n_edge, n_nodes), 256), ib = align_up(n_edge * sizeof(uint64_t), 256);
+    void* mem = nullptr;
+    if (int rc = zg_hip_alloc(ctx, 2 * pb + 2 * ib, &mem)) return rc;
+    zg_hip_edge_plan* pl = new zg_hip_edge_plan;
+    pl->mem = mem;
+    pl->by_tgt = carve_plan(mem, n_edge, n_nodes);
+    pl->by_src = carve_plan((char*)mem + pb, n_edge, n_nodes);
+    pl->src_dev = (uint64_t*)((char*)mem + 2 * pb);
+    pl->tgt_dev = (uint64_t*)((char*)mem + 2 * pb + ib);
+    pl->n_edge = n_edge;
+    pl->n_nodes = n_nodes;
+    int rc = zg_hip_memcpy_d2d(ctx, pl->src_dev, src_indices, n_edge * sizeof(uint64_t));  // device or pinned source
+    if (!rc) rc = zg_hip_memcpy_d2d(ctx, pl->tgt_dev, tgt_indices, n_edge * sizeof(uint64_t));
+    if (!rc) rc = build_plan(ctx, pl->tgt_dev, pl->by_tgt, pl->src_dev);
+    if (!rc) rc = build_plan(ctx, pl->src_dev, pl->by_src, pl->tgt_dev);
+    if (rc) {
+        zg_hip_free(ctx, mem);
+        delete pl;
+        return rc;
+    }
+    *out = pl;
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_edge_plan_free(zg_hip_ctx* ctx, zg_hip_edge_plan* plan) {
+    ZG_CTX(ctx);
+    if (!plan) return ZG_HIP_OK;
+    ZG_NOT_CAPTURING(ctx, "edge_plan_free");
+    ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));  // kernels that read the plan may still be queued
+    int rc = zg_hip_free(ctx, plan->mem);
+    delete plan;
+    return rc;
+}
+
+// dst[tgt[e]] += src[e] in edge order (zg_hip_scatter_add with offsets = the plan's targets)
+ZG_API int zg_hip_scatter_add_planned(zg_hip_ctx* ctx, const float* src, const zg_hip_edge_plan* plan, float* dst) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(plan && src && dst, "scatter_add_planned: null pointer");
+    hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(plan->n_nodes, 256)), dim3(256), 0,
+                       ctx->stream, src, plan->by_tgt.row_ptr, plan->by_tgt.perm, dst, plan->n_nodes);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,
+                                                 const zg_hip_edge_plan* plan, size_t stride) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(plan && dst && h && deg, "scatter_gcn_deg_scaled_planned: null pointer");
+    ZG_REQUIRE(stride > 0, "scatter_gcn_deg_scaled_planned: stride is 0");
+    const size_t n_nodes = plan->n_nodes;
+    const int g = group_for(stride);
+    const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
+                                        plan->by_tgt.row_ptr, plan->by_tgt.peer, n_nodes, stride));
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx* ctx, const float* grad_output, const float* h,
+                                                     const float* deg, const zg_hip_edge_plan* plan, float* grad_h,
+                                                     float* grad_deg, size_t stride) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(plan && grad_output && h && deg && grad_h && grad_deg, "scatter_gcn_deg_scaled_bwd_planned: null pointer");
+    ZG_REQUIRE(stride > 0, "scatter_gcn_deg_scaled_bwd_planned: stride is 0");
+    const size_t n_nodes = plan->n_nodes, n_edge = plan->n_edge;
+    const size_t tb = align_up(n_edge * sizeof(float), 256);
+    char* mem = (char*)workspace(ctx, 2 * tb);
+    if (!mem) return ZG_HIP_EOOM;
+    float* term_src = (float*)mem;
+    float* term_tgt = (float*)(mem + tb);
+    const int g = group_for(stride);
+    const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
+                                        grad_output, deg, plan->by_src.row_ptr, plan->by_src.peer, n_nodes, stride));
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
+                       grad_output, h, deg, plan->src_dev, plan->tgt_dev, n_edge, n_nodes, stride, term_src, term_tgt);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
+                       grad_deg, term_src, term_tgt, plan->by_src.row_ptr, plan->by_src.perm, plan->by_tgt.row_ptr,
+                       plan->by_tgt.perm, n_nodes);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}

@@ -394,6 +394,22 @@ class HipDevice:
         self._call("zg_hip_scatter_gcn_deg_scaled_bwd", grad_output.ptr, h.ptr, deg.ptr, src_indices.ptr,
                    tgt_indices.ptr, grad_h.ptr, grad_deg.ptr, stride, n_edge, deg.n)
 
+    # the same three ops on an edge plan built once for an edge list that does not change
+    def edge_plan(self, src_indices: DevBuf, tgt_indices: DevBuf, n_nodes: int) -> "EdgePlan":
+        h = ctypes.c_void_p()
+        self._call("zg_hip_edge_plan_create", src_indices.ptr, tgt_indices.ptr, src_indices.n, n_nodes, ctypes.byref(h))
+        return EdgePlan(self, h, src_indices, tgt_indices, n_nodes)
+
+    def _op_scatter_add_planned(self, src, plan, dst):
+        self._call("zg_hip_scatter_add_planned", src.ptr, plan.handle, dst.ptr)
+
+    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride):
+        self._call("zg_hip_scatter_gcn_deg_scaled_planned", dst.ptr, h.ptr, deg.ptr, plan.handle, stride)
+
+    def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride):
+        self._call("zg_hip_scatter_gcn_deg_scaled_bwd_planned", grad_output.ptr, h.ptr, deg.ptr, plan.handle, grad_h.ptr,
+                   grad_deg.ptr, stride)
+
     # losses
     def _op_smce_fwd(self, logits, target, probs, loss, rows, cols):
         self._call("zg_hip_smce_fwd", logits.ptr, target.ptr, probs.ptr, loss.ptr, rows, cols)
@@ -476,6 +492,19 @@ class Graph:
         if self._h is not None:
             self._dev._call("zg_hip_graph_free", self._h)
             self._h = None
+
+
+class EdgePlan:
+    """Both destination orderings of an edge list, built once (zg_hip_edge_plan_create)."""
+
+    def __init__(self, dev, handle, src_indices, tgt_indices, n_nodes):
+        self._dev, self.handle = dev, handle
+        self.src_indices, self.tgt_indices, self.n_nodes = src_indices, tgt_indices, n_nodes
+
+    def free(self) -> None:
+        if self.handle is not None:
+            self._dev._call("zg_hip_edge_plan_free", self.handle)
+            self.handle = None
 
 
 class Event:

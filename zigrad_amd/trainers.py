@@ -590,6 +590,8 @@ class GCNTrainer(GraphSteps):
         self.edge_index = d.mem_alloc_host(U64, 2 * self.E)
         d.mem_transfer(np.concatenate([inp["src"], inp["tgt"]]), self.edge_index, "HtoD")
         self.src, self.tgt = self.edge_index.sub(0, self.E), self.edge_index.sub(self.E, self.E)
+        # fused: the edge list is the dataset's and never changes, so its segment plans are built once
+        self.plan = d.edge_plan(self.src, self.tgt, self.N) if fused else None
         self.label_m = d.from_numpy(inp["onehot"][: self.n_train])
         self._init_loss_slot()
         self.last_grads = None
@@ -611,7 +613,10 @@ class GCNTrainer(GraphSteps):
         d.mem_fill(ones_edges, 1.0)
         contrib = d.mem_cache_alloc(F32, N)
         d.mem_fill(contrib, 0.0)
-        d.dispatch("scatter_add", src=ones_edges, offsets=self.tgt, dst=contrib)
+        if self.plan is not None:
+            d.dispatch("scatter_add_planned", src=ones_edges, plan=self.plan, dst=contrib)
+        else:
+            d.dispatch("scatter_add", src=ones_edges, offsets=self.tgt, dst=contrib)
         d.mem_cache_free(ones_edges)
         d.dispatch("add", x=contrib, y=deg, z=deg)  # deg._add(deg_contrib)
         d.mem_cache_free(contrib)
@@ -620,8 +625,11 @@ class GCNTrainer(GraphSteps):
         d.mem_cache_free(deg)
         y = d.mem_cache_alloc(F32, N * fan_out)
         d.mem_fill(y, 0.0)
-        d.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg_norm, src_indices=self.src, tgt_indices=self.tgt,
-                   stride=fan_out, n_edge=E)
+        if self.plan is not None:
+            d.dispatch("scatter_gcn_deg_scaled_planned", dst=y, h=h, deg=deg_norm, plan=self.plan, stride=fan_out)
+        else:
+            d.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg_norm, src_indices=self.src, tgt_indices=self.tgt,
+                       stride=fan_out, n_edge=E)
         d.dispatch("add", x=self.b[l], y=y, z=y)  # y._add(bias)
         return {"x": x_in, "h": h, "deg": deg_norm, "y": y}
 
@@ -633,8 +641,12 @@ class GCNTrainer(GraphSteps):
         d.mem_fill(g_h, 0.0)
         g_deg = d.mem_cache_alloc(F32, N)
         d.mem_fill(g_deg, 0.0)
-        d.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=g_y, h=saved["h"], deg=saved["deg"], src_indices=self.src,
-                   tgt_indices=self.tgt, grad_h=g_h, grad_deg=g_deg, stride=fan_out, n_edge=E)
+        if self.plan is not None:
+            d.dispatch("scatter_gcn_deg_scaled_bwd_planned", grad_output=g_y, h=saved["h"], deg=saved["deg"], plan=self.plan,
+                       grad_h=g_h, grad_deg=g_deg, stride=fan_out)
+        else:
+            d.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=g_y, h=saved["h"], deg=saved["deg"], src_indices=self.src,
+                       tgt_indices=self.tgt, grad_h=g_h, grad_deg=g_deg, stride=fan_out, n_edge=E)
         d.mem_cache_free(g_y)
         d.mem_cache_free(saved["y"])
         d.mem_cache_free(g_deg)  # deg itself needs no gradient: the chain stops at rsqrt (src/ndtensor.zig:1009)

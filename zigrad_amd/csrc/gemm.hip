@@ -85,10 +85,13 @@ struct Tile {
     // fast path: `base` is the tile origin (uniform), `off` this thread's byte offset of piece i.  A buffer load
     // takes the base as a scalar resource and the offset as one 32-bit VGPR, so moving along k costs scalar adds
     // only (a flat global load needs a 64-bit vector add per piece and tile).
-    __device__ __forceinline__ void load_fast(int i, const float* __restrict__ base, unsigned off) {
+    // `bytes` = size of the buffer from `base` on: a load that starts beyond it returns zeros instead of touching
+    // memory (the loads of the last tiles of a k that ends inside a tile can pass the end of the operand).
+    __device__ __forceinline__ void load_fast(int i, const float* __restrict__ base, unsigned off,
+                                              unsigned bytes = 0xffffffffu) {
         typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
         const __amdgpu_buffer_rsrc_t rsrc =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)0xffffffffu, 0x00020000);
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)bytes, 0x00020000);
         r[i] = __builtin_bit_cast(floatx4, (uintx4)__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
     }
 
@@ -130,6 +133,24 @@ struct Tile {
         // lds_thread_base = buffer + lds_offset(0); the further pieces sit at compile-time distances
         constexpr int STEP = KMAJOR ? (kGemmThreads / (kBK / 4)) * LD : (kGemmThreads / (BMN / 4)) * LD;
         *reinterpret_cast<floatx4*>(lds_thread_base + i * STEP) = r[i];
+    }
+    // the same store for a tile that starts at k0 and may reach past k_end: values at k >= k_end become zero
+    __device__ __forceinline__ void store_masked(float* __restrict__ lds_thread_base, int i, size_t k0,
+                                                 size_t k_end) const {
+        constexpr int STEP = KMAJOR ? (kGemmThreads / (kBK / 4)) * LD : (kGemmThreads / (BMN / 4)) * LD;
+        int tmn, tk;
+        coords(i, tmn, tk);
+        const size_t k = k0 + tk;
+        floatx4 v = r[i];
+        if (KMAJOR) {
+            if (k + 0 >= k_end) v.x = 0.f;
+            if (k + 1 >= k_end) v.y = 0.f;
+            if (k + 2 >= k_end) v.z = 0.f;
+            if (k + 3 >= k_end) v.w = 0.f;
+        } else if (k >= k_end) {
+            v = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+        *reinterpret_cast<floatx4*>(lds_thread_base + i * STEP) = v;
     }
 };
 
@@ -212,7 +233,9 @@ __device__ __forceinline__ void tile_coords(unsigned pid, unsigned tiles_m, unsi
     tn = in_group / gsize;
 }
 
-// MODE 0 (fast): whole tiles, aligned operands, an even number of k-tiles; no bounds checks anywhere.
+// MODE 0 (fast): whole tiles in m and n, aligned operands; no bounds checks in the loop.  A k that is not a whole
+//                number of tile pairs is handled by the last two pairs of steps: their loads see the operand's true
+//                size (buffer bounds: nothing past the end is touched) and their LDS writes zero what lies past k.
 // MODE 1 (edge): as fast, but M and N may end inside a tile: the per-thread load offsets are clamped to the last
 //                valid row / 4-column piece once, before the loop (rows and columns past the edge then hold copies
 //                of valid data, which only reach C elements that are never stored), and the epilogue checks bounds.
@@ -258,6 +281,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     const size_t k_end = (k_begin + g.split_tiles * BK < g.K) ? k_begin + g.split_tiles * BK : g.K;
     // 32-bit tile counter: there is no scalar 64-bit ordered compare, and a vector compare in the loop costs MFMA time
     const unsigned KT = (unsigned)((k_end - k_begin + BK - 1) / BK);
+    // fast / edge kernels: a k range that is not a whole number of tile pairs ends in tiles whose values past k_end
+    // are zeroed on their way into LDS (the last two pairs of steps run the masking variant of the step)
+    const bool ragged_k = !SAFE && (k_end - k_begin) % (2 * BK) != 0;
     constexpr int NM = TM * TN;         // MFMAs per step
     constexpr int NMF = 4 * NM;         // MFMAs per k-group
     constexpr int NR = FA::N + FB::N;   // fragment reads per k-group
@@ -292,25 +318,47 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     }
     const float* const a_org = A_KMAJOR ? A + m0 * g.lda : A + m0;  // tile origin at k = 0
     const float* const b_org = B_KMAJOR ? B + n0 * g.ldb : B + n0;
+    // one past the last element of each operand
+    const float* const a_end = A_KMAJOR ? A + (g.M - 1) * g.lda + g.K : A + (g.K - 1) * g.lda + g.M;
+    const float* const b_end = B_KMAJOR ? B + (g.N - 1) * g.ldb + g.K : B + (g.K - 1) * g.ldb + g.N;
+    auto bytes_left = [](const float* base, const float* end) {
+        const size_t n = base < end ? (size_t)(end - base) * sizeof(float) : 0;
+        return (unsigned)(n < 0xffffffffull ? n : 0xffffffffull);
+    };
 
     // Tiles wait in registers for two tile times between their global loads and their LDS writes (slot t % 2),
     // which covers the HBM latency also when a workgroup has a CU to itself.
     TA ta[2];
     TB tb[2];
-    auto load_op = [&](auto slot_tag, int v, size_t k0) {
+    auto load_op = [&](auto slot_tag, int v, size_t k0, auto bounded_tag) {
         constexpr int S = decltype(slot_tag)::value;
+        constexpr bool BOUNDED = decltype(bounded_tag)::value;  // give the buffer its true size (last tiles only)
         if (v < TA::NV) {
-            if (!SAFE) ta[S].load_fast(v, a_org + (A_KMAJOR ? k0 : k0 * g.lda), a_off[v]);
-            else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
+            if (!SAFE) {
+                const float* base = a_org + (A_KMAJOR ? k0 : k0 * g.lda);
+                ta[S].load_fast(v, base, a_off[v], BOUNDED ? bytes_left(base, a_end) : 0xffffffffu);
+            } else {
+                ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
+            }
         } else {
-            if (!SAFE) tb[S].load_fast(v - TA::NV, b_org + (B_KMAJOR ? k0 : k0 * g.ldb), b_off[v - TA::NV]);
-            else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
+            if (!SAFE) {
+                const float* base = b_org + (B_KMAJOR ? k0 : k0 * g.ldb);
+                tb[S].load_fast(v - TA::NV, base, b_off[v - TA::NV], BOUNDED ? bytes_left(base, b_end) : 0xffffffffu);
+            } else {
+                tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
+            }
         }
     };
-    auto store_op = [&](auto slot_tag, int w, int buf) {
+    // k0: first k of the tile being stored (used by the masking variant only)
+    auto store_op = [&](auto slot_tag, int w, int buf, size_t k0, auto masked_tag) {
         constexpr int S = decltype(slot_tag)::value;
-        if (w < TA::NV) ta[S].store_op(a_wr + buf * TA::ELEMS, w);
-        else tb[S].store_op(b_wr + buf * TB::ELEMS, w - TA::NV);
+        if constexpr (decltype(masked_tag)::value) {
+            if (w < TA::NV) ta[S].store_masked(a_wr + buf * TA::ELEMS, w, k0, k_end);
+            else tb[S].store_masked(b_wr + buf * TB::ELEMS, w - TA::NV, k0, k_end);
+        } else {
+            if (w < TA::NV) ta[S].store_op(a_wr + buf * TA::ELEMS, w);
+            else tb[S].store_op(b_wr + buf * TB::ELEMS, w - TA::NV);
+        }
     };
     // fragment register sets: k-group 0 of a tile lives in set 0, k-group 1 in set 1
     FA fa[2];
@@ -332,11 +380,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     constexpr int E0 = NL + NR + NL;
     constexpr int PER0 = (E0 + NMF - 1) / NMF;
     constexpr int PER1 = (NR + (NMF + 1) / 2 - 1) / ((NMF + 1) / 2);  // reads land in the first half of group 1
-    auto tile_step = [&](unsigned kt, auto parity_tag) {
+    auto tile_step = [&](unsigned kt, auto parity_tag, auto masked_tag) {
         constexpr int S = decltype(parity_tag)::value;  // kt % 2: LDS buffer and register slot of this tile
         using SCur = std::integral_constant<int, S>;
         using SNext = std::integral_constant<int, S ^ 1>;
         const size_t k_load = k_begin + (size_t)((SAFE || kt + 2 < KT) ? kt + 2 : KT - 1) * BK;
+        const size_t k_store = k_begin + (size_t)(kt + 1) * BK;
 #pragma unroll
         for (int grp = 0; grp < 2; grp++) {
 #pragma unroll
@@ -348,9 +397,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
                 if (grp == 0) {
 #pragma unroll
                     for (int e = n * PER0; e < (n + 1) * PER0 && e < E0; e++) {
-                        if (e < NL) load_op(SCur{}, e, k_load);              // slot S is free: tile kt is in LDS
+                        if (e < NL) load_op(SCur{}, e, k_load, masked_tag);  // slot S is free: tile kt is in LDS
                         else if (e < NL + NR) read_op(1, e - NL, S, 1);
-                        else store_op(SNext{}, e - NL - NR, S ^ 1);
+                        else store_op(SNext{}, e - NL - NR, S ^ 1, k_store, masked_tag);
                     }
                 } else {
 #pragma unroll
@@ -366,14 +415,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     };
     using P0 = std::integral_constant<int, 0>;
     using P1 = std::integral_constant<int, 1>;
+    using Plain = std::false_type;
+    using Masked = std::true_type;
 
     // prologue: tile 0 goes straight to LDS buffer 0, tile 1 starts its flight in slot 1
 #pragma unroll
-    for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin);
+    for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Masked{});
 #pragma unroll
-    for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0));
+    for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0), Masked{});
+    if (ragged_k) {
 #pragma unroll
-    for (int w = 0; w < NL; w++) store_op(P0{}, w, 0);
+        for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Masked{});
+    } else {
+#pragma unroll
+        for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Plain{});
+    }
     __syncthreads();
 #pragma unroll
     for (int n = 0; n < NR; n++) read_op(0, n, 0, 0);
@@ -381,9 +437,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 
     // Tiles go in pairs so that the loop body is one straight run of MFMAs.  The fast kernels are only used for
     // an even number of tiles; in the checked kernels a tile past the end of k loads as zeros and adds nothing.
-    for (unsigned kt = 0; kt < KT; kt += 2) {
-        tile_step(kt, P0{});
-        tile_step(kt + 1, P1{});
+    const unsigned kt_plain = !ragged_k ? KT : (KT > 4 ? ((KT + 1) & ~1u) - 4 : 0);
+    unsigned kt = 0;
+    for (; kt < kt_plain; kt += 2) {
+        tile_step(kt, P0{}, Plain{});
+        tile_step(kt + 1, P1{}, Plain{});
+    }
+    if constexpr (!SAFE) {
+        for (; kt < KT; kt += 2) {  // ragged k only: the last two pairs, whose stores may hold values past k_end
+            tile_step(kt, P0{}, Masked{});
+            tile_step(kt + 1, P1{}, Masked{});
+        }
     }
 
     // epilogue.  Accumulator register r of lane l belongs to block row (r/4)*8 + (l/32)*4 + r%4 and block
@@ -698,16 +762,18 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.a_vec = aligned16(A) && lda % 4 == 0 && a_chunk % 4 == 0;
     g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
 
-    // Kernel mode per tile shape: fast (whole tiles, aligned, even number of k-tiles), edge (aligned, ragged in m
-    // and n only) or checked (everything else), see gemm_kernel.
+    // Kernel mode per tile shape: fast (whole tiles in m and n), edge (ragged in m and n) or checked (C not
+    // 16-byte aligned, huge leading dimensions, or an m / n that would split a 16-byte piece), see gemm_kernel.
     const bool c_vec = aligned16(C) && ldc % 4 == 0 && c_chunk % 4 == 0;
     const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
-    const bool aligned = g.a_vec && g.b_vec && c_vec && small_ld;
+    // A and B go through 16-byte buffer loads, which the memory system serves at any 4-byte alignment (measured: an
+    // odd leading dimension costs a few percent); only C's vector stores need their natural alignment
+    const bool aligned = c_vec && small_ld;
     const bool mn_ok = (a_kmajor || m % 4 == 0) && (b_kmajor || n % 4 == 0);
     auto tiles = [&](size_t bm, size_t bn) { return ceil_div_sz(m, bm) * ceil_div_sz(n, bn) * batches; };
     auto mode = [&](size_t bm, size_t bn) {
-        if (!aligned || !mn_ok || k % (2 * kBK) != 0) return 2;
-        return (m % bm == 0 && n % bn == 0) ? 0 : 1;
+        if (!aligned || !mn_ok) return 2;
+        return (m % bm == 0 && n % bn == 0) ? 0 : 1;  // any k: the last tiles are masked on their way into LDS
     };
     // Tile choice by estimated time.  A CU works through its workgroups at a rate that depends on the tile shape
     // but hardly on how many of them share the CU (measured fraction of a CU's MFMA peak: 0.92 / 0.89 / 0.79),
@@ -719,30 +785,6 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     const size_t kt_total = ceil_div_sz(k, kBK);
     g.split_tiles = kt_total;
     g.split_stride = 0;
-
-    // A deep, aligned product whose k is not a whole number of tile pairs: the bulk of k goes through the fast /
-    // edge kernels and the remainder (fewer than 32 values of k) is accumulated by a second, checked pass with
-    // beta = 1.  The second pass re-reads and re-writes C, so this only pays when k is long.
-    const size_t k_main = k / (2 * kBK) * (2 * kBK);
-    if (depth == 0 && aligned && mn_ok && k_main < k && k_main >= 16 * kBK && tiles(64, 64) >= n_cu) {
-        const float* a_tail = trans_a ? A + k_main * lda : A + k_main;
-        const float* b_tail = trans_b ? B + k_main : B + k_main * ldb;
-        if (int rc = gemm_dispatch(ctx, name, A, B, C, m, n, k_main, trans_a, trans_b, lda, ldb, ldc, alpha, beta, batches,
-                                   nba, nbb, a_chunk, b_chunk, c_chunk, 1))
-            return rc;
-        // epilogue extras belong to the finished sum: bias and ReLU ride in the second pass; a gate cannot (it
-        // shares the epilogue's registers with the old C values) and runs as the separate op it replaces
-        const bool gate_after = extras && extras->gate;
-        const GemmExtras tail_extras = {extras ? extras->bias : nullptr, nullptr, extras ? extras->relu : 0};
-        if (int rc = gemm_dispatch(ctx, name, a_tail, b_tail, C, m, n, k - k_main, trans_a, trans_b, lda, ldb, ldc, alpha,
-                                   1.f, batches, nba, nbb, a_chunk, b_chunk, c_chunk, 1, extras ? &tail_extras : nullptr))
-            return rc;
-        if (gate_after) {
-            ZG_REQUIRE(ldc == n && batches == 1, "%s: a gated product needs a dense C", name);
-            return zg_hip_relu_inplace_bwd(ctx, extras->gate, C, m * n);
-        }
-        return ZG_HIP_OK;
-    }
 
     // the unstaged kernel: short k on up to one block per CU, or a longer k when C is only a handful of blocks (the
     // first layer of the batch-64 MLP, 64 x 128 x 784: 6 us in one launch against 14 us split and reduced)
@@ -783,7 +825,8 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
             gs.gate = nullptr;
             gs.relu = 0;
             // the partial-product buffer is 256-byte aligned and dense: its own alignment rule is n % 4 == 0
-            const int split_mode = (mode(64, 64) != 2 && n % 4 == 0 && (m * n) % 4 == 0) ? mode(64, 64) : 2;
+            const bool split_ok = small_ld && mn_ok && n % 4 == 0 && (m * n) % 4 == 0;
+            const int split_mode = split_ok ? ((m % 64 == 0 && n % 64 == 0) ? 0 : 1) : 2;
             int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
             if (rc) return rc;
             size_t blocks = ceil_div_sz(m * n, 256);

@@ -45,6 +45,9 @@ SHAPES = [
     (128, 64, 2048), (64, 64, 4096), (70, 50, 1000),
     # aligned but ragged in m and n (edge kernels: clamped loads, guarded stores), with and without a k remainder
     (2072, 1300, 1028), (4100, 2060, 100), (2072, 1300, 1024), (1000, 1000, 512), (100, 68, 64), (4, 4, 32),
+    # nothing a multiple of anything: odd m, n, k and (with the padding rule below) odd leading dimensions, so pieces
+    # of 16 bytes straddle the edges of the operands, C takes scalar stores and the last k-tiles are masked
+    (1023, 1021, 1019), (515, 259, 1031), (258, 1026, 2050), (1025, 3, 1025), (5, 1027, 513),
 ]
 
 

@@ -196,6 +196,9 @@ struct GemmArgs {
     // C + y * split_stride (the launcher points C at a buffer of partial products); one split = the whole of k
     size_t split_tiles, split_stride;
     int a_vec, b_vec;  // 16-byte vector loads are legal for this operand
+    int c_vec;         // vector stores to C are legal (alignment, ldc and n multiples of 4)
+    int bounded_tail;  // edge kernels: an m or n that ends inside a 16-byte piece reads a few floats past the
+                       // operand's end in the last k rows, so the last tiles must load through bounded descriptors
     // Optional epilogue of the fused Linear entry points, applied to v = alpha * acc + beta * C in this order:
     // v += bias[col]; v = max(v, 0) when relu; v = 0 where gate[row][col] <= 0 (gate laid out like C, only with
     // beta == 0).  All null / 0 for the plain products.
@@ -233,15 +236,16 @@ __device__ __forceinline__ void tile_coords(unsigned pid, unsigned tiles_m, unsi
     tn = in_group / gsize;
 }
 
-// MODE 0 (fast): whole tiles in m and n, aligned operands; no bounds checks in the loop.  A k that is not a whole
+// MODE 0 (fast): whole tiles in m and n, C fit for vector stores; no bounds checks in the loop.  A k that is not a whole
 //                number of tile pairs is handled by the last two pairs of steps: their loads see the operand's true
 //                size (buffer bounds: nothing past the end is touched) and their LDS writes zero what lies past k.
-// MODE 1 (edge): as fast, but M and N may end inside a tile: the per-thread load offsets are clamped to the last
-//                valid row / 4-column piece once, before the loop (rows and columns past the edge then hold copies
-//                of valid data, which only reach C elements that are never stored), and the epilogue checks bounds.
-//                Needs M % 4 == 0 (N % 4 == 0) when A (B) is not k-contiguous, so that a 16-byte piece is never
-//                half inside.  The loop is the fast loop.
-// MODE 2 (checked): every load checked and zero-filled, scalar loads where 16-byte loads are not legal.
+// MODE 1 (edge): as fast, but M and N may end inside a tile and C may need scalar stores: the per-thread load
+//                offsets are clamped once, before the loop, to the last valid row or to the 16-byte piece that holds
+//                it (rows and columns past the edge then hold copies of valid data or whatever follows the edge in
+//                memory, which only reach C elements that are never stored), and the epilogue checks bounds.  When
+//                such a piece sticks out of the operand (M or N not a multiple of 4 with a non-k-contiguous operand)
+//                the last tiles load through bounded descriptors like the tail of a ragged k.  The loop is the fast loop.
+// MODE 2 (checked): every load checked and zero-filled; only for leading dimensions beyond 32-bit byte offsets.
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int MODE>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     constexpr bool SAFE = MODE == 2;
@@ -283,7 +287,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     const unsigned KT = (unsigned)((k_end - k_begin + BK - 1) / BK);
     // fast / edge kernels: a k range that is not a whole number of tile pairs ends in tiles whose values past k_end
     // are zeroed on their way into LDS (the last two pairs of steps run the masking variant of the step)
-    const bool ragged_k = !SAFE && (k_end - k_begin) % (2 * BK) != 0;
+    const bool ragged_k = !SAFE && ((k_end - k_begin) % (2 * BK) != 0 || (MODE == 1 && g.bounded_tail != 0));
     constexpr int NM = TM * TN;         // MFMAs per step
     constexpr int NMF = 4 * NM;         // MFMAs per k-group
     constexpr int NR = FA::N + FB::N;   // fragment reads per k-group
@@ -301,7 +305,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         int tmn, tk;
         TA::coords(i, tmn, tk);
         if (MODE == 1) {
-            const size_t last = A_KMAJOR ? g.M - 1 : g.M - 4;
+            const size_t last = A_KMAJOR ? g.M - 1 : (g.M - 1) / 4 * 4;  // the row, or the piece that holds row M - 1
             if (m0 + tmn > last) tmn = (int)(last - m0);
         }
         a_off[i] = (unsigned)((A_KMAJOR ? tmn * g.lda + tk : tk * g.lda + tmn) * sizeof(float));
@@ -311,7 +315,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         int tmn, tk;
         TB::coords(i, tmn, tk);
         if (MODE == 1) {
-            const size_t last = B_KMAJOR ? g.N - 1 : g.N - 4;
+            const size_t last = B_KMAJOR ? g.N - 1 : (g.N - 1) / 4 * 4;
             if (n0 + tmn > last) tmn = (int)(last - n0);
         }
         b_off[i] = (unsigned)((B_KMAJOR ? tmn * g.ldb + tk : tk * g.ldb + tmn) * sizeof(float));
@@ -471,6 +475,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     constexpr bool VEC_C = !SAFE && !B_KMAJOR && TN > 1;
     using VC = typename VecOf<VEC_C ? TN : 1>::type;
+    const bool vec_c = VEC_C && (MODE == 0 || g.c_vec != 0);  // edge kernels also serve a C that needs scalar stores
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         float res[TN][16], old[TN][16];
@@ -495,7 +500,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         if (use_old) {  // the old C values, or the gate values when gated
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                if (VEC_C) {
+                if (vec_c) {
                     VC o = {};
                     if (in_range(0, r)) o = *reinterpret_cast<const VC*>(optr[0] + (size_t)row_of(r) * g.ldc);
 #pragma unroll
@@ -535,7 +540,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            if (VEC_C) {
+            if (vec_c) {
                 VC o;
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
@@ -762,18 +767,18 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.a_vec = aligned16(A) && lda % 4 == 0 && a_chunk % 4 == 0;
     g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
 
-    // Kernel mode per tile shape: fast (whole tiles in m and n), edge (ragged in m and n) or checked (C not
-    // 16-byte aligned, huge leading dimensions, or an m / n that would split a 16-byte piece), see gemm_kernel.
-    const bool c_vec = aligned16(C) && ldc % 4 == 0 && c_chunk % 4 == 0;
+    // Kernel mode per tile shape: fast (whole tiles in m and n, C fit for vector stores), edge (everything else) or
+    // checked (leading dimensions too large for 32-bit byte offsets), see gemm_kernel.
+    const bool c_vec = aligned16(C) && ldc % 4 == 0 && c_chunk % 4 == 0 && n % 4 == 0;
     const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
     // A and B go through 16-byte buffer loads, which the memory system serves at any 4-byte alignment (measured: an
-    // odd leading dimension costs a few percent); only C's vector stores need their natural alignment
-    const bool aligned = c_vec && small_ld;
-    const bool mn_ok = (a_kmajor || m % 4 == 0) && (b_kmajor || n % 4 == 0);
+    // odd leading dimension costs a few percent); the fast kernels store C in vectors, the edge kernels also in scalars
+    g.c_vec = c_vec;
+    g.bounded_tail = (!a_kmajor && m % 4 != 0) || (!b_kmajor && n % 4 != 0);
     auto tiles = [&](size_t bm, size_t bn) { return ceil_div_sz(m, bm) * ceil_div_sz(n, bn) * batches; };
     auto mode = [&](size_t bm, size_t bn) {
-        if (!aligned || !mn_ok) return 2;
-        return (m % bm == 0 && n % bn == 0) ? 0 : 1;  // any k: the last tiles are masked on their way into LDS
+        if (!small_ld) return 2;
+        return (m % bm == 0 && n % bn == 0 && c_vec) ? 0 : 1;  // any k: the last tiles are masked on their way into LDS
     };
     // Tile choice by estimated time.  A CU works through its workgroups at a rate that depends on the tile shape
     // but hardly on how many of them share the CU (measured fraction of a CU's MFMA peak: 0.92 / 0.89 / 0.79),
@@ -824,9 +829,8 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
             gs.bias = nullptr;  // the extras belong to the sum of the partial products: the reduce kernel applies them
             gs.gate = nullptr;
             gs.relu = 0;
-            // the partial-product buffer is 256-byte aligned and dense: its own alignment rule is n % 4 == 0
-            const bool split_ok = small_ld && mn_ok && n % 4 == 0 && (m * n) % 4 == 0;
-            const int split_mode = split_ok ? ((m % 64 == 0 && n % 64 == 0) ? 0 : 1) : 2;
+            gs.c_vec = n % 4 == 0 && (m * n) % 4 == 0;  // the partial-product buffer is 256-byte aligned and dense
+            const int split_mode = !small_ld ? 2 : ((m % 64 == 0 && n % 64 == 0 && gs.c_vec) ? 0 : 1);
             int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
             if (rc) return rc;
             size_t blocks = ceil_div_sz(m * n, 256);

@@ -79,6 +79,23 @@ def test_matmul_variants(oracle, hip, m, n, k, ta, tb):
         assert rel_fro(got[:, :n], ref[:, :n]) <= TOL
 
 
+@pytest.mark.parametrize("ta,tb", [(False, True), (True, False)])
+def test_matmul_with_a_leading_dimension_beyond_32_bit_offsets(hip, ta, tb):
+    """lda = 2^21 floats: a 256-row tile no longer fits 32-bit byte offsets, so the checked kernels take over."""
+    r = rng(77 + ta)
+    m, n, k, ld = 24, 40, 72, 1 << 21
+    if ta:  # A stored [k, lda] with m valid columns, B stored [k, ldb]
+        A = np.zeros((k, ld), np.float32); A[:, :m] = r.standard_normal((k, m))
+        B = np.zeros((k, ld), np.float32); B[:, :n] = r.standard_normal((k, n))
+        truth = A[:, :m].astype(np.float64).T @ B[:, :n].astype(np.float64)
+    else:   # A stored [m, lda] with k valid columns, B stored [n, ldb]
+        A = np.zeros((m, ld), np.float32); A[:, :k] = r.standard_normal((m, k))
+        B = np.zeros((n, ld), np.float32); B[:, :k] = r.standard_normal((n, k))
+        truth = A[:, :k].astype(np.float64) @ B[:, :k].astype(np.float64).T
+    got = run_matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, ta, tb, ld, ld, n, 1.0, 0.0)
+    assert rel_fro(got, truth) <= TOL
+
+
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 def test_matmul_exact_on_integers(oracle, hip, ta, tb):
     """Small integers make every product and partial sum exact in fp32: results must agree bit for bit."""

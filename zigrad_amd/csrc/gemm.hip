@@ -577,9 +577,15 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
         else if (!a_kmajor && b_kmajor) ZG_GEMM(false, true, MD); \
         else ZG_GEMM(false, false, MD);                         \
     } while (0)
-    if (mode == 0) ZG_GEMM_LAYOUT(0);
-    else if (mode == 1) ZG_GEMM_LAYOUT(1);
-    else ZG_GEMM_LAYOUT(2);
+    if (mode == 0) {
+        ZG_GEMM_LAYOUT(0);
+    } else if (mode == 1) {
+        ZG_GEMM_LAYOUT(1);
+    } else {
+        // the checked kernels exist for the 64 x 64 tile only: they serve leading dimensions beyond 32-bit byte offsets
+        if constexpr (BM == 64 && BN == 64) ZG_GEMM_LAYOUT(2);
+        else ZG_REQUIRE(false, "gemm: no checked kernel for this tile");
+    }
 #undef ZG_GEMM_LAYOUT
 #undef ZG_GEMM
     ZG_LAUNCH_CHECK();
@@ -791,6 +797,7 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.split_tiles = kt_total;
     g.split_stride = 0;
 
+    if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
     // the unstaged kernel: short k on up to one block per CU, or a longer k when C is only a handful of blocks (the
     // first layer of the batch-64 MLP, 64 x 128 x 784: 6 us in one launch against 14 us split and reduced)
     if ((k <= 256 && tiles(32, 32) <= n_cu) || (k <= 2048 && tiles(32, 32) <= 16))

@@ -423,14 +423,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     using Masked = std::true_type;
 
     // prologue: tile 0 goes straight to LDS buffer 0, tile 1 starts its flight in slot 1
+    if (__builtin_expect(ragged_k, 0)) {
 #pragma unroll
-    for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Masked{});
+        for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Masked{});
 #pragma unroll
-    for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0), Masked{});
-    if (ragged_k) {
+        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + (KT > 1 ? BK : 0), Masked{});
 #pragma unroll
         for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Masked{});
     } else {
+#pragma unroll
+        for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Plain{});
+#pragma unroll
+        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0), Plain{});
 #pragma unroll
         for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Plain{});
     }
@@ -448,9 +452,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         tile_step(kt + 1, P1{}, Plain{});
     }
     if constexpr (!SAFE) {
-        for (; kt < KT; kt += 2) {  // ragged k only: the last two pairs, whose stores may hold values past k_end
-            tile_step(kt, P0{}, Masked{});
-            tile_step(kt + 1, P1{}, Masked{});
+        if (__builtin_expect(kt < KT, 0)) {  // ragged k only: the last two pairs, whose stores may hold values past k_end
+            do {
+                tile_step(kt, P0{}, Masked{});
+                tile_step(kt + 1, P1{}, Masked{});
+                kt += 2;
+            } while (kt < KT);
         }
     }
 

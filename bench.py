@@ -334,6 +334,30 @@ def run_small(dev, kind, steps, graph=True, fused=False):
     return out
 
 
+def run_c_harness(dims, batch, steps):
+    """The same eager batch-64 step issued from plain C (tests/c_harness/mlp_step.c): what the op-by-op path costs
+    without an interpreter between the calls.  None when the binary has not been built."""
+    import subprocess
+    import tempfile
+
+    from zigrad_amd.build import C_HARNESS_BIN
+    from zigrad_amd.trainers import mlp_inputs
+
+    if not C_HARNESS_BIN.exists():
+        return None
+    params, x, onehot, _ = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data="uniform")
+    with tempfile.NamedTemporaryFile(suffix=".bin") as f:
+        for a in (*params, x, onehot):
+            f.write(np.ascontiguousarray(a, np.float32).tobytes())
+        f.flush()
+        run = subprocess.run([str(C_HARNESS_BIN), f.name, str(steps), str(batch), *map(str, dims)], capture_output=True,
+                             text=True, timeout=300)
+    if run.returncode != 0:
+        raise RuntimeError("tests/c_harness/mlp_step failed: " + run.stderr)
+    us = float(run.stdout.strip().splitlines()[-1].split()[1])
+    return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": "eager, same op sequence, caller in C"}
+
+
 def cpu_baseline(dims, batch, budget_steps=2):
     """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share."""
     from oracle.oracle_device import OracleDevice
@@ -433,6 +457,7 @@ def main():
             fs = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=True, fused=True)
             result["mlp_b64"]["fused"] = {"steps_per_s": 200 / fs[0], "ms_per_step": fs[0] / 200 * 1e3,
                                                  "graph_replay": {"steps_per_s": 200 / fs[2], "ms_per_step": fs[2] / 200 * 1e3}}
+        result["mlp_b64"]["c_caller"] = run_c_harness([784, 128, 64, 10], 64, 2000)
         result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
         result["gcn"] = run_small(dev, "gcn", 100, graph=not args.no_graph)
         result["dqn"] = run_small(dev, "dqn", 200, graph=not args.no_graph)

@@ -186,3 +186,19 @@ def test_fused_adam_step_replays_from_an_execution_graph(hip):
     for a, b in zip(eager.param_buffers(), graph.param_buffers()):
         assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b))
     graph.free_graph()
+
+
+def test_fused_gcn_step_with_an_edge_plan_replays_from_an_execution_graph(hip):
+    from zigrad_amd.trainers import GCNTrainer, gcn_inputs
+
+    inp = gcn_inputs(n_nodes=500, n_features=200, n_pairs=1500, n_train=40, hidden=16, seed=3)
+    eager, graph = GCNTrainer(hip, inp, fused=True), GCNTrainer(hip, inp, fused=True)
+    graph.step()
+    eager.step()
+    graph.capture()
+    for _ in range(4):
+        assert eager.step() == graph.step_graph()
+        hip.sync()
+    for a, b in zip(eager.param_buffers(), graph.param_buffers()):
+        assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b))
+    graph.free_graph()

@@ -376,11 +376,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // pinned with sched_barrier (left alone, the scheduler sinks every load next to its use):
     //   group 0: global loads of tile t+2, fragment reads of group 1, LDS writes of tile t+1; then the barrier
     //   group 1: fragment reads of group 0 of tile t+1
-    // Every tile runs the same code, the last ones included: past the end of k the fast kernels repeat the loads
-    // of the last tile (in bounds, never consumed), the checked kernels load zeros, and the LDS writes and the
-    // barrier still happen.  One loop body without peeled
-    // tails keeps the accumulators in one place.  The tile's parity is a template argument, so all LDS
-    // addresses are immediates.
+    // Every tile runs the same code, the last ones included: past the end of k the fast and edge kernels repeat the
+    // loads of the last tile, the checked kernels load zeros, and the LDS writes and the barrier still happen.  One
+    // loop body without peeled tails keeps the accumulators in one place.  The tile's parity is a template
+    // argument, so all LDS addresses are immediates.  The masking variant of the step (second template flag) is the
+    // same instruction stream with bounded loads and k-masked LDS writes; it only runs for the last two pairs of
+    // steps of a ragged k range.
     constexpr int E0 = NL + NR + NL;
     constexpr int PER0 = (E0 + NMF - 1) / NMF;
     constexpr int PER1 = (NR + (NMF + 1) / 2 - 1) / ((NMF + 1) / 2);  // reads land in the first half of group 1
@@ -443,8 +444,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     for (int n = 0; n < NR; n++) read_op(0, n, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 
-    // Tiles go in pairs so that the loop body is one straight run of MFMAs.  The fast kernels are only used for
-    // an even number of tiles; in the checked kernels a tile past the end of k loads as zeros and adds nothing.
+    // Tiles go in pairs so that the loop body is one straight run of MFMAs.  A tile past the end of k adds nothing:
+    // the masking steps zero it on its way into LDS, the checked kernels load it as zeros.
     const unsigned kt_plain = !ragged_k ? KT : (KT > 4 ? ((KT + 1) & ~1u) - 4 : 0);
     unsigned kt = 0;
     for (; kt < kt_plain; kt += 2) {

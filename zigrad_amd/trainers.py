@@ -141,7 +141,6 @@ class GraphSteps:
     recorded once as an execution graph (src/device/cuda_device.zig:558-611) and replayed with one launch."""
 
     graph = None
-    graph_loss = None
     _capturing = False
 
     _loss_pinned = None

@@ -9,7 +9,6 @@ from __future__ import annotations
 
 import math
 
-import numpy as np
 
 from .device import DevBuf, F32, U64
 

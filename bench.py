@@ -233,13 +233,13 @@ def timed_steps(dev, step_fn, steps):
 
 
 def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3, graph=False,
-            late_read=False, fused=False):
+            late_read=False, fused=False, clip=True):
     """Returns (seconds, last loss) for `steps` eager steps; with graph=True also the same for `steps` replays of
     the step recorded as an execution graph (the loss is read back every step in both modes)."""
     from zigrad_amd.trainers import MLPTrainer, mlp_inputs
 
     params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data=data)
-    tr = MLPTrainer(dev, dims, batch, optimizer=optimizer, lr=lr, clip=True, loss_mode=loss_mode, fused=fused)
+    tr = MLPTrainer(dev, dims, batch, optimizer=optimizer, lr=lr, clip=clip, loss_mode=loss_mode, fused=fused)
     tr.load_params(params)
     tr.set_batch(x, onehot, labels)
     for _ in range(warmup):
@@ -457,6 +457,10 @@ def main():
             fs = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=True, fused=True)
             result["mlp_b64"]["fused"] = {"steps_per_s": 200 / fs[0], "ms_per_step": fs[0] / 200 * 1e3,
                                                  "graph_replay": {"steps_per_s": 200 / fs[2], "ms_per_step": fs[2] / 200 * 1e3}}
+            # the example itself switches the gradient clip off (examples/mnist/src/main-simple.zig:29-34)
+            nc = run_mlp(dev, [784, 128, 64, 10], 64, "sgd", 200, 20, "uniform", None, "onehot", lr=0.01, graph=True, clip=False)
+            result["mlp_b64"]["clip_off"] = {"steps_per_s": 200 / nc[0], "ms_per_step": nc[0] / 200 * 1e3,
+                                             "graph_replay": {"steps_per_s": 200 / nc[2], "ms_per_step": nc[2] / 200 * 1e3}}
         result["mlp_b64"]["c_caller"] = run_c_harness([784, 128, 64, 10], 64, 2000)
         result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
         result["gcn"] = run_small(dev, "gcn", 100, graph=not args.no_graph)

@@ -143,7 +143,7 @@ def test_unary_inplace_and_empty(oracle, hip):
 # ----------------------------------------------------------------------------------------------
 # BLAS level 1 style ops and flat reductions
 # ----------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("n", [1, 5, 1000, 65536, 65537, 1 << 20, (1 << 22) + 13])
+@pytest.mark.parametrize("n", [1, 5, 1000, 65536, 65537, 131072, 131073, 1 << 20, (1 << 22) + 13])
 def test_flat_reductions(oracle, hip, n):
     r = rng(n)
     x = r.standard_normal(n).astype(np.float32)

@@ -358,12 +358,12 @@ def run_c_harness(dims, batch, steps):
     return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": "eager, same op sequence, caller in C"}
 
 
-def cpu_baseline(dims, batch, budget_steps=2):
-    """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share."""
+def cpu_baseline(dims, batch, budget_steps=2, threads=None):
+    """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share (or `threads`)."""
     from oracle.oracle_device import OracleDevice
 
     odev = OracleDevice()
-    cores = min(16, os.cpu_count() or 1)
+    cores = threads or min(16, os.cpu_count() or 1)
     cores = odev.set_threads(cores)
     dt, _ = run_mlp(odev, dims, batch, "adam", steps=budget_steps, warmup=1, data="normal")
     return {
@@ -473,6 +473,7 @@ def main():
         result["ops"] = op_suite(dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH)
+        result["cpu_baseline_1_thread"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH, budget_steps=1, threads=1)
         # the same CPU oracle on the batch-64 MLP, the configuration the reference runs today
         from oracle.oracle_device import OracleDevice
 

@@ -591,6 +591,7 @@ class GCNTrainer(GraphSteps):
         self.src, self.tgt = self.edge_index.sub(0, self.E), self.edge_index.sub(self.E, self.E)
         # fused: the edge list is the dataset's and never changes, so its segment plans are built once
         self.plan = d.edge_plan(self.src, self.tgt, self.N) if fused else None
+        self._deg_norm = None
         self.label_m = d.from_numpy(inp["onehot"][: self.n_train])
         self._init_loss_slot()
         self.last_grads = None
@@ -601,11 +602,13 @@ class GCNTrainer(GraphSteps):
     def grad_buffers(self):
         return [self.Wg[0], self.bg[0], self.Wg[1], self.bg[1]]
 
-    def _conv_forward(self, l, x_in):
+    def _degree_norm(self) -> DevBuf:
+        """deg^-1/2 with deg = 1 + in-degree, as GraphConvLayer.forward computes it on every call
+        (examples/gcn/src/model.zig:116-224).  With an edge plan the graph is known not to change, so the fused
+        trainer computes it once (during its first, eager step) and every layer reads that one buffer."""
         d, N, E = self.dev, self.N, self.E
-        fan_in, fan_out = self.dims[l], self.dims[l + 1]
-        h = d.mem_cache_alloc(F32, N * fan_out)
-        host.bmm_acc_(d, x_in, [N, fan_in], self.W[l], [fan_out, fan_in], h, trans_a=False, trans_b=True)
+        if self._deg_norm is not None:
+            return self._deg_norm
         deg = d.mem_cache_alloc(F32, N)
         d.mem_fill(deg, 1.0)
         ones_edges = d.mem_cache_alloc(F32, E)
@@ -622,6 +625,19 @@ class GCNTrainer(GraphSteps):
         deg_norm = d.mem_cache_alloc(F32, N)
         d.dispatch("rsqrt_fwd", x=deg, y=deg_norm, eps=self.EPS)
         d.mem_cache_free(deg)
+        if self.plan is not None:
+            self._deg_norm = d.mem_alloc(F32, N)
+            d.mem_copy(deg_norm, self._deg_norm)
+            d.mem_cache_free(deg_norm)
+            return self._deg_norm
+        return deg_norm
+
+    def _conv_forward(self, l, x_in):
+        d, N, E = self.dev, self.N, self.E
+        fan_in, fan_out = self.dims[l], self.dims[l + 1]
+        h = d.mem_cache_alloc(F32, N * fan_out)
+        host.bmm_acc_(d, x_in, [N, fan_in], self.W[l], [fan_out, fan_in], h, trans_a=False, trans_b=True)
+        deg_norm = self._degree_norm()
         y = d.mem_cache_alloc(F32, N * fan_out)
         d.mem_fill(y, 0.0)
         if self.plan is not None:
@@ -649,7 +665,8 @@ class GCNTrainer(GraphSteps):
         d.mem_cache_free(g_y)
         d.mem_cache_free(saved["y"])
         d.mem_cache_free(g_deg)  # deg itself needs no gradient: the chain stops at rsqrt (src/ndtensor.zig:1009)
-        d.mem_cache_free(saved["deg"])
+        if saved["deg"] is not self._deg_norm:
+            d.mem_cache_free(saved["deg"])
         g_x = None
         if need_input_grad:
             g_x = d.mem_cache_alloc(F32, N * fan_in)

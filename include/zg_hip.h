@@ -233,12 +233,16 @@ typedef struct zg_hip_edge_plan zg_hip_edge_plan;
 int zg_hip_edge_plan_create(zg_hip_ctx *ctx, const uint64_t *src_indices, const uint64_t *tgt_indices, size_t n_edge,
                             size_t n_nodes, zg_hip_edge_plan **out);
 int zg_hip_edge_plan_free(zg_hip_ctx *ctx, zg_hip_edge_plan *plan);
-int zg_hip_scatter_add_planned(zg_hip_ctx *ctx, const float *src, const zg_hip_edge_plan *plan, float *dst);
+/* accumulate != 0: add into the outputs, as the unplanned ops do; accumulate == 0: the outputs are written (every
+ * element, zeros where no edge arrives), so the caller needs no zero fill.  grad_deg may be null when the degrees need
+ * no gradient (they are data of the graph; the reference's chain stops there too, src/ndtensor.zig:1009). */
+int zg_hip_scatter_add_planned(zg_hip_ctx *ctx, const float *src, const zg_hip_edge_plan *plan, float *dst,
+                               int accumulate);
 int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx *ctx, float *dst, const float *h, const float *deg,
-                                          const zg_hip_edge_plan *plan, size_t stride);
+                                          const zg_hip_edge_plan *plan, size_t stride, int accumulate);
 int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx *ctx, const float *grad_output, const float *h,
                                               const float *deg, const zg_hip_edge_plan *plan, float *grad_h,
-                                              float *grad_deg, size_t stride);
+                                              float *grad_deg, size_t stride, int accumulate);
 
 /* ---------------------------------------------------------------------------------------------
  * losses: the host loops of src/nn/loss.zig:94-305 as device ops (new op names; the reference

@@ -186,17 +186,30 @@ class OracleDevice(HipDevice):
 
         return EdgePlan(self, None, src_indices, tgt_indices, n_nodes)
 
-    def _op_scatter_add_planned(self, src, plan, dst):
+    def _op_scatter_add_planned(self, src, plan, dst, accumulate=True):
+        if not accumulate:
+            self.mem_fill(dst, 0.0)
         self.dispatch("scatter_add", src=src, offsets=plan.tgt_indices, dst=dst)
 
-    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride):
+    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride, accumulate=True):
+        if not accumulate:
+            self.mem_fill(dst, 0.0)
         self.dispatch("scatter_gcn_deg_scaled", dst=dst, h=h, deg=deg, src_indices=plan.src_indices,
                       tgt_indices=plan.tgt_indices, stride=stride, n_edge=plan.src_indices.n)
 
-    def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride):
+    def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride, accumulate=True):
+        unused = grad_deg is None
+        if unused:
+            grad_deg = self.mem_alloc(grad_h.dtype, plan.n_nodes)
+        if not accumulate or unused:
+            self.mem_fill(grad_deg, 0.0)
+        if not accumulate:
+            self.mem_fill(grad_h, 0.0)
         self.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=grad_output, h=h, deg=deg, src_indices=plan.src_indices,
                       tgt_indices=plan.tgt_indices, grad_h=grad_h, grad_deg=grad_deg, stride=stride,
                       n_edge=plan.src_indices.n)
+        if unused:
+            self.mem_free(grad_deg)
 
     # -- the list entry points are the per-tensor ops in a loop --------------------------------------------
     def _op_sgd_step_multi(self, params, grads, lr, clip, max_norm, delta, zero_grads):

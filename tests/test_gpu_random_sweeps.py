@@ -240,6 +240,30 @@ def test_planned_scatter_ops_equal_the_unplanned_ones(oracle, hip, n_nodes, n_ed
                                                              "tgt_indices": tgt, "grad_h": gh0.copy(), "grad_deg": gd0.copy(),
                                                              "stride": stride, "n_edge": n_edge}, ["grad_h", "grad_deg"])
         assert np.array_equal(got["grad_h"], want["grad_h"]) and np.array_equal(got["grad_deg"], want["grad_deg"]), rep
+        # written instead of accumulated: outputs start as NaN and must come out as if they had started as zeros
+        # (every element, also where no edge arrives); the degree gradient may be left out
+        nan_n, nan_ns = np.full(n_nodes, np.nan, np.float32), np.full(n_nodes * stride, np.nan, np.float32)
+        got = run_op(hip, "scatter_add_planned", {"src": vals, "plan": plan, "dst": nan_n.copy(), "accumulate": False}, ["dst"])["dst"]
+        want = run_op(oracle, "scatter_add", {"src": vals, "offsets": tgt, "dst": np.zeros(n_nodes, np.float32)}, ["dst"])["dst"]
+        assert np.array_equal(got, want), (rep, "scatter_add fresh")
+        got = run_op(hip, "scatter_gcn_deg_scaled_planned", {"dst": nan_ns.copy(), "h": h, "deg": deg, "plan": plan,
+                                                              "stride": stride, "accumulate": False}, ["dst"])["dst"]
+        want = run_op(oracle, "scatter_gcn_deg_scaled", {"dst": np.zeros(n_nodes * stride, np.float32), "h": h, "deg": deg,
+                                                         "src_indices": src, "tgt_indices": tgt, "stride": stride,
+                                                         "n_edge": n_edge}, ["dst"])["dst"]
+        assert np.array_equal(got, want), (rep, "fwd fresh")
+        want = run_op(oracle, "scatter_gcn_deg_scaled_bwd", {"grad_output": go, "h": h, "deg": deg, "src_indices": src,
+                                                             "tgt_indices": tgt, "grad_h": np.zeros(n_nodes * stride, np.float32),
+                                                             "grad_deg": np.zeros(n_nodes, np.float32), "stride": stride,
+                                                             "n_edge": n_edge}, ["grad_h", "grad_deg"])
+        got = run_op(hip, "scatter_gcn_deg_scaled_bwd_planned", {"grad_output": go, "h": h, "deg": deg, "plan": plan,
+                                                                  "grad_h": nan_ns.copy(), "grad_deg": nan_n.copy(),
+                                                                  "stride": stride, "accumulate": False}, ["grad_h", "grad_deg"])
+        assert np.array_equal(got["grad_h"], want["grad_h"]) and np.array_equal(got["grad_deg"], want["grad_deg"]), rep
+        got = run_op(hip, "scatter_gcn_deg_scaled_bwd_planned", {"grad_output": go, "h": h, "deg": deg, "plan": plan,
+                                                                  "grad_h": nan_ns.copy(), "grad_deg": None, "stride": stride,
+                                                                  "accumulate": False}, ["grad_h"])
+        assert np.array_equal(got["grad_h"], want["grad_h"]), (rep, "no degree gradient")
     plan.free()
     hip.mem_free(s_buf)
     hip.mem_free(t_buf)

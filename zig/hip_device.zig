@@ -491,15 +491,16 @@ pub const EdgePlan = struct {
 };
 pub fn scatter_add_planned(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
-    check(c.zg_hip_scatter_add_planned(self.ctx, p.src.ptr, p.plan.plan, p.dst.ptr));
+    check(c.zg_hip_scatter_add_planned(self.ctx, p.src.ptr, p.plan.plan, p.dst.ptr, @intFromBool(p.accumulate)));
 }
 pub fn scatter_gcn_deg_scaled_planned(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
-    check(c.zg_hip_scatter_gcn_deg_scaled_planned(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.stride));
+    check(c.zg_hip_scatter_gcn_deg_scaled_planned(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.stride, @intFromBool(p.accumulate)));
 }
 pub fn scatter_gcn_deg_scaled_bwd_planned(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
-    check(c.zg_hip_scatter_gcn_deg_scaled_bwd_planned(self.ctx, p.grad_output.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.grad_h.ptr, p.grad_deg.ptr, p.stride));
+    const gd: ?[*]T = if (p.grad_deg) |g| g.ptr else null; // optional: the degrees are data of the graph
+    check(c.zg_hip_scatter_gcn_deg_scaled_bwd_planned(self.ctx, p.grad_output.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.grad_h.ptr, gd, p.stride, @intFromBool(p.accumulate)));
 }
 
 /// A Linear layer's forward in one launch: y = act(x . w^T + bias), the arithmetic of `bmm_acc(trans_b)` +

@@ -246,13 +246,17 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
 // ------------------------------------------------------------------------------------------------
 
 // dst[b] += src[e] for the bucket's entries in input order; one thread per destination
+// `fresh`: dst is write-only (treated as zero on entry), so the caller needs no zero fill
 __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_ptr, const uint32_t* perm, float* dst,
-                                         size_t nb) {
+                                         size_t nb, bool fresh) {
     size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nb) return;
     const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
-    if (s == e) return;
-    float acc = dst[b];
+    if (s == e) {
+        if (fresh) dst[b] = 0.f;
+        return;
+    }
+    float acc = fresh ? 0.f : dst[b];
     for (uint32_t k = s; k < e; k++) acc = __fadd_rn(acc, src[perm[k]]);
     dst[b] = acc;
 }
@@ -281,15 +285,19 @@ __global__ __launch_bounds__(256) void row_scatter_apply_kernel(const float* src
 template <int G>
 __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const float* h, const float* deg,
                                                              const uint32_t* row_ptr, const uint32_t* peer,
-                                                             size_t n_nodes, size_t stride) {
+                                                             size_t n_nodes, size_t stride, bool fresh) {
     const size_t t = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     if (t >= n_nodes) return;
     const int lane = threadIdx.x % G;
     const uint32_t s0 = row_ptr[t], s1 = row_ptr[t + 1];
-    if (s0 == s1) return;
+    if (s0 == s1) {
+        if (fresh)
+            for (size_t j = lane; j < stride; j += G) dst[t * stride + j] = 0.f;
+        return;
+    }
     const float dt = deg[t];
     for (size_t j = lane; j < stride; j += G) {
-        float acc = dst[t * stride + j];
+        float acc = fresh ? 0.f : dst[t * stride + j];
         for (uint32_t k = s0; k < s1; k += 4) {
             uint32_t sv[4];
             float dv[4], hv[4];
@@ -313,15 +321,19 @@ __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const fl
 template <int G>
 __global__ __launch_bounds__(256) void gcn_bwd_gradh_kernel(float* grad_h, const float* go, const float* deg,
                                                              const uint32_t* row_ptr, const uint32_t* peer,
-                                                             size_t n_nodes, size_t stride) {
+                                                             size_t n_nodes, size_t stride, bool fresh) {
     const size_t s = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     if (s >= n_nodes) return;
     const int lane = threadIdx.x % G;
     const uint32_t s0 = row_ptr[s], s1 = row_ptr[s + 1];
-    if (s0 == s1) return;
+    if (s0 == s1) {
+        if (fresh)
+            for (size_t j = lane; j < stride; j += G) grad_h[s * stride + j] = 0.f;
+        return;
+    }
     const float ds = deg[s];
     for (size_t j = lane; j < stride; j += G) {
-        float acc = grad_h[s * stride + j];
+        float acc = fresh ? 0.f : grad_h[s * stride + j];
         for (uint32_t k = s0; k < s1; k += 4) {
             uint32_t tv[4];
             float dv[4], gv[4];
@@ -364,12 +376,15 @@ __global__ void gcn_bwd_edge_terms_kernel(const float* go, const float* h, const
 // grad_deg[v] += terms of the edges touching v, merged in edge order (an edge v->v adds its source term first)
 __global__ void gcn_bwd_graddeg_kernel(float* grad_deg, const float* term_src, const float* term_tgt,
                                        const uint32_t* rp_src, const uint32_t* perm_src, const uint32_t* rp_tgt,
-                                       const uint32_t* perm_tgt, size_t n_nodes) {
+                                       const uint32_t* perm_tgt, size_t n_nodes, bool fresh) {
     size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (v >= n_nodes) return;
     uint32_t a = rp_src[v], a1 = rp_src[v + 1], b = rp_tgt[v], b1 = rp_tgt[v + 1];
-    if (a == a1 && b == b1) return;
-    float acc = grad_deg[v];
+    if (a == a1 && b == b1) {
+        if (fresh) grad_deg[v] = 0.f;
+        return;
+    }
+    float acc = fresh ? 0.f : grad_deg[v];
     while (a < a1 || b < b1) {
         const uint32_t ea = (a < a1) ? perm_src[a] : 0xffffffffu;
         const uint32_t eb = (b < b1) ? perm_tgt[b] : 0xffffffffu;
@@ -503,7 +518,7 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
     Plan pl = carve_plan(mem, n, dst_len);
     if (int rc = build_plan(ctx, offsets, pl)) return rc;
     hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(dst_len, 256)), dim3(256), 0, ctx->stream,
-                       src, pl.row_ptr, pl.perm, dst, dst_len);
+                       src, pl.row_ptr, pl.perm, dst, dst_len, false);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
@@ -563,7 +578,7 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const floa
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
-                                        pl.row_ptr, pl.peer, n_nodes, stride));
+                                        pl.row_ptr, pl.peer, n_nodes, stride, false));
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
@@ -590,13 +605,14 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
-                                        grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride));
+                                        grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride, false));
     ZG_LAUNCH_CHECK();
     hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
                        grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride, term_src, term_tgt);
     ZG_LAUNCH_CHECK();
     hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
-                       grad_deg, term_src, term_tgt, by_src.row_ptr, by_src.perm, by_tgt.row_ptr, by_tgt.perm, n_nodes);
+                       grad_deg, term_src, term_tgt, by_src.row_ptr, by_src.perm, by_tgt.row_ptr, by_tgt.perm, n_nodes,
+                       false);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
@@ -659,17 +675,18 @@ ZG_API int zg_hip_edge_plan_free(zg_hip_ctx* ctx, zg_hip_edge_plan* plan) {
 }
 
 // dst[tgt[e]] += src[e] in edge order (zg_hip_scatter_add with offsets = the plan's targets)
-ZG_API int zg_hip_scatter_add_planned(zg_hip_ctx* ctx, const float* src, const zg_hip_edge_plan* plan, float* dst) {
+ZG_API int zg_hip_scatter_add_planned(zg_hip_ctx* ctx, const float* src, const zg_hip_edge_plan* plan, float* dst,
+                                      int accumulate) {
     ZG_CTX(ctx);
     ZG_REQUIRE(plan && src && dst, "scatter_add_planned: null pointer");
     hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(plan->n_nodes, 256)), dim3(256), 0,
-                       ctx->stream, src, plan->by_tgt.row_ptr, plan->by_tgt.perm, dst, plan->n_nodes);
+                       ctx->stream, src, plan->by_tgt.row_ptr, plan->by_tgt.perm, dst, plan->n_nodes, accumulate == 0);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
 
 ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,
-                                                 const zg_hip_edge_plan* plan, size_t stride) {
+                                                 const zg_hip_edge_plan* plan, size_t stride, int accumulate) {
     ZG_CTX(ctx);
     ZG_REQUIRE(plan && dst && h && deg, "scatter_gcn_deg_scaled_planned: null pointer");
     ZG_REQUIRE(stride > 0, "scatter_gcn_deg_scaled_planned: stride is 0");
@@ -677,16 +694,17 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, co
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
-                                        plan->by_tgt.row_ptr, plan->by_tgt.peer, n_nodes, stride));
+                                        plan->by_tgt.row_ptr, plan->by_tgt.peer, n_nodes, stride, accumulate == 0));
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
 
 ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx* ctx, const float* grad_output, const float* h,
                                                      const float* deg, const zg_hip_edge_plan* plan, float* grad_h,
-                                                     float* grad_deg, size_t stride) {
+                                                     float* grad_deg, size_t stride, int accumulate) {
     ZG_CTX(ctx);
-    ZG_REQUIRE(plan && grad_output && h && deg && grad_h && grad_deg, "scatter_gcn_deg_scaled_bwd_planned: null pointer");
+    ZG_REQUIRE(plan && grad_output && h && deg && grad_h, "scatter_gcn_deg_scaled_bwd_planned: null pointer");
+    const bool fresh = accumulate == 0;
     ZG_REQUIRE(stride > 0, "scatter_gcn_deg_scaled_bwd_planned: stride is 0");
     const size_t n_nodes = plan->n_nodes, n_edge = plan->n_edge;
     const size_t tb = align_up(n_edge * sizeof(float), 256);
@@ -697,14 +715,15 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx* ctx, const floa
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
-                                        grad_output, deg, plan->by_src.row_ptr, plan->by_src.peer, n_nodes, stride));
+                                        grad_output, deg, plan->by_src.row_ptr, plan->by_src.peer, n_nodes, stride, fresh));
     ZG_LAUNCH_CHECK();
+    if (!grad_deg) return ZG_HIP_OK;  // the degrees need no gradient (they are data of the graph)
     hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
                        grad_output, h, deg, plan->src_dev, plan->tgt_dev, n_edge, n_nodes, stride, term_src, term_tgt);
     ZG_LAUNCH_CHECK();
     hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
                        grad_deg, term_src, term_tgt, plan->by_src.row_ptr, plan->by_src.perm, plan->by_tgt.row_ptr,
-                       plan->by_tgt.perm, n_nodes);
+                       plan->by_tgt.perm, n_nodes, fresh);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

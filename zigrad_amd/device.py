@@ -400,15 +400,16 @@ class HipDevice:
         self._call("zg_hip_edge_plan_create", src_indices.ptr, tgt_indices.ptr, src_indices.n, n_nodes, ctypes.byref(h))
         return EdgePlan(self, h, src_indices, tgt_indices, n_nodes)
 
-    def _op_scatter_add_planned(self, src, plan, dst):
-        self._call("zg_hip_scatter_add_planned", src.ptr, plan.handle, dst.ptr)
+    def _op_scatter_add_planned(self, src, plan, dst, accumulate=True):
+        self._call("zg_hip_scatter_add_planned", src.ptr, plan.handle, dst.ptr, int(accumulate))
 
-    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride):
-        self._call("zg_hip_scatter_gcn_deg_scaled_planned", dst.ptr, h.ptr, deg.ptr, plan.handle, stride)
+    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride, accumulate=True):
+        self._call("zg_hip_scatter_gcn_deg_scaled_planned", dst.ptr, h.ptr, deg.ptr, plan.handle, stride, int(accumulate))
 
-    def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride):
+    def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride, accumulate=True):
+        """grad_deg may be None: the degree gradient is then not computed."""
         self._call("zg_hip_scatter_gcn_deg_scaled_bwd_planned", grad_output.ptr, h.ptr, deg.ptr, plan.handle, grad_h.ptr,
-                   grad_deg.ptr, stride)
+                   grad_deg.ptr if grad_deg is not None else None, stride, int(accumulate))
 
     # losses
     def _op_smce_fwd(self, logits, target, probs, loss, rows, cols):

@@ -639,10 +639,11 @@ class GCNTrainer(GraphSteps):
         host.bmm_acc_(d, x_in, [N, fan_in], self.W[l], [fan_out, fan_in], h, trans_a=False, trans_b=True)
         deg_norm = self._degree_norm()
         y = d.mem_cache_alloc(F32, N * fan_out)
-        d.mem_fill(y, 0.0)
-        if self.plan is not None:
-            d.dispatch("scatter_gcn_deg_scaled_planned", dst=y, h=h, deg=deg_norm, plan=self.plan, stride=fan_out)
+        if self.plan is not None:  # written, not accumulated: no zero fill
+            d.dispatch("scatter_gcn_deg_scaled_planned", dst=y, h=h, deg=deg_norm, plan=self.plan, stride=fan_out,
+                       accumulate=False)
         else:
+            d.mem_fill(y, 0.0)
             d.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg_norm, src_indices=self.src, tgt_indices=self.tgt,
                        stride=fan_out, n_edge=E)
         d.dispatch("add", x=self.b[l], y=y, z=y)  # y._add(bias)
@@ -653,18 +654,20 @@ class GCNTrainer(GraphSteps):
         fan_in, fan_out = self.dims[l], self.dims[l + 1]
         host.unbroadcast_(d, g_y, [N, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
         g_h = d.mem_cache_alloc(F32, N * fan_out)
-        d.mem_fill(g_h, 0.0)
-        g_deg = d.mem_cache_alloc(F32, N)
-        d.mem_fill(g_deg, 0.0)
         if self.plan is not None:
+            # written, not accumulated (no zero fill), and without the degree gradient, which nobody reads: the
+            # chain stops at rsqrt (src/ndtensor.zig:1009) and the degrees are data of the graph
             d.dispatch("scatter_gcn_deg_scaled_bwd_planned", grad_output=g_y, h=saved["h"], deg=saved["deg"], plan=self.plan,
-                       grad_h=g_h, grad_deg=g_deg, stride=fan_out)
+                       grad_h=g_h, grad_deg=None, stride=fan_out, accumulate=False)
         else:
+            d.mem_fill(g_h, 0.0)
+            g_deg = d.mem_cache_alloc(F32, N)
+            d.mem_fill(g_deg, 0.0)
             d.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=g_y, h=saved["h"], deg=saved["deg"], src_indices=self.src,
                        tgt_indices=self.tgt, grad_h=g_h, grad_deg=g_deg, stride=fan_out, n_edge=E)
+            d.mem_cache_free(g_deg)  # deg itself needs no gradient: the chain stops at rsqrt (src/ndtensor.zig:1009)
         d.mem_cache_free(g_y)
         d.mem_cache_free(saved["y"])
-        d.mem_cache_free(g_deg)  # deg itself needs no gradient: the chain stops at rsqrt (src/ndtensor.zig:1009)
         if saved["deg"] is not self._deg_norm:
             d.mem_cache_free(saved["deg"])
         g_x = None

@@ -93,6 +93,43 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float*
     }
 }
 
+// The update loop of the one-workgroup kernels: four independent elements in flight per thread (the loop is latency
+// bound: one element per trip cost a memory round trip each), same arithmetic per element as sgd_kernel / adam_kernel.
+template <bool ADAM>
+__device__ __forceinline__ void update_in_workgroup(float* p, float* g, float* m, float* v, size_t n, bool scale, float f,
+                                                    float lr_t, float b1, float b2, float omb1, float omb2, float eps,
+                                                    bool zero_grads) {
+    const size_t nt = blockDim.x;
+    for (size_t base = threadIdx.x; base < n; base += 4 * nt) {
+        float gv[4], pv[4], mv[4], vv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const size_t i = base + (size_t)u * nt;
+            const bool ok = i < n;
+            gv[u] = ok ? g[i] : 0.f;
+            pv[u] = ok ? p[i] : 0.f;
+            mv[u] = (ADAM && ok) ? m[i] : 0.f;
+            vv[u] = (ADAM && ok) ? v[i] : 1.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const size_t i = base + (size_t)u * nt;
+            if (i >= n) continue;
+            if (ADAM) {
+                adam_elem(pv[u], gv[u], mv[u], vv[u], scale, f, lr_t, b1, b2, omb1, omb2, eps);
+                m[i] = mv[u];
+                v[i] = vv[u];
+                p[i] = pv[u];
+            } else {
+                if (scale) gv[u] = __fmul_rn(gv[u], f);
+                p[i] = __fadd_rn(pv[u], __fmul_rn(lr_t, gv[u]));
+            }
+            if (zero_grads) g[i] = 0.f;
+            else if (scale) g[i] = gv[u];
+        }
+    }
+}
+
 // Small tensors with the gradient clip on: one workgroup computes the norm exactly as flat_single_kernel does (same
 // per-thread accumulation and the same combine tree), publishes the clip factor, and goes on to the update.
 // One launch instead of two; the arithmetic per element is that of sgd_kernel / adam_kernel, so the values are
@@ -116,23 +153,7 @@ __global__ __launch_bounds__(kFlatSingle) void clipped_update_small_kernel(float
     const float f = factor_s;
     const bool scale = f != 1.0f;
     const float lr_t = (ADAM && lr_t_ptr) ? lr_t_ptr[0] : step_scale;  // SGD: step_scale = -lr
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
-        float gv = g[i];
-        if (ADAM) {
-            float pv = p[i], mv = m[i], vv = v[i];
-            adam_elem(pv, gv, mv, vv, scale, f, lr_t, b1, b2, omb1, omb2, eps);
-            if (scale) g[i] = gv;
-            m[i] = mv;
-            v[i] = vv;
-            p[i] = pv;
-        } else {
-            if (scale) {
-                gv = __fmul_rn(gv, f);
-                g[i] = gv;
-            }
-            p[i] = __fadd_rn(p[i], __fmul_rn(lr_t, gv));
-        }
-    }
+    update_in_workgroup<ADAM>(p, g, m, v, n, scale, f, lr_t, b1, b2, omb1, omb2, eps, false);
 }
 
 // The same update for up to kMultiMax small tensors in one launch: workgroup b does what
@@ -172,21 +193,7 @@ __global__ __launch_bounds__(kFlatSingle) void update_multi_kernel(MultiArgs a) 
     }
     const bool scale = f != 1.0f;
     const float lr_t = (ADAM && a.lr_t_mem) ? a.lr_t_mem[b] : a.lr_t[b];
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
-        float gv = g[i];
-        if (ADAM) {
-            float pv = p[i], mv = m[i], vv = v[i];
-            adam_elem(pv, gv, mv, vv, scale, f, lr_t, a.b1, a.b2, a.omb1, a.omb2, a.eps);
-            m[i] = mv;
-            v[i] = vv;
-            p[i] = pv;
-        } else {
-            if (scale) gv = __fmul_rn(gv, f);
-            p[i] = __fadd_rn(p[i], __fmul_rn(lr_t, gv));
-        }
-        if (a.zero_grads) g[i] = 0.f;
-        else if (scale) g[i] = gv;
-    }
+    update_in_workgroup<ADAM>(p, g, m, v, n, scale, f, lr_t, a.b1, a.b2, a.omb1, a.omb2, a.eps, a.zero_grads != 0);
 }
 
 static int update_grid(zg_hip_ctx* ctx, size_t n) {

@@ -222,6 +222,14 @@ int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx *ctx, const float *grad_output,
                                       const uint64_t *src_indices, const uint64_t *tgt_indices, float *grad_h,
                                       float *grad_deg, size_t stride, size_t n_edge, size_t n_nodes);
 
+/* CSR forms (src/device/host_device.zig:1325-1353).  scatter_add_csr: dst[j] += src[i] for j in [row_ptr[i],
+ * row_ptr[i + 1]), row_ptr non-decreasing with n_segments + 1 entries.  segment_sum_csr: dst[i] = the sum of
+ * src[row_offsets[i] .. row_offsets[i + 1]) (written, not accumulated). */
+int zg_hip_scatter_add_csr(zg_hip_ctx *ctx, const float *src, const uint64_t *row_ptr, size_t n_segments, float *dst,
+                           size_t dst_len);
+int zg_hip_segment_sum_csr(zg_hip_ctx *ctx, const float *src, size_t src_len, const uint64_t *row_offsets,
+                           size_t n_segments, float *dst);
+
 /* Edge plans.  The three ops above sort the edge list by destination on every call, because the reference hands
  * them bare index slices (examples/gcn/src/model.zig:116-224 builds them per forward).  For an edge list that does
  * not change between calls (the dataset's graph, examples/gcn/src/dataset.zig:110-127) the analysis can be done

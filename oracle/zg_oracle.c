@@ -779,6 +779,24 @@ int zo_gather_offsets(const uint64_t *src_shape, const uint64_t *idx_shape, size
 }
 
 /* src/device/host_device.zig:1039-1087: dst[offsets[i]] += src[i], in index order */
+/* src/device/host_device.zig:1325-1335 */
+void zo_scatter_add_csr(const float *src, const uint64_t *row_ptr, size_t n_segments, float *dst, size_t dst_len) {
+    for (size_t i = 0; i < n_segments; i++) {
+        const float value = src[i];
+        for (uint64_t j = row_ptr[i]; j < row_ptr[i + 1] && j < dst_len; j++) dst[j] += value;
+    }
+}
+
+/* src/device/host_device.zig:1337-1353; the host sums each segment in SIMD lanes (vsum_contig), here sequentially:
+ * the order is not pinned by the reference */
+void zo_segment_sum_csr(const float *src, size_t src_len, const uint64_t *row_offsets, size_t n_segments, float *dst) {
+    for (size_t i = 0; i < n_segments; i++) {
+        float s = 0.0f;
+        for (uint64_t j = row_offsets[i]; j < row_offsets[i + 1] && j < src_len; j++) s += src[j];
+        dst[i] = s;
+    }
+}
+
 void zo_scatter_add(const float *src, const uint64_t *offsets, size_t n, float *dst, size_t dst_len) {
     (void)dst_len;
     for (size_t i = 0; i < n; i++) dst[offsets[i]] += src[i];

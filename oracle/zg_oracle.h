@@ -107,6 +107,8 @@ void zo_mem_random(float *x, size_t n, int kind, uint64_t fan, uint64_t seed);
 int zo_gather_offsets(const uint64_t *src_shape, const uint64_t *idx_shape, size_t rank, const uint64_t *indices,
                       size_t dim, uint64_t *offsets);
 void zo_scatter_add(const float *src, const uint64_t *offsets, size_t n, float *dst, size_t dst_len);
+void zo_scatter_add_csr(const float *src, const uint64_t *row_ptr, size_t n_segments, float *dst, size_t dst_len);
+void zo_segment_sum_csr(const float *src, size_t src_len, const uint64_t *row_offsets, size_t n_segments, float *dst);
 void zo_index_select_fwd(const float *src, size_t src_len, const uint64_t *indices, size_t n_idx, size_t stride,
                          float *dst);
 void zo_index_select_bwd(const float *y_grad, const uint64_t *indices, size_t n_idx, size_t stride, float *x_grad,

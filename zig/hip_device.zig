@@ -410,6 +410,14 @@ pub fn scatter_add(self: *const Self, T: type, p: opspec.scatter_add(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_scatter_add(self.ctx, p.src.ptr, @ptrCast(p.offsets.ptr), p.src.len, p.dst.ptr, p.dst.len));
 }
+pub fn scatter_add_csr(self: *const Self, T: type, p: opspec.scatter_add_csr(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_scatter_add_csr(self.ctx, p.src.ptr, @ptrCast(p.row_ptr.ptr), p.src.len, p.dst.ptr, p.dst.len));
+}
+pub fn segment_sum_csr(self: *const Self, T: type, p: opspec.segment_sum_csr(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_segment_sum_csr(self.ctx, p.src.ptr, p.src.len, @ptrCast(p.row_offsets.ptr), p.dst.len, p.dst.ptr));
+}
 pub fn scatter_gcn_deg_scaled(self: *const Self, T: type, p: opspec.scatter_gcn_deg_scaled(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_scatter_gcn_deg_scaled(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, @ptrCast(p.src_indices.ptr), @ptrCast(p.tgt_indices.ptr), p.stride, p.n_edge, p.deg.len));

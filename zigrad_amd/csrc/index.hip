@@ -618,6 +618,70 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
 }
 
 // ------------------------------------------------------------------------------------------------
+// CSR forms (src/device/host_device.zig:1325-1353): segments are given by their boundaries, so no plan is needed.
+// ------------------------------------------------------------------------------------------------
+namespace zg {
+
+// dst[j] += src[i] for j in [row_ptr[i], row_ptr[i + 1]): one wave per segment.  A boundary beyond dst is clipped.
+__global__ __launch_bounds__(256) void scatter_add_csr_kernel(const float* src, const uint64_t* row_ptr, size_t n_seg,
+                                                               float* dst, size_t dst_len) {
+    const size_t i = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n_seg) return;
+    const int lane = threadIdx.x & 63;
+    uint64_t s = row_ptr[i], e = row_ptr[i + 1];
+    if (e > dst_len) e = dst_len;
+    const float v = src[i];
+    for (uint64_t j = s + lane; j < e; j += 64) dst[j] = __fadd_rn(dst[j], v);
+}
+
+// dst[i] = sum of src[row_ptr[i] .. row_ptr[i + 1]): one wave per segment, four loads in flight per lane, lanes
+// combined by a fixed butterfly (the host sums in SIMD lanes: there is no order to match)
+__global__ __launch_bounds__(256) void segment_sum_csr_kernel(const float* src, size_t src_len, const uint64_t* row_ptr,
+                                                               size_t n_seg, float* dst) {
+    const size_t i = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n_seg) return;
+    const int lane = threadIdx.x & 63;
+    uint64_t s = row_ptr[i], e = row_ptr[i + 1];
+    if (e > src_len) e = src_len;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    uint64_t j = s + lane;
+    for (; j + 192 < e; j += 256) {
+        a0 += src[j];
+        a1 += src[j + 64];
+        a2 += src[j + 128];
+        a3 += src[j + 192];
+    }
+    for (; j < e; j += 64) a0 += src[j];
+    float acc = (a0 + a1) + (a2 + a3);
+    for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
+    if (lane == 0) dst[i] = acc;
+}
+
+}  // namespace zg
+
+ZG_API int zg_hip_scatter_add_csr(zg_hip_ctx* ctx, const float* src, const uint64_t* row_ptr, size_t n_segments,
+                                  float* dst, size_t dst_len) {
+    ZG_CTX(ctx);
+    if (n_segments == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(src && row_ptr && dst, "scatter_add_csr: null pointer");
+    hipLaunchKernelGGL(scatter_add_csr_kernel, dim3((unsigned)ceil_div_sz(n_segments, 4)), dim3(256), 0, ctx->stream, src,
+                       row_ptr, n_segments, dst, dst_len);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_segment_sum_csr(zg_hip_ctx* ctx, const float* src, size_t src_len, const uint64_t* row_offsets,
+                                  size_t n_segments, float* dst) {
+    ZG_CTX(ctx);
+    if (n_segments == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(src && row_offsets && dst, "segment_sum_csr: null pointer");
+    hipLaunchKernelGGL(segment_sum_csr_kernel, dim3((unsigned)ceil_div_sz(n_segments, 4)), dim3(256), 0, ctx->stream, src,
+                       src_len, row_offsets, n_segments, dst);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
 // Edge plans: the segment plans of an edge list that does not change between calls (a dataset's graph), built once.
 // The planned ops launch the same apply kernels on the same plans as the ops above, so their results are identical;
 // what they save is the plan construction (five launches per plan, two plans in the backward op).

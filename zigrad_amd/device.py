@@ -379,6 +379,16 @@ class HipDevice:
             raise ValueError("scatter_add: offsets.len != src.len")
         self._call("zg_hip_scatter_add", src.ptr, offsets.ptr, src.n, dst.ptr, dst.n)
 
+    def _op_scatter_add_csr(self, src, row_ptr, dst):
+        if row_ptr.n != src.n + 1:
+            raise ValueError("scatter_add_csr: row_ptr.len != src.len + 1")
+        self._call("zg_hip_scatter_add_csr", src.ptr, row_ptr.ptr, src.n, dst.ptr, dst.n)
+
+    def _op_segment_sum_csr(self, src, row_offsets, dst):
+        if row_offsets.n != dst.n + 1:
+            raise ValueError("segment_sum_csr: row_offsets.len != dst.len + 1")
+        self._call("zg_hip_segment_sum_csr", src.ptr, src.n, row_offsets.ptr, dst.n, dst.ptr)
+
     def _op_index_select_fwd(self, src, indices, stride, dst):
         self._call("zg_hip_index_select_fwd", src.ptr, src.n, indices.ptr, indices.n, stride, dst.ptr)
 

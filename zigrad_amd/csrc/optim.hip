@@ -93,17 +93,18 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float*
     }
 }
 
-// The update loop of the one-workgroup kernels: four independent elements in flight per thread (the loop is latency
+// The update loop of the one-workgroup kernels: eight independent elements in flight per thread (the loop is latency
 // bound: one element per trip cost a memory round trip each), same arithmetic per element as sgd_kernel / adam_kernel.
+constexpr int kInFlight = 8;  // elements per thread and trip
 template <bool ADAM>
 __device__ __forceinline__ void update_in_workgroup(float* p, float* g, float* m, float* v, size_t n, bool scale, float f,
                                                     float lr_t, float b1, float b2, float omb1, float omb2, float eps,
                                                     bool zero_grads) {
     const size_t nt = blockDim.x;
-    for (size_t base = threadIdx.x; base < n; base += 4 * nt) {
-        float gv[4], pv[4], mv[4], vv[4];
+    for (size_t base = threadIdx.x; base < n; base += kInFlight * nt) {
+        float gv[kInFlight], pv[kInFlight], mv[kInFlight], vv[kInFlight];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kInFlight; u++) {
             const size_t i = base + (size_t)u * nt;
             const bool ok = i < n;
             gv[u] = ok ? g[i] : 0.f;
@@ -112,7 +113,7 @@ __device__ __forceinline__ void update_in_workgroup(float* p, float* g, float* m
             vv[u] = (ADAM && ok) ? v[i] : 1.f;
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kInFlight; u++) {
             const size_t i = base + (size_t)u * nt;
             if (i >= n) continue;
             if (ADAM) {

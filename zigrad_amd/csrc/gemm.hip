@@ -11,7 +11,8 @@
 // A wave cannot overlap its own non-MFMA instructions with its MFMAs to any useful degree (measured: every
 // LDS or global instruction in the loop costs about its issue time), so the loop is built to need few of them:
 //   * LDS keeps each operand tile in the orientation it has in HBM ([mn][k] for a k-contiguous operand,
-//     [k][mn] otherwise), so a tile moves HBM -> registers -> LDS with 16-byte loads and 16-byte LDS writes only.
+//     [k][mn] otherwise), so a tile moves HBM -> registers -> LDS with 16-byte loads and 16-byte LDS writes only;
+//     the [mn][k] form is XOR-swizzled, the other padded, so that no LDS access conflicts on banks.
 //   * An MFMA sums over two k values, one per lane half, and it does not matter which two as long as A and B
 //     agree.  Lane half h takes k = 8g + 4h + c in step c of k-group g.  A lane of a k-contiguous operand then
 //     reads its 4 steps of one 32-row block with one ds_read_b128; a lane of the other kind reads, per step,
@@ -51,10 +52,12 @@ struct VecOf<4> {
 // One operand tile: `BMN` rows in the m (or n) direction by kBK along k.
 // KMAJOR: element (mn, k) lives at ptr[mn * ld + k]   (A not transposed, B transposed); LDS holds [mn][k]
 // else  : element (mn, k) lives at ptr[k * ld + mn]   (A transposed, B not transposed); LDS holds [k][mn]
-// The 4-float row padding makes the 16-byte fragment reads of 16 consecutive lanes hit 64 distinct banks.
+// [k][mn] rows carry 4 floats of padding.  [mn][k] rows are 16 floats with no padding; the 16-byte piece kq of row
+// mn sits at column kq ^ ((mn >> 2) & 3), so that both the LDS writes (4 pieces of 4 adjacent rows per 16 lanes) and
+// the fragment reads (one piece of 16 adjacent rows per 16 lanes) touch 64 distinct banks.
 template <int BMN, bool KMAJOR>
 struct Tile {
-    static constexpr int LD = KMAJOR ? kBK + 4 : BMN + 4;            // LDS row stride in floats
+    static constexpr int LD = KMAJOR ? kBK : BMN + 4;                // LDS row stride in floats
     static constexpr int ELEMS = KMAJOR ? BMN * LD : kBK * LD;       // floats per LDS buffer
     static constexpr int NV = BMN * kBK / 4 / kGemmThreads;          // 16-byte pieces per thread
     floatx4 r[NV];
@@ -79,7 +82,7 @@ struct Tile {
     static __device__ __forceinline__ int lds_offset(int i) {
         int mn, k;
         coords(i, mn, k);
-        return KMAJOR ? mn * LD + k : k * LD + mn;
+        return KMAJOR ? mn * LD + (((k >> 2) ^ ((mn >> 2) & 3)) << 2) : k * LD + mn;
     }
 
     // fast path: `base` is the tile origin (uniform), `off` this thread's byte offset of piece i.  A buffer load
@@ -162,13 +165,16 @@ struct Frag {
     static constexpr int N = KMAJOR ? T : 4;  // LDS reads per k-group
     V v[N];
 
-    // this lane's read base inside an LDS buffer: w0 = first row of the wave's slab
-    static __device__ __forceinline__ int lane_base(int w0, int l32, int lk) {
-        return KMAJOR ? (w0 + l32) * Tl::LD + lk * 4 : (lk * 4) * Tl::LD + w0 + l32 * T;
+    // this lane's read base inside an LDS buffer for k-group g: w0 = first row of the wave's slab.  A k-contiguous
+    // tile is swizzled (see Tile), which makes the column of piece 2g + lk a per-lane constant for each g; the other
+    // layout reaches group g through an immediate offset, so its two bases are the same.
+    static __device__ __forceinline__ int lane_base(int w0, int l32, int lk, int g) {
+        const int row = w0 + l32;
+        return KMAJOR ? row * Tl::LD + ((((g << 1) + lk) ^ ((row >> 2) & 3)) << 2) : (lk * 4) * Tl::LD + w0 + l32 * T;
     }
-    // n-th read of k-group g
+    // n-th read of k-group g; lane_ptr = buffer + lane_base(.., g)
     __device__ __forceinline__ void read_op(int n, const float* __restrict__ lane_ptr, int g) {
-        if (KMAJOR) v[n] = *reinterpret_cast<const V*>(lane_ptr + n * 32 * Tl::LD + g * 8);
+        if (KMAJOR) v[n] = *reinterpret_cast<const V*>(lane_ptr + n * 32 * Tl::LD);
         else v[n] = *reinterpret_cast<const V*>(lane_ptr + (g * 8 + n) * Tl::LD);
     }
     // operand of block t in step c
@@ -297,8 +303,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // path) the byte offsets of its pieces from the tile origin in HBM
     float* const a_wr = As0 + TA::lds_offset(0);
     float* const b_wr = Bs0 + TB::lds_offset(0);
-    const float* const a_rd = As0 + FA::lane_base(wm0, l32, lk);
-    const float* const b_rd = Bs0 + FB::lane_base(wn0, l32, lk);
+    const float* const a_rd[2] = {As0 + FA::lane_base(wm0, l32, lk, 0), As0 + FA::lane_base(wm0, l32, lk, 1)};
+    const float* const b_rd[2] = {Bs0 + FB::lane_base(wn0, l32, lk, 0), Bs0 + FB::lane_base(wn0, l32, lk, 1)};
     unsigned a_off[TA::NV], b_off[TB::NV];
 #pragma unroll
     for (int i = 0; i < TA::NV; i++) {
@@ -368,8 +374,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     FA fa[2];
     FB fb[2];
     auto read_op = [&](int set, int n, int buf, int grp) {
-        if (n < FA::N) fa[set].read_op(n, a_rd + buf * TA::ELEMS, grp);
-        else fb[set].read_op(n - FA::N, b_rd + buf * TB::ELEMS, grp);
+        if (n < FA::N) fa[set].read_op(n, a_rd[grp] + buf * TA::ELEMS, grp);
+        else fb[set].read_op(n - FA::N, b_rd[grp] + buf * TB::ELEMS, grp);
     };
 
     // One tile = two k-groups of 4 steps of NM MFMAs.  The other instructions are dealt out behind the MFMAs,

@@ -340,23 +340,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // which covers the HBM latency also when a workgroup has a CU to itself.
     TA ta[2];
     TB tb[2];
+    // Fast / edge kernels address a tile through running tile-origin pointers (a_tile, b_tile) that tile_step moves
+    // along k with scalar adds; the checked kernels address through k0.
+    const float* a_tile = a_org;
+    const float* b_tile = b_org;
+    const size_t a_step = A_KMAJOR ? (size_t)BK : (size_t)BK * g.lda;  // elements between the origins of two tiles
+    const size_t b_step = B_KMAJOR ? (size_t)BK : (size_t)BK * g.ldb;
     auto load_op = [&](auto slot_tag, int v, size_t k0, auto bounded_tag) {
         constexpr int S = decltype(slot_tag)::value;
         constexpr bool BOUNDED = decltype(bounded_tag)::value;  // give the buffer its true size (last tiles only)
         if (v < TA::NV) {
-            if (!SAFE) {
-                const float* base = a_org + (A_KMAJOR ? k0 : k0 * g.lda);
-                ta[S].load_fast(v, base, a_off[v], BOUNDED ? bytes_left(base, a_end) : 0xffffffffu);
-            } else {
-                ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
-            }
+            if (!SAFE) ta[S].load_fast(v, a_tile, a_off[v], BOUNDED ? bytes_left(a_tile, a_end) : 0xffffffffu);
+            else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
         } else {
-            if (!SAFE) {
-                const float* base = b_org + (B_KMAJOR ? k0 : k0 * g.ldb);
-                tb[S].load_fast(v - TA::NV, base, b_off[v - TA::NV], BOUNDED ? bytes_left(base, b_end) : 0xffffffffu);
-            } else {
-                tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
-            }
+            if (!SAFE) tb[S].load_fast(v - TA::NV, b_tile, b_off[v - TA::NV], BOUNDED ? bytes_left(b_tile, b_end) : 0xffffffffu);
+            else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
         }
     };
     // k0: first k of the tile being stored (used by the masking variant only)
@@ -395,7 +393,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         constexpr int S = decltype(parity_tag)::value;  // kt % 2: LDS buffer and register slot of this tile
         using SCur = std::integral_constant<int, S>;
         using SNext = std::integral_constant<int, S ^ 1>;
-        const size_t k_load = k_begin + (size_t)((SAFE || kt + 2 < KT) ? kt + 2 : KT - 1) * BK;
+        // this step loads tile min(kt + 2, KT - 1) (the checked kernels: tile kt + 2, zeros past the end)
+        const size_t k_load = k_begin + (size_t)(kt + 2) * BK;
         const size_t k_store = k_begin + (size_t)(kt + 1) * BK;
 #pragma unroll
         for (int grp = 0; grp < 2; grp++) {
@@ -419,6 +418,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (grp == 0) {
+                if (!SAFE && kt + 3 < KT) {  // the loads of this step are out: move on to the next step's tile
+                    a_tile += a_step;
+                    b_tile += b_step;
+                }
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -430,21 +433,32 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     using Masked = std::true_type;
 
     // prologue: tile 0 goes straight to LDS buffer 0, tile 1 starts its flight in slot 1
+    a_tile += (A_KMAJOR ? k_begin : k_begin * g.lda);
+    b_tile += (B_KMAJOR ? k_begin : k_begin * g.ldb);
+    auto advance = [&](unsigned next_tile) {  // to the origin of tile min(next_tile, KT - 1)
+        if (!SAFE && next_tile < KT) {
+            a_tile += a_step;
+            b_tile += b_step;
+        }
+    };
     if (__builtin_expect(ragged_k, 0)) {
 #pragma unroll
         for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Masked{});
+        advance(1);
 #pragma unroll
-        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + (KT > 1 ? BK : 0), Masked{});
+        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + BK, Masked{});
 #pragma unroll
         for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Masked{});
     } else {
 #pragma unroll
         for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Plain{});
+        advance(1);
 #pragma unroll
-        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0), Plain{});
+        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + BK, Plain{});
 #pragma unroll
         for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Plain{});
     }
+    advance(2);
     __syncthreads();
 #pragma unroll
     for (int n = 0; n < NR; n++) read_op(0, n, 0, 0);

@@ -340,8 +340,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // which covers the HBM latency also when a workgroup has a CU to itself.
     TA ta[2];
     TB tb[2];
-    // Fast / edge kernels address a tile through running tile-origin pointers (a_tile, b_tile) that tile_step moves
-    // along k with scalar adds; the checked kernels address through k0.
+    // Fast / edge kernels: a k-contiguous operand is addressed through a running tile-origin pointer (a_tile, b_tile)
+    // that tile_step moves along k with one scalar add; a strided operand's origin is recomputed from k0 for every
+    // tile.  (Running pointers for the strided operands as well save a few scalar instructions per tile and 0.5 % of
+    // the TN product's time, but its workgroups then drift apart in k and the L2 of each XCD misses 1.6 x as many
+    // bytes: measured 509 -> 790..950 MiB per 4096-cubed product.)  The checked kernels address through k0.
     const float* a_tile = a_org;
     const float* b_tile = b_org;
     const size_t a_step = A_KMAJOR ? (size_t)BK : (size_t)BK * g.lda;  // elements between the origins of two tiles
@@ -350,11 +353,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         constexpr int S = decltype(slot_tag)::value;
         constexpr bool BOUNDED = decltype(bounded_tag)::value;  // give the buffer its true size (last tiles only)
         if (v < TA::NV) {
-            if (!SAFE) ta[S].load_fast(v, a_tile, a_off[v], BOUNDED ? bytes_left(a_tile, a_end) : 0xffffffffu);
-            else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
+            if (!SAFE) {
+                const float* org = A_KMAJOR ? a_tile : a_org + k0 * g.lda;
+                ta[S].load_fast(v, org, a_off[v], BOUNDED ? bytes_left(org, a_end) : 0xffffffffu);
+            } else ta[S].load_safe(v, A, g.lda, m0, k0, g.M, k_end, g.a_vec != 0);
         } else {
-            if (!SAFE) tb[S].load_fast(v - TA::NV, b_tile, b_off[v - TA::NV], BOUNDED ? bytes_left(b_tile, b_end) : 0xffffffffu);
-            else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
+            if (!SAFE) {
+                const float* org = B_KMAJOR ? b_tile : b_org + k0 * g.ldb;
+                tb[S].load_fast(v - TA::NV, org, b_off[v - TA::NV], BOUNDED ? bytes_left(org, b_end) : 0xffffffffu);
+            } else tb[S].load_safe(v - TA::NV, B, g.ldb, n0, k0, g.N, k_end, g.b_vec != 0);
         }
     };
     // k0: first k of the tile being stored (used by the masking variant only)
@@ -394,7 +401,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         using SCur = std::integral_constant<int, S>;
         using SNext = std::integral_constant<int, S ^ 1>;
         // this step loads tile min(kt + 2, KT - 1) (the checked kernels: tile kt + 2, zeros past the end)
-        const size_t k_load = k_begin + (size_t)(kt + 2) * BK;
+        const size_t k_load = k_begin + (size_t)((SAFE || kt + 2 < KT) ? kt + 2 : KT - 1) * BK;
         const size_t k_store = k_begin + (size_t)(kt + 1) * BK;
 #pragma unroll
         for (int grp = 0; grp < 2; grp++) {
@@ -446,7 +453,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Masked{});
         advance(1);
 #pragma unroll
-        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + BK, Masked{});
+        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0), Masked{});
 #pragma unroll
         for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Masked{});
     } else {
@@ -454,7 +461,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         for (int v = 0; v < NL; v++) load_op(P0{}, v, k_begin, Plain{});
         advance(1);
 #pragma unroll
-        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + BK, Plain{});
+        for (int v = 0; v < NL; v++) load_op(P1{}, v, k_begin + ((SAFE || KT > 1) ? BK : 0), Plain{});
 #pragma unroll
         for (int w = 0; w < NL; w++) store_op(P0{}, w, 0, k_begin, Plain{});
     }

@@ -259,6 +259,11 @@ int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx *ctx, const float *grad
 int zg_hip_smce_fwd(zg_hip_ctx *ctx, const float *logits, const float *target, float *probs, float *loss,
                     size_t rows, size_t cols);
 int zg_hip_smce_bwd(zg_hip_ctx *ctx, const float *probs, const float *target, float *grad, size_t rows, size_t cols);
+/* smce_fwd followed by the loss's backward with upstream gradient 1 (loss.backward() on the scalar loss,
+ * src/nn/loss.zig:150-159): grad (+)= (probs - target)/rows.  Same values as the two calls; a batch of at most
+ * 256 rows x 32 columns (64 x 256, 16 x 4096) takes one launch.  accumulate == 0: grad is written, not read. */
+int zg_hip_smce_fwd_bwd(zg_hip_ctx *ctx, const float *logits, const float *target, float *probs, float *loss,
+                        float *grad, size_t rows, size_t cols, int accumulate);
 /* integer-label form: one pass over the logits forward (online softmax), lse[rows] kept for backward */
 int zg_hip_smce_label_fwd(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, float *lse, float *loss,
                           size_t rows, size_t cols);

@@ -252,6 +252,13 @@ class OracleDevice(HipDevice):
     def _x_zg_hip_scatter_gcn_deg_scaled_bwd(self, go, h, deg, s, t, gh, gd, stride, n_edge, n_nodes):
         return self._o.cdll.zo_scatter_gcn_deg_scaled_bwd(go, h, deg, s, t, gh, gd, stride, n_edge)
 
+    def _x_zg_hip_smce_fwd_bwd(self, logits, target, probs, loss, grad, rows, cols, accumulate):
+        # the forward followed by CceBwd with an upstream gradient of 1 (src/nn/loss.zig:130-159)
+        if not accumulate:
+            ctypes.memset(grad, 0, rows * cols * 4)
+        self._o.cdll.zo_smce_fwd(logits, target, probs, loss, rows, cols)
+        self._o.cdll.zo_smce_bwd(probs, target, grad, rows, cols)
+
     def _x_zg_hip_smce_label_bwd(self, logits, labels, lse, grad, rows, cols, accumulate):
         if not accumulate:
             ctypes.memset(grad, 0, rows * cols * 4)

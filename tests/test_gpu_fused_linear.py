@@ -202,3 +202,39 @@ def test_fused_gcn_step_with_an_edge_plan_replays_from_an_execution_graph(hip):
     for a, b in zip(eager.param_buffers(), graph.param_buffers()):
         assert np.array_equal(hip.to_numpy(a), hip.to_numpy(b))
     graph.free_graph()
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 10), (140, 7), (256, 32), (257, 32), (1, 1), (64, 256), (65, 256), (16, 4096),
+                                       (17, 4096), (3, 1000), (5, 33), (700, 1024), (2, 5000)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_smce_fwd_bwd_equals_forward_then_backward(oracle, hip, rows, cols, accumulate):
+    """One call against smce_fwd + smce_bwd (src/nn/loss.zig:130-159) on the same device, bit for bit, on both sides
+    of the one-launch limit; against the CPU oracle's composition to 1e-5."""
+    r = np.random.default_rng(rows * 131 + cols)
+    logits = r.standard_normal((rows, cols)).astype(np.float32)  # label probabilities stay above the 1e-7 clamp
+    target = np.zeros((rows, cols), np.float32)
+    target[np.arange(rows), r.integers(0, cols, rows)] = 1.0
+    g0 = r.standard_normal((rows, cols)).astype(np.float32)
+    nan = np.full((rows, cols), np.nan, np.float32)
+    p = {"logits": logits, "target": target, "probs": nan.copy(), "loss": np.full(1, np.nan, np.float32),
+         "grad": g0.copy() if accumulate else nan.copy(), "rows": rows, "cols": cols, "accumulate": accumulate}
+    got = run_op(hip, "smce_fwd_bwd", dict(p), ["probs", "loss", "grad"])
+    fwd = run_op(hip, "smce_fwd", {"logits": logits, "target": target, "probs": nan.copy(), "loss": np.zeros(1, np.float32),
+                                   "rows": rows, "cols": cols}, ["probs", "loss"])
+    bwd = run_op(hip, "smce_bwd", {"probs": fwd["probs"], "target": target,
+                                   "grad": g0.copy() if accumulate else np.zeros((rows, cols), np.float32),
+                                   "rows": rows, "cols": cols}, ["grad"])
+    assert np.array_equal(got["probs"], fwd["probs"])
+    assert np.array_equal(got["loss"], fwd["loss"])
+    assert np.array_equal(got["grad"], bwd["grad"])
+    ref = run_op(oracle, "smce_fwd_bwd", dict(p), ["probs", "loss", "grad"])
+    for name in ("probs", "loss", "grad"):
+        assert np.linalg.norm(got[name].ravel() - ref[name].ravel()) <= 1e-5 * (np.linalg.norm(ref[name].ravel()) + 1e-6), name
+    # closed form: rows of the written gradient sum to zero, the loss is the mean of -log clamp(p[label])
+    if not accumulate:
+        assert np.abs(got["grad"].reshape(rows, cols).astype(np.float64).sum(axis=1)).max() <= 1e-6
+    x = logits.astype(np.float64)
+    lse = np.log(np.exp(x - x.max(axis=1, keepdims=True)).sum(axis=1)) + x.max(axis=1)
+    p_label = np.clip(np.exp((x * target).sum(axis=1) - lse), 1e-7, np.float64(np.float32(1.0 - 1e-7)))  # the clamp of loss.zig:143
+    want = np.mean(-np.log(p_label))
+    assert abs(float(got["loss"][0]) - want) <= 1e-5 * (abs(want) + 1e-3)

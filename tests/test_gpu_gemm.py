@@ -186,6 +186,22 @@ def test_bmm_acc_split_k_batches(oracle, hip):
     assert rel_fro(res[1], res[0]) <= TOL
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 128, 784), (40, 40, 16384), (33, 31, 16392), (500, 500, 300), (16, 1433, 2708)])
+def test_small_products_with_a_long_k_repeat_bit_for_bit(hip, m, n, k):
+    """A small C with a long k is cut into ranges of k over several workgroups per tile of C, and the partial tiles
+    are added in range order by a second kernel: repeated launches give the same bits, and the values match float64
+    to the tolerance."""
+    r = rng(m + n + k)
+    A = r.standard_normal((m, k)).astype(np.float32)
+    B = r.standard_normal((n, k)).astype(np.float32)
+    C0 = r.standard_normal((m, n)).astype(np.float32)
+    outs = [run_matmul(hip, A, B, C0.copy(), m, n, k, False, True, k, k, n, 1.0, 1.0) for _ in range(4)]
+    for o in outs[1:]:
+        assert np.array_equal(o, outs[0])
+    truth = A.astype(np.float64) @ B.astype(np.float64).T + C0
+    assert rel_fro(outs[0], truth) <= TOL
+
+
 def test_bmm_32x512_cubed(oracle, hip):
     """The microbenchmark shape: batch 32 of 512 x 512 x 512, transposed-B layout as well."""
     r = rng(77)

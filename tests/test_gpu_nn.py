@@ -195,7 +195,8 @@ def test_gather_offsets_bit_exact(oracle, hip):
         np.testing.assert_array_equal(res[1], want.ravel().astype(np.uint64))
 
 
-@pytest.mark.parametrize("n,dst_len", [(64, 128), (13264, 2708), (100000, 17), (5000, 300000), (1, 1), (40000, 5000)])
+@pytest.mark.parametrize("n,dst_len", [(64, 128), (13264, 2708), (100000, 17), (5000, 300000), (1, 1), (40000, 5000),
+                                        (256, 7), (257, 7), (200, 1), (255, 1000)])
 def test_scatter_add_bit_exact(oracle, hip, n, dst_len):
     """Order of accumulation per destination equals the host loop's, so the floats agree bit for bit."""
     r = rng(n + dst_len)

@@ -442,6 +442,11 @@ pub fn smce_bwd(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
     check(c.zg_hip_smce_bwd(self.ctx, p.probs.ptr, p.target.ptr, p.grad.ptr, p.rows, p.cols));
 }
+/// smce_fwd and the backward of the scalar loss in one call (upstream gradient 1): p.grad (+)= (probs - target)/rows.
+pub fn smce_fwd_bwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smce_fwd_bwd(self.ctx, p.logits.ptr, p.target.ptr, p.probs.ptr, p.loss.ptr, p.grad.ptr, p.rows, p.cols, @intFromBool(p.accumulate)));
+}
 pub fn smooth_l1_fwd(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
     check(c.zg_hip_smooth_l1_fwd(self.ctx, p.pred.ptr, p.target.ptr, p.pred.len, p.beta, p.loss.ptr));

@@ -842,9 +842,13 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.split_stride = 0;
 
     if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
-    // the unstaged kernel: short k on up to one block per CU, or a longer k when C is only a handful of blocks (the
-    // first layer of the batch-64 MLP, 64 x 128 x 784: 6 us in one launch against 14 us split and reduced)
-    if ((k <= 256 && tiles(32, 32) <= n_cu) || (k <= 2048 && tiles(32, 32) <= 16))
+    // the unstaged kernel: short k on up to one block per CU, or k up to 512 when C is only a handful of blocks.
+    // Beyond that the split product below is faster even with its second launch (64 x 128 x 784, the first layer of
+    // the batch-64 MLP: 7.6 us of kernel time split and reduced against 11 us here; 128 x 128 x 1024: 8.6 against 16).
+    // Cutting k over several workgroups inside this kernel, with the last one to arrive adding the partial blocks,
+    // was measured too: the device-scope fences it needs write back and invalidate the L2, 10 us for 32 workgroups
+    // and 65 us for 500.
+    if ((k <= 256 && tiles(32, 32) <= n_cu) || (k <= 512 && tiles(32, 32) <= 16))
         return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
 
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);

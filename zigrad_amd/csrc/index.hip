@@ -261,6 +261,43 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
     dst[b] = acc;
 }
 
+// The whole of scatter_add for at most kScatterSmallMax entries in one launch of one workgroup: thread i owns entry i,
+// and the first entry of each destination walks the later entries in input order, so the additions happen in the
+// order of the host loop.  Offsets at or beyond `nb` are skipped, as the bucket path skips them.
+constexpr int kScatterSmallMax = 256;
+__global__ __launch_bounds__(kScatterSmallMax) void scatter_add_small_kernel(const float* src, const uint64_t* offsets,
+                                                                             int n, float* dst, size_t nb) {
+    __shared__ uint64_t s_off[kScatterSmallMax];
+    __shared__ float s_src[kScatterSmallMax];
+    const int i = threadIdx.x;
+    // slots past n hold an offset no destination has, so the walk below can run in whole groups of eight
+    s_off[i] = (i < n) ? offsets[i] : ~0ull;
+    s_src[i] = (i < n) ? src[i] : 0.f;
+    __syncthreads();
+    if (i >= n) return;
+    const uint64_t k = s_off[i];
+    if (k >= nb) return;
+    float acc = dst[k];
+    bool first = true;
+    const int n8 = (n + 7) & ~7;
+    for (int j0 = 0; j0 < n8; j0 += 8) {
+        uint64_t o[8];
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {  // eight LDS reads in flight, then the additions in input order
+            o[u] = s_off[j0 + u];
+            v[u] = s_src[j0 + u];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const bool same = o[u] == k;
+            first = first && !(same && j0 + u < i);
+            acc = (same && j0 + u >= i) ? __fadd_rn(acc, v[u]) : acc;
+        }
+    }
+    if (first) dst[k] = acc;
+}
+
 // rows of `stride` elements: dst[b, :] = src_row(e) + dst[b, :] in input order.  G threads per destination row.
 // MODE 0: index_select backward  (x_grad[row] = y_grad[e] + x_grad[row], src/ndtensor.zig:1461-1465)
 template <int G>
@@ -513,6 +550,12 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
     ZG_REQUIRE(src && offsets && dst, "scatter_add: null pointer");
     ZG_REQUIRE(dst_len > 0, "scatter_add: empty destination");
     ZG_REQUIRE(n < 0xffffffffull && dst_len < 0xffffffffull, "scatter_add: sizes beyond 2^32-1");
+    if (n <= (size_t)kScatterSmallMax) {
+        hipLaunchKernelGGL(scatter_add_small_kernel, dim3(1), dim3(kScatterSmallMax), 0, ctx->stream, src, offsets, (int)n,
+                           dst, dst_len);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     void* mem = workspace(ctx, plan_bytes(n, dst_len));
     if (!mem) return ZG_HIP_EOOM;
     Plan pl = carve_plan(mem, n, dst_len);

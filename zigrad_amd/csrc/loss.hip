@@ -313,46 +313,97 @@ static bool long_row_ok(const float* a, const float* b, const float* c, size_t r
            rows <= 0x7fffffffull;
 }
 
-// src/nn/loss.zig:150-159
+// src/nn/loss.zig:150-159.  ACC false: the gradient is written, not accumulated (same values as accumulating
+// into zeros, without reading them).
+template <bool ACC>
 __global__ __launch_bounds__(kBlock) void smce_bwd_kernel(const float* probs, const float* target, float* grad, size_t n,
                                                            float denom) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x, nt = (size_t)gridDim.x * kBlock;
     const bool vec = ((reinterpret_cast<uintptr_t>(probs) | reinterpret_cast<uintptr_t>(target) |
                        reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
+    auto term = [&](float g, float p, float t) {
+        const float d = __fdiv_rn(__fsub_rn(p, t), denom);
+        return ACC ? __fadd_rn(g, d) : d;
+    };
     if (vec) {
         const size_t n4 = n >> 2;
         const float4* p4 = reinterpret_cast<const float4*>(probs);
         const float4* t4 = reinterpret_cast<const float4*>(target);
         float4* g4 = reinterpret_cast<float4*>(grad);
-        // three streams in, one out: two 16-byte pieces per stream in flight per thread
+        const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        // three streams in (two when the gradient is only written), one out: two 16-byte pieces per stream in
+        // flight per thread
         for (size_t j = i; j < n4; j += 2 * nt) {
             const size_t j2 = j + nt;
             const bool two = j2 < n4;
-            float4 p = nt_load(p4 + j), t = nt_load(t4 + j), g = nt_load(g4 + j);
+            float4 p = nt_load(p4 + j), t = nt_load(t4 + j), g = ACC ? nt_load(g4 + j) : zero4;
             float4 q = p, u = t, h = g;
             if (two) {
                 q = nt_load(p4 + j2);
                 u = nt_load(t4 + j2);
-                h = nt_load(g4 + j2);
+                if (ACC) h = nt_load(g4 + j2);
             }
-            g.x = __fadd_rn(g.x, __fdiv_rn(__fsub_rn(p.x, t.x), denom));
-            g.y = __fadd_rn(g.y, __fdiv_rn(__fsub_rn(p.y, t.y), denom));
-            g.z = __fadd_rn(g.z, __fdiv_rn(__fsub_rn(p.z, t.z), denom));
-            g.w = __fadd_rn(g.w, __fdiv_rn(__fsub_rn(p.w, t.w), denom));
+            g.x = term(g.x, p.x, t.x);
+            g.y = term(g.y, p.y, t.y);
+            g.z = term(g.z, p.z, t.z);
+            g.w = term(g.w, p.w, t.w);
             nt_store(g, g4 + j);
             if (two) {
-                h.x = __fadd_rn(h.x, __fdiv_rn(__fsub_rn(q.x, u.x), denom));
-                h.y = __fadd_rn(h.y, __fdiv_rn(__fsub_rn(q.y, u.y), denom));
-                h.z = __fadd_rn(h.z, __fdiv_rn(__fsub_rn(q.z, u.z), denom));
-                h.w = __fadd_rn(h.w, __fdiv_rn(__fsub_rn(q.w, u.w), denom));
+                h.x = term(h.x, q.x, u.x);
+                h.y = term(h.y, q.y, u.y);
+                h.z = term(h.z, q.z, u.z);
+                h.w = term(h.w, q.w, u.w);
                 nt_store(h, g4 + j2);
             }
         }
-        for (size_t j = (n4 << 2) + i; j < n; j += nt)
-            grad[j] = __fadd_rn(grad[j], __fdiv_rn(__fsub_rn(probs[j], target[j]), denom));
+        for (size_t j = (n4 << 2) + i; j < n; j += nt) grad[j] = term(ACC ? grad[j] : 0.f, probs[j], target[j]);
     } else {
-        for (; i < n; i += nt) grad[i] = __fadd_rn(grad[i], __fdiv_rn(__fsub_rn(probs[i], target[i]), denom));
+        for (; i < n; i += nt) grad[i] = term(ACC ? grad[i] : 0.f, probs[i], target[i]);
     }
+}
+
+// smce_fwd and the loss's backward (upstream gradient 1) of a batch small enough for one workgroup, in one launch:
+// kFlatSingle / TPR rows of at most 4096 columns.  Per row the arithmetic is softmax_rows_kernel's, per gradient
+// element smce_bwd_kernel's, and the mean over the rows is formed as flat_single_kernel forms it, so every value
+// equals what the separate launches produce.
+template <int TPR, bool ACC>
+__global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* logits, const float* target, float* probs,
+                                                                 float* loss, float* grad, size_t rows, size_t cols) {
+    static_assert(TPR <= kWave, "a row is reduced inside one wave");
+    __shared__ __align__(16) float row_loss[kFlatSingle / TPR];
+    __shared__ float smem[kFlatSingle / kWave];
+    const int lane = threadIdx.x % TPR;
+    const size_t row = threadIdx.x / TPR;
+    const bool live = row < rows;
+    const float denom = (float)rows;
+    OnlineAccT acc = OnlineAcc::init();
+    if (live) acc = row_online<TPR>(logits + row * cols, cols, lane);
+    acc = group_reduce<OnlineAcc, TPR>(acc);
+    float part = 0.f;
+    if (live) {
+        const float l = __fadd_rn(acc.m, logf(acc.s));
+        const float* xr = logits + row * cols;
+        const float* tr = target + row * cols;
+        float* pr = probs + row * cols;
+        float* gr = grad + row * cols;
+        for (size_t j = lane; j < cols; j += TPR) {
+            const float p = expf(__fsub_rn(xr[j], l));
+            const float t = tr[j];
+            pr[j] = p;
+            if (t != 0.f) {
+                const float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
+                part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
+            }
+            const float d = __fdiv_rn(__fsub_rn(p, t), denom);
+            gr[j] = ACC ? __fadd_rn(gr[j], d) : d;
+        }
+    }
+    part = group_reduce<SumAcc, TPR>(part);
+    if (live && lane == 0) row_loss[row] = part;
+    __syncthreads();
+    float s = flat_accumulate<TermId, 1>(row_loss, nullptr, rows, 0.f, threadIdx.x, blockDim.x);
+    s = block_reduce<SumAcc>(s, smem);
+    if (threadIdx.x == 0) FinDivN{loss, denom}(s);
 }
 
 // src/nn/loss.zig:232-245: x_g += y * (y_g - sum_j y_j * y_g_j) per row
@@ -472,8 +523,43 @@ ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* tar
     const size_t n = rows * cols;
     size_t blocks = ceil_div_sz(n, (size_t)kBlock * 8);
     if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
-    hipLaunchKernelGGL(smce_bwd_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad, n,
-                       (float)rows);
+    hipLaunchKernelGGL(smce_bwd_kernel<true>, dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad,
+                       n, (float)rows);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_smce_fwd_bwd(zg_hip_ctx* ctx, const float* logits, const float* target, float* probs, float* loss,
+                               float* grad, size_t rows, size_t cols, int accumulate) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(logits && target && probs && loss && grad, "smce_fwd_bwd: null pointer");
+    if (int rc = check_rows("smce_fwd_bwd", rows, cols)) return rc;
+    const int tpr = pick_tpr(cols);
+    if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr)) {
+#define ZG_SMALL(T)                                                                                                    \
+    if (accumulate)                                                                                                    \
+        hipLaunchKernelGGL((smce_small_kernel<T, true>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,   \
+                           probs, loss, grad, rows, cols);                                                             \
+    else                                                                                                               \
+        hipLaunchKernelGGL((smce_small_kernel<T, false>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,  \
+                           probs, loss, grad, rows, cols)
+        if (tpr == 4) { ZG_SMALL(4); }
+        else if (tpr == 16) { ZG_SMALL(16); }
+        else { ZG_SMALL(64); }
+#undef ZG_SMALL
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    if (int rc = zg_hip_smce_fwd(ctx, logits, target, probs, loss, rows, cols)) return rc;
+    const size_t n = rows * cols;
+    size_t blocks = ceil_div_sz(n, (size_t)kBlock * 8);
+    if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
+    if (accumulate)
+        hipLaunchKernelGGL(smce_bwd_kernel<true>, dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad,
+                           n, (float)rows);
+    else
+        hipLaunchKernelGGL(smce_bwd_kernel<false>, dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, probs, target,
+                           grad, n, (float)rows);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

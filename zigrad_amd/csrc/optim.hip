@@ -135,6 +135,7 @@ __device__ __forceinline__ void update_in_workgroup(float* p, float* g, float* m
 // per-thread accumulation and the same combine tree), publishes the clip factor, and goes on to the update.
 // One launch instead of two; the arithmetic per element is that of sgd_kernel / adam_kernel, so the values are
 // the same.  `factor_out` keeps the slot the two-kernel path fills.
+constexpr size_t kClippedSingleMax = 4096;  // Adam: beyond this the update alone keeps one compute unit busy for microseconds
 template <bool ADAM>
 __global__ __launch_bounds__(kFlatSingle) void clipped_update_small_kernel(float* p, float* g, float* m, float* v,
                                                                            size_t n, float step_scale,
@@ -157,11 +158,16 @@ __global__ __launch_bounds__(kFlatSingle) void clipped_update_small_kernel(float
     update_in_workgroup<ADAM>(p, g, m, v, n, scale, f, lr_t, b1, b2, omb1, omb2, eps, false);
 }
 
-// The same update for up to kMultiMax small tensors in one launch: workgroup b does what
-// clipped_update_small_kernel does for tensor b (same accumulation tree for the norm, same arithmetic per element),
-// reads its lr_t from memory when asked to, and with `zero_grads` leaves the gradient zero instead of clipped
-// (optim.step() followed by model.zero_grad(), examples/mnist/src/main-simple.zig:70-71).
+// The same update for up to kMultiMax small tensors in two launches (one without the clip).  norm_multi_kernel:
+// workgroup b forms tensor b's clip factor as clipped_update_small_kernel does (same accumulation tree).
+// update_multi_kernel: the tensors are cut into slices of kMultiSlice elements, one workgroup each, so that a tensor
+// of tens of thousands of elements is spread over many compute units (the update is arithmetic-bound on one); each
+// workgroup looks up its tensor's factor, reads its lr_t from memory when asked to, and with `zero_grads` leaves the
+// gradient zero instead of clipped (optim.step() followed by model.zero_grad(),
+// examples/mnist/src/main-simple.zig:70-71).  The arithmetic per element is that of sgd_kernel / adam_kernel.
 constexpr int kMultiMax = 16;
+constexpr int kMultiThreads = 256;
+constexpr int kMultiSlice = kMultiThreads * kInFlight;  // one trip of update_in_workgroup
 struct MultiArgs {
     float* p[kMultiMax];
     float* g[kMultiMax];
@@ -169,32 +175,33 @@ struct MultiArgs {
     float* v[kMultiMax];
     size_t n[kMultiMax];
     float lr_t[kMultiMax];       // Adam: lr_t per tensor; SGD: -lr
+    int wg_first[kMultiMax + 1]; // update_multi_kernel: tensor b owns workgroups wg_first[b] .. wg_first[b + 1] - 1
     const float* lr_t_mem;       // Adam under replay: lr_t_mem[b] is read when the kernel runs (null: use lr_t[b])
+    float* factors;              // clip factor per tensor, written by norm_multi_kernel
     float b1, b2, omb1, omb2, eps, max_norm, delta;
-    int clip, zero_grads;
+    int clip, zero_grads, count;
 };
 
-template <bool ADAM>
-__global__ __launch_bounds__(kFlatSingle) void update_multi_kernel(MultiArgs a) {
+__global__ __launch_bounds__(kFlatSingle) void norm_multi_kernel(MultiArgs a) {
     __shared__ float smem[kFlatSingle / kWave];
-    __shared__ float factor_s;
     const int b = blockIdx.x;
-    float* const p = a.p[b];
-    float* const g = a.g[b];
-    float* const m = a.m[b];
-    float* const v = a.v[b];
-    const size_t n = a.n[b];
-    float f = 1.0f;
-    if (a.clip) {
-        float acc = flat_accumulate<TermSq, 1>(g, nullptr, n, 0.f, threadIdx.x, blockDim.x);
-        acc = block_reduce<SumAcc>(acc, smem);
-        if (threadIdx.x == 0) FinClipFactor{&factor_s, a.max_norm, a.delta}(acc);
-        __syncthreads();
-        f = factor_s;
-    }
+    float acc = flat_accumulate<TermSq, 1>(a.g[b], nullptr, a.n[b], 0.f, threadIdx.x, blockDim.x);
+    acc = block_reduce<SumAcc>(acc, smem);
+    if (threadIdx.x == 0) FinClipFactor{a.factors + b, a.max_norm, a.delta}(acc);
+}
+
+template <bool ADAM>
+__global__ __launch_bounds__(kMultiThreads) void update_multi_kernel(MultiArgs a) {
+    int b = 0;
+    while (b + 1 < a.count && (int)blockIdx.x >= a.wg_first[b + 1]) b++;
+    const size_t off = (size_t)((int)blockIdx.x - a.wg_first[b]) * kMultiSlice;
+    const size_t left = a.n[b] - off;
+    const size_t n = left < (size_t)kMultiSlice ? left : (size_t)kMultiSlice;
+    const float f = a.clip ? a.factors[b] : 1.0f;
     const bool scale = f != 1.0f;
     const float lr_t = (ADAM && a.lr_t_mem) ? a.lr_t_mem[b] : a.lr_t[b];
-    update_in_workgroup<ADAM>(p, g, m, v, n, scale, f, lr_t, a.b1, a.b2, a.omb1, a.omb2, a.eps, a.zero_grads != 0);
+    update_in_workgroup<ADAM>(a.p[b] + off, a.g[b] + off, ADAM ? a.m[b] + off : nullptr, ADAM ? a.v[b] + off : nullptr, n,
+                              scale, f, lr_t, a.b1, a.b2, a.omb1, a.omb2, a.eps, a.zero_grads != 0);
 }
 
 static int update_grid(zg_hip_ctx* ctx, size_t n) {
@@ -242,7 +249,7 @@ static int adam_launch(zg_hip_ctx* ctx, float* param, float* grad, float* m, flo
                        float delta) {
     const float omb1 = 1.0f - beta1, omb2 = 1.0f - beta2;
     float* factor = ctx->scalar_slot + 1;
-    if (clip && n <= kFlatSingleMax) {
+    if (clip && n <= kClippedSingleMax) {
         hipLaunchKernelGGL((clipped_update_small_kernel<true>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, param, grad,
                            m, v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, max_norm, delta, factor);
     } else if (clip) {
@@ -296,8 +303,14 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
     auto flush = [&]() -> int {
         if (!filled) return ZG_HIP_OK;
         a.lr_t_mem = (adam && lr_t_in_memory) ? lr_t + first : nullptr;
-        if (adam) hipLaunchKernelGGL((update_multi_kernel<true>), dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
-        else hipLaunchKernelGGL((update_multi_kernel<false>), dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
+        a.count = filled;
+        if (clip) {
+            hipLaunchKernelGGL(norm_multi_kernel, dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
+            ZG_LAUNCH_CHECK();
+        }
+        const unsigned grid = (unsigned)a.wg_first[filled];
+        if (adam) hipLaunchKernelGGL((update_multi_kernel<true>), dim3(grid), dim3(kMultiThreads), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((update_multi_kernel<false>), dim3(grid), dim3(kMultiThreads), 0, ctx->stream, a);
         filled = 0;
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
@@ -311,6 +324,8 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
     a.delta = delta;
     a.clip = clip;
     a.zero_grads = zero_grads;
+    a.factors = ctx->scalar_slot + 16;  // kMultiMax floats of the context's 64
+    a.wg_first[0] = 0;
     for (size_t i = 0; i < n_tensors; i++) {
         const size_t n = lens[i];
         if (n == 0) {  // keeps lr_t_mem's indexing dense: an empty tensor ends the batch
@@ -326,6 +341,7 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
             a.v[filled] = adam ? vs[i] : nullptr;
             a.n[filled] = n;
             a.lr_t[filled] = adam ? (lr_t_in_memory ? 0.f : lr_t[i]) : -lr;
+            a.wg_first[filled + 1] = a.wg_first[filled] + (int)ceil_div_sz(n, kMultiSlice);
             if (++filled == kMultiMax)
                 if (int rc = flush()) return rc;
             continue;

@@ -280,7 +280,7 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks < 1) chunks = 1;
     if (chunks > 64) chunks = 64;  // keeps the partials buffer and the serial tail of the final stage small
-    if (outer * R * inner <= 65536) chunks = 1;  // a second launch costs more than the rows a chunk split would save
+    if (outer * R * inner <= 16384) chunks = 1;  // a second launch costs more than the rows a chunk split would save
     const size_t rows_per_chunk = ceil_div_sz(R, chunks);
     chunks = ceil_div_sz(R, rows_per_chunk);
     ZG_REQUIRE(outer <= 65535, "axis reduction: %zu leading slices exceed the grid limit", outer);

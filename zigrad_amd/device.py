@@ -428,6 +428,10 @@ class HipDevice:
     def _op_smce_bwd(self, probs, target, grad, rows, cols):
         self._call("zg_hip_smce_bwd", probs.ptr, target.ptr, grad.ptr, rows, cols)
 
+    def _op_smce_fwd_bwd(self, logits, target, probs, loss, grad, rows, cols, accumulate=True):
+        self._call("zg_hip_smce_fwd_bwd", logits.ptr, target.ptr, probs.ptr, loss.ptr, grad.ptr, rows, cols,
+                   int(bool(accumulate)))
+
     def _op_smce_label_fwd(self, logits, labels, lse, loss, rows, cols):
         self._call("zg_hip_smce_label_fwd", logits.ptr, labels.ptr, lse.ptr, loss.ptr, rows, cols)
 

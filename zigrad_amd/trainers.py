@@ -412,25 +412,33 @@ class MLPTrainer(GraphSteps):
         acts = self.net.forward(self.x, B)
         logits = acts[-1]
         loss = d.mem_cache_alloc(F32, 1)
-        if self.loss_mode == "onehot":
-            saved = d.mem_cache_alloc(F32, B * C)  # sm_preds
-            d.dispatch("smce_fwd", logits=logits, target=self.onehot, probs=saved, loss=loss, rows=B, cols=C)
+        if self.optim.fused and self.loss_mode == "onehot":
+            # forward and the loss's backward in one call; the gradient is written, so it needs no zero fill
+            saved, g = d.mem_cache_alloc(F32, B * C), d.mem_cache_alloc(F32, B * C)
+            d.dispatch("smce_fwd_bwd", logits=logits, target=self.onehot, probs=saved, loss=loss, grad=g, rows=B, cols=C,
+                       accumulate=False)
+            loss_val = self._read_loss(loss) if read_loss is True else None
+            d.mem_cache_free(saved)
         else:
-            saved = d.mem_cache_alloc(F32, B)  # per-row log-sum-exp
-            d.dispatch("smce_label_fwd", logits=logits, labels=self.labels, lse=saved, loss=loss, rows=B, cols=C)
-        loss_val = self._read_loss(loss) if read_loss is True else None  # loss.get(0): a blocking read before backward
+            if self.loss_mode == "onehot":
+                saved = d.mem_cache_alloc(F32, B * C)  # sm_preds
+                d.dispatch("smce_fwd", logits=logits, target=self.onehot, probs=saved, loss=loss, rows=B, cols=C)
+            else:
+                saved = d.mem_cache_alloc(F32, B)  # per-row log-sum-exp
+                d.dispatch("smce_label_fwd", logits=logits, labels=self.labels, lse=saved, loss=loss, rows=B, cols=C)
+            loss_val = self._read_loss(loss) if read_loss is True else None  # loss.get(0): a blocking read before backward
 
-        # backward
-        loss_grad = d.mem_cache_alloc(F32, 1)
-        d.mem_fill(loss_grad, 1.0)
-        g = d.mem_cache_alloc(F32, B * C)
-        d.mem_fill(g, 0.0)
-        if self.loss_mode == "onehot":
-            d.dispatch("smce_bwd", probs=saved, target=self.onehot, grad=g, rows=B, cols=C)
-        else:
-            d.dispatch("smce_label_bwd", logits=logits, labels=self.labels, lse=saved, grad=g, rows=B, cols=C, accumulate=True)
-        d.mem_cache_free(saved)
-        d.mem_cache_free(loss_grad)
+            # backward
+            loss_grad = d.mem_cache_alloc(F32, 1)
+            d.mem_fill(loss_grad, 1.0)
+            g = d.mem_cache_alloc(F32, B * C)
+            d.mem_fill(g, 0.0)
+            if self.loss_mode == "onehot":
+                d.dispatch("smce_bwd", probs=saved, target=self.onehot, grad=g, rows=B, cols=C)
+            else:
+                d.dispatch("smce_label_bwd", logits=logits, labels=self.labels, lse=saved, grad=g, rows=B, cols=C, accumulate=True)
+            d.mem_cache_free(saved)
+            d.mem_cache_free(loss_grad)
         self.net.backward(acts, g, B)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
@@ -688,14 +696,19 @@ class GCNTrainer(GraphSteps):
         out_m = d.mem_cache_alloc(F32, M * C)  # MaskLayer.forward: the labelled rows, here one contiguous prefix
         d.mem_copy(s2["y"].sub(0, M * C), out_m)
         probs, loss = d.mem_cache_alloc(F32, M * C), d.mem_cache_alloc(F32, 1)
-        d.dispatch("smce_fwd", logits=out_m, target=self.label_m, probs=probs, loss=loss, rows=M, cols=C)
-        loss_val = self._read_loss(loss)
-        # backward
-        loss_grad = d.mem_cache_alloc(F32, 1)
-        d.mem_fill(loss_grad, 1.0)
         g_m = d.mem_cache_alloc(F32, M * C)
-        d.mem_fill(g_m, 0.0)
-        d.dispatch("smce_bwd", probs=probs, target=self.label_m, grad=g_m, rows=M, cols=C)
+        loss_grad = d.mem_cache_alloc(F32, 1)
+        if self.optim.fused:  # forward and the loss's backward in one call, the gradient written without a zero fill
+            d.dispatch("smce_fwd_bwd", logits=out_m, target=self.label_m, probs=probs, loss=loss, grad=g_m, rows=M, cols=C,
+                       accumulate=False)
+            loss_val = self._read_loss(loss)
+        else:
+            d.dispatch("smce_fwd", logits=out_m, target=self.label_m, probs=probs, loss=loss, rows=M, cols=C)
+            loss_val = self._read_loss(loss)
+            # backward
+            d.mem_fill(loss_grad, 1.0)
+            d.mem_fill(g_m, 0.0)
+            d.dispatch("smce_bwd", probs=probs, target=self.label_m, grad=g_m, rows=M, cols=C)
         g2 = d.mem_cache_alloc(F32, N * C)
         d.mem_fill(g2, 0.0)
         d.mem_copy(g_m, g2.sub(0, M * C))  # MaskLayer.backward

@@ -185,6 +185,7 @@ struct MultiArgs {
 __global__ __launch_bounds__(kFlatSingle) void norm_multi_kernel(MultiArgs a) {
     __shared__ float smem[kFlatSingle / kWave];
     const int b = blockIdx.x;
+    if (a.n[b] > kFlatSingleMax) return;  // its factor came from the two-stage reduction, launched before this kernel
     float acc = flat_accumulate<TermSq, 1>(a.g[b], nullptr, a.n[b], 0.f, threadIdx.x, blockDim.x);
     acc = block_reduce<SumAcc>(acc, smem);
     if (threadIdx.x == 0) FinClipFactor{a.factors + b, a.max_norm, a.delta}(acc);
@@ -290,7 +291,10 @@ ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float
     return adam_launch(ctx, param, grad, m, v, n, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);
 }
 
-// Parameter lists: tensors of up to kFlatSingleMax elements share launches, larger ones take the per-tensor path.
+// Parameter lists: tensors of up to kMultiBigMax elements share the update launch (those beyond kFlatSingleMax get
+// their clip factor from the two-stage norm reduction of the per-tensor path first, so the values stay the same);
+// larger ones take the per-tensor path with its 16-byte grid-stride kernels.
+constexpr size_t kMultiBigMax = (size_t)1 << 20;
 static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_tensors, float* const* params,
                       float* const* grads, float* const* ms, float* const* vs, const size_t* lens, const float* lr_t,
                       int lr_t_in_memory, float lr, float beta1, float beta2, float epsilon, int clip, float max_norm,
@@ -333,8 +337,13 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
             continue;
         }
         ZG_REQUIRE(params[i] && grads[i] && (!adam || (ms[i] && vs[i])), "%s: null pointer in tensor %zu", name, i);
-        if (n <= kFlatSingleMax) {
+        if (n <= kMultiBigMax) {
             if (filled == 0) first = i;
+            if (clip && n > kFlatSingleMax) {
+                int rc = flat_reduce<TermSq, 1>(ctx, grads[i], nullptr, n, 0.f,
+                                                FinClipFactor{a.factors + filled, max_norm, delta});
+                if (rc) return rc;
+            }
             a.p[filled] = params[i];
             a.g[filled] = grads[i];
             a.m[filled] = adam ? ms[i] : nullptr;

@@ -149,6 +149,29 @@ def test_optimizer_list_entry_points_equal_the_per_tensor_ops(hip, kind, clip, z
             assert np.array_equal(x, y), (sizes[i], which)
 
 
+def test_optimizer_list_with_a_tensor_listed_twice_updates_it_twice(hip):
+    """Shared weights that appear twice in the parameter list get two updates, the second on the result of the first,
+    as the per-tensor loop gives them (src/nn/optim.zig:100-122)."""
+    r = np.random.default_rng(11)
+    n = 5000
+    p0, g0 = r.standard_normal(n).astype(np.float32), (3.0 * r.standard_normal(n)).astype(np.float32)
+    q0, h0 = r.standard_normal(77).astype(np.float32), r.standard_normal(77).astype(np.float32)
+    out = []
+    for multi in (False, True):
+        p, g, q, h = (hip.from_numpy(a) for a in (p0, g0, q0, h0))
+        if multi:
+            hip.dispatch("sgd_step_multi", params=[p, q, p], grads=[g, h, g], lr=0.1, clip=True, max_norm=10.0, delta=1e-6,
+                         zero_grads=False)
+        else:
+            for a, b in ((p, g), (q, h), (p, g)):
+                hip.dispatch("sgd_step", param=a, grad=b, lr=0.1, clip=True, max_norm=10.0, delta=1e-6)
+        out.append([hip.to_numpy(t) for t in (p, g, q, h)])
+        for t in (p, g, q, h):
+            hip.mem_free(t)
+    for x, y in zip(*out):
+        assert np.array_equal(x, y)
+
+
 def test_dqn_and_gcn_steps_with_and_without_fusion_agree_exactly(hip):
     from zigrad_amd.trainers import DQNTrainer, GCNTrainer, dqn_inputs, gcn_inputs
 

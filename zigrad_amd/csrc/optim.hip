@@ -176,7 +176,7 @@ struct MultiArgs {
     size_t n[kMultiMax];
     float lr_t[kMultiMax];       // Adam: lr_t per tensor; SGD: -lr
     int wg_first[kMultiMax + 1]; // update_multi_kernel: tensor b owns workgroups wg_first[b] .. wg_first[b + 1] - 1
-    const float* lr_t_mem;       // Adam under replay: lr_t_mem[b] is read when the kernel runs (null: use lr_t[b])
+    const float* lr_t_mem[kMultiMax];  // Adam under replay: *lr_t_mem[b] is read when the kernel runs (null: use lr_t[b])
     float* factors;              // clip factor per tensor, written by norm_multi_kernel
     float b1, b2, omb1, omb2, eps, max_norm, delta;
     int clip, zero_grads, count;
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kMultiThreads) void update_multi_kernel(MultiArgs a
     const size_t n = left < (size_t)kMultiSlice ? left : (size_t)kMultiSlice;
     const float f = a.clip ? a.factors[b] : 1.0f;
     const bool scale = f != 1.0f;
-    const float lr_t = (ADAM && a.lr_t_mem) ? a.lr_t_mem[b] : a.lr_t[b];
+    const float lr_t = (ADAM && a.lr_t_mem[b]) ? a.lr_t_mem[b][0] : a.lr_t[b];
     update_in_workgroup<ADAM>(a.p[b] + off, a.g[b] + off, ADAM ? a.m[b] + off : nullptr, ADAM ? a.v[b] + off : nullptr, n,
                               scale, f, lr_t, a.b1, a.b2, a.omb1, a.omb2, a.eps, a.zero_grads != 0);
 }
@@ -291,7 +291,8 @@ ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float
     return adam_launch(ctx, param, grad, m, v, n, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);
 }
 
-// Parameter lists: tensors of up to kMultiBigMax elements share the update launch (those beyond kFlatSingleMax get
+// Parameter lists (the tensors are independent, so the launches need not follow the list order; a tensor listed
+// twice is the exception and is handled below): tensors of up to kMultiBigMax elements share the update launch (those beyond kFlatSingleMax get
 // their clip factor from the two-stage norm reduction of the per-tensor path first, so the values stay the same);
 // larger ones take the per-tensor path with its 16-byte grid-stride kernels.
 constexpr size_t kMultiBigMax = (size_t)1 << 20;
@@ -303,10 +304,8 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
     ZG_REQUIRE(!adam || n_tensors == 0 || (ms && vs && lr_t), "%s: null list", name);
     MultiArgs a;
     int filled = 0;
-    size_t first = 0;  // list index of the batch's first tensor (lr_t_mem is indexed by workgroup)
     auto flush = [&]() -> int {
         if (!filled) return ZG_HIP_OK;
-        a.lr_t_mem = (adam && lr_t_in_memory) ? lr_t + first : nullptr;
         a.count = filled;
         if (clip) {
             hipLaunchKernelGGL(norm_multi_kernel, dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
@@ -332,13 +331,14 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
     a.wg_first[0] = 0;
     for (size_t i = 0; i < n_tensors; i++) {
         const size_t n = lens[i];
-        if (n == 0) {  // keeps lr_t_mem's indexing dense: an empty tensor ends the batch
-            if (int rc = flush()) return rc;
-            continue;
-        }
+        if (n == 0) continue;
         ZG_REQUIRE(params[i] && grads[i] && (!adam || (ms[i] && vs[i])), "%s: null pointer in tensor %zu", name, i);
+        // a tensor that is listed twice is updated twice, in list order: the second update waits for the first
+        bool listed = false;
+        for (int b = 0; b < filled; b++) listed = listed || a.p[b] == params[i] || a.g[b] == grads[i];
+        if (listed)
+            if (int rc = flush()) return rc;
         if (n <= kMultiBigMax) {
-            if (filled == 0) first = i;
             if (clip && n > kFlatSingleMax) {
                 int rc = flat_reduce<TermSq, 1>(ctx, grads[i], nullptr, n, 0.f,
                                                 FinClipFactor{a.factors + filled, max_norm, delta});
@@ -350,12 +350,12 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
             a.v[filled] = adam ? vs[i] : nullptr;
             a.n[filled] = n;
             a.lr_t[filled] = adam ? (lr_t_in_memory ? 0.f : lr_t[i]) : -lr;
+            a.lr_t_mem[filled] = (adam && lr_t_in_memory) ? lr_t + i : nullptr;
             a.wg_first[filled + 1] = a.wg_first[filled] + (int)ceil_div_sz(n, kMultiSlice);
             if (++filled == kMultiMax)
                 if (int rc = flush()) return rc;
             continue;
         }
-        if (int rc = flush()) return rc;
         int rc;
         if (adam)
             rc = adam_launch(ctx, params[i], grads[i], ms[i], vs[i], n, lr_t_in_memory ? 0.f : lr_t[i],

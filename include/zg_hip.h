@@ -142,6 +142,13 @@ int zg_hip_linear_fwd(zg_hip_ctx *ctx, const float *x, const float *w, const flo
  * ReLU output that fed the layer (null: no mask).  With accumulate == 0 gx is not read and needs no zero fill. */
 int zg_hip_linear_bwd_input(zg_hip_ctx *ctx, const float *gy, const float *w, const float *act_in, float *gx,
                             size_t batch, size_t fan_in, size_t fan_out, int accumulate);
+/* The whole backward of the layer for a final output gradient gy[batch, fan_out] (the two products of BmmAccBwd,
+ * src/ndtensor.zig:1092-1136, the bias's unbroadcast, src/device/host_device.zig:709-780, and the ReLU backward of the
+ * layer before): gw[fan_out, fan_in] += gy^T . x;  gb[fan_out] += column sums of gy (null: none);
+ * gx[batch, fan_in] = gy . w, zero where act_in <= 0 (gx null: no input gradient; act_in null: no mask).
+ * One launch for a small layer, the separate ops otherwise; the same values either way. */
+int zg_hip_linear_bwd(zg_hip_ctx *ctx, const float *gy, const float *x, const float *w, const float *act_in, float *gw,
+                      float *gb, float *gx, size_t batch, size_t fan_in, size_t fan_out);
 int zg_hip_outer(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *A, float alpha);
 /* B = A^T + alpha*B; B is not read when alpha == 0 (the reference hands in uninitialised B then:
  * src/ndarray.zig:794-802) */

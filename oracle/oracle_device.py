@@ -243,6 +243,19 @@ class OracleDevice(HipDevice):
         if act_in:
             c.zo_relu_inplace_bwd(act_in, gx, batch * fan_in)
 
+    def _x_zg_hip_linear_bwd(self, gy, x, w, act_in, gw, gb, gx, batch, fan_in, fan_out):
+        # dB and dA of BmmAccBwd for MATMUL_ABt (src/ndtensor.zig:1092-1136), the bias's fold over the batch
+        # (src/device/host_device.zig:709-780) and relu_inplace_bwd of the layer before (:543-547)
+        c = self._o.cdll
+        c.zo_matmul(gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, fan_in, fan_in, 1.0, 1.0)
+        if gb:
+            shape_x, shape_y = (ctypes.c_uint64 * 2)(batch, fan_out), (ctypes.c_uint64 * 1)(fan_out)
+            c.zo_unbroadcast(gy, shape_x, 2, gb, shape_y, 1, None, 0, 1.0, 1.0)
+        if gx:
+            c.zo_matmul(gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in, 1.0, 0.0)
+            if act_in:
+                c.zo_relu_inplace_bwd(act_in, gx, batch * fan_in)
+
     def _x_zg_hip_axpy(self, x, y, n, alpha, alpha_on_device):
         return self._o.cdll.zo_axpy(x, y, n, alpha)  # host memory either way
 

@@ -73,6 +73,46 @@ def test_linear_bwd_input_equals_product_then_relu_backward(hip, shape, accumula
     assert np.linalg.norm(got - want) <= 1e-5 * (np.linalg.norm(want) + 1e-3), shape
 
 
+@pytest.mark.parametrize("shape", SHAPES + [(64, 4, 128), (64, 128, 2), (128, 128, 128), (256, 100, 64), (257, 100, 64)])
+@pytest.mark.parametrize("with_gx,with_gb", [(True, True), (False, True), (True, False)])
+def test_linear_bwd_equals_the_separate_ops(oracle, hip, shape, with_gx, with_gb):
+    """One call against the weight-gradient product, the bias's unbroadcast and linear_bwd_input on the same device,
+    bit for bit (small layers take one launch, the others the separate ops); against float64 and the CPU oracle's
+    composition to 1e-5."""
+    B, I, O = shape
+    r = np.random.default_rng(B * 7 + I * 3 + O + 5)
+    gy = r.standard_normal((B, O)).astype(np.float32)
+    x = np.maximum(r.standard_normal((B, I)), 0.0).astype(np.float32)  # a ReLU output: layer input and mask
+    w = (r.standard_normal((O, I)) / np.sqrt(O)).astype(np.float32)
+    gw0 = r.standard_normal((O, I)).astype(np.float32)
+    gb0 = r.standard_normal(O).astype(np.float32)
+    p = {"gy": gy, "x": x, "w": w, "act_in": x if with_gx else None, "gw": gw0.copy(), "gb": gb0.copy() if with_gb else None,
+         "gx": np.full((B, I), np.nan, np.float32) if with_gx else None, "batch": B, "fan_in": I, "fan_out": O}
+    outs = ["gw"] + (["gb"] if with_gb else []) + (["gx"] if with_gx else [])
+    got = run_op(hip, "linear_bwd", dict(p), outs)
+    ref_gw = run_op(hip, "matmul", {"A": gy, "B": x, "C": gw0.copy(), "m": O, "n": I, "k": B, "trans_a": True,
+                                    "trans_b": False, "lda": O, "ldb": I, "ldc": I, "alpha": 1.0, "beta": 1.0}, ["C"])["C"]
+    assert np.array_equal(got["gw"], ref_gw), shape
+    want_gw = gy.astype(np.float64).T @ x.astype(np.float64) + gw0
+    assert np.linalg.norm(got["gw"] - want_gw) <= 1e-5 * (np.linalg.norm(want_gw) + 1e-3)
+    if with_gb:
+        ref_gb = run_op(hip, "unbroadcast", {"x": gy, "x_shape": [B, O], "y": gb0.copy(), "y_shape": [O], "alpha": 1.0,
+                                             "beta": 1.0}, ["y"])["y"]
+        assert np.array_equal(got["gb"], ref_gb), shape
+        want_gb = gy.astype(np.float64).sum(axis=0) + gb0
+        assert np.linalg.norm(got["gb"] - want_gb) <= 1e-5 * (np.linalg.norm(want_gb) + 1e-3)
+    if with_gx:
+        ref_gx = run_op(hip, "linear_bwd_input", {"gy": gy, "w": w, "act_in": x, "gx": np.full((B, I), np.nan, np.float32),
+                                                  "batch": B, "fan_in": I, "fan_out": O, "accumulate": False}, ["gx"])["gx"]
+        assert np.array_equal(got["gx"], ref_gx), shape
+        want_gx = np.where(x > 0, gy.astype(np.float64) @ w.astype(np.float64), 0.0)
+        assert np.linalg.norm(got["gx"] - want_gx) <= 1e-5 * (np.linalg.norm(want_gx) + 1e-3)
+    if B * I * O <= 1 << 22:
+        ref = run_op(oracle, "linear_bwd", dict(p), outs)
+        for name in outs:
+            assert np.linalg.norm(got[name] - ref[name]) <= 1e-5 * (np.linalg.norm(ref[name]) + 1e-3), (shape, name)
+
+
 @pytest.mark.parametrize("dims,batch,optimizer", [([784, 128, 64, 10], 64, "sgd"), ([100, 260, 130, 7], 50, "adam"),
                                                   ([512, 768, 384, 32], 512, "adam")])
 def test_train_steps_with_and_without_fusion_agree_exactly(hip, dims, batch, optimizer):

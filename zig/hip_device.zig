@@ -531,6 +531,16 @@ pub fn linear_bwd_input(self: *const Self, T: type, p: anytype) void {
     const act: ?[*]const T = if (p.act_in) |a| a.ptr else null;
     check(c.zg_hip_linear_bwd_input(self.ctx, p.gy.ptr, p.w.ptr, act, p.gx.ptr, p.batch, p.fan_in, p.fan_out, @intFromBool(p.accumulate)));
 }
+/// The whole backward of a Linear layer for a final output gradient: gw += gy^T . x, gb += column sums of gy
+/// (`p.gb` optional), gx = gy . w zeroed where `p.act_in` <= 0 (`p.gx`, `p.act_in` optional): the two products of
+/// BmmAccBwd (src/ndtensor.zig:1092-1136), the bias's unbroadcast and relu_inplace_bwd of the layer before.
+pub fn linear_bwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    const act: ?[*]const T = if (p.act_in) |a| a.ptr else null;
+    const gb: ?[*]T = if (p.gb) |b| b.ptr else null;
+    const gx: ?[*]T = if (p.gx) |g| g.ptr else null;
+    check(c.zg_hip_linear_bwd(self.ctx, p.gy.ptr, p.x.ptr, p.w.ptr, act, p.gw.ptr, gb, gx, p.batch, p.fan_in, p.fan_out));
+}
 
 /// Adam update whose `lr_t` is read from memory when the kernel runs (`p.lr_t` points to device memory or
 /// to `mem_alloc_indices`-style pinned host memory).  A step recorded with `capture.open()` can then be

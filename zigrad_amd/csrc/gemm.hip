@@ -22,6 +22,7 @@
 // Workgroup ids are remapped so that the workgroups resident on one XCD (ids congruent modulo 8) cover a
 // compact patch of C and share their A rows / B columns in that XCD's L2.
 #include "common.h"
+#include "reduce.cuh"
 
 #include <type_traits>
 
@@ -634,11 +635,10 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
 // of group g: k = 8g + 4h + c), so a k-contiguous operand is one 16-byte load per lane and group; every load is
 // guarded and zero-filled, so any shape and alignment is served.  The four partial blocks are added in wave
 // order through LDS: the result does not depend on scheduling.
+// `block` is the 32x32 block of C (row-major over tiles_n), z the batch, `part` 16 KiB of the caller's LDS.
 template <bool A_KMAJOR, bool B_KMAJOR>
-__global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
-    __shared__ float part[4][16][64];
-    const size_t m0 = (size_t)(blockIdx.x / g.tiles_n) * 32, n0 = (size_t)(blockIdx.x % g.tiles_n) * 32;
-    const size_t z = blockIdx.z;
+__device__ __forceinline__ void gemm_tiny_block(const GemmArgs& g, unsigned block, size_t z, float (*part)[16][64]) {
+    const size_t m0 = (size_t)(block / g.tiles_n) * 32, n0 = (size_t)(block % g.tiles_n) * 32;
     const float* A = g.A + (z % g.nba) * g.a_chunk;
     const float* B = g.B + (z % g.nbb) * g.b_chunk;
     float* C = g.C + z * g.c_chunk;
@@ -715,6 +715,37 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
     }
 }
 
+template <bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
+    __shared__ float part[4][16][64];
+    gemm_tiny_block<A_KMAJOR, B_KMAJOR>(g, blockIdx.x, blockIdx.z, part);
+}
+
+// The backward of a small Linear layer in one launch: the workgroups of the weight-gradient product (gw += gy^T x),
+// those of the input-gradient product (gx = gy w, masked by the ReLU output that fed the layer) and those of the bias
+// gradient (gb += column sums of gy) side by side.  Each workgroup runs the block of gemm_tiny_kernel or of
+// col_reduce_kernel it would run in the separate launches, so the values are the same; the three results are
+// independent of each other.
+struct LinearBwdArgs {
+    GemmArgs gw, gx;
+    unsigned n_w, n_x;  // workgroups of the two products (n_x = 0: no input gradient)
+    const float* gy;    // [R, inner]
+    float* gb;          // null: no bias gradient
+    size_t R, inner;
+    int log2_cx;
+};
+template <int V>
+__global__ __launch_bounds__(kGemmThreads) void linear_bwd_small_kernel(LinearBwdArgs a) {
+    __shared__ float part[4][16][64];
+    static_assert(sizeof(part) >= sizeof(float) * kBlock * V && kBlock == kGemmThreads, "LDS of the column sums");
+    const unsigned b = blockIdx.x;
+    if (b < a.n_w) gemm_tiny_block<false, false>(a.gw, b, 0, part);
+    else if (b < a.n_w + a.n_x) gemm_tiny_block<true, false>(a.gx, b - a.n_w, 0, part);
+    else
+        col_reduce_block<AxisSum, V>(a.gy, a.gb, nullptr, a.R, a.inner, a.log2_cx, a.R, 1.f, 1.f, b - a.n_w - a.n_x, 0, 0,
+                                     1, &part[0][0][0]);
+}
+
 static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, size_t batches) {
     g.tiles_m = (unsigned)ceil_div_sz(g.M, 32);
     g.tiles_n = (unsigned)ceil_div_sz(g.N, 32);
@@ -772,6 +803,53 @@ struct GemmExtras {
     int relu;
 };
 
+// the operand fields every kernel reads (the staged kernels' launcher adds the tile geometry and the split)
+static GemmArgs gemm_args(const float* A, const float* B, float* C, size_t m, size_t n, size_t k, int trans_a, int trans_b,
+                          size_t lda, size_t ldb, size_t ldc, float alpha, float beta, size_t nba, size_t nbb,
+                          size_t a_chunk, size_t b_chunk, size_t c_chunk, const GemmExtras* extras) {
+    GemmArgs g;
+    g.A = A;
+    g.B = B;
+    g.C = C;
+    g.M = m;
+    g.N = n;
+    g.K = k;
+    g.lda = lda;
+    g.ldb = ldb;
+    g.ldc = ldc;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.bias = extras ? extras->bias : nullptr;
+    g.gate = extras ? extras->gate : nullptr;
+    g.relu = extras ? extras->relu : 0;
+    g.nba = nba;
+    g.nbb = nbb;
+    g.a_chunk = a_chunk;
+    g.b_chunk = b_chunk;
+    g.c_chunk = c_chunk;
+    g.a_vec = aligned16(A) && lda % 4 == 0 && a_chunk % 4 == 0;
+    g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
+    g.tiles_m = (unsigned)ceil_div_sz(m, 32);  // the unstaged kernel's blocks; the staged launcher sets its own
+    g.tiles_n = (unsigned)ceil_div_sz(n, 32);
+    g.split_tiles = 0;
+    g.split_stride = 0;
+    g.c_vec = 0;
+    g.bounded_tail = 0;
+    return g;
+}
+
+// The unstaged kernel serves short k on up to one 32 x 32 block of C per CU, or k up to 512 when C is only a handful
+// of blocks.  Beyond that the split product is faster even with its second launch (64 x 128 x 784, the first layer
+// of the batch-64 MLP: 7.6 us of kernel time split and reduced against 11 us unstaged; 128 x 128 x 1024: 8.6 against
+// 16).  Cutting k over several workgroups inside the unstaged kernel, with the last one to arrive adding the partial
+// blocks, was measured too: the device-scope fences it needs write back and invalidate the L2, 10 us for 32
+// workgroups and 65 us for 500.
+static bool gemm_is_tiny(size_t m, size_t n, size_t k, size_t batches, size_t lda, size_t ldb, size_t n_cu) {
+    const size_t blocks = ceil_div_sz(m, 32) * ceil_div_sz(n, 32) * batches;
+    const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
+    return small_ld && ((k <= 256 && blocks <= n_cu) || (k <= 512 && blocks <= 16));
+}
+
 static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
                          size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta,
                          size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk,
@@ -793,29 +871,9 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    GemmArgs g;
-    g.A = A;
-    g.B = B;
-    g.C = C;
-    g.M = m;
-    g.N = n;
-    g.K = k;
-    g.lda = lda;
-    g.ldb = ldb;
-    g.ldc = ldc;
-    g.alpha = alpha;
-    g.beta = beta;
-    g.bias = extras ? extras->bias : nullptr;
-    g.gate = extras ? extras->gate : nullptr;
-    g.relu = extras ? extras->relu : 0;
-    g.nba = nba;
-    g.nbb = nbb;
-    g.a_chunk = a_chunk;
-    g.b_chunk = b_chunk;
-    g.c_chunk = c_chunk;
+    GemmArgs g = gemm_args(A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, nba, nbb, a_chunk, b_chunk,
+                           c_chunk, extras);
     const bool a_kmajor = !trans_a, b_kmajor = trans_b != 0;
-    g.a_vec = aligned16(A) && lda % 4 == 0 && a_chunk % 4 == 0;
-    g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
 
     // Kernel mode per tile shape: fast (whole tiles in m and n, C fit for vector stores), edge (everything else) or
     // checked (leading dimensions too large for 32-bit byte offsets), see gemm_kernel.
@@ -842,14 +900,7 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     g.split_stride = 0;
 
     if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
-    // the unstaged kernel: short k on up to one block per CU, or k up to 512 when C is only a handful of blocks.
-    // Beyond that the split product below is faster even with its second launch (64 x 128 x 784, the first layer of
-    // the batch-64 MLP: 7.6 us of kernel time split and reduced against 11 us here; 128 x 128 x 1024: 8.6 against 16).
-    // Cutting k over several workgroups inside this kernel, with the last one to arrive adding the partial blocks,
-    // was measured too: the device-scope fences it needs write back and invalidate the L2, 10 us for 32 workgroups
-    // and 65 us for 500.
-    if ((k <= 256 && tiles(32, 32) <= n_cu) || (k <= 512 && tiles(32, 32) <= 16))
-        return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
+    if (gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
 
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
     if (c_large <= c_mid && c_large <= c_small)
@@ -998,6 +1049,56 @@ ZG_API int zg_hip_linear_bwd_input(zg_hip_ctx* ctx, const float* gy, const float
     const GemmExtras ex = {nullptr, act_in, 0};
     return gemm_dispatch(ctx, "linear_bwd_input", gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in, 1.f, 0.f,
                          1, 1, 1, 0, 0, 0, 0, act_in ? &ex : nullptr);
+}
+
+// The backward of a Linear layer y = x . w^T + b whose output gradient gy is final (src/ndtensor.zig:1092-1136 for the
+// two products, the bias's unbroadcast, and the ReLU backward of the layer before):
+//   gw += gy^T . x;   gb += column sums of gy (gb may be null);   gx = gy . w, zeroed where act_in <= 0 (gx may be
+//   null: no input gradient; act_in may be null: no mask).
+// A layer small enough for the unstaged product kernel and the one-chunk column sum takes one launch; any other
+// layer takes the separate ops.  Same values either way.
+ZG_API int zg_hip_linear_bwd(zg_hip_ctx* ctx, const float* gy, const float* x, const float* w, const float* act_in,
+                             float* gw, float* gb, float* gx, size_t batch, size_t fan_in, size_t fan_out) {
+    ZG_CTX(ctx);
+    if (batch == 0 || fan_in == 0 || fan_out == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(gy && x && gw, "linear_bwd: null pointer");
+    ZG_REQUIRE(!gx || w, "linear_bwd: an input gradient needs the weights");
+    const size_t n_cu = (size_t)ctx->n_cu;
+    const bool small = gemm_is_tiny(fan_out, fan_in, batch, 1, fan_out, fan_in, n_cu) &&
+                       (!gx || gemm_is_tiny(batch, fan_in, fan_out, 1, fan_out, fan_in, n_cu)) &&
+                       (!gb || batch * fan_out <= kColSingleChunkMax);
+    if (!small) {
+        if (gb) {
+            const uint64_t gy_shape[2] = {batch, fan_out}, gb_shape[1] = {fan_out};
+            if (int rc = zg_hip_unbroadcast(ctx, gy, gy_shape, 2, gb, gb_shape, 1, nullptr, 0, 1.f, 1.f)) return rc;
+        }
+        if (gx)
+            if (int rc = zg_hip_linear_bwd_input(ctx, gy, w, act_in, gx, batch, fan_in, fan_out, 0)) return rc;
+        return gemm_dispatch(ctx, "linear_bwd", gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, fan_in, fan_in, 1.f, 1.f,
+                             1, 1, 1, 0, 0, 0);
+    }
+    LinearBwdArgs a;
+    a.gw = gemm_args(gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, fan_in, fan_in, 1.f, 1.f, 1, 1, 0, 0, 0, nullptr);
+    a.n_w = a.gw.tiles_m * a.gw.tiles_n;
+    a.gx = a.gw;
+    a.n_x = 0;
+    if (gx) {
+        const GemmExtras ex = {nullptr, act_in, 0};
+        a.gx = gemm_args(gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in, 1.f, 0.f, 1, 1, 0, 0, 0,
+                         act_in ? &ex : nullptr);
+        a.n_x = a.gx.tiles_m * a.gx.tiles_n;
+    }
+    const ColReduceShape cs = col_reduce_shape(gy, fan_out);
+    a.gy = gy;
+    a.gb = gb;
+    a.R = batch;
+    a.inner = fan_out;
+    a.log2_cx = cs.log2_cx;
+    const unsigned grid = a.n_w + a.n_x + (gb ? (unsigned)cs.gx : 0u);
+    if (cs.V == 4) hipLaunchKernelGGL(linear_bwd_small_kernel<4>, dim3(grid), dim3(kGemmThreads), 0, ctx->stream, a);
+    else hipLaunchKernelGGL(linear_bwd_small_kernel<1>, dim3(grid), dim3(kGemmThreads), 0, ctx->stream, a);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
 }
 
 ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_shape, const float* B,

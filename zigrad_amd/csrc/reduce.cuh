@@ -313,4 +313,122 @@ static __global__ __launch_bounds__(kBlock) void scale_by_device_factor_kernel(f
 }
 
 
+// ------------------------------------------------------------------------------------------------
+// sums along the first or a middle axis of [outer, R, inner] (used by reduce.hip and by the fused Linear backward)
+// ------------------------------------------------------------------------------------------------
+struct AxisSum {
+    using P = SumAcc;
+    using Out = float;
+    static __device__ __forceinline__ float term(float v, uint32_t) { return v; }
+    static __device__ __forceinline__ void store(Out* y, size_t o, float s, float alpha, float beta) {
+        float r = __fmul_rn(alpha, s);
+        y[o] = (beta == 0.f) ? r : __fadd_rn(r, __fmul_rn(beta, y[o]));
+    }
+};
+
+// inner > 1: column-style.  Workgroup = cx column-threads x ry row-threads (cx*ry = 256), each thread owns V
+// adjacent columns and walks rows ty, ty+ry, ... of its row chunk.  grid = (column groups, row chunks, outer).
+// With one row chunk the result is stored directly; otherwise per-chunk partials go to `partials`
+// laid out [outer, chunks, inner] and col_final_kernel combines them in chunk order.
+// The block coordinates are arguments (bx: column group, by: row chunk of n_chunks, bz: outer slice) and `smem` is
+// kBlock * V accumulators of the caller's LDS, so that another kernel can run this block beside other work.
+template <class A, int V>
+__device__ __forceinline__ void col_reduce_block(const float* x, typename A::Out* y, typename A::P::Acc* partials,
+                                                 size_t R, size_t inner, int log2_cx, size_t rows_per_chunk,
+                                                 float alpha, float beta, unsigned bx, unsigned by, unsigned bz,
+                                                 unsigned n_chunks, typename A::P::Acc* smem) {
+    using P = typename A::P;
+    using Acc = typename P::Acc;
+    const int cx = 1 << log2_cx, ry = kBlock >> log2_cx;
+    const int tx = threadIdx.x & (cx - 1), ty = threadIdx.x >> log2_cx;
+    const size_t colv = (size_t)bx * cx + tx;  // in units of V columns
+    const size_t col0 = colv * V;
+    const size_t outer = bz;
+    const size_t r_begin = (size_t)by * rows_per_chunk;
+    size_t r_end = r_begin + rows_per_chunk;
+    if (r_end > R) r_end = R;
+    Acc acc[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) acc[v] = P::init();
+    const bool active = col0 < inner;
+    if (active) {
+        const float* xb = x + outer * R * inner + col0;
+        size_t r = r_begin + ty;
+        if constexpr (V == 4) {
+            for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
+                float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
+                float4 v1 = *reinterpret_cast<const float4*>(xb + (r + ry) * inner);
+                float4 v2 = *reinterpret_cast<const float4*>(xb + (r + 2 * (size_t)ry) * inner);
+                float4 v3 = *reinterpret_cast<const float4*>(xb + (r + 3 * (size_t)ry) * inner);
+                const float4 vs[4] = {v0, v1, v2, v3};
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    uint32_t rr = (uint32_t)(r + (size_t)u * ry);
+                    acc[0] = P::combine(acc[0], A::term(vs[u].x, rr));
+                    acc[1 % V] = P::combine(acc[1 % V], A::term(vs[u].y, rr));
+                    acc[2 % V] = P::combine(acc[2 % V], A::term(vs[u].z, rr));
+                    acc[3 % V] = P::combine(acc[3 % V], A::term(vs[u].w, rr));
+                }
+            }
+            for (; r < r_end; r += ry) {
+                float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
+                uint32_t rr = (uint32_t)r;
+                acc[0] = P::combine(acc[0], A::term(v0.x, rr));
+                acc[1 % V] = P::combine(acc[1 % V], A::term(v0.y, rr));
+                acc[2 % V] = P::combine(acc[2 % V], A::term(v0.z, rr));
+                acc[3 % V] = P::combine(acc[3 % V], A::term(v0.w, rr));
+            }
+        } else {
+            for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
+                float v0 = xb[r * inner], v1 = xb[(r + ry) * inner], v2 = xb[(r + 2 * (size_t)ry) * inner],
+                      v3 = xb[(r + 3 * (size_t)ry) * inner];
+                acc[0] = P::combine(acc[0], A::term(v0, (uint32_t)r));
+                acc[0] = P::combine(acc[0], A::term(v1, (uint32_t)(r + ry)));
+                acc[0] = P::combine(acc[0], A::term(v2, (uint32_t)(r + 2 * (size_t)ry)));
+                acc[0] = P::combine(acc[0], A::term(v3, (uint32_t)(r + 3 * (size_t)ry)));
+            }
+            for (; r < r_end; r += ry) acc[0] = P::combine(acc[0], A::term(xb[r * inner], (uint32_t)r));
+        }
+    }
+    // combine the ry row-threads of each column in ty order
+#pragma unroll
+    for (int v = 0; v < V; v++) smem[threadIdx.x * V + v] = acc[v];
+    __syncthreads();
+    if (ty == 0 && active) {
+        for (int t = 1; t < ry; t++) {
+#pragma unroll
+            for (int v = 0; v < V; v++) acc[v] = P::combine(acc[v], smem[((t << log2_cx) + tx) * V + v]);
+        }
+#pragma unroll
+        for (int v = 0; v < V; v++) {
+            size_t c = col0 + v;
+            if (c < inner) {
+                if (n_chunks == 1)
+                    A::store(y, outer * inner + c, acc[v], alpha, beta);
+                else
+                    partials[(outer * n_chunks + by) * inner + c] = acc[v];
+            }
+        }
+    }
+}
+
+
+// Launch geometry of col_reduce_block for rows of `inner` elements starting at x: V columns per thread, 2^log2_cx
+// column-threads per workgroup, gx column groups.
+struct ColReduceShape {
+    int V, log2_cx;
+    size_t gx;
+};
+static inline ColReduceShape col_reduce_shape(const float* x, size_t inner) {
+    ColReduceShape s;
+    s.V = ((inner % 4 == 0) && aligned16(x)) ? 4 : 1;
+    const size_t colv = inner / s.V;
+    s.log2_cx = 0;
+    // at most 64 column threads (1 KiB of a row per workgroup with V = 4): more workgroups, fewer partials
+    while ((1u << s.log2_cx) < colv && s.log2_cx < 6) s.log2_cx++;
+    s.gx = ceil_div_sz(colv, (size_t)1 << s.log2_cx);
+    return s;
+}
+constexpr size_t kColSingleChunkMax = 16384;  // up to this many elements the rows are not split into chunks
+
 }  // namespace zg

@@ -52,15 +52,6 @@ static int stream_grid(zg_hip_ctx* ctx, size_t n, size_t per_thread) {
 // ------------------------------------------------------------------------------------------------
 // reductions along an axis.  x is viewed as [outer, R, inner]; R is reduced.
 // ------------------------------------------------------------------------------------------------
-struct AxisSum {
-    using P = SumAcc;
-    using Out = float;
-    static __device__ __forceinline__ float term(float v, uint32_t) { return v; }
-    static __device__ __forceinline__ void store(Out* y, size_t o, float s, float alpha, float beta) {
-        float r = __fmul_rn(alpha, s);
-        y[o] = (beta == 0.f) ? r : __fadd_rn(r, __fmul_rn(beta, y[o]));
-    }
-};
 struct AxisMax {
     using P = MaxAcc;
     using Out = float;
@@ -126,89 +117,15 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
     if (lane == 0 && row < rows) A::store(y, row, acc, alpha, beta);
 }
 
-// inner > 1: column-style.  Workgroup = cx column-threads x ry row-threads (cx*ry = 256), each thread owns V
-// adjacent columns and walks rows ty, ty+ry, ... of its row chunk.  grid = (column groups, row chunks, outer).
-// With one row chunk the result is stored directly; otherwise per-chunk partials go to `partials`
-// laid out [outer, chunks, inner] and col_final_kernel combines them in chunk order.
+// inner > 1: column-style, see col_reduce_block
 template <class A, int V>
 __global__ __launch_bounds__(kBlock) void col_reduce_kernel(const float* x, typename A::Out* y,
                                                              typename A::P::Acc* partials, size_t R, size_t inner,
                                                              int log2_cx, size_t rows_per_chunk, float alpha,
                                                              float beta) {
-    using P = typename A::P;
-    using Acc = typename P::Acc;
-    __shared__ Acc smem[kBlock * V];
-    const int cx = 1 << log2_cx, ry = kBlock >> log2_cx;
-    const int tx = threadIdx.x & (cx - 1), ty = threadIdx.x >> log2_cx;
-    const size_t colv = (size_t)blockIdx.x * cx + tx;  // in units of V columns
-    const size_t col0 = colv * V;
-    const size_t outer = blockIdx.z;
-    const size_t r_begin = (size_t)blockIdx.y * rows_per_chunk;
-    size_t r_end = r_begin + rows_per_chunk;
-    if (r_end > R) r_end = R;
-    Acc acc[V];
-#pragma unroll
-    for (int v = 0; v < V; v++) acc[v] = P::init();
-    const bool active = col0 < inner;
-    if (active) {
-        const float* xb = x + outer * R * inner + col0;
-        size_t r = r_begin + ty;
-        if constexpr (V == 4) {
-            for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
-                float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
-                float4 v1 = *reinterpret_cast<const float4*>(xb + (r + ry) * inner);
-                float4 v2 = *reinterpret_cast<const float4*>(xb + (r + 2 * (size_t)ry) * inner);
-                float4 v3 = *reinterpret_cast<const float4*>(xb + (r + 3 * (size_t)ry) * inner);
-                const float4 vs[4] = {v0, v1, v2, v3};
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    uint32_t rr = (uint32_t)(r + (size_t)u * ry);
-                    acc[0] = P::combine(acc[0], A::term(vs[u].x, rr));
-                    acc[1 % V] = P::combine(acc[1 % V], A::term(vs[u].y, rr));
-                    acc[2 % V] = P::combine(acc[2 % V], A::term(vs[u].z, rr));
-                    acc[3 % V] = P::combine(acc[3 % V], A::term(vs[u].w, rr));
-                }
-            }
-            for (; r < r_end; r += ry) {
-                float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
-                uint32_t rr = (uint32_t)r;
-                acc[0] = P::combine(acc[0], A::term(v0.x, rr));
-                acc[1 % V] = P::combine(acc[1 % V], A::term(v0.y, rr));
-                acc[2 % V] = P::combine(acc[2 % V], A::term(v0.z, rr));
-                acc[3 % V] = P::combine(acc[3 % V], A::term(v0.w, rr));
-            }
-        } else {
-            for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
-                float v0 = xb[r * inner], v1 = xb[(r + ry) * inner], v2 = xb[(r + 2 * (size_t)ry) * inner],
-                      v3 = xb[(r + 3 * (size_t)ry) * inner];
-                acc[0] = P::combine(acc[0], A::term(v0, (uint32_t)r));
-                acc[0] = P::combine(acc[0], A::term(v1, (uint32_t)(r + ry)));
-                acc[0] = P::combine(acc[0], A::term(v2, (uint32_t)(r + 2 * (size_t)ry)));
-                acc[0] = P::combine(acc[0], A::term(v3, (uint32_t)(r + 3 * (size_t)ry)));
-            }
-            for (; r < r_end; r += ry) acc[0] = P::combine(acc[0], A::term(xb[r * inner], (uint32_t)r));
-        }
-    }
-    // combine the ry row-threads of each column in ty order
-#pragma unroll
-    for (int v = 0; v < V; v++) smem[threadIdx.x * V + v] = acc[v];
-    __syncthreads();
-    if (ty == 0 && active) {
-        for (int t = 1; t < ry; t++) {
-#pragma unroll
-            for (int v = 0; v < V; v++) acc[v] = P::combine(acc[v], smem[((t << log2_cx) + tx) * V + v]);
-        }
-#pragma unroll
-        for (int v = 0; v < V; v++) {
-            size_t c = col0 + v;
-            if (c < inner) {
-                if (gridDim.y == 1)
-                    A::store(y, outer * inner + c, acc[v], alpha, beta);
-                else
-                    partials[(outer * gridDim.y + blockIdx.y) * inner + c] = acc[v];
-            }
-        }
-    }
+    __shared__ typename A::P::Acc smem[kBlock * V];
+    col_reduce_block<A, V>(x, y, partials, R, inner, log2_cx, rows_per_chunk, alpha, beta, blockIdx.x, blockIdx.y,
+                           blockIdx.z, gridDim.y, smem);
 }
 
 // Workgroup = 64 adjacent outputs x 4 waves; wave w combines chunks w, w+4, w+8, ... of its outputs with all its
@@ -265,14 +182,11 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    const bool v4 = (inner % 4 == 0) && aligned16(x);
-    const int V = v4 ? 4 : 1;
-    const size_t colv = inner / V;
-    int log2_cx = 0;
-    // at most 64 column threads (1 KiB of a row per workgroup with V = 4): more workgroups, fewer partials
-    while ((1u << log2_cx) < colv && log2_cx < 6) log2_cx++;
-    const int cx = 1 << log2_cx, ry = kBlock >> log2_cx;
-    const size_t gx = ceil_div_sz(colv, cx);
+    const ColReduceShape cs = col_reduce_shape(x, inner);
+    const bool v4 = cs.V == 4;
+    const int log2_cx = cs.log2_cx;
+    const int ry = kBlock >> log2_cx;
+    const size_t gx = cs.gx;
     // row chunks: enough workgroups to cover the machine several times, but at least 4 trips of ry rows each
     size_t want = (size_t)ctx->n_cu * 8;
     size_t chunks = ceil_div_sz(want, gx * outer);
@@ -280,7 +194,7 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks < 1) chunks = 1;
     if (chunks > 64) chunks = 64;  // keeps the partials buffer and the serial tail of the final stage small
-    if (outer * R * inner <= 16384) chunks = 1;  // a second launch costs more than the rows a chunk split would save
+    if (outer * R * inner <= kColSingleChunkMax) chunks = 1;  // a second launch costs more than a chunk split saves
     const size_t rows_per_chunk = ceil_div_sz(R, chunks);
     chunks = ceil_div_sz(R, rows_per_chunk);
     ZG_REQUIRE(outer <= 65535, "axis reduction: %zu leading slices exceed the grid limit", outer);

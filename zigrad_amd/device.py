@@ -289,6 +289,12 @@ class HipDevice:
         self._call("zg_hip_linear_bwd_input", gy.ptr, w.ptr, act_in.ptr if act_in is not None else None, gx.ptr, batch,
                    fan_in, fan_out, int(accumulate))
 
+    def _op_linear_bwd(self, gy, x, w, act_in, gw, gb, gx, batch, fan_in, fan_out):
+        """gw += gy^T . x; gb += column sums of gy (None: none); gx = gy . w, zeroed where act_in <= 0 (None: none)."""
+        opt = lambda b: b.ptr if b is not None else None
+        self._call("zg_hip_linear_bwd", gy.ptr, x.ptr, opt(w), opt(act_in), gw.ptr, opt(gb), opt(gx), batch, fan_in,
+                   fan_out)
+
     def _op_outer(self, x, y, A, alpha):
         self._call("zg_hip_outer", x.ptr, x.n, y.ptr, y.n, A.ptr, alpha)
 

@@ -312,14 +312,9 @@ class MLP:
             if self.fused:
                 # g arrives with this layer's ReLU backward applied (by the product that made it); the input
                 # gradient is written, not accumulated, so it needs no zero fill
-                host.unbroadcast_(d, g, [batch, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
-                g_prev = None
-                if l > 0:
-                    g_prev = d.mem_cache_alloc(F32, batch * fan_in)
-                    d.dispatch("linear_bwd_input", gy=g, w=self.W[l], act_in=acts[l], gx=g_prev, batch=batch,
-                               fan_in=fan_in, fan_out=fan_out, accumulate=False)
-                host.bmm_acc_backward(d, False, True, acts[l], [batch, fan_in], self.W[l], [fan_out, fan_in], g,
-                                      [batch, fan_out], None, self.Wg[l])
+                g_prev = d.mem_cache_alloc(F32, batch * fan_in) if l > 0 else None
+                d.dispatch("linear_bwd", gy=g, x=acts[l], w=self.W[l], act_in=acts[l] if l > 0 else None, gw=self.Wg[l],
+                           gb=self.bg[l], gx=g_prev, batch=batch, fan_in=fan_in, fan_out=fan_out)
                 d.mem_cache_free(y)
                 d.mem_cache_free(g)
                 g = g_prev

@@ -253,8 +253,11 @@ int zg_hip_edge_plan_free(zg_hip_ctx *ctx, zg_hip_edge_plan *plan);
  * no gradient (they are data of the graph; the reference's chain stops there too, src/ndtensor.zig:1009). */
 int zg_hip_scatter_add_planned(zg_hip_ctx *ctx, const float *src, const zg_hip_edge_plan *plan, float *dst,
                                int accumulate);
+/* bias (null: none) and relu (0: none) are the tail of a graph-convolution layer, applied to every row after its
+ * edges: dst[t, :] = max(dst[t, :] + bias, 0), the `y._add(self.bias)` of examples/gcn/src/model.zig:110 and the `relu_` of :36 */
 int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx *ctx, float *dst, const float *h, const float *deg,
-                                          const zg_hip_edge_plan *plan, size_t stride, int accumulate);
+                                          const zg_hip_edge_plan *plan, const float *bias, int relu, size_t stride,
+                                          int accumulate);
 int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx *ctx, const float *grad_output, const float *h,
                                               const float *deg, const zg_hip_edge_plan *plan, float *grad_h,
                                               float *grad_deg, size_t stride, int accumulate);

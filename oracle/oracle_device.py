@@ -191,11 +191,15 @@ class OracleDevice(HipDevice):
             self.mem_fill(dst, 0.0)
         self.dispatch("scatter_add", src=src, offsets=plan.tgt_indices, dst=dst)
 
-    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride, accumulate=True):
+    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride, accumulate=True, bias=None, relu=False):
         if not accumulate:
             self.mem_fill(dst, 0.0)
         self.dispatch("scatter_gcn_deg_scaled", dst=dst, h=h, deg=deg, src_indices=plan.src_indices,
                       tgt_indices=plan.tgt_indices, stride=stride, n_edge=plan.src_indices.n)
+        if bias is not None:  # y._add(self.bias), examples/gcn/src/model.zig:110
+            self.dispatch("add", x=bias, y=dst, z=dst)
+        if relu:              # relu_ on the layer's output, examples/gcn/src/model.zig:36
+            self.dispatch("relu_fwd", x=dst, y=dst)
 
     def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride, accumulate=True):
         unused = grad_deg is None

@@ -252,6 +252,20 @@ def test_planned_scatter_ops_equal_the_unplanned_ones(oracle, hip, n_nodes, n_ed
                                                          "src_indices": src, "tgt_indices": tgt, "stride": stride,
                                                          "n_edge": n_edge}, ["dst"])["dst"]
         assert np.array_equal(got, want), (rep, "fwd fresh")
+        # the layer's tail in the same launch: + bias per column, then relu (isolated nodes get relu(bias))
+        bias = r.standard_normal(stride).astype(np.float32)
+        for relu in (False, True):
+            got = run_op(hip, "scatter_gcn_deg_scaled_planned", {"dst": nan_ns.copy(), "h": h, "deg": deg, "plan": plan,
+                                                                  "stride": stride, "accumulate": False, "bias": bias,
+                                                                  "relu": relu}, ["dst"])["dst"]
+            tail = want.reshape(n_nodes, stride) + bias[None, :]
+            tail = np.where(tail > 0, tail, np.float32(0)) if relu else tail
+            assert np.array_equal(got, tail.ravel()), (rep, "fwd tail", relu)
+            ref = run_op(oracle, "scatter_gcn_deg_scaled_planned", {"dst": nan_ns.copy(), "h": h, "deg": deg,
+                                                                    "plan": oracle.edge_plan(oracle.from_numpy(src), oracle.from_numpy(tgt), n_nodes),
+                                                                    "stride": stride, "accumulate": False, "bias": bias,
+                                                                    "relu": relu}, ["dst"])["dst"]
+            assert np.array_equal(got, ref), (rep, "fwd tail against the oracle's three ops", relu)
         want = run_op(oracle, "scatter_gcn_deg_scaled_bwd", {"grad_output": go, "h": h, "deg": deg, "src_indices": src,
                                                              "tgt_indices": tgt, "grad_h": np.zeros(n_nodes * stride, np.float32),
                                                              "grad_deg": np.zeros(n_nodes, np.float32), "stride": stride,

@@ -508,7 +508,8 @@ pub fn scatter_add_planned(self: *const Self, T: type, p: anytype) void {
 }
 pub fn scatter_gcn_deg_scaled_planned(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
-    check(c.zg_hip_scatter_gcn_deg_scaled_planned(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.stride, @intFromBool(p.accumulate)));
+    const bias: ?[*]const T = if (p.bias) |b| b.ptr else null;  // the layer's tail: + bias, then relu when asked
+    check(c.zg_hip_scatter_gcn_deg_scaled_planned(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, bias, @intFromBool(p.relu), p.stride, @intFromBool(p.accumulate)));
 }
 pub fn scatter_gcn_deg_scaled_bwd_planned(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);

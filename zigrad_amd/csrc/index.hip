@@ -318,20 +318,18 @@ __global__ __launch_bounds__(256) void row_scatter_apply_kernel(const float* src
 
 // dst[t, :] += (deg[s] * deg[t]) * h[s, :] over the edges into t, in edge order.  `peer` holds the source of each
 // edge in that order; four edges are loaded at a time (the loads do not depend on the running sum) and then added
-// one after the other.
+// one after the other.  Optional tail of a graph-convolution layer: + bias[j], then max(., 0) (the IEEE operations of
+// the separate add and relu ops).
 template <int G>
 __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const float* h, const float* deg,
                                                              const uint32_t* row_ptr, const uint32_t* peer,
-                                                             size_t n_nodes, size_t stride, bool fresh) {
+                                                             size_t n_nodes, size_t stride, bool fresh,
+                                                             const float* bias, bool relu) {
     const size_t t = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     if (t >= n_nodes) return;
     const int lane = threadIdx.x % G;
     const uint32_t s0 = row_ptr[t], s1 = row_ptr[t + 1];
-    if (s0 == s1) {
-        if (fresh)
-            for (size_t j = lane; j < stride; j += G) dst[t * stride + j] = 0.f;
-        return;
-    }
+    if (s0 == s1 && !fresh && !bias && !relu) return;
     const float dt = deg[t];
     for (size_t j = lane; j < stride; j += G) {
         float acc = fresh ? 0.f : dst[t * stride + j];
@@ -350,6 +348,8 @@ __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const fl
             for (int u = 0; u < 4; u++)
                 if (sv[u] < n_nodes) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(dv[u], dt), hv[u]));
         }
+        if (bias) acc = __fadd_rn(acc, bias[j]);
+        if (relu) acc = acc > 0.f ? acc : 0.f;
         dst[t * stride + j] = acc;
     }
 }
@@ -621,7 +621,7 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const floa
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
-                                        pl.row_ptr, pl.peer, n_nodes, stride, false));
+                                        pl.row_ptr, pl.peer, n_nodes, stride, false, (const float*)nullptr, false));
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
@@ -793,7 +793,8 @@ ZG_API int zg_hip_scatter_add_planned(zg_hip_ctx* ctx, const float* src, const z
 }
 
 ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,
-                                                 const zg_hip_edge_plan* plan, size_t stride, int accumulate) {
+                                                 const zg_hip_edge_plan* plan, const float* bias, int relu, size_t stride,
+                                                 int accumulate) {
     ZG_CTX(ctx);
     ZG_REQUIRE(plan && dst && h && deg, "scatter_gcn_deg_scaled_planned: null pointer");
     ZG_REQUIRE(stride > 0, "scatter_gcn_deg_scaled_planned: stride is 0");
@@ -801,7 +802,8 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, co
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
-                                        plan->by_tgt.row_ptr, plan->by_tgt.peer, n_nodes, stride, accumulate == 0));
+                                        plan->by_tgt.row_ptr, plan->by_tgt.peer, n_nodes, stride, accumulate == 0, bias,
+                                        relu != 0));
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, size_t 
         }
         tid += n4 << 2;
     }
-    for (size_t i = vec ? tid : tid; i < n; i += nt) {
+    for (size_t i = tid; i < n; i += nt) {
         float gv = g[i];
         if (scale) {
             gv = __fmul_rn(gv, f);

@@ -419,8 +419,9 @@ class HipDevice:
     def _op_scatter_add_planned(self, src, plan, dst, accumulate=True):
         self._call("zg_hip_scatter_add_planned", src.ptr, plan.handle, dst.ptr, int(accumulate))
 
-    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride, accumulate=True):
-        self._call("zg_hip_scatter_gcn_deg_scaled_planned", dst.ptr, h.ptr, deg.ptr, plan.handle, stride, int(accumulate))
+    def _op_scatter_gcn_deg_scaled_planned(self, dst, h, deg, plan, stride, accumulate=True, bias=None, relu=False):
+        self._call("zg_hip_scatter_gcn_deg_scaled_planned", dst.ptr, h.ptr, deg.ptr, plan.handle,
+                   bias.ptr if bias is not None else None, int(bool(relu)), stride, int(accumulate))
 
     def _op_scatter_gcn_deg_scaled_bwd_planned(self, grad_output, h, deg, plan, grad_h, grad_deg, stride, accumulate=True):
         """grad_deg may be None: the degree gradient is then not computed."""

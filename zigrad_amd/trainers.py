@@ -635,24 +635,30 @@ class GCNTrainer(GraphSteps):
             return self._deg_norm
         return deg_norm
 
-    def _conv_forward(self, l, x_in):
+    def _conv_forward(self, l, x_in, relu=False):
+        """h = x W^T, y = aggregate(h) + b (GraphConvLayer.forward, examples/gcn/src/model.zig:100-112); `relu` applies
+        the model's relu_ to y as well (:36)."""
         d, N, E = self.dev, self.N, self.E
         fan_in, fan_out = self.dims[l], self.dims[l + 1]
         h = d.mem_cache_alloc(F32, N * fan_out)
         host.bmm_acc_(d, x_in, [N, fan_in], self.W[l], [fan_out, fan_in], h, trans_a=False, trans_b=True)
         deg_norm = self._degree_norm()
         y = d.mem_cache_alloc(F32, N * fan_out)
-        if self.plan is not None:  # written, not accumulated: no zero fill
+        if self.plan is not None:  # written, not accumulated (no zero fill); bias and relu in the same launch
             d.dispatch("scatter_gcn_deg_scaled_planned", dst=y, h=h, deg=deg_norm, plan=self.plan, stride=fan_out,
-                       accumulate=False)
+                       accumulate=False, bias=self.b[l], relu=relu)
         else:
             d.mem_fill(y, 0.0)
             d.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg_norm, src_indices=self.src, tgt_indices=self.tgt,
                        stride=fan_out, n_edge=E)
-        d.dispatch("add", x=self.b[l], y=y, z=y)  # y._add(bias)
+            d.dispatch("add", x=self.b[l], y=y, z=y)  # y._add(bias)
+            if relu:
+                d.dispatch("relu_fwd", x=y, y=y)
         return {"x": x_in, "h": h, "deg": deg_norm, "y": y}
 
-    def _conv_backward(self, l, saved, g_y, need_input_grad):
+    def _conv_backward(self, l, saved, g_y, need_input_grad, act_in=None):
+        """`act_in` (fused trainer only): the ReLU output that fed this layer; its backward is then applied to the
+        input gradient by the product that writes it."""
         d, N, E = self.dev, self.N, self.E
         fan_in, fan_out = self.dims[l], self.dims[l + 1]
         host.unbroadcast_(d, g_y, [N, fan_out], self.bg[l], [fan_out], alpha=1.0, beta=1.0)
@@ -673,20 +679,22 @@ class GCNTrainer(GraphSteps):
         d.mem_cache_free(saved["y"])
         if saved["deg"] is not self._deg_norm:
             d.mem_cache_free(saved["deg"])
-        g_x = None
-        if need_input_grad:
-            g_x = d.mem_cache_alloc(F32, N * fan_in)
-            d.mem_fill(g_x, 0.0)
-        host.bmm_acc_backward(d, False, True, saved["x"], [N, fan_in], self.W[l], [fan_out, fan_in], g_h, [N, fan_out],
-                              g_x, self.Wg[l])
+        g_x = d.mem_cache_alloc(F32, N * fan_in) if need_input_grad else None
+        if self.optim.fused:  # the input gradient is written (no zero fill) with the ReLU backward applied
+            d.dispatch("linear_bwd", gy=g_h, x=saved["x"], w=self.W[l], act_in=act_in, gw=self.Wg[l], gb=None, gx=g_x,
+                       batch=N, fan_in=fan_in, fan_out=fan_out)
+        else:
+            if need_input_grad:
+                d.mem_fill(g_x, 0.0)
+            host.bmm_acc_backward(d, False, True, saved["x"], [N, fan_in], self.W[l], [fan_out, fan_in], g_h, [N, fan_out],
+                                  g_x, self.Wg[l])
         d.mem_cache_free(g_h)
         d.mem_cache_free(saved["h"])
         return g_x
 
     def step(self, keep_grads: bool = False) -> float:
         d, N, C, M = self.dev, self.N, self.dims[-1], self.n_train
-        s1 = self._conv_forward(0, self.x)
-        d.dispatch("relu_fwd", x=s1["y"], y=s1["y"])
+        s1 = self._conv_forward(0, self.x, relu=True)
         s2 = self._conv_forward(1, s1["y"])
         out_m = d.mem_cache_alloc(F32, M * C)  # MaskLayer.forward: the labelled rows, here one contiguous prefix
         d.mem_copy(s2["y"].sub(0, M * C), out_m)
@@ -709,8 +717,11 @@ class GCNTrainer(GraphSteps):
         d.mem_copy(g_m, g2.sub(0, M * C))  # MaskLayer.backward
         for t in (probs, loss, loss_grad, g_m, out_m):
             d.mem_cache_free(t)
-        g1 = self._conv_backward(1, s2, g2, need_input_grad=True)
-        d.dispatch("relu_inplace_bwd", x=s1["y"], x_g=g1)
+        if self.optim.fused:
+            g1 = self._conv_backward(1, s2, g2, need_input_grad=True, act_in=s1["y"])
+        else:
+            g1 = self._conv_backward(1, s2, g2, need_input_grad=True)
+            d.dispatch("relu_inplace_bwd", x=s1["y"], x_g=g1)
         self._conv_backward(0, s1, g1, need_input_grad=False)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]

@@ -73,7 +73,8 @@ def test_linear_bwd_input_equals_product_then_relu_backward(hip, shape, accumula
     assert np.linalg.norm(got - want) <= 1e-5 * (np.linalg.norm(want) + 1e-3), shape
 
 
-@pytest.mark.parametrize("shape", SHAPES + [(64, 4, 128), (64, 128, 2), (128, 128, 128), (256, 100, 64), (257, 100, 64)])
+@pytest.mark.parametrize("shape", SHAPES + [(64, 4, 128), (64, 128, 2), (128, 128, 128), (256, 100, 64), (257, 100, 64),
+                                            (10, 128, 1), (256, 38, 1), (1, 20, 30), (1, 1, 1)])
 @pytest.mark.parametrize("with_gx,with_gb", [(True, True), (False, True), (True, False)])
 def test_linear_bwd_equals_the_separate_ops(oracle, hip, shape, with_gx, with_gb):
     """One call against the weight-gradient product, the bias's unbroadcast and linear_bwd_input on the same device,

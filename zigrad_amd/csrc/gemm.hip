@@ -1066,7 +1066,8 @@ ZG_API int zg_hip_linear_bwd(zg_hip_ctx* ctx, const float* gy, const float* x, c
     const size_t n_cu = (size_t)ctx->n_cu;
     const bool small = gemm_is_tiny(fan_out, fan_in, batch, 1, fan_out, fan_in, n_cu) &&
                        (!gx || gemm_is_tiny(batch, fan_in, fan_out, 1, fan_out, fan_in, n_cu)) &&
-                       (!gb || batch * fan_out <= kColSingleChunkMax);
+                       // a single column or a single row takes other kernels in the separate op (row sums, a copy)
+                       (!gb || (batch > 1 && fan_out > 1 && batch * fan_out <= kColSingleChunkMax));
     if (!small) {
         if (gb) {
             const uint64_t gy_shape[2] = {batch, fan_out}, gb_shape[1] = {fan_out};

@@ -334,7 +334,7 @@ def run_small(dev, kind, steps, graph=True, fused=False):
     return out
 
 
-def run_c_harness(dims, batch, steps):
+def run_c_harness(dims, batch, steps, fused=False):
     """The same eager batch-64 step issued from plain C (tests/c_harness/mlp_step.c): what the op-by-op path costs
     without an interpreter between the calls.  None when the binary has not been built."""
     import subprocess
@@ -350,12 +350,13 @@ def run_c_harness(dims, batch, steps):
         for a in (*params, x, onehot):
             f.write(np.ascontiguousarray(a, np.float32).tobytes())
         f.flush()
-        run = subprocess.run([str(C_HARNESS_BIN), f.name, str(steps), str(batch), *map(str, dims)], capture_output=True,
-                             text=True, timeout=300)
+        run = subprocess.run([str(C_HARNESS_BIN), f.name, str(steps), str(batch), *map(str, dims), *(["fused"] if fused else [])],
+                             capture_output=True, text=True, timeout=300)
     if run.returncode != 0:
         raise RuntimeError("tests/c_harness/mlp_step failed: " + run.stderr)
     us = float(run.stdout.strip().splitlines()[-1].split()[1])
-    return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": "eager, same op sequence, caller in C"}
+    what = "eager, fused entry points, caller in C" if fused else "eager, same op sequence, caller in C"
+    return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": what}
 
 
 def cpu_baseline(dims, batch, budget_steps=2, threads=None):
@@ -462,6 +463,8 @@ def main():
             result["mlp_b64"]["clip_off"] = {"steps_per_s": 200 / nc[0], "ms_per_step": nc[0] / 200 * 1e3,
                                              "graph_replay": {"steps_per_s": 200 / nc[2], "ms_per_step": nc[2] / 200 * 1e3}}
         result["mlp_b64"]["c_caller"] = run_c_harness([784, 128, 64, 10], 64, 2000)
+        if "fused" in result["mlp_b64"]:
+            result["mlp_b64"]["fused"]["c_caller"] = run_c_harness([784, 128, 64, 10], 64, 2000, fused=True)
         result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
         result["gcn"] = run_small(dev, "gcn", 100, graph=not args.no_graph)
         result["dqn"] = run_small(dev, "dqn", 200, graph=not args.no_graph)

@@ -4,7 +4,10 @@
  * (W1 b1 W2 b2 W3 b3 x onehot), runs `steps` SGD steps (lr 0.01, per-tensor clip 10 / 1e-6), prints the loss of every
  * step and the time per step.
  *
- *   mlp_step <input.bin> <steps> <batch> <d0> <d1> <d2> <d3>
+ *   mlp_step <input.bin> <steps> <batch> <d0> <d1> <d2> <d3> [fused]
+ *
+ * With `fused` the step goes through the fused entry points instead (linear_fwd, smce_fwd_bwd, linear_bwd,
+ * sgd_step_multi): the same values in 13 launches instead of 43.
  */
 #include <stdio.h>
 #include <stdlib.h>
@@ -57,10 +60,11 @@ static void bmm(const float *A, const float *B, float *C, size_t M, size_t N, si
 }
 
 int main(int argc, char **argv) {
-    if (argc != 8) {
-        fprintf(stderr, "usage: %s input.bin steps batch d0 d1 d2 d3\n", argv[0]);
+    if (argc != 8 && argc != 9) {
+        fprintf(stderr, "usage: %s input.bin steps batch d0 d1 d2 d3 [fused]\n", argv[0]);
         return 2;
     }
+    const int fused = argc == 9;
     const int steps = atoi(argv[2]);
     const size_t B = (size_t)atol(argv[3]);
     size_t d[LAYERS + 1];
@@ -97,9 +101,39 @@ int main(int argc, char **argv) {
             CHECK(zg_hip_sync(ctx));
             clock_gettime(CLOCK_MONOTONIC, &t0);
         }
-        /* forward: y = x . W^T, y += bias, relu in place (not after the last layer) */
         cached act[LAYERS + 1];
         act[0].ptr = x;
+        if (fused) {
+            for (int l = 0; l < LAYERS; l++) {
+                act[l + 1] = cache_alloc(B * d[l + 1]);
+                CHECK(zg_hip_linear_fwd(ctx, act[l].ptr, W[l], b[l], act[l + 1].ptr, B, d[l], d[l + 1], l + 1 < LAYERS));
+            }
+            cached loss = cache_alloc(1), probs = cache_alloc(B * C), g = cache_alloc(B * C);
+            CHECK(zg_hip_smce_fwd_bwd(ctx, act[LAYERS].ptr, onehot, probs.ptr, loss.ptr, g.ptr, B, C, 0));
+            float loss_host = 0.0f;
+            CHECK(zg_hip_memcpy_d2h(ctx, &loss_host, loss.ptr, sizeof(float)));
+            printf("loss %.9g\n", loss_host);
+            cache_free(probs);
+            cache_free(loss);
+            for (int l = LAYERS - 1; l >= 0; l--) {
+                cached g_prev = {NULL, 0};
+                if (l > 0) g_prev = cache_alloc(B * d[l]);
+                CHECK(zg_hip_linear_bwd(ctx, g.ptr, act[l].ptr, W[l], l > 0 ? act[l].ptr : NULL, Wg[l], bg[l], g_prev.ptr, B,
+                                        d[l], d[l + 1]));
+                cache_free(act[l + 1]);
+                cache_free(g);
+                g = g_prev;
+            }
+            float *params[2 * LAYERS], *grads[2 * LAYERS];
+            size_t lens[2 * LAYERS];
+            for (int l = 0; l < LAYERS; l++) {
+                params[2 * l] = W[l], grads[2 * l] = Wg[l], lens[2 * l] = d[l + 1] * d[l];
+                params[2 * l + 1] = b[l], grads[2 * l + 1] = bg[l], lens[2 * l + 1] = d[l + 1];
+            }
+            CHECK(zg_hip_sgd_step_multi(ctx, 2 * LAYERS, params, grads, lens, 0.01f, 1, 10.0f, 1e-6f, 1));
+            continue;
+        }
+        /* forward: y = x . W^T, y += bias, relu in place (not after the last layer) */
         for (int l = 0; l < LAYERS; l++) {
             act[l + 1] = cache_alloc(B * d[l + 1]);
             bmm(act[l].ptr, W[l], act[l + 1].ptr, B, d[l + 1], d[l], 0, 1, d[l], d[l], 0.0f);

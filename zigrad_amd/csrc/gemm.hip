@@ -635,21 +635,26 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
 // of group g: k = 8g + 4h + c), so a k-contiguous operand is one 16-byte load per lane and group; every load is
 // guarded and zero-filled, so any shape and alignment is served.  The four partial blocks are added in wave
 // order through LDS: the result does not depend on scheduling.
-// `block` is the 32x32 block of C (row-major over tiles_n), z the batch, `part` 16 KiB of the caller's LDS.
+// `block` is the 32x32 block of C (row-major over tiles_n), z the batch, `part` 16 KiB of the caller's LDS.  With
+// g.split_tiles != 0 the workgroup takes the groups [split * split_tiles, (split + 1) * split_tiles) of k only and
+// writes its block at C + split * split_stride (the launcher points C at a buffer of partial products).
 template <bool A_KMAJOR, bool B_KMAJOR>
-__device__ __forceinline__ void gemm_tiny_block(const GemmArgs& g, unsigned block, size_t z, float (*part)[16][64]) {
+__device__ __forceinline__ void gemm_tiny_block(const GemmArgs& g, unsigned block, unsigned split, size_t z,
+                                                float (*part)[16][64]) {
     const size_t m0 = (size_t)(block / g.tiles_n) * 32, n0 = (size_t)(block % g.tiles_n) * 32;
     const float* A = g.A + (z % g.nba) * g.a_chunk;
     const float* B = g.B + (z % g.nbb) * g.b_chunk;
-    float* C = g.C + z * g.c_chunk;
+    float* C = g.C + z * g.c_chunk + (size_t)split * g.split_stride;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, lk = lane >> 5;
     const size_t K = g.K, groups = (K + 7) / 8;
+    const size_t grp_begin = (size_t)split * g.split_tiles;
+    const size_t grp_end = (g.split_tiles && grp_begin + g.split_tiles < groups) ? grp_begin + g.split_tiles : groups;
 
     auto fragment = [&](const float* P, bool kmajor, size_t ld, size_t idx, size_t limit, bool vec_ok, size_t grp) {
         floatx4 v = {0.f, 0.f, 0.f, 0.f};
         const size_t k0 = grp * 8 + (size_t)lk * 4;
-        if (idx < limit && k0 < K) {
+        if (idx < limit && grp < grp_end && k0 < K) {
             if (kmajor) {
                 const float* q = P + idx * ld + k0;
                 if (vec_ok && k0 + 4 <= K) {
@@ -676,17 +681,17 @@ __device__ __forceinline__ void gemm_tiny_block(const GemmArgs& g, unsigned bloc
     // 32 groups (k = 256) per round, 8 per wave: all of a wave's operand loads of a round are issued before its first
     // MFMA, so a round costs one memory round trip instead of one per group.  Most callers need a single round.
     constexpr int kMaxGroups = 8;
-    for (size_t base = 0; base < groups; base += 4 * kMaxGroups) {
+    for (size_t base = grp_begin; base < grp_end; base += 4 * kMaxGroups) {
         floatx4 a_frag[kMaxGroups], b_frag[kMaxGroups];
 #pragma unroll
         for (int i = 0; i < kMaxGroups; i++) {
             const size_t grp = base + (size_t)wave + 4 * (size_t)i;
-            a_frag[i] = frag_a(grp);  // zero beyond k
+            a_frag[i] = frag_a(grp);  // zero beyond the range
             b_frag[i] = frag_b(grp);
         }
 #pragma unroll
         for (int i = 0; i < kMaxGroups; i++) {
-            if (base + (size_t)wave + 4 * (size_t)i < groups) {
+            if (base + (size_t)wave + 4 * (size_t)i < grp_end) {
 #pragma unroll
                 for (int c = 0; c < 4; c++)
                     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_frag[i][c], b_frag[i][c], acc, 0, 0, 0);
@@ -718,7 +723,7 @@ __device__ __forceinline__ void gemm_tiny_block(const GemmArgs& g, unsigned bloc
 template <bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(kGemmThreads) void gemm_tiny_kernel(GemmArgs g) {
     __shared__ float part[4][16][64];
-    gemm_tiny_block<A_KMAJOR, B_KMAJOR>(g, blockIdx.x, blockIdx.z, part);
+    gemm_tiny_block<A_KMAJOR, B_KMAJOR>(g, blockIdx.x, blockIdx.y, blockIdx.z, part);
 }
 
 // The backward of a small Linear layer in one launch: the workgroups of the weight-gradient product (gw += gy^T x),
@@ -739,17 +744,19 @@ __global__ __launch_bounds__(kGemmThreads) void linear_bwd_small_kernel(LinearBw
     __shared__ float part[4][16][64];
     static_assert(sizeof(part) >= sizeof(float) * kBlock * V && kBlock == kGemmThreads, "LDS of the column sums");
     const unsigned b = blockIdx.x;
-    if (b < a.n_w) gemm_tiny_block<false, false>(a.gw, b, 0, part);
-    else if (b < a.n_w + a.n_x) gemm_tiny_block<true, false>(a.gx, b - a.n_w, 0, part);
+    if (b < a.n_w) gemm_tiny_block<false, false>(a.gw, b, 0, 0, part);
+    else if (b < a.n_w + a.n_x) gemm_tiny_block<true, false>(a.gx, b - a.n_w, 0, 0, part);
     else
         col_reduce_block<AxisSum, V>(a.gy, a.gb, nullptr, a.R, a.inner, a.log2_cx, a.R, 1.f, 1.f, b - a.n_w - a.n_x, 0, 0,
                                      1, &part[0][0][0]);
 }
 
-static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, size_t batches) {
+static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, size_t batches,
+                            size_t splits = 1) {
     g.tiles_m = (unsigned)ceil_div_sz(g.M, 32);
     g.tiles_n = (unsigned)ceil_div_sz(g.N, 32);
-    dim3 grid(g.tiles_m * g.tiles_n, 1, (unsigned)batches), block(kGemmThreads);
+    if (splits == 1) g.split_tiles = g.split_stride = 0;  // the whole of k in one workgroup per block
+    dim3 grid(g.tiles_m * g.tiles_n, (unsigned)splits, (unsigned)batches), block(kGemmThreads);
     if (a_kmajor && b_kmajor) hipLaunchKernelGGL((gemm_tiny_kernel<true, true>), grid, block, 0, ctx->stream, g);
     else if (a_kmajor && !b_kmajor) hipLaunchKernelGGL((gemm_tiny_kernel<true, false>), grid, block, 0, ctx->stream, g);
     else if (!a_kmajor && b_kmajor) hipLaunchKernelGGL((gemm_tiny_kernel<false, true>), grid, block, 0, ctx->stream, g);
@@ -901,6 +908,39 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
 
     if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
     if (gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
+    // Skinny weight-gradient products with a long k (one side of C at most 32 wide, both operands stored k-strided:
+    // the 16-wide layer of the GCN, 16 x 1433 over 2708 nodes): 64-wide tiles would compute mostly padding, so the
+    // unstaged kernel takes ranges of k (one round of 256 per workgroup, at most 32 ranges) and the split-k reduction
+    // adds the partial blocks: 11.9 us against 15.3 us.  With a k-contiguous operand the unstaged kernel's loads are
+    // 16 bytes per row and lane, which costs more than the padding (2708 x 16 x 1433: 17.8 us against 14.1 us).
+    if (!a_kmajor && !b_kmajor && (m <= 32 || n <= 32) && k > 512 && tiles(32, 32) <= n_cu) {
+        const size_t groups = ceil_div_sz(k, 8);
+        size_t splits = ceil_div_sz(groups, 32);
+        if (splits > 32) splits = 32;
+        size_t per = ceil_div_sz(groups, splits);
+        per = (per + 3) & ~(size_t)3;  // whole turns of the four waves
+        splits = ceil_div_sz(groups, per);
+        float* part = (float*)workspace(ctx, batches * splits * m * n * sizeof(float));
+        if (!part) return ZG_HIP_EOOM;
+        GemmArgs gs = g;
+        gs.C = part;
+        gs.ldc = n;
+        gs.c_chunk = splits * m * n;
+        gs.split_tiles = per;
+        gs.split_stride = m * n;
+        gs.alpha = 1.f;
+        gs.beta = 0.f;
+        gs.bias = nullptr;  // the extras belong to the sum of the partial products: the reduce kernel applies them
+        gs.gate = nullptr;
+        gs.relu = 0;
+        if (int rc = launch_gemm_tiny(ctx, gs, a_kmajor, b_kmajor, batches, splits)) return rc;
+        size_t blocks = ceil_div_sz(m * n, 256);
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks, 1, (unsigned)batches), dim3(256), 0, ctx->stream,
+                           part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk, g.bias, g.gate, g.relu);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
 
     const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
     if (c_large <= c_mid && c_large <= c_small)

@@ -1,5 +1,6 @@
 // fp32 GEMM family on the CDNA4 matrix cores: matmul, bmm_acc (all four transpose variants, alpha/beta,
-// explicit leading dimensions), matvec, outer, transpose.
+// explicit leading dimensions), the fused Linear entry points built on them (forward with bias and ReLU in the
+// epilogue, masked input gradient, a small layer's whole backward in one launch), matvec, outer, transpose.
 //
 // Reference semantics: cblas_sgemm(RowMajor, ...) as called from src/device/host_device.zig:242-250 and
 // the batch loop of :277-313.

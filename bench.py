@@ -386,6 +386,10 @@ def main():
     ap.add_argument("--no-ops", action="store_true", help="skip the op microbenchmark suite")
     ap.add_argument("--loss-mode", default="onehot", choices=["onehot", "label"])
     ap.add_argument("--no-small", action="store_true", help="skip the latency-bound configurations (keeps profiler output small)")
+    ap.add_argument("--trace-small", choices=["mlp_b64", "gcn", "dqn"],
+                    help="run 30 eager steps of one latency-bound configuration and exit (for rocprofv3 --kernel-trace: "
+                         "the profiler cannot trace graph replays, the eager steps launch the same kernels)")
+    ap.add_argument("--trace-fused", action="store_true", help="with --trace-small: through the fused entry points")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the execution-graph replays (rocprofv3's kernel tracing crashes inside hipGraphLaunch)")
     args = ap.parse_args()
@@ -396,6 +400,28 @@ def main():
     from zigrad_amd import HipDevice
 
     dev = HipDevice(0)
+    if args.trace_small:
+        from zigrad_amd.trainers import DQNTrainer, GCNTrainer, MLPTrainer, dqn_inputs, gcn_inputs, mlp_inputs
+
+        if args.trace_small == "mlp_b64":
+            dims, batch = [784, 128, 64, 10], 64
+            params, x, onehot, labels = mlp_inputs(dims, batch, data="uniform")
+            tr = MLPTrainer(dev, dims, batch, optimizer="sgd", lr=0.01, clip=True, fused=args.trace_fused)
+            tr.load_params(params)
+            tr.set_batch(x, onehot, labels)
+        elif args.trace_small == "gcn":
+            tr = GCNTrainer(dev, gcn_inputs(seed=0), lr=0.01, clip=True, fused=args.trace_fused)
+        else:
+            dims, batch = [4, 128, 128, 2], 64
+            params, _, _, _ = mlp_inputs(dims, batch)
+            tr = DQNTrainer(dev, dims, batch, lr=1e-3, gamma=0.99, clip=True, fused=args.trace_fused)
+            tr.load_params(params)
+            tr.set_batch(dqn_inputs(batch=batch))
+        for _ in range(30):
+            tr.step()
+        dev.sync()
+        print(json.dumps({"traced": args.trace_small, "fused": args.trace_fused, "steps": 30}))
+        return
     copy_calibration(dev)
     timer = GemmTimer(dev)
     timer.install()

@@ -215,6 +215,10 @@ int zg_hip_broadcast(zg_hip_ctx *ctx, const float *x, size_t xl, float *y, size_
  * 0 ok, 1 InvalidIndexShape, 2 IndexOutOfBounds */
 int zg_hip_gather_offsets(zg_hip_ctx *ctx, const uint64_t *src_shape, const uint64_t *idx_shape, size_t rank,
                           const uint64_t *indices, size_t dim, uint64_t *offsets, int *status);
+/* the whole of NDArray.gather (src/ndarray.zig:593-633) in one launch: the offsets as above (kept: the backward
+ * scatters through them) and dst[i] = src[offsets[i]] */
+int zg_hip_gather(zg_hip_ctx *ctx, const float *src, const uint64_t *src_shape, const uint64_t *idx_shape, size_t rank,
+                  const uint64_t *indices, size_t dim, uint64_t *offsets, float *dst, int *status);
 int zg_hip_scatter_add(zg_hip_ctx *ctx, const float *src, const uint64_t *offsets, size_t n, float *dst,
                        size_t dst_len);
 int zg_hip_index_select_fwd(zg_hip_ctx *ctx, const float *src, size_t src_len, const uint64_t *indices, size_t n_idx,

@@ -288,6 +288,13 @@ class OracleDevice(HipDevice):
         ish, _ = _shape(idx_shape)
         return int(self._o.cdll.zo_gather_offsets(ss, ish, r, indices.ptr, dim, offsets.ptr))
 
+    def gather(self, src, src_shape, idx_shape, indices, dim, offsets, dst, check=True):
+        # NDArray.gather (src/ndarray.zig:593-633): the offsets loop, then mem_take
+        status = self.gather_offsets(src_shape, idx_shape, indices, dim, offsets, check=check)
+        if status == 0:
+            self.mem_take(src, offsets, dst)
+        return status
+
     def unbroadcast_scratch_len(self, x_shape, y_shape):
         from zigrad_amd.device import _shape
 

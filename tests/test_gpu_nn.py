@@ -195,6 +195,44 @@ def test_gather_offsets_bit_exact(oracle, hip):
         np.testing.assert_array_equal(res[1], want.ravel().astype(np.uint64))
 
 
+def test_gather_in_one_launch_equals_offsets_then_take(oracle, hip):
+    """zg_hip_gather against gather_offsets + mem_take on the device and against the oracle's host loops, bit for bit;
+    an index beyond the source's dim is reported when the status is asked for."""
+    from zigrad_amd.device import F32, U64
+
+    r = rng(2)
+    for src_shape, idx_shape, dim in [([64, 2], [64, 1], 1), ([5, 6, 7], [5, 4, 7], 1), ([5, 6, 7], [3, 6, 2], 0), ([9], [4], 0),
+                                       ([300, 40], [300, 40], 1)]:
+        n = int(np.prod(idx_shape))
+        idx = r.integers(0, src_shape[dim], n).astype(np.uint64)
+        src = r.standard_normal(int(np.prod(src_shape))).astype(np.float32)
+        res = []
+        for dev in (oracle, hip):
+            S, I = dev.from_numpy(src), dev.from_numpy(idx)
+            O, D = dev.from_numpy(np.zeros(n, np.uint64)), dev.from_numpy(np.full(n, np.nan, np.float32))
+            assert dev.gather(S, src_shape, idx_shape, I, dim, O, D, check=(n % 2 == 0)) == 0
+            dev.sync()
+            res.append((dev.to_numpy(O), dev.to_numpy(D)))
+        O2, D2 = hip.from_numpy(np.zeros(n, np.uint64)), hip.from_numpy(np.full(n, np.nan, np.float32))
+        S, I = hip.from_numpy(src), hip.from_numpy(idx)
+        assert hip.gather_offsets(src_shape, idx_shape, I, dim, O2) == 0
+        hip.mem_take(S, O2, D2)
+        hip.sync()
+        np.testing.assert_array_equal(res[1][0], hip.to_numpy(O2))
+        np.testing.assert_array_equal(res[1][1], hip.to_numpy(D2))
+        np.testing.assert_array_equal(res[0][0], res[1][0])
+        np.testing.assert_array_equal(res[0][1], res[1][1])
+        want = np.take_along_axis(src.reshape(src_shape)[tuple(slice(0, s) if i != dim else slice(None) for i, s in enumerate(idx_shape))],
+                                  idx.reshape(idx_shape).astype(np.int64), axis=dim)
+        np.testing.assert_array_equal(res[1][1], want.ravel())
+    bad = np.array([0, 1, 7, 1], np.uint64)  # 7 >= 2
+    S, I = hip.from_numpy(np.arange(8, dtype=np.float32)), hip.from_numpy(bad)
+    O, D = hip.from_numpy(np.zeros(4, np.uint64)), hip.from_numpy(np.zeros(4, np.float32))
+    assert hip.gather(S, [4, 2], [4, 1], I, 1, O, D, check=True) == 2
+    assert hip.gather(S, [4, 2], [4, 1], I, 1, O, D, check=False) == 0  # unchecked: the bad entry is skipped silently
+    hip.sync()
+
+
 @pytest.mark.parametrize("n,dst_len", [(64, 128), (13264, 2708), (100000, 17), (5000, 300000), (1, 1), (40000, 5000),
                                         (256, 7), (257, 7), (200, 1), (255, 1000)])
 def test_scatter_add_bit_exact(oracle, hip, n, dst_len):

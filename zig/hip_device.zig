@@ -434,6 +434,16 @@ pub fn scatter_gcn_deg_scaled_bwd(self: *const Self, T: type, p: opspec.scatter_
 //   sgd_step / adam_step                                     src/nn/optim.zig:100-122, 177-234
 //   argmax_along, gather_offsets, index_select_fwd / _bwd    examples/mnist/src/main-simple.zig:124, src/ndarray.zig:607-624,
 //                                                            src/ndtensor.zig:1437-1513
+/// NDArray.gather (src/ndarray.zig:593-633) as one device op: the offsets (kept for the backward's scatter_add) and
+/// the gathered values.  `p.check` reads the out-of-bounds status back (one blocking 4-byte copy).
+pub fn gather(self: *const Self, T: type, p: anytype) !void {
+    comptime only_f32(T);
+    var status: c_int = 0;
+    const rc = c.zg_hip_gather(self.ctx, p.src.ptr, @ptrCast(p.src_shape.ptr), @ptrCast(p.idx_shape.ptr), p.src_shape.len, @ptrCast(p.indices.ptr), p.dim, @ptrCast(p.offsets.ptr), p.dst.ptr, if (p.check) &status else null);
+    if (status == 1) return error.InvalidIndexShape;
+    if (status == 2) return error.IndexOutOfBounds;
+    check(rc);
+}
 pub fn smce_fwd(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
     check(c.zg_hip_smce_fwd(self.ctx, p.logits.ptr, p.target.ptr, p.probs.ptr, p.loss.ptr, p.rows, p.cols));

@@ -440,8 +440,11 @@ __global__ void gcn_bwd_graddeg_kernel(float* grad_deg, const float* term_src, c
 struct GatherMeta {
     uint64_t v[24];  // [idx_strides(8) | src_strides(8) | src_shape(8)]
 };
+// offsets[i] = flat position in the source of idx coordinate i with its `dim` coordinate replaced by indices[i]
+// (src/ndarray.zig:607-624); with `src` the values are taken in the same pass (mem_take, :625-633).  An index
+// beyond the source's dim raises the status flag (when there is one) and yields offset 0 and no value.
 __global__ void gather_offsets_kernel(const uint64_t* indices, size_t n, int rank, size_t dim, GatherMeta gm,
-                                      uint64_t* offsets, int* status) {
+                                      uint64_t* offsets, int* status, const float* src, float* dst) {
     const uint64_t* meta = gm.v;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
@@ -457,10 +460,11 @@ __global__ void gather_offsets_kernel(const uint64_t* indices, size_t n, int ran
         off += c * meta[8 + d];
     }
     if (bad) {
-        *status = 2;
+        if (status) *status = 2;
         offsets[i] = 0;
     } else {
         offsets[i] = off;
+        if (src) dst[i] = src[off];
     }
 }
 
@@ -496,16 +500,16 @@ static int group_for(size_t stride) {
 
 using namespace zg;
 
-ZG_API int zg_hip_gather_offsets(zg_hip_ctx* ctx, const uint64_t* src_shape, const uint64_t* idx_shape, size_t rank,
-                                 const uint64_t* indices, size_t dim, uint64_t* offsets, int* status) {
-    ZG_CTX(ctx);
-    ZG_REQUIRE(src_shape && idx_shape && indices && offsets, "gather_offsets: null pointer");
-    ZG_REQUIRE(rank >= 1 && rank <= 8 && dim < rank, "gather_offsets: bad rank %zu / dim %zu", rank, dim);
+static int gather_impl(zg_hip_ctx* ctx, const char* name, const uint64_t* src_shape, const uint64_t* idx_shape, size_t rank,
+                       const uint64_t* indices, size_t dim, uint64_t* offsets, int* status, const float* src,
+                       float* dst) {
+    ZG_REQUIRE(src_shape && idx_shape && indices && offsets, "%s: null pointer", name);
+    ZG_REQUIRE(rank >= 1 && rank <= 8 && dim < rank, "%s: bad rank %zu / dim %zu", name, rank, dim);
     if (status) *status = 0;
     for (size_t i = 0; i < rank; i++) {
         if (i != dim && idx_shape[i] > src_shape[i]) {  // src/ndarray.zig:602-604
             if (status) *status = 1;
-            set_error("gather_offsets: InvalidIndexShape at dim %zu", i);
+            set_error("%s: InvalidIndexShape at dim %zu", name, i);
             return ZG_HIP_EINVAL;
         }
     }
@@ -522,25 +526,41 @@ ZG_API int zg_hip_gather_offsets(zg_hip_ctx* ctx, const uint64_t* src_shape, con
     }
     const size_t n = (size_t)a;
     if (n == 0) return ZG_HIP_OK;
-    int* d_status = (int*)(ctx->scalar_slot + 2);
-    hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(64), 0, ctx->stream, (uint32_t*)d_status, (size_t)1,
-                       (uint32_t*)nullptr, (size_t)0);
-    ZG_LAUNCH_CHECK();
+    // the out-of-bounds flag costs a launch to clear, so it exists only for callers that read it
+    int* d_status = status ? (int*)(ctx->scalar_slot + 2) : nullptr;
+    if (d_status) {
+        hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(64), 0, ctx->stream, (uint32_t*)d_status, (size_t)1,
+                           (uint32_t*)nullptr, (size_t)0);
+        ZG_LAUNCH_CHECK();
+    }
     hipLaunchKernelGGL(gather_offsets_kernel, dim3((unsigned)ceil_div_sz(n, 256)), dim3(256), 0, ctx->stream, indices, n,
-                       (int)rank, dim, gm, offsets, d_status);
+                       (int)rank, dim, gm, offsets, d_status, src, dst);
     ZG_LAUNCH_CHECK();
     if (status) {
-        ZG_NOT_CAPTURING(ctx, "gather_offsets with a status read-back");
+        ZG_NOT_CAPTURING(ctx, "a gather with a status read-back");
         int h = 0;
         ZG_HIP_TRY(hipMemcpyAsync(&h, d_status, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
         *status = h;
         if (h) {
-            set_error("gather_offsets: IndexOutOfBounds");
+            set_error("%s: IndexOutOfBounds", name);
             return ZG_HIP_EINVAL;
         }
     }
     return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_gather_offsets(zg_hip_ctx* ctx, const uint64_t* src_shape, const uint64_t* idx_shape, size_t rank,
+                                 const uint64_t* indices, size_t dim, uint64_t* offsets, int* status) {
+    ZG_CTX(ctx);
+    return gather_impl(ctx, "gather_offsets", src_shape, idx_shape, rank, indices, dim, offsets, status, nullptr, nullptr);
+}
+
+ZG_API int zg_hip_gather(zg_hip_ctx* ctx, const float* src, const uint64_t* src_shape, const uint64_t* idx_shape,
+                         size_t rank, const uint64_t* indices, size_t dim, uint64_t* offsets, float* dst, int* status) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(src && dst, "gather: null pointer");
+    return gather_impl(ctx, "gather", src_shape, idx_shape, rank, indices, dim, offsets, status, src, dst);
 }
 
 ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t* offsets, size_t n, float* dst,

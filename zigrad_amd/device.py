@@ -380,6 +380,21 @@ class HipDevice:
             raise
         return st.value
 
+    def gather(self, src: DevBuf, src_shape, idx_shape, indices: DevBuf, dim: int, offsets: DevBuf, dst: DevBuf,
+               check: bool = True) -> int:
+        """Offsets and values of NDArray.gather in one launch; returns the status gather_offsets returns."""
+        ss, r = _shape(src_shape)
+        ish, _ = _shape(idx_shape)
+        st = ctypes.c_int(0)
+        try:
+            self._call("zg_hip_gather", src.ptr, ss, ish, r, indices.ptr, dim, offsets.ptr, dst.ptr,
+                       ctypes.byref(st) if check else None)
+        except ZgHipError:
+            if st.value:
+                return st.value
+            raise
+        return st.value
+
     def _op_scatter_add(self, src, offsets, dst):
         if offsets.n != src.n:
             raise ValueError("scatter_add: offsets.len != src.len")

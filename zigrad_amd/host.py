@@ -122,15 +122,12 @@ def gather(dev, src: DevBuf, src_shape, indices: DevBuf, idx_shape, dim: int, re
     # the reference takes the offsets from the raw allocator (its own "TODO: cache?"); on a GPU that would be a
     # hipMalloc/hipFree pair per call, so they come from the caching allocator (free with mem_cache_free)
     offsets = dev.mem_cache_alloc(U64, n)
-    status = dev.gather_offsets(src_shape, idx_shape, indices, dim, offsets, check=check)
-    if status == 1:
-        dev.mem_cache_free(offsets)
-        raise ValueError("InvalidIndexShape")
-    if status == 2:
-        dev.mem_cache_free(offsets)
-        raise IndexError("IndexOutOfBounds")
     values = dev.mem_cache_alloc(F32, n)
-    dev.mem_take(src, offsets, values)
+    status = dev.gather(src, src_shape, idx_shape, indices, dim, offsets, values, check=check)
+    if status:
+        dev.mem_cache_free(values)
+        dev.mem_cache_free(offsets)
+        raise ValueError("InvalidIndexShape") if status == 1 else IndexError("IndexOutOfBounds")
     if return_offsets:
         return values, offsets
     dev.mem_cache_free(offsets)

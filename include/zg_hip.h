@@ -289,6 +289,10 @@ int zg_hip_softmax_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t rows, s
 int zg_hip_softmax_bwd(zg_hip_ctx *ctx, const float *y, const float *y_g, float *x_g, size_t rows, size_t cols);
 int zg_hip_smooth_l1_fwd(zg_hip_ctx *ctx, const float *pred, const float *target, size_t n, float beta, float *loss);
 int zg_hip_smooth_l1_bwd(zg_hip_ctx *ctx, const float *pred, const float *target, float *grad, size_t n, float beta);
+/* smooth_l1_fwd followed by the backward of the scalar loss (upstream gradient 1): grad (+)= d loss / d pred; one
+ * launch for up to 4096 elements.  accumulate == 0: grad is written, not read. */
+int zg_hip_smooth_l1_fwd_bwd(zg_hip_ctx *ctx, const float *pred, const float *target, float *grad, size_t n, float beta,
+                             float *loss, int accumulate);
 int zg_hip_mse_fwd(zg_hip_ctx *ctx, const float *pred, const float *target, size_t n, float *loss);
 int zg_hip_mse_bwd(zg_hip_ctx *ctx, const float *pred, const float *target, float *grad, size_t n);
 

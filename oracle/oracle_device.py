@@ -269,6 +269,13 @@ class OracleDevice(HipDevice):
     def _x_zg_hip_scatter_gcn_deg_scaled_bwd(self, go, h, deg, s, t, gh, gd, stride, n_edge, n_nodes):
         return self._o.cdll.zo_scatter_gcn_deg_scaled_bwd(go, h, deg, s, t, gh, gd, stride, n_edge)
 
+    def _x_zg_hip_smooth_l1_fwd_bwd(self, pred, target, grad, n, beta, loss, accumulate):
+        # the forward followed by the loss's backward with an upstream gradient of 1 (src/nn/loss.zig:259-305)
+        if not accumulate:
+            ctypes.memset(grad, 0, n * 4)
+        self._o.cdll.zo_smooth_l1_fwd(pred, target, n, beta, loss)
+        self._o.cdll.zo_smooth_l1_bwd(pred, target, grad, n, beta)
+
     def _x_zg_hip_smce_fwd_bwd(self, logits, target, probs, loss, grad, rows, cols, accumulate):
         # the forward followed by CceBwd with an upstream gradient of 1 (src/nn/loss.zig:130-159)
         if not accumulate:

@@ -303,3 +303,30 @@ def test_smce_fwd_bwd_equals_forward_then_backward(oracle, hip, rows, cols, accu
     p_label = np.clip(np.exp((x * target).sum(axis=1) - lse), 1e-7, np.float64(np.float32(1.0 - 1e-7)))  # the clamp of loss.zig:143
     want = np.mean(-np.log(p_label))
     assert abs(float(got["loss"][0]) - want) <= 1e-5 * (abs(want) + 1e-3)
+
+
+@pytest.mark.parametrize("n", [1, 64, 4096, 4097, 100001])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_smooth_l1_fwd_bwd_equals_forward_then_backward(oracle, hip, n, accumulate):
+    """One call against smooth_l1_fwd + smooth_l1_bwd (src/nn/loss.zig:259-305) on the same device, bit for bit, on
+    both sides of the one-launch limit; against the closed form and the CPU oracle's composition to 1e-5."""
+    r = np.random.default_rng(n)
+    pred = (2.0 * r.standard_normal(n)).astype(np.float32)
+    target = r.standard_normal(n).astype(np.float32)
+    g0 = r.standard_normal(n).astype(np.float32)
+    p = {"pred": pred, "target": target, "grad": g0.copy() if accumulate else np.full(n, np.nan, np.float32), "beta": 1.0,
+         "loss": np.full(1, np.nan, np.float32), "accumulate": accumulate}
+    got = run_op(hip, "smooth_l1_fwd_bwd", dict(p), ["grad", "loss"])
+    fwd = run_op(hip, "smooth_l1_fwd", {"pred": pred, "target": target, "beta": 1.0, "loss": np.zeros(1, np.float32)}, ["loss"])
+    bwd = run_op(hip, "smooth_l1_bwd", {"pred": pred, "target": target, "grad": g0.copy() if accumulate else np.zeros(n, np.float32),
+                                        "beta": 1.0}, ["grad"])
+    assert np.array_equal(got["loss"], fwd["loss"])
+    assert np.array_equal(got["grad"], bwd["grad"])
+    d = pred.astype(np.float64) - target
+    want_loss = np.mean(np.where(np.abs(d) < 1.0, 0.5 * d * d, np.abs(d) - 0.5))
+    want_grad = np.where(np.abs(d) < 1.0, d, np.sign(d)) / n + (g0 if accumulate else 0.0)
+    assert abs(float(got["loss"][0]) - want_loss) <= 1e-5 * (abs(want_loss) + 1e-6)
+    assert np.linalg.norm(got["grad"] - want_grad) <= 1e-5 * (np.linalg.norm(want_grad) + 1e-9)
+    ref = run_op(oracle, "smooth_l1_fwd_bwd", dict(p), ["grad", "loss"])
+    assert np.linalg.norm(got["grad"] - ref["grad"]) <= 1e-5 * (np.linalg.norm(ref["grad"]) + 1e-9)
+    assert abs(float(got["loss"][0]) - float(ref["loss"][0])) <= 1e-5 * (abs(float(ref["loss"][0])) + 1e-6)

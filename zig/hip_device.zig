@@ -461,6 +461,11 @@ pub fn smooth_l1_fwd(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
     check(c.zg_hip_smooth_l1_fwd(self.ctx, p.pred.ptr, p.target.ptr, p.pred.len, p.beta, p.loss.ptr));
 }
+/// smooth_l1_fwd and the backward of the scalar loss in one call: p.grad (+)= d loss / d pred.
+pub fn smooth_l1_fwd_bwd(self: *const Self, T: type, p: anytype) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smooth_l1_fwd_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len, p.beta, p.loss.ptr, @intFromBool(p.accumulate)));
+}
 pub fn smooth_l1_bwd(self: *const Self, T: type, p: anytype) void {
     comptime only_f32(T);
     check(c.zg_hip_smooth_l1_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len, p.beta));

@@ -78,6 +78,15 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 inline int ceil_div(size_t a, size_t b) {
     return (int)((a + b - 1) / b);
 }
+// d(mean smooth-L1)/d(pred) of one element (src/nn/loss.zig:259-305): (pred - target) / (beta * n) where
+// |pred - target| < beta, sign(pred - target) / n elsewhere
+__device__ __forceinline__ float smooth_l1_grad(float pred, float target, float beta, float n) {
+    const float d = __fsub_rn(pred, target);
+    if (fabsf(d) < beta) return __fdiv_rn(d, __fmul_rn(beta, n));
+    const float sg = (d > 0.f) ? 1.f : ((d < 0.f) ? -1.f : 0.f);
+    return __fdiv_rn(sg, n);
+}
+
 inline size_t ceil_div_sz(size_t a, size_t b) {
     return (a + b - 1) / b;
 }

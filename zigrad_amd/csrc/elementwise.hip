@@ -278,9 +278,7 @@ ZG_OP(ScaleOp, return __fmul_rn(a, p0);)
 ZG_OP(ScaledCopy, return __fadd_rn(__fmul_rn(p0, a), __fmul_rn(p1, b));)
 ZG_OP(ScaledCopyNoRead, return __fmul_rn(p0, a);)
 // smooth-l1 / mse backward: a = pred, b = target, c = grad; p0 = beta or scale, p1 = n
-ZG_OP(SmoothL1Bwd, float d = __fsub_rn(a, b);
-      if (fabsf(d) < p0) return __fadd_rn(c, __fdiv_rn(d, __fmul_rn(p0, p1)));
-      float sg = (d > 0.f) ? 1.f : ((d < 0.f) ? -1.f : 0.f); return __fadd_rn(c, __fdiv_rn(sg, p1));)
+ZG_OP(SmoothL1Bwd, return __fadd_rn(c, smooth_l1_grad(a, b, p0, p1));)
 ZG_OP(MseBwd, return __fadd_rn(c, __fmul_rn(p0, __fsub_rn(a, b)));)
 
 }  // namespace zg

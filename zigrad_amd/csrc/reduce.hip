@@ -320,6 +320,43 @@ ZG_API int zg_hip_smooth_l1_fwd(zg_hip_ctx* ctx, const float* pred, const float*
     return flat_reduce<TermSmoothL1, 2>(ctx, pred, target, n, beta, FinDivN{loss, (float)n});
 }
 
+// smooth_l1_fwd followed by the backward of the scalar loss (upstream gradient 1): grad (+)= d loss / d pred.  Up to
+// kSmoothL1SmallMax elements take one launch of one workgroup, which forms the mean as flat_single_kernel does and
+// the gradient elements as the separate backward op does; larger inputs take the separate launches.
+constexpr size_t kSmoothL1SmallMax = 4096;
+template <bool ACC>
+__global__ __launch_bounds__(kFlatSingle) void smooth_l1_small_kernel(const float* pred, const float* target, float* grad,
+                                                                      size_t n, float beta, float* loss) {
+    __shared__ float smem[kFlatSingle / kWave];
+    float acc = flat_accumulate<TermSmoothL1, 2>(pred, target, n, beta, threadIdx.x, blockDim.x);
+    acc = block_reduce<SumAcc>(acc, smem);
+    if (threadIdx.x == 0) FinDivN{loss, (float)n}(acc);
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float d = smooth_l1_grad(pred[i], target[i], beta, (float)n);
+        grad[i] = ACC ? __fadd_rn(grad[i], d) : d;
+    }
+}
+
+ZG_API int zg_hip_smooth_l1_fwd_bwd(zg_hip_ctx* ctx, const float* pred, const float* target, float* grad, size_t n,
+                                    float beta, float* loss, int accumulate) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(pred && target && grad && loss && n > 0, "smooth_l1_fwd_bwd: null or empty operand");
+    if (n <= kSmoothL1SmallMax) {
+        if (accumulate)
+            hipLaunchKernelGGL(smooth_l1_small_kernel<true>, dim3(1), dim3(kFlatSingle), 0, ctx->stream, pred, target, grad, n,
+                               beta, loss);
+        else
+            hipLaunchKernelGGL(smooth_l1_small_kernel<false>, dim3(1), dim3(kFlatSingle), 0, ctx->stream, pred, target, grad,
+                               n, beta, loss);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    if (int rc = zg_hip_smooth_l1_fwd(ctx, pred, target, n, beta, loss)) return rc;
+    if (!accumulate)
+        if (int rc = zg_hip_mem_fill(ctx, grad, n, 0.f)) return rc;
+    return zg_hip_smooth_l1_bwd(ctx, pred, target, grad, n, beta);
+}
+
 ZG_API int zg_hip_mse_fwd(zg_hip_ctx* ctx, const float* pred, const float* target, size_t n, float* loss) {
     ZG_CTX(ctx);
     ZG_REQUIRE(pred && target && loss && n > 0, "mse_fwd: null or empty operand");

@@ -469,6 +469,9 @@ class HipDevice:
     def _op_smooth_l1_bwd(self, pred, target, grad, beta):
         self._call("zg_hip_smooth_l1_bwd", pred.ptr, target.ptr, grad.ptr, pred.n, beta)
 
+    def _op_smooth_l1_fwd_bwd(self, pred, target, grad, beta, loss, accumulate=True):
+        self._call("zg_hip_smooth_l1_fwd_bwd", pred.ptr, target.ptr, grad.ptr, pred.n, beta, loss.ptr, int(bool(accumulate)))
+
     def _op_mse_fwd(self, pred, target, loss): self._call("zg_hip_mse_fwd", pred.ptr, target.ptr, pred.n, loss.ptr)
     def _op_mse_bwd(self, pred, target, grad): self._call("zg_hip_mse_bwd", pred.ptr, target.ptr, grad.ptr, pred.n)
 

@@ -515,15 +515,19 @@ class DQNTrainer(GraphSteps):
         q_all = acts[-1]
         q, offsets = host.gather(d, q_all, [B, A], self.actions, [B, 1], 1, return_offsets=True, check=False)
         loss = d.mem_cache_alloc(F32, 1)
-        d.dispatch("smooth_l1_fwd", pred=q, target=targets, beta=1.0, loss=loss)
-        if not self.optim.fused:  # the fused optimizer step leaves the gradients zero for the next step
-            self.policy.zero_grad()
-        # backward
         loss_grad = d.mem_cache_alloc(F32, 1)
-        d.mem_fill(loss_grad, 1.0)
         g_q = d.mem_cache_alloc(F32, B)
-        d.mem_fill(g_q, 0.0)
-        d.dispatch("smooth_l1_bwd", pred=q, target=targets, grad=g_q, beta=1.0)
+        if self.optim.fused:
+            # forward and the loss's backward in one call, the gradient written (no fills); the fused optimizer step
+            # leaves the parameter gradients zero for the next step
+            d.dispatch("smooth_l1_fwd_bwd", pred=q, target=targets, grad=g_q, beta=1.0, loss=loss, accumulate=False)
+        else:
+            d.dispatch("smooth_l1_fwd", pred=q, target=targets, beta=1.0, loss=loss)
+            self.policy.zero_grad()
+            # backward
+            d.mem_fill(loss_grad, 1.0)
+            d.mem_fill(g_q, 0.0)
+            d.dispatch("smooth_l1_bwd", pred=q, target=targets, grad=g_q, beta=1.0)
         g_all = d.mem_cache_alloc(F32, B * A)
         d.mem_fill(g_all, 0.0)
         d.dispatch("scatter_add", src=g_q, offsets=offsets, dst=g_all)  # GatherBwd, src/ndtensor.zig:1367-1380

@@ -120,3 +120,29 @@ def test_oracle_list_optimizers_follow_the_per_tensor_recurrence(oracle, kind):
     # the clip rescaled the second gradient in place to max_norm, and left the others alone
     assert abs(np.linalg.norm(oracle.to_numpy(G[1]).astype(np.float64)) - max_norm) <= 1e-3
     assert np.array_equal(oracle.to_numpy(G[0]), g0[0])
+
+
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_oracle_smooth_l1_fwd_bwd(oracle, accumulate):
+    r = np.random.default_rng(9)
+    n = 200
+    pred, target = (2.0 * r.standard_normal(n)).astype(np.float32), r.standard_normal(n).astype(np.float32)
+    g0 = r.standard_normal(n).astype(np.float32)
+    got = run_op(oracle, "smooth_l1_fwd_bwd", {"pred": pred, "target": target, "grad": g0.copy() if accumulate else np.full(n, np.nan, np.float32),
+                                               "beta": 1.0, "loss": np.full(1, np.nan, np.float32), "accumulate": accumulate},
+                 ["grad", "loss"])
+    d = pred.astype(np.float64) - target
+    assert abs(float(got["loss"][0]) - np.mean(np.where(np.abs(d) < 1.0, 0.5 * d * d, np.abs(d) - 0.5))) <= 1e-6
+    assert _close(got["grad"], np.where(np.abs(d) < 1.0, d, np.sign(d)) / n + (g0 if accumulate else 0.0))
+
+
+def test_oracle_gather_in_one_call(oracle):
+    r = np.random.default_rng(4)
+    src = r.standard_normal((5, 6, 7)).astype(np.float32)
+    idx = r.integers(0, 6, (5, 4, 7)).astype(np.uint64)
+    S, I = oracle.from_numpy(src), oracle.from_numpy(idx)
+    O, D = oracle.from_numpy(np.zeros(idx.size, np.uint64)), oracle.from_numpy(np.full(idx.size, np.nan, np.float32))
+    assert oracle.gather(S, [5, 6, 7], [5, 4, 7], I, 1, O, D) == 0
+    want = np.take_along_axis(src[:, :, :], idx.astype(np.int64), axis=1)
+    assert np.array_equal(oracle.to_numpy(D), want.ravel())
+    assert np.array_equal(src.ravel()[oracle.to_numpy(O).astype(np.int64)], want.ravel())

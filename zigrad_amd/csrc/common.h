@@ -22,7 +22,7 @@ constexpr size_t kPoolAlign = 256; // min split size of the block pools, bytes
 
 void set_error(const char* fmt, ...);
 
-struct BlockPool;  // allocator.cpp
+struct BlockPool;  // runtime.hip
 
 }  // namespace zg
 
@@ -45,7 +45,7 @@ struct zg_hip_ctx {
     // fixed buffer for the per-workgroup partials of flat reductions (64 KiB)
     void* partials = nullptr;
 
-    // caching allocator state (allocator.cpp)
+    // caching allocator state (runtime.hip)
     zg::BlockPool* small_pool = nullptr;
     zg::BlockPool* large_pool = nullptr;
     size_t small_pool_bytes = 0;

@@ -281,6 +281,15 @@ int zg_hip_smce_fwd_bwd(zg_hip_ctx *ctx, const float *logits, const float *targe
 /* integer-label form: one pass over the logits forward (online softmax), lse[rows] kept for backward */
 int zg_hip_smce_label_fwd(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, float *lse, float *loss,
                           size_t rows, size_t cols);
+/* No counterpart in the reference: zg_hip_smce_label_fwd for callers that cannot allocate (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It calls no allocator of any kind: the per-row loss
+ * terms and the partial sums live in a fixed array in the library's device image (1 MiB + 8 KiB per GPU, held until
+ * the process ends) instead of the context's grow-only workspace.  At most 262144 rows; more is rejected with
+ * ZG_HIP_EINVAL before any launch.  Same kernels and the same values as zg_hip_smce_label_fwd.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (two contexts, two streams) race; calls on one context are ordered
+ * by its stream. */
+int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, float *lse,
+                                  float *loss, size_t rows, size_t cols);
 /* accumulate != 0: grad += (p - onehot)/rows (the reference's `+=`, src/nn/loss.zig:157);
  * accumulate == 0: grad is overwritten (valid when the caller knows grad is a fresh zero buffer) */
 int zg_hip_smce_label_bwd(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, const float *lse,

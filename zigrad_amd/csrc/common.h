@@ -45,6 +45,10 @@ struct zg_hip_ctx {
     // fixed buffer for the per-workgroup partials of flat reductions (64 KiB)
     void* partials = nullptr;
 
+    // address, on this context's device, of the fixed scratch array of the allocation-free entry point (loss.hip)
+    void* noalloc_scratch = nullptr;
+    size_t noalloc_scratch_bytes = 0;
+
     // caching allocator state (runtime.hip)
     zg::BlockPool* small_pool = nullptr;
     zg::BlockPool* large_pool = nullptr;
@@ -74,6 +78,9 @@ namespace zg {
 
 // Returns a workspace of at least `bytes` bytes (256-byte aligned), or nullptr with the error set.
 void* workspace(zg_hip_ctx* ctx, size_t bytes);
+
+// Looks up the device address of the fixed scratch array (loss.hip); the context's device must be current.
+int noalloc_setup(zg_hip_ctx* ctx);
 
 inline int ceil_div(size_t a, size_t b) {
     return (int)((a + b - 1) / b);

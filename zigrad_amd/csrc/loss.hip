@@ -450,6 +450,30 @@ static int pick_tpr(size_t cols) {
         default: { constexpr int T = 256; CALL; } break;  \
     }
 
+// Scratch of the entry point that allocates nothing (zg_hip_smce_label_fwd_noalloc): the per-row loss terms, then
+// the per-workgroup partials of their sum.  One copy per GPU for the life of the process; every call on a GPU uses
+// it, so calls that overlap on one GPU race.  Nothing in it has to start at zero: each call writes every entry it
+// later reads.
+constexpr size_t kNoAllocMaxRows = (size_t)1 << 18;
+constexpr size_t kNoAllocRowBytes = kNoAllocMaxRows * sizeof(float);
+constexpr size_t kNoAllocBytes = kNoAllocRowBytes + kMaxPartials * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
+
+// `scratch` is a host-side stand-in in host code, not a device address: the address on the current device is
+// looked up once per context (zg_hip_init calls this with the context's device current) and used from then on.
+int noalloc_setup(zg_hip_ctx* ctx) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        set_error("init: hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+        return ZG_HIP_ERUNTIME;
+    }
+    ctx->noalloc_scratch = p;
+    ctx->noalloc_scratch_bytes = kNoAllocBytes;
+    return ZG_HIP_OK;
+}
+
 static int check_rows(const char* name, size_t rows, size_t cols) {
     ZG_REQUIRE(rows > 0 && cols > 0, "%s: empty matrix (%zu x %zu)", name, rows, cols);
     ZG_REQUIRE(rows <= 0x7fffffffull * 64, "%s: too many rows", name);
@@ -473,6 +497,24 @@ ZG_API int zg_hip_smce_label_fwd(zg_hip_ctx* ctx, const float* logits, const uin
                                             labels, lse, row_loss, rows, cols));
     ZG_LAUNCH_CHECK();
     return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows});
+}
+
+ZG_API int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, float* lse,
+                                         float* loss, size_t rows, size_t cols) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(logits && labels && lse && loss, "smce_label_fwd_noalloc: null pointer");
+    if (int rc = check_rows("smce_label_fwd_noalloc", rows, cols)) return rc;
+    ZG_REQUIRE(rows <= kNoAllocMaxRows, "smce_label_fwd_noalloc: %zu rows exceed the fixed scratch (at most %zu rows)",
+               rows, kNoAllocMaxRows);
+    ZG_REQUIRE(ctx->noalloc_scratch != nullptr, "smce_label_fwd_noalloc: the context has no scratch address");
+    float* row_loss = (float*)ctx->noalloc_scratch;
+    void* partials = (char*)ctx->noalloc_scratch + kNoAllocRowBytes;
+    const int tpr = pick_tpr(cols);
+    const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
+    ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
+                                            labels, lse, row_loss, rows, cols));
+    ZG_LAUNCH_CHECK();
+    return flat_reduce_into<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows}, partials);
 }
 
 ZG_API int zg_hip_smce_label_bwd(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, const float* lse,

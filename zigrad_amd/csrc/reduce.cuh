@@ -265,8 +265,10 @@ __global__ __launch_bounds__(kFlatBlock) void flat_final_kernel(const typename P
     if (threadIdx.x == 0) fin(acc);
 }
 
+// `partials` holds the per-workgroup results of the two-launch form: room for kMaxPartials accumulators.
 template <class T, int NIN, class Fin>
-static int flat_reduce(zg_hip_ctx* ctx, const float* a, const float* b, size_t n, float p0, Fin fin) {
+static int flat_reduce_into(zg_hip_ctx* ctx, const float* a, const float* b, size_t n, float p0, Fin fin,
+                            void* partials_mem) {
     using P = typename T::P;
     if (n <= kFlatSingleMax) {
         hipLaunchKernelGGL((flat_single_kernel<T, NIN, Fin>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, a, b, n, p0,
@@ -279,7 +281,7 @@ static int flat_reduce(zg_hip_ctx* ctx, const float* a, const float* b, size_t n
     if (cap > (size_t)kMaxPartials) cap = kMaxPartials;
     if (blocks > cap) blocks = cap;
     static_assert(kMaxPartials * sizeof(typename P::Acc) <= (64 << 10), "partials buffer too small");
-    auto* partials = (typename P::Acc*)ctx->partials;
+    auto* partials = (typename P::Acc*)partials_mem;
     hipLaunchKernelGGL((flat_partial_kernel<T, NIN>), dim3((unsigned)blocks), dim3(kFlatBlock), 0, ctx->stream, a, b, n,
                        p0, partials);
     ZG_LAUNCH_CHECK();
@@ -287,6 +289,11 @@ static int flat_reduce(zg_hip_ctx* ctx, const float* a, const float* b, size_t n
                        fin);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
+}
+
+template <class T, int NIN, class Fin>
+static int flat_reduce(zg_hip_ctx* ctx, const float* a, const float* b, size_t n, float p0, Fin fin) {
+    return flat_reduce_into<T, NIN, Fin>(ctx, a, b, n, p0, fin, ctx->partials);
 }
 
 // x *= factor[0], skipped entirely when the factor is exactly 1

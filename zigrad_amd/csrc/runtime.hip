@@ -287,24 +287,37 @@ ZG_API int zg_hip_device_count(int* count) {
     return ZG_HIP_OK;
 }
 
-ZG_API int zg_hip_init(int device_id, zg_hip_ctx** out) {
-    ZG_REQUIRE(out != nullptr, "init: null output");
-    int n = 0;
-    ZG_HIP_TRY(hipGetDeviceCount(&n));
-    ZG_REQUIRE(device_id >= 0 && device_id < n, "init: device %d not present (%d devices)", device_id, n);
-    ZG_HIP_TRY(hipSetDevice(device_id));
-    zg_hip_ctx* ctx = new zg_hip_ctx();
-    ctx->device = device_id;
+static int init_resources(zg_hip_ctx* ctx) {
     hipDeviceProp_t prop;
-    ZG_HIP_TRY(hipGetDeviceProperties(&prop, device_id));
+    ZG_HIP_TRY(hipGetDeviceProperties(&prop, ctx->device));
     ctx->n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     ctx->total_mem = prop.totalGlobalMem;
     // one stream, default priority, in-order: the reference's device model (src/device/cuda_device.zig:126-144)
     ZG_HIP_TRY(hipStreamCreateWithFlags(&ctx->stream, hipStreamDefault));
     ZG_HIP_TRY(hipMalloc((void**)&ctx->scalar_slot, 256));
     ZG_HIP_TRY(hipMalloc(&ctx->partials, 64 << 10));
+    return noalloc_setup(ctx);
+}
+
+ZG_API int zg_hip_init(int device_id, zg_hip_ctx** out) {
+    ZG_REQUIRE(out != nullptr, "init: null output");
+    *out = nullptr;
+    int n = 0;
+    ZG_HIP_TRY(hipGetDeviceCount(&n));
+    ZG_REQUIRE(device_id >= 0 && device_id < n, "init: device %d not present (%d devices)", device_id, n);
+    ZG_HIP_TRY(hipSetDevice(device_id));
+    zg_hip_ctx* ctx = new zg_hip_ctx();
+    ctx->device = device_id;
     ctx->small_pool_bytes = (size_t)64 << 20;
     ctx->large_pool_bytes = (size_t)1 << 30;
+    if (int rc = init_resources(ctx)) {
+        // a context that failed part-way owns whatever it got so far
+        if (ctx->scalar_slot) (void)hipFree(ctx->scalar_slot);
+        if (ctx->partials) (void)hipFree(ctx->partials);
+        if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return rc;
+    }
     *out = ctx;
     return ZG_HIP_OK;
 }

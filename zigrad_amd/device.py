@@ -457,6 +457,10 @@ class HipDevice:
     def _op_smce_label_fwd(self, logits, labels, lse, loss, rows, cols):
         self._call("zg_hip_smce_label_fwd", logits.ptr, labels.ptr, lse.ptr, loss.ptr, rows, cols)
 
+    def _op_smce_label_fwd_noalloc(self, logits, labels, lse, loss, rows, cols):
+        """smce_label_fwd without any allocation: fixed scratch in the library's device image, at most 262144 rows."""
+        self._call("zg_hip_smce_label_fwd_noalloc", logits.ptr, labels.ptr, lse.ptr, loss.ptr, rows, cols)
+
     def _op_smce_label_bwd(self, logits, labels, lse, grad, rows, cols, accumulate=True):
         self._call("zg_hip_smce_label_bwd", logits.ptr, labels.ptr, lse.ptr, grad.ptr, rows, cols, int(accumulate))
 

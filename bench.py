@@ -233,7 +233,7 @@ def timed_steps(dev, step_fn, steps):
 
 
 def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_mode="onehot", lr=1e-3, graph=False,
-            late_read=False, fused=False, clip=True):
+            late_read=False, fused=False, clip=True, loss_log=None):
     """Returns (seconds, last loss) for `steps` eager steps; with graph=True also the same for `steps` replays of
     the step recorded as an execution graph (the loss is read back every step in both modes)."""
     from zigrad_amd.trainers import MLPTrainer, mlp_inputs
@@ -243,7 +243,9 @@ def run_mlp(dev, dims, batch, optimizer, steps, warmup, data, timer=None, loss_m
     tr.load_params(params)
     tr.set_batch(x, onehot, labels)
     for _ in range(warmup):
-        tr.step()
+        l = tr.step()
+        if loss_log is not None:  # the loss of every step from the first, for the cross-check against the oracle
+            loss_log.append(l)
     if timer is not None:
         timer.on = True
     dt, loss = timed_steps(dev, tr.step, steps)
@@ -359,15 +361,18 @@ def run_c_harness(dims, batch, steps, fused=False):
     return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": what}
 
 
-def cpu_baseline(dims, batch, budget_steps=2, threads=None):
+def cpu_baseline(dims, batch, budget_steps=2, threads=None, loss_mode="onehot"):
     """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share (or `threads`)."""
     from oracle.oracle_device import OracleDevice
 
     odev = OracleDevice()
     cores = threads or min(16, os.cpu_count() or 1)
     cores = odev.set_threads(cores)
-    dt, _ = run_mlp(odev, dims, batch, "adam", steps=budget_steps, warmup=1, data="normal")
+    log = []
+    dt, _ = run_mlp(odev, dims, batch, "adam", steps=budget_steps, warmup=1, data="normal", loss_mode=loss_mode,
+                    loss_log=log)
     return {
+        "first_step_loss": log[0],
         "value": budget_steps / dt,
         "unit": "steps/s",
         "cores": cores,
@@ -425,8 +430,9 @@ def main():
     copy_calibration(dev)
     timer = GemmTimer(dev)
     timer.install()
+    gpu_losses = []
     dt, loss, dt_late, _ = run_mlp(dev, WIDE_DIMS, WIDE_BATCH, "adam", args.steps, args.warmup, "normal", timer, args.loss_mode,
-                                   late_read=True)
+                                   late_read=True, loss_log=gpu_losses)
     ms_per_step = dt / args.steps * 1e3
     gemm_ms = timer.total_ms()
     n_launch = len(timer.pairs)
@@ -501,8 +507,16 @@ def main():
     if not args.no_ops:
         result["ops"] = op_suite(dev)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH)
+        result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH, loss_mode=args.loss_mode)
+        # the oracle ran the same first step from the same parameters and batch: its loss must be the device's
+        if gpu_losses:
+            o, g = result["cpu_baseline"]["first_step_loss"], gpu_losses[0]
+            rel = abs(o - g) / max(1.0, abs(o))
+            result["parity_check"] = {"what": "loss of the first train step, device against the CPU oracle",
+                                      "device": g, "oracle": o, "rel_diff": rel, "bound": 1e-4, "ok": rel <= 1e-4}
+        result["cpu_baseline"].pop("first_step_loss", None)
         result["cpu_baseline_1_thread"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH, budget_steps=1, threads=1)
+        result["cpu_baseline_1_thread"].pop("first_step_loss", None)
         # the same CPU oracle on the batch-64 MLP, the configuration the reference runs today
         from oracle.oracle_device import OracleDevice
 
@@ -528,6 +542,8 @@ def main():
         result["cpu_baseline"] = None
     dev.deinit()
     print(json.dumps(result))
+    if result.get("parity_check") and not result["parity_check"]["ok"]:
+        sys.exit("bench.py: the device's first-step loss differs from the CPU oracle's by more than 1e-4")
 
 
 if __name__ == "__main__":

@@ -319,6 +319,9 @@ class OracleDevice(HipDevice):
         code = {"uniform": 0, "normal": 1, "kaiming": 2}[kind]
         self._o.cdll.zo_mem_random(buf.ptr, buf.n, code, int(fan), int(seed))
 
+    def adam_lr_t(self, lr, beta1, beta2, t) -> float:
+        return float(self._o.cdll.zo_adam_lr_t(int(t), lr, beta1, beta2))
+
     def mem_take(self, src, idxs, dst):
         self._o.cdll.zo_mem_take(src.ptr, src.n, idxs.ptr, idxs.n, dst.ptr)
 

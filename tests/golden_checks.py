@@ -219,7 +219,87 @@ def check_losses(dev):
     np.testing.assert_allclose(g["grad"] * 6, f32(c["expected_grad_times_6"]), rtol=1e-6)
 
 
+def check_mul_div_backward(dev):
+    """t3 = t1 * t2 and t3 = t1 / t2 followed by backward() with an upstream gradient of ones: the op sequences of
+    MulBwd / DivBwd (src/ndtensor.zig:836-907), gradient buffers zero-filled on first touch."""
+    for key, op, bwd, fwd_key in (("mul_backward", "mul", host.mul_backward, "expected_product"),
+                                  ("div_backward", "div", host.div_backward, "expected_quotient")):
+        c = G[key]
+        a, b = dev.from_numpy(f32(c["t1"])), dev.from_numpy(f32(c["t2"]))
+        z, z_shape = host.elwise(dev, op, a, c["t1_shape"], b, c["t2_shape"])
+        dev.sync()
+        np.testing.assert_array_equal(dev.to_numpy(z), f32(c[fwd_key]))
+        zg = dev.from_numpy(np.ones(len(c[fwd_key]), np.float32))
+        ag, bg = dev.from_numpy(np.zeros(len(c["t1"]), np.float32)), dev.from_numpy(np.zeros(len(c["t2"]), np.float32))
+        bwd(dev, a, c["t1_shape"], b, c["t2_shape"], zg, z_shape, ag, bg)
+        dev.sync()
+        want_a = np.float32(1.0) / f32(c["t2"]) if c.get("grad_t1_is_fp32_reciprocal_of_t2") else f32(c["grad_t1"])
+        np.testing.assert_array_equal(dev.to_numpy(ag), want_a)
+        np.testing.assert_array_equal(dev.to_numpy(bg), f32(c["grad_t2"]))
+        dev.mem_cache_free(z)
+    # broadcasting operands: the gradient of the short one is folded back (same closures, shapes (2,3) and (3,))
+    a_np, b_np = f32([[1, 2, 3], [4, 5, 6]]), f32([2, 4, 8])
+    a, b = dev.from_numpy(a_np.ravel()), dev.from_numpy(b_np)
+    zg = dev.from_numpy(np.ones(6, np.float32))
+    ag, bg = dev.from_numpy(np.zeros(6, np.float32)), dev.from_numpy(np.zeros(3, np.float32))
+    host.mul_backward(dev, a, [2, 3], b, [3], zg, [2, 3], ag, bg)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(ag), np.tile(b_np, 2))
+    np.testing.assert_array_equal(dev.to_numpy(bg), a_np.sum(axis=0))
+    ag, bg = dev.from_numpy(np.zeros(6, np.float32)), dev.from_numpy(np.zeros(3, np.float32))
+    host.div_backward(dev, a, [2, 3], b, [3], zg, [2, 3], ag, bg)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(ag), np.tile(1 / b_np, 2))
+    np.testing.assert_array_equal(dev.to_numpy(bg), -(a_np / (b_np * b_np)).sum(axis=0))  # powers of two: exact
+
+
+def check_matvec_dot_backward(dev):
+    """y = A x and z = t1 . t2 followed by backward(): MatvecBwd issues outer + matvec, DotBwd two axpy whose alpha
+    is read through a pointer to the result's one-element gradient in device memory (src/ndtensor.zig:1142-1252)."""
+    c = G["matvec_backward"]
+    A, x = dev.from_numpy(f32(c["A"])), dev.from_numpy(f32(c["x"]))
+    rows, cols = c["A_shape"]
+    y = dev.from_numpy(np.full(rows, np.nan, np.float32))
+    dev.dispatch("matvec", A=A, x=x, y=y, m=rows, n=cols, trans_a=False, alpha=1.0, beta=0.0)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(y), f32(c["expected_y"]))
+    yg = dev.from_numpy(np.ones(rows, np.float32))
+    Ag, xg = dev.from_numpy(np.zeros(rows * cols, np.float32)), dev.from_numpy(np.zeros(cols, np.float32))
+    host.matvec_backward(dev, A, c["A_shape"], x, yg, Ag, xg)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(Ag), f32(c["grad_A"]))
+    np.testing.assert_array_equal(dev.to_numpy(xg), f32(c["grad_x"]))
+    # an upstream gradient that is not all ones separates outer(dy, x) from outer(x, dy) and A^T dy from A dy
+    yg = dev.from_numpy(f32([2, -1]))
+    Ag, xg = dev.from_numpy(np.zeros(4, np.float32)), dev.from_numpy(np.zeros(2, np.float32))
+    x2 = dev.from_numpy(f32([3, 5]))
+    host.matvec_backward(dev, A, c["A_shape"], x2, yg, Ag, xg)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(Ag), f32([6, 10, -3, -5]))
+    np.testing.assert_array_equal(dev.to_numpy(xg), f32([2 * 1 - 3, 2 * 2 - 4]))
+
+    c = G["dot_backward"]
+    t1, t2 = dev.from_numpy(f32(c["t1"])), dev.from_numpy(f32(c["t2"]))
+    z = dev.from_numpy(np.zeros(1, np.float32))
+    dev.dispatch("dot", x=t1, y=t2, z=z)
+    dev.sync()
+    assert dev.to_numpy(z)[0] == c["expected"]
+    zg = dev.from_numpy(np.ones(1, np.float32))  # backward() of a scalar: gradient 1, resident on the device
+    g1, g2 = dev.from_numpy(np.zeros(3, np.float32)), dev.from_numpy(np.zeros(3, np.float32))
+    host.dot_backward(dev, t1, t2, zg, g1, g2)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(g1), f32(c["grad_t1"]))
+    np.testing.assert_array_equal(dev.to_numpy(g2), f32(c["grad_t2"]))
+    # alpha really is read from the gradient: a different upstream value scales both
+    zg = dev.from_numpy(f32([-0.5]))
+    host.dot_backward(dev, t1, t2, zg, g1, g2)
+    dev.sync()
+    np.testing.assert_array_equal(dev.to_numpy(g1), f32(c["grad_t1"]) * 0.5)
+    np.testing.assert_array_equal(dev.to_numpy(g2), f32(c["grad_t2"]) * 0.5)
+
+
 ALL_CHECKS = [
     check_clip_nrm2, check_clamp, check_add_sub_scalar, check_dot, check_bmm, check_matvec, check_sum_max_along,
     check_gather, check_sum, check_add_broadcast_grad, check_matmul_backward, check_pow_sqrt, check_losses,
+    check_mul_div_backward, check_matvec_dot_backward,
 ]

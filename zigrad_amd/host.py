@@ -132,3 +132,70 @@ def gather(dev, src: DevBuf, src_shape, indices: DevBuf, idx_shape, dim: int, re
         return values, offsets
     dev.mem_cache_free(offsets)
     return values, None
+
+
+def broadcast_shape(a, b) -> list[int]:
+    """Right-aligned broadcast of two shapes (reference: Shape.broadcast, src/ndarray/shape.zig:247-264)."""
+    return _broadcast_batch(list(a), list(b))
+
+
+def elwise(dev, op: str, x: DevBuf, x_shape, y: DevBuf, y_shape):
+    """z = x op y into a fresh buffer of the broadcast shape.  Reference: NDArray.elwise_alloc,
+    src/ndarray.zig:231-246 (the device op does the modulo broadcasting).  Returns (z, z_shape); free z with
+    mem_cache_free."""
+    z_shape = broadcast_shape(x_shape, y_shape)
+    z = dev.mem_cache_alloc(F32, _prod(z_shape))
+    dev.dispatch(op, x=x, y=y, z=z)
+    return z, z_shape
+
+
+def mul_backward(dev, a: DevBuf, a_shape, b: DevBuf, b_shape, c_grad: DevBuf, c_shape, a_grad: DevBuf | None,
+                 b_grad: DevBuf | None) -> None:
+    """The device ops MulBwd issues (src/ndtensor.zig:836-868): a.grad += unbroadcast(b * dc),
+    b.grad += unbroadcast(a * dc)."""
+    for own_grad, own_shape, other, other_shape in ((a_grad, a_shape, b, b_shape), (b_grad, b_shape, a, a_shape)):
+        if own_grad is None:
+            continue
+        t, t_shape = elwise(dev, "mul", other, other_shape, c_grad, c_shape)
+        unbroadcast_(dev, t, t_shape, own_grad, own_shape, alpha=1.0, beta=1.0)
+        dev.mem_cache_free(t)
+
+
+def div_backward(dev, a: DevBuf, a_shape, b: DevBuf, b_shape, c_grad: DevBuf, c_shape, a_grad: DevBuf | None,
+                 b_grad: DevBuf | None) -> None:
+    """The device ops DivBwd issues (src/ndtensor.zig:871-907): a.grad += unbroadcast(dc / b);
+    b.grad -= unbroadcast((dc * a) / (b * b))  (alpha = -1, beta = 1)."""
+    if a_grad is not None:
+        t, t_shape = elwise(dev, "div", c_grad, c_shape, b, b_shape)
+        unbroadcast_(dev, t, t_shape, a_grad, a_shape, alpha=1.0, beta=1.0)
+        dev.mem_cache_free(t)
+    if b_grad is not None:
+        num, num_shape = elwise(dev, "mul", c_grad, c_shape, a, a_shape)
+        bsq, bsq_shape = elwise(dev, "mul", b, b_shape, b, b_shape)
+        t, t_shape = elwise(dev, "div", num, num_shape, bsq, bsq_shape)
+        dev.mem_cache_free(num)
+        dev.mem_cache_free(bsq)
+        unbroadcast_(dev, t, t_shape, b_grad, b_shape, alpha=-1.0, beta=1.0)
+        dev.mem_cache_free(t)
+
+
+def dot_backward(dev, a: DevBuf, b: DevBuf, c_grad: DevBuf, a_grad: DevBuf | None, b_grad: DevBuf | None) -> None:
+    """DotBwd (src/ndtensor.zig:1142-1160): two axpy whose alpha is the one-element gradient of the result, read
+    through a pointer into device memory."""
+    if a_grad is not None:
+        dev.dispatch("axpy", x=b, y=a_grad, alpha=c_grad)
+    if b_grad is not None:
+        dev.dispatch("axpy", x=a, y=b_grad, alpha=c_grad)
+
+
+def matvec_backward(dev, A: DevBuf, a_shape, x: DevBuf, y_grad: DevBuf, A_grad: DevBuf | None, x_grad: DevBuf | None,
+                    trans_a: bool = False) -> None:
+    """MatvecBwd (src/ndtensor.zig:1225-1252): A.grad += outer(dy, x) (operands swapped when trans_a);
+    x.grad += op(A)^T . dy, issued with the reference's own m / n (the matrix's dimensions exchanged and the
+    transpose flag flipped), which describes the stored matrix correctly only when it is square."""
+    rows, cols = int(a_shape[0]), int(a_shape[1])
+    if A_grad is not None:
+        dev.dispatch("outer", x=(x if trans_a else y_grad), y=(y_grad if trans_a else x), A=A_grad, alpha=1.0)
+    if x_grad is not None:
+        m, n = (cols, rows) if not trans_a else (rows, cols)
+        dev.dispatch("matvec", A=A, x=y_grad, y=x_grad, m=m, n=n, trans_a=not trans_a, alpha=1.0, beta=1.0)

@@ -399,12 +399,23 @@ class MLPTrainer(GraphSteps):
         """Train on batch buffers owned by the caller (a BatchStager slot) from the next step on."""
         self.x, self.onehot, self.labels = x, onehot, labels
 
-    def step(self, read_loss=True, keep_grads: bool = False):
+    def step(self, read_loss=True, keep_grads: bool = False, keep_acts: bool = False, force: dict | None = None):
         """One train step.  read_loss=True reads the loss where the reference's loop does (loss.get(0) before
         backward, examples/mnist/src/main-simple.zig:67): the host blocks there and the GPU idles until the backward
-        launches arrive.  read_loss="late" moves the same read behind the optimizer step, so the queue never drains."""
+        launches arrive.  read_loss="late" moves the same read behind the optimizer step, so the queue never drains.
+
+        keep_acts / keep_grads read the layer outputs / the gradients back into last_acts / last_grads.
+        force = {"acts": [...], "grads": [...]} (host arrays, either key optional) overwrites the layer outputs after
+        the forward pass and the gradients after the backward pass: two devices can then run the backward pass and
+        the optimizer from identical inputs, which takes the ReLU's discontinuity at zero out of a comparison (an
+        output that rounds to +1e-7 on one device and to 0 on the other gates a whole gradient row differently)."""
         d, B, C = self.dev, self.batch, self.dims[-1]
         acts = self.net.forward(self.x, B)
+        if keep_acts:
+            self.last_acts = [d.to_numpy(a) for a in acts[1:]]
+        if force and "acts" in force:
+            for buf, a in zip(acts[1:], force["acts"]):
+                d.mem_transfer(a, buf, "HtoD")
         logits = acts[-1]
         loss = d.mem_cache_alloc(F32, 1)
         if self.optim.fused and self.loss_mode == "onehot":
@@ -437,6 +448,9 @@ class MLPTrainer(GraphSteps):
         self.net.backward(acts, g, B)
         if keep_grads:
             self.last_grads = [d.to_numpy(b) for b in self.grad_buffers()]
+        if force and "grads" in force:
+            for buf, g_host in zip(self.grad_buffers(), force["grads"]):
+                d.mem_transfer(g_host, buf, "HtoD")
         if not self.optim.step_and_zero_grad():
             self.optim.step()
             self.net.zero_grad()  # model.zero_grad()

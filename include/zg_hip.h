@@ -83,15 +83,23 @@ int zg_hip_free(zg_hip_ctx *ctx, void *ptr);                    /* mem_free:  sr
 int zg_hip_host_alloc(zg_hip_ctx *ctx, size_t bytes, void **out); /* pinned, device-readable host memory */
 int zg_hip_host_free(zg_hip_ctx *ctx, void *ptr);
 
-/* The library's own caching allocator (block pools over two mapped regions + grow-only scratch),
- * the C++ counterpart of CachingAllocator(DataHandler) (src/allocators/caching_allocator.zig:15-162)
- * for callers that do not bring Zigrad's.  `block` is the DeviceData.ctx of the reference
- * (src/allocators/device_data.zig:32-40). A zero-byte request yields (NULL, 0). */
+/* The library's own caching allocator (two block pools, small <= 1 MiB and large, over segments obtained on
+ * demand, + grow-only scratch), the C++ counterpart of CachingAllocator(DataHandler)
+ * (src/allocators/caching_allocator.zig:15-162): blocks are split on allocation and fused with free neighbours on
+ * release (src/allocators/block_pool.zig:185-324), every operation in constant time.  `block` is the DeviceData.ctx
+ * of the reference (src/allocators/device_data.zig:32-40): an opaque non-zero handle that zg_hip_mem_cache_free
+ * takes back together with the pointer.  A zero-byte request yields (NULL, 0).  cache_configure sets the size of the
+ * segments each pool grows by. */
 int zg_hip_cache_configure(zg_hip_ctx *ctx, size_t small_pool_bytes, size_t large_pool_bytes);
 int zg_hip_mem_cache_alloc(zg_hip_ctx *ctx, size_t bytes, void **out, uint64_t *block);
 int zg_hip_mem_cache_free(zg_hip_ctx *ctx, void *ptr, uint64_t block);
 int zg_hip_mem_scratch(zg_hip_ctx *ctx, size_t bytes, void **out); /* src/allocators/caching_allocator.zig:133-156 */
 int zg_hip_clear_cache(zg_hip_ctx *ctx);
+/* *yes = 1 when ptr lies in memory this context handed out as device memory (cache pools, zg_hip_alloc /
+ * zg_hip_pool_map regions, the scratch buffer), else 0.  The reference's callers pass host scalars and device slices
+ * through the same parameters (src/ndarray.zig:251 and src/nn/optim.zig:117 against src/ndtensor.zig:1146-1150); a
+ * binding tells them apart with this range test. */
+int zg_hip_is_device_ptr(zg_hip_ctx *ctx, const void *ptr, int *yes);
 int zg_hip_cache_stats(zg_hip_ctx *ctx, size_t *bytes_in_use, size_t *bytes_mapped, uint64_t *n_device_allocs);
 
 /* ---------------------------------------------------------------------------------------------

@@ -77,6 +77,32 @@ def test_zig_veneer_calls_match_the_header():
         assert n_args == len(protos[name][1]), f"{name}: veneer passes {n_args} arguments, header declares {len(protos[name][1])}"
 
 
+def test_zig_veneer_uses_only_what_the_reference_allocators_export():
+    """The binding imports src/allocators.zig: every `allocators.<name>` it names must be a `pub` declaration of
+    that file, and it must not reach into the allocator objects (no `self.cache.<method>` that the reference's
+    CachingAllocator lacks: the binding keeps no allocator object at all)."""
+    import re
+    from pathlib import Path
+
+    import pytest
+
+    text = (Path(__file__).resolve().parents[1] / "zig" / "hip_device.zig").read_text()
+    text = re.sub(r"//[^\n]*", "", text)
+    assert not re.search(r"\bself\.cache\b", text), "the binding is meant to go through zg_hip_mem_cache_* only"
+    used = set(re.findall(r"\ballocators\.(\w+)", text)) - {"zig"}  # "../allocators.zig" is the import itself
+    assert used, "the binding no longer imports src/allocators.zig?"
+    ref = Path("/root/reference/src/allocators.zig")
+    if not ref.exists():
+        pytest.skip("the reference checkout is not present on this machine")
+    exported = set(re.findall(r"(?m)^pub (?:const|fn) (\w+)", ref.read_text()))
+    assert used <= exported, f"not exported by the reference's src/allocators.zig: {sorted(used - exported)}"
+    # the members of the DataHandler contract (src/allocators/block_pool.zig:103-173) are all present
+    handler = text[text.index("pub const DataHandler = struct"):]
+    handler = handler[:handler.index("\n};")]
+    for member in ("min_split_size", "fn map(", "fn unmap(", "fn alloc(", "fn free(", "fn page_size(", "fn reset(", "fn deinit("):
+        assert member in handler, member
+
+
 def test_header_is_plain_c_and_links_from_a_c_program(tmp_path):
     """include/zg_hip.h compiles as C11 with gcc (no C++ in the boundary) and a C program linked against the library
     can call it: device count and the error string, nothing that needs a GPU."""

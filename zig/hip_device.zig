@@ -18,10 +18,10 @@ const c = @cImport(@cInclude("zg_hip.h"));
 const opspec = @import("opspec.zig");
 const RandType = @import("device_common.zig").RandType;
 const TransferDirection = @import("device_common.zig").TransferDirection;
-const CachingAllocator = @import("../allocators.zig").CachingAllocator(DataHandler);
-const DeviceData = @import("../allocators.zig").DeviceData;
-const Error = @import("../allocators.zig").Error;
-const adjust_map_size = @import("../allocators.zig").adjust_map_size;
+const allocators = @import("../allocators.zig");
+const DeviceData = allocators.DeviceData;
+const Error = allocators.Error;
+const adjust_map_size = allocators.adjust_map_size;
 
 pub const DeviceReference = @import("device_reference.zig");
 const Self = @This();
@@ -30,10 +30,13 @@ fn check(rc: c_int) void {
     if (rc != 0) std.debug.panic("zg_hip: {s}", .{std.mem.span(c.zg_hip_last_error())});
 }
 
-/// The per-device handler src/allocators/caching_allocator.zig is generic over.
-/// `map` hands the block pool one contiguous device region; `map_alloc` is left out on purpose
-/// (src/allocators/block_pool.zig:115 makes it optional): the region is physically backed when mapped.
-const DataHandler = struct {
+/// The per-device handler src/allocators/caching_allocator.zig is generic over, for a build that wants Zigrad's own
+/// `CachingAllocator(HipDevice.DataHandler)` over device memory (every member the contract names:
+/// src/allocators/block_pool.zig:103-173).  `map` hands the block pool one contiguous device region; `map_alloc` is
+/// left out on purpose (src/allocators/block_pool.zig:115 makes it optional): the region is physically backed when
+/// mapped.  The device below does NOT use it: its mem_cache_* methods go through the library's allocator
+/// (zg_hip_mem_cache_*), the one the library's tests cover and the one that knows about execution graphs.
+pub const DataHandler = struct {
     pub const min_split_size = 256; // bytes; every block is then 256-byte aligned, enough for 128-bit accesses
 
     ctx: *c.zg_hip_ctx,
@@ -70,8 +73,14 @@ const DataHandler = struct {
     }
 };
 
+/// Segment sizes of the library's two block pools (the counterpart of CachingAllocator.Options,
+/// src/allocators/caching_allocator.zig:41-44); null keeps the library's defaults (64 MiB and 1 GiB).
+pub const Options = struct {
+    small_pool_size: ?usize = null,
+    large_pool_size: ?usize = null,
+};
+
 ctx: *c.zg_hip_ctx,
-cache: CachingAllocator,
 /// one device float that host-side scalar operands are staged through (see `dev_scalar`)
 scalar_slot: [*]f32,
 
@@ -85,22 +94,22 @@ pub fn init(device_number: u32) Self {
     return init_advanced(device_number, .{});
 }
 
-pub fn init_advanced(device_number: u32, opts: CachingAllocator.Options) Self {
+pub fn init_advanced(device_number: u32, opts: Options) Self {
     var ctx: ?*c.zg_hip_ctx = null;
     check(c.zg_hip_init(@intCast(device_number), &ctx));
+    if (opts.small_pool_size != null or opts.large_pool_size != null)
+        check(c.zg_hip_cache_configure(ctx.?, opts.small_pool_size orelse (64 << 20), opts.large_pool_size orelse (1 << 30)));
     var slot: ?*anyopaque = null;
     check(c.zg_hip_alloc(ctx.?, 256, &slot));
     return .{
         .ctx = ctx.?,
-        .cache = CachingAllocator.init(.{ .ctx = ctx.? }, opts),
         .scalar_slot = @ptrCast(@alignCast(slot.?)),
     };
 }
 
 pub fn deinit(self: *Self) void {
     self.sync();
-    self.cache.deinit();
-    check(c.zg_hip_deinit(self.ctx));
+    check(c.zg_hip_deinit(self.ctx)); // frees the pools, the scratch buffer and every raw allocation still live
     self.* = undefined;
 }
 
@@ -117,7 +126,7 @@ pub fn sync(self: *const Self) void {
 }
 
 pub fn clear_cache(self: *Self) void {
-    self.cache.clear();
+    check(c.zg_hip_clear_cache(self.ctx));
 }
 
 // --------------------------------------------------------------------------------------------------
@@ -127,8 +136,9 @@ pub fn clear_cache(self: *Self) void {
 // `mem_alloc_indices` (pinned, device-readable); scalars are staged here.
 // --------------------------------------------------------------------------------------------------
 fn is_device_ptr(self: *const Self, p: *const anyopaque) bool {
-    const a = @intFromPtr(p);
-    return self.cache.owns(a); // two contiguous pool mappings: an O(1) range test (src/allocators/block_pool.zig:118)
+    var yes: c_int = 0;
+    check(c.zg_hip_is_device_ptr(self.ctx, p, &yes)); // a range test over the pools' segments and the raw allocations
+    return yes != 0;
 }
 
 fn dev_scalar(self: *const Self, T: type, s: []const T) [*]const T {
@@ -148,14 +158,22 @@ pub fn mem_alloc_indices(self: *Self, n: usize) ![]usize {
 // --------------------------------------------------------------------------------------------------
 // memory API (src/device/device_reference.zig:29-123)
 // --------------------------------------------------------------------------------------------------
+/// `ctx` of the returned DeviceData is the library's block handle (the reference keeps its *Block there:
+/// src/allocators/device_data.zig:32-40, src/allocators/block_pool.zig:262-269); views carry 0 and are never freed.
 pub fn mem_cache_alloc(self: *Self, T: type, n: usize) !DeviceData(T) {
-    return self.cache.alloc(T, n);
+    if (n == 0) return .{ .raw = &.{}, .ctx = 0 }; // src/allocators/caching_allocator.zig:81-85
+    var ptr: ?*anyopaque = null;
+    var block: u64 = 0;
+    if (c.zg_hip_mem_cache_alloc(self.ctx, n * @sizeOf(T), &ptr, &block) != 0) return Error.DeviceOOM;
+    const p: [*]T = @ptrCast(@alignCast(ptr.?));
+    return .{ .raw = p[0..n], .ctx = @intCast(block) };
 }
 pub fn mem_cache_free(self: *Self, data: anytype) void {
-    self.cache.free(data);
+    if (data.raw.len == 0 or data.ctx == 0) return; // src/allocators/caching_allocator.zig:111-112
+    check(c.zg_hip_mem_cache_free(self.ctx, @constCast(@ptrCast(data.raw.ptr)), @intCast(data.ctx)));
 }
 pub fn mem_cache_dupe(self: *Self, T: type, src: []const T) !DeviceData(T) {
-    const dst = try self.cache.alloc(T, src.len);
+    const dst = try self.mem_cache_alloc(T, src.len);
     // callers pass host stack values here (src/nn/loss.zig:163), so pick the direction by where src lives
     if (self.is_device_ptr(src.ptr)) self.mem_copy(T, src, dst.raw) else self.mem_transfer(T, src, dst.raw, .HtoD);
     return dst;
@@ -180,7 +198,11 @@ pub fn mem_dupe(self: *Self, T: type, src: []const T) ![]T {
     return dst;
 }
 pub fn mem_scratch(self: *Self, T: type, n: usize) []T {
-    return self.cache.alloc_scratch(T, n);
+    if (n == 0) return &.{};
+    var ptr: ?*anyopaque = null;
+    check(c.zg_hip_mem_scratch(self.ctx, n * @sizeOf(T), &ptr)); // grow-only, src/allocators/caching_allocator.zig:133-156
+    const p: [*]T = @ptrCast(@alignCast(ptr.?));
+    return p[0..n];
 }
 pub fn mem_fill(self: *const Self, T: type, slice: []T, value: T) void {
     switch (T) {
@@ -567,8 +589,9 @@ pub fn adam_step_at(self: *const Self, T: type, p: anytype) void {
 }
 
 /// The ExecutionGraph of the reference's second device (src/device/cuda_device.zig:558-611), same four calls.
-/// Between `open` and `save` every op is recorded instead of executed; `mem_cache_free` inside a capture parks
-/// the block with the graph, so the recorded addresses stay private to it until `free`.
+/// Between `open` and `save` every op is recorded instead of executed.  Cache blocks handed out or returned while
+/// recording may be reused by later allocations of the same recording; whatever part of them is free at `save`
+/// stays with the graph, so the recorded addresses remain private to it until `free`.
 pub const ExecutionGraph = struct {
     ctx: *c.zg_hip_ctx,
     graph: ?*c.zg_hip_graph = null,

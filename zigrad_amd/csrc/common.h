@@ -62,10 +62,11 @@ struct zg_hip_ctx {
     hipStream_t copy_stream = nullptr;
     hipEvent_t ev_compute = nullptr, ev_copy = nullptr;
 
-    // execution-graph capture (runtime.hip): while `capturing`, cache blocks that are freed are parked here
-    // instead of going back to the pool, so a replay never meets another owner at those addresses
+    // execution-graph capture (runtime.hip): while `capturing`, the address range of every cache block handed out
+    // or returned is noted; the free part of those ranges stays with the graph when the recording ends, so a
+    // replay never meets another owner at those addresses
     bool capturing = false;
-    std::vector<std::pair<void*, uint64_t>> capture_parked;
+    std::vector<std::pair<char*, size_t>> capture_touched;
     int live_graphs = 0;
     std::vector<void*> retired_ws;  // outgrown workspaces that an instantiated graph may still name
 

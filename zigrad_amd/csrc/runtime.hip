@@ -5,8 +5,8 @@
 // DataHandler primitives src/allocators/caching_allocator.zig expects from a device.
 #include "common.h"
 
+#include <algorithm>
 #include <cmath>
-#include <mutex>
 
 namespace zg {
 
@@ -51,37 +51,123 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Block pool: a coalescing free-list allocator over device segments obtained with hipMalloc.
-// Counterpart of src/allocators/block_pool.zig:103-412 (split on alloc, fuse with free neighbours on
-// free); segments are added on demand instead of mapping one region of the whole device up front, so
-// steady-state training never reaches hipMalloc once the working set has been seen.
+// Block pool: a coalescing allocator over device segments obtained with hipMalloc, with every operation in
+// constant time.  Counterpart of src/allocators/block_pool.zig:103-412 (split on alloc, fuse with free
+// neighbours on free, free blocks filed by size order); segments are added on demand instead of mapping
+// one region of the whole device up front, so steady-state training never reaches hipMalloc once the
+// working set has been seen.
+//
+// A block is a node of two doubly linked lists: the blocks of its segment in address order (for fusing)
+// and the free blocks of its size class.  Size classes are exact up to 7 units of 256 bytes and four per
+// power of two above that; a bitmap of the non-empty classes finds the first class whose blocks all fit.
+// The handle the caller keeps (DeviceData.ctx in the reference, src/allocators/device_data.zig:32-40) is
+// the node's address, so freeing looks nothing up; nodes live in slabs, which makes a stale or foreign
+// handle detectable by a range test.
 // ------------------------------------------------------------------------------------------------
 struct Block {
     char* ptr;
     size_t size;
-    bool free;
-    int segment;
+    Block *prev, *next;    // neighbours in address order within the segment
+    Block *fprev, *fnext;  // neighbours in the free list of the size class (fnext also chains unused nodes)
+    BlockPool* pool;
+    uint8_t state;         // kNodeUnused, kFree, kLive
+};
+enum : uint8_t { kNodeUnused = 0, kFree = 1, kLive = 2 };
+
+struct Segment {
+    char* base;
+    size_t bytes;
+    Block* first;
 };
 
 struct BlockPool {
-    size_t segment_bytes;
-    size_t min_split;
-    std::vector<void*> segments;
-    std::map<char*, Block> blocks;                 // by address
-    std::multimap<size_t, char*> free_by_size;     // free blocks by size
+    static constexpr int kClasses = 8 + 4 * 48;
+    static constexpr int kSlabNodes = 1024;
+    size_t segment_bytes = 0;
+    size_t min_split = kPoolAlign;
+    std::vector<Segment> segments;
+    std::vector<Block*> slabs;
+    Block* unused_nodes = nullptr;
+    Block* free_head[kClasses] = {};
+    uint64_t class_bits[(kClasses + 63) / 64] = {};
     size_t in_use = 0;
     size_t mapped = 0;
 
-    void erase_free(const Block& b) {
-        auto range = free_by_size.equal_range(b.size);
-        for (auto it = range.first; it != range.second; ++it) {
-            if (it->second == b.ptr) {
-                free_by_size.erase(it);
-                return;
+    // ---- nodes ----
+    Block* new_node() {
+        if (!unused_nodes) {
+            Block* slab = new Block[kSlabNodes]();
+            slabs.push_back(slab);
+            for (int i = kSlabNodes - 1; i >= 0; i--) {
+                slab[i].state = kNodeUnused;
+                slab[i].fnext = unused_nodes;
+                unused_nodes = &slab[i];
             }
+        }
+        Block* b = unused_nodes;
+        unused_nodes = b->fnext;
+        *b = Block{};
+        b->pool = this;
+        return b;
+    }
+    void drop_node(Block* b) {
+        b->state = kNodeUnused;
+        b->fnext = unused_nodes;
+        unused_nodes = b;
+    }
+    bool is_node(const void* h) const {
+        for (Block* slab : slabs) {
+            const char* lo = (const char*)slab;
+            const char* p = (const char*)h;
+            if (p >= lo && p < lo + sizeof(Block) * kSlabNodes) return (size_t)(p - lo) % sizeof(Block) == 0;
+        }
+        return false;
+    }
+
+    // ---- size classes ----
+    // class of a block of `units` (largest class whose lower bound is <= units)
+    static int class_floor(size_t units) {
+        if (units < 8) return (int)units;
+        const int fl = 63 - __builtin_clzll((unsigned long long)units);
+        const int sl = (int)((units >> (fl - 2)) & 3);
+        return 8 + (fl - 3) * 4 + sl;
+    }
+    // smallest class all of whose blocks hold `units`
+    static int class_ceil(size_t units) {
+        if (units < 8) return (int)units;
+        const int fl = 63 - __builtin_clzll((unsigned long long)units);
+        return class_floor(units + (((size_t)1 << (fl - 2)) - 1));
+    }
+    void push_free(Block* b) {
+        const int c = class_floor(b->size / min_split);
+        b->state = kFree;
+        b->fprev = nullptr;
+        b->fnext = free_head[c];
+        if (free_head[c]) free_head[c]->fprev = b;
+        free_head[c] = b;
+        class_bits[c >> 6] |= (uint64_t)1 << (c & 63);
+    }
+    void pop_free(Block* b) {
+        const int c = class_floor(b->size / min_split);
+        if (b->fprev) b->fprev->fnext = b->fnext;
+        else free_head[c] = b->fnext;
+        if (b->fnext) b->fnext->fprev = b->fprev;
+        if (!free_head[c]) class_bits[c >> 6] &= ~((uint64_t)1 << (c & 63));
+        b->fprev = b->fnext = nullptr;
+    }
+    int first_class_from(int c) const {
+        constexpr int kWords = (kClasses + 63) / 64;
+        if (c >= kClasses) return -1;
+        int w = c >> 6;
+        uint64_t bits = class_bits[w] & (~(uint64_t)0 << (c & 63));
+        while (true) {
+            if (bits) return (w << 6) + __builtin_ctzll(bits);
+            if (++w >= kWords) return -1;
+            bits = class_bits[w];
         }
     }
 
+    // ---- segments ----
     bool add_segment(zg_hip_ctx* ctx, size_t at_least) {
         if (ctx->capturing) return false;  // no driver allocation inside a graph capture
         size_t bytes = segment_bytes;
@@ -97,78 +183,122 @@ struct BlockPool {
             }
         }
         ctx->n_device_allocs++;
-        int seg = (int)segments.size();
-        segments.push_back(p);
         mapped += bytes;
-        Block b{(char*)p, bytes, true, seg};
-        blocks[b.ptr] = b;
-        free_by_size.insert({bytes, b.ptr});
+        Block* b = new_node();
+        b->ptr = (char*)p;
+        b->size = bytes;
+        segments.push_back(Segment{(char*)p, bytes, b});
+        push_free(b);
         return true;
     }
 
-    void* alloc(zg_hip_ctx* ctx, size_t bytes) {
-        size_t need = (bytes + min_split - 1) / min_split * min_split;
-        auto it = free_by_size.lower_bound(need);
-        if (it == free_by_size.end()) {
-            if (!add_segment(ctx, need)) return nullptr;
-            it = free_by_size.lower_bound(need);
-            if (it == free_by_size.end()) return nullptr;
-        }
-        char* p = it->second;
-        free_by_size.erase(it);
-        Block& b = blocks[p];
-        if (b.size - need >= min_split) {
-            Block rest{p + need, b.size - need, true, b.segment};
-            b.size = need;
-            blocks[rest.ptr] = rest;
-            free_by_size.insert({rest.size, rest.ptr});
-        }
-        b.free = false;
-        in_use += b.size;
-        return p;
+    // the tail of `b` beyond `keep` bytes becomes a block of its own, filed as free
+    void split_tail(Block* b, size_t keep) {
+        Block* rest = new_node();
+        rest->ptr = b->ptr + keep;
+        rest->size = b->size - keep;
+        rest->prev = b;
+        rest->next = b->next;
+        if (b->next) b->next->prev = rest;
+        b->next = rest;
+        b->size = keep;
+        push_free(rest);
     }
 
-    bool release(void* ptr) {
-        auto it = blocks.find((char*)ptr);
-        if (it == blocks.end() || it->second.free) return false;
-        Block& b = it->second;
-        in_use -= b.size;
-        b.free = true;
-        // fuse with the next block of the same segment
-        auto nx = std::next(it);
-        if (nx != blocks.end() && nx->second.free && nx->second.segment == b.segment &&
-            nx->second.ptr == b.ptr + b.size) {
-            erase_free(nx->second);
-            b.size += nx->second.size;
-            blocks.erase(nx);
+    Block* alloc(zg_hip_ctx* ctx, size_t bytes) {
+        const size_t need = (bytes + min_split - 1) / min_split * min_split;
+        const size_t units = need / min_split;
+        Block* b = nullptr;
+        // a block of the request's own class may fit (it does when it was freed by the same caller a step ago)
+        const int cf = class_floor(units);
+        int tries = 0;
+        for (Block* c = free_head[cf]; c && tries < 4; c = c->fnext, tries++)
+            if (c->size >= need) {
+                b = c;
+                break;
+            }
+        if (!b) {
+            int c = first_class_from(class_ceil(units));
+            if (c < 0) {
+                if (!add_segment(ctx, need)) return nullptr;
+                c = first_class_from(class_ceil(units));
+                if (c < 0) return nullptr;
+            }
+            b = free_head[c];
         }
-        // fuse with the previous block
-        if (it != blocks.begin()) {
-            auto pv = std::prev(it);
-            if (pv->second.free && pv->second.segment == b.segment && pv->second.ptr + pv->second.size == b.ptr) {
-                erase_free(pv->second);
-                pv->second.size += b.size;
-                blocks.erase(it);
-                it = pv;
+        pop_free(b);
+        if (b->size - need >= min_split) split_tail(b, need);
+        b->state = kLive;
+        in_use += b->size;
+        return b;
+    }
+
+    // `b` must be a live block of this pool
+    void release(Block* b) {
+        in_use -= b->size;
+        Block* nx = b->next;
+        if (nx && nx->state == kFree) {
+            pop_free(nx);
+            b->size += nx->size;
+            b->next = nx->next;
+            if (nx->next) nx->next->prev = b;
+            drop_node(nx);
+        }
+        Block* pv = b->prev;
+        if (pv && pv->state == kFree) {
+            pop_free(pv);
+            pv->size += b->size;
+            pv->next = b->next;
+            if (b->next) b->next->prev = pv;
+            drop_node(b);
+            b = pv;
+        }
+        push_free(b);
+    }
+
+    bool owns_live(const void* handle, const void* ptr) const {
+        if (!is_node(handle)) return false;
+        const Block* b = (const Block*)handle;
+        return b->pool == this && b->state == kLive && b->ptr == (const char*)ptr;
+    }
+
+    bool contains(const void* p) const {
+        for (const Segment& s : segments)
+            if ((const char*)p >= s.base && (const char*)p < s.base + s.bytes) return true;
+        return false;
+    }
+
+    // Takes every free byte of [lo, hi) out of circulation (as live blocks appended to `held`): the part of the
+    // range that callers still own is left alone.  Used when a recorded graph keeps naming addresses.
+    void reserve_range(char* lo, char* hi, std::vector<Block*>& held) {
+        for (Segment& s : segments) {
+            if (hi <= s.base || lo >= s.base + s.bytes) continue;
+            for (Block* b = s.first; b && b->ptr < hi; b = b->next) {
+                if (b->ptr + b->size <= lo || b->state != kFree) continue;
+                pop_free(b);
+                if (b->ptr < lo) {  // keep the front free, continue with the part inside the range
+                    const size_t front = (size_t)(lo - b->ptr);
+                    split_tail(b, front);  // files the tail as free
+                    push_free(b);
+                    b = b->next;
+                    pop_free(b);
+                }
+                if (b->ptr + b->size > hi) split_tail(b, (size_t)(hi - b->ptr));
+                b->state = kLive;
+                in_use += b->size;
+                held.push_back(b);
             }
         }
-        free_by_size.insert({it->second.size, it->second.ptr});
-        return true;
-    }
-
-    bool owns(void* ptr) const {
-        return blocks.find((char*)ptr) != blocks.end();
-    }
-    bool owns_live(void* ptr) const {
-        auto it = blocks.find((char*)ptr);
-        return it != blocks.end() && !it->second.free;
     }
 
     void destroy() {
-        for (void* s : segments) (void)hipFree(s);
+        for (Segment& s : segments) (void)hipFree(s.base);
         segments.clear();
-        blocks.clear();
-        free_by_size.clear();
+        for (Block* slab : slabs) delete[] slab;
+        slabs.clear();
+        unused_nodes = nullptr;
+        for (auto& h : free_head) h = nullptr;
+        for (auto& w : class_bits) w = 0;
         in_use = mapped = 0;
     }
 };
@@ -418,15 +548,33 @@ ZG_API int zg_hip_staging_wait(zg_hip_ctx* ctx) {
 struct zg_hip_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
-    std::vector<std::pair<void*, uint64_t>> parked;  // cache blocks freed inside the capture
+    std::vector<Block*> held;  // the cache memory the recorded ops name, kept out of the pools while the graph lives
 };
 
-static void unpark(zg_hip_ctx* ctx, std::vector<std::pair<void*, uint64_t>>& parked) {
-    for (auto& pb : parked) {
-        BlockPool* pool = pb.second == 2 ? ctx->large_pool : ctx->small_pool;
-        if (pool) (void)pool->release(pb.first);
+static void release_held(std::vector<Block*>& held) {
+    for (Block* b : held) b->pool->release(b);
+    held.clear();
+}
+
+// The address ranges of every cache block handed out or returned while recording, merged; whatever part of
+// them is free when the recording ends belongs to the graph from then on.
+static void hold_touched_ranges(zg_hip_ctx* ctx, std::vector<Block*>& held) {
+    auto& r = ctx->capture_touched;
+    std::sort(r.begin(), r.end());
+    size_t i = 0;
+    while (i < r.size()) {
+        char* lo = r[i].first;
+        char* hi = lo + r[i].second;
+        size_t j = i + 1;
+        while (j < r.size() && r[j].first <= hi) {
+            if (r[j].first + r[j].second > hi) hi = r[j].first + r[j].second;
+            j++;
+        }
+        for (BlockPool* pool : {ctx->small_pool, ctx->large_pool})
+            if (pool) pool->reserve_range(lo, hi, held);
+        i = j;
     }
-    parked.clear();
+    r.clear();
 }
 
 ZG_API int zg_hip_graph_open(zg_hip_ctx* ctx) {
@@ -434,6 +582,7 @@ ZG_API int zg_hip_graph_open(zg_hip_ctx* ctx) {
     ZG_NOT_CAPTURING(ctx, "graph_open");
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
     ZG_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capture_touched.clear();
     ctx->capturing = true;
     return ZG_HIP_OK;
 }
@@ -451,7 +600,7 @@ ZG_API int zg_hip_graph_save(zg_hip_ctx* ctx, zg_hip_graph** out) {
     hipError_t e = hipStreamEndCapture(ctx->stream, &g);
     if (e != hipSuccess || g == nullptr) {
         (void)hipGetLastError();
-        unpark(ctx, ctx->capture_parked);
+        ctx->capture_touched.clear();
         set_error("graph_save: hipStreamEndCapture failed: %s", hipGetErrorString(e));
         return ZG_HIP_ERUNTIME;
     }
@@ -460,14 +609,14 @@ ZG_API int zg_hip_graph_save(zg_hip_ctx* ctx, zg_hip_graph** out) {
     if (e != hipSuccess) {
         (void)hipGetLastError();
         (void)hipGraphDestroy(g);
-        unpark(ctx, ctx->capture_parked);
+        ctx->capture_touched.clear();
         set_error("graph_save: hipGraphInstantiate failed: %s", hipGetErrorString(e));
         return ZG_HIP_ERUNTIME;
     }
     zg_hip_graph* gr = new zg_hip_graph();
     gr->graph = g;
     gr->exec = exec;
-    gr->parked.swap(ctx->capture_parked);
+    hold_touched_ranges(ctx, gr->held);
     ctx->live_graphs++;
     *out = gr;
     return ZG_HIP_OK;
@@ -488,7 +637,7 @@ ZG_API int zg_hip_graph_free(zg_hip_ctx* ctx, zg_hip_graph* graph) {
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));  // a replay may still be running
     if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
     if (graph->graph) (void)hipGraphDestroy(graph->graph);
-    unpark(ctx, graph->parked);
+    release_held(graph->held);
     ctx->live_graphs--;
     delete graph;
     return ZG_HIP_OK;
@@ -649,8 +798,8 @@ ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uin
     bool large = bytes > kLargeThreshold;
     BlockPool*& pool = large ? ctx->large_pool : ctx->small_pool;
     if (!pool) pool = make_pool(large ? ctx->large_pool_bytes : ctx->small_pool_bytes);
-    void* p = pool->alloc(ctx, bytes);
-    if (!p) {
+    Block* b = pool->alloc(ctx, bytes);
+    if (!b) {
         if (ctx->capturing) {
             set_error("mem_cache_alloc: the pool would have to grow for %zu bytes while an execution graph is being "
                       "captured; run the same ops once eagerly first", bytes);
@@ -659,25 +808,50 @@ ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uin
         set_error("mem_cache_alloc: out of device memory for %zu bytes", bytes);
         return ZG_HIP_EOOM;
     }
-    *out = p;
-    *block = large ? 2 : 1;
+    if (ctx->capturing) ctx->capture_touched.push_back({b->ptr, b->size});
+    *out = b->ptr;
+    *block = (uint64_t)(uintptr_t)b;
     return ZG_HIP_OK;
 }
 
 ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     ZG_CTX(ctx);
     if (!ptr || block == 0) return ZG_HIP_OK;  // views and empty data: src/allocators/caching_allocator.zig:111-112
-    ZG_REQUIRE(block == 1 || block == 2, "mem_cache_free: bad block handle %llu", (unsigned long long)block);
-    BlockPool* pool = block == 2 ? ctx->large_pool : ctx->small_pool;
-    if (ctx->capturing) {
-        // the graph being recorded names this address: the block stays out of the pool until the graph is freed
-        ZG_REQUIRE(pool && pool->owns_live(ptr), "mem_cache_free: %p is not a live block of this pool", ptr);
-        ctx->capture_parked.push_back({ptr, block});
-        return ZG_HIP_OK;
+    Block* b = (Block*)(uintptr_t)block;
+    BlockPool* pool = nullptr;
+    for (BlockPool* p : {ctx->small_pool, ctx->large_pool})
+        if (p && p->owns_live(b, ptr)) pool = p;
+    ZG_REQUIRE(pool != nullptr, "mem_cache_free: %p with handle %llx is not a live block of this context's pools", ptr,
+               (unsigned long long)block);
+    // While recording, the block goes back to the pool like any other, so a later allocation of the same recording
+    // may reuse it (the graph keeps the stream's order); its range is noted, and whatever part of the noted ranges is
+    // free when the recording ends stays with the graph.  Outside a recording, stream order makes reuse safe: a
+    // later op that receives this block runs after every op already enqueued on the same stream.
+    if (ctx->capturing) ctx->capture_touched.push_back({b->ptr, b->size});
+    pool->release(b);
+    return ZG_HIP_OK;
+}
+
+// Whether `ptr` lies in memory this context handed out as device memory (cache pools, raw allocations, scratch):
+// what a binding needs to tell a device slice from a host scalar (the reference's callers pass both through the
+// same parameter: src/ndarray.zig:251, src/nn/optim.zig:117 against src/ndtensor.zig:1146-1150).
+ZG_API int zg_hip_is_device_ptr(zg_hip_ctx* ctx, const void* ptr, int* yes) {
+    ZG_CTX(ctx);
+    ZG_REQUIRE(yes != nullptr, "is_device_ptr: null output");
+    *yes = 0;
+    if (!ptr) return ZG_HIP_OK;
+    for (BlockPool* p : {ctx->small_pool, ctx->large_pool})
+        if (p && p->contains(ptr)) *yes = 1;
+    if (!*yes && ctx->scratch && (const char*)ptr >= (const char*)ctx->scratch &&
+        (const char*)ptr < (const char*)ctx->scratch + ctx->scratch_bytes)
+        *yes = 1;
+    if (!*yes && !ctx->raw_allocs.empty()) {
+        auto it = ctx->raw_allocs.upper_bound(const_cast<void*>(ptr));
+        if (it != ctx->raw_allocs.begin()) {
+            --it;
+            if ((const char*)ptr < (const char*)it->first + it->second) *yes = 1;
+        }
     }
-    // Stream order makes reuse safe: a later op that receives this block runs after every op
-    // already enqueued on the same stream.
-    ZG_REQUIRE(pool && pool->release(ptr), "mem_cache_free: %p is not a live block of this pool", ptr);
     return ZG_HIP_OK;
 }
 
@@ -686,9 +860,12 @@ ZG_API int zg_hip_mem_scratch(zg_hip_ctx* ctx, size_t bytes, void** out) {
     ZG_REQUIRE(out != nullptr, "mem_scratch: null output");
     if (bytes > ctx->scratch_bytes) {
         ZG_NOT_CAPTURING(ctx, "mem_scratch (growing)");
-        ZG_REQUIRE(ctx->live_graphs == 0, "mem_scratch: cannot grow while an execution graph may name the old buffer");
         ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
-        if (ctx->scratch) ZG_HIP_TRY(hipFree(ctx->scratch));
+        if (ctx->scratch) {
+            // an instantiated graph may have recorded the old address: keep it alive until the context goes
+            if (ctx->live_graphs > 0) ctx->retired_ws.push_back(ctx->scratch);
+            else ZG_HIP_TRY(hipFree(ctx->scratch));
+        }
         ctx->scratch = nullptr;
         ctx->scratch_bytes = 0;
         size_t want = (bytes + kPoolAlign - 1) / kPoolAlign * kPoolAlign;

@@ -177,6 +177,16 @@ class HipDevice:
     def clear_cache(self) -> None:
         self._call("zg_hip_clear_cache")
 
+    def cache_configure(self, small_pool_bytes: int, large_pool_bytes: int) -> None:
+        """Segment sizes of the two block pools (CachingAllocator.Options, src/allocators/caching_allocator.zig:41-44);
+        only before the first cache allocation or after clear_cache()."""
+        self._call("zg_hip_cache_configure", int(small_pool_bytes), int(large_pool_bytes))
+
+    def is_device_ptr(self, ptr: int) -> bool:
+        yes = ctypes.c_int(0)
+        self._call("zg_hip_is_device_ptr", ctypes.c_void_p(ptr), ctypes.byref(yes))
+        return bool(yes.value)
+
     def cache_stats(self) -> dict:
         u, m, a = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_uint64()
         self._call("zg_hip_cache_stats", ctypes.byref(u), ctypes.byref(m), ctypes.byref(a))

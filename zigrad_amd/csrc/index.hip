@@ -22,8 +22,16 @@ struct Plan {
     uint32_t* peer;      // n: optional payload (the other endpoint of an edge) in the order of perm
     uint32_t* peer_tmp;  // n: the payload in the order of perm_tmp
     uint32_t* tile_sums; // scan scratch
+    uint32_t* long_list; // [0] = number of long buckets, then their ids (at most n / kLongBucket of them)
     size_t n, nb;
 };
+
+// A bucket with more entries than this is "long": its entries are added by a whole wave (loads in parallel, additions
+// still one after the other in input order) instead of by one thread.
+constexpr uint32_t kLongBucket = 256;
+// Up to this length a bucket is put back into input order by ranking every entry against every other (len^2 / 64
+// loads per lane); beyond it the bucket is rebuilt in order by one pass over the input.
+constexpr uint32_t kRankMax = 1024;
 
 constexpr int kScanTile = 2048;  // elements per workgroup of the scan (256 threads x 8)
 
@@ -33,7 +41,8 @@ static size_t align_up(size_t v, size_t a) {
 
 static size_t plan_bytes(size_t n, size_t nb) {
     size_t tiles = ceil_div_sz(nb + 1, kScanTile);
-    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 4 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256);
+    return align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 4 * align_up(n * 4, 256) + align_up((tiles + 1) * 4, 256) +
+           align_up((n / kLongBucket + 2) * 4, 256);
 }
 
 static Plan carve_plan(void* mem, size_t n, size_t nb) {
@@ -54,13 +63,16 @@ static Plan carve_plan(void* mem, size_t n, size_t nb) {
     pl.peer_tmp = (uint32_t*)p;
     p += align_up(n * 4, 256);
     pl.tile_sums = (uint32_t*)p;
+    p += align_up((ceil_div_sz(nb + 1, kScanTile) + 1) * 4, 256);
+    pl.long_list = (uint32_t*)p;
     return pl;
 }
 
-__global__ void zero_u32_kernel(uint32_t* a, size_t na, uint32_t* b, size_t nb) {
+__global__ void zero_u32_kernel(uint32_t* a, size_t na, uint32_t* b, size_t nb, uint32_t* one = nullptr) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
     for (size_t k = i; k < na; k += nt) a[k] = 0;
     for (size_t k = i; k < nb; k += nt) b[k] = 0;
+    if (i == 0 && one) one[0] = 0;
 }
 
 // key = idx[e] / divisor (divisor 1 for plain indices)
@@ -192,12 +204,17 @@ __global__ void place_kernel(const uint64_t* keys, size_t n, size_t nb, const ui
 // Put each bucket back into ascending input position: rank of an entry = number of smaller entries
 // in its bucket.  One wave per bucket.
 // With `peer_tmp` the payload is laid out in the same order, so that the apply kernels read it next to perm.
+// Buckets of more than kLongBucket entries are listed in `long_list`; those of more than kRankMax entries are left
+// to order_long_segments_kernel (ranking them here would cost len^2 loads in one wave).
 __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
-                                                              uint32_t* perm, const uint32_t* peer_tmp, uint32_t* peer) {
+                                                              uint32_t* perm, const uint32_t* peer_tmp, uint32_t* peer,
+                                                              uint32_t* long_list) {
     const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= nb) return;
     const int lane = threadIdx.x & 63;
     const uint32_t s = row_ptr[b], len = row_ptr[b + 1] - s;
+    if (len > kLongBucket && lane == 0) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)b;
+    if (len > kRankMax) return;
     for (uint32_t i = lane; i < len; i += 64) {
         const uint32_t id = perm_tmp[s + i];
         uint32_t rank = 0;
@@ -207,12 +224,72 @@ __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row
     }
 }
 
+// The buckets of more than kRankMax entries, rebuilt in input order: one workgroup per such bucket walks the whole
+// key array, 4096 entries a round, and writes the positions whose key is the bucket's, in order (a workgroup-wide
+// prefix sum of the per-thread match counts gives each thread its place).  Cost: one read of the key array per very
+// long bucket, and there are at most n / kRankMax of them.
+constexpr int kOrderLongThreads = 1024;
+__global__ __launch_bounds__(kOrderLongThreads) void order_long_segments_kernel(const uint64_t* keys, size_t n,
+                                                                                const uint32_t* row_ptr,
+                                                                                const uint32_t* long_list, uint32_t* perm,
+                                                                                const uint64_t* payload, uint32_t* peer) {
+    __shared__ uint32_t wave_tot[kOrderLongThreads / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n_long = long_list[0];
+    for (uint32_t li = blockIdx.x; li < n_long; li += gridDim.x) {
+        const uint32_t b = long_list[1 + li];
+        const uint32_t s = row_ptr[b], len = row_ptr[b + 1] - s;
+        if (len <= kRankMax) continue;  // ordered by order_segments_kernel already (uniform over the workgroup)
+        uint32_t written = 0;
+        for (size_t e0 = 0; e0 < n; e0 += (size_t)kOrderLongThreads * 4) {
+            const size_t mine = e0 + (size_t)threadIdx.x * 4;
+            bool hit[4];
+            uint32_t cnt = 0;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                hit[u] = (mine + u < n) && keys[mine + u] == (uint64_t)b;
+                cnt += hit[u] ? 1u : 0u;
+            }
+            uint32_t inc = cnt;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t t = __shfl_up(inc, d, 64);
+                if (lane >= d) inc += t;
+            }
+            __syncthreads();  // wave_tot of the previous round has been read by everyone
+            if (lane == 63) wave_tot[wave] = inc;
+            __syncthreads();
+            uint32_t before = 0, total = 0;
+            for (int w = 0; w < kOrderLongThreads / 64; w++) {
+                const uint32_t t = wave_tot[w];
+                before += (w < wave) ? t : 0u;
+                total += t;
+            }
+            uint32_t pos = s + written + before + inc - cnt;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (hit[u]) {
+                    if (pos < s + len) {  // cannot fail: the histogram counted the same matches
+                        perm[pos] = (uint32_t)(mine + u);
+                        if (payload) {
+                            const uint64_t v = payload[mine + u];
+                            peer[pos] = v < 0xffffffffull ? (uint32_t)v : 0xffffffffu;
+                        }
+                    }
+                    pos++;
+                }
+            }
+            written += total;
+        }
+    }
+}
+
 static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, const uint64_t* payload = nullptr) {
     hipStream_t st = ctx->stream;
     const size_t n = pl.n, nb = pl.nb;
     const int g_n = (int)(ceil_div_sz(n ? n : 1, 256) > 4096 ? 4096 : ceil_div_sz(n ? n : 1, 256));
     const int g_b = (int)(ceil_div_sz(nb + 1, 256) > 4096 ? 4096 : ceil_div_sz(nb + 1, 256));
-    hipLaunchKernelGGL(zero_u32_kernel, dim3(g_b), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.cursor, nb);
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(g_b), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.cursor, nb, pl.long_list);
     ZG_LAUNCH_CHECK();
     if (n) {
         hipLaunchKernelGGL(histogram_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr);
@@ -235,8 +312,15 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
                            pl.peer_tmp);
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(nb, 4)), dim3(256), 0, st, pl.row_ptr, nb,
-                           pl.perm_tmp, pl.perm, payload ? pl.peer_tmp : (const uint32_t*)nullptr, pl.peer);
+                           pl.perm_tmp, pl.perm, payload ? pl.peer_tmp : (const uint32_t*)nullptr, pl.peer, pl.long_list);
         ZG_LAUNCH_CHECK();
+        if (n > kRankMax) {  // only then can a bucket be too long to rank; the workgroups exit at once when none is
+            size_t grid = n / kRankMax;
+            if (grid > 1024) grid = 1024;
+            hipLaunchKernelGGL(order_long_segments_kernel, dim3((unsigned)grid), dim3(kOrderLongThreads), 0, st, keys, n,
+                               pl.row_ptr, pl.long_list, pl.perm, payload, pl.peer);
+            ZG_LAUNCH_CHECK();
+        }
     }
     return ZG_HIP_OK;
 }
@@ -256,9 +340,46 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
         if (fresh) dst[b] = 0.f;
         return;
     }
+    if (e - s > kLongBucket) return;  // scatter_add_apply_long_kernel's
     float acc = fresh ? 0.f : dst[b];
     for (uint32_t k = s; k < e; k++) acc = __fadd_rn(acc, src[perm[k]]);
     dst[b] = acc;
+}
+
+// The long buckets: one wave per destination.  The wave loads 64 contributions at a time (the loads do not depend
+// on the running sum), then adds them one after the other in input order, every lane forming the same sum.
+__global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float* src, const uint32_t* row_ptr,
+                                                                      const uint32_t* perm, const uint32_t* long_list,
+                                                                      float* dst, bool fresh) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t n_long = long_list[0];
+    const uint32_t wave0 = blockIdx.x * 4 + (threadIdx.x >> 6), n_waves = gridDim.x * 4;
+    for (uint32_t li = wave0; li < n_long; li += n_waves) {
+        const uint32_t b = long_list[1 + li];
+        const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
+        float acc = fresh ? 0.f : dst[b];
+        for (uint32_t k0 = s; k0 < e; k0 += 64) {
+            const uint32_t k = k0 + lane;
+            const float v = (k < e) ? src[perm[k]] : 0.f;
+            const int cnt = (e - k0 < 64u) ? (int)(e - k0) : 64;
+            for (int j = 0; j < cnt; j++) acc = __fadd_rn(acc, __shfl(v, j, 64));
+        }
+        if (lane == 0) dst[b] = acc;
+    }
+}
+
+static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Plan& pl, float* dst, bool fresh) {
+    hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(pl.nb, 256)), dim3(256), 0, ctx->stream, src,
+                       pl.row_ptr, pl.perm, dst, pl.nb, fresh);
+    ZG_LAUNCH_CHECK();
+    if (pl.n > kLongBucket) {
+        size_t grid = ceil_div_sz(pl.n / kLongBucket, 4);
+        if (grid > 2048) grid = 2048;
+        hipLaunchKernelGGL(scatter_add_apply_long_kernel, dim3((unsigned)grid), dim3(256), 0, ctx->stream, src, pl.row_ptr,
+                           pl.perm, pl.long_list, dst, fresh);
+        ZG_LAUNCH_CHECK();
+    }
+    return ZG_HIP_OK;
 }
 
 // The whole of scatter_add for at most kScatterSmallMax entries in one launch of one workgroup: thread i owns entry i,
@@ -530,7 +651,7 @@ static int gather_impl(zg_hip_ctx* ctx, const char* name, const uint64_t* src_sh
     int* d_status = status ? (int*)(ctx->scalar_slot + 2) : nullptr;
     if (d_status) {
         hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(64), 0, ctx->stream, (uint32_t*)d_status, (size_t)1,
-                           (uint32_t*)nullptr, (size_t)0);
+                           (uint32_t*)nullptr, (size_t)0, (uint32_t*)nullptr);
         ZG_LAUNCH_CHECK();
     }
     hipLaunchKernelGGL(gather_offsets_kernel, dim3((unsigned)ceil_div_sz(n, 256)), dim3(256), 0, ctx->stream, indices, n,
@@ -580,10 +701,7 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
     if (!mem) return ZG_HIP_EOOM;
     Plan pl = carve_plan(mem, n, dst_len);
     if (int rc = build_plan(ctx, offsets, pl)) return rc;
-    hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(dst_len, 256)), dim3(256), 0, ctx->stream,
-                       src, pl.row_ptr, pl.perm, dst, dst_len, false);
-    ZG_LAUNCH_CHECK();
-    return ZG_HIP_OK;
+    return launch_scatter_add_apply(ctx, src, pl, dst, false);
 }
 
 ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src_len, const uint64_t* indices,
@@ -806,10 +924,7 @@ ZG_API int zg_hip_scatter_add_planned(zg_hip_ctx* ctx, const float* src, const z
                                       int accumulate) {
     ZG_CTX(ctx);
     ZG_REQUIRE(plan && src && dst, "scatter_add_planned: null pointer");
-    hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(plan->n_nodes, 256)), dim3(256), 0,
-                       ctx->stream, src, plan->by_tgt.row_ptr, plan->by_tgt.perm, dst, plan->n_nodes, accumulate == 0);
-    ZG_LAUNCH_CHECK();
-    return ZG_HIP_OK;
+    return launch_scatter_add_apply(ctx, src, plan->by_tgt, dst, accumulate == 0);
 }
 
 ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,

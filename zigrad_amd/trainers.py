@@ -95,7 +95,7 @@ class Optimizer:
 
     def prepare_replay(self) -> None:
         """Host part of one replayed step: advance the per-tensor counter and publish each tensor's lr_t.
-        The previous replay must have finished (the trainers read the loss back every step)."""
+        The previous replay must have finished (GraphSteps.step_graph waits for it when the loss was not read)."""
         if self.kind != "adam":
             return
         for i in range(len(self.params)):
@@ -174,12 +174,20 @@ class GraphSteps:
             self.optim.capturing = False
             self.graph = self.dev.graph_save()
 
+    _replay_pending = False
+
     def step_graph(self, read_loss: bool = True):
+        # Adam's recorded kernels read each tensor's lr_t from pinned host memory when they run: the slots may only
+        # be rewritten once the previous replay has finished
+        if self._replay_pending and self.optim.kind == "adam":
+            self.dev.sync()
         self.optim.prepare_replay()
         self.graph.run()
         if not read_loss:
+            self._replay_pending = True
             return None
         self.dev.sync()
+        self._replay_pending = False
         return float(self._loss_view[0])
 
     def free_graph(self) -> None:

@@ -59,9 +59,22 @@ def gemm_bytes_per_step(dims, batch):
     return total
 
 
-# HBM-side bytes per GEMM launch (average over the step's 8 launches), from two rocprofv3 counter runs of this
-# script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the copy_calibration kernel.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 492.0e6
+# HBM-side bytes per GEMM launch (average over the step's 8 launches): measured by two rocprofv3 counter runs of this
+# script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the copy_calibration kernel.  The
+# figure is read from the committed summary of those runs, so it cannot drift from it; without the file it is null.
+GEMM_TRAFFIC_PROFILE = Path(__file__).resolve().parent / "profiles" / "gemm_kernel_wide_mlp_step_hbm_traffic.txt"
+
+
+def gemm_traffic_bytes_per_launch(path=GEMM_TRAFFIC_PROFILE):
+    """The 'All N launches ...: X MB per launch on average (B bytes).' line of the traffic summary -> B, else None."""
+    import re
+
+    try:
+        text = Path(path).read_text()
+    except OSError:
+        return None
+    m = re.search(r"^All \d+ launches.*per launch on average \((\d+) bytes\)", text, re.M)
+    return float(m.group(1)) if m else None
 
 
 class GemmTimer:
@@ -337,7 +350,7 @@ def run_small(dev, kind, steps, graph=True, fused=False):
 
 
 def run_c_harness(dims, batch, steps, fused=False):
-    """The same eager batch-64 step issued from plain C (tests/c_harness/mlp_step.c): what the op-by-op path costs
+    """The same eager batch-64 step issued from plain C (examples/c_caller/mlp_step.c): what the op-by-op path costs
     without an interpreter between the calls.  None when the binary has not been built."""
     import subprocess
     import tempfile
@@ -355,7 +368,7 @@ def run_c_harness(dims, batch, steps, fused=False):
         run = subprocess.run([str(C_HARNESS_BIN), f.name, str(steps), str(batch), *map(str, dims), *(["fused"] if fused else [])],
                              capture_output=True, text=True, timeout=300)
     if run.returncode != 0:
-        raise RuntimeError("tests/c_harness/mlp_step failed: " + run.stderr)
+        raise RuntimeError("examples/c_caller/mlp_step failed: " + run.stderr)
     us = float(run.stdout.strip().splitlines()[-1].split()[1])
     what = "eager, fused entry points, caller in C" if fused else "eager, same op sequence, caller in C"
     return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": what}
@@ -460,7 +473,7 @@ def main():
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": gemm_traffic_bytes_per_launch(),
             "traffic_unit": "bytes per launch (L2 misses to the fabric, rocprofv3 FETCH_SIZE + WRITE_SIZE)",
             "algorithmic_bytes_per_launch": gemm_bytes_per_step(WIDE_DIMS, WIDE_BATCH) / 8,
             "kernel": "gemm_kernel (fp32 MFMA 32x32x2), 8 launches per step",

@@ -1,4 +1,4 @@
-"""The batch-64 MLP train step driven from plain C through the C ABI (tests/c_harness/mlp_step.c) gives, step for
+"""The batch-64 MLP train step driven from plain C through the C ABI (examples/c_caller/mlp_step.c) gives, step for
 step, the losses the Python trainer gives on the same parameters and batch: the boundary needs nothing from Python."""
 from __future__ import annotations
 

@@ -78,18 +78,18 @@ def build(force: bool = False, jobs: int | None = None) -> Path:
     return LIB_PATH
 
 
-C_HARNESS_SRC = PKG_DIR.parent / "tests" / "c_harness" / "mlp_step.c"
+C_HARNESS_SRC = PKG_DIR.parent / "examples" / "c_caller" / "mlp_step.c"
 C_HARNESS_BIN = C_HARNESS_SRC.with_suffix("")
 
 
 def build_c_harness() -> Path:
-    """The plain-C caller of the C ABI (tests/c_harness/mlp_step.c), linked against the library in its tree."""
+    """The plain-C caller of the C ABI (examples/c_caller/mlp_step.c), linked against the library in its tree."""
     cmd = ["gcc", "-std=c11", "-O2", "-Wall", "-Werror", "-D_POSIX_C_SOURCE=199309L", f"-I{PKG_DIR.parent / 'include'}",
            str(C_HARNESS_SRC), "-o", str(C_HARNESS_BIN), f"-L{PKG_DIR}", "-lzg_hip", "-Wl,-rpath,$ORIGIN/../../zigrad_amd"]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("gcc failed for tests/c_harness/mlp_step.c")
+        raise RuntimeError("gcc failed for examples/c_caller/mlp_step.c")
     return C_HARNESS_BIN
 
 

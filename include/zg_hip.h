@@ -249,6 +249,18 @@ int zg_hip_scatter_add_csr(zg_hip_ctx *ctx, const float *src, const uint64_t *ro
 int zg_hip_segment_sum_csr(zg_hip_ctx *ctx, const float *src, size_t src_len, const uint64_t *row_offsets,
                            size_t n_segments, float *dst);
 
+/* Kept plans.  When the index arrays of zg_hip_scatter_add, zg_hip_index_select_bwd, zg_hip_scatter_gcn_deg_scaled or
+ * zg_hip_scatter_gcn_deg_scaled_bwd lie in zg_hip_host_alloc memory (where the reference's callers write them with
+ * host loops, examples/gcn/src/model.zig:204-205), the context keeps the destination ordering it computed, a host
+ * copy of the arrays' contents and a device copy for the kernels.  A later call whose arrays hold the same values
+ * (compared on the host, byte for byte, when the call is made) runs the same apply kernels on the kept ordering
+ * instead of computing it again: same values, five to six launches fewer per ordering.  At most 16 orderings are
+ * kept (least recently used goes first).  A recorded graph keeps the orderings it used, and zg_hip_graph_run returns
+ * ZG_HIP_EINVAL when one of those arrays no longer holds what it held at the recording.  Index arrays in device
+ * memory are analysed on every call.  `hits` / `builds` count calls served from a kept ordering / orderings computed
+ * and kept; no counterpart in the reference. */
+int zg_hip_plan_cache_stats(zg_hip_ctx *ctx, uint64_t *hits, uint64_t *builds);
+
 /* Edge plans.  The three ops above sort the edge list by destination on every call, because the reference hands
  * them bare index slices (examples/gcn/src/model.zig:116-224 builds them per forward).  For an edge list that does
  * not change between calls (the dataset's graph, examples/gcn/src/dataset.zig:110-127) the analysis can be done

@@ -23,6 +23,15 @@ constexpr size_t kPoolAlign = 256; // min split size of the block pools, bytes
 void set_error(const char* fmt, ...);
 
 struct BlockPool;  // runtime.hip
+struct PlanCache;  // index.hip
+struct CachedPlan;
+
+// One use of a cached segment plan by an op call: the entry and the caller's index arrays it was matched against.
+struct PlanUse {
+    CachedPlan* entry;
+    const uint64_t* keys;
+    const uint64_t* payload;
+};
 
 }  // namespace zg
 
@@ -70,6 +79,11 @@ struct zg_hip_ctx {
     int live_graphs = 0;
     std::vector<void*> retired_ws;  // outgrown workspaces that an instantiated graph may still name
 
+    // segment plans of index arrays in pinned host memory, kept between calls and matched by content (index.hip);
+    // plan_uses: the cached plans the ops of the recording in progress launched their kernels on
+    zg::PlanCache* plan_cache = nullptr;
+    std::vector<zg::PlanUse> plan_uses;
+
     // regions handed out by pool_map/alloc, for ownership checks at free time
     std::map<void*, size_t> raw_allocs;
     std::map<void*, size_t> host_allocs;
@@ -79,6 +93,13 @@ namespace zg {
 
 // Returns a workspace of at least `bytes` bytes (256-byte aligned), or nullptr with the error set.
 void* workspace(zg_hip_ctx* ctx, size_t bytes);
+
+// Cached segment plans (index.hip).  destroy: at deinit.  retain: a saved graph takes (+1) or drops (-1) its plans,
+// which are never evicted while a graph names them.  validate: before a replay, every index array the recording
+// matched must still hold what it held then, or the replay would scatter by a stale plan.
+void plan_cache_destroy(zg_hip_ctx* ctx);
+void plan_uses_retain(const std::vector<PlanUse>& uses, int delta);
+int plan_uses_validate(zg_hip_ctx* ctx, const std::vector<PlanUse>& uses);
 
 // Looks up the device address of the fixed scratch array (loss.hip); the context's device must be current.
 int noalloc_setup(zg_hip_ctx* ctx);

@@ -326,6 +326,160 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
 }
 
 // ------------------------------------------------------------------------------------------------
+// Plan cache.  The reference's callers keep their index arrays (edge lists, gather offsets) in memory the host
+// writes, here pinned host memory from zg_hip_host_alloc, and pass the same arrays call after call: a graph
+// convolution step builds eight plans of the same two arrays.  A context therefore keeps the plans it built for
+// such arrays, together with a host copy of what the arrays held and a device copy for the kernels, and a later
+// call whose arrays hold the same values (compared on the host, byte for byte, at the time of the call) launches
+// its apply kernels on the kept plan.  Same plan, same kernels, same results; what is saved is five to six launches
+// per plan and the kernels' reads of the indices across the bus.  Arrays in device memory cannot be compared without
+// waiting for the GPU and take the uncached path.  A hit while an execution graph is being recorded is noted in the
+// context so that the saved graph keeps the plan alive and zg_hip_graph_run can refuse a replay after the caller
+// has rewritten the arrays.
+// ------------------------------------------------------------------------------------------------
+constexpr size_t kPlanCacheMax = 16;
+constexpr size_t kPlanCacheMaxEntries = (size_t)1 << 24;  // longer index arrays are not worth a host comparison per call
+
+struct CachedPlan {
+    std::vector<uint64_t> keys_host, payload_host;  // what the arrays held when the plan was built
+    void* mem = nullptr;                             // one device allocation: the plan, then the device copies
+    Plan plan;
+    uint64_t* keys_dev = nullptr;
+    uint64_t* payload_dev = nullptr;  // null: built without payload
+    uint64_t last_use = 0;
+    int graph_refs = 0;
+};
+
+struct PlanCache {
+    std::vector<CachedPlan*> entries;
+    uint64_t clock = 0;
+    uint64_t hits = 0, builds = 0;
+};
+
+static bool in_pinned_host(zg_hip_ctx* ctx, const void* p, size_t bytes) {
+    auto it = ctx->host_allocs.upper_bound(const_cast<void*>(p));
+    if (it == ctx->host_allocs.begin()) return false;
+    --it;
+    const char* lo = (const char*)it->first;
+    return (const char*)p >= lo && (const char*)p + bytes <= lo + it->second;
+}
+
+// What an op launches its apply kernels on: a plan and device-readable copies of the arrays it was built from.
+struct PlanRef {
+    Plan plan;
+    const uint64_t* keys;
+    const uint64_t* payload;
+};
+
+// True when `out` names a cached plan for these arrays (found, or built and kept by this call).  False: the caller
+// builds the plan in the workspace as before (*rc says whether that is because of an error).
+static bool plan_from_cache(zg_hip_ctx* ctx, const uint64_t* keys, const uint64_t* payload, size_t n, size_t nb,
+                            PlanRef* out, int* rc) {
+    *rc = ZG_HIP_OK;
+    if (n == 0 || n > kPlanCacheMaxEntries) return false;
+    const size_t bytes = n * sizeof(uint64_t);
+    if (!in_pinned_host(ctx, keys, bytes) || (payload && !in_pinned_host(ctx, payload, bytes))) return false;
+    if (!ctx->plan_cache) ctx->plan_cache = new PlanCache();
+    PlanCache& pc = *ctx->plan_cache;
+    CachedPlan* hit = nullptr;
+    for (CachedPlan* e : pc.entries) {
+        if (e->plan.n != n || e->plan.nb != nb) continue;
+        if (payload && !e->payload_dev) continue;  // an entry with a payload also serves a call without one
+        if (memcmp(e->keys_host.data(), keys, bytes) != 0) continue;
+        if (payload && memcmp(e->payload_host.data(), payload, bytes) != 0) continue;
+        hit = e;
+        break;
+    }
+    if (!hit) {
+        if (ctx->capturing) return false;  // building one allocates; the recording builds its plan in the workspace
+        if (pc.entries.size() >= kPlanCacheMax) {
+            size_t victim = pc.entries.size();
+            for (size_t i = 0; i < pc.entries.size(); i++)
+                if (pc.entries[i]->graph_refs == 0 &&
+                    (victim == pc.entries.size() || pc.entries[i]->last_use < pc.entries[victim]->last_use))
+                    victim = i;
+            if (victim == pc.entries.size()) return false;  // every entry is named by a saved graph
+            if (hipStreamSynchronize(ctx->stream) != hipSuccess) return false;  // queued kernels may read the victim
+            CachedPlan* v = pc.entries[victim];
+            zg_hip_free(ctx, v->mem);
+            delete v;
+            pc.entries.erase(pc.entries.begin() + victim);
+        }
+        const size_t pb = align_up(plan_bytes(n, nb), 256), ib = align_up(bytes, 256);
+        void* mem = nullptr;
+        if ((*rc = zg_hip_alloc(ctx, pb + (payload ? 2 : 1) * ib, &mem))) return false;
+        CachedPlan* e = new CachedPlan();
+        e->mem = mem;
+        e->plan = carve_plan(mem, n, nb);
+        e->keys_dev = (uint64_t*)((char*)mem + pb);
+        e->keys_host.assign(keys, keys + n);
+        // the device copies are taken from the host snapshots' source at the same moment; both are pinned memory
+        *rc = zg_hip_memcpy_d2d(ctx, e->keys_dev, keys, bytes);
+        if (!*rc && payload) {
+            e->payload_dev = (uint64_t*)((char*)mem + pb + ib);
+            e->payload_host.assign(payload, payload + n);
+            *rc = zg_hip_memcpy_d2d(ctx, e->payload_dev, payload, bytes);
+        }
+        if (!*rc) *rc = build_plan(ctx, e->keys_dev, e->plan, e->payload_dev);
+        if (*rc) {
+            (void)hipStreamSynchronize(ctx->stream);
+            zg_hip_free(ctx, mem);
+            delete e;
+            return false;
+        }
+        pc.entries.push_back(e);
+        pc.builds++;
+        hit = e;
+    } else {
+        pc.hits++;
+    }
+    hit->last_use = ++pc.clock;
+    if (ctx->capturing) ctx->plan_uses.push_back(PlanUse{hit, keys, payload});
+    out->plan = hit->plan;
+    out->keys = hit->keys_dev;
+    out->payload = hit->payload_dev;
+    return true;
+}
+
+void plan_cache_destroy(zg_hip_ctx* ctx) {
+    if (!ctx->plan_cache) return;
+    for (CachedPlan* e : ctx->plan_cache->entries) {
+        zg_hip_free(ctx, e->mem);
+        delete e;
+    }
+    delete ctx->plan_cache;
+    ctx->plan_cache = nullptr;
+}
+
+void plan_uses_retain(const std::vector<PlanUse>& uses, int delta) {
+    for (const PlanUse& u : uses) u.entry->graph_refs += delta;
+}
+
+int plan_uses_validate(zg_hip_ctx* ctx, const std::vector<PlanUse>& uses) {
+    // an array that compared equal to one snapshot equals every snapshot the recording matched it against
+    const void* seen[2 * kPlanCacheMax];
+    size_t n_seen = 0;
+    auto check = [&](const uint64_t* p, const std::vector<uint64_t>& snap) -> int {
+        for (size_t i = 0; i < n_seen; i++)
+            if (seen[i] == p) return ZG_HIP_OK;
+        const size_t bytes = snap.size() * sizeof(uint64_t);
+        ZG_REQUIRE(in_pinned_host(ctx, p, bytes),
+                   "graph_run: an index array named by the recording is no longer a zg_hip_host_alloc allocation");
+        ZG_REQUIRE(memcmp(p, snap.data(), bytes) == 0,
+                   "graph_run: an index array was rewritten after the step was recorded; the recorded kernels would "
+                   "scatter by its old contents (record the step again)");
+        if (n_seen < 2 * kPlanCacheMax) seen[n_seen++] = p;
+        return ZG_HIP_OK;
+    };
+    for (const PlanUse& u : uses) {
+        if (int rc = check(u.keys, u.entry->keys_host)) return rc;
+        if (u.payload)
+            if (int rc = check(u.payload, u.entry->payload_host)) return rc;
+    }
+    return ZG_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
 // apply kernels
 // ------------------------------------------------------------------------------------------------
 
@@ -697,11 +851,16 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    void* mem = workspace(ctx, plan_bytes(n, dst_len));
-    if (!mem) return ZG_HIP_EOOM;
-    Plan pl = carve_plan(mem, n, dst_len);
-    if (int rc = build_plan(ctx, offsets, pl)) return rc;
-    return launch_scatter_add_apply(ctx, src, pl, dst, false);
+    PlanRef pr;
+    int rc = 0;
+    if (!plan_from_cache(ctx, offsets, nullptr, n, dst_len, &pr, &rc)) {
+        if (rc) return rc;
+        void* mem = workspace(ctx, plan_bytes(n, dst_len));
+        if (!mem) return ZG_HIP_EOOM;
+        pr.plan = carve_plan(mem, n, dst_len);
+        if ((rc = build_plan(ctx, offsets, pr.plan))) return rc;
+    }
+    return launch_scatter_add_apply(ctx, src, pr.plan, dst, false);
 }
 
 ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src_len, const uint64_t* indices,
@@ -727,10 +886,16 @@ ZG_API int zg_hip_index_select_bwd(zg_hip_ctx* ctx, const float* y_grad, const u
     ZG_REQUIRE(x_len >= stride, "index_select_bwd: gradient shorter than one row");
     const size_t nb = x_len / stride;
     ZG_REQUIRE(n_idx < 0xffffffffull && nb < 0xffffffffull, "index_select_bwd: sizes beyond 2^32-1");
-    void* mem = workspace(ctx, plan_bytes(n_idx, nb));
-    if (!mem) return ZG_HIP_EOOM;
-    Plan pl = carve_plan(mem, n_idx, nb);
-    if (int rc = build_plan(ctx, indices, pl)) return rc;
+    PlanRef pr;
+    int rc = 0;
+    if (!plan_from_cache(ctx, indices, nullptr, n_idx, nb, &pr, &rc)) {
+        if (rc) return rc;
+        void* mem = workspace(ctx, plan_bytes(n_idx, nb));
+        if (!mem) return ZG_HIP_EOOM;
+        pr.plan = carve_plan(mem, n_idx, nb);
+        if ((rc = build_plan(ctx, indices, pr.plan))) return rc;
+    }
+    const Plan& pl = pr.plan;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(nb, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((row_scatter_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, y_grad,
@@ -752,10 +917,16 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const floa
     if (n_edge == 0) return ZG_HIP_OK;
     ZG_REQUIRE(dst && h && deg && src_indices && tgt_indices, "scatter_gcn_deg_scaled: null pointer");
     if (int rc = check_gcn("scatter_gcn_deg_scaled", stride, n_edge, n_nodes)) return rc;
-    void* mem = workspace(ctx, plan_bytes(n_edge, n_nodes));
-    if (!mem) return ZG_HIP_EOOM;
-    Plan pl = carve_plan(mem, n_edge, n_nodes);
-    if (int rc = build_plan(ctx, tgt_indices, pl, src_indices)) return rc;
+    PlanRef pr;
+    int rc = 0;
+    if (!plan_from_cache(ctx, tgt_indices, src_indices, n_edge, n_nodes, &pr, &rc)) {
+        if (rc) return rc;
+        void* mem = workspace(ctx, plan_bytes(n_edge, n_nodes));
+        if (!mem) return ZG_HIP_EOOM;
+        pr.plan = carve_plan(mem, n_edge, n_nodes);
+        if ((rc = build_plan(ctx, tgt_indices, pr.plan, src_indices))) return rc;
+    }
+    const Plan& pl = pr.plan;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
@@ -777,12 +948,26 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     const size_t tb = align_up(n_edge * sizeof(float), 256);
     char* mem = (char*)workspace(ctx, 2 * pb + 2 * tb);
     if (!mem) return ZG_HIP_EOOM;
-    Plan by_src = carve_plan(mem, n_edge, n_nodes);
-    Plan by_tgt = carve_plan(mem + pb, n_edge, n_nodes);
     float* term_src = (float*)(mem + 2 * pb);
     float* term_tgt = (float*)(mem + 2 * pb + tb);
-    if (int rc = build_plan(ctx, src_indices, by_src, tgt_indices)) return rc;
-    if (int rc = build_plan(ctx, tgt_indices, by_tgt)) return rc;
+    PlanRef rs, rt;
+    int rc = 0;
+    if (!plan_from_cache(ctx, src_indices, tgt_indices, n_edge, n_nodes, &rs, &rc)) {
+        if (rc) return rc;
+        rs.plan = carve_plan(mem, n_edge, n_nodes);
+        if ((rc = build_plan(ctx, src_indices, rs.plan, tgt_indices))) return rc;
+        rs.keys = src_indices;
+        rs.payload = tgt_indices;
+    }
+    if (!plan_from_cache(ctx, tgt_indices, nullptr, n_edge, n_nodes, &rt, &rc)) {
+        if (rc) return rc;
+        rt.plan = carve_plan(mem + pb, n_edge, n_nodes);
+        if ((rc = build_plan(ctx, tgt_indices, rt.plan))) return rc;
+    }
+    const Plan &by_src = rs.plan, &by_tgt = rt.plan;
+    // the edge-term kernel reads both arrays entry by entry: from the cache's device copies when there are any
+    src_indices = rs.keys;
+    tgt_indices = rs.payload;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
@@ -859,6 +1044,13 @@ ZG_API int zg_hip_segment_sum_csr(zg_hip_ctx* ctx, const float* src, size_t src_
     hipLaunchKernelGGL(segment_sum_csr_kernel, dim3((unsigned)ceil_div_sz(n_segments, 4)), dim3(256), 0, ctx->stream, src,
                        src_len, row_offsets, n_segments, dst);
     ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_plan_cache_stats(zg_hip_ctx* ctx, uint64_t* hits, uint64_t* builds) {
+    ZG_CTX(ctx);
+    if (hits) *hits = ctx->plan_cache ? ctx->plan_cache->hits : 0;
+    if (builds) *builds = ctx->plan_cache ? ctx->plan_cache->builds : 0;
     return ZG_HIP_OK;
 }
 

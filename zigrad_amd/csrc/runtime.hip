@@ -455,6 +455,7 @@ ZG_API int zg_hip_init(int device_id, zg_hip_ctx** out) {
 ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
     ZG_CTX(ctx);
     (void)hipStreamSynchronize(ctx->stream);
+    plan_cache_destroy(ctx);  // its device memory is in raw_allocs; this frees the host side
     if (ctx->small_pool) {
         ctx->small_pool->destroy();
         delete ctx->small_pool;
@@ -549,6 +550,7 @@ struct zg_hip_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     std::vector<Block*> held;  // the cache memory the recorded ops name, kept out of the pools while the graph lives
+    std::vector<PlanUse> plan_uses;  // cached segment plans the recorded kernels read, and the index arrays they stand for
 };
 
 static void release_held(std::vector<Block*>& held) {
@@ -583,6 +585,7 @@ ZG_API int zg_hip_graph_open(zg_hip_ctx* ctx) {
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
     ZG_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capture_touched.clear();
+    ctx->plan_uses.clear();
     ctx->capturing = true;
     return ZG_HIP_OK;
 }
@@ -601,6 +604,7 @@ ZG_API int zg_hip_graph_save(zg_hip_ctx* ctx, zg_hip_graph** out) {
     if (e != hipSuccess || g == nullptr) {
         (void)hipGetLastError();
         ctx->capture_touched.clear();
+        ctx->plan_uses.clear();
         set_error("graph_save: hipStreamEndCapture failed: %s", hipGetErrorString(e));
         return ZG_HIP_ERUNTIME;
     }
@@ -610,6 +614,7 @@ ZG_API int zg_hip_graph_save(zg_hip_ctx* ctx, zg_hip_graph** out) {
         (void)hipGetLastError();
         (void)hipGraphDestroy(g);
         ctx->capture_touched.clear();
+        ctx->plan_uses.clear();
         set_error("graph_save: hipGraphInstantiate failed: %s", hipGetErrorString(e));
         return ZG_HIP_ERUNTIME;
     }
@@ -617,6 +622,8 @@ ZG_API int zg_hip_graph_save(zg_hip_ctx* ctx, zg_hip_graph** out) {
     gr->graph = g;
     gr->exec = exec;
     hold_touched_ranges(ctx, gr->held);
+    gr->plan_uses.swap(ctx->plan_uses);
+    plan_uses_retain(gr->plan_uses, +1);
     ctx->live_graphs++;
     *out = gr;
     return ZG_HIP_OK;
@@ -626,6 +633,8 @@ ZG_API int zg_hip_graph_run(zg_hip_ctx* ctx, zg_hip_graph* graph) {
     ZG_CTX(ctx);
     ZG_NOT_CAPTURING(ctx, "graph_run");
     ZG_REQUIRE(graph != nullptr && graph->exec != nullptr, "graph_run: null or unsaved graph");
+    if (!graph->plan_uses.empty())
+        if (int rc = plan_uses_validate(ctx, graph->plan_uses)) return rc;
     ZG_HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
     return ZG_HIP_OK;
 }
@@ -638,6 +647,7 @@ ZG_API int zg_hip_graph_free(zg_hip_ctx* ctx, zg_hip_graph* graph) {
     if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
     if (graph->graph) (void)hipGraphDestroy(graph->graph);
     release_held(graph->held);
+    plan_uses_retain(graph->plan_uses, -1);
     ctx->live_graphs--;
     delete graph;
     return ZG_HIP_OK;

@@ -435,6 +435,12 @@ class HipDevice:
         self._call("zg_hip_scatter_gcn_deg_scaled_bwd", grad_output.ptr, h.ptr, deg.ptr, src_indices.ptr,
                    tgt_indices.ptr, grad_h.ptr, grad_deg.ptr, stride, n_edge, deg.n)
 
+    def plan_cache_stats(self) -> dict:
+        """Calls served from a kept destination ordering / orderings computed and kept (pinned index arrays only)."""
+        h, b = ctypes.c_uint64(), ctypes.c_uint64()
+        self._call("zg_hip_plan_cache_stats", ctypes.byref(h), ctypes.byref(b))
+        return {"hits": h.value, "builds": b.value}
+
     # the same three ops on an edge plan built once for an edge list that does not change
     def edge_plan(self, src_indices: DevBuf, tgt_indices: DevBuf, n_nodes: int) -> "EdgePlan":
         h = ctypes.c_void_p()

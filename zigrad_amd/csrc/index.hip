@@ -346,6 +346,11 @@ struct CachedPlan {
     Plan plan;
     uint64_t* keys_dev = nullptr;
     uint64_t* payload_dev = nullptr;  // null: built without payload
+    // scatter_gcn_deg_scaled_bwd on an entry with a payload (keys = sources, payload = targets): the incidence plan
+    // of the degree gradient, built by the first such call outside a recording
+    void* inc_mem = nullptr;
+    Plan inc;
+    uint32_t* slot_of = nullptr;  // 2 n
     uint64_t last_use = 0;
     int graph_refs = 0;
 };
@@ -369,6 +374,7 @@ struct PlanRef {
     Plan plan;
     const uint64_t* keys;
     const uint64_t* payload;
+    CachedPlan* entry = nullptr;  // null: built in the workspace by the caller
 };
 
 // True when `out` names a cached plan for these arrays (found, or built and kept by this call).  False: the caller
@@ -402,6 +408,7 @@ static bool plan_from_cache(zg_hip_ctx* ctx, const uint64_t* keys, const uint64_
             if (hipStreamSynchronize(ctx->stream) != hipSuccess) return false;  // queued kernels may read the victim
             CachedPlan* v = pc.entries[victim];
             zg_hip_free(ctx, v->mem);
+            if (v->inc_mem) zg_hip_free(ctx, v->inc_mem);
             delete v;
             pc.entries.erase(pc.entries.begin() + victim);
         }
@@ -438,6 +445,44 @@ static bool plan_from_cache(zg_hip_ctx* ctx, const uint64_t* keys, const uint64_
     out->plan = hit->plan;
     out->keys = hit->keys_dev;
     out->payload = hit->payload_dev;
+    out->entry = hit;
+    return true;
+}
+
+__global__ void interleave_keys_kernel(const uint64_t* src_idx, const uint64_t* tgt_idx, size_t n_edge, uint64_t* keys,
+                                       uint32_t* slot_of);
+__global__ void invert_perm_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm, uint32_t* slot_of);
+
+// The incidence plan of an entry whose keys are edge sources and whose payload is edge targets; false when it does
+// not exist and cannot be built now (recording, or an error: *rc).
+static bool incidence_plan(zg_hip_ctx* ctx, CachedPlan* e, int* rc) {
+    *rc = ZG_HIP_OK;
+    if (e->inc_mem) return true;
+    if (ctx->capturing || !e->payload_dev) return false;
+    const size_t n2 = 2 * e->plan.n, nb = e->plan.nb;
+    if (n2 >= 0xffffffffull) return false;
+    const size_t pb = align_up(plan_bytes(n2, nb), 256), kb = align_up(n2 * sizeof(uint64_t), 256);
+    void* mem = nullptr;
+    if ((*rc = zg_hip_alloc(ctx, pb + kb + align_up(n2 * sizeof(uint32_t), 256), &mem))) return false;
+    Plan inc = carve_plan(mem, n2, nb);
+    uint64_t* keys = (uint64_t*)((char*)mem + pb);
+    uint32_t* slot_of = (uint32_t*)((char*)mem + pb + kb);
+    hipLaunchKernelGGL(interleave_keys_kernel, dim3((unsigned)ceil_div_sz(e->plan.n, 256)), dim3(256), 0, ctx->stream,
+                       e->keys_dev, e->payload_dev, e->plan.n, keys, slot_of);
+    *rc = build_plan(ctx, keys, inc);
+    if (!*rc) {
+        hipLaunchKernelGGL(invert_perm_kernel, dim3((unsigned)ceil_div_sz(n2, 256)), dim3(256), 0, ctx->stream, inc.row_ptr,
+                           nb, inc.perm, slot_of);
+        if (hipGetLastError() != hipSuccess) *rc = ZG_HIP_ERUNTIME;
+    }
+    if (*rc) {
+        (void)hipStreamSynchronize(ctx->stream);
+        zg_hip_free(ctx, mem);
+        return false;
+    }
+    e->inc_mem = mem;
+    e->inc = inc;
+    e->slot_of = slot_of;
     return true;
 }
 
@@ -445,6 +490,7 @@ void plan_cache_destroy(zg_hip_ctx* ctx) {
     if (!ctx->plan_cache) return;
     for (CachedPlan* e : ctx->plan_cache->entries) {
         zg_hip_free(ctx, e->mem);
+        if (e->inc_mem) zg_hip_free(ctx, e->inc_mem);
         delete e;
     }
     delete ctx->plan_cache;
@@ -496,7 +542,18 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
     }
     if (e - s > kLongBucket) return;  // scatter_add_apply_long_kernel's
     float acc = fresh ? 0.f : dst[b];
-    for (uint32_t k = s; k < e; k++) acc = __fadd_rn(acc, src[perm[k]]);
+    // eight entries' loads at a time (positions, then values: two round trips), the additions still in input order
+    for (uint32_t k = s; k < e; k += 8) {
+        uint32_t pv[8];
+        float sv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) pv[u] = (k + u < e) ? perm[k + u] : 0u;
+#pragma unroll
+        for (int u = 0; u < 8; u++) sv[u] = (k + u < e) ? src[pv[u]] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (k + u < e) acc = __fadd_rn(acc, sv[u]);
+    }
     dst[b] = acc;
 }
 
@@ -707,6 +764,67 @@ __global__ void gcn_bwd_graddeg_kernel(float* grad_deg, const float* term_src, c
             acc = __fadd_rn(acc, term_tgt[eb]);
             b++;
         }
+    }
+    grad_deg[v] = acc;
+}
+
+// The same sums through an incidence plan: the 2 * n_edge endpoint items (item 2e = edge e's source, item 2e + 1 = its
+// target) bucketed by node.  Ascending item order inside a bucket is the merged order above and the order of the
+// host loop (per edge: the source's term, then the target's).  slot_of[item] is the item's position in bucket order
+// (0xffffffff: its node is out of range), so the edge kernel writes each term where the node's thread will read
+// it, and that thread reads one contiguous run, eight loads at a time: no chain of dependent index loads.
+__global__ void interleave_keys_kernel(const uint64_t* src_idx, const uint64_t* tgt_idx, size_t n_edge, uint64_t* keys,
+                                       uint32_t* slot_of) {
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_edge) return;
+    keys[2 * e] = src_idx[e];
+    keys[2 * e + 1] = tgt_idx[e];
+    slot_of[2 * e] = 0xffffffffu;
+    slot_of[2 * e + 1] = 0xffffffffu;
+}
+
+__global__ void invert_perm_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm, uint32_t* slot_of) {
+    size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (k < row_ptr[nb]) slot_of[perm[k]] = (uint32_t)k;
+}
+
+__global__ void gcn_bwd_edge_terms_slots_kernel(const float* go, const float* h, const float* deg,
+                                                const uint64_t* src_idx, const uint64_t* tgt_idx, size_t n_edge,
+                                                size_t n_nodes, size_t stride, const uint32_t* slot_of, float* terms) {
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_edge) return;
+    const uint64_t s = src_idx[e], t = tgt_idx[e];
+    const uint32_t slot_s = slot_of[2 * e], slot_t = slot_of[2 * e + 1];
+    float gs = 0.f, gt = 0.f;
+    if (s < n_nodes && t < n_nodes) {
+        const float ds = deg[s], dt = deg[t];
+        for (size_t j = 0; j < stride; j++) {
+            const float g = go[t * stride + j], hv = h[s * stride + j];
+            gs = __fadd_rn(gs, __fmul_rn(__fmul_rn(g, dt), hv));
+            gt = __fadd_rn(gt, __fmul_rn(__fmul_rn(g, ds), hv));
+        }
+    }
+    if (slot_s != 0xffffffffu) terms[slot_s] = gs;
+    if (slot_t != 0xffffffffu) terms[slot_t] = gt;
+}
+
+__global__ void gcn_bwd_graddeg_slots_kernel(float* grad_deg, const float* terms, const uint32_t* row_ptr,
+                                             size_t n_nodes, bool fresh) {
+    size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= n_nodes) return;
+    const uint32_t s = row_ptr[v], e = row_ptr[v + 1];
+    if (s == e) {
+        if (fresh) grad_deg[v] = 0.f;
+        return;
+    }
+    float acc = fresh ? 0.f : grad_deg[v];
+    for (uint32_t k = s; k < e; k += 8) {
+        float tv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) tv[u] = (k + u < e) ? terms[k + u] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (k + u < e) acc = __fadd_rn(acc, tv[u]);
     }
     grad_deg[v] = acc;
 }
@@ -959,7 +1077,9 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
         rs.keys = src_indices;
         rs.payload = tgt_indices;
     }
-    if (!plan_from_cache(ctx, tgt_indices, nullptr, n_edge, n_nodes, &rt, &rc)) {
+    const bool by_incidence = rs.entry && incidence_plan(ctx, rs.entry, &rc);
+    if (rc) return rc;
+    if (!by_incidence && !plan_from_cache(ctx, tgt_indices, nullptr, n_edge, n_nodes, &rt, &rc)) {
         if (rc) return rc;
         rt.plan = carve_plan(mem + pb, n_edge, n_nodes);
         if ((rc = build_plan(ctx, tgt_indices, rt.plan))) return rc;
@@ -973,6 +1093,18 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
                                         grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride, false));
     ZG_LAUNCH_CHECK();
+    if (by_incidence) {
+        // 2 * n_edge terms in bucket order; the two separate term arrays' room holds them
+        float* terms = term_src;
+        hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0,
+                           ctx->stream, grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride,
+                           rs.entry->slot_of, terms);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0,
+                           ctx->stream, grad_deg, terms, rs.entry->inc.row_ptr, n_nodes, false);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
                        grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride, term_src, term_tgt);
     ZG_LAUNCH_CHECK();

@@ -132,6 +132,15 @@ int zg_hip_div(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_
 int zg_hip_dot(zg_hip_ctx *ctx, const float *x, const float *y, size_t n, float *z);
 int zg_hip_matvec(zg_hip_ctx *ctx, const float *A, const float *x, float *y, size_t m, size_t n, int trans_a,
                   float alpha, float beta);
+/* How a product of this shape would be launched by the staged kernels (no counterpart in the reference; for tests
+ * and for reading profiles).  out[0] kind: 0 one launch, 1 k cut over several workgroups per tile and the partial
+ * tiles added in a fixed order by a second kernel, 2 C cut into a block of whole 256 x 128 tiles plus strips that are
+ * launched as products of their own; out[1] tile: 0 = 256 x 128, 1 = 128 x 128, 2 = 64 x 64; out[2], out[3] number of k
+ * ranges and k-tiles (of 16) per range; out[4], out[5] tile rows and columns of the main block; out[6] the planner's
+ * estimate in microseconds.  Products served by the unstaged small-product kernels are not planned this way.
+ * ctx may be null (256 compute units are assumed); nothing is launched. */
+int zg_hip_gemm_plan(zg_hip_ctx *ctx, size_t m, size_t n, size_t k, size_t batches, int64_t *out);
+
 /* row-major C = alpha*op(A)*op(B) + beta*C; C is not read when beta == 0 */
 int zg_hip_matmul(zg_hip_ctx *ctx, const float *A, const float *B, float *C, size_t m, size_t n, size_t k,
                   int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta);

@@ -1,0 +1,40 @@
+"""The launch planner of the staged GEMM kernels (host arithmetic only: no GPU needed).  The products of the headline
+train step and of the op suite must keep their single launches; shapes whose tile count leaves the last round of
+workgroups mostly empty are cut into a block of whole rounds plus strips, or along k."""
+from __future__ import annotations
+
+import pytest
+
+from zigrad_amd.device import gemm_plan
+
+
+@pytest.mark.parametrize("shape,tile", [
+    ((4096, 4096, 4096), (256, 128)),   # the op suite's matmul and five of the wide MLP's eight products
+    ((4096, 1024, 4096), (128, 128)),   # last layer forward
+    ((1024, 4096, 4096), (128, 128)),   # last layer weight gradient
+    ((4096, 4096, 1024), (256, 128)),   # last layer input gradient
+    ((512, 512, 512, 32), (256, 128)),  # the op suite's batched product
+])
+def test_benchmark_products_stay_single_launches(shape, tile):
+    p = gemm_plan(*shape)
+    assert p["kind"] == "single" and p["tile"] == tile and p["splits"] == 1
+
+
+def test_off_grid_cubes_are_cut_into_whole_rounds_plus_strips():
+    p = gemm_plan(3072, 3072, 3072)   # 288 large tiles: 252 in the main block (one round of 256 CUs), a strip of 36
+    assert p["kind"] == "parts" and p["main_tiles"] == (12, 21)
+    p = gemm_plan(4100, 4100, 4100)   # 4096 x 4096 is two exact rounds; 4 rows and 4 columns are left over
+    assert p["kind"] == "parts" and p["main_tiles"] == (16, 32)
+
+
+def test_deep_products_on_few_tiles_are_cut_along_k():
+    for shape in ((64, 128, 784), (2708, 16, 1433)):   # first layer of the batch-64 MLP, first layer of the GCN
+        p = gemm_plan(*shape)
+        assert p["kind"] == "split_k" and p["tile"] == (64, 64) and p["splits"] >= 2
+        assert p["k_tiles_per_split"] % 2 == 0 and p["splits"] * p["k_tiles_per_split"] * 16 >= shape[2]
+
+
+def test_plans_are_a_function_of_the_shape_only():
+    assert gemm_plan(3072, 3072, 3072) == gemm_plan(3072, 3072, 3072)
+    with pytest.raises(Exception):
+        gemm_plan(0, 16, 16)

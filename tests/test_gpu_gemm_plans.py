@@ -1,0 +1,85 @@
+"""Products that the planner launches in parts (a block of whole rounds plus strips) or with k cut over several
+workgroups per large tile: against float64 products in full, bit-exact on integer-valued operands, with accumulation,
+and through the fused Linear entry points (bias, ReLU and gate must land on the right strip)."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from conftest import run_op
+from zigrad_amd.device import F32
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def _matmul(hip, A, B, C0, m, n, k, ta, tb, alpha, beta):
+    a, b, c = hip.from_numpy(A), hip.from_numpy(B), hip.from_numpy(C0)
+    hip.dispatch("matmul", A=a, B=b, C=c, m=m, n=n, k=k, trans_a=ta, trans_b=tb, lda=A.shape[1], ldb=B.shape[1], ldc=n,
+                 alpha=alpha, beta=beta)
+    out = hip.to_numpy(c).reshape(m, n)
+    for x in (a, b, c):
+        hip.mem_free(x)
+    return out
+
+
+@pytest.mark.parametrize("shape", [(3072, 3072, 3072), (4100, 4100, 1030), (3600, 2308, 1541)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_products_launched_in_parts_match_float64(hip, shape, ta, tb):
+    m, n, k = shape
+    assert hip.gemm_plan(m, n, k)["kind"] == "parts", hip.gemm_plan(m, n, k)
+    r = np.random.default_rng(m + 3 * n + 7 * k + 2 * ta + tb)
+    A = r.standard_normal((k, m) if ta else (m, k), dtype=np.float32)
+    B = r.standard_normal((n, k) if tb else (k, n), dtype=np.float32)
+    C0 = r.standard_normal((m, n), dtype=np.float32)
+    opA = (A.T if ta else A).astype(np.float64)
+    opB = (B.T if tb else B).astype(np.float64)
+    prod = opA @ opB
+    got = _matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, ta, tb, 1.0, 0.0)
+    assert np.linalg.norm(got - prod) <= TOL * np.linalg.norm(prod)
+    # every strip separately: an error confined to a few rows or columns must not hide in the whole-matrix norm
+    for sl in (np.s_[-4:, :], np.s_[:, -4:], np.s_[: m // 2, n // 2:], np.s_[m // 2:, : n // 2]):
+        assert np.linalg.norm(got[sl] - prod[sl]) <= TOL * np.linalg.norm(prod[sl])
+    got = _matmul(hip, A, B, C0, m, n, k, ta, tb, 0.5, 2.0)
+    want = 0.5 * prod + 2.0 * C0
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+
+
+def test_parts_and_split_products_are_exact_on_small_integers(hip):
+    for (m, n, k) in ((3072, 3072, 3072), (4100, 4100, 1030)):
+        r = np.random.default_rng(m)
+        A = r.integers(-3, 4, (m, k)).astype(np.float32)
+        B = r.integers(-3, 4, (n, k)).astype(np.float32)  # stored [n, k]: the forward layout of a Linear layer
+        got = _matmul(hip, A, B, np.zeros((m, n), np.float32), m, n, k, False, True, 1.0, 0.0)
+        want = (A.astype(np.int64) @ B.astype(np.int64).T).astype(np.float32)  # |entries| < 2^24: exact in fp32
+        assert np.array_equal(got, want)
+
+
+def test_fused_linear_entry_points_on_a_product_launched_in_parts(hip):
+    Bt, I, O = 2560, 1024, 3328  # batch, fan_in, fan_out
+    assert hip.gemm_plan(Bt, O, I)["kind"] == "parts", hip.gemm_plan(Bt, O, I)
+    r = np.random.default_rng(77)
+    x = r.standard_normal((Bt, I)).astype(np.float32)
+    w = (r.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
+    b = r.standard_normal(O).astype(np.float32)
+    got = run_op(hip, "linear_fwd", {"x": x, "w": w, "bias": b, "y": np.full((Bt, O), np.nan, np.float32), "batch": Bt,
+                                     "fan_in": I, "fan_out": O, "relu": True}, ["y"])["y"].reshape(Bt, O)
+    y = run_op(hip, "matmul", {"A": x, "B": w, "C": np.zeros((Bt, O), np.float32), "m": Bt, "n": O, "k": I,
+                               "trans_a": False, "trans_b": True, "lda": I, "ldb": I, "ldc": O, "alpha": 1.0, "beta": 0.0},
+               ["C"])["C"]
+    y = run_op(hip, "add", {"x": b, "y": y, "z": np.zeros_like(y)}, ["z"])["z"]
+    y = run_op(hip, "relu_fwd", {"x": y, "y": np.zeros_like(y)}, ["y"])["y"].reshape(Bt, O)
+    assert np.array_equal(got, y)
+    want = np.maximum(x.astype(np.float64) @ w.astype(np.float64).T + b, 0.0)
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+    # input gradient with the ReLU gate of the layer below: gx = (gy W) where act > 0
+    I2, O2 = 3328, 1024
+    assert hip.gemm_plan(Bt, I2, O2)["kind"] == "parts"
+    gy = r.standard_normal((Bt, O2)).astype(np.float32)
+    w2 = (r.standard_normal((O2, I2)) / np.sqrt(O2)).astype(np.float32)
+    act = np.maximum(r.standard_normal((Bt, I2)), 0.0).astype(np.float32)
+    got = run_op(hip, "linear_bwd_input", {"gy": gy, "w": w2, "act_in": act, "gx": np.full((Bt, I2), np.nan, np.float32),
+                                            "batch": Bt, "fan_in": I2, "fan_out": O2, "accumulate": False}, ["gx"])["gx"]
+    want = np.where(act > 0, gy.astype(np.float64) @ w2.astype(np.float64), 0.0)
+    assert np.linalg.norm(got.reshape(Bt, I2) - want) <= TOL * np.linalg.norm(want)
+    assert np.all(got.reshape(Bt, I2)[act <= 0] == 0.0)

@@ -23,6 +23,7 @@ constexpr size_t kPoolAlign = 256; // min split size of the block pools, bytes
 void set_error(const char* fmt, ...);
 
 struct BlockPool;  // runtime.hip
+struct GemmPlanCache;  // gemm.hip
 struct PlanCache;  // index.hip
 struct CachedPlan;
 
@@ -84,6 +85,9 @@ struct zg_hip_ctx {
     zg::PlanCache* plan_cache = nullptr;
     std::vector<zg::PlanUse> plan_uses;
 
+    // launch plans of the staged GEMM kernels, by shape (gemm.hip)
+    zg::GemmPlanCache* gemm_plans = nullptr;
+
     // regions handed out by pool_map/alloc, for ownership checks at free time
     std::map<void*, size_t> raw_allocs;
     std::map<void*, size_t> host_allocs;
@@ -98,6 +102,7 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 // which are never evicted while a graph names them.  validate: before a replay, every index array the recording
 // matched must still hold what it held then, or the replay would scatter by a stale plan.
 void plan_cache_destroy(zg_hip_ctx* ctx);
+void gemm_plans_destroy(zg_hip_ctx* ctx);
 void plan_uses_retain(const std::vector<PlanUse>& uses, int delta);
 int plan_uses_validate(zg_hip_ctx* ctx, const std::vector<PlanUse>& uses);
 

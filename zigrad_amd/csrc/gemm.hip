@@ -805,6 +805,215 @@ __global__ void scale_c_kernel(float* C, size_t M, size_t N, size_t ldc, float b
     }
 }
 
+// The same sum, four columns per thread: for a C fit for 16-byte accesses and no gate.
+__global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(const float* P, float* C, size_t M, size_t N, size_t ldc,
+                                                                 int splits, float alpha, float beta, size_t c_chunk,
+                                                                 const float* bias, int relu) {
+    const size_t z = blockIdx.z;
+    const float4* p = reinterpret_cast<const float4*>(P + z * (size_t)splits * M * N);
+    float* c = C + z * c_chunk;
+    const size_t n4 = M * N / 4, stride4 = M * N / 4;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += nt) {
+        float4 acc = p[i];
+        int s = 1;
+        for (; s + 3 < splits; s += 4) {  // four loads in flight, added in split order
+            const float4 v0 = p[(size_t)s * stride4 + i], v1 = p[(size_t)(s + 1) * stride4 + i],
+                         v2 = p[(size_t)(s + 2) * stride4 + i], v3 = p[(size_t)(s + 3) * stride4 + i];
+            acc.x += v0.x; acc.y += v0.y; acc.z += v0.z; acc.w += v0.w;
+            acc.x += v1.x; acc.y += v1.y; acc.z += v1.z; acc.w += v1.w;
+            acc.x += v2.x; acc.y += v2.y; acc.z += v2.z; acc.w += v2.w;
+            acc.x += v3.x; acc.y += v3.y; acc.z += v3.z; acc.w += v3.w;
+        }
+        for (; s < splits; s++) {
+            const float4 v = p[(size_t)s * stride4 + i];
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+        const size_t e = 4 * i, r = e / N, col = e % N;  // N is a multiple of 4: the four share a row
+        float4* cp = reinterpret_cast<float4*>(c + r * ldc + col);
+        float4 v = make_float4(alpha * acc.x, alpha * acc.y, alpha * acc.z, alpha * acc.w);
+        if (beta != 0.f) {
+            const float4 o = *cp;
+            v.x += beta * o.x; v.y += beta * o.y; v.z += beta * o.z; v.w += beta * o.w;
+        }
+        const bool hb = bias != nullptr;
+        v.x = gemm_extras(v.x, hb, hb ? bias[col] : 0.f, relu != 0);
+        v.y = gemm_extras(v.y, hb, hb ? bias[col + 1] : 0.f, relu != 0);
+        v.z = gemm_extras(v.z, hb, hb ? bias[col + 2] : 0.f, relu != 0);
+        v.w = gemm_extras(v.w, hb, hb ? bias[col + 3] : 0.f, relu != 0);
+        *cp = v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Launch planning for the staged kernels.  A CU works through its workgroups at a rate that depends on the tile
+// shape but hardly on how many of them share the CU, so a launch takes (rounds the grid needs) x (time of one tile)
+// plus a fixed cost (launch, first loads, the write of C by workgroups that all finish together).  When the tile
+// count leaves the last round mostly empty, two other shapes of launch are priced with the same model: k cut over
+// several workgroups per tile with a second kernel adding the partial tiles in a fixed order, and C cut into a block
+// of whole large tiles that fills whole rounds plus one or two strips that are products of their own.  Plans depend
+// on the shape only and are kept per context.
+// ------------------------------------------------------------------------------------------------
+struct GemmTileKind {
+    size_t bm, bn;
+    double eff;  // fraction of a CU's MFMA peak inside the loop
+};
+static const GemmTileKind kGemmTiles[3] = {{256, 128, 0.975}, {128, 128, 0.90}, {64, 64, 0.82}};
+constexpr double kCuFlopsPerUs = 2.4e9 * 256 / 1e6;  // one CU: 256 fp32 MFMA FLOP per clock at 2.4 GHz
+constexpr double kLaunchFixedUs = 8.0;
+constexpr double kReduceFixedUs = 4.0, kReduceBytesPerUs = 4.0e6;
+
+struct GemmPlan {
+    enum Kind { kPlain, kSplit, kParts } kind = kPlain;
+    int tile = 2;
+    size_t splits = 1, per = 0;  // kSplit: number of k ranges and k-tiles per range
+    size_t rm = 0, rn = 0;       // kParts: the main block is rm x rn tiles of 256 x 128
+    double us = 0;               // the model's estimate
+};
+
+struct GemmPlanKey {
+    size_t m, n, k, batches;
+    int layout;
+    bool operator<(const GemmPlanKey& o) const {
+        if (m != o.m) return m < o.m;
+        if (n != o.n) return n < o.n;
+        if (k != o.k) return k < o.k;
+        if (batches != o.batches) return batches < o.batches;
+        return layout < o.layout;
+    }
+};
+struct GemmPlanCache {
+    std::map<GemmPlanKey, GemmPlan> plans;
+};
+
+void gemm_plans_destroy(zg_hip_ctx* ctx) {
+    delete ctx->gemm_plans;
+    ctx->gemm_plans = nullptr;
+}
+
+static double gemm_tile_us(int tile, size_t kk) {
+    const GemmTileKind& t = kGemmTiles[tile];
+    return 2.0 * (double)(t.bm * t.bn) * (double)kk / (kCuFlopsPerUs * t.eff);
+}
+static size_t gemm_tiles_of(int tile, size_t m, size_t n, size_t batches) {
+    return ceil_div_sz(m, kGemmTiles[tile].bm) * ceil_div_sz(n, kGemmTiles[tile].bn) * batches;
+}
+
+// Other shapes of launch are priced only when the model puts the plan in hand more than 12 % above the time the
+// product would take with every CU busy at the large tile's rate.
+static bool gemm_plan_is_slow(double us, size_t m, size_t n, size_t k, size_t batches, size_t n_cu) {
+    const double ideal = 2.0 * (double)m * (double)n * (double)k * (double)batches / ((double)n_cu * kCuFlopsPerUs * 0.975);
+    return us > 1.12 * ideal + kLaunchFixedUs;
+}
+
+// One launch (plus the reduction when k is cut) for the whole product: the choice made before planning existed
+// (`legacy`: rounds x padded tile work over 0.92 / 0.89 / 0.79, and the 64 x 64 split for few tiles and a deep k), and,
+// when the model finds that slow, the best cut of k for any tile if the model prices it at least 8 % faster.
+static GemmPlan gemm_plan_single(size_t m, size_t n, size_t k, size_t batches, size_t n_cu) {
+    const size_t kt_total = ceil_div_sz(k, kBK);
+    static const double legacy_eff[3] = {0.92, 0.89, 0.79};
+    GemmPlan lp;
+    double best = 0;
+    for (int t = 0; t < 3; t++) {
+        const double c = (double)ceil_div_sz(gemm_tiles_of(t, m, n, batches), n_cu) *
+                         (double)(kGemmTiles[t].bm * kGemmTiles[t].bn) / legacy_eff[t];
+        if (t == 0 || c < best) {  // ties go to the larger tile
+            best = c;
+            lp.tile = t;
+        }
+    }
+    auto model = [&](int tile, size_t splits, size_t per) {
+        const size_t wgs = gemm_tiles_of(tile, m, n, batches) * splits;
+        double us = (double)ceil_div_sz(wgs, n_cu) * gemm_tile_us(tile, splits == 1 ? k : per * kBK) + kLaunchFixedUs;
+        if (splits > 1) us += kReduceFixedUs + (double)(splits + 2) * (double)(m * n * batches) * 4.0 / kReduceBytesPerUs;
+        return us;
+    };
+    if (lp.tile == 2) {
+        const size_t t64 = gemm_tiles_of(2, m, n, batches);
+        if (t64 < n_cu && kt_total >= 16) {
+            size_t splits = ceil_div_sz(2 * n_cu, t64);
+            if (splits > kt_total / 4) splits = kt_total / 4;
+            if (splits > 64) splits = 64;
+            size_t per = ceil_div_sz(kt_total, splits);
+            per += per & 1;
+            splits = ceil_div_sz(kt_total, per);
+            // Worth it only when the k-tiles saved on the busiest CU outweigh the second launch and the short loops:
+            // a 64x64 k-tile step takes about 0.27 us, the split's fixed costs about 6 us (768-cubed: 15.5 us whole,
+            // 20 us split four ways).
+            const double whole = (double)kt_total, busiest = (double)(ceil_div_sz(t64 * splits, n_cu) * per);
+            if (splits >= 2 && (whole - busiest) * 0.27 > 6.0) {
+                lp.kind = GemmPlan::kSplit;
+                lp.splits = splits;
+                lp.per = per;
+            }
+        }
+    }
+    lp.us = model(lp.tile, lp.splits, lp.per);
+    if (lp.kind == GemmPlan::kSplit) return lp;
+    if (!gemm_plan_is_slow(lp.us, m, n, k, batches, n_cu) || kt_total < 32) return lp;
+    GemmPlan bp = lp;
+    for (int t = 0; t < 3; t++) {
+        for (size_t want = 2; want <= 16; want++) {
+            size_t per = ceil_div_sz(kt_total, want);
+            per += per & 1;
+            if (per < 8) break;  // ranges shorter than 128 values of k are all prologue
+            const size_t splits = ceil_div_sz(kt_total, per);
+            if (splits < 2) continue;
+            const double us = model(t, splits, per);
+            if (us < bp.us) {
+                bp.kind = GemmPlan::kSplit;
+                bp.tile = t;
+                bp.splits = splits;
+                bp.per = per;
+                bp.us = us;
+            }
+        }
+    }
+    return (bp.us < 0.92 * lp.us) ? bp : lp;
+}
+
+static GemmPlan gemm_plan_compute(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth) {
+    GemmPlan best = gemm_plan_single(m, n, k, batches, n_cu);
+    // C in parts: only for one product (no batch), at the top level, when the single launch is slow by the model
+    const size_t tm_f = m / 256, tn_f = n / 128;
+    if (depth == 0 && batches == 1 && tm_f >= 1 && tn_f >= 1) {
+        if (gemm_plan_is_slow(best.us, m, n, k, 1, n_cu)) {
+            GemmPlan bp = best;
+            const size_t rm_lo = tm_f > 6 ? tm_f - 6 : 1, rn_lo = tn_f > 6 ? tn_f - 6 : 1;
+            for (size_t rm = tm_f; rm >= rm_lo; rm--) {
+                for (size_t rn = tn_f; rn >= rn_lo; rn--) {
+                    const size_t main_tiles = rm * rn;
+                    const double main_fill = (double)main_tiles / (double)(ceil_div_sz(main_tiles, n_cu) * n_cu);
+                    if (main_fill < 0.95) continue;
+                    double us = (double)ceil_div_sz(main_tiles, n_cu) * gemm_tile_us(0, k) + kLaunchFixedUs;
+                    const size_t m1 = rm * 256, n1 = rn * 128;
+                    if (n > n1) us += gemm_plan_single(m1, n - n1, k, 1, n_cu).us;
+                    if (m > m1) us += gemm_plan_single(m - m1, n, k, 1, n_cu).us;
+                    if (us < bp.us) {
+                        bp.kind = GemmPlan::kParts;
+                        bp.rm = rm;
+                        bp.rn = rn;
+                        bp.us = us;
+                    }
+                }
+            }
+            if (bp.us < 0.92 * best.us) best = bp;
+        }
+    }
+    return best;
+}
+
+static GemmPlan gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_t batches, bool a_kmajor, bool b_kmajor,
+                          int depth) {
+    if (!ctx->gemm_plans) ctx->gemm_plans = new GemmPlanCache();
+    const GemmPlanKey key{m, n, k, batches, (a_kmajor ? 1 : 0) | (b_kmajor ? 2 : 0) | (depth ? 4 : 0)};
+    auto it = ctx->gemm_plans->plans.find(key);
+    if (it != ctx->gemm_plans->plans.end()) return it->second;
+    const GemmPlan best = gemm_plan_compute((size_t)ctx->n_cu, m, n, k, batches, depth);
+    ctx->gemm_plans->plans[key] = best;
+    return best;
+}
+
 struct GemmExtras {
     const float* bias;
     const float* gate;
@@ -896,13 +1105,7 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         if (!small_ld) return 2;
         return (m % bm == 0 && n % bn == 0 && c_vec) ? 0 : 1;  // any k: the last tiles are masked on their way into LDS
     };
-    // Tile choice by estimated time.  A CU works through its workgroups at a rate that depends on the tile shape
-    // but hardly on how many of them share the CU (measured fraction of a CU's MFMA peak: 0.92 / 0.89 / 0.79),
-    // so the time is the number of rounds the grid needs times the padded work of one tile over that rate.
     const size_t n_cu = (size_t)ctx->n_cu;
-    auto cost = [&](size_t bm, size_t bn, double eff) {
-        return (double)ceil_div_sz(tiles(bm, bn), n_cu) * (double)(bm * bn) / eff;
-    };
     const size_t kt_total = ceil_div_sz(k, kBK);
     g.split_tiles = kt_total;
     g.split_stride = 0;
@@ -943,51 +1146,72 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
         return ZG_HIP_OK;
     }
 
-    const double c_large = cost(256, 128, 0.92), c_mid = cost(128, 128, 0.89), c_small = cost(64, 64, 0.79);
-    if (c_large <= c_mid && c_large <= c_small)
-        return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, mode(256, 128), batches);
-    if (c_mid <= c_small) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, mode(128, 128), batches);
-    // A deep product with too few C tiles to give every CU a workgroup: split k over several workgroups per tile
-    // (an even number of k-tiles each), let each write its partial tile to the workspace, and add the partials in
-    // split order in a second kernel.  The order is fixed, so the result does not depend on scheduling.
-    const size_t t64 = tiles(64, 64);
-    if (t64 < n_cu && kt_total >= 16) {
-        size_t splits = ceil_div_sz(2 * n_cu, t64);
-        if (splits > kt_total / 4) splits = kt_total / 4;
-        if (splits > 64) splits = 64;
-        size_t per = ceil_div_sz(kt_total, splits);
-        per += per & 1;
-        splits = ceil_div_sz(kt_total, per);
-        // Worth it only when the k-tiles saved on the busiest CU outweigh the second launch and the short loops:
-        // a 64x64 k-tile step takes about 0.27 us, the split's fixed costs about 6 us (768-cubed: 15.5 us whole,
-        // 20 us split four ways).
-        const double whole = (double)kt_total, busiest = (double)(ceil_div_sz(t64 * splits, n_cu) * per);
-        if (splits >= 2 && (whole - busiest) * 0.27 > 6.0) {
-            float* part = (float*)workspace(ctx, batches * splits * m * n * sizeof(float));
-            if (!part) return ZG_HIP_EOOM;
-            GemmArgs gs = g;
-            gs.C = part;
-            gs.ldc = n;
-            gs.c_chunk = splits * m * n;
-            gs.split_tiles = per;
-            gs.split_stride = m * n;
-            gs.alpha = 1.f;
-            gs.beta = 0.f;
-            gs.bias = nullptr;  // the extras belong to the sum of the partial products: the reduce kernel applies them
-            gs.gate = nullptr;
-            gs.relu = 0;
-            gs.c_vec = n % 4 == 0 && (m * n) % 4 == 0;  // the partial-product buffer is 256-byte aligned and dense
-            const int split_mode = !small_ld ? 2 : ((m % 64 == 0 && n % 64 == 0 && gs.c_vec) ? 0 : 1);
-            int rc = launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
-            if (rc) return rc;
-            size_t blocks = ceil_div_sz(m * n, 256);
-            if (blocks > 2048) blocks = 2048;
+    // ---- plan: which tile, whether k is cut, whether C is cut into a block of whole rounds plus strips ----
+    const GemmPlan plan = gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth);
+    if (plan.kind == GemmPlan::kParts) {
+        // C = [ main | right ] over [ bottom ]: main is rm x rn whole large tiles (a whole number of rounds, or nearly),
+        // the strips are products of their own and go through this function again (they may cut k, not C).
+        const size_t m1 = plan.rm * 256, n1 = plan.rn * 128;
+        struct Part {
+            size_t r0, c0, mm, nn;
+        } parts[3] = {{0, 0, m1, n1}, {0, n1, m1, n - n1}, {m1, 0, m - m1, n}};
+        for (const Part& pt : parts) {
+            if (pt.mm == 0 || pt.nn == 0) continue;
+            const float* As = trans_a ? A + pt.r0 : A + pt.r0 * lda;
+            const float* Bs = trans_b ? B + pt.c0 * ldb : B + pt.c0;
+            float* Cs = C + pt.r0 * ldc + pt.c0;
+            GemmExtras ex;
+            if (extras) {
+                ex.bias = extras->bias ? extras->bias + pt.c0 : nullptr;
+                ex.gate = extras->gate ? extras->gate + (pt.r0 * ldc + pt.c0) : nullptr;
+                ex.relu = extras->relu;
+            }
+            if (int rc = gemm_dispatch(ctx, name, As, Bs, Cs, pt.mm, pt.nn, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta,
+                                       1, 1, 1, 0, 0, 0, depth + 1, extras ? &ex : nullptr))
+                return rc;
+        }
+        return ZG_HIP_OK;
+    }
+    const int tile = plan.tile;  // 0: 256 x 128, 1: 128 x 128, 2: 64 x 64
+    const size_t bm = kGemmTiles[tile].bm, bn = kGemmTiles[tile].bn;
+    if (plan.kind == GemmPlan::kSplit) {
+        // k is cut over several workgroups per tile (an even number of k-tiles each); each writes its partial tile to the
+        // workspace and a second kernel adds the partials in split order: the order is fixed, so the result does not
+        // depend on scheduling.
+        const size_t splits = plan.splits, per = plan.per;
+        float* part = (float*)workspace(ctx, batches * splits * m * n * sizeof(float));
+        if (!part) return ZG_HIP_EOOM;
+        GemmArgs gs = g;
+        gs.C = part;
+        gs.ldc = n;
+        gs.c_chunk = splits * m * n;
+        gs.split_tiles = per;
+        gs.split_stride = m * n;
+        gs.alpha = 1.f;
+        gs.beta = 0.f;
+        gs.bias = nullptr;  // the extras belong to the sum of the partial products: the reduce kernel applies them
+        gs.gate = nullptr;
+        gs.relu = 0;
+        gs.c_vec = n % 4 == 0 && (m * n) % 4 == 0;  // the partial-product buffer is 256-byte aligned and dense
+        const int split_mode = !small_ld ? 2 : ((m % bm == 0 && n % bn == 0 && gs.c_vec) ? 0 : 1);
+        int rc = tile == 0   ? launch_gemm<256, 128>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches)
+                 : tile == 1 ? launch_gemm<128, 128>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches)
+                             : launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
+        if (rc) return rc;
+        const bool vec4 = gs.c_vec && c_vec && !g.gate;
+        size_t blocks = ceil_div_sz(vec4 ? m * n / 4 : m * n, 256);
+        if (blocks > 4096) blocks = 4096;
+        if (vec4)
+            hipLaunchKernelGGL(splitk_reduce_vec4_kernel, dim3((unsigned)blocks, 1, (unsigned)batches), dim3(256), 0,
+                               ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk, g.bias, g.relu);
+        else
             hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks, 1, (unsigned)batches), dim3(256), 0,
                                ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk, g.bias, g.gate, g.relu);
-            ZG_LAUNCH_CHECK();
-            return ZG_HIP_OK;
-        }
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
     }
+    if (tile == 0) return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, mode(256, 128), batches);
+    if (tile == 1) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, mode(128, 128), batches);
     return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, mode(64, 64), batches);
 }
 
@@ -1053,6 +1277,20 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* A, float* B
 }  // namespace zg
 
 using namespace zg;
+
+ZG_API int zg_hip_gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_t batches, int64_t* out) {
+    ZG_REQUIRE(out != nullptr, "gemm_plan: null output");
+    ZG_REQUIRE(m > 0 && n > 0 && k > 0 && batches > 0, "gemm_plan: empty product");
+    const GemmPlan p = gemm_plan_compute(ctx ? (size_t)ctx->n_cu : 256, m, n, k, batches, 0);
+    out[0] = (int64_t)p.kind;
+    out[1] = p.tile;
+    out[2] = (int64_t)p.splits;
+    out[3] = (int64_t)p.per;
+    out[4] = (int64_t)p.rm;
+    out[5] = (int64_t)p.rn;
+    out[6] = (int64_t)(p.us + 0.5);
+    return ZG_HIP_OK;
+}
 
 ZG_API int zg_hip_matmul(zg_hip_ctx* ctx, const float* A, const float* B, float* C, size_t m, size_t n, size_t k,
                          int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {

@@ -455,6 +455,7 @@ ZG_API int zg_hip_init(int device_id, zg_hip_ctx** out) {
 ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
     ZG_CTX(ctx);
     (void)hipStreamSynchronize(ctx->stream);
+    gemm_plans_destroy(ctx);
     plan_cache_destroy(ctx);  // its device memory is in raw_allocs; this frees the host side
     if (ctx->small_pool) {
         ctx->small_pool->destroy();

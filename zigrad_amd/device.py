@@ -435,6 +435,10 @@ class HipDevice:
         self._call("zg_hip_scatter_gcn_deg_scaled_bwd", grad_output.ptr, h.ptr, deg.ptr, src_indices.ptr,
                    tgt_indices.ptr, grad_h.ptr, grad_deg.ptr, stride, n_edge, deg.n)
 
+    def gemm_plan(self, m: int, n: int, k: int, batches: int = 1) -> dict:
+        """How the staged GEMM kernels would launch this product (see zg_hip_gemm_plan)."""
+        return gemm_plan(m, n, k, batches, self)
+
     def plan_cache_stats(self) -> dict:
         """Calls served from a kept destination ordering / orderings computed and kept (pinned index arrays only)."""
         h, b = ctypes.c_uint64(), ctypes.c_uint64()
@@ -537,6 +541,17 @@ class HipDevice:
         out = ctypes.c_float()
         self._lib.call("zg_hip_adam_lr_t", lr, beta1, beta2, int(t), ctypes.byref(out))
         return out.value
+
+
+def gemm_plan(m: int, n: int, k: int, batches: int = 1, dev: "HipDevice | None" = None) -> dict:
+    """zg_hip_gemm_plan as a dict; without a device the planner assumes 256 compute units (no GPU needed)."""
+    from ._lib import lib
+
+    out = (ctypes.c_int64 * 7)()
+    lib().call("zg_hip_gemm_plan", dev._ctx if dev is not None else None, m, n, k, batches, out)
+    kinds, tiles = ("single", "split_k", "parts"), ((256, 128), (128, 128), (64, 64))
+    return {"kind": kinds[out[0]], "tile": tiles[out[1]], "splits": out[2], "k_tiles_per_split": out[3],
+            "main_tiles": (out[4], out[5]), "estimate_us": out[6]}
 
 
 class Graph:

@@ -175,7 +175,8 @@ def op_suite(dev, quick=False, cpu=False):
 
     # GEMM 4096^3: NN, TN (A transposed), NT (B transposed)
     n = 4096
-    A, B, C = dev_normal(n * n), dev_normal(n * n), dev_normal(n * n)
+    big = n * n if cpu else 4100 * 4100  # the largest operand any product below takes
+    A, B, C = dev_normal(big), dev_normal(big), dev_normal(big)
     for tag, ta, tb in (("matmul_4096_nn", False, False), ("matmul_4096_tn", True, False), ("matmul_4096_nt", False, True)):
         t = timed(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=n, n=n, k=n, trans_a=ta, trans_b=tb, lda=n, ldb=n,
                                                ldc=n, alpha=1.0, beta=0.0), iters)
@@ -185,6 +186,20 @@ def op_suite(dev, quick=False, cpu=False):
     t = timed(dev, lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, s, s], B_shape=[nb, s, s], C_shape=[nb, s, s],
                                            trans_a=False, trans_b=False, lda=s, ldb=s, ldc=s, alpha=1.0, beta=0.0), iters * 5)
     out["bmm_32x512"] = tfl(2 * nb * s ** 3, t)
+    if not cpu:
+        # products off the large tile's grid (not part of the named op suite: cubes whose tile count does not fill whole
+        # rounds of compute units, and the graph convolution's skinny first layer, which is bound by reading X)
+        for m_, n_, k_ in ((1536, 1536, 1536), (3072, 3072, 3072), (4100, 4100, 4100)):
+            t = timed(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=m_, n=n_, k=k_, trans_a=False, trans_b=True,
+                                                   lda=k_, ldb=k_, ldc=n_, alpha=1.0, beta=0.0), iters * (4 if m_ < 2048 else 1))
+            out[f"matmul_{m_}_nt"] = {**tfl(2 * m_ * n_ * k_, t), "plan": dev.gemm_plan(m_, n_, k_)["kind"]}
+        m_, n_, k_ = 2708, 16, 1433
+        t = timed(dev, lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=m_, n=n_, k=k_, trans_a=False, trans_b=True, lda=k_,
+                                               ldb=k_, ldc=n_, alpha=1.0, beta=0.0), iters * 10)
+        nbytes = 4 * (m_ * k_ + n_ * k_ + m_ * n_)
+        out["matmul_2708x16x1433_nt"] = {**tfl(2 * m_ * n_ * k_, t), "gbs": nbytes / (t["ms"] * 1e-3) / 1e9,
+                                         "frac_hbm": nbytes / (t["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                         "bound": "hbm (0.25 FLOP per byte of X at N = 16)"}
     for b in (A, B, C):
         dev.mem_free(b)
 

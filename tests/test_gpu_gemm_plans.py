@@ -83,3 +83,87 @@ def test_fused_linear_entry_points_on_a_product_launched_in_parts(hip):
     want = np.where(act > 0, gy.astype(np.float64) @ w2.astype(np.float64), 0.0)
     assert np.linalg.norm(got.reshape(Bt, I2) - want) <= TOL * np.linalg.norm(want)
     assert np.all(got.reshape(Bt, I2)[act <= 0] == 0.0)
+
+
+@pytest.mark.parametrize("shape", [(2708, 16, 1433), (2708, 7, 1433), (1000, 1, 300), (513, 32, 257), (4096, 17, 1024),
+                                   (600, 8, 2050), (515, 9, 4099), (2048, 24, 256)])
+def test_tall_narrow_products_of_k_contiguous_operands(hip, shape):
+    """[m, k] x [n, k]^T with n <= 32 (the graph convolution's first layer; k is cut over several workgroups per tile):
+    against float64, with accumulation, with padded leading dimensions, and through linear_fwd (bias and ReLU in the
+    same launch) against the three separate ops."""
+    m, n, k = shape
+    r = np.random.default_rng(m + n + k)
+    A = r.standard_normal((m, k), dtype=np.float32)
+    B = r.standard_normal((n, k), dtype=np.float32)
+    C0 = r.standard_normal((m, n), dtype=np.float32)
+    prod = A.astype(np.float64) @ B.astype(np.float64).T
+    got = _matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, False, True, 1.0, 0.0)
+    assert np.linalg.norm(got - prod) <= TOL * np.linalg.norm(prod)
+    assert np.abs(got - prod).max() <= 8 * TOL * np.sqrt(k)
+    got = _matmul(hip, A, B, C0, m, n, k, False, True, -0.5, 1.0)
+    want = -0.5 * prod + C0
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+    # a row stride larger than k (a view into a wider matrix) and an output wider than n
+    Aw = r.standard_normal((m, k + 3), dtype=np.float32)
+    a, b, c = hip.from_numpy(Aw), hip.from_numpy(B), hip.from_numpy(np.full((m, n + 5), 7.0, np.float32))
+    hip.dispatch("matmul", A=a, B=b, C=c, m=m, n=n, k=k, trans_a=False, trans_b=True, lda=k + 3, ldb=k, ldc=n + 5,
+                 alpha=1.0, beta=0.0)
+    out = hip.to_numpy(c).reshape(m, n + 5)
+    want = Aw[:, :k].astype(np.float64) @ B.astype(np.float64).T
+    assert np.linalg.norm(out[:, :n] - want) <= TOL * np.linalg.norm(want)
+    assert np.all(out[:, n:] == 7.0)
+    for x in (a, b, c):
+        hip.mem_free(x)
+    bias = r.standard_normal(n).astype(np.float32)
+    fused = run_op(hip, "linear_fwd", {"x": A, "w": B, "bias": bias, "y": np.full((m, n), np.nan, np.float32), "batch": m,
+                                       "fan_in": k, "fan_out": n, "relu": True}, ["y"])["y"].reshape(m, n)
+    y = _matmul(hip, A, B, np.zeros((m, n), np.float32), m, n, k, False, True, 1.0, 0.0)
+    y = run_op(hip, "add", {"x": bias, "y": y, "z": np.zeros_like(y)}, ["z"])["z"]
+    y = run_op(hip, "relu_fwd", {"x": y, "y": np.zeros_like(y)}, ["y"])["y"].reshape(m, n)
+    assert np.array_equal(fused, y)
+
+
+def test_tall_narrow_product_is_exact_on_small_integers(hip):
+    m, n, k = 2708, 16, 1433
+    r = np.random.default_rng(4)
+    A = r.integers(0, 2, (m, k)).astype(np.float32)       # binary features, as in the benchmark's graph
+    B = r.integers(-4, 5, (n, k)).astype(np.float32)
+    got = _matmul(hip, A, B, np.zeros((m, n), np.float32), m, n, k, False, True, 1.0, 0.0)
+    assert np.array_equal(got, (A.astype(np.int64) @ B.astype(np.int64).T).astype(np.float32))
+
+
+@pytest.mark.parametrize("m,n", [(5000, 300), (70000, 33), (64, 64), (63, 1), (1, 700), (4096, 4096), (130, 257)])
+def test_transposed_matvec_over_many_rows(oracle, hip, m, n):
+    """y = alpha A^T x + beta y with the rows split over workgroups (src/device/host_device.zig:232-240)."""
+    r = np.random.default_rng(m * 3 + n)
+    A = r.standard_normal((m, n), dtype=np.float32)
+    x = r.standard_normal(m, dtype=np.float32)
+    y0 = r.standard_normal(n, dtype=np.float32)
+    want = 0.75 * (A.astype(np.float64).T @ x.astype(np.float64)) + 0.5 * y0
+    p = {"A": A, "x": x, "y": y0.copy(), "m": m, "n": n, "trans_a": True, "alpha": 0.75, "beta": 0.5}
+    got = run_op(hip, "matvec", dict(p), ["y"])["y"]
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+    if m * n <= 1 << 22:
+        ref = run_op(oracle, "matvec", dict(p), ["y"])["y"]
+        assert np.linalg.norm(got - ref) <= TOL * np.linalg.norm(ref)
+    got = run_op(hip, "matvec", {**p, "y": np.full(n, np.nan, np.float32), "beta": 0.0}, ["y"])["y"]  # y is not read
+    want0 = 0.75 * (A.astype(np.float64).T @ x.astype(np.float64))
+    assert np.linalg.norm(got - want0) <= TOL * np.linalg.norm(want0)
+
+
+def test_more_batches_than_one_grid_dimension_holds(hip):
+    """bmm_acc over 70000 batches (a grid's z dimension ends at 65535): per-batch operands, and one B for all."""
+    nb, s = 70000, 4
+    r = np.random.default_rng(12)
+    A = r.integers(-3, 4, (nb, s, s)).astype(np.float32)
+    B = r.integers(-3, 4, (nb, s, s)).astype(np.float32)
+    for shared_b in (False, True):
+        Bop = B[:1] if shared_b else B
+        a, b, c = hip.from_numpy(A), hip.from_numpy(Bop), hip.mem_alloc(F32, nb * s * s)
+        hip.dispatch("bmm_acc", A=a, B=b, C=c, A_shape=[nb, s, s], B_shape=[Bop.shape[0], s, s], C_shape=[nb, s, s],
+                     trans_a=False, trans_b=False, lda=s, ldb=s, ldc=s, alpha=1.0, beta=0.0)
+        got = hip.to_numpy(c).reshape(nb, s, s)
+        want = np.matmul(A, Bop if not shared_b else np.broadcast_to(Bop, A.shape))
+        assert np.array_equal(got, want)  # small integers: exact
+        for x in (a, b, c):
+            hip.mem_free(x)

@@ -39,7 +39,7 @@ def sources() -> list[Path]:
 
 
 def _headers_mtime() -> float:
-    hdrs = list(CSRC.glob("*.h")) + list(CSRC.glob("*.cuh")) + [PKG_DIR.parent / "include" / "zg_hip.h"]
+    hdrs = list(CSRC.glob("*.h")) + [PKG_DIR.parent / "include" / "zg_hip.h"]
     return max(h.stat().st_mtime for h in hdrs)
 
 

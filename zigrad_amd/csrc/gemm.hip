@@ -23,7 +23,7 @@
 // Workgroup ids are remapped so that the workgroups resident on one XCD (ids congruent modulo 8) cover a
 // compact patch of C and share their A rows / B columns in that XCD's L2.
 #include "common.h"
-#include "reduce.cuh"
+#include "reduce_device.h"
 
 #include <type_traits>
 
@@ -1077,8 +1077,28 @@ static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, cons
     ZG_REQUIRE(lda >= (trans_a ? m : k) && lda >= 1, "%s: lda %zu too small", name, lda);
     ZG_REQUIRE(ldb >= (trans_b ? k : n) && ldb >= 1, "%s: ldb %zu too small", name, ldb);
     ZG_REQUIRE(ldc >= n, "%s: ldc %zu < n %zu", name, ldc, n);
-    ZG_REQUIRE(batches <= 65535, "%s: more than 65535 batches", name);
     ZG_REQUIRE(nba >= 1 && nbb >= 1, "%s: zero operand batches", name);
+    if (batches > 65535) {
+        // the batch index is the grid's z dimension (at most 65535): longer batches go in runs.  The operand batch
+        // index of run-relative batch z is (z0 + z) % nb; a run that starts at a multiple of nb, or an operand with a
+        // single batch, keeps the kernel's own z % nb valid, which a run length that nba and nbb both divide ensures.
+        ZG_REQUIRE((nba == 1 || nba == batches) && (nbb == 1 || nbb == batches),
+                   "%s: more than 65535 batches with operands that repeat every %zu / %zu batches", name, nba, nbb);
+        for (size_t z0 = 0; z0 < batches; z0 += 65535) {
+            const size_t run = batches - z0 < 65535 ? batches - z0 : 65535;
+            GemmExtras ex;
+            if (extras) {
+                ex = *extras;
+                if (ex.gate) ex.gate += z0 * c_chunk;
+            }
+            if (int rc = gemm_dispatch(ctx, name, nba == 1 ? A : A + z0 * a_chunk, nbb == 1 ? B : B + z0 * b_chunk,
+                                       C + z0 * c_chunk, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, run,
+                                       nba == 1 ? 1 : run, nbb == 1 ? 1 : run, a_chunk, b_chunk, c_chunk, depth,
+                                       extras ? &ex : nullptr))
+                return rc;
+        }
+        return ZG_HIP_OK;
+    }
     if (k == 0 || alpha == 0.f) {
         if (beta == 1.f) return ZG_HIP_OK;
         size_t blocks = ceil_div_sz(m * n, 256);
@@ -1233,13 +1253,44 @@ __global__ __launch_bounds__(256) void gemv_n_kernel(const float* A, const float
     if (lane == 0) y[row] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[row];
 }
 
-// y = alpha * A^T x + beta * y, A is [m, n] row-major, y has n entries: thread per column, rows in order
-__global__ __launch_bounds__(256) void gemv_t_kernel(const float* A, const float* x, float* y, size_t m, size_t n,
-                                                      float alpha, float beta) {
+// y = alpha * A^T x + beta * y, A is [m, n] row-major, y has n entries.  A workgroup owns 64 columns and one chunk of
+// rows: its four waves take every fourth row of the chunk (each wave reads 256 contiguous bytes of a row), their
+// sums are added in wave order through LDS.  One chunk: the result is written here; several: the chunk sums go to
+// `part` [chunks][n] and gemv_t_final_kernel adds them in chunk order.
+__global__ __launch_bounds__(256) void gemv_t_kernel(const float* A, const float* x, float* y, float* part, size_t m,
+                                                      size_t n, size_t rows_per_chunk, float alpha, float beta) {
+    __shared__ float s_part[4][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const size_t col = (size_t)blockIdx.x * 64 + tx;
+    const size_t r0 = (size_t)blockIdx.y * rows_per_chunk;
+    const size_t r1 = r0 + rows_per_chunk < m ? r0 + rows_per_chunk : m;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (col < n) {
+        size_t i = r0 + ty;
+        for (; i + 12 < r1; i += 16) {  // four loads in flight per thread
+            const float a0 = A[i * n + col], a1 = A[(i + 4) * n + col], a2 = A[(i + 8) * n + col], a3 = A[(i + 12) * n + col];
+            s0 += a0 * x[i];
+            s1 += a1 * x[i + 4];
+            s2 += a2 * x[i + 8];
+            s3 += a3 * x[i + 12];
+        }
+        for (; i < r1; i += 4) s0 += A[i * n + col] * x[i];
+    }
+    s_part[ty][tx] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (ty == 0 && col < n) {
+        const float s = ((s_part[0][tx] + s_part[1][tx]) + s_part[2][tx]) + s_part[3][tx];
+        if (part) part[(size_t)blockIdx.y * n + col] = s;
+        else y[col] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[col];
+    }
+}
+
+__global__ __launch_bounds__(256) void gemv_t_final_kernel(const float* part, float* y, size_t n, size_t chunks, float alpha,
+                                                            float beta) {
     const size_t col = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (col >= n) return;
-    float s = 0.f;
-    for (size_t i = 0; i < m; i++) s += A[i * n + col] * x[i];
+    float s = part[col];
+    for (size_t c = 1; c < chunks; c++) s += part[c * n + col];
     y[col] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[col];
 }
 
@@ -1404,9 +1455,29 @@ ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float*
     if (!trans_a)
         hipLaunchKernelGGL(gemv_n_kernel, dim3((unsigned)ceil_div_sz(m, 4)), dim3(256), 0, ctx->stream, A, x, y, m, n,
                            alpha, beta);
-    else
-        hipLaunchKernelGGL(gemv_t_kernel, dim3((unsigned)ceil_div_sz(n, 256)), dim3(256), 0, ctx->stream, A, x, y, m, n,
-                           alpha, beta);
+    else {
+        // enough row chunks to put about two workgroups on every CU, at least 64 rows each, at most 64 chunks
+        const size_t col_blocks = ceil_div_sz(n, 64);
+        size_t chunks = ceil_div_sz(2 * (size_t)ctx->n_cu, col_blocks);
+        if (chunks > m / 64) chunks = m / 64;
+        if (chunks > 64) chunks = 64;
+        if (chunks < 1) chunks = 1;
+        const size_t rows_per_chunk = ceil_div_sz(m, chunks);
+        chunks = ceil_div_sz(m, rows_per_chunk);
+        float* part = nullptr;
+        if (chunks > 1) {
+            part = (float*)workspace(ctx, chunks * n * sizeof(float));
+            if (!part) return ZG_HIP_EOOM;
+        }
+        ZG_REQUIRE(col_blocks <= 0x7fffffffull, "matvec: too many columns");
+        hipLaunchKernelGGL(gemv_t_kernel, dim3((unsigned)col_blocks, (unsigned)chunks), dim3(256), 0, ctx->stream, A, x, y,
+                           part, m, n, rows_per_chunk, alpha, beta);
+        ZG_LAUNCH_CHECK();
+        if (chunks > 1) {
+            hipLaunchKernelGGL(gemv_t_final_kernel, dim3((unsigned)ceil_div_sz(n, 256)), dim3(256), 0, ctx->stream, part, y,
+                               n, chunks, alpha, beta);
+        }
+    }
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

@@ -4,7 +4,7 @@
 // needs a single pass (online max / sum-of-exponentials); the one-hot forward needs two (it must write
 // the probabilities the reference keeps for backward).  Row losses are written to a buffer and summed
 // by a fixed-order reduction, so the loss value does not depend on scheduling.
-#include "reduce.cuh"
+#include "reduce_device.h"
 
 namespace zg {
 

@@ -4,7 +4,7 @@
 //
 // HBM traffic per element: SGD reads p,g and writes p (12 B; +4 B when the clip changes g);
 // Adam reads p,g,m,v and writes p,m,v (28 B; +4 B when the clip changes g).
-#include "reduce.cuh"
+#include "reduce_device.h"
 
 namespace zg {
 

@@ -5,7 +5,7 @@
 // launches (per-block partials, then one block that combines the partials in a fixed order); there is
 // no cross-workgroup communication inside a kernel and no floating-point atomics, so results do not
 // depend on scheduling.
-#include "reduce.cuh"
+#include "reduce_device.h"
 
 namespace zg {
 

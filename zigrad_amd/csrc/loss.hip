@@ -361,6 +361,83 @@ __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(cons
     }
 }
 
+// Rows of 260 to 1024 columns in batches of a thousand rows or more (the wide classifier's [4096, 1024] logits): a wave
+// per row holds the row in registers (at most 4 float4 per lane), so the logits are read once and the row's
+// reductions stay inside the wave: three passes of the matrix instead of four, no LDS, no barrier.
+constexpr int kWaveRowVec = 4;
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* logits, const float* target, float* probs,
+                                                                    float* row_loss, size_t rows, size_t cols) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t row = (size_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (row >= rows) return;  // whole waves leave together: no barrier follows
+    const size_t c4 = cols >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
+    const float4* t4 = reinterpret_cast<const float4*>(MODE ? target + row * cols : logits);
+    float4* p4 = reinterpret_cast<float4*>(probs + row * cols);
+    const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    float4 v[kWaveRowVec], t[kWaveRowVec];
+#pragma unroll
+    for (int u = 0; u < kWaveRowVec; u++) {
+        const size_t j = lane + (size_t)u * kWave;
+        v[u] = (j < c4) ? nt_load(x4 + j) : ninf;
+    }
+    if (MODE) {
+#pragma unroll
+        for (int u = 0; u < kWaveRowVec; u++) {
+            const size_t j = lane + (size_t)u * kWave;
+            t[u] = (j < c4) ? nt_load(t4 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    OnlineAccT acc = OnlineAcc::init();
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < kWaveRowVec; u++) mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
+    if (mx != -INFINITY) {
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < kWaveRowVec; u++)
+            sum += fexp(v[u].x - mx) + fexp(v[u].y - mx) + fexp(v[u].z - mx) + fexp(v[u].w - mx);
+        acc.m = mx;
+        acc.s = sum;
+    }
+    acc = group_reduce<OnlineAcc, kWave>(acc);
+    const float l = __fadd_rn(acc.m, logf(acc.s));
+    float part = 0.f;
+#pragma unroll
+    for (int u = 0; u < kWaveRowVec; u++) {
+        const size_t j = lane + (size_t)u * kWave;
+        if (j < c4) {
+            float4 p;
+            p.x = fexp(__fsub_rn(v[u].x, l));
+            p.y = fexp(__fsub_rn(v[u].y, l));
+            p.z = fexp(__fsub_rn(v[u].z, l));
+            p.w = fexp(__fsub_rn(v[u].w, l));
+            nt_store(p, p4 + j);
+            if (MODE) {
+                const float pv[4] = {p.x, p.y, p.z, p.w}, tv[4] = {t[u].x, t[u].y, t[u].z, t[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (tv[e] != 0.f) {
+                        const float safe = fminf(fmaxf(pv[e], 1e-7f), 1.0f - 1e-7f);
+                        part = __fsub_rn(part, __fmul_rn(tv[e], logf(safe)));
+                    }
+                }
+            }
+        }
+    }
+    if (MODE) {
+        part = group_reduce<SumAcc, kWave>(part);
+        if (lane == 0) row_loss[row] = part;
+    }
+}
+
+static bool wave_row_ok(const float* a, const float* b, const float* c, size_t rows, size_t cols) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
+    return cols > 256 && cols <= (size_t)kWave * kWaveRowVec * 4 && cols % 4 == 0 && (bits & 15u) == 0 && rows >= 1024 &&
+           rows <= 0x7fffffffull;
+}
+
 static bool long_row_ok(const float* a, const float* b, const float* c, size_t rows, size_t cols) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
     return cols > 4096 && cols % 4 == 0 && cols <= (size_t)kLongRowThreads * kLongRowVec * 4 && (bits & 15u) == 0 &&
@@ -629,6 +706,9 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
     if (long_row_ok(logits, target, probs, rows, cols)) {
         hipLaunchKernelGGL((softmax_long_rows_kernel<1>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
                            logits, target, probs, row_loss, cols);
+    } else if (wave_row_ok(logits, target, probs, rows, cols)) {
+        hipLaunchKernelGGL((softmax_wave_rows_kernel<1>), dim3((unsigned)ceil_div_sz(rows, kBlock / kWave)), dim3(kBlock), 0,
+                           ctx->stream, logits, target, probs, row_loss, rows, cols);
     } else {
         const int tpr = pick_tpr(cols);
         const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
@@ -693,6 +773,9 @@ ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t 
     if (long_row_ok(x, x, y, rows, cols)) {
         hipLaunchKernelGGL((softmax_long_rows_kernel<0>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream, x,
                            (const float*)nullptr, y, (float*)nullptr, cols);
+    } else if (wave_row_ok(x, x, y, rows, cols)) {
+        hipLaunchKernelGGL((softmax_wave_rows_kernel<0>), dim3((unsigned)ceil_div_sz(rows, kBlock / kWave)), dim3(kBlock), 0,
+                           ctx->stream, x, (const float*)nullptr, y, (float*)nullptr, rows, cols);
     } else {
         const int tpr = pick_tpr(cols);
         const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);

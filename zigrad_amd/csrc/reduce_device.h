@@ -244,13 +244,52 @@ __global__ __launch_bounds__(kFlatSingle) void flat_single_kernel(const float* a
     if (threadIdx.x == 0) fin(acc);
 }
 
+// The first stage of the two-launch form.  A workgroup walks the input in chunks of kFlatChunk consecutive 16-byte
+// pieces (16 KiB per stream), four pieces per thread in flight: consecutive workgroups on consecutive chunks keep
+// DRAM pages open, which a grid-stride walk of the whole array does not (67 MB of squares: 18 -> 11 us).
+constexpr int kFlatU = 4;
+constexpr size_t kFlatChunk = (size_t)kFlatBlock * kFlatU;
 template <class T, int NIN>
 __global__ __launch_bounds__(kFlatBlock) void flat_partial_kernel(const float* a, const float* b, size_t n, float p0,
                                                                    typename T::P::Acc* partials) {
     using P = typename T::P;
     __shared__ typename P::Acc smem[kFlatBlock / kWave];
-    typename P::Acc acc = flat_accumulate<T, NIN>(a, b, n, p0, (size_t)blockIdx.x * kFlatBlock + threadIdx.x,
-                                                  (size_t)gridDim.x * kFlatBlock);
+    typename P::Acc acc = P::init();
+    const bool vec = ((reinterpret_cast<uintptr_t>(a) | (NIN > 1 ? reinterpret_cast<uintptr_t>(b) : 0)) & 15u) == 0;
+    if (vec) {
+        const size_t n4 = n >> 2;
+        const float4* a4 = reinterpret_cast<const float4*>(a);
+        const float4* b4 = reinterpret_cast<const float4*>(b);
+        for (size_t c0 = (size_t)blockIdx.x * kFlatChunk; c0 < n4; c0 += (size_t)gridDim.x * kFlatChunk) {
+            float4 u[kFlatU], w[kFlatU];
+#pragma unroll
+            for (int k = 0; k < kFlatU; k++) {
+                const size_t i = c0 + threadIdx.x + (size_t)k * kFlatBlock;
+                u[k] = make_float4(0, 0, 0, 0);
+                w[k] = u[k];
+                if (i < n4) {
+                    u[k] = a4[i];
+                    if (NIN > 1) w[k] = b4[i];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kFlatU; k++) {
+                const size_t i = c0 + threadIdx.x + (size_t)k * kFlatBlock;
+                if (i < n4) {
+                    acc = P::combine(acc, T::term(u[k].x, w[k].x, 4 * i + 0, p0));
+                    acc = P::combine(acc, T::term(u[k].y, w[k].y, 4 * i + 1, p0));
+                    acc = P::combine(acc, T::term(u[k].z, w[k].z, 4 * i + 2, p0));
+                    acc = P::combine(acc, T::term(u[k].w, w[k].w, 4 * i + 3, p0));
+                }
+            }
+        }
+        const size_t tid = (size_t)blockIdx.x * kFlatBlock + threadIdx.x, nthreads = (size_t)gridDim.x * kFlatBlock;
+        for (size_t t = (n4 << 2) + tid; t < n; t += nthreads)
+            acc = P::combine(acc, T::term(a[t], NIN > 1 ? b[t] : 0.f, t, p0));
+    } else {
+        acc = flat_accumulate<T, NIN>(a, b, n, p0, (size_t)blockIdx.x * kFlatBlock + threadIdx.x,
+                                      (size_t)gridDim.x * kFlatBlock);
+    }
     acc = block_reduce<P>(acc, smem);
     if (threadIdx.x == 0) partials[blockIdx.x] = acc;
 }
@@ -276,7 +315,7 @@ static int flat_reduce_into(zg_hip_ctx* ctx, const float* a, const float* b, siz
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    size_t blocks = ceil_div_sz(n, (size_t)kFlatBlock * 16);
+    size_t blocks = ceil_div_sz(n, kFlatChunk * 4);  // one chunk per workgroup until the partials buffer is full
     size_t cap = (size_t)ctx->n_cu * 8;
     if (cap > (size_t)kMaxPartials) cap = kMaxPartials;
     if (blocks > cap) blocks = cap;

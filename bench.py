@@ -410,6 +410,80 @@ def cpu_baseline(dims, batch, budget_steps=2, threads=None, loss_mode="onehot"):
     }
 
 
+VENDOR_SHAPES = [(4096, 4096, 4096, 1), (512, 512, 512, 32), (4096, 1024, 4096, 1), (3072, 3072, 3072, 1), (4100, 4100, 4100, 1),
+                 (2048, 2048, 2048, 1), (1536, 1536, 1536, 1), (1024, 1024, 1024, 1), (768, 768, 768, 1), (64, 128, 784, 1),
+                 (2708, 16, 1433, 1)]
+
+
+def vendor_gemm_child():
+    """The vendor leg, in a process of its own (torch brings its own HIP runtime): one JSON list of ms per shape."""
+    import torch
+
+    torch.backends.cuda.matmul.allow_tf32 = False
+    tdev = torch.device("cuda:0")
+    out = []
+    for m, n, k, nb in VENDOR_SHAPES:
+        iters = max(5, min(200, int(3e11 / (2.0 * m * n * k * nb))))
+        ta = torch.randn(nb, m, k, device=tdev) if nb > 1 else torch.randn(m, k, device=tdev)
+        tb = torch.randn(nb, n, k, device=tdev) if nb > 1 else torch.randn(n, k, device=tdev)
+        tc = torch.empty(nb, m, n, device=tdev) if nb > 1 else torch.empty(m, n, device=tdev)
+        tfn = (lambda: torch.bmm(ta, tb.transpose(1, 2), out=tc)) if nb > 1 else (lambda: torch.matmul(ta, tb.t(), out=tc))
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < 60.0:
+            for _ in range(iters):
+                tfn()
+            torch.cuda.synchronize()
+        ms = []
+        for _ in range(10):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                tfn()
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1) / iters)
+        out.append(sorted(ms)[5])
+        del ta, tb, tc
+    print(json.dumps(out))
+
+
+def vendor_gemm_table():
+    """A yardstick, not part of the product: fp32 products through this library and through the vendor's GEMM (torch's
+    matmul / bmm on the same GPU, TF32 off), same shapes (C = A B^T, B stored [n, k]), same timing method (60 ms of
+    warm-up, median of 10 event-bracketed batches), one process each, run one after the other."""
+    import subprocess
+
+    from zigrad_amd import HipDevice
+    from zigrad_amd.device import F32
+
+    dev = HipDevice(0)
+    ours = []
+    for m, n, k, nb in VENDOR_SHAPES:
+        iters = max(5, min(200, int(3e11 / (2.0 * m * n * k * nb))))
+        A, B, C = dev.mem_alloc(F32, nb * m * k), dev.mem_alloc(F32, nb * n * k), dev.mem_alloc(F32, nb * m * n)
+        dev.mem_random(A, "normal", seed=1)
+        dev.mem_random(B, "normal", seed=2)
+        if nb == 1:
+            fn = lambda: dev.dispatch("matmul", A=A, B=B, C=C, m=m, n=n, k=k, trans_a=False, trans_b=True, lda=k, ldb=k,
+                                      ldc=n, alpha=1.0, beta=0.0)
+        else:
+            fn = lambda: dev.dispatch("bmm_acc", A=A, B=B, C=C, A_shape=[nb, m, k], B_shape=[nb, k, n], C_shape=[nb, m, n],
+                                      trans_a=False, trans_b=True, lda=k, ldb=k, ldc=n, alpha=1.0, beta=0.0)
+        ours.append(time_op(dev, fn, iters)["ms"])
+        for b in (A, B, C):
+            dev.mem_free(b)
+    dev.deinit()
+    run = subprocess.run([sys.executable, str(Path(__file__).resolve()), "--vendor-gemm-child"], capture_output=True,
+                         text=True, timeout=600)
+    if run.returncode != 0:
+        sys.exit("the vendor leg failed: " + run.stderr[-2000:])
+    theirs = json.loads(run.stdout.strip().splitlines()[-1])
+    print(f"{'m x n x k (batch)':>28} {'this library':>22} {'vendor (torch.matmul)':>26}")
+    for (m, n, k, nb), a, b in zip(VENDOR_SHAPES, ours, theirs):
+        frac = lambda t: 2.0 * m * n * k * nb / (t * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS * 100
+        print(f"{m:>6} x {n:>5} x {k:>5} ({nb:>2}) {a * 1e3:>12.1f} us {frac(a):5.1f} % {b * 1e3:>16.1f} us {frac(b):5.1f} %")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -425,7 +499,16 @@ def main():
     ap.add_argument("--trace-fused", action="store_true", help="with --trace-small: through the fused entry points")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the execution-graph replays (rocprofv3's kernel tracing crashes inside hipGraphLaunch)")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="print a table of fp32 products through this library and through the vendor GEMM (torch) and exit")
+    ap.add_argument("--vendor-gemm-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.vendor_gemm_child:
+        vendor_gemm_child()
+        return
+    if args.vendor_gemm:
+        vendor_gemm_table()
+        return
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the hot path is single-device and this build uses no second GPU "
                  "(run with --gpus 1)")

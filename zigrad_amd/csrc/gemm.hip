@@ -815,19 +815,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(const float* P,
     const size_t n4 = M * N / 4, stride4 = M * N / 4;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
     for (; i < n4; i += nt) {
-        float4 acc = p[i];
-        int s = 1;
-        for (; s + 3 < splits; s += 4) {  // four loads in flight, added in split order
-            const float4 v0 = p[(size_t)s * stride4 + i], v1 = p[(size_t)(s + 1) * stride4 + i],
-                         v2 = p[(size_t)(s + 2) * stride4 + i], v3 = p[(size_t)(s + 3) * stride4 + i];
-            acc.x += v0.x; acc.y += v0.y; acc.z += v0.z; acc.w += v0.w;
-            acc.x += v1.x; acc.y += v1.y; acc.z += v1.z; acc.w += v1.w;
-            acc.x += v2.x; acc.y += v2.y; acc.z += v2.z; acc.w += v2.w;
-            acc.x += v3.x; acc.y += v3.y; acc.z += v3.z; acc.w += v3.w;
-        }
-        for (; s < splits; s++) {
-            const float4 v = p[(size_t)s * stride4 + i];
-            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s0 = 0; s0 < splits; s0 += 8) {  // eight partial tiles' loads in flight, added in split order
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (s0 + u < splits) v[u] = p[(size_t)(s0 + u) * stride4 + i];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (s0 + u < splits) {
+                    if (s0 + u == 0) {
+                        acc = v[u];  // the first partial tile starts the sum (no 0 + x: keeps a -0 as it is)
+                    } else {
+                        acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w;
+                    }
+                }
+            }
         }
         const size_t e = 4 * i, r = e / N, col = e % N;  // N is a multiple of 4: the four share a row
         float4* cp = reinterpret_cast<float4*>(c + r * ldc + col);

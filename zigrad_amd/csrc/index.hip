@@ -24,6 +24,7 @@ struct Plan {
     uint32_t* tile_sums; // scan scratch
     uint32_t* long_list; // [0] = number of long buckets, then their ids (at most n / kLongBucket of them)
     size_t n, nb;
+    long n_long;         // host copy of long_list[0] where the host has read it back (kept plans), else -1
 };
 
 // A bucket with more entries than this is "long": its entries are added by a whole wave (loads in parallel, additions
@@ -50,6 +51,7 @@ static Plan carve_plan(void* mem, size_t n, size_t nb) {
     Plan pl;
     pl.n = n;
     pl.nb = nb;
+    pl.n_long = -1;
     pl.row_ptr = (uint32_t*)p;
     p += align_up((nb + 1) * 4, 256);
     pl.cursor = (uint32_t*)p;
@@ -428,6 +430,14 @@ static bool plan_from_cache(zg_hip_ctx* ctx, const uint64_t* keys, const uint64_
             *rc = zg_hip_memcpy_d2d(ctx, e->payload_dev, payload, bytes);
         }
         if (!*rc) *rc = build_plan(ctx, e->keys_dev, e->plan, e->payload_dev);
+        if (!*rc) {
+            // how many long buckets there are is read back once, so that later calls skip the long-bucket kernel's
+            // launch when there is none (the usual case: a graph's edge list)
+            uint32_t n_long = 0;
+            if (hipMemcpyAsync(&n_long, e->plan.long_list, sizeof(n_long), hipMemcpyDeviceToHost, ctx->stream) == hipSuccess &&
+                hipStreamSynchronize(ctx->stream) == hipSuccess)
+                e->plan.n_long = (long)n_long;
+        }
         if (*rc) {
             (void)hipStreamSynchronize(ctx->stream);
             zg_hip_free(ctx, mem);
@@ -583,7 +593,7 @@ static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Pla
     hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(pl.nb, 256)), dim3(256), 0, ctx->stream, src,
                        pl.row_ptr, pl.perm, dst, pl.nb, fresh);
     ZG_LAUNCH_CHECK();
-    if (pl.n > kLongBucket) {
+    if (pl.n > kLongBucket && pl.n_long != 0) {
         size_t grid = ceil_div_sz(pl.n / kLongBucket, 4);
         if (grid > 2048) grid = 2048;
         hipLaunchKernelGGL(scatter_add_apply_long_kernel, dim3((unsigned)grid), dim3(256), 0, ctx->stream, src, pl.row_ptr,
@@ -790,7 +800,8 @@ __global__ void invert_perm_kernel(const uint32_t* row_ptr, size_t nb, const uin
 
 __global__ void gcn_bwd_edge_terms_slots_kernel(const float* go, const float* h, const float* deg,
                                                 const uint64_t* src_idx, const uint64_t* tgt_idx, size_t n_edge,
-                                                size_t n_nodes, size_t stride, const uint32_t* slot_of, float* terms) {
+                                                size_t n_nodes, size_t stride, const uint32_t* slot_of, float* terms,
+                                                bool vec4) {
     size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n_edge) return;
     const uint64_t s = src_idx[e], t = tgt_idx[e];
@@ -798,10 +809,34 @@ __global__ void gcn_bwd_edge_terms_slots_kernel(const float* go, const float* h,
     float gs = 0.f, gt = 0.f;
     if (s < n_nodes && t < n_nodes) {
         const float ds = deg[s], dt = deg[t];
-        for (size_t j = 0; j < stride; j++) {
-            const float g = go[t * stride + j], hv = h[s * stride + j];
+        const float* gr = go + t * stride;
+        const float* hr = h + s * stride;
+        auto term = [&](float g, float hv) {
             gs = __fadd_rn(gs, __fmul_rn(__fmul_rn(g, dt), hv));
             gt = __fadd_rn(gt, __fmul_rn(__fmul_rn(g, ds), hv));
+        };
+        if (vec4) {  // stride a multiple of 4 and both matrices 16-byte aligned: a row is whole 16-byte pieces
+            for (size_t j = 0; j < stride; j += 16) {  // up to four pieces of each row in flight
+                float4 gv[4], hv[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    if (j + 4 * u < stride) {
+                        gv[u] = *reinterpret_cast<const float4*>(gr + j + 4 * u);
+                        hv[u] = *reinterpret_cast<const float4*>(hr + j + 4 * u);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    if (j + 4 * u < stride) {
+                        term(gv[u].x, hv[u].x);
+                        term(gv[u].y, hv[u].y);
+                        term(gv[u].z, hv[u].z);
+                        term(gv[u].w, hv[u].w);
+                    }
+                }
+            }
+        } else {
+            for (size_t j = 0; j < stride; j++) term(gr[j], hr[j]);
         }
     }
     if (slot_s != 0xffffffffu) terms[slot_s] = gs;
@@ -1098,7 +1133,7 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
         float* terms = term_src;
         hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0,
                            ctx->stream, grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride,
-                           rs.entry->slot_of, terms);
+                           rs.entry->slot_of, terms, stride % 4 == 0 && aligned16(grad_output) && aligned16(h));
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0,
                            ctx->stream, grad_deg, terms, rs.entry->inc.row_ptr, n_nodes, false);

@@ -200,6 +200,7 @@ struct GemmArgs {
     size_t nba, nbb;
     size_t a_chunk, b_chunk, c_chunk;
     unsigned tiles_m, tiles_n;
+    unsigned flat_batches;  // staged kernels: number of batches folded into grid.x (0: the batch is grid.z)
     // split-K: workgroup y handles k-tiles [y * split_tiles, (y + 1) * split_tiles) and writes its C tile at
     // C + y * split_stride (the launcher points C at a buffer of partial products); one split = the whole of k
     size_t split_tiles, split_stride;
@@ -229,11 +230,11 @@ __device__ __forceinline__ float gemm_extras(float v, bool has_bias, float bias,
 // that stop sharing L2 lines after a few dozen k-tiles.  Each half is a run of 32 consecutive ids; 4 rows x 8
 // columns is the shape of such a run with the fewest A and B panel bytes for the 256 x 128 tile (8 rows x 4
 // columns fetched 47 % more from the fabric, measured with FETCH_SIZE).
-__device__ __forceinline__ void tile_coords(unsigned pid, unsigned tiles_m, unsigned tiles_n, unsigned& tm,
+__device__ __forceinline__ unsigned xcd_contiguous(unsigned pid, unsigned total) {
+    return ((total & 7u) == 0) ? (pid & 7u) * (total >> 3) + (pid >> 3) : pid;
+}
+__device__ __forceinline__ void tile_coords(unsigned id, unsigned tiles_m, unsigned tiles_n, unsigned& tm,
                                             unsigned& tn) {
-    const unsigned total = tiles_m * tiles_n;
-    unsigned id = pid;
-    if ((total & 7u) == 0) id = (pid & 7u) * (total >> 3) + (pid >> 3);
     constexpr unsigned GM = 4;
     const unsigned per_group = GM * tiles_n;
     const unsigned group = id / per_group;
@@ -268,9 +269,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     float* const As0 = lds;
     float* const Bs0 = lds + 2 * TA::ELEMS;
 
+    // Batched products with few tiles per batch fold the batch into grid.x (flat_batches != 0): the contiguous run of
+    // logical ids an XCD gets then holds whole batches, so the tiles that share a batch's A and B panels share an L2.
+    // With the batch in grid.z the hardware deals the tiles of one batch out over all eight XCDs and every tile
+    // fetches its panels alone (32 x 512 x 512 x 4096: 513 -> 46x us).
     unsigned tm, tn;
-    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
-    const size_t z = blockIdx.z;
+    size_t z = blockIdx.z;
+    {
+        const unsigned per_batch = g.tiles_m * g.tiles_n;
+        if (g.flat_batches) {
+            const unsigned id = xcd_contiguous(blockIdx.x, per_batch * g.flat_batches);
+            z = id / per_batch;
+            tile_coords(id % per_batch, g.tiles_m, g.tiles_n, tm, tn);
+        } else {
+            tile_coords(xcd_contiguous(blockIdx.x, per_batch), g.tiles_m, g.tiles_n, tm, tn);
+        }
+    }
     const float* A = g.A + (z % g.nba) * g.a_chunk;
     const float* B = g.B + (z % g.nbb) * g.b_chunk;
     float* C = g.C + z * g.c_chunk + (size_t)blockIdx.y * g.split_stride;
@@ -601,6 +615,12 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
     g.tiles_n = (unsigned)ceil_div_sz(g.N, BN);
     const size_t kt_total = ceil_div_sz(g.K, kBK);
     dim3 grid(g.tiles_m * g.tiles_n, (unsigned)ceil_div_sz(kt_total, g.split_tiles), (unsigned)batches), block(kGemmThreads);
+    const size_t flat = (size_t)grid.x * batches;
+    g.flat_batches = 0;
+    if (batches > 1 && grid.y == 1 && flat % 8 == 0 && flat < 0x7fffffffull) {
+        g.flat_batches = (unsigned)batches;
+        grid = dim3((unsigned)flat, 1, 1);
+    }
 #define ZG_GEMM(AK, BKM, MD)                                                                                  \
     do {                                                                                                      \
         constexpr size_t lds_bytes = 2 * (size_t)(Tile<BM, AK>::ELEMS + Tile<BN, BKM>::ELEMS) * sizeof(float); \
@@ -1051,6 +1071,7 @@ static GemmArgs gemm_args(const float* A, const float* B, float* C, size_t m, si
     g.b_vec = aligned16(B) && ldb % 4 == 0 && b_chunk % 4 == 0;
     g.tiles_m = (unsigned)ceil_div_sz(m, 32);  // the unstaged kernel's blocks; the staged launcher sets its own
     g.tiles_n = (unsigned)ceil_div_sz(n, 32);
+    g.flat_batches = 0;
     g.split_tiles = 0;
     g.split_stride = 0;
     g.c_vec = 0;

@@ -264,7 +264,8 @@ int zg_hip_segment_sum_csr(zg_hip_ctx *ctx, const float *src, size_t src_len, co
  * copy of the arrays' contents and a device copy for the kernels.  A later call whose arrays hold the same values
  * (compared on the host, byte for byte, when the call is made) runs the same apply kernels on the kept ordering
  * instead of computing it again: same values, five to six launches fewer per ordering.  At most 16 orderings are
- * kept (least recently used goes first).  A recorded graph keeps the orderings it used, and zg_hip_graph_run returns
+ * kept (least recently used goes first), for arrays of up to 65536 entries (longer ones cost more to compare than
+ * to analyse).  A recorded graph keeps the orderings it used, and zg_hip_graph_run returns
  * ZG_HIP_EINVAL when one of those arrays no longer holds what it held at the recording.  Index arrays in device
  * memory are analysed on every call.  `hits` / `builds` count calls served from a kept ordering / orderings computed
  * and kept; no counterpart in the reference. */

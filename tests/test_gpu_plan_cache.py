@@ -170,3 +170,19 @@ def test_a_recorded_step_refuses_to_replay_over_a_rewritten_index_array(oracle, 
     g.free()
     for b in (a, s, d):
         hip.mem_free(b)
+
+
+def test_long_pinned_index_arrays_are_analysed_every_call(oracle, hip):
+    """Beyond 65536 entries the host comparison would cost more than the analysis: nothing is kept, results as ever."""
+    r = np.random.default_rng(5)
+    n, n_dst = 70_000, 900
+    off = r.integers(0, n_dst, n).astype(np.uint64)
+    src = r.standard_normal(n).astype(np.float32)
+    dst0 = np.zeros(n_dst, np.float32)
+    want = run_op(oracle, "scatter_add", {"src": src, "offsets": off, "dst": dst0.copy()}, ["dst"])["dst"]
+    a = _pinned(hip, off)
+    before = hip.plan_cache_stats()
+    for _ in range(2):
+        np.testing.assert_array_equal(_scatter(hip, src, a, dst0), want)
+    assert hip.plan_cache_stats() == before
+    hip.mem_free(a)

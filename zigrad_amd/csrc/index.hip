@@ -340,7 +340,9 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
 // has rewritten the arrays.
 // ------------------------------------------------------------------------------------------------
 constexpr size_t kPlanCacheMax = 16;
-constexpr size_t kPlanCacheMaxEntries = (size_t)1 << 24;  // longer index arrays are not worth a host comparison per call
+// The host comparison costs about 50 us per MB; the five to six launches it saves take 20 to 30 us of GPU time and
+// about as much host time, so arrays of more than 64 Ki entries (512 KiB) are analysed on the GPU every call.
+constexpr size_t kPlanCacheMaxEntries = (size_t)1 << 16;
 
 struct CachedPlan {
     std::vector<uint64_t> keys_host, payload_host;  // what the arrays held when the plan was built

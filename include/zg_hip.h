@@ -108,6 +108,12 @@ int zg_hip_cache_stats(zg_hip_ctx *ctx, size_t *bytes_in_use, size_t *bytes_mapp
 int zg_hip_memcpy_h2d(zg_hip_ctx *ctx, void *dst, const void *src_host, size_t bytes); /* mem_transfer .HtoD */
 int zg_hip_memcpy_d2h(zg_hip_ctx *ctx, void *dst_host, const void *src, size_t bytes); /* .DtoH, blocking */
 int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes);      /* mem_copy / .DtoD */
+/* mem_fill (src/device/host_device.zig:876-884).  The fill is queued inside the context and launched together with
+ * any other waiting fills (up to 16, one kernel) at the start of the next call on this context that is not a float fill
+ * or a cache allocation: callers zero gradients tensor by tensor (examples/mnist/src/model.zig:57-62) and one launch per
+ * tensor costs more than the fills.  Every later call on the context, zg_hip_sync, zg_hip_stream and a recording's
+ * end included, therefore finds the memory filled; only work queued on the raw stream obtained EARLIER from
+ * zg_hip_stream, with no call on the context in between, could overtake a waiting fill. */
 int zg_hip_mem_fill(zg_hip_ctx *ctx, float *x, size_t n, float value);
 int zg_hip_mem_fill_u8(zg_hip_ctx *ctx, void *x, size_t n, uint8_t value);
 int zg_hip_mem_fill_u64(zg_hip_ctx *ctx, uint64_t *x, size_t n, uint64_t value);

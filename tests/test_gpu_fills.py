@@ -1,0 +1,117 @@
+"""Float fills wait in the context and go out as one launch with the next call that is not a fill
+(src/device/host_device.zig:876-884 fills at once; callers zero gradients tensor by tensor).  Whatever the caller does
+next must see every fill: later fills win over earlier ones on the same memory, a freed block's fill does not land on
+its next owner, more fills than the queue holds, odd offsets and lengths, and fills recorded into a graph."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from zigrad_amd.device import F32
+
+pytestmark = pytest.mark.gpu
+
+
+def test_many_fills_of_odd_pieces_then_a_read(hip):
+    r = np.random.default_rng(0)
+    n = 300_000
+    buf = hip.from_numpy(np.full(n, -1.0, np.float32))
+    want = np.full(n, -1.0, np.float32)
+    pos = 0
+    k = 0
+    while pos < n and k < 40:  # 40 fills: the queue (16) is sent more than once
+        length = int(r.integers(1, 20_000))
+        off = pos + int(r.integers(0, 7))  # 4-byte aligned only
+        if off + length > n:
+            break
+        hip.mem_fill(buf.sub(off, length), float(k))
+        want[off:off + length] = k
+        pos = off + length
+        k += 1
+    np.testing.assert_array_equal(hip.to_numpy(buf), want)  # the read comes after every fill
+    hip.mem_free(buf)
+
+
+def test_a_later_fill_wins_where_two_overlap(hip):
+    buf = hip.mem_alloc(F32, 10_000)
+    hip.mem_fill(buf, 1.0)
+    hip.mem_fill(buf.sub(100, 5000), 2.0)
+    hip.mem_fill(buf.sub(4000, 3000), 3.0)
+    hip.mem_fill(buf.sub(0, 1), 4.0)
+    want = np.full(10_000, 1.0, np.float32)
+    want[100:5100] = 2.0
+    want[4000:7000] = 3.0
+    want[0] = 4.0
+    np.testing.assert_array_equal(hip.to_numpy(buf), want)
+    hip.mem_free(buf)
+
+
+def test_a_fill_then_an_op_on_the_same_memory(hip):
+    n = 5000
+    a = hip.from_numpy(np.arange(n, dtype=np.float32))
+    b = hip.mem_alloc(F32, n)
+    hip.mem_fill(b, 0.5)
+    hip.dispatch("add", x=a, y=b, z=b)  # reads the filled values, in place
+    np.testing.assert_array_equal(hip.to_numpy(b), np.arange(n, dtype=np.float32) + 0.5)
+    hip.mem_fill(a, 0.0)
+    hip.dispatch("relu_fwd", x=b, y=a)  # overwrites what the waiting fill wrote: the fill must not come after it
+    np.testing.assert_array_equal(hip.to_numpy(a), np.arange(n, dtype=np.float32) + 0.5)
+    for x in (a, b):
+        hip.mem_free(x)
+
+
+def test_a_fill_of_a_block_that_is_freed_does_not_reach_its_next_owner(hip):
+    n = 4096
+    first = hip.mem_cache_alloc(F32, n)
+    hip.mem_fill(first, 9.0)
+    hip.mem_cache_free(first)                 # the fill is sent before the block returns to the pool
+    second = hip.mem_cache_alloc(F32, n)      # most likely the same block
+    hip.mem_transfer(np.full(n, 1.0, np.float32), second, "HtoD")
+    hip.sync()
+    np.testing.assert_array_equal(hip.to_numpy(second), np.full(n, 1.0, np.float32))
+    # allocations in between leave fills waiting; they still all arrive
+    bufs = []
+    for i in range(20):
+        b = hip.mem_cache_alloc(F32, 1000 + i)
+        hip.mem_fill(b, float(i))
+        bufs.append(b)
+    for i, b in enumerate(bufs):
+        np.testing.assert_array_equal(hip.to_numpy(b), np.full(1000 + i, float(i), np.float32))
+        hip.mem_cache_free(b)
+    hip.mem_cache_free(second)
+
+
+def test_fills_recorded_into_a_graph_replay_with_it(hip):
+    n = 3000
+    a, b, out = hip.mem_alloc(F32, n), hip.mem_alloc(F32, n), hip.mem_alloc(F32, n)
+    hip.mem_fill(a, 0.0)
+    hip.mem_fill(b, 0.0)
+    hip.mem_fill(out, 0.0)
+    hip.sync()
+    hip.mem_fill(a, 7.0)  # waiting when the recording starts: sent before it, not recorded
+    hip.graph_open()
+    hip.mem_fill(a, 2.0)
+    hip.mem_fill(b, 3.0)
+    hip.dispatch("add", x=a, y=b, z=out)
+    hip.mem_fill(b, 1.0)  # waiting when the recording ends: recorded
+    g = hip.graph_save()
+    for _ in range(3):
+        hip.mem_transfer(np.full(n, -5.0, np.float32), a, "HtoD")
+        hip.mem_transfer(np.full(n, -5.0, np.float32), b, "HtoD")
+        g.run()
+        hip.sync()
+        np.testing.assert_array_equal(hip.to_numpy(out), np.full(n, 5.0, np.float32))
+        np.testing.assert_array_equal(hip.to_numpy(b), np.full(n, 1.0, np.float32))
+        np.testing.assert_array_equal(hip.to_numpy(a), np.full(n, 2.0, np.float32))
+    g.free()
+    for x in (a, b, out):
+        hip.mem_free(x)
+
+
+def test_one_large_fill_and_its_tail(hip):
+    n = (1 << 24) + 3
+    buf = hip.mem_alloc(F32, n)
+    hip.mem_fill(buf, 1.25)
+    got = hip.to_numpy(buf)
+    assert got[0] == 1.25 and got[-1] == 1.25 and np.all(got == 1.25)
+    hip.mem_free(buf)

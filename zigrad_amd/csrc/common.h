@@ -40,6 +40,14 @@ struct zg_hip_event {
     hipEvent_t ev;
 };
 
+// A float fill that has been asked for and not launched yet (runtime.hip).
+struct zg_pending_fill {
+    float* x;
+    size_t n;
+    float value;
+};
+constexpr int kMaxPendingFills = 16;
+
 struct zg_hip_ctx {
     int device = 0;
     int n_cu = 256;
@@ -85,6 +93,13 @@ struct zg_hip_ctx {
     zg::PlanCache* plan_cache = nullptr;
     std::vector<zg::PlanUse> plan_uses;
 
+    // Float fills wait here until the next call that is not a fill (or an allocation) and then go out as one launch:
+    // callers zero their gradients tensor by tensor (examples/mnist/src/model.zig:57-62: one fill per parameter), and a
+    // launch per tensor costs more than the fills themselves.  Every entry point starts with ZG_CTX, which sends
+    // the waiting fills first, so no call can see memory that a fill has not reached yet.
+    zg_pending_fill pending_fills[kMaxPendingFills];
+    int n_pending_fills = 0;
+
     // launch plans of the staged GEMM kernels, by shape (gemm.hip)
     zg::GemmPlanCache* gemm_plans = nullptr;
 
@@ -101,6 +116,9 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 // Cached segment plans (index.hip).  destroy: at deinit.  retain: a saved graph takes (+1) or drops (-1) its plans,
 // which are never evicted while a graph names them.  validate: before a replay, every index array the recording
 // matched must still hold what it held then, or the replay would scatter by a stale plan.
+// Launches the fills that are waiting in the context (one kernel for all of them).
+int flush_fills(zg_hip_ctx* ctx);
+
 void plan_cache_destroy(zg_hip_ctx* ctx);
 void gemm_plans_destroy(zg_hip_ctx* ctx);
 void plan_uses_retain(const std::vector<PlanUse>& uses, int delta);
@@ -157,7 +175,15 @@ inline bool aligned16(const void* p) {
         }                                                                                        \
     } while (0)
 
-#define ZG_CTX(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
+// First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
+#define ZG_CTX(ctx)                                          \
+    ZG_REQUIRE((ctx) != nullptr, "null context");            \
+    if ((ctx)->n_pending_fills) {                            \
+        if (int _rc_fill = zg::flush_fills(ctx)) return _rc_fill; \
+    }
+// The same for the few calls that leave waiting fills alone: the fills themselves, and allocations (a block that is
+// handed out is free, so no waiting fill names it; a block that is freed goes through ZG_CTX).
+#define ZG_CTX_KEEP_FILLS(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.
 #define ZG_NOT_CAPTURING(ctx, who)                                                                       \

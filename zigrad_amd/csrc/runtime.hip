@@ -662,7 +662,9 @@ ZG_API int zg_hip_total_memory(zg_hip_ctx* ctx, size_t* bytes) {
 }
 
 ZG_API void* zg_hip_stream(zg_hip_ctx* ctx) {
-    return ctx ? (void*)ctx->stream : nullptr;
+    if (!ctx) return nullptr;
+    (void)flush_fills(ctx);  // work the caller queues on the stream itself must find every fill already there
+    return (void*)ctx->stream;
 }
 
 ZG_API int zg_hip_event_create(zg_hip_ctx* ctx, zg_hip_event** out) {
@@ -801,7 +803,7 @@ ZG_API int zg_hip_cache_configure(zg_hip_ctx* ctx, size_t small_pool_bytes, size
 }
 
 ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uint64_t* block) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
     ZG_REQUIRE(out != nullptr && block != nullptr, "mem_cache_alloc: null output");
     *out = nullptr;
     *block = 0;
@@ -974,25 +976,74 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
     return ZG_HIP_OK;
 }
 
+// Up to kMaxPendingFills float fills in one launch: workgroup b fills one slice of kFillSlice floats of the fill
+// that owns it (wg_first is the running count of slices).  Slices of a 16-byte aligned array are written in
+// 16-byte pieces, four per thread.
+constexpr size_t kFillSlice = 4096;
+struct MultiFillArgs {
+    float* x[kMaxPendingFills];
+    size_t n[kMaxPendingFills];
+    float value[kMaxPendingFills];
+    unsigned wg_first[kMaxPendingFills + 1];
+    int count;
+};
+__global__ __launch_bounds__(kBlock) void multi_fill_kernel(MultiFillArgs a) {
+    int e = 0;
+    while (e + 1 < a.count && blockIdx.x >= a.wg_first[e + 1]) e++;
+    const size_t s0 = (size_t)(blockIdx.x - a.wg_first[e]) * kFillSlice;
+    float* x = a.x[e] + s0;
+    const size_t n = a.n[e] - s0 < kFillSlice ? a.n[e] - s0 : kFillSlice;
+    const float v = a.value[e];
+    size_t done = 0;
+    if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+        const size_t n4 = n >> 2;
+        const float4 v4 = make_float4(v, v, v, v);
+        for (size_t i = threadIdx.x; i < n4; i += kBlock) reinterpret_cast<float4*>(x)[i] = v4;
+        done = n4 << 2;
+    }
+    for (size_t i = done + threadIdx.x; i < n; i += kBlock) x[i] = v;
+}
+
+namespace zg {
+int flush_fills(zg_hip_ctx* ctx) {
+    const int count = ctx->n_pending_fills;
+    if (count == 0) return ZG_HIP_OK;
+    ctx->n_pending_fills = 0;  // whatever happens below, the same fills are not sent twice
+    MultiFillArgs a;
+    size_t wgs = 0;
+    for (int i = 0; i < count; i++) {
+        a.x[i] = ctx->pending_fills[i].x;
+        a.n[i] = ctx->pending_fills[i].n;
+        a.value[i] = ctx->pending_fills[i].value;
+        a.wg_first[i] = (unsigned)wgs;
+        wgs += ceil_div_sz(a.n[i], kFillSlice);
+    }
+    a.wg_first[count] = (unsigned)wgs;
+    a.count = count;
+    hipLaunchKernelGGL(multi_fill_kernel, dim3((unsigned)wgs), dim3(kBlock), 0, ctx->stream, a);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+}  // namespace zg
+
 ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x != nullptr, "mem_fill: null pointer");
-    if (aligned16(x) && n >= 4) {
-        size_t n4 = n / 4;
-        hipLaunchKernelGGL(fill4_kernel, dim3(grid_for(ctx, n4, kBlock)), dim3(kBlock), 0, ctx->stream, (float4*)x, n4,
-                           value);
-        ZG_LAUNCH_CHECK();
-        size_t tail = n - n4 * 4;
-        if (tail) {
-            hipLaunchKernelGGL(fill_kernel<float>, dim3(1), dim3(64), 0, ctx->stream, x + n4 * 4, tail, value);
-            ZG_LAUNCH_CHECK();
-        }
-    } else {
-        hipLaunchKernelGGL(fill_kernel<float>, dim3(grid_for(ctx, n, kBlock)), dim3(kBlock), 0, ctx->stream, x, n,
-                           value);
-        ZG_LAUNCH_CHECK();
+    // The fill waits for the next call that is not a fill.  Two waiting fills never overlap (workgroups of one launch
+    // would race, and the later fill must win), and their slices must fit one grid.
+    size_t wgs = ceil_div_sz(n, kFillSlice);
+    bool send_first = ctx->n_pending_fills == kMaxPendingFills;
+    for (int i = 0; i < ctx->n_pending_fills && !send_first; i++) {
+        const zg_pending_fill& p = ctx->pending_fills[i];
+        if (x < p.x + p.n && p.x < x + n) send_first = true;
+        wgs += ceil_div_sz(p.n, kFillSlice);
     }
+    if (wgs > 0x7fffffffull) send_first = true;
+    if (send_first)
+        if (int rc = flush_fills(ctx)) return rc;
+    ZG_REQUIRE(ceil_div_sz(n, kFillSlice) <= 0x7fffffffull, "mem_fill: more than 2^43 elements");
+    ctx->pending_fills[ctx->n_pending_fills++] = zg_pending_fill{x, n, value};
     return ZG_HIP_OK;
 }
 

@@ -113,7 +113,9 @@ int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
  * or a cache allocation: callers zero gradients tensor by tensor (examples/mnist/src/model.zig:57-62) and one launch per
  * tensor costs more than the fills.  Every later call on the context, zg_hip_sync, zg_hip_stream and a recording's
  * end included, therefore finds the memory filled; only work queued on the raw stream obtained EARLIER from
- * zg_hip_stream, with no call on the context in between, could overtake a waiting fill. */
+ * zg_hip_stream, with no call on the context in between, could overtake a waiting fill.  A waiting fill of +0.0 over
+ * exactly the dense output of zg_hip_matmul / zg_hip_bmm_acc with beta = 1, or the gradient of zg_hip_smce_bwd, is not
+ * launched at all: the op writes what it would have added to the zeros. */
 int zg_hip_mem_fill(zg_hip_ctx *ctx, float *x, size_t n, float value);
 int zg_hip_mem_fill_u8(zg_hip_ctx *ctx, void *x, size_t n, uint8_t value);
 int zg_hip_mem_fill_u64(zg_hip_ctx *ctx, uint64_t *x, size_t n, uint64_t value);

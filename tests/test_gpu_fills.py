@@ -115,3 +115,73 @@ def test_one_large_fill_and_its_tail(hip):
     got = hip.to_numpy(buf)
     assert got[0] == 1.25 and got[-1] == 1.25 and np.all(got == 1.25)
     hip.mem_free(buf)
+
+
+def test_an_accumulating_product_takes_over_a_waiting_zero_fill(hip):
+    """ensure_grad(0) then `C += A B` (src/ndtensor.zig:221-228, :1092-1136): the product writes C instead of adding to
+    zeros; any other fill value, a padded C or a refused product leaves the fill's effect in place."""
+    from zigrad_amd._lib import ZgHipError
+
+    r = np.random.default_rng(1)
+    m, n, k = 96, 80, 64
+    A = r.standard_normal((m, k), dtype=np.float32)
+    B = r.standard_normal((k, n), dtype=np.float32)
+    a, b = hip.from_numpy(A), hip.from_numpy(B)
+    c = hip.from_numpy(np.full(m * n, np.nan, np.float32))
+    prod = (A.astype(np.float64) @ B.astype(np.float64))
+
+    def matmul(cbuf, ldc=n, lda=k, beta=1.0):
+        hip.dispatch("matmul", A=a, B=b, C=cbuf, m=m, n=n, k=k, trans_a=False, trans_b=False, lda=lda, ldb=n, ldc=ldc,
+                     alpha=1.0, beta=beta)
+
+    hip.mem_fill(c, 0.0)
+    matmul(c)
+    got = hip.to_numpy(c).reshape(m, n)
+    assert np.linalg.norm(got - prod) <= 1e-5 * np.linalg.norm(prod)
+    matmul(c)  # nothing waiting now: a true accumulation
+    assert np.linalg.norm(hip.to_numpy(c).reshape(m, n) - 2 * prod) <= 1e-5 * np.linalg.norm(2 * prod)
+    hip.mem_fill(c, 1.0)  # not zero: stays a fill
+    matmul(c)
+    assert np.linalg.norm(hip.to_numpy(c).reshape(m, n) - (prod + 1.0)) <= 1e-5 * np.linalg.norm(prod + 1.0)
+    hip.mem_fill(c, 0.0)  # batched form, one batch: the same rule
+    hip.dispatch("bmm_acc", A=a, B=b, C=c, A_shape=[1, m, k], B_shape=[1, k, n], C_shape=[1, m, n], trans_a=False,
+                 trans_b=False, lda=k, ldb=n, ldc=n, alpha=1.0, beta=1.0)
+    assert np.linalg.norm(hip.to_numpy(c).reshape(m, n) - prod) <= 1e-5 * np.linalg.norm(prod)
+    # a C with padding between rows: the fill covers the padding too and is launched as a fill
+    wide = hip.from_numpy(np.full(m * (n + 8), np.nan, np.float32))
+    hip.mem_fill(wide, 0.0)
+    matmul(wide, ldc=n + 8)
+    w = hip.to_numpy(wide).reshape(m, n + 8)
+    assert np.linalg.norm(w[:, :n] - prod) <= 1e-5 * np.linalg.norm(prod) and np.all(w[:, n:] == 0.0)
+    # a refused product (lda too small) after a zero fill: C holds the zeros
+    hip.mem_transfer(np.full(m * n, np.nan, np.float32), c, "HtoD")
+    hip.mem_fill(c, 0.0)
+    with pytest.raises(ZgHipError):
+        matmul(c, lda=k - 1)
+    assert np.all(hip.to_numpy(c) == 0.0)
+    for x in (a, b, c, wide):
+        hip.mem_free(x)
+
+
+def test_the_loss_backward_takes_over_a_waiting_zero_fill(oracle, hip):
+    from conftest import run_op
+
+    r = np.random.default_rng(2)
+    rows, cols = 64, 10
+    logits = r.standard_normal((rows, cols)).astype(np.float32)
+    onehot = np.eye(cols, dtype=np.float32)[r.integers(0, cols, rows)]
+    fw = run_op(oracle, "smce_fwd", {"logits": logits, "target": onehot, "probs": np.zeros_like(logits),
+                                     "loss": np.zeros(1, np.float32), "rows": rows, "cols": cols}, ["probs"])
+    probs = fw["probs"]
+    want = run_op(oracle, "smce_bwd", {"probs": probs, "target": onehot, "grad": np.zeros_like(logits), "rows": rows,
+                                       "cols": cols}, ["grad"])["grad"]
+    p, t = hip.from_numpy(probs), hip.from_numpy(onehot)
+    g = hip.from_numpy(np.full(rows * cols, np.nan, np.float32))
+    hip.mem_fill(g, 0.0)
+    hip.dispatch("smce_bwd", probs=p, target=t, grad=g, rows=rows, cols=cols)
+    got = hip.to_numpy(g).reshape(rows, cols)
+    assert np.array_equal(got, want)
+    hip.dispatch("smce_bwd", probs=p, target=t, grad=g, rows=rows, cols=cols)  # now it accumulates
+    assert np.array_equal(hip.to_numpy(g).reshape(rows, cols), want + want)
+    for x in (p, t, g):
+        hip.mem_free(x)

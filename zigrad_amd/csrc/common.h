@@ -118,6 +118,11 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 // matched must still hold what it held then, or the replay would scatter by a stale plan.
 // Launches the fills that are waiting in the context (one kernel for all of them).
 int flush_fills(zg_hip_ctx* ctx);
+// An op that adds into x[0 .. n) asks whether a fill of exactly that range with +0.0 is still waiting.  If so the fill
+// is dropped and true comes back: the op then writes its result instead of adding it to zeros it would have to read
+// (ensure_grad(0) followed by an accumulating backward op, src/ndtensor.zig:221-228), the same values without the
+// fill's launch and without the read.
+bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n);
 
 void plan_cache_destroy(zg_hip_ctx* ctx);
 void gemm_plans_destroy(zg_hip_ctx* ctx);

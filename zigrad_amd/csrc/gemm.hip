@@ -1369,8 +1369,14 @@ ZG_API int zg_hip_gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_
 
 ZG_API int zg_hip_matmul(zg_hip_ctx* ctx, const float* A, const float* B, float* C, size_t m, size_t n, size_t k,
                          int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
-    ZG_CTX(ctx);
-    return gemm_dispatch(ctx, "matmul", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, 1, 1, 1, 0, 0, 0);
+    ZG_CTX_KEEP_FILLS(ctx);
+    // C += ... into a C whose zero fill has not been launched yet: write instead (no fill, no read of C)
+    const bool zeroed = beta == 1.f && C && ldc == n && k > 0 && alpha != 0.f && absorb_zero_fill(ctx, C, m * n);
+    if (int rc = flush_fills(ctx)) return rc;
+    const int rc = gemm_dispatch(ctx, "matmul", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, zeroed ? 0.f : beta,
+                                 1, 1, 1, 0, 0, 0);
+    if (rc && zeroed) (void)zg_hip_mem_fill(ctx, C, m * n, 0.f);  // the product was refused: the zeros are still owed
+    return rc;
 }
 
 // y = act(x . w^T + bias): one launch where the product is one launch (the bias add and the ReLU ride in the GEMM
@@ -1459,10 +1465,19 @@ ZG_API int zg_hip_linear_bwd(zg_hip_ctx* ctx, const float* gy, const float* x, c
 ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_shape, const float* B,
                           const uint64_t* B_shape, float* C, const uint64_t* C_shape, int trans_a, int trans_b,
                           size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
     ZG_REQUIRE(A_shape && B_shape && C_shape, "bmm_acc: null shape");
     const size_t nba = A_shape[0], nbb = B_shape[0], nbc = C_shape[0];
     const size_t m = C_shape[1], n = C_shape[2], k = A_shape[2];
+    // C += ... into a C whose zero fill has not been launched yet (ensure_grad(0) then BmmAccBwd,
+    // src/ndtensor.zig:221-228, :1092-1136): write instead (no fill, no read of C)
+    const bool zeroed = beta == 1.f && C && ldc == n && k > 0 && alpha != 0.f && absorb_zero_fill(ctx, C, nbc * m * n);
+    if (int rc = flush_fills(ctx)) return rc;
+    if (zeroed) {
+        const int rc = zg_hip_bmm_acc(ctx, A, A_shape, B, B_shape, C, C_shape, trans_a, trans_b, lda, ldb, ldc, alpha, 0.f);
+        if (rc) (void)zg_hip_mem_fill(ctx, C, nbc * m * n, 0.f);  // the product was refused: the zeros are still owed
+        return rc;
+    }
     ZG_REQUIRE(A_shape[1] == m, "bmm_acc: A rows %llu != C rows %zu", (unsigned long long)A_shape[1], m);
     ZG_REQUIRE(B_shape[1] == k && B_shape[2] == n, "bmm_acc: B shape does not match [%zu, %zu]", k, n);
     if (nbc == 0) return ZG_HIP_OK;

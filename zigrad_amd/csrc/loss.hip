@@ -664,7 +664,7 @@ ZG_API int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx* ctx, const float* logits, c
 
 ZG_API int zg_hip_smce_label_bwd(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, const float* lse,
                                  float* grad, size_t rows, size_t cols, int accumulate) {
-    ZG_CTX(ctx);
+    ZG_CTX(ctx);  // (a gradient fill that is still waiting is launched here: this form is not the reference's own)
     ZG_REQUIRE(logits && labels && lse && grad, "smce_label_bwd: null pointer");
     if (int rc = check_rows("smce_label_bwd", rows, cols)) return rc;
     const bool aligned = ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
@@ -721,13 +721,20 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
 
 ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* target, float* grad, size_t rows,
                            size_t cols) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
     ZG_REQUIRE(probs && target && grad, "smce_bwd: null pointer");
     if (int rc = check_rows("smce_bwd", rows, cols)) return rc;
+    // the gradient's zero fill (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: then write, not add
+    const bool fresh = absorb_zero_fill(ctx, grad, rows * cols);
+    if (int rc = flush_fills(ctx)) return rc;
     const size_t n = rows * cols;
     const unsigned blocks = smce_bwd_grid(n);
-    hipLaunchKernelGGL(smce_bwd_kernel<true>, dim3(blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad,
-                       n, (float)rows);
+    if (fresh)
+        hipLaunchKernelGGL(smce_bwd_kernel<false>, dim3(blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad, n,
+                           (float)rows);
+    else
+        hipLaunchKernelGGL(smce_bwd_kernel<true>, dim3(blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad, n,
+                           (float)rows);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

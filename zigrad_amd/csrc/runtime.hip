@@ -1024,6 +1024,19 @@ int flush_fills(zg_hip_ctx* ctx) {
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
+bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
+    for (int i = 0; i < ctx->n_pending_fills; i++) {
+        const zg_pending_fill& p = ctx->pending_fills[i];
+        uint32_t bits;
+        memcpy(&bits, &p.value, sizeof(bits));
+        if (p.x == x && p.n == n && bits == 0u) {  // +0.0 only: x + (-0.0) and x differ for x = +0.0
+            for (int j = i + 1; j < ctx->n_pending_fills; j++) ctx->pending_fills[j - 1] = ctx->pending_fills[j];
+            ctx->n_pending_fills--;
+            return true;
+        }
+    }
+    return false;
+}
 }  // namespace zg
 
 ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {

@@ -140,6 +140,15 @@ int zg_hip_div(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_
 int zg_hip_dot(zg_hip_ctx *ctx, const float *x, const float *y, size_t n, float *z);
 int zg_hip_matvec(zg_hip_ctx *ctx, const float *A, const float *x, float *y, size_t m, size_t n, int trans_a,
                   float alpha, float beta);
+/* Timing of the products, for benchmarks (no counterpart in the reference).  While on, the launches of every product
+ * (zg_hip_matmul, zg_hip_bmm_acc, the fused Linear entry points: the product's kernel with whatever its epilogue
+ * carries, plus the reduction or the strips when the product is cut) are bracketed by a pair of events on the
+ * context's stream at the moment they are queued.  zg_hip_gemm_timing(ctx, 1) clears the count and starts,
+ * zg_hip_gemm_timing(ctx, 0) stops; zg_hip_gemm_timing_read waits for the stream and returns the summed time between
+ * the pairs and the number of products.  Nothing is bracketed while a graph is being recorded. */
+int zg_hip_gemm_timing(zg_hip_ctx *ctx, int enable);
+int zg_hip_gemm_timing_read(zg_hip_ctx *ctx, double *total_ms, uint64_t *products);
+
 /* How a product of this shape would be launched by the staged kernels (no counterpart in the reference; for tests
  * and for reading profiles).  out[0] kind: 0 one launch, 1 k cut over several workgroups per tile and the partial
  * tiles added in a fixed order by a second kernel, 2 C cut into a block of whole 256 x 128 tiles plus strips that are
@@ -149,7 +158,20 @@ int zg_hip_matvec(zg_hip_ctx *ctx, const float *A, const float *x, float *y, siz
  * ctx may be null (256 compute units are assumed); nothing is launched. */
 int zg_hip_gemm_plan(zg_hip_ctx *ctx, size_t m, size_t n, size_t k, size_t batches, int64_t *out);
 
-/* row-major C = alpha*op(A)*op(B) + beta*C; C is not read when beta == 0 */
+/* row-major C = alpha*op(A)*op(B) + beta*C; C is not read when beta == 0.
+ * Products that wait.  Two kinds of single (unbatched) product with a dense C (ldc == n) are not launched by the call
+ * that asks for them but by the NEXT call on the context, whatever it is:
+ *   - a layer's forward product, C = A B^T with beta == 0 (x.bmm_acc(W, trans_b), examples/mnist/src/model.zig:107):
+ *     if the next call is zg_hip_add of a row of n values onto C in place (bias.add_(y), :108) the row is added in the
+ *     product's epilogue and the product waits one more call; if the next call is zg_hip_relu_fwd of C in place
+ *     (:38-46) the ReLU is applied in the epilogue too and the product is launched;
+ *   - an input-gradient product, C += A B with beta == 1 onto a C whose zero fill is still waiting (ensure_grad(0) then
+ *     BmmAccBwd, src/ndtensor.zig:221-228, :1107-1109): one following product that touches none of its operands (the
+ *     weight gradient, :1126-1128) is launched ahead of it; if the next call is zg_hip_relu_inplace_bwd on C
+ *     (src/nn/nn.zig:44-50) the mask is applied in the epilogue and the product is launched.
+ * Any other call (a read, a fill, a free, an allocation, another op, zg_hip_sync, the end of a recording) launches the
+ * waiting product first, unchanged.  The values are those of the separate calls, bit for bit: the epilogue does the
+ * same IEEE operations in the same order.  An argument error is reported by the call that asks for the product. */
 int zg_hip_matmul(zg_hip_ctx *ctx, const float *A, const float *B, float *C, size_t m, size_t n, size_t k,
                   int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta);
 /* shapes are host arrays of 3: {batches, rows, cols} of the logical (post-transpose) operands */

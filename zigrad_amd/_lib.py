@@ -17,6 +17,7 @@ LIB_PATH = PKG_DIR / "libzg_hip.so"
 _SCALARS = {
     "int": ctypes.c_int,
     "float": ctypes.c_float,
+    "double": ctypes.c_double,
     "size_t": ctypes.c_size_t,
     "uint64_t": ctypes.c_uint64,
     "uint8_t": ctypes.c_uint8,

@@ -48,6 +48,23 @@ struct zg_pending_fill {
 };
 constexpr int kMaxPendingFills = 16;
 
+// A single (unbatched) product C = alpha op(A) op(B) that has been asked for and not launched yet (gemm.hip).
+struct zg_deferred_gemm {
+    bool active = false;
+    int kind = 0;         // 1: a layer's forward product (A as stored, B transposed); 2: an input-gradient product
+    bool zeroed = false;  // the product took over a waiting zero fill of C (it was asked for as C += ...)
+    const float* A = nullptr;
+    const float* B = nullptr;
+    float* C = nullptr;
+    size_t m = 0, n = 0, k = 0, lda = 0, ldb = 0, ldc = 0;
+    int trans_a = 0, trans_b = 0;
+    float alpha = 1.f;
+    const float* bias = nullptr;  // attached by a following row-broadcast add onto C
+    const float* gate = nullptr;  // attached by a following relu_inplace_bwd on C
+    int relu = 0;                 // attached by a following in-place relu_fwd on C
+    const char* name = "matmul";
+};
+
 struct zg_hip_ctx {
     int device = 0;
     int n_cu = 256;
@@ -100,6 +117,15 @@ struct zg_hip_ctx {
     zg_pending_fill pending_fills[kMaxPendingFills];
     int n_pending_fills = 0;
 
+    // A layer's forward product waits one call for the bias add and the ReLU that the reference's Linear layer issues
+    // right after it (examples/mnist/src/model.zig:104-110, :38-46), and an input-gradient product waits for the
+    // relu_inplace_bwd that masks it (src/nn/nn.zig:44-50), letting one independent product (the weight gradient,
+    // src/ndtensor.zig:1126-1128) pass: what follows is then done in the product's epilogue, the same IEEE operations
+    // in the same order, instead of in one more pass over the output each.  Any other call launches the product as it
+    // is, first thing (ZG_CTX), so no call ever sees memory the product has not reached; fills and a waiting product
+    // never coexist (a fill launches the product first, a product launches the fills first).
+    zg_deferred_gemm deferred;
+
     // launch plans of the staged GEMM kernels, by shape (gemm.hip)
     zg::GemmPlanCache* gemm_plans = nullptr;
 
@@ -118,6 +144,15 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 // matched must still hold what it held then, or the replay would scatter by a stale plan.
 // Launches the fills that are waiting in the context (one kernel for all of them).
 int flush_fills(zg_hip_ctx* ctx);
+// Launches the waiting product, with whatever was attached to it (gemm.hip).
+int flush_deferred_gemm(zg_hip_ctx* ctx);
+// The waiting product, then the waiting fills: what ZG_CTX does before a call's own work.
+int flush_pending(zg_hip_ctx* ctx);
+// A call that may be absorbed by the waiting product: true when it was (then *rc is the call's result and the caller
+// returns it), false when the call has to run as usual.
+bool deferred_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);
+bool deferred_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc);
+bool deferred_take_relu_mask(zg_hip_ctx* ctx, const float* x, const float* x_g, size_t n, int* rc);
 // An op that adds into x[0 .. n) asks whether a fill of exactly that range with +0.0 is still waiting.  If so the fill
 // is dropped and true comes back: the op then writes its result instead of adding it to zeros it would have to read
 // (ensure_grad(0) followed by an accumulating backward op, src/ndtensor.zig:221-228), the same values without the
@@ -183,11 +218,12 @@ inline bool aligned16(const void* p) {
 // First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
 #define ZG_CTX(ctx)                                          \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
-    if ((ctx)->n_pending_fills) {                            \
-        if (int _rc_fill = zg::flush_fills(ctx)) return _rc_fill; \
+    if ((ctx)->n_pending_fills || (ctx)->deferred.active) {  \
+        if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
     }
-// The same for the few calls that leave waiting fills alone: the fills themselves, and allocations (a block that is
-// handed out is free, so no waiting fill names it; a block that is freed goes through ZG_CTX).
+// The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the
+// calls a product may absorb, and cache allocations (a block that is handed out is free, so no waiting fill names it;
+// a block that is freed goes through ZG_CTX).
 #define ZG_CTX_KEEP_FILLS(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.

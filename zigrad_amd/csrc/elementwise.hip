@@ -294,6 +294,8 @@ using namespace zg;
     }
 
 ZG_API int zg_hip_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
+    // a bias row added onto the output of a product that is still waiting becomes part of that product's launch
+    if (ctx && ctx->deferred.active && deferred_take_add(ctx, x, xl, y, yl, z, zl)) return ZG_HIP_OK;
     return binary_op<AddOp>(ctx, "add", x, xl, y, yl, z, zl);
 }
 ZG_API int zg_hip_sub(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
@@ -339,6 +341,9 @@ ZG_API int zg_hip_exp_bwd(zg_hip_ctx* ctx, float* x_g, const float* y, const flo
     return launch_map<ExpBwd, 3>(ctx, x_g, y, x_g, y_g, n);
 }
 ZG_API int zg_hip_relu_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) {
+    // in place on the output of a product that is still waiting: done in that product's epilogue
+    int taken_rc = 0;
+    if (ctx && ctx->deferred.active && deferred_take_relu(ctx, x, y, n, &taken_rc)) return taken_rc;
     ZG_CHECK_N("relu_fwd", n, x, y);
     return launch_map<ReluFwd, 1>(ctx, y, x, nullptr, nullptr, n);
 }
@@ -347,6 +352,9 @@ ZG_API int zg_hip_relu_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, const fl
     return launch_map<ReluBwd, 3>(ctx, x_g, x, x_g, y_g, n);
 }
 ZG_API int zg_hip_relu_inplace_bwd(zg_hip_ctx* ctx, const float* x, float* x_g, size_t n) {
+    // the mask of an input gradient whose product is still waiting: applied in that product's epilogue
+    int taken_rc = 0;
+    if (ctx && ctx->deferred.active && deferred_take_relu_mask(ctx, x, x_g, n, &taken_rc)) return taken_rc;
     ZG_CHECK_N("relu_inplace_bwd", n, x, x_g);
     return launch_map<ReluInplaceBwd, 2>(ctx, x_g, x, x_g, nullptr, n);
 }

@@ -907,9 +907,18 @@ struct GemmPlanKey {
 };
 struct GemmPlanCache {
     std::map<GemmPlanKey, GemmPlan> plans;
+    // zg_hip_gemm_timing: event pairs around every product launched while it is on
+    bool timing = false, in_bracket = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> pairs;
+    size_t used = 0;
 };
 
 void gemm_plans_destroy(zg_hip_ctx* ctx) {
+    if (ctx->gemm_plans)
+        for (auto& pr : ctx->gemm_plans->pairs) {
+            (void)hipEventDestroy(pr.first);
+            (void)hipEventDestroy(pr.second);
+        }
     delete ctx->gemm_plans;
     ctx->gemm_plans = nullptr;
 }
@@ -1091,16 +1100,56 @@ static bool gemm_is_tiny(size_t m, size_t n, size_t k, size_t batches, size_t ld
     return small_ld && ((k <= 256 && blocks <= n_cu) || (k <= 512 && blocks <= 16));
 }
 
-static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
-                         size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta,
-                         size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk,
-                         int depth = 0, const GemmExtras* extras = nullptr) {
-    if (m == 0 || n == 0 || batches == 0) return ZG_HIP_OK;
+static int gemm_validate(const char* name, const float* A, const float* B, const float* C, size_t m, size_t n, size_t k,
+                         int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc) {
     ZG_REQUIRE(A && B && C, "%s: null pointer", name);
     // cblas argument rules for row-major storage
     ZG_REQUIRE(lda >= (trans_a ? m : k) && lda >= 1, "%s: lda %zu too small", name, lda);
     ZG_REQUIRE(ldb >= (trans_b ? k : n) && ldb >= 1, "%s: ldb %zu too small", name, ldb);
     ZG_REQUIRE(ldc >= n, "%s: ldc %zu < n %zu", name, ldc, n);
+    return ZG_HIP_OK;
+}
+
+static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m,
+                              size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha,
+                              float beta, size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk,
+                              size_t c_chunk, int depth, const GemmExtras* extras);
+
+// Every product goes through here.  With zg_hip_gemm_timing on, the launches of one product (its kernel, and the
+// reduction or the strips when it is cut) are bracketed by a pair of events on the context's stream.
+static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
+                         size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta,
+                         size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk,
+                         int depth = 0, const GemmExtras* extras = nullptr) {
+    GemmPlanCache* pc = ctx->gemm_plans;
+    const bool bracket = pc && pc->timing && !pc->in_bracket && !ctx->capturing && m > 0 && n > 0 && batches > 0;
+    if (!bracket)
+        return gemm_dispatch_body(ctx, name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, batches, nba, nbb,
+                                  a_chunk, b_chunk, c_chunk, depth, extras);
+    if (pc->used == pc->pairs.size()) {
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        ZG_HIP_TRY(hipEventCreate(&e0));
+        ZG_HIP_TRY(hipEventCreate(&e1));
+        pc->pairs.emplace_back(e0, e1);
+    }
+    auto& pr = pc->pairs[pc->used];
+    ZG_HIP_TRY(hipEventRecord(pr.first, ctx->stream));
+    pc->in_bracket = true;
+    const int rc = gemm_dispatch_body(ctx, name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, batches, nba,
+                                      nbb, a_chunk, b_chunk, c_chunk, depth, extras);
+    pc->in_bracket = false;
+    if (rc) return rc;
+    ZG_HIP_TRY(hipEventRecord(pr.second, ctx->stream));
+    pc->used++;
+    return ZG_HIP_OK;
+}
+
+static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m,
+                              size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha,
+                              float beta, size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk,
+                              size_t c_chunk, int depth, const GemmExtras* extras) {
+    if (m == 0 || n == 0 || batches == 0) return ZG_HIP_OK;
+    if (int rc = gemm_validate(name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc)) return rc;
     ZG_REQUIRE(nba >= 1 && nbb >= 1, "%s: zero operand batches", name);
     if (batches > 65535) {
         // the batch index is the grid's z dimension (at most 65535): longer batches go in runs.  The operand batch
@@ -1353,6 +1402,31 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* A, float* B
 
 using namespace zg;
 
+ZG_API int zg_hip_gemm_timing(zg_hip_ctx* ctx, int enable) {
+    ZG_CTX(ctx);
+    if (!ctx->gemm_plans) ctx->gemm_plans = new GemmPlanCache();
+    if (enable) ctx->gemm_plans->used = 0;
+    ctx->gemm_plans->timing = enable != 0;
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_gemm_timing_read(zg_hip_ctx* ctx, double* total_ms, uint64_t* products) {
+    ZG_CTX(ctx);
+    ZG_NOT_CAPTURING(ctx, "gemm_timing_read");
+    ZG_REQUIRE(total_ms && products, "gemm_timing_read: null output");
+    *total_ms = 0.0;
+    *products = 0;
+    if (!ctx->gemm_plans) return ZG_HIP_OK;
+    ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    for (size_t i = 0; i < ctx->gemm_plans->used; i++) {
+        float ms = 0.f;
+        ZG_HIP_TRY(hipEventElapsedTime(&ms, ctx->gemm_plans->pairs[i].first, ctx->gemm_plans->pairs[i].second));
+        *total_ms += (double)ms;
+    }
+    *products = ctx->gemm_plans->used;
+    return ZG_HIP_OK;
+}
+
 ZG_API int zg_hip_gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_t batches, int64_t* out) {
     ZG_REQUIRE(out != nullptr, "gemm_plan: null output");
     ZG_REQUIRE(m > 0 && n > 0 && k > 0 && batches > 0, "gemm_plan: empty product");
@@ -1367,20 +1441,138 @@ ZG_API int zg_hip_gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_
     return ZG_HIP_OK;
 }
 
-ZG_API int zg_hip_matmul(zg_hip_ctx* ctx, const float* A, const float* B, float* C, size_t m, size_t n, size_t k,
-                         int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
-    ZG_CTX_KEEP_FILLS(ctx);
-    // C += ... into a C whose zero fill has not been launched yet: write instead (no fill, no read of C)
-    const bool zeroed = beta == 1.f && C && ldc == n && k > 0 && alpha != 0.f && absorb_zero_fill(ctx, C, m * n);
-    if (int rc = flush_fills(ctx)) return rc;
-    const int rc = gemm_dispatch(ctx, "matmul", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, zeroed ? 0.f : beta,
-                                 1, 1, 1, 0, 0, 0);
-    if (rc && zeroed) (void)zg_hip_mem_fill(ctx, C, m * n, 0.f);  // the product was refused: the zeros are still owed
+// ------------------------------------------------------------------------------------------------
+// Products that wait for what follows them (see zg_hip_ctx::deferred)
+// ------------------------------------------------------------------------------------------------
+namespace zg {
+
+struct ByteRange {
+    const char* lo;
+    const char* hi;
+};
+static ByteRange operand_range(const float* p, size_t rows, size_t cols, size_t ld) {
+    const char* lo = reinterpret_cast<const char*>(p);
+    return ByteRange{lo, lo + ((rows - 1) * ld + cols) * sizeof(float)};
+}
+static bool ranges_meet(ByteRange a, ByteRange b) {
+    return a.lo < b.hi && b.lo < a.hi;
+}
+
+int flush_deferred_gemm(zg_hip_ctx* ctx) {
+    zg_deferred_gemm d = ctx->deferred;
+    if (!d.active) return ZG_HIP_OK;
+    ctx->deferred.active = false;
+    GemmExtras ex{d.bias, d.gate, d.relu};
+    const bool any = d.bias || d.gate || d.relu;
+    const int rc = gemm_dispatch(ctx, d.name, d.A, d.B, d.C, d.m, d.n, d.k, d.trans_a, d.trans_b, d.lda, d.ldb, d.ldc, d.alpha,
+                                 0.f, 1, 1, 1, 0, 0, 0, 0, any ? &ex : nullptr);
+    if (rc && d.zeroed) (void)zg_hip_mem_fill(ctx, d.C, d.m * d.n, 0.f);  // the product failed: the zeros are still owed
     return rc;
 }
 
-// y = act(x . w^T + bias): one launch where the product is one launch (the bias add and the ReLU ride in the GEMM
-// epilogue or in the split-k reduction), with the arithmetic of the three separate ops.
+// bias.add_(y): z = x + y over the product's output, one operand the output itself, the other a row of n values
+bool deferred_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl) {
+    zg_deferred_gemm& d = ctx->deferred;
+    if (!d.active || d.kind != 1 || d.bias || d.relu || z != d.C || zl != d.m * d.n || d.n == zl) return false;
+    const float* row = nullptr;
+    if (y == d.C && yl == zl && xl == d.n) row = x;
+    else if (x == d.C && xl == zl && yl == d.n) row = y;
+    if (!row) return false;
+    if (ranges_meet(operand_range(row, 1, d.n, d.n), operand_range(d.C, d.m, d.n, d.ldc))) return false;
+    d.bias = row;
+    return true;
+}
+
+// relu_(y) in place on the product's output: the last thing a layer's forward pass does, so the product goes out
+bool deferred_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc) {
+    zg_deferred_gemm& d = ctx->deferred;
+    if (!d.active || d.kind != 1 || d.relu || x != d.C || y != d.C || n != d.m * d.n) return false;
+    d.relu = 1;
+    *rc = flush_deferred_gemm(ctx);
+    return true;
+}
+
+// relu_inplace_bwd(x, x_g) on the product's output x_g: x_g = 0 where x <= 0, x laid out like the output
+bool deferred_take_relu_mask(zg_hip_ctx* ctx, const float* x, const float* x_g, size_t n, int* rc) {
+    zg_deferred_gemm& d = ctx->deferred;
+    if (!d.active || d.kind != 2 || d.gate || x_g != d.C || n != d.m * d.n || !x) return false;
+    if (ranges_meet(operand_range(x, d.m, d.n, d.n), operand_range(d.C, d.m, d.n, d.ldc))) return false;
+    d.gate = x;
+    *rc = flush_deferred_gemm(ctx);
+    return true;
+}
+
+// matmul and bmm_acc.  In order: a waiting zero fill of exactly C turns C += ... into C = ...; the other fills go out;
+// a product that is already waiting either lets this one pass (it waits for its mask and this one touches none of
+// its operands: the weight-gradient product after the input-gradient product) or goes out first; then this product
+// waits itself if it is a layer's forward product or an input-gradient product, or is launched.
+static int gemm_entry(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
+                      size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta,
+                      size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk, size_t c_chunk) {
+    const bool plain = batches == 1 && m > 0 && n > 0 && k > 0 && alpha != 0.f && A && B && C && ldc == n;
+    const bool zeroed = beta == 1.f && C && ldc == n && k > 0 && alpha != 0.f && m > 0 && n > 0 && batches > 0 &&
+                        absorb_zero_fill(ctx, C, batches * m * n);
+    const float beta_eff = zeroed ? 0.f : beta;
+    if (int rc = flush_fills(ctx)) return rc;
+    auto launch_now = [&]() {
+        const int rc = gemm_dispatch(ctx, name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta_eff, batches, nba,
+                                     nbb, a_chunk, b_chunk, c_chunk);
+        if (rc && zeroed) (void)zg_hip_mem_fill(ctx, C, batches * m * n, 0.f);  // refused: the zeros are still owed
+        return rc;
+    };
+    if (ctx->deferred.active) {
+        const zg_deferred_gemm& d = ctx->deferred;
+        bool pass = false;
+        if (d.kind == 2 && plain && gemm_validate(name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc) == ZG_HIP_OK) {
+            const ByteRange dA = operand_range(d.A, d.trans_a ? d.k : d.m, d.trans_a ? d.m : d.k, d.lda);
+            const ByteRange dB = operand_range(d.B, d.trans_b ? d.n : d.k, d.trans_b ? d.k : d.n, d.ldb);
+            const ByteRange dC = operand_range(d.C, d.m, d.n, d.ldc);
+            const ByteRange tA = operand_range(A, trans_a ? k : m, trans_a ? m : k, lda);
+            const ByteRange tB = operand_range(B, trans_b ? n : k, trans_b ? k : n, ldb);
+            const ByteRange tC = operand_range(C, m, n, ldc);
+            pass = !ranges_meet(tC, dA) && !ranges_meet(tC, dB) && !ranges_meet(tC, dC) && !ranges_meet(dC, tA) &&
+                   !ranges_meet(dC, tB);
+        }
+        if (pass) return launch_now();
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
+    }
+    const int kind = (!trans_a && trans_b) ? 1 : ((!trans_a && !trans_b && zeroed) ? 2 : 0);
+    if (plain && beta_eff == 0.f && kind != 0) {
+        if (int rc = gemm_validate(name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc)) {
+            if (zeroed) (void)zg_hip_mem_fill(ctx, C, m * n, 0.f);
+            return rc;
+        }
+        zg_deferred_gemm& d = ctx->deferred;
+        d = zg_deferred_gemm{};
+        d.active = true;
+        d.kind = kind;
+        d.zeroed = zeroed;
+        d.A = A;
+        d.B = B;
+        d.C = C;
+        d.m = m;
+        d.n = n;
+        d.k = k;
+        d.lda = lda;
+        d.ldb = ldb;
+        d.ldc = ldc;
+        d.trans_a = trans_a;
+        d.trans_b = trans_b;
+        d.alpha = alpha;
+        d.name = name;
+        return ZG_HIP_OK;
+    }
+    return launch_now();
+}
+
+}  // namespace zg
+
+ZG_API int zg_hip_matmul(zg_hip_ctx* ctx, const float* A, const float* B, float* C, size_t m, size_t n, size_t k,
+                         int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
+    ZG_CTX_KEEP_FILLS(ctx);
+    return gemm_entry(ctx, "matmul", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, 1, 1, 1, 0, 0, 0);
+}
+
 ZG_API int zg_hip_linear_fwd(zg_hip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, size_t batch,
                              size_t fan_in, size_t fan_out, int relu) {
     ZG_CTX(ctx);
@@ -1469,21 +1661,11 @@ ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_sha
     ZG_REQUIRE(A_shape && B_shape && C_shape, "bmm_acc: null shape");
     const size_t nba = A_shape[0], nbb = B_shape[0], nbc = C_shape[0];
     const size_t m = C_shape[1], n = C_shape[2], k = A_shape[2];
-    // C += ... into a C whose zero fill has not been launched yet (ensure_grad(0) then BmmAccBwd,
-    // src/ndtensor.zig:221-228, :1092-1136): write instead (no fill, no read of C)
-    const bool zeroed = beta == 1.f && C && ldc == n && k > 0 && alpha != 0.f && absorb_zero_fill(ctx, C, nbc * m * n);
-    if (int rc = flush_fills(ctx)) return rc;
-    if (zeroed) {
-        const int rc = zg_hip_bmm_acc(ctx, A, A_shape, B, B_shape, C, C_shape, trans_a, trans_b, lda, ldb, ldc, alpha, 0.f);
-        if (rc) (void)zg_hip_mem_fill(ctx, C, nbc * m * n, 0.f);  // the product was refused: the zeros are still owed
-        return rc;
-    }
     ZG_REQUIRE(A_shape[1] == m, "bmm_acc: A rows %llu != C rows %zu", (unsigned long long)A_shape[1], m);
     ZG_REQUIRE(B_shape[1] == k && B_shape[2] == n, "bmm_acc: B shape does not match [%zu, %zu]", k, n);
-    if (nbc == 0) return ZG_HIP_OK;
-    ZG_REQUIRE(nba >= 1 && nbb >= 1, "bmm_acc: zero operand batches");
-    return gemm_dispatch(ctx, "bmm_acc", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, nbc, nba, nbb,
-                         A_shape[1] * A_shape[2], B_shape[1] * B_shape[2], C_shape[1] * C_shape[2]);
+    if (nbc > 0) ZG_REQUIRE(nba >= 1 && nbb >= 1, "bmm_acc: zero operand batches");
+    return gemm_entry(ctx, "bmm_acc", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, nbc, nba ? nba : 1,
+                      nbb ? nbb : 1, A_shape[1] * A_shape[2], B_shape[1] * B_shape[2], C_shape[1] * C_shape[2]);
 }
 
 ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float* y, size_t m, size_t n, int trans_a,

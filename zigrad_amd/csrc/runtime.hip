@@ -663,7 +663,7 @@ ZG_API int zg_hip_total_memory(zg_hip_ctx* ctx, size_t* bytes) {
 
 ZG_API void* zg_hip_stream(zg_hip_ctx* ctx) {
     if (!ctx) return nullptr;
-    (void)flush_fills(ctx);  // work the caller queues on the stream itself must find every fill already there
+    (void)flush_pending(ctx);  // work the caller queues on the stream itself must find everything already there
     return (void*)ctx->stream;
 }
 
@@ -804,6 +804,8 @@ ZG_API int zg_hip_cache_configure(zg_hip_ctx* ctx, size_t small_pool_bytes, size
 
 ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uint64_t* block) {
     ZG_CTX_KEEP_FILLS(ctx);
+    if (ctx->deferred.active)  // what a waiting product waits for comes right after it, not after an allocation
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
     ZG_REQUIRE(out != nullptr && block != nullptr, "mem_cache_alloc: null output");
     *out = nullptr;
     *block = 0;
@@ -1024,6 +1026,12 @@ int flush_fills(zg_hip_ctx* ctx) {
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
+int flush_pending(zg_hip_ctx* ctx) {
+    if (ctx->deferred.active)
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
+    return flush_fills(ctx);
+}
+
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
     for (int i = 0; i < ctx->n_pending_fills; i++) {
         const zg_pending_fill& p = ctx->pending_fills[i];
@@ -1041,6 +1049,8 @@ bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
 
 ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {
     ZG_CTX_KEEP_FILLS(ctx);
+    if (ctx->deferred.active)  // a waiting product goes first: the fill may be of one of its operands
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x != nullptr, "mem_fill: null pointer");
     // The fill waits for the next call that is not a fill.  Two waiting fills never overlap (workgroups of one launch

@@ -439,6 +439,16 @@ class HipDevice:
         """How the staged GEMM kernels would launch this product (see zg_hip_gemm_plan)."""
         return gemm_plan(m, n, k, batches, self)
 
+    def gemm_timing(self, on: bool) -> None:
+        """Start (clearing the count) or stop bracketing every product's launches with events on the stream."""
+        self._call("zg_hip_gemm_timing", int(bool(on)))
+
+    def gemm_timing_read(self) -> tuple[float, int]:
+        """(summed milliseconds between the event pairs, number of products) since timing was last started."""
+        ms, cnt = ctypes.c_double(), ctypes.c_uint64()
+        self._call("zg_hip_gemm_timing_read", ctypes.byref(ms), ctypes.byref(cnt))
+        return ms.value, cnt.value
+
     def plan_cache_stats(self) -> dict:
         """Calls served from a kept destination ordering / orderings computed and kept (pinned index arrays only)."""
         h, b = ctypes.c_uint64(), ctypes.c_uint64()

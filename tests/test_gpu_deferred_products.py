@@ -183,3 +183,73 @@ def test_an_input_gradient_waits_only_for_products_that_leave_it_alone(hip):
     assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
     for b in (gyb, wb, ab, gx, out):
         hip.mem_free(b)
+
+
+@pytest.mark.parametrize("shape", [(64, 128, 64), (256, 512, 384), (1024, 1024, 1024)])
+def test_frees_of_the_backward_pass_do_not_disturb_a_waiting_input_gradient(hip, shape):
+    """The reference frees a layer's output and its gradient as soon as the layer's backward has run, which is before the
+    mask of the input gradient arrives: blocks that hold an operand of the waiting product go back to the pool when the
+    product has been launched, others at once; the pool ends where it started."""
+    B, I, O = shape
+    r = np.random.default_rng(B + I + O)
+    gy = r.standard_normal((B, O)).astype(np.float32)
+    w = (r.standard_normal((O, I)) / np.sqrt(O)).astype(np.float32)
+    act = np.maximum(r.standard_normal((B, I)), 0.0).astype(np.float32)
+    wb, ab = hip.from_numpy(w), hip.from_numpy(act)
+    gw0 = r.standard_normal((O, I)).astype(np.float32)
+    outs = []
+    in_use0 = hip.cache_stats()["bytes_in_use"]
+    for eager in (False, True):
+        step = hip.sync if eager else (lambda: None)
+        y = hip.mem_cache_alloc(F32, B * O)            # the layer's output: freed after the layer's backward
+        g = hip.mem_cache_alloc(F32, B * O)            # its gradient: an operand of both products
+        hip.mem_transfer(gy, g, "HtoD")
+        gw = hip.from_numpy(gw0)
+        gx = hip.mem_cache_alloc(F32, B * I)
+        hip.mem_fill(gx, 0.0)
+        step()
+        hip.dispatch("bmm_acc", A=g, B=wb, C=gx, A_shape=[1, B, O], B_shape=[1, O, I], C_shape=[1, B, I], trans_a=False,
+                     trans_b=False, lda=O, ldb=I, ldc=I, alpha=1.0, beta=1.0)
+        step()
+        hip.dispatch("bmm_acc", A=g, B=ab, C=gw, A_shape=[1, O, B], B_shape=[1, B, I], C_shape=[1, O, I], trans_a=True,
+                     trans_b=False, lda=O, ldb=I, ldc=I, alpha=1.0, beta=1.0)
+        step()
+        hip.mem_cache_free(y)
+        hip.mem_cache_free(g)
+        step()
+        hip.dispatch("relu_inplace_bwd", x=ab, x_g=gx)
+        step()
+        # memory handed out now must not be what the waiting product still had to read
+        scratch = hip.mem_cache_alloc(F32, B * O)
+        hip.mem_fill(scratch, 123.0)
+        outs.append((hip.to_numpy(gx).reshape(B, I), hip.to_numpy(gw).reshape(O, I)))
+        hip.mem_cache_free(scratch)
+        hip.mem_cache_free(gx)
+        hip.mem_free(gw)
+    hip.sync()
+    assert hip.cache_stats()["bytes_in_use"] == in_use0
+    (gx_a, gw_a), (gx_b, gw_b) = outs
+    assert np.array_equal(gx_a, gx_b) and np.array_equal(gw_a, gw_b)
+    want = np.where(act > 0, gy.astype(np.float64) @ w.astype(np.float64), 0.0)
+    assert np.linalg.norm(gx_a - want) <= 1e-5 * (np.linalg.norm(want) + 1e-3)
+    for b in (wb, ab):
+        hip.mem_free(b)
+
+
+def test_giving_a_block_back_twice_while_its_free_waits_is_refused(hip):
+    B, I, O = 64, 32, 48
+    r = np.random.default_rng(3)
+    g = hip.mem_cache_alloc(F32, B * O)
+    hip.mem_transfer(r.standard_normal(B * O).astype(np.float32), g, "HtoD")
+    wb = hip.from_numpy(r.standard_normal(O * I).astype(np.float32))
+    gx = hip.mem_cache_alloc(F32, B * I)
+    hip.mem_fill(gx, 0.0)
+    hip.dispatch("bmm_acc", A=g, B=wb, C=gx, A_shape=[1, B, O], B_shape=[1, O, I], C_shape=[1, B, I], trans_a=False,
+                 trans_b=False, lda=O, ldb=I, ldc=I, alpha=1.0, beta=1.0)
+    ptr, block = g.ptr, g.block
+    hip.mem_cache_free(g)
+    with pytest.raises(ZgHipError):
+        hip._call("zg_hip_mem_cache_free", ptr, block)
+    hip.sync()
+    hip.mem_cache_free(gx)
+    hip.mem_free(wb)

@@ -125,6 +125,14 @@ struct zg_hip_ctx {
     // is, first thing (ZG_CTX), so no call ever sees memory the product has not reached; fills and a waiting product
     // never coexist (a fill launches the product first, a product launches the fills first).
     zg_deferred_gemm deferred;
+    // Cache blocks that were given back while a waiting input-gradient product still names them as operands (the
+    // reference frees a node's gradient as soon as its backward has run, src/ndtensor.zig eager teardown): they return
+    // to the pool right after the product is launched.
+    struct {
+        void* ptr;
+        uint64_t block;
+    } deferred_frees[4];
+    int n_deferred_frees = 0;
 
     // launch plans of the staged GEMM kernels, by shape (gemm.hip)
     zg::GemmPlanCache* gemm_plans = nullptr;
@@ -146,6 +154,8 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 int flush_fills(zg_hip_ctx* ctx);
 // Launches the waiting product, with whatever was attached to it (gemm.hip).
 int flush_deferred_gemm(zg_hip_ctx* ctx);
+// Returns to the pools the blocks whose free waited for the product (runtime.hip); called once it is launched.
+void run_deferred_frees(zg_hip_ctx* ctx);
 // The waiting product, then the waiting fills: what ZG_CTX does before a call's own work.
 int flush_pending(zg_hip_ctx* ctx);
 // A call that may be absorbed by the waiting product: true when it was (then *rc is the call's result and the caller

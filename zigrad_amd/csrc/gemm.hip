@@ -1467,6 +1467,7 @@ int flush_deferred_gemm(zg_hip_ctx* ctx) {
     const int rc = gemm_dispatch(ctx, d.name, d.A, d.B, d.C, d.m, d.n, d.k, d.trans_a, d.trans_b, d.lda, d.ldb, d.ldc, d.alpha,
                                  0.f, 1, 1, 1, 0, 0, 0, 0, any ? &ex : nullptr);
     if (rc && d.zeroed) (void)zg_hip_mem_fill(ctx, d.C, d.m * d.n, 0.f);  // the product failed: the zeros are still owed
+    run_deferred_frees(ctx);  // blocks that hold its operands and were given back while it waited
     return rc;
 }
 

@@ -829,21 +829,69 @@ ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uin
     return ZG_HIP_OK;
 }
 
+static void release_block(zg_hip_ctx* ctx, Block* b) {
+    // While recording, the block goes back to the pool like any other, so a later allocation of the same recording
+    // may reuse it (the graph keeps the stream's order); its range is noted, and whatever part of the noted ranges is
+    // free when the recording ends stays with the graph.  Outside a recording, stream order makes reuse safe: a
+    // later op that receives this block runs after every op already enqueued on the same stream.
+    if (ctx->capturing) ctx->capture_touched.push_back({b->ptr, b->size});
+    b->pool->release(b);
+}
+
+namespace zg {
+void run_deferred_frees(zg_hip_ctx* ctx) {
+    const int n = ctx->n_deferred_frees;
+    ctx->n_deferred_frees = 0;
+    for (int i = 0; i < n; i++) release_block(ctx, (Block*)(uintptr_t)ctx->deferred_frees[i].block);
+}
+}  // namespace zg
+
 ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
-    ZG_CTX(ctx);
-    if (!ptr || block == 0) return ZG_HIP_OK;  // views and empty data: src/allocators/caching_allocator.zig:111-112
+    ZG_CTX_KEEP_FILLS(ctx);
+    if (ctx->n_pending_fills)  // a fill of the block that is given back must not land on its next owner
+        if (int rc = flush_fills(ctx)) return rc;
+    if (!ptr || block == 0) {  // views and empty data: src/allocators/caching_allocator.zig:111-112
+        if (ctx->deferred.active) return flush_deferred_gemm(ctx);
+        return ZG_HIP_OK;
+    }
     Block* b = (Block*)(uintptr_t)block;
     BlockPool* pool = nullptr;
     for (BlockPool* p : {ctx->small_pool, ctx->large_pool})
         if (p && p->owns_live(b, ptr)) pool = p;
     ZG_REQUIRE(pool != nullptr, "mem_cache_free: %p with handle %llx is not a live block of this context's pools", ptr,
                (unsigned long long)block);
-    // While recording, the block goes back to the pool like any other, so a later allocation of the same recording
-    // may reuse it (the graph keeps the stream's order); its range is noted, and whatever part of the noted ranges is
-    // free when the recording ends stays with the graph.  Outside a recording, stream order makes reuse safe: a
-    // later op that receives this block runs after every op already enqueued on the same stream.
-    if (ctx->capturing) ctx->capture_touched.push_back({b->ptr, b->size});
-    pool->release(b);
+    if (ctx->deferred.active) {
+        // An input-gradient product that waits for its mask outlives the frees of the backward pass it belongs to
+        // (the layer's output, the output gradient).  A block none of its operands lies in goes back at once; one that
+        // holds an operand goes back when the product has been launched.
+        const zg_deferred_gemm& d = ctx->deferred;
+        bool keep_waiting = d.kind == 2;
+        for (int i = 0; i < ctx->n_deferred_frees; i++)
+            ZG_REQUIRE(ctx->deferred_frees[i].block != block, "mem_cache_free: %p was already given back", ptr);
+        if (keep_waiting) {
+            const char *lo = b->ptr, *hi = b->ptr + b->size;
+            auto meets = [&](const float* p, size_t rows, size_t cols, size_t ld) {
+                const char* plo = (const char*)p;
+                const char* phi = plo + ((rows - 1) * ld + cols) * sizeof(float);
+                return plo < hi && lo < phi;
+            };
+            const bool operand = meets(d.A, d.trans_a ? d.k : d.m, d.trans_a ? d.m : d.k, d.lda) ||
+                                 meets(d.B, d.trans_b ? d.n : d.k, d.trans_b ? d.k : d.n, d.ldb) ||
+                                 meets(d.C, d.m, d.n, d.ldc);
+            if (!operand) {
+                release_block(ctx, b);
+                return ZG_HIP_OK;
+            }
+            if (ctx->n_deferred_frees < 4) {
+                ctx->deferred_frees[ctx->n_deferred_frees].ptr = ptr;
+                ctx->deferred_frees[ctx->n_deferred_frees].block = block;
+                ctx->n_deferred_frees++;
+                return ZG_HIP_OK;
+            }
+        }
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
+    }
+    release_block(ctx, b);
     return ZG_HIP_OK;
 }
 

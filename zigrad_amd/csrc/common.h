@@ -65,6 +65,22 @@ struct zg_deferred_gemm {
     const char* name = "matmul";
 };
 
+// Optimizer steps of small tensors that have been asked for and not launched yet (optim.hip).
+constexpr int kMaxPendingSteps = 16;
+struct zg_pending_steps {
+    int count = 0;
+    int kind = 0;  // 0 SGD, 1 Adam with lr_t by value, 2 Adam with lr_t read from memory when the kernel runs
+    float* p[kMaxPendingSteps];
+    float* g[kMaxPendingSteps];
+    float* m[kMaxPendingSteps];
+    float* v[kMaxPendingSteps];
+    size_t n[kMaxPendingSteps];
+    float lr_t[kMaxPendingSteps];            // kind 1
+    const float* lr_t_mem[kMaxPendingSteps]; // kind 2
+    float lr = 0.f, b1 = 0.f, b2 = 0.f, eps = 0.f, max_norm = 0.f, delta = 0.f;
+    int clip = 0;
+};
+
 struct zg_hip_ctx {
     int device = 0;
     int n_cu = 256;
@@ -134,6 +150,11 @@ struct zg_hip_ctx {
     } deferred_frees[4];
     int n_deferred_frees = 0;
 
+    // Optimizer steps of tensors of up to 2^20 elements wait here while the calls that follow are more optimizer steps
+    // with the same settings (Optimizer.step() walks its parameter list, src/nn/optim.zig:100-122, :177-234) and then
+    // leave in the two launches of the parameter-list kernels instead of one to three launches each; same values.
+    zg_pending_steps steps;
+
     // launch plans of the staged GEMM kernels, by shape (gemm.hip)
     zg::GemmPlanCache* gemm_plans = nullptr;
 
@@ -154,6 +175,8 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 int flush_fills(zg_hip_ctx* ctx);
 // Launches the waiting product, with whatever was attached to it (gemm.hip).
 int flush_deferred_gemm(zg_hip_ctx* ctx);
+// Launches the optimizer steps that are waiting (optim.hip).
+int flush_steps(zg_hip_ctx* ctx);
 // Returns to the pools the blocks whose free waited for the product (runtime.hip); called once it is launched.
 void run_deferred_frees(zg_hip_ctx* ctx);
 // The waiting product, then the waiting fills: what ZG_CTX does before a call's own work.
@@ -228,7 +251,7 @@ inline bool aligned16(const void* p) {
 // First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
 #define ZG_CTX(ctx)                                          \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
-    if ((ctx)->n_pending_fills || (ctx)->deferred.active) {  \
+    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->steps.count) {  \
         if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
     }
 // The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the

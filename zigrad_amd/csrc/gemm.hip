@@ -1515,6 +1515,8 @@ static int gemm_entry(zg_hip_ctx* ctx, const char* name, const float* A, const f
                         absorb_zero_fill(ctx, C, batches * m * n);
     const float beta_eff = zeroed ? 0.f : beta;
     if (int rc = flush_fills(ctx)) return rc;
+    if (ctx->steps.count)
+        if (int rc = flush_steps(ctx)) return rc;
     auto launch_now = [&]() {
         const int rc = gemm_dispatch(ctx, name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta_eff, batches, nba,
                                      nbb, a_chunk, b_chunk, c_chunk);

@@ -726,7 +726,7 @@ ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* tar
     if (int rc = check_rows("smce_bwd", rows, cols)) return rc;
     // the gradient's zero fill (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: then write, not add
     const bool fresh = absorb_zero_fill(ctx, grad, rows * cols);
-    if (int rc = flush_fills(ctx)) return rc;
+    if (int rc = flush_pending(ctx)) return rc;
     const size_t n = rows * cols;
     const unsigned blocks = smce_bwd_grid(n);
     if (fresh)

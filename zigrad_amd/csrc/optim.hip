@@ -216,11 +216,8 @@ static int update_grid(zg_hip_ctx* ctx, size_t n) {
 
 using namespace zg;
 
-ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n, float lr, int clip, float max_norm,
-                           float delta) {
-    ZG_CTX(ctx);
-    if (n == 0) return ZG_HIP_OK;
-    ZG_REQUIRE(param && grad, "sgd_step: null pointer");
+static int sgd_launch(zg_hip_ctx* ctx, float* param, float* grad, size_t n, float lr, int clip, float max_norm,
+                      float delta) {
     float* factor = ctx->scalar_slot + 1;
     if (clip && n <= kFlatSingleMax) {
         hipLaunchKernelGGL((clipped_update_small_kernel<false>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, param, grad,
@@ -266,14 +263,106 @@ static int adam_launch(zg_hip_ctx* ctx, float* param, float* grad, float* m, flo
     return ZG_HIP_OK;
 }
 
+constexpr size_t kMultiBigMax = (size_t)1 << 20;
+static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_tensors, float* const* params,
+                      float* const* grads, float* const* ms, float* const* vs, const size_t* lens, const float* lr_t,
+                      int lr_t_in_memory, float lr, float beta1, float beta2, float epsilon, int clip, float max_norm,
+                      float delta, int zero_grads);
+
+namespace zg {
+// The waiting steps: one of them alone takes the per-tensor launches it would have taken, several take the
+// parameter-list kernels (the same arithmetic per element and the same norm trees: the values do not depend on which).
+int flush_steps(zg_hip_ctx* ctx) {
+    zg_pending_steps q = ctx->steps;
+    ctx->steps.count = 0;
+    if (q.count == 0) return ZG_HIP_OK;
+    if (q.count == 1) {
+        if (q.kind == 0) return sgd_launch(ctx, q.p[0], q.g[0], q.n[0], q.lr, q.clip, q.max_norm, q.delta);
+        return adam_launch(ctx, q.p[0], q.g[0], q.m[0], q.v[0], q.n[0], q.lr_t[0], q.kind == 2 ? q.lr_t_mem[0] : nullptr, q.b1,
+                           q.b2, q.eps, q.clip, q.max_norm, q.delta);
+    }
+    if (q.kind == 2) {
+        // lr_t read from memory: the list kernels take one base pointer and index it, so the tensors go one by one
+        // unless their lr_t slots are consecutive floats
+        bool consecutive = true;
+        for (int i = 1; i < q.count; i++) consecutive = consecutive && q.lr_t_mem[i] == q.lr_t_mem[0] + i;
+        if (!consecutive) {
+            for (int i = 0; i < q.count; i++)
+                if (int rc = adam_launch(ctx, q.p[i], q.g[i], q.m[i], q.v[i], q.n[i], 0.f, q.lr_t_mem[i], q.b1, q.b2, q.eps,
+                                         q.clip, q.max_norm, q.delta))
+                    return rc;
+            return ZG_HIP_OK;
+        }
+        return step_multi(ctx, "adam_step_at", true, (size_t)q.count, q.p, q.g, q.m, q.v, q.n, q.lr_t_mem[0], 1, 0.f, q.b1, q.b2,
+                          q.eps, q.clip, q.max_norm, q.delta, 0);
+    }
+    return step_multi(ctx, q.kind ? "adam_step" : "sgd_step", q.kind != 0, (size_t)q.count, q.p, q.g, q.m, q.v, q.n, q.lr_t, 0,
+                      q.lr, q.b1, q.b2, q.eps, q.clip, q.max_norm, q.delta, 0);
+}
+}  // namespace zg
+
+// One optimizer step of one tensor.  Up to 2^20 elements it joins the waiting steps when it has their settings and names
+// none of their tensors (otherwise they are sent first); a larger tensor is launched at once, ahead of waiting steps
+// that do not name it.
+static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, float* m, float* v, size_t n, float lr,
+                      float lr_t, const float* lr_t_mem, float b1, float b2, float eps, int clip, float max_norm,
+                      float delta) {
+    if (ctx->deferred.active || ctx->n_pending_fills) {  // the gradients come from them
+        if (ctx->deferred.active)
+            if (int rc = flush_deferred_gemm(ctx)) return rc;
+        if (int rc = flush_fills(ctx)) return rc;
+    }
+    zg_pending_steps& q = ctx->steps;
+    bool named = false;
+    for (int i = 0; i < q.count; i++)
+        named = named || q.p[i] == param || q.g[i] == grad || (kind && (q.m[i] == m || q.v[i] == v));
+    const bool same = q.count == 0 || (q.kind == kind && q.clip == clip && q.max_norm == max_norm && q.delta == delta &&
+                                       (kind ? (q.b1 == b1 && q.b2 == b2 && q.eps == eps) : q.lr == lr));
+    if (n > kMultiBigMax) {
+        if (named)
+            if (int rc = flush_steps(ctx)) return rc;
+        if (kind == 0) return sgd_launch(ctx, param, grad, n, lr, clip, max_norm, delta);
+        return adam_launch(ctx, param, grad, m, v, n, lr_t, lr_t_mem, b1, b2, eps, clip, max_norm, delta);
+    }
+    if (named || !same || q.count == kMaxPendingSteps)
+        if (int rc = flush_steps(ctx)) return rc;
+    if (q.count == 0) {
+        q.kind = kind;
+        q.lr = lr;
+        q.b1 = b1;
+        q.b2 = b2;
+        q.eps = eps;
+        q.clip = clip;
+        q.max_norm = max_norm;
+        q.delta = delta;
+    }
+    const int i = q.count++;
+    q.p[i] = param;
+    q.g[i] = grad;
+    q.m[i] = m;
+    q.v[i] = v;
+    q.n[i] = n;
+    q.lr_t[i] = lr_t;
+    q.lr_t_mem[i] = lr_t_mem;
+    return ZG_HIP_OK;
+}
+
+ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n, float lr, int clip, float max_norm,
+                           float delta) {
+    ZG_CTX_KEEP_FILLS(ctx);
+    if (n == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(param && grad, "sgd_step: null pointer");
+    return step_entry(ctx, 0, param, grad, nullptr, nullptr, n, lr, 0.f, nullptr, 0.f, 0.f, 0.f, clip, max_norm, delta);
+}
+
 ZG_API int zg_hip_adam_step(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n, uint64_t t,
                             float lr, float beta1, float beta2, float epsilon, int clip, float max_norm, float delta) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad && m && v, "adam_step: null pointer");
     ZG_REQUIRE(t >= 1, "adam_step: t must be >= 1");
-    return adam_launch(ctx, param, grad, m, v, n, adam_lr_t(lr, beta1, beta2, t), nullptr, beta1, beta2, epsilon, clip,
-                       max_norm, delta);
+    return step_entry(ctx, 1, param, grad, m, v, n, 0.f, adam_lr_t(lr, beta1, beta2, t), nullptr, beta1, beta2, epsilon, clip,
+                      max_norm, delta);
 }
 
 ZG_API int zg_hip_adam_lr_t(float lr, float beta1, float beta2, uint64_t t, float* lr_t) {
@@ -285,17 +374,16 @@ ZG_API int zg_hip_adam_lr_t(float lr, float beta1, float beta2, uint64_t t, floa
 ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n,
                                const float* lr_t, float beta1, float beta2, float epsilon, int clip, float max_norm,
                                float delta) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad && m && v && lr_t, "adam_step_at: null pointer");
-    return adam_launch(ctx, param, grad, m, v, n, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);
+    return step_entry(ctx, 2, param, grad, m, v, n, 0.f, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);
 }
 
 // Parameter lists (the tensors are independent, so the launches need not follow the list order; a tensor listed
 // twice is the exception and is handled below): tensors of up to kMultiBigMax elements share the update launch (those beyond kFlatSingleMax get
 // their clip factor from the two-stage norm reduction of the per-tensor path first, so the values stay the same);
 // larger ones take the per-tensor path with its 16-byte grid-stride kernels.
-constexpr size_t kMultiBigMax = (size_t)1 << 20;
 static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_tensors, float* const* params,
                       float* const* grads, float* const* ms, float* const* vs, const size_t* lens, const float* lr_t,
                       int lr_t_in_memory, float lr, float beta1, float beta2, float epsilon, int clip, float max_norm,
@@ -361,7 +449,7 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
             rc = adam_launch(ctx, params[i], grads[i], ms[i], vs[i], n, lr_t_in_memory ? 0.f : lr_t[i],
                              lr_t_in_memory ? lr_t + i : nullptr, beta1, beta2, epsilon, clip, max_norm, delta);
         else
-            rc = zg_hip_sgd_step(ctx, params[i], grads[i], n, lr, clip, max_norm, delta);
+            rc = sgd_launch(ctx, params[i], grads[i], n, lr, clip, max_norm, delta);
         if (rc) return rc;
         if (zero_grads)
             if ((rc = zg_hip_mem_fill(ctx, grads[i], n, 0.f))) return rc;

@@ -806,6 +806,8 @@ ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uin
     ZG_CTX_KEEP_FILLS(ctx);
     if (ctx->deferred.active)  // what a waiting product waits for comes right after it, not after an allocation
         if (int rc = flush_deferred_gemm(ctx)) return rc;
+    if (ctx->steps.count)
+        if (int rc = flush_steps(ctx)) return rc;
     ZG_REQUIRE(out != nullptr && block != nullptr, "mem_cache_alloc: null output");
     *out = nullptr;
     *block = 0;
@@ -850,6 +852,8 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     ZG_CTX_KEEP_FILLS(ctx);
     if (ctx->n_pending_fills)  // a fill of the block that is given back must not land on its next owner
         if (int rc = flush_fills(ctx)) return rc;
+    if (ctx->steps.count)
+        if (int rc = flush_steps(ctx)) return rc;
     if (!ptr || block == 0) {  // views and empty data: src/allocators/caching_allocator.zig:111-112
         if (ctx->deferred.active) return flush_deferred_gemm(ctx);
         return ZG_HIP_OK;
@@ -1075,9 +1079,11 @@ int flush_fills(zg_hip_ctx* ctx) {
     return ZG_HIP_OK;
 }
 int flush_pending(zg_hip_ctx* ctx) {
+    // at most one kind is waiting at a time, except fills next to allocations: each kind's own calls send the others first
     if (ctx->deferred.active)
         if (int rc = flush_deferred_gemm(ctx)) return rc;
-    return flush_fills(ctx);
+    if (int rc = flush_fills(ctx)) return rc;
+    return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
 }
 
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
@@ -1099,6 +1105,8 @@ ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {
     ZG_CTX_KEEP_FILLS(ctx);
     if (ctx->deferred.active)  // a waiting product goes first: the fill may be of one of its operands
         if (int rc = flush_deferred_gemm(ctx)) return rc;
+    if (ctx->steps.count)  // and so do waiting optimizer steps: zero_grad fills the gradients they read
+        if (int rc = flush_steps(ctx)) return rc;
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x != nullptr, "mem_fill: null pointer");
     // The fill waits for the next call that is not a fill.  Two waiting fills never overlap (workgroups of one launch

@@ -65,6 +65,15 @@ struct zg_deferred_gemm {
     const char* name = "matmul";
 };
 
+// The bias gradient of a small Linear layer (gb += column sums of gy, one launch of the column kernel) that has been
+// asked for and not launched yet: the layer's two products follow it and can share its launch (gemm.hip).
+struct zg_waiting_bias {
+    bool active = false;
+    const float* gy = nullptr;  // [R, inner]
+    float* gb = nullptr;        // [inner]
+    size_t R = 0, inner = 0;
+};
+
 // Optimizer steps of small tensors that have been asked for and not launched yet (optim.hip).
 constexpr int kMaxPendingSteps = 16;
 struct zg_pending_steps {
@@ -141,6 +150,11 @@ struct zg_hip_ctx {
     // is, first thing (ZG_CTX), so no call ever sees memory the product has not reached; fills and a waiting product
     // never coexist (a fill launches the product first, a product launches the fills first).
     zg_deferred_gemm deferred;
+    // The backward pass of a small Linear layer, gathered call by call: the bias gradient (asked for first), the
+    // input-gradient product (`deferred`, kind 2, waiting for its mask) and the weight-gradient product that follows
+    // it leave in one launch when the mask arrives.
+    zg_deferred_gemm deferred_w;
+    zg_waiting_bias bias_wait;
     // Cache blocks that were given back while a waiting input-gradient product still names them as operands (the
     // reference frees a node's gradient as soon as its backward has run, src/ndtensor.zig eager teardown): they return
     // to the pool right after the product is launched.
@@ -173,8 +187,16 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 // matched must still hold what it held then, or the replay would scatter by a stale plan.
 // Launches the fills that are waiting in the context (one kernel for all of them).
 int flush_fills(zg_hip_ctx* ctx);
-// Launches the waiting product, with whatever was attached to it (gemm.hip).
+// Launches the waiting product with whatever was attached to it, and the waiting bias gradient and weight-gradient
+// product of the same layer (gemm.hip).  gemm_group_waiting: whether any of the three waits.
 int flush_deferred_gemm(zg_hip_ctx* ctx);
+inline bool gemm_group_waiting(const zg_hip_ctx* ctx) {
+    return ctx->deferred.active || ctx->deferred_w.active || ctx->bias_wait.active;
+}
+// Whether [lo, hi) meets an operand of the waiting products or of the waiting bias gradient.
+bool gemm_group_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
+// The single-chunk column sum y += column sums of x[R, inner] (reduce.hip), the launch the waiting bias gradient owes.
+int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner);
 // Launches the optimizer steps that are waiting (optim.hip).
 int flush_steps(zg_hip_ctx* ctx);
 // Returns to the pools the blocks whose free waited for the product (runtime.hip); called once it is launched.
@@ -251,7 +273,7 @@ inline bool aligned16(const void* p) {
 // First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
 #define ZG_CTX(ctx)                                          \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
-    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->steps.count) {  \
+    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count) {  \
         if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
     }
 // The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the

@@ -1115,6 +1115,36 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
                               float beta, size_t batches, size_t nba, size_t nbb, size_t a_chunk, size_t b_chunk,
                               size_t c_chunk, int depth, const GemmExtras* extras);
 
+// One launch for the backward of a small Linear layer (linear_bwd_small_kernel): gw = gw_beta * gw + gy^T x (x with
+// leading dimension ldx), gx = gy w masked by act_in (w with leading dimension ldw; gx null: none), gb += column sums of
+// gy (gb null: none).  The caller has checked that each job is one the kernel's blocks take.
+static int launch_linear_bwd_small(zg_hip_ctx* ctx, const float* gy, const float* x, size_t ldx, const float* w, size_t ldw,
+                                   const float* act_in, float* gw, float gw_beta, float* gb, float* gx, size_t batch,
+                                   size_t fan_in, size_t fan_out) {
+    LinearBwdArgs a;
+    a.gw = gemm_args(gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, ldx, fan_in, 1.f, gw_beta, 1, 1, 0, 0, 0, nullptr);
+    a.n_w = a.gw.tiles_m * a.gw.tiles_n;
+    a.gx = a.gw;
+    a.n_x = 0;
+    if (gx) {
+        const GemmExtras ex = {nullptr, act_in, 0};
+        a.gx = gemm_args(gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, ldw, fan_in, 1.f, 0.f, 1, 1, 0, 0, 0,
+                         act_in ? &ex : nullptr);
+        a.n_x = a.gx.tiles_m * a.gx.tiles_n;
+    }
+    const ColReduceShape cs = col_reduce_shape(gy, fan_out);
+    a.gy = gy;
+    a.gb = gb;
+    a.R = batch;
+    a.inner = fan_out;
+    a.log2_cx = cs.log2_cx;
+    const unsigned grid = a.n_w + a.n_x + (gb ? (unsigned)cs.gx : 0u);
+    if (cs.V == 4) hipLaunchKernelGGL(linear_bwd_small_kernel<4>, dim3(grid), dim3(kGemmThreads), 0, ctx->stream, a);
+    else hipLaunchKernelGGL(linear_bwd_small_kernel<1>, dim3(grid), dim3(kGemmThreads), 0, ctx->stream, a);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
 // Every product goes through here.  With zg_hip_gemm_timing on, the launches of one product (its kernel, and the
 // reduction or the strips when it is cut) are bracketed by a pair of events on the context's stream.
 static int gemm_dispatch(zg_hip_ctx* ctx, const char* name, const float* A, const float* B, float* C, size_t m, size_t n,
@@ -1458,16 +1488,57 @@ static bool ranges_meet(ByteRange a, ByteRange b) {
     return a.lo < b.hi && b.lo < a.hi;
 }
 
+static ByteRange product_a_range(const zg_deferred_gemm& d) {
+    return operand_range(d.A, d.trans_a ? d.k : d.m, d.trans_a ? d.m : d.k, d.lda);
+}
+static ByteRange product_b_range(const zg_deferred_gemm& d) {
+    return operand_range(d.B, d.trans_b ? d.n : d.k, d.trans_b ? d.k : d.n, d.ldb);
+}
+static ByteRange product_c_range(const zg_deferred_gemm& d) {
+    return operand_range(d.C, d.m, d.n, d.ldc);
+}
+
+bool gemm_group_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi) {
+    const ByteRange r{lo, hi};
+    auto product = [&](const zg_deferred_gemm& d) {
+        return d.active && (ranges_meet(r, product_a_range(d)) || ranges_meet(r, product_b_range(d)) ||
+                            ranges_meet(r, product_c_range(d)));
+    };
+    const zg_waiting_bias& b = ctx->bias_wait;
+    return product(ctx->deferred) || product(ctx->deferred_w) ||
+           (b.active && (ranges_meet(r, operand_range(b.gy, b.R, b.inner, b.inner)) ||
+                         ranges_meet(r, operand_range(b.gb, 1, b.inner, b.inner))));
+}
+
+// Whatever waits of a layer's backward pass goes out: in one launch when the weight-gradient product was recorded (it
+// is only recorded when every waiting member fits linear_bwd_small_kernel), else the bias gradient's column sum and
+// the product with what was attached to it.
 int flush_deferred_gemm(zg_hip_ctx* ctx) {
-    zg_deferred_gemm d = ctx->deferred;
-    if (!d.active) return ZG_HIP_OK;
+    const zg_deferred_gemm d = ctx->deferred, w = ctx->deferred_w;
+    const zg_waiting_bias b = ctx->bias_wait;
+    if (!d.active && !w.active && !b.active) return ZG_HIP_OK;
     ctx->deferred.active = false;
-    GemmExtras ex{d.bias, d.gate, d.relu};
-    const bool any = d.bias || d.gate || d.relu;
-    const int rc = gemm_dispatch(ctx, d.name, d.A, d.B, d.C, d.m, d.n, d.k, d.trans_a, d.trans_b, d.lda, d.ldb, d.ldc, d.alpha,
-                                 0.f, 1, 1, 1, 0, 0, 0, 0, any ? &ex : nullptr);
-    if (rc && d.zeroed) (void)zg_hip_mem_fill(ctx, d.C, d.m * d.n, 0.f);  // the product failed: the zeros are still owed
-    run_deferred_frees(ctx);  // blocks that hold its operands and were given back while it waited
+    ctx->deferred_w.active = false;
+    ctx->bias_wait.active = false;
+    int rc = ZG_HIP_OK;
+    if (w.active) {
+        rc = launch_linear_bwd_small(ctx, w.A, w.B, w.ldb, d.active ? d.B : nullptr, d.active ? d.ldb : 0,
+                                     d.active ? d.gate : nullptr, w.C, w.zeroed ? 0.f : 1.f, b.active ? b.gb : nullptr,
+                                     d.active ? d.C : nullptr, w.k, w.n, w.m);
+    } else {
+        if (b.active) rc = launch_bias_col_sum(ctx, b.gy, b.gb, b.R, b.inner);
+        if (!rc && d.active) {
+            GemmExtras ex{d.bias, d.gate, d.relu};
+            const bool any = d.bias || d.gate || d.relu;
+            rc = gemm_dispatch(ctx, d.name, d.A, d.B, d.C, d.m, d.n, d.k, d.trans_a, d.trans_b, d.lda, d.ldb, d.ldc, d.alpha,
+                               0.f, 1, 1, 1, 0, 0, 0, 0, any ? &ex : nullptr);
+        }
+    }
+    if (rc) {  // a product failed: the zeros its output was owed are still owed
+        if (d.active && d.zeroed) (void)zg_hip_mem_fill(ctx, d.C, d.m * d.n, 0.f);
+        if (w.active && w.zeroed) (void)zg_hip_mem_fill(ctx, w.C, w.m * w.n, 0.f);
+    }
+    run_deferred_frees(ctx);  // blocks that hold operands and were given back while the work waited
     return rc;
 }
 
@@ -1523,21 +1594,71 @@ static int gemm_entry(zg_hip_ctx* ctx, const char* name, const float* A, const f
         if (rc && zeroed) (void)zg_hip_mem_fill(ctx, C, batches * m * n, 0.f);  // refused: the zeros are still owed
         return rc;
     };
+    const size_t n_cu = (size_t)ctx->n_cu;
+    const ByteRange tC = (plain && C) ? operand_range(C, m, n, ldc) : ByteRange{nullptr, nullptr};
+    // a weight-gradient product the one-launch layer backward can take: gw (+)= gy^T x, gy dense
+    const bool w_shape = plain && trans_a && !trans_b && alpha == 1.f && (beta_eff == 0.f || beta_eff == 1.f) && lda == m &&
+                         gemm_is_tiny(m, n, k, 1, lda, ldb, n_cu) &&
+                         gemm_validate(name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc) == ZG_HIP_OK;
+    auto record_w = [&]() {
+        zg_deferred_gemm& w = ctx->deferred_w;
+        w = zg_deferred_gemm{};
+        w.active = true;
+        w.zeroed = beta_eff == 0.f;
+        w.A = A;
+        w.B = B;
+        w.C = C;
+        w.m = m;
+        w.n = n;
+        w.k = k;
+        w.lda = lda;
+        w.ldb = ldb;
+        w.ldc = ldc;
+        w.trans_a = 1;
+        w.trans_b = 0;
+        w.name = name;
+    };
+    const zg_waiting_bias& bw = ctx->bias_wait;
+    const bool clear_of_bias =
+        !bw.active || !plain ||
+        (!ranges_meet(tC, operand_range(bw.gy, bw.R, bw.inner, bw.inner)) &&
+         !ranges_meet(tC, operand_range(bw.gb, 1, bw.inner, bw.inner)) &&
+         !ranges_meet(operand_range(bw.gb, 1, bw.inner, bw.inner), operand_range(A, trans_a ? k : m, trans_a ? m : k, lda)) &&
+         !ranges_meet(operand_range(bw.gb, 1, bw.inner, bw.inner), operand_range(B, trans_b ? n : k, trans_b ? k : n, ldb)));
     if (ctx->deferred.active) {
         const zg_deferred_gemm& d = ctx->deferred;
         bool pass = false;
-        if (d.kind == 2 && plain && gemm_validate(name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc) == ZG_HIP_OK) {
-            const ByteRange dA = operand_range(d.A, d.trans_a ? d.k : d.m, d.trans_a ? d.m : d.k, d.lda);
-            const ByteRange dB = operand_range(d.B, d.trans_b ? d.n : d.k, d.trans_b ? d.k : d.n, d.ldb);
-            const ByteRange dC = operand_range(d.C, d.m, d.n, d.ldc);
+        if (d.kind == 2 && plain && !ctx->deferred_w.active && clear_of_bias &&
+            gemm_validate(name, A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc) == ZG_HIP_OK) {
+            const ByteRange dA = product_a_range(d), dB = product_b_range(d), dC = product_c_range(d);
             const ByteRange tA = operand_range(A, trans_a ? k : m, trans_a ? m : k, lda);
             const ByteRange tB = operand_range(B, trans_b ? n : k, trans_b ? k : n, ldb);
-            const ByteRange tC = operand_range(C, m, n, ldc);
             pass = !ranges_meet(tC, dA) && !ranges_meet(tC, dB) && !ranges_meet(tC, dC) && !ranges_meet(dC, tA) &&
                    !ranges_meet(dC, tB);
         }
-        if (pass) return launch_now();
+        if (pass) {
+            // the layer's weight-gradient product after its input-gradient product: both small and fed by the same
+            // dense gy, it waits too and the layer's backward leaves in one launch; else it goes out now
+            if (w_shape && A == d.A && d.alpha == 1.f && d.lda == d.k && m == d.k && k == d.m && n == d.n &&
+                gemm_is_tiny(d.m, d.n, d.k, 1, d.lda, d.ldb, n_cu)) {
+                record_w();
+                return ZG_HIP_OK;
+            }
+            return launch_now();
+        }
         if (int rc = flush_deferred_gemm(ctx)) return rc;
+    } else if (bw.active) {
+        // only a bias gradient waits: the layer's input-gradient product may join it (below), its weight-gradient
+        // product takes it along now (a first layer has no input gradient); anything else sends it out first
+        const bool same_gy = plain && A == bw.gy && clear_of_bias;
+        if (same_gy && w_shape && m == bw.inner && k == bw.R) {
+            record_w();
+            return flush_deferred_gemm(ctx);
+        }
+        const bool joins = same_gy && !trans_a && !trans_b && zeroed && beta_eff == 0.f && m == bw.R && k == bw.inner &&
+                           lda == k;
+        if (!joins)
+            if (int rc = flush_deferred_gemm(ctx)) return rc;
     }
     const int kind = (!trans_a && trans_b) ? 1 : ((!trans_a && !trans_b && zeroed) ? 2 : 0);
     if (plain && beta_eff == 0.f && kind != 0) {
@@ -1633,28 +1754,7 @@ ZG_API int zg_hip_linear_bwd(zg_hip_ctx* ctx, const float* gy, const float* x, c
         return gemm_dispatch(ctx, "linear_bwd", gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, fan_in, fan_in, 1.f, 1.f,
                              1, 1, 1, 0, 0, 0);
     }
-    LinearBwdArgs a;
-    a.gw = gemm_args(gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, fan_in, fan_in, 1.f, 1.f, 1, 1, 0, 0, 0, nullptr);
-    a.n_w = a.gw.tiles_m * a.gw.tiles_n;
-    a.gx = a.gw;
-    a.n_x = 0;
-    if (gx) {
-        const GemmExtras ex = {nullptr, act_in, 0};
-        a.gx = gemm_args(gy, w, gx, batch, fan_in, fan_out, 0, 0, fan_out, fan_in, fan_in, 1.f, 0.f, 1, 1, 0, 0, 0,
-                         act_in ? &ex : nullptr);
-        a.n_x = a.gx.tiles_m * a.gx.tiles_n;
-    }
-    const ColReduceShape cs = col_reduce_shape(gy, fan_out);
-    a.gy = gy;
-    a.gb = gb;
-    a.R = batch;
-    a.inner = fan_out;
-    a.log2_cx = cs.log2_cx;
-    const unsigned grid = a.n_w + a.n_x + (gb ? (unsigned)cs.gx : 0u);
-    if (cs.V == 4) hipLaunchKernelGGL(linear_bwd_small_kernel<4>, dim3(grid), dim3(kGemmThreads), 0, ctx->stream, a);
-    else hipLaunchKernelGGL(linear_bwd_small_kernel<1>, dim3(grid), dim3(kGemmThreads), 0, ctx->stream, a);
-    ZG_LAUNCH_CHECK();
-    return ZG_HIP_OK;
+    return launch_linear_bwd_small(ctx, gy, x, fan_in, w, fan_in, act_in, gw, 1.f, gb, gx, batch, fan_in, fan_out);
 }
 
 ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_shape, const float* B,

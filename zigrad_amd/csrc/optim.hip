@@ -307,8 +307,8 @@ int flush_steps(zg_hip_ctx* ctx) {
 static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, float* m, float* v, size_t n, float lr,
                       float lr_t, const float* lr_t_mem, float b1, float b2, float eps, int clip, float max_norm,
                       float delta) {
-    if (ctx->deferred.active || ctx->n_pending_fills) {  // the gradients come from them
-        if (ctx->deferred.active)
+    if (gemm_group_waiting(ctx) || ctx->n_pending_fills) {  // the gradients come from them
+        if (gemm_group_waiting(ctx))
             if (int rc = flush_deferred_gemm(ctx)) return rc;
         if (int rc = flush_fills(ctx)) return rc;
     }

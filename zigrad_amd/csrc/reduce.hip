@@ -249,6 +249,10 @@ static int sum_along_impl(zg_hip_ctx* ctx, const float* x, const uint64_t* x_sha
     return axis_reduce<AxisSum>(ctx, x, y, outer, R, inner, alpha, beta);
 }
 
+int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner) {
+    return axis_reduce<AxisSum>(ctx, x, y, 1, R, inner, 1.f, 1.f);
+}
+
 }  // namespace zg
 
 using namespace zg;
@@ -467,6 +471,18 @@ ZG_API int zg_hip_unbroadcast(zg_hip_ctx* ctx, const float* x, const uint64_t* x
     if (xr > yr) {
         const size_t dif = xr - yr;
         const size_t row = prod(xs, 0, dif), col = prod(xs, dif, xr);
+        if (ones == 0 && alpha == 1.f && beta == 1.f && row > 1 && col > 1 && row * col <= kColSingleChunkMax &&
+            (x + row * col <= y || y + col <= x)) {
+            // y += column sums of x in one launch of the column kernel: a small layer's bias gradient
+            // (src/ndtensor.zig:780-796).  It waits for the layer's two products, which can share its launch.
+            zg_waiting_bias& b = ctx->bias_wait;
+            b.active = true;
+            b.gy = x;
+            b.gb = y;
+            b.R = row;
+            b.inner = col;
+            return ZG_HIP_OK;
+        }
         int rc = axis_reduce<AxisSum>(ctx, x, ones == 0 ? y : scratch, 1, row, col, alpha, beta);
         if (rc) return rc;
         if (ones == 0) return ZG_HIP_OK;

@@ -804,7 +804,9 @@ ZG_API int zg_hip_cache_configure(zg_hip_ctx* ctx, size_t small_pool_bytes, size
 
 ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uint64_t* block) {
     ZG_CTX_KEEP_FILLS(ctx);
-    if (ctx->deferred.active)  // what a waiting product waits for comes right after it, not after an allocation
+    // what a waiting product waits for comes right after it, not after an allocation; a bias gradient that waits
+    // alone stays (the input gradient its layer's products write is allocated next, and a new block holds no operand)
+    if (ctx->deferred.active)
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (ctx->steps.count)
         if (int rc = flush_steps(ctx)) return rc;
@@ -855,7 +857,7 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     if (ctx->steps.count)
         if (int rc = flush_steps(ctx)) return rc;
     if (!ptr || block == 0) {  // views and empty data: src/allocators/caching_allocator.zig:111-112
-        if (ctx->deferred.active) return flush_deferred_gemm(ctx);
+        if (gemm_group_waiting(ctx)) return flush_deferred_gemm(ctx);
         return ZG_HIP_OK;
     }
     Block* b = (Block*)(uintptr_t)block;
@@ -864,25 +866,16 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
         if (p && p->owns_live(b, ptr)) pool = p;
     ZG_REQUIRE(pool != nullptr, "mem_cache_free: %p with handle %llx is not a live block of this context's pools", ptr,
                (unsigned long long)block);
-    if (ctx->deferred.active) {
+    if (gemm_group_waiting(ctx)) {
         // An input-gradient product that waits for its mask outlives the frees of the backward pass it belongs to
-        // (the layer's output, the output gradient).  A block none of its operands lies in goes back at once; one that
-        // holds an operand goes back when the product has been launched.
-        const zg_deferred_gemm& d = ctx->deferred;
-        bool keep_waiting = d.kind == 2;
+        // (the layer's output, the output gradient), and so do the bias gradient and the weight-gradient product
+        // that wait with it.  A block none of their operands lies in goes back at once; one that holds an operand
+        // goes back when they have been launched.
+        const bool keep_waiting = !ctx->deferred.active || ctx->deferred.kind == 2;
         for (int i = 0; i < ctx->n_deferred_frees; i++)
             ZG_REQUIRE(ctx->deferred_frees[i].block != block, "mem_cache_free: %p was already given back", ptr);
         if (keep_waiting) {
-            const char *lo = b->ptr, *hi = b->ptr + b->size;
-            auto meets = [&](const float* p, size_t rows, size_t cols, size_t ld) {
-                const char* plo = (const char*)p;
-                const char* phi = plo + ((rows - 1) * ld + cols) * sizeof(float);
-                return plo < hi && lo < phi;
-            };
-            const bool operand = meets(d.A, d.trans_a ? d.k : d.m, d.trans_a ? d.m : d.k, d.lda) ||
-                                 meets(d.B, d.trans_b ? d.n : d.k, d.trans_b ? d.k : d.n, d.ldb) ||
-                                 meets(d.C, d.m, d.n, d.ldc);
-            if (!operand) {
+            if (!gemm_group_touches(ctx, b->ptr, b->ptr + b->size)) {
                 release_block(ctx, b);
                 return ZG_HIP_OK;
             }
@@ -1080,7 +1073,7 @@ int flush_fills(zg_hip_ctx* ctx) {
 }
 int flush_pending(zg_hip_ctx* ctx) {
     // at most one kind is waiting at a time, except fills next to allocations: each kind's own calls send the others first
-    if (ctx->deferred.active)
+    if (gemm_group_waiting(ctx))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (int rc = flush_fills(ctx)) return rc;
     return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
@@ -1103,7 +1096,10 @@ bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
 
 ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {
     ZG_CTX_KEEP_FILLS(ctx);
-    if (ctx->deferred.active)  // a waiting product goes first: the fill may be of one of its operands
+    // a waiting product goes first: the fill may be of one of its operands; a bias gradient that waits alone stays
+    // unless the fill meets what it reads or writes (the zero fill of the layer's input gradient comes next)
+    if (ctx->deferred.active ||
+        (x && n && gemm_group_waiting(ctx) && gemm_group_touches(ctx, (const char*)x, (const char*)(x + n))))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (ctx->steps.count)  // and so do waiting optimizer steps: zero_grad fills the gradients they read
         if (int rc = flush_steps(ctx)) return rc;

@@ -167,8 +167,10 @@ int zg_hip_gemm_plan(zg_hip_ctx *ctx, size_t m, size_t n, size_t k, size_t batch
  *     (:38-46) the ReLU is applied in the epilogue too and the product is launched;
  *   - an input-gradient product, C += A B with beta == 1 onto a C whose zero fill is still waiting (ensure_grad(0) then
  *     BmmAccBwd, src/ndtensor.zig:221-228, :1107-1109): one following product that touches none of its operands (the
- *     weight gradient, :1126-1128) is launched ahead of it; if the next call is zg_hip_relu_inplace_bwd on C
- *     (src/nn/nn.zig:44-50) the mask is applied in the epilogue and the product is launched.
+ *     weight gradient, :1126-1128) is launched ahead of it, or, when both products are small enough for the unstaged
+ *     kernel and read the same dense A, waits with it; if the next call is zg_hip_relu_inplace_bwd on C
+ *     (src/nn/nn.zig:44-50) the mask is applied in the epilogue and the product is launched, in one launch with the
+ *     weight-gradient product and the layer's bias gradient (see zg_hip_unbroadcast) when those wait too.
  * Any other call (a read, a fill, a free, an allocation, another op, zg_hip_sync, the end of a recording) launches the
  * waiting product first, unchanged.  The values are those of the separate calls, bit for bit: the epilogue does the
  * same IEEE operations in the same order.  An argument error is reported by the call that asks for the product. */
@@ -247,6 +249,10 @@ int zg_hip_argmax_along(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape
 /* scratch sizing rule of NDArray.unbroadcast_ (src/ndarray.zig:701-719), in floats */
 size_t zg_hip_unbroadcast_scratch_len(const uint64_t *x_shape, size_t x_rank, const uint64_t *y_shape,
                                       size_t y_rank);
+/* unbroadcast (src/device/host_device.zig:709-780).  The form a Linear layer's bias gradient takes (y += sums over the
+ * leading dimensions of x, alpha = beta = 1, at most 16384 elements of x) waits inside the context like a product
+ * (see zg_hip_matmul): the layer's input-gradient and weight-gradient products follow it (src/ndtensor.zig:780-796,
+ * 1092-1136) and, when they are small too, the three leave in one launch.  Any other call sends it out first. */
 int zg_hip_unbroadcast(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape, size_t x_rank, float *y,
                        const uint64_t *y_shape, size_t y_rank, float *scratch, size_t scratch_len, float alpha,
                        float beta);

@@ -6,6 +6,7 @@ import pytest
 from scipy.special import logsumexp, softmax
 
 from conftest import rel_fro, run_op
+from zigrad_amd.device import F32
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-5
@@ -24,6 +25,36 @@ def both(oracle, hip, name, params, outputs):
 # ----------------------------------------------------------------------------------------------
 # softmax / cross-entropy
 # ----------------------------------------------------------------------------------------------
+def _smce_fwd_hip(hip, x, t):
+    rows, cols = x.shape
+    xb, tb = hip.from_numpy(x), hip.from_numpy(t)
+    pb, lb = hip.mem_alloc(F32, rows * cols), hip.mem_alloc(F32, 1)
+    hip.dispatch("smce_fwd", logits=xb, target=tb, probs=pb, loss=lb, rows=rows, cols=cols)
+    out = hip.to_numpy(pb).reshape(rows, cols), float(hip.to_numpy(lb)[0])
+    for b in (xb, tb, pb, lb):
+        hip.mem_free(b)
+    return out
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 10), (256, 32), (140, 7), (64, 200), (16, 3000), (1, 4), (255, 2)])
+def test_smce_fwd_small_batches_equal_the_two_launch_path(hip, rows, cols):
+    """A batch that fits one workgroup takes one launch (rows and their mean); the same rows inside a batch too large
+    for it take the row kernel and the reduction.  Per row the probabilities must be the same bits; the mean is held to
+    the float64 closed form."""
+    r = rng(rows + 31 * cols)
+    x = (r.standard_normal((rows, cols)) * 3).astype(np.float32)
+    t = np.zeros((rows, cols), np.float32)
+    t[np.arange(rows), r.integers(0, cols, rows)] = 1.0
+    p_small, loss_small = _smce_fwd_hip(hip, x, t)
+    big = 1200 // rows + 2
+    p_big, _ = _smce_fwd_hip(hip, np.tile(x, (big, 1)), np.tile(t, (big, 1)))
+    np.testing.assert_array_equal(p_small, p_big[:rows])
+    x64 = x.astype(np.float64)
+    p_lab = np.exp((x64 * t).sum(axis=1) - logsumexp(x64, axis=1))
+    want = float(np.mean(-np.log(np.clip(p_lab, np.float32(1e-7), np.float32(1.0) - np.float32(1e-7)))))
+    assert abs(loss_small - want) <= 1e-5 * max(1.0, abs(want))
+
+
 SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001), (9, 4100)]
 
 

@@ -86,6 +86,7 @@ struct zg_pending_steps {
     size_t n[kMaxPendingSteps];
     float lr_t[kMaxPendingSteps];            // kind 1
     const float* lr_t_mem[kMaxPendingSteps]; // kind 2
+    bool zero[kMaxPendingSteps];             // a zero fill of exactly this gradient arrived while the step waited
     float lr = 0.f, b1 = 0.f, b2 = 0.f, eps = 0.f, max_norm = 0.f, delta = 0.f;
     int clip = 0;
 };
@@ -197,8 +198,10 @@ inline bool gemm_group_waiting(const zg_hip_ctx* ctx) {
 bool gemm_group_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
 // The single-chunk column sum y += column sums of x[R, inner] (reduce.hip), the launch the waiting bias gradient owes.
 int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner);
-// Launches the optimizer steps that are waiting (optim.hip).
-int flush_steps(zg_hip_ctx* ctx);
+// Launches the optimizer steps that are waiting (optim.hip).  Gradients whose zero fill was taken over are zeroed by
+// the update kernel when every waiting step has one; otherwise their fills are launched after the steps, or, with
+// requeue_fills, put back among the waiting fills for the caller (zg_hip_mem_fill) to send with its own.
+int flush_steps(zg_hip_ctx* ctx, bool requeue_fills = false);
 // Returns to the pools the blocks whose free waited for the product (runtime.hip); called once it is launched.
 void run_deferred_frees(zg_hip_ctx* ctx);
 // The waiting product, then the waiting fills: what ZG_CTX does before a call's own work.

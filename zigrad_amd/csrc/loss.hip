@@ -510,8 +510,8 @@ static unsigned smce_bwd_grid(size_t n) {
 // smce_fwd and the loss's backward (upstream gradient 1) of a batch small enough for one workgroup, in one launch:
 // kFlatSingle / TPR rows of at most 4096 columns.  Per row the arithmetic is softmax_rows_kernel's, per gradient
 // element smce_bwd_kernel's, and the mean over the rows is formed as flat_single_kernel forms it, so every value
-// equals what the separate launches produce.
-template <int TPR, bool ACC>
+// equals what the separate launches produce.  GRAD: 0 no gradient (smce_fwd alone), 1 written, 2 added to.
+template <int TPR, int GRAD>
 __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* logits, const float* target, float* probs,
                                                                  float* loss, float* grad, size_t rows, size_t cols) {
     static_assert(TPR <= kWave, "a row is reduced inside one wave");
@@ -539,8 +539,10 @@ __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* lo
                 const float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
                 part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
             }
-            const float d = __fdiv_rn(__fsub_rn(p, t), denom);
-            gr[j] = ACC ? __fadd_rn(gr[j], d) : d;
+            if (GRAD) {
+                const float d = __fdiv_rn(__fsub_rn(p, t), denom);
+                gr[j] = (GRAD == 2) ? __fadd_rn(gr[j], d) : d;
+            }
         }
     }
     part = group_reduce<SumAcc, TPR>(part);
@@ -701,6 +703,16 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
     ZG_CTX(ctx);
     ZG_REQUIRE(logits && target && probs && loss, "smce_fwd: null pointer");
     if (int rc = check_rows("smce_fwd", rows, cols)) return rc;
+    {
+        // a batch small enough for one workgroup: rows and their mean in one launch
+        const int tpr = pick_tpr(cols);
+        if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr)) {
+            ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_small_kernel<(T <= kWave ? T : kWave), 0>), dim3(1), dim3(kFlatSingle),
+                                                    0, ctx->stream, logits, target, probs, loss, (float*)nullptr, rows, cols));
+            ZG_LAUNCH_CHECK();
+            return ZG_HIP_OK;
+        }
+    }
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
     if (long_row_ok(logits, target, probs, rows, cols)) {
@@ -748,10 +760,10 @@ ZG_API int zg_hip_smce_fwd_bwd(zg_hip_ctx* ctx, const float* logits, const float
     if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr)) {
 #define ZG_SMALL(T)                                                                                                    \
     if (accumulate)                                                                                                    \
-        hipLaunchKernelGGL((smce_small_kernel<T, true>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,   \
+        hipLaunchKernelGGL((smce_small_kernel<T, 2>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,      \
                            probs, loss, grad, rows, cols);                                                             \
     else                                                                                                               \
-        hipLaunchKernelGGL((smce_small_kernel<T, false>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,  \
+        hipLaunchKernelGGL((smce_small_kernel<T, 1>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,      \
                            probs, loss, grad, rows, cols)
         if (tpr == 4) { ZG_SMALL(4); }
         else if (tpr == 16) { ZG_SMALL(16); }

@@ -272,10 +272,7 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
 namespace zg {
 // The waiting steps: one of them alone takes the per-tensor launches it would have taken, several take the
 // parameter-list kernels (the same arithmetic per element and the same norm trees: the values do not depend on which).
-int flush_steps(zg_hip_ctx* ctx) {
-    zg_pending_steps q = ctx->steps;
-    ctx->steps.count = 0;
-    if (q.count == 0) return ZG_HIP_OK;
+static int launch_steps(zg_hip_ctx* ctx, const zg_pending_steps& q, int zero_grads) {
     if (q.count == 1) {
         if (q.kind == 0) return sgd_launch(ctx, q.p[0], q.g[0], q.n[0], q.lr, q.clip, q.max_norm, q.delta);
         return adam_launch(ctx, q.p[0], q.g[0], q.m[0], q.v[0], q.n[0], q.lr_t[0], q.kind == 2 ? q.lr_t_mem[0] : nullptr, q.b1,
@@ -294,10 +291,33 @@ int flush_steps(zg_hip_ctx* ctx) {
             return ZG_HIP_OK;
         }
         return step_multi(ctx, "adam_step_at", true, (size_t)q.count, q.p, q.g, q.m, q.v, q.n, q.lr_t_mem[0], 1, 0.f, q.b1, q.b2,
-                          q.eps, q.clip, q.max_norm, q.delta, 0);
+                          q.eps, q.clip, q.max_norm, q.delta, zero_grads);
     }
     return step_multi(ctx, q.kind ? "adam_step" : "sgd_step", q.kind != 0, (size_t)q.count, q.p, q.g, q.m, q.v, q.n, q.lr_t, 0,
-                      q.lr, q.b1, q.b2, q.eps, q.clip, q.max_norm, q.delta, 0);
+                      q.lr, q.b1, q.b2, q.eps, q.clip, q.max_norm, q.delta, zero_grads);
+}
+
+int flush_steps(zg_hip_ctx* ctx, bool requeue_fills) {
+    const zg_pending_steps q = ctx->steps;
+    ctx->steps.count = 0;
+    if (q.count == 0) return ZG_HIP_OK;
+    int n_zero = 0;
+    for (int i = 0; i < q.count; i++) n_zero += q.zero[i] ? 1 : 0;
+    // zero_grad() after step(): when every waiting step's gradient is to be zeroed and the list kernels run, the update
+    // kernel stores the zeros as it reads the gradients (zg_hip_*_step_multi with zero_grads)
+    bool in_kernel = n_zero == q.count && q.count > 1;
+    if (in_kernel && q.kind == 2)
+        for (int i = 1; i < q.count; i++) in_kernel = in_kernel && q.lr_t_mem[i] == q.lr_t_mem[0] + i;
+    const int rc = launch_steps(ctx, q, in_kernel ? 1 : 0);
+    if (n_zero && !(in_kernel && rc == ZG_HIP_OK)) {  // the zeros are owed as fills, after the steps
+        if (ctx->n_pending_fills + n_zero > kMaxPendingFills)
+            if (int rcf = flush_fills(ctx)) return rc ? rc : rcf;
+        for (int i = 0; i < q.count; i++)
+            if (q.zero[i]) ctx->pending_fills[ctx->n_pending_fills++] = zg_pending_fill{q.g[i], q.n[i], 0.f};
+        if (!requeue_fills)
+            if (int rcf = flush_fills(ctx)) return rc ? rc : rcf;
+    }
+    return rc;
 }
 }  // namespace zg
 
@@ -344,6 +364,7 @@ static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, floa
     q.n[i] = n;
     q.lr_t[i] = lr_t;
     q.lr_t_mem[i] = lr_t_mem;
+    q.zero[i] = false;
     return ZG_HIP_OK;
 }
 

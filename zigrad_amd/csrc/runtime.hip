@@ -1101,8 +1101,21 @@ ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {
     if (ctx->deferred.active ||
         (x && n && gemm_group_waiting(ctx) && gemm_group_touches(ctx, (const char*)x, (const char*)(x + n))))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
-    if (ctx->steps.count)  // and so do waiting optimizer steps: zero_grad fills the gradients they read
-        if (int rc = flush_steps(ctx)) return rc;
+    if (ctx->steps.count) {
+        // zero_grad() after step() (examples/mnist/src/model.zig:57-62): a zero fill of exactly the gradient of a waiting
+        // step is taken over by the step, whose kernel stores the zeros once it has read the gradient; any other fill
+        // sends the steps out first (it may be of something they read), and zeros taken over so far leave with it
+        zg_pending_steps& q = ctx->steps;
+        uint32_t bits;
+        memcpy(&bits, &value, sizeof(bits));
+        if (bits == 0u && x && n)
+            for (int i = 0; i < q.count; i++)
+                if (q.g[i] == x && q.n[i] == n && !q.zero[i]) {
+                    q.zero[i] = true;
+                    return ZG_HIP_OK;
+                }
+        if (int rc = flush_steps(ctx, true)) return rc;
+    }
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x != nullptr, "mem_fill: null pointer");
     // The fill waits for the next call that is not a fill.  Two waiting fills never overlap (workgroups of one launch

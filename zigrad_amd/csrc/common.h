@@ -74,6 +74,21 @@ struct zg_waiting_bias {
     size_t R = 0, inner = 0;
 };
 
+// The aggregation of a graph-convolution layer (scatter_gcn_deg_scaled) whose plan is ready and whose apply kernel has
+// not been launched yet: the layer's bias add and ReLU follow it and run as the kernel's tail (index.hip).
+struct zg_waiting_scatter {
+    bool active = false;
+    float* dst = nullptr;
+    const float* h = nullptr;
+    const float* deg = nullptr;
+    const uint32_t* row_ptr = nullptr;
+    const uint32_t* peer = nullptr;
+    size_t n_nodes = 0, stride = 0;
+    bool fresh = false;           // written, not added to (the output's zero fill was taken over)
+    const float* bias = nullptr;  // attached by a following row-broadcast add onto dst
+    int relu = 0;                 // attached by a following in-place relu_fwd on dst
+};
+
 // Optimizer steps of small tensors that have been asked for and not launched yet (optim.hip).
 constexpr int kMaxPendingSteps = 16;
 struct zg_pending_steps {
@@ -156,6 +171,7 @@ struct zg_hip_ctx {
     // it leave in one launch when the mask arrives.
     zg_deferred_gemm deferred_w;
     zg_waiting_bias bias_wait;
+    zg_waiting_scatter scatter_wait;
     // Cache blocks that were given back while a waiting input-gradient product still names them as operands (the
     // reference frees a node's gradient as soon as its backward has run, src/ndtensor.zig eager teardown): they return
     // to the pool right after the product is launched.
@@ -198,6 +214,11 @@ inline bool gemm_group_waiting(const zg_hip_ctx* ctx) {
 bool gemm_group_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
 // The single-chunk column sum y += column sums of x[R, inner] (reduce.hip), the launch the waiting bias gradient owes.
 int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner);
+// Launches the waiting graph-convolution aggregation with what was attached to it (index.hip); the two hooks are for
+// zg_hip_add and zg_hip_relu_fwd, like deferred_take_add / deferred_take_relu below.
+int flush_scatter(zg_hip_ctx* ctx);
+bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);
+bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc);
 // Launches the optimizer steps that are waiting (optim.hip).  Gradients whose zero fill was taken over are zeroed by
 // the update kernel when every waiting step has one; otherwise their fills are launched after the steps, or, with
 // requeue_fills, put back among the waiting fills for the caller (zg_hip_mem_fill) to send with its own.
@@ -276,13 +297,19 @@ inline bool aligned16(const void* p) {
 // First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
 #define ZG_CTX(ctx)                                          \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
-    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count) {  \
+    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
+        (ctx)->scatter_wait.active) {                        \
         if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
     }
 // The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the
 // calls a product may absorb, and cache allocations (a block that is handed out is free, so no waiting fill names it;
 // a block that is freed goes through ZG_CTX).
-#define ZG_CTX_KEEP_FILLS(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
+// A waiting aggregation only waits for the add and the ReLU, which look at it before they get here: it goes out.
+#define ZG_CTX_KEEP_FILLS(ctx)                                   \
+    ZG_REQUIRE((ctx) != nullptr, "null context");                \
+    if ((ctx)->scatter_wait.active) {                            \
+        if (int _rc_sc = zg::flush_scatter(ctx)) return _rc_sc;  \
+    }
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.
 #define ZG_NOT_CAPTURING(ctx, who)                                                                       \

@@ -296,6 +296,7 @@ using namespace zg;
 ZG_API int zg_hip_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
     // a bias row added onto the output of a product that is still waiting becomes part of that product's launch
     if (ctx && ctx->deferred.active && deferred_take_add(ctx, x, xl, y, yl, z, zl)) return ZG_HIP_OK;
+    if (ctx && ctx->scatter_wait.active && scatter_take_add(ctx, x, xl, y, yl, z, zl)) return ZG_HIP_OK;
     return binary_op<AddOp>(ctx, "add", x, xl, y, yl, z, zl);
 }
 ZG_API int zg_hip_sub(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
@@ -344,6 +345,7 @@ ZG_API int zg_hip_relu_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n) 
     // in place on the output of a product that is still waiting: done in that product's epilogue
     int taken_rc = 0;
     if (ctx && ctx->deferred.active && deferred_take_relu(ctx, x, y, n, &taken_rc)) return taken_rc;
+    if (ctx && ctx->scatter_wait.active && scatter_take_relu(ctx, x, y, n, &taken_rc)) return taken_rc;
     ZG_CHECK_N("relu_fwd", n, x, y);
     return launch_map<ReluFwd, 1>(ctx, y, x, nullptr, nullptr, n);
 }

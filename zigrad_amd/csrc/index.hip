@@ -1059,6 +1059,43 @@ ZG_API int zg_hip_index_select_bwd(zg_hip_ctx* ctx, const float* y_grad, const u
     return ZG_HIP_OK;
 }
 
+namespace zg {
+int flush_scatter(zg_hip_ctx* ctx) {
+    const zg_waiting_scatter w = ctx->scatter_wait;
+    if (!w.active) return ZG_HIP_OK;
+    ctx->scatter_wait.active = false;
+    const int g = group_for(w.stride);
+    const unsigned grid = (unsigned)ceil_div_sz(w.n_nodes, 256 / g);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, w.dst, w.h, w.deg,
+                                        w.row_ptr, w.peer, w.n_nodes, w.stride, w.fresh, w.bias, w.relu != 0));
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// y._add(bias): z = x + y in place on the aggregation's output, the other operand a row of `stride` values
+bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl) {
+    zg_waiting_scatter& w = ctx->scatter_wait;
+    const size_t n = w.n_nodes * w.stride;
+    if (!w.active || w.bias || w.relu || z != w.dst || zl != n || w.stride == n) return false;
+    const float* row = nullptr;
+    if (y == w.dst && yl == n && xl == w.stride) row = x;
+    else if (x == w.dst && xl == n && yl == w.stride) row = y;
+    if (!row) return false;
+    if (row < w.dst + n && w.dst < row + w.stride) return false;
+    w.bias = row;
+    return true;
+}
+
+// relu_(y) in place on the aggregation's output: the last thing the layer does, so the kernel goes out
+bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc) {
+    zg_waiting_scatter& w = ctx->scatter_wait;
+    if (!w.active || w.relu || x != w.dst || y != w.dst || n != w.n_nodes * w.stride) return false;
+    w.relu = 1;
+    *rc = flush_scatter(ctx);
+    return true;
+}
+}  // namespace zg
+
 static int check_gcn(const char* name, size_t stride, size_t n_edge, size_t n_nodes) {
     ZG_REQUIRE(stride > 0 && n_nodes > 0, "%s: stride and n_nodes must be positive", name);
     ZG_REQUIRE(n_edge < 0xffffffffull && n_nodes < 0xffffffffull, "%s: sizes beyond 2^32-1", name);
@@ -1068,25 +1105,43 @@ static int check_gcn(const char* name, size_t stride, size_t n_edge, size_t n_no
 ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,
                                          const uint64_t* src_indices, const uint64_t* tgt_indices, size_t stride,
                                          size_t n_edge, size_t n_nodes) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
+    // the output's zero fill (the layer allocates it zeroed, examples/gcn/src/model.zig:100-112) may still be waiting:
+    // then the sums are written instead of added to zeros
+    const bool fresh = n_edge > 0 && dst && stride > 0 && n_nodes > 0 && absorb_zero_fill(ctx, dst, n_nodes * stride);
+    auto owed = [&](int rc_in) {  // refused after the fill was taken over: the zeros are still owed
+        if (fresh) (void)zg_hip_mem_fill(ctx, dst, n_nodes * stride, 0.f);
+        return rc_in;
+    };
+    if (int rc = flush_pending(ctx)) return owed(rc);
     if (n_edge == 0) return ZG_HIP_OK;
-    ZG_REQUIRE(dst && h && deg && src_indices && tgt_indices, "scatter_gcn_deg_scaled: null pointer");
-    if (int rc = check_gcn("scatter_gcn_deg_scaled", stride, n_edge, n_nodes)) return rc;
+    if (!(dst && h && deg && src_indices && tgt_indices)) {
+        set_error("scatter_gcn_deg_scaled: null pointer");
+        return owed(ZG_HIP_EINVAL);
+    }
+    if (int rc = check_gcn("scatter_gcn_deg_scaled", stride, n_edge, n_nodes)) return owed(rc);
     PlanRef pr;
     int rc = 0;
     if (!plan_from_cache(ctx, tgt_indices, src_indices, n_edge, n_nodes, &pr, &rc)) {
-        if (rc) return rc;
+        if (rc) return owed(rc);
         void* mem = workspace(ctx, plan_bytes(n_edge, n_nodes));
-        if (!mem) return ZG_HIP_EOOM;
+        if (!mem) return owed(ZG_HIP_EOOM);
         pr.plan = carve_plan(mem, n_edge, n_nodes);
-        if ((rc = build_plan(ctx, tgt_indices, pr.plan, src_indices))) return rc;
+        if ((rc = build_plan(ctx, tgt_indices, pr.plan, src_indices))) return owed(rc);
     }
-    const Plan& pl = pr.plan;
-    const int g = group_for(stride);
-    const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
-    ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, dst, h, deg,
-                                        pl.row_ptr, pl.peer, n_nodes, stride, false, (const float*)nullptr, false));
-    ZG_LAUNCH_CHECK();
+    // The plan is ready; the apply kernel waits for the layer's bias add and ReLU (examples/gcn/src/model.zig:100-112,
+    // :36), which become its tail.  Whatever else comes next launches it first.
+    zg_waiting_scatter& w = ctx->scatter_wait;
+    w = zg_waiting_scatter{};
+    w.active = true;
+    w.dst = dst;
+    w.h = h;
+    w.deg = deg;
+    w.row_ptr = pr.plan.row_ptr;
+    w.peer = pr.plan.peer;
+    w.n_nodes = n_nodes;
+    w.stride = stride;
+    w.fresh = fresh;
     return ZG_HIP_OK;
 }
 
@@ -1094,7 +1149,18 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
                                              const float* deg, const uint64_t* src_indices,
                                              const uint64_t* tgt_indices, float* grad_h, float* grad_deg, size_t stride,
                                              size_t n_edge, size_t n_nodes) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_FILLS(ctx);
+    // the zero fills of the two gradients (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: a gradient
+    // whose fill is taken over is written instead of added to zeros
+    const bool sized = n_edge > 0 && stride > 0 && n_nodes > 0;
+    const bool fresh_h = sized && grad_h && absorb_zero_fill(ctx, grad_h, n_nodes * stride);
+    const bool fresh_d = sized && grad_deg && absorb_zero_fill(ctx, grad_deg, n_nodes);
+    if (int rc = flush_pending(ctx)) {
+        if (fresh_h) (void)zg_hip_mem_fill(ctx, grad_h, n_nodes * stride, 0.f);
+        if (fresh_d) (void)zg_hip_mem_fill(ctx, grad_deg, n_nodes, 0.f);
+        return rc;
+    }
+    const int rc_body = [&]() -> int {
     if (n_edge == 0) return ZG_HIP_OK;
     ZG_REQUIRE(grad_output && h && deg && src_indices && tgt_indices && grad_h && grad_deg,
                "scatter_gcn_deg_scaled_bwd: null pointer");
@@ -1128,7 +1194,7 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
-                                        grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride, false));
+                                        grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride, fresh_h));
     ZG_LAUNCH_CHECK();
     if (by_incidence) {
         // 2 * n_edge terms in bucket order; the two separate term arrays' room holds them
@@ -1138,7 +1204,7 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
                            rs.entry->slot_of, terms, stride % 4 == 0 && aligned16(grad_output) && aligned16(h));
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0,
-                           ctx->stream, grad_deg, terms, rs.entry->inc.row_ptr, n_nodes, false);
+                           ctx->stream, grad_deg, terms, rs.entry->inc.row_ptr, n_nodes, fresh_d);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
@@ -1147,9 +1213,15 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     ZG_LAUNCH_CHECK();
     hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
                        grad_deg, term_src, term_tgt, by_src.row_ptr, by_src.perm, by_tgt.row_ptr, by_tgt.perm, n_nodes,
-                       false);
+                       fresh_d);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
+    }();
+    if (rc_body) {  // refused before its kernels ran: the zeros that were taken over are still owed
+        if (fresh_h) (void)zg_hip_mem_fill(ctx, grad_h, n_nodes * stride, 0.f);
+        if (fresh_d) (void)zg_hip_mem_fill(ctx, grad_deg, n_nodes, 0.f);
+    }
+    return rc_body;
 }
 
 // ------------------------------------------------------------------------------------------------

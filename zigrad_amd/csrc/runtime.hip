@@ -1073,6 +1073,8 @@ int flush_fills(zg_hip_ctx* ctx) {
 }
 int flush_pending(zg_hip_ctx* ctx) {
     // at most one kind is waiting at a time, except fills next to allocations: each kind's own calls send the others first
+    if (ctx->scatter_wait.active)
+        if (int rc = flush_scatter(ctx)) return rc;
     if (gemm_group_waiting(ctx))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (int rc = flush_fills(ctx)) return rc;

@@ -114,8 +114,10 @@ int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
  * tensor costs more than the fills.  Every later call on the context, zg_hip_sync, zg_hip_stream and a recording's
  * end included, therefore finds the memory filled; only work queued on the raw stream obtained EARLIER from
  * zg_hip_stream, with no call on the context in between, could overtake a waiting fill.  A waiting fill of +0.0 over
- * exactly the dense output of zg_hip_matmul / zg_hip_bmm_acc with beta = 1, or the gradient of zg_hip_smce_bwd, is not
- * launched at all: the op writes what it would have added to the zeros. */
+ * exactly the dense output of zg_hip_matmul / zg_hip_bmm_acc with beta = 1, the gradient of zg_hip_smce_bwd, the output
+ * of zg_hip_scatter_gcn_deg_scaled or a gradient of zg_hip_scatter_gcn_deg_scaled_bwd is not
+ * launched at all: the op writes what it would have added to the zeros; one over exactly the gradient of an optimizer
+ * step that is itself still waiting (zero_grad() after step()) is stored by the step's update kernel. */
 int zg_hip_mem_fill(zg_hip_ctx *ctx, float *x, size_t n, float value);
 int zg_hip_mem_fill_u8(zg_hip_ctx *ctx, void *x, size_t n, uint8_t value);
 int zg_hip_mem_fill_u64(zg_hip_ctx *ctx, uint64_t *x, size_t n, uint64_t value);
@@ -278,7 +280,12 @@ int zg_hip_index_select_fwd(zg_hip_ctx *ctx, const float *src, size_t src_len, c
                             size_t stride, float *dst);
 int zg_hip_index_select_bwd(zg_hip_ctx *ctx, const float *y_grad, const uint64_t *indices, size_t n_idx,
                             size_t stride, float *x_grad, size_t x_len);
-/* n_nodes = number of rows of dst/h (the reference derives it from the slices' lengths) */
+/* n_nodes = number of rows of dst/h (the reference derives it from the slices' lengths).
+ * Like the products (see zg_hip_matmul), the aggregation works with the calls around it: a waiting zero fill of exactly
+ * dst (or of exactly grad_h / grad_deg in the backward) is taken over and the sums are written instead of added to
+ * zeros; and the forward's kernel is launched by the NEXT call on the context: zg_hip_add of a row of `stride` values
+ * onto dst in place (y._add(bias), examples/gcn/src/model.zig:110) and zg_hip_relu_fwd of dst in place (:36) become the
+ * kernel's tail, any other call launches it first, unchanged.  Same values, bit for bit. */
 int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx *ctx, float *dst, const float *h, const float *deg,
                                   const uint64_t *src_indices, const uint64_t *tgt_indices, size_t stride,
                                   size_t n_edge, size_t n_nodes);

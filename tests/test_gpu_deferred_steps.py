@@ -167,3 +167,27 @@ def test_the_next_step_accumulates_into_gradients_zeroed_by_the_update_kernel(hi
     assert np.all(hip.to_numpy(gb) == 0.0)
     for t in (w, b, gw, gb, gyb, xb):
         hip.mem_free(t)
+
+
+def test_a_step_whose_tensors_overlap_a_waiting_steps_goes_after_it(hip):
+    """The gradient of one step is the parameter of the next (or overlaps it): the two must not share a launch."""
+    r = np.random.default_rng(29)
+    n = 640
+    init = [r.standard_normal(4096).astype(np.float32) for _ in range(3)]
+    outs = []
+    for eager in (False, True):
+        a, b, c = (hip.from_numpy(x) for x in init)
+        step = hip.sync if eager else (lambda: None)
+        hip.dispatch("sgd_step", param=a.sub(0, n), grad=b.sub(0, n), lr=0.01, clip=True, max_norm=10.0, delta=1e-6)
+        step()
+        hip.mem_fill(b.sub(0, n), 0.0)
+        step()
+        hip.dispatch("sgd_step", param=b, grad=c, lr=0.01, clip=True, max_norm=10.0, delta=1e-6)      # writes what the first reads
+        step()
+        hip.dispatch("sgd_step", param=c.sub(100, n), grad=a.sub(8, n), lr=0.01, clip=True, max_norm=10.0, delta=1e-6)
+        step()
+        outs.append([hip.to_numpy(t) for t in (a, b, c)])
+        for t in (a, b, c):
+            hip.mem_free(t)
+    for x, y in zip(*outs):
+        assert np.array_equal(x, y)

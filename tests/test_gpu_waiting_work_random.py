@@ -1,0 +1,243 @@
+"""Random call sequences against the work that waits inside the context (fills, products, bias gradients, optimizer
+steps, graph-convolution aggregations).  Whatever the order of calls and however their operands overlap, the memory a
+caller can observe must be what the same calls leave behind when every one of them is launched on its own, which a
+synchronisation after each call forces.  Seeded; every buffer is compared bit for bit at the end of a sequence and at
+random points inside it."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from zigrad_amd import host
+from zigrad_amd.device import F32, U64
+
+pytestmark = pytest.mark.gpu
+
+N_BUF = 10
+BUF_LEN = 64 * 64   # every buffer can hold a 64 x 64 matrix
+DIMS = [1, 7, 16, 32, 33, 64]
+
+
+class _Run:
+    def __init__(self, hip, seed, eager):
+        self.hip, self.eager = hip, eager
+        self.r = np.random.default_rng(seed)             # the same stream of choices in both runs
+        init = np.random.default_rng(seed + 10_000)
+        self.bufs = [hip.from_numpy((init.standard_normal(BUF_LEN) * 0.1).astype(np.float32)) for _ in range(N_BUF)]
+        # Adam's moments live in buffers of their own (the second moment must stay non-negative)
+        self.moments = [(hip.from_numpy(np.zeros(BUF_LEN, np.float32)), hip.from_numpy(np.zeros(BUF_LEN, np.float32)))
+                        for _ in range(3)]
+        self.temps = []                                   # cache allocations that are alive
+        n_nodes, n_edge = 40, 150
+        self.graph = (n_nodes, n_edge)
+        self.src = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
+        self.tgt = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
+        self.reads = []
+        self.t = 0
+
+    def done(self):
+        if self.eager:
+            self.hip.sync()
+
+    def picks(self, *sizes):
+        """One view per size, each in a different buffer (or live temp), so the operands of one call never overlap;
+        calls that follow each other meet on the same buffers all the time."""
+        pool = list(self.bufs) + list(self.temps)
+        order = self.r.permutation(len(pool))
+        out, used = [], set()
+        for n in sizes:
+            for j in order:
+                if int(j) not in used and pool[int(j)].n >= n:
+                    used.add(int(j))
+                    b = pool[int(j)]
+                    off = int(self.r.integers(0, b.n - n + 1)) if self.r.random() < 0.3 else 0
+                    off -= off % 4
+                    out.append(b.sub(off, n))
+                    break
+            else:
+                raise AssertionError("no buffer left")
+        return out
+
+    def pick(self, n):
+        return self.picks(n)[0]
+
+    # ---- the calls -------------------------------------------------------------------------------------------------
+    def op_fill(self):
+        n = int(self.r.choice([1, 10, 64, 1024, BUF_LEN]))
+        v = float(self.r.choice([0.0, 0.0, 0.125, -0.0, 0.5]))
+        self.hip.mem_fill(self.pick(n), v)
+
+    def op_matmul(self):
+        m, n, k = (int(self.r.choice(DIMS)) for _ in range(3))
+        ta, tb = bool(self.r.integers(0, 2)), bool(self.r.integers(0, 2))
+        beta = float(self.r.choice([0.0, 1.0, 1.0]))
+        a, b, c = self.picks(m * k, k * n, m * n)
+        if self.r.random() < 0.5:
+            self.hip.mem_fill(c, 0.0)      # ensure_grad(0) before an accumulating product
+            self.done()
+        self.hip.dispatch("matmul", A=a, B=b, C=c, m=m, n=n, k=k, trans_a=ta, trans_b=tb, lda=(m if ta else k),
+                          ldb=(k if tb else n), ldc=n, alpha=1.0, beta=beta)
+        self.last_c = (c, m, n)
+
+    def op_add_row(self):
+        """A bias row onto the last product's output, or onto something else."""
+        m, n = int(self.r.choice(DIMS)), int(self.r.choice(DIMS))
+        c, row = self.picks(m * n, n)
+        if getattr(self, "last_c", None) is not None and self.r.random() < 0.7:
+            c, m, n = self.last_c
+            row = self.pick(n)
+            if row.ptr < c.ptr + 4 * c.n and c.ptr < row.ptr + 4 * row.n:
+                return
+        if self.r.random() < 0.5:
+            self.hip.dispatch("add", x=row, y=c, z=c)
+        else:
+            self.hip.dispatch("add", x=c, y=row, z=c)
+
+    def op_relu(self):
+        if getattr(self, "last_c", None) is not None and self.r.random() < 0.7:
+            c = self.last_c[0]
+        else:
+            c = self.pick(int(self.r.choice([64, 1024])))
+        other = self.pick(c.n)
+        if self.r.random() < 0.8 or (other.ptr < c.ptr + 4 * c.n and c.ptr < other.ptr + 4 * other.n):
+            self.hip.dispatch("relu_fwd", x=c, y=c)
+        else:
+            self.hip.dispatch("relu_fwd", x=c, y=other)
+
+    def op_relu_mask(self):
+        if getattr(self, "last_c", None) is not None and self.r.random() < 0.7:
+            g = self.last_c[0]
+        else:
+            g = self.pick(int(self.r.choice([64, 1024])))
+        x = self.pick(g.n)
+        if x.ptr < g.ptr + 4 * g.n and g.ptr < x.ptr + 4 * x.n:
+            return
+        self.hip.dispatch("relu_inplace_bwd", x=x, x_g=g)
+
+    def op_layer_backward(self):
+        """unbroadcast, zero fill, dX, dW, frees, mask: the reference's order, on random buffers."""
+        B, I, O = (int(self.r.choice([2, 16, 33, 64])) for _ in range(3))
+        g, w, x, gw, gb = self.picks(B * O, O * I, B * I, O * I, O)
+        g_temp = None
+        if self.r.random() < 0.5:          # the output gradient in a cache block that is freed before the mask arrives
+            g_temp = self.hip.mem_cache_alloc(F32, B * O)
+            self.hip.mem_copy(g, g_temp)
+            self.done()
+            g = g_temp
+        host.unbroadcast_(self.hip, g, [B, O], gb, [O], alpha=1.0, beta=1.0)
+        self.done()
+        gx = self.hip.mem_cache_alloc(F32, B * I)
+        self.hip.mem_fill(gx, 0.0)
+        self.done()
+        if self.r.random() < 0.8:
+            host.bmm_acc_(self.hip, g, [B, O], w, [O, I], gx, False, False, 1.0, 1.0)
+            self.done()
+        host.bmm_acc_(self.hip, g, [B, O], x, [B, I], gw, True, False, 1.0, 1.0)
+        self.done()
+        if g_temp is not None:
+            self.hip.mem_cache_free(g_temp)
+            self.done()
+        if self.r.random() < 0.7:
+            self.hip.dispatch("relu_inplace_bwd", x=x, x_g=gx)
+            self.done()
+        self.temps.append(gx)
+
+    def op_unbroadcast(self):
+        R, inner = int(self.r.choice([2, 16, 64])), int(self.r.choice([2, 10, 64]))
+        x, y = self.picks(R * inner, inner)
+        host.unbroadcast_(self.hip, x, [R, inner], y, [inner], alpha=1.0, beta=1.0)
+
+    def op_step(self):
+        n = int(self.r.choice([10, 640, BUF_LEN]))
+        i, j = (int(v) for v in self.r.choice(N_BUF, 2, replace=False))
+        p, g = self.bufs[i].sub(0, n), self.bufs[j].sub(0, n)
+        if self.r.random() < 0.5:
+            self.hip.dispatch("sgd_step", param=p, grad=g, lr=0.01, clip=True, max_norm=10.0, delta=1e-6)
+        else:
+            m, v = self.moments[int(self.r.integers(0, len(self.moments)))]
+            self.t += 1
+            self.hip.dispatch("adam_step", param=p, grad=g, m=m.sub(0, n), v=v.sub(0, n), t=self.t, lr=0.01, beta1=0.9,
+                              beta2=0.999, epsilon=1e-8, clip=True, max_norm=10.0, delta=1e-6)
+        if self.r.random() < 0.6:
+            self.done()
+            self.hip.mem_fill(g, 0.0)      # zero_grad() after step()
+
+    def op_scatter(self):
+        n_nodes, n_edge = self.graph
+        stride = int(self.r.choice([4, 7, 16]))
+        y, h, deg, bias = self.picks(n_nodes * stride, n_nodes * stride, n_nodes, stride)
+        if self.r.random() < 0.6:
+            self.hip.mem_fill(y, 0.0)
+            self.done()
+        self.hip.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg, src_indices=self.src, tgt_indices=self.tgt,
+                          stride=stride, n_edge=n_edge)
+        self.done()
+        if self.r.random() < 0.7:
+            self.hip.dispatch("add", x=bias, y=y, z=y)
+            self.done()
+        if self.r.random() < 0.5:
+            self.hip.dispatch("relu_fwd", x=y, y=y)
+
+    def op_alloc(self):
+        n = int(self.r.choice([16, 1024, BUF_LEN]))
+        t = self.hip.mem_cache_alloc(F32, n)
+        self.hip.mem_fill(t, float(self.r.choice([0.0, 0.25])))
+        self.temps.append(t)
+
+    def op_free(self):
+        if self.temps:
+            t = self.temps.pop(int(self.r.integers(0, len(self.temps))))
+            self.hip.mem_cache_free(t)
+
+    def op_copy(self):
+        n = int(self.r.choice([16, 1000, BUF_LEN]))
+        a, b = self.picks(n, n)
+        self.hip.mem_copy(a, b)
+
+    def op_elementwise(self):
+        n = int(self.r.choice([64, 1024, BUF_LEN]))
+        a, b = self.picks(n, n)
+        which = int(self.r.integers(0, 3))
+        if which == 0:
+            self.hip.dispatch("add", x=a, y=b, z=b)
+        elif which == 1:
+            self.hip.dispatch("mul", x=a, y=b, z=b)
+        else:
+            self.hip.dispatch("tanh_fwd", x=a, y=b)
+
+    def op_read(self):
+        self.reads.append(self.hip.to_numpy(self.bufs[int(self.r.integers(0, N_BUF))]).view(np.uint32).copy())
+
+    def run(self, n_ops):
+        ops = [self.op_fill, self.op_matmul, self.op_add_row, self.op_relu, self.op_relu_mask, self.op_layer_backward,
+               self.op_unbroadcast, self.op_step, self.op_scatter, self.op_alloc, self.op_free, self.op_read, self.op_copy,
+               self.op_elementwise]
+        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1], float)
+        for _ in range(n_ops):
+            ops[int(self.r.choice(len(ops), p=weights / weights.sum()))]()
+            self.done()
+        out = [self.hip.to_numpy(b).view(np.uint32).copy() for b in self.bufs]
+        for t in self.temps:
+            out.append(self.hip.to_numpy(t).view(np.uint32).copy())
+            self.hip.mem_cache_free(t)
+        for m, v in self.moments:
+            out += [self.hip.to_numpy(m).view(np.uint32).copy(), self.hip.to_numpy(v).view(np.uint32).copy()]
+        for b in self.bufs + [self.src, self.tgt] + [x for mv in self.moments for x in mv]:
+            self.hip.mem_free(b)
+        return out, self.reads
+
+
+@pytest.mark.parametrize("seed", range(200))
+def test_random_sequences_leave_what_one_launch_per_call_leaves(hip, seed):
+    in_use0 = hip.cache_stats()["bytes_in_use"]
+    lazy, lazy_reads = _Run(hip, seed, eager=False).run(80)
+    want, want_reads = _Run(hip, seed, eager=True).run(80)
+    assert len(lazy) == len(want) and len(lazy_reads) == len(want_reads)
+    if not all(np.all(np.isfinite(b.view(np.float32))) for b in want):
+        pytest.skip("the sequence overflowed: NaN payloads are not part of the contract")
+    for i, (a, b) in enumerate(zip(lazy_reads, want_reads)):
+        assert np.array_equal(a, b), f"seed {seed}: read {i} differs"
+    for i, (a, b) in enumerate(zip(lazy, want)):
+        assert np.array_equal(a, b), f"seed {seed}: buffer {i} differs in {np.count_nonzero(a != b)} elements"
+    hip.sync()
+    assert hip.cache_stats()["bytes_in_use"] == in_use0

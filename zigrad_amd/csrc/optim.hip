@@ -333,9 +333,18 @@ static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, floa
         if (int rc = flush_fills(ctx)) return rc;
     }
     zg_pending_steps& q = ctx->steps;
+    // a step that touches memory a waiting step touches (the same tensor again, or buffers that overlap in any way)
+    // must not share its launch: the waiting steps go first
     bool named = false;
-    for (int i = 0; i < q.count; i++)
-        named = named || q.p[i] == param || q.g[i] == grad || (kind && (q.m[i] == m || q.v[i] == v));
+    {
+        const float* mine[4] = {param, grad, kind ? m : nullptr, kind ? v : nullptr};
+        for (int i = 0; i < q.count && !named; i++) {
+            const float* theirs[4] = {q.p[i], q.g[i], q.kind ? q.m[i] : nullptr, q.kind ? q.v[i] : nullptr};
+            for (const float* a : mine)
+                for (const float* b : theirs)
+                    named = named || (a && b && a < b + q.n[i] && b < a + n);
+        }
+    }
     const bool same = q.count == 0 || (q.kind == kind && q.clip == clip && q.max_norm == max_norm && q.delta == delta &&
                                        (kind ? (q.b1 == b1 && q.b2 == b2 && q.eps == eps) : q.lr == lr));
     if (n > kMultiBigMax) {

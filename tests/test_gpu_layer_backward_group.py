@@ -229,3 +229,41 @@ def test_products_that_are_not_the_layers_own_send_the_bias_gradient_out_first(h
     assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
     for t in (g, gb, a, b, out):
         hip.mem_free(t)
+
+
+def test_a_mask_that_lies_in_the_weight_gradient_is_read_after_the_weight_gradient_is_written(hip):
+    """relu_inplace_bwd whose mask operand is the buffer the waiting weight-gradient product writes: the separate calls
+    mask by the NEW weight gradient, so the three must not leave in one launch with that mask."""
+    B = O = 32
+    I = 48
+    r = np.random.default_rng(12)
+    gy = r.standard_normal((B, O)).astype(np.float32)
+    w = r.standard_normal((O, I)).astype(np.float32)
+    x = r.standard_normal((B, I)).astype(np.float32)
+    gw0 = r.standard_normal((O, I)).astype(np.float32)
+    outs = []
+    for eager in (False, True):
+        step = hip.sync if eager else (lambda: None)
+        g, wb, xb, gwb = hip.from_numpy(gy), hip.from_numpy(w), hip.from_numpy(x), hip.from_numpy(gw0)
+        gb = hip.from_numpy(np.zeros(O, np.float32))
+        host.unbroadcast_(hip, g, [B, O], gb, [O], alpha=1.0, beta=1.0)
+        step()
+        gx = hip.mem_cache_alloc(F32, B * I)
+        hip.mem_fill(gx, 0.0)
+        step()
+        host.bmm_acc_(hip, g, [B, O], wb, [O, I], gx, False, False, 1.0, 1.0)
+        step()
+        host.bmm_acc_(hip, g, [B, O], xb, [B, I], gwb, True, False, 1.0, 1.0)
+        step()
+        hip.dispatch("relu_inplace_bwd", x=gwb, x_g=gx)      # O * I == B * I: the weight gradient as the mask
+        step()
+        outs.append((hip.to_numpy(gx), hip.to_numpy(gwb), hip.to_numpy(gb)))
+        hip.mem_cache_free(gx)
+        for t in (g, wb, xb, gwb, gb):
+            hip.mem_free(t)
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
+    new_gw = gy.astype(np.float64).T @ x.astype(np.float64) + gw0
+    want = np.where(new_gw.ravel() > 0, (gy.astype(np.float64) @ w.astype(np.float64)).ravel(), 0.0)
+    sure = np.abs(new_gw.ravel()) > 1e-4          # away from the mask's threshold, where rounding cannot flip it
+    assert np.allclose(outs[0][0][sure], want[sure], rtol=1e-4, atol=1e-5)

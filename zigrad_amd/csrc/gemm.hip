@@ -1568,7 +1568,14 @@ bool deferred_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t 
 bool deferred_take_relu_mask(zg_hip_ctx* ctx, const float* x, const float* x_g, size_t n, int* rc) {
     zg_deferred_gemm& d = ctx->deferred;
     if (!d.active || d.kind != 2 || d.gate || x_g != d.C || n != d.m * d.n || !x) return false;
-    if (ranges_meet(operand_range(x, d.m, d.n, d.n), operand_range(d.C, d.m, d.n, d.ldc))) return false;
+    const ByteRange xr = operand_range(x, d.m, d.n, d.n);
+    if (ranges_meet(xr, operand_range(d.C, d.m, d.n, d.ldc))) return false;
+    // a mask that lies in what the weight-gradient product or the bias gradient of the same launch write must be
+    // read after they ran: then the mask is not taken over and the call sends everything out first
+    if (ctx->deferred_w.active && ranges_meet(xr, product_c_range(ctx->deferred_w))) return false;
+    if (ctx->bias_wait.active &&
+        ranges_meet(xr, operand_range(ctx->bias_wait.gb, 1, ctx->bias_wait.inner, ctx->bias_wait.inner)))
+        return false;
     d.gate = x;
     *rc = flush_deferred_gemm(ctx);
     return true;

@@ -8,8 +8,10 @@
 
 namespace zg {
 
+// zero_g: the gradient is left zero instead of clipped (zero_grad() right after step(): one pass less over it)
 template <bool CLIP>
-__global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, size_t n, float nlr, const float* factor) {
+__global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, size_t n, float nlr, const float* factor,
+                                                      bool zero_g) {
     const float f = CLIP ? factor[0] : 1.0f;
     const bool scale = CLIP && (f != 1.0f);
     const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g)) & 15u) == 0;
@@ -25,8 +27,9 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, size_t 
                 gv.y = __fmul_rn(gv.y, f);
                 gv.z = __fmul_rn(gv.z, f);
                 gv.w = __fmul_rn(gv.w, f);
-                g4[i] = gv;
+                if (!zero_g) g4[i] = gv;
             }
+            if (zero_g) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             pv.x = __fadd_rn(pv.x, __fmul_rn(nlr, gv.x));
             pv.y = __fadd_rn(pv.y, __fmul_rn(nlr, gv.y));
             pv.z = __fadd_rn(pv.z, __fmul_rn(nlr, gv.z));
@@ -39,8 +42,9 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, size_t 
         float gv = g[i];
         if (scale) {
             gv = __fmul_rn(gv, f);
-            g[i] = gv;
+            if (!zero_g) g[i] = gv;
         }
+        if (zero_g) g[i] = 0.f;
         p[i] = __fadd_rn(p[i], __fmul_rn(nlr, gv));
     }
 }
@@ -57,7 +61,8 @@ __device__ __forceinline__ void adam_elem(float& p, float& g, float& m, float& v
 template <bool CLIP>
 __global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float* m, float* v, size_t n,
                                                        float lr_t_value, const float* lr_t_ptr, float b1, float b2,
-                                                       float omb1, float omb2, float eps, const float* factor) {
+                                                       float omb1, float omb2, float eps, const float* factor,
+                                                       bool zero_g) {
     const float lr_t = lr_t_ptr ? lr_t_ptr[0] : lr_t_value;
     const float f = CLIP ? factor[0] : 1.0f;
     const bool scale = CLIP && (f != 1.0f);
@@ -76,7 +81,8 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float*
             adam_elem(pv.y, gv.y, mv.y, vv.y, scale, f, lr_t, b1, b2, omb1, omb2, eps);
             adam_elem(pv.z, gv.z, mv.z, vv.z, scale, f, lr_t, b1, b2, omb1, omb2, eps);
             adam_elem(pv.w, gv.w, mv.w, vv.w, scale, f, lr_t, b1, b2, omb1, omb2, eps);
-            if (scale) g4[i] = gv;
+            if (zero_g) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            else if (scale) g4[i] = gv;
             m4[i] = mv;
             v4[i] = vv;
             p4[i] = pv;
@@ -86,7 +92,8 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* p, float* g, float*
     for (size_t i = tid; i < n; i += nt) {
         float pv = p[i], gv = g[i], mv = m[i], vv = v[i];
         adam_elem(pv, gv, mv, vv, scale, f, lr_t, b1, b2, omb1, omb2, eps);
-        if (scale) g[i] = gv;
+        if (zero_g) g[i] = 0.f;
+        else if (scale) g[i] = gv;
         m[i] = mv;
         v[i] = vv;
         p[i] = pv;
@@ -178,15 +185,35 @@ struct MultiArgs {
     int wg_first[kMultiMax + 1]; // update_multi_kernel: tensor b owns workgroups wg_first[b] .. wg_first[b + 1] - 1
     const float* lr_t_mem[kMultiMax];  // Adam under replay: *lr_t_mem[b] is read when the kernel runs (null: use lr_t[b])
     float* factors;              // clip factor per tensor, written by norm_multi_kernel
+    float* partials[kMultiMax];  // tensors beyond kFlatSingleMax: the first-stage sums of norm_partials_multi_kernel
+    int n_partials[kMultiMax];   //   and how many (0: the tensor's norm is formed by one workgroup)
+    int part_first[kMultiMax + 1];  // norm_partials_multi_kernel: tensor b owns workgroups part_first[b] .. part_first[b + 1] - 1
     float b1, b2, omb1, omb2, eps, max_norm, delta;
     int clip, zero_grads, count;
 };
 
+// First stage of the squared norms of the tensors beyond kFlatSingleMax, all in one launch: each workgroup runs the
+// block of flat_partial_kernel it would run in the tensor's own launch.
+__global__ __launch_bounds__(kFlatBlock) void norm_partials_multi_kernel(MultiArgs a) {
+    __shared__ float smem[kFlatBlock / kWave];
+    int b = 0;
+    while (b + 1 < a.count && (int)blockIdx.x >= a.part_first[b + 1]) b++;
+    flat_partial_block<TermSq, 1>(a.g[b], nullptr, a.n[b], 0.f, a.partials[b], (size_t)((int)blockIdx.x - a.part_first[b]),
+                                  (size_t)a.n_partials[b], smem);
+}
+
 __global__ __launch_bounds__(kFlatSingle) void norm_multi_kernel(MultiArgs a) {
     __shared__ float smem[kFlatSingle / kWave];
     const int b = blockIdx.x;
-    if (a.n[b] > kFlatSingleMax) return;  // its factor came from the two-stage reduction, launched before this kernel
-    float acc = flat_accumulate<TermSq, 1>(a.g[b], nullptr, a.n[b], 0.f, threadIdx.x, blockDim.x);
+    float acc = 0.f;
+    if (a.n_partials[b]) {
+        // the second stage as flat_final_kernel runs it: kFlatBlock threads gather, the others hold zeros, which
+        // leave every sum of the combine tree as it is
+        if (threadIdx.x < kFlatBlock)
+            for (int i = threadIdx.x; i < a.n_partials[b]; i += kFlatBlock) acc = SumAcc::combine(acc, a.partials[b][i]);
+    } else {
+        acc = flat_accumulate<TermSq, 1>(a.g[b], nullptr, a.n[b], 0.f, threadIdx.x, blockDim.x);
+    }
     acc = block_reduce<SumAcc>(acc, smem);
     if (threadIdx.x == 0) FinClipFactor{a.factors + b, a.max_norm, a.delta}(acc);
 }
@@ -227,10 +254,10 @@ static int sgd_launch(zg_hip_ctx* ctx, float* param, float* grad, size_t n, floa
         int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
         if (rc) return rc;
         hipLaunchKernelGGL((sgd_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, n,
-                           -lr, factor);
+                           -lr, factor, false);
     } else {
         hipLaunchKernelGGL((sgd_kernel<false>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad,
-                           n, -lr, factor);
+                           n, -lr, factor, false);
     }
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
@@ -254,10 +281,10 @@ static int adam_launch(zg_hip_ctx* ctx, float* param, float* grad, float* m, flo
         int rc = flat_reduce<TermSq, 1>(ctx, grad, nullptr, n, 0.f, FinClipFactor{factor, max_norm, delta});
         if (rc) return rc;
         hipLaunchKernelGGL((adam_kernel<true>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad, m,
-                           v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, factor);
+                           v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, factor, false);
     } else {
         hipLaunchKernelGGL((adam_kernel<false>), dim3(update_grid(ctx, n)), dim3(kBlock), 0, ctx->stream, param, grad,
-                           m, v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, factor);
+                           m, v, n, lr_t, lr_t_ptr, beta1, beta2, omb1, omb2, epsilon, factor, false);
     }
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
@@ -321,9 +348,8 @@ int flush_steps(zg_hip_ctx* ctx, bool requeue_fills) {
 }
 }  // namespace zg
 
-// One optimizer step of one tensor.  Up to 2^20 elements it joins the waiting steps when it has their settings and names
-// none of their tensors (otherwise they are sent first); a larger tensor is launched at once, ahead of waiting steps
-// that do not name it.
+// One optimizer step of one tensor.  It joins the waiting steps when it has their settings and touches none of their
+// tensors (otherwise they are sent first).
 static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, float* m, float* v, size_t n, float lr,
                       float lr_t, const float* lr_t_mem, float b1, float b2, float eps, int clip, float max_norm,
                       float delta) {
@@ -347,12 +373,6 @@ static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, floa
     }
     const bool same = q.count == 0 || (q.kind == kind && q.clip == clip && q.max_norm == max_norm && q.delta == delta &&
                                        (kind ? (q.b1 == b1 && q.b2 == b2 && q.eps == eps) : q.lr == lr));
-    if (n > kMultiBigMax) {
-        if (named)
-            if (int rc = flush_steps(ctx)) return rc;
-        if (kind == 0) return sgd_launch(ctx, param, grad, n, lr, clip, max_norm, delta);
-        return adam_launch(ctx, param, grad, m, v, n, lr_t, lr_t_mem, b1, b2, eps, clip, max_norm, delta);
-    }
     if (named || !same || q.count == kMaxPendingSteps)
         if (int rc = flush_steps(ctx)) return rc;
     if (q.count == 0) {
@@ -411,9 +431,10 @@ ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float
 }
 
 // Parameter lists (the tensors are independent, so the launches need not follow the list order; a tensor listed
-// twice is the exception and is handled below): tensors of up to kMultiBigMax elements share the update launch (those beyond kFlatSingleMax get
-// their clip factor from the two-stage norm reduction of the per-tensor path first, so the values stay the same);
-// larger ones take the per-tensor path with its 16-byte grid-stride kernels.
+// twice is the exception and is handled below): the clip factors of all tensors of a batch come from two launches (the
+// first stage of the two-stage norm of every tensor beyond kFlatSingleMax, with the blocks and the combine tree of the
+// per-tensor path, then one workgroup per tensor), tensors of up to kMultiBigMax elements share the update launch, and
+// larger ones take the per-tensor update kernels with their 16-byte grid-stride walks.
 static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_tensors, float* const* params,
                       float* const* grads, float* const* ms, float* const* vs, const size_t* lens, const float* lr_t,
                       int lr_t_in_memory, float lr, float beta1, float beta2, float epsilon, int clip, float max_norm,
@@ -422,18 +443,53 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
     ZG_REQUIRE(!adam || n_tensors == 0 || (ms && vs && lr_t), "%s: null list", name);
     MultiArgs a;
     int filled = 0;
+    size_t partials_used = 0;  // floats of the context's partials buffer handed to this batch
+    const size_t partials_room = ((size_t)64 << 10) / sizeof(float);
+    // One batch: the first stage of the norms of its larger tensors (one launch), every tensor's clip factor (one
+    // launch), the update of the tensors of up to kMultiBigMax elements in slices (one launch), and the update of
+    // each larger tensor by the per-tensor kernel, which reads its factor from the batch's slot.
     auto flush = [&]() -> int {
         if (!filled) return ZG_HIP_OK;
         a.count = filled;
         if (clip) {
+            if (a.part_first[filled] > 0) {
+                hipLaunchKernelGGL(norm_partials_multi_kernel, dim3((unsigned)a.part_first[filled]), dim3(kFlatBlock), 0,
+                                   ctx->stream, a);
+                ZG_LAUNCH_CHECK();
+            }
             hipLaunchKernelGGL(norm_multi_kernel, dim3(filled), dim3(kFlatSingle), 0, ctx->stream, a);
             ZG_LAUNCH_CHECK();
         }
         const unsigned grid = (unsigned)a.wg_first[filled];
-        if (adam) hipLaunchKernelGGL((update_multi_kernel<true>), dim3(grid), dim3(kMultiThreads), 0, ctx->stream, a);
-        else hipLaunchKernelGGL((update_multi_kernel<false>), dim3(grid), dim3(kMultiThreads), 0, ctx->stream, a);
+        if (grid) {
+            if (adam) hipLaunchKernelGGL((update_multi_kernel<true>), dim3(grid), dim3(kMultiThreads), 0, ctx->stream, a);
+            else hipLaunchKernelGGL((update_multi_kernel<false>), dim3(grid), dim3(kMultiThreads), 0, ctx->stream, a);
+            ZG_LAUNCH_CHECK();
+        }
+        for (int b = 0; b < filled; b++) {
+            const size_t n = a.n[b];
+            if (n <= kMultiBigMax) continue;
+            const float* factor = a.factors + b;
+            const dim3 g(update_grid(ctx, n)), t(kBlock);
+            if (adam) {
+                if (clip)
+                    hipLaunchKernelGGL((adam_kernel<true>), g, t, 0, ctx->stream, a.p[b], a.g[b], a.m[b], a.v[b], n, a.lr_t[b],
+                                       a.lr_t_mem[b], a.b1, a.b2, a.omb1, a.omb2, a.eps, factor, zero_grads != 0);
+                else
+                    hipLaunchKernelGGL((adam_kernel<false>), g, t, 0, ctx->stream, a.p[b], a.g[b], a.m[b], a.v[b], n, a.lr_t[b],
+                                       a.lr_t_mem[b], a.b1, a.b2, a.omb1, a.omb2, a.eps, factor, zero_grads != 0);
+            } else {
+                if (clip)
+                    hipLaunchKernelGGL((sgd_kernel<true>), g, t, 0, ctx->stream, a.p[b], a.g[b], n, a.lr_t[b], factor,
+                                       zero_grads != 0);
+                else
+                    hipLaunchKernelGGL((sgd_kernel<false>), g, t, 0, ctx->stream, a.p[b], a.g[b], n, a.lr_t[b], factor,
+                                       zero_grads != 0);
+            }
+            ZG_LAUNCH_CHECK();
+        }
         filled = 0;
-        ZG_LAUNCH_CHECK();
+        partials_used = 0;
         return ZG_HIP_OK;
     };
     a.b1 = beta1;
@@ -447,6 +503,7 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
     a.zero_grads = zero_grads;
     a.factors = ctx->scalar_slot + 16;  // kMultiMax floats of the context's 64
     a.wg_first[0] = 0;
+    a.part_first[0] = 0;
     for (size_t i = 0; i < n_tensors; i++) {
         const size_t n = lens[i];
         if (n == 0) continue;
@@ -454,35 +511,24 @@ static int step_multi(zg_hip_ctx* ctx, const char* name, bool adam, size_t n_ten
         // a tensor that is listed twice is updated twice, in list order: the second update waits for the first
         bool listed = false;
         for (int b = 0; b < filled; b++) listed = listed || a.p[b] == params[i] || a.g[b] == grads[i];
-        if (listed)
+        const size_t parts = (clip && n > kFlatSingleMax) ? flat_partial_blocks(ctx, n) : 0;
+        if (listed || partials_used + parts > partials_room)
             if (int rc = flush()) return rc;
-        if (n <= kMultiBigMax) {
-            if (clip && n > kFlatSingleMax) {
-                int rc = flat_reduce<TermSq, 1>(ctx, grads[i], nullptr, n, 0.f,
-                                                FinClipFactor{a.factors + filled, max_norm, delta});
-                if (rc) return rc;
-            }
-            a.p[filled] = params[i];
-            a.g[filled] = grads[i];
-            a.m[filled] = adam ? ms[i] : nullptr;
-            a.v[filled] = adam ? vs[i] : nullptr;
-            a.n[filled] = n;
-            a.lr_t[filled] = adam ? (lr_t_in_memory ? 0.f : lr_t[i]) : -lr;
-            a.lr_t_mem[filled] = (adam && lr_t_in_memory) ? lr_t + i : nullptr;
-            a.wg_first[filled + 1] = a.wg_first[filled] + (int)ceil_div_sz(n, kMultiSlice);
-            if (++filled == kMultiMax)
-                if (int rc = flush()) return rc;
-            continue;
-        }
-        int rc;
-        if (adam)
-            rc = adam_launch(ctx, params[i], grads[i], ms[i], vs[i], n, lr_t_in_memory ? 0.f : lr_t[i],
-                             lr_t_in_memory ? lr_t + i : nullptr, beta1, beta2, epsilon, clip, max_norm, delta);
-        else
-            rc = sgd_launch(ctx, params[i], grads[i], n, lr, clip, max_norm, delta);
-        if (rc) return rc;
-        if (zero_grads)
-            if ((rc = zg_hip_mem_fill(ctx, grads[i], n, 0.f))) return rc;
+        a.p[filled] = params[i];
+        a.g[filled] = grads[i];
+        a.m[filled] = adam ? ms[i] : nullptr;
+        a.v[filled] = adam ? vs[i] : nullptr;
+        a.n[filled] = n;
+        a.lr_t[filled] = adam ? (lr_t_in_memory ? 0.f : lr_t[i]) : -lr;
+        a.lr_t_mem[filled] = (adam && lr_t_in_memory) ? lr_t + i : nullptr;
+        a.partials[filled] = parts ? (float*)ctx->partials + partials_used : nullptr;
+        a.n_partials[filled] = (int)parts;
+        a.part_first[filled + 1] = a.part_first[filled] + (int)parts;
+        partials_used += parts;
+        // tensors beyond kMultiBigMax keep the per-tensor update kernels (16-byte grid-stride walks): no slices
+        a.wg_first[filled + 1] = a.wg_first[filled] + (n <= kMultiBigMax ? (int)ceil_div_sz(n, kMultiSlice) : 0);
+        if (++filled == kMultiMax)
+            if (int rc = flush()) return rc;
     }
     return flush();
 }

@@ -249,18 +249,20 @@ __global__ __launch_bounds__(kFlatSingle) void flat_single_kernel(const float* a
 // DRAM pages open, which a grid-stride walk of the whole array does not (67 MB of squares: 18 -> 11 us).
 constexpr int kFlatU = 4;
 constexpr size_t kFlatChunk = (size_t)kFlatBlock * kFlatU;
+// Workgroup `block` of `nblocks` of that stage (a device function so that a launch over several arrays can run the
+// same blocks, see optim.hip).
 template <class T, int NIN>
-__global__ __launch_bounds__(kFlatBlock) void flat_partial_kernel(const float* a, const float* b, size_t n, float p0,
-                                                                   typename T::P::Acc* partials) {
+__device__ __forceinline__ void flat_partial_block(const float* a, const float* b, size_t n, float p0,
+                                                   typename T::P::Acc* partials, size_t block, size_t nblocks,
+                                                   typename T::P::Acc* smem) {
     using P = typename T::P;
-    __shared__ typename P::Acc smem[kFlatBlock / kWave];
     typename P::Acc acc = P::init();
     const bool vec = ((reinterpret_cast<uintptr_t>(a) | (NIN > 1 ? reinterpret_cast<uintptr_t>(b) : 0)) & 15u) == 0;
     if (vec) {
         const size_t n4 = n >> 2;
         const float4* a4 = reinterpret_cast<const float4*>(a);
         const float4* b4 = reinterpret_cast<const float4*>(b);
-        for (size_t c0 = (size_t)blockIdx.x * kFlatChunk; c0 < n4; c0 += (size_t)gridDim.x * kFlatChunk) {
+        for (size_t c0 = block * kFlatChunk; c0 < n4; c0 += nblocks * kFlatChunk) {
             float4 u[kFlatU], w[kFlatU];
 #pragma unroll
             for (int k = 0; k < kFlatU; k++) {
@@ -283,15 +285,21 @@ __global__ __launch_bounds__(kFlatBlock) void flat_partial_kernel(const float* a
                 }
             }
         }
-        const size_t tid = (size_t)blockIdx.x * kFlatBlock + threadIdx.x, nthreads = (size_t)gridDim.x * kFlatBlock;
+        const size_t tid = block * kFlatBlock + threadIdx.x, nthreads = nblocks * kFlatBlock;
         for (size_t t = (n4 << 2) + tid; t < n; t += nthreads)
             acc = P::combine(acc, T::term(a[t], NIN > 1 ? b[t] : 0.f, t, p0));
     } else {
-        acc = flat_accumulate<T, NIN>(a, b, n, p0, (size_t)blockIdx.x * kFlatBlock + threadIdx.x,
-                                      (size_t)gridDim.x * kFlatBlock);
+        acc = flat_accumulate<T, NIN>(a, b, n, p0, block * kFlatBlock + threadIdx.x, nblocks * kFlatBlock);
     }
     acc = block_reduce<P>(acc, smem);
-    if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+    if (threadIdx.x == 0) partials[block] = acc;
+}
+
+template <class T, int NIN>
+__global__ __launch_bounds__(kFlatBlock) void flat_partial_kernel(const float* a, const float* b, size_t n, float p0,
+                                                                   typename T::P::Acc* partials) {
+    __shared__ typename T::P::Acc smem[kFlatBlock / kWave];
+    flat_partial_block<T, NIN>(a, b, n, p0, partials, blockIdx.x, gridDim.x, smem);
 }
 
 template <class P, class Fin>
@@ -302,6 +310,14 @@ __global__ __launch_bounds__(kFlatBlock) void flat_final_kernel(const typename P
     for (int i = threadIdx.x; i < n_partials; i += kFlatBlock) acc = P::combine(acc, partials[i]);
     acc = block_reduce<P>(acc, smem);
     if (threadIdx.x == 0) fin(acc);
+}
+
+// Workgroups of the first stage for n elements: one chunk per workgroup until the partials buffer is full.
+static inline size_t flat_partial_blocks(const zg_hip_ctx* ctx, size_t n) {
+    size_t blocks = ceil_div_sz(n, kFlatChunk * 4);
+    size_t cap = (size_t)ctx->n_cu * 8;
+    if (cap > (size_t)kMaxPartials) cap = kMaxPartials;
+    return blocks > cap ? cap : blocks;
 }
 
 // `partials` holds the per-workgroup results of the two-launch form: room for kMaxPartials accumulators.
@@ -315,10 +331,7 @@ static int flat_reduce_into(zg_hip_ctx* ctx, const float* a, const float* b, siz
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    size_t blocks = ceil_div_sz(n, kFlatChunk * 4);  // one chunk per workgroup until the partials buffer is full
-    size_t cap = (size_t)ctx->n_cu * 8;
-    if (cap > (size_t)kMaxPartials) cap = kMaxPartials;
-    if (blocks > cap) blocks = cap;
+    const size_t blocks = flat_partial_blocks(ctx, n);
     static_assert(kMaxPartials * sizeof(typename P::Acc) <= (64 << 10), "partials buffer too small");
     auto* partials = (typename P::Acc*)partials_mem;
     hipLaunchKernelGGL((flat_partial_kernel<T, NIN>), dim3((unsigned)blocks), dim3(kFlatBlock), 0, ctx->stream, a, b, n,

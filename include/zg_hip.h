@@ -382,10 +382,11 @@ int zg_hip_mse_bwd(zg_hip_ctx *ctx, const float *pred, const float *target, floa
  * optimizers: src/nn/optim.zig:100-122 (SGD.update) and :177-234 (Adam.update) as one op per
  * parameter tensor.  `clip` != 0 applies the reference's per-tensor clip_nrm2 to grad first
  * (grad is modified in place, as in the reference).
- * A step of a tensor of up to 2^20 elements is not launched by its own call: it waits while the calls that follow are
- * more steps with the same settings on other tensors (an optimizer walks its parameter list) and the run then leaves in
- * the two launches of the parameter-list kernels below; any other call on the context launches what is waiting first.
- * Same values, bit for bit, as a launch per call.
+ * A step is not launched by its own call: it waits while the calls that follow are more steps with the same settings
+ * on tensors that do not overlap the waiting ones (an optimizer walks its parameter list), and the run then leaves
+ * through the parameter-list kernels below (the clip factors of all tensors in two launches, then the updates); a
+ * zero fill of exactly a waiting step's gradient (zero_grad() after step()) is stored by its update kernel; any other
+ * call on the context launches what is waiting first.  Same values, bit for bit, as a launch per call.
  * ------------------------------------------------------------------------------------------- */
 int zg_hip_sgd_step(zg_hip_ctx *ctx, float *param, float *grad, size_t n, float lr, int clip, float max_norm,
                     float delta);

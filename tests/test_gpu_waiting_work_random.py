@@ -19,8 +19,8 @@ DIMS = [1, 7, 16, 32, 33, 64]
 
 
 class _Run:
-    def __init__(self, hip, seed, eager):
-        self.hip, self.eager = hip, eager
+    def __init__(self, hip, seed, eager, reads=True):
+        self.hip, self.eager, self.seed, self.with_reads = hip, eager, seed, reads
         self.r = np.random.default_rng(seed)             # the same stream of choices in both runs
         init = np.random.default_rng(seed + 10_000)
         self.bufs = [hip.from_numpy((init.standard_normal(BUF_LEN) * 0.1).astype(np.float32)) for _ in range(N_BUF)]
@@ -206,9 +206,15 @@ class _Run:
             self.hip.dispatch("tanh_fwd", x=a, y=b)
 
     def op_read(self):
+        if not self.with_reads:
+            return
         self.reads.append(self.hip.to_numpy(self.bufs[int(self.r.integers(0, N_BUF))]).view(np.uint32).copy())
 
-    def run(self, n_ops):
+    def ops(self, n_ops):
+        """The sequence of this run's seed, from the start: every call of ops() makes the same choices."""
+        self.r = np.random.default_rng(self.seed)
+        self.t = 0
+        self.last_c = None
         ops = [self.op_fill, self.op_matmul, self.op_add_row, self.op_relu, self.op_relu_mask, self.op_layer_backward,
                self.op_unbroadcast, self.op_step, self.op_scatter, self.op_alloc, self.op_free, self.op_read, self.op_copy,
                self.op_elementwise]
@@ -216,15 +222,27 @@ class _Run:
         for _ in range(n_ops):
             ops[int(self.r.choice(len(ops), p=weights / weights.sum()))]()
             self.done()
+        self.kept = list(self.temps)
+
+    def free_temps(self):
+        for t in self.temps:
+            self.hip.mem_cache_free(t)
+        self.temps = []
+
+    def finish(self):
         out = [self.hip.to_numpy(b).view(np.uint32).copy() for b in self.bufs]
         for t in self.temps:
             out.append(self.hip.to_numpy(t).view(np.uint32).copy())
-            self.hip.mem_cache_free(t)
+        self.free_temps()
         for m, v in self.moments:
             out += [self.hip.to_numpy(m).view(np.uint32).copy(), self.hip.to_numpy(v).view(np.uint32).copy()]
         for b in self.bufs + [self.src, self.tgt] + [x for mv in self.moments for x in mv]:
             self.hip.mem_free(b)
         return out, self.reads
+
+    def run(self, n_ops):
+        self.ops(n_ops)
+        return self.finish()
 
 
 @pytest.mark.parametrize("seed", range(200))
@@ -238,6 +256,40 @@ def test_random_sequences_leave_what_one_launch_per_call_leaves(hip, seed):
     for i, (a, b) in enumerate(zip(lazy_reads, want_reads)):
         assert np.array_equal(a, b), f"seed {seed}: read {i} differs"
     for i, (a, b) in enumerate(zip(lazy, want)):
+        assert np.array_equal(a, b), f"seed {seed}: buffer {i} differs in {np.count_nonzero(a != b)} elements"
+    hip.sync()
+    assert hip.cache_stats()["bytes_in_use"] == in_use0
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_recorded_random_sequences_replay_what_the_eager_calls_leave(hip, seed):
+    """The same sequences recorded as an execution graph (nothing runs while recording; waiting work is launched into
+    the recording) and replayed three times, against the same calls issued three times with one launch per call."""
+    n_ops, reps = 50, 3
+    in_use0 = hip.cache_stats()["bytes_in_use"]
+    eager = _Run(hip, seed, eager=True, reads=False)
+    for _ in range(reps):
+        eager.ops(n_ops)
+        eager.free_temps()
+    want, _ = eager.finish()
+    rec = _Run(hip, seed, eager=False, reads=False)
+    rec.ops(n_ops)          # once eagerly: the allocator and the workspace reach their final size
+    rec.free_temps()
+    hip.sync()
+    hip.graph_open()
+    try:
+        rec.ops(n_ops)
+        rec.free_temps()
+    finally:
+        graph = hip.graph_save()
+    for _ in range(reps - 1):
+        graph.run()
+    hip.sync()
+    got, _ = rec.finish()
+    graph.free()
+    if not all(np.all(np.isfinite(b.view(np.float32))) for b in want):
+        pytest.skip("the sequence overflowed: NaN payloads are not part of the contract")
+    for i, (a, b) in enumerate(zip(got, want)):
         assert np.array_equal(a, b), f"seed {seed}: buffer {i} differs in {np.count_nonzero(a != b)} elements"
     hip.sync()
     assert hip.cache_stats()["bytes_in_use"] == in_use0

@@ -360,7 +360,9 @@ int zg_hip_smce_label_fwd(zg_hip_ctx *ctx, const float *logits, const uint64_t *
  * the process ends) instead of the context's grow-only workspace.  At most 262144 rows; more is rejected with
  * ZG_HIP_EINVAL before any launch.  Same kernels and the same values as zg_hip_smce_label_fwd.  All calls on one GPU
  * share the array: calls that overlap on one GPU (two contexts, two streams) race; calls on one context are ordered
- * by its stream. */
+ * by its stream.  Work that earlier calls left waiting in the context (see zg_hip_mem_fill, zg_hip_matmul) is launched
+ * first, as by every call; it needs no memory either: what a waiting product uses was reserved by the call that
+ * queued it. */
 int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx *ctx, const float *logits, const uint64_t *labels, float *lse,
                                   float *loss, size_t rows, size_t cols);
 /* accumulate != 0: grad += (p - onehot)/rows (the reference's `+=`, src/nn/loss.zig:157);

@@ -87,3 +87,43 @@ def test_noalloc_makes_no_device_allocation(hip):
             dev.mem_free(b)
     finally:
         dev.deinit()
+
+
+def test_noalloc_launches_waiting_work_without_allocating():
+    """A product whose k is cut over workgroups (its partial tiles live in the context's workspace) is queued and
+    still waiting when the allocation-free entry point is called: the entry point launches it first.  The workspace
+    the product needs was reserved by the call that queued it, so the allocation-free call makes no driver allocation
+    (it reports one if it happens), and both results are right.  A context of its own: its workspace starts empty."""
+    from zigrad_amd.device import F32, U64, HipDevice
+
+    dev = HipDevice(0)
+    try:
+        r = np.random.default_rng(5)
+        m, n, k = 256, 1024, 16384          # eight large tiles: k is cut, tens of MB of partial tiles
+        assert dev.gemm_plan(m, n, k, 1)["kind"] == "split_k"
+        A = (r.standard_normal((m, k)) * 0.1).astype(np.float32)
+        W = (r.standard_normal((n, k)) * 0.1).astype(np.float32)
+        a, w = dev.from_numpy(A), dev.from_numpy(W)
+        c = dev.mem_alloc(F32, m * n)
+        rows, cols = 3000, 50
+        x, lab = _case(7, rows, cols)
+        xb, lb = dev.from_numpy(x.ravel()), dev.from_numpy(lab)
+        lse, loss = dev.mem_alloc(F32, rows), dev.mem_alloc(F32, 1)
+        dev.sync()
+        before = dev.cache_stats()["n_device_allocs"]
+        dev.dispatch("matmul", A=a, B=w, C=c, m=m, n=n, k=k, trans_a=False, trans_b=True, lda=k, ldb=k, ldc=n, alpha=1.0,
+                     beta=0.0)                                  # a layer's forward product: waits for its bias add
+        dev.dispatch("smce_label_fwd_noalloc", logits=xb, labels=lb, lse=lse, loss=loss, rows=rows, cols=cols)
+        after = dev.cache_stats()["n_device_allocs"]
+        got = dev.to_numpy(c).reshape(m, n)
+        want = A.astype(np.float64) @ W.astype(np.float64).T
+        assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
+        x64 = x.astype(np.float64)
+        lse64 = np.log(np.exp(x64 - x64.max(axis=1, keepdims=True)).sum(axis=1)) + x64.max(axis=1)
+        assert np.allclose(dev.to_numpy(lse), lse64, rtol=1e-6, atol=1e-6)
+        # the product's workspace was allocated by the matmul call (at most one growth), nothing by the other
+        assert after - before <= 1
+        for b in (a, w, c, xb, lb, lse, loss):
+            dev.mem_free(b)
+    finally:
+        dev.deinit()

@@ -1338,6 +1338,41 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, mode(64, 64), batches);
 }
 
+// The workspace a single product of this shape asks for when it is dispatched (the partial tiles of a k that is cut),
+// following gemm_dispatch_body's choices.  A product that waits reserves it when it is queued, so that the call
+// which later launches it, whichever that is, allocates nothing.
+static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda,
+                                  size_t ldb, int depth) {
+    if (m == 0 || n == 0 || k == 0) return 0;
+    const bool a_kmajor = !trans_a, b_kmajor = trans_b != 0;
+    const size_t n_cu = (size_t)ctx->n_cu;
+    const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
+    if (!small_ld || gemm_is_tiny(m, n, k, 1, lda, ldb, n_cu)) return 0;
+    if (!a_kmajor && !b_kmajor && (m <= 32 || n <= 32) && k > 512 && ceil_div_sz(m, 32) * ceil_div_sz(n, 32) <= n_cu) {
+        const size_t groups = ceil_div_sz(k, 8);
+        size_t splits = ceil_div_sz(groups, 32);
+        if (splits > 32) splits = 32;
+        size_t per = ceil_div_sz(groups, splits);
+        per = (per + 3) & ~(size_t)3;
+        splits = ceil_div_sz(groups, per);
+        return splits * m * n * sizeof(float);
+    }
+    const GemmPlan plan = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth);
+    if (plan.kind == GemmPlan::kParts) {
+        const size_t m1 = plan.rm * 256, n1 = plan.rn * 128;
+        const size_t shapes[3][2] = {{m1, n1}, {m1, n - n1}, {m - m1, n}};
+        size_t need = 0;
+        for (const auto& sh : shapes) {
+            if (sh[0] == 0 || sh[1] == 0) continue;
+            const size_t part = gemm_workspace_need(ctx, sh[0], sh[1], k, trans_a, trans_b, lda, ldb, depth + 1);
+            need = part > need ? part : need;
+        }
+        return need;
+    }
+    if (plan.kind == GemmPlan::kSplit) return plan.splits * m * n * sizeof(float);
+    return 0;
+}
+
 // ------------------------------------------------------------------------------------------------
 // matvec / outer / transpose
 // ------------------------------------------------------------------------------------------------
@@ -1673,6 +1708,12 @@ static int gemm_entry(zg_hip_ctx* ctx, const char* name, const float* A, const f
             if (zeroed) (void)zg_hip_mem_fill(ctx, C, m * n, 0.f);
             return rc;
         }
+        // whichever call launches the product later must not have to grow the workspace for it
+        if (const size_t need = gemm_workspace_need(ctx, m, n, k, trans_a, trans_b, lda, ldb, 0))
+            if (!workspace(ctx, need)) {
+                if (zeroed) (void)zg_hip_mem_fill(ctx, C, m * n, 0.f);
+                return ZG_HIP_EOOM;
+            }
         zg_deferred_gemm& d = ctx->deferred;
         d = zg_deferred_gemm{};
         d.active = true;

@@ -25,7 +25,13 @@
  *     and panic on failure (src/device/device_reference.zig:20-22); the Zig
  *     binding turns a non-zero return into @panic.
  *   - argument checks happen on the host before any launch; a rejected call
- *     launches nothing.
+ *     launches nothing;
+ *   - "in order" describes what a caller can observe, not when kernels are launched: some calls (float fills, a
+ *     layer's products, its bias gradient, optimizer steps, the graph-convolution aggregation) are held inside the
+ *     context for the calls that usually follow them and leave in fewer launches with the same values, and every
+ *     other call launches what is held first (the comments at those entry points say what is held and for what);
+ *   - a context belongs to one host thread at a time (the reference's devices are not shared between threads
+ *     either); different contexts may be used from different threads.
  */
 #ifndef ZG_HIP_H
 #define ZG_HIP_H

@@ -120,6 +120,8 @@ struct zg_hip_ctx {
     float* scalar_slot = nullptr;
     // fixed buffer for the per-workgroup partials of flat reductions (64 KiB)
     void* partials = nullptr;
+    // pinned host memory that small device-to-host copies go through (runtime.hip)
+    void* d2h_slot = nullptr;
 
     // address, on this context's device, of the fixed scratch array of the allocation-free entry point (loss.hip)
     void* noalloc_scratch = nullptr;

@@ -204,6 +204,8 @@ void* workspace(zg_hip_ctx* ctx, size_t bytes);
 // Cached segment plans (index.hip).  destroy: at deinit.  retain: a saved graph takes (+1) or drops (-1) its plans,
 // which are never evicted while a graph names them.  validate: before a replay, every index array the recording
 // matched must still hold what it held then, or the replay would scatter by a stale plan.
+// Blocking copy of a few bytes (at most 4096) from device memory to pageable host memory (runtime.hip).
+int small_d2h(zg_hip_ctx* ctx, void* dst_host, const void* src, size_t bytes);
 // Launches the fills that are waiting in the context (one kernel for all of them).
 int flush_fills(zg_hip_ctx* ctx);
 // Launches the waiting product with whatever was attached to it, and the waiting bias gradient and weight-gradient

@@ -969,8 +969,7 @@ static int gather_impl(zg_hip_ctx* ctx, const char* name, const uint64_t* src_sh
     if (status) {
         ZG_NOT_CAPTURING(ctx, "a gather with a status read-back");
         int h = 0;
-        ZG_HIP_TRY(hipMemcpyAsync(&h, d_status, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
-        ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        if (int rc = small_d2h(ctx, &h, d_status, sizeof(int))) return rc;
         *status = h;
         if (h) {
             set_error("%s: IndexOutOfBounds", name);

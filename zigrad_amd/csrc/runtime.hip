@@ -996,22 +996,26 @@ ZG_API int zg_hip_memcpy_h2d(zg_hip_ctx* ctx, void* dst, const void* src_host, s
     return ZG_HIP_OK;
 }
 
+namespace zg {
+// A scalar read (loss.get(0), src/ndtensor.zig:524-528; an op's status word): a copy kernel into the context's pinned
+// slot, the wait for the stream, and a host copy.  The driver's own path for a few bytes into pageable memory costs
+// 25 us more per call (the batch-64 train step from C: 99 -> 75-85 us).  At most kSmallD2H bytes.
+int small_d2h(zg_hip_ctx* ctx, void* dst_host, const void* src, size_t bytes) {
+    hipLaunchKernelGGL(copy_kernel<uint8_t>, dim3(1), dim3(kBlock), 0, ctx->stream, (uint8_t*)ctx->d2h_slot,
+                       (const uint8_t*)src, bytes);
+    ZG_LAUNCH_CHECK();
+    ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    memcpy(dst_host, ctx->d2h_slot, bytes);
+    return ZG_HIP_OK;
+}
+}  // namespace zg
+
 ZG_API int zg_hip_memcpy_d2h(zg_hip_ctx* ctx, void* dst_host, const void* src, size_t bytes) {
     ZG_CTX(ctx);
     ZG_NOT_CAPTURING(ctx, "memcpy_d2h");
     if (bytes == 0) return ZG_HIP_OK;
     ZG_REQUIRE(dst_host && src, "memcpy_d2h: null pointer");
-    if (bytes <= kSmallD2H) {
-        // a scalar read (loss.get(0), src/ndtensor.zig:524-528): a copy kernel into the context's pinned slot, the wait
-        // for the stream, and a host copy.  The driver's own path for a few bytes into pageable memory costs 25 us
-        // more per call (the batch-64 train step from C: 99 -> 75 us).
-        hipLaunchKernelGGL(copy_kernel<uint8_t>, dim3(1), dim3(kBlock), 0, ctx->stream, (uint8_t*)ctx->d2h_slot,
-                           (const uint8_t*)src, bytes);
-        ZG_LAUNCH_CHECK();
-        ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
-        memcpy(dst_host, ctx->d2h_slot, bytes);
-        return ZG_HIP_OK;
-    }
+    if (bytes <= kSmallD2H) return small_d2h(ctx, dst_host, src, bytes);
     ZG_HIP_TRY(hipMemcpyAsync(dst_host, src, bytes, hipMemcpyDefault, ctx->stream));
     ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
     return ZG_HIP_OK;

@@ -178,6 +178,31 @@ class _Run:
         if self.r.random() < 0.5:
             self.hip.dispatch("relu_fwd", x=y, y=y)
 
+    def op_scatter_bwd(self):
+        n_nodes, n_edge = self.graph
+        stride = int(self.r.choice([4, 7, 16]))
+        go, h, deg, gh, gd = self.picks(n_nodes * stride, n_nodes * stride, n_nodes, n_nodes * stride, n_nodes)
+        if self.r.random() < 0.6:
+            self.hip.mem_fill(gh, 0.0)
+            self.done()
+        if self.r.random() < 0.6:
+            self.hip.mem_fill(gd, 0.0)
+            self.done()
+        self.hip.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=go, h=h, deg=deg, src_indices=self.src,
+                          tgt_indices=self.tgt, grad_h=gh, grad_deg=gd, stride=stride, n_edge=n_edge)
+
+    def op_loss(self):
+        rows, cols = int(self.r.choice([8, 64])), int(self.r.choice([7, 10]))
+        logits, target, probs, loss, grad = self.picks(rows * cols, rows * cols, rows * cols, 1, rows * cols)
+        self.hip.dispatch("smce_fwd", logits=logits, target=target, probs=probs, loss=loss, rows=rows, cols=cols)
+        self.done()
+        self.hip.mem_fill(self.pick(1), 1.0)         # the upstream gradient of the loss
+        self.done()
+        if self.r.random() < 0.7:
+            self.hip.mem_fill(grad, 0.0)
+            self.done()
+        self.hip.dispatch("smce_bwd", probs=probs, target=target, grad=grad, rows=rows, cols=cols)
+
     def op_alloc(self):
         n = int(self.r.choice([16, 1024, BUF_LEN]))
         t = self.hip.mem_cache_alloc(F32, n)
@@ -217,8 +242,8 @@ class _Run:
         self.last_c = None
         ops = [self.op_fill, self.op_matmul, self.op_add_row, self.op_relu, self.op_relu_mask, self.op_layer_backward,
                self.op_unbroadcast, self.op_step, self.op_scatter, self.op_alloc, self.op_free, self.op_read, self.op_copy,
-               self.op_elementwise]
-        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1], float)
+               self.op_elementwise, self.op_scatter_bwd, self.op_loss]
+        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1], float)
         for _ in range(n_ops):
             ops[int(self.r.choice(len(ops), p=weights / weights.sum()))]()
             self.done()

@@ -125,7 +125,8 @@ int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
  * exactly the dense output of zg_hip_matmul / zg_hip_bmm_acc with beta = 1, the gradient of zg_hip_smce_bwd, the output
  * of zg_hip_scatter_gcn_deg_scaled or a gradient of zg_hip_scatter_gcn_deg_scaled_bwd is not
  * launched at all: the op writes what it would have added to the zeros; one over exactly the gradient of an optimizer
- * step that is itself still waiting (zero_grad() after step()) is stored by the step's update kernel. */
+ * step that is itself still waiting (zero_grad() after step()) is stored by the step's update kernel; and a waiting
+ * fill that lies inside a cache block handed back with zg_hip_mem_cache_free is dropped (nobody can read it any more). */
 int zg_hip_mem_fill(zg_hip_ctx *ctx, float *x, size_t n, float value);
 int zg_hip_mem_fill_u8(zg_hip_ctx *ctx, void *x, size_t n, uint8_t value);
 int zg_hip_mem_fill_u64(zg_hip_ctx *ctx, uint64_t *x, size_t n, uint64_t value);

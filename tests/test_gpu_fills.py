@@ -185,3 +185,55 @@ def test_the_loss_backward_takes_over_a_waiting_zero_fill(oracle, hip):
     assert np.array_equal(hip.to_numpy(g).reshape(rows, cols), want + want)
     for x in (p, t, g):
         hip.mem_free(x)
+
+
+def test_a_waiting_fill_of_a_block_that_is_given_back_never_lands(hip):
+    """The fill of a cache block that is freed while the fill still waits is dropped; whoever gets the block next must
+    not see it arrive later.  Fills of other memory that waited beside it still happen."""
+    n = 5000
+    other = hip.mem_alloc(F32, 300)
+    t = hip.mem_cache_alloc(F32, n)
+    hip.mem_fill(t, 5.0)
+    hip.mem_fill(other, 2.0)
+    hip.mem_cache_free(t)
+    u = hip.mem_cache_alloc(F32, n)              # the same block again, most likely
+    data = np.arange(n, dtype=np.float32)
+    hip.mem_transfer(data, u, "HtoD")
+    hip.sync()
+    assert np.array_equal(hip.to_numpy(u), data)
+    assert np.all(hip.to_numpy(other) == 2.0)
+    # a view into a live block is not the block: freeing the view's parent drops nothing that lies elsewhere
+    v = hip.mem_cache_alloc(F32, n)
+    hip.mem_fill(v.sub(0, 100), 9.0)
+    hip.mem_fill(other, 3.0)
+    hip.mem_cache_free(u)
+    assert np.all(hip.to_numpy(v)[:100] == 9.0) and np.all(hip.to_numpy(other) == 3.0)
+    hip.mem_cache_free(v)
+    hip.mem_free(other)
+
+
+def test_the_loss_backward_leaves_unrelated_fills_waiting_and_sees_related_ones(hip):
+    rows, cols = 64, 10
+    r = np.random.default_rng(2)
+    p = r.random((rows, cols)).astype(np.float32)
+    t = np.zeros((rows, cols), np.float32)
+    t[np.arange(rows), r.integers(0, cols, rows)] = 1.0
+    pb, tb = hip.from_numpy(p), hip.from_numpy(t)
+    g = hip.mem_cache_alloc(F32, rows * cols)
+    up = hip.mem_cache_alloc(F32, 1)
+    hip.mem_fill(up, 1.0)                        # the upstream gradient: unrelated to the three operands
+    hip.mem_fill(g, 0.0)
+    hip.dispatch("smce_bwd", probs=pb, target=tb, grad=g, rows=rows, cols=cols)
+    assert np.all(hip.to_numpy(up) == 1.0)       # still filled when somebody does read it
+    want = ((p - t) / np.float32(rows)).astype(np.float32)
+    assert np.array_equal(hip.to_numpy(g).reshape(rows, cols), want)
+    # a fill of the probabilities that waits when the backward is asked for must be seen by it
+    hip.mem_fill(pb, 0.5)
+    hip.mem_fill(g, 0.0)
+    hip.dispatch("smce_bwd", probs=pb, target=tb, grad=g, rows=rows, cols=cols)
+    want = ((np.float32(0.5) - t) / np.float32(rows)).astype(np.float32)
+    assert np.array_equal(hip.to_numpy(g).reshape(rows, cols), want)
+    hip.mem_cache_free(g)
+    hip.mem_cache_free(up)
+    hip.mem_free(pb)
+    hip.mem_free(tb)

@@ -231,6 +231,9 @@ int flush_steps(zg_hip_ctx* ctx, bool requeue_fills = false);
 void run_deferred_frees(zg_hip_ctx* ctx);
 // The waiting product, then the waiting fills: what ZG_CTX does before a call's own work.
 int flush_pending(zg_hip_ctx* ctx);
+// The same except that waiting fills stay waiting unless one of them meets one of the `count` byte ranges the caller
+// is about to read or write (runtime.hip).
+int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count);
 // A call that may be absorbed by the waiting product: true when it was (then *rc is the call's result and the caller
 // returns it), false when the call has to run as usual.
 bool deferred_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);

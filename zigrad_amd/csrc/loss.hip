@@ -748,7 +748,16 @@ ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* tar
     if (int rc = check_rows("smce_bwd", rows, cols)) return rc;
     // the gradient's zero fill (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: then write, not add
     const bool fresh = absorb_zero_fill(ctx, grad, rows * cols);
-    if (int rc = flush_pending(ctx)) return rc;
+    {
+        // a fill that meets none of the three operands keeps waiting (the loss's upstream gradient is filled right
+        // before this call and read by nobody: src/nn/loss.zig:150-159 folds it into the 1/rows factor)
+        const void* ops[3] = {probs, target, grad};
+        const size_t bytes[3] = {rows * cols * sizeof(float), rows * cols * sizeof(float), rows * cols * sizeof(float)};
+        if (int rc = flush_pending_but_fills(ctx, ops, bytes, 3)) {
+            if (fresh) (void)zg_hip_mem_fill(ctx, grad, rows * cols, 0.f);
+            return rc;
+        }
+    }
     const size_t n = rows * cols;
     const unsigned blocks = smce_bwd_grid(n);
     if (fresh)

@@ -856,11 +856,10 @@ void run_deferred_frees(zg_hip_ctx* ctx) {
 
 ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     ZG_CTX_KEEP_FILLS(ctx);
-    if (ctx->n_pending_fills)  // a fill of the block that is given back must not land on its next owner
-        if (int rc = flush_fills(ctx)) return rc;
     if (ctx->steps.count)
         if (int rc = flush_steps(ctx)) return rc;
     if (!ptr || block == 0) {  // views and empty data: src/allocators/caching_allocator.zig:111-112
+        if (int rc = flush_fills(ctx)) return rc;
         if (gemm_group_waiting(ctx)) return flush_deferred_gemm(ctx);
         return ZG_HIP_OK;
     }
@@ -868,8 +867,32 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     BlockPool* pool = nullptr;
     for (BlockPool* p : {ctx->small_pool, ctx->large_pool})
         if (p && p->owns_live(b, ptr)) pool = p;
+    if (pool == nullptr) (void)flush_fills(ctx);
     ZG_REQUIRE(pool != nullptr, "mem_cache_free: %p with handle %llx is not a live block of this context's pools", ptr,
                (unsigned long long)block);
+    if (ctx->n_pending_fills) {
+        // A fill must not land on the block's next owner.  One that lies wholly inside the block that is given back
+        // has no reader left (the block's contents are nobody's once it is free) and is dropped: the upstream gradient
+        // of a loss is filled, never read by the fused loss backward, and freed.  One that straddles the block's end
+        // sends all waiting fills out instead; the others keep waiting.
+        const char *lo = b->ptr, *hi = b->ptr + b->size;
+        bool straddles = false;
+        for (int i = 0; i < ctx->n_pending_fills; i++) {
+            const char* x0 = (const char*)ctx->pending_fills[i].x;
+            const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
+            straddles = straddles || (x0 < hi && lo < x1 && !(lo <= x0 && x1 <= hi));
+        }
+        if (straddles) {
+            if (int rc = flush_fills(ctx)) return rc;
+        } else {
+            int kept = 0;
+            for (int i = 0; i < ctx->n_pending_fills; i++) {
+                const char* x0 = (const char*)ctx->pending_fills[i].x;
+                if (!(lo <= x0 && x0 < hi)) ctx->pending_fills[kept++] = ctx->pending_fills[i];
+            }
+            ctx->n_pending_fills = kept;
+        }
+    }
     if (gemm_group_waiting(ctx)) {
         // An input-gradient product that waits for its mask outlives the frees of the backward pass it belongs to
         // (the layer's output, the output gradient), and so do the bias gradient and the weight-gradient product
@@ -1098,6 +1121,24 @@ int flush_pending(zg_hip_ctx* ctx) {
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (int rc = flush_fills(ctx)) return rc;
     return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
+}
+
+int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
+    if (ctx->scatter_wait.active)
+        if (int rc = flush_scatter(ctx)) return rc;
+    if (gemm_group_waiting(ctx))
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
+    if (ctx->steps.count)
+        if (int rc = flush_steps(ctx)) return rc;
+    for (int i = 0; i < ctx->n_pending_fills; i++) {
+        const char* x0 = (const char*)ctx->pending_fills[i].x;
+        const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
+        for (int j = 0; j < count; j++) {
+            const char* p0 = (const char*)ptrs[j];
+            if (p0 && x0 < p0 + bytes[j] && p0 < x1) return flush_fills(ctx);
+        }
+    }
+    return ZG_HIP_OK;
 }
 
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {

@@ -34,6 +34,7 @@ class _Run:
         self.tgt = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
         self.reads = []
         self.t = 0
+        self.last_c = None
 
     def done(self):
         if self.eager:
@@ -83,7 +84,7 @@ class _Run:
         """A bias row onto the last product's output, or onto something else."""
         m, n = int(self.r.choice(DIMS)), int(self.r.choice(DIMS))
         c, row = self.picks(m * n, n)
-        if getattr(self, "last_c", None) is not None and self.r.random() < 0.7:
+        if self.last_c is not None and self.r.random() < 0.7:
             c, m, n = self.last_c
             row = self.pick(n)
             if row.ptr < c.ptr + 4 * c.n and c.ptr < row.ptr + 4 * row.n:
@@ -94,7 +95,7 @@ class _Run:
             self.hip.dispatch("add", x=c, y=row, z=c)
 
     def op_relu(self):
-        if getattr(self, "last_c", None) is not None and self.r.random() < 0.7:
+        if self.last_c is not None and self.r.random() < 0.7:
             c = self.last_c[0]
         else:
             c = self.pick(int(self.r.choice([64, 1024])))
@@ -105,7 +106,7 @@ class _Run:
             self.hip.dispatch("relu_fwd", x=c, y=other)
 
     def op_relu_mask(self):
-        if getattr(self, "last_c", None) is not None and self.r.random() < 0.7:
+        if self.last_c is not None and self.r.random() < 0.7:
             g = self.last_c[0]
         else:
             g = self.pick(int(self.r.choice([64, 1024])))
@@ -135,6 +136,7 @@ class _Run:
         host.bmm_acc_(self.hip, g, [B, O], x, [B, I], gw, True, False, 1.0, 1.0)
         self.done()
         if g_temp is not None:
+            self.forget_if_in(g_temp)
             self.hip.mem_cache_free(g_temp)
             self.done()
         if self.r.random() < 0.7:
@@ -209,9 +211,16 @@ class _Run:
         self.hip.mem_fill(t, float(self.r.choice([0.0, 0.25])))
         self.temps.append(t)
 
+    def forget_if_in(self, t):
+        """The last product's output may lie in a temporary: once that is given back it must not be used again."""
+        c = self.last_c
+        if c is not None and t.ptr <= c[0].ptr < t.ptr + 4 * t.n:
+            self.last_c = None
+
     def op_free(self):
         if self.temps:
             t = self.temps.pop(int(self.r.integers(0, len(self.temps))))
+            self.forget_if_in(t)
             self.hip.mem_cache_free(t)
 
     def op_copy(self):

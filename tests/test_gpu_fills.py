@@ -237,3 +237,49 @@ def test_the_loss_backward_leaves_unrelated_fills_waiting_and_sees_related_ones(
     hip.mem_cache_free(up)
     hip.mem_free(pb)
     hip.mem_free(tb)
+
+
+def test_a_refused_call_still_owes_the_zeros_it_took_over(hip):
+    """An op that takes over a waiting zero fill and is then refused (an argument error) must leave the zeros behind:
+    the caller asked for them and the refused op wrote nothing."""
+    from zigrad_amd._lib import ZgHipError
+    from zigrad_amd.device import U64
+
+    m, n, k = 24, 16, 8
+    a = hip.from_numpy(np.ones(m * k, np.float32))
+    b = hip.from_numpy(np.ones(k * n, np.float32))
+    c = hip.from_numpy(np.full(m * n, 7.0, np.float32))
+    hip.mem_fill(c, 0.0)
+    with pytest.raises(ZgHipError):      # lda smaller than k
+        hip.dispatch("matmul", A=a, B=b, C=c, m=m, n=n, k=k, trans_a=False, trans_b=False, lda=k - 1, ldb=n, ldc=n,
+                     alpha=1.0, beta=1.0)
+    assert np.all(hip.to_numpy(c) == 0.0)
+    # the graph-convolution aggregation and its backward
+    n_nodes, stride, n_edge = 12, 4, 30
+    r = np.random.default_rng(1)
+    src = hip.from_numpy(r.integers(0, n_nodes, n_edge).astype(np.uint64))
+    tgt = hip.from_numpy(r.integers(0, n_nodes, n_edge).astype(np.uint64))
+    h = hip.from_numpy(r.standard_normal(n_nodes * stride).astype(np.float32))
+    deg = hip.from_numpy(np.ones(n_nodes, np.float32))
+    y = hip.from_numpy(np.full(n_nodes * stride, 3.0, np.float32))
+    hip.mem_fill(y, 0.0)
+    with pytest.raises(ZgHipError):      # no node features
+        hip._call("zg_hip_scatter_gcn_deg_scaled", y.ptr, None, deg.ptr, src.ptr, tgt.ptr, stride, n_edge, n_nodes)
+    assert np.all(hip.to_numpy(y) == 0.0)
+    gh = hip.from_numpy(np.full(n_nodes * stride, 3.0, np.float32))
+    gd = hip.from_numpy(np.full(n_nodes, 3.0, np.float32))
+    hip.mem_fill(gh, 0.0)
+    hip.mem_fill(gd, 0.0)
+    with pytest.raises(ZgHipError):      # no upstream gradient
+        hip._call("zg_hip_scatter_gcn_deg_scaled_bwd", None, h.ptr, deg.ptr, src.ptr, tgt.ptr, gh.ptr, gd.ptr, stride,
+                  n_edge, n_nodes)
+    assert np.all(hip.to_numpy(gh) == 0.0) and np.all(hip.to_numpy(gd) == 0.0)
+    # the loss backward
+    g = hip.from_numpy(np.full(40, 2.0, np.float32))
+    p = hip.from_numpy(np.full(40, 0.1, np.float32))
+    hip.mem_fill(g, 0.0)
+    with pytest.raises(ZgHipError):      # no target
+        hip._call("zg_hip_smce_bwd", p.ptr, None, g.ptr, 4, 10)
+    assert np.all(hip.to_numpy(g) == 0.0)
+    for t in (a, b, c, src, tgt, h, deg, y, gh, gd, g, p):
+        hip.mem_free(t)

@@ -228,6 +228,55 @@ def op_suite(dev, quick=False, cpu=False):
     out["sum_axis1_8192x4096"] = gbs((rows * cols + rows) * 4, ms)
     ms = timed(dev, lambda: dev.dispatch("max_along", x=X, x_shape=[rows, cols], y=yrow, dim=1), iters * 5)
     out["max_axis1_8192x4096"] = gbs((rows * cols + rows) * 4, ms)
+    if not cpu:
+        # the rest of the op surface at the same size (not in the named suite): unary ops forward and backward, a
+        # same-size binary op, reductions along the other axis, argmax, the optimizer updates of a [4096,4096] weight,
+        # row gathers.  Bytes are the algorithmic ones: every operand read once, every result written once.
+        n_el = rows * cols
+        G, Y = dev_normal(n_el), dev_normal(n_el)
+        extra = {}
+        for name in ("relu_fwd", "tanh_fwd", "sigm_fwd", "exp_fwd"):
+            ms = timed(dev, lambda: dev.dispatch(name, x=X, y=Z), iters * 5)
+            extra[f"{name}_8192x4096"] = gbs(2 * n_el * 4, ms)
+        ms = timed(dev, lambda: dev.dispatch("relu_bwd", x=X, x_g=G, y_g=Y), iters * 5)
+        extra["relu_bwd_8192x4096"] = gbs(4 * n_el * 4, ms)
+        for name in ("tanh_bwd", "sigm_bwd", "exp_bwd"):
+            ms = timed(dev, lambda: dev.dispatch(name, x_g=G, y=Z, y_g=Y), iters * 5)
+            extra[f"{name}_8192x4096"] = gbs(4 * n_el * 4, ms)
+        ms = timed(dev, lambda: dev.dispatch("relu_inplace_bwd", x=X, x_g=G), iters * 5)
+        extra["relu_inplace_bwd_8192x4096"] = gbs(3 * n_el * 4, ms)
+        ms = timed(dev, lambda: dev.dispatch("mul", x=X, y=Y, z=Z), iters * 5)
+        extra["mul_8192x4096"] = gbs(3 * n_el * 4, ms)
+        ycol = dev.mem_alloc(F32, cols)
+        ms = timed(dev, lambda: dev.dispatch("sum_along", x=X, x_shape=[rows, cols], y=ycol, dim=0), iters * 5)
+        extra["sum_axis0_8192x4096"] = gbs((n_el + cols) * 4, ms)
+        yarg = dev.mem_alloc(U64, rows)
+        ms = timed(dev, lambda: dev.dispatch("argmax_along", x=X, x_shape=[rows, cols], y=yarg, dim=1), iters * 5)
+        extra["argmax_axis1_8192x4096"] = gbs(n_el * 4 + rows * 8, ms)
+        ysc = dev.mem_alloc(F32, 1)
+        ms = timed(dev, lambda: dev.dispatch("nrm2", x=X, y=ysc), iters * 5)
+        extra["nrm2_33M"] = gbs(n_el * 4, ms)
+        n_w = 4096 * 4096
+        P, Gw, M1, V1 = (X.sub(0, n_w), G.sub(0, n_w), Y.sub(0, n_w), Z.sub(0, n_w))
+        dev.mem_fill(M1, 0.0)
+        dev.mem_fill(V1, 0.0)
+        ms = timed(dev, lambda: dev.dispatch("sgd_step", param=P, grad=Gw, lr=1e-6, clip=False, max_norm=10.0, delta=1e-6),
+                   iters * 5)
+        extra["sgd_step_16.8M"] = gbs(3 * n_w * 4, ms)
+        ms = timed(dev, lambda: dev.dispatch("adam_step", param=P, grad=Gw, m=M1, v=V1, t=10, lr=1e-6, beta1=0.9, beta2=0.999,
+                                             epsilon=1e-8, clip=False, max_norm=10.0, delta=1e-6), iters * 5)
+        extra["adam_step_16.8M"] = gbs(7 * n_w * 4, ms)
+        ms = timed(dev, lambda: dev.dispatch("adam_step", param=P, grad=Gw, m=M1, v=V1, t=10, lr=1e-6, beta1=0.9, beta2=0.999,
+                                             epsilon=1e-8, clip=True, max_norm=10.0, delta=1e-6), iters * 5)
+        extra["adam_step_clip_16.8M"] = gbs(8 * n_w * 4, ms)
+        n_idx, stride = 65536, 256
+        idx = dev.from_numpy(r.integers(0, n_el // stride, n_idx).astype(np.uint64))
+        ms = timed(dev, lambda: dev.dispatch("index_select_fwd", src=X, indices=idx, stride=stride, dst=Z.sub(0, n_idx * stride)),
+                   iters * 5)
+        extra["index_select_fwd_65536x256"] = gbs(2 * n_idx * stride * 4 + n_idx * 8, ms)
+        out["other_ops"] = extra
+        for b in (G, Y, ycol, yarg, ysc, idx):
+            dev.mem_free(b)
     for b in (X, bias, Z, yrow):
         dev.mem_free(b)
 
@@ -632,6 +681,7 @@ def main():
                 result[kind]["fused"] = {k: f[k] for k in ("steps_per_s", "ms_per_step", "graph_replay")}
     if not args.no_ops:
         result["ops"] = op_suite(dev)
+        result["other_ops"] = result["ops"].pop("other_ops", None)  # the op surface outside the named suite
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH, loss_mode=args.loss_mode)
         # the oracle ran the same first step from the same parameters and batch: its loss must be the device's

@@ -909,6 +909,33 @@ __global__ void index_select_fwd_kernel(const float* src, size_t src_len, const 
     }
 }
 
+// The same for rows of whole 16-byte pieces: G lanes share a row (G a power of two up to the wave), four rows per lane
+// group in flight (two or eight measured no better: a gather of random 1 KiB rows runs at the rate DRAM opens pages) (their indices are loaded first, then their pieces), one piece per lane and trip along the row.
+template <int G>
+__global__ __launch_bounds__(256) void index_select_fwd_vec4_kernel(const float4* src, size_t src_rows, const uint64_t* indices,
+                                                                     size_t n_idx, size_t s4, float4* dst) {
+    constexpr int kRows = 4;
+    const int lane = threadIdx.x % G;
+    const size_t slot = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G, n_slots = (size_t)gridDim.x * (256 / G);
+    for (size_t d0 = slot; d0 < n_idx; d0 += kRows * n_slots) {
+        uint64_t r[kRows];
+#pragma unroll
+        for (int u = 0; u < kRows; u++) {
+            const size_t d = d0 + (size_t)u * n_slots;
+            r[u] = d < n_idx ? indices[d] : ~(uint64_t)0;
+        }
+        for (size_t j = lane; j < s4; j += G) {
+            float4 v[kRows];
+#pragma unroll
+            for (int u = 0; u < kRows; u++)
+                if (r[u] < src_rows) v[u] = src[r[u] * s4 + j];
+#pragma unroll
+            for (int u = 0; u < kRows; u++)
+                if (r[u] < src_rows) dst[(d0 + (size_t)u * n_slots) * s4 + j] = v[u];
+        }
+    }
+}
+
 static int group_for(size_t stride) {
     if (stride <= 4) return 4;
     if (stride <= 8) return 8;
@@ -1024,6 +1051,18 @@ ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src
     ZG_REQUIRE(src && indices && dst, "index_select_fwd: null pointer");
     ZG_REQUIRE(src_len >= stride, "index_select_fwd: source shorter than one row");
     const size_t total = n_idx * stride;
+    if (stride % 4 == 0 && aligned16(src) && aligned16(dst)) {
+        // rows of whole 16-byte pieces: a lane group per row (an out-of-range index is skipped, as below)
+        const size_t s4 = stride / 4;
+        const int g = group_for(s4);
+        size_t vblocks = ceil_div_sz(n_idx, (size_t)(256 / g) * 4);
+        if (vblocks > (size_t)ctx->n_cu * 16) vblocks = (size_t)ctx->n_cu * 16;
+        ZG_G_DISPATCH(g, hipLaunchKernelGGL((index_select_fwd_vec4_kernel<G>), dim3((unsigned)vblocks), dim3(256), 0,
+                                            ctx->stream, (const float4*)src, src_len / stride, indices, n_idx, s4,
+                                            (float4*)dst));
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     size_t blocks = ceil_div_sz(total, 256);
     if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
     hipLaunchKernelGGL(index_select_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, src, src_len, indices,

@@ -111,7 +111,10 @@ class GemmTimer:
         return range(self.count)
 
 
-def time_op(dev, fn, iters, warm_ms=60.0, batches=10):
+OP_WARM_MS = 60.0  # --short-ops lowers it: under a profiler every warm-up call is a row of output
+
+
+def time_op(dev, fn, iters, warm_ms=None, batches=10):
     """Median (and p10/p90) per-call time in ms over `batches` event-bracketed runs of `iters` back-to-back calls.
 
     The warm-up runs for at least `warm_ms` of wall time: the GPU raises its clock only under sustained load, and a
@@ -127,6 +130,7 @@ def time_op(dev, fn, iters, warm_ms=60.0, batches=10):
         ms.sort()
         pick = lambda q: ms[min(len(ms) - 1, int(q * len(ms)))]
         return {"ms": pick(0.5), "ms_p10": pick(0.1), "ms_p90": pick(0.9)}
+    warm_ms = OP_WARM_MS if warm_ms is None else warm_ms
     t0 = time.perf_counter()
     while True:
         for _ in range(iters):
@@ -552,6 +556,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops", action="store_true", help="skip the op microbenchmark suite")
+    ap.add_argument("--short-ops", action="store_true",
+                    help="op suite with a 2 ms warm-up and a quarter of the repetitions: for runs under a profiler, which "
+                         "reads the kernels' durations itself and writes a row per launch")
     ap.add_argument("--loss-mode", default="onehot", choices=["onehot", "label"])
     ap.add_argument("--no-small", action="store_true", help="skip the latency-bound configurations (keeps profiler output small)")
     ap.add_argument("--trace-small", choices=["mlp_b64", "gcn", "dqn"],
@@ -680,7 +687,10 @@ def main():
                 f = run_small(dev, kind, n, graph=True, fused=True)
                 result[kind]["fused"] = {k: f[k] for k in ("steps_per_s", "ms_per_step", "graph_replay")}
     if not args.no_ops:
-        result["ops"] = op_suite(dev)
+        if args.short_ops:
+            global OP_WARM_MS
+            OP_WARM_MS = 2.0
+        result["ops"] = op_suite(dev, quick=args.short_ops)
         result["other_ops"] = result["ops"].pop("other_ops", None)  # the op surface outside the named suite
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(WIDE_DIMS, WIDE_BATCH, loss_mode=args.loss_mode)

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(kBlock) void col_reduce_kernel(const float* x, type
 }
 
 // Workgroup = 64 adjacent outputs x 4 waves; wave w combines chunks w, w+4, w+8, ... of its outputs with all its
-// loads in flight at once (chunks <= 64, so at most 16 per thread), then the four wave results are combined in
+// loads in flight at once (16 per thread and round of 64 chunks), then the four wave results are combined in
 // wave order.  The order is fixed, so the result does not depend on scheduling.
 template <class A>
 __global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::Acc* partials, typename A::Out* y,
@@ -144,16 +144,18 @@ __global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::
     if (o < n_out) {
         const size_t outer = o / inner, c = o % inner;
         const Acc* pp = partials + (outer * chunks) * inner + c;
-        Acc t[16];
+        for (int base = 0; base < chunks; base += 64) {  // 64 chunks per round: 16 loads in flight per thread
+            Acc t[16];
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
-            const int k = w + 4 * u;
-            if (k < chunks) t[u] = pp[(size_t)k * inner];
-        }
+            for (int u = 0; u < 16; u++) {
+                const int k = base + w + 4 * u;
+                if (k < chunks) t[u] = pp[(size_t)k * inner];
+            }
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
-            const int k = w + 4 * u;
-            if (k < chunks) acc = P::combine(acc, t[u]);
+            for (int u = 0; u < 16; u++) {
+                const int k = base + w + 4 * u;
+                if (k < chunks) acc = P::combine(acc, t[u]);
+            }
         }
     }
     smem[threadIdx.x] = acc;
@@ -182,7 +184,8 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    const ColReduceShape cs = col_reduce_shape(x, inner);
+    const bool wide = inner >= 1024 && R >= 256 && outer * R * inner > kColSingleChunkMax;
+    const ColReduceShape cs = col_reduce_shape(x, inner, wide);
     const bool v4 = cs.V == 4;
     const int log2_cx = cs.log2_cx;
     const int ry = kBlock >> log2_cx;
@@ -193,7 +196,10 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     size_t max_chunks = ceil_div_sz(R, (size_t)ry * 4);
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks < 1) chunks = 1;
-    if (chunks > 64) chunks = 64;  // keeps the partials buffer and the serial tail of the final stage small
+    // keeps the partials buffer and the serial tail of the final stage small (the wide shape has a quarter of the
+    // column groups, so it takes more chunks for enough workgroups)
+    const size_t chunk_cap = (wide && ry == 1) ? 256 : 64;
+    if (chunks > chunk_cap) chunks = chunk_cap;
     if (outer * R * inner <= kColSingleChunkMax) chunks = 1;  // a second launch costs more than a chunk split saves
     const size_t rows_per_chunk = ceil_div_sz(R, chunks);
     chunks = ceil_div_sz(R, rows_per_chunk);

@@ -414,6 +414,20 @@ __device__ __forceinline__ void col_reduce_block(const float* x, typename A::Out
         const float* xb = x + outer * R * inner + col0;
         size_t r = r_begin + ty;
         if constexpr (V == 4) {
+            // eight rows in flight while there are eight left, then four, then one by one: always combined in row order
+            for (; r + 7 * (size_t)ry < r_end; r += 8 * (size_t)ry) {
+                float4 vs[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) vs[u] = *reinterpret_cast<const float4*>(xb + (r + (size_t)u * ry) * inner);
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    uint32_t rr = (uint32_t)(r + (size_t)u * ry);
+                    acc[0] = P::combine(acc[0], A::term(vs[u].x, rr));
+                    acc[1 % V] = P::combine(acc[1 % V], A::term(vs[u].y, rr));
+                    acc[2 % V] = P::combine(acc[2 % V], A::term(vs[u].z, rr));
+                    acc[3 % V] = P::combine(acc[3 % V], A::term(vs[u].w, rr));
+                }
+            }
             for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
                 float4 v0 = *reinterpret_cast<const float4*>(xb + r * inner);
                 float4 v1 = *reinterpret_cast<const float4*>(xb + (r + ry) * inner);
@@ -478,13 +492,18 @@ struct ColReduceShape {
     int V, log2_cx;
     size_t gx;
 };
-static inline ColReduceShape col_reduce_shape(const float* x, size_t inner) {
+// `wide`: all 256 threads side by side (4 KiB of a row per workgroup and trip with V = 4, neighbouring workgroups on the
+// neighbouring 4 KiB), each walking the rows of its chunk one after the other: for matrices of many long rows, where
+// the narrow shape's four pieces of 1 KiB from four different rows per trip leave the bandwidth to the luck of how the
+// rows fall on the memory channels (column sums of [8192,4096]: 19 to 32 us depending on the allocation).
+static inline ColReduceShape col_reduce_shape(const float* x, size_t inner, bool wide = false) {
     ColReduceShape s;
     s.V = ((inner % 4 == 0) && aligned16(x)) ? 4 : 1;
     const size_t colv = inner / s.V;
     s.log2_cx = 0;
-    // at most 64 column threads (1 KiB of a row per workgroup with V = 4): more workgroups, fewer partials
-    while ((1u << s.log2_cx) < colv && s.log2_cx < 6) s.log2_cx++;
+    // narrow: at most 64 column threads (1 KiB of a row per workgroup with V = 4): more workgroups, fewer partials
+    const int max_log2 = (wide && s.V == 4) ? 8 : 6;
+    while ((1u << s.log2_cx) < colv && s.log2_cx < max_log2) s.log2_cx++;
     s.gx = ceil_div_sz(colv, (size_t)1 << s.log2_cx);
     return s;
 }

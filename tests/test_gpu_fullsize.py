@@ -123,3 +123,118 @@ def test_smce_label_8192x32000_invariants(hip):
     assert np.array_equal(hip.to_numpy(grad.sub(5 * N, N)), 2 * first)
     for b in (logits, grad, blk, lab, lse, loss, rs):
         hip.mem_free(b)
+
+
+def test_unary_ops_and_their_backward_8192x4096(oracle, hip):
+    """The unary ops at the op suite's size against the oracle on the same data: relu exactly (no rounding), the
+    transcendental ones to 1e-6 (the device's expf/tanhf and the host's are both within an ulp or two of the truth)."""
+    from conftest import run_op
+
+    rows, cols = 8192, 4096
+    n = rows * cols
+    r = np.random.default_rng(21)
+    X = r.standard_normal(n, dtype=np.float32)
+    YG = r.standard_normal(n, dtype=np.float32)
+    G0 = r.standard_normal(n, dtype=np.float32)
+    x, yg, g, y = hip.from_numpy(X), hip.from_numpy(YG), hip.from_numpy(G0), hip.mem_alloc(F32, n)
+    for name in ("relu_fwd", "tanh_fwd", "sigm_fwd", "exp_fwd"):
+        hip.dispatch(name, x=x, y=y)
+        got = hip.to_numpy(y)
+        want = run_op(oracle, name, {"x": X, "y": np.zeros(n, np.float32)}, ["y"])["y"]
+        if name == "relu_fwd":
+            assert np.array_equal(got, want)
+        else:
+            assert np.linalg.norm(got - want) <= 1e-6 * np.linalg.norm(want), name
+    # backward: x_g += f'(.) * y_g on the same buffers the benchmark uses them on
+    hip.dispatch("relu_bwd", x=x, x_g=g, y_g=yg)
+    want = run_op(oracle, "relu_bwd", {"x": X, "x_g": G0.copy(), "y_g": YG}, ["x_g"])["x_g"]
+    assert np.array_equal(hip.to_numpy(g), want)
+    T = np.tanh(X)
+    t = hip.from_numpy(T)
+    for name in ("tanh_bwd", "sigm_bwd", "exp_bwd"):
+        hip.mem_transfer(G0, g, "HtoD")
+        hip.dispatch(name, x_g=g, y=t, y_g=yg)
+        want = run_op(oracle, name, {"x_g": G0.copy(), "y": T, "y_g": YG}, ["x_g"])["x_g"]
+        assert np.linalg.norm(hip.to_numpy(g) - want) <= 1e-6 * np.linalg.norm(want), name
+    hip.mem_transfer(G0, g, "HtoD")
+    hip.dispatch("relu_inplace_bwd", x=x, x_g=g)
+    assert np.array_equal(hip.to_numpy(g), np.where(X > 0, G0, np.float32(0.0)))
+    hip.dispatch("mul", x=x, y=yg, z=y)
+    assert np.array_equal(hip.to_numpy(y), X * YG)          # one rounding per element: exact
+    for b in (x, yg, g, y, t):
+        hip.mem_free(b)
+
+
+def test_reductions_along_the_other_axis_and_norms_8192x4096(hip):
+    rows, cols = 8192, 4096
+    r = np.random.default_rng(22)
+    X = r.standard_normal((rows, cols), dtype=np.float32)
+    x = hip.from_numpy(X)
+    ycol = hip.mem_alloc(F32, cols)
+    hip.dispatch("sum_along", x=x, x_shape=[rows, cols], y=ycol, dim=0)
+    want = X.astype(np.float64).sum(axis=0)
+    assert np.linalg.norm(hip.to_numpy(ycol) - want) <= TOL * np.linalg.norm(want)
+    hip.dispatch("max_along", x=x, x_shape=[rows, cols], y=ycol, dim=0)
+    assert np.array_equal(hip.to_numpy(ycol), X.max(axis=0))
+    icol = hip.mem_alloc(U64, cols)
+    hip.dispatch("argmax_along", x=x, x_shape=[rows, cols], y=icol, dim=0)
+    assert np.array_equal(hip.to_numpy(icol), X.argmax(axis=0).astype(np.uint64))
+    one = hip.mem_alloc(F32, 1)
+    hip.dispatch("nrm2", x=x, y=one)
+    truth = np.sqrt((X.astype(np.float64) ** 2).sum())
+    assert abs(float(hip.to_numpy(one)[0]) - truth) <= 2e-6 * truth
+    # the bias gradient of the wide MLP's layers: unbroadcast of [4096,4096] and [4096,1024] to a row, accumulated
+    from zigrad_amd import host
+    for c in (4096, 1024):
+        G = r.standard_normal((4096, c), dtype=np.float32)
+        b0 = r.standard_normal(c, dtype=np.float32)
+        gb, bb = hip.from_numpy(G), hip.from_numpy(b0)
+        host.unbroadcast_(hip, gb, [4096, c], bb, [c], alpha=1.0, beta=1.0)
+        want = G.astype(np.float64).sum(axis=0) + b0
+        assert np.linalg.norm(hip.to_numpy(bb) - want) <= TOL * np.linalg.norm(want)
+        hip.mem_free(gb)
+        hip.mem_free(bb)
+    for b in (x, ycol, icol, one):
+        hip.mem_free(b)
+
+
+def test_optimizer_updates_of_a_4096x4096_weight(oracle, hip):
+    """SGD and Adam on 16.8 M parameters, clip off and on, against the oracle on the same data."""
+    from conftest import run_op
+
+    n = 4096 * 4096
+    r = np.random.default_rng(23)
+    P = r.standard_normal(n, dtype=np.float32)
+    G = (r.standard_normal(n, dtype=np.float32) * np.float32(0.01))
+    M0 = (r.standard_normal(n, dtype=np.float32) * np.float32(0.01))
+    V0 = (r.random(n, dtype=np.float32) * np.float32(1e-4))
+    for clip in (False, True):
+        p, g = hip.from_numpy(P), hip.from_numpy(G)
+        hip.dispatch("sgd_step", param=p, grad=g, lr=0.01, clip=clip, max_norm=10.0, delta=1e-6)
+        want = run_op(oracle, "sgd_step", {"param": P.copy(), "grad": G.copy(), "lr": 0.01, "clip": clip, "max_norm": 10.0,
+                                           "delta": 1e-6}, ["param", "grad"])
+        assert np.linalg.norm(hip.to_numpy(p) - want["param"]) <= 1e-6 * np.linalg.norm(want["param"])
+        assert np.linalg.norm(hip.to_numpy(g) - want["grad"]) <= 1e-6 * np.linalg.norm(want["grad"])
+        hip.mem_transfer(P, p, "HtoD")
+        hip.mem_transfer(G, g, "HtoD")
+        m, v = hip.from_numpy(M0), hip.from_numpy(V0)
+        kw = dict(t=7, lr=1e-3, beta1=0.9, beta2=0.999, epsilon=1e-8, clip=clip, max_norm=10.0, delta=1e-6)
+        hip.dispatch("adam_step", param=p, grad=g, m=m, v=v, **kw)
+        want = run_op(oracle, "adam_step", {"param": P.copy(), "grad": G.copy(), "m": M0.copy(), "v": V0.copy(), **kw},
+                      ["param", "m", "v"])
+        for name, buf in (("param", p), ("m", m), ("v", v)):
+            assert np.linalg.norm(hip.to_numpy(buf) - want[name]) <= 1e-6 * np.linalg.norm(want[name]), (clip, name)
+        for b in (p, g, m, v):
+            hip.mem_free(b)
+
+
+def test_gather_of_random_rows_65536x256(hip):
+    n_rows, stride, n_idx = 131072, 256, 65536
+    r = np.random.default_rng(24)
+    S = r.standard_normal((n_rows, stride), dtype=np.float32)
+    idx = r.integers(0, n_rows, n_idx).astype(np.uint64)
+    s, i, d = hip.from_numpy(S), hip.from_numpy(idx), hip.mem_alloc(F32, n_idx * stride)
+    hip.dispatch("index_select_fwd", src=s, indices=i, stride=stride, dst=d)
+    assert np.array_equal(hip.to_numpy(d).reshape(n_idx, stride), S[idx.astype(np.int64)])
+    for b in (s, i, d):
+        hip.mem_free(b)

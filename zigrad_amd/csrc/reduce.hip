@@ -129,7 +129,7 @@ __global__ __launch_bounds__(kBlock) void col_reduce_kernel(const float* x, type
 }
 
 // Workgroup = 64 adjacent outputs x 4 waves; wave w combines chunks w, w+4, w+8, ... of its outputs with all its
-// loads in flight at once (16 per thread and round of 64 chunks), then the four wave results are combined in
+// loads in flight at once (16 per thread up to 64 chunks, rounds of 32 beyond), then the four wave results are combined in
 // wave order.  The order is fixed, so the result does not depend on scheduling.
 template <class A>
 __global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::Acc* partials, typename A::Out* y,
@@ -144,17 +144,31 @@ __global__ __launch_bounds__(kBlock) void col_final_kernel(const typename A::P::
     if (o < n_out) {
         const size_t outer = o / inner, c = o % inner;
         const Acc* pp = partials + (outer * chunks) * inner + c;
-        for (int base = 0; base < chunks; base += 64) {  // 64 chunks per round: 16 loads in flight per thread
+        if (chunks <= 64) {  // one round: 16 loads in flight per thread
             Acc t[16];
 #pragma unroll
             for (int u = 0; u < 16; u++) {
-                const int k = base + w + 4 * u;
+                const int k = w + 4 * u;
                 if (k < chunks) t[u] = pp[(size_t)k * inner];
             }
 #pragma unroll
             for (int u = 0; u < 16; u++) {
-                const int k = base + w + 4 * u;
+                const int k = w + 4 * u;
                 if (k < chunks) acc = P::combine(acc, t[u]);
+            }
+        } else {
+            for (int base = 0; base < chunks; base += 128) {  // 128 chunks per round: 32 loads in flight per thread
+                Acc t[32];
+#pragma unroll
+                for (int u = 0; u < 32; u++) {
+                    const int k = base + w + 4 * u;
+                    if (k < chunks) t[u] = pp[(size_t)k * inner];
+                }
+#pragma unroll
+                for (int u = 0; u < 32; u++) {
+                    const int k = base + w + 4 * u;
+                    if (k < chunks) acc = P::combine(acc, t[u]);
+                }
             }
         }
     }

@@ -278,8 +278,31 @@ def op_suite(dev, quick=False, cpu=False):
         ms = timed(dev, lambda: dev.dispatch("index_select_fwd", src=X, indices=idx, stride=stride, dst=Z.sub(0, n_idx * stride)),
                    iters * 5)
         extra["index_select_fwd_65536x256"] = gbs(2 * n_idx * stride * 4 + n_idx * 8, ms)
+        # the deterministic scatter ops on a graph larger than the GCN configuration's (100 k nodes, 1 M edges, 64
+        # features): with the destination ordering computed on every call (bare index slices in device memory, as the
+        # reference hands them over) and with an edge plan made once for a graph that does not change
+        n_nodes, n_edge, feat = 100_000, 1_000_000, 64
+        e_src = dev.from_numpy(r.integers(0, n_nodes, n_edge).astype(np.uint64))
+        e_tgt = dev.from_numpy(r.integers(0, n_nodes, n_edge).astype(np.uint64))
+        h_buf, y_buf = X.sub(0, n_nodes * feat), Z.sub(0, n_nodes * feat)
+        deg = dev.mem_alloc(F32, n_nodes)
+        dev.mem_fill(deg, 1.0)
+        gcn_bytes = n_edge * feat * 4 + 2 * n_nodes * feat * 4 + n_edge * 16
+        ms = timed(dev, lambda: dev.dispatch("scatter_gcn_deg_scaled", dst=y_buf, h=h_buf, deg=deg, src_indices=e_src,
+                                             tgt_indices=e_tgt, stride=feat, n_edge=n_edge), iters)
+        extra["scatter_gcn_1Medges_x64_ordering_per_call"] = {**gbs(gcn_bytes, ms), "edges_per_us": n_edge / (ms["ms"] * 1e3)}
+        plan = dev.edge_plan(e_src, e_tgt, n_nodes)
+        ms = timed(dev, lambda: dev.dispatch("scatter_gcn_deg_scaled_planned", dst=y_buf, h=h_buf, deg=deg, plan=plan,
+                                             stride=feat, accumulate=True), iters)
+        extra["scatter_gcn_1Medges_x64_planned"] = {**gbs(gcn_bytes, ms), "edges_per_us": n_edge / (ms["ms"] * 1e3)}
+        vals = Y.sub(0, n_edge)
+        ms = timed(dev, lambda: dev.dispatch("scatter_add", src=vals, offsets=e_tgt, dst=y_buf.sub(0, n_nodes)), iters)
+        extra["scatter_add_1M_into_100k_ordering_per_call"] = {**ms, "entries_per_us": n_edge / (ms["ms"] * 1e3)}
+        ms = timed(dev, lambda: dev.dispatch("scatter_add_planned", src=vals, plan=plan, dst=y_buf.sub(0, n_nodes)), iters * 5)
+        extra["scatter_add_1M_into_100k_planned"] = {**ms, "entries_per_us": n_edge / (ms["ms"] * 1e3)}
+        plan.free()
         out["other_ops"] = extra
-        for b in (G, Y, ycol, yarg, ysc, idx):
+        for b in (G, Y, ycol, yarg, ysc, idx, e_src, e_tgt, deg):
             dev.mem_free(b)
     for b in (X, bias, Z, yrow):
         dev.mem_free(b)

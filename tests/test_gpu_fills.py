@@ -243,7 +243,6 @@ def test_a_refused_call_still_owes_the_zeros_it_took_over(hip):
     """An op that takes over a waiting zero fill and is then refused (an argument error) must leave the zeros behind:
     the caller asked for them and the refused op wrote nothing."""
     from zigrad_amd._lib import ZgHipError
-    from zigrad_amd.device import U64
 
     m, n, k = 24, 16, 8
     a = hip.from_numpy(np.ones(m * k, np.float32))

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from zigrad_amd import host
-from zigrad_amd.device import F32, U64
+from zigrad_amd.device import F32
 
 pytestmark = pytest.mark.gpu
 

@@ -94,7 +94,7 @@ def test_noalloc_launches_waiting_work_without_allocating():
     still waiting when the allocation-free entry point is called: the entry point launches it first.  The workspace
     the product needs was reserved by the call that queued it, so the allocation-free call makes no driver allocation
     (it reports one if it happens), and both results are right.  A context of its own: its workspace starts empty."""
-    from zigrad_amd.device import F32, U64, HipDevice
+    from zigrad_amd.device import F32, HipDevice
 
     dev = HipDevice(0)
     try:

@@ -294,7 +294,11 @@ int zg_hip_index_select_bwd(zg_hip_ctx *ctx, const float *y_grad, const uint64_t
  * dst (or of exactly grad_h / grad_deg in the backward) is taken over and the sums are written instead of added to
  * zeros; and the forward's kernel is launched by the NEXT call on the context: zg_hip_add of a row of `stride` values
  * onto dst in place (y._add(bias), examples/gcn/src/model.zig:110) and zg_hip_relu_fwd of dst in place (:36) become the
- * kernel's tail, any other call launches it first, unchanged.  Same values, bit for bit. */
+ * kernel's tail, any other call launches it first, unchanged.  Same values, bit for bit.  The backward launches the
+ * feature gradient at once and holds the two launches of the degree gradient for the next call: the reference's layer
+ * computes grad_deg into a buffer it gives back unread (the degrees are data of the graph, src/ndtensor.zig:1009), and
+ * a zg_hip_mem_cache_free of the block that holds all of grad_deg while they wait drops them; any other call launches
+ * them first. */
 int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx *ctx, float *dst, const float *h, const float *deg,
                                   const uint64_t *src_indices, const uint64_t *tgt_indices, size_t stride,
                                   size_t n_edge, size_t n_nodes);

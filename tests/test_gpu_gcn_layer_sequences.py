@@ -195,3 +195,50 @@ def test_layer_backward_with_waiting_zero_fills(oracle, hip, shape, pinned, zero
                                                          "n_edge": n_edge}, ["grad_h", "grad_deg"])
     np.testing.assert_array_equal(got[0], want["grad_h"].reshape(n_nodes, stride))
     np.testing.assert_array_equal(got[1], want["grad_deg"])
+
+
+@pytest.mark.parametrize("shape", [(2708, 13264, 16), (300, 2000, 5), (50, 5000, 64)])
+@pytest.mark.parametrize("pinned", [True, False])
+def test_a_degree_gradient_that_is_given_back_unread_is_never_computed_and_changes_nothing(oracle, hip, shape, pinned):
+    """The layer computes the degree gradient into a buffer it frees at once (the degrees are data of the graph,
+    src/ndtensor.zig:1009).  The two launches that compute it wait for the next call; a free of their output drops
+    them.  The feature gradient must be what it always was, a later owner of the freed block must not be written to,
+    and a degree gradient that IS read later (after frees of other blocks) must be right."""
+    n_nodes, n_edge, stride = shape
+    g = _graph(*shape, seed=7)
+    src, tgt, h, deg, _ = g
+    go = np.random.default_rng(8).standard_normal((n_nodes, stride)).astype(np.float32)
+    want = run_op(oracle, "scatter_gcn_deg_scaled_bwd", {"grad_output": go.ravel(), "h": h.ravel(), "deg": deg, "src_indices": src,
+                                                         "tgt_indices": tgt, "grad_h": np.zeros(n_nodes * stride, np.float32),
+                                                         "grad_deg": np.zeros(n_nodes, np.float32), "stride": stride,
+                                                         "n_edge": n_edge}, ["grad_h", "grad_deg"])
+    sb, tb = _index(hip, src, pinned), _index(hip, tgt, pinned)
+    hb, db, gob = hip.from_numpy(h), hip.from_numpy(deg), hip.from_numpy(go)
+    in_use0 = hip.cache_stats()["bytes_in_use"]
+    for read_it in (False, True):
+        gh = hip.mem_cache_alloc(F32, n_nodes * stride)
+        gd = hip.mem_cache_alloc(F32, n_nodes)
+        other = hip.mem_cache_alloc(F32, 64)
+        hip.mem_fill(gh, 0.0)
+        hip.mem_fill(gd, 0.0)
+        hip.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=gob, h=hb, deg=db, src_indices=sb, tgt_indices=tb, grad_h=gh,
+                     grad_deg=gd, stride=stride, n_edge=n_edge)
+        if read_it:
+            hip.mem_cache_free(other)              # a free of another block: the waiting work goes out, nothing is lost
+            np.testing.assert_array_equal(hip.to_numpy(gd), want["grad_deg"])
+            hip.mem_cache_free(gd)
+        else:
+            hip.mem_cache_free(gd)                 # unread: dropped
+            t = hip.mem_cache_alloc(F32, n_nodes)  # the same block again, most likely
+            marker = np.arange(n_nodes, dtype=np.float32)
+            hip.mem_transfer(marker, t, "HtoD")
+            hip.sync()
+            np.testing.assert_array_equal(hip.to_numpy(t), marker)
+            hip.mem_cache_free(t)
+            hip.mem_cache_free(other)
+        np.testing.assert_array_equal(hip.to_numpy(gh), want["grad_h"])
+        hip.mem_cache_free(gh)
+    hip.sync()
+    assert hip.cache_stats()["bytes_in_use"] == in_use0
+    for b in (sb, tb, hb, db, gob):
+        hip.mem_free(b)

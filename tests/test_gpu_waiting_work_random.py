@@ -184,14 +184,23 @@ class _Run:
         n_nodes, n_edge = self.graph
         stride = int(self.r.choice([4, 7, 16]))
         go, h, deg, gh, gd = self.picks(n_nodes * stride, n_nodes * stride, n_nodes, n_nodes * stride, n_nodes)
+        gd_temp = None
+        if self.r.random() < 0.5:          # the degree gradient in a block of its own that is given back unread
+            gd_temp = gd = self.hip.mem_cache_alloc(F32, n_nodes)
         if self.r.random() < 0.6:
             self.hip.mem_fill(gh, 0.0)
             self.done()
-        if self.r.random() < 0.6:
+        if self.r.random() < 0.6 or gd_temp is not None:
             self.hip.mem_fill(gd, 0.0)
             self.done()
         self.hip.dispatch("scatter_gcn_deg_scaled_bwd", grad_output=go, h=h, deg=deg, src_indices=self.src,
                           tgt_indices=self.tgt, grad_h=gh, grad_deg=gd, stride=stride, n_edge=n_edge)
+        if gd_temp is not None:
+            self.done()
+            if self.r.random() < 0.3:
+                self.hip.mem_fill(self.pick(16), 0.5)     # something else first: the degree gradient is computed after all
+                self.done()
+            self.hip.mem_cache_free(gd_temp)
 
     def op_loss(self):
         rows, cols = int(self.r.choice([8, 64])), int(self.r.choice([7, 10]))

@@ -89,6 +89,33 @@ struct zg_waiting_scatter {
     int relu = 0;                 // attached by a following in-place relu_fwd on dst
 };
 
+// The degree gradient of scatter_gcn_deg_scaled_bwd (two launches: the edge terms, then their sums per node), asked
+// for and not launched yet: the reference's graph-convolution layer computes it into a buffer that it gives back
+// unread (the degrees are data of the graph, src/ndtensor.zig:1009), and a job whose output block is freed while
+// it waits is dropped (index.hip).
+struct zg_waiting_graddeg {
+    bool active = false;
+    bool by_incidence = false;
+    const float* grad_output = nullptr;
+    const float* h = nullptr;
+    const float* deg = nullptr;
+    const uint64_t* src_idx = nullptr;
+    const uint64_t* tgt_idx = nullptr;
+    size_t n_edge = 0, n_nodes = 0, stride = 0;
+    float* grad_deg = nullptr;
+    bool fresh = false;
+    // by_incidence: terms in bucket order
+    const uint32_t* slot_of = nullptr;
+    const uint32_t* inc_row_ptr = nullptr;
+    // otherwise: two term arrays and the two orderings
+    float* term_src = nullptr;
+    float* term_tgt = nullptr;
+    const uint32_t* rp_src = nullptr;
+    const uint32_t* perm_src = nullptr;
+    const uint32_t* rp_tgt = nullptr;
+    const uint32_t* perm_tgt = nullptr;
+};
+
 // Optimizer steps of small tensors that have been asked for and not launched yet (optim.hip).
 constexpr int kMaxPendingSteps = 16;
 struct zg_pending_steps {
@@ -174,6 +201,7 @@ struct zg_hip_ctx {
     zg_deferred_gemm deferred_w;
     zg_waiting_bias bias_wait;
     zg_waiting_scatter scatter_wait;
+    zg_waiting_graddeg graddeg_wait;
     // Cache blocks that were given back while a waiting input-gradient product still names them as operands (the
     // reference frees a node's gradient as soon as its backward has run, src/ndtensor.zig eager teardown): they return
     // to the pool right after the product is launched.
@@ -221,6 +249,8 @@ int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, siz
 // Launches the waiting graph-convolution aggregation with what was attached to it (index.hip); the two hooks are for
 // zg_hip_add and zg_hip_relu_fwd, like deferred_take_add / deferred_take_relu below.
 int flush_scatter(zg_hip_ctx* ctx);
+// Launches the waiting degree gradient (index.hip).
+int flush_graddeg(zg_hip_ctx* ctx);
 bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);
 bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc);
 // Launches the optimizer steps that are waiting (optim.hip).  Gradients whose zero fill was taken over are zeroed by
@@ -305,7 +335,7 @@ inline bool aligned16(const void* p) {
 #define ZG_CTX(ctx)                                          \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
     if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
-        (ctx)->scatter_wait.active) {                        \
+        (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active) { \
         if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
     }
 // The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the
@@ -316,7 +346,13 @@ inline bool aligned16(const void* p) {
     ZG_REQUIRE((ctx) != nullptr, "null context");                \
     if ((ctx)->scatter_wait.active) {                            \
         if (int _rc_sc = zg::flush_scatter(ctx)) return _rc_sc;  \
+    }                                                            \
+    if ((ctx)->graddeg_wait.active) {                            \
+        if (int _rc_gd = zg::flush_graddeg(ctx)) return _rc_gd;  \
     }
+// zg_hip_mem_cache_free alone looks at the waiting degree gradient before it decides: the block that is given back may
+// be the one it would write.
+#define ZG_CTX_KEEP_ALL(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.
 #define ZG_NOT_CAPTURING(ctx, who)                                                                       \

@@ -1110,6 +1110,32 @@ int flush_scatter(zg_hip_ctx* ctx) {
     return ZG_HIP_OK;
 }
 
+int flush_graddeg(zg_hip_ctx* ctx) {
+    const zg_waiting_graddeg w = ctx->graddeg_wait;
+    if (!w.active) return ZG_HIP_OK;
+    ctx->graddeg_wait.active = false;
+    if (w.by_incidence) {
+        // 2 * n_edge terms in bucket order; the two separate term arrays' room holds them
+        float* terms = w.term_src;
+        hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel, dim3((unsigned)ceil_div_sz(w.n_edge, 256)), dim3(256), 0,
+                           ctx->stream, w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride,
+                           w.slot_of, terms, w.stride % 4 == 0 && aligned16(w.grad_output) && aligned16(w.h));
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(w.n_nodes, 256)), dim3(256), 0,
+                           ctx->stream, w.grad_deg, terms, w.inc_row_ptr, w.n_nodes, w.fresh);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(w.n_edge, 256)), dim3(256), 0, ctx->stream,
+                       w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride, w.term_src,
+                       w.term_tgt);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(w.n_nodes, 256)), dim3(256), 0, ctx->stream,
+                       w.grad_deg, w.term_src, w.term_tgt, w.rp_src, w.perm_src, w.rp_tgt, w.perm_tgt, w.n_nodes, w.fresh);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
 // y._add(bias): z = x + y in place on the aggregation's output, the other operand a row of `stride` values
 bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl) {
     zg_waiting_scatter& w = ctx->scatter_wait;
@@ -1234,25 +1260,34 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
                                         grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride, fresh_h));
     ZG_LAUNCH_CHECK();
+    // The degree gradient waits: whatever comes next launches it (its orderings and term arrays live in the cache or in
+    // the workspace, which no call touches before it has sent waiting work out), except a free of the block it would
+    // write, which drops it.
+    zg_waiting_graddeg& w = ctx->graddeg_wait;
+    w = zg_waiting_graddeg{};
+    w.active = true;
+    w.by_incidence = by_incidence;
+    w.grad_output = grad_output;
+    w.h = h;
+    w.deg = deg;
+    w.src_idx = src_indices;
+    w.tgt_idx = tgt_indices;
+    w.n_edge = n_edge;
+    w.n_nodes = n_nodes;
+    w.stride = stride;
+    w.grad_deg = grad_deg;
+    w.fresh = fresh_d;
+    w.term_src = term_src;
+    w.term_tgt = term_tgt;
     if (by_incidence) {
-        // 2 * n_edge terms in bucket order; the two separate term arrays' room holds them
-        float* terms = term_src;
-        hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0,
-                           ctx->stream, grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride,
-                           rs.entry->slot_of, terms, stride % 4 == 0 && aligned16(grad_output) && aligned16(h));
-        ZG_LAUNCH_CHECK();
-        hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0,
-                           ctx->stream, grad_deg, terms, rs.entry->inc.row_ptr, n_nodes, fresh_d);
-        ZG_LAUNCH_CHECK();
-        return ZG_HIP_OK;
+        w.slot_of = rs.entry->slot_of;
+        w.inc_row_ptr = rs.entry->inc.row_ptr;
+    } else {
+        w.rp_src = by_src.row_ptr;
+        w.perm_src = by_src.perm;
+        w.rp_tgt = by_tgt.row_ptr;
+        w.perm_tgt = by_tgt.perm;
     }
-    hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
-                       grad_output, h, deg, src_indices, tgt_indices, n_edge, n_nodes, stride, term_src, term_tgt);
-    ZG_LAUNCH_CHECK();
-    hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
-                       grad_deg, term_src, term_tgt, by_src.row_ptr, by_src.perm, by_tgt.row_ptr, by_tgt.perm, n_nodes,
-                       fresh_d);
-    ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
     }();
     if (rc_body) {  // refused before its kernels ran: the zeros that were taken over are still owed

@@ -855,7 +855,22 @@ void run_deferred_frees(zg_hip_ctx* ctx) {
 }  // namespace zg
 
 ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_CTX_KEEP_ALL(ctx);
+    if (ctx->scatter_wait.active)
+        if (int rc = flush_scatter(ctx)) return rc;
+    if (ctx->graddeg_wait.active) {
+        // a waiting degree gradient whose whole output lies in the block that is given back has no reader left and is
+        // dropped (the reference's layer frees it unread); any other free sends it out first
+        const zg_waiting_graddeg& w = ctx->graddeg_wait;
+        const Block* gb = (const Block*)(uintptr_t)block;
+        bool dead = false;
+        if (ptr && block)
+            for (BlockPool* p : {ctx->small_pool, ctx->large_pool})
+                if (p && p->owns_live(const_cast<Block*>(gb), ptr))
+                    dead = gb->ptr <= (const char*)w.grad_deg && (const char*)(w.grad_deg + w.n_nodes) <= gb->ptr + gb->size;
+        if (dead) ctx->graddeg_wait.active = false;
+        else if (int rc = flush_graddeg(ctx)) return rc;
+    }
     if (ctx->steps.count)
         if (int rc = flush_steps(ctx)) return rc;
     if (!ptr || block == 0) {  // views and empty data: src/allocators/caching_allocator.zig:111-112
@@ -1117,6 +1132,8 @@ int flush_pending(zg_hip_ctx* ctx) {
     // at most one kind is waiting at a time, except fills next to allocations: each kind's own calls send the others first
     if (ctx->scatter_wait.active)
         if (int rc = flush_scatter(ctx)) return rc;
+    if (ctx->graddeg_wait.active)
+        if (int rc = flush_graddeg(ctx)) return rc;
     if (gemm_group_waiting(ctx))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (int rc = flush_fills(ctx)) return rc;
@@ -1126,6 +1143,8 @@ int flush_pending(zg_hip_ctx* ctx) {
 int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
     if (ctx->scatter_wait.active)
         if (int rc = flush_scatter(ctx)) return rc;
+    if (ctx->graddeg_wait.active)
+        if (int rc = flush_graddeg(ctx)) return rc;
     if (gemm_group_waiting(ctx))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (ctx->steps.count)

@@ -139,6 +139,16 @@ int zg_hip_mem_random(zg_hip_ctx *ctx, float *x, size_t n, int kind, uint64_t fa
 /* ---------------------------------------------------------------------------------------------
  * elementwise binary (src/device/host_device.zig:205-219, :975-1019; opspec.zig:19-57)
  * requires max(xl,yl) % min(xl,yl) == 0 and zl == max(xl,yl); z may alias x or y
+ *
+ * Small elementwise ops wait.  These four with operands of one length or one operand of a single float, the unary
+ * forward and backward ops below, zg_hip_scale and the elementwise loss gradients, on at most 65536 elements, are not
+ * launched by their own call: up to eight that follow each other with the same length leave in one launch, in which
+ * thread i carries element i through the ops in call order (a caller's chain r + gamma * max_q * (1 - done) is one
+ * launch, not four).  An op joins only when every element it shares with a waiting op is shared at the same index (the
+ * same n floats, in place or not) and no waiting op writes a one-float operand; otherwise, and on any other call but
+ * zg_hip_mem_cache_alloc and zg_hip_mem_cache_free (a caller allocates each result just before its op and frees the
+ * temporaries afterwards; the pool keeps a freed block's memory), the waiting ops are launched first.  Same values,
+ * bit for bit, as a launch per call.
  * ------------------------------------------------------------------------------------------- */
 int zg_hip_add(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
 int zg_hip_sub(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);

@@ -1,0 +1,200 @@
+"""Small elementwise ops of one length wait in the context and go out as one launch (the reference launches each at
+once: src/device/host_device.zig:300-420).  Every result must be bit-identical to the ops run one launch each, which
+is what the same calls with a synchronisation after each of them give."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from zigrad_amd.device import F32
+
+pytestmark = pytest.mark.gpu
+
+
+def both_ways(hip, body):
+    """body(step) issues the calls and returns the buffers to compare; step() is called after every call."""
+    outs = []
+    for sync_each in (False, True):
+        step = hip.sync if sync_each else (lambda: None)
+        bufs = body(step)
+        outs.append([hip.to_numpy(b).view(np.uint32).copy() for b in bufs])
+        for b in bufs:
+            hip.mem_free(b)
+    for lazy, eager in zip(*outs):
+        np.testing.assert_array_equal(lazy, eager)
+    return outs[0]
+
+
+def test_td_target_chain_with_allocations_and_frees_between(hip):
+    """The op chain of a DQN target (examples/dqn/src/dqn_agent.zig:173-186): every op's output is allocated just
+    before it and the temporaries are given back afterwards."""
+    r = np.random.default_rng(0)
+    B = 64
+    q = r.standard_normal(B).astype(np.float32)
+    done = (r.random(B) < 0.3).astype(np.float32)
+    rew = r.standard_normal(B).astype(np.float32)
+
+    def body(step):
+        qd, dd, rd = hip.from_numpy(q), hip.from_numpy(done), hip.from_numpy(rew)
+        gamma, one = hip.from_numpy(np.float32([0.99])), hip.from_numpy(np.float32([1.0]))
+        out = hip.mem_alloc(F32, B)
+        disc = hip.mem_cache_alloc(F32, B); step()
+        hip.dispatch("mul", x=qd, y=gamma, z=disc); step()
+        nd = hip.mem_cache_alloc(F32, B); step()
+        hip.dispatch("sub", x=one, y=dd, z=nd); step()
+        masked = hip.mem_cache_alloc(F32, B); step()
+        hip.dispatch("mul", x=disc, y=nd, z=masked); step()
+        tgt = hip.mem_cache_alloc(F32, B); step()
+        hip.dispatch("add", x=rd, y=masked, z=tgt); step()
+        for t in (disc, nd, masked):
+            hip.mem_cache_free(t); step()
+        again = hip.mem_cache_alloc(F32, B); step()       # receives a block the waiting ops still use
+        hip.dispatch("relu_fwd", x=tgt, y=again); step()
+        hip.mem_copy(again, out); step()
+        hip.mem_cache_free(again); hip.mem_cache_free(tgt)
+        for t in (qd, dd, rd, gamma, one):
+            hip.mem_free(t)
+        return [out]
+
+    got = both_ways(hip, body)[0].view(np.float32)
+    want = np.maximum(rew + (q * np.float32(0.99)) * (np.float32(1.0) - done), 0)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_in_place_ops_and_results_feeding_later_ops(hip):
+    r = np.random.default_rng(1)
+    n = 1000
+    a0, b0 = r.standard_normal(n).astype(np.float32), r.standard_normal(n).astype(np.float32)
+
+    def body(step):
+        a, b, c = hip.from_numpy(a0), hip.from_numpy(b0), hip.mem_alloc(F32, n)
+        hip.dispatch("add", x=a, y=b, z=c); step()
+        hip.dispatch("mul", x=c, y=c, z=c); step()
+        hip.dispatch("tanh_fwd", x=c, y=a); step()        # overwrites an operand of the first op
+        hip.dispatch("sub", x=a, y=b, z=b); step()
+        hip.dispatch("scale", x=b, alpha=0.25); step()
+        hip.dispatch("relu_fwd", x=b, y=b); step()
+        hip.dispatch("sigm_fwd", x=c, y=c); step()
+        return [a, b, c]
+
+    a, b, c = (x.view(np.float32) for x in both_ways(hip, body))
+    s = (a0 + b0) * (a0 + b0)
+    np.testing.assert_allclose(a, np.tanh(s), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(b, np.maximum((a - b0) * np.float32(0.25), 0), rtol=0, atol=0)
+    np.testing.assert_allclose(c, 1 / (1 + np.exp(-s.astype(np.float64))), rtol=1e-5, atol=1e-6)
+
+
+def test_more_ops_than_the_queue_holds_and_a_change_of_length(hip):
+    n = 777
+    x0 = np.linspace(-2, 2, n).astype(np.float32)
+
+    def body(step):
+        x, y = hip.from_numpy(x0), hip.from_numpy(np.ones(n, np.float32))
+        for _ in range(21):
+            hip.dispatch("add", x=x, y=y, z=x); step()
+        hip.dispatch("mul", x=x.sub(0, 100), y=x.sub(0, 100), z=y.sub(0, 100)); step()   # another length: a new run
+        hip.dispatch("add", x=x, y=y, z=y); step()
+        return [x, y]
+
+    x, y = (v.view(np.float32) for v in both_ways(hip, body))
+    want_x = x0.copy()
+    for _ in range(21):
+        want_x = want_x + np.float32(1)
+    np.testing.assert_array_equal(x, want_x)
+    want_y = np.ones(n, np.float32)
+    want_y[:100] = x[:100] * x[:100]
+    np.testing.assert_array_equal(y, x + want_y)
+
+
+def test_views_that_overlap_out_of_step_do_not_share_a_launch(hip):
+    """Element i of the second op reads what the first wrote at i + 4: two launches, or thread i would read before
+    thread i + 4 has written."""
+    n = 4096
+    x0 = np.arange(n + 8, dtype=np.float32)
+
+    def body(step):
+        buf, one = hip.from_numpy(x0), hip.from_numpy(np.ones(n, np.float32))
+        out = hip.mem_alloc(F32, n)
+        hip.dispatch("add", x=buf.sub(4, n), y=one, z=buf.sub(4, n)); step()
+        hip.dispatch("mul", x=buf.sub(0, n), y=one, z=out); step()       # reads the shifted view
+        hip.dispatch("add", x=out, y=one, z=buf.sub(8, n)); step()       # writes over what the ops before read
+        return [buf, out, one]
+
+    buf, out, _ = (v.view(np.float32) for v in both_ways(hip, body))
+    mid = x0.copy()
+    mid[4:4 + n] += 1
+    np.testing.assert_array_equal(out, mid[:n])
+    mid[8:8 + n] = out + 1
+    np.testing.assert_array_equal(buf, mid)
+
+
+def test_a_one_float_operand_written_by_an_op_of_the_run(hip):
+    n = 64
+    v0 = np.arange(n, dtype=np.float32)
+
+    def body(step):
+        v, s, w = hip.from_numpy(v0), hip.from_numpy(np.float32([2.0, 0, 0, 0])), hip.mem_alloc(F32, n)
+        hip.dispatch("mul", x=v, y=s.sub(0, 1), z=w); step()
+        hip.dispatch("add", x=s.sub(0, 1), y=s.sub(0, 1), z=s.sub(0, 1)); step()   # the scalar doubles: length 1
+        hip.dispatch("mul", x=w, y=s.sub(0, 1), z=w); step()
+        hip.dispatch("scale", x=s, alpha=0.5); step()                               # length 4, covers the scalar
+        hip.dispatch("add", x=s.sub(0, 1), y=w, z=w); step()
+        return [w, s]
+
+    w, s = (x.view(np.float32) for x in both_ways(hip, body))
+    np.testing.assert_array_equal(w, v0 * 2 * 4 + 2)
+    np.testing.assert_array_equal(s, np.float32([2, 0, 0, 0]))
+
+
+def test_long_operands_and_other_calls_between(hip):
+    """Ops past the waiting length take their own launches; a call of another kind (a fill, a reduction, a read) sends
+    the waiting ops out first."""
+    n = 70_000
+    x0 = np.linspace(0, 1, n).astype(np.float32)
+
+    def body(step):
+        x, y = hip.from_numpy(x0), hip.mem_alloc(F32, n)
+        small = hip.mem_alloc(F32, 256)
+        hip.dispatch("add", x=x, y=x, z=y); step()                       # too long to wait
+        hip.dispatch("mul", x=y.sub(0, 256), y=y.sub(0, 256), z=small); step()
+        hip.mem_fill(y.sub(0, 256), 3.0); step()                         # overwrites an operand of the waiting op
+        hip.dispatch("add", x=small, y=y.sub(0, 256), z=small); step()
+        total = hip.mem_alloc(F32, 1)
+        hip.dispatch("sum", x=small, y=total); step()
+        hip.dispatch("mul", x=small, y=total, z=small); step()
+        return [y, small, total]
+
+    y, small, total = (v.view(np.float32) for v in both_ways(hip, body))
+    want_small = (2 * x0[:256]) ** 2 + 3
+    np.testing.assert_array_equal(y[256:], 2 * x0[256:])
+    np.testing.assert_array_equal(y[:256], np.full(256, 3, np.float32))
+    np.testing.assert_allclose(total[0], want_small.sum(dtype=np.float64), rtol=1e-6)
+    np.testing.assert_array_equal(small, want_small * total[0])
+
+
+def test_a_run_recorded_into_a_graph_replays(hip):
+    n = 512
+    x0 = np.linspace(-1, 1, n).astype(np.float32)
+    x, y = hip.from_numpy(x0), hip.from_numpy(np.zeros(n, np.float32))
+    half = hip.from_numpy(np.float32([0.5]))
+
+    def calls():
+        t = hip.mem_cache_alloc(F32, n)
+        hip.dispatch("mul", x=x, y=half, z=t)
+        hip.dispatch("add", x=t, y=y, z=y)
+        hip.dispatch("relu_fwd", x=y, y=y)
+        hip.mem_cache_free(t)
+
+    calls()                                   # eager once: the pool grows outside the recording
+    hip.graph_open()
+    calls()
+    g = hip.graph_save()
+    want = np.maximum(x0 * np.float32(0.5), 0)
+    for k in range(2, 6):
+        g.run()
+        hip.sync()
+        want = np.maximum(x0 * np.float32(0.5) + want, 0)
+        np.testing.assert_array_equal(hip.to_numpy(y), want)
+    g.free()
+    for b in (x, y, half):
+        hip.mem_free(b)

@@ -248,6 +248,66 @@ class _Run:
         else:
             self.hip.dispatch("tanh_fwd", x=a, y=b)
 
+    def op_map_run(self):
+        """A run of small elementwise ops of one length over a few buffers: results feeding later ops, in-place forms,
+        one-float operands, and now and then a view shifted against one an earlier op of the run wrote."""
+        n = int(self.r.choice([1, 64, 1000, 4096]))
+        picked = self.picks(n, n, n, n, 1, 1)     # six different buffers: a one-float operand never lies in an output
+        views, scalars = picked[:4], picked[4:]
+        fresh = []                                        # outputs allocated inside the run, as a caller's op chain does
+        for _ in range(int(self.r.integers(2, 6))):
+            x, y, z = (views[int(v)] for v in self.r.integers(0, len(views), 3))
+            if fresh and self.r.random() < 0.3:           # given back while the ops that use it may still wait
+                t = fresh.pop(int(self.r.integers(0, len(fresh))))
+                views = [v for v in views if v.ptr != t.ptr]
+                self.hip.mem_cache_free(t)
+                continue
+            if self.r.random() < 0.3:
+                z = self.hip.mem_cache_alloc(F32, n)
+                fresh.append(z)
+                views = views + [z]
+                kind = int(self.r.integers(0, 3))         # a new block holds nothing: ops that only write it
+                if kind == 0:
+                    self.hip.dispatch(str(self.r.choice(["add", "sub", "mul"])), x=x, y=y, z=z)
+                elif kind == 1:
+                    self.hip.dispatch("mul", x=x, y=scalars[0], z=z)
+                else:
+                    self.hip.dispatch("tanh_fwd", x=x, y=z)
+                self.done()
+                continue
+            if self.r.random() < 0.15 and n > 8:          # shifted against a buffer of the run
+                base = views[int(self.r.integers(0, len(views)))]
+                room = [b for b in self.bufs + self.temps + fresh if b.ptr <= base.ptr < b.ptr + 4 * b.n][0]
+                off = (base.ptr - room.ptr) // 4 + 4
+                if off + n <= room.n:
+                    x = room.sub(off, n)
+            if x.ptr != z.ptr and x.ptr < z.ptr + 4 * n and z.ptr < x.ptr + 4 * n:
+                continue                                  # an op that reads a shifted view of its own output races with itself
+            kind = int(self.r.integers(0, 8))
+            if kind == 0:
+                self.hip.dispatch(str(self.r.choice(["add", "sub", "mul"])), x=x, y=y, z=z)
+            elif kind == 1:
+                s = scalars[int(self.r.integers(0, 2))]
+                if self.r.random() < 0.5:
+                    self.hip.dispatch(str(self.r.choice(["add", "mul", "sub"])), x=s, y=y, z=z)
+                else:
+                    self.hip.dispatch(str(self.r.choice(["add", "mul", "sub"])), x=x, y=s, z=z)
+            elif kind == 2:
+                self.hip.dispatch(str(self.r.choice(["relu_fwd", "tanh_fwd", "sigm_fwd"])), x=x, y=z)
+            elif kind == 3:
+                self.hip.dispatch("relu_fwd", x=z, y=z)
+            elif kind == 4 and x.ptr != z.ptr and y.ptr != z.ptr:
+                self.hip.dispatch(str(self.r.choice(["relu_bwd"])), x=x, x_g=z, y_g=y)
+            elif kind == 5 and x.ptr != z.ptr and y.ptr != z.ptr:
+                self.hip.dispatch(str(self.r.choice(["tanh_bwd", "sigm_bwd"])), x_g=z, y=x, y_g=y)
+            elif kind == 6 and x.ptr != z.ptr:
+                self.hip.dispatch(str(self.r.choice(["relu_inplace_bwd", "tanh_inplace_bwd"])), x=x, x_g=z)
+            elif kind == 7:
+                self.hip.dispatch("scale", x=z, alpha=0.5)
+            self.done()
+        for t in fresh:
+            self.hip.mem_cache_free(t)
+
     def op_read(self):
         if not self.with_reads:
             return
@@ -260,8 +320,8 @@ class _Run:
         self.last_c = None
         ops = [self.op_fill, self.op_matmul, self.op_add_row, self.op_relu, self.op_relu_mask, self.op_layer_backward,
                self.op_unbroadcast, self.op_step, self.op_scatter, self.op_alloc, self.op_free, self.op_read, self.op_copy,
-               self.op_elementwise, self.op_scatter_bwd, self.op_loss]
-        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1], float)
+               self.op_elementwise, self.op_scatter_bwd, self.op_loss, self.op_map_run]
+        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1, 3], float)
         for _ in range(n_ops):
             ops[int(self.r.choice(len(ops), p=weights / weights.sum()))]()
             self.done()

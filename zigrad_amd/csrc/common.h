@@ -116,6 +116,27 @@ struct zg_waiting_graddeg {
     const uint32_t* perm_tgt = nullptr;
 };
 
+// Small elementwise ops of one length that have been asked for and not launched yet (elementwise.hip): the reference's
+// autograd issues runs of them (a target r + gamma * max * (1 - done), a degree normalisation rsqrt(deg + count)), and
+// a run leaves as one launch in which thread i carries element i through every op in call order.
+constexpr int kMaxWaitingMaps = 8;
+constexpr size_t kWaitingMapMaxLen = 65536;
+struct zg_map_op {
+    int code;           // which functor (elementwise.hip)
+    int nin;            // array operands read: a, then b, then c
+    int scalar;         // 0: every operand has one element per output; 1: b is one float; 2: a is one float
+    float* out;
+    const float* a;
+    const float* b;
+    const float* c;
+    float p0, p1;
+};
+struct zg_waiting_maps {
+    int count = 0;
+    size_t n = 0;
+    zg_map_op op[kMaxWaitingMaps];
+};
+
 // Optimizer steps of small tensors that have been asked for and not launched yet (optim.hip).
 constexpr int kMaxPendingSteps = 16;
 struct zg_pending_steps {
@@ -202,6 +223,7 @@ struct zg_hip_ctx {
     zg_waiting_bias bias_wait;
     zg_waiting_scatter scatter_wait;
     zg_waiting_graddeg graddeg_wait;
+    zg_waiting_maps maps;
     // Cache blocks that were given back while a waiting input-gradient product still names them as operands (the
     // reference frees a node's gradient as soon as its backward has run, src/ndtensor.zig eager teardown): they return
     // to the pool right after the product is launched.
@@ -251,6 +273,9 @@ int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, siz
 int flush_scatter(zg_hip_ctx* ctx);
 // Launches the waiting degree gradient (index.hip).
 int flush_graddeg(zg_hip_ctx* ctx);
+// Launches the waiting elementwise ops as one kernel (elementwise.hip); flush_pending_but_maps: everything else.
+int flush_maps(zg_hip_ctx* ctx);
+int flush_pending_but_maps(zg_hip_ctx* ctx);
 bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);
 bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc);
 // Launches the optimizer steps that are waiting (optim.hip).  Gradients whose zero fill was taken over are zeroed by
@@ -335,12 +360,11 @@ inline bool aligned16(const void* p) {
 #define ZG_CTX(ctx)                                          \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
     if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
-        (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active) { \
+        (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active || (ctx)->maps.count) { \
         if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
     }
 // The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the
-// calls a product may absorb, and cache allocations (a block that is handed out is free, so no waiting fill names it;
-// a block that is freed goes through ZG_CTX).
+// calls a product may absorb.
 // A waiting aggregation only waits for the add and the ReLU, which look at it before they get here: it goes out.
 #define ZG_CTX_KEEP_FILLS(ctx)                                   \
     ZG_REQUIRE((ctx) != nullptr, "null context");                \
@@ -349,9 +373,21 @@ inline bool aligned16(const void* p) {
     }                                                            \
     if ((ctx)->graddeg_wait.active) {                            \
         if (int _rc_gd = zg::flush_graddeg(ctx)) return _rc_gd;  \
+    }                                                            \
+    if ((ctx)->maps.count) {                                     \
+        if (int _rc_mp = zg::flush_maps(ctx)) return _rc_mp;     \
     }
-// zg_hip_mem_cache_free alone looks at the waiting degree gradient before it decides: the block that is given back may
-// be the one it would write.
+// The small elementwise ops: everything else that waits goes out, the waiting elementwise ops stay (the call joins
+// them or sends them out itself).
+#define ZG_CTX_KEEP_MAPS(ctx)                                    \
+    ZG_REQUIRE((ctx) != nullptr, "null context");                \
+    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
+        (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active) { \
+        if (int _rc_km = zg::flush_pending_but_maps(ctx)) return _rc_km; \
+    }
+// The cache's allocations and frees look at each kind of waiting work themselves: a block that is handed out is free,
+// so nothing that waits names it; a block that is given back may be the one a waiting degree gradient would write, or
+// hold operands of waiting elementwise ops, which the pool's memory outlives.
 #define ZG_CTX_KEEP_ALL(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.

@@ -71,10 +71,24 @@ static int map_grid(zg_hip_ctx* ctx, size_t items, int per_block) {
     return (int)(blocks < 1 ? 1 : blocks);
 }
 
+// Waiting elementwise ops (see zg_waiting_maps): chain_code<Op>() is the op's number in the one-launch kernel, -1 for
+// an op that always takes its own launch; chain_push queues an op, sending the waiting ones out first when it cannot
+// join them; false: the caller launches the op itself (after flush_maps).
+template <class Op> constexpr int chain_code() { return -1; }
+static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* out, const float* a, const float* b,
+                       const float* c, size_t n, float p0, float p1, int* rc);
+
 template <class Op, int NIN>
 static int launch_map(zg_hip_ctx* ctx, float* out, const float* a, const float* b, const float* c, size_t n,
                       float p0 = 0.f, float p1 = 0.f) {
     if (n == 0) return ZG_HIP_OK;
+    {
+        int rc = ZG_HIP_OK;
+        if (chain_code<Op>() >= 0 && chain_push(ctx, chain_code<Op>(), NIN, 0, out, a, b, c, n, p0, p1, &rc)) return rc;
+        if (rc) return rc;
+        if (ctx->maps.count)
+            if ((rc = flush_maps(ctx))) return rc;
+    }
     bool vec = aligned16(out) && aligned16(a) && (NIN < 2 || aligned16(b)) && (NIN < 3 || aligned16(c)) && n >= 4;
     if (vec) {
         int grid = map_grid(ctx, n >> 2, kBlock * kUnroll);
@@ -188,7 +202,7 @@ __global__ void broadcast_modulo_kernel(float* y, const float* x, size_t xl, siz
 template <class B>
 static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t xl, const float* y, size_t yl, float* z,
                      size_t zl) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_MAPS(ctx);
     ZG_REQUIRE(xl > 0 && yl > 0 && zl > 0, "%s: empty operand", name);
     ZG_REQUIRE(x && y && z, "%s: null pointer", name);
     const size_t mx = xl > yl ? xl : yl, mn = xl < yl ? xl : yl;
@@ -198,6 +212,13 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
 
     if (xl == yl) return launch_map<Bin2<B>, 2>(ctx, z, x, y, nullptr, zl);
     if (mn == 1) {
+        {
+            int rc = ZG_HIP_OK;
+            if (chain_push(ctx, chain_code<Bin2<B>>(), 2, xl == 1 ? 2 : 1, z, x, y, nullptr, zl, 0.f, 0.f, &rc)) return rc;
+            if (rc) return rc;
+        }
+        if (ctx->maps.count)
+            if (int rc = flush_maps(ctx)) return rc;
         int grid = map_grid(ctx, (zl + 3) / 4, kBlock);
         if (xl == 1)
             hipLaunchKernelGGL((bin_scalar_kernel<B, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, y, x, zl);
@@ -206,6 +227,8 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
+    if (ctx->maps.count)
+        if (int rc = flush_maps(ctx)) return rc;
     const bool short_lhs = xl < yl;
     const float* lng = short_lhs ? y : x;
     const float* sht = short_lhs ? x : y;
@@ -281,12 +304,112 @@ ZG_OP(ScaledCopyNoRead, return __fmul_rn(p0, a);)
 ZG_OP(SmoothL1Bwd, return __fadd_rn(c, smooth_l1_grad(a, b, p0, p1));)
 ZG_OP(MseBwd, return __fadd_rn(c, __fmul_rn(p0, __fsub_rn(a, b)));)
 
+// ------------------------------------------------------------------------------------------------
+// waiting elementwise ops: one launch for a run of small ops of one length
+// ------------------------------------------------------------------------------------------------
+#define ZG_CHAIN_OPS(X)                                                                                              \
+    X(0, Bin2<AddOp>) X(1, Bin2<SubOp>) X(2, Bin2<MulOp>) X(3, Bin2<DivOp>) X(4, PowFwd) X(5, SqrtFwd) X(6, RsqrtFwd) \
+    X(7, ExpFwd) X(8, ReluFwd) X(9, TanhFwd) X(10, SigmFwd) X(11, ClampFwd) X(12, PowBwd) X(13, SqrtBwd)             \
+    X(14, RsqrtBwd) X(15, ExpBwd) X(16, ReluBwd) X(17, ReluInplaceBwd) X(18, TanhBwd) X(19, TanhInplaceBwd)          \
+    X(20, SigmBwd) X(21, SigmInplaceBwd) X(22, ClampBwd) X(23, ScaleOp) X(24, SmoothL1Bwd) X(25, MseBwd)
+#define ZG_CHAIN_CODE(N, OP) template <> constexpr int chain_code<OP>() { return N; }
+ZG_CHAIN_OPS(ZG_CHAIN_CODE)
+#undef ZG_CHAIN_CODE
+
+struct MapChainArgs {
+    zg_map_op op[kMaxWaitingMaps];
+    int count;
+    size_t n;
+};
+// Thread i carries element i through the ops in call order: each op loads its operands from memory and stores its
+// result, so an op that reads what an earlier one wrote (always at the same index: the queue admits nothing else) gets
+// it from its own store.  The arithmetic is each op's functor, as in its own kernel.
+__global__ __launch_bounds__(kBlock) void map_chain_kernel(MapChainArgs g) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= g.n) return;
+    for (int k = 0; k < g.count; k++) {
+        const zg_map_op& o = g.op[k];
+        const float a = o.a[o.scalar == 2 ? 0 : i];
+        const float b = o.nin > 1 ? o.b[o.scalar == 1 ? 0 : i] : 0.f;
+        const float c = o.nin > 2 ? o.c[i] : 0.f;
+        float r = 0.f;
+        switch (o.code) {
+#define ZG_CHAIN_CASE(N, OP) case N: r = OP::f(a, b, c, o.p0, o.p1); break;
+            ZG_CHAIN_OPS(ZG_CHAIN_CASE)
+#undef ZG_CHAIN_CASE
+        }
+        o.out[i] = r;
+    }
+}
+
+int flush_maps(zg_hip_ctx* ctx) {
+    zg_waiting_maps& q = ctx->maps;
+    if (q.count == 0) return ZG_HIP_OK;
+    MapChainArgs g;
+    for (int k = 0; k < q.count; k++) g.op[k] = q.op[k];
+    g.count = q.count;
+    g.n = q.n;
+    q.count = 0;
+    hipLaunchKernelGGL(map_chain_kernel, dim3((unsigned)ceil_div_sz(g.n, kBlock)), dim3(kBlock), 0, ctx->stream, g);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
+// Two accesses of which one writes may share a launch when they cannot meet, or when they are the same n elements (then
+// thread i alone touches element i of both, in call order).  A one-float operand is read by every thread, so nothing in
+// the run may write it.
+struct MapRange {
+    const char* lo;
+    const char* hi;
+    bool per_element;
+};
+static bool map_ranges_conflict(const MapRange& w, const MapRange& o) {
+    if (!(w.lo < o.hi && o.lo < w.hi)) return false;
+    return !(w.per_element && o.per_element && w.lo == o.lo && w.hi == o.hi);
+}
+static int map_op_ranges(const zg_map_op& o, size_t n, MapRange* r) {  // r[0] is the output
+    int m = 0;
+    auto put = [&](const float* p, bool scalar) {
+        r[m++] = MapRange{(const char*)p, (const char*)(p + (scalar ? 1 : n)), !scalar};
+    };
+    put(o.out, false);
+    put(o.a, o.scalar == 2);
+    if (o.nin > 1) put(o.b, o.scalar == 1);
+    if (o.nin > 2) put(o.c, false);
+    return m;
+}
+
+static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* out, const float* a, const float* b,
+                       const float* c, size_t n, float p0, float p1, int* rc) {
+    *rc = ZG_HIP_OK;
+    if (code < 0 || n == 0 || n > kWaitingMapMaxLen) return false;
+    zg_map_op o{code, nin, scalar, out, a, b, c, p0, p1};
+    MapRange mine[4];
+    const int n_mine = map_op_ranges(o, n, mine);
+    // the op's own operands: in place is fine, a shifted overlap is not (its own kernel would race too: let it)
+    for (int j = 1; j < n_mine; j++)
+        if (map_ranges_conflict(mine[0], mine[j])) return false;
+    zg_waiting_maps& q = ctx->maps;
+    bool joins = q.count > 0 && q.count < kMaxWaitingMaps && q.n == n;
+    for (int k = 0; k < q.count && joins; k++) {
+        MapRange theirs[4];
+        const int n_theirs = map_op_ranges(q.op[k], q.n, theirs);
+        for (int j = 0; j < n_mine && joins; j++) joins = !map_ranges_conflict(theirs[0], mine[j]);   // they write
+        for (int j = 1; j < n_theirs && joins; j++) joins = !map_ranges_conflict(mine[0], theirs[j]);  // I write
+    }
+    if (q.count > 0 && !joins)
+        if ((*rc = flush_maps(ctx))) return false;
+    if (q.count == 0) q.n = n;
+    q.op[q.count++] = o;
+    return true;
+}
+
 }  // namespace zg
 
 using namespace zg;
 
 #define ZG_CHECK_N(name, n, ...)                                         \
-    ZG_CTX(ctx);                                                         \
+    ZG_CTX_KEEP_MAPS(ctx);                                               \
     if ((n) == 0) return ZG_HIP_OK;                                      \
     {                                                                    \
         const void* _ptrs[] = {__VA_ARGS__};                             \

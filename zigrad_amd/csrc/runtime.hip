@@ -807,7 +807,13 @@ ZG_API int zg_hip_cache_configure(zg_hip_ctx* ctx, size_t small_pool_bytes, size
 }
 
 ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uint64_t* block) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_CTX_KEEP_ALL(ctx);
+    // waiting fills stay (a block that is handed out is free, so no waiting fill names it), and so do waiting
+    // elementwise ops: a new block holds no operand of theirs, and a caller allocates each op's output just before it
+    if (ctx->scatter_wait.active)
+        if (int rc = flush_scatter(ctx)) return rc;
+    if (ctx->graddeg_wait.active)
+        if (int rc = flush_graddeg(ctx)) return rc;
     // what a waiting product waits for comes right after it, not after an allocation; a bias gradient that waits
     // alone stays (the input gradient its layer's products write is allocated next, and a new block holds no operand)
     if (ctx->deferred.active)
@@ -856,6 +862,9 @@ void run_deferred_frees(zg_hip_ctx* ctx) {
 
 ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
     ZG_CTX_KEEP_ALL(ctx);
+    // Waiting elementwise ops stay: the pool keeps the block's memory, so they may still read and write it when they
+    // are launched, and whoever receives the block next either joins them (in call order, element by element) or sends
+    // them out first.
     if (ctx->scatter_wait.active)
         if (int rc = flush_scatter(ctx)) return rc;
     if (ctx->graddeg_wait.active) {
@@ -1130,6 +1139,11 @@ int flush_fills(zg_hip_ctx* ctx) {
 }
 int flush_pending(zg_hip_ctx* ctx) {
     // at most one kind is waiting at a time, except fills next to allocations: each kind's own calls send the others first
+    if (ctx->maps.count)
+        if (int rc = flush_maps(ctx)) return rc;
+    return flush_pending_but_maps(ctx);
+}
+int flush_pending_but_maps(zg_hip_ctx* ctx) {
     if (ctx->scatter_wait.active)
         if (int rc = flush_scatter(ctx)) return rc;
     if (ctx->graddeg_wait.active)
@@ -1141,6 +1155,8 @@ int flush_pending(zg_hip_ctx* ctx) {
 }
 
 int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
+    if (ctx->maps.count)
+        if (int rc = flush_maps(ctx)) return rc;
     if (ctx->scatter_wait.active)
         if (int rc = flush_scatter(ctx)) return rc;
     if (ctx->graddeg_wait.active)

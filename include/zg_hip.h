@@ -123,8 +123,10 @@ int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
  * end included, therefore finds the memory filled; only work queued on the raw stream obtained EARLIER from
  * zg_hip_stream, with no call on the context in between, could overtake a waiting fill.  A waiting fill of +0.0 over
  * exactly the dense output of zg_hip_matmul / zg_hip_bmm_acc with beta = 1, the gradient of zg_hip_smce_bwd, the output
- * of zg_hip_scatter_gcn_deg_scaled or a gradient of zg_hip_scatter_gcn_deg_scaled_bwd is not
- * launched at all: the op writes what it would have added to the zeros; one over exactly the gradient of an optimizer
+ * of zg_hip_scatter_gcn_deg_scaled, a gradient of zg_hip_scatter_gcn_deg_scaled_bwd or the destination of
+ * zg_hip_scatter_add is not launched at all: the op writes what it would have added to the zeros; a waiting fill of any
+ * value over exactly the output of a small elementwise op (see below) is taken over likewise, and one inside the output
+ * of zg_hip_max_along, which writes every element and reads none, is dropped; one over exactly the gradient of an optimizer
  * step that is itself still waiting (zero_grad() after step()) is stored by the step's update kernel; and a waiting
  * fill that lies inside a cache block handed back with zg_hip_mem_cache_free is dropped (nobody can read it any more). */
 int zg_hip_mem_fill(zg_hip_ctx *ctx, float *x, size_t n, float value);
@@ -147,8 +149,8 @@ int zg_hip_mem_random(zg_hip_ctx *ctx, float *x, size_t n, int kind, uint64_t fa
  * launch, not four).  An op joins only when every element it shares with a waiting op is shared at the same index (the
  * same n floats, in place or not) and no waiting op writes a one-float operand; otherwise, and on any other call but
  * zg_hip_mem_cache_alloc and zg_hip_mem_cache_free (a caller allocates each result just before its op and frees the
- * temporaries afterwards; the pool keeps a freed block's memory), the waiting ops are launched first.  Same values,
- * bit for bit, as a launch per call.
+ * temporaries afterwards; the pool keeps a freed block's memory), the waiting ops are launched first.  Waiting float
+ * fills that meet none of an op's operands stay waiting.  Same values, bit for bit, as a launch per call.
  * ------------------------------------------------------------------------------------------- */
 int zg_hip_add(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
 int zg_hip_sub(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);

@@ -198,3 +198,149 @@ def test_a_run_recorded_into_a_graph_replays(hip):
     g.free()
     for b in (x, y, half):
         hip.mem_free(b)
+
+
+@pytest.mark.parametrize("value", [0.0, -0.0, 0.25])
+def test_a_fill_of_exactly_the_output_is_taken_over(hip, value):
+    """ensure_grad(0) followed by an accumulating backward op (src/ndtensor.zig:221-228): the op takes the fill's value
+    where it would have read the output, whatever the value, and other waiting fills are left alone."""
+    r = np.random.default_rng(3)
+    n = 300
+    x0, g0 = r.standard_normal(n).astype(np.float32), r.standard_normal(n).astype(np.float32)
+    g0[::7] = -0.0
+    x0[::7] = 1.0
+
+    def body(step):
+        x, yg = hip.from_numpy(x0), hip.from_numpy(g0)
+        xg, other, z = hip.from_numpy(np.ones(n, np.float32)), hip.from_numpy(np.ones(n, np.float32)), hip.mem_alloc(F32, n)
+        hip.mem_fill(other, 7.0); step()
+        hip.mem_fill(xg, value); step()
+        hip.dispatch("relu_bwd", x=x, x_g=xg, y_g=yg); step()          # xg = fill + (x > 0 ? yg : 0)
+        hip.mem_fill(z, value); step()
+        hip.dispatch("mul", x=x, y=yg, z=z); step()                     # overwrites the filled output
+        hip.mem_fill(xg.sub(0, n // 2), value); step()                  # only part of the output: must be seen
+        hip.dispatch("tanh_inplace_bwd", x=x, x_g=xg); step()
+        hip.dispatch("add", x=other, y=z, z=z); step()                  # reads the fill that kept waiting
+        return [xg, z, other, x, yg]
+
+    xg, z, other = (v.view(np.float32) for v in both_ways(hip, body)[:3])
+    want = np.float32(value) + np.where(x0 > 0, g0, np.float32(0))
+    want[:n // 2] = np.float32(value)
+    want = want * (np.float32(1) - x0 * x0)
+    np.testing.assert_array_equal(xg.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    np.testing.assert_array_equal(other, np.full(n, 7, np.float32))
+    np.testing.assert_array_equal(z, np.float32(7) + x0 * g0)
+
+
+def test_max_along_over_a_filled_output(hip):
+    """NDArray.max_along zero-fills its output and then writes every element (src/ndarray.zig:567): the fill is never
+    launched; a fill that reaches past the output is."""
+    r = np.random.default_rng(4)
+    rows, cols = 64, 2
+    q0 = r.standard_normal(rows * cols).astype(np.float32)
+
+    def body(step):
+        q, room = hip.from_numpy(q0), hip.from_numpy(np.full(rows + 8, -1, np.float32))
+        hip.mem_fill(room.sub(0, rows), 0.0); step()
+        hip.dispatch("max_along", x=q, x_shape=[rows, cols], y=room.sub(0, rows), y_shape=[rows], dim=1); step()
+        first = hip.mem_alloc(F32, rows)
+        hip.mem_copy(room.sub(0, rows), first); step()
+        hip.mem_fill(room.sub(4, rows + 4), 2.0); step()               # sticks out of the output
+        hip.dispatch("max_along", x=q, x_shape=[rows, cols], y=room.sub(0, rows), y_shape=[rows], dim=1); step()
+        return [first, room, q]
+
+    first, room = (v.view(np.float32) for v in both_ways(hip, body)[:2])
+    want = q0.reshape(rows, cols).max(axis=1)
+    np.testing.assert_array_equal(first, want)
+    np.testing.assert_array_equal(room[:rows], want)
+    np.testing.assert_array_equal(room[rows:], np.float32([2, 2, 2, 2, 2, 2, 2, 2]))
+
+
+@pytest.mark.parametrize("n,nb", [(64, 128), (200, 50), (1000, 300), (5000, 20000)])
+def test_scatter_add_into_a_destination_whose_zero_fill_waits(hip, n, nb):
+    """GatherBwd (src/ndtensor.zig:1367-1380): the gradient is zero-filled, then scattered into; the zeros of the
+    untouched elements come from the scatter's own launch.  Other fills are not taken over."""
+    r = np.random.default_rng(n)
+    src0 = r.standard_normal(n).astype(np.float32)
+    off0 = r.integers(0, nb + nb // 8, n).astype(np.uint64)               # a few past the end: skipped
+
+    def body(step):
+        src, off = hip.from_numpy(src0), hip.from_numpy(off0)
+        a, b, c = (hip.from_numpy(np.full(nb, 9, np.float32)) for _ in range(3))
+        hip.mem_fill(a, 0.0); step()
+        hip.dispatch("scatter_add", src=src, offsets=off, dst=a); step()
+        hip.mem_fill(b, 0.5); step()
+        hip.dispatch("scatter_add", src=src, offsets=off, dst=b); step()
+        hip.mem_fill(c.sub(0, nb // 2), 0.0); step()
+        hip.dispatch("scatter_add", src=src, offsets=off, dst=c); step()
+        return [a, b, c, src, off]
+
+    a, b, c = (v.view(np.float32) for v in both_ways(hip, body)[:3])
+
+    def scattered(start):
+        out = start.copy()
+        for i in range(n):
+            if off0[i] < nb:
+                out[off0[i]] = np.float32(out[off0[i]] + src0[i])
+        return out
+
+    half = np.full(nb, 9, np.float32)
+    half[:nb // 2] = 0
+    np.testing.assert_array_equal(a, scattered(np.zeros(nb, np.float32)))
+    np.testing.assert_array_equal(b, scattered(np.full(nb, 0.5, np.float32)))
+    np.testing.assert_array_equal(c, scattered(half))
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 10), (3000, 16), (2708, 7)])
+def test_a_bias_gradient_takes_over_the_zero_fill_of_zero_grad(hip, rows, cols):
+    """zero_grad(), then the backward pass: the bias gradient's column sums (src/ndtensor.zig:780-796) are written
+    instead of added to zeros, in the one-launch and in the two-launch form; the fills of other gradients keep waiting
+    and are seen by whoever reads them."""
+    from zigrad_amd import host
+    r = np.random.default_rng(rows)
+    g0 = r.standard_normal((rows, cols)).astype(np.float32)
+
+    def body(step):
+        g = hip.from_numpy(g0.ravel())
+        gb, gb2, other = (hip.from_numpy(np.full(cols, 5, np.float32)) for _ in range(3))
+        hip.mem_fill(other, 0.0); step()
+        hip.mem_fill(gb, 0.0); step()
+        host.unbroadcast_(hip, g, [rows, cols], gb, [cols], alpha=1.0, beta=1.0); step()
+        hip.mem_fill(gb2, 0.5); step()                                   # not zero: added to
+        host.unbroadcast_(hip, g, [rows, cols], gb2, [cols], alpha=1.0, beta=1.0); step()
+        hip.dispatch("add", x=gb, y=other, z=other); step()
+        return [gb, gb2, other, g]
+
+    gb, gb2, other = (v.view(np.float32) for v in both_ways(hip, body)[:3])
+    np.testing.assert_allclose(gb, g0.sum(axis=0, dtype=np.float64), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gb2, 0.5 + g0.sum(axis=0, dtype=np.float64), rtol=1e-5, atol=1e-5)
+    np.testing.assert_array_equal(other, gb)
+
+
+def test_a_fill_that_waits_past_a_product_is_seen_by_the_bias_row_and_the_mask_it_takes_later(hip):
+    """Fills that meet none of a product's operands keep waiting while the product waits for its bias add or its mask;
+    when that call names memory such a fill covers, the fill goes out first."""
+    from zigrad_amd import host
+    r = np.random.default_rng(9)
+    B, I, O = 16, 32, 8
+    x0 = r.standard_normal((B, I)).astype(np.float32)
+    w0 = r.standard_normal((O, I)).astype(np.float32)
+    g0 = r.standard_normal((B, O)).astype(np.float32)
+
+    def body(step):
+        x, w, g = hip.from_numpy(x0.ravel()), hip.from_numpy(w0.ravel()), hip.from_numpy(g0.ravel())
+        bias, mask = hip.from_numpy(np.full(O, 3, np.float32)), hip.from_numpy(np.full(B * I, -1, np.float32))
+        y, gx = hip.from_numpy(np.full(B * O, 7, np.float32)), hip.from_numpy(np.full(B * I, 7, np.float32))
+        hip.mem_fill(bias, 0.5); step()                                   # waits past the product below
+        hip.mem_fill(y, 0.0); step()
+        host.bmm_acc_(hip, x, [B, I], w, [O, I], y, False, True, 1.0, 1.0); step()    # y = x w^T, waits for its bias
+        hip.dispatch("add", x=bias, y=y, z=y); step()
+        hip.mem_fill(mask, 1.0); step()                                   # waits past the product below
+        hip.mem_fill(gx, 0.0); step()
+        host.bmm_acc_(hip, g, [B, O], w, [O, I], gx, False, False, 1.0, 1.0); step()  # gx = g w, waits for its mask
+        hip.dispatch("relu_inplace_bwd", x=mask, x_g=gx); step()
+        return [y, gx, x, w, g, bias, mask]
+
+    y, gx = (v.view(np.float32) for v in both_ways(hip, body)[:2])
+    np.testing.assert_allclose(y.reshape(B, O), x0 @ w0.T + 0.5, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gx.reshape(B, I), g0 @ w0, rtol=1e-5, atol=1e-5)   # the mask is all ones: nothing zeroed

@@ -32,6 +32,7 @@ class _Run:
         self.graph = (n_nodes, n_edge)
         self.src = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
         self.tgt = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
+        self.offs = hip.from_numpy(init.integers(0, 300, 1000).astype(np.uint64))   # scatter_add: one-launch and planned
         self.reads = []
         self.t = 0
         self.last_c = None
@@ -125,6 +126,11 @@ class _Run:
             self.hip.mem_copy(g, g_temp)
             self.done()
             g = g_temp
+        if self.r.random() < 0.5:          # zero_grad() before the backward pass: the fills wait for the ops that add
+            for t in (gw, gb, self.pick(int(self.r.choice([16, 640])))):
+                if self.r.random() < 0.8:
+                    self.hip.mem_fill(t, 0.0)
+                    self.done()
         host.unbroadcast_(self.hip, g, [B, O], gb, [O], alpha=1.0, beta=1.0)
         self.done()
         gx = self.hip.mem_cache_alloc(F32, B * I)
@@ -147,6 +153,14 @@ class _Run:
     def op_unbroadcast(self):
         R, inner = int(self.r.choice([2, 16, 64])), int(self.r.choice([2, 10, 64]))
         x, y = self.picks(R * inner, inner)
+        how = self.r.random()
+        if how < 0.4:
+            self.hip.mem_fill(y, 0.0)
+        elif how < 0.5:
+            self.hip.mem_fill(y.sub(0, inner // 2), 0.0)
+        elif how < 0.6:
+            self.hip.mem_fill(y, 0.25)
+        self.done()
         host.unbroadcast_(self.hip, x, [R, inner], y, [inner], alpha=1.0, beta=1.0)
 
     def op_step(self):
@@ -201,6 +215,41 @@ class _Run:
                 self.hip.mem_fill(self.pick(16), 0.5)     # something else first: the degree gradient is computed after all
                 self.done()
             self.hip.mem_cache_free(gd_temp)
+
+    def op_scatter_add(self):
+        """GatherBwd: a zero fill of the gradient, then the scatter into it (small and planned forms), sometimes with
+        another fill or a fill of only part of the destination before it."""
+        n = int(self.r.choice([64, 200, 1000]))
+        nb = int(self.r.choice([150, 300]))                     # some offsets past the end: skipped
+        src, dst = self.picks(n, nb)
+        how = self.r.random()
+        if how < 0.5:
+            self.hip.mem_fill(dst, 0.0)
+        elif how < 0.65:
+            self.hip.mem_fill(dst.sub(0, nb // 2), 0.0)
+        elif how < 0.75:
+            self.hip.mem_fill(dst, 0.25)
+        self.done()
+        if self.r.random() < 0.3:
+            self.hip.mem_fill(self.pick(16), 0.5)
+            self.done()
+        self.hip.dispatch("scatter_add", src=src, offsets=self.offs.sub(0, n), dst=dst)
+
+    def op_max_along(self):
+        rows, cols = int(self.r.choice([8, 64])), int(self.r.choice([2, 7, 33]))
+        x, y = self.picks(rows * cols, rows)
+        how = self.r.random()
+        if how < 0.5:
+            self.hip.mem_fill(y, 0.0)                           # NDArray.max_along zero-fills its output
+        elif how < 0.65:
+            self.hip.mem_fill(y.sub(0, rows // 2), 0.5)
+        elif how < 0.75:
+            room = [b for b in self.bufs + self.temps if b.ptr <= y.ptr < b.ptr + 4 * b.n][0]
+            off = (y.ptr - room.ptr) // 4
+            if off + rows + 4 <= room.n:
+                self.hip.mem_fill(room.sub(off, rows + 4), 0.75)  # sticks out of the output: must be seen
+        self.done()
+        self.hip.dispatch("max_along", x=x, x_shape=[rows, cols], y=y, y_shape=[rows], dim=1)
 
     def op_loss(self):
         rows, cols = int(self.r.choice([8, 64])), int(self.r.choice([7, 10]))
@@ -283,6 +332,11 @@ class _Run:
                     x = room.sub(off, n)
             if x.ptr != z.ptr and x.ptr < z.ptr + 4 * n and z.ptr < x.ptr + 4 * n:
                 continue                                  # an op that reads a shifted view of its own output races with itself
+            if self.r.random() < 0.3:                     # ensure_grad(0), or any other fill, right before the op
+                f = self.r.random()
+                target = z if f < 0.7 else (z.sub(0, n // 2) if n > 1 and f < 0.85 else x)
+                self.hip.mem_fill(target, float(self.r.choice([0.0, 0.0, 0.25, -0.0])))
+                self.done()
             kind = int(self.r.integers(0, 8))
             if kind == 0:
                 self.hip.dispatch(str(self.r.choice(["add", "sub", "mul"])), x=x, y=y, z=z)
@@ -320,8 +374,9 @@ class _Run:
         self.last_c = None
         ops = [self.op_fill, self.op_matmul, self.op_add_row, self.op_relu, self.op_relu_mask, self.op_layer_backward,
                self.op_unbroadcast, self.op_step, self.op_scatter, self.op_alloc, self.op_free, self.op_read, self.op_copy,
-               self.op_elementwise, self.op_scatter_bwd, self.op_loss, self.op_map_run]
-        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1, 3], float)
+               self.op_elementwise, self.op_scatter_bwd, self.op_loss, self.op_map_run, self.op_scatter_add,
+               self.op_max_along]
+        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1, 3, 1, 1], float)
         for _ in range(n_ops):
             ops[int(self.r.choice(len(ops), p=weights / weights.sum()))]()
             self.done()
@@ -339,7 +394,7 @@ class _Run:
         self.free_temps()
         for m, v in self.moments:
             out += [self.hip.to_numpy(m).view(np.uint32).copy(), self.hip.to_numpy(v).view(np.uint32).copy()]
-        for b in self.bufs + [self.src, self.tgt] + [x for mv in self.moments for x in mv]:
+        for b in self.bufs + [self.src, self.tgt, self.offs] + [x for mv in self.moments for x in mv]:
             self.hip.mem_free(b)
         return out, self.reads
 

@@ -72,6 +72,8 @@ struct zg_waiting_bias {
     const float* gy = nullptr;  // [R, inner]
     float* gb = nullptr;        // [inner]
     size_t R = 0, inner = 0;
+    bool fresh = false;         // gb's zero fill was taken over: the sums are written (a sum of floats that starts from
+                                // +0.0 is never -0.0, so s and s + 0.0 are the same bits)
 };
 
 // The aggregation of a graph-convolution layer (scatter_gcn_deg_scaled) whose plan is ready and whose apply kernel has
@@ -125,6 +127,8 @@ struct zg_map_op {
     int code;           // which functor (elementwise.hip)
     int nin;            // array operands read: a, then b, then c
     int scalar;         // 0: every operand has one element per output; 1: b is one float; 2: a is one float
+    int subst;          // bit 0 / 1 / 2: operand a / b / c is the output itself, over which a fill was still waiting when
+    float subst_value;  // the op was asked for: the op takes the fill's value instead of loading, and the fill is dropped
     float* out;
     const float* a;
     const float* b;
@@ -267,15 +271,24 @@ inline bool gemm_group_waiting(const zg_hip_ctx* ctx) {
 // Whether [lo, hi) meets an operand of the waiting products or of the waiting bias gradient.
 bool gemm_group_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
 // The single-chunk column sum y += column sums of x[R, inner] (reduce.hip), the launch the waiting bias gradient owes.
-int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner);
+int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner, bool fresh);
 // Launches the waiting graph-convolution aggregation with what was attached to it (index.hip); the two hooks are for
 // zg_hip_add and zg_hip_relu_fwd, like deferred_take_add / deferred_take_relu below.
 int flush_scatter(zg_hip_ctx* ctx);
 // Launches the waiting degree gradient (index.hip).
 int flush_graddeg(zg_hip_ctx* ctx);
-// Launches the waiting elementwise ops as one kernel (elementwise.hip); flush_pending_but_maps: everything else.
+// Launches the waiting elementwise ops as one kernel (elementwise.hip); flush_pending_but_maps: everything else;
+// flush_pending_but_maps_and_fills: everything but the two (no waiting fill ever meets an operand of a waiting
+// elementwise op, so the two kinds may leave in either order).
 int flush_maps(zg_hip_ctx* ctx);
 int flush_pending_but_maps(zg_hip_ctx* ctx);
+int flush_pending_but_maps_and_fills(zg_hip_ctx* ctx);
+// Whether a waiting fill meets one of the byte ranges; take_fill_exact: a waiting fill of exactly x[0 .. n) is dropped
+// and its value handed over (the caller overwrites all of the range and uses the value where it would have read it);
+// drop_fills_inside: waiting fills that lie wholly inside a range the caller overwrites without reading it.
+bool fills_touch(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count);
+bool take_fill_exact(zg_hip_ctx* ctx, const float* x, size_t n, float* value);
+void drop_fills_inside(zg_hip_ctx* ctx, const void* lo, size_t bytes);
 bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);
 bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc);
 // Launches the optimizer steps that are waiting (optim.hip).  Gradients whose zero fill was taken over are zeroed by
@@ -377,13 +390,14 @@ inline bool aligned16(const void* p) {
     if ((ctx)->maps.count) {                                     \
         if (int _rc_mp = zg::flush_maps(ctx)) return _rc_mp;     \
     }
-// The small elementwise ops: everything else that waits goes out, the waiting elementwise ops stay (the call joins
-// them or sends them out itself).
+// The small elementwise ops: the waiting elementwise ops stay (the call joins them or sends them out itself) and so do
+// the waiting fills (the call sends them out if one meets its operands, or takes over the one that covers its output);
+// everything else that waits goes out.
 #define ZG_CTX_KEEP_MAPS(ctx)                                    \
     ZG_REQUIRE((ctx) != nullptr, "null context");                \
-    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
-        (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active) { \
-        if (int _rc_km = zg::flush_pending_but_maps(ctx)) return _rc_km; \
+    if ((ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || (ctx)->scatter_wait.active || \
+        (ctx)->graddeg_wait.active) {                            \
+        if (int _rc_km = zg::flush_pending_but_maps_and_fills(ctx)) return _rc_km; \
     }
 // The cache's allocations and frees look at each kind of waiting work themselves: a block that is handed out is free,
 // so nothing that waits names it; a block that is given back may be the one a waiting degree gradient would write, or

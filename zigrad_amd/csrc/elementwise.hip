@@ -77,6 +77,19 @@ static int map_grid(zg_hip_ctx* ctx, size_t items, int per_block) {
 template <class Op> constexpr int chain_code() { return -1; }
 static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* out, const float* a, const float* b,
                        const float* c, size_t n, float p0, float p1, int* rc);
+// An elementwise op that takes its own launch: the waiting elementwise ops go out first, and the waiting fills too when
+// one of them meets an operand (lengths in floats; null operands are skipped).
+static int settle_before_launch(zg_hip_ctx* ctx, const float* out, size_t n_out, const float* a, size_t n_a,
+                                const float* b, size_t n_b, const float* c, size_t n_c) {
+    if (ctx->maps.count)
+        if (int rc = flush_maps(ctx)) return rc;
+    if (ctx->n_pending_fills) {
+        const void* ptrs[4] = {out, a, b, c};
+        const size_t bytes[4] = {n_out * sizeof(float), n_a * sizeof(float), n_b * sizeof(float), n_c * sizeof(float)};
+        if (fills_touch(ctx, ptrs, bytes, 4)) return flush_fills(ctx);
+    }
+    return ZG_HIP_OK;
+}
 
 template <class Op, int NIN>
 static int launch_map(zg_hip_ctx* ctx, float* out, const float* a, const float* b, const float* c, size_t n,
@@ -86,8 +99,7 @@ static int launch_map(zg_hip_ctx* ctx, float* out, const float* a, const float* 
         int rc = ZG_HIP_OK;
         if (chain_code<Op>() >= 0 && chain_push(ctx, chain_code<Op>(), NIN, 0, out, a, b, c, n, p0, p1, &rc)) return rc;
         if (rc) return rc;
-        if (ctx->maps.count)
-            if ((rc = flush_maps(ctx))) return rc;
+        if ((rc = settle_before_launch(ctx, out, n, a, n, NIN > 1 ? b : nullptr, n, NIN > 2 ? c : nullptr, n))) return rc;
     }
     bool vec = aligned16(out) && aligned16(a) && (NIN < 2 || aligned16(b)) && (NIN < 3 || aligned16(c)) && n >= 4;
     if (vec) {
@@ -217,8 +229,7 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
             if (chain_push(ctx, chain_code<Bin2<B>>(), 2, xl == 1 ? 2 : 1, z, x, y, nullptr, zl, 0.f, 0.f, &rc)) return rc;
             if (rc) return rc;
         }
-        if (ctx->maps.count)
-            if (int rc = flush_maps(ctx)) return rc;
+        if (int rc = settle_before_launch(ctx, z, zl, x, xl, y, yl, nullptr, 0)) return rc;
         int grid = map_grid(ctx, (zl + 3) / 4, kBlock);
         if (xl == 1)
             hipLaunchKernelGGL((bin_scalar_kernel<B, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, y, x, zl);
@@ -227,8 +238,7 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    if (ctx->maps.count)
-        if (int rc = flush_maps(ctx)) return rc;
+    if (int rc = settle_before_launch(ctx, z, zl, x, xl, y, yl, nullptr, 0)) return rc;
     const bool short_lhs = xl < yl;
     const float* lng = short_lhs ? y : x;
     const float* sht = short_lhs ? x : y;
@@ -329,9 +339,9 @@ __global__ __launch_bounds__(kBlock) void map_chain_kernel(MapChainArgs g) {
     if (i >= g.n) return;
     for (int k = 0; k < g.count; k++) {
         const zg_map_op& o = g.op[k];
-        const float a = o.a[o.scalar == 2 ? 0 : i];
-        const float b = o.nin > 1 ? o.b[o.scalar == 1 ? 0 : i] : 0.f;
-        const float c = o.nin > 2 ? o.c[i] : 0.f;
+        const float a = (o.subst & 1) ? o.subst_value : o.a[o.scalar == 2 ? 0 : i];
+        const float b = o.nin > 1 ? ((o.subst & 2) ? o.subst_value : o.b[o.scalar == 1 ? 0 : i]) : 0.f;
+        const float c = o.nin > 2 ? ((o.subst & 4) ? o.subst_value : o.c[i]) : 0.f;
         float r = 0.f;
         switch (o.code) {
 #define ZG_CHAIN_CASE(N, OP) case N: r = OP::f(a, b, c, o.p0, o.p1); break;
@@ -383,12 +393,33 @@ static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* ou
                        const float* c, size_t n, float p0, float p1, int* rc) {
     *rc = ZG_HIP_OK;
     if (code < 0 || n == 0 || n > kWaitingMapMaxLen) return false;
-    zg_map_op o{code, nin, scalar, out, a, b, c, p0, p1};
+    zg_map_op o{code, nin, scalar, 0, 0.f, out, a, b, c, p0, p1};
     MapRange mine[4];
-    const int n_mine = map_op_ranges(o, n, mine);
+    int n_mine = map_op_ranges(o, n, mine);
     // the op's own operands: in place is fine, a shifted overlap is not (its own kernel would race too: let it)
     for (int j = 1; j < n_mine; j++)
         if (map_ranges_conflict(mine[0], mine[j])) return false;
+    // From here on the op is queued.  A fill of exactly its output that is still waiting has no other reader: the op
+    // overwrites all of it, and where the output is also an operand (x_g += ..., in place) it takes the fill's value
+    // instead of loading it (ensure_grad(0) followed by an accumulating backward, src/ndtensor.zig:221-228).  Other
+    // fills that meet an operand go out first; the rest keep waiting.
+    if (ctx->n_pending_fills) {
+        float value = 0.f;
+        if (take_fill_exact(ctx, out, n, &value)) {
+            o.subst_value = value;
+            if (scalar != 2 && a == out) o.subst |= 1;
+            if (nin > 1 && scalar != 1 && b == out) o.subst |= 2;
+            if (nin > 2 && c == out) o.subst |= 4;
+        }
+        const void* ptrs[4];
+        size_t bytes[4];
+        for (int j = 0; j < n_mine; j++) {
+            ptrs[j] = mine[j].lo;
+            bytes[j] = (size_t)(mine[j].hi - mine[j].lo);
+        }
+        if (fills_touch(ctx, ptrs, bytes, n_mine))
+            if ((*rc = flush_fills(ctx))) return false;
+    }
     zg_waiting_maps& q = ctx->maps;
     bool joins = q.count > 0 && q.count < kMaxWaitingMaps && q.n == n;
     for (int k = 0; k < q.count && joins; k++) {

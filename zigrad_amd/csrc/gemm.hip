@@ -757,6 +757,7 @@ struct LinearBwdArgs {
     unsigned n_w, n_x;  // workgroups of the two products (n_x = 0: no input gradient)
     const float* gy;    // [R, inner]
     float* gb;          // null: no bias gradient
+    float gb_beta;      // 1: gb += sums; 0: gb = sums (its zero fill was taken over)
     size_t R, inner;
     int log2_cx;
 };
@@ -768,7 +769,7 @@ __global__ __launch_bounds__(kGemmThreads) void linear_bwd_small_kernel(LinearBw
     if (b < a.n_w) gemm_tiny_block<false, false>(a.gw, b, 0, 0, part);
     else if (b < a.n_w + a.n_x) gemm_tiny_block<true, false>(a.gx, b - a.n_w, 0, 0, part);
     else
-        col_reduce_block<AxisSum, V>(a.gy, a.gb, nullptr, a.R, a.inner, a.log2_cx, a.R, 1.f, 1.f, b - a.n_w - a.n_x, 0, 0,
+        col_reduce_block<AxisSum, V>(a.gy, a.gb, nullptr, a.R, a.inner, a.log2_cx, a.R, 1.f, a.gb_beta, b - a.n_w - a.n_x, 0, 0,
                                      1, &part[0][0][0]);
 }
 
@@ -1119,8 +1120,8 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
 // leading dimension ldx), gx = gy w masked by act_in (w with leading dimension ldw; gx null: none), gb += column sums of
 // gy (gb null: none).  The caller has checked that each job is one the kernel's blocks take.
 static int launch_linear_bwd_small(zg_hip_ctx* ctx, const float* gy, const float* x, size_t ldx, const float* w, size_t ldw,
-                                   const float* act_in, float* gw, float gw_beta, float* gb, float* gx, size_t batch,
-                                   size_t fan_in, size_t fan_out) {
+                                   const float* act_in, float* gw, float gw_beta, float* gb, float gb_beta, float* gx,
+                                   size_t batch, size_t fan_in, size_t fan_out) {
     LinearBwdArgs a;
     a.gw = gemm_args(gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, ldx, fan_in, 1.f, gw_beta, 1, 1, 0, 0, 0, nullptr);
     a.n_w = a.gw.tiles_m * a.gw.tiles_n;
@@ -1135,6 +1136,7 @@ static int launch_linear_bwd_small(zg_hip_ctx* ctx, const float* gy, const float
     const ColReduceShape cs = col_reduce_shape(gy, fan_out);
     a.gy = gy;
     a.gb = gb;
+    a.gb_beta = gb_beta;
     a.R = batch;
     a.inner = fan_out;
     a.log2_cx = cs.log2_cx;
@@ -1559,9 +1561,9 @@ int flush_deferred_gemm(zg_hip_ctx* ctx) {
     if (w.active) {
         rc = launch_linear_bwd_small(ctx, w.A, w.B, w.ldb, d.active ? d.B : nullptr, d.active ? d.ldb : 0,
                                      d.active ? d.gate : nullptr, w.C, w.zeroed ? 0.f : 1.f, b.active ? b.gb : nullptr,
-                                     d.active ? d.C : nullptr, w.k, w.n, w.m);
+                                     b.active && b.fresh ? 0.f : 1.f, d.active ? d.C : nullptr, w.k, w.n, w.m);
     } else {
-        if (b.active) rc = launch_bias_col_sum(ctx, b.gy, b.gb, b.R, b.inner);
+        if (b.active) rc = launch_bias_col_sum(ctx, b.gy, b.gb, b.R, b.inner, b.fresh);
         if (!rc && d.active) {
             GemmExtras ex{d.bias, d.gate, d.relu};
             const bool any = d.bias || d.gate || d.relu;
@@ -1572,9 +1574,19 @@ int flush_deferred_gemm(zg_hip_ctx* ctx) {
     if (rc) {  // a product failed: the zeros its output was owed are still owed
         if (d.active && d.zeroed) (void)zg_hip_mem_fill(ctx, d.C, d.m * d.n, 0.f);
         if (w.active && w.zeroed) (void)zg_hip_mem_fill(ctx, w.C, w.m * w.n, 0.f);
+        if (b.active && b.fresh) (void)zg_hip_mem_fill(ctx, b.gb, b.inner, 0.f);
     }
     run_deferred_frees(ctx);  // blocks that hold operands and were given back while the work waited
     return rc;
+}
+
+// An operand that joins waiting work after the fact (a bias row, a mask): the waiting fills meet none of the operands the
+// work already has, but one may meet this one; then the fills go out first.  False: they could not be launched.
+static bool fills_clear_of(zg_hip_ctx* ctx, const float* p, size_t n) {
+    const void* ptrs[1] = {p};
+    const size_t bytes[1] = {n * sizeof(float)};
+    if (!ctx->n_pending_fills || !fills_touch(ctx, ptrs, bytes, 1)) return true;
+    return flush_fills(ctx) == ZG_HIP_OK;
 }
 
 // bias.add_(y): z = x + y over the product's output, one operand the output itself, the other a row of n values
@@ -1586,6 +1598,7 @@ bool deferred_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* 
     else if (x == d.C && xl == zl && yl == d.n) row = y;
     if (!row) return false;
     if (ranges_meet(operand_range(row, 1, d.n, d.n), operand_range(d.C, d.m, d.n, d.ldc))) return false;
+    if (!fills_clear_of(ctx, row, d.n)) return false;
     d.bias = row;
     return true;
 }
@@ -1611,6 +1624,7 @@ bool deferred_take_relu_mask(zg_hip_ctx* ctx, const float* x, const float* x_g, 
     if (ctx->bias_wait.active &&
         ranges_meet(xr, operand_range(ctx->bias_wait.gb, 1, ctx->bias_wait.inner, ctx->bias_wait.inner)))
         return false;
+    if (!fills_clear_of(ctx, x, n)) return false;
     d.gate = x;
     *rc = flush_deferred_gemm(ctx);
     return true;
@@ -1627,7 +1641,21 @@ static int gemm_entry(zg_hip_ctx* ctx, const char* name, const float* A, const f
     const bool zeroed = beta == 1.f && C && ldc == n && k > 0 && alpha != 0.f && m > 0 && n > 0 && batches > 0 &&
                         absorb_zero_fill(ctx, C, batches * m * n);
     const float beta_eff = zeroed ? 0.f : beta;
-    if (int rc = flush_fills(ctx)) return rc;
+    // the other waiting fills go out if one meets an operand; the rest stay (the zero_grad() fills of the layers whose
+    // backward pass comes later, each taken over by the op that accumulates into it)
+    if (ctx->n_pending_fills) {
+        bool touched = !plain;
+        if (plain) {
+            const ByteRange rs[3] = {operand_range(A, trans_a ? k : m, trans_a ? m : k, lda),
+                                     operand_range(B, trans_b ? n : k, trans_b ? k : n, ldb), operand_range(C, m, n, ldc)};
+            const void* ptrs[3] = {rs[0].lo, rs[1].lo, rs[2].lo};
+            const size_t bytes[3] = {(size_t)(rs[0].hi - rs[0].lo), (size_t)(rs[1].hi - rs[1].lo),
+                                     (size_t)(rs[2].hi - rs[2].lo)};
+            touched = fills_touch(ctx, ptrs, bytes, 3);
+        }
+        if (touched)
+            if (int rc = flush_fills(ctx)) return rc;
+    }
     if (ctx->steps.count)
         if (int rc = flush_steps(ctx)) return rc;
     auto launch_now = [&]() {
@@ -1802,7 +1830,7 @@ ZG_API int zg_hip_linear_bwd(zg_hip_ctx* ctx, const float* gy, const float* x, c
         return gemm_dispatch(ctx, "linear_bwd", gy, x, gw, fan_out, fan_in, batch, 1, 0, fan_out, fan_in, fan_in, 1.f, 1.f,
                              1, 1, 1, 0, 0, 0);
     }
-    return launch_linear_bwd_small(ctx, gy, x, fan_in, w, fan_in, act_in, gw, 1.f, gb, gx, batch, fan_in, fan_out);
+    return launch_linear_bwd_small(ctx, gy, x, fan_in, w, fan_in, act_in, gw, 1.f, gb, 1.f, gx, batch, fan_in, fan_out);
 }
 
 ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_shape, const float* B,

@@ -608,20 +608,25 @@ static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Pla
 // The whole of scatter_add for at most kScatterSmallMax entries in one launch of one workgroup: thread i owns entry i,
 // and the first entry of each destination walks the later entries in input order, so the additions happen in the
 // order of the host loop.  Offsets at or beyond `nb` are skipped, as the bucket path skips them.
+// With `fresh` the destination's zero fill was taken over: the workgroup zeroes all of dst first and the sums start
+// from +0.0 instead of what dst held (at most kScatterSmallFreshMax destinations).
 constexpr int kScatterSmallMax = 256;
+constexpr size_t kScatterSmallFreshMax = 16384;
 __global__ __launch_bounds__(kScatterSmallMax) void scatter_add_small_kernel(const float* src, const uint64_t* offsets,
-                                                                             int n, float* dst, size_t nb) {
+                                                                             int n, float* dst, size_t nb, bool fresh) {
     __shared__ uint64_t s_off[kScatterSmallMax];
     __shared__ float s_src[kScatterSmallMax];
     const int i = threadIdx.x;
     // slots past n hold an offset no destination has, so the walk below can run in whole groups of eight
     s_off[i] = (i < n) ? offsets[i] : ~0ull;
     s_src[i] = (i < n) ? src[i] : 0.f;
-    __syncthreads();
+    if (fresh)
+        for (size_t e = i; e < nb; e += kScatterSmallMax) dst[e] = 0.f;
+    __syncthreads();  // also orders the zeros before the sums stored below (one workgroup, global memory)
     if (i >= n) return;
     const uint64_t k = s_off[i];
     if (k >= nb) return;
-    float acc = dst[k];
+    float acc = fresh ? 0.f : dst[k];
     bool first = true;
     const int n8 = (n + 7) & ~7;
     for (int j0 = 0; j0 < n8; j0 += 8) {
@@ -1021,27 +1026,47 @@ ZG_API int zg_hip_gather(zg_hip_ctx* ctx, const float* src, const uint64_t* src_
 
 ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t* offsets, size_t n, float* dst,
                               size_t dst_len) {
-    ZG_CTX(ctx);
-    if (n == 0) return ZG_HIP_OK;
-    ZG_REQUIRE(src && offsets && dst, "scatter_add: null pointer");
-    ZG_REQUIRE(dst_len > 0, "scatter_add: empty destination");
-    ZG_REQUIRE(n < 0xffffffffull && dst_len < 0xffffffffull, "scatter_add: sizes beyond 2^32-1");
-    if (n <= (size_t)kScatterSmallMax) {
+    ZG_CTX_KEEP_ALL(ctx);
+    const bool args_ok = n == 0 || (src && offsets && dst && dst_len > 0 && n < 0xffffffffull && dst_len < 0xffffffffull);
+    if (n == 0 || !args_ok) {
+        if (int rc = flush_pending(ctx)) return rc;
+        if (n == 0) return ZG_HIP_OK;
+        ZG_REQUIRE(src && offsets && dst, "scatter_add: null pointer");
+        ZG_REQUIRE(dst_len > 0, "scatter_add: empty destination");
+        ZG_REQUIRE(false, "scatter_add: sizes beyond 2^32-1");
+    }
+    // A zero fill of exactly dst that still waits is taken over: the sums are written, untouched elements get their
+    // zero from the same launch (GatherBwd fills the gradient, then scatters into it: src/ndtensor.zig:1367-1380).
+    // The other waiting fills stay unless they meet an operand.
+    const bool small = n <= (size_t)kScatterSmallMax;
+    const char *s0 = (const char*)src, *s1 = s0 + n * sizeof(float), *d0 = (const char*)dst, *d1 = d0 + dst_len * sizeof(float);
+    const bool fresh = !(s0 < d1 && d0 < s1) && (!small || dst_len <= kScatterSmallFreshMax) &&
+                       absorb_zero_fill(ctx, dst, dst_len);
+    auto owed = [&](int rc_in) {  // refused after the fill was taken over: the zeros are still owed
+        if (fresh) (void)zg_hip_mem_fill(ctx, dst, dst_len, 0.f);
+        return rc_in;
+    };
+    {
+        const void* ptrs[3] = {src, offsets, dst};
+        const size_t bytes[3] = {n * sizeof(float), n * sizeof(uint64_t), dst_len * sizeof(float)};
+        if (int rc = flush_pending_but_fills(ctx, ptrs, bytes, 3)) return owed(rc);
+    }
+    if (small) {
         hipLaunchKernelGGL(scatter_add_small_kernel, dim3(1), dim3(kScatterSmallMax), 0, ctx->stream, src, offsets, (int)n,
-                           dst, dst_len);
+                           dst, dst_len, fresh);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
     PlanRef pr;
     int rc = 0;
     if (!plan_from_cache(ctx, offsets, nullptr, n, dst_len, &pr, &rc)) {
-        if (rc) return rc;
+        if (rc) return owed(rc);
         void* mem = workspace(ctx, plan_bytes(n, dst_len));
-        if (!mem) return ZG_HIP_EOOM;
+        if (!mem) return owed(ZG_HIP_EOOM);
         pr.plan = carve_plan(mem, n, dst_len);
-        if ((rc = build_plan(ctx, offsets, pr.plan))) return rc;
+        if ((rc = build_plan(ctx, offsets, pr.plan))) return owed(rc);
     }
-    return launch_scatter_add_apply(ctx, src, pr.plan, dst, false);
+    return launch_scatter_add_apply(ctx, src, pr.plan, dst, fresh);
 }
 
 ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src_len, const uint64_t* indices,

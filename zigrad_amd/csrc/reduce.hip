@@ -269,8 +269,8 @@ static int sum_along_impl(zg_hip_ctx* ctx, const float* x, const uint64_t* x_sha
     return axis_reduce<AxisSum>(ctx, x, y, outer, R, inner, alpha, beta);
 }
 
-int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner) {
-    return axis_reduce<AxisSum>(ctx, x, y, 1, R, inner, 1.f, 1.f);
+int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner, bool fresh) {
+    return axis_reduce<AxisSum>(ctx, x, y, 1, R, inner, 1.f, fresh ? 0.f : 1.f);
 }
 
 }  // namespace zg
@@ -397,11 +397,32 @@ ZG_API int zg_hip_sum_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_s
 
 ZG_API int zg_hip_max_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, float* y,
                             size_t y_len, size_t dim) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_ALL(ctx);
     int rc = check_axis_args("max_along", x, x_shape, x_rank, y, y_len, dim);
-    if (rc) return rc;
+    if (rc == ZG_HIP_OK && y_len != prod(x_shape, 0, x_rank) / x_shape[dim]) {
+        set_error("max_along: y.len %zu != %zu", y_len, prod(x_shape, 0, x_rank) / (size_t)x_shape[dim]);
+        rc = ZG_HIP_EINVAL;
+    }
+    if (rc) {  // refused: what waits is launched as by any other call
+        (void)flush_pending(ctx);
+        return rc;
+    }
     const size_t outer = prod(x_shape, 0, dim), R = x_shape[dim], inner = prod(x_shape, dim + 1, x_rank);
-    ZG_REQUIRE(y_len == outer * inner, "max_along: y.len %zu != %zu", y_len, outer * inner);
+    {
+        // every element of y is written and none is read: a fill inside y that still waits has no reader left
+        // (NDArray.max_along zero-fills its output first, src/ndarray.zig:567); the other waiting fills stay unless
+        // they meet x or y
+        const char *x0 = (const char*)x, *x1 = x0 + outer * R * inner * sizeof(float);
+        const char *y0 = (const char*)y, *y1 = y0 + y_len * sizeof(float);
+        if (x0 < y1 && y0 < x1) {
+            if ((rc = flush_pending(ctx))) return rc;
+        } else {
+            drop_fills_inside(ctx, y, y_len * sizeof(float));
+            const void* ptrs[2] = {x, y};
+            const size_t bytes[2] = {(size_t)(x1 - x0), (size_t)(y1 - y0)};
+            if ((rc = flush_pending_but_fills(ctx, ptrs, bytes, 2))) return rc;
+        }
+    }
     return axis_reduce<AxisMax>(ctx, x, y, outer, R, inner, 1.f, 0.f);
 }
 
@@ -453,7 +474,13 @@ __global__ __launch_bounds__(kBlock) void scaled_copy_kernel(const float* x, flo
 ZG_API int zg_hip_unbroadcast(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape_in, size_t x_rank_in, float* y,
                               const uint64_t* y_shape_in, size_t y_rank_in, float* scratch, size_t scratch_len,
                               float alpha, float beta) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_ALL(ctx);
+    // what waits goes out before this call's first launch (below); a refused call sends it out too
+    struct Settle {
+        zg_hip_ctx* ctx;
+        bool done = false;
+        ~Settle() { if (!done) (void)flush_pending(ctx); }
+    } settle{ctx};
     ZG_REQUIRE(x && y && x_shape_in && y_shape_in, "unbroadcast: null pointer");
     ZG_REQUIRE(x_rank_in >= 1 && x_rank_in <= 8 && y_rank_in >= 1 && y_rank_in <= 8, "unbroadcast: rank not in 1..8");
     ZG_REQUIRE(x_rank_in >= y_rank_in, "unbroadcast: x rank %zu < y rank %zu", x_rank_in, y_rank_in);
@@ -462,6 +489,8 @@ ZG_API int zg_hip_unbroadcast(zg_hip_ctx* ctx, const float* x, const uint64_t* x
                y_len);
     ZG_REQUIRE(x != y, "unbroadcast: input and output alias");
     if (x_len == y_len) {
+        settle.done = true;
+        if (int rc = flush_pending(ctx)) return rc;
         hipLaunchKernelGGL(scaled_copy_kernel, dim3(stream_grid(ctx, x_len, 4)), dim3(kBlock), 0, ctx->stream, x, y,
                            x_len, alpha, beta);
         ZG_LAUNCH_CHECK();
@@ -488,21 +517,38 @@ ZG_API int zg_hip_unbroadcast(zg_hip_ctx* ctx, const float* x, const uint64_t* x
         if (ones == 0) ZG_REQUIRE(col <= y_len, "unbroadcast: fold writes %zu elements into y of %zu", col, y_len);
         else ZG_REQUIRE(scratch && col <= scratch_len, "unbroadcast: scratch of %zu floats needed, %zu given", col, scratch_len);
     }
+    settle.done = true;
+    if (xr > yr && ones == 0 && alpha == 1.f && beta == 1.f && (x + x_len <= y || y + y_len <= x)) {
+        // y += column sums of x, a bias gradient (src/ndtensor.zig:780-796).  A zero fill of exactly y that still
+        // waits (zero_grad() before the backward pass) is taken over: the sums are written.  The other waiting fills
+        // stay unless they meet x or y; everything else that waits goes out.
+        const size_t dif = xr - yr;
+        const size_t row = prod(xs, 0, dif), col = prod(xs, dif, xr);
+        const bool fresh = absorb_zero_fill(ctx, y, col);
+        const void* ptrs[2] = {x, y};
+        const size_t bytes[2] = {x_len * sizeof(float), col * sizeof(float)};
+        int rc = flush_pending_but_fills(ctx, ptrs, bytes, 2);
+        if (rc == ZG_HIP_OK) {
+            if (row > 1 && col > 1 && row * col <= kColSingleChunkMax) {
+                // one launch of the column kernel: it waits for the layer's two products, which can share its launch
+                zg_waiting_bias& b = ctx->bias_wait;
+                b.active = true;
+                b.gy = x;
+                b.gb = y;
+                b.R = row;
+                b.inner = col;
+                b.fresh = fresh;
+                return ZG_HIP_OK;
+            }
+            rc = axis_reduce<AxisSum>(ctx, x, y, 1, row, col, 1.f, fresh ? 0.f : 1.f);
+        }
+        if (rc && fresh) (void)zg_hip_mem_fill(ctx, y, col, 0.f);  // refused: the zeros are still owed
+        return rc;
+    }
+    if (int rc = flush_pending(ctx)) return rc;
     if (xr > yr) {
         const size_t dif = xr - yr;
         const size_t row = prod(xs, 0, dif), col = prod(xs, dif, xr);
-        if (ones == 0 && alpha == 1.f && beta == 1.f && row > 1 && col > 1 && row * col <= kColSingleChunkMax &&
-            (x + row * col <= y || y + col <= x)) {
-            // y += column sums of x in one launch of the column kernel: a small layer's bias gradient
-            // (src/ndtensor.zig:780-796).  It waits for the layer's two products, which can share its launch.
-            zg_waiting_bias& b = ctx->bias_wait;
-            b.active = true;
-            b.gy = x;
-            b.gb = y;
-            b.R = row;
-            b.inner = col;
-            return ZG_HIP_OK;
-        }
         int rc = axis_reduce<AxisSum>(ctx, x, ones == 0 ? y : scratch, 1, row, col, alpha, beta);
         if (rc) return rc;
         if (ones == 0) return ZG_HIP_OK;

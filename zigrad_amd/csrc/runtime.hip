@@ -1069,9 +1069,21 @@ ZG_API int zg_hip_memcpy_d2h(zg_hip_ctx* ctx, void* dst_host, const void* src, s
 }
 
 ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t bytes) {
-    ZG_CTX(ctx);
-    if (bytes == 0) return ZG_HIP_OK;
-    ZG_REQUIRE(dst && src, "memcpy_d2d: null pointer");
+    ZG_CTX_KEEP_ALL(ctx);
+    if (bytes == 0 || !dst || !src) {
+        if (int rc = flush_pending(ctx)) return rc;
+        if (bytes == 0) return ZG_HIP_OK;
+        ZG_REQUIRE(dst && src, "memcpy_d2d: null pointer");
+    }
+    {
+        // waiting fills that meet neither range stay; one that lies inside a destination the copy overwrites without
+        // reading it has no reader left
+        const char *s0 = (const char*)src, *d0 = (const char*)dst;
+        if (s0 + bytes <= d0 || d0 + bytes <= s0) drop_fills_inside(ctx, dst, bytes);
+        const void* ptrs[2] = {src, dst};
+        const size_t lens[2] = {bytes, bytes};
+        if (int rc = flush_pending_but_fills(ctx, ptrs, lens, 2)) return rc;
+    }
     if (ctx->capturing) {
         // recorded as a kernel node like everything else in the graph
         const bool v16 = aligned16(dst) && aligned16(src) && bytes % 16 == 0;
@@ -1153,6 +1165,49 @@ int flush_pending_but_maps(zg_hip_ctx* ctx) {
     if (int rc = flush_fills(ctx)) return rc;
     return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
 }
+int flush_pending_but_maps_and_fills(zg_hip_ctx* ctx) {
+    if (ctx->scatter_wait.active)
+        if (int rc = flush_scatter(ctx)) return rc;
+    if (ctx->graddeg_wait.active)
+        if (int rc = flush_graddeg(ctx)) return rc;
+    if (gemm_group_waiting(ctx))
+        if (int rc = flush_deferred_gemm(ctx)) return rc;
+    return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
+}
+
+bool fills_touch(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
+    for (int i = 0; i < ctx->n_pending_fills; i++) {
+        const char* x0 = (const char*)ctx->pending_fills[i].x;
+        const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
+        for (int j = 0; j < count; j++) {
+            const char* p0 = (const char*)ptrs[j];
+            if (p0 && x0 < p0 + bytes[j] && p0 < x1) return true;
+        }
+    }
+    return false;
+}
+bool take_fill_exact(zg_hip_ctx* ctx, const float* x, size_t n, float* value) {
+    for (int i = 0; i < ctx->n_pending_fills; i++) {
+        const zg_pending_fill& p = ctx->pending_fills[i];
+        if (p.x == x && p.n == n) {
+            *value = p.value;
+            for (int j = i + 1; j < ctx->n_pending_fills; j++) ctx->pending_fills[j - 1] = ctx->pending_fills[j];
+            ctx->n_pending_fills--;
+            return true;
+        }
+    }
+    return false;
+}
+void drop_fills_inside(zg_hip_ctx* ctx, const void* lo_, size_t bytes) {
+    const char *lo = (const char*)lo_, *hi = lo + bytes;
+    int kept = 0;
+    for (int i = 0; i < ctx->n_pending_fills; i++) {
+        const char* x0 = (const char*)ctx->pending_fills[i].x;
+        const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
+        if (!(lo <= x0 && x1 <= hi)) ctx->pending_fills[kept++] = ctx->pending_fills[i];
+    }
+    ctx->n_pending_fills = kept;
+}
 
 int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
     if (ctx->maps.count)
@@ -1165,15 +1220,7 @@ int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size
         if (int rc = flush_deferred_gemm(ctx)) return rc;
     if (ctx->steps.count)
         if (int rc = flush_steps(ctx)) return rc;
-    for (int i = 0; i < ctx->n_pending_fills; i++) {
-        const char* x0 = (const char*)ctx->pending_fills[i].x;
-        const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
-        for (int j = 0; j < count; j++) {
-            const char* p0 = (const char*)ptrs[j];
-            if (p0 && x0 < p0 + bytes[j] && p0 < x1) return flush_fills(ctx);
-        }
-    }
-    return ZG_HIP_OK;
+    return fills_touch(ctx, ptrs, bytes, count) ? flush_fills(ctx) : ZG_HIP_OK;
 }
 
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {

@@ -48,6 +48,10 @@ SHAPES = [
     # nothing a multiple of anything: odd m, n, k and (with the padding rule below) odd leading dimensions, so pieces
     # of 16 bytes straddle the edges of the operands, C takes scalar stores and the last k-tiles are masked
     (1023, 1021, 1019), (515, 259, 1031), (258, 1026, 2050), (1025, 3, 1025), (5, 1027, 513),
+    # tall with at most 16 columns and a k of 512 to 2048
+    (512, 16, 512), (600, 1, 2048), (4096, 10, 1000), (513, 15, 577), (1000, 16, 2049), (511, 16, 600), (700, 17, 600),
+    # at most 16 rows, wide, over a long k
+    (16, 256, 512), (7, 1433, 2708), (1, 300, 5000), (16, 257, 32768), (15, 1000, 513), (16, 255, 600), (17, 300, 600),
 ]
 
 
@@ -186,7 +190,8 @@ def test_bmm_acc_split_k_batches(oracle, hip):
     assert rel_fro(res[1], res[0]) <= TOL
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 784), (40, 40, 16384), (33, 31, 16392), (500, 500, 300), (16, 1433, 2708)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 784), (40, 40, 16384), (33, 31, 16392), (500, 500, 300), (16, 1433, 2708),
+                                   (2708, 16, 1433), (1000, 7, 600)])
 def test_small_products_with_a_long_k_repeat_bit_for_bit(hip, m, n, k):
     """A small C with a long k is cut into ranges of k over several workgroups per tile of C, and the partial tiles
     are added in range order by a second kernel: repeated launches give the same bits, and the values match float64

@@ -477,6 +477,58 @@ def run_c_harness(dims, batch, steps, fused=False):
     return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": what}
 
 
+def run_c_dqn(dims, batch, steps):
+    """The DQN update issued op by op from plain C (examples/c_caller/dqn_step.c).  None when the binary has not been
+    built."""
+    import subprocess
+    import tempfile
+
+    from zigrad_amd.build import C_DQN_BIN
+    from zigrad_amd.trainers import dqn_inputs, mlp_inputs
+
+    if not C_DQN_BIN.exists():
+        return None
+    params, _, _, _ = mlp_inputs(dims, batch)
+    b = dqn_inputs(batch=batch)
+    with tempfile.NamedTemporaryFile(suffix=".bin") as f:
+        for a in (*params, b["states"], b["next_states"], b["rewards"], b["dones"]):
+            f.write(np.ascontiguousarray(a, np.float32).tobytes())
+        f.write(np.ascontiguousarray(b["actions"], np.uint64).tobytes())
+        f.flush()
+        run = subprocess.run([str(C_DQN_BIN), f.name, str(steps), str(batch), *map(str, dims)], capture_output=True, text=True,
+                             timeout=300)
+    if run.returncode != 0:
+        raise RuntimeError("examples/c_caller/dqn_step failed: " + run.stderr)
+    us = float(run.stdout.strip().splitlines()[-1].split()[1])
+    return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": "eager, same op sequence, caller in C"}
+
+
+def run_c_gcn(steps):
+    """The GCN step issued op by op from plain C (examples/c_caller/gcn_step.c).  None when the binary has not been
+    built."""
+    import subprocess
+    import tempfile
+
+    from zigrad_amd.build import C_GCN_BIN
+    from zigrad_amd.trainers import gcn_inputs
+
+    if not C_GCN_BIN.exists():
+        return None
+    inp = gcn_inputs(seed=0)
+    with tempfile.NamedTemporaryFile(suffix=".bin") as f:
+        for a in (*inp["params"], inp["x"], inp["onehot"][: inp["n_train"]]):
+            f.write(np.ascontiguousarray(a, np.float32).tobytes())
+        f.write(np.ascontiguousarray(inp["src"], np.uint64).tobytes())
+        f.write(np.ascontiguousarray(inp["tgt"], np.uint64).tobytes())
+        f.flush()
+        argv = [inp["x"].shape[0], *inp["dims"], inp["src"].size, inp["n_train"]]
+        run = subprocess.run([str(C_GCN_BIN), f.name, str(steps), *map(str, argv)], capture_output=True, text=True, timeout=300)
+    if run.returncode != 0:
+        raise RuntimeError("examples/c_caller/gcn_step failed: " + run.stderr)
+    us = float(run.stdout.strip().splitlines()[-1].split()[1])
+    return {"steps_per_s": 1e6 / us, "ms_per_step": us / 1e3, "workload": "eager, same op sequence, caller in C"}
+
+
 def cpu_baseline(dims, batch, budget_steps=2, threads=None, loss_mode="onehot"):
     """The oracle on the host cores: the same step sequence, BLAS threads = the box's CPU share (or `threads`)."""
     from oracle.oracle_device import OracleDevice
@@ -704,7 +756,9 @@ def main():
             result["mlp_b64"]["fused"]["c_caller"] = run_c_harness([784, 128, 64, 10], 64, 2000, fused=True)
         result["input_pipeline"] = run_input_pipeline(dev, WIDE_DIMS, WIDE_BATCH, max(5, args.steps // 2), 2)
         result["gcn"] = run_small(dev, "gcn", 100, graph=not args.no_graph)
+        result["gcn"]["c_caller"] = run_c_gcn(1000)
         result["dqn"] = run_small(dev, "dqn", 200, graph=not args.no_graph)
+        result["dqn"]["c_caller"] = run_c_dqn([4, 128, 128, 2], 64, 2000)
         if not args.no_graph:
             for kind, n in (("gcn", 100), ("dqn", 200)):
                 f = run_small(dev, kind, n, graph=True, fused=True)

@@ -80,16 +80,21 @@ def build(force: bool = False, jobs: int | None = None) -> Path:
 
 C_HARNESS_SRC = PKG_DIR.parent / "examples" / "c_caller" / "mlp_step.c"
 C_HARNESS_BIN = C_HARNESS_SRC.with_suffix("")
+C_DQN_SRC = PKG_DIR.parent / "examples" / "c_caller" / "dqn_step.c"
+C_DQN_BIN = C_DQN_SRC.with_suffix("")
+C_GCN_SRC = PKG_DIR.parent / "examples" / "c_caller" / "gcn_step.c"
+C_GCN_BIN = C_GCN_SRC.with_suffix("")
 
 
 def build_c_harness() -> Path:
-    """The plain-C caller of the C ABI (examples/c_caller/mlp_step.c), linked against the library in its tree."""
-    cmd = ["gcc", "-std=c11", "-O2", "-Wall", "-Werror", "-D_POSIX_C_SOURCE=199309L", f"-I{PKG_DIR.parent / 'include'}",
-           str(C_HARNESS_SRC), "-o", str(C_HARNESS_BIN), f"-L{PKG_DIR}", "-lzg_hip", "-Wl,-rpath,$ORIGIN/../../zigrad_amd"]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("gcc failed for examples/c_caller/mlp_step.c")
+    """The plain-C callers of the C ABI (examples/c_caller/*.c), linked against the library in its tree."""
+    for src, out in ((C_HARNESS_SRC, C_HARNESS_BIN), (C_DQN_SRC, C_DQN_BIN), (C_GCN_SRC, C_GCN_BIN)):
+        cmd = ["gcc", "-std=c11", "-O2", "-Wall", "-Werror", "-D_POSIX_C_SOURCE=199309L", f"-I{PKG_DIR.parent / 'include'}",
+               str(src), "-o", str(out), f"-L{PKG_DIR}", "-lzg_hip", "-Wl,-rpath,$ORIGIN/../../zigrad_amd"]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            sys.stderr.write(res.stdout + res.stderr)
+            raise RuntimeError(f"gcc failed for {src}")
     return C_HARNESS_BIN
 
 

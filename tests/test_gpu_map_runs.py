@@ -344,3 +344,31 @@ def test_a_fill_that_waits_past_a_product_is_seen_by_the_bias_row_and_the_mask_i
     y, gx = (v.view(np.float32) for v in both_ways(hip, body)[:2])
     np.testing.assert_allclose(y.reshape(B, O), x0 @ w0.T + 0.5, rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(gx.reshape(B, I), g0 @ w0, rtol=1e-5, atol=1e-5)   # the mask is all ones: nothing zeroed
+
+
+@pytest.mark.parametrize("n,nb", [(100, 40), (3000, 500)])
+def test_scatter_add_of_a_source_whose_fill_waits(hip, n, nb):
+    """Counting with a buffer of ones (the GCN's degrees, examples/gcn/src/model.zig:116-224): the source's fill need
+    not be launched for the scatter, but whoever reads the source afterwards finds it filled."""
+    r = np.random.default_rng(n)
+    off0 = r.integers(0, nb, n).astype(np.uint64)
+
+    def body(step):
+        off = hip.from_numpy(off0)
+        ones, counts, deg = hip.from_numpy(np.full(n, 9, np.float32)), hip.from_numpy(np.full(nb, 9, np.float32)), hip.mem_alloc(F32, nb)
+        later = hip.mem_alloc(F32, n)
+        hip.mem_fill(deg, 1.0); step()
+        hip.mem_fill(ones, 1.0); step()
+        hip.mem_fill(counts, 0.0); step()
+        hip.dispatch("scatter_add", src=ones, offsets=off, dst=counts); step()
+        hip.dispatch("add", x=counts, y=deg, z=deg); step()
+        hip.dispatch("rsqrt_fwd", x=deg, y=deg, eps=1e-12); step()
+        hip.dispatch("scale", x=ones, alpha=3.0); step()                # reads the source after all
+        hip.mem_copy(ones, later); step()
+        return [deg, counts, later, ones, off]
+
+    deg, counts, later = (v.view(np.float32) for v in both_ways(hip, body)[:3])
+    want = np.bincount(off0.astype(np.int64), minlength=nb).astype(np.float32)
+    np.testing.assert_array_equal(counts, want)
+    np.testing.assert_allclose(deg, 1 / np.sqrt(1 + want.astype(np.float64)), rtol=1e-6)
+    np.testing.assert_array_equal(later, np.full(n, 3, np.float32))

@@ -233,6 +233,9 @@ class _Run:
         if self.r.random() < 0.3:
             self.hip.mem_fill(self.pick(16), 0.5)
             self.done()
+        if self.r.random() < 0.3:                                # a buffer of ones scattered to count (the GCN's degrees)
+            self.hip.mem_fill(src if self.r.random() < 0.7 else src.sub(0, n // 2), 1.0)
+            self.done()
         self.hip.dispatch("scatter_add", src=src, offsets=self.offs.sub(0, n), dst=dst)
 
     def op_max_along(self):

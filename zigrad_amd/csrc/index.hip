@@ -543,8 +543,9 @@ int plan_uses_validate(zg_hip_ctx* ctx, const std::vector<PlanUse>& uses) {
 
 // dst[b] += src[e] for the bucket's entries in input order; one thread per destination
 // `fresh`: dst is write-only (treated as zero on entry), so the caller needs no zero fill
+// src null: every contribution is `src_const` (a source whose fill with one value is still waiting is not read)
 __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_ptr, const uint32_t* perm, float* dst,
-                                         size_t nb, bool fresh) {
+                                         size_t nb, bool fresh, float src_const) {
     size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nb) return;
     const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
@@ -561,7 +562,7 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
 #pragma unroll
         for (int u = 0; u < 8; u++) pv[u] = (k + u < e) ? perm[k + u] : 0u;
 #pragma unroll
-        for (int u = 0; u < 8; u++) sv[u] = (k + u < e) ? src[pv[u]] : 0.f;
+        for (int u = 0; u < 8; u++) sv[u] = (k + u < e) ? (src ? src[pv[u]] : src_const) : 0.f;
 #pragma unroll
         for (int u = 0; u < 8; u++)
             if (k + u < e) acc = __fadd_rn(acc, sv[u]);
@@ -573,7 +574,7 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
 // on the running sum), then adds them one after the other in input order, every lane forming the same sum.
 __global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float* src, const uint32_t* row_ptr,
                                                                       const uint32_t* perm, const uint32_t* long_list,
-                                                                      float* dst, bool fresh) {
+                                                                      float* dst, bool fresh, float src_const) {
     const int lane = threadIdx.x & 63;
     const uint32_t n_long = long_list[0];
     const uint32_t wave0 = blockIdx.x * 4 + (threadIdx.x >> 6), n_waves = gridDim.x * 4;
@@ -583,7 +584,7 @@ __global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float
         float acc = fresh ? 0.f : dst[b];
         for (uint32_t k0 = s; k0 < e; k0 += 64) {
             const uint32_t k = k0 + lane;
-            const float v = (k < e) ? src[perm[k]] : 0.f;
+            const float v = (k < e) ? (src ? src[perm[k]] : src_const) : 0.f;
             const int cnt = (e - k0 < 64u) ? (int)(e - k0) : 64;
             for (int j = 0; j < cnt; j++) acc = __fadd_rn(acc, __shfl(v, j, 64));
         }
@@ -591,15 +592,16 @@ __global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float
     }
 }
 
-static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Plan& pl, float* dst, bool fresh) {
+static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Plan& pl, float* dst, bool fresh,
+                                    float src_const = 0.f) {
     hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(pl.nb, 256)), dim3(256), 0, ctx->stream, src,
-                       pl.row_ptr, pl.perm, dst, pl.nb, fresh);
+                       pl.row_ptr, pl.perm, dst, pl.nb, fresh, src_const);
     ZG_LAUNCH_CHECK();
     if (pl.n > kLongBucket && pl.n_long != 0) {
         size_t grid = ceil_div_sz(pl.n / kLongBucket, 4);
         if (grid > 2048) grid = 2048;
         hipLaunchKernelGGL(scatter_add_apply_long_kernel, dim3((unsigned)grid), dim3(256), 0, ctx->stream, src, pl.row_ptr,
-                           pl.perm, pl.long_list, dst, fresh);
+                           pl.perm, pl.long_list, dst, fresh, src_const);
         ZG_LAUNCH_CHECK();
     }
     return ZG_HIP_OK;
@@ -613,13 +615,14 @@ static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Pla
 constexpr int kScatterSmallMax = 256;
 constexpr size_t kScatterSmallFreshMax = 16384;
 __global__ __launch_bounds__(kScatterSmallMax) void scatter_add_small_kernel(const float* src, const uint64_t* offsets,
-                                                                             int n, float* dst, size_t nb, bool fresh) {
+                                                                             int n, float* dst, size_t nb, bool fresh,
+                                                                             float src_const) {
     __shared__ uint64_t s_off[kScatterSmallMax];
     __shared__ float s_src[kScatterSmallMax];
     const int i = threadIdx.x;
     // slots past n hold an offset no destination has, so the walk below can run in whole groups of eight
     s_off[i] = (i < n) ? offsets[i] : ~0ull;
-    s_src[i] = (i < n) ? src[i] : 0.f;
+    s_src[i] = (i < n) ? (src ? src[i] : src_const) : 0.f;  // src null: every contribution is src_const
     if (fresh)
         for (size_t e = i; e < nb; e += kScatterSmallMax) dst[e] = 0.f;
     __syncthreads();  // also orders the zeros before the sums stored below (one workgroup, global memory)
@@ -1040,20 +1043,32 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
     // The other waiting fills stay unless they meet an operand.
     const bool small = n <= (size_t)kScatterSmallMax;
     const char *s0 = (const char*)src, *s1 = s0 + n * sizeof(float), *d0 = (const char*)dst, *d1 = d0 + dst_len * sizeof(float);
-    const bool fresh = !(s0 < d1 && d0 < s1) && (!small || dst_len <= kScatterSmallFreshMax) &&
-                       absorb_zero_fill(ctx, dst, dst_len);
+    const bool apart = !(s0 < d1 && d0 < s1);
+    const bool fresh = apart && (!small || dst_len <= kScatterSmallFreshMax) && absorb_zero_fill(ctx, dst, dst_len);
+    // A source that is exactly a fill still waiting (a buffer of ones scattered to count edges, examples/gcn/src/
+    // model.zig:116-224) is not read: its value is the contribution.  The fill stays queued for whoever reads the
+    // buffer next; a caller that frees it right away never pays for it.
+    float src_const = 0.f;
+    bool const_src = false;
+    if (apart)
+        for (int i = 0; i < ctx->n_pending_fills && !const_src; i++)
+            if (ctx->pending_fills[i].x == src && ctx->pending_fills[i].n == n) {
+                const_src = true;
+                src_const = ctx->pending_fills[i].value;
+            }
     auto owed = [&](int rc_in) {  // refused after the fill was taken over: the zeros are still owed
         if (fresh) (void)zg_hip_mem_fill(ctx, dst, dst_len, 0.f);
         return rc_in;
     };
     {
-        const void* ptrs[3] = {src, offsets, dst};
+        const void* ptrs[3] = {const_src ? nullptr : src, offsets, dst};
         const size_t bytes[3] = {n * sizeof(float), n * sizeof(uint64_t), dst_len * sizeof(float)};
         if (int rc = flush_pending_but_fills(ctx, ptrs, bytes, 3)) return owed(rc);
     }
+    const float* src_read = const_src ? nullptr : src;
     if (small) {
-        hipLaunchKernelGGL(scatter_add_small_kernel, dim3(1), dim3(kScatterSmallMax), 0, ctx->stream, src, offsets, (int)n,
-                           dst, dst_len, fresh);
+        hipLaunchKernelGGL(scatter_add_small_kernel, dim3(1), dim3(kScatterSmallMax), 0, ctx->stream, src_read, offsets,
+                           (int)n, dst, dst_len, fresh, src_const);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
@@ -1066,7 +1081,7 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
         pr.plan = carve_plan(mem, n, dst_len);
         if ((rc = build_plan(ctx, offsets, pr.plan))) return owed(rc);
     }
-    return launch_scatter_add_apply(ctx, src, pr.plan, dst, fresh);
+    return launch_scatter_add_apply(ctx, src_read, pr.plan, dst, fresh, src_const);
 }
 
 ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src_len, const uint64_t* indices,

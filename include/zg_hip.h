@@ -115,7 +115,9 @@ int zg_hip_memcpy_h2d(zg_hip_ctx *ctx, void *dst, const void *src_host, size_t b
 /* .DtoH, blocking.  Up to 4096 bytes (NDTensor.get of a scalar, src/ndtensor.zig:524-528) travel through pinned memory of
  * the context: a copy kernel on the stream, the wait for the stream, a host copy. */
 int zg_hip_memcpy_d2h(zg_hip_ctx *ctx, void *dst_host, const void *src, size_t bytes);
-int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes);      /* mem_copy / .DtoD */
+/* mem_copy / .DtoD.  A waiting float fill of at most 2^20 elements that covers the destination and more, and is clear of
+ * the source, leaves in the copy's launch (a gradient zero-filled, then rows copied into it). */
+int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes);
 /* mem_fill (src/device/host_device.zig:876-884).  The fill is queued inside the context and launched together with
  * any other waiting fills (up to 16, one kernel) at the start of the next call on this context that is not a float fill
  * or a cache allocation: callers zero gradients tensor by tensor (examples/mnist/src/model.zig:57-62) and one launch per

@@ -372,3 +372,25 @@ def test_scatter_add_of_a_source_whose_fill_waits(hip, n, nb):
     np.testing.assert_array_equal(counts, want)
     np.testing.assert_allclose(deg, 1 / np.sqrt(1 + want.astype(np.float64)), rtol=1e-6)
     np.testing.assert_array_equal(later, np.full(n, 3, np.float32))
+
+
+@pytest.mark.parametrize("total,off,n", [(18956, 0, 980), (5000, 1234, 77), (300, 299, 1), (4096, 0, 4096)])
+def test_rows_copied_into_a_gradient_whose_zero_fill_waits(hip, total, off, n):
+    """MaskLayer.backward (examples/gcn/src/model.zig:343-348): the full gradient is zero-filled, then the labelled rows
+    are copied into it; fill and copy leave in one launch, and a fill that waits elsewhere is left alone."""
+    r = np.random.default_rng(total)
+    rows0 = r.standard_normal(n).astype(np.float32)
+
+    def body(step):
+        rows, full, other = hip.from_numpy(rows0), hip.from_numpy(np.full(total, 9, np.float32)), hip.mem_alloc(F32, 64)
+        hip.mem_fill(other, 2.0); step()
+        hip.mem_fill(full, 0.0); step()
+        hip.mem_copy(rows, full.sub(off, n)); step()
+        hip.dispatch("scale", x=full, alpha=2.0); step()
+        return [full, other, rows]
+
+    full, other = (v.view(np.float32) for v in both_ways(hip, body)[:2])
+    want = np.zeros(total, np.float32)
+    want[off:off + n] = rows0
+    np.testing.assert_array_equal(full, want * 2)
+    np.testing.assert_array_equal(other, np.full(64, 2, np.float32))

@@ -287,6 +287,13 @@ class _Run:
     def op_copy(self):
         n = int(self.r.choice([16, 1000, BUF_LEN]))
         a, b = self.picks(n, n)
+        if self.r.random() < 0.4:                   # MaskLayer.backward: a zero-filled gradient, then rows copied into it
+            room = [t for t in self.bufs + self.temps if t.ptr <= b.ptr < t.ptr + 4 * t.n][0]
+            lo = (b.ptr - room.ptr) // 4
+            lo0 = max(0, lo - int(self.r.integers(0, 40)))
+            hi0 = min(room.n, lo + n + int(self.r.integers(0, 40)))
+            self.hip.mem_fill(room.sub(lo0, hi0 - lo0), float(self.r.choice([0.0, 0.5])))
+            self.done()
         self.hip.mem_copy(a, b)
 
     def op_elementwise(self):

@@ -321,6 +321,14 @@ __global__ void copy_kernel(T* __restrict__ dst, const T* __restrict__ src, size
     for (; i < n; i += nt) dst[i] = src[i];
 }
 
+// A fill of x[0 .. n) with v and a copy of n_copy floats to x + off in one pass: a zero-filled gradient whose leading rows
+// are then overwritten (MaskLayer.backward, examples/gcn/src/model.zig:343-348).
+__global__ void fill_and_copy_kernel(float* __restrict__ x, size_t n, float v, size_t off, const float* __restrict__ src,
+                                     size_t n_copy) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += nt) x[i] = (i >= off && i - off < n_copy) ? src[i - off] : v;
+}
+
 template <typename T>
 __global__ void fill_kernel(T* __restrict__ x, size_t n, T v) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1080,9 +1088,37 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
         // reading it has no reader left
         const char *s0 = (const char*)src, *d0 = (const char*)dst;
         if (s0 + bytes <= d0 || d0 + bytes <= s0) drop_fills_inside(ctx, dst, bytes);
+        // a waiting float fill that covers the destination and more (a gradient zeroed, then its leading rows
+        // overwritten) and is clear of the source leaves together with the copy, in one launch
+        int host_fill = -1;
+        if (bytes % sizeof(float) == 0 && ((uintptr_t)dst | (uintptr_t)src) % sizeof(float) == 0)
+            for (int i = 0; i < ctx->n_pending_fills && host_fill < 0; i++) {
+                const char* x0 = (const char*)ctx->pending_fills[i].x;
+                const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
+                if (x0 <= d0 && d0 + bytes <= x1 && (s0 + bytes <= x0 || x1 <= s0) &&
+                    ctx->pending_fills[i].n <= ((size_t)1 << 20))  // a long fill keeps its own kernel's wide stores
+                    host_fill = i;
+            }
+        zg_pending_fill f{};
+        if (host_fill >= 0) {
+            f = ctx->pending_fills[host_fill];
+            for (int j = host_fill + 1; j < ctx->n_pending_fills; j++) ctx->pending_fills[j - 1] = ctx->pending_fills[j];
+            ctx->n_pending_fills--;
+        }
         const void* ptrs[2] = {src, dst};
         const size_t lens[2] = {bytes, bytes};
-        if (int rc = flush_pending_but_fills(ctx, ptrs, lens, 2)) return rc;
+        int rc = flush_pending_but_fills(ctx, ptrs, lens, 2);
+        if (host_fill >= 0) {
+            if (rc) {  // refused: the fill is still owed
+                (void)zg_hip_mem_fill(ctx, f.x, f.n, f.value);
+                return rc;
+            }
+            hipLaunchKernelGGL(fill_and_copy_kernel, dim3(grid_for(ctx, f.n, kBlock)), dim3(kBlock), 0, ctx->stream, f.x, f.n,
+                               f.value, (size_t)((const float*)dst - f.x), (const float*)src, bytes / sizeof(float));
+            ZG_LAUNCH_CHECK();
+            return ZG_HIP_OK;
+        }
+        if (rc) return rc;
     }
     if (ctx->capturing) {
         // recorded as a kernel node like everything else in the graph

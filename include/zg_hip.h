@@ -128,7 +128,8 @@ int zg_hip_memcpy_d2d(zg_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
  * of zg_hip_scatter_gcn_deg_scaled, a gradient of zg_hip_scatter_gcn_deg_scaled_bwd or the destination of
  * zg_hip_scatter_add is not launched at all: the op writes what it would have added to the zeros (and a source of
  * zg_hip_scatter_add that is exactly a fill still waiting is not read: the fill's value is every contribution, and the
- * fill stays queued for later readers); a waiting fill of any
+ * fill stays queued for later readers; such a count into a zeroed destination of at most 65536 elements whose offsets
+ * were seen before waits with the small elementwise ops below); a waiting fill of any
  * value over exactly the output of a small elementwise op (see below) is taken over likewise, and one inside the output
  * of zg_hip_max_along, which writes every element and reads none, is dropped; one over exactly the gradient of an optimizer
  * step that is itself still waiting (zero_grad() after step()) is stored by the step's update kernel; and a waiting

@@ -281,6 +281,10 @@ int flush_graddeg(zg_hip_ctx* ctx);
 // flush_pending_but_maps_and_fills: everything but the two (no waiting fill ever meets an operand of a waiting
 // elementwise op, so the two kinds may leave in either order).
 int flush_maps(zg_hip_ctx* ctx);
+// Queues out[i] = c added to +0.0 (row_ptr[i + 1] - row_ptr[i]) times, i < n, with the waiting elementwise ops: what
+// scatter_add of a constant source into a destination of zeros comes to once the offsets are sorted into buckets
+// (index.hip).  False: not queued (*rc says whether something failed), the caller launches its own kernel.
+bool maps_push_count(zg_hip_ctx* ctx, float* out, const uint32_t* row_ptr, size_t n, float c, int* rc);
 int flush_pending_but_maps(zg_hip_ctx* ctx);
 int flush_pending_but_maps_and_fills(zg_hip_ctx* ctx);
 // Whether a waiting fill meets one of the byte ranges; take_fill_exact: a waiting fill of exactly x[0 .. n) is dropped

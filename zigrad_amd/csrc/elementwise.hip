@@ -326,6 +326,7 @@ ZG_OP(MseBwd, return __fadd_rn(c, __fmul_rn(p0, __fsub_rn(a, b)));)
 ZG_CHAIN_OPS(ZG_CHAIN_CODE)
 #undef ZG_CHAIN_CODE
 
+constexpr int kChainCountCode = 26;  // out[i] = p0 added (a[i + 1] - a[i]) times, a an array of uint32 bucket bounds
 struct MapChainArgs {
     zg_map_op op[kMaxWaitingMaps];
     int count;
@@ -339,6 +340,14 @@ __global__ __launch_bounds__(kBlock) void map_chain_kernel(MapChainArgs g) {
     if (i >= g.n) return;
     for (int k = 0; k < g.count; k++) {
         const zg_map_op& o = g.op[k];
+        if (o.code == kChainCountCode) {
+            const uint32_t* bounds = reinterpret_cast<const uint32_t*>(o.a);
+            const uint32_t cnt = bounds[i + 1] - bounds[i];
+            float r = 0.f;
+            for (uint32_t e = 0; e < cnt; e++) r = __fadd_rn(r, o.p0);
+            o.out[i] = r;
+            continue;
+        }
         const float a = (o.subst & 1) ? o.subst_value : o.a[o.scalar == 2 ? 0 : i];
         const float b = o.nin > 1 ? ((o.subst & 2) ? o.subst_value : o.b[o.scalar == 1 ? 0 : i]) : 0.f;
         const float c = o.nin > 2 ? ((o.subst & 4) ? o.subst_value : o.c[i]) : 0.f;
@@ -383,6 +392,10 @@ static int map_op_ranges(const zg_map_op& o, size_t n, MapRange* r) {  // r[0] i
         r[m++] = MapRange{(const char*)p, (const char*)(p + (scalar ? 1 : n)), !scalar};
     };
     put(o.out, false);
+    if (o.code == kChainCountCode) {  // n + 1 bucket bounds, read by neighbouring threads: nothing in the run may write them
+        r[m++] = MapRange{(const char*)o.a, (const char*)o.a + (n + 1) * sizeof(uint32_t), false};
+        return m;
+    }
     put(o.a, o.scalar == 2);
     if (o.nin > 1) put(o.b, o.scalar == 1);
     if (o.nin > 2) put(o.c, false);
@@ -433,6 +446,11 @@ static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* ou
     if (q.count == 0) q.n = n;
     q.op[q.count++] = o;
     return true;
+}
+
+bool maps_push_count(zg_hip_ctx* ctx, float* out, const uint32_t* row_ptr, size_t n, float c, int* rc) {
+    return chain_push(ctx, kChainCountCode, 1, 0, out, reinterpret_cast<const float*>(row_ptr), nullptr, nullptr, n, c, 0.f,
+                      rc);
 }
 
 }  // namespace zg

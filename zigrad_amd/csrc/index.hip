@@ -1081,6 +1081,14 @@ ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t*
         pr.plan = carve_plan(mem, n, dst_len);
         if ((rc = build_plan(ctx, offsets, pr.plan))) return owed(rc);
     }
+    if (const_src && fresh && pr.plan.n_long == 0 && dst_len <= kWaitingMapMaxLen) {
+        // counting: every destination gets the constant added once per entry of its bucket, which needs neither the
+        // source nor the order of the entries; it waits with the small elementwise ops (the GCN adds one and takes
+        // the reciprocal square root next, examples/gcn/src/model.zig:116-224: one launch for the three)
+        int rc_push = ZG_HIP_OK;
+        if (maps_push_count(ctx, dst, pr.plan.row_ptr, dst_len, src_const, &rc_push)) return rc_push;
+        if (rc_push) return owed(rc_push);
+    }
     return launch_scatter_add_apply(ctx, src_read, pr.plan, dst, fresh, src_const);
 }
 

@@ -1186,7 +1186,8 @@ int flush_fills(zg_hip_ctx* ctx) {
     return ZG_HIP_OK;
 }
 int flush_pending(zg_hip_ctx* ctx) {
-    // at most one kind is waiting at a time, except fills next to allocations: each kind's own calls send the others first
+    // Work of different kinds that waits at the same time touches disjoint memory (each kind's calls send out whatever
+    // meets their operands before they queue), so the kinds may leave in any order.
     if (ctx->maps.count)
         if (int rc = flush_maps(ctx)) return rc;
     return flush_pending_but_maps(ctx);

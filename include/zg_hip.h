@@ -107,6 +107,10 @@ int zg_hip_clear_cache(zg_hip_ctx *ctx);
  * binding tells them apart with this range test. */
 int zg_hip_is_device_ptr(zg_hip_ctx *ctx, const void *ptr, int *yes);
 int zg_hip_cache_stats(zg_hip_ctx *ctx, size_t *bytes_in_use, size_t *bytes_mapped, uint64_t *n_device_allocs);
+/* Kernels launched by the library in this process so far, device-to-device copies included (no counterpart in the
+ * reference; for tests and for reading profiles: how many launches an op sequence costs).  Work still waiting in the
+ * context is not counted and is not sent out by this call. */
+int zg_hip_launch_count(zg_hip_ctx *ctx, uint64_t *launches);
 
 /* ---------------------------------------------------------------------------------------------
  * memory ops (src/device/host_device.zig:919-958)

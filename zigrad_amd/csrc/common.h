@@ -2,6 +2,18 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+// Every kernel launch of the library is counted (zg_hip_launch_count): the launches an op sequence costs are what the
+// work that waits inside the context is there to cut, and tests hold them to what was measured.
+namespace zg {
+extern unsigned long long launches_issued;
+}
+#undef hipLaunchKernelGGL
+#define hipLaunchKernelGGL(kernelName, numBlocks, numThreads, memPerBlock, streamId, ...)              \
+    do {                                                                                               \
+        ++zg::launches_issued;                                                                         \
+        (kernelName)<<<(numBlocks), (numThreads), (memPerBlock), (streamId)>>>(__VA_ARGS__);           \
+    } while (0)
+
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>

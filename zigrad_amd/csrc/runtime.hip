@@ -1021,6 +1021,16 @@ ZG_API int zg_hip_clear_cache(zg_hip_ctx* ctx) {
     return ZG_HIP_OK;
 }
 
+namespace zg {
+unsigned long long launches_issued = 0;
+}
+
+ZG_API int zg_hip_launch_count(zg_hip_ctx* ctx, uint64_t* launches) {
+    ZG_REQUIRE(ctx != nullptr && launches != nullptr, "launch_count: null argument");
+    *launches = launches_issued;  // nothing is sent out: what waits in the context has not been launched and is not counted
+    return ZG_HIP_OK;
+}
+
 ZG_API int zg_hip_cache_stats(zg_hip_ctx* ctx, size_t* bytes_in_use, size_t* bytes_mapped, uint64_t* n_device_allocs) {
     ZG_CTX(ctx);
     size_t u = 0, m = 0;
@@ -1133,6 +1143,7 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
+    ++launches_issued;  // the driver's copy kernel
     ZG_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, ctx->stream));
     return ZG_HIP_OK;
 }

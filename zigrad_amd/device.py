@@ -192,6 +192,13 @@ class HipDevice:
         self._call("zg_hip_cache_stats", ctypes.byref(u), ctypes.byref(m), ctypes.byref(a))
         return {"bytes_in_use": u.value, "bytes_mapped": m.value, "n_device_allocs": a.value}
 
+    def launch_count(self) -> int:
+        """Kernels the library has launched in this process so far (device-to-device copies included); work that
+        still waits in the context is not counted."""
+        n = ctypes.c_uint64()
+        self._call("zg_hip_launch_count", ctypes.byref(n))
+        return n.value
+
     def mem_fill(self, buf: DevBuf, value) -> None:
         if buf.dtype == F32:
             self._call("zg_hip_mem_fill", buf.ptr, buf.n, float(value))

@@ -440,8 +440,11 @@ def run_small(dev, kind, steps, graph=True, fused=False):
         what = "DQN update 4-128-128-2, batch 64, frozen target net, gather, smooth-L1, Adam lr 1e-3"
     for _ in range(10):
         tr.step()
+    dev.sync()
+    launches = dev.launch_count()
     dt, _ = timed_steps(dev, tr.step, steps)
-    out = {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "workload": what}
+    launches = (dev.launch_count() - launches) / steps
+    out = {"steps_per_s": steps / dt, "ms_per_step": dt / steps * 1e3, "workload": what, "launches_per_step": launches}
     if graph and hasattr(tr, "capture"):
         tr.capture()
         for _ in range(10):

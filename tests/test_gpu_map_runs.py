@@ -354,17 +354,21 @@ def test_scatter_add_of_a_source_whose_fill_waits(hip, n, nb):
     off0 = r.integers(0, nb, n).astype(np.uint64)
 
     def body(step):
-        off = hip.from_numpy(off0)
+        # the offsets in pinned host memory: from the second round on the library has their buckets, and the count
+        # waits with the add and the rsqrt that follow it
+        off = hip.mem_alloc_host(np.uint64, n)
+        hip.mem_transfer(off0, off, "HtoD")
         ones, counts, deg = hip.from_numpy(np.full(n, 9, np.float32)), hip.from_numpy(np.full(nb, 9, np.float32)), hip.mem_alloc(F32, nb)
         later = hip.mem_alloc(F32, n)
-        hip.mem_fill(deg, 1.0); step()
-        hip.mem_fill(ones, 1.0); step()
-        hip.mem_fill(counts, 0.0); step()
-        hip.dispatch("scatter_add", src=ones, offsets=off, dst=counts); step()
-        hip.dispatch("add", x=counts, y=deg, z=deg); step()
-        hip.dispatch("rsqrt_fwd", x=deg, y=deg, eps=1e-12); step()
-        hip.dispatch("scale", x=ones, alpha=3.0); step()                # reads the source after all
-        hip.mem_copy(ones, later); step()
+        for _ in range(3):
+            hip.mem_fill(deg, 1.0); step()
+            hip.mem_fill(ones, 1.0); step()
+            hip.mem_fill(counts, 0.0); step()
+            hip.dispatch("scatter_add", src=ones, offsets=off, dst=counts); step()
+            hip.dispatch("add", x=counts, y=deg, z=deg); step()
+            hip.dispatch("rsqrt_fwd", x=deg, y=deg, eps=1e-12); step()
+            hip.dispatch("scale", x=ones, alpha=3.0); step()            # reads the source after all
+            hip.mem_copy(ones, later); step()
         return [deg, counts, later, ones, off]
 
     deg, counts, later = (v.view(np.float32) for v in both_ways(hip, body)[:3])

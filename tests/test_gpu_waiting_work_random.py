@@ -32,7 +32,10 @@ class _Run:
         self.graph = (n_nodes, n_edge)
         self.src = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
         self.tgt = hip.from_numpy(init.integers(0, n_nodes, n_edge).astype(np.uint64))
-        self.offs = hip.from_numpy(init.integers(0, 300, 1000).astype(np.uint64))   # scatter_add: one-launch and planned
+        # scatter_add, one-launch and planned forms; in pinned host memory, where the library keeps the buckets it sorted
+        # the offsets into from call to call (what lets a count of a constant wait with the elementwise ops)
+        self.offs = hip.mem_alloc_host(np.uint64, 1000)
+        hip.mem_transfer(init.integers(0, 300, 1000).astype(np.uint64), self.offs, "HtoD")
         self.reads = []
         self.t = 0
         self.last_c = None
@@ -237,6 +240,12 @@ class _Run:
             self.hip.mem_fill(src if self.r.random() < 0.7 else src.sub(0, n // 2), 1.0)
             self.done()
         self.hip.dispatch("scatter_add", src=src, offsets=self.offs.sub(0, n), dst=dst)
+        if self.r.random() < 0.4:                                # deg + count, then a unary op, as the GCN's layers go on
+            self.done()
+            other = self.pick(nb)
+            self.hip.dispatch("add", x=dst, y=other, z=other)
+            self.done()
+            self.hip.dispatch("tanh_fwd", x=other, y=other)      # (rsqrt of arbitrary data would bring NaNs in)
 
     def op_max_along(self):
         rows, cols = int(self.r.choice([8, 64])), int(self.r.choice([2, 7, 33]))

@@ -797,16 +797,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, floa
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
     for (; i < M * N; i += nt) {
         float acc = p[i];
-        int s = 1;
-        for (; s + 3 < splits; s += 4) {  // four loads in flight, added in split order
-            const float v0 = p[(size_t)s * M * N + i], v1 = p[(size_t)(s + 1) * M * N + i],
-                        v2 = p[(size_t)(s + 2) * M * N + i], v3 = p[(size_t)(s + 3) * M * N + i];
-            acc += v0;
-            acc += v1;
-            acc += v2;
-            acc += v3;
+        for (int s0 = 1; s0 < splits; s0 += 8) {  // eight loads in flight, added in split order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (s0 + u < splits) v[u] = p[(size_t)(s0 + u) * M * N + i];
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (s0 + u < splits) acc += v[u];
         }
-        for (; s < splits; s++) acc += p[(size_t)s * M * N + i];
         const size_t r = i / N, col = i % N;
         float v = alpha * acc;
         if (beta != 0.f) v += beta * c[r * ldc + col];

@@ -142,6 +142,9 @@ class OracleDevice(HipDevice):
     def clear_cache(self):
         pass
 
+    def launch_count(self) -> int:
+        return 0  # nothing is launched: every op runs on the host when it is called
+
     def cache_stats(self):
         return {"bytes_in_use": 0, "bytes_mapped": 0, "n_device_allocs": self.n_allocs}
 

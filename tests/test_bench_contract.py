@@ -40,3 +40,15 @@ def test_gemm_traffic_comes_from_the_committed_counter_summary(tmp_path):
     alg = bench.gemm_bytes_per_step(bench.WIDE_DIMS, bench.WIDE_BATCH) / 8
     assert alg <= got <= 10 * alg
     assert bench.gemm_traffic_bytes_per_launch(tmp_path / "absent.txt") is None
+
+
+def test_the_cpu_legs_of_the_small_configurations_run_on_the_oracle_device():
+    """bench.py times the DQN update and the GCN step on the CPU oracle beside the GPU: the function that runs them must
+    work with a device that launches nothing."""
+    sys.path.insert(0, str(ROOT))
+    import bench
+    from oracle.oracle_device import OracleDevice
+
+    for kind in ("dqn", "gcn"):
+        out = bench.run_small(OracleDevice(), kind, 2, graph=False)
+        assert out["ms_per_step"] > 0 and "launches_per_step" not in out

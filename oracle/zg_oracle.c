@@ -691,9 +691,10 @@ void zo_mem_take(const float *src, size_t src_len, const uint64_t *idxs, size_t 
 }
 
 /* src/device/host_device.zig:931-945 defines WHAT is drawn (U[0,1), N(0,1), N(0,1)*sqrt(2/fan));
- * the stream itself comes from Zig's std.Random and is not reproducible here ("parity unpinned").
- * Generator used instead: splitmix64-seeded xoshiro256++, uniform = top 24 bits * 2^-24,
- * normal = Box-Muller on two uniforms (cosine branch), evaluated in fp32. */
+ * the stream comes from a host std.Random the caller passes, whose Ziggurat normals are not
+ * reproducible here, so the stream is this documented one: splitmix64-seeded xoshiro256++,
+ * uniform = top 24 bits * 2^-24, normal = Box-Muller on two uniforms (cosine branch) in fp32.
+ * Pinned by the generators' published known-answer vectors through an independent restatement. */
 static uint64_t rotl64(uint64_t x, int k) {
     return (x << k) | (x >> (64 - k));
 }

@@ -375,6 +375,94 @@ def check_mem_ops(dev):
     exact(dev.to_numpy(dst), [13.5, 0, 4.5, 4.5, 10.5])
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# mem_random (src/device/host_device.zig:931-945 fixes WHAT is drawn: U[0,1), N(0,1), N(0,1) * sqrt(2 / fan)).
+# The stream is the documented one: splitmix64 seeding -> xoshiro256++ -> top 24 bits -> Box-Muller (cosine branch).
+# It is written here a further time, in Python integers, and that copy is first held to the published known-answer
+# vectors of the two generators (Vigna's splitmix64.c from seed 0 and from 1234567; xoshiro256++ from state
+# {1, 2, 3, 4}, the vector of the generator's reference implementation that Zig's std.Random.Xoshiro256 test and
+# Rust's rand_xoshiro repeat), so a wrong constant, rotate or shift in every copy cannot pass.
+# ---------------------------------------------------------------------------------------------------------------
+_M64 = (1 << 64) - 1
+
+
+def _splitmix64(seed, count):
+    z, out = seed & _M64, []
+    for _ in range(count):
+        z = (z + 0x9E3779B97F4A7C15) & _M64
+        v = z
+        v = ((v ^ (v >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+        v = ((v ^ (v >> 27)) * 0x94D049BB133111EB) & _M64
+        out.append(v ^ (v >> 31))
+    return out
+
+
+def _xoshiro256pp(state, count):
+    def rotl(x, k):
+        return ((x << k) | (x >> (64 - k))) & _M64
+
+    s, out = list(state), []
+    for _ in range(count):
+        out.append((rotl((s[0] + s[3]) & _M64, 23) + s[0]) & _M64)
+        t = (s[1] << 17) & _M64
+        s[2] ^= s[0]
+        s[3] ^= s[1]
+        s[1] ^= s[2]
+        s[0] ^= s[3]
+        s[2] ^= t
+        s[3] = rotl(s[3], 45)
+    return out
+
+
+def _documented_uniforms(seed, count):
+    """float64 values of the documented stream's uniforms: every one is k * 2^-24, exact in fp32 and fp64"""
+    return np.asarray([w >> 40 for w in _xoshiro256pp(_splitmix64(seed, 4), count)], np.float64) / 16777216.0
+
+
+def check_mem_random(dev):
+    assert _splitmix64(0, 5) == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F, 0xF88BB8A8724C81EC,
+                                 0x1B39896A51A8749B]
+    assert _splitmix64(1234567, 5) == [6457827717110365317, 3203168211198807973, 9817491932198370423,
+                                       4593380528125082431, 16408922859458223821]
+    assert _xoshiro256pp([1, 2, 3, 4], 10) == [
+        41943041, 58720359, 3588806011781223, 3591011842654386, 9228616714210784205, 9973669472204895162,
+        14011001112246962877, 12406186145184390807, 15849039046786891736, 10450023813501588000]
+
+    def draw(n, kind, seed, fan=0):
+        b = dev.mem_alloc(np.float32, n)
+        dev.mem_fill(b, np.nan)
+        dev.mem_random(b, kind, seed=seed, fan=fan)
+        dev.sync()
+        out = dev.to_numpy(b).copy()
+        dev.mem_free(b)
+        return out
+
+    fan = 784
+    for seed in (0, 81761, 2**63 + 12345):
+        for n in (16, 1, 257):
+            u = _documented_uniforms(seed, 2 * n)
+            exact(draw(n, "uniform", seed), u[:n])  # one word per uniform, in order
+            # normal i takes words 2i and 2i+1: radius from 1 - u (so the logarithm never sees 0), angle from the
+            # second; cos near its zeros keeps only absolute accuracy (the fp32 angle is rounded), hence atol
+            want = np.sqrt(-2.0 * np.log(1.0 - u[0::2])) * np.cos(2.0 * np.pi * u[1::2])
+            close(draw(n, "normal", seed), want, rtol=2e-6, atol=5e-6)
+            close(draw(n, "kaiming", seed, fan), want * np.sqrt(2.0 / fan), rtol=3e-6, atol=5e-6 * np.sqrt(2.0 / fan))
+    assert not np.array_equal(draw(16, "uniform", 1), draw(16, "uniform", 2))  # the seed is used
+    # distribution (what the reference's contract fixes): moments, range and independence of neighbours on 10^6
+    # draws; every bound is five or more standard errors wide
+    n = 1_000_000
+    u = r64(draw(n, "uniform", 7))
+    assert u.min() >= 0.0 and u.max() < 1.0
+    assert abs(u.mean() - 0.5) < 5 * np.sqrt(1 / 12 / n) and abs(u.var() - 1 / 12) < 5e-4
+    assert np.all(np.abs(np.histogram(u, bins=16, range=(0, 1))[0] / n - 1 / 16) < 5 * np.sqrt(1 / 16 / n))
+    for kind, sd in (("normal", 1.0), ("kaiming", np.sqrt(2.0 / fan))):
+        z = r64(draw(n, kind, 11, fan)) / sd
+        assert abs(z.mean()) < 5 / np.sqrt(n) and abs(z.var() - 1.0) < 5 * np.sqrt(2 / n)
+        assert abs(np.mean(z ** 3)) < 5 * np.sqrt(15 / n) and abs(np.mean(z ** 4) - 3.0) < 5 * np.sqrt(96 / n)
+        assert abs(np.mean(z[:-1] * z[1:])) < 5 / np.sqrt(n)
+        assert abs(np.mean(np.abs(z) < 1.0) - 0.6826894921) < 5 * np.sqrt(0.2167 / n)
+
+
 def check_gather_offsets(dev):
     """offsets[i] = flat position in src of the index tensor's coordinate i with coordinate `dim` replaced by the
     index value (src/ndarray.zig:607-624), brute force over a rank-3 case with an index tensor smaller than src."""
@@ -602,7 +690,7 @@ def check_optimizers(dev):
 ALL_CHECKS = [
     check_binary_all_regimes, check_dot_axpy_scale_nrm2, check_matvec_outer_transpose, check_matmul_layouts,
     check_unary_forward, check_unary_backward, check_max_fwd_bwd, check_axis_reductions, check_unbroadcast,
-    check_broadcast, check_mem_ops, check_gather_offsets, check_scatter_and_select, check_csr_ops, check_gcn_scatter,
+    check_broadcast, check_mem_ops, check_mem_random, check_gather_offsets, check_scatter_and_select, check_csr_ops, check_gcn_scatter,
     check_softmax_and_smce, check_regression_losses, check_optimizers,
 ]
 
@@ -654,6 +742,7 @@ PINS = {
     "zo_broadcast": ["check_broadcast"],
     "zo_mem_fill": ["check_mem_ops"],
     "zo_mem_sequence": ["check_mem_ops"],
+    "zo_mem_random": ["check_mem_random"],
     "zo_mem_take": ["check_mem_ops", "golden:check_gather"],
     "zo_gather_offsets": ["check_gather_offsets", "golden:check_gather"],
     "zo_scatter_add": ["check_scatter_and_select"],
@@ -678,7 +767,6 @@ PINS = {
     "zo_adam_lr_t": ["check_optimizers"],
 }
 
-# declared but deliberately without a pin: the generator's stream cannot be reproduced without the reference's
-# toolchain ("parity unpinned" in the oracle's header); the zo_blas_* calls select a backend and compute nothing
-UNPINNED = {"zo_mem_random"}
+# declared but deliberately without a pin: none.  The zo_blas_* calls select a backend and compute nothing.
+UNPINNED = set()
 NOT_ARITHMETIC = {"zo_blas_name", "zo_blas_set_threads", "zo_blas_force_builtin"}

@@ -114,10 +114,9 @@ int main(int argc, char **argv) {
     float *dones = (float *)upload(f, B, sizeof(float));
     uint64_t *actions = (uint64_t *)upload(f, B, sizeof(uint64_t));
     fclose(f);
-    const float gamma_host = 0.99f, one_host = 1.0f;
-    float *gamma = (float *)device_alloc(sizeof(float)), *one = (float *)device_alloc(sizeof(float));
-    CHECK(zg_hip_memcpy_h2d(ctx, gamma, &gamma_host, sizeof(float)));
-    CHECK(zg_hip_memcpy_h2d(ctx, one, &one_host, sizeof(float)));
+    /* gamma and 1 stay on the host: scalar operands go to the device by value, as a binding passes the one-element
+     * host slice of NDArray's scalar ops (src/ndarray.zig:247-257) */
+    const float gamma = 0.99f, one = 1.0f;
 
     uint64_t t = 0; /* Adam's counter: once per parameter tensor update (src/nn/optim.zig:189) */
     struct timespec t0, t1;
@@ -137,9 +136,9 @@ int main(int argc, char **argv) {
         CHECK(zg_hip_max_along(ctx, act_t[LAYERS].ptr, q_shape, 2, max_next.ptr, B, 1));
         for (int l = 1; l <= LAYERS; l++) cache_free(act_t[l]);
         cached disc = cache_alloc(B);
-        CHECK(zg_hip_mul(ctx, max_next.ptr, B, gamma, 1, disc.ptr, B));
+        CHECK(zg_hip_mul_scalar(ctx, max_next.ptr, B, gamma, 0, disc.ptr));
         cached not_done = cache_alloc(B);
-        CHECK(zg_hip_sub(ctx, one, 1, dones, B, not_done.ptr, B));
+        CHECK(zg_hip_sub_scalar(ctx, dones, B, one, 1, not_done.ptr)); /* 1 - done: the scalar is the left operand */
         cached masked = cache_alloc(B);
         CHECK(zg_hip_mul(ctx, disc.ptr, B, not_done.ptr, B, masked.ptr, B));
         cached targets = cache_alloc(B);

@@ -86,7 +86,14 @@ int zg_hip_pool_map(zg_hip_ctx *ctx, size_t bytes, void **out);  /* one contiguo
 int zg_hip_pool_unmap(zg_hip_ctx *ctx, void *ptr);
 int zg_hip_alloc(zg_hip_ctx *ctx, size_t bytes, void **out);    /* mem_alloc: src/device/host_device.zig:890-898 */
 int zg_hip_free(zg_hip_ctx *ctx, void *ptr);                    /* mem_free:  src/device/host_device.zig:900-903 */
-int zg_hip_host_alloc(zg_hip_ctx *ctx, size_t bytes, void **out); /* pinned, device-readable host memory */
+/* Pinned host memory that the host reads and writes through the pointer and the kernels read and write in place (no
+ * counterpart in the reference, whose one device is the host): what a binding serves every `usize` allocation from,
+ * because the reference's callers fill and read index tensors with host loops over `.raw` (NDArray.gather,
+ * src/ndarray.zig:607-624; the GCN's edge lists, examples/gcn/src/model.zig:204-205).  Blocks of up to 16 MiB that are
+ * given back are kept (256 MiB at most, until zg_hip_clear_cache) and reused for requests of the same power-of-two
+ * size class, so a tensor of indices per train step costs no driver call; a reused block is handed out only after the
+ * stream has passed the point at which it was given back. */
+int zg_hip_host_alloc(zg_hip_ctx *ctx, size_t bytes, void **out);
 int zg_hip_host_free(zg_hip_ctx *ctx, void *ptr);
 
 /* The library's own caching allocator (two block pools, small <= 1 MiB and large, over segments obtained on
@@ -104,7 +111,8 @@ int zg_hip_clear_cache(zg_hip_ctx *ctx);
 /* *yes = 1 when ptr lies in memory this context handed out as device memory (cache pools, zg_hip_alloc /
  * zg_hip_pool_map regions, the scratch buffer), else 0.  The reference's callers pass host scalars and device slices
  * through the same parameters (src/ndarray.zig:251 and src/nn/optim.zig:117 against src/ndtensor.zig:1146-1150); a
- * binding tells them apart with this range test. */
+ * binding tells them apart with this range test.  A pure host-side lookup: nothing is launched and work that waits in
+ * the context keeps waiting. */
 int zg_hip_is_device_ptr(zg_hip_ctx *ctx, const void *ptr, int *yes);
 int zg_hip_cache_stats(zg_hip_ctx *ctx, size_t *bytes_in_use, size_t *bytes_mapped, uint64_t *n_device_allocs);
 /* Kernels launched by the library in this process so far, device-to-device copies included (no counterpart in the
@@ -165,6 +173,16 @@ int zg_hip_add(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_
 int zg_hip_sub(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
 int zg_hip_mul(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
 int zg_hip_div(zg_hip_ctx *ctx, const float *x, size_t xl, const float *y, size_t yl, float *z, size_t zl);
+/* The same four ops with the one-float operand passed BY VALUE: z[i] = x[i] o s, or s o x[i] when scalar_is_lhs.
+ * NDArray.add_scalar & co hand the op a scalar that lives on the caller's stack (src/ndarray.zig:247-257:
+ * `.y = &.{s}`), which HostDevice reads in place (src/device/host_device.zig:975-1019) and a kernel cannot.  By value
+ * the scalar is a kernel argument: no copy to the device, no wait, the call joins the small elementwise ops that wait
+ * (above) and can be recorded into an execution graph.  z may alias x.  A binding calls these when an operand of
+ * zg_hip_add & co has length 1 and zg_hip_is_device_ptr says it is not device memory. */
+int zg_hip_add_scalar(zg_hip_ctx *ctx, const float *x, size_t n, float s, int scalar_is_lhs, float *z);
+int zg_hip_sub_scalar(zg_hip_ctx *ctx, const float *x, size_t n, float s, int scalar_is_lhs, float *z);
+int zg_hip_mul_scalar(zg_hip_ctx *ctx, const float *x, size_t n, float s, int scalar_is_lhs, float *z);
+int zg_hip_div_scalar(zg_hip_ctx *ctx, const float *x, size_t n, float s, int scalar_is_lhs, float *z);
 
 /* ---------------------------------------------------------------------------------------------
  * linear algebra (src/device/host_device.zig:224-346)

@@ -103,6 +103,20 @@ class OracleDevice(HipDevice):
     def force_builtin_blas(self, on: bool) -> None:
         self._o.cdll.zo_blas_force_builtin(int(on))
 
+    # the by-value scalar forms: HostDevice reads the caller's one-element slice in place
+    # (src/ndarray.zig:247-257, src/device/host_device.zig:975-1019), so the oracle gets a one-element array
+    def _scalar_form(self, op, x, n, s, scalar_is_lhs, z):
+        one = np.asarray([s], np.float32)
+        fn = getattr(self._o.cdll, "zo_" + op)
+        if scalar_is_lhs:
+            return fn(one.ctypes.data, 1, x, n, z, n)
+        return fn(x, n, one.ctypes.data, 1, z, n)
+
+    def _x_zg_hip_add_scalar(self, *a): return self._scalar_form("add", *a)
+    def _x_zg_hip_sub_scalar(self, *a): return self._scalar_form("sub", *a)
+    def _x_zg_hip_mul_scalar(self, *a): return self._scalar_form("mul", *a)
+    def _x_zg_hip_div_scalar(self, *a): return self._scalar_form("div", *a)
+
     # -- memory --------------------------------------------------------------------------------
     def _new(self, dtype, n, kind):
         dtype = np.dtype(dtype)

@@ -63,6 +63,18 @@ def check_binary_all_regimes(dev):
     x2 = f32(r.standard_normal(24))
     out = run_op(dev, "div", {"x": x2, "y": x, "z": x2}, ["z"])
     exact(out["z"], x2 / x[np.arange(24) % 6])
+    # a host scalar on either side (NDArray.add_scalar: `.y = &.{s}`, src/ndarray.zig:247-257): the same IEEE operation
+    # as the one-float device operand; sizes either side of the vector path and of the small-op queue, in place too
+    for n in (1, 3, 24, 4099, 70001):
+        v = f32(r.uniform(0.5, 3.0, n) * r.choice([-1, 1], n))
+        for s in (np.float32(-1.75), np.float32(0.3)):
+            for name, fn in ops.items():
+                out = run_op(dev, name, {"x": v, "y": float(s), "z": np.full(n, np.nan, np.float32)}, ["z"])
+                exact(out["z"], fn(v, s))
+                out = run_op(dev, name, {"x": float(s), "y": v, "z": np.full(n, np.nan, np.float32)}, ["z"])
+                exact(out["z"], fn(s, v))
+        out = run_op(dev, "sub", {"x": 2.5, "y": v, "z": v}, ["z"])
+        exact(out["z"], np.float32(2.5) - v)
 
 
 # ---------------------------------------------------------------------------------------------------------------

@@ -125,3 +125,39 @@ def test_scratch_may_grow_while_a_graph_is_alive(hip):
     hip.sync()
     g.free()
     hip.mem_cache_free(x)
+
+
+def test_pinned_host_blocks_are_kept_and_reused_in_stream_order(hip):
+    """A binding serves every `usize` tensor from pinned host memory (the reference's callers fill index tensors with
+    host loops, src/ndarray.zig:607-624): a block given back is handed out again for the same size class, the next
+    owner's host writes cannot reach a kernel that was queued before the block was given back, and every take reads the
+    indices its own call was given."""
+    U64 = np.uint64
+    n, m = 3000, 50000
+    src0 = np.arange(m, dtype=np.float32) * 0.5
+    src = hip.from_numpy(src0)
+    r = np.random.default_rng(9)
+    seen, outs, wants = set(), [], []
+    for it in range(40):
+        idx = hip.mem_alloc_host(U64, n)
+        seen.add(idx.ptr)
+        want = r.integers(0, m, n).astype(U64)
+        hip.host_view(idx)[:] = want            # a host loop writes the indices
+        out = hip.mem_alloc(F32, n)
+        hip.mem_take(src, idx, out)             # queued, not waited for
+        hip.mem_free(idx)                       # given back while the kernel may still be running
+        outs.append(out)
+        wants.append(want)
+    assert len(seen) <= 2, "blocks of one size class are reused, not obtained from the driver every time"
+    for out, want in zip(outs, wants):
+        np.testing.assert_array_equal(hip.to_numpy(out), src0[want])
+        hip.mem_free(out)
+    # another size class does not get the kept block; a larger request than the block's class neither
+    a = hip.mem_alloc_host(U64, 8)
+    b = hip.mem_alloc_host(U64, n * 4)
+    assert a.ptr not in seen and b.ptr not in seen
+    hip.mem_free(a)
+    hip.mem_free(b)
+    hip.mem_free(src)
+    with pytest.raises(ZgHipError):
+        hip._call("zg_hip_host_free", 12345)    # not a pointer of this context

@@ -35,11 +35,12 @@ def test_batch_64_mlp_step(hip, fused, want):
     assert launches_per_step(hip, tr) == want
 
 
+@pytest.mark.parametrize("device_scalars", [False, True], ids=["host_scalars", "device_scalars"])
 @pytest.mark.parametrize("fused,want", [(False, 18), (True, 17)])
-def test_dqn_update(hip, fused, want):
+def test_dqn_update(hip, fused, want, device_scalars):
     dims, batch = [4, 128, 128, 2], 64
     params, _, _, _ = mlp_inputs(dims, batch)
-    tr = DQNTrainer(hip, dims, batch, lr=1e-3, gamma=0.99, clip=True, fused=fused)
+    tr = DQNTrainer(hip, dims, batch, lr=1e-3, gamma=0.99, clip=True, fused=fused, device_scalars=device_scalars)
     tr.load_params(params)
     tr.set_batch(dqn_inputs(batch=batch))
     assert launches_per_step(hip, tr) == want

@@ -61,6 +61,68 @@ def test_td_target_chain_with_allocations_and_frees_between(hip):
     np.testing.assert_array_equal(got, want)
 
 
+def test_td_target_chain_with_host_scalars_is_one_launch_and_can_be_recorded(hip):
+    """gamma and 1 as host scalars (NDArray's scalar ops pass `&.{s}`, src/ndarray.zig:247-257): they travel by value, so
+    the chain still leaves as one launch, equals the chain with one-float device operands bit for bit, and a recording
+    accepts it (a copy of the scalar to the device would not be recordable)."""
+    r = np.random.default_rng(5)
+    B = 64
+    q = r.standard_normal(B).astype(np.float32)
+    done = (r.random(B) < 0.3).astype(np.float32)
+    rew = r.standard_normal(B).astype(np.float32)
+    qd, dd, rd = hip.from_numpy(q), hip.from_numpy(done), hip.from_numpy(rew)
+    gamma_d, one_d = hip.from_numpy(np.float32([0.99])), hip.from_numpy(np.float32([1.0]))
+    disc, nd, masked, tgt = (hip.mem_alloc(F32, B) for _ in range(4))
+
+    def chain(gamma, one):
+        hip.dispatch("mul", x=qd, y=gamma, z=disc)
+        hip.dispatch("sub", x=one, y=dd, z=nd)
+        hip.dispatch("mul", x=disc, y=nd, z=masked)
+        hip.dispatch("add", x=rd, y=masked, z=tgt)
+
+    chain(gamma_d, one_d)
+    want = hip.to_numpy(tgt).copy()
+    np.testing.assert_array_equal(want, rew + (q * np.float32(0.99)) * (np.float32(1.0) - done))
+    hip.mem_fill(tgt, np.nan)
+    hip.sync()
+    before = hip.launch_count()
+    chain(0.99, 1.0)
+    hip.sync()
+    assert hip.launch_count() - before == 1
+    np.testing.assert_array_equal(hip.to_numpy(tgt), want)
+    # recorded and replayed, with eager work and a synchronisation between the replays
+    hip.graph_open()
+    chain(0.99, 1.0)
+    g = hip.graph_save()
+    for _ in range(3):
+        hip.mem_fill(tgt, np.nan)
+        hip.sync()
+        g.run()
+        np.testing.assert_array_equal(hip.to_numpy(tgt), want)
+    g.free()
+    for b in (qd, dd, rd, gamma_d, one_d, disc, nd, masked, tgt):
+        hip.mem_free(b)
+
+
+def test_host_scalar_ops_alone_and_in_runs_match_a_launch_each(hip):
+    n = 1000
+    x0 = np.linspace(-3, 3, n).astype(np.float32)
+
+    def body(step):
+        x, y = hip.from_numpy(x0), hip.mem_alloc(F32, n)
+        hip.dispatch("div", x=2.0, y=x, z=y); step()
+        hip.dispatch("add", x=y, y=-0.5, z=y); step()
+        hip.dispatch("mul", x=3.0, y=y, z=x); step()
+        hip.dispatch("sub", x=x, y=0.125, z=x); step()
+        hip.dispatch("div", x=x, y=7.0, z=x); step()
+        return [x, y]
+
+    x, y = (v.view(np.float32) for v in both_ways(hip, body))
+    want_y = np.float32(2.0) / x0 + np.float32(-0.5)
+    np.testing.assert_array_equal(y, want_y)
+    np.testing.assert_array_equal(x, (np.float32(3.0) * want_y - np.float32(0.125)) / np.float32(7.0))
+
+
 def test_in_place_ops_and_results_feeding_later_ops(hip):
     r = np.random.default_rng(1)
     n = 1000

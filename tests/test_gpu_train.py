@@ -101,3 +101,25 @@ def test_dqn_steps_match_oracle(oracle, hip):
         assert rel_fro(b2, a) <= STEP_TOL
     for a, b2 in zip(po, ph):
         assert rel_fro(b2, a) <= STEP_TOL
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_dqn_with_host_scalars_equals_dqn_with_device_scalars(hip, fused):
+    """gamma and 1 by value (NDArray's scalar ops, src/ndarray.zig:247-257) against gamma and 1 as one-element device
+    tensors (examples/dqn/src/dqn_agent.zig:173-181): the same IEEE operations, so the same bits after ten updates."""
+    from zigrad_amd.trainers import DQNTrainer, dqn_inputs
+
+    dims, batch = [4, 128, 128, 2], 64
+    params, _, _, _ = mlp_inputs(dims, batch)
+    b = dqn_inputs(batch=batch)
+    runs = []
+    for device_scalars in (False, True):
+        tr = DQNTrainer(hip, dims, batch, lr=1e-3, gamma=0.99, clip=True, fused=fused, device_scalars=device_scalars)
+        tr.load_params(params)
+        tr.set_batch(b)
+        losses = [tr.step() for _ in range(10)]
+        hip.sync()
+        runs.append((losses, [hip.to_numpy(p) for p in tr.param_buffers()]))
+    assert runs[0][0] == runs[1][0]
+    for a, b2 in zip(runs[0][1], runs[1][1]):
+        np.testing.assert_array_equal(a, b2)

@@ -81,8 +81,6 @@ pub const Options = struct {
 };
 
 ctx: *c.zg_hip_ctx,
-/// one device float that host-side scalar operands are staged through (see `dev_scalar`)
-scalar_slot: [*]f32,
 
 pub fn device_count() u32 {
     var n: c_int = 0;
@@ -99,12 +97,7 @@ pub fn init_advanced(device_number: u32, opts: Options) Self {
     check(c.zg_hip_init(@intCast(device_number), &ctx));
     if (opts.small_pool_size != null or opts.large_pool_size != null)
         check(c.zg_hip_cache_configure(ctx.?, opts.small_pool_size orelse (64 << 20), opts.large_pool_size orelse (1 << 30)));
-    var slot: ?*anyopaque = null;
-    check(c.zg_hip_alloc(ctx.?, 256, &slot));
-    return .{
-        .ctx = ctx.?,
-        .scalar_slot = @ptrCast(@alignCast(slot.?)),
-    };
+    return .{ .ctx = ctx.? };
 }
 
 pub fn deinit(self: *Self) void {
@@ -130,29 +123,35 @@ pub fn clear_cache(self: *Self) void {
 }
 
 // --------------------------------------------------------------------------------------------------
-// Host-pointer hazards.  Callers that grew up on the host device hand over host memory in three places:
-// the scalar operand of add_scalar & co (src/ndarray.zig:251), axpy's alpha (src/nn/optim.zig:117) and index
-// slices filled by host loops (examples/gcn/src/model.zig:204-205).  Index slices must be allocated with
-// `mem_alloc_indices` (pinned, device-readable); scalars are staged here.
+// Host-pointer hazards.  Callers that grew up on the host device touch host memory in three places, and none of
+// them has to change:
+//   - the scalar operand of add_scalar & co is a one-element slice on the caller's stack (src/ndarray.zig:247-257):
+//     `binary` below passes it BY VALUE (zg_hip_add_scalar ...), so nothing is copied or waited for;
+//   - axpy's alpha (src/nn/optim.zig:117) is read on the host at call time (`axpy` below);
+//   - `usize` buffers are read and written through `.raw` by host loops (NDArray.gather, src/ndarray.zig:607-624;
+//     the GCN's edge lists, examples/gcn/src/model.zig:204-205): every allocation of `usize` elements, cached or
+//     not, is pinned host memory that the kernels read in place, and every device op that writes one is followed
+//     by a wait, so the host loops see what HostDevice would show them.
 // --------------------------------------------------------------------------------------------------
 fn is_device_ptr(self: *const Self, p: *const anyopaque) bool {
     var yes: c_int = 0;
-    check(c.zg_hip_is_device_ptr(self.ctx, p, &yes)); // a range test over the pools' segments and the raw allocations
+    check(c.zg_hip_is_device_ptr(self.ctx, p, &yes)); // a host-side range test; launches nothing, flushes nothing
     return yes != 0;
 }
 
-fn dev_scalar(self: *const Self, T: type, s: []const T) [*]const T {
-    if (s.len != 1 or self.is_device_ptr(s.ptr)) return s.ptr;
-    check(c.zg_hip_memcpy_h2d(self.ctx, self.scalar_slot, s.ptr, @sizeOf(T)));
-    return @ptrCast(self.scalar_slot);
+/// DeviceData.ctx of a cached `usize` allocation: pinned host memory, not a block of the device pools.
+const host_tag: usize = std.math.maxInt(usize);
+
+fn host_alloc(self: *const Self, T: type, n: usize) ![]T {
+    var ptr: ?*anyopaque = null;
+    if (c.zg_hip_host_alloc(self.ctx, n * @sizeOf(T), &ptr) != 0) return Error.DeviceOOM;
+    const p: [*]T = @ptrCast(@alignCast(ptr.?));
+    return p[0..n];
 }
 
-/// usize buffers the host may write and the kernels may read (edge lists, gather indices).
+/// Kept for callers that ask for index memory by name; `mem_alloc(usize, n)` returns the same kind of memory.
 pub fn mem_alloc_indices(self: *Self, n: usize) ![]usize {
-    var ptr: ?*anyopaque = null;
-    if (c.zg_hip_host_alloc(self.ctx, n * @sizeOf(usize), &ptr) != 0) return Error.DeviceOOM;
-    const p: [*]usize = @ptrCast(@alignCast(ptr.?));
-    return p[0..n];
+    return self.host_alloc(usize, n);
 }
 
 // --------------------------------------------------------------------------------------------------
@@ -162,6 +161,7 @@ pub fn mem_alloc_indices(self: *Self, n: usize) ![]usize {
 /// src/allocators/device_data.zig:32-40, src/allocators/block_pool.zig:262-269); views carry 0 and are never freed.
 pub fn mem_cache_alloc(self: *Self, T: type, n: usize) !DeviceData(T) {
     if (n == 0) return .{ .raw = &.{}, .ctx = 0 }; // src/allocators/caching_allocator.zig:81-85
+    if (T == usize) return .{ .raw = try self.host_alloc(T, n), .ctx = host_tag }; // host loops read and write it
     var ptr: ?*anyopaque = null;
     var block: u64 = 0;
     if (c.zg_hip_mem_cache_alloc(self.ctx, n * @sizeOf(T), &ptr, &block) != 0) return Error.DeviceOOM;
@@ -170,6 +170,7 @@ pub fn mem_cache_alloc(self: *Self, T: type, n: usize) !DeviceData(T) {
 }
 pub fn mem_cache_free(self: *Self, data: anytype) void {
     if (data.raw.len == 0 or data.ctx == 0) return; // src/allocators/caching_allocator.zig:111-112
+    if (data.ctx == host_tag) return check(c.zg_hip_host_free(self.ctx, @constCast(@ptrCast(data.raw.ptr))));
     check(c.zg_hip_mem_cache_free(self.ctx, @constCast(@ptrCast(data.raw.ptr)), @intCast(data.ctx)));
 }
 pub fn mem_cache_dupe(self: *Self, T: type, src: []const T) !DeviceData(T) {
@@ -180,6 +181,7 @@ pub fn mem_cache_dupe(self: *Self, T: type, src: []const T) !DeviceData(T) {
 }
 pub fn mem_alloc(self: *Self, T: type, n: usize) ![]T {
     if (n == 0) return &.{};
+    if (T == usize) return self.host_alloc(T, n); // NDArray.gather fills its offsets with a host loop
     var ptr: ?*anyopaque = null;
     if (c.zg_hip_alloc(self.ctx, n * @sizeOf(T), &ptr) != 0) return Error.DeviceOOM;
     const p: [*]T = @ptrCast(@alignCast(ptr.?));
@@ -190,6 +192,7 @@ pub fn mem_alloc_byte_mask(self: *Self, n: usize) ![]u8 {
 }
 pub fn mem_free(self: *Self, slice: anytype) void {
     if (slice.len == 0) return;
+    if (std.meta.Elem(@TypeOf(slice)) == usize) return check(c.zg_hip_host_free(self.ctx, @constCast(@ptrCast(slice.ptr))));
     check(c.zg_hip_free(self.ctx, @constCast(@ptrCast(slice.ptr))));
 }
 pub fn mem_dupe(self: *Self, T: type, src: []const T) ![]T {
@@ -211,9 +214,11 @@ pub fn mem_fill(self: *const Self, T: type, slice: []T, value: T) void {
         usize => check(c.zg_hip_mem_fill_u64(self.ctx, @ptrCast(slice.ptr), slice.len, value)),
         else => @compileError("HipDevice.mem_fill: unsupported element type " ++ @typeName(T)),
     }
+    if (T == usize) self.sync(); // host-visible memory: a host loop may read it next
 }
 pub fn mem_copy(self: *const Self, T: type, src: []const T, dst: []T) void {
     check(c.zg_hip_memcpy_d2d(self.ctx, dst.ptr, src.ptr, src.len * @sizeOf(T)));
+    if (T == usize) self.sync(); // host-visible memory: a host loop may read it next
 }
 pub fn mem_transfer(self: *const Self, T: type, src: []const T, dst: []T, dir: TransferDirection) void {
     const n = src.len * @sizeOf(T);
@@ -222,6 +227,7 @@ pub fn mem_transfer(self: *const Self, T: type, src: []const T, dst: []T, dir: T
         .DtoH => check(c.zg_hip_memcpy_d2h(self.ctx, dst.ptr, src.ptr, n)), // blocks: NDTensor.get reads right after
         .DtoD => check(c.zg_hip_memcpy_d2d(self.ctx, dst.ptr, src.ptr, n)),
     }
+    if (T == usize and dir == .DtoD) self.sync(); // the other two directions have waited already
 }
 pub fn mem_sequence(self: *const Self, T: type, slice: []T, initial: T, step: T) void {
     comptime std.debug.assert(T == f32);
@@ -259,21 +265,56 @@ fn only_f32(T: type) void {
     if (T != f32) @compileError("HipDevice implements f32 ops; got " ++ @typeName(T));
 }
 
+/// z = x o y with the reference's broadcasting (src/device/host_device.zig:975-1019).  An operand of one element
+/// that is not device memory is a scalar on the caller's stack (NDArray.add_scalar: `.y = &.{s}`,
+/// src/ndarray.zig:247-257) and is passed by value.
+const BinaryOp = enum { add, sub, mul, div };
+fn binary(self: *const Self, comptime op: BinaryOp, x: []const f32, y: []const f32, z: []f32) void {
+    const x_host = x.len == 1 and !self.is_device_ptr(x.ptr);
+    const y_host = y.len == 1 and !self.is_device_ptr(y.ptr);
+    if (x_host and y_host) {
+        // both operands on the host: the one result is formed where HostDevice forms it, the same fp32 operation
+        const v: f32 = switch (op) {
+            .add => x[0] + y[0],
+            .sub => x[0] - y[0],
+            .mul => x[0] * y[0],
+            .div => x[0] / y[0],
+        };
+        return check(c.zg_hip_mem_fill(self.ctx, z.ptr, z.len, v));
+    }
+    if (x_host or y_host) {
+        const vec = if (y_host) x else y;
+        const s = if (y_host) y[0] else x[0];
+        const lhs: c_int = @intFromBool(x_host);
+        return check(switch (op) {
+            .add => c.zg_hip_add_scalar(self.ctx, vec.ptr, vec.len, s, lhs, z.ptr),
+            .sub => c.zg_hip_sub_scalar(self.ctx, vec.ptr, vec.len, s, lhs, z.ptr),
+            .mul => c.zg_hip_mul_scalar(self.ctx, vec.ptr, vec.len, s, lhs, z.ptr),
+            .div => c.zg_hip_div_scalar(self.ctx, vec.ptr, vec.len, s, lhs, z.ptr),
+        });
+    }
+    check(switch (op) {
+        .add => c.zg_hip_add(self.ctx, x.ptr, x.len, y.ptr, y.len, z.ptr, z.len),
+        .sub => c.zg_hip_sub(self.ctx, x.ptr, x.len, y.ptr, y.len, z.ptr, z.len),
+        .mul => c.zg_hip_mul(self.ctx, x.ptr, x.len, y.ptr, y.len, z.ptr, z.len),
+        .div => c.zg_hip_div(self.ctx, x.ptr, x.len, y.ptr, y.len, z.ptr, z.len),
+    });
+}
 pub fn add(self: *const Self, T: type, p: opspec.add(T)) void {
     comptime only_f32(T);
-    check(c.zg_hip_add(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+    self.binary(.add, p.x, p.y, p.z);
 }
 pub fn sub(self: *const Self, T: type, p: opspec.sub(T)) void {
     comptime only_f32(T);
-    check(c.zg_hip_sub(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+    self.binary(.sub, p.x, p.y, p.z);
 }
 pub fn mul(self: *const Self, T: type, p: opspec.mul(T)) void {
     comptime only_f32(T);
-    check(c.zg_hip_mul(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+    self.binary(.mul, p.x, p.y, p.z);
 }
 pub fn div(self: *const Self, T: type, p: opspec.div(T)) void {
     comptime only_f32(T);
-    check(c.zg_hip_div(self.ctx, self.dev_scalar(T, p.x), p.x.len, self.dev_scalar(T, p.y), p.y.len, p.z.ptr, p.z.len));
+    self.binary(.div, p.x, p.y, p.z);
 }
 pub fn dot(self: *const Self, T: type, p: opspec.dot(T)) void {
     comptime only_f32(T);

@@ -260,6 +260,18 @@ struct zg_hip_ctx {
     // regions handed out by pool_map/alloc, for ownership checks at free time
     std::map<void*, size_t> raw_allocs;
     std::map<void*, size_t> host_allocs;
+    // Pinned host blocks that were given back and are kept for the next zg_hip_host_alloc of their size class
+    // (runtime.hip): a binding serves every `usize` tensor from pinned memory, one or more per train step, and the
+    // driver's pinned allocation and release cost far more than a step's kernels.  `done` marks the point on the
+    // stream after which no queued kernel reads the block; the next owner waits for it before it gets the block.
+    struct HostBlock {
+        void* ptr;
+        size_t cap;
+        hipEvent_t done;
+    };
+    std::map<void*, size_t> host_caps;  // capacity (size class) of every live pinned allocation
+    std::vector<HostBlock> host_free_blocks;
+    size_t host_cached_bytes = 0;
 };
 
 namespace zg {

@@ -310,6 +310,15 @@ ZG_OP(ScaleOp, return __fmul_rn(a, p0);)
 // broadcast / scaled copy: a = x, b = y -> alpha*x + beta*y
 ZG_OP(ScaledCopy, return __fadd_rn(__fmul_rn(p0, a), __fmul_rn(p1, b));)
 ZG_OP(ScaledCopyNoRead, return __fmul_rn(p0, a);)
+// binary ops with one operand passed by value: a = the array's element, p0 = the scalar; R: x o s, L: s o x
+ZG_OP(AddScalarR, return __fadd_rn(a, p0);)
+ZG_OP(AddScalarL, return __fadd_rn(p0, a);)
+ZG_OP(SubScalarR, return __fsub_rn(a, p0);)
+ZG_OP(SubScalarL, return __fsub_rn(p0, a);)
+ZG_OP(MulScalarR, return __fmul_rn(a, p0);)
+ZG_OP(MulScalarL, return __fmul_rn(p0, a);)
+ZG_OP(DivScalarR, return __fdiv_rn(a, p0);)
+ZG_OP(DivScalarL, return __fdiv_rn(p0, a);)
 // smooth-l1 / mse backward: a = pred, b = target, c = grad; p0 = beta or scale, p1 = n
 ZG_OP(SmoothL1Bwd, return __fadd_rn(c, smooth_l1_grad(a, b, p0, p1));)
 ZG_OP(MseBwd, return __fadd_rn(c, __fmul_rn(p0, __fsub_rn(a, b)));)
@@ -321,7 +330,9 @@ ZG_OP(MseBwd, return __fadd_rn(c, __fmul_rn(p0, __fsub_rn(a, b)));)
     X(0, Bin2<AddOp>) X(1, Bin2<SubOp>) X(2, Bin2<MulOp>) X(3, Bin2<DivOp>) X(4, PowFwd) X(5, SqrtFwd) X(6, RsqrtFwd) \
     X(7, ExpFwd) X(8, ReluFwd) X(9, TanhFwd) X(10, SigmFwd) X(11, ClampFwd) X(12, PowBwd) X(13, SqrtBwd)             \
     X(14, RsqrtBwd) X(15, ExpBwd) X(16, ReluBwd) X(17, ReluInplaceBwd) X(18, TanhBwd) X(19, TanhInplaceBwd)          \
-    X(20, SigmBwd) X(21, SigmInplaceBwd) X(22, ClampBwd) X(23, ScaleOp) X(24, SmoothL1Bwd) X(25, MseBwd)
+    X(20, SigmBwd) X(21, SigmInplaceBwd) X(22, ClampBwd) X(23, ScaleOp) X(24, SmoothL1Bwd) X(25, MseBwd)          \
+    X(27, AddScalarR) X(28, AddScalarL) X(29, SubScalarR) X(30, SubScalarL) X(31, MulScalarR) X(32, MulScalarL)      \
+    X(33, DivScalarR) X(34, DivScalarL)
 #define ZG_CHAIN_CODE(N, OP) template <> constexpr int chain_code<OP>() { return N; }
 ZG_CHAIN_OPS(ZG_CHAIN_CODE)
 #undef ZG_CHAIN_CODE
@@ -479,6 +490,28 @@ ZG_API int zg_hip_mul(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y
 }
 ZG_API int zg_hip_div(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, float* z, size_t zl) {
     return binary_op<DivOp>(ctx, "div", x, xl, y, yl, z, zl);
+}
+
+// The scalar operand of add_scalar & co (src/ndarray.zig:251: `.y = &.{s}`, a value on the caller's stack) by value: it
+// travels as a kernel argument, so nothing is copied to the device, a small op joins the waiting elementwise ops, and
+// the call can be recorded into an execution graph.  Same IEEE operation as the two-array form on a one-float operand.
+template <class OpR, class OpL>
+static int scalar_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t n, float s, int scalar_is_lhs, float* z) {
+    ZG_CHECK_N(name, n, x, z);
+    if (scalar_is_lhs) return launch_map<OpL, 1>(ctx, z, x, nullptr, nullptr, n, s);
+    return launch_map<OpR, 1>(ctx, z, x, nullptr, nullptr, n, s);
+}
+ZG_API int zg_hip_add_scalar(zg_hip_ctx* ctx, const float* x, size_t n, float s, int scalar_is_lhs, float* z) {
+    return scalar_op<AddScalarR, AddScalarL>(ctx, "add_scalar", x, n, s, scalar_is_lhs, z);
+}
+ZG_API int zg_hip_sub_scalar(zg_hip_ctx* ctx, const float* x, size_t n, float s, int scalar_is_lhs, float* z) {
+    return scalar_op<SubScalarR, SubScalarL>(ctx, "sub_scalar", x, n, s, scalar_is_lhs, z);
+}
+ZG_API int zg_hip_mul_scalar(zg_hip_ctx* ctx, const float* x, size_t n, float s, int scalar_is_lhs, float* z) {
+    return scalar_op<MulScalarR, MulScalarL>(ctx, "mul_scalar", x, n, s, scalar_is_lhs, z);
+}
+ZG_API int zg_hip_div_scalar(zg_hip_ctx* ctx, const float* x, size_t n, float s, int scalar_is_lhs, float* z) {
+    return scalar_op<DivScalarR, DivScalarL>(ctx, "div_scalar", x, n, s, scalar_is_lhs, z);
 }
 
 ZG_API int zg_hip_pow_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t n, float e) {

@@ -484,6 +484,10 @@ ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
     if (ctx->d2h_slot) (void)hipHostFree(ctx->d2h_slot);
     for (auto& kv : ctx->raw_allocs) (void)hipFree(kv.first);
     for (auto& kv : ctx->host_allocs) (void)hipHostFree(kv.first);
+    for (auto& b : ctx->host_free_blocks) {
+        (void)hipEventDestroy(b.done);
+        (void)hipHostFree(b.ptr);
+    }
     if (ctx->copy_stream) {
         (void)hipStreamSynchronize(ctx->copy_stream);
         (void)hipEventDestroy(ctx->ev_compute);
@@ -770,34 +774,73 @@ ZG_API int zg_hip_free(zg_hip_ctx* ctx, void* ptr) {
     return raw_free(ctx, ptr, "free");
 }
 
+// Pinned host memory.  Size classes are powers of two from 256 bytes; blocks of up to 16 MiB that are given back are
+// kept (up to 256 MiB in all) and handed out again to requests of the same class.
+constexpr size_t kHostBlockKeepMax = (size_t)16 << 20;
+constexpr size_t kHostCacheMax = (size_t)256 << 20;
+static size_t host_size_class(size_t bytes) {
+    size_t cap = 256;
+    while (cap < bytes) cap <<= 1;
+    return cap;
+}
+
 ZG_API int zg_hip_host_alloc(zg_hip_ctx* ctx, size_t bytes, void** out) {
     ZG_CTX(ctx);
     ZG_NOT_CAPTURING(ctx, "host_alloc");
     ZG_REQUIRE(out != nullptr, "host_alloc: null output");
     *out = nullptr;
     if (bytes == 0) return ZG_HIP_OK;
+    ZG_REQUIRE(bytes <= ((size_t)1 << 62), "host_alloc: %zu bytes", bytes);
+    const size_t cap = host_size_class(bytes);
     void* p = nullptr;
-    hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocDefault);
-    if (e != hipSuccess) {
-        (void)hipGetLastError();
-        set_error("host_alloc: hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
-        return ZG_HIP_EOOM;
+    for (size_t i = 0; i < ctx->host_free_blocks.size() && !p; i++) {
+        if (ctx->host_free_blocks[i].cap != cap) continue;
+        zg_hip_ctx::HostBlock b = ctx->host_free_blocks[i];
+        // kernels queued before the block was given back may still read it: wait for that point of the stream
+        ZG_HIP_TRY(hipEventSynchronize(b.done));
+        (void)hipEventDestroy(b.done);
+        ctx->host_free_blocks.erase(ctx->host_free_blocks.begin() + (long)i);
+        ctx->host_cached_bytes -= cap;
+        p = b.ptr;
+    }
+    if (!p) {
+        hipError_t e = hipHostMalloc(&p, cap, hipHostMallocDefault);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("host_alloc: hipHostMalloc(%zu) failed: %s", cap, hipGetErrorString(e));
+            return ZG_HIP_EOOM;
+        }
     }
     ctx->host_allocs[p] = bytes;
+    ctx->host_caps[p] = cap;
     *out = p;
     return ZG_HIP_OK;
 }
 
 ZG_API int zg_hip_host_free(zg_hip_ctx* ctx, void* ptr) {
-    ZG_CTX(ctx);
+    ZG_CTX(ctx);  // whatever waits in the context may read the block: it is launched first
     ZG_NOT_CAPTURING(ctx, "host_free");
     if (!ptr) return ZG_HIP_OK;
     auto it = ctx->host_allocs.find(ptr);
     ZG_REQUIRE(it != ctx->host_allocs.end(), "host_free: pointer %p was not allocated by this context", ptr);
-    ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    const size_t cap = ctx->host_caps[ptr];
     if (ctx->copy_stream) ZG_HIP_TRY(hipStreamSynchronize(ctx->copy_stream));
-    ZG_HIP_TRY(hipHostFree(ptr));
+    if (cap <= kHostBlockKeepMax && ctx->host_cached_bytes + cap <= kHostCacheMax) {
+        hipEvent_t done = nullptr;
+        ZG_HIP_TRY(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+        hipError_t e = hipEventRecord(done, ctx->stream);
+        if (e != hipSuccess) {
+            (void)hipEventDestroy(done);
+            ZG_HIP_TRY(e);
+        }
+        ctx->host_free_blocks.push_back(zg_hip_ctx::HostBlock{ptr, cap, done});
+        ctx->host_cached_bytes += cap;
+    } else {
+        ZG_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        ZG_HIP_TRY(hipHostFree(ptr));
+    }
     ctx->host_allocs.erase(it);
+    ctx->host_caps.erase(ptr);
     return ZG_HIP_OK;
 }
 
@@ -955,7 +998,7 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
 // what a binding needs to tell a device slice from a host scalar (the reference's callers pass both through the
 // same parameter: src/ndarray.zig:251, src/nn/optim.zig:117 against src/ndtensor.zig:1146-1150).
 ZG_API int zg_hip_is_device_ptr(zg_hip_ctx* ctx, const void* ptr, int* yes) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_ALL(ctx);  // a lookup in host tables: a binding asks before every op with a one-float operand
     ZG_REQUIRE(yes != nullptr, "is_device_ptr: null output");
     *yes = 0;
     if (!ptr) return ZG_HIP_OK;
@@ -1018,6 +1061,12 @@ ZG_API int zg_hip_clear_cache(zg_hip_ctx* ctx) {
         ctx->scratch = nullptr;
         ctx->scratch_bytes = 0;
     }
+    for (auto& b : ctx->host_free_blocks) {  // the stream has been waited for: nothing reads them any more
+        (void)hipEventDestroy(b.done);
+        (void)hipHostFree(b.ptr);
+    }
+    ctx->host_free_blocks.clear();
+    ctx->host_cached_bytes = 0;
     return ZG_HIP_OK;
 }
 

@@ -44,6 +44,16 @@ class DevBuf:
         return DevBuf(self.ptr + offset * self.dtype.itemsize, n, self.dtype, 0, "view")
 
 
+def _host_scalar(v):
+    """The float value of a host-side scalar operand, None for a device buffer."""
+    if isinstance(v, DevBuf):
+        return None
+    a = np.asarray(v, dtype=np.float32)
+    if a.size != 1:
+        raise ValueError("a host operand of an elementwise op must be a single value")
+    return float(a.reshape(())[()])
+
+
 def _shape(shape) -> tuple[ctypes.Array, int]:
     arr = (ctypes.c_uint64 * len(shape))(*[int(s) for s in shape])
     return arr, len(shape)
@@ -269,7 +279,17 @@ class HipDevice:
 
     # elementwise binary
     def _bin(self, cname, x, y, z):
-        self._call(cname, x.ptr, x.n, y.ptr, y.n, z.ptr, z.n)
+        """x or y may be a host scalar (a Python / numpy number or a one-element numpy array): what NDArray.add_scalar
+        hands the op as `.y = &.{s}` (src/ndarray.zig:247-257).  It goes to the by-value entry point."""
+        xs, ys = _host_scalar(x), _host_scalar(y)
+        if xs is None and ys is None:
+            self._call(cname, x.ptr, x.n, y.ptr, y.n, z.ptr, z.n)
+        elif xs is not None and ys is not None:
+            raise ValueError(f"{cname}: both operands are host scalars")
+        elif ys is not None:
+            self._call(cname + "_scalar", x.ptr, x.n, ys, 0, z.ptr)
+        else:
+            self._call(cname + "_scalar", y.ptr, y.n, xs, 1, z.ptr)
 
     def _op_add(self, x, y, z): self._bin("zg_hip_add", x, y, z)
     def _op_sub(self, x, y, z): self._bin("zg_hip_sub", x, y, z)

@@ -485,7 +485,8 @@ class DQNTrainer(GraphSteps):
     smooth-L1 loss, Adam.  Op order follows DQNAgent.train (examples/dqn/src/dqn_agent.zig:125-228) without
     its host-side clamps, on the network 4 -> 128 -> 128 -> 2."""
 
-    def __init__(self, dev, dims=(4, 128, 128, 2), batch=64, lr=1e-3, gamma=0.99, clip=True, fused=False):
+    def __init__(self, dev, dims=(4, 128, 128, 2), batch=64, lr=1e-3, gamma=0.99, clip=True, fused=False,
+                 device_scalars=False):
         self.dev, self.dims, self.batch, self.gamma = dev, list(dims), batch, gamma
         self.optim = Optimizer(dev, "adam", lr, clip, fused=fused)
         self.policy = MLP(dev, dims, self.optim, fused=fused)
@@ -494,8 +495,14 @@ class DQNTrainer(GraphSteps):
         self.states, self.next_states = dev.mem_alloc(F32, B * S), dev.mem_alloc(F32, B * S)
         self.actions = dev.mem_alloc(U64, B)
         self.rewards, self.dones = dev.mem_alloc(F32, B), dev.mem_alloc(F32, B)
-        self.gamma_t = dev.from_numpy(np.asarray([gamma], np.float32))
-        self.one_t = dev.from_numpy(np.asarray([1.0], np.float32))
+        # gamma and 1: host scalars, as NDArray's scalar ops hand them over (`.y = &.{s}`, src/ndarray.zig:247-257);
+        # with device_scalars they are one-element tensors in device memory, the form the example builds
+        # (examples/dqn/src/dqn_agent.zig:173-181).  Same values either way.
+        if device_scalars:
+            self.gamma_t = dev.from_numpy(np.asarray([gamma], np.float32))
+            self.one_t = dev.from_numpy(np.asarray([1.0], np.float32))
+        else:
+            self.gamma_t, self.one_t = float(np.float32(gamma)), 1.0
         self._init_loss_slot()
         self.last_grads = None
 

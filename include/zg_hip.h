@@ -30,6 +30,17 @@
  *     layer's products, its bias gradient, optimizer steps, the graph-convolution aggregation) are held inside the
  *     context for the calls that usually follow them and leave in fewer launches with the same values, and every
  *     other call launches what is held first (the comments at those entry points say what is held and for what);
+ *   - OPERAND LIFETIME.  Because work is held, a call that returned ZG_HIP_OK may still name its operands: every
+ *     pointer handed to a call (device operands, pinned host index arrays, a pinned or device alpha / lr_t) must stay
+ *     valid AND unchanged until the next call on the context that launches what is held: zg_hip_sync, zg_hip_flush,
+ *     zg_hip_stream, or any op that is not itself held.  Memory from this context's own allocators may be given back
+ *     at once (the free calls know what is held).  A caller that mixes its own HIP calls with the library's -- its own
+ *     hipMalloc / hipFree of operands, hipDeviceSynchronize followed by its own hipMemcpy of a result, kernels on a
+ *     stream handle fetched EARLIER from zg_hip_stream -- must call zg_hip_flush (or zg_hip_stream again) first, or
+ *     switch holding off for the context with zg_hip_set_holding(ctx, 0): then every call launches its own work
+ *     before it returns and the in-order stream alone decides what is visible, as in a library that holds nothing.
+ *     An error of held work (a failed launch) is reported by the call that launches it, not by the call that queued
+ *     it; with holding off it is reported by the next call on the context;
  *   - a context belongs to one host thread at a time (the reference's devices are not shared between threads
  *     either); different contexts may be used from different threads.
  */
@@ -65,10 +76,21 @@ enum { ZG_RAND_UNIFORM = 0, ZG_RAND_NORMAL = 1, ZG_RAND_KAIMING = 2 };
 const char *zg_hip_last_error(void);
 int zg_hip_device_count(int *count);
 int zg_hip_init(int device_id, zg_hip_ctx **out);
+/* Launches what waits, waits for the stream and releases everything the context owns.  The context is gone afterwards
+ * whatever is returned; a non-zero return reports an error of work that was still held. */
 int zg_hip_deinit(zg_hip_ctx *ctx);
 int zg_hip_sync(zg_hip_ctx *ctx);
+/* Launches whatever earlier calls left waiting in the context and returns without waiting for the stream (no
+ * counterpart in the reference, which holds nothing).  For callers that are about to touch operands or results with
+ * HIP calls of their own; see OPERAND LIFETIME above. */
+int zg_hip_flush(zg_hip_ctx *ctx);
+/* enable = 0: from now on every call launches its own work before it returns (what waits now is launched first);
+ * enable = 1 (the state of a new context): calls may leave work waiting for the calls that follow.  Values are the
+ * same either way; holding only saves launches. */
+int zg_hip_set_holding(zg_hip_ctx *ctx, int enable);
 int zg_hip_total_memory(zg_hip_ctx *ctx, size_t *bytes);
-/* the HIP stream every op is enqueued on, as an opaque pointer (hipStream_t) */
+/* the HIP stream every op is enqueued on, as an opaque pointer (hipStream_t).  What waits in the context is launched
+ * first; NULL when that fails (zg_hip_last_error has the reason) or ctx is NULL. */
 void *zg_hip_stream(zg_hip_ctx *ctx);
 
 /* timing helpers on the context's stream (hipEvent_t underneath) */
@@ -114,8 +136,9 @@ int zg_hip_clear_cache(zg_hip_ctx *ctx);
  * binding tells them apart with this range test.  A pure host-side lookup: nothing is launched and work that waits in
  * the context keeps waiting. */
 int zg_hip_is_device_ptr(zg_hip_ctx *ctx, const void *ptr, int *yes);
+/* host counters; nothing is launched and what waits keeps waiting */
 int zg_hip_cache_stats(zg_hip_ctx *ctx, size_t *bytes_in_use, size_t *bytes_mapped, uint64_t *n_device_allocs);
-/* Kernels launched by the library in this process so far, device-to-device copies included (no counterpart in the
+/* Kernels launched by the library in this process so far (all contexts together), device-to-device copies included (no counterpart in the
  * reference; for tests and for reading profiles: how many launches an op sequence costs).  Work still waiting in the
  * context is not counted and is not sent out by this call. */
 int zg_hip_launch_count(zg_hip_ctx *ctx, uint64_t *launches);

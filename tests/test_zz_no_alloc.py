@@ -113,6 +113,7 @@ def test_noalloc_launches_waiting_work_without_allocating():
         before = dev.cache_stats()["n_device_allocs"]
         dev.dispatch("matmul", A=a, B=w, C=c, m=m, n=n, k=k, trans_a=False, trans_b=True, lda=k, ldb=k, ldc=n, alpha=1.0,
                      beta=0.0)                                  # a layer's forward product: waits for its bias add
+        queued = dev.cache_stats()["n_device_allocs"]           # a host counter: the product keeps waiting
         dev.dispatch("smce_label_fwd_noalloc", logits=xb, labels=lb, lse=lse, loss=loss, rows=rows, cols=cols)
         after = dev.cache_stats()["n_device_allocs"]
         got = dev.to_numpy(c).reshape(m, n)
@@ -121,8 +122,10 @@ def test_noalloc_launches_waiting_work_without_allocating():
         x64 = x.astype(np.float64)
         lse64 = np.log(np.exp(x64 - x64.max(axis=1, keepdims=True)).sum(axis=1)) + x64.max(axis=1)
         assert np.allclose(dev.to_numpy(lse), lse64, rtol=1e-6, atol=1e-6)
-        # the product's workspace was allocated by the matmul call (at most one growth), nothing by the other
-        assert after - before <= 1
+        # the product's workspace was allocated by the matmul call (one growth), nothing by the allocation-free call
+        # although it is the one that launched the product
+        assert queued - before == 1
+        assert after == queued
         for b in (a, w, c, xb, lb, lse, loss):
             dev.mem_free(b)
     finally:

@@ -4,13 +4,14 @@
 
 // Every kernel launch of the library is counted (zg_hip_launch_count): the launches an op sequence costs are what the
 // work that waits inside the context is there to cut, and tests hold them to what was measured.
+#include <atomic>
 namespace zg {
-extern unsigned long long launches_issued;
+extern std::atomic<unsigned long long> launches_issued;  // process-wide: contexts on different threads share it
 }
 #undef hipLaunchKernelGGL
 #define hipLaunchKernelGGL(kernelName, numBlocks, numThreads, memPerBlock, streamId, ...)              \
     do {                                                                                               \
-        ++zg::launches_issued;                                                                         \
+        zg::launches_issued.fetch_add(1, std::memory_order_relaxed);                                                                       \
         (kernelName)<<<(numBlocks), (numThreads), (memPerBlock), (streamId)>>>(__VA_ARGS__);           \
     } while (0)
 
@@ -223,6 +224,11 @@ struct zg_hip_ctx {
     // the waiting fills first, so no call can see memory that a fill has not reached yet.
     zg_pending_fill pending_fills[kMaxPendingFills];
     int n_pending_fills = 0;
+    // hold_work false (zg_hip_set_holding): nothing stays waiting past the call that queued it, for callers that mix
+    // their own HIP calls with the library's.  late_error: what launching held work at the end of such a call
+    // returned; the next call on the context reports it.
+    bool hold_work = true;
+    int late_error = 0;
 
     // A layer's forward product waits one call for the bias add and the ReLU that the reference's Linear layer issues
     // right after it (examples/mnist/src/model.zig:104-110, :38-46), and an input-gradient product waits for the
@@ -317,6 +323,10 @@ int flush_pending_but_maps_and_fills(zg_hip_ctx* ctx);
 bool fills_touch(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count);
 bool take_fill_exact(zg_hip_ctx* ctx, const float* x, size_t n, float* value);
 void drop_fills_inside(zg_hip_ctx* ctx, const void* lo, size_t bytes);
+// The same, handing the dropped fills to the caller (`out` holds kMaxPendingFills): a call that then fails owes them
+// back (requeue_fills), because the memory was not overwritten after all.
+int take_fills_inside(zg_hip_ctx* ctx, const void* lo, size_t bytes, zg_pending_fill* out);
+void requeue_fills(zg_hip_ctx* ctx, const zg_pending_fill* fills, int count);
 bool scatter_take_add(zg_hip_ctx* ctx, const float* x, size_t xl, const float* y, size_t yl, const float* z, size_t zl);
 bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, int* rc);
 // Launches the optimizer steps that are waiting (optim.hip).  Gradients whose zero fill was taken over are zeroed by
@@ -340,6 +350,20 @@ bool deferred_take_relu_mask(zg_hip_ctx* ctx, const float* x, const float* x_g, 
 // (ensure_grad(0) followed by an accumulating backward op, src/ndtensor.zig:221-228), the same values without the
 // fill's launch and without the read.
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n);
+
+inline bool anything_waits(const zg_hip_ctx* ctx) {
+    return ctx->n_pending_fills || ctx->deferred.active || ctx->deferred_w.active || ctx->bias_wait.active ||
+           ctx->steps.count || ctx->scatter_wait.active || ctx->graddeg_wait.active || ctx->maps.count;
+}
+// Lives for the length of an entry point (the ZG_CTX* macros declare one): with holding switched off, whatever the
+// call queued is launched before the call returns.
+struct HoldGuard {
+    zg_hip_ctx* ctx;
+    ~HoldGuard() {
+        if (ctx && !ctx->hold_work && anything_waits(ctx))
+            if (int rc = flush_pending(ctx)) ctx->late_error = rc;
+    }
+};
 
 void plan_cache_destroy(zg_hip_ctx* ctx);
 void gemm_plans_destroy(zg_hip_ctx* ctx);
@@ -398,8 +422,17 @@ inline bool aligned16(const void* p) {
     } while (0)
 
 // First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
-#define ZG_CTX(ctx)                                          \
+#define ZG_CTX_ENTER(ctx)                                    \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
+    zg::HoldGuard _zg_hold_guard{(ctx)};                     \
+    (void)_zg_hold_guard;                                    \
+    if ((ctx)->late_error) {                                 \
+        const int _rc_late = (ctx)->late_error;              \
+        (ctx)->late_error = 0;                               \
+        return _rc_late;                                     \
+    }
+#define ZG_CTX(ctx)                                          \
+    ZG_CTX_ENTER(ctx)                                        \
     if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
         (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active || (ctx)->maps.count) { \
         if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
@@ -408,7 +441,7 @@ inline bool aligned16(const void* p) {
 // calls a product may absorb.
 // A waiting aggregation only waits for the add and the ReLU, which look at it before they get here: it goes out.
 #define ZG_CTX_KEEP_FILLS(ctx)                                   \
-    ZG_REQUIRE((ctx) != nullptr, "null context");                \
+    ZG_CTX_ENTER(ctx)                                            \
     if ((ctx)->scatter_wait.active) {                            \
         if (int _rc_sc = zg::flush_scatter(ctx)) return _rc_sc;  \
     }                                                            \
@@ -422,7 +455,7 @@ inline bool aligned16(const void* p) {
 // the waiting fills (the call sends them out if one meets its operands, or takes over the one that covers its output);
 // everything else that waits goes out.
 #define ZG_CTX_KEEP_MAPS(ctx)                                    \
-    ZG_REQUIRE((ctx) != nullptr, "null context");                \
+    ZG_CTX_ENTER(ctx)                                            \
     if ((ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || (ctx)->scatter_wait.active || \
         (ctx)->graddeg_wait.active) {                            \
         if (int _rc_km = zg::flush_pending_but_maps_and_fills(ctx)) return _rc_km; \
@@ -430,7 +463,7 @@ inline bool aligned16(const void* p) {
 // The cache's allocations and frees look at each kind of waiting work themselves: a block that is handed out is free,
 // so nothing that waits names it; a block that is given back may be the one a waiting degree gradient would write, or
 // hold operands of waiting elementwise ops, which the pool's memory outlives.
-#define ZG_CTX_KEEP_ALL(ctx) ZG_REQUIRE((ctx) != nullptr, "null context")
+#define ZG_CTX_KEEP_ALL(ctx) ZG_CTX_ENTER(ctx)
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.
 #define ZG_NOT_CAPTURING(ctx, who)                                                                       \

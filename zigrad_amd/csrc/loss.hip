@@ -648,11 +648,16 @@ ZG_API int zg_hip_smce_label_fwd(zg_hip_ctx* ctx, const float* logits, const uin
 
 ZG_API int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, float* lse,
                                          float* loss, size_t rows, size_t cols) {
-    // work that earlier calls left waiting is launched by ZG_CTX below, like this call's own kernels without an
-    // allocation (a waiting product reserved its workspace when it was queued): the count of driver allocations is
-    // compared at the end and a difference is reported
+    // work that earlier calls left waiting is launched by ZG_CTX below, without an allocation (a waiting product reserved
+    // its workspace when it was queued): the count of driver allocations is compared before any kernel of this call is
+    // queued, so a call that reports a difference has launched nothing of its own
     const uint64_t allocs_before = ctx ? ctx->n_device_allocs : 0;
     ZG_CTX(ctx);
+    if (ctx->n_device_allocs != allocs_before) {
+        set_error("smce_label_fwd_noalloc: %llu driver allocation(s) were made while waiting work was launched",
+                  (unsigned long long)(ctx->n_device_allocs - allocs_before));
+        return ZG_HIP_ERUNTIME;
+    }
     ZG_REQUIRE(logits && labels && lse && loss, "smce_label_fwd_noalloc: null pointer");
     if (int rc = check_rows("smce_label_fwd_noalloc", rows, cols)) return rc;
     ZG_REQUIRE(rows <= kNoAllocMaxRows, "smce_label_fwd_noalloc: %zu rows exceed the fixed scratch (at most %zu rows)",
@@ -665,13 +670,7 @@ ZG_API int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx* ctx, const float* logits, c
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
                                             labels, lse, row_loss, rows, cols));
     ZG_LAUNCH_CHECK();
-    if (int rc = flat_reduce_into<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows}, partials)) return rc;
-    if (ctx->n_device_allocs != allocs_before) {
-        set_error("smce_label_fwd_noalloc: %llu driver allocation(s) were made while waiting work was launched",
-                  (unsigned long long)(ctx->n_device_allocs - allocs_before));
-        return ZG_HIP_ERUNTIME;
-    }
-    return ZG_HIP_OK;
+    return flat_reduce_into<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows}, partials);
 }
 
 ZG_API int zg_hip_smce_label_bwd(zg_hip_ctx* ctx, const float* logits, const uint64_t* labels, const float* lse,

@@ -408,6 +408,8 @@ ZG_API int zg_hip_max_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_s
         return rc;
     }
     const size_t outer = prod(x_shape, 0, dim), R = x_shape[dim], inner = prod(x_shape, dim + 1, x_rank);
+    zg_pending_fill dropped[kMaxPendingFills];
+    int n_dropped = 0;
     {
         // every element of y is written and none is read: a fill inside y that still waits has no reader left
         // (NDArray.max_along zero-fills its output first, src/ndarray.zig:567); the other waiting fills stay unless
@@ -417,13 +419,15 @@ ZG_API int zg_hip_max_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_s
         if (x0 < y1 && y0 < x1) {
             if ((rc = flush_pending(ctx))) return rc;
         } else {
-            drop_fills_inside(ctx, y, y_len * sizeof(float));
+            n_dropped = take_fills_inside(ctx, y, y_len * sizeof(float), dropped);
             const void* ptrs[2] = {x, y};
             const size_t bytes[2] = {(size_t)(x1 - x0), (size_t)(y1 - y0)};
-            if ((rc = flush_pending_but_fills(ctx, ptrs, bytes, 2))) return rc;
+            rc = flush_pending_but_fills(ctx, ptrs, bytes, 2);
         }
     }
-    return axis_reduce<AxisMax>(ctx, x, y, outer, R, inner, 1.f, 0.f);
+    if (rc == ZG_HIP_OK) rc = axis_reduce<AxisMax>(ctx, x, y, outer, R, inner, 1.f, 0.f);
+    if (rc) requeue_fills(ctx, dropped, n_dropped);  // refused: y was not overwritten, its fills are still owed
+    return rc;
 }
 
 ZG_API int zg_hip_argmax_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, uint64_t* y,

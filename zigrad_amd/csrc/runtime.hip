@@ -464,7 +464,11 @@ ZG_API int zg_hip_init(int device_id, zg_hip_ctx** out) {
 }
 
 ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
-    ZG_CTX(ctx);
+    ZG_REQUIRE(ctx != nullptr, "null context");
+    // held work is launched first; if that fails the error is returned, but the context is torn down all the same
+    int held_rc = ctx->late_error;
+    if (anything_waits(ctx))
+        if (int rc = flush_pending(ctx)) held_rc = held_rc ? held_rc : rc;
     (void)hipStreamSynchronize(ctx->stream);
     gemm_plans_destroy(ctx);
     plan_cache_destroy(ctx);  // its device memory is in raw_allocs; this frees the host side
@@ -496,6 +500,20 @@ ZG_API int zg_hip_deinit(zg_hip_ctx* ctx) {
     }
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
+    return held_rc;
+}
+
+// Launches whatever waits in the context, without waiting for the stream (no counterpart in the reference).
+ZG_API int zg_hip_flush(zg_hip_ctx* ctx) {
+    ZG_CTX(ctx);
+    return ZG_HIP_OK;
+}
+
+// Whether calls may leave work waiting in the context for the calls that follow (default) or launch their own work
+// before they return.
+ZG_API int zg_hip_set_holding(zg_hip_ctx* ctx, int enable) {
+    ZG_CTX(ctx);  // what waits now goes out either way
+    ctx->hold_work = enable != 0;
     return ZG_HIP_OK;
 }
 
@@ -679,7 +697,9 @@ ZG_API int zg_hip_total_memory(zg_hip_ctx* ctx, size_t* bytes) {
 
 ZG_API void* zg_hip_stream(zg_hip_ctx* ctx) {
     if (!ctx) return nullptr;
-    (void)flush_pending(ctx);  // work the caller queues on the stream itself must find everything already there
+    // work the caller queues on the stream itself must find everything already there; if what waits cannot be launched
+    // the stream is not handed out (zg_hip_last_error says why)
+    if (flush_pending(ctx) != ZG_HIP_OK) return nullptr;
     return (void*)ctx->stream;
 }
 
@@ -1071,17 +1091,17 @@ ZG_API int zg_hip_clear_cache(zg_hip_ctx* ctx) {
 }
 
 namespace zg {
-unsigned long long launches_issued = 0;
+std::atomic<unsigned long long> launches_issued{0};
 }
 
 ZG_API int zg_hip_launch_count(zg_hip_ctx* ctx, uint64_t* launches) {
     ZG_REQUIRE(ctx != nullptr && launches != nullptr, "launch_count: null argument");
-    *launches = launches_issued;  // nothing is sent out: what waits in the context has not been launched and is not counted
+    *launches = launches_issued.load(std::memory_order_relaxed);  // nothing is sent out: what waits in the context has not been launched and is not counted
     return ZG_HIP_OK;
 }
 
 ZG_API int zg_hip_cache_stats(zg_hip_ctx* ctx, size_t* bytes_in_use, size_t* bytes_mapped, uint64_t* n_device_allocs) {
-    ZG_CTX(ctx);
+    ZG_CTX_KEEP_ALL(ctx);  // host counters only: what waits keeps waiting
     size_t u = 0, m = 0;
     for (BlockPool* p : {ctx->small_pool, ctx->large_pool}) {
         if (p) {
@@ -1142,11 +1162,14 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
         if (bytes == 0) return ZG_HIP_OK;
         ZG_REQUIRE(dst && src, "memcpy_d2d: null pointer");
     }
+    // fills dropped below are owed back if the copy is then refused
+    zg_pending_fill dropped[kMaxPendingFills];
+    int n_dropped = 0;
     {
         // waiting fills that meet neither range stay; one that lies inside a destination the copy overwrites without
         // reading it has no reader left
         const char *s0 = (const char*)src, *d0 = (const char*)dst;
-        if (s0 + bytes <= d0 || d0 + bytes <= s0) drop_fills_inside(ctx, dst, bytes);
+        if (s0 + bytes <= d0 || d0 + bytes <= s0) n_dropped = take_fills_inside(ctx, dst, bytes, dropped);
         // a waiting float fill that covers the destination and more (a gradient zeroed, then its leading rows
         // overwritten) and is clear of the source leaves together with the copy, in one launch
         int host_fill = -1;
@@ -1168,8 +1191,9 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
         const size_t lens[2] = {bytes, bytes};
         int rc = flush_pending_but_fills(ctx, ptrs, lens, 2);
         if (host_fill >= 0) {
-            if (rc) {  // refused: the fill is still owed
+            if (rc) {  // refused: the fills are still owed
                 (void)zg_hip_mem_fill(ctx, f.x, f.n, f.value);
+                requeue_fills(ctx, dropped, n_dropped);
                 return rc;
             }
             hipLaunchKernelGGL(fill_and_copy_kernel, dim3(grid_for(ctx, f.n, kBlock)), dim3(kBlock), 0, ctx->stream, f.x, f.n,
@@ -1177,7 +1201,10 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
             ZG_LAUNCH_CHECK();
             return ZG_HIP_OK;
         }
-        if (rc) return rc;
+        if (rc) {
+            requeue_fills(ctx, dropped, n_dropped);
+            return rc;
+        }
     }
     if (ctx->capturing) {
         // recorded as a kernel node like everything else in the graph
@@ -1192,8 +1219,11 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    ++launches_issued;  // the driver's copy kernel
-    ZG_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, ctx->stream));
+    launches_issued.fetch_add(1, std::memory_order_relaxed);  // the driver's copy kernel
+    if (hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, ctx->stream)) {
+        requeue_fills(ctx, dropped, n_dropped);
+        ZG_HIP_TRY(e);
+    }
     return ZG_HIP_OK;
 }
 
@@ -1295,15 +1325,23 @@ bool take_fill_exact(zg_hip_ctx* ctx, const float* x, size_t n, float* value) {
     }
     return false;
 }
-void drop_fills_inside(zg_hip_ctx* ctx, const void* lo_, size_t bytes) {
+int take_fills_inside(zg_hip_ctx* ctx, const void* lo_, size_t bytes, zg_pending_fill* out) {
     const char *lo = (const char*)lo_, *hi = lo + bytes;
-    int kept = 0;
+    int kept = 0, taken = 0;
     for (int i = 0; i < ctx->n_pending_fills; i++) {
         const char* x0 = (const char*)ctx->pending_fills[i].x;
         const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
         if (!(lo <= x0 && x1 <= hi)) ctx->pending_fills[kept++] = ctx->pending_fills[i];
+        else if (out) out[taken++] = ctx->pending_fills[i];
     }
     ctx->n_pending_fills = kept;
+    return taken;
+}
+void drop_fills_inside(zg_hip_ctx* ctx, const void* lo, size_t bytes) {
+    (void)take_fills_inside(ctx, lo, bytes, nullptr);
+}
+void requeue_fills(zg_hip_ctx* ctx, const zg_pending_fill* fills, int count) {
+    for (int i = 0; i < count; i++) (void)zg_hip_mem_fill(ctx, fills[i].x, fills[i].n, fills[i].value);
 }
 
 int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {

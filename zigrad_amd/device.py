@@ -90,6 +90,14 @@ class HipDevice:
     def sync(self) -> None:
         self._call("zg_hip_sync")
 
+    def flush(self) -> None:
+        """Launch what earlier calls left waiting in the context, without waiting for the stream."""
+        self._call("zg_hip_flush")
+
+    def set_holding(self, enable: bool) -> None:
+        """False: every call launches its own work before it returns (for callers that mix in their own HIP calls)."""
+        self._call("zg_hip_set_holding", int(bool(enable)))
+
     def _call(self, name: str, *args) -> None:
         self._lib.call(name, self._ctx, *args)
 

@@ -490,75 +490,116 @@ pub fn scatter_gcn_deg_scaled_bwd(self: *const Self, T: type, p: opspec.scatter_
     check(c.zg_hip_scatter_gcn_deg_scaled_bwd(self.ctx, p.grad_output.ptr, p.h.ptr, p.deg.ptr, @ptrCast(p.src_indices.ptr), @ptrCast(p.tgt_indices.ptr), p.grad_h.ptr, p.grad_deg.ptr, p.stride, p.n_edge, p.deg.len));
 }
 
-// New op names for what the reference computes with host loops over `.raw` (they need the matching
-// parameter structs added to opspec.zig, field names as used below, and the call sites switched to dispatch):
+// New op names for what the reference computes with host loops over `.raw`.  Their parameter structs are in
+// zig/opspec_additions.zig (to be appended to src/device/opspec.zig); the call sites that switch to dispatch:
 //   smce_fwd / smce_bwd / smce_label_fwd / smce_label_bwd   src/nn/loss.zig:130-215
+//   softmax_fwd / softmax_bwd                                src/nn/loss.zig:217-257
 //   smooth_l1_fwd / smooth_l1_bwd / mse_fwd / mse_bwd        src/nn/loss.zig:94-127, 259-305
 //   sgd_step / adam_step                                     src/nn/optim.zig:100-122, 177-234
 //   argmax_along, gather_offsets, index_select_fwd / _bwd    examples/mnist/src/main-simple.zig:124, src/ndarray.zig:607-624,
 //                                                            src/ndtensor.zig:1437-1513
-/// NDArray.gather (src/ndarray.zig:593-633) as one device op: the offsets (kept for the backward's scatter_add) and
-/// the gathered values.  `p.check` reads the out-of-bounds status back (one blocking 4-byte copy).
-pub fn gather(self: *const Self, T: type, p: anytype) !void {
+pub fn argmax_along(self: *const Self, T: type, p: opspec.argmax_along(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_argmax_along(self.ctx, p.x.ptr, @ptrCast(p.x_shape.ptr), p.x_shape.len, @ptrCast(p.y.ptr), p.y.len, p.dim));
+    self.sync(); // `y` is host-visible index memory: the caller's loop reads it next
+}
+/// The offsets loop of NDArray.gather (src/ndarray.zig:607-624) on the device.  `p.check` reads the status back.
+pub fn gather_offsets(self: *const Self, T: type, p: opspec.gather_offsets(T)) !void {
     comptime only_f32(T);
     var status: c_int = 0;
-    const rc = c.zg_hip_gather(self.ctx, p.src.ptr, @ptrCast(p.src_shape.ptr), @ptrCast(p.idx_shape.ptr), p.src_shape.len, @ptrCast(p.indices.ptr), p.dim, @ptrCast(p.offsets.ptr), p.dst.ptr, if (p.check) &status else null);
+    const status_ptr: ?*c_int = if (p.check) &status else null;
+    const rc = c.zg_hip_gather_offsets(self.ctx, @ptrCast(p.src_shape.ptr), @ptrCast(p.idx_shape.ptr), p.src_shape.len, @ptrCast(p.indices.ptr), p.dim, @ptrCast(p.offsets.ptr), status_ptr);
     if (status == 1) return error.InvalidIndexShape;
     if (status == 2) return error.IndexOutOfBounds;
     check(rc);
 }
-pub fn smce_fwd(self: *const Self, T: type, p: anytype) void {
+pub fn index_select_fwd(self: *const Self, T: type, p: opspec.index_select_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_index_select_fwd(self.ctx, p.src.ptr, p.src.len, @ptrCast(p.indices.ptr), p.indices.len, p.stride, p.dst.ptr));
+}
+pub fn index_select_bwd(self: *const Self, T: type, p: opspec.index_select_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_index_select_bwd(self.ctx, p.y_grad.ptr, @ptrCast(p.indices.ptr), p.indices.len, p.stride, p.x_grad.ptr, p.x_grad.len));
+}
+pub fn smce_label_fwd(self: *const Self, T: type, p: opspec.smce_label_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smce_label_fwd(self.ctx, p.logits.ptr, @ptrCast(p.labels.ptr), p.lse.ptr, p.loss.ptr, p.rows, p.cols));
+}
+pub fn smce_label_bwd(self: *const Self, T: type, p: opspec.smce_label_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_smce_label_bwd(self.ctx, p.logits.ptr, @ptrCast(p.labels.ptr), p.lse.ptr, p.grad.ptr, p.rows, p.cols, @intFromBool(p.accumulate)));
+}
+pub fn softmax_fwd(self: *const Self, T: type, p: opspec.softmax_fwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_softmax_fwd(self.ctx, p.x.ptr, p.y.ptr, p.rows, p.cols));
+}
+pub fn softmax_bwd(self: *const Self, T: type, p: opspec.softmax_bwd(T)) void {
+    comptime only_f32(T);
+    check(c.zg_hip_softmax_bwd(self.ctx, p.y.ptr, p.y_g.ptr, p.x_g.ptr, p.rows, p.cols));
+}
+/// NDArray.gather (src/ndarray.zig:593-633) as one device op: the offsets (kept for the backward's scatter_add) and
+/// the gathered values.  `p.check` reads the out-of-bounds status back (one blocking 4-byte copy).
+pub fn gather(self: *const Self, T: type, p: opspec.gather(T)) !void {
+    comptime only_f32(T);
+    var status: c_int = 0;
+    const status_ptr: ?*c_int = if (p.check) &status else null;
+    const rc = c.zg_hip_gather(self.ctx, p.src.ptr, @ptrCast(p.src_shape.ptr), @ptrCast(p.idx_shape.ptr), p.src_shape.len, @ptrCast(p.indices.ptr), p.dim, @ptrCast(p.offsets.ptr), p.dst.ptr, status_ptr);
+    if (status == 1) return error.InvalidIndexShape;
+    if (status == 2) return error.IndexOutOfBounds;
+    check(rc);
+}
+pub fn smce_fwd(self: *const Self, T: type, p: opspec.smce_fwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_smce_fwd(self.ctx, p.logits.ptr, p.target.ptr, p.probs.ptr, p.loss.ptr, p.rows, p.cols));
 }
-pub fn smce_bwd(self: *const Self, T: type, p: anytype) void {
+pub fn smce_bwd(self: *const Self, T: type, p: opspec.smce_bwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_smce_bwd(self.ctx, p.probs.ptr, p.target.ptr, p.grad.ptr, p.rows, p.cols));
 }
 /// smce_fwd and the backward of the scalar loss in one call (upstream gradient 1): p.grad (+)= (probs - target)/rows.
-pub fn smce_fwd_bwd(self: *const Self, T: type, p: anytype) void {
+pub fn smce_fwd_bwd(self: *const Self, T: type, p: opspec.smce_fwd_bwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_smce_fwd_bwd(self.ctx, p.logits.ptr, p.target.ptr, p.probs.ptr, p.loss.ptr, p.grad.ptr, p.rows, p.cols, @intFromBool(p.accumulate)));
 }
-pub fn smooth_l1_fwd(self: *const Self, T: type, p: anytype) void {
+pub fn smooth_l1_fwd(self: *const Self, T: type, p: opspec.smooth_l1_fwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_smooth_l1_fwd(self.ctx, p.pred.ptr, p.target.ptr, p.pred.len, p.beta, p.loss.ptr));
 }
 /// smooth_l1_fwd and the backward of the scalar loss in one call: p.grad (+)= d loss / d pred.
-pub fn smooth_l1_fwd_bwd(self: *const Self, T: type, p: anytype) void {
+pub fn smooth_l1_fwd_bwd(self: *const Self, T: type, p: opspec.smooth_l1_fwd_bwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_smooth_l1_fwd_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len, p.beta, p.loss.ptr, @intFromBool(p.accumulate)));
 }
-pub fn smooth_l1_bwd(self: *const Self, T: type, p: anytype) void {
+pub fn smooth_l1_bwd(self: *const Self, T: type, p: opspec.smooth_l1_bwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_smooth_l1_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len, p.beta));
 }
-pub fn mse_fwd(self: *const Self, T: type, p: anytype) void {
+pub fn mse_fwd(self: *const Self, T: type, p: opspec.mse_fwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_mse_fwd(self.ctx, p.pred.ptr, p.target.ptr, p.pred.len, p.loss.ptr));
 }
-pub fn mse_bwd(self: *const Self, T: type, p: anytype) void {
+pub fn mse_bwd(self: *const Self, T: type, p: opspec.mse_bwd(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_mse_bwd(self.ctx, p.pred.ptr, p.target.ptr, p.grad.ptr, p.pred.len));
 }
-pub fn sgd_step(self: *const Self, T: type, p: anytype) void {
+pub fn sgd_step(self: *const Self, T: type, p: opspec.sgd_step(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_sgd_step(self.ctx, p.param.ptr, p.grad.ptr, p.param.len, p.lr, @intFromBool(p.clip), p.max_norm, p.delta));
 }
-pub fn adam_step(self: *const Self, T: type, p: anytype) void {
+pub fn adam_step(self: *const Self, T: type, p: opspec.adam_step(T)) void {
     comptime only_f32(T);
-    check(c.zg_hip_adam_step(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.t, p.lr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
+    check(c.zg_hip_adam_step(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, @intCast(p.t), p.lr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
 }
 
 /// Optimizer.step() over a whole parameter list (src/nn/optim.zig:100-122, :177-234), optionally followed by
 /// model.zero_grad(): small tensors share launches.  `p.params`, `p.grads` (and `p.ms`, `p.vs`) are slices of
 /// device pointers, `p.lens` their element counts; Adam's `p.lr_t` holds one step size per tensor
 /// (`adam_lr_t` with that tensor's counter), in host memory unless `p.lr_t_in_memory`.
-pub fn sgd_step_multi(self: *const Self, T: type, p: anytype) void {
+pub fn sgd_step_multi(self: *const Self, T: type, p: opspec.sgd_step_multi(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_sgd_step_multi(self.ctx, p.params.len, p.params.ptr, p.grads.ptr, p.lens.ptr, p.lr, @intFromBool(p.clip), p.max_norm, p.delta, @intFromBool(p.zero_grads)));
 }
-pub fn adam_step_multi(self: *const Self, T: type, p: anytype) void {
+pub fn adam_step_multi(self: *const Self, T: type, p: opspec.adam_step_multi(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_adam_step_multi(self.ctx, p.params.len, p.params.ptr, p.grads.ptr, p.ms.ptr, p.vs.ptr, p.lens.ptr, p.lr_t.ptr, @intFromBool(p.lr_t_in_memory), p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta, @intFromBool(p.zero_grads)));
 }
@@ -580,16 +621,16 @@ pub const EdgePlan = struct {
         self.plan = null;
     }
 };
-pub fn scatter_add_planned(self: *const Self, T: type, p: anytype) void {
+pub fn scatter_add_planned(self: *const Self, T: type, p: opspec.scatter_add_planned(T)) void {
     comptime only_f32(T);
     check(c.zg_hip_scatter_add_planned(self.ctx, p.src.ptr, p.plan.plan, p.dst.ptr, @intFromBool(p.accumulate)));
 }
-pub fn scatter_gcn_deg_scaled_planned(self: *const Self, T: type, p: anytype) void {
+pub fn scatter_gcn_deg_scaled_planned(self: *const Self, T: type, p: opspec.scatter_gcn_deg_scaled_planned(T)) void {
     comptime only_f32(T);
     const bias: ?[*]const T = if (p.bias) |b| b.ptr else null;  // the layer's tail: + bias, then relu when asked
     check(c.zg_hip_scatter_gcn_deg_scaled_planned(self.ctx, p.dst.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, bias, @intFromBool(p.relu), p.stride, @intFromBool(p.accumulate)));
 }
-pub fn scatter_gcn_deg_scaled_bwd_planned(self: *const Self, T: type, p: anytype) void {
+pub fn scatter_gcn_deg_scaled_bwd_planned(self: *const Self, T: type, p: opspec.scatter_gcn_deg_scaled_bwd_planned(T)) void {
     comptime only_f32(T);
     const gd: ?[*]T = if (p.grad_deg) |g| g.ptr else null; // optional: the degrees are data of the graph
     check(c.zg_hip_scatter_gcn_deg_scaled_bwd_planned(self.ctx, p.grad_output.ptr, p.h.ptr, p.deg.ptr, p.plan.plan, p.grad_h.ptr, gd, p.stride, @intFromBool(p.accumulate)));
@@ -597,7 +638,7 @@ pub fn scatter_gcn_deg_scaled_bwd_planned(self: *const Self, T: type, p: anytype
 
 /// A Linear layer's forward in one launch: y = act(x . w^T + bias), the arithmetic of `bmm_acc(trans_b)` +
 /// `bias.add_` + `relu_` (examples/mnist/src/model.zig:104-110, :38-46).  `p.bias` is an optional slice.
-pub fn linear_fwd(self: *const Self, T: type, p: anytype) void {
+pub fn linear_fwd(self: *const Self, T: type, p: opspec.linear_fwd(T)) void {
     comptime only_f32(T);
     const bias: ?[*]const T = if (p.bias) |b| b.ptr else null;
     check(c.zg_hip_linear_fwd(self.ctx, p.x.ptr, p.w.ptr, bias, p.y.ptr, p.batch, p.fan_in, p.fan_out, @intFromBool(p.relu)));
@@ -605,7 +646,7 @@ pub fn linear_fwd(self: *const Self, T: type, p: anytype) void {
 /// The input gradient of a Linear layer with the ReLU backward of the layer before it in one launch:
 /// gx = (accumulate ? gx : 0) + gy . w, zeroed where `p.act_in` (that ReLU's output, optional) is <= 0:
 /// the dA product of BmmAccBwd (src/ndtensor.zig:1092-1136) + relu_inplace_bwd (src/device/host_device.zig:543-547).
-pub fn linear_bwd_input(self: *const Self, T: type, p: anytype) void {
+pub fn linear_bwd_input(self: *const Self, T: type, p: opspec.linear_bwd_input(T)) void {
     comptime only_f32(T);
     const act: ?[*]const T = if (p.act_in) |a| a.ptr else null;
     check(c.zg_hip_linear_bwd_input(self.ctx, p.gy.ptr, p.w.ptr, act, p.gx.ptr, p.batch, p.fan_in, p.fan_out, @intFromBool(p.accumulate)));
@@ -613,7 +654,7 @@ pub fn linear_bwd_input(self: *const Self, T: type, p: anytype) void {
 /// The whole backward of a Linear layer for a final output gradient: gw += gy^T . x, gb += column sums of gy
 /// (`p.gb` optional), gx = gy . w zeroed where `p.act_in` <= 0 (`p.gx`, `p.act_in` optional): the two products of
 /// BmmAccBwd (src/ndtensor.zig:1092-1136), the bias's unbroadcast and relu_inplace_bwd of the layer before.
-pub fn linear_bwd(self: *const Self, T: type, p: anytype) void {
+pub fn linear_bwd(self: *const Self, T: type, p: opspec.linear_bwd(T)) void {
     comptime only_f32(T);
     const act: ?[*]const T = if (p.act_in) |a| a.ptr else null;
     const gb: ?[*]T = if (p.gb) |b| b.ptr else null;
@@ -624,9 +665,9 @@ pub fn linear_bwd(self: *const Self, T: type, p: anytype) void {
 /// Adam update whose `lr_t` is read from memory when the kernel runs (`p.lr_t` points to device memory or
 /// to `mem_alloc_indices`-style pinned host memory).  A step recorded with `capture.open()` can then be
 /// replayed for every later step: the host only rewrites `lr_t` between replays.
-pub fn adam_step_at(self: *const Self, T: type, p: anytype) void {
+pub fn adam_step_at(self: *const Self, T: type, p: opspec.adam_step_at(T)) void {
     comptime only_f32(T);
-    check(c.zg_hip_adam_step_at(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.lr_t, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
+    check(c.zg_hip_adam_step_at(self.ctx, p.param.ptr, p.grad.ptr, p.m.ptr, p.v.ptr, p.param.len, p.lr_t.ptr, p.beta1, p.beta2, p.epsilon, @intFromBool(p.clip), p.max_norm, p.delta));
 }
 
 /// The ExecutionGraph of the reference's second device (src/device/cuda_device.zig:558-611), same four calls.

@@ -5,7 +5,7 @@
 // holds the short operand in registers while it walks down the rows of the long one.
 // Arithmetic is kept as separate fp32 multiplies and adds (no contraction) so each element rounds
 // exactly like the host loop it replaces.
-#include "common.h"
+#include "reduce_device.h"
 
 namespace zg {
 
@@ -24,15 +24,21 @@ __global__ __launch_bounds__(kBlock) void map_vec4_kernel(float* out, const floa
     float4* o4 = reinterpret_cast<float4*>(out);
     size_t base = (size_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * (kBlock * kUnroll);
+    // Three or more streams run at 71-76 % of HBM bandwidth through the caches and at 83-88 % with the non-temporal
+    // hint on what is touched once (measured on [8192,4096]: mul 70.6 -> 60.5 us, relu_bwd 88.5 -> 76.3 us).  An operand
+    // that is also the output keeps plain accesses (its line is written right after it is read), and an in-place op of
+    // two streams is fastest with plain accesses throughout (56.8 us against 58.6).
+    const bool aliased = out == a || (NIN > 1 && out == b) || (NIN > 2 && out == c);
+    const bool nt = NIN > 1 && !(NIN == 2 && aliased);  // (one input, one output: 39.3 us plain, 42.0 us with the hint)
     for (; base < n4; base += stride) {
         float4 va[kUnroll], vb[kUnroll], vc[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             size_t i = base + (size_t)u * kBlock;
             if (i < n4) {
-                va[u] = a4[i];
-                if (NIN > 1) vb[u] = b4[i];
-                if (NIN > 2) vc[u] = c4[i];
+                va[u] = (nt && a != out) ? nt_load(a4 + i) : a4[i];
+                if (NIN > 1) vb[u] = (nt && b != out) ? nt_load(b4 + i) : b4[i];
+                if (NIN > 2) vc[u] = (nt && c != out) ? nt_load(c4 + i) : c4[i];
             }
         }
 #pragma unroll
@@ -44,7 +50,8 @@ __global__ __launch_bounds__(kBlock) void map_vec4_kernel(float* out, const floa
                 r.y = Op::f(va[u].y, NIN > 1 ? vb[u].y : 0.f, NIN > 2 ? vc[u].y : 0.f, p0, p1);
                 r.z = Op::f(va[u].z, NIN > 1 ? vb[u].z : 0.f, NIN > 2 ? vc[u].z : 0.f, p0, p1);
                 r.w = Op::f(va[u].w, NIN > 1 ? vb[u].w : 0.f, NIN > 2 ? vc[u].w : 0.f, p0, p1);
-                o4[i] = r;
+                if (nt && !aliased) nt_store(r, o4 + i);
+                else o4[i] = r;
             }
         }
     }

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
             const size_t c4 = cols >> 2;
             size_t j = lane;
             for (; j + 3 * TPR < c4; j += 4 * TPR) {
-                float4 v0 = x4[j], v1 = x4[j + TPR], v2 = x4[j + 2 * TPR], v3 = x4[j + 3 * TPR];
+                float4 v0 = nt_load(x4 + j), v1 = nt_load(x4 + j + TPR), v2 = nt_load(x4 + j + 2 * TPR), v3 = nt_load(x4 + j + 3 * TPR);
                 const float4 vs[4] = {v0, v1, v2, v3};
 #pragma unroll
                 for (int u = 0; u < 4; u++) {

@@ -481,7 +481,7 @@ int zg_hip_adam_step_at(zg_hip_ctx *ctx, float *param, float *grad, float *m, fl
                         float beta1, float beta2, float epsilon, int clip, float max_norm, float delta);
 
 /* The optimizer step over a whole parameter list, as Optimizer.step() walks it (src/nn/optim.zig:100-122, :177-234):
- * tensors of up to 65536 elements share launches (one workgroup per tensor, 16 tensors per launch), larger ones
+ * tensors of up to 131072 elements share launches (one workgroup per tensor, 16 tensors per launch), larger ones
  * take the per-tensor kernels; values are those of the per-tensor calls.  The lists are host arrays of n_tensors
  * entries.  zero_grads != 0 also leaves every gradient zero: optim.step() followed by model.zero_grad()
  * (examples/mnist/src/main-simple.zig:70-71, examples/mnist/src/model.zig:57-62) without the fills.

@@ -11,7 +11,7 @@ from zigrad_amd.device import F32
 
 pytestmark = pytest.mark.gpu
 
-SIZES = [7, 640, 4096, 4097, 8192, 65536, 65537, 100_352, 1 << 20, (1 << 20) + 4, 128, 1]
+SIZES = [7, 640, 4096, 4097, 8192, 65536, 65537, 100_352, 131072, 131073, 1 << 20, (1 << 20) + 4, 128, 1]
 
 
 def _run(hip, kind, sizes, eager, clip, vary_lr=False, repeat_first=False):

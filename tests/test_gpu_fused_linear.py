@@ -151,12 +151,12 @@ def test_fused_step_replays_from_an_execution_graph(hip):
 @pytest.mark.parametrize("clip,zero", [(True, True), (True, False), (False, True)])
 def test_optimizer_list_entry_points_equal_the_per_tensor_ops(hip, kind, clip, zero):
     """Sizes either side of every limit (update slices of 2048, Adam's one-workgroup path up to 4096, the one-launch
-    norm up to 65536, the shared update launch up to 2^20), a list longer than one launch holds (16), gradients large
+    norm up to 131072, the shared update launch up to 2^20), a list longer than one launch holds (16), gradients large
     enough that the clip is active for some tensors and not for others."""
     from zigrad_amd.device import F32
 
     r = np.random.default_rng(7)
-    sizes = [1, 10, 128, 640, 2048, 2049, 4096, 4097, 8192, 65536, 65537, 100352, 3, 64, (1 << 20), (1 << 20) + 4] + [int(r.integers(1, 5000)) for _ in range(14)]
+    sizes = [1, 10, 128, 640, 2048, 2049, 4096, 4097, 8192, 65536, 65537, 100352, 131072, 131073, 3, 64, (1 << 20), (1 << 20) + 4] + [int(r.integers(1, 5000)) for _ in range(14)]
     host = [(r.standard_normal(n).astype(np.float32), (r.standard_normal(n) * r.choice([0.01, 3.0])).astype(np.float32),
              (r.standard_normal(n) * 0.1).astype(np.float32), (r.random(n) * 0.1).astype(np.float32)) for n in sizes]
     beta1, beta2, eps, lr = 0.9, 0.999, 1e-8, 0.01

@@ -25,7 +25,7 @@ def launches_per_step(hip, tr, steps=6):
     return total // steps
 
 
-@pytest.mark.parametrize("fused,want", [(False, 13), (True, 12)])
+@pytest.mark.parametrize("fused,want", [(False, 12), (True, 11)])
 def test_batch_64_mlp_step(hip, fused, want):
     dims, batch = [784, 128, 64, 10], 64
     params, x, onehot, labels = mlp_inputs(dims, batch, seed_weights=0, seed_data=1, data="uniform")

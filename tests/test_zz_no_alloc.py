@@ -27,9 +27,9 @@ def _run(dev, name, x, lab):
     return out["lse"], out["loss"]
 
 
-# first call: more than 65536 rows, so the sum of the row terms takes the two-launch form and uses the partials
+# first call: more than 131072 rows, so the sum of the row terms takes the two-launch form and uses the partials
 # part of the array; second call: few rows (single-launch sum) over stale contents
-@pytest.mark.parametrize("shapes", [[(70001, 24), (300, 40)], [(4096, 1000), (17, 7)], [(262144, 8), (65537, 8)]])
+@pytest.mark.parametrize("shapes", [[(140001, 12), (300, 40)], [(4096, 1000), (17, 7)], [(262144, 8), (131073, 8)], [(70001, 24), (65537, 8)]])
 def test_noalloc_matches_the_allocating_entry_point(hip, oracle, shapes):
     results = []
     for k, (rows, cols) in enumerate(shapes):

@@ -27,6 +27,9 @@ def _skewed_offsets(r, n, n_dst, hubs):
     (60_000, 50, [(0, 257), (1, 256), (2, 1024), (3, 1025), (49, 20_000)]),  # either side of both limits
     (5_000, 3, []),                                                    # every bucket long, none huge
     (300_000, 200_000, [(199_999, 3000), (7, 1500)]),                  # mostly tiny buckets, two long ones
+    (400_000, 1000, [(3, 200_000)]),                                   # the same through the radix build (>= 262144 entries)
+    (300_000, 50, [(0, 257), (1, 256), (2, 1024), (3, 1025), (49, 100_000)]),
+    (270_000, 3, []),
 ])
 def test_scatter_add_with_hub_destinations_equals_the_host_loop(oracle, hip, n, n_dst, hubs):
     r = np.random.default_rng(n + n_dst)
@@ -86,3 +89,51 @@ def test_index_select_bwd_and_gcn_with_a_hub_equal_the_host_loops(oracle, hip):
                                                      "grad_deg": np.zeros(n_nodes, np.float32)}, ["grad_h", "grad_deg"])
     np.testing.assert_array_equal(got["grad_h"], want["grad_h"])
     np.testing.assert_array_equal(got["grad_deg"], want["grad_deg"])
+
+
+@pytest.mark.parametrize("n", [262143, 262144, 262145, 266241, 300000])
+@pytest.mark.parametrize("n_dst", [1, 255, 256, 257, 65535, 65536, 1 << 20])
+def test_scatter_add_either_side_of_the_radix_build_limits(oracle, hip, n, n_dst):
+    """From 262144 entries on the destination ordering is built by a stable radix sort, 8 bits a pass: one, two and three
+    passes (n_dst up to 255, 65535, beyond), tiles that end inside the input, the shortest input that takes this build and
+    the longest that does not.  Equal to the host's sequential loop bit for bit."""
+    r = np.random.default_rng(n * 31 + n_dst)
+    off = r.integers(0, n_dst, n).astype(np.uint64)
+    src = r.standard_normal(n).astype(np.float32)
+    dst0 = r.standard_normal(n_dst).astype(np.float32)
+    p = {"src": src, "offsets": off, "dst": dst0.copy()}
+    want = run_op(oracle, "scatter_add", p, ["dst"])["dst"]
+    got = run_op(hip, "scatter_add", {**p, "dst": dst0.copy()}, ["dst"])["dst"]
+    np.testing.assert_array_equal(got, want)
+
+
+def test_gcn_scatter_through_the_radix_build_equals_the_host_loops(oracle, hip):
+    """An edge list long enough for the radix build (>= 262144 edges), with hubs: the payload (the other endpoint of an
+    edge) travels with its entry, forward and backward, and the incidence ordering of the degree gradient (2 x edges)."""
+    r = np.random.default_rng(12)
+    n_nodes, n_edge, f = 3000, 280_000, 5
+    tgt = _skewed_offsets(r, n_edge, n_nodes, [(11, 60_000), (5, 300)])
+    src = _skewed_offsets(r, n_edge, n_nodes, [(12, 30_000)])
+    h = r.standard_normal(n_nodes * f).astype(np.float32)
+    deg = r.uniform(0.2, 1.0, n_nodes).astype(np.float32)
+    fw = {"dst": np.zeros(n_nodes * f, np.float32), "h": h, "deg": deg, "src_indices": src, "tgt_indices": tgt,
+          "stride": f, "n_edge": n_edge}
+    want = run_op(oracle, "scatter_gcn_deg_scaled", fw, ["dst"])["dst"]
+    got = run_op(hip, "scatter_gcn_deg_scaled", {**fw, "dst": np.zeros(n_nodes * f, np.float32)}, ["dst"])["dst"]
+    np.testing.assert_array_equal(got, want)
+    bw = {"grad_output": r.standard_normal(n_nodes * f).astype(np.float32), "h": h, "deg": deg, "src_indices": src,
+          "tgt_indices": tgt, "grad_h": np.zeros(n_nodes * f, np.float32), "grad_deg": np.zeros(n_nodes, np.float32),
+          "stride": f, "n_edge": n_edge}
+    want = run_op(oracle, "scatter_gcn_deg_scaled_bwd", bw, ["grad_h", "grad_deg"])
+    got = run_op(hip, "scatter_gcn_deg_scaled_bwd", {**bw, "grad_h": np.zeros(n_nodes * f, np.float32),
+                                                     "grad_deg": np.zeros(n_nodes, np.float32)}, ["grad_h", "grad_deg"])
+    np.testing.assert_array_equal(got["grad_h"], want["grad_h"])
+    np.testing.assert_array_equal(got["grad_deg"], want["grad_deg"])
+    # index_select backward through the same build
+    rows, stride, n_idx = 64, 3, 270_000
+    indices = _skewed_offsets(r, n_idx, rows, [(2, 100_000)])
+    p = {"y_grad": r.standard_normal(n_idx * stride).astype(np.float32), "indices": indices, "stride": stride,
+         "x_grad": r.standard_normal(rows * stride).astype(np.float32)}
+    want = run_op(oracle, "index_select_bwd", {**p, "x_grad": p["x_grad"].copy()}, ["x_grad"])["x_grad"]
+    got = run_op(hip, "index_select_bwd", {**p, "x_grad": p["x_grad"].copy()}, ["x_grad"])["x_grad"]
+    np.testing.assert_array_equal(got, want)

@@ -298,8 +298,14 @@ int flush_deferred_gemm(zg_hip_ctx* ctx);
 inline bool gemm_group_waiting(const zg_hip_ctx* ctx) {
     return ctx->deferred.active || ctx->deferred_w.active || ctx->bias_wait.active;
 }
-// Whether [lo, hi) meets an operand of the waiting products or of the waiting bias gradient.
+// Whether [lo, hi) meets an operand of the waiting products or of the waiting bias gradient (gemm.hip), of the waiting
+// optimizer steps (optim.hip), of the waiting aggregation or degree gradient (index.hip), of the waiting elementwise
+// ops (elementwise.hip): what kind_touches asks, kind by kind.
 bool gemm_group_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
+bool steps_touch(const zg_hip_ctx* ctx, const char* lo, const char* hi);
+bool scatter_wait_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
+bool graddeg_wait_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi);
+bool maps_touch(const zg_hip_ctx* ctx, const char* lo, const char* hi);
 // The single-chunk column sum y += column sums of x[R, inner] (reduce.hip), the launch the waiting bias gradient owes.
 int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, size_t inner, bool fresh);
 // Launches the waiting graph-convolution aggregation with what was attached to it (index.hip); the two hooks are for
@@ -307,16 +313,12 @@ int launch_bias_col_sum(zg_hip_ctx* ctx, const float* x, float* y, size_t R, siz
 int flush_scatter(zg_hip_ctx* ctx);
 // Launches the waiting degree gradient (index.hip).
 int flush_graddeg(zg_hip_ctx* ctx);
-// Launches the waiting elementwise ops as one kernel (elementwise.hip); flush_pending_but_maps: everything else;
-// flush_pending_but_maps_and_fills: everything but the two (no waiting fill ever meets an operand of a waiting
-// elementwise op, so the two kinds may leave in either order).
+// Launches the waiting elementwise ops as one kernel (elementwise.hip).
 int flush_maps(zg_hip_ctx* ctx);
 // Queues out[i] = c added to +0.0 (row_ptr[i + 1] - row_ptr[i]) times, i < n, with the waiting elementwise ops: what
 // scatter_add of a constant source into a destination of zeros comes to once the offsets are sorted into buckets
 // (index.hip).  False: not queued (*rc says whether something failed), the caller launches its own kernel.
 bool maps_push_count(zg_hip_ctx* ctx, float* out, const uint32_t* row_ptr, size_t n, float c, int* rc);
-int flush_pending_but_maps(zg_hip_ctx* ctx);
-int flush_pending_but_maps_and_fills(zg_hip_ctx* ctx);
 // Whether a waiting fill meets one of the byte ranges; take_fill_exact: a waiting fill of exactly x[0 .. n) is dropped
 // and its value handed over (the caller overwrites all of the range and uses the value where it would have read it);
 // drop_fills_inside: waiting fills that lie wholly inside a range the caller overwrites without reading it.
@@ -335,10 +337,44 @@ bool scatter_take_relu(zg_hip_ctx* ctx, const float* x, const float* y, size_t n
 int flush_steps(zg_hip_ctx* ctx, bool requeue_fills = false);
 // Returns to the pools the blocks whose free waited for the product (runtime.hip); called once it is launched.
 void run_deferred_frees(zg_hip_ctx* ctx);
-// The waiting product, then the waiting fills: what ZG_CTX does before a call's own work.
-int flush_pending(zg_hip_ctx* ctx);
-// The same except that waiting fills stay waiting unless one of them meets one of the `count` byte ranges the caller
-// is about to read or write (runtime.hip).
+// ------------------------------------------------------------------------------------------------
+// The one mechanism behind every kind of waiting work.  A kind is a bit; for each kind the context can say whether
+// work of that kind waits (waiting_kinds), launch it (flush_kinds, always in the order maps, aggregation, degree
+// gradient, products, fills, steps: kinds that wait at the same time touch disjoint memory, so any fixed order does),
+// and tell whether it would read or write a byte range (kind_touches).  An entry point starts with
+// ZG_ENTER(ctx, keep): everything that waits is launched except the kinds in `keep`, which the entry point looks at
+// itself (to join them, to take them over, or to launch them only if they meet its operands: flush_touching).
+// ------------------------------------------------------------------------------------------------
+enum : unsigned {
+    kWaitFills = 1u,     // float fills (runtime.hip)
+    kWaitProducts = 2u,  // a layer's forward or input-gradient product, the weight-gradient product and the bias
+                         // gradient that wait with it (gemm.hip)
+    kWaitSteps = 4u,     // optimizer steps (optim.hip)
+    kWaitScatter = 8u,   // a graph-convolution aggregation (index.hip)
+    kWaitGradDeg = 16u,  // a degree gradient (index.hip)
+    kWaitMaps = 32u,     // small elementwise ops (elementwise.hip)
+    kWaitAll = 63u,
+};
+struct ByteSpan {
+    const void* p;
+    size_t bytes;
+};
+inline unsigned waiting_kinds(const zg_hip_ctx* ctx) {
+    return (ctx->n_pending_fills ? kWaitFills : 0u) |
+           ((ctx->deferred.active || ctx->deferred_w.active || ctx->bias_wait.active) ? kWaitProducts : 0u) |
+           (ctx->steps.count ? kWaitSteps : 0u) | (ctx->scatter_wait.active ? kWaitScatter : 0u) |
+           (ctx->graddeg_wait.active ? kWaitGradDeg : 0u) | (ctx->maps.count ? kWaitMaps : 0u);
+}
+// Launches what waits of the given kinds (runtime.hip).
+int flush_kinds(zg_hip_ctx* ctx, unsigned kinds);
+// Whether waiting work of one kind reads or writes any byte of the spans (null spans are skipped).
+bool kind_touches(const zg_hip_ctx* ctx, unsigned kind, const ByteSpan* spans, int count);
+// Of the given kinds, launches those whose waiting work meets the spans; the others keep waiting.
+int flush_touching(zg_hip_ctx* ctx, unsigned kinds, const ByteSpan* spans, int count);
+// Everything that waits: what a call that knows nothing about waiting work starts with.
+inline int flush_pending(zg_hip_ctx* ctx) { return flush_kinds(ctx, kWaitAll); }
+// Everything but the fills, and the fills too when one of them meets one of the `count` byte ranges the caller is about
+// to read or write.
 int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count);
 // A call that may be absorbed by the waiting product: true when it was (then *rc is the call's result and the caller
 // returns it), false when the call has to run as usual.
@@ -351,10 +387,7 @@ bool deferred_take_relu_mask(zg_hip_ctx* ctx, const float* x, const float* x_g, 
 // fill's launch and without the read.
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n);
 
-inline bool anything_waits(const zg_hip_ctx* ctx) {
-    return ctx->n_pending_fills || ctx->deferred.active || ctx->deferred_w.active || ctx->bias_wait.active ||
-           ctx->steps.count || ctx->scatter_wait.active || ctx->graddeg_wait.active || ctx->maps.count;
-}
+inline bool anything_waits(const zg_hip_ctx* ctx) { return waiting_kinds(ctx) != 0u; }
 // Lives for the length of an entry point (the ZG_CTX* macros declare one): with holding switched off, whatever the
 // call queued is launched before the call returns.
 struct HoldGuard {
@@ -421,7 +454,8 @@ inline bool aligned16(const void* p) {
         }                                                                                        \
     } while (0)
 
-// First statement of every entry point: a context, and no fill still waiting when the call's own work is queued.
+// What ZG_ENTER starts with: a context, the guard for contexts that hold nothing, and the error that launching held
+// work at the end of an earlier call left behind.
 #define ZG_CTX_ENTER(ctx)                                    \
     ZG_REQUIRE((ctx) != nullptr, "null context");            \
     zg::HoldGuard _zg_hold_guard{(ctx)};                     \
@@ -431,39 +465,15 @@ inline bool aligned16(const void* p) {
         (ctx)->late_error = 0;                               \
         return _rc_late;                                     \
     }
-#define ZG_CTX(ctx)                                          \
-    ZG_CTX_ENTER(ctx)                                        \
-    if ((ctx)->n_pending_fills || (ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || \
-        (ctx)->scatter_wait.active || (ctx)->graddeg_wait.active || (ctx)->maps.count) { \
-        if (int _rc_fill = zg::flush_pending(ctx)) return _rc_fill; \
+// First statement of every entry point.  `keep`: the kinds of waiting work (kWait* bits) the entry point deals with
+// itself; everything else that waits is launched before the call's own work is queued, so no call can observe memory
+// that waiting work has not reached.  ZG_CTX is the common case: the entry point knows nothing of waiting work.
+#define ZG_ENTER(ctx, keep)                                                                    \
+    ZG_CTX_ENTER(ctx)                                                                          \
+    if (const unsigned _zg_w = zg::waiting_kinds(ctx) & ~(unsigned)(keep)) {                   \
+        if (int _rc_w = zg::flush_kinds(ctx, _zg_w)) return _rc_w;                             \
     }
-// The same for the few calls that decide themselves what happens to waiting work: the fills, the products and the
-// calls a product may absorb.
-// A waiting aggregation only waits for the add and the ReLU, which look at it before they get here: it goes out.
-#define ZG_CTX_KEEP_FILLS(ctx)                                   \
-    ZG_CTX_ENTER(ctx)                                            \
-    if ((ctx)->scatter_wait.active) {                            \
-        if (int _rc_sc = zg::flush_scatter(ctx)) return _rc_sc;  \
-    }                                                            \
-    if ((ctx)->graddeg_wait.active) {                            \
-        if (int _rc_gd = zg::flush_graddeg(ctx)) return _rc_gd;  \
-    }                                                            \
-    if ((ctx)->maps.count) {                                     \
-        if (int _rc_mp = zg::flush_maps(ctx)) return _rc_mp;     \
-    }
-// The small elementwise ops: the waiting elementwise ops stay (the call joins them or sends them out itself) and so do
-// the waiting fills (the call sends them out if one meets its operands, or takes over the one that covers its output);
-// everything else that waits goes out.
-#define ZG_CTX_KEEP_MAPS(ctx)                                    \
-    ZG_CTX_ENTER(ctx)                                            \
-    if ((ctx)->deferred.active || (ctx)->bias_wait.active || (ctx)->steps.count || (ctx)->scatter_wait.active || \
-        (ctx)->graddeg_wait.active) {                            \
-        if (int _rc_km = zg::flush_pending_but_maps_and_fills(ctx)) return _rc_km; \
-    }
-// The cache's allocations and frees look at each kind of waiting work themselves: a block that is handed out is free,
-// so nothing that waits names it; a block that is given back may be the one a waiting degree gradient would write, or
-// hold operands of waiting elementwise ops, which the pool's memory outlives.
-#define ZG_CTX_KEEP_ALL(ctx) ZG_CTX_ENTER(ctx)
+#define ZG_CTX(ctx) ZG_ENTER(ctx, 0u)
 
 // Entry points that synchronise, allocate from the driver or touch host memory cannot be recorded into a graph.
 #define ZG_NOT_CAPTURING(ctx, who)                                                                       \

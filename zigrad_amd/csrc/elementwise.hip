@@ -88,14 +88,10 @@ static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* ou
 // one of them meets an operand (lengths in floats; null operands are skipped).
 static int settle_before_launch(zg_hip_ctx* ctx, const float* out, size_t n_out, const float* a, size_t n_a,
                                 const float* b, size_t n_b, const float* c, size_t n_c) {
-    if (ctx->maps.count)
-        if (int rc = flush_maps(ctx)) return rc;
-    if (ctx->n_pending_fills) {
-        const void* ptrs[4] = {out, a, b, c};
-        const size_t bytes[4] = {n_out * sizeof(float), n_a * sizeof(float), n_b * sizeof(float), n_c * sizeof(float)};
-        if (fills_touch(ctx, ptrs, bytes, 4)) return flush_fills(ctx);
-    }
-    return ZG_HIP_OK;
+    if (int rc = flush_kinds(ctx, kWaitMaps)) return rc;
+    const ByteSpan spans[4] = {{out, n_out * sizeof(float)}, {a, n_a * sizeof(float)}, {b, n_b * sizeof(float)},
+                               {c, n_c * sizeof(float)}};
+    return flush_touching(ctx, kWaitFills, spans, 4);
 }
 
 template <class Op, int NIN>
@@ -221,7 +217,7 @@ __global__ void broadcast_modulo_kernel(float* y, const float* x, size_t xl, siz
 template <class B>
 static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t xl, const float* y, size_t yl, float* z,
                      size_t zl) {
-    ZG_CTX_KEEP_MAPS(ctx);
+    ZG_ENTER(ctx, kWaitMaps | kWaitFills);
     ZG_REQUIRE(xl > 0 && yl > 0 && zl > 0, "%s: empty operand", name);
     ZG_REQUIRE(x && y && z, "%s: null pointer", name);
     const size_t mx = xl > yl ? xl : yl, mn = xl < yl ? xl : yl;
@@ -420,6 +416,17 @@ static int map_op_ranges(const zg_map_op& o, size_t n, MapRange* r) {  // r[0] i
     return m;
 }
 
+bool maps_touch(const zg_hip_ctx* ctx, const char* lo, const char* hi) {
+    const zg_waiting_maps& q = ctx->maps;
+    for (int k = 0; k < q.count; k++) {
+        MapRange r[4];
+        const int m = map_op_ranges(q.op[k], q.n, r);
+        for (int j = 0; j < m; j++)
+            if (r[j].lo < hi && lo < r[j].hi) return true;
+    }
+    return false;
+}
+
 static bool chain_push(zg_hip_ctx* ctx, int code, int nin, int scalar, float* out, const float* a, const float* b,
                        const float* c, size_t n, float p0, float p1, int* rc) {
     *rc = ZG_HIP_OK;
@@ -476,7 +483,7 @@ bool maps_push_count(zg_hip_ctx* ctx, float* out, const uint32_t* row_ptr, size_
 using namespace zg;
 
 #define ZG_CHECK_N(name, n, ...)                                         \
-    ZG_CTX_KEEP_MAPS(ctx);                                               \
+    ZG_ENTER(ctx, kWaitMaps | kWaitFills);                                               \
     if ((n) == 0) return ZG_HIP_OK;                                      \
     {                                                                    \
         const void* _ptrs[] = {__VA_ARGS__};                             \

@@ -1768,7 +1768,7 @@ static int gemm_entry(zg_hip_ctx* ctx, const char* name, const float* A, const f
 
 ZG_API int zg_hip_matmul(zg_hip_ctx* ctx, const float* A, const float* B, float* C, size_t m, size_t n, size_t k,
                          int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     return gemm_entry(ctx, "matmul", A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, 1, 1, 1, 0, 0, 0);
 }
 
@@ -1835,7 +1835,7 @@ ZG_API int zg_hip_linear_bwd(zg_hip_ctx* ctx, const float* gy, const float* x, c
 ZG_API int zg_hip_bmm_acc(zg_hip_ctx* ctx, const float* A, const uint64_t* A_shape, const float* B,
                           const uint64_t* B_shape, float* C, const uint64_t* C_shape, int trans_a, int trans_b,
                           size_t lda, size_t ldb, size_t ldc, float alpha, float beta) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     ZG_REQUIRE(A_shape && B_shape && C_shape, "bmm_acc: null shape");
     const size_t nba = A_shape[0], nbb = B_shape[0], nbc = C_shape[0];
     const size_t m = C_shape[1], n = C_shape[2], k = A_shape[2];

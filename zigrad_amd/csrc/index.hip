@@ -1292,7 +1292,7 @@ ZG_API int zg_hip_gather(zg_hip_ctx* ctx, const float* src, const uint64_t* src_
 
 ZG_API int zg_hip_scatter_add(zg_hip_ctx* ctx, const float* src, const uint64_t* offsets, size_t n, float* dst,
                               size_t dst_len) {
-    ZG_CTX_KEEP_ALL(ctx);
+    ZG_ENTER(ctx, kWaitAll);
     const bool args_ok = n == 0 || (src && offsets && dst && dst_len > 0 && n < 0xffffffffull && dst_len < 0xffffffffull);
     if (n == 0 || !args_ok) {
         if (int rc = flush_pending(ctx)) return rc;
@@ -1409,6 +1409,26 @@ ZG_API int zg_hip_index_select_bwd(zg_hip_ctx* ctx, const float* y_grad, const u
 }
 
 namespace zg {
+static bool span_meets(const void* p, size_t bytes, const char* lo, const char* hi) {
+    return p && (const char*)p < hi && lo < (const char*)p + bytes;
+}
+// (the orderings and term arrays of both live in plan memory that no caller can name)
+bool scatter_wait_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi) {
+    const zg_waiting_scatter& w = ctx->scatter_wait;
+    if (!w.active) return false;
+    const size_t n = w.n_nodes * w.stride * sizeof(float);
+    return span_meets(w.dst, n, lo, hi) || span_meets(w.h, n, lo, hi) || span_meets(w.deg, w.n_nodes * sizeof(float), lo, hi) ||
+           span_meets(w.bias, w.stride * sizeof(float), lo, hi);
+}
+bool graddeg_wait_touches(const zg_hip_ctx* ctx, const char* lo, const char* hi) {
+    const zg_waiting_graddeg& w = ctx->graddeg_wait;
+    if (!w.active) return false;
+    const size_t n = w.n_nodes * w.stride * sizeof(float);
+    return span_meets(w.grad_output, n, lo, hi) || span_meets(w.h, n, lo, hi) ||
+           span_meets(w.deg, w.n_nodes * sizeof(float), lo, hi) || span_meets(w.grad_deg, w.n_nodes * sizeof(float), lo, hi) ||
+           span_meets(w.src_idx, w.n_edge * sizeof(uint64_t), lo, hi) || span_meets(w.tgt_idx, w.n_edge * sizeof(uint64_t), lo, hi);
+}
+
 int flush_scatter(zg_hip_ctx* ctx) {
     const zg_waiting_scatter w = ctx->scatter_wait;
     if (!w.active) return ZG_HIP_OK;
@@ -1480,7 +1500,7 @@ static int check_gcn(const char* name, size_t stride, size_t n_edge, size_t n_no
 ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const float* h, const float* deg,
                                          const uint64_t* src_indices, const uint64_t* tgt_indices, size_t stride,
                                          size_t n_edge, size_t n_nodes) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     // the output's zero fill (the layer allocates it zeroed, examples/gcn/src/model.zig:100-112) may still be waiting:
     // then the sums are written instead of added to zeros
     const bool fresh = n_edge > 0 && dst && stride > 0 && n_nodes > 0 && absorb_zero_fill(ctx, dst, n_nodes * stride);
@@ -1524,7 +1544,7 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
                                              const float* deg, const uint64_t* src_indices,
                                              const uint64_t* tgt_indices, float* grad_h, float* grad_deg, size_t stride,
                                              size_t n_edge, size_t n_nodes) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     // the zero fills of the two gradients (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: a gradient
     // whose fill is taken over is written instead of added to zeros
     const bool sized = n_edge > 0 && stride > 0 && n_nodes > 0;

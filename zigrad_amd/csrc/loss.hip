@@ -742,7 +742,7 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
 
 ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* target, float* grad, size_t rows,
                            size_t cols) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     ZG_REQUIRE(probs && target && grad, "smce_bwd: null pointer");
     if (int rc = check_rows("smce_bwd", rows, cols)) return rc;
     // the gradient's zero fill (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: then write, not add

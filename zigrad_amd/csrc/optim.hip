@@ -324,6 +324,17 @@ static int launch_steps(zg_hip_ctx* ctx, const zg_pending_steps& q, int zero_gra
                       q.lr, q.b1, q.b2, q.eps, q.clip, q.max_norm, q.delta, zero_grads);
 }
 
+bool steps_touch(const zg_hip_ctx* ctx, const char* lo, const char* hi) {
+    const zg_pending_steps& q = ctx->steps;
+    for (int i = 0; i < q.count; i++) {
+        const float* arrays[4] = {q.p[i], q.g[i], q.m[i], q.v[i]};
+        for (const float* a : arrays)
+            if (a && (const char*)a < hi && lo < (const char*)(a + q.n[i])) return true;
+        if (q.kind == 2 && q.lr_t_mem[i] && (const char*)q.lr_t_mem[i] < hi && lo < (const char*)(q.lr_t_mem[i] + 1)) return true;
+    }
+    return false;
+}
+
 int flush_steps(zg_hip_ctx* ctx, bool requeue_fills) {
     const zg_pending_steps q = ctx->steps;
     ctx->steps.count = 0;
@@ -399,7 +410,7 @@ static int step_entry(zg_hip_ctx* ctx, int kind, float* param, float* grad, floa
 
 ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n, float lr, int clip, float max_norm,
                            float delta) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad, "sgd_step: null pointer");
     return step_entry(ctx, 0, param, grad, nullptr, nullptr, n, lr, 0.f, nullptr, 0.f, 0.f, 0.f, clip, max_norm, delta);
@@ -407,7 +418,7 @@ ZG_API int zg_hip_sgd_step(zg_hip_ctx* ctx, float* param, float* grad, size_t n,
 
 ZG_API int zg_hip_adam_step(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n, uint64_t t,
                             float lr, float beta1, float beta2, float epsilon, int clip, float max_norm, float delta) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad && m && v, "adam_step: null pointer");
     ZG_REQUIRE(t >= 1, "adam_step: t must be >= 1");
@@ -424,7 +435,7 @@ ZG_API int zg_hip_adam_lr_t(float lr, float beta1, float beta2, uint64_t t, floa
 ZG_API int zg_hip_adam_step_at(zg_hip_ctx* ctx, float* param, float* grad, float* m, float* v, size_t n,
                                const float* lr_t, float beta1, float beta2, float epsilon, int clip, float max_norm,
                                float delta) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(param && grad && m && v && lr_t, "adam_step_at: null pointer");
     return step_entry(ctx, 2, param, grad, m, v, n, 0.f, 0.f, lr_t, beta1, beta2, epsilon, clip, max_norm, delta);

@@ -397,7 +397,7 @@ ZG_API int zg_hip_sum_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_s
 
 ZG_API int zg_hip_max_along(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape, size_t x_rank, float* y,
                             size_t y_len, size_t dim) {
-    ZG_CTX_KEEP_ALL(ctx);
+    ZG_ENTER(ctx, kWaitAll);
     int rc = check_axis_args("max_along", x, x_shape, x_rank, y, y_len, dim);
     if (rc == ZG_HIP_OK && y_len != prod(x_shape, 0, x_rank) / x_shape[dim]) {
         set_error("max_along: y.len %zu != %zu", y_len, prod(x_shape, 0, x_rank) / (size_t)x_shape[dim]);
@@ -478,7 +478,7 @@ __global__ __launch_bounds__(kBlock) void scaled_copy_kernel(const float* x, flo
 ZG_API int zg_hip_unbroadcast(zg_hip_ctx* ctx, const float* x, const uint64_t* x_shape_in, size_t x_rank_in, float* y,
                               const uint64_t* y_shape_in, size_t y_rank_in, float* scratch, size_t scratch_len,
                               float alpha, float beta) {
-    ZG_CTX_KEEP_ALL(ctx);
+    ZG_ENTER(ctx, kWaitAll);
     // what waits goes out before this call's first launch (below); a refused call sends it out too
     struct Settle {
         zg_hip_ctx* ctx;

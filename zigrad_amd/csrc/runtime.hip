@@ -878,7 +878,7 @@ ZG_API int zg_hip_cache_configure(zg_hip_ctx* ctx, size_t small_pool_bytes, size
 }
 
 ZG_API int zg_hip_mem_cache_alloc(zg_hip_ctx* ctx, size_t bytes, void** out, uint64_t* block) {
-    ZG_CTX_KEEP_ALL(ctx);
+    ZG_ENTER(ctx, kWaitAll);
     // waiting fills stay (a block that is handed out is free, so no waiting fill names it), and so do waiting
     // elementwise ops: a new block holds no operand of theirs, and a caller allocates each op's output just before it
     if (ctx->scatter_wait.active)
@@ -932,7 +932,7 @@ void run_deferred_frees(zg_hip_ctx* ctx) {
 }  // namespace zg
 
 ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
-    ZG_CTX_KEEP_ALL(ctx);
+    ZG_ENTER(ctx, kWaitAll);
     // Waiting elementwise ops stay: the pool keeps the block's memory, so they may still read and write it when they
     // are launched, and whoever receives the block next either joins them (in call order, element by element) or sends
     // them out first.
@@ -1018,7 +1018,7 @@ ZG_API int zg_hip_mem_cache_free(zg_hip_ctx* ctx, void* ptr, uint64_t block) {
 // what a binding needs to tell a device slice from a host scalar (the reference's callers pass both through the
 // same parameter: src/ndarray.zig:251, src/nn/optim.zig:117 against src/ndtensor.zig:1146-1150).
 ZG_API int zg_hip_is_device_ptr(zg_hip_ctx* ctx, const void* ptr, int* yes) {
-    ZG_CTX_KEEP_ALL(ctx);  // a lookup in host tables: a binding asks before every op with a one-float operand
+    ZG_ENTER(ctx, kWaitAll);  // a lookup in host tables: a binding asks before every op with a one-float operand
     ZG_REQUIRE(yes != nullptr, "is_device_ptr: null output");
     *yes = 0;
     if (!ptr) return ZG_HIP_OK;
@@ -1101,7 +1101,7 @@ ZG_API int zg_hip_launch_count(zg_hip_ctx* ctx, uint64_t* launches) {
 }
 
 ZG_API int zg_hip_cache_stats(zg_hip_ctx* ctx, size_t* bytes_in_use, size_t* bytes_mapped, uint64_t* n_device_allocs) {
-    ZG_CTX_KEEP_ALL(ctx);  // host counters only: what waits keeps waiting
+    ZG_ENTER(ctx, kWaitAll);  // host counters only: what waits keeps waiting
     size_t u = 0, m = 0;
     for (BlockPool* p : {ctx->small_pool, ctx->large_pool}) {
         if (p) {
@@ -1156,7 +1156,7 @@ ZG_API int zg_hip_memcpy_d2h(zg_hip_ctx* ctx, void* dst_host, const void* src, s
 }
 
 ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t bytes) {
-    ZG_CTX_KEEP_ALL(ctx);
+    ZG_ENTER(ctx, kWaitAll);
     if (bytes == 0 || !dst || !src) {
         if (int rc = flush_pending(ctx)) return rc;
         if (bytes == 0) return ZG_HIP_OK;
@@ -1275,43 +1275,61 @@ int flush_fills(zg_hip_ctx* ctx) {
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
-int flush_pending(zg_hip_ctx* ctx) {
+int flush_kinds(zg_hip_ctx* ctx, unsigned kinds) {
     // Work of different kinds that waits at the same time touches disjoint memory (each kind's calls send out whatever
-    // meets their operands before they queue), so the kinds may leave in any order.
-    if (ctx->maps.count)
+    // meets their operands before they queue), so the kinds may leave in any order; this one is fixed.
+    if ((kinds & kWaitMaps) && ctx->maps.count)
         if (int rc = flush_maps(ctx)) return rc;
-    return flush_pending_but_maps(ctx);
-}
-int flush_pending_but_maps(zg_hip_ctx* ctx) {
-    if (ctx->scatter_wait.active)
+    if ((kinds & kWaitScatter) && ctx->scatter_wait.active)
         if (int rc = flush_scatter(ctx)) return rc;
-    if (ctx->graddeg_wait.active)
+    if ((kinds & kWaitGradDeg) && ctx->graddeg_wait.active)
         if (int rc = flush_graddeg(ctx)) return rc;
-    if (gemm_group_waiting(ctx))
+    if ((kinds & kWaitProducts) && gemm_group_waiting(ctx))
         if (int rc = flush_deferred_gemm(ctx)) return rc;
-    if (int rc = flush_fills(ctx)) return rc;
-    return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
+    if ((kinds & kWaitFills) && ctx->n_pending_fills)
+        if (int rc = flush_fills(ctx)) return rc;
+    if ((kinds & kWaitSteps) && ctx->steps.count)
+        if (int rc = flush_steps(ctx)) return rc;
+    return ZG_HIP_OK;
 }
-int flush_pending_but_maps_and_fills(zg_hip_ctx* ctx) {
-    if (ctx->scatter_wait.active)
-        if (int rc = flush_scatter(ctx)) return rc;
-    if (ctx->graddeg_wait.active)
-        if (int rc = flush_graddeg(ctx)) return rc;
-    if (gemm_group_waiting(ctx))
-        if (int rc = flush_deferred_gemm(ctx)) return rc;
-    return ctx->steps.count ? flush_steps(ctx) : ZG_HIP_OK;
+
+bool kind_touches(const zg_hip_ctx* ctx, unsigned kind, const ByteSpan* spans, int count) {
+    for (int j = 0; j < count; j++) {
+        const char* lo = (const char*)spans[j].p;
+        if (!lo || spans[j].bytes == 0) continue;
+        const char* hi = lo + spans[j].bytes;
+        bool hit = false;
+        switch (kind) {
+            case kWaitFills:
+                for (int i = 0; i < ctx->n_pending_fills && !hit; i++) {
+                    const char* x0 = (const char*)ctx->pending_fills[i].x;
+                    hit = x0 < hi && lo < x0 + ctx->pending_fills[i].n * sizeof(float);
+                }
+                break;
+            case kWaitProducts: hit = gemm_group_waiting(ctx) && gemm_group_touches(ctx, lo, hi); break;
+            case kWaitSteps: hit = steps_touch(ctx, lo, hi); break;
+            case kWaitScatter: hit = scatter_wait_touches(ctx, lo, hi); break;
+            case kWaitGradDeg: hit = graddeg_wait_touches(ctx, lo, hi); break;
+            case kWaitMaps: hit = maps_touch(ctx, lo, hi); break;
+            default: break;
+        }
+        if (hit) return true;
+    }
+    return false;
+}
+
+int flush_touching(zg_hip_ctx* ctx, unsigned kinds, const ByteSpan* spans, int count) {
+    unsigned hit = 0;
+    for (unsigned kind = 1; kind <= kWaitMaps; kind <<= 1)
+        if ((kinds & kind) && (waiting_kinds(ctx) & kind) && kind_touches(ctx, kind, spans, count)) hit |= kind;
+    return hit ? flush_kinds(ctx, hit) : ZG_HIP_OK;
 }
 
 bool fills_touch(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
-    for (int i = 0; i < ctx->n_pending_fills; i++) {
-        const char* x0 = (const char*)ctx->pending_fills[i].x;
-        const char* x1 = x0 + ctx->pending_fills[i].n * sizeof(float);
-        for (int j = 0; j < count; j++) {
-            const char* p0 = (const char*)ptrs[j];
-            if (p0 && x0 < p0 + bytes[j] && p0 < x1) return true;
-        }
-    }
-    return false;
+    ByteSpan spans[8];
+    const int n = count < 8 ? count : 8;
+    for (int j = 0; j < n; j++) spans[j] = ByteSpan{ptrs[j], bytes[j]};
+    return kind_touches(ctx, kWaitFills, spans, n);
 }
 bool take_fill_exact(zg_hip_ctx* ctx, const float* x, size_t n, float* value) {
     for (int i = 0; i < ctx->n_pending_fills; i++) {
@@ -1345,17 +1363,11 @@ void requeue_fills(zg_hip_ctx* ctx, const zg_pending_fill* fills, int count) {
 }
 
 int flush_pending_but_fills(zg_hip_ctx* ctx, const void* const* ptrs, const size_t* bytes, int count) {
-    if (ctx->maps.count)
-        if (int rc = flush_maps(ctx)) return rc;
-    if (ctx->scatter_wait.active)
-        if (int rc = flush_scatter(ctx)) return rc;
-    if (ctx->graddeg_wait.active)
-        if (int rc = flush_graddeg(ctx)) return rc;
-    if (gemm_group_waiting(ctx))
-        if (int rc = flush_deferred_gemm(ctx)) return rc;
-    if (ctx->steps.count)
-        if (int rc = flush_steps(ctx)) return rc;
-    return fills_touch(ctx, ptrs, bytes, count) ? flush_fills(ctx) : ZG_HIP_OK;
+    if (int rc = flush_kinds(ctx, kWaitAll & ~kWaitFills)) return rc;
+    ByteSpan spans[8];
+    const int n = count < 8 ? count : 8;
+    for (int j = 0; j < n; j++) spans[j] = ByteSpan{ptrs[j], bytes[j]};
+    return flush_touching(ctx, kWaitFills, spans, n);
 }
 
 bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
@@ -1374,12 +1386,15 @@ bool absorb_zero_fill(zg_hip_ctx* ctx, const float* x, size_t n) {
 }  // namespace zg
 
 ZG_API int zg_hip_mem_fill(zg_hip_ctx* ctx, float* x, size_t n, float value) {
-    ZG_CTX_KEEP_FILLS(ctx);
+    ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
     // a waiting product goes first: the fill may be of one of its operands; a bias gradient that waits alone stays
     // unless the fill meets what it reads or writes (the zero fill of the layer's input gradient comes next)
-    if (ctx->deferred.active ||
-        (x && n && gemm_group_waiting(ctx) && gemm_group_touches(ctx, (const char*)x, (const char*)(x + n))))
-        if (int rc = flush_deferred_gemm(ctx)) return rc;
+    if (ctx->deferred.active) {
+        if (int rc = flush_kinds(ctx, kWaitProducts)) return rc;
+    } else if (x && n) {
+        const ByteSpan span{x, n * sizeof(float)};
+        if (int rc = flush_touching(ctx, kWaitProducts, &span, 1)) return rc;
+    }
     if (ctx->steps.count) {
         // zero_grad() after step() (examples/mnist/src/model.zig:57-62): a zero fill of exactly the gradient of a waiting
         // step is taken over by the step, whose kernel stores the zeros once it has read the gradient; any other fill

@@ -419,18 +419,26 @@ __global__ __launch_bounds__(kRxBins * kRxScanParts) void rx_scan_kernel(uint32_
 }
 
 // Entry e of a tile belongs to round r = (e / 256) and wave w: "wave-round" q = 4 r + w, lanes in input order, so
-// (q, lane) ascending is input order.  Rank of an entry = entries of its digit in earlier wave-rounds of the tile (a
-// prefix over q of table[q][digit]) + entries of its digit in lower lanes of its own wave-round (ballots).
+// (q, lane) ascending is input order.  Rank of an entry among the tile's entries of its digit = entries of its digit in
+// earlier wave-rounds (a prefix over q of table[q][digit]) + entries of its digit in lower lanes of its own wave-round
+// (ballots).  The tile is then put in digit order in LDS and written out from there, so that the lanes of a store
+// instruction write runs of consecutive addresses (one run per digit present) instead of 64 scattered words.
 __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* __restrict__ keys_in,
                                                                 const uint32_t* __restrict__ vals_in, size_t n, int shift,
                                                                 const uint32_t* __restrict__ starts,
                                                                 uint32_t* __restrict__ keys_out,
                                                                 uint32_t* __restrict__ vals_out) {
     constexpr int Q = kRxPerThread * (kRxThreads / 64);
-    __shared__ uint16_t table[Q][kRxBins];
-    __shared__ uint32_t first[kRxBins];
+    // the ranking table, then (once every entry knows its place) the tile in digit order: keys, then values
+    __shared__ __align__(16) uint32_t lds[Q * kRxBins / 2];
+    static_assert(sizeof(lds) == 2 * kRxTile * sizeof(uint32_t), "the sorted tile reuses the table's memory");
+    uint16_t(*table)[kRxBins] = reinterpret_cast<uint16_t(*)[kRxBins]>(lds);
+    __shared__ uint32_t first[kRxBins];       // where the tile's entries of a digit go in the output
+    __shared__ uint32_t tile_start[kRxBins];  // where they start in the sorted tile
+    __shared__ uint32_t wave_tot[kRxThreads / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t base = (size_t)blockIdx.x * kRxTile;
+    const uint32_t in_tile = (uint32_t)((n - base < (size_t)kRxTile) ? n - base : (size_t)kRxTile);
     uint32_t key[kRxPerThread], val[kRxPerThread];
     uint16_t rank[kRxPerThread];
 #pragma unroll
@@ -440,7 +448,7 @@ __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* 
         val[r] = (e < n && vals_in) ? vals_in[e] : (uint32_t)e;
     }
     const uint32_t my_first = starts[(size_t)blockIdx.x * kRxBins + threadIdx.x];
-    for (int i = threadIdx.x; i < Q * kRxBins / 2; i += kRxThreads) reinterpret_cast<uint32_t*>(&table[0][0])[i] = 0;
+    for (int i = threadIdx.x; i < Q * kRxBins / 2; i += kRxThreads) lds[i] = 0;
     first[threadIdx.x] = my_first;
     __syncthreads();
 #pragma unroll
@@ -460,7 +468,7 @@ __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* 
         if (live && below == 0) table[r * (kRxThreads / 64) + wave][digit] = (uint16_t)__popcll(peers);
     }
     __syncthreads();
-    {  // thread d: exclusive prefix over the wave-rounds of digit d
+    {  // thread d: exclusive prefix over the wave-rounds of digit d, then over the digits of the tile
         const int d = threadIdx.x;
         uint16_t c[Q];
 #pragma unroll
@@ -471,16 +479,46 @@ __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* 
             table[q][d] = (uint16_t)run;
             run += c[q];
         }
+        uint32_t inc = run;
+#pragma unroll
+        for (int s = 1; s < 64; s <<= 1) {
+            const uint32_t v = __shfl_up(inc, s, 64);
+            if (lane >= s) inc += v;
+        }
+        if (lane == 63) wave_tot[wave] = inc;
+        __syncthreads();
+        uint32_t start = inc - run;
+        for (int w = 0; w < wave; w++) start += wave_tot[w];
+        tile_start[d] = start;
     }
     __syncthreads();
+    uint32_t place[kRxPerThread];
+#pragma unroll
+    for (int r = 0; r < kRxPerThread; r++) {
+        const uint32_t digit = (key[r] >> shift) & (kRxBins - 1);
+        place[r] = tile_start[digit] + table[r * (kRxThreads / 64) + wave][digit] + rank[r];
+    }
+    __syncthreads();  // the table has been read by everyone: its memory now takes the sorted tile
+    uint32_t* skey = lds;
+    uint32_t* sval = lds + kRxTile;
 #pragma unroll
     for (int r = 0; r < kRxPerThread; r++) {
         const size_t e = base + (size_t)r * kRxThreads + threadIdx.x;
         if (e < n) {
-            const uint32_t digit = (key[r] >> shift) & (kRxBins - 1);
-            const uint32_t pos = first[digit] + table[r * (kRxThreads / 64) + wave][digit] + rank[r];
-            keys_out[pos] = key[r];
-            vals_out[pos] = val[r];
+            skey[place[r]] = key[r];
+            sval[place[r]] = val[r];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kRxPerThread; r++) {
+        const uint32_t j = (uint32_t)r * kRxThreads + threadIdx.x;
+        if (j < in_tile) {
+            const uint32_t k = skey[j];
+            const uint32_t digit = (k >> shift) & (kRxBins - 1);
+            const uint32_t pos = first[digit] + (j - tile_start[digit]);
+            keys_out[pos] = k;
+            vals_out[pos] = sval[j];
         }
     }
 }

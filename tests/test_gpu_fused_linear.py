@@ -270,7 +270,9 @@ def test_fused_gcn_step_with_an_edge_plan_replays_from_an_execution_graph(hip):
 
 
 @pytest.mark.parametrize("rows,cols", [(64, 10), (140, 7), (256, 32), (257, 32), (1, 1), (64, 256), (65, 256), (16, 4096),
-                                       (17, 4096), (3, 1000), (5, 33), (700, 1024), (2, 5000)])
+                                       (17, 4096), (3, 1000), (5, 33), (700, 1024), (2, 5000),
+                                       # one pass over rows held in registers: a wave per row, a workgroup per row
+                                       (1024, 1024), (1500, 260), (1100, 1000), (3, 8192), (2, 32768), (5, 4100)])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_smce_fwd_bwd_equals_forward_then_backward(oracle, hip, rows, cols, accumulate):
     """One call against smce_fwd + smce_bwd (src/nn/loss.zig:130-159) on the same device, bit for bit, on both sides

@@ -276,10 +276,13 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* logit
 // MODE 1 reads the target row as well; its loads are issued before the reduction so they are in flight under it.
 constexpr int kLongRowThreads = 1024;
 constexpr int kLongRowVec = 8;
-template <int MODE>
+// GRAD (with MODE 1): 1 the loss's gradient (p - t) / denom is written to grad as well, 2 it is added to grad: the
+// backward pass of the scalar loss in the same pass over the row (smce_bwd_kernel's arithmetic per element).
+template <int MODE, int GRAD = 0>
 __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(const float* logits, const float* target,
                                                                             float* probs, float* row_loss,
-                                                                            size_t cols) {
+                                                                            size_t cols, float* grad = nullptr,
+                                                                            float denom = 1.f) {
     __shared__ OnlineAccT smem[kLongRowThreads / kWave];
     __shared__ float lsum[kLongRowThreads / kWave];
     __shared__ OnlineAccT total_s;
@@ -288,6 +291,7 @@ __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(cons
     const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
     const float4* t4 = reinterpret_cast<const float4*>(MODE ? target + row * cols : logits);
     float4* p4 = reinterpret_cast<float4*>(probs + row * cols);
+    float4* g4 = reinterpret_cast<float4*>(GRAD ? grad + row * cols : probs);
     const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     float4 v[kLongRowVec], t[kLongRowVec];
 #pragma unroll
@@ -346,6 +350,21 @@ __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(cons
                         part = __fsub_rn(part, __fmul_rn(tv[e], logf(safe)));
                     }
                 }
+                if (GRAD) {
+                    float4 d;
+                    d.x = __fdiv_rn(__fsub_rn(p.x, t[u].x), denom);
+                    d.y = __fdiv_rn(__fsub_rn(p.y, t[u].y), denom);
+                    d.z = __fdiv_rn(__fsub_rn(p.z, t[u].z), denom);
+                    d.w = __fdiv_rn(__fsub_rn(p.w, t[u].w), denom);
+                    if (GRAD == 2) {
+                        const float4 g = nt_load(g4 + j);
+                        d.x = __fadd_rn(g.x, d.x);
+                        d.y = __fadd_rn(g.y, d.y);
+                        d.z = __fadd_rn(g.z, d.z);
+                        d.w = __fadd_rn(g.w, d.w);
+                    }
+                    nt_store(d, g4 + j);
+                }
             }
         }
     }
@@ -365,9 +384,10 @@ __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(cons
 // per row holds the row in registers (at most 4 float4 per lane), so the logits are read once and the row's
 // reductions stay inside the wave: three passes of the matrix instead of four, no LDS, no barrier.
 constexpr int kWaveRowVec = 4;
-template <int MODE>
+template <int MODE, int GRAD = 0>
 __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* logits, const float* target, float* probs,
-                                                                    float* row_loss, size_t rows, size_t cols) {
+                                                                    float* row_loss, size_t rows, size_t cols,
+                                                                    float* grad = nullptr, float denom = 1.f) {
     const int lane = threadIdx.x & (kWave - 1);
     const size_t row = (size_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
     if (row >= rows) return;  // whole waves leave together: no barrier follows
@@ -375,6 +395,7 @@ __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* 
     const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
     const float4* t4 = reinterpret_cast<const float4*>(MODE ? target + row * cols : logits);
     float4* p4 = reinterpret_cast<float4*>(probs + row * cols);
+    float4* g4 = reinterpret_cast<float4*>(GRAD ? grad + row * cols : probs);
     const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     float4 v[kWaveRowVec], t[kWaveRowVec];
 #pragma unroll
@@ -422,6 +443,21 @@ __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* 
                         const float safe = fminf(fmaxf(pv[e], 1e-7f), 1.0f - 1e-7f);
                         part = __fsub_rn(part, __fmul_rn(tv[e], logf(safe)));
                     }
+                }
+                if (GRAD) {
+                    float4 d;
+                    d.x = __fdiv_rn(__fsub_rn(p.x, t[u].x), denom);
+                    d.y = __fdiv_rn(__fsub_rn(p.y, t[u].y), denom);
+                    d.z = __fdiv_rn(__fsub_rn(p.z, t[u].z), denom);
+                    d.w = __fdiv_rn(__fsub_rn(p.w, t[u].w), denom);
+                    if (GRAD == 2) {
+                        const float4 g = nt_load(g4 + j);
+                        d.x = __fadd_rn(g.x, d.x);
+                        d.y = __fadd_rn(g.y, d.y);
+                        d.z = __fadd_rn(g.z, d.z);
+                        d.w = __fadd_rn(g.w, d.w);
+                    }
+                    nt_store(d, g4 + j);
                 }
             }
         }
@@ -790,8 +826,36 @@ ZG_API int zg_hip_smce_fwd_bwd(zg_hip_ctx* ctx, const float* logits, const float
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    if (int rc = zg_hip_smce_fwd(ctx, logits, target, probs, loss, rows, cols)) return rc;
+    // rows a wave or a workgroup holds in registers: probabilities, loss terms and gradient in one pass over the logits
+    // and the target (four streams instead of the six of forward + backward); the gradient must not lie on the inputs
     const size_t n = rows * cols;
+    auto apart = [&](const float* a) { return a + n <= grad || grad + n <= a; };
+    const bool one_pass = aligned16(grad) && apart(logits) && apart(target) && apart(probs) &&
+                          (long_row_ok(logits, target, probs, rows, cols) || wave_row_ok(logits, target, probs, rows, cols));
+    if (one_pass) {
+        float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
+        if (!row_loss) return ZG_HIP_EOOM;
+        const float denom = (float)rows;
+        if (long_row_ok(logits, target, probs, rows, cols)) {
+            if (accumulate)
+                hipLaunchKernelGGL((softmax_long_rows_kernel<1, 2>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
+                                   logits, target, probs, row_loss, cols, grad, denom);
+            else
+                hipLaunchKernelGGL((softmax_long_rows_kernel<1, 1>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
+                                   logits, target, probs, row_loss, cols, grad, denom);
+        } else {
+            const dim3 grid((unsigned)ceil_div_sz(rows, kBlock / kWave));
+            if (accumulate)
+                hipLaunchKernelGGL((softmax_wave_rows_kernel<1, 2>), grid, dim3(kBlock), 0, ctx->stream, logits, target, probs,
+                                   row_loss, rows, cols, grad, denom);
+            else
+                hipLaunchKernelGGL((softmax_wave_rows_kernel<1, 1>), grid, dim3(kBlock), 0, ctx->stream, logits, target, probs,
+                                   row_loss, rows, cols, grad, denom);
+        }
+        ZG_LAUNCH_CHECK();
+        return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, denom});
+    }
+    if (int rc = zg_hip_smce_fwd(ctx, logits, target, probs, loss, rows, cols)) return rc;
     const unsigned blocks = smce_bwd_grid(n);
     if (accumulate)
         hipLaunchKernelGGL(smce_bwd_kernel<true>, dim3(blocks), dim3(kBlock), 0, ctx->stream, probs, target, grad,

@@ -282,3 +282,20 @@ def test_a_refused_call_still_owes_the_zeros_it_took_over(hip):
     assert np.all(hip.to_numpy(g) == 0.0)
     for t in (a, b, c, src, tgt, h, deg, y, gh, gd, g, p):
         hip.mem_free(t)
+
+
+def test_a_refused_max_along_still_owes_the_fill_it_dropped(hip):
+    """max_along overwrites its output without reading it, so a fill of the output that still waits is dropped
+    (NDArray.max_along zero-fills first, src/ndarray.zig:567).  When the call is then refused after that point (more
+    leading slices than a grid holds), nothing was overwritten and the fill must still land."""
+    from zigrad_amd._lib import ZgHipError
+
+    outer, R, inner = 70_000, 2, 3          # dim 1 of [70000, 2, 3]: 70000 leading slices exceed the grid's 65535
+    x = hip.from_numpy(np.ones(outer * R * inner, np.float32))
+    y = hip.from_numpy(np.full(outer * inner, 7.0, np.float32))
+    hip.mem_fill(y, 0.5)
+    with pytest.raises(ZgHipError):
+        hip.dispatch("max_along", x=x, x_shape=[outer, R, inner], y=y, y_shape=[outer, inner], dim=1)
+    assert np.all(hip.to_numpy(y) == 0.5)
+    hip.mem_free(x)
+    hip.mem_free(y)

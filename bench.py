@@ -331,6 +331,11 @@ def op_suite(dev, quick=False, cpu=False):
     out["smce_onehot_fwd_8192x32000"] = gbs(3 * 4 * M * N, ms)
     ms = timed(dev, lambda: dev.dispatch("smce_bwd", probs=probs, target=target, grad=grad, rows=M, cols=N), iters // 2)
     out["smce_onehot_bwd_8192x32000"] = gbs(4 * 4 * M * N, ms)
+    # forward and the loss's backward in one pass over rows held in registers (the fused entry point): logits and target
+    # in, probabilities and the written gradient out
+    ms = timed(dev, lambda: dev.dispatch("smce_fwd_bwd", logits=logits, target=target, probs=probs, loss=loss, grad=grad,
+                                            rows=M, cols=N, accumulate=False), iters // 2)
+    out["smce_onehot_fwd_bwd_one_pass_8192x32000"] = gbs(4 * 4 * M * N, ms)
     for b in (logits, grad, labels, lse, loss, target, probs):
         dev.mem_free(b)
     return out

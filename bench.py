@@ -291,6 +291,20 @@ def op_suite(dev, quick=False, cpu=False):
         ms = timed(dev, lambda: dev.dispatch("scatter_gcn_deg_scaled", dst=y_buf, h=h_buf, deg=deg, src_indices=e_src,
                                              tgt_indices=e_tgt, stride=feat, n_edge=n_edge), iters)
         extra["scatter_gcn_1Medges_x64_ordering_per_call"] = {**gbs(gcn_bytes, ms), "edges_per_us": n_edge / (ms["ms"] * 1e3)}
+        # the same with the target array rewritten before every call (a copy of 8 MB inside the timed region, about
+        # 3 us): the ordering the library keeps for the array is found stale on the GPU and built again, and after a few
+        # such calls the library stops keeping one for this array
+        e_alt = [e_tgt, dev.from_numpy(r.integers(0, n_nodes, n_edge).astype(np.uint64))]
+        e_cur, flip = dev.mem_alloc(U64, n_edge), [0]
+
+        def rewritten(op, **kw):
+            flip[0] ^= 1
+            dev.mem_copy(e_alt[flip[0]], e_cur)
+            dev.dispatch(op, **kw)
+
+        ms = timed(dev, lambda: rewritten("scatter_gcn_deg_scaled", dst=y_buf, h=h_buf, deg=deg, src_indices=e_src,
+                                          tgt_indices=e_cur, stride=feat, n_edge=n_edge), iters)
+        extra["scatter_gcn_1Medges_x64_indices_rewritten_every_call"] = {**gbs(gcn_bytes, ms), "edges_per_us": n_edge / (ms["ms"] * 1e3)}
         plan = dev.edge_plan(e_src, e_tgt, n_nodes)
         ms = timed(dev, lambda: dev.dispatch("scatter_gcn_deg_scaled_planned", dst=y_buf, h=h_buf, deg=deg, plan=plan,
                                              stride=feat, accumulate=True), iters)
@@ -298,11 +312,13 @@ def op_suite(dev, quick=False, cpu=False):
         vals = Y.sub(0, n_edge)
         ms = timed(dev, lambda: dev.dispatch("scatter_add", src=vals, offsets=e_tgt, dst=y_buf.sub(0, n_nodes)), iters)
         extra["scatter_add_1M_into_100k_ordering_per_call"] = {**ms, "entries_per_us": n_edge / (ms["ms"] * 1e3)}
+        ms = timed(dev, lambda: rewritten("scatter_add", src=vals, offsets=e_cur, dst=y_buf.sub(0, n_nodes)), iters)
+        extra["scatter_add_1M_into_100k_indices_rewritten_every_call"] = {**ms, "entries_per_us": n_edge / (ms["ms"] * 1e3)}
         ms = timed(dev, lambda: dev.dispatch("scatter_add_planned", src=vals, plan=plan, dst=y_buf.sub(0, n_nodes)), iters * 5)
         extra["scatter_add_1M_into_100k_planned"] = {**ms, "entries_per_us": n_edge / (ms["ms"] * 1e3)}
         plan.free()
         out["other_ops"] = extra
-        for b in (G, Y, ycol, yarg, ysc, idx, e_src, e_tgt, deg):
+        for b in (G, Y, ycol, yarg, ysc, idx, e_src, e_tgt, e_alt[1], e_cur, deg):
             dev.mem_free(b)
     for b in (X, bias, Z, yrow):
         dev.mem_free(b)

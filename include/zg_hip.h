@@ -384,9 +384,18 @@ int zg_hip_segment_sum_csr(zg_hip_ctx *ctx, const float *src, size_t src_len, co
  * instead of computing it again: same values, five to six launches fewer per ordering.  At most 16 orderings are
  * kept (least recently used goes first), for arrays of up to 65536 entries (longer ones cost more to compare than
  * to analyse).  A recorded graph keeps the orderings it used, and zg_hip_graph_run returns
- * ZG_HIP_EINVAL when one of those arrays no longer holds what it held at the recording.  Index arrays in device
- * memory are analysed on every call.  `hits` / `builds` count calls served from a kept ordering / orderings computed
- * and kept; no counterpart in the reference. */
+ * ZG_HIP_EINVAL when one of those arrays no longer holds what it held at the recording.  Shorter index arrays in
+ * device memory are analysed on every call.
+ * Arrays of 262144 to 2^24 entries, in device memory or in zg_hip_host_alloc memory, are kept differently: under the
+ * ADDRESSES of the arrays, with 32-bit copies of their contents beside the ordering, and every call starts with a
+ * kernel that compares the arrays with the copies ON THE GPU.  Unchanged arrays skip the rebuild (the kernels of the
+ * build are launched and return at once), changed ones are ordered again in place; either way the call works on the
+ * arrays as they are when its kernels run, whoever rewrote them, so a recorded graph stays valid when the arrays are
+ * rewritten between replays.  An array that turns out to change on most calls is dropped from the cache and analysed
+ * on every call like a short one (the address is tried again 1024 calls later).  These entries count in `hits` when
+ * the address was found, whether or not the contents had changed.
+ * `hits` / `builds` count calls served from a kept ordering / orderings computed and kept; no counterpart in the
+ * reference. */
 int zg_hip_plan_cache_stats(zg_hip_ctx *ctx, uint64_t *hits, uint64_t *builds);
 
 /* Edge plans.  The three ops above sort the edge list by destination on every call, because the reference hands

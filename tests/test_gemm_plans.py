@@ -21,10 +21,26 @@ def test_benchmark_products_stay_single_launches(shape, tile):
 
 
 def test_off_grid_cubes_are_cut_into_whole_rounds_plus_strips():
-    p = gemm_plan(3072, 3072, 3072)   # 288 large tiles: 252 in the main block (one round of 256 CUs), a strip of 36
-    assert p["kind"] == "parts" and p["main_tiles"] == (12, 21)
     p = gemm_plan(4100, 4100, 4100)   # 4096 x 4096 is two exact rounds; 4 rows and 4 columns are left over
     assert p["kind"] == "parts" and p["main_tiles"] == (16, 32)
+    p = gemm_plan(3600, 2308, 1541)
+    assert p["kind"] == "parts"
+
+
+def test_whole_tiles_that_leave_a_round_part_empty_get_their_tail_in_pieces():
+    p = gemm_plan(1536, 1536, 1536)   # 576 tiles of 64 x 64: two rounds of 256 whole, 64 tiles in 4 pieces each = 256 pieces
+    assert p["kind"] == "tail_in_pieces" and p["tile"] == (64, 64) and p["whole_tiles"] == 512 and p["splits"] == 4
+    assert p["k_tiles_per_split"] == 24
+    p = gemm_plan(3072, 3072, 3072)   # 576 tiles of 128 x 128
+    assert p["kind"] == "tail_in_pieces" and p["tile"] == (128, 128) and p["whole_tiles"] == 512
+    for shape in ((1536, 1536, 1234), (2560, 2560, 2560), (3584, 3584, 3584), (2560, 3328, 1024)):
+        p = gemm_plan(*shape)
+        assert p["kind"] == "tail_in_pieces" and p["whole_tiles"] % 256 == 0 and p["whole_tiles"] > 0
+        assert p["k_tiles_per_split"] % 2 == 0 and p["k_tiles_per_split"] >= 8
+        assert (p["splits"] - 1) * p["k_tiles_per_split"] * 16 < shape[2] <= p["splits"] * p["k_tiles_per_split"] * 16
+    # nothing to gain: a whole number of rounds, fewer tiles than CUs, tiles that end inside C, a batch
+    for shape in ((2048, 2048, 2048), (4096, 4096, 4096), (768, 768, 768), (1540, 1536, 1536), (1536, 1536, 1536, 2)):
+        assert gemm_plan(*shape)["kind"] != "tail_in_pieces", shape
 
 
 def test_deep_products_on_few_tiles_are_cut_along_k():

@@ -15,7 +15,7 @@ from zigrad_amd.device import F32
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(64, 784, 128), (64, 64, 10), (33, 70, 129), (256, 512, 384), (250, 512, 380), (1024, 1024, 1024),
-          (130, 1433, 16), (2048, 1000, 1024), (2560, 1024, 3328), (2, 5, 3)]
+          (130, 1433, 16), (2048, 1000, 1024), (2560, 1024, 3328), (2560, 1024, 3332), (2, 5, 3)]
 
 
 def _forward(hip, x, w, bias, relu, bias_first, eager):

@@ -1,6 +1,7 @@
-"""Products that the planner launches in parts (a block of whole rounds plus strips) or with k cut over several
-workgroups per large tile: against float64 products in full, bit-exact on integer-valued operands, with accumulation,
-and through the fused Linear entry points (bias, ReLU and gate must land on the right strip)."""
+"""Products that the planner launches in parts (a block of whole rounds plus strips), with the tiles of the last round
+cut into pieces along k, or with k cut over several workgroups per large tile: against float64 products in full,
+bit-exact on integer-valued operands, with accumulation, and through the fused Linear entry points (bias, ReLU and gate
+must land on the right strip or tile)."""
 from __future__ import annotations
 
 import numpy as np
@@ -23,11 +24,15 @@ def _matmul(hip, A, B, C0, m, n, k, ta, tb, alpha, beta):
     return out
 
 
-@pytest.mark.parametrize("shape", [(3072, 3072, 3072), (4100, 4100, 1030), (3600, 2308, 1541)])
+# (3072, 3072, 3072): 128 x 128 tiles, 4 pieces of 48 k-tiles; (1536, 1536, 1234): 64 x 64 tiles, a k that ends inside a
+# k-tile, so the last piece is short and masked; (2560, 3328, 1024): 8 pieces of 8 k-tiles, the shortest range allowed
+@pytest.mark.parametrize("shape,kind", [((4100, 4100, 1030), "parts"), ((3600, 2308, 1541), "parts"),
+                                        ((3072, 3072, 3072), "tail_in_pieces"), ((1536, 1536, 1234), "tail_in_pieces"),
+                                        ((2560, 3328, 1024), "tail_in_pieces")])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-def test_products_launched_in_parts_match_float64(hip, shape, ta, tb):
+def test_products_launched_in_parts_or_with_the_tail_in_pieces_match_float64(hip, shape, kind, ta, tb):
     m, n, k = shape
-    assert hip.gemm_plan(m, n, k)["kind"] == "parts", hip.gemm_plan(m, n, k)
+    assert hip.gemm_plan(m, n, k)["kind"] == kind, hip.gemm_plan(m, n, k)
     r = np.random.default_rng(m + 3 * n + 7 * k + 2 * ta + tb)
     A = r.standard_normal((k, m) if ta else (m, k), dtype=np.float32)
     B = r.standard_normal((n, k) if tb else (k, n), dtype=np.float32)
@@ -38,7 +43,9 @@ def test_products_launched_in_parts_match_float64(hip, shape, ta, tb):
     got = _matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, ta, tb, 1.0, 0.0)
     assert np.linalg.norm(got - prod) <= TOL * np.linalg.norm(prod)
     # every strip separately: an error confined to a few rows or columns must not hide in the whole-matrix norm
-    for sl in (np.s_[-4:, :], np.s_[:, -4:], np.s_[: m // 2, n // 2:], np.s_[m // 2:, : n // 2]):
+    # (the tiles cut into pieces are the last of the walk over C: its bottom rows)
+    for sl in (np.s_[-4:, :], np.s_[:, -4:], np.s_[: m // 2, n // 2:], np.s_[m // 2:, : n // 2], np.s_[-256:, -128:],
+               np.s_[-64:, :64]):
         assert np.linalg.norm(got[sl] - prod[sl]) <= TOL * np.linalg.norm(prod[sl])
     got = _matmul(hip, A, B, C0, m, n, k, ta, tb, 0.5, 2.0)
     want = 0.5 * prod + 2.0 * C0
@@ -46,7 +53,7 @@ def test_products_launched_in_parts_match_float64(hip, shape, ta, tb):
 
 
 def test_parts_and_split_products_are_exact_on_small_integers(hip):
-    for (m, n, k) in ((3072, 3072, 3072), (4100, 4100, 1030)):
+    for (m, n, k) in ((3072, 3072, 3072), (4100, 4100, 1030), (1536, 1536, 1536)):
         r = np.random.default_rng(m)
         A = r.integers(-3, 4, (m, k)).astype(np.float32)
         B = r.integers(-3, 4, (n, k)).astype(np.float32)  # stored [n, k]: the forward layout of a Linear layer
@@ -55,9 +62,10 @@ def test_parts_and_split_products_are_exact_on_small_integers(hip):
         assert np.array_equal(got, want)
 
 
-def test_fused_linear_entry_points_on_a_product_launched_in_parts(hip):
-    Bt, I, O = 2560, 1024, 3328  # batch, fan_in, fan_out
-    assert hip.gemm_plan(Bt, O, I)["kind"] == "parts", hip.gemm_plan(Bt, O, I)
+@pytest.mark.parametrize("wide,kind", [(3332, "parts"), (3328, "tail_in_pieces")])
+def test_fused_linear_entry_points_on_a_product_launched_in_parts_or_with_the_tail_in_pieces(hip, wide, kind):
+    Bt, I, O = 2560, 1024, wide  # batch, fan_in, fan_out
+    assert hip.gemm_plan(Bt, O, I)["kind"] == kind, hip.gemm_plan(Bt, O, I)
     r = np.random.default_rng(77)
     x = r.standard_normal((Bt, I)).astype(np.float32)
     w = (r.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
@@ -73,8 +81,8 @@ def test_fused_linear_entry_points_on_a_product_launched_in_parts(hip):
     want = np.maximum(x.astype(np.float64) @ w.astype(np.float64).T + b, 0.0)
     assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
     # input gradient with the ReLU gate of the layer below: gx = (gy W) where act > 0
-    I2, O2 = 3328, 1024
-    assert hip.gemm_plan(Bt, I2, O2)["kind"] == "parts"
+    I2, O2 = wide, 1024
+    assert hip.gemm_plan(Bt, I2, O2)["kind"] == kind
     gy = r.standard_normal((Bt, O2)).astype(np.float32)
     w2 = (r.standard_normal((O2, I2)) / np.sqrt(O2)).astype(np.float32)
     act = np.maximum(r.standard_normal((Bt, I2)), 0.0).astype(np.float32)

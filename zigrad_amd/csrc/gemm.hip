@@ -204,6 +204,14 @@ struct GemmArgs {
     // split-K: workgroup y handles k-tiles [y * split_tiles, (y + 1) * split_tiles) and writes its C tile at
     // C + y * split_stride (the launcher points C at a buffer of partial products); one split = the whole of k
     size_t split_tiles, split_stride;
+    // Tail in pieces (staged kernels, one unbatched product of whole tiles; tail_splits == 0: off).  The first
+    // tail_first workgroups (a whole number of rounds of the CUs) compute whole tiles as ever; the tiles that would
+    // start one more round are cut along k instead, tail_splits workgroups per tile with split_tiles k-tiles each,
+    // and piece p of tail tile t goes to tail_part + (t * tail_splits + p) * BM * BN as a dense BM x BN block with no
+    // epilogue arithmetic; gemm_tail_reduce_kernel adds a tile's pieces in piece order and applies alpha, beta and the
+    // extras.  Every CU then carries the same work instead of a quarter of them carrying one tile more.
+    unsigned tail_first, tail_splits;
+    float* tail_part;
     int a_vec, b_vec;  // 16-byte vector loads are legal for this operand
     int c_vec;         // vector stores to C are legal (alignment, ldc and n multiples of 4)
     int bounded_tail;  // edge kernels: an m or n that ends inside a 16-byte piece reads a few floats past the
@@ -275,7 +283,19 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // fetches its panels alone (32 x 512 x 512 x 4096: 513 -> 46x us).
     unsigned tm, tn;
     size_t z = blockIdx.z;
-    {
+    unsigned split = blockIdx.y;
+    bool piece = false;     // a k range of a tail tile: goes to the partial buffer as it is
+    unsigned piece_id = 0;
+    if (g.tail_splits) {
+        if (blockIdx.x < g.tail_first) {
+            tile_coords(xcd_contiguous(blockIdx.x, g.tail_first), g.tiles_m, g.tiles_n, tm, tn);
+        } else {
+            piece = true;
+            piece_id = blockIdx.x - g.tail_first;
+            split = piece_id % g.tail_splits;
+            tile_coords(g.tail_first + piece_id / g.tail_splits, g.tiles_m, g.tiles_n, tm, tn);
+        }
+    } else {
         const unsigned per_batch = g.tiles_m * g.tiles_n;
         if (g.flat_batches) {
             const unsigned id = xcd_contiguous(blockIdx.x, per_batch * g.flat_batches);
@@ -287,8 +307,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     }
     const float* A = g.A + (z % g.nba) * g.a_chunk;
     const float* B = g.B + (z % g.nbb) * g.b_chunk;
-    float* C = g.C + z * g.c_chunk + (size_t)blockIdx.y * g.split_stride;
     const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+    // where the tile's element (0, 0) is stored, and the row pitch there
+    float* const c_org = piece ? g.tail_part + (size_t)piece_id * (BM * BN)
+                               : g.C + z * g.c_chunk + (size_t)split * g.split_stride + m0 * g.ldc + n0;
+    const size_t c_ld = piece ? (size_t)BN : g.ldc;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
@@ -303,8 +326,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     // this workgroup's range of k
-    const size_t k_begin = (size_t)blockIdx.y * g.split_tiles * BK;
-    const size_t k_end = (k_begin + g.split_tiles * BK < g.K) ? k_begin + g.split_tiles * BK : g.K;
+    const bool whole_k = g.tail_splits && !piece;
+    const size_t k_begin = whole_k ? 0 : (size_t)split * g.split_tiles * BK;
+    const size_t k_end = (whole_k || k_begin + g.split_tiles * BK >= g.K) ? g.K : k_begin + g.split_tiles * BK;
     // 32-bit tile counter: there is no scalar 64-bit ordered compare, and a vector compare in the loop costs MFMA time
     const unsigned KT = (unsigned)((k_end - k_begin + BK - 1) / BK);
     // fast / edge kernels: a k range that is not a whole number of tile pairs ends in tiles whose values past k_end
@@ -510,9 +534,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // instruction writes two 128-byte row segments; otherwise a lane owns TN adjacent columns and stores them as
     // one vector.  With beta != 0 the old values of a row of blocks are read together before any is used; C is
     // not read at all when beta == 0.
-    const float alpha = g.alpha, beta = g.beta;
+    const float alpha = piece ? 1.f : g.alpha, beta = piece ? 0.f : g.beta;
     const bool use_c = beta != 0.f;
-    const bool has_bias = g.bias != nullptr, relu = g.relu != 0, gated = g.gate != nullptr;  // gated implies !use_c
+    // gated implies !use_c
+    const bool has_bias = !piece && g.bias != nullptr, relu = !piece && g.relu != 0, gated = !piece && g.gate != nullptr;
     // the gate value of a C element sits at the same offset from g.gate as the element from g.C
     const ptrdiff_t gate_bytes = gated ? reinterpret_cast<const char*>(g.gate) - reinterpret_cast<const char*>(g.C) : 0;
 
@@ -536,7 +561,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const size_t col = n0 + wn0 + FB::index_of(j, l32);
-            cptr[j] = C + (m0 + wm0 + FA::index_of(i, lk * 4)) * g.ldc + col;
+            cptr[j] = c_org + (size_t)(wm0 + FA::index_of(i, lk * 4)) * c_ld + (col - n0);
             optr[j] = reinterpret_cast<const float*>(reinterpret_cast<const char*>(cptr[j]) + gate_bytes);
             bias_v[j] = (has_bias && (MODE == 0 || col < g.N)) ? g.bias[col] : 0.f;
         }
@@ -553,7 +578,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             for (int r = 0; r < 16; r++) {
                 if (vec_c) {
                     VC o = {};
-                    if (in_range(0, r)) o = *reinterpret_cast<const VC*>(optr[0] + (size_t)row_of(r) * g.ldc);
+                    if (in_range(0, r)) o = *reinterpret_cast<const VC*>(optr[0] + (size_t)row_of(r) * c_ld);
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
                         if constexpr (VEC_C) old[j][r] = o[j];
@@ -561,7 +586,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
                 } else {
 #pragma unroll
                     for (int j = 0; j < TN; j++)
-                        old[j][r] = in_range(j, r) ? optr[j][(size_t)row_of(r) * g.ldc] : 0.f;
+                        old[j][r] = in_range(j, r) ? optr[j][(size_t)row_of(r) * c_ld] : 0.f;
                 }
             }
         }
@@ -597,11 +622,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
                 for (int j = 0; j < TN; j++) {
                     if constexpr (VEC_C) o[j] = res[j][r];
                 }
-                if (in_range(0, r)) *reinterpret_cast<VC*>(cptr[0] + (size_t)row_of(r) * g.ldc) = o;
+                if (in_range(0, r)) *reinterpret_cast<VC*>(cptr[0] + (size_t)row_of(r) * c_ld) = o;
             } else {
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    if (in_range(j, r)) cptr[j][(size_t)row_of(r) * g.ldc] = res[j][r];
+                    if (in_range(j, r)) cptr[j][(size_t)row_of(r) * c_ld] = res[j][r];
             }
         }
         // one row of blocks at a time
@@ -615,9 +640,10 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
     g.tiles_n = (unsigned)ceil_div_sz(g.N, BN);
     const size_t kt_total = ceil_div_sz(g.K, kBK);
     dim3 grid(g.tiles_m * g.tiles_n, (unsigned)ceil_div_sz(kt_total, g.split_tiles), (unsigned)batches), block(kGemmThreads);
+    if (g.tail_splits) grid = dim3(g.tail_first + (g.tiles_m * g.tiles_n - g.tail_first) * g.tail_splits, 1, 1);
     const size_t flat = (size_t)grid.x * batches;
     g.flat_batches = 0;
-    if (batches > 1 && grid.y == 1 && flat % 8 == 0 && flat < 0x7fffffffull) {
+    if (!g.tail_splits && batches > 1 && grid.y == 1 && flat % 8 == 0 && flat < 0x7fffffffull) {
         g.flat_batches = (unsigned)batches;
         grid = dim3((unsigned)flat, 1, 1);
     }
@@ -868,6 +894,56 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(const float* P,
     }
 }
 
+// The tail tiles of a product launched with its tail in pieces (GemmArgs::tail_part): C tile = alpha * (the tile's
+// pieces, added in piece order) + beta * C, then the extras.  A thread owns four adjacent columns of one row.
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(GemmArgs g) {
+    constexpr unsigned V4 = BM * BN / 4, PER_TILE = V4 / 256;
+    const unsigned t = blockIdx.x / PER_TILE, q = (blockIdx.x % PER_TILE) * 256 + threadIdx.x;
+    unsigned tm, tn;
+    tile_coords(g.tail_first + t, g.tiles_m, g.tiles_n, tm, tn);
+    const unsigned row = q / (BN / 4), col = (q % (BN / 4)) * 4;
+    const float4* p = reinterpret_cast<const float4*>(g.tail_part + (size_t)t * g.tail_splits * (BM * BN)) + q;
+    float4 acc = p[0];
+    for (unsigned s0 = 1; s0 < g.tail_splits; s0 += 8) {  // eight pieces' loads in flight, added in piece order
+        float4 v[8];
+#pragma unroll
+        for (unsigned u = 0; u < 8; u++)
+            if (s0 + u < g.tail_splits) v[u] = p[(size_t)(s0 + u) * V4];
+#pragma unroll
+        for (unsigned u = 0; u < 8; u++) {
+            if (s0 + u < g.tail_splits) {
+                acc.x += v[u].x;
+                acc.y += v[u].y;
+                acc.z += v[u].z;
+                acc.w += v[u].w;
+            }
+        }
+    }
+    const size_t at = ((size_t)tm * BM + row) * g.ldc + (size_t)tn * BN + col;
+    float r[4] = {g.alpha * acc.x, g.alpha * acc.y, g.alpha * acc.z, g.alpha * acc.w};
+    if (g.beta != 0.f) {
+        const float4 old = *reinterpret_cast<const float4*>(g.C + at);
+        r[0] += g.beta * old.x;
+        r[1] += g.beta * old.y;
+        r[2] += g.beta * old.z;
+        r[3] += g.beta * old.w;
+    }
+    if (g.bias || g.relu) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            r[j] = gemm_extras(r[j], g.bias != nullptr, g.bias ? g.bias[(size_t)tn * BN + col + j] : 0.f, g.relu != 0);
+    }
+    if (g.gate) {
+        const float4 gv = *reinterpret_cast<const float4*>(g.gate + at);
+        r[0] = gv.x <= 0.f ? 0.f : r[0];
+        r[1] = gv.y <= 0.f ? 0.f : r[1];
+        r[2] = gv.z <= 0.f ? 0.f : r[2];
+        r[3] = gv.w <= 0.f ? 0.f : r[3];
+    }
+    *reinterpret_cast<float4*>(g.C + at) = make_float4(r[0], r[1], r[2], r[3]);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Launch planning for the staged kernels.  A CU works through its workgroups at a rate that depends on the tile
 // shape but hardly on how many of them share the CU, so a launch takes (rounds the grid needs) x (time of one tile)
@@ -887,9 +963,10 @@ constexpr double kLaunchFixedUs = 8.0;
 constexpr double kReduceFixedUs = 4.0, kReduceBytesPerUs = 4.0e6;
 
 struct GemmPlan {
-    enum Kind { kPlain, kSplit, kParts } kind = kPlain;
+    enum Kind { kPlain, kSplit, kParts, kTail } kind = kPlain;
     int tile = 2;
-    size_t splits = 1, per = 0;  // kSplit: number of k ranges and k-tiles per range
+    size_t splits = 1, per = 0;  // kSplit, kTail: number of k ranges and k-tiles per range
+    size_t whole = 0;            // kTail: tiles computed whole (a whole number of rounds)
     size_t rm = 0, rn = 0;       // kParts: the main block is rm x rn tiles of 256 x 128
     double us = 0;               // the model's estimate
 };
@@ -937,6 +1014,8 @@ static bool gemm_plan_is_slow(double us, size_t m, size_t n, size_t k, size_t ba
     const double ideal = 2.0 * (double)m * (double)n * (double)k * (double)batches / ((double)n_cu * kCuFlopsPerUs * 0.975);
     return us > 1.12 * ideal + kLaunchFixedUs;
 }
+
+static GemmPlan gemm_plan_compute_untailed(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth);
 
 // One launch (plus the reduction when k is cut) for the whole product: the choice made before planning existed
 // (`legacy`: rounds x padded tile work over 0.92 / 0.89 / 0.79, and the 64 x 64 split for few tiles and a deep k), and,
@@ -1004,7 +1083,70 @@ static GemmPlan gemm_plan_single(size_t m, size_t n, size_t k, size_t batches, s
     return (bp.us < 0.92 * lp.us) ? bp : lp;
 }
 
-static GemmPlan gemm_plan_compute(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth) {
+// The tail in pieces (GemmArgs::tail_part) for one unbatched product of whole tiles that needs more than one round:
+// with T tiles on n_cu CUs, R = T / n_cu whole rounds and L = T % n_cu tiles left over, a plain launch takes R + 1
+// tile times although the last round keeps only L of the CUs busy.  Cutting each left-over tile into s ranges of k
+// gives L * s pieces of 1 / s tile each, spread over all CUs: R + ceil(L * s / n_cu) / s tile times, plus the second
+// kernel that adds the pieces.  Measured per-round efficiencies (fraction of a CU's MFMA peak while a round runs: 0.975
+// / 0.98 / 0.92 for the three tiles) are about equal, so what separates the tiles in this range of sizes is how much
+// of the last round is empty, and with the tail in pieces the larger tiles win again: 1536-cubed 69 -> 58 us
+// (64 x 64, s = 4), 2560-cubed 285 -> 243 us (64 x 64, s = 4), 3072-cubed 412 (in parts) -> 395 us (128 x 128, s = 4),
+// 3584-cubed 93.5 % of the matrix peak (128 x 128, s = 8).
+static const double kRoundEff[3] = {0.975, 0.98, 0.92};
+constexpr double kPieceFixedUs = 1.5, kTailReduceFixedUs = 3.0;
+
+static double gemm_rounds_us(int tile, double rounds, size_t k) {
+    const GemmTileKind& t = kGemmTiles[tile];
+    return kLaunchFixedUs + rounds * 2.0 * (double)(t.bm * t.bn) * (double)k / (kCuFlopsPerUs * kRoundEff[tile]);
+}
+
+static bool gemm_plan_tail(size_t m, size_t n, size_t k, size_t n_cu, GemmPlan* out) {
+    const size_t kt_total = ceil_div_sz(k, kBK);
+    bool found = false;
+    for (int t = 0; t < 3; t++) {
+        const size_t bm = kGemmTiles[t].bm, bn = kGemmTiles[t].bn;
+        if (m % bm || n % bn) continue;
+        const size_t T = (m / bm) * (n / bn), R = T / n_cu, L = T % n_cu;
+        if (R == 0 || L == 0 || T >= 0x7fffffffull / 16) continue;
+        for (size_t want = 2; want <= 8; want++) {
+            size_t per = ceil_div_sz(kt_total, want);
+            per += per & 1;
+            if (per < 8) break;  // ranges shorter than 128 values of k are all prologue
+            const size_t s = ceil_div_sz(kt_total, per);
+            if (s < 2) continue;
+            const size_t piece_rounds = ceil_div_sz(L * s, n_cu);
+            const double us = gemm_rounds_us(t, (double)R + (double)piece_rounds * (double)per / (double)kt_total, k) +
+                              kPieceFixedUs * (double)piece_rounds + kTailReduceFixedUs +
+                              (double)((s + 1) * L * bm * bn) * 4.0 / kReduceBytesPerUs;
+            if (!found || us < out->us) {
+                found = true;
+                out->kind = GemmPlan::kTail;
+                out->tile = t;
+                out->splits = s;
+                out->per = per;
+                out->whole = R * n_cu;
+                out->us = us;
+            }
+        }
+    }
+    return found;
+}
+
+static GemmPlan gemm_plan_compute(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth,
+                                  bool allow_tail = true) {
+    GemmPlan best = gemm_plan_compute_untailed(n_cu, m, n, k, batches, depth);
+    GemmPlan tail;
+    if (allow_tail && batches == 1 && gemm_plan_tail(m, n, k, n_cu, &tail)) {
+        // against the plan in hand priced the same way (a plain launch: its rounds at the measured efficiencies)
+        double in_hand = best.us;
+        if (best.kind == GemmPlan::kPlain)
+            in_hand = gemm_rounds_us(best.tile, (double)ceil_div_sz(gemm_tiles_of(best.tile, m, n, 1), n_cu), k);
+        if (tail.us < 0.95 * in_hand) return tail;
+    }
+    return best;
+}
+
+static GemmPlan gemm_plan_compute_untailed(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth) {
     GemmPlan best = gemm_plan_single(m, n, k, batches, n_cu);
     // C in parts: only for one product (no batch), at the top level, when the single launch is slow by the model
     const size_t tm_f = m / 256, tn_f = n / 128;
@@ -1035,13 +1177,15 @@ static GemmPlan gemm_plan_compute(size_t n_cu, size_t m, size_t n, size_t k, siz
     return best;
 }
 
+// allow_tail: C is fit for the fast kernels' vector stores (the pieces and their sums are written that way)
 static GemmPlan gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_t batches, bool a_kmajor, bool b_kmajor,
-                          int depth) {
+                          int depth, bool allow_tail) {
     if (!ctx->gemm_plans) ctx->gemm_plans = new GemmPlanCache();
-    const GemmPlanKey key{m, n, k, batches, (a_kmajor ? 1 : 0) | (b_kmajor ? 2 : 0) | (depth ? 4 : 0)};
+    const GemmPlanKey key{m, n, k, batches,
+                          (a_kmajor ? 1 : 0) | (b_kmajor ? 2 : 0) | (depth ? 4 : 0) | (allow_tail ? 8 : 0)};
     auto it = ctx->gemm_plans->plans.find(key);
     if (it != ctx->gemm_plans->plans.end()) return it->second;
-    const GemmPlan best = gemm_plan_compute((size_t)ctx->n_cu, m, n, k, batches, depth);
+    const GemmPlan best = gemm_plan_compute((size_t)ctx->n_cu, m, n, k, batches, depth, allow_tail);
     ctx->gemm_plans->plans[key] = best;
     return best;
 }
@@ -1083,6 +1227,8 @@ static GemmArgs gemm_args(const float* A, const float* B, float* C, size_t m, si
     g.flat_batches = 0;
     g.split_tiles = 0;
     g.split_stride = 0;
+    g.tail_first = g.tail_splits = 0;
+    g.tail_part = nullptr;
     g.c_vec = 0;
     g.bounded_tail = 0;
     return g;
@@ -1271,7 +1417,7 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     }
 
     // ---- plan: which tile, whether k is cut, whether C is cut into a block of whole rounds plus strips ----
-    const GemmPlan plan = gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth);
+    const GemmPlan plan = gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth, c_vec && small_ld);
     if (plan.kind == GemmPlan::kParts) {
         // C = [ main | right ] over [ bottom ]: main is rm x rn whole large tiles (a whole number of rounds, or nearly),
         // the strips are products of their own and go through this function again (they may cut k, not C).
@@ -1334,6 +1480,26 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
+    if (plan.kind == GemmPlan::kTail) {
+        // whole tiles for a whole number of rounds, the remaining tiles in pieces along k, one more kernel for their sums
+        const size_t tail_tiles = tiles(bm, bn) - plan.whole;
+        float* part = (float*)workspace(ctx, tail_tiles * plan.splits * bm * bn * sizeof(float));
+        if (!part) return ZG_HIP_EOOM;
+        g.tail_first = (unsigned)plan.whole;
+        g.tail_splits = (unsigned)plan.splits;
+        g.tail_part = part;
+        g.split_tiles = plan.per;
+        int rc = tile == 0   ? launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, 0, 1)
+                 : tile == 1 ? launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, 0, 1)
+                             : launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 0, 1);
+        if (rc) return rc;
+        const unsigned blocks = (unsigned)(tail_tiles * (bm * bn / 1024));
+        if (tile == 0) hipLaunchKernelGGL((gemm_tail_reduce_kernel<256, 128>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+        else if (tile == 1) hipLaunchKernelGGL((gemm_tail_reduce_kernel<128, 128>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+        else hipLaunchKernelGGL((gemm_tail_reduce_kernel<64, 64>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     if (tile == 0) return launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, mode(256, 128), batches);
     if (tile == 1) return launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, mode(128, 128), batches);
     return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, mode(64, 64), batches);
@@ -1342,6 +1508,8 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
 // The workspace a single product of this shape asks for when it is dispatched (the partial tiles of a k that is cut),
 // following gemm_dispatch_body's choices.  A product that waits reserves it when it is queued, so that the call
 // which later launches it, whichever that is, allocates nothing.
+static size_t gemm_workspace_need_untailed(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b,
+                                           size_t lda, size_t ldb, int depth);
 static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda,
                                   size_t ldb, int depth) {
     if (m == 0 || n == 0 || k == 0) return 0;
@@ -1358,7 +1526,21 @@ static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k,
         splits = ceil_div_sz(groups, per);
         return splits * m * n * sizeof(float);
     }
-    const GemmPlan plan = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth);
+    // whether C will be fit for vector stores is not known here: the larger of the two plans' needs
+    const GemmPlan tailed = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth, true);
+    size_t tail_need = 0;
+    if (tailed.kind == GemmPlan::kTail) {
+        const size_t bm = kGemmTiles[tailed.tile].bm, bn = kGemmTiles[tailed.tile].bn;
+        tail_need = ((m / bm) * (n / bn) - tailed.whole) * tailed.splits * bm * bn * sizeof(float);
+    }
+    const size_t other_need = gemm_workspace_need_untailed(ctx, m, n, k, trans_a, trans_b, lda, ldb, depth);
+    return tail_need > other_need ? tail_need : other_need;
+}
+
+static size_t gemm_workspace_need_untailed(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b,
+                                           size_t lda, size_t ldb, int depth) {
+    const bool a_kmajor = !trans_a, b_kmajor = trans_b != 0;
+    const GemmPlan plan = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth, false);
     if (plan.kind == GemmPlan::kParts) {
         const size_t m1 = plan.rm * 256, n1 = plan.rn * 128;
         const size_t shapes[3][2] = {{m1, n1}, {m1, n - n1}, {m - m1, n}};
@@ -1501,7 +1683,7 @@ ZG_API int zg_hip_gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_
     out[1] = p.tile;
     out[2] = (int64_t)p.splits;
     out[3] = (int64_t)p.per;
-    out[4] = (int64_t)p.rm;
+    out[4] = (int64_t)(p.kind == GemmPlan::kTail ? p.whole : p.rm);
     out[5] = (int64_t)p.rn;
     out[6] = (int64_t)(p.us + 0.5);
     return ZG_HIP_OK;

@@ -594,9 +594,11 @@ def gemm_plan(m: int, n: int, k: int, batches: int = 1, dev: "HipDevice | None" 
 
     out = (ctypes.c_int64 * 7)()
     lib().call("zg_hip_gemm_plan", dev._ctx if dev is not None else None, m, n, k, batches, out)
-    kinds, tiles = ("single", "split_k", "parts"), ((256, 128), (128, 128), (64, 64))
+    kinds, tiles = ("single", "split_k", "parts", "tail_in_pieces"), ((256, 128), (128, 128), (64, 64))
+    tail = kinds[out[0]] == "tail_in_pieces"
     return {"kind": kinds[out[0]], "tile": tiles[out[1]], "splits": out[2], "k_tiles_per_split": out[3],
-            "main_tiles": (out[4], out[5]), "estimate_us": out[6]}
+            "main_tiles": (0, 0) if tail else (out[4], out[5]), "whole_tiles": out[4] if tail else 0,
+            "estimate_us": out[6]}
 
 
 class Graph:

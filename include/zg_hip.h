@@ -225,9 +225,11 @@ int zg_hip_gemm_timing_read(zg_hip_ctx *ctx, double *total_ms, uint64_t *product
 /* How a product of this shape would be launched by the staged kernels (no counterpart in the reference; for tests
  * and for reading profiles).  out[0] kind: 0 one launch, 1 k cut over several workgroups per tile and the partial
  * tiles added in a fixed order by a second kernel, 2 C cut into a block of whole 256 x 128 tiles plus strips that are
- * launched as products of their own; out[1] tile: 0 = 256 x 128, 1 = 128 x 128, 2 = 64 x 64; out[2], out[3] number of k
- * ranges and k-tiles (of 16) per range; out[4], out[5] tile rows and columns of the main block; out[6] the planner's
- * estimate in microseconds.  Products served by the unstaged small-product kernels are not planned this way.
+ * launched as products of their own, 3 the tail in pieces: a whole number of rounds of tiles computed whole and, in the
+ * same launch, the tiles that would start one more (mostly empty) round cut along k into pieces, which a second kernel
+ * adds tile by tile in a fixed order; out[1] tile: 0 = 256 x 128, 1 = 128 x 128, 2 = 64 x 64; out[2], out[3] number of k
+ * ranges and k-tiles (of 16) per range; out[4], out[5] tile rows and columns of the main block (kind 2), or out[4] the
+ * number of tiles computed whole (kind 3); out[6] the planner's estimate in microseconds.  Products served by the unstaged small-product kernels are not planned this way.
  * ctx may be null (256 compute units are assumed); nothing is launched. */
 int zg_hip_gemm_plan(zg_hip_ctx *ctx, size_t m, size_t n, size_t k, size_t batches, int64_t *out);
 

@@ -24,11 +24,13 @@ def _matmul(hip, A, B, C0, m, n, k, ta, tb, alpha, beta):
     return out
 
 
-# (3072, 3072, 3072): 128 x 128 tiles, 4 pieces of 48 k-tiles; (1536, 1536, 1234): 64 x 64 tiles, a k that ends inside a
+# tail in pieces: (3072, 3072, 3072): 128 x 128 tiles, 4 pieces of 48 k-tiles; (1536, 1536, 1234): 64 x 64 tiles, a k that ends inside a
 # k-tile, so the last piece is short and masked; (2560, 3328, 1024): 8 pieces of 8 k-tiles, the shortest range allowed
 @pytest.mark.parametrize("shape,kind", [((4100, 4100, 1030), "parts"), ((3600, 2308, 1541), "parts"),
                                         ((3072, 3072, 3072), "tail_in_pieces"), ((1536, 1536, 1234), "tail_in_pieces"),
-                                        ((2560, 3328, 1024), "tail_in_pieces")])
+                                        ((2560, 3328, 1024), "tail_in_pieces"),
+                                        # tiles that end inside C (the edge kernels), and a C that takes scalar stores
+                                        ((1498, 1530, 1000), "tail_in_pieces"), ((1498, 1531, 1003), "tail_in_pieces")])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 def test_products_launched_in_parts_or_with_the_tail_in_pieces_match_float64(hip, shape, kind, ta, tb):
     m, n, k = shape
@@ -62,9 +64,10 @@ def test_parts_and_split_products_are_exact_on_small_integers(hip):
         assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("wide,kind", [(3332, "parts"), (3328, "tail_in_pieces")])
-def test_fused_linear_entry_points_on_a_product_launched_in_parts_or_with_the_tail_in_pieces(hip, wide, kind):
-    Bt, I, O = 2560, 1024, wide  # batch, fan_in, fan_out
+@pytest.mark.parametrize("Bt,I,wide,kind", [(2560, 1024, 3332, "parts"), (2560, 1024, 3328, "tail_in_pieces"),
+                                            (1498, 1000, 1530, "tail_in_pieces"), (1498, 1003, 1531, "tail_in_pieces")])
+def test_fused_linear_entry_points_on_a_product_launched_in_parts_or_with_the_tail_in_pieces(hip, Bt, I, wide, kind):
+    O = wide  # batch Bt, fan_in I, fan_out O
     assert hip.gemm_plan(Bt, O, I)["kind"] == kind, hip.gemm_plan(Bt, O, I)
     r = np.random.default_rng(77)
     x = r.standard_normal((Bt, I)).astype(np.float32)
@@ -81,7 +84,7 @@ def test_fused_linear_entry_points_on_a_product_launched_in_parts_or_with_the_ta
     want = np.maximum(x.astype(np.float64) @ w.astype(np.float64).T + b, 0.0)
     assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
     # input gradient with the ReLU gate of the layer below: gx = (gy W) where act > 0
-    I2, O2 = wide, 1024
+    I2, O2 = wide, I
     assert hip.gemm_plan(Bt, I2, O2)["kind"] == kind
     gy = r.standard_normal((Bt, O2)).astype(np.float32)
     w2 = (r.standard_normal((O2, I2)) / np.sqrt(O2)).astype(np.float32)

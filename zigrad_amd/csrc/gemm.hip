@@ -263,7 +263,9 @@ __device__ __forceinline__ void tile_coords(unsigned id, unsigned tiles_m, unsig
 //                such a piece sticks out of the operand (M or N not a multiple of 4 with a non-k-contiguous operand)
 //                the last tiles load through bounded descriptors like the tail of a ragged k.  The loop is the fast loop.
 // MODE 2 (checked): every load checked and zero-filled; only for leading dimensions beyond 32-bit byte offsets.
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int MODE>
+// TAILS: the launch has its tail in pieces (GemmArgs::tail_part); instantiated for the 128 x 128 and 64 x 64 tiles only
+// (the 256 x 128 kernels' register budget has no room for it, and the planner never asks them).
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int MODE, bool TAILS = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     constexpr bool SAFE = MODE == 2;
     constexpr int BK = kBK;
@@ -286,7 +288,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     unsigned split = blockIdx.y;
     bool piece = false;     // a k range of a tail tile: goes to the partial buffer as it is
     unsigned piece_id = 0;
-    if (g.tail_splits) {
+    if constexpr (TAILS) {
         if (blockIdx.x < g.tail_first) {
             tile_coords(xcd_contiguous(blockIdx.x, g.tail_first), g.tiles_m, g.tiles_n, tm, tn);
         } else {
@@ -308,10 +310,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     const float* A = g.A + (z % g.nba) * g.a_chunk;
     const float* B = g.B + (z % g.nbb) * g.b_chunk;
     const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
-    // where the tile's element (0, 0) is stored, and the row pitch there
-    float* const c_org = piece ? g.tail_part + (size_t)piece_id * (BM * BN)
-                               : g.C + z * g.c_chunk + (size_t)split * g.split_stride + m0 * g.ldc + n0;
-    const size_t c_ld = piece ? (size_t)BN : g.ldc;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
@@ -326,7 +324,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     // this workgroup's range of k
-    const bool whole_k = g.tail_splits && !piece;
+    const bool whole_k = TAILS && !piece;
     const size_t k_begin = whole_k ? 0 : (size_t)split * g.split_tiles * BK;
     const size_t k_end = (whole_k || k_begin + g.split_tiles * BK >= g.K) ? g.K : k_begin + g.split_tiles * BK;
     // 32-bit tile counter: there is no scalar 64-bit ordered compare, and a vector compare in the loop costs MFMA time
@@ -534,6 +532,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     // instruction writes two 128-byte row segments; otherwise a lane owns TN adjacent columns and stores them as
     // one vector.  With beta != 0 the old values of a row of blocks are read together before any is used; C is
     // not read at all when beta == 0.
+    // where the tile's element (0, 0) is stored, and the row pitch there
+    float* const c_org = piece ? g.tail_part + (size_t)piece_id * (BM * BN)
+                               : g.C + z * g.c_chunk + (size_t)split * g.split_stride + m0 * g.ldc + n0;
+    const size_t c_ld = piece ? (size_t)BN : g.ldc;
     const float alpha = piece ? 1.f : g.alpha, beta = piece ? 0.f : g.beta;
     const bool use_c = beta != 0.f;
     // gated implies !use_c
@@ -551,7 +553,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     constexpr bool VEC_C = !SAFE && !B_KMAJOR && TN > 1;
     using VC = typename VecOf<VEC_C ? TN : 1>::type;
-    const bool vec_c = VEC_C && (MODE == 0 || g.c_vec != 0);  // edge kernels also serve a C that needs scalar stores
+    const bool vec_c = VEC_C && (MODE == 0 || g.c_vec != 0 || piece);  // edge kernels also serve a C that needs scalar stores
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         float res[TN][16], old[TN][16];
@@ -568,7 +570,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs g) {
         constexpr int RSTEP = A_KMAJOR ? 1 : TM;  // tile rows between consecutive block rows
         auto row_of = [&](int r) { return ((r >> 2) * 8 + (r & 3)) * RSTEP; };  // relative to block row lk*4
         auto in_range = [&](int j, int r) {
-            if (MODE == 0) return true;
+            if (MODE == 0 || piece) return true;  // a piece is a whole dense tile in the partial buffer
             const size_t row = m0 + wm0 + FA::index_of(i, lk * 4 + (r >> 2) * 8 + (r & 3));
             const size_t col = n0 + wn0 + FB::index_of(j, l32);
             return row < g.M && col < g.N;
@@ -647,11 +649,17 @@ static int launch_gemm(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajo
         g.flat_batches = (unsigned)batches;
         grid = dim3((unsigned)flat, 1, 1);
     }
-#define ZG_GEMM(AK, BKM, MD)                                                                                  \
-    do {                                                                                                      \
-        constexpr size_t lds_bytes = 2 * (size_t)(Tile<BM, AK>::ELEMS + Tile<BN, BKM>::ELEMS) * sizeof(float); \
-        static_assert(lds_bytes <= 64 * 1024, "tile buffers exceed the default dynamic LDS limit");           \
-        hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, MD>), grid, block, lds_bytes, ctx->stream, g);       \
+#define ZG_GEMM(AK, BKM, MD)                                                                                        \
+    do {                                                                                                            \
+        constexpr size_t lds_bytes = 2 * (size_t)(Tile<BM, AK>::ELEMS + Tile<BN, BKM>::ELEMS) * sizeof(float);       \
+        static_assert(lds_bytes <= 64 * 1024, "tile buffers exceed the default dynamic LDS limit");                 \
+        if constexpr (BM * BN <= 128 * 128 && MD != 2) {                                                            \
+            if (g.tail_splits) {                                                                                    \
+                hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, MD, true>), grid, block, lds_bytes, ctx->stream, g); \
+                break;                                                                                              \
+            }                                                                                                       \
+        }                                                                                                           \
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, AK, BKM, MD>), grid, block, lds_bytes, ctx->stream, g);             \
     } while (0)
 #define ZG_GEMM_LAYOUT(MD)                                      \
     do {                                                        \
@@ -895,14 +903,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(const float* P,
 }
 
 // The tail tiles of a product launched with its tail in pieces (GemmArgs::tail_part): C tile = alpha * (the tile's
-// pieces, added in piece order) + beta * C, then the extras.  A thread owns four adjacent columns of one row.
+// pieces, added in piece order) + beta * C, then the extras.  A thread owns four adjacent columns of one row; where C
+// is not fit for 16-byte accesses, or the four columns reach past n, it handles them one by one.
 template <int BM, int BN>
 __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(GemmArgs g) {
     constexpr unsigned V4 = BM * BN / 4, PER_TILE = V4 / 256;
     const unsigned t = blockIdx.x / PER_TILE, q = (blockIdx.x % PER_TILE) * 256 + threadIdx.x;
     unsigned tm, tn;
     tile_coords(g.tail_first + t, g.tiles_m, g.tiles_n, tm, tn);
-    const unsigned row = q / (BN / 4), col = (q % (BN / 4)) * 4;
+    const size_t row = (size_t)tm * BM + q / (BN / 4), col = (size_t)tn * BN + (q % (BN / 4)) * 4;
+    if (row >= g.M || col >= g.N) return;
     const float4* p = reinterpret_cast<const float4*>(g.tail_part + (size_t)t * g.tail_splits * (BM * BN)) + q;
     float4 acc = p[0];
     for (unsigned s0 = 1; s0 < g.tail_splits; s0 += 8) {  // eight pieces' loads in flight, added in piece order
@@ -920,28 +930,36 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(GemmArgs g) {
             }
         }
     }
-    const size_t at = ((size_t)tm * BM + row) * g.ldc + (size_t)tn * BN + col;
+    const size_t at = row * g.ldc + col;
+    const bool vec = g.c_vec != 0 && col + 4 <= g.N;
+    const int live = vec ? 4 : (int)(g.N - col < 4 ? g.N - col : 4);
     float r[4] = {g.alpha * acc.x, g.alpha * acc.y, g.alpha * acc.z, g.alpha * acc.w};
     if (g.beta != 0.f) {
-        const float4 old = *reinterpret_cast<const float4*>(g.C + at);
-        r[0] += g.beta * old.x;
-        r[1] += g.beta * old.y;
-        r[2] += g.beta * old.z;
-        r[3] += g.beta * old.w;
+        float old[4] = {0.f, 0.f, 0.f, 0.f};
+        if (vec) {
+            const float4 o = *reinterpret_cast<const float4*>(g.C + at);
+            old[0] = o.x, old[1] = o.y, old[2] = o.z, old[3] = o.w;
+        } else {
+            for (int j = 0; j < live; j++) old[j] = g.C[at + j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) r[j] += g.beta * old[j];
     }
     if (g.bias || g.relu) {
 #pragma unroll
         for (int j = 0; j < 4; j++)
-            r[j] = gemm_extras(r[j], g.bias != nullptr, g.bias ? g.bias[(size_t)tn * BN + col + j] : 0.f, g.relu != 0);
+            r[j] = gemm_extras(r[j], g.bias != nullptr, (g.bias && j < live) ? g.bias[col + j] : 0.f, g.relu != 0);
     }
     if (g.gate) {
-        const float4 gv = *reinterpret_cast<const float4*>(g.gate + at);
-        r[0] = gv.x <= 0.f ? 0.f : r[0];
-        r[1] = gv.y <= 0.f ? 0.f : r[1];
-        r[2] = gv.z <= 0.f ? 0.f : r[2];
-        r[3] = gv.w <= 0.f ? 0.f : r[3];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (j < live && g.gate[at + j] <= 0.f) r[j] = 0.f;
     }
-    *reinterpret_cast<float4*>(g.C + at) = make_float4(r[0], r[1], r[2], r[3]);
+    if (vec) {
+        *reinterpret_cast<float4*>(g.C + at) = make_float4(r[0], r[1], r[2], r[3]);
+    } else {
+        for (int j = 0; j < live; j++) g.C[at + j] = r[j];
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1092,22 +1110,32 @@ static GemmPlan gemm_plan_single(size_t m, size_t n, size_t k, size_t batches, s
 // of the last round is empty, and with the tail in pieces the larger tiles win again: 1536-cubed 69 -> 58 us
 // (64 x 64, s = 4), 2560-cubed 285 -> 243 us (64 x 64, s = 4), 3072-cubed 412 (in parts) -> 395 us (128 x 128, s = 4),
 // 3584-cubed 93.5 % of the matrix peak (128 x 128, s = 8).
+// (the 64 x 64 tile reads four times the operand bytes per flop of the 128 x 128 tile and falls to 0.85 when the
+// operands outgrow what the L2s and the Infinity Cache keep of them between tiles: 3000-cubed and up)
 static const double kRoundEff[3] = {0.975, 0.98, 0.92};
+constexpr double kSmallTileBigOperandsEff = 0.85;
+constexpr size_t kSmallTileBigOperands = (size_t)64 << 20;
 constexpr double kPieceFixedUs = 1.5, kTailReduceFixedUs = 3.0;
 
-static double gemm_rounds_us(int tile, double rounds, size_t k) {
+static double gemm_rounds_us(int tile, double rounds, size_t m, size_t n, size_t k) {
     const GemmTileKind& t = kGemmTiles[tile];
-    return kLaunchFixedUs + rounds * 2.0 * (double)(t.bm * t.bn) * (double)k / (kCuFlopsPerUs * kRoundEff[tile]);
+    const double eff = (tile == 2 && (m + n) * k * sizeof(float) > kSmallTileBigOperands) ? kSmallTileBigOperandsEff
+                                                                                           : kRoundEff[tile];
+    return kLaunchFixedUs + rounds * 2.0 * (double)(t.bm * t.bn) * (double)k / (kCuFlopsPerUs * eff);
 }
 
 static bool gemm_plan_tail(size_t m, size_t n, size_t k, size_t n_cu, GemmPlan* out) {
     const size_t kt_total = ceil_div_sz(k, kBK);
     bool found = false;
-    for (int t = 0; t < 3; t++) {
+    for (int t = 1; t < 3; t++) {  // the 128 x 128 and 64 x 64 kernels
         const size_t bm = kGemmTiles[t].bm, bn = kGemmTiles[t].bn;
-        if (m % bm || n % bn) continue;
-        const size_t T = (m / bm) * (n / bn), R = T / n_cu, L = T % n_cu;
+        const size_t T = ceil_div_sz(m, bm) * ceil_div_sz(n, bn), R = T / n_cu, L = T % n_cu;
         if (R == 0 || L == 0 || T >= 0x7fffffffull / 16) continue;
+        // Two 128 x 128 workgroups share a CU, and a CU that finishes early takes the next two in line: past three rounds
+        // the CUs have drifted far enough apart that the pieces pile up on a few of them (4608-cubed, five rounds: 1537 us
+        // against 1350 in parts; 5632-cubed, seven rounds: 2558 against 2502 whole).  The 64 x 64 tile runs six to eight
+        // workgroups per CU and keeps its gain (2560-cubed, six rounds: 286 -> 258 us).
+        if (t == 1 && R > 3) continue;
         for (size_t want = 2; want <= 8; want++) {
             size_t per = ceil_div_sz(kt_total, want);
             per += per & 1;
@@ -1115,7 +1143,7 @@ static bool gemm_plan_tail(size_t m, size_t n, size_t k, size_t n_cu, GemmPlan* 
             const size_t s = ceil_div_sz(kt_total, per);
             if (s < 2) continue;
             const size_t piece_rounds = ceil_div_sz(L * s, n_cu);
-            const double us = gemm_rounds_us(t, (double)R + (double)piece_rounds * (double)per / (double)kt_total, k) +
+            const double us = gemm_rounds_us(t, (double)R + (double)piece_rounds * (double)per / (double)kt_total, m, n, k) +
                               kPieceFixedUs * (double)piece_rounds + kTailReduceFixedUs +
                               (double)((s + 1) * L * bm * bn) * 4.0 / kReduceBytesPerUs;
             if (!found || us < out->us) {
@@ -1132,16 +1160,18 @@ static bool gemm_plan_tail(size_t m, size_t n, size_t k, size_t n_cu, GemmPlan* 
     return found;
 }
 
-static GemmPlan gemm_plan_compute(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth,
-                                  bool allow_tail = true) {
+static GemmPlan gemm_plan_compute(size_t n_cu, size_t m, size_t n, size_t k, size_t batches, int depth) {
     GemmPlan best = gemm_plan_compute_untailed(n_cu, m, n, k, batches, depth);
     GemmPlan tail;
-    if (allow_tail && batches == 1 && gemm_plan_tail(m, n, k, n_cu, &tail)) {
+    if (batches == 1 && depth == 0 && gemm_plan_tail(m, n, k, n_cu, &tail)) {
         // against the plan in hand priced the same way (a plain launch: its rounds at the measured efficiencies)
         double in_hand = best.us;
         if (best.kind == GemmPlan::kPlain)
-            in_hand = gemm_rounds_us(best.tile, (double)ceil_div_sz(gemm_tiles_of(best.tile, m, n, 1), n_cu), k);
-        if (tail.us < 0.95 * in_hand) return tail;
+            in_hand = gemm_rounds_us(best.tile, (double)ceil_div_sz(gemm_tiles_of(best.tile, m, n, 1), n_cu), m, n, k);
+        // Tiles that end inside C take the edge kernels, where the gain is less regular (4100 x 4100 x 1030 measured
+        // none at all with any tile or number of pieces, 3000-cubed 438 -> 391 us): the model has to promise more there.
+        const bool whole_tiles = m % kGemmTiles[tail.tile].bm == 0 && n % kGemmTiles[tail.tile].bn == 0;
+        if (tail.us < (whole_tiles ? 0.97 : 0.92) * in_hand) return tail;
     }
     return best;
 }
@@ -1177,15 +1207,13 @@ static GemmPlan gemm_plan_compute_untailed(size_t n_cu, size_t m, size_t n, size
     return best;
 }
 
-// allow_tail: C is fit for the fast kernels' vector stores (the pieces and their sums are written that way)
 static GemmPlan gemm_plan(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, size_t batches, bool a_kmajor, bool b_kmajor,
-                          int depth, bool allow_tail) {
+                          int depth) {
     if (!ctx->gemm_plans) ctx->gemm_plans = new GemmPlanCache();
-    const GemmPlanKey key{m, n, k, batches,
-                          (a_kmajor ? 1 : 0) | (b_kmajor ? 2 : 0) | (depth ? 4 : 0) | (allow_tail ? 8 : 0)};
+    const GemmPlanKey key{m, n, k, batches, (a_kmajor ? 1 : 0) | (b_kmajor ? 2 : 0) | (depth ? 4 : 0)};
     auto it = ctx->gemm_plans->plans.find(key);
     if (it != ctx->gemm_plans->plans.end()) return it->second;
-    const GemmPlan best = gemm_plan_compute((size_t)ctx->n_cu, m, n, k, batches, depth, allow_tail);
+    const GemmPlan best = gemm_plan_compute((size_t)ctx->n_cu, m, n, k, batches, depth);
     ctx->gemm_plans->plans[key] = best;
     return best;
 }
@@ -1417,7 +1445,7 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     }
 
     // ---- plan: which tile, whether k is cut, whether C is cut into a block of whole rounds plus strips ----
-    const GemmPlan plan = gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth, c_vec && small_ld);
+    const GemmPlan plan = gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth);
     if (plan.kind == GemmPlan::kParts) {
         // C = [ main | right ] over [ bottom ]: main is rm x rn whole large tiles (a whole number of rounds, or nearly),
         // the strips are products of their own and go through this function again (they may cut k, not C).
@@ -1489,13 +1517,12 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
         g.tail_splits = (unsigned)plan.splits;
         g.tail_part = part;
         g.split_tiles = plan.per;
-        int rc = tile == 0   ? launch_gemm<256, 128>(ctx, g, a_kmajor, b_kmajor, 0, 1)
-                 : tile == 1 ? launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, 0, 1)
-                             : launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 0, 1);
+        const int md = mode(bm, bn);
+        int rc = tile == 1 ? launch_gemm<128, 128>(ctx, g, a_kmajor, b_kmajor, md, 1)
+                           : launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, md, 1);
         if (rc) return rc;
         const unsigned blocks = (unsigned)(tail_tiles * (bm * bn / 1024));
-        if (tile == 0) hipLaunchKernelGGL((gemm_tail_reduce_kernel<256, 128>), dim3(blocks), dim3(256), 0, ctx->stream, g);
-        else if (tile == 1) hipLaunchKernelGGL((gemm_tail_reduce_kernel<128, 128>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+        if (tile == 1) hipLaunchKernelGGL((gemm_tail_reduce_kernel<128, 128>), dim3(blocks), dim3(256), 0, ctx->stream, g);
         else hipLaunchKernelGGL((gemm_tail_reduce_kernel<64, 64>), dim3(blocks), dim3(256), 0, ctx->stream, g);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
@@ -1508,8 +1535,6 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
 // The workspace a single product of this shape asks for when it is dispatched (the partial tiles of a k that is cut),
 // following gemm_dispatch_body's choices.  A product that waits reserves it when it is queued, so that the call
 // which later launches it, whichever that is, allocates nothing.
-static size_t gemm_workspace_need_untailed(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b,
-                                           size_t lda, size_t ldb, int depth);
 static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda,
                                   size_t ldb, int depth) {
     if (m == 0 || n == 0 || k == 0) return 0;
@@ -1526,21 +1551,11 @@ static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k,
         splits = ceil_div_sz(groups, per);
         return splits * m * n * sizeof(float);
     }
-    // whether C will be fit for vector stores is not known here: the larger of the two plans' needs
-    const GemmPlan tailed = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth, true);
-    size_t tail_need = 0;
-    if (tailed.kind == GemmPlan::kTail) {
-        const size_t bm = kGemmTiles[tailed.tile].bm, bn = kGemmTiles[tailed.tile].bn;
-        tail_need = ((m / bm) * (n / bn) - tailed.whole) * tailed.splits * bm * bn * sizeof(float);
+    const GemmPlan plan = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth);
+    if (plan.kind == GemmPlan::kTail) {
+        const size_t bm = kGemmTiles[plan.tile].bm, bn = kGemmTiles[plan.tile].bn;
+        return (ceil_div_sz(m, bm) * ceil_div_sz(n, bn) - plan.whole) * plan.splits * bm * bn * sizeof(float);
     }
-    const size_t other_need = gemm_workspace_need_untailed(ctx, m, n, k, trans_a, trans_b, lda, ldb, depth);
-    return tail_need > other_need ? tail_need : other_need;
-}
-
-static size_t gemm_workspace_need_untailed(zg_hip_ctx* ctx, size_t m, size_t n, size_t k, int trans_a, int trans_b,
-                                           size_t lda, size_t ldb, int depth) {
-    const bool a_kmajor = !trans_a, b_kmajor = trans_b != 0;
-    const GemmPlan plan = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth, false);
     if (plan.kind == GemmPlan::kParts) {
         const size_t m1 = plan.rm * 256, n1 = plan.rn * 128;
         const size_t shapes[3][2] = {{m1, n1}, {m1, n - n1}, {m - m1, n}};

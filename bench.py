@@ -577,8 +577,8 @@ def cpu_baseline(dims, batch, budget_steps=2, threads=None, loss_mode="onehot"):
 
 
 VENDOR_SHAPES = [(4096, 4096, 4096, 1), (512, 512, 512, 32), (4096, 1024, 4096, 1), (3072, 3072, 3072, 1), (4100, 4100, 4100, 1),
-                 (2048, 2048, 2048, 1), (1536, 1536, 1536, 1), (1024, 1024, 1024, 1), (768, 768, 768, 1), (64, 128, 784, 1),
-                 (2708, 16, 1433, 1)]
+                 (3584, 3584, 3584, 1), (3000, 3000, 3000, 1), (2560, 2560, 2560, 1), (2048, 2048, 2048, 1), (1792, 1792, 1792, 1),
+                 (1536, 1536, 1536, 1), (1024, 1024, 1024, 1), (768, 768, 768, 1), (64, 128, 784, 1), (2708, 16, 1433, 1)]
 
 
 def vendor_gemm_child():

@@ -43,6 +43,7 @@ class _Run:
         self.lr_slot = hip.mem_alloc(F32, 1)
         self.u64_out = hip.mem_alloc(np.uint64, 4096)
         self.plan = hip.edge_plan(self.src, self.tgt, n_nodes)
+        self.long = None    # index arrays long enough for the orderings kept by address (made on first use)
         self.reads = []
         self.t = 0
         self.last_c = None
@@ -253,6 +254,49 @@ class _Run:
             self.hip.dispatch("add", x=dst, y=other, z=other)
             self.done()
             self.hip.dispatch("tanh_fwd", x=other, y=other)      # (rsqrt of arbitrary data would bring NaNs in)
+
+    def op_scatter_long(self):
+        """Index arrays of 270000 entries in device memory: their orderings are kept under the arrays' addresses and
+        checked on the GPU by every call; the arrays are rewritten in place now and then (a device copy), and what waits
+        in the context when the ordering is rebuilt (an aggregation waiting for its bias, a count) must not be lost."""
+        n_nodes, n = self.graph[0], 270_000
+        if self.long is None:
+            init = np.random.default_rng(self.seed + 20_000)
+            mk = lambda hi: self.hip.from_numpy(init.integers(0, hi, n).astype(np.uint64))
+            self.long = {"offs": mk(300), "offs_alt": [mk(300), mk(300)], "src": mk(n_nodes), "tgt": mk(n_nodes),
+                         "tgt_alt": [mk(n_nodes), mk(n_nodes)],
+                         "vals": self.hip.from_numpy((init.standard_normal(n) * 0.01).astype(np.float32))}
+        L = self.long
+        if self.r.random() < 0.35:
+            which = int(self.r.integers(0, 2))
+            if self.r.random() < 0.5:
+                self.hip.mem_copy(L["offs_alt"][which], L["offs"])
+            else:
+                self.hip.mem_copy(L["tgt_alt"][which], L["tgt"])
+            self.done()
+        if self.r.random() < 0.5:
+            nb = int(self.r.choice([150, 300]))
+            dst = self.pick(nb)
+            if self.r.random() < 0.6:
+                self.hip.mem_fill(dst, 0.0)
+                self.done()
+            self.hip.dispatch("scatter_add", src=L["vals"], offsets=L["offs"], dst=dst)
+        else:
+            stride = 4
+            y, h, deg, bias = self.picks(n_nodes * stride, n_nodes * stride, n_nodes, stride)
+            self.hip.dispatch("scale", x=h, alpha=0.01)      # 270000 edges into 40 nodes: keep the sums small
+            self.done()
+            if self.r.random() < 0.6:
+                self.hip.mem_fill(y, 0.0)
+                self.done()
+            self.hip.dispatch("scatter_gcn_deg_scaled", dst=y, h=h, deg=deg, src_indices=L["src"], tgt_indices=L["tgt"],
+                              stride=stride, n_edge=n)
+            self.done()
+            if self.r.random() < 0.7:
+                self.hip.dispatch("add", x=bias, y=y, z=y)
+                self.done()
+            if self.r.random() < 0.4:       # the next long call finds the aggregation still waiting
+                self.hip.dispatch("scatter_add", src=L["vals"], offsets=L["offs"], dst=self.pick(300))
 
     def op_max_along(self):
         rows, cols = int(self.r.choice([8, 64])), int(self.r.choice([2, 7, 33]))
@@ -589,8 +633,8 @@ class _Run:
         ops = [self.op_fill, self.op_matmul, self.op_add_row, self.op_relu, self.op_relu_mask, self.op_layer_backward,
                self.op_unbroadcast, self.op_step, self.op_scatter, self.op_alloc, self.op_free, self.op_read, self.op_copy,
                self.op_elementwise, self.op_scatter_bwd, self.op_loss, self.op_map_run, self.op_scatter_add,
-               self.op_max_along, self.op_plain]
-        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1, 3, 1, 1, 6], float)
+               self.op_max_along, self.op_plain, self.op_scatter_long]
+        weights = np.array([3, 4, 3, 3, 2, 2, 2, 3, 2, 1, 2, 1, 1, 1, 1, 1, 3, 1, 1, 6, 0.5], float)
         self.trace = []
         for _ in range(n_ops):
             op = ops[int(self.r.choice(len(ops), p=weights / weights.sum()))]
@@ -612,6 +656,10 @@ class _Run:
         for m, v in self.moments:
             out += [self.hip.to_numpy(m).view(np.uint32).copy(), self.hip.to_numpy(v).view(np.uint32).copy()]
         self.plan.free()
+        if self.long is not None:
+            for v in self.long.values():
+                for b in (v if isinstance(v, list) else [v]):
+                    self.hip.mem_free(b)
         for b in self.bufs + [self.src, self.tgt, self.offs, self.idx, self.row_ptr, self.seg_bounds, self.u64_out, self.lr_slot] + \
                 [x for mv in self.moments for x in mv]:
             self.hip.mem_free(b)
@@ -676,7 +724,7 @@ def test_the_sequences_call_every_op_entry_point_the_header_declares(hip, monkey
         return real(name, *args)
 
     monkeypatch.setattr(hip._lib, "call", recording)
-    for seed in range(60):
+    for seed in range(200):
         _Run(hip, seed, eager=False).run(80)
     declared = set(parse_header())
     missing = declared - NOT_IN_SEQUENCES - called

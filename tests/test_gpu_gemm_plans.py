@@ -134,6 +134,49 @@ def test_tall_narrow_products_of_k_contiguous_operands(hip, shape):
     assert np.array_equal(fused, y)
 
 
+@pytest.mark.parametrize("shape", [(64, 128, 784), (100, 30, 384), (100, 30, 383), (256, 256, 2048), (256, 256, 2049),
+                                   (250, 251, 1000), (257, 256, 600), (17, 33, 2047), (16, 16, 400), (64, 128, 1433)])
+def test_deep_products_of_k_contiguous_operands_either_side_of_the_one_launch_kernels_limits(hip, shape):
+    """[m, k] x [n, k]^T with 384 <= k <= 2048 on at most 256 blocks of 16 x 16 takes one launch of a kernel of its own
+    (a Linear layer's forward at a small batch); the shapes here sit on both sides of each limit, with edges inside a
+    block, a k that ends inside a chunk of 16 and inside a 16-byte piece: against float64, accumulating, with padded
+    leading dimensions, exact on small integers, and with bias and ReLU against the three separate ops."""
+    m, n, k = shape
+    r = np.random.default_rng(m * 7 + n * 3 + k)
+    A = r.standard_normal((m, k), dtype=np.float32)
+    B = r.standard_normal((n, k), dtype=np.float32)
+    C0 = r.standard_normal((m, n), dtype=np.float32)
+    prod = A.astype(np.float64) @ B.astype(np.float64).T
+    got = _matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, False, True, 1.0, 0.0)
+    assert np.linalg.norm(got - prod) <= TOL * np.linalg.norm(prod)
+    assert np.abs(got - prod).max() <= 8 * TOL * np.sqrt(k)
+    got = _matmul(hip, A, B, C0, m, n, k, False, True, 0.25, -2.0)
+    want = 0.25 * prod - 2.0 * C0
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+    Ai = r.integers(-3, 4, (m, k)).astype(np.float32)
+    Bi = r.integers(-3, 4, (n, k)).astype(np.float32)
+    got = _matmul(hip, Ai, Bi, np.zeros((m, n), np.float32), m, n, k, False, True, 1.0, 0.0)
+    assert np.array_equal(got, (Ai.astype(np.int64) @ Bi.astype(np.int64).T).astype(np.float32))
+    # views into wider matrices: row strides k + 3 and k + 1 (rows that start at any 4-byte alignment), an output wider than n
+    Aw, Bw = r.standard_normal((m, k + 3), dtype=np.float32), r.standard_normal((n, k + 1), dtype=np.float32)
+    a, b, c = hip.from_numpy(Aw), hip.from_numpy(Bw), hip.from_numpy(np.full((m, n + 5), 7.0, np.float32))
+    hip.dispatch("matmul", A=a, B=b, C=c, m=m, n=n, k=k, trans_a=False, trans_b=True, lda=k + 3, ldb=k + 1, ldc=n + 5,
+                 alpha=1.0, beta=0.0)
+    out = hip.to_numpy(c).reshape(m, n + 5)
+    want = Aw[:, :k].astype(np.float64) @ Bw[:, :k].astype(np.float64).T
+    assert np.linalg.norm(out[:, :n] - want) <= TOL * np.linalg.norm(want)
+    assert np.all(out[:, n:] == 7.0)
+    for x in (a, b, c):
+        hip.mem_free(x)
+    bias = r.standard_normal(n).astype(np.float32)
+    fused = run_op(hip, "linear_fwd", {"x": A, "w": B, "bias": bias, "y": np.full((m, n), np.nan, np.float32), "batch": m,
+                                       "fan_in": k, "fan_out": n, "relu": True}, ["y"])["y"].reshape(m, n)
+    y = _matmul(hip, A, B, np.zeros((m, n), np.float32), m, n, k, False, True, 1.0, 0.0)
+    y = run_op(hip, "add", {"x": bias, "y": y, "z": np.zeros_like(y)}, ["z"])["z"]
+    y = run_op(hip, "relu_fwd", {"x": y, "y": np.zeros_like(y)}, ["y"])["y"].reshape(m, n)
+    assert np.array_equal(fused, y)
+
+
 def test_tall_narrow_product_is_exact_on_small_integers(hip):
     m, n, k = 2708, 16, 1433
     r = np.random.default_rng(4)

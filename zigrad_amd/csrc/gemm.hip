@@ -821,6 +821,81 @@ static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_
     return ZG_HIP_OK;
 }
 
+// Deep products on a few blocks (a Linear layer's forward at a small batch: 64 x 128 over k = 784; the graph
+// convolution's first layer, 2708 x 16 over k = 1433): C = alpha * A B^T + beta * C with both operands k-contiguous, one
+// 16 x 16 block of C per workgroup, so that even 64 x 128 gives 32 workgroups something to fetch.  The four waves deal
+// k out in chunks of 16 (wave w takes chunks w, w + 4, ...); lane (r, q) of a wave loads values 4 q .. 4 q + 3 of its
+// chunk for row r of A and for column r of B, sixteen bytes each, twelve chunks' loads in flight before the first is
+// used, and element c of the two pieces feeds MFMA c of the chunk (v_mfma_f32_16x16x4_f32 adds over q in hardware).
+// The waves' blocks are added in wave order through LDS; thread t finishes C element (t / 16, t % 16).  One launch
+// where cutting k over workgroups takes two: 64 x 128 x 784 7.8 -> 5.4 us, 2708 x 16 x 1433 12.3 -> 7.8 us,
+// 256 x 256 x 1024 9.9 -> 6.6 us.
+constexpr int kDeepBatch = 12;  // chunks in flight per wave
+
+__global__ __launch_bounds__(256) void gemm_deep_kernel(GemmArgs g) {
+    __shared__ float part[4][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const size_t tm = blockIdx.x / g.tiles_n, tn = blockIdx.x % g.tiles_n;
+    size_t row = tm * 16 + r, col = tn * 16 + r;
+    if (row >= g.M) row = g.M - 1;  // rows and columns past the edge repeat the last one; their sums are never stored
+    if (col >= g.N) col = g.N - 1;
+    // 16-byte buffer loads (served at any 4-byte alignment) from the block's first row, lane offsets in bytes
+    typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+    const float* a_rows = g.A + tm * 16 * g.lda;
+    const float* b_rows = g.B + tn * 16 * g.ldb;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a_rows), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(b_rows), 0, -1, 0x00020000);
+    const unsigned a_off = (unsigned)(((row - tm * 16) * g.lda + 4 * q) * sizeof(float));
+    const unsigned b_off = (unsigned)(((col - tn * 16) * g.ldb + 4 * q) * sizeof(float));
+    const unsigned chunks = (unsigned)((g.K + 15) / 16);
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    // four values of k from chunk * 16 + 4 q on, zeros past K (the one chunk that K ends in loads value by value)
+    auto piece = [&](__amdgpu_buffer_rsrc_t rsrc, const float* rows, unsigned off, unsigned chunk) {
+        const unsigned k0 = chunk * 16 + 4 * (unsigned)q;
+        if (k0 + 4 <= g.K) return __builtin_bit_cast(floatx4, (uintx4)__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(off + chunk * 64), 0, 0));
+        floatx4 p;
+#pragma unroll
+        for (int c = 0; c < 4; c++) p[c] = (k0 + c < g.K) ? rows[off / 4 + chunk * 16 + c] : 0.f;
+        return p;
+    };
+    for (unsigned c0 = wave; c0 < chunks; c0 += 4 * kDeepBatch) {
+        floatx4 av[kDeepBatch], bv[kDeepBatch];
+#pragma unroll
+        for (int i = 0; i < kDeepBatch; i++) {
+            const unsigned chunk = c0 + 4 * i;
+            if (chunk < chunks) {
+                av[i] = piece(a_rsrc, a_rows, a_off, chunk);
+                bv[i] = piece(b_rsrc, b_rows, b_off, chunk);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kDeepBatch; i++) {
+            if (c0 + 4 * i < chunks) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i][c], bv[i][c], acc, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) part[wave][lane][i] = acc[i];
+    __syncthreads();
+    // accumulator i of lane (r, q) is C element (4 q + i, r) of the block
+    const int er = threadIdx.x >> 4, ec = threadIdx.x & 15;
+    const int src_lane = (er >> 2) * 16 + ec, src_i = er & 3;
+    float sum = part[0][src_lane][src_i];
+#pragma unroll
+    for (int w = 1; w < 4; w++) sum += part[w][src_lane][src_i];
+    const size_t orow = tm * 16 + er, ocol = tn * 16 + ec;
+    if (orow >= g.M || ocol >= g.N) return;
+    const size_t at = orow * g.ldc + ocol;
+    float v = g.alpha * sum;
+    if (g.beta != 0.f) v += g.beta * g.C[at];
+    v = gemm_extras(v, g.bias != nullptr, g.bias ? g.bias[ocol] : 0.f, g.relu != 0);
+    if (g.gate && g.gate[at] <= 0.f) v = 0.f;
+    g.C[at] = v;
+}
+
 // C = alpha * (sum of the split-K partial products, in split order) + beta * C.  P is [batch][split][M][N] dense.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, float* C, size_t M, size_t N, size_t ldc,
                                                             int splits, float alpha, float beta, size_t c_chunk,
@@ -1274,6 +1349,15 @@ static bool gemm_is_tiny(size_t m, size_t n, size_t k, size_t batches, size_t ld
     return small_ld && ((k <= 256 && blocks <= n_cu) || (k <= 512 && blocks <= 16));
 }
 
+// One unbatched product of k-contiguous operands with a long k on at most a CU's worth of 16 x 16 blocks: gemm_deep_kernel.
+// (Below k = 384 the unstaged kernel or one round of 64 x 64 tiles does as well.  A load instruction of this kernel
+// touches 64 bytes in each of 16 rows, which the memory system serves slowly when the rows are far apart: at k = 4096
+// a workgroup's loads take 19 us and the staged kernels with k cut over workgroups win again; measured break-even
+// between k = 2048 and 3072.)
+static bool gemm_is_deep(size_t m, size_t n, size_t k, size_t batches, bool a_kmajor, bool b_kmajor, size_t n_cu) {
+    return batches == 1 && a_kmajor && b_kmajor && k >= 384 && k <= 2048 && ceil_div_sz(m, 16) * ceil_div_sz(n, 16) <= n_cu;
+}
+
 static int gemm_validate(const char* name, const float* A, const float* B, const float* C, size_t m, size_t n, size_t k,
                          int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc) {
     ZG_REQUIRE(A && B && C, "%s: null pointer", name);
@@ -1410,6 +1494,13 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
 
     if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
     if (gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
+    if (gemm_is_deep(m, n, k, batches, a_kmajor, b_kmajor, n_cu)) {
+        g.tiles_m = (unsigned)ceil_div_sz(m, 16);
+        g.tiles_n = (unsigned)ceil_div_sz(n, 16);
+        hipLaunchKernelGGL(gemm_deep_kernel, dim3(g.tiles_m * g.tiles_n), dim3(256), 0, ctx->stream, g);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     // Skinny weight-gradient products with a long k (one side of C at most 32 wide, both operands stored k-strided:
     // the 16-wide layer of the GCN, 16 x 1433 over 2708 nodes): 64-wide tiles would compute mostly padding, so the
     // unstaged kernel takes ranges of k (one round of 256 per workgroup, at most 32 ranges) and the split-k reduction
@@ -1542,6 +1633,7 @@ static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k,
     const size_t n_cu = (size_t)ctx->n_cu;
     const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
     if (!small_ld || gemm_is_tiny(m, n, k, 1, lda, ldb, n_cu)) return 0;
+    if (gemm_is_deep(m, n, k, 1, a_kmajor, b_kmajor, n_cu)) return 0;
     if (!a_kmajor && !b_kmajor && (m <= 32 || n <= 32) && k > 512 && ceil_div_sz(m, 32) * ceil_div_sz(n, 32) <= n_cu) {
         const size_t groups = ceil_div_sz(k, 8);
         size_t splits = ceil_div_sz(groups, 32);

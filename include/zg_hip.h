@@ -229,7 +229,9 @@ int zg_hip_gemm_timing_read(zg_hip_ctx *ctx, double *total_ms, uint64_t *product
  * same launch, the tiles that would start one more (mostly empty) round cut along k into pieces, which a second kernel
  * adds tile by tile in a fixed order; out[1] tile: 0 = 256 x 128, 1 = 128 x 128, 2 = 64 x 64; out[2], out[3] number of k
  * ranges and k-tiles (of 16) per range; out[4], out[5] tile rows and columns of the main block (kind 2), or out[4] the
- * number of tiles computed whole (kind 3); out[6] the planner's estimate in microseconds.  Products served by the unstaged small-product kernels are not planned this way.
+ * number of tiles computed whole (kind 3); out[6] the planner's estimate in microseconds.  Products served by the
+ * unstaged small-product kernels, or by the one-launch kernel for deep products of k-contiguous operands on a few
+ * blocks (384 <= k <= 2048, at most a CU's worth of 16 x 16 blocks of C), are not planned this way.
  * ctx may be null (256 compute units are assumed); nothing is launched. */
 int zg_hip_gemm_plan(zg_hip_ctx *ctx, size_t m, size_t n, size_t k, size_t batches, int64_t *out);
 

@@ -48,7 +48,7 @@ def _tally(hip):
 @pytest.mark.parametrize("where", ["device", "pinned"])
 def test_scatter_add_follows_an_array_rewritten_in_place(oracle, hip, where):
     r = np.random.default_rng(3)
-    n_dst = 70_000   # three 8-bit passes
+    n_dst = 70_000   # 17 bits of destination: two 9-bit passes
     off = r.integers(0, n_dst, N).astype(np.uint64)
     src = r.standard_normal(N).astype(np.float32)
     dst0 = r.standard_normal(n_dst).astype(np.float32)

@@ -92,11 +92,12 @@ def test_index_select_bwd_and_gcn_with_a_hub_equal_the_host_loops(oracle, hip):
 
 
 @pytest.mark.parametrize("n", [262143, 262144, 262145, 266241, 300000])
-@pytest.mark.parametrize("n_dst", [1, 255, 256, 257, 65535, 65536, 1 << 20])
+@pytest.mark.parametrize("n_dst", [1, 255, 256, 257, 511, 512, 65535, 65536, 262143, 262144, 1 << 20])
 def test_scatter_add_either_side_of_the_radix_build_limits(oracle, hip, n, n_dst):
-    """From 262144 entries on the destination ordering is built by a stable radix sort, 8 bits a pass: one, two and three
-    passes (n_dst up to 255, 65535, beyond), tiles that end inside the input, the shortest input that takes this build and
-    the longest that does not.  Equal to the host's sequential loop bit for bit."""
+    """From 262144 entries on the destination ordering is built by a stable radix sort, 8 bits a pass, or 9 where that
+    saves a pass: one pass of 8 (n_dst up to 255) or of 9 (up to 511), two of 8 (up to 65535) or of 9 (up to 262143),
+    three beyond; tiles that end inside the input, the shortest input that takes this build and the longest that does
+    not.  Equal to the host's sequential loop bit for bit."""
     r = np.random.default_rng(n * 31 + n_dst)
     off = r.integers(0, n_dst, n).astype(np.uint64)
     src = r.standard_normal(n).astype(np.float32)

@@ -54,7 +54,9 @@ static size_t align_up(size_t v, size_t a) {
 // 1100 us against 510 us; at a quarter of a million entries the two take the same time.
 constexpr size_t kRadixMinEntries = (size_t)1 << 18;
 constexpr int kRxThreads = 256, kRxPerThread = 16, kRxTile = kRxThreads * kRxPerThread;  // entries per workgroup
-constexpr int kRxBits = 8, kRxBins = 1 << kRxBits;                                       // digit width
+// digit width: 8 bits a pass, or 9 where that saves a pass (17, 18 and 25 to 27 bits of bucket number: two passes instead
+// of three for 65 K to 262 K buckets); the kernels take it as a template argument
+constexpr int kRxMaxBins = 512;
 static bool radix_build_applies(size_t n, size_t nb) {
     return n >= kRadixMinEntries && nb < ((size_t)1 << 31);
 }
@@ -64,7 +66,7 @@ static size_t plan_bytes(size_t n, size_t nb) {
     size_t bytes = align_up((nb + 1) * 4, 256) + align_up(nb * 4, 256) + 4 * align_up(n * 4, 256) +
                    align_up((tiles + 1) * 4, 256) + align_up((n / kLongBucket + 2) * 4, 256);
     if (radix_build_applies(n, nb))
-        bytes += 3 * align_up(n * 4, 256) + align_up(ceil_div_sz(n, kRxTile) * kRxBins * 4, 256);
+        bytes += 3 * align_up(n * 4, 256) + align_up(ceil_div_sz(n, kRxTile) * kRxMaxBins * 4, 256);
     return bytes;
 }
 
@@ -329,22 +331,24 @@ __global__ __launch_bounds__(kOrderLongThreads) void order_long_segments_kernel(
 // ------------------------------------------------------------------------------------------------
 // A kept plan is rebuilt only when the arrays it was built from have changed.  `gate` (null: build unconditionally) is
 // two words in device memory.  The first kernel of a build compares the arrays with the 32-bit copies the plan keeps
-// (keys32, peer0), brings the copies up to date and sets gate[0] where it finds a difference; the first scan (one
-// workgroup) moves gate[0] to gate[1] and clears gate[0] for the next build; every later kernel returns at once when
-// gate[1] is zero.  No kernel reads a word that another workgroup of the same launch writes.
+// (keys32, peer0), brings the copies up to date and sets gate[0] where it finds a difference; the first scan copies
+// gate[0] to gate[1]; every later kernel returns at once when gate[1] is zero, and the first scatter pass, which reads
+// gate[1] only, clears gate[0] for the next build.  No kernel reads a word that another workgroup of the same launch
+// writes.
 struct RxGate {
     const uint32_t* in = nullptr;  // the kernel runs when this is null or points at a non-zero word
-    uint32_t* move_to = nullptr;   // first scan only: receives *in ...
-    uint32_t* clear = nullptr;     // ... and this word (the one the compare kernel sets) is cleared
+    uint32_t* move_to = nullptr;   // first scan only: receives *in
     uint32_t* tally = nullptr;     // first scan only: [0] builds skipped, [1] builds done, in device memory ...
     uint32_t* tally_host = nullptr;  // ... and mirrored into pinned host memory, where the host reads it without waiting
 };
 
+template <int BITS>
 __global__ __launch_bounds__(kRxThreads) void rx_count_first_kernel(const uint64_t* keys, const uint64_t* payload, size_t n,
                                                                     uint32_t nb, uint32_t* keys32, uint32_t* peer0,
                                                                     uint32_t* counts, uint32_t* gate) {
+    constexpr int kRxBins = 1 << BITS;
     __shared__ uint32_t hist[kRxBins];
-    hist[threadIdx.x] = 0;
+    for (int i = threadIdx.x; i < kRxBins; i += kRxThreads) hist[i] = 0;
     __syncthreads();
     const size_t base = (size_t)blockIdx.x * kRxTile;
     bool changed = false;
@@ -375,14 +379,16 @@ __global__ __launch_bounds__(kRxThreads) void rx_count_first_kernel(const uint64
     }
     if (gate && __any(changed) && (threadIdx.x & 63) == 0) gate[0] = 1u;  // every writer stores the same value
     __syncthreads();
-    counts[(size_t)blockIdx.x * kRxBins + threadIdx.x] = hist[threadIdx.x];
+    for (int i = threadIdx.x; i < kRxBins; i += kRxThreads) counts[(size_t)blockIdx.x * kRxBins + i] = hist[i];
 }
 
+template <int BITS>
 __global__ __launch_bounds__(kRxThreads) void rx_count_kernel(const uint32_t* keys32, size_t n, int shift, uint32_t* counts,
                                                               const uint32_t* gate) {
     if (gate && *gate == 0) return;
+    constexpr int kRxBins = 1 << BITS;
     __shared__ uint32_t hist[kRxBins];
-    hist[threadIdx.x] = 0;
+    for (int i = threadIdx.x; i < kRxBins; i += kRxThreads) hist[i] = 0;
     __syncthreads();
     const size_t base = (size_t)blockIdx.x * kRxTile;
 #pragma unroll 4
@@ -391,34 +397,38 @@ __global__ __launch_bounds__(kRxThreads) void rx_count_kernel(const uint32_t* ke
         if (e < n) atomicAdd(&hist[(keys32[e] >> shift) & (kRxBins - 1)], 1u);
     }
     __syncthreads();
-    counts[(size_t)blockIdx.x * kRxBins + threadIdx.x] = hist[threadIdx.x];
+    for (int i = threadIdx.x; i < kRxBins; i += kRxThreads) counts[(size_t)blockIdx.x * kRxBins + i] = hist[i];
 }
 
 // counts[tile][digit] -> first output position of that tile's entries with that digit: all of digit 0 by tile, then
-// all of digit 1, ...  One workgroup of 1024 threads: thread (part, d) owns a quarter of the tiles of digit d, so a
-// thread's two walks over its counts are a few batches of independent loads (a thread per digit took 20 us on 245 tiles).
-constexpr int kRxScanParts = 4;
-__global__ __launch_bounds__(kRxBins * kRxScanParts) void rx_scan_kernel(uint32_t* __restrict__ counts, size_t n_tiles,
-                                                                         RxGate gate, uint32_t* long_list) {
+// all of digit 1, ...  A workgroup of 1024 threads takes 256 digits: thread (part, d) owns a quarter of the tiles of
+// digit d, so a thread's two walks over its counts are a few batches of independent loads (a thread per digit took
+// 20 us on 245 tiles, and so did one workgroup for 512 digits).  With 9-bit digits a second workgroup takes the upper
+// 256 and finds what lies before them without the first one's help.
+constexpr int kRxScanThreads = 1024, kRxScanDigits = 256, kRxScanParts = kRxScanThreads / kRxScanDigits;
+template <int BITS>
+__global__ __launch_bounds__(kRxScanThreads) void rx_scan_kernel(uint32_t* __restrict__ counts, size_t n_tiles, RxGate gate,
+                                                                  uint32_t* long_list, uint32_t n_entries) {
+    constexpr int kRxBins = 1 << BITS;
+    static_assert(kRxBins <= 2 * kRxScanDigits, "the second workgroup finds its base from the total: two groups at most");
     if (gate.in) {
+        // every workgroup of this launch reads the word; the one that set it is cleared by a later launch (the first
+        // scatter pass), which does not read it
         const uint32_t go = *gate.in;
-        if (gate.move_to) {      // the first scan of a gated build: one workgroup, so every thread has read the word
-            __syncthreads();     // before thread 0 clears it
-            if (threadIdx.x == 0) {
-                *gate.move_to = go;
-                *gate.clear = 0u;
-                const uint32_t seen = gate.tally[go ? 1 : 0] + 1u;
-                gate.tally[go ? 1 : 0] = seen;
-                gate.tally_host[go ? 1 : 0] = seen;
-            }
+        if (gate.move_to && blockIdx.x == 0 && threadIdx.x == 0) {
+            *gate.move_to = go;
+            const uint32_t seen = gate.tally[go ? 1 : 0] + 1u;
+            gate.tally[go ? 1 : 0] = seen;
+            gate.tally_host[go ? 1 : 0] = seen;
         }
         if (go == 0) return;
     }
-    if (long_list && threadIdx.x == 0) long_list[0] = 0;  // first scan: the finish kernel appends to the list
-    __shared__ uint32_t part_sum[kRxScanParts][kRxBins];
-    __shared__ uint32_t digit_base[kRxBins];
-    __shared__ uint32_t wave_tot[kRxBins / 64];
-    const int d = threadIdx.x & (kRxBins - 1), part = threadIdx.x / kRxBins;
+    if (long_list && blockIdx.x == 0 && threadIdx.x == 0) long_list[0] = 0;  // first scan: the finish kernel appends to the list
+    __shared__ uint32_t part_sum[kRxScanParts][kRxScanDigits];
+    __shared__ uint32_t digit_base[kRxScanDigits];
+    __shared__ uint32_t wave_tot[kRxScanDigits / 64];
+    const int dl = threadIdx.x & (kRxScanDigits - 1), part = threadIdx.x / kRxScanDigits;
+    const int d = blockIdx.x * kRxScanDigits + dl;  // 256 digits a workgroup: one workgroup, or two for 9-bit digits
     const size_t per_part = (n_tiles + kRxScanParts - 1) / kRxScanParts;
     const size_t t0 = (size_t)part * per_part, t1 = (t0 + per_part < n_tiles) ? t0 + per_part : n_tiles;
     uint32_t total = 0;
@@ -430,13 +440,13 @@ __global__ __launch_bounds__(kRxBins * kRxScanParts) void rx_scan_kernel(uint32_
 #pragma unroll
         for (int u = 0; u < 16; u++) total += c[u];
     }
-    part_sum[part][d] = total;
+    part_sum[part][dl] = total;
     __syncthreads();
     if (part == 0) {
-        const int lane = d & 63, wave = d >> 6;
+        const int lane = dl & 63, wave = dl >> 6;
         uint32_t all = 0;
 #pragma unroll
-        for (int p = 0; p < kRxScanParts; p++) all += part_sum[p][d];
+        for (int p = 0; p < kRxScanParts; p++) all += part_sum[p][dl];
         uint32_t inc = all;
 #pragma unroll
         for (int s = 1; s < 64; s <<= 1) {
@@ -444,12 +454,19 @@ __global__ __launch_bounds__(kRxBins * kRxScanParts) void rx_scan_kernel(uint32_
             if (lane >= s) inc += v;
         }
         if (lane == 63) wave_tot[wave] = inc;
-        digit_base[d] = inc - all;  // within the wave; the earlier waves' totals are added below
+        digit_base[dl] = inc - all;  // within the wave; the earlier waves' totals are added below
     }
     __syncthreads();
-    uint32_t run = digit_base[d];
-    for (int w = 0; w < (d >> 6); w++) run += wave_tot[w];
-    for (int p = 0; p < part; p++) run += part_sum[p][d];
+    uint32_t run = digit_base[dl];
+    for (int w = 0; w < (dl >> 6); w++) run += wave_tot[w];
+    if (blockIdx.x != 0) {
+        // the second workgroup's digits come after all of the first's: every entry has one digit, so what lies before
+        // them is the number of entries less what this workgroup counted
+        uint32_t group = 0;
+        for (int w = 0; w < kRxScanDigits / 64; w++) group += wave_tot[w];
+        run += n_entries - group;
+    }
+    for (int p = 0; p < part; p++) run += part_sum[p][dl];
     for (t = t0; t < t1; t += 16) {
         uint32_t c[16];
 #pragma unroll
@@ -467,16 +484,21 @@ __global__ __launch_bounds__(kRxBins * kRxScanParts) void rx_scan_kernel(uint32_
 // earlier wave-rounds (a prefix over q of table[q][digit]) + entries of its digit in lower lanes of its own wave-round
 // (ballots).  The tile is then put in digit order in LDS and written out from there, so that the lanes of a store
 // instruction write runs of consecutive addresses (one run per digit present) instead of 64 scattered words.
+template <int BITS>
 __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* __restrict__ keys_in,
                                                                 const uint32_t* __restrict__ vals_in, size_t n, int shift,
                                                                 const uint32_t* __restrict__ starts,
                                                                 uint32_t* __restrict__ keys_out,
-                                                                uint32_t* __restrict__ vals_out, const uint32_t* gate) {
+                                                                uint32_t* __restrict__ vals_out, const uint32_t* gate,
+                                                                uint32_t* gate_clear) {
     if (gate && *gate == 0) return;
+    if (gate_clear && blockIdx.x == 0 && threadIdx.x == 0) *gate_clear = 0u;  // the word no workgroup of this launch reads
+    constexpr int kRxBits = BITS, kRxBins = 1 << BITS;
+    constexpr int DPT = kRxBins / kRxThreads;  // digits a thread owns in the prefix step: t * DPT .. t * DPT + DPT - 1
     constexpr int Q = kRxPerThread * (kRxThreads / 64);
     // the ranking table, then (once every entry knows its place) the tile in digit order: keys, then values
     __shared__ __align__(16) uint32_t lds[Q * kRxBins / 2];
-    static_assert(sizeof(lds) == 2 * kRxTile * sizeof(uint32_t), "the sorted tile reuses the table's memory");
+    static_assert(sizeof(lds) >= 2 * kRxTile * sizeof(uint32_t), "the sorted tile reuses the table's memory");
     uint16_t(*table)[kRxBins] = reinterpret_cast<uint16_t(*)[kRxBins]>(lds);
     __shared__ uint32_t first[kRxBins];       // where the tile's entries of a digit go in the output
     __shared__ uint32_t tile_start[kRxBins];  // where they start in the sorted tile
@@ -492,9 +514,12 @@ __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* 
         key[r] = e < n ? keys_in[e] : 0xffffffffu;
         val[r] = (e < n && vals_in) ? vals_in[e] : (uint32_t)e;
     }
-    const uint32_t my_first = starts[(size_t)blockIdx.x * kRxBins + threadIdx.x];
+    uint32_t my_first[DPT];
+#pragma unroll
+    for (int j = 0; j < DPT; j++) my_first[j] = starts[(size_t)blockIdx.x * kRxBins + threadIdx.x + j * kRxThreads];
     for (int i = threadIdx.x; i < Q * kRxBins / 2; i += kRxThreads) lds[i] = 0;
-    first[threadIdx.x] = my_first;
+#pragma unroll
+    for (int j = 0; j < DPT; j++) first[threadIdx.x + j * kRxThreads] = my_first[j];
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kRxPerThread; r++) {
@@ -513,18 +538,24 @@ __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* 
         if (live && below == 0) table[r * (kRxThreads / 64) + wave][digit] = (uint16_t)__popcll(peers);
     }
     __syncthreads();
-    {  // thread d: exclusive prefix over the wave-rounds of digit d, then over the digits of the tile
-        const int d = threadIdx.x;
-        uint16_t c[Q];
+    {  // a thread's digits: exclusive prefix over the wave-rounds of each, then over the digits of the tile
+        uint32_t tot[DPT], mine = 0;
 #pragma unroll
-        for (int q = 0; q < Q; q++) c[q] = table[q][d];  // all reads first: one LDS round trip, not Q
-        uint32_t run = 0;
+        for (int j = 0; j < DPT; j++) {
+            const int d = threadIdx.x * DPT + j;
+            uint16_t c[Q];
 #pragma unroll
-        for (int q = 0; q < Q; q++) {
-            table[q][d] = (uint16_t)run;
-            run += c[q];
+            for (int q = 0; q < Q; q++) c[q] = table[q][d];  // all reads first: one LDS round trip, not Q
+            uint32_t run = 0;
+#pragma unroll
+            for (int q = 0; q < Q; q++) {
+                table[q][d] = (uint16_t)run;
+                run += c[q];
+            }
+            tot[j] = run;
+            mine += run;
         }
-        uint32_t inc = run;
+        uint32_t inc = mine;
 #pragma unroll
         for (int s = 1; s < 64; s <<= 1) {
             const uint32_t v = __shfl_up(inc, s, 64);
@@ -532,9 +563,13 @@ __global__ __launch_bounds__(kRxThreads) void rx_scatter_kernel(const uint32_t* 
         }
         if (lane == 63) wave_tot[wave] = inc;
         __syncthreads();
-        uint32_t start = inc - run;
+        uint32_t start = inc - mine;
         for (int w = 0; w < wave; w++) start += wave_tot[w];
-        tile_start[d] = start;
+#pragma unroll
+        for (int j = 0; j < DPT; j++) {
+            tile_start[threadIdx.x * DPT + j] = start;
+            start += tot[j];
+        }
     }
     __syncthreads();
     uint32_t place[kRxPerThread];
@@ -609,40 +644,42 @@ static int build_plan_radix(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& p
     const unsigned n_tiles = (unsigned)ceil_div_sz(n, kRxTile);
     int bits = 1;
     while (((size_t)1 << bits) <= nb) bits++;  // values 0 .. nb (nb itself marks a key outside the buckets)
-    const int passes = (bits + kRxBits - 1) / kRxBits;
+    const bool nine = (bits + 8) / 9 < (bits + 7) / 8;  // 9-bit digits where they save a pass
+    const int digit = nine ? 9 : 8, passes = (bits + digit - 1) / digit;
     // the last pass must land in pl.perm: the positions alternate between perm_tmp and perm
     uint32_t* vals[2] = {(passes & 1) ? pl.perm_tmp : pl.perm, (passes & 1) ? pl.perm : pl.perm_tmp};
     // keys: pass 0 reads rx_in0 and writes rx_keys[1], pass 1 writes rx_keys[0], ...
     const uint32_t* later = gate ? gate + 1 : nullptr;
-    hipLaunchKernelGGL(rx_count_first_kernel, dim3(n_tiles), dim3(kRxThreads), 0, st, keys, payload, n, (uint32_t)nb,
-                       pl.rx_in0, pl.rx_peer0, pl.rx_counts, gate);
-    ZG_LAUNCH_CHECK();
+#define ZG_RX(KERNEL, GRID, BLOCK, ...)                                                                \
+    do {                                                                                               \
+        if (nine) hipLaunchKernelGGL((KERNEL<9>), GRID, BLOCK, 0, st, __VA_ARGS__);                    \
+        else hipLaunchKernelGGL((KERNEL<8>), GRID, BLOCK, 0, st, __VA_ARGS__);                         \
+        ZG_LAUNCH_CHECK();                                                                             \
+    } while (0)
+    ZG_RX(rx_count_first_kernel, dim3(n_tiles), dim3(kRxThreads), keys, payload, n, (uint32_t)nb, pl.rx_in0, pl.rx_peer0,
+          pl.rx_counts, gate);
     for (int p = 0; p < passes; p++) {
         const uint32_t* kin = p == 0 ? pl.rx_in0 : pl.rx_keys[p & 1];
         uint32_t* kout = pl.rx_keys[(p & 1) ^ 1];
         if (p > 0) {
-            hipLaunchKernelGGL(rx_count_kernel, dim3(n_tiles), dim3(kRxThreads), 0, st, kin, n, p * kRxBits, pl.rx_counts, later);
-            ZG_LAUNCH_CHECK();
+            ZG_RX(rx_count_kernel, dim3(n_tiles), dim3(kRxThreads), kin, n, p * digit, pl.rx_counts, later);
         }
         RxGate g;
         if (gate) {
             g.in = p == 0 ? gate : later;
             if (p == 0) {
                 g.move_to = gate + 1;
-                g.clear = gate;
                 g.tally = gate + 2;
                 g.tally_host = tally_host;
             }
         }
-        hipLaunchKernelGGL(rx_scan_kernel, dim3(1), dim3(kRxBins * kRxScanParts), 0, st, pl.rx_counts, (size_t)n_tiles, g,
-                           p == 0 ? pl.long_list : (uint32_t*)nullptr);
-        ZG_LAUNCH_CHECK();
+        ZG_RX(rx_scan_kernel, dim3(nine ? 2 : 1), dim3(kRxScanThreads), pl.rx_counts, (size_t)n_tiles, g,
+              p == 0 ? pl.long_list : (uint32_t*)nullptr, (uint32_t)n);
         // pass 0 reads no positions (an entry's position is its index); pass p writes vals[(p + 1) & 1]... in turn
-        hipLaunchKernelGGL(rx_scatter_kernel, dim3(n_tiles), dim3(kRxThreads), 0, st, kin,
-                           p == 0 ? (const uint32_t*)nullptr : vals[p & 1], n, p * kRxBits, pl.rx_counts, kout,
-                           vals[(p & 1) ^ 1], later);
-        ZG_LAUNCH_CHECK();
+        ZG_RX(rx_scatter_kernel, dim3(n_tiles), dim3(kRxThreads), kin, p == 0 ? (const uint32_t*)nullptr : vals[p & 1], n,
+              p * digit, pl.rx_counts, kout, vals[(p & 1) ^ 1], later, (gate && p == 0) ? gate : (uint32_t*)nullptr);
     }
+#undef ZG_RX
     hipLaunchKernelGGL(rx_finish_kernel, dim3((unsigned)ceil_div_sz(n + 1, 256)), dim3(256), 0, st, pl.rx_keys[passes & 1], n,
                        nb, pl.perm, payload ? pl.rx_peer0 : (const uint32_t*)nullptr, pl.peer, pl.row_ptr, pl.long_list, later);
     ZG_LAUNCH_CHECK();

@@ -180,7 +180,9 @@ int zg_hip_mem_random(zg_hip_ctx *ctx, float *x, size_t n, int kind, uint64_t fa
 
 /* ---------------------------------------------------------------------------------------------
  * elementwise binary (src/device/host_device.zig:205-219, :975-1019; opspec.zig:19-57)
- * requires max(xl,yl) % min(xl,yl) == 0 and zl == max(xl,yl); z may alias x or y
+ * requires max(xl,yl) % min(xl,yl) == 0 and zl == max(xl,yl); z may alias x or y.  Empty operands: zl == 0 with x and
+ * y each empty or one float (not both one float) does nothing, as the host's loops do; an empty operand against a
+ * longer one is refused (the host's loop would not end).
  *
  * Small elementwise ops wait.  These four with operands of one length or one operand of a single float, the unary
  * forward and backward ops below, zg_hip_scale and the elementwise loss gradients, on at most 65536 elements, are not
@@ -209,6 +211,9 @@ int zg_hip_div_scalar(zg_hip_ctx *ctx, const float *x, size_t n, float s, int sc
 
 /* ---------------------------------------------------------------------------------------------
  * linear algebra (src/device/host_device.zig:224-346)
+ * On no elements (n == 0) dot, sum and nrm2 write 0, as the BLAS calls behind the reference do; scale, axpy and
+ * clip_nrm2 do nothing.  A product with k == 0 leaves C = beta C and does not look at A and B (they may be null);
+ * with m == 0 or n == 0 there is nothing to do.
  * ------------------------------------------------------------------------------------------- */
 int zg_hip_dot(zg_hip_ctx *ctx, const float *x, const float *y, size_t n, float *z);
 int zg_hip_matvec(zg_hip_ctx *ctx, const float *A, const float *x, float *y, size_t m, size_t n, int trans_a,
@@ -434,6 +439,8 @@ int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx *ctx, const float *grad
 int zg_hip_smce_fwd(zg_hip_ctx *ctx, const float *logits, const float *target, float *probs, float *loss,
                     size_t rows, size_t cols);
 int zg_hip_smce_bwd(zg_hip_ctx *ctx, const float *probs, const float *target, float *grad, size_t rows, size_t cols);
+/* (An empty matrix: zg_hip_smce_bwd, zg_hip_softmax_fwd and zg_hip_softmax_bwd do nothing, like the host's loops over
+ * no rows; the forward losses, which divide by the number of rows or elements, refuse it with ZG_HIP_EINVAL.) */
 /* smce_fwd followed by the loss's backward with upstream gradient 1 (loss.backward() on the scalar loss,
  * src/nn/loss.zig:150-159): grad (+)= (probs - target)/rows.  Same values as the two calls; a batch of at most
  * 256 rows x 32 columns (64 x 256, 16 x 4096) takes one launch.  accumulate == 0: grad is written, not read. */

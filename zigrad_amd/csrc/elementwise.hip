@@ -218,6 +218,10 @@ template <class B>
 static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t xl, const float* y, size_t yl, float* z,
                      size_t zl) {
     ZG_ENTER(ctx, kWaitMaps | kWaitFills);
+    // An empty result from empty or one-element operands is what the host's loops make of it: nothing
+    // (src/device/host_device.zig:975-1019: equal lengths, or a scalar against an empty slice).  An empty operand
+    // against a longer one never ends there and is refused here.
+    if (zl == 0 && xl <= 1 && yl <= 1 && xl + yl < 2) return ZG_HIP_OK;
     ZG_REQUIRE(xl > 0 && yl > 0 && zl > 0, "%s: empty operand", name);
     ZG_REQUIRE(x && y && z, "%s: null pointer", name);
     const size_t mx = xl > yl ? xl : yl, mn = xl < yl ? xl : yl;

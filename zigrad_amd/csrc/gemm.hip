@@ -1360,7 +1360,7 @@ static bool gemm_is_deep(size_t m, size_t n, size_t k, size_t batches, bool a_km
 
 static int gemm_validate(const char* name, const float* A, const float* B, const float* C, size_t m, size_t n, size_t k,
                          int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc) {
-    ZG_REQUIRE(A && B && C, "%s: null pointer", name);
+    ZG_REQUIRE(C && (k == 0 || (A && B)), "%s: null pointer", name);  // with k == 0 the operands are not read: C = beta C
     // cblas argument rules for row-major storage
     ZG_REQUIRE(lda >= (trans_a ? m : k) && lda >= 1, "%s: lda %zu too small", name, lda);
     ZG_REQUIRE(ldb >= (trans_b ? k : n) && ldb >= 1, "%s: ldb %zu too small", name, ldb);

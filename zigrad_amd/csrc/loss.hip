@@ -779,6 +779,7 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
 ZG_API int zg_hip_smce_bwd(zg_hip_ctx* ctx, const float* probs, const float* target, float* grad, size_t rows,
                            size_t cols) {
     ZG_ENTER(ctx, kWaitFills | kWaitProducts | kWaitSteps);
+    if (rows == 0 || cols == 0) return ZG_HIP_OK;  // the host's loop over no rows (src/nn/loss.zig:157-171)
     ZG_REQUIRE(probs && target && grad, "smce_bwd: null pointer");
     if (int rc = check_rows("smce_bwd", rows, cols)) return rc;
     // the gradient's zero fill (ensure_grad(0), src/ndtensor.zig:221-228) may still be waiting: then write, not add
@@ -869,6 +870,7 @@ ZG_API int zg_hip_smce_fwd_bwd(zg_hip_ctx* ctx, const float* logits, const float
 
 ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t rows, size_t cols) {
     ZG_CTX(ctx);
+    if (rows == 0 || cols == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x && y, "softmax_fwd: null pointer");
     if (int rc = check_rows("softmax_fwd", rows, cols)) return rc;
     if (long_row_ok(x, x, y, rows, cols)) {
@@ -889,6 +891,7 @@ ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t 
 
 ZG_API int zg_hip_softmax_bwd(zg_hip_ctx* ctx, const float* y, const float* y_g, float* x_g, size_t rows, size_t cols) {
     ZG_CTX(ctx);
+    if (rows == 0 || cols == 0) return ZG_HIP_OK;
     ZG_REQUIRE(y && y_g && x_g, "softmax_bwd: null pointer");
     if (int rc = check_rows("softmax_bwd", rows, cols)) return rc;
     const int tpr = pick_tpr(cols);

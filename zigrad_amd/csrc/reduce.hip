@@ -279,18 +279,21 @@ using namespace zg;
 
 ZG_API int zg_hip_sum(zg_hip_ctx* ctx, const float* x, size_t n, float* y) {
     ZG_CTX(ctx);
+    if (n == 0 && y) return zg_hip_mem_fill(ctx, y, 1, 0.f);  // the BLAS call on no elements: 0 (src/device/host_device.zig:315-321)
     ZG_REQUIRE(x && y && n > 0, "sum: null or empty operand");
     return flat_reduce<TermAbs, 1>(ctx, x, nullptr, n, 0.f, FinStore{y});
 }
 
 ZG_API int zg_hip_nrm2(zg_hip_ctx* ctx, const float* x, size_t n, float* y) {
     ZG_CTX(ctx);
+    if (n == 0 && y) return zg_hip_mem_fill(ctx, y, 1, 0.f);  // (src/device/host_device.zig:331)
     ZG_REQUIRE(x && y && n > 0, "nrm2: null or empty operand");
     return flat_reduce<TermSq, 1>(ctx, x, nullptr, n, 0.f, FinSqrt{y});
 }
 
 ZG_API int zg_hip_dot(zg_hip_ctx* ctx, const float* x, const float* y, size_t n, float* z) {
     ZG_CTX(ctx);
+    if (n == 0 && z) return zg_hip_mem_fill(ctx, z, 1, 0.f);  // (src/device/host_device.zig:224)
     ZG_REQUIRE(x && y && z && n > 0, "dot: null or empty operand");
     return flat_reduce<TermDot, 2>(ctx, x, y, n, 0.f, FinStore{z});
 }

@@ -314,7 +314,9 @@ int zg_hip_sigm_bwd(zg_hip_ctx *ctx, float *x_g, const float *y, const float *y_
 int zg_hip_sigm_inplace_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, size_t n);
 int zg_hip_clamp_fwd(zg_hip_ctx *ctx, const float *x, float *y, size_t n, float lo, float hi);
 int zg_hip_clamp_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, const float *y_g, size_t n, float lo, float hi);
-int zg_hip_max_fwd(zg_hip_ctx *ctx, const float *x, size_t n, float *y); /* x[isamax(x)]: largest |x|, first on ties */
+/* x[isamax(x)]: the element of largest |x|, the first on ties (src/device/host_device.zig:573-580).  A NaN counts as
+ * larger than anything and the first one wins, as mkl_rt, the BLAS the reference names, documents for i?amax. */
+int zg_hip_max_fwd(zg_hip_ctx *ctx, const float *x, size_t n, float *y);
 int zg_hip_max_bwd(zg_hip_ctx *ctx, const float *x, float *x_g, size_t n, const float *y, const float *y_g);
 
 /* ---------------------------------------------------------------------------------------------

@@ -449,9 +449,15 @@ void zo_max_fwd(const float *x, size_t n, float *y) {
     if (use_blas() && g_blas.isamax) {
         idx = g_blas.isamax((int)n, x, 1);
     } else {
+        /* a NaN counts as larger than anything, the first one wins: what mkl_rt documents for i?amax (the plain
+         * comparison loop of the Fortran routine would skip NaNs unless one comes first) */
         float best = -1.f;
         for (size_t i = 0; i < n; i++) {
             float a = fabsf(x[i]);
+            if (a != a) {
+                idx = i;
+                break;
+            }
             if (a > best) {
                 best = a;
                 idx = i;

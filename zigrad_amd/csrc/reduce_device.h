@@ -56,21 +56,25 @@ struct ArgmaxAcc {
 };
 
 // |value| + position + signed value: the element cblas_isamax picks (first index of the largest |x|)
+// The element of largest magnitude, first on ties (cblas_isamax).  Magnitudes are compared as the bit patterns of |x|,
+// which order like the values for everything finite and infinite and put every NaN above them (all NaNs count alike):
+// an array that holds a NaN yields its first NaN, as the BLAS the reference is built with documents (mkl_rt), instead
+// of an element that only looks like the maximum.
 struct AbsArgAccT {
-    float a;
+    uint32_t a;  // bits of |x|, any NaN as 0x7f800001
     uint32_t i;
     float v;
 };
 struct AbsArgmaxAcc {
     using Acc = AbsArgAccT;
-    static __device__ __forceinline__ Acc init() { return Acc{-1.0f, 0xffffffffu, 0.f}; }
+    static __device__ __forceinline__ Acc init() { return Acc{0u, 0xffffffffu, 0.f}; }
     static __device__ __forceinline__ Acc combine(Acc x, Acc y) {
         bool take_y = (y.a > x.a) || (y.a == x.a && y.i < x.i);
         return take_y ? y : x;
     }
     static __device__ __forceinline__ Acc shfl_xor(Acc x, int m) {
         Acc r;
-        r.a = __shfl_xor(x.a, m, kWave);
+        r.a = (uint32_t)__shfl_xor((int)x.a, m, kWave);
         r.i = (uint32_t)__shfl_xor((int)x.i, m, kWave);
         r.v = __shfl_xor(x.v, m, kWave);
         return r;
@@ -143,7 +147,8 @@ struct TermSqDiff {
 struct TermAbsArg {
     using P = AbsArgmaxAcc;
     static __device__ __forceinline__ AbsArgAccT term(float a, float, size_t i, float) {
-        return AbsArgAccT{fabsf(a), (uint32_t)i, a};
+        const uint32_t bits = __float_as_uint(a) & 0x7fffffffu;
+        return AbsArgAccT{bits > 0x7f800000u ? 0x7f800001u : bits, (uint32_t)i, a};
     }
 };
 

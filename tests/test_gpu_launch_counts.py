@@ -46,7 +46,7 @@ def test_dqn_update(hip, fused, want, device_scalars):
     assert launches_per_step(hip, tr) == want
 
 
-@pytest.mark.parametrize("fused,want", [(False, 24), (True, 21)])
+@pytest.mark.parametrize("fused,want", [(False, 22), (True, 19)])
 def test_gcn_step(hip, fused, want):
     tr = GCNTrainer(hip, gcn_inputs(seed=0), lr=0.01, clip=True, fused=fused)
     assert launches_per_step(hip, tr) == want

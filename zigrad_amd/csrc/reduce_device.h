@@ -478,6 +478,15 @@ __device__ __forceinline__ void col_reduce_block(const float* x, typename A::Out
                 acc[3 % V] = P::combine(acc[3 % V], A::term(v0.w, rr));
             }
         } else {
+            // sixteen rows in flight while there are sixteen left (a single workgroup walking thousands of short rows
+            // waits for memory once per trip), then four, then one by one: always combined in row order
+            for (; r + 15 * (size_t)ry < r_end; r += 16 * (size_t)ry) {
+                float vs[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) vs[u] = xb[(r + (size_t)u * ry) * inner];
+#pragma unroll
+                for (int u = 0; u < 16; u++) acc[0] = P::combine(acc[0], A::term(vs[u], (uint32_t)(r + (size_t)u * ry)));
+            }
             for (; r + 3 * (size_t)ry < r_end; r += 4 * (size_t)ry) {
                 float v0 = xb[r * inner], v1 = xb[(r + ry) * inner], v2 = xb[(r + 2 * (size_t)ry) * inner],
                       v3 = xb[(r + 3 * (size_t)ry) * inner];
@@ -533,6 +542,6 @@ static inline ColReduceShape col_reduce_shape(const float* x, size_t inner, bool
     s.gx = ceil_div_sz(colv, (size_t)1 << s.log2_cx);
     return s;
 }
-constexpr size_t kColSingleChunkMax = 16384;  // up to this many elements the rows are not split into chunks
+constexpr size_t kColSingleChunkMax = 65536;  // up to this many elements the rows are not split into chunks
 
 }  // namespace zg

@@ -334,7 +334,7 @@ int zg_hip_argmax_along(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape
 size_t zg_hip_unbroadcast_scratch_len(const uint64_t *x_shape, size_t x_rank, const uint64_t *y_shape,
                                       size_t y_rank);
 /* unbroadcast (src/device/host_device.zig:709-780).  The form a Linear layer's bias gradient takes (y += sums over the
- * leading dimensions of x, alpha = beta = 1, at most 16384 elements of x) waits inside the context like a product
+ * leading dimensions of x, alpha = beta = 1, at most 65536 elements of x) waits inside the context like a product
  * (see zg_hip_matmul): the layer's input-gradient and weight-gradient products follow it (src/ndtensor.zig:780-796,
  * 1092-1136) and, when they are small too, the three leave in one launch.  Any other call sends it out first. */
 int zg_hip_unbroadcast(zg_hip_ctx *ctx, const float *x, const uint64_t *x_shape, size_t x_rank, float *y,

@@ -135,7 +135,9 @@ def test_tall_narrow_products_of_k_contiguous_operands(hip, shape):
 
 
 @pytest.mark.parametrize("shape", [(64, 128, 784), (100, 30, 384), (100, 30, 383), (256, 256, 2048), (256, 256, 2049),
-                                   (250, 251, 1000), (257, 256, 600), (17, 33, 2047), (16, 16, 400), (64, 128, 1433)])
+                                   (250, 251, 1000), (257, 256, 600), (17, 33, 2047), (16, 16, 400), (64, 128, 1433),
+                                   # k of 384 to 512 on up to 16 blocks of 32 x 32, which the unstaged kernel would take too
+                                   (64, 64, 512), (128, 128, 512), (100, 30, 385), (96, 96, 513), (16, 16, 512)])
 def test_deep_products_of_k_contiguous_operands_either_side_of_the_one_launch_kernels_limits(hip, shape):
     """[m, k] x [n, k]^T with 384 <= k <= 2048 on at most 256 blocks of 16 x 16 takes one launch of a kernel of its own
     (a Linear layer's forward at a small batch); the shapes here sit on both sides of each limit, with edges inside a

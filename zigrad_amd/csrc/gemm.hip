@@ -1350,6 +1350,8 @@ static bool gemm_is_tiny(size_t m, size_t n, size_t k, size_t batches, size_t ld
 }
 
 // One unbatched product of k-contiguous operands with a long k on at most a CU's worth of 16 x 16 blocks: gemm_deep_kernel.
+// It goes before the unstaged kernel where both apply (k of 384 to 512 on up to 16 blocks of 32 x 32: 64 x 64 x 512
+// 8.1 -> 5.6 us, 128 x 64 x 512 8.2 -> 4.8 us).
 // (Below k = 384 the unstaged kernel or one round of 64 x 64 tiles does as well.  A load instruction of this kernel
 // touches 64 bytes in each of 16 rows, which the memory system serves slowly when the rows are far apart: at k = 4096
 // a workgroup's loads take 19 us and the staged kernels with k cut over workgroups win again; measured break-even
@@ -1493,8 +1495,9 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     g.split_stride = 0;
 
     if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
-    if (gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
-    if (gemm_is_deep(m, n, k, batches, a_kmajor, b_kmajor, n_cu)) {
+    const bool deep = gemm_is_deep(m, n, k, batches, a_kmajor, b_kmajor, n_cu);
+    if (!deep && gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
+    if (deep) {
         g.tiles_m = (unsigned)ceil_div_sz(m, 16);
         g.tiles_n = (unsigned)ceil_div_sz(n, 16);
         hipLaunchKernelGGL(gemm_deep_kernel, dim3(g.tiles_m * g.tiles_n), dim3(256), 0, ctx->stream, g);

@@ -52,6 +52,21 @@ def test_deep_products_on_few_tiles_are_cut_along_k():
         assert p["k_tiles_per_split"] % 2 == 0 and p["splits"] * p["k_tiles_per_split"] * 16 >= shape[2]
 
 
+def test_ranges_of_k_on_few_tiles_get_a_compute_unit_each_and_stay_long():
+    # up to 32 tiles of 64 x 64: at most one range per compute unit and at most 16 ranges (256 values of k and more each
+    # at k = 4096), and a product of 25 k-tiles is cut once every range has a compute unit to itself
+    for shape in ((256, 256, 4096), (64, 64, 4096), (500, 64, 4096), (500, 256, 2048), (1024, 64, 2048), (500, 64, 385)):
+        p = gemm_plan(*shape)
+        tiles = -(-shape[0] // 64) * -(-shape[1] // 64)
+        assert p["kind"] == "split_k" and p["tile"] == (64, 64), shape
+        assert 2 <= p["splits"] <= 16 and tiles * p["splits"] <= 256, (shape, p)
+        assert (p["splits"] - 1) * p["k_tiles_per_split"] * 16 < shape[2] <= p["splits"] * p["k_tiles_per_split"] * 16
+    assert gemm_plan(256, 256, 4096)["k_tiles_per_split"] == 16
+    # ranges that would need a second round keep the higher bar: these stay whole
+    for shape in ((768, 768, 768), (1024, 500, 512)):
+        assert gemm_plan(*shape)["kind"] == "single", shape
+
+
 def test_plans_are_a_function_of_the_shape_only():
     assert gemm_plan(3072, 3072, 3072) == gemm_plan(3072, 3072, 3072)
     with pytest.raises(Exception):

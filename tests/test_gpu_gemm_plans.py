@@ -188,6 +188,28 @@ def test_tall_narrow_product_is_exact_on_small_integers(hip):
     assert np.array_equal(got, (A.astype(np.int64) @ B.astype(np.int64).T).astype(np.float32))
 
 
+@pytest.mark.parametrize("shape", [(500, 64, 385), (256, 256, 4096), (100, 100, 4099), (500, 256, 2048), (64, 64, 4096),
+                                   (1024, 64, 2050), (130, 70, 1000), (16, 16, 4096)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (True, True)])
+def test_products_on_few_tiles_cut_into_ranges_of_k(hip, shape, ta, tb):
+    """Few 64 x 64 tiles over a long k (in the layouts the one-launch kernels do not take): ranges of k on separate
+    workgroups and a reduction, the last range shorter than the others, against float64 and accumulating."""
+    m, n, k = shape
+    r = np.random.default_rng(m + 3 * n + 7 * k)
+    A = r.standard_normal((k, m) if ta else (m, k), dtype=np.float32)
+    B = r.standard_normal((n, k) if tb else (k, n), dtype=np.float32)
+    C0 = r.standard_normal((m, n), dtype=np.float32)
+    a64 = (A.T if ta else A).astype(np.float64)
+    b64 = (B.T if tb else B).astype(np.float64)
+    prod = a64 @ b64
+    got = _matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, ta, tb, 1.0, 0.0)
+    assert np.linalg.norm(got - prod) <= TOL * np.linalg.norm(prod)
+    assert np.abs(got - prod).max() <= 8 * TOL * np.sqrt(k)
+    got = _matmul(hip, A, B, C0, m, n, k, ta, tb, -0.5, 1.0)
+    want = C0 - 0.5 * prod
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+
+
 @pytest.mark.parametrize("m,n", [(5000, 300), (70000, 33), (64, 64), (63, 1), (1, 700), (4096, 4096), (130, 257)])
 def test_transposed_matvec_over_many_rows(oracle, hip, m, n):
     """y = alpha A^T x + beta y with the rows split over workgroups (src/device/host_device.zig:232-240)."""

@@ -1135,17 +1135,22 @@ static GemmPlan gemm_plan_single(size_t m, size_t n, size_t k, size_t batches, s
     if (lp.tile == 2) {
         const size_t t64 = gemm_tiles_of(2, m, n, batches);
         if (t64 < n_cu && kt_total >= 16) {
-            size_t splits = ceil_div_sz(2 * n_cu, t64);
+            // a range of k per CU for up to 32 tiles, two per CU beyond (500 x 256 x 2048, 32 tiles: 15.5 us in 16 ranges,
+            // 12.9 us in 8), and at most 16 ranges: shorter ones are mostly prologue and the reduction reads them all
+            // (256 x 256 x 4096: 17.0 us in 64 ranges of 64 values of k, 13.1 us in 16 of 256)
+            size_t splits = ceil_div_sz((t64 <= 32 ? 1 : 2) * n_cu, t64);
             if (splits > kt_total / 4) splits = kt_total / 4;
-            if (splits > 64) splits = 64;
+            if (splits > 16) splits = 16;
             size_t per = ceil_div_sz(kt_total, splits);
             per += per & 1;
             splits = ceil_div_sz(kt_total, per);
             // Worth it only when the k-tiles saved on the busiest CU outweigh the second launch and the short loops:
-            // a 64x64 k-tile step takes about 0.27 us, the split's fixed costs about 6 us (768-cubed: 15.5 us whole,
-            // 20 us split four ways).
+            // a 64x64 k-tile step takes about 0.27 us, the split's fixed costs about 4 us when every range has a CU
+            // to itself (500 x 64 x 385: 12.4 us whole, 8.2 us in five ranges) and 6 us when the ranges take a second
+            // round (768-cubed: 15.5 us whole, 20 us split four ways; 1024 x 500 x 512: 11.4 against 14.6).
             const double whole = (double)kt_total, busiest = (double)(ceil_div_sz(t64 * splits, n_cu) * per);
-            if (splits >= 2 && (whole - busiest) * 0.27 > 6.0) {
+            const double fixed_us = t64 * splits <= n_cu ? 4.0 : 6.0;
+            if (splits >= 2 && (whole - busiest) * 0.27 > fixed_us) {
                 lp.kind = GemmPlan::kSplit;
                 lp.splits = splits;
                 lp.per = per;

@@ -272,7 +272,11 @@ def test_fused_gcn_step_with_an_edge_plan_replays_from_an_execution_graph(hip):
 @pytest.mark.parametrize("rows,cols", [(64, 10), (140, 7), (256, 32), (257, 32), (1, 1), (64, 256), (65, 256), (16, 4096),
                                        (17, 4096), (3, 1000), (5, 33), (700, 1024), (2, 5000),
                                        # one pass over rows held in registers: a wave per row, a workgroup per row
-                                       (1024, 1024), (1500, 260), (1100, 1000), (3, 8192), (2, 32768), (5, 4100)])
+                                       (1024, 1024), (1500, 260), (1100, 1000), (3, 8192), (2, 32768), (5, 4100),
+                                       # 4, 16 and 64 lanes per row on either side of the one-launch limit; a workgroup of
+                                       # 256 threads per row with 4 and with 8 pieces each
+                                       (3000, 8), (300, 32), (700, 36), (65, 256), (1500, 256), (17, 1024), (40, 1028),
+                                       (21, 2048), (9, 4096), (6, 8192), (5, 8196)])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_smce_fwd_bwd_equals_forward_then_backward(oracle, hip, rows, cols, accumulate):
     """One call against smce_fwd + smce_bwd (src/nn/loss.zig:130-159) on the same device, bit for bit, on both sides

@@ -36,7 +36,11 @@ def _smce_fwd_hip(hip, x, t):
     return out
 
 
-@pytest.mark.parametrize("rows,cols", [(64, 10), (256, 32), (140, 7), (64, 200), (16, 3000), (1, 4), (255, 2)])
+@pytest.mark.parametrize("rows,cols", [(64, 10), (256, 32), (140, 7), (64, 200), (16, 3000), (1, 4), (255, 2),
+                                       # rows that a larger batch holds in registers: 4, 16 and 64 lanes per row
+                                       (200, 8), (50, 28), (64, 256), (16, 260), (16, 1000), (3, 1024), (9, 36),
+                                       # more than 1024 columns: the small batch takes the row kernels as well
+                                       (16, 2048), (5, 4096), (7, 1030)])
 def test_smce_fwd_small_batches_equal_the_two_launch_path(hip, rows, cols):
     """A batch that fits one workgroup takes one launch (rows and their mean); the same rows inside a batch too large
     for it take the row kernel and the reduction.  Per row the probabilities must be the same bits; the mean is held to
@@ -55,7 +59,10 @@ def test_smce_fwd_small_batches_equal_the_two_launch_path(hip, rows, cols):
     assert abs(loss_small - want) <= 1e-5 * max(1.0, abs(want))
 
 
-SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001), (9, 4100)]
+SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001), (9, 4100),
+               # rows held in registers by 4, 16 or 64 lanes, by a workgroup of 256 threads (4 or 8 pieces each) or of 1024
+               (3000, 8), (3000, 32), (700, 36), (1500, 256), (40, 260), (300, 1024), (40, 1028), (21, 2048), (9, 4096),
+               (7, 5000), (6, 8192), (5, 8196), (3, 20000), (2, 32768)]
 
 
 @pytest.mark.parametrize("rows,cols", SMCE_SHAPES)
@@ -119,7 +126,10 @@ def test_smce_clamp_edge(oracle, hip):
     assert abs(b["loss"][0] - want) <= 1e-5 * want and abs(a["loss"][0] - want) <= 1e-5 * want
 
 
-@pytest.mark.parametrize("rows,cols", [(64, 10), (5, 3000), (1, 7), (3, 8192), (2, 32768), (2, 32772)])
+@pytest.mark.parametrize("rows,cols", [(64, 10), (5, 3000), (1, 7), (3, 8192), (2, 32768), (2, 32772),
+                                       # every shape of the kernels that hold a row in registers, and rows beside them
+                                       (1000, 4), (700, 32), (300, 36), (1500, 256), (70, 260), (300, 1024), (33, 1028),
+                                       (21, 4096), (9, 4100), (5, 8196), (3, 32764), (70, 1030), (500, 30)])
 def test_softmax_fwd_bwd(oracle, hip, rows, cols):
     r = rng(rows + cols)
     x = r.standard_normal((rows, cols)).astype(np.float32)

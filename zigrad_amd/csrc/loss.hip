@@ -270,15 +270,17 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* logit
     }
 }
 
-// Long rows (up to 32768 columns, 16-byte aligned): one workgroup of 1024 threads per row keeps the whole row in
-// registers (at most 8 float4 per thread), so the logits are read from HBM once: max / sum-of-exponentials over
+// Long rows (1028 to 32768 columns, 16-byte aligned): one workgroup of NT threads per row keeps the whole row in
+// registers (at most VEC float4 per thread), so the logits are read from HBM once: max / sum-of-exponentials over
 // the registers, one workgroup reduction, then the probabilities (and the loss terms) from the same registers.
 // MODE 1 reads the target row as well; its loads are issued before the reduction so they are in flight under it.
-constexpr int kLongRowThreads = 1024;
-constexpr int kLongRowVec = 8;
+// Three shapes by row length, so that a thread has several loads in flight and a compute unit several rows:
+// 256 threads x 4 float4 up to 4096 columns, 256 x 8 up to 8192, 1024 x 8 beyond.
+constexpr int kLongRowMaxThreads = 1024;
+constexpr int kLongRowMaxVec = 8;
 // GRAD (with MODE 1): 1 the loss's gradient (p - t) / denom is written to grad as well, 2 it is added to grad: the
 // backward pass of the scalar loss in the same pass over the row (smce_bwd_kernel's arithmetic per element).
-template <int MODE, int GRAD = 0>
+template <int kLongRowThreads, int kLongRowVec, int MODE, int GRAD = 0>
 __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(const float* logits, const float* target,
                                                                             float* probs, float* row_loss,
                                                                             size_t cols, float* grad = nullptr,
@@ -380,17 +382,17 @@ __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(cons
     }
 }
 
-// Rows of 260 to 1024 columns in batches of a thousand rows or more (the wide classifier's [4096, 1024] logits): a wave
-// per row holds the row in registers (at most 4 float4 per lane), so the logits are read once and the row's
-// reductions stay inside the wave: three passes of the matrix instead of four, no LDS, no barrier.
+// Rows of up to 1024 columns (the wide classifier's [4096, 1024] logits): TPR lanes of a wave per row (16 up to 256
+// columns, a whole wave beyond) hold the row in registers (at most 4 float4 per lane), so the logits are read once and
+// the row's reductions stay inside the wave: three passes of the matrix instead of four, no LDS, no barrier.
 constexpr int kWaveRowVec = 4;
-template <int MODE, int GRAD = 0>
+template <int TPR, int MODE, int GRAD = 0>
 __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* logits, const float* target, float* probs,
                                                                     float* row_loss, size_t rows, size_t cols,
                                                                     float* grad = nullptr, float denom = 1.f) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const size_t row = (size_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    if (row >= rows) return;  // whole waves leave together: no barrier follows
+    const int lane = threadIdx.x & (TPR - 1);
+    const size_t row = (size_t)blockIdx.x * (kBlock / TPR) + threadIdx.x / TPR;
+    if (row >= rows) return;  // the lanes of a row leave together: no barrier follows, and shuffles stay inside the row
     const size_t c4 = cols >> 2;
     const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
     const float4* t4 = reinterpret_cast<const float4*>(MODE ? target + row * cols : logits);
@@ -400,13 +402,13 @@ __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* 
     float4 v[kWaveRowVec], t[kWaveRowVec];
 #pragma unroll
     for (int u = 0; u < kWaveRowVec; u++) {
-        const size_t j = lane + (size_t)u * kWave;
+        const size_t j = lane + (size_t)u * TPR;
         v[u] = (j < c4) ? nt_load(x4 + j) : ninf;
     }
     if (MODE) {
 #pragma unroll
         for (int u = 0; u < kWaveRowVec; u++) {
-            const size_t j = lane + (size_t)u * kWave;
+            const size_t j = lane + (size_t)u * TPR;
             t[u] = (j < c4) ? nt_load(t4 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
@@ -422,12 +424,12 @@ __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* 
         acc.m = mx;
         acc.s = sum;
     }
-    acc = group_reduce<OnlineAcc, kWave>(acc);
+    acc = group_reduce<OnlineAcc, TPR>(acc);
     const float l = __fadd_rn(acc.m, logf(acc.s));
     float part = 0.f;
 #pragma unroll
     for (int u = 0; u < kWaveRowVec; u++) {
-        const size_t j = lane + (size_t)u * kWave;
+        const size_t j = lane + (size_t)u * TPR;
         if (j < c4) {
             float4 p;
             p.x = fexp(__fsub_rn(v[u].x, l));
@@ -463,22 +465,49 @@ __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* 
         }
     }
     if (MODE) {
-        part = group_reduce<SumAcc, kWave>(part);
+        part = group_reduce<SumAcc, TPR>(part);
         if (lane == 0) row_loss[row] = part;
     }
 }
 
 static bool wave_row_ok(const float* a, const float* b, const float* c, size_t rows, size_t cols) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
-    return cols > 256 && cols <= (size_t)kWave * kWaveRowVec * 4 && cols % 4 == 0 && (bits & 15u) == 0 && rows >= 1024 &&
-           rows <= 0x7fffffffull;
+    return cols <= (size_t)kWave * kWaveRowVec * 4 && cols % 4 == 0 && (bits & 15u) == 0 && rows <= 0x7fffffffull;
 }
 
 static bool long_row_ok(const float* a, const float* b, const float* c, size_t rows, size_t cols) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
-    return cols > 4096 && cols % 4 == 0 && cols <= (size_t)kLongRowThreads * kLongRowVec * 4 && (bits & 15u) == 0 &&
+    return cols > 1024 && cols % 4 == 0 && cols <= (size_t)kLongRowMaxThreads * kLongRowMaxVec * 4 && (bits & 15u) == 0 &&
            rows <= 0x7fffffffull;
 }
+
+// Launches softmax_wave_rows_kernel<.., MODE, GRAD> with the lanes per row that fit the row length (wave_row_ok holds).
+#define ZG_WAVE_ROWS(MODE, GRAD, ...)                                                                                  \
+    do {                                                                                                               \
+        if (cols <= 32) /* the lanes per row of pick_tpr, which the one-workgroup kernel for small batches follows */   \
+            hipLaunchKernelGGL((softmax_wave_rows_kernel<4, MODE, GRAD>), dim3((unsigned)ceil_div_sz(rows, kBlock / 4)), \
+                               dim3(kBlock), 0, ctx->stream, __VA_ARGS__);                                             \
+        else if (cols <= 16 * kWaveRowVec * 4)                                                                         \
+            hipLaunchKernelGGL((softmax_wave_rows_kernel<16, MODE, GRAD>), dim3((unsigned)ceil_div_sz(rows, kBlock / 16)), \
+                               dim3(kBlock), 0, ctx->stream, __VA_ARGS__);                                             \
+        else                                                                                                           \
+            hipLaunchKernelGGL((softmax_wave_rows_kernel<kWave, MODE, GRAD>),                                          \
+                               dim3((unsigned)ceil_div_sz(rows, kBlock / kWave)), dim3(kBlock), 0, ctx->stream, __VA_ARGS__); \
+    } while (0)
+
+// Launches softmax_long_rows_kernel<.., MODE, GRAD> in the shape that fits the row length (long_row_ok holds).
+#define ZG_LONG_ROWS(MODE, GRAD, ...)                                                                                  \
+    do {                                                                                                               \
+        if (cols <= 4096)                                                                                              \
+            hipLaunchKernelGGL((softmax_long_rows_kernel<256, 4, MODE, GRAD>), dim3((unsigned)rows), dim3(256), 0, ctx->stream, \
+                               __VA_ARGS__);                                                                           \
+        else if (cols <= 8192)                                                                                         \
+            hipLaunchKernelGGL((softmax_long_rows_kernel<256, 8, MODE, GRAD>), dim3((unsigned)rows), dim3(256), 0, ctx->stream, \
+                               __VA_ARGS__);                                                                           \
+        else                                                                                                           \
+            hipLaunchKernelGGL((softmax_long_rows_kernel<1024, 8, MODE, GRAD>), dim3((unsigned)rows), dim3(1024), 0,   \
+                               ctx->stream, __VA_ARGS__);                                                              \
+    } while (0)
 
 // src/nn/loss.zig:150-159.  ACC false: the gradient is written, not accumulated (same values as accumulating
 // into zeros, without reading them).
@@ -544,9 +573,11 @@ static unsigned smce_bwd_grid(size_t n) {
 }
 
 // smce_fwd and the loss's backward (upstream gradient 1) of a batch small enough for one workgroup, in one launch:
-// kFlatSingle / TPR rows of at most 4096 columns.  Per row the arithmetic is softmax_rows_kernel's, per gradient
-// element smce_bwd_kernel's, and the mean over the rows is formed as flat_single_kernel forms it, so every value
-// equals what the separate launches produce.  GRAD: 0 no gradient (smce_fwd alone), 1 written, 2 added to.
+// kFlatSingle / TPR rows of at most 4096 columns (rows of more than 1024 columns that the register-resident row kernels
+// take go there instead: 8 x 4096 21 us here, 7.7 us through them and the reduction of the row terms).  Per row the
+// arithmetic is that of the row kernel a larger batch of such rows takes (softmax_rows_kernel, or the lanes-per-row
+// kernel with its exponential), per gradient element smce_bwd_kernel's, and the mean over the rows is formed as
+// flat_single_kernel forms it.  GRAD: 0 no gradient (smce_fwd alone), 1 written, 2 added to.
 template <int TPR, int GRAD>
 __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* logits, const float* target, float* probs,
                                                                  float* loss, float* grad, size_t rows, size_t cols) {
@@ -561,6 +592,10 @@ __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* lo
     if (live) acc = row_online<TPR>(logits + row * cols, cols, lane);
     acc = group_reduce<OnlineAcc, TPR>(acc);
     float part = 0.f;
+    // rows the register-resident kernels take in a larger batch (wave_row_ok) get their exponential, so that a row's
+    // probabilities do not depend on the size of the batch it arrives in
+    const bool fast = cols % 4 == 0 && ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(target) |
+                                         reinterpret_cast<uintptr_t>(probs)) & 15u) == 0;
     if (live) {
         const float l = __fadd_rn(acc.m, logf(acc.s));
         const float* xr = logits + row * cols;
@@ -568,7 +603,7 @@ __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* lo
         float* pr = probs + row * cols;
         float* gr = grad + row * cols;
         for (size_t j = lane; j < cols; j += TPR) {
-            const float p = expf(__fsub_rn(xr[j], l));
+            const float p = fast ? fexp(__fsub_rn(xr[j], l)) : expf(__fsub_rn(xr[j], l));
             const float t = tr[j];
             pr[j] = p;
             if (t != 0.f) {
@@ -616,6 +651,63 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
             size_t k = row * cols + j;
             x_g[k] = __fadd_rn(x_g[k], __fmul_rn(y[k], __fsub_rn(y_g[k], part)));
         }
+}
+
+// The same with the rows of y and y_g held in registers (16-byte aligned rows of up to 32768 columns): NT threads per row
+// (lanes of a wave up to 1024 columns, a workgroup beyond), at most VEC float4 of each operand per thread, all loads of
+// the row in flight at once: one pass over the three operands instead of two passes of single values.
+template <int NT, int VEC>
+__global__ __launch_bounds__(NT <= kWave ? kBlock : NT) void softmax_bwd_rows_kernel(const float* y, const float* y_g,
+                                                                                      float* x_g, size_t rows, size_t cols) {
+    constexpr int kThreads = NT <= kWave ? kBlock : NT;
+    __shared__ float smem[kThreads / kWave];
+    __shared__ float bcast;
+    const int lane = threadIdx.x % NT;
+    const size_t row = (size_t)blockIdx.x * (kThreads / NT) + threadIdx.x / NT;
+    const bool live = row < rows;  // a workgroup per row (NT > 64) is always live: every thread reaches the barriers
+    const size_t c4 = cols >> 2;
+    const float4* a4 = reinterpret_cast<const float4*>(y + (live ? row : 0) * cols);
+    const float4* b4 = reinterpret_cast<const float4*>(y_g + (live ? row : 0) * cols);
+    float4* g4 = reinterpret_cast<float4*>(x_g + (live ? row : 0) * cols);
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 a[VEC], b[VEC], g[VEC];
+#pragma unroll
+    for (int u = 0; u < VEC; u++) {
+        const size_t j = lane + (size_t)u * NT;
+        const bool in = live && j < c4;
+        a[u] = in ? nt_load(a4 + j) : zero;
+        b[u] = in ? nt_load(b4 + j) : zero;
+        g[u] = in ? nt_load(g4 + j) : zero;
+    }
+    float part = 0.f;
+#pragma unroll
+    for (int u = 0; u < VEC; u++) {
+        part = __fadd_rn(part, __fmul_rn(a[u].x, b[u].x));
+        part = __fadd_rn(part, __fmul_rn(a[u].y, b[u].y));
+        part = __fadd_rn(part, __fmul_rn(a[u].z, b[u].z));
+        part = __fadd_rn(part, __fmul_rn(a[u].w, b[u].w));
+    }
+    if (NT <= kWave) {
+        part = group_reduce<SumAcc, (NT <= kWave ? NT : kWave)>(part);
+    } else {
+        part = block_reduce<SumAcc>(part, smem);
+        __syncthreads();
+        if (threadIdx.x == 0) bcast = part;
+        __syncthreads();
+        part = bcast;
+    }
+#pragma unroll
+    for (int u = 0; u < VEC; u++) {
+        const size_t j = lane + (size_t)u * NT;
+        if (live && j < c4) {
+            float4 o;
+            o.x = __fadd_rn(g[u].x, __fmul_rn(a[u].x, __fsub_rn(b[u].x, part)));
+            o.y = __fadd_rn(g[u].y, __fmul_rn(a[u].y, __fsub_rn(b[u].y, part)));
+            o.z = __fadd_rn(g[u].z, __fmul_rn(a[u].z, __fsub_rn(b[u].z, part)));
+            o.w = __fadd_rn(g[u].w, __fmul_rn(a[u].w, __fsub_rn(b[u].w, part)));
+            nt_store(o, g4 + j);
+        }
+    }
 }
 
 static int pick_tpr(size_t cols) {
@@ -751,7 +843,7 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
     {
         // a batch small enough for one workgroup: rows and their mean in one launch
         const int tpr = pick_tpr(cols);
-        if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr)) {
+        if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr) && !long_row_ok(logits, target, probs, rows, cols)) {
             ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_small_kernel<(T <= kWave ? T : kWave), 0>), dim3(1), dim3(kFlatSingle),
                                                     0, ctx->stream, logits, target, probs, loss, (float*)nullptr, rows, cols));
             ZG_LAUNCH_CHECK();
@@ -761,11 +853,9 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
     if (long_row_ok(logits, target, probs, rows, cols)) {
-        hipLaunchKernelGGL((softmax_long_rows_kernel<1>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
-                           logits, target, probs, row_loss, cols);
+        ZG_LONG_ROWS(1, 0, logits, target, probs, row_loss, cols, (float*)nullptr, 1.f);
     } else if (wave_row_ok(logits, target, probs, rows, cols)) {
-        hipLaunchKernelGGL((softmax_wave_rows_kernel<1>), dim3((unsigned)ceil_div_sz(rows, kBlock / kWave)), dim3(kBlock), 0,
-                           ctx->stream, logits, target, probs, row_loss, rows, cols);
+        ZG_WAVE_ROWS(1, 0, logits, target, probs, row_loss, rows, cols, (float*)nullptr, 1.f);
     } else {
         const int tpr = pick_tpr(cols);
         const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
@@ -812,7 +902,7 @@ ZG_API int zg_hip_smce_fwd_bwd(zg_hip_ctx* ctx, const float* logits, const float
     ZG_REQUIRE(logits && target && probs && loss && grad, "smce_fwd_bwd: null pointer");
     if (int rc = check_rows("smce_fwd_bwd", rows, cols)) return rc;
     const int tpr = pick_tpr(cols);
-    if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr)) {
+    if (tpr <= kWave && rows <= (size_t)(kFlatSingle / tpr) && !long_row_ok(logits, target, probs, rows, cols)) {
 #define ZG_SMALL(T)                                                                                                    \
     if (accumulate)                                                                                                    \
         hipLaunchKernelGGL((smce_small_kernel<T, 2>), dim3(1), dim3(kFlatSingle), 0, ctx->stream, logits, target,      \
@@ -838,20 +928,11 @@ ZG_API int zg_hip_smce_fwd_bwd(zg_hip_ctx* ctx, const float* logits, const float
         if (!row_loss) return ZG_HIP_EOOM;
         const float denom = (float)rows;
         if (long_row_ok(logits, target, probs, rows, cols)) {
-            if (accumulate)
-                hipLaunchKernelGGL((softmax_long_rows_kernel<1, 2>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
-                                   logits, target, probs, row_loss, cols, grad, denom);
-            else
-                hipLaunchKernelGGL((softmax_long_rows_kernel<1, 1>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream,
-                                   logits, target, probs, row_loss, cols, grad, denom);
+            if (accumulate) ZG_LONG_ROWS(1, 2, logits, target, probs, row_loss, cols, grad, denom);
+            else ZG_LONG_ROWS(1, 1, logits, target, probs, row_loss, cols, grad, denom);
         } else {
-            const dim3 grid((unsigned)ceil_div_sz(rows, kBlock / kWave));
-            if (accumulate)
-                hipLaunchKernelGGL((softmax_wave_rows_kernel<1, 2>), grid, dim3(kBlock), 0, ctx->stream, logits, target, probs,
-                                   row_loss, rows, cols, grad, denom);
-            else
-                hipLaunchKernelGGL((softmax_wave_rows_kernel<1, 1>), grid, dim3(kBlock), 0, ctx->stream, logits, target, probs,
-                                   row_loss, rows, cols, grad, denom);
+            if (accumulate) ZG_WAVE_ROWS(1, 2, logits, target, probs, row_loss, rows, cols, grad, denom);
+            else ZG_WAVE_ROWS(1, 1, logits, target, probs, row_loss, rows, cols, grad, denom);
         }
         ZG_LAUNCH_CHECK();
         return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, denom});
@@ -874,11 +955,9 @@ ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t 
     ZG_REQUIRE(x && y, "softmax_fwd: null pointer");
     if (int rc = check_rows("softmax_fwd", rows, cols)) return rc;
     if (long_row_ok(x, x, y, rows, cols)) {
-        hipLaunchKernelGGL((softmax_long_rows_kernel<0>), dim3((unsigned)rows), dim3(kLongRowThreads), 0, ctx->stream, x,
-                           (const float*)nullptr, y, (float*)nullptr, cols);
+        ZG_LONG_ROWS(0, 0, x, (const float*)nullptr, y, (float*)nullptr, cols, (float*)nullptr, 1.f);
     } else if (wave_row_ok(x, x, y, rows, cols)) {
-        hipLaunchKernelGGL((softmax_wave_rows_kernel<0>), dim3((unsigned)ceil_div_sz(rows, kBlock / kWave)), dim3(kBlock), 0,
-                           ctx->stream, x, (const float*)nullptr, y, (float*)nullptr, rows, cols);
+        ZG_WAVE_ROWS(0, 0, x, (const float*)nullptr, y, (float*)nullptr, rows, cols, (float*)nullptr, 1.f);
     } else {
         const int tpr = pick_tpr(cols);
         const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
@@ -894,6 +973,20 @@ ZG_API int zg_hip_softmax_bwd(zg_hip_ctx* ctx, const float* y, const float* y_g,
     if (rows == 0 || cols == 0) return ZG_HIP_OK;
     ZG_REQUIRE(y && y_g && x_g, "softmax_bwd: null pointer");
     if (int rc = check_rows("softmax_bwd", rows, cols)) return rc;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(y_g) | reinterpret_cast<uintptr_t>(x_g);
+    if (cols % 4 == 0 && (bits & 15u) == 0 && cols <= 32768 && rows <= 0x7fffffffull) {
+#define ZG_BWD_ROWS(NT, VEC, ROWS_PER_WG)                                                                              \
+    hipLaunchKernelGGL((softmax_bwd_rows_kernel<NT, VEC>), dim3((unsigned)ceil_div_sz(rows, ROWS_PER_WG)),             \
+                       dim3(NT <= kWave ? kBlock : NT), 0, ctx->stream, y, y_g, x_g, rows, cols)
+        if (cols <= 256) ZG_BWD_ROWS(16, 4, kBlock / 16);
+        else if (cols <= 1024) ZG_BWD_ROWS(64, 4, kBlock / 64);
+        else if (cols <= 4096) ZG_BWD_ROWS(256, 4, 1);
+        else if (cols <= 8192) ZG_BWD_ROWS(256, 8, 1);
+        else ZG_BWD_ROWS(1024, 8, 1);
+#undef ZG_BWD_ROWS
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     const int tpr = pick_tpr(cols);
     const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, y, y_g,

@@ -207,7 +207,13 @@ def test_axpy_scale_clip(oracle, hip, n):
 # ----------------------------------------------------------------------------------------------
 AXIS_SHAPES = [([64, 10], 1), ([64, 10], 0), ([64, 2], 1), ([2708, 16], 0), ([1000, 4096], 1), ([1000, 4096], 0),
                ([33, 1001], 1), ([33, 1001], 0), ([6, 50, 7], 1), ([3, 4, 5, 6], 2), ([2, 3, 4], 0), ([4, 20000], 1),
-               ([5, 70000], 1), ([70000, 3], 0), ([1, 5, 8], 1)]
+               ([5, 70000], 1), ([70000, 3], 0), ([1, 5, 8], 1),
+               # few long rows, cut into segments and combined in a second launch: a single row, a row length that is
+               # no multiple of four, rows that end inside a segment, a reduced first axis of a vector
+               ([1, 300000], 1), ([3, 262145], 1), ([7, 140002], 1), ([64, 16384], 1), ([100, 20000], 1), ([300000], 0),
+               ([300, 16388], 1), ([2, 3, 140000], 2),
+               # rows whose last trip of loads is partial
+               ([700, 1000], 1), ([300, 1028], 1), ([900, 260], 1), ([50, 2044], 1)]
 
 
 @pytest.mark.parametrize("shape,dim", AXIS_SHAPES)
@@ -229,6 +235,25 @@ def test_sum_max_argmax_along(oracle, hip, shape, dim):
     a, b = both(oracle, hip, "argmax_along", {"x": x, "x_shape": shape, "y": np.zeros(out_n, np.uint64), "dim": dim}, ["y"])
     np.testing.assert_array_equal(a["y"], b["y"])
     np.testing.assert_array_equal(b["y"], np.argmax(x.reshape(shape), axis=dim).ravel().astype(np.uint64))
+
+
+def test_argmax_ties_across_the_segments_of_a_long_row_take_the_first(oracle, hip):
+    cols = 200_000
+    x = np.zeros((3, cols), np.float32)
+    x[0, [5000, 70000, 199999]] = 2.0      # equal maxima in three segments
+    x[1, [150000, 150001]] = 1.0
+    x[2, :] = -np.inf                       # nothing to find: the host loop answers 0
+    a, b = both(oracle, hip, "argmax_along", {"x": x.ravel(), "x_shape": [3, cols], "y": np.zeros(3, np.uint64), "dim": 1}, ["y"])
+    np.testing.assert_array_equal(a["y"], b["y"])
+    np.testing.assert_array_equal(b["y"], np.asarray([5000, 150000, 0], np.uint64))
+    a, b = both(oracle, hip, "max_along", {"x": x.ravel(), "x_shape": [3, cols], "y": np.zeros(3, np.float32), "dim": 1}, ["y"])
+    np.testing.assert_array_equal(a["y"], b["y"])
+    # integer values: the sum is exact in any order, with alpha and beta applied once
+    xi = rng(5).integers(-4, 5, (5, 131075)).astype(np.float32)
+    y0 = np.arange(5, dtype=np.float32)
+    out = run_op(hip, "sum_along", {"x": xi.ravel(), "x_shape": [5, 131075], "y": y0.copy(), "dim": 1, "alpha": 2.0, "beta": -1.0},
+                 ["y"])["y"]
+    np.testing.assert_array_equal(out, 2.0 * xi.astype(np.float64).sum(axis=1) - y0)
 
 
 def test_argmax_ties_take_first(oracle, hip):

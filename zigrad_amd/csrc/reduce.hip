@@ -83,8 +83,12 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
         if (vec) {
             const float4* x4 = reinterpret_cast<const float4*>(xr);
             const size_t c4 = cols >> 2;
-            size_t j = lane;
-            for (; j + 3 * TPR < c4; j += 4 * TPR) {
+            // whole trips of four loads per lane, then one partial trip whose loads are in flight together as well, the
+            // ones past the row's end left out: the trip count is the same for every lane, so a row of 1000 columns takes
+            // one memory round trip like a row of 1024 (lanes that finish one by one cost a quarter more)
+            size_t j0 = 0;
+            for (; j0 + 4 * TPR <= c4; j0 += 4 * TPR) {
+                const size_t j = j0 + lane;
                 float4 v0 = nt_load(x4 + j), v1 = nt_load(x4 + j + TPR), v2 = nt_load(x4 + j + 2 * TPR), v3 = nt_load(x4 + j + 3 * TPR);
                 const float4 vs[4] = {v0, v1, v2, v3};
 #pragma unroll
@@ -96,13 +100,23 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
                     acc = P::combine(acc, A::term(vs[u].w, c + 3));
                 }
             }
-            for (; j < c4; j += TPR) {
-                float4 v = x4[j];
-                uint32_t c = (uint32_t)(4 * j);
-                acc = P::combine(acc, A::term(v.x, c + 0));
-                acc = P::combine(acc, A::term(v.y, c + 1));
-                acc = P::combine(acc, A::term(v.z, c + 2));
-                acc = P::combine(acc, A::term(v.w, c + 3));
+            if (j0 < c4) {
+                const size_t j = j0 + lane;
+                const bool streamed = cols >= 512;  // rows of a few hundred bytes are read faster through the caches
+                float4 vs[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    if (j + (size_t)u * TPR < c4) vs[u] = streamed ? nt_load(x4 + j + (size_t)u * TPR) : x4[j + (size_t)u * TPR];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    if (j + (size_t)u * TPR < c4) {
+                        uint32_t c = (uint32_t)(4 * (j + (size_t)u * TPR));
+                        acc = P::combine(acc, A::term(vs[u].x, c + 0));
+                        acc = P::combine(acc, A::term(vs[u].y, c + 1));
+                        acc = P::combine(acc, A::term(vs[u].z, c + 2));
+                        acc = P::combine(acc, A::term(vs[u].w, c + 3));
+                    }
+                }
             }
         } else {
             for (size_t j = lane; j < cols; j += TPR) acc = P::combine(acc, A::term(xr[j], (uint32_t)j));
@@ -115,6 +129,50 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
         acc = block_reduce<P>(acc, smem);
     }
     if (lane == 0 && row < rows) A::store(y, row, acc, alpha, beta);
+}
+
+// inner == 1 with few, long rows (a handful of rows of a million columns would keep a handful of workgroups busy): the
+// rows are cut into segments of `seg` columns (a multiple of 4), workgroup (s, r) reduces segment s of row r and leaves
+// its result at partials[s * rows + r]; col_final_kernel then combines a row's segments in a fixed order.
+template <class A>
+__global__ __launch_bounds__(kBlock) void row_segments_kernel(const float* x, typename A::P::Acc* partials, size_t rows,
+                                                               size_t cols, size_t seg) {
+    using P = typename A::P;
+    __shared__ typename P::Acc smem[kBlock / kWave];
+    const size_t s = blockIdx.x, row = blockIdx.y;
+    const size_t c_begin = s * seg, c_end = c_begin + seg < cols ? c_begin + seg : cols;
+    const float* xr = x + row * cols;
+    typename P::Acc acc = P::init();
+    const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15u) == 0) && (cols % 4 == 0);
+    if (vec) {
+        const float4* x4 = reinterpret_cast<const float4*>(xr);
+        const size_t j_end = c_end >> 2;
+        size_t j = (c_begin >> 2) + threadIdx.x;
+        for (; j + 3 * kBlock < j_end; j += 4 * kBlock) {
+            const float4 vs[4] = {nt_load(x4 + j), nt_load(x4 + j + kBlock), nt_load(x4 + j + 2 * kBlock),
+                                  nt_load(x4 + j + 3 * kBlock)};
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t c = (uint32_t)(4 * (j + (size_t)u * kBlock));
+                acc = P::combine(acc, A::term(vs[u].x, c + 0));
+                acc = P::combine(acc, A::term(vs[u].y, c + 1));
+                acc = P::combine(acc, A::term(vs[u].z, c + 2));
+                acc = P::combine(acc, A::term(vs[u].w, c + 3));
+            }
+        }
+        for (; j < j_end; j += kBlock) {
+            const float4 v = x4[j];
+            const uint32_t c = (uint32_t)(4 * j);
+            acc = P::combine(acc, A::term(v.x, c + 0));
+            acc = P::combine(acc, A::term(v.y, c + 1));
+            acc = P::combine(acc, A::term(v.z, c + 2));
+            acc = P::combine(acc, A::term(v.w, c + 3));
+        }
+    } else {
+        for (size_t j = c_begin + threadIdx.x; j < c_end; j += kBlock) acc = P::combine(acc, A::term(xr[j], (uint32_t)j));
+    }
+    acc = block_reduce<P>(acc, smem);
+    if (threadIdx.x == 0) partials[s * rows + row] = acc;
 }
 
 // inner > 1: column-style, see col_reduce_block
@@ -187,6 +245,27 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     if (outer == 0 || R == 0 || inner == 0) return ZG_HIP_OK;
     if (inner == 1) {
         const size_t rows = outer, cols = R;
+        // few long rows: segments of at least 4096 columns, about eight workgroups per compute unit, then a row's segments
+        // are combined by the column kernel's final pass (7 x 1048576: 137 -> 9 us; 64 x 262144: 40 -> 13 us)
+        // (below a million elements or so, rows of up to 65536 columns are done sooner in the one launch: 7 x 65536
+        // 5.1 against 7.6 us)
+        if (rows < 2 * (size_t)ctx->n_cu && (cols >= 131072 || (cols >= 16384 && rows * cols >= ((size_t)1 << 20)))) {
+            const size_t want = ceil_div_sz(8 * (size_t)ctx->n_cu, rows);
+            size_t seg = ceil_div_sz(ceil_div_sz(cols, want), 1024) * 1024;
+            if (seg < 4096) seg = 4096;
+            const size_t n_seg = ceil_div_sz(cols, seg);
+            if (n_seg >= 2) {
+                Acc* partials = (Acc*)workspace(ctx, n_seg * rows * sizeof(Acc));
+                if (!partials) return ZG_HIP_EOOM;
+                hipLaunchKernelGGL((row_segments_kernel<A>), dim3((unsigned)n_seg, (unsigned)rows), dim3(kBlock), 0, ctx->stream,
+                                   x, partials, rows, cols, seg);
+                ZG_LAUNCH_CHECK();
+                hipLaunchKernelGGL((col_final_kernel<A>), dim3((unsigned)ceil_div_sz(rows, 64)), dim3(kBlock), 0, ctx->stream,
+                                   partials, y, rows, rows, (int)n_seg, alpha, beta);
+                ZG_LAUNCH_CHECK();
+                return ZG_HIP_OK;
+            }
+        }
 #define ZG_ROW(TPR)                                                                                          \
     hipLaunchKernelGGL((row_reduce_kernel<A, TPR>), dim3((unsigned)ceil_div_sz(rows, kBlock / TPR)), dim3(kBlock), 0, \
                        ctx->stream, x, y, rows, cols, alpha, beta)

@@ -226,7 +226,11 @@ def test_bmm_32x512_cubed(oracle, hip):
         assert rel_fro(res[1], res[0]) <= TOL
 
 
-@pytest.mark.parametrize("m,n", [(2, 2), (64, 784), (1000, 33), (5, 4097)])
+@pytest.mark.parametrize("m,n", [(2, 2), (64, 784), (1000, 33), (5, 4097),
+                                 # every lanes-per-row shape of the row kernel, rows cut into segments, a reduced axis cut
+                                 # into many chunks, tiles of the transpose that end inside the matrix
+                                 (3, 300000), (7, 20000), (300, 16384), (100000, 8), (5000, 64), (4096, 256), (70000, 12),
+                                 (130, 5000), (64, 64), (256, 1000), (1000, 1024), (68, 132), (1, 70000), (70000, 1)])
 def test_matvec_outer_transpose(oracle, hip, m, n):
     r = rng(m + n)
     A = r.standard_normal((m, n)).astype(np.float32)

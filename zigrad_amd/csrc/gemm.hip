@@ -1675,68 +1675,214 @@ static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k,
 // matvec / outer / transpose
 // ------------------------------------------------------------------------------------------------
 
-// y = alpha * A x + beta * y, A is [m, n] row-major: one wave per row
-__global__ __launch_bounds__(256) void gemv_n_kernel(const float* A, const float* x, float* y, size_t m, size_t n,
-                                                      float alpha, float beta) {
-    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= m) return;
-    const int lane = threadIdx.x & 63;
-    const float* a = A + row * n;
-    float s = 0.f;
-    for (size_t j = lane; j < n; j += 64) s += a[j] * x[j];
+// y = alpha * A x + beta * y, A is [m, n] row-major (cblas_sgemv, src/device/host_device.zig:232-240).  TPR threads per row
+// (4, 16 or 64 lanes of a wave, or a whole workgroup), 256 / TPR rows per workgroup; a thread has four 16-byte loads of
+// its row in flight (and the matching pieces of x, which stay in the caches), the partial sums of the four are added
+// in a fixed order and the threads of a row combine by shuffles (through LDS for a workgroup).  Long rows on few
+// workgroups are cut into segments of `seg` columns (blockIdx.y): the segment sums go to part [segments][m] and
+// vec_final_kernel adds them in segment order.  VEC false: any alignment, any n, value by value.
+template <int TPR, bool VEC>
+__global__ __launch_bounds__(256) void gemv_rows_kernel(const float* A, const float* x, float* y, float* part, size_t m,
+                                                         size_t n, size_t seg, float alpha, float beta) {
+    __shared__ float smem[256 / kWave];
+    const int lane = threadIdx.x % TPR;
+    const size_t row = (size_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
+    const bool live = row < m;
+    const size_t c0 = (size_t)blockIdx.y * seg, c1 = c0 + seg < n ? c0 + seg : n;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (live) {
+        const float* a = A + row * n;
+        if (VEC) {
+            const float4* a4 = reinterpret_cast<const float4*>(a);
+            const float4* x4 = reinterpret_cast<const float4*>(x);
+            const size_t j1 = c1 >> 2;
+            auto dot4 = [](float4 u, float4 v) { return ((u.x * v.x + u.y * v.y) + u.z * v.z) + u.w * v.w; };
+            size_t j0 = c0 >> 2;
+            for (; j0 + 4 * TPR <= j1; j0 += 4 * TPR) {
+                const size_t j = j0 + lane;
+                const float4 u0 = a4[j], u1 = a4[j + TPR], u2 = a4[j + 2 * TPR], u3 = a4[j + 3 * TPR];
+                s0 += dot4(u0, x4[j]);
+                s1 += dot4(u1, x4[j + TPR]);
+                s2 += dot4(u2, x4[j + 2 * TPR]);
+                s3 += dot4(u3, x4[j + 3 * TPR]);
+            }
+            if (j0 < j1) {  // the last, partial trip: its loads in flight together, the ones past the end left out
+                const size_t j = j0 + lane;
+                float4 u[4];
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
-    if (lane == 0) y[row] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[row];
+                for (int k = 0; k < 4; k++)
+                    if (j + (size_t)k * TPR < j1) u[k] = a4[j + (size_t)k * TPR];
+                if (j < j1) s0 += dot4(u[0], x4[j]);
+                if (j + TPR < j1) s1 += dot4(u[1], x4[j + TPR]);
+                if (j + 2 * TPR < j1) s2 += dot4(u[2], x4[j + 2 * TPR]);
+                if (j + 3 * TPR < j1) s3 += dot4(u[3], x4[j + 3 * TPR]);
+            }
+        } else {
+            size_t j = c0 + lane;
+            for (; j + 3 * TPR < c1; j += 4 * TPR) {
+                const float u0 = a[j], u1 = a[j + TPR], u2 = a[j + 2 * TPR], u3 = a[j + 3 * TPR];
+                s0 += u0 * x[j];
+                s1 += u1 * x[j + TPR];
+                s2 += u2 * x[j + 2 * TPR];
+                s3 += u3 * x[j + 3 * TPR];
+            }
+            for (; j < c1; j += TPR) s0 += a[j] * x[j];
+        }
+    }
+    float s = (s0 + s1) + (s2 + s3);
+    if (TPR <= kWave) {
+        s = group_reduce<SumAcc, (TPR <= kWave ? TPR : kWave)>(s);
+    } else {
+        s = block_reduce<SumAcc>(s, smem);
+    }
+    if (live && lane == 0) {
+        if (part) part[(size_t)blockIdx.y * m + row] = s;
+        else y[row] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[row];
+    }
 }
 
-// y = alpha * A^T x + beta * y, A is [m, n] row-major, y has n entries.  A workgroup owns 64 columns and one chunk of
-// rows: its four waves take every fourth row of the chunk (each wave reads 256 contiguous bytes of a row), their
-// sums are added in wave order through LDS.  One chunk: the result is written here; several: the chunk sums go to
-// `part` [chunks][n] and gemv_t_final_kernel adds them in chunk order.
+// y[o] = alpha * (part[0][o] + part[1][o] + ...) + beta * y[o] for partial results [chunks][n_out]: a workgroup owns 64
+// adjacent outputs, wave w adds chunks w, w + 4, ... with sixteen loads in flight, and the four wave sums are added in
+// wave order.
+__global__ __launch_bounds__(256) void vec_final_kernel(const float* part, float* y, size_t n_out, size_t chunks, float alpha,
+                                                         float beta) {
+    __shared__ float smem[4][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const size_t o = (size_t)blockIdx.x * 64 + lane;
+    float s = 0.f;
+    if (o < n_out) {
+        for (size_t base = 0; base < chunks; base += 64) {
+            float t[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const size_t k = base + (size_t)w + 4 * (size_t)u;
+                t[u] = k < chunks ? part[k * n_out + o] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 16; u++) s += t[u];
+        }
+    }
+    smem[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && o < n_out) {
+        s = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
+        y[o] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[o];
+    }
+}
+
+// y = alpha * A^T x + beta * y, A is [m, n] row-major, y has n entries.  A workgroup is cx column-threads by ry = 256 / cx
+// row-threads and owns cx * V adjacent columns and one chunk of rows: a thread walks rows ty, ty + ry, ... of the chunk
+// with eight loads of V columns in flight (V = 4: 16 bytes), multiplies by x[row] and adds in row order; the row-threads
+// of a column combine in ty order through LDS.  One chunk: the result is written here; several: the chunk sums go to
+// part [chunks][n] and vec_final_kernel adds them in chunk order.
+template <int V>
 __global__ __launch_bounds__(256) void gemv_t_kernel(const float* A, const float* x, float* y, float* part, size_t m,
-                                                      size_t n, size_t rows_per_chunk, float alpha, float beta) {
-    __shared__ float s_part[4][64];
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const size_t col = (size_t)blockIdx.x * 64 + tx;
+                                                      size_t n, int log2_cx, size_t rows_per_chunk, float alpha, float beta) {
+    __shared__ float smem[256 * V];
+    const int cx = 1 << log2_cx, ry = 256 >> log2_cx;
+    const int tx = threadIdx.x & (cx - 1), ty = threadIdx.x >> log2_cx;
+    const size_t col0 = ((size_t)blockIdx.x * cx + tx) * V;
     const size_t r0 = (size_t)blockIdx.y * rows_per_chunk;
     const size_t r1 = r0 + rows_per_chunk < m ? r0 + rows_per_chunk : m;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    if (col < n) {
-        size_t i = r0 + ty;
-        for (; i + 12 < r1; i += 16) {  // four loads in flight per thread
-            const float a0 = A[i * n + col], a1 = A[(i + 4) * n + col], a2 = A[(i + 8) * n + col], a3 = A[(i + 12) * n + col];
-            s0 += a0 * x[i];
-            s1 += a1 * x[i + 4];
-            s2 += a2 * x[i + 8];
-            s3 += a3 * x[i + 12];
+    float acc[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) acc[v] = 0.f;
+    const bool active = col0 < n;
+    if (active) {
+        const float* ab = A + col0;
+        size_t r = r0 + ty;
+        if constexpr (V == 4) {
+            for (; r + 7 * (size_t)ry < r1; r += 8 * (size_t)ry) {
+                float4 u[8];
+                float xs[8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    u[k] = *reinterpret_cast<const float4*>(ab + (r + (size_t)k * ry) * n);
+                    xs[k] = x[r + (size_t)k * ry];
+                }
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    acc[0] += u[k].x * xs[k];
+                    acc[1 % V] += u[k].y * xs[k];
+                    acc[2 % V] += u[k].z * xs[k];
+                    acc[3 % V] += u[k].w * xs[k];
+                }
+            }
+            for (; r < r1; r += ry) {
+                const float4 u = *reinterpret_cast<const float4*>(ab + r * n);
+                const float xv = x[r];
+                acc[0] += u.x * xv;
+                acc[1 % V] += u.y * xv;
+                acc[2 % V] += u.z * xv;
+                acc[3 % V] += u.w * xv;
+            }
+        } else {
+            for (; r + 7 * (size_t)ry < r1; r += 8 * (size_t)ry) {
+                float u[8], xs[8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    u[k] = ab[(r + (size_t)k * ry) * n];
+                    xs[k] = x[r + (size_t)k * ry];
+                }
+#pragma unroll
+                for (int k = 0; k < 8; k++) acc[0] += u[k] * xs[k];
+            }
+            for (; r < r1; r += ry) acc[0] += ab[r * n] * x[r];
         }
-        for (; i < r1; i += 4) s0 += A[i * n + col] * x[i];
     }
-    s_part[ty][tx] = (s0 + s1) + (s2 + s3);
+#pragma unroll
+    for (int v = 0; v < V; v++) smem[threadIdx.x * V + v] = acc[v];
     __syncthreads();
-    if (ty == 0 && col < n) {
-        const float s = ((s_part[0][tx] + s_part[1][tx]) + s_part[2][tx]) + s_part[3][tx];
-        if (part) part[(size_t)blockIdx.y * n + col] = s;
-        else y[col] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[col];
+    if (ty == 0 && active) {
+        for (int t = 1; t < ry; t++) {
+#pragma unroll
+            for (int v = 0; v < V; v++) acc[v] += smem[((t << log2_cx) + tx) * V + v];
+        }
+#pragma unroll
+        for (int v = 0; v < V; v++) {
+            const size_t c = col0 + v;
+            if (c < n) {
+                if (part) part[(size_t)blockIdx.y * n + c] = acc[v];
+                else y[c] = (beta == 0.f) ? alpha * acc[v] : alpha * acc[v] + beta * y[c];
+            }
+        }
     }
 }
 
-__global__ __launch_bounds__(256) void gemv_t_final_kernel(const float* part, float* y, size_t n, size_t chunks, float alpha,
-                                                            float beta) {
-    const size_t col = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (col >= n) return;
-    float s = part[col];
-    for (size_t c = 1; c < chunks; c++) s += part[c * n + col];
-    y[col] = (beta == 0.f) ? alpha * s : alpha * s + beta * y[col];
-}
-
-// A += alpha * x y^T   (cblas_sger, src/device/host_device.zig:252-258)
+// A += alpha * x y^T   (cblas_sger, src/device/host_device.zig:252-258).  VEC: 16-byte pieces of a row of A (rows that start
+// on 16-byte boundaries), four per thread in flight.
+template <bool VEC>
 __global__ __launch_bounds__(256) void ger_kernel(const float* x, size_t xl, const float* y, size_t yl, float* A,
                                                    float alpha) {
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, nt = (size_t)gridDim.x * 256;
-    for (; i < xl * yl; i += nt) {
-        size_t r = i / yl, c = i % yl;
-        A[i] = __fadd_rn(A[i], __fmul_rn(__fmul_rn(alpha, x[r]), y[c]));
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, nt = (size_t)gridDim.x * 256;
+    if (VEC) {
+        const size_t yl4 = yl >> 2, n4 = xl * yl4;
+        float4* a4 = reinterpret_cast<float4*>(A);
+        const float4* y4 = reinterpret_cast<const float4*>(y);
+        auto piece = [&](size_t i, float4 a) {
+            const size_t r = i / yl4, c = i % yl4;
+            const float ax = __fmul_rn(alpha, x[r]);
+            const float4 yv = y4[c];
+            a.x = __fadd_rn(a.x, __fmul_rn(ax, yv.x));
+            a.y = __fadd_rn(a.y, __fmul_rn(ax, yv.y));
+            a.z = __fadd_rn(a.z, __fmul_rn(ax, yv.z));
+            a.w = __fadd_rn(a.w, __fmul_rn(ax, yv.w));
+            return a;
+        };
+        size_t i = tid;
+        for (; i + 3 * nt < n4; i += 4 * nt) {
+            const float4 u0 = nt_load(a4 + i), u1 = nt_load(a4 + i + nt), u2 = nt_load(a4 + i + 2 * nt), u3 = nt_load(a4 + i + 3 * nt);
+            nt_store(piece(i, u0), a4 + i);
+            nt_store(piece(i + nt, u1), a4 + i + nt);
+            nt_store(piece(i + 2 * nt, u2), a4 + i + 2 * nt);
+            nt_store(piece(i + 3 * nt, u3), a4 + i + 3 * nt);
+        }
+        for (; i < n4; i += nt) a4[i] = piece(i, a4[i]);
+    } else {
+        for (size_t i = tid; i < xl * yl; i += nt) {
+            const size_t r = i / yl, c = i % yl;
+            A[i] = __fadd_rn(A[i], __fmul_rn(__fmul_rn(alpha, x[r]), y[c]));
+        }
     }
 }
 
@@ -1757,6 +1903,56 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* A, float* B
             float v = tile[tx][r];
             float* b = B + j * m + i;
             *b = (alpha == 0.f) ? v : __fadd_rn(v, __fmul_rn(alpha, *b));
+        }
+    }
+}
+
+// The same through a 64 x 64 tile with 16-byte accesses on both sides (m and n multiples of 4, A and B on 16-byte
+// boundaries): thread (tx, ty) of 16 x 16 reads pieces tx of rows ty, ty + 16, ... of the tile of A, and writes pieces
+// tx of rows ty, ty + 16, ... of the tile of B, whose four values come from four rows of the LDS tile.
+__global__ __launch_bounds__(256) void transpose_vec_kernel(const float* A, float* B, size_t m, size_t n, float alpha) {
+    __shared__ float tile[64][65];
+    const size_t bi = (size_t)blockIdx.y * 64, bj = (size_t)blockIdx.x * 64;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    float4 u[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const size_t i = bi + ty + 16 * k, j = bj + 4 * tx;
+        if (i < m && j < n) u[k] = *reinterpret_cast<const float4*>(A + i * n + j);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const size_t i = bi + ty + 16 * k, j = bj + 4 * tx;
+        if (i < m && j < n) {
+            float* t = &tile[ty + 16 * k][4 * tx];
+            t[0] = u[k].x;
+            t[1] = u[k].y;
+            t[2] = u[k].z;
+            t[3] = u[k].w;
+        }
+    }
+    __syncthreads();
+    float4 old[4];
+    if (alpha != 0.f) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const size_t j = bj + ty + 16 * k, i = bi + 4 * tx;  // B[j, i .. i + 3]
+            if (j < n && i < m) old[k] = *reinterpret_cast<const float4*>(B + j * m + i);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int r = ty + 16 * k;
+        const size_t j = bj + r, i = bi + 4 * tx;
+        if (j < n && i < m) {
+            float4 v = make_float4(tile[4 * tx][r], tile[4 * tx + 1][r], tile[4 * tx + 2][r], tile[4 * tx + 3][r]);
+            if (alpha != 0.f) {
+                v.x = __fadd_rn(v.x, __fmul_rn(alpha, old[k].x));
+                v.y = __fadd_rn(v.y, __fmul_rn(alpha, old[k].y));
+                v.z = __fadd_rn(v.z, __fmul_rn(alpha, old[k].z));
+                v.w = __fadd_rn(v.w, __fmul_rn(alpha, old[k].w));
+            }
+            *reinterpret_cast<float4*>(B + j * m + i) = v;
         }
     }
 }
@@ -2148,16 +2344,69 @@ ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float*
     ZG_CTX(ctx);
     if (m == 0 || n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(A && x && y, "matvec: null pointer");
-    if (!trans_a)
-        hipLaunchKernelGGL(gemv_n_kernel, dim3((unsigned)ceil_div_sz(m, 4)), dim3(256), 0, ctx->stream, A, x, y, m, n,
-                           alpha, beta);
-    else {
-        // enough row chunks to put about two workgroups on every CU, at least 64 rows each, at most 64 chunks
-        const size_t col_blocks = ceil_div_sz(n, 64);
-        size_t chunks = ceil_div_sz(2 * (size_t)ctx->n_cu, col_blocks);
-        if (chunks > m / 64) chunks = m / 64;
-        if (chunks > 64) chunks = 64;
-        if (chunks < 1) chunks = 1;
+    const size_t n_cu = (size_t)ctx->n_cu;
+    if (!trans_a) {
+        const bool vec = aligned16(A) && aligned16(x) && n % 4 == 0;
+        // lanes per row by row length; a whole workgroup for rows of more than 4096 columns
+        const int tpr = n <= 64 ? 4 : n <= 256 ? 16 : n <= 4096 ? 64 : 256;
+        const size_t wgs = ceil_div_sz(m, (size_t)(256 / tpr));
+        ZG_REQUIRE(wgs <= 0x7fffffffull, "matvec: too many rows");
+        // few long rows: segments of at least 4096 columns, about eight workgroups per compute unit
+        size_t seg = n, n_seg = 1;
+        if (tpr == 256 && m < 2 * n_cu && n >= 16384) {
+            seg = ceil_div_sz(ceil_div_sz(n, ceil_div_sz(8 * n_cu, m)), 1024) * 1024;
+            if (seg < 4096) seg = 4096;
+            n_seg = ceil_div_sz(n, seg);
+            if (n_seg > 65535) {
+                n_seg = 65535;
+                seg = ceil_div_sz(ceil_div_sz(n, n_seg), 1024) * 1024;
+                n_seg = ceil_div_sz(n, seg);
+            }
+        }
+        float* part = nullptr;
+        if (n_seg > 1) {
+            part = (float*)workspace(ctx, n_seg * m * sizeof(float));
+            if (!part) return ZG_HIP_EOOM;
+        }
+        const dim3 grid((unsigned)wgs, (unsigned)n_seg);
+#define ZG_GEMV(T)                                                                                                     \
+    do {                                                                                                               \
+        if (vec) hipLaunchKernelGGL((gemv_rows_kernel<T, true>), grid, dim3(256), 0, ctx->stream, A, x, y, part, m, n, seg, \
+                                    alpha, beta);                                                                      \
+        else hipLaunchKernelGGL((gemv_rows_kernel<T, false>), grid, dim3(256), 0, ctx->stream, A, x, y, part, m, n, seg, \
+                                alpha, beta);                                                                          \
+    } while (0)
+        if (tpr == 4) ZG_GEMV(4);
+        else if (tpr == 16) ZG_GEMV(16);
+        else if (tpr == 64) ZG_GEMV(64);
+        else ZG_GEMV(256);
+#undef ZG_GEMV
+        ZG_LAUNCH_CHECK();
+        if (n_seg > 1)
+            hipLaunchKernelGGL(vec_final_kernel, dim3((unsigned)ceil_div_sz(m, 64)), dim3(256), 0, ctx->stream, part, y, m,
+                               n_seg, alpha, beta);
+    } else {
+        // column-threads as the column reductions have them: 4 columns per thread where rows start on 16-byte
+        // boundaries, at most 64 column-threads (1 KiB of a row) per workgroup
+        const int V = (n % 4 == 0 && aligned16(A)) ? 4 : 1;
+        const size_t colv = n / V;
+        int log2_cx = 0;
+        // 16 row-threads (and 16 column-threads) where a row-thread gets four rows or more, fewer for shorter matrices
+        // (7 x 1048576: 11.5 us with 16 row-threads, 5.7 us with 4; 64 x 1048576: 50.5 us with 4, 39.1 us with 16)
+        const int cx_max = m >= 64 ? 4 : m >= 32 ? 5 : 6;
+        while (((size_t)1 << log2_cx) < colv && log2_cx < cx_max) log2_cx++;
+        // narrower column groups (down to 16 column-threads) while they are fewer than two per compute unit: a wide matrix
+        // of few rows then needs no row chunks at all
+        while (log2_cx > 4 && ceil_div_sz(colv, (size_t)1 << log2_cx) < 2 * n_cu) log2_cx--;
+        const size_t gx = ceil_div_sz(colv, (size_t)1 << log2_cx);
+        const size_t ry = (size_t)256 >> log2_cx;
+        // row chunks: about two workgroups per compute unit, at least 64 rows and eight trips of ry rows each, at most 1024
+        size_t chunks = ceil_div_sz(2 * n_cu, gx);
+        size_t max_chunks = ceil_div_sz(m, ry * 8);
+        if (max_chunks > m / 64) max_chunks = m / 64;
+        if (chunks > max_chunks) chunks = max_chunks;
+        if (chunks > 1024) chunks = 1024;
+        if (m * n <= kColSingleChunkMax || chunks < 1) chunks = 1;
         const size_t rows_per_chunk = ceil_div_sz(m, chunks);
         chunks = ceil_div_sz(m, rows_per_chunk);
         float* part = nullptr;
@@ -2165,14 +2414,18 @@ ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float*
             part = (float*)workspace(ctx, chunks * n * sizeof(float));
             if (!part) return ZG_HIP_EOOM;
         }
-        ZG_REQUIRE(col_blocks <= 0x7fffffffull, "matvec: too many columns");
-        hipLaunchKernelGGL(gemv_t_kernel, dim3((unsigned)col_blocks, (unsigned)chunks), dim3(256), 0, ctx->stream, A, x, y,
-                           part, m, n, rows_per_chunk, alpha, beta);
+        ZG_REQUIRE(gx <= 0x7fffffffull, "matvec: too many columns");
+        const dim3 grid((unsigned)gx, (unsigned)chunks);
+        if (V == 4)
+            hipLaunchKernelGGL(gemv_t_kernel<4>, grid, dim3(256), 0, ctx->stream, A, x, y, part, m, n, log2_cx, rows_per_chunk,
+                               alpha, beta);
+        else
+            hipLaunchKernelGGL(gemv_t_kernel<1>, grid, dim3(256), 0, ctx->stream, A, x, y, part, m, n, log2_cx, rows_per_chunk,
+                               alpha, beta);
         ZG_LAUNCH_CHECK();
-        if (chunks > 1) {
-            hipLaunchKernelGGL(gemv_t_final_kernel, dim3((unsigned)ceil_div_sz(n, 256)), dim3(256), 0, ctx->stream, part, y,
-                               n, chunks, alpha, beta);
-        }
+        if (chunks > 1)
+            hipLaunchKernelGGL(vec_final_kernel, dim3((unsigned)ceil_div_sz(n, 64)), dim3(256), 0, ctx->stream, part, y, n,
+                               chunks, alpha, beta);
     }
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
@@ -2182,9 +2435,11 @@ ZG_API int zg_hip_outer(zg_hip_ctx* ctx, const float* x, size_t xl, const float*
     ZG_CTX(ctx);
     if (xl == 0 || yl == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x && y && A, "outer: null pointer");
-    size_t blocks = ceil_div_sz(xl * yl, 256);
+    const bool vec = aligned16(A) && aligned16(y) && yl % 4 == 0;
+    size_t blocks = ceil_div_sz(xl * yl, vec ? 256 * 16 : 256);
     if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
-    hipLaunchKernelGGL(ger_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, x, xl, y, yl, A, alpha);
+    if (vec) hipLaunchKernelGGL(ger_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, x, xl, y, yl, A, alpha);
+    else hipLaunchKernelGGL(ger_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, x, xl, y, yl, A, alpha);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }
@@ -2194,6 +2449,12 @@ ZG_API int zg_hip_transpose(zg_hip_ctx* ctx, const float* A, float* B, size_t m,
     if (m == 0 || n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(A && B, "transpose: null pointer");
     ZG_REQUIRE(A != B, "transpose: in-place transpose is not supported");
+    if (aligned16(A) && aligned16(B) && m % 4 == 0 && n % 4 == 0 && ceil_div_sz(m, 64) <= 65535) {
+        dim3 grid((unsigned)ceil_div_sz(n, 64), (unsigned)ceil_div_sz(m, 64));
+        hipLaunchKernelGGL(transpose_vec_kernel, grid, dim3(256), 0, ctx->stream, A, B, m, n, alpha);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     dim3 grid((unsigned)ceil_div_sz(n, 32), (unsigned)ceil_div_sz(m, 32));
     ZG_REQUIRE(grid.y <= 65535, "transpose: too many rows");
     hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, ctx->stream, A, B, m, n, alpha);

@@ -1,6 +1,7 @@
 """Scatter ops on skewed index sets: one destination that receives a hundred thousand contributions, buckets on
 both sides of the limits the plan uses (256 entries: a wave instead of a thread adds them; 1024: the bucket is put
-back into input order by a pass over the input instead of all-pairs ranking).  The sums must still equal the host's
+back into input order by a pass over the input instead of all-pairs ranking), through the short build and through
+the radix build (262144 entries and more, or 64 entries and more per destination).  The sums must still equal the host's
 sequential loop bit for bit (src/device/host_device.zig:1039-1087, :1356-1403; src/ndtensor.zig:1437-1513)."""
 from __future__ import annotations
 
@@ -30,6 +31,12 @@ def _skewed_offsets(r, n, n_dst, hubs):
     (400_000, 1000, [(3, 200_000)]),                                   # the same through the radix build (>= 262144 entries)
     (300_000, 50, [(0, 257), (1, 256), (2, 1024), (3, 1025), (49, 100_000)]),
     (270_000, 3, []),
+    # few destinations for the entries (64 and more each on average): the radix build from 512 entries on
+    (600, 3, []), (1000, 1, []), (4097, 17, [(16, 3000)]), (512, 8, []), (511, 7, []),
+    # hubs among many destinations below 262144 entries: the short build with its long buckets
+    (200_000, 4000, [(3, 100_000)]),
+    (60_000, 1000, [(0, 257), (1, 256), (2, 1024), (3, 1025), (999, 20_000)]),
+    (130_000, 100_000, [(99_999, 3000), (7, 1500)]),
 ])
 def test_scatter_add_with_hub_destinations_equals_the_host_loop(oracle, hip, n, n_dst, hubs):
     r = np.random.default_rng(n + n_dst)

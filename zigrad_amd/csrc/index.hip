@@ -51,14 +51,19 @@ static size_t align_up(size_t v, size_t a) {
 // coherent with each other, so device-scope atomics are served by the memory side) and the short build spends two per
 // entry; the radix build spends none but takes ten launches of at least 4 to 5 us each.  Measured, ordering only: one
 // million entries into 100 k buckets 145 us (atomics) against 112 us (radix), eight million into a million about
-// 1100 us against 510 us; at a quarter of a million entries the two take the same time.
+// 1100 us against 510 us; at a quarter of a million entries the two take the same time, and below that the short
+// build is the faster one on keys that do not repeat much (13264 entries into 2708 buckets: 24 us against 47 us).
 constexpr size_t kRadixMinEntries = (size_t)1 << 18;
 constexpr int kRxThreads = 256, kRxPerThread = 16, kRxTile = kRxThreads * kRxPerThread;  // entries per workgroup
 // digit width: 8 bits a pass, or 9 where that saves a pass (17, 18 and 25 to 27 bits of bucket number: two passes instead
 // of three for 65 K to 262 K buckets); the kernels take it as a template argument
 constexpr int kRxMaxBins = 512;
 static bool radix_build_applies(size_t n, size_t nb) {
-    return n >= kRadixMinEntries && nb < ((size_t)1 << 31);
+    // few destinations for many entries (64 and more each on average): the short build's atomics all land on the same
+    // few addresses and its buckets are long to rank (13264 entries into 17 buckets: 217 us against 35 us; into 1000
+    // buckets: 24 us against 48 us)
+    const bool crowded = n >= 512 && n / 64 >= nb;
+    return (n >= kRadixMinEntries || crowded) && nb < ((size_t)1 << 31);
 }
 
 static size_t plan_bytes(size_t n, size_t nb) {
@@ -239,23 +244,37 @@ __global__ void place_kernel(const uint64_t* keys, size_t n, size_t nb, const ui
 }
 
 // Put each bucket back into ascending input position: rank of an entry = number of smaller entries
-// in its bucket.  One wave per bucket.
+// in its bucket.  One wave per bucket; the bucket's positions are first copied to LDS, from where every lane reads
+// them four at a time (all lanes the same address), so that a bucket of a thousand entries costs a thousand LDS reads
+// per lane and not a thousand trips to the L1 each (1000 entries in one bucket: 1.2 ms that way).
 // With `peer_tmp` the payload is laid out in the same order, so that the apply kernels read it next to perm.
 // Buckets of more than kLongBucket entries are listed in `long_list`; those of more than kRankMax entries are left
-// to order_long_segments_kernel (ranking them here would cost len^2 loads in one wave).
+// to order_long_segments_kernel.
 __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
                                                               uint32_t* perm, const uint32_t* peer_tmp, uint32_t* peer,
                                                               uint32_t* long_list) {
-    const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (b >= nb) return;
-    const int lane = threadIdx.x & 63;
-    const uint32_t s = row_ptr[b], len = row_ptr[b + 1] - s;
-    if (len > kLongBucket && lane == 0) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)b;
-    if (len > kRankMax) return;
+    __shared__ __align__(16) uint32_t ids[4][kRankMax];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t b = (size_t)blockIdx.x * 4 + wave;
+    uint32_t s = 0, len = 0;
+    if (b < nb) {
+        s = row_ptr[b];
+        len = row_ptr[b + 1] - s;
+        if (len > kLongBucket && lane == 0) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)b;
+    }
+    const bool here = b < nb && len <= kRankMax;
+    const uint32_t len4 = (len + 3) & ~3u;
+    if (here)
+        for (uint32_t i = lane; i < len4; i += 64) ids[wave][i] = i < len ? perm_tmp[s + i] : 0xffffffffu;  // no position is above the padding
+    __syncthreads();
+    if (!here) return;
     for (uint32_t i = lane; i < len; i += 64) {
-        const uint32_t id = perm_tmp[s + i];
+        const uint32_t id = ids[wave][i];
         uint32_t rank = 0;
-        for (uint32_t j = 0; j < len; j++) rank += (perm_tmp[s + j] < id) ? 1u : 0u;
+        for (uint32_t j = 0; j < len4; j += 4) {
+            const uint4 q = *reinterpret_cast<const uint4*>(&ids[wave][j]);
+            rank += (q.x < id ? 1u : 0u) + (q.y < id ? 1u : 0u) + (q.z < id ? 1u : 0u) + (q.w < id ? 1u : 0u);
+        }
         perm[s + rank] = id;
         if (peer_tmp) peer[s + rank] = peer_tmp[s + i];
     }
@@ -920,7 +939,8 @@ static bool plan_from_cache(zg_hip_ctx* ctx, const uint64_t* keys, const uint64_
                             PlanRef* out, int* rc) {
     *rc = ZG_HIP_OK;
     if (n == 0) return false;
-    if (radix_build_applies(n, nb) && n <= kValidatedMaxEntries) return plan_validated(ctx, keys, payload, n, nb, out, rc);
+    if (radix_build_applies(n, nb) && n >= kRadixMinEntries && n <= kValidatedMaxEntries)
+        return plan_validated(ctx, keys, payload, n, nb, out, rc);
     if (n > kPlanCacheMaxEntries) return false;
     const size_t bytes = n * sizeof(uint64_t);
     if (!in_pinned_host(ctx, keys, bytes) || (payload && !in_pinned_host(ctx, payload, bytes))) return false;
@@ -1105,10 +1125,12 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
 }
 
 // The long buckets: one wave per destination.  The wave loads 64 contributions at a time (the loads do not depend
-// on the running sum), then adds them one after the other in input order, every lane forming the same sum.
+// on the running sum, and the next 64 are in flight meanwhile), then adds them one after the other in input order, every
+// lane forming the same sum.
 __global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float* src, const uint32_t* row_ptr,
                                                                       const uint32_t* perm, const uint32_t* long_list,
                                                                       float* dst, bool fresh, float src_const) {
+    __shared__ __align__(16) float vals[4][2][64];
     const int lane = threadIdx.x & 63;
     const uint32_t n_long = long_list[0];
     const uint32_t wave0 = blockIdx.x * 4 + (threadIdx.x >> 6), n_waves = gridDim.x * 4;
@@ -1116,11 +1138,28 @@ __global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float
         const uint32_t b = long_list[1 + li];
         const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
         float acc = fresh ? 0.f : dst[b];
+        auto fetch = [&](uint32_t k) { return (k < e) ? (src ? src[perm[k]] : src_const) : 0.f; };
+        float v = fetch(s + lane);
         for (uint32_t k0 = s; k0 < e; k0 += 64) {
-            const uint32_t k = k0 + lane;
-            const float v = (k < e) ? (src ? src[perm[k]] : src_const) : 0.f;
+            const float v_next = fetch(k0 + 64 + lane);  // in flight under the 64 additions (two memory round trips)
             const int cnt = (e - k0 < 64u) ? (int)(e - k0) : 64;
-            for (int j = 0; j < cnt; j++) acc = __fadd_rn(acc, __shfl(v, j, 64));
+            // the 64 values go through LDS: every lane reads them back four at a time (all lanes the same address, a
+            // broadcast) and adds them in order, so that the chain of additions is all that is serial (a shuffle per value
+            // costs 45 ns an entry, a scalar lane read 12 ns, this 4 ns).  LDS serves a wave's accesses in order, and the
+            // two halves of `vals` alternate, so the wave needs no barrier with itself.
+            float* slot = vals[threadIdx.x >> 6][(k0 - s) / 64 & 1];
+            slot[lane] = v;
+            __builtin_amdgcn_wave_barrier();
+            if (cnt == 64) {
+#pragma unroll
+                for (int j = 0; j < 64; j += 4) {
+                    const float4 q = *reinterpret_cast<const float4*>(slot + j);
+                    acc = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(acc, q.x), q.y), q.z), q.w);
+                }
+            } else {
+                for (int j = 0; j < cnt; j++) acc = __fadd_rn(acc, slot[j]);
+            }
+            v = v_next;
         }
         if (lane == 0) dst[b] = acc;
     }

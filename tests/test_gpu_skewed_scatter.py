@@ -98,6 +98,23 @@ def test_index_select_bwd_and_gcn_with_a_hub_equal_the_host_loops(oracle, hip):
     np.testing.assert_array_equal(got["grad_deg"], want["grad_deg"])
 
 
+@pytest.mark.parametrize("rows,stride,n_idx,hubs", [
+    (64, 1, 40_000, [(2, 25_000)]), (300, 16, 20_000, [(7, 257), (8, 256), (299, 9000)]), (5000, 70, 9_000, [(0, 3000)]),
+    (30, 300, 9_000, []), (100_000, 3, 300_000, [(5, 100_000), (99_999, 300)]),
+])
+def test_index_select_bwd_of_rows_selected_many_times(oracle, hip, rows, stride, n_idx, hubs):
+    """Rows that more than 256 entries select are added up by a wave per column (the entries' loads in flight 64 at a
+    time), the others by a thread group per row; through the short and the radix build.  Bit for bit the host's loop
+    (src/ndtensor.zig:1461-1465)."""
+    r = np.random.default_rng(rows + stride + n_idx)
+    indices = _skewed_offsets(r, n_idx, rows, hubs)
+    p = {"y_grad": r.standard_normal(n_idx * stride).astype(np.float32), "indices": indices, "stride": stride,
+         "x_grad": r.standard_normal(rows * stride).astype(np.float32)}
+    want = run_op(oracle, "index_select_bwd", {**p, "x_grad": p["x_grad"].copy()}, ["x_grad"])["x_grad"]
+    got = run_op(hip, "index_select_bwd", {**p, "x_grad": p["x_grad"].copy()}, ["x_grad"])["x_grad"]
+    np.testing.assert_array_equal(got, want)
+
+
 @pytest.mark.parametrize("n", [262143, 262144, 262145, 266241, 300000])
 @pytest.mark.parametrize("n_dst", [1, 255, 256, 257, 511, 512, 65535, 65536, 262143, 262144, 1 << 20])
 def test_scatter_add_either_side_of_the_radix_build_limits(oracle, hip, n, n_dst):

@@ -98,6 +98,9 @@ struct zg_waiting_scatter {
     const float* deg = nullptr;
     const uint32_t* row_ptr = nullptr;
     const uint32_t* peer = nullptr;
+    const uint32_t* long_list = nullptr;  // the ordering's buckets of many entries, which a second kernel adds up
+    size_t n_entries = 0;
+    long n_long = -1;
     size_t n_nodes = 0, stride = 0;
     bool fresh = false;           // written, not added to (the output's zero fill was taken over)
     const float* bias = nullptr;  // attached by a following row-broadcast add onto dst
@@ -122,6 +125,7 @@ struct zg_waiting_graddeg {
     // by_incidence: terms in bucket order
     const uint32_t* slot_of = nullptr;
     const uint32_t* inc_row_ptr = nullptr;
+    const uint32_t* inc_long_list = nullptr;  // the nodes of more than 256 terms, which a second kernel adds up
     // otherwise: two term arrays and the two orderings
     float* term_src = nullptr;
     float* term_tgt = nullptr;
@@ -129,6 +133,11 @@ struct zg_waiting_graddeg {
     const uint32_t* perm_src = nullptr;
     const uint32_t* rp_tgt = nullptr;
     const uint32_t* perm_tgt = nullptr;
+    // room for the terms of every node laid out in the order they are added (null: the node's two lists are merged as
+    // they are read), the row pointers of that layout and the list of nodes with many terms
+    float* merged = nullptr;
+    uint32_t* rp_merged = nullptr;
+    uint32_t* long_merged = nullptr;
 };
 
 // Small elementwise ops of one length that have been asked for and not launched yet (elementwise.hip): the reference's

@@ -1107,7 +1107,7 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
         if (fresh) dst[b] = 0.f;
         return;
     }
-    if (e - s > kLongBucket) return;  // scatter_add_apply_long_kernel's
+    if (e - s > kLongBucket) return;  // long_bucket_kernel's
     float acc = fresh ? 0.f : dst[b];
     // eight entries' loads at a time (positions, then values: two round trips), the additions still in input order
     for (uint32_t k = s; k < e; k += 8) {
@@ -1124,14 +1124,56 @@ __global__ void scatter_add_apply_kernel(const float* src, const uint32_t* row_p
     dst[b] = acc;
 }
 
-// The long buckets: one wave per destination.  The wave loads 64 contributions at a time (the loads do not depend
-// on the running sum, and the next 64 are in flight meanwhile), then adds them one after the other in input order, every
-// lane forming the same sum.
-// With rows of `stride` elements (index_select backward) a wave takes one column of one long destination row.
-__global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float* src, const uint32_t* row_ptr,
-                                                                      const uint32_t* perm, const uint32_t* long_list,
-                                                                      float* dst, bool fresh, float src_const,
-                                                                      size_t stride) {
+// The long buckets: one wave per destination element (a destination row of `stride` elements: a wave per column).  The
+// wave loads 64 contributions at a time (the loads do not depend on the running sum, and the next 64 are in flight
+// meanwhile), then adds them one after the other in input order, every lane forming the same sum.  The 64 values go
+// through LDS: every lane reads them back four at a time (all lanes the same address, a broadcast), so that the chain of
+// additions is all that is serial (a shuffle per value costs 45 ns an entry, a scalar lane read 12 ns, this 10 ns).  LDS
+// serves a wave's accesses in order, and the two halves of `vals` alternate, so the wave needs no barrier with itself.
+// F::value(k, b, col, stride, ok) is entry k's contribution to column col of destination b; ok false: the entry is
+// skipped (an edge whose other endpoint is no node).  Optional tail of a graph-convolution layer as in
+// gcn_fwd_apply_kernel: + bias[col], then max(., 0).
+struct LongScatterAdd {
+    const float* src;  // null: every contribution is src_const
+    const uint32_t* perm;
+    float src_const;
+    __device__ __forceinline__ float value(uint32_t k, uint32_t, size_t col, size_t stride, bool& ok) const {
+        ok = true;
+        return src ? src[(size_t)perm[k] * stride + col] : src_const;
+    }
+};
+struct LongGcnFwd {  // (deg[s] * deg[t]) * h[s, col] over the edges into t = b
+    const float* h;
+    const float* deg;
+    const uint32_t* peer;
+    size_t n_nodes;
+    __device__ __forceinline__ float value(uint32_t k, uint32_t b, size_t col, size_t stride, bool& ok) const {
+        const uint32_t sv = peer[k];
+        ok = sv < n_nodes;
+        return ok ? __fmul_rn(__fmul_rn(deg[sv], deg[b]), h[(size_t)sv * stride + col]) : 0.f;
+    }
+};
+struct LongTerms {  // the degree-gradient terms of a node, laid out in the order they are added
+    const float* terms;
+    __device__ __forceinline__ float value(uint32_t k, uint32_t, size_t, size_t, bool& ok) const {
+        ok = true;
+        return terms[k];
+    }
+};
+struct LongGcnGradH {  // (go[t, col] * deg[s]) * deg[t] over the edges out of s = b
+    const float* go;
+    const float* deg;
+    const uint32_t* peer;
+    size_t n_nodes;
+    __device__ __forceinline__ float value(uint32_t k, uint32_t b, size_t col, size_t stride, bool& ok) const {
+        const uint32_t tv = peer[k];
+        ok = tv < n_nodes;
+        return ok ? __fmul_rn(__fmul_rn(go[(size_t)tv * stride + col], deg[b]), deg[tv]) : 0.f;
+    }
+};
+template <class F>
+__global__ __launch_bounds__(256) void long_bucket_kernel(F f, const uint32_t* row_ptr, const uint32_t* long_list, float* dst,
+                                                           bool fresh, size_t stride, const float* bias, bool relu) {
     __shared__ __align__(16) float vals[4][2][64];
     const int lane = threadIdx.x & 63;
     const size_t n_jobs = (size_t)long_list[0] * stride;
@@ -1142,31 +1184,50 @@ __global__ __launch_bounds__(256) void scatter_add_apply_long_kernel(const float
         const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
         float* out = dst + (size_t)b * stride + col;
         float acc = fresh ? 0.f : out[0];
-        auto fetch = [&](uint32_t k) { return (k < e) ? (src ? src[(size_t)perm[k] * stride + col] : src_const) : 0.f; };
-        float v = fetch(s + lane);
+        auto fetch = [&](uint32_t k, bool& ok) {
+            ok = false;
+            return (k < e) ? f.value(k, b, col, stride, ok) : 0.f;
+        };
+        bool ok;
+        float v = fetch(s + lane, ok);
         for (uint32_t k0 = s; k0 < e; k0 += 64) {
-            const float v_next = fetch(k0 + 64 + lane);  // in flight under the 64 additions (two memory round trips)
-            const int cnt = (e - k0 < 64u) ? (int)(e - k0) : 64;
-            // the 64 values go through LDS: every lane reads them back four at a time (all lanes the same address, a
-            // broadcast) and adds them in order, so that the chain of additions is all that is serial (a shuffle per value
-            // costs 45 ns an entry, a scalar lane read 12 ns, this 4 ns).  LDS serves a wave's accesses in order, and the
-            // two halves of `vals` alternate, so the wave needs no barrier with itself.
+            bool ok_next;
+            const float v_next = fetch(k0 + 64 + lane, ok_next);
+            const unsigned long long mask = __ballot(ok);
             float* slot = vals[threadIdx.x >> 6][(k0 - s) / 64 & 1];
             slot[lane] = v;
             __builtin_amdgcn_wave_barrier();
-            if (cnt == 64) {
+            if (mask == ~0ull) {
 #pragma unroll
                 for (int j = 0; j < 64; j += 4) {
                     const float4 q = *reinterpret_cast<const float4*>(slot + j);
                     acc = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(acc, q.x), q.y), q.z), q.w);
                 }
             } else {
-                for (int j = 0; j < cnt; j++) acc = __fadd_rn(acc, slot[j]);
+                for (int j = 0; j < 64; j++)
+                    if ((mask >> j) & 1ull) acc = __fadd_rn(acc, slot[j]);
             }
             v = v_next;
+            ok = ok_next;
         }
+        if (bias) acc = __fadd_rn(acc, bias[col]);
+        if (relu) acc = acc > 0.f ? acc : 0.f;
         if (lane == 0) out[0] = acc;
     }
+}
+
+// Launches long_bucket_kernel over the long buckets of `pl` (n_long: the host's count of them, -1 unknown).
+template <class F>
+static int launch_long_buckets(zg_hip_ctx* ctx, const F& f, const uint32_t* row_ptr, const uint32_t* long_list, size_t n_entries,
+                               long n_long, float* dst, bool fresh, size_t stride, const float* bias = nullptr,
+                               bool relu = false) {
+    if (n_entries <= kLongBucket || n_long == 0) return ZG_HIP_OK;
+    size_t grid = ceil_div_sz((n_entries / kLongBucket) * stride, 4);
+    if (grid > 2048) grid = 2048;
+    hipLaunchKernelGGL((long_bucket_kernel<F>), dim3((unsigned)grid), dim3(256), 0, ctx->stream, f, row_ptr, long_list, dst,
+                       fresh, stride, bias, relu);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
 }
 
 static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Plan& pl, float* dst, bool fresh,
@@ -1174,14 +1235,7 @@ static int launch_scatter_add_apply(zg_hip_ctx* ctx, const float* src, const Pla
     hipLaunchKernelGGL(scatter_add_apply_kernel, dim3((unsigned)ceil_div_sz(pl.nb, 256)), dim3(256), 0, ctx->stream, src,
                        pl.row_ptr, pl.perm, dst, pl.nb, fresh, src_const);
     ZG_LAUNCH_CHECK();
-    if (pl.n > kLongBucket && pl.n_long != 0) {
-        size_t grid = ceil_div_sz(pl.n / kLongBucket, 4);
-        if (grid > 2048) grid = 2048;
-        hipLaunchKernelGGL(scatter_add_apply_long_kernel, dim3((unsigned)grid), dim3(256), 0, ctx->stream, src, pl.row_ptr,
-                           pl.perm, pl.long_list, dst, fresh, src_const, (size_t)1);
-        ZG_LAUNCH_CHECK();
-    }
-    return ZG_HIP_OK;
+    return launch_long_buckets(ctx, LongScatterAdd{src, pl.perm, src_const}, pl.row_ptr, pl.long_list, pl.n, pl.n_long, dst, fresh, 1);
 }
 
 // The whole of scatter_add for at most kScatterSmallMax entries in one launch of one workgroup: thread i owns entry i,
@@ -1238,7 +1292,7 @@ __global__ __launch_bounds__(256) void row_scatter_apply_kernel(const float* src
     const int lane = threadIdx.x % G;
     const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
     if (s == e) return;
-    if (e - s > kLongBucket) return;  // scatter_add_apply_long_kernel's, a wave per column
+    if (e - s > kLongBucket) return;  // long_bucket_kernel's, a wave per column
     for (size_t j = lane; j < stride; j += G) {
         float acc = dst[b * stride + j];
         // eight entries' loads at a time (positions, then row elements: two round trips), the additions still in input
@@ -1272,6 +1326,7 @@ __global__ __launch_bounds__(256) void gcn_fwd_apply_kernel(float* dst, const fl
     const int lane = threadIdx.x % G;
     const uint32_t s0 = row_ptr[t], s1 = row_ptr[t + 1];
     if (s0 == s1 && !fresh && !bias && !relu) return;
+    if (s1 - s0 > kLongBucket) return;  // long_bucket_kernel's, a wave per column
     const float dt = deg[t];
     for (size_t j = lane; j < stride; j += G) {
         float acc = fresh ? 0.f : dst[t * stride + j];
@@ -1310,6 +1365,7 @@ __global__ __launch_bounds__(256) void gcn_bwd_gradh_kernel(float* grad_h, const
             for (size_t j = lane; j < stride; j += G) grad_h[s * stride + j] = 0.f;
         return;
     }
+    if (s1 - s0 > kLongBucket) return;  // long_bucket_kernel's, a wave per column
     const float ds = deg[s];
     for (size_t j = lane; j < stride; j += G) {
         float acc = fresh ? 0.f : grad_h[s * stride + j];
@@ -1332,11 +1388,66 @@ __global__ __launch_bounds__(256) void gcn_bwd_gradh_kernel(float* grad_h, const
     }
 }
 
-// per-edge degree-gradient terms, each summed over the feature dim in index order (one thread per edge)
+// The two degree-gradient terms of an edge, each summed over the feature dimension in index order, for rows of more than
+// 16 features: a thread per edge, but the rows reach it through LDS.  A wave copies 32 columns of the two rows of each of
+// its 64 edges into LDS with loads that follow the rows (32 lanes on the 128 contiguous bytes of a row, two edges per
+// instruction), then every lane walks its own edge's 32 values in order; left to itself a lane reads its rows value by
+// value and every load instruction of the wave touches 64 different rows (a million edges of 64 features: 1766 us that
+// way, 12 times what the bytes take).  Called by every thread of a workgroup of kEtThreads.
+constexpr int kEtThreads = 128, kEtCols = 32;
+constexpr size_t kEtStagedMinStride = 16;  // rows of up to 64 bytes are one cache line either way
+__device__ __forceinline__ void edge_terms_staged(const float* go, const float* h, const float* deg, uint64_t s, uint64_t t,
+                                                  bool valid, size_t stride, float& gs, float& gt) {
+    __shared__ float tg[kEtThreads / 64][64][kEtCols + 1], th[kEtThreads / 64][64][kEtCols + 1];
+    __shared__ uint32_t ss[kEtThreads / 64][64], ts[kEtThreads / 64][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    ss[w][lane] = valid ? (uint32_t)s : 0xffffffffu;
+    ts[w][lane] = valid ? (uint32_t)t : 0xffffffffu;
+    const float ds = valid ? deg[s] : 0.f, dt = valid ? deg[t] : 0.f;
+    gs = 0.f;
+    gt = 0.f;
+    const int col = lane & 31;
+    for (size_t c0 = 0; c0 < stride; c0 += kEtCols) {
+        __syncthreads();  // the node numbers are in place, and the last chunk has been used up
+        const size_t c = c0 + col;
+#pragma unroll 8
+        for (int it = 0; it < 32; it++) {
+            const int ed = it * 2 + (lane >> 5);
+            const uint32_t se = ss[w][ed], te = ts[w][ed];
+            const bool ok = se != 0xffffffffu && c < stride;
+            tg[w][ed][col] = ok ? go[(size_t)te * stride + c] : 0.f;
+            th[w][ed][col] = ok ? h[(size_t)se * stride + c] : 0.f;
+        }
+        __syncthreads();
+        if (valid) {
+            const int lim = stride - c0 < (size_t)kEtCols ? (int)(stride - c0) : kEtCols;
+            for (int j = 0; j < lim; j++) {
+                const float g = tg[w][lane][j], hv = th[w][lane][j];
+                gs = __fadd_rn(gs, __fmul_rn(__fmul_rn(g, dt), hv));
+                gt = __fadd_rn(gt, __fmul_rn(__fmul_rn(g, ds), hv));
+            }
+        }
+    }
+}
+
+// STAGED: the workgroup is kEtThreads wide and the rows go through LDS (edge_terms_staged)
+template <bool STAGED>
 __global__ void gcn_bwd_edge_terms_kernel(const float* go, const float* h, const float* deg, const uint64_t* src_idx,
                                           const uint64_t* tgt_idx, size_t n_edge, size_t n_nodes, size_t stride,
-                                          float* term_src, float* term_tgt) {
+                                          float* term_src, float* term_tgt, uint32_t* zero_me) {
     size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (zero_me && e == 0) zero_me[0] = 0;  // the counter of a list that a later kernel appends to
+    if (STAGED) {
+        const bool in = e < n_edge;
+        const uint64_t s = in ? src_idx[e] : 0, t = in ? tgt_idx[e] : 0;
+        float gs, gt;
+        edge_terms_staged(go, h, deg, s, t, in && s < n_nodes && t < n_nodes, stride, gs, gt);
+        if (in) {
+            term_src[e] = gs;
+            term_tgt[e] = gt;
+        }
+        return;
+    }
     if (e >= n_edge) return;
     const uint64_t s = src_idx[e], t = tgt_idx[e];
     float gs = 0.f, gt = 0.f;
@@ -1398,11 +1509,24 @@ __global__ void invert_perm_kernel(const uint32_t* row_ptr, size_t nb, const uin
     if (k < row_ptr[nb]) slot_of[perm[k]] = (uint32_t)k;
 }
 
+template <bool STAGED>
 __global__ void gcn_bwd_edge_terms_slots_kernel(const float* go, const float* h, const float* deg,
                                                 const uint64_t* src_idx, const uint64_t* tgt_idx, size_t n_edge,
                                                 size_t n_nodes, size_t stride, const uint32_t* slot_of, float* terms,
                                                 bool vec4) {
     size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (STAGED) {
+        const bool in = e < n_edge;
+        const uint64_t s = in ? src_idx[e] : 0, t = in ? tgt_idx[e] : 0;
+        float gs, gt;
+        edge_terms_staged(go, h, deg, s, t, in && s < n_nodes && t < n_nodes, stride, gs, gt);
+        if (in) {
+            const uint32_t slot_s = slot_of[2 * e], slot_t = slot_of[2 * e + 1];
+            if (slot_s != 0xffffffffu) terms[slot_s] = gs;
+            if (slot_t != 0xffffffffu) terms[slot_t] = gt;
+        }
+        return;
+    }
     if (e >= n_edge) return;
     const uint64_t s = src_idx[e], t = tgt_idx[e];
     const uint32_t slot_s = slot_of[2 * e], slot_t = slot_of[2 * e + 1];
@@ -1443,6 +1567,55 @@ __global__ void gcn_bwd_edge_terms_slots_kernel(const float* go, const float* h,
     if (slot_t != 0xffffffffu) terms[slot_t] = gt;
 }
 
+// The degree gradient of a node is the sum of its edges' terms in edge order, the source term of an edge before its target
+// term; a node's edges are in two lists (by source, by target), each in edge order.  Instead of merging the two lists
+// while adding (a node of a hundred thousand edges: one dependent load after the other, 140 ns a term), every term is
+// first put where it belongs in the merged order, which it can find on its own: entry i of the node's source list goes
+// behind the i source terms before it and the target terms of earlier edges (a binary search of the target list), entry
+// j of the target list behind j target terms and the source terms of edges up to its own.  The merged lists of all nodes
+// lie one after the other, node v's at rp_src[v] + rp_tgt[v]; then the terms are contiguous per node and are added by
+// gcn_bwd_graddeg_slots_kernel, or by long_bucket_kernel for a node of many terms.
+__global__ void graddeg_rows_kernel(const uint32_t* rp_src, const uint32_t* rp_tgt, size_t n_nodes, uint32_t* rp_merged,
+                                    uint32_t* long_list) {
+    const size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v > n_nodes) return;
+    const uint32_t at = rp_src[v] + rp_tgt[v];
+    rp_merged[v] = at;
+    if (v < n_nodes && rp_src[v + 1] + rp_tgt[v + 1] - at > kLongBucket) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)v;
+}
+
+__global__ void graddeg_place_kernel(const uint64_t* src_idx, const uint64_t* tgt_idx, const float* term_src,
+                                     const float* term_tgt, const uint32_t* rp_src, const uint32_t* perm_src,
+                                     const uint32_t* rp_tgt, const uint32_t* perm_tgt, size_t n_nodes, size_t n_edge,
+                                     float* merged) {
+    const size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= n_edge) return;
+    if (k < rp_src[n_nodes]) {  // entry k of the by-source ordering
+        const uint32_t e = perm_src[k];
+        const size_t v = (size_t)src_idx[e];
+        const uint32_t* other = perm_tgt + rp_tgt[v];
+        uint32_t lo = 0, hi = rp_tgt[v + 1] - rp_tgt[v];  // target terms of edges before e
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (other[mid] < e) lo = mid + 1;
+            else hi = mid;
+        }
+        merged[(size_t)rp_tgt[v] + k + lo] = term_src[e];
+    }
+    if (k < rp_tgt[n_nodes]) {  // entry k of the by-target ordering
+        const uint32_t e = perm_tgt[k];
+        const size_t v = (size_t)tgt_idx[e];
+        const uint32_t* other = perm_src + rp_src[v];
+        uint32_t lo = 0, hi = rp_src[v + 1] - rp_src[v];  // source terms of edges up to e
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (other[mid] <= e) lo = mid + 1;
+            else hi = mid;
+        }
+        merged[(size_t)rp_src[v] + k + lo] = term_tgt[e];
+    }
+}
+
 __global__ void gcn_bwd_graddeg_slots_kernel(float* grad_deg, const float* terms, const uint32_t* row_ptr,
                                              size_t n_nodes, bool fresh) {
     size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1452,6 +1625,7 @@ __global__ void gcn_bwd_graddeg_slots_kernel(float* grad_deg, const float* terms
         if (fresh) grad_deg[v] = 0.f;
         return;
     }
+    if (e - s > kLongBucket) return;  // long_bucket_kernel's
     float acc = fresh ? 0.f : grad_deg[v];
     for (uint32_t k = s; k < e; k += 8) {
         float tv[8];
@@ -1732,16 +1906,10 @@ ZG_API int zg_hip_index_select_bwd(zg_hip_ctx* ctx, const float* y_grad, const u
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((row_scatter_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, y_grad,
                                         pl.row_ptr, pl.perm, x_grad, nb, stride));
     ZG_LAUNCH_CHECK();
-    if (pl.n > kLongBucket && pl.n_long != 0) {
-        // rows that more than kLongBucket entries select: a wave per column, 64 entries' loads in flight (a row selected
-        // ten thousand times: 4.6 ms a thread group walking its entries one by one, 0.2 ms this way)
-        size_t long_grid = ceil_div_sz((pl.n / kLongBucket) * stride, 4);
-        if (long_grid > 2048) long_grid = 2048;
-        hipLaunchKernelGGL(scatter_add_apply_long_kernel, dim3((unsigned)long_grid), dim3(256), 0, ctx->stream, y_grad,
-                           pl.row_ptr, pl.perm, pl.long_list, x_grad, false, 0.f, stride);
-        ZG_LAUNCH_CHECK();
-    }
-    return ZG_HIP_OK;
+    // rows that more than kLongBucket entries select: a wave per column, 64 entries' loads in flight (a row selected
+    // ten thousand times: 4.6 ms a thread group walking its entries one by one, 0.2 ms this way)
+    return launch_long_buckets(ctx, LongScatterAdd{y_grad, pl.perm, 0.f}, pl.row_ptr, pl.long_list, pl.n, pl.n_long, x_grad, false,
+                               stride);
 }
 
 namespace zg {
@@ -1774,7 +1942,32 @@ int flush_scatter(zg_hip_ctx* ctx) {
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_fwd_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, w.dst, w.h, w.deg,
                                         w.row_ptr, w.peer, w.n_nodes, w.stride, w.fresh, w.bias, w.relu != 0));
     ZG_LAUNCH_CHECK();
-    return ZG_HIP_OK;
+    return launch_long_buckets(ctx, LongGcnFwd{w.h, w.deg, w.peer, w.n_nodes}, w.row_ptr, w.long_list, w.n_entries, w.n_long,
+                               w.dst, w.fresh, w.stride, w.bias, w.relu != 0);
+}
+
+// The sums of the degree-gradient terms through the merged layout (see graddeg_rows_kernel); `long_list[0]` is zero.
+static int launch_graddeg_merged(zg_hip_ctx* ctx, const uint64_t* src_idx, const uint64_t* tgt_idx, const float* term_src,
+                                 const float* term_tgt, const uint32_t* rp_src, const uint32_t* perm_src,
+                                 const uint32_t* rp_tgt, const uint32_t* perm_tgt, size_t n_nodes, size_t n_edge, float* merged,
+                                 uint32_t* rp_merged, uint32_t* long_list, float* grad_deg, bool fresh) {
+    hipLaunchKernelGGL(graddeg_rows_kernel, dim3((unsigned)ceil_div_sz(n_nodes + 1, 256)), dim3(256), 0, ctx->stream, rp_src,
+                       rp_tgt, n_nodes, rp_merged, long_list);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(graddeg_place_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream, src_idx,
+                       tgt_idx, term_src, term_tgt, rp_src, perm_src, rp_tgt, perm_tgt, n_nodes, n_edge, merged);
+    ZG_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
+                       grad_deg, merged, rp_merged, n_nodes, fresh);
+    ZG_LAUNCH_CHECK();
+    return launch_long_buckets(ctx, LongTerms{merged}, rp_merged, long_list, 2 * n_edge, -1, grad_deg, fresh, 1);
+}
+
+// Room behind the two term arrays for the merged layout: 2 * n_edge terms, n_nodes + 1 row pointers, the list of long nodes.
+static size_t graddeg_merged_bytes(size_t n_edge, size_t n_nodes) {
+    if (2 * n_edge >= 0xffffffffull) return 0;  // positions would not fit 32 bits: the lists are merged as they are read
+    return align_up(2 * n_edge * sizeof(float), 256) + align_up((n_nodes + 1) * sizeof(uint32_t), 256) +
+           align_up((2 * n_edge / kLongBucket + 2) * sizeof(uint32_t), 256);
 }
 
 int flush_graddeg(zg_hip_ctx* ctx) {
@@ -1784,19 +1977,32 @@ int flush_graddeg(zg_hip_ctx* ctx) {
     if (w.by_incidence) {
         // 2 * n_edge terms in bucket order; the two separate term arrays' room holds them
         float* terms = w.term_src;
-        hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel, dim3((unsigned)ceil_div_sz(w.n_edge, 256)), dim3(256), 0,
-                           ctx->stream, w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride,
-                           w.slot_of, terms, w.stride % 4 == 0 && aligned16(w.grad_output) && aligned16(w.h));
+        if (w.stride > kEtStagedMinStride)
+            hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel<true>, dim3((unsigned)ceil_div_sz(w.n_edge, kEtThreads)),
+                               dim3(kEtThreads), 0, ctx->stream, w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge,
+                               w.n_nodes, w.stride, w.slot_of, terms, false);
+        else
+            hipLaunchKernelGGL(gcn_bwd_edge_terms_slots_kernel<false>, dim3((unsigned)ceil_div_sz(w.n_edge, 256)), dim3(256), 0,
+                               ctx->stream, w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride,
+                               w.slot_of, terms, w.stride % 4 == 0 && aligned16(w.grad_output) && aligned16(w.h));
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(gcn_bwd_graddeg_slots_kernel, dim3((unsigned)ceil_div_sz(w.n_nodes, 256)), dim3(256), 0,
                            ctx->stream, w.grad_deg, terms, w.inc_row_ptr, w.n_nodes, w.fresh);
         ZG_LAUNCH_CHECK();
-        return ZG_HIP_OK;
+        return launch_long_buckets(ctx, LongTerms{terms}, w.inc_row_ptr, w.inc_long_list, 2 * w.n_edge, -1, w.grad_deg, w.fresh, 1);
     }
-    hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(w.n_edge, 256)), dim3(256), 0, ctx->stream,
-                       w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride, w.term_src,
-                       w.term_tgt);
+    if (w.stride > kEtStagedMinStride)
+        hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel<true>, dim3((unsigned)ceil_div_sz(w.n_edge, kEtThreads)), dim3(kEtThreads),
+                           0, ctx->stream, w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride,
+                           w.term_src, w.term_tgt, w.long_merged);
+    else
+        hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel<false>, dim3((unsigned)ceil_div_sz(w.n_edge, 256)), dim3(256), 0,
+                           ctx->stream, w.grad_output, w.h, w.deg, w.src_idx, w.tgt_idx, w.n_edge, w.n_nodes, w.stride,
+                           w.term_src, w.term_tgt, w.long_merged);
     ZG_LAUNCH_CHECK();
+    if (w.merged)
+        return launch_graddeg_merged(ctx, w.src_idx, w.tgt_idx, w.term_src, w.term_tgt, w.rp_src, w.perm_src, w.rp_tgt,
+                                     w.perm_tgt, w.n_nodes, w.n_edge, w.merged, w.rp_merged, w.long_merged, w.grad_deg, w.fresh);
     hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(w.n_nodes, 256)), dim3(256), 0, ctx->stream,
                        w.grad_deg, w.term_src, w.term_tgt, w.rp_src, w.perm_src, w.rp_tgt, w.perm_tgt, w.n_nodes, w.fresh);
     ZG_LAUNCH_CHECK();
@@ -1870,6 +2076,9 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled(zg_hip_ctx* ctx, float* dst, const floa
     w.deg = deg;
     w.row_ptr = pr.plan.row_ptr;
     w.peer = pr.plan.peer;
+    w.long_list = pr.plan.long_list;
+    w.n_entries = pr.plan.n;
+    w.n_long = pr.plan.n_long;
     w.n_nodes = n_nodes;
     w.stride = stride;
     w.fresh = fresh;
@@ -1898,10 +2107,12 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     if (int rc = check_gcn("scatter_gcn_deg_scaled_bwd", stride, n_edge, n_nodes)) return rc;
     const size_t pb = align_up(plan_bytes(n_edge, n_nodes), 256);
     const size_t tb = align_up(n_edge * sizeof(float), 256);
-    char* mem = (char*)workspace(ctx, 2 * pb + 2 * tb);
+    const size_t mb = graddeg_merged_bytes(n_edge, n_nodes);
+    char* mem = (char*)workspace(ctx, 2 * pb + 2 * tb + mb);
     if (!mem) return ZG_HIP_EOOM;
     float* term_src = (float*)(mem + 2 * pb);
     float* term_tgt = (float*)(mem + 2 * pb + tb);
+    char* merged_mem = mb ? mem + 2 * pb + 2 * tb : nullptr;
     PlanRef rs, rt;
     int rc = 0;
     if (!plan_from_cache(ctx, src_indices, tgt_indices, n_edge, n_nodes, &rs, &rc)) {
@@ -1927,6 +2138,9 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
                                         grad_output, deg, by_src.row_ptr, by_src.peer, n_nodes, stride, fresh_h));
     ZG_LAUNCH_CHECK();
+    if (int rc2 = launch_long_buckets(ctx, LongGcnGradH{grad_output, deg, by_src.peer, n_nodes}, by_src.row_ptr, by_src.long_list,
+                                      by_src.n, by_src.n_long, grad_h, fresh_h, stride))
+        return rc2;
     // The degree gradient waits: whatever comes next launches it (its orderings and term arrays live in the cache or in
     // the workspace, which no call touches before it has sent waiting work out), except a free of the block it would
     // write, which drops it.
@@ -1949,11 +2163,18 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd(zg_hip_ctx* ctx, const float* grad_
     if (by_incidence) {
         w.slot_of = rs.entry->slot_of;
         w.inc_row_ptr = rs.entry->inc.row_ptr;
+        w.inc_long_list = rs.entry->inc.long_list;
     } else {
         w.rp_src = by_src.row_ptr;
         w.perm_src = by_src.perm;
         w.rp_tgt = by_tgt.row_ptr;
         w.perm_tgt = by_tgt.perm;
+        if (merged_mem) {
+            w.merged = (float*)merged_mem;
+            w.rp_merged = (uint32_t*)(merged_mem + align_up(2 * n_edge * sizeof(float), 256));
+            w.long_merged = (uint32_t*)(merged_mem + align_up(2 * n_edge * sizeof(float), 256) +
+                                        align_up((n_nodes + 1) * sizeof(uint32_t), 256));
+        }
     }
     return ZG_HIP_OK;
     }();
@@ -2073,6 +2294,19 @@ ZG_API int zg_hip_edge_plan_create(zg_hip_ctx* ctx, const uint64_t* src_indices,
     if (!rc) rc = zg_hip_memcpy_d2d(ctx, pl->tgt_dev, tgt_indices, n_edge * sizeof(uint64_t));
     if (!rc) rc = build_plan(ctx, pl->tgt_dev, pl->by_tgt, pl->src_dev);
     if (!rc) rc = build_plan(ctx, pl->src_dev, pl->by_src, pl->tgt_dev);
+    if (!rc) {
+        // how many nodes have more than kLongBucket edges is read back once: the calls that use the plan skip the launch of
+        // the kernel for such nodes when there is none
+        uint32_t n_long[2] = {0, 0};
+        if (hipMemcpyAsync(&n_long[0], pl->by_tgt.long_list, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream) == hipSuccess &&
+            hipMemcpyAsync(&n_long[1], pl->by_src.long_list, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream) == hipSuccess &&
+            hipStreamSynchronize(ctx->stream) == hipSuccess) {
+            pl->by_tgt.n_long = (long)n_long[0];
+            pl->by_src.n_long = (long)n_long[1];
+        } else {
+            (void)hipGetLastError();  // the counts stay unknown: the kernel is launched and finds the lists empty or not
+        }
+    }
     if (rc) {
         zg_hip_free(ctx, mem);
         delete pl;
@@ -2113,7 +2347,8 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_planned(zg_hip_ctx* ctx, float* dst, co
                                         plan->by_tgt.row_ptr, plan->by_tgt.peer, n_nodes, stride, accumulate == 0, bias,
                                         relu != 0));
     ZG_LAUNCH_CHECK();
-    return ZG_HIP_OK;
+    return launch_long_buckets(ctx, LongGcnFwd{h, deg, plan->by_tgt.peer, n_nodes}, plan->by_tgt.row_ptr, plan->by_tgt.long_list,
+                               plan->by_tgt.n, plan->by_tgt.n_long, dst, accumulate == 0, stride, bias, relu != 0);
 }
 
 ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx* ctx, const float* grad_output, const float* h,
@@ -2125,19 +2360,36 @@ ZG_API int zg_hip_scatter_gcn_deg_scaled_bwd_planned(zg_hip_ctx* ctx, const floa
     ZG_REQUIRE(stride > 0, "scatter_gcn_deg_scaled_bwd_planned: stride is 0");
     const size_t n_nodes = plan->n_nodes, n_edge = plan->n_edge;
     const size_t tb = align_up(n_edge * sizeof(float), 256);
-    char* mem = (char*)workspace(ctx, 2 * tb);
+    const size_t mb = graddeg_merged_bytes(n_edge, n_nodes);
+    char* mem = (char*)workspace(ctx, 2 * tb + mb);
     if (!mem) return ZG_HIP_EOOM;
     float* term_src = (float*)mem;
     float* term_tgt = (float*)(mem + tb);
+    float* merged = mb ? (float*)(mem + 2 * tb) : nullptr;
+    uint32_t* rp_merged = mb ? (uint32_t*)(mem + 2 * tb + align_up(2 * n_edge * sizeof(float), 256)) : nullptr;
+    uint32_t* long_merged = mb ? (uint32_t*)((char*)rp_merged + align_up((n_nodes + 1) * sizeof(uint32_t), 256)) : nullptr;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(n_nodes, 256 / g);
     ZG_G_DISPATCH(g, hipLaunchKernelGGL((gcn_bwd_gradh_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, grad_h,
                                         grad_output, deg, plan->by_src.row_ptr, plan->by_src.peer, n_nodes, stride, fresh));
     ZG_LAUNCH_CHECK();
+    if (int rc = launch_long_buckets(ctx, LongGcnGradH{grad_output, deg, plan->by_src.peer, n_nodes}, plan->by_src.row_ptr,
+                                     plan->by_src.long_list, plan->by_src.n, plan->by_src.n_long, grad_h, fresh, stride))
+        return rc;
     if (!grad_deg) return ZG_HIP_OK;  // the degrees need no gradient (they are data of the graph)
-    hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
-                       grad_output, h, deg, plan->src_dev, plan->tgt_dev, n_edge, n_nodes, stride, term_src, term_tgt);
+    if (stride > kEtStagedMinStride)
+        hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel<true>, dim3((unsigned)ceil_div_sz(n_edge, kEtThreads)), dim3(kEtThreads), 0,
+                           ctx->stream, grad_output, h, deg, plan->src_dev, plan->tgt_dev, n_edge, n_nodes, stride, term_src,
+                           term_tgt, long_merged);
+    else
+        hipLaunchKernelGGL(gcn_bwd_edge_terms_kernel<false>, dim3((unsigned)ceil_div_sz(n_edge, 256)), dim3(256), 0, ctx->stream,
+                           grad_output, h, deg, plan->src_dev, plan->tgt_dev, n_edge, n_nodes, stride, term_src, term_tgt,
+                           long_merged);
     ZG_LAUNCH_CHECK();
+    if (merged)
+        return launch_graddeg_merged(ctx, plan->src_dev, plan->tgt_dev, term_src, term_tgt, plan->by_src.row_ptr,
+                                     plan->by_src.perm, plan->by_tgt.row_ptr, plan->by_tgt.perm, n_nodes, n_edge, merged, rp_merged,
+                                     long_merged, grad_deg, fresh);
     hipLaunchKernelGGL(gcn_bwd_graddeg_kernel, dim3((unsigned)ceil_div_sz(n_nodes, 256)), dim3(256), 0, ctx->stream,
                        grad_deg, term_src, term_tgt, plan->by_src.row_ptr, plan->by_src.perm, plan->by_tgt.row_ptr,
                        plan->by_tgt.perm, n_nodes, fresh);

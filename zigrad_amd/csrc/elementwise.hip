@@ -73,7 +73,10 @@ __global__ __launch_bounds__(kBlock) void map_scalar_kernel(float* out, const fl
 
 static int map_grid(zg_hip_ctx* ctx, size_t items, int per_block) {
     size_t blocks = ceil_div_sz(items, (size_t)per_block);
-    size_t cap = (size_t)ctx->n_cu * 32;
+    // one trip per thread at any size (a capped grid whose threads stride through the array is 2 to 5 % slower beyond
+    // 33 M elements)
+    (void)ctx;
+    size_t cap = 0x7fffffffull;
     if (blocks > cap) blocks = cap;
     return (int)(blocks < 1 ? 1 : blocks);
 }

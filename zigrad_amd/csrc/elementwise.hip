@@ -255,11 +255,9 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
     if (mn % 4 == 0 && aligned16(lng) && aligned16(sht) && aligned16(z)) {
         size_t p4 = mn / 4, rows = mx / mn;
         unsigned gx = (unsigned)ceil_div_sz(p4, kRbX);
-        // enough row groups to fill the machine, each thread then loops over the rest
-        size_t want_blocks = (size_t)ctx->n_cu * 16;
-        size_t gy = ceil_div_sz(want_blocks, gx);
-        size_t max_gy = ceil_div_sz(rows, (size_t)kRbY * kRbRows);
-        if (gy > max_gy) gy = max_gy;
+        // a workgroup per group of rows, up to the grid's limit (65536 rows of 4096: 466 -> 370 us against 16 workgroups
+        // per compute unit whose threads loop over the rest)
+        size_t gy = ceil_div_sz(rows, (size_t)kRbY * kRbRows);
         if (gy < 1) gy = 1;
         if (gy > 65535) gy = 65535;
         dim3 grid(gx, (unsigned)gy), block(kRbX, kRbY);

@@ -1868,7 +1868,9 @@ ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src
         const size_t s4 = stride / 4;
         const int g = group_for(s4);
         size_t vblocks = ceil_div_sz(n_idx, (size_t)(256 / g) * 4);
-        if (vblocks > (size_t)ctx->n_cu * 16) vblocks = (size_t)ctx->n_cu * 16;
+        // a workgroup per 16 to 64 rows at any count (a million rows of 1 KiB: 355 -> 339 us against a grid capped at 16
+        // workgroups per compute unit)
+        if (vblocks > 0x7fffffffull) vblocks = 0x7fffffffull;
         ZG_G_DISPATCH(g, hipLaunchKernelGGL((index_select_fwd_vec4_kernel<G>), dim3((unsigned)vblocks), dim3(256), 0,
                                             ctx->stream, (const float4*)src, src_len / stride, indices, n_idx, s4,
                                             (float4*)dst));
@@ -1876,7 +1878,7 @@ ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src
         return ZG_HIP_OK;
     }
     size_t blocks = ceil_div_sz(total, 256);
-    if (blocks > (size_t)ctx->n_cu * 16) blocks = (size_t)ctx->n_cu * 16;
+    if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
     hipLaunchKernelGGL(index_select_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, src, src_len, indices,
                        n_idx, stride, dst);
     ZG_LAUNCH_CHECK();

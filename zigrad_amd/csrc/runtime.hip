@@ -360,9 +360,12 @@ __global__ void take_kernel(const float* __restrict__ src, const uint64_t* __res
     }
 }
 
-static int grid_for(zg_hip_ctx* ctx, size_t work_items, int block) {
+// capped = 16 workgroups per compute unit, threads looping over the rest: the better choice where a thread moves four
+// bytes per trip (sequence on 134 M elements: 99 us capped, 116 us with a thread per element); kernels whose threads move
+// 8 or 16 bytes per trip take a workgroup per chunk at any size (fill of 134 M 64-bit words: 208 -> 163 us)
+static int grid_for(zg_hip_ctx* ctx, size_t work_items, int block, bool capped = true) {
     size_t blocks = ceil_div_sz(work_items, (size_t)block);
-    size_t cap = (size_t)ctx->n_cu * 16;
+    size_t cap = capped ? (size_t)ctx->n_cu * 16 : 0x7fffffffull;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     return (int)blocks;
@@ -1211,7 +1214,7 @@ ZG_API int zg_hip_memcpy_d2d(zg_hip_ctx* ctx, void* dst, const void* src, size_t
         const bool v16 = aligned16(dst) && aligned16(src) && bytes % 16 == 0;
         const size_t units = v16 ? bytes / 16 : bytes;
         if (v16)
-            hipLaunchKernelGGL(copy_kernel<uint4>, dim3(grid_for(ctx, units, kBlock)), dim3(kBlock), 0, ctx->stream,
+            hipLaunchKernelGGL(copy_kernel<uint4>, dim3(grid_for(ctx, units, kBlock, false)), dim3(kBlock), 0, ctx->stream,
                                (uint4*)dst, (const uint4*)src, units);
         else
             hipLaunchKernelGGL(copy_kernel<uint8_t>, dim3(grid_for(ctx, units, kBlock)), dim3(kBlock), 0, ctx->stream,
@@ -1443,7 +1446,7 @@ ZG_API int zg_hip_mem_fill_u64(zg_hip_ctx* ctx, uint64_t* x, size_t n, uint64_t 
     ZG_CTX(ctx);
     if (n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x != nullptr, "mem_fill_u64: null pointer");
-    hipLaunchKernelGGL(fill_kernel<uint64_t>, dim3(grid_for(ctx, n, kBlock)), dim3(kBlock), 0, ctx->stream, x, n,
+    hipLaunchKernelGGL(fill_kernel<uint64_t>, dim3(grid_for(ctx, n, kBlock, false)), dim3(kBlock), 0, ctx->stream, x, n,
                        value);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;

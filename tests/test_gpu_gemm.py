@@ -230,7 +230,10 @@ def test_bmm_32x512_cubed(oracle, hip):
                                  # every lanes-per-row shape of the row kernel, rows cut into segments, a reduced axis cut
                                  # into many chunks, tiles of the transpose that end inside the matrix
                                  (3, 300000), (7, 20000), (300, 16384), (100000, 8), (5000, 64), (4096, 256), (70000, 12),
-                                 (130, 5000), (64, 64), (256, 1000), (1000, 1024), (68, 132), (1, 70000), (70000, 1)])
+                                 (130, 5000), (64, 64), (256, 1000), (1000, 1024), (68, 132), (1, 70000), (70000, 1),
+                                 # transposes whose tiles are numbered down the diagonals (wide, both sides multiples of 1024)
+                                 # and the tall counterpart that is not
+                                 (1024, 1024), (1024, 3072), (2048, 1024)])
 def test_matvec_outer_transpose(oracle, hip, m, n):
     r = rng(m + n)
     A = r.standard_normal((m, n)).astype(np.float32)

@@ -1910,9 +1910,22 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* A, float* B
 // The same through a 64 x 64 tile with 16-byte accesses on both sides (m and n multiples of 4, A and B on 16-byte
 // boundaries): thread (tx, ty) of 16 x 16 reads pieces tx of rows ty, ty + 16, ... of the tile of A, and writes pieces
 // tx of rows ty, ty + 16, ... of the tile of B, whose four values come from four rows of the LDS tile.
-__global__ __launch_bounds__(256) void transpose_vec_kernel(const float* A, float* B, size_t m, size_t n, float alpha) {
+// Tiles are numbered along the rows of A; `diagonal` numbers them down the diagonals instead (tile row = id mod gy, tile
+// column = id / gy + tile row), so that the tiles in flight differ in both their column of A and their column of B: with
+// both row lengths multiples of 4 KiB, tiles of one row of A write to addresses a multiple of 4 KiB apart, which land on
+// few memory channels (4096 x 4096: 23.4 -> 20.5 us, 8192 x 8192: 123 -> 103 us).
+__global__ __launch_bounds__(256) void transpose_vec_kernel(const float* A, float* B, size_t m, size_t n, float alpha,
+                                                            bool diagonal, unsigned gx, unsigned gy) {
     __shared__ float tile[64][65];
-    const size_t bi = (size_t)blockIdx.y * 64, bj = (size_t)blockIdx.x * 64;
+    unsigned bx, by;
+    if (diagonal) {
+        by = blockIdx.x % gy;
+        bx = (blockIdx.x / gy + by) % gx;
+    } else {
+        bx = blockIdx.x % gx;
+        by = blockIdx.x / gx;
+    }
+    const size_t bi = (size_t)by * 64, bj = (size_t)bx * 64;
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     float4 u[4];
 #pragma unroll
@@ -2450,9 +2463,13 @@ ZG_API int zg_hip_transpose(zg_hip_ctx* ctx, const float* A, float* B, size_t m,
     if (m == 0 || n == 0) return ZG_HIP_OK;
     ZG_REQUIRE(A && B, "transpose: null pointer");
     ZG_REQUIRE(A != B, "transpose: in-place transpose is not supported");
-    if (aligned16(A) && aligned16(B) && m % 4 == 0 && n % 4 == 0 && ceil_div_sz(m, 64) <= 65535) {
-        dim3 grid((unsigned)ceil_div_sz(n, 64), (unsigned)ceil_div_sz(m, 64));
-        hipLaunchKernelGGL(transpose_vec_kernel, grid, dim3(256), 0, ctx->stream, A, B, m, n, alpha);
+    if (aligned16(A) && aligned16(B) && m % 4 == 0 && n % 4 == 0 && ceil_div_sz(m, 64) * ceil_div_sz(n, 64) <= 0x7fffffffull) {
+        const unsigned gx = (unsigned)ceil_div_sz(n, 64), gy = (unsigned)ceil_div_sz(m, 64);
+        // wide matrices only: on 65536 x 4096 and on row lengths that are no multiple of 4 KiB the order along the rows
+        // is 3 to 8 % faster
+        const bool diagonal = n % 1024 == 0 && m % 1024 == 0 && n >= m;
+        dim3 grid((unsigned)((size_t)gx * gy));
+        hipLaunchKernelGGL(transpose_vec_kernel, grid, dim3(256), 0, ctx->stream, A, B, m, n, alpha, diagonal, gx, gy);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }

@@ -213,7 +213,9 @@ AXIS_SHAPES = [([64, 10], 1), ([64, 10], 0), ([64, 2], 1), ([2708, 16], 0), ([10
                ([1, 300000], 1), ([3, 262145], 1), ([7, 140002], 1), ([64, 16384], 1), ([100, 20000], 1), ([300000], 0),
                ([300, 16388], 1), ([2, 3, 140000], 2),
                # rows whose last trip of loads is partial
-               ([700, 1000], 1), ([300, 1028], 1), ([900, 260], 1), ([50, 2044], 1)]
+               ([700, 1000], 1), ([300, 1028], 1), ([900, 260], 1), ([50, 2044], 1),
+               # tall matrices of one column group: 128 chunks of rows from 64 MiB, 256 from 256 MiB
+               ([262149, 64], 0), ([65541, 256], 0), ([1048581, 68], 0)]
 
 
 @pytest.mark.parametrize("shape,dim", AXIS_SHAPES)
@@ -226,7 +228,10 @@ def test_sum_max_argmax_along(oracle, hip, shape, dim):
     y0 = r.standard_normal(out_n).astype(np.float32)
     a, b = both(oracle, hip, "sum_along", {"x": x, "x_shape": shape, "y": y0, "dim": dim, "alpha": 1.0, "beta": 1.0}, ["y"])
     truth = x64.sum(axis=dim).ravel() + y0
-    assert rel_fro(b["y"], truth) <= TOL and rel_fro(a["y"], truth) <= TOL
+    # the host's running float sum over a million terms drifts further from the exact sum than 1e-5 (1.6e-5 measured);
+    # the device's partial sums stay at 4e-7
+    tol_host = TOL if shape[dim] <= (1 << 19) else 1e-4
+    assert rel_fro(b["y"], truth) <= TOL and rel_fro(a["y"], truth) <= tol_host
     if out_n > 1:
         a, b = both(oracle, hip, "sum_along", {"x": x, "x_shape": shape, "y": np.full(out_n, 7.0, np.float32), "dim": dim}, ["y"])
         assert rel_fro(b["y"], x64.sum(axis=dim).ravel()) <= TOL

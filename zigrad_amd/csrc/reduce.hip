@@ -292,7 +292,17 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
     if (chunks < 1) chunks = 1;
     // keeps the partials buffer and the serial tail of the final stage small (the wide shape has a quarter of the
     // column groups, so it takes more chunks for enough workgroups)
-    const size_t chunk_cap = (wide && ry == 1) ? 256 : 64;
+    size_t chunk_cap = (wide && ry == 1) ? 256 : 64;
+    if (!(wide && ry == 1)) {
+        // tall matrices of few columns: with 64 chunks a matrix of a single column group runs on 64 workgroups (4194304 x
+        // 64: 361 us, 37 % of 8 TB/s).  128 workgroups in all from 64 MiB and 256 from 256 MiB, so chunks of 512 KiB at
+        // least (4194304 x 64: 187 us, 1048576 x 64: 62 -> 43 us, 262144 x 256: 62 -> 41 us); more than that and the
+        // final stage, one workgroup per 64 outputs walking every chunk, costs what the first stage gains
+        const size_t total = outer * R * inner;
+        const size_t groups = total >= ((size_t)1 << 26) ? 256 : total >= ((size_t)1 << 24) ? 128 : 64;
+        size_t c = groups / (gx * outer);
+        if (c > chunk_cap) chunk_cap = c;
+    }
     if (chunks > chunk_cap) chunks = chunk_cap;
     if (outer * R * inner <= kColSingleChunkMax) chunks = 1;  // a second launch costs more than a chunk split saves
     const size_t rows_per_chunk = ceil_div_sz(R, chunks);

@@ -62,7 +62,10 @@ def test_smce_fwd_small_batches_equal_the_two_launch_path(hip, rows, cols):
 SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (17, 32000), (300, 257), (5, 70001), (9, 4100),
                # rows held in registers by 4, 16 or 64 lanes, by a workgroup of 256 threads (4 or 8 pieces each) or of 1024
                (3000, 8), (3000, 32), (700, 36), (1500, 256), (40, 260), (300, 1024), (40, 1028), (21, 2048), (9, 4096),
-               (7, 5000), (6, 8192), (5, 8196), (3, 20000), (2, 32768)]
+               (7, 5000), (6, 8192), (5, 8196), (3, 20000), (2, 32768),
+               # rows that start off a 16-byte boundary: heads and tails of one to three values, pieces that hold the end
+               # of one row and the start of the next, rows too long for the registers
+               (1000, 5), (999, 6), (501, 11), (40, 4099), (7, 33001), (3, 70002), (2, 131072), (2000, 3), (5000, 1)]
 
 
 @pytest.mark.parametrize("rows,cols", SMCE_SHAPES)
@@ -82,8 +85,9 @@ def test_smce_onehot_and_label(oracle, hip, rows, cols):
     loss = float(np.mean(-np.log(np.clip(p_lab, np.float32(1e-7), np.float32(1.0) - np.float32(1e-7)))))
     # The host loop adds the exponentials of a row one after the other in fp32; for rows of tens of thousands
     # of columns that alone drifts past 1e-5 from the exact value.  The device result is held to 1e-5 against
-    # fp64; the oracle is held to 1e-5 where its own summation error allows it and to 2e-4 beyond.
-    oracle_tol = TOL if cols <= 4096 else 2e-4
+    # fp64; the oracle is held to 1e-5 where its own summation error allows it, to 2e-4 up to rows of 70002 columns
+    # and to 1e-3 beyond (3.3e-4 measured on rows of 131072).
+    oracle_tol = TOL if cols <= 4096 else 2e-4 if cols <= 70002 else 1e-3
     assert rel_fro(b["probs"], sm) <= TOL and rel_fro(a["probs"], sm) <= oracle_tol
     assert rel_fro(b["probs"], a["probs"]) <= max(TOL, 1.1 * rel_fro(a["probs"], sm) + 1e-6)
     assert abs(b["loss"][0] - loss) <= 1e-5 * max(1.0, abs(loss))
@@ -129,7 +133,9 @@ def test_smce_clamp_edge(oracle, hip):
 @pytest.mark.parametrize("rows,cols", [(64, 10), (5, 3000), (1, 7), (3, 8192), (2, 32768), (2, 32772),
                                        # every shape of the kernels that hold a row in registers, and rows beside them
                                        (1000, 4), (700, 32), (300, 36), (1500, 256), (70, 260), (300, 1024), (33, 1028),
-                                       (21, 4096), (9, 4100), (5, 8196), (3, 32764), (70, 1030), (500, 30)])
+                                       (21, 4096), (9, 4100), (5, 8196), (3, 32764), (70, 1030), (500, 30),
+                                       # rows that start off a 16-byte boundary, rows too long for the registers
+                                       (999, 6), (501, 11), (40, 4099), (7, 33001), (3, 70002), (2000, 3)])
 def test_softmax_fwd_bwd(oracle, hip, rows, cols):
     r = rng(rows + cols)
     x = r.standard_normal((rows, cols)).astype(np.float32)

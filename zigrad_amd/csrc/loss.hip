@@ -41,22 +41,45 @@ __device__ __forceinline__ void online_push(OnlineAccT& a, float x) {
     a.s = __fadd_rn(a.s, expf(__fsub_rn(x, a.m)));
 }
 
-// one pass over a row: per-thread online accumulation, then a group reduction
+// Elements of a row before its first 16-byte boundary (0 to 3, fewer for a row that ends before it).
+__device__ __forceinline__ size_t row_head(const float* xr, size_t cols) {
+    const size_t h = (size_t)((0 - (reinterpret_cast<uintptr_t>(xr) >> 2)) & 3);
+    return h < cols ? h : cols;
+}
+
+// one pass over a row: per-thread online accumulation, then a group reduction.  A row starts wherever row * cols puts
+// it: the elements before its first 16-byte boundary and after its last whole 16-byte piece (at most three each) are
+// pushed one by one by the first lanes, the pieces between are read 16 bytes at a time.  (A row of 32001 or 50257
+// columns read value by value ran at 37 % of 8 TB/s where 32000 columns reach 83 %.)
+// Rows of fewer than 8 * TPR columns that are not whole 16-byte pieces are pushed value by value by all lanes: with one
+// or two pieces per lane the head and the tail cost more than the pieces save ([4194304, 7]: 151 us value by value,
+// 204 us in pieces).  KEEP: plain loads, for a caller whose second pass reads the row again; else the row is read with
+// the non-temporal hint.
 template <int TPR>
+__device__ __forceinline__ bool row_in_pieces(size_t h, size_t cols) {
+    return (h == 0 && cols % 4 == 0) || cols >= (size_t)8 * TPR;
+}
+template <int TPR, bool KEEP = false>
 __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, int lane) {
+    static_assert(TPR >= 4, "the first lanes take the head and the tail of a row");
     OnlineAccT acc = OnlineAcc::init();
-    const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15u) == 0) && (cols % 4 == 0);
-    if (vec) {
-        const float4* x4 = reinterpret_cast<const float4*>(xr);
-        const size_t c4 = cols >> 2;
+    const size_t h = row_head(xr, cols);
+    auto load = [](const float4* p) { return KEEP ? *p : nt_load(p); };
+    if (!row_in_pieces<TPR>(h, cols)) {
+        for (size_t j = lane; j < cols; j += TPR)
+            if (xr[j] != -INFINITY) online_push(acc, xr[j]);
+    } else {
+        if ((size_t)lane < h && xr[lane] != -INFINITY) online_push(acc, xr[lane]);
+        const float4* x4 = reinterpret_cast<const float4*>(xr + h);
+        const size_t c4 = (cols - h) >> 2;
         // four 16-byte loads in flight per thread; past the end of the row they are replaced by -inf, which adds
         // exp(-inf) = 0, so the last partial round takes the same path as the others
         const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
         for (size_t j = lane; j < c4; j += 4 * TPR) {
-            const float4 v0 = nt_load(x4 + j);
-            const float4 v1 = (j + TPR < c4) ? nt_load(x4 + j + TPR) : ninf;
-            const float4 v2 = (j + 2 * TPR < c4) ? nt_load(x4 + j + 2 * TPR) : ninf;
-            const float4 v3 = (j + 3 * TPR < c4) ? nt_load(x4 + j + 3 * TPR) : ninf;
+            const float4 v0 = load(x4 + j);
+            const float4 v1 = (j + TPR < c4) ? load(x4 + j + TPR) : ninf;
+            const float4 v2 = (j + 2 * TPR < c4) ? load(x4 + j + 2 * TPR) : ninf;
+            const float4 v3 = (j + 3 * TPR < c4) ? load(x4 + j + 3 * TPR) : ninf;
             // one rescale per 16 elements: fold the 16 into the running max first
             float mx = fmaxf(fmaxf(fmaxf(v0.x, v0.y), fmaxf(v0.z, v0.w)), fmaxf(fmaxf(v1.x, v1.y), fmaxf(v1.z, v1.w)));
             mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(v2.x, v2.y), fmaxf(v2.z, v2.w)), fmaxf(fmaxf(v3.x, v3.y), fmaxf(v3.z, v3.w))));
@@ -72,10 +95,84 @@ __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, i
             s += fexp(v3.x - acc.m) + fexp(v3.y - acc.m) + fexp(v3.z - acc.m) + fexp(v3.w - acc.m);
             acc.s += s;
         }
-    } else {
-        for (size_t j = lane; j < cols; j += TPR) online_push(acc, xr[j]);
+        const size_t tail = h + (c4 << 2) + (size_t)lane;
+        if (tail < cols && xr[tail] != -INFINITY) online_push(acc, xr[tail]);
     }
     return acc;
+}
+
+// Second pass over a row: probabilities exp(x - l) written out; MODE 1 also returns this lane's part of the row's loss
+// term sum_j -t_j * log(clamp(p_j)); GRAD 1 writes (p - t) / denom to the gradient row, GRAD 2 adds it.  Where the rows
+// of all the arrays involved start at the same offset from a 16-byte boundary, the row is walked like row_online walks
+// it (head, 16-byte pieces with four in flight per lane, tail); rows of fewer than 8 * TPR columns and rows that start at
+// different offsets go value by value.  Each element's arithmetic is the same either way.
+template <int TPR, int MODE, int GRAD>
+__device__ __forceinline__ float row_probs(const float* xr, const float* tr, float* pr, float* gr, size_t cols, int lane,
+                                           float l, float denom, bool fast) {
+    float part = 0.f;
+    auto element = [&](float x, float t, float g, float& p, float& d) {
+        p = fast ? fexp(__fsub_rn(x, l)) : expf(__fsub_rn(x, l));
+        if (MODE) {
+            if (t != 0.f) {  // a zero target adds t * log(.) = 0: skipping it changes nothing and saves the log
+                const float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
+                part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
+            }
+            if (GRAD) {
+                d = __fdiv_rn(__fsub_rn(p, t), denom);
+                if (GRAD == 2) d = __fadd_rn(g, d);
+            }
+        }
+    };
+    auto scalar = [&](size_t j) {
+        float p, dd = 0.f;
+        element(xr[j], MODE ? tr[j] : 0.f, GRAD == 2 ? gr[j] : 0.f, p, dd);
+        pr[j] = p;
+        if (GRAD) gr[j] = dd;
+    };
+    uintptr_t differ = reinterpret_cast<uintptr_t>(xr) ^ reinterpret_cast<uintptr_t>(pr);
+    if (MODE) differ |= reinterpret_cast<uintptr_t>(xr) ^ reinterpret_cast<uintptr_t>(tr);
+    if (GRAD) differ |= reinterpret_cast<uintptr_t>(xr) ^ reinterpret_cast<uintptr_t>(gr);
+    if ((differ & 15u) != 0 || cols < (size_t)8 * TPR) {
+        for (size_t j = lane; j < cols; j += TPR) scalar(j);
+        return part;
+    }
+    const size_t h = row_head(xr, cols);
+    if ((size_t)lane < h) scalar(lane);
+    const size_t c4 = (cols - h) >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(xr + h);
+    const float4* t4 = reinterpret_cast<const float4*>(MODE ? tr + h : xr + h);
+    float4* p4 = reinterpret_cast<float4*>(pr + h);
+    float4* g4 = reinterpret_cast<float4*>(GRAD ? gr + h : pr + h);
+    constexpr int U = 4;
+    for (size_t j0 = lane; j0 < c4; j0 += (size_t)U * TPR) {
+        float4 v[U], t[U], g[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t j = j0 + (size_t)u * TPR;
+            if (j < c4) {
+                v[u] = nt_load(x4 + j);
+                if (MODE) t[u] = nt_load(t4 + j);
+                if (GRAD == 2) g[u] = nt_load(g4 + j);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t j = j0 + (size_t)u * TPR;
+            if (j < c4) {
+                float4 p, dd = make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 tt = MODE ? t[u] : dd, gg = GRAD == 2 ? g[u] : dd;
+                element(v[u].x, tt.x, gg.x, p.x, dd.x);
+                element(v[u].y, tt.y, gg.y, p.y, dd.y);
+                element(v[u].z, tt.z, gg.z, p.z, dd.z);
+                element(v[u].w, tt.w, gg.w, p.w, dd.w);
+                nt_store(p, p4 + j);
+                if (GRAD) nt_store(dd, g4 + j);
+            }
+        }
+    }
+    const size_t tail = h + (c4 << 2) + (size_t)lane;
+    if (tail < cols) scalar(tail);
+    return part;
 }
 
 template <int TPR>
@@ -116,63 +213,20 @@ __global__ __launch_bounds__(kBlock) void smce_label_fwd_kernel(const float* log
     }
 }
 
-// grad (+)= (exp(x - lse[row]) - onehot) / rows, elementwise over the whole matrix.
-// grid: x over chunks of 4 * kBlock float4 columns of one row, y over rows (looped).  A thread has four 16-byte
-// loads (eight when accumulating) in flight: with one, the resident waves cannot cover the HBM latency.
+// grad (+)= (exp(x - lse[row]) - onehot) / rows, elementwise over the whole matrix, value by value: for operands that
+// are not on 16-byte boundaries and rows of fewer than four columns.
 template <bool ACC>
-__global__ __launch_bounds__(kBlock) void smce_label_bwd_kernel(const float* logits, const uint64_t* labels,
-                                                                 const float* lse, float* grad, size_t rows,
-                                                                 size_t cols, float denom) {
+__global__ __launch_bounds__(kBlock) void smce_label_bwd_values_kernel(const float* logits, const uint64_t* labels,
+                                                                        const float* lse, float* grad, size_t n,
+                                                                        size_t cols, float denom) {
     const float inv_denom = __fdiv_rn(1.0f, denom);  // exact for power-of-two batch sizes, else within 1 ulp of x/denom
-    const bool vec = (((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(grad)) & 15u) == 0) &&
-                     (cols % 4 == 0);
-    constexpr int U = 4;
-    for (size_t row = blockIdx.y; row < rows; row += gridDim.y) {
-        const float l = lse[row];
-        const uint64_t lab = labels[row];
-        const float* xr = logits + row * cols;
-        float* gr = grad + row * cols;
-        if (vec) {
-            const size_t c4 = cols >> 2;
-            const float4* x4 = reinterpret_cast<const float4*>(xr);
-            float4* g4 = reinterpret_cast<float4*>(gr);
-            for (size_t j0 = (size_t)blockIdx.x * (kBlock * U) + threadIdx.x; j0 < c4; j0 += (size_t)gridDim.x * (kBlock * U)) {
-                float4 v[U], g[U];
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const size_t j = j0 + (size_t)u * kBlock;
-                    if (j < c4) {
-                        v[u] = nt_load(x4 + j);
-                        if (ACC) g[u] = nt_load(g4 + j);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const size_t j = j0 + (size_t)u * kBlock;
-                    if (j < c4) {
-                        const size_t c = 4 * j;
-                        float d0 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].x, l)), (c + 0 == lab) ? 1.f : 0.f), inv_denom);
-                        float d1 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].y, l)), (c + 1 == lab) ? 1.f : 0.f), inv_denom);
-                        float d2 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].z, l)), (c + 2 == lab) ? 1.f : 0.f), inv_denom);
-                        float d3 = __fmul_rn(__fsub_rn(fexp(__fsub_rn(v[u].w, l)), (c + 3 == lab) ? 1.f : 0.f), inv_denom);
-                        float4 o;
-                        o.x = ACC ? __fadd_rn(g[u].x, d0) : d0;
-                        o.y = ACC ? __fadd_rn(g[u].y, d1) : d1;
-                        o.z = ACC ? __fadd_rn(g[u].z, d2) : d2;
-                        o.w = ACC ? __fadd_rn(g[u].w, d3) : d3;
-                        nt_store(o, g4 + j);
-                    }
-                }
-            }
-        } else {
-            for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += (size_t)gridDim.x * kBlock) {
-                float d = __fmul_rn(__fsub_rn(fexp(__fsub_rn(xr[j], l)), (j == lab) ? 1.f : 0.f), inv_denom);
-                gr[j] = ACC ? __fadd_rn(gr[j], d) : d;
-            }
-        }
+    const size_t nt = (size_t)gridDim.x * kBlock;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += nt) {
+        const size_t r = i / cols, c = i - r * cols;
+        const float d = __fmul_rn(__fsub_rn(fexp(__fsub_rn(logits[i], lse[r])), (c == labels[r]) ? 1.f : 0.f), inv_denom);
+        grad[i] = ACC ? __fadd_rn(grad[i], d) : d;
     }
 }
-
 
 // The same update with the matrix walked as one flat array: workgroup b owns float4 b*1024 .. b*1024+1023 of both
 // streams, whatever rows they fall in (rows of at least 256 float4, so a piece crosses at most a few row ends).
@@ -228,6 +282,80 @@ __global__ __launch_bounds__(kBlock) void smce_label_bwd_flat_kernel(const float
 }
 
 
+// The same for rows of any length of at least four columns (both matrices on 16-byte boundaries): the matrix is still
+// walked as one flat array of 16-byte pieces, and a piece may end one row and begin the next, so a thread fetches lse
+// and label of the row its piece starts in and of the one after, and each of the four values takes the pair of its own
+// row.  The n % 4 values after the last whole piece are done one by one.  (One workgroup per row, the form this
+// replaces, ran [1048576, 10] at 4 % of 8 TB/s and [8192, 50257] at 50 %.)
+template <bool ACC>
+__global__ __launch_bounds__(kBlock) void smce_label_bwd_any_kernel(const float* logits, const uint64_t* labels,
+                                                                     const float* lse, float* grad, size_t n, size_t cols,
+                                                                     size_t rows, float denom) {
+    const float inv_denom = __fdiv_rn(1.0f, denom);
+    const float4* x4 = reinterpret_cast<const float4*>(logits);
+    float4* g4 = reinterpret_cast<float4*>(grad);
+    const size_t n4 = n >> 2;
+    for (size_t c0 = (size_t)blockIdx.x * kLabelBwdChunk; c0 < n4; c0 += (size_t)gridDim.x * kLabelBwdChunk) {
+        const size_t e0 = c0 << 2, r0 = e0 / cols, rem = e0 - r0 * cols;
+        float4 v[kLabelBwdU], g[kLabelBwdU];
+        float l0[kLabelBwdU], l1[kLabelBwdU];
+        uint64_t lab0[kLabelBwdU], lab1[kLabelBwdU];
+        size_t col[kLabelBwdU];  // column of the piece's first value
+#pragma unroll
+        for (int u = 0; u < kLabelBwdU; u++) {
+            const size_t j = c0 + threadIdx.x + (size_t)u * kBlock;
+            size_t o = rem + 4 * (threadIdx.x + (size_t)u * kBlock), r = r0;  // o < cols + 4 * kLabelBwdChunk
+            if (cols >= 4 * kLabelBwdChunk) {
+                if (o >= cols) {
+                    o -= cols;
+                    r++;
+                }
+            } else {
+                const uint32_t q = (uint32_t)o / (uint32_t)cols;
+                o -= (size_t)q * cols;
+                r += q;
+            }
+            col[u] = o;
+            if (j < n4) {
+                const size_t r1 = r + 1 < rows ? r + 1 : r;
+                v[u] = nt_load(x4 + j);
+                if (ACC) g[u] = nt_load(g4 + j);
+                l0[u] = lse[r];
+                l1[u] = lse[r1];
+                lab0[u] = labels[r];
+                lab1[u] = labels[r1];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kLabelBwdU; u++) {
+            const size_t j = c0 + threadIdx.x + (size_t)u * kBlock;
+            if (j < n4) {
+                auto value = [&](float x, size_t c) {
+                    const bool next = c >= cols;  // at most one row end inside a piece: cols >= 4
+                    const float l = next ? l1[u] : l0[u];
+                    const uint64_t lab = next ? lab1[u] : lab0[u];
+                    const size_t cc = next ? c - cols : c;
+                    return __fmul_rn(__fsub_rn(fexp(__fsub_rn(x, l)), (cc == lab) ? 1.f : 0.f), inv_denom);
+                };
+                const float d0 = value(v[u].x, col[u]), d1 = value(v[u].y, col[u] + 1), d2 = value(v[u].z, col[u] + 2),
+                            d3 = value(v[u].w, col[u] + 3);
+                float4 o;
+                o.x = ACC ? __fadd_rn(g[u].x, d0) : d0;
+                o.y = ACC ? __fadd_rn(g[u].y, d1) : d1;
+                o.z = ACC ? __fadd_rn(g[u].z, d2) : d2;
+                o.w = ACC ? __fadd_rn(g[u].w, d3) : d3;
+                nt_store(o, g4 + j);
+            }
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const size_t i = (n4 << 2) + threadIdx.x, r = i / cols, c = i - r * cols;
+        const float d = __fmul_rn(__fsub_rn(fexp(__fsub_rn(logits[i], lse[r])), (c == labels[r]) ? 1.f : 0.f), inv_denom);
+        grad[i] = ACC ? __fadd_rn(grad[i], d) : d;
+    }
+}
+
+
 // one-hot targets (the reference's form): probabilities are written out; the row's loss term is
 // sum_j -t_j * log(clamp(p_j)).  MODE 0: softmax only (no target, no loss).
 template <int TPR, int MODE>
@@ -240,25 +368,13 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* logit
     const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
     const bool live = row < rows;
     OnlineAccT acc = OnlineAcc::init();
-    if (live) acc = row_online<TPR>(logits + row * cols, cols, lane);
+    if (live) acc = row_online<TPR, true>(logits + row * cols, cols, lane);
     acc = row_group_reduce<TPR>(acc, smem);
     float part = 0.f;
     if (live) {
         const float l = __fadd_rn(acc.m, logf(acc.s));
-        const float* xr = logits + row * cols;
-        const float* tr = MODE ? target + row * cols : nullptr;
-        float* pr = probs + row * cols;
-        for (size_t j = lane; j < cols; j += TPR) {
-            float p = expf(__fsub_rn(xr[j], l));
-            pr[j] = p;
-            if (MODE) {
-                float t = tr[j];
-                if (t != 0.f) {  // a zero target adds t * log(.) = 0: skipping it changes nothing and saves the log
-                    float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
-                    part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
-                }
-            }
-        }
+        part = row_probs<TPR, MODE, 0>(logits + row * cols, MODE ? target + row * cols : nullptr, probs + row * cols,
+                                       nullptr, cols, lane, l, 1.f, false);
     }
     if (MODE) {
         if (TPR <= kWave) {
@@ -589,7 +705,7 @@ __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* lo
     const bool live = row < rows;
     const float denom = (float)rows;
     OnlineAccT acc = OnlineAcc::init();
-    if (live) acc = row_online<TPR>(logits + row * cols, cols, lane);
+    if (live) acc = row_online<TPR, true>(logits + row * cols, cols, lane);
     acc = group_reduce<OnlineAcc, TPR>(acc);
     float part = 0.f;
     // rows the register-resident kernels take in a larger batch (wave_row_ok) get their exponential, so that a row's
@@ -598,23 +714,8 @@ __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* lo
                                          reinterpret_cast<uintptr_t>(probs)) & 15u) == 0;
     if (live) {
         const float l = __fadd_rn(acc.m, logf(acc.s));
-        const float* xr = logits + row * cols;
-        const float* tr = target + row * cols;
-        float* pr = probs + row * cols;
-        float* gr = grad + row * cols;
-        for (size_t j = lane; j < cols; j += TPR) {
-            const float p = fast ? fexp(__fsub_rn(xr[j], l)) : expf(__fsub_rn(xr[j], l));
-            const float t = tr[j];
-            pr[j] = p;
-            if (t != 0.f) {
-                const float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
-                part = __fsub_rn(part, __fmul_rn(t, logf(safe)));
-            }
-            if (GRAD) {
-                const float d = __fdiv_rn(__fsub_rn(p, t), denom);
-                gr[j] = (GRAD == 2) ? __fadd_rn(gr[j], d) : d;
-            }
-        }
+        part = row_probs<TPR, 1, GRAD>(logits + row * cols, target + row * cols, probs + row * cols,
+                                       GRAD ? grad + row * cols : nullptr, cols, lane, l, denom, fast);
     }
     part = group_reduce<SumAcc, TPR>(part);
     if (live && lane == 0) row_loss[row] = part;
@@ -635,8 +736,43 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
     const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
     const bool live = row < rows;
     float part = 0.f;
-    if (live)
-        for (size_t j = lane; j < cols; j += TPR) part = __fadd_rn(part, __fmul_rn(y[row * cols + j], y_g[row * cols + j]));
+    const float* yr = y + row * cols;
+    const float* gr = y_g + row * cols;
+    float* xr = x_g + row * cols;
+    // rows of the three operands that start at the same offset from a 16-byte boundary are walked in 16-byte pieces, the
+    // values before the first boundary and after the last whole piece by the first lanes (rows of 32001 columns value
+    // by value: 31 % of 8 TB/s)
+    const bool pieces = live && cols >= (size_t)8 * TPR &&
+                        (((reinterpret_cast<uintptr_t>(yr) ^ reinterpret_cast<uintptr_t>(gr)) |
+                          (reinterpret_cast<uintptr_t>(yr) ^ reinterpret_cast<uintptr_t>(xr))) & 15u) == 0;
+    const size_t h = live ? row_head(yr, cols) : 0, c4 = (cols - h) >> 2, tail = h + (c4 << 2) + (size_t)lane;
+    const float4* y4 = reinterpret_cast<const float4*>(yr + h);
+    const float4* q4 = reinterpret_cast<const float4*>(gr + h);
+    float4* x4 = reinterpret_cast<float4*>(xr + h);
+    if (pieces) {
+        auto dot4 = [](float4 a, float4 b) {
+            return __fadd_rn(__fadd_rn(__fmul_rn(a.x, b.x), __fmul_rn(a.y, b.y)), __fadd_rn(__fmul_rn(a.z, b.z), __fmul_rn(a.w, b.w)));
+        };
+        if ((size_t)lane < h) part = __fmul_rn(yr[lane], gr[lane]);
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        for (size_t j = lane; j < c4; j += 4 * TPR) {
+            const bool in1 = j + TPR < c4, in2 = j + 2 * TPR < c4, in3 = j + 3 * TPR < c4;
+            // plain loads: the second pass reads both rows again
+            const float4 a0 = y4[j], b0 = q4[j];
+            const float4 a1 = in1 ? y4[j + TPR] : zero, b1 = in1 ? q4[j + TPR] : zero;
+            const float4 a2 = in2 ? y4[j + 2 * TPR] : zero, b2 = in2 ? q4[j + 2 * TPR] : zero;
+            const float4 a3 = in3 ? y4[j + 3 * TPR] : zero, b3 = in3 ? q4[j + 3 * TPR] : zero;
+            s0 = __fadd_rn(s0, dot4(a0, b0));
+            s1 = __fadd_rn(s1, dot4(a1, b1));
+            s2 = __fadd_rn(s2, dot4(a2, b2));
+            s3 = __fadd_rn(s3, dot4(a3, b3));
+        }
+        part = __fadd_rn(part, __fadd_rn(__fadd_rn(s0, s1), __fadd_rn(s2, s3)));
+        if (tail < cols) part = __fadd_rn(part, __fmul_rn(yr[tail], gr[tail]));
+    } else if (live) {
+        for (size_t j = lane; j < cols; j += TPR) part = __fadd_rn(part, __fmul_rn(yr[j], gr[j]));
+    }
     if (TPR <= kWave) {
         part = group_reduce<SumAcc, (TPR <= kWave ? TPR : kWave)>(part);
     } else {
@@ -646,11 +782,33 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
         __syncthreads();
         part = bcast;
     }
-    if (live)
-        for (size_t j = lane; j < cols; j += TPR) {
-            size_t k = row * cols + j;
-            x_g[k] = __fadd_rn(x_g[k], __fmul_rn(y[k], __fsub_rn(y_g[k], part)));
+    if (pieces) {
+        if ((size_t)lane < h) xr[lane] = __fadd_rn(xr[lane], __fmul_rn(yr[lane], __fsub_rn(gr[lane], part)));
+        for (size_t j0 = lane; j0 < c4; j0 += 2 * TPR) {
+            const size_t j1 = j0 + TPR;
+            const bool in1 = j1 < c4;
+            const float4 a0 = nt_load(y4 + j0), b0 = nt_load(q4 + j0), x0 = nt_load(x4 + j0);
+            float4 a1 = a0, b1 = b0, x1 = x0;
+            if (in1) {
+                a1 = nt_load(y4 + j1);
+                b1 = nt_load(q4 + j1);
+                x1 = nt_load(x4 + j1);
+            }
+            auto upd = [&](float4 a, float4 b, float4 x) {
+                float4 o;
+                o.x = __fadd_rn(x.x, __fmul_rn(a.x, __fsub_rn(b.x, part)));
+                o.y = __fadd_rn(x.y, __fmul_rn(a.y, __fsub_rn(b.y, part)));
+                o.z = __fadd_rn(x.z, __fmul_rn(a.z, __fsub_rn(b.z, part)));
+                o.w = __fadd_rn(x.w, __fmul_rn(a.w, __fsub_rn(b.w, part)));
+                return o;
+            };
+            nt_store(upd(a0, b0, x0), x4 + j0);
+            if (in1) nt_store(upd(a1, b1, x1), x4 + j1);
         }
+        if (tail < cols) xr[tail] = __fadd_rn(xr[tail], __fmul_rn(yr[tail], __fsub_rn(gr[tail], part)));
+    } else if (live) {
+        for (size_t j = lane; j < cols; j += TPR) xr[j] = __fadd_rn(xr[j], __fmul_rn(yr[j], __fsub_rn(gr[j], part)));
+    }
 }
 
 // The same with the rows of y and y_g held in registers (16-byte aligned rows of up to 32768 columns): NT threads per row
@@ -820,17 +978,28 @@ ZG_API int zg_hip_smce_label_bwd(zg_hip_ctx* ctx, const float* logits, const uin
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    // one workgroup per (row, chunk of 4 * kBlock float4 columns); rows beyond the grid limit are looped over
-    size_t gx = ceil_div_sz((cols + 3) / 4, (size_t)kBlock * 4);
-    if (gx > 1024) gx = 1024;
-    size_t gy = rows < 65535 ? rows : 65535;
-    dim3 grid((unsigned)gx, (unsigned)gy);
+    const size_t n = rows * cols;
+    if (aligned && cols >= 4 && cols < 0xffffffffull) {
+        size_t blocks = ceil_div_sz(n >> 2, kLabelBwdChunk);
+        if (blocks < 1) blocks = 1;
+        if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
+        if (accumulate)
+            hipLaunchKernelGGL((smce_label_bwd_any_kernel<true>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream,
+                               logits, labels, lse, grad, n, cols, rows, (float)rows);
+        else
+            hipLaunchKernelGGL((smce_label_bwd_any_kernel<false>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream,
+                               logits, labels, lse, grad, n, cols, rows, (float)rows);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    size_t blocks = ceil_div_sz(n, kBlock);
+    if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
     if (accumulate)
-        hipLaunchKernelGGL((smce_label_bwd_kernel<true>), grid, dim3(kBlock), 0, ctx->stream, logits, labels, lse, grad,
-                           rows, cols, (float)rows);
+        hipLaunchKernelGGL((smce_label_bwd_values_kernel<true>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, logits,
+                           labels, lse, grad, n, cols, (float)rows);
     else
-        hipLaunchKernelGGL((smce_label_bwd_kernel<false>), grid, dim3(kBlock), 0, ctx->stream, logits, labels, lse,
-                           grad, rows, cols, (float)rows);
+        hipLaunchKernelGGL((smce_label_bwd_values_kernel<false>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream,
+                           logits, labels, lse, grad, n, cols, (float)rows);
     ZG_LAUNCH_CHECK();
     return ZG_HIP_OK;
 }

@@ -114,6 +114,33 @@ def test_smce_onehot_and_label(oracle, hip, rows, cols):
     assert rel_fro(go, want) <= oracle_tol
 
 
+@pytest.mark.parametrize("rows,cols", [(5, 5), (70, 10), (40, 130), (9, 1001), (3, 4099), (2000, 7)])
+def test_rows_that_begin_with_minus_infinity(oracle, hip, rows, cols):
+    """Masked logits: -inf in the first columns (and elsewhere) of rows that are read value by value or in pieces with a
+    head.  The running maximum must not form exp(-inf - -inf) before it has seen a finite value."""
+    r = rng(rows * 3 + cols)
+    x = (r.standard_normal((rows, cols)) * 2).astype(np.float32)
+    x[:, 0] = -np.inf
+    x[::2, 1] = -np.inf
+    x[1::3, cols - 1] = -np.inf
+    lab = np.full(rows, 2, np.uint64)
+    t = np.zeros((rows, cols), np.float32)
+    t[:, 2] = 1.0
+    one = np.zeros(1, np.float32)
+    sm = softmax(x.astype(np.float64), axis=1)
+    a, b = both(oracle, hip, "smce_fwd", {"logits": x, "target": t, "probs": np.zeros_like(x), "loss": one, "rows": rows,
+                                          "cols": cols}, ["probs", "loss"])
+    assert np.isfinite(b["probs"]).all() and np.isfinite(b["loss"]).all()
+    assert rel_fro(b["probs"], sm) <= TOL and rel_fro(a["probs"], sm) <= TOL
+    assert abs(b["loss"][0] - a["loss"][0]) <= TOL * max(1.0, abs(a["loss"][0]))
+    a, b = both(oracle, hip, "softmax_fwd", {"x": x, "y": np.zeros_like(x), "rows": rows, "cols": cols}, ["y"])
+    assert rel_fro(b["y"], sm) <= TOL
+    a2, b2 = both(oracle, hip, "smce_label_fwd", {"logits": x, "labels": lab, "lse": np.zeros(rows, np.float32), "loss": one,
+                                                  "rows": rows, "cols": cols}, ["lse", "loss"])
+    assert rel_fro(b2["lse"], logsumexp(x.astype(np.float64), axis=1)) <= 1e-6
+    assert abs(b2["loss"][0] - a2["loss"][0]) <= TOL * max(1.0, abs(a2["loss"][0]))
+
+
 def test_smce_clamp_edge(oracle, hip):
     """A vanishing probability is clamped to 1e-7 in the loss only (src/nn/loss.zig:143)."""
     x = np.asarray([[100.0, 0.0, 0.0], [0.0, 0.0, 50.0]], np.float32)

@@ -1817,6 +1817,17 @@ __global__ __launch_bounds__(256) void gemv_t_kernel(const float* A, const float
                 acc[3 % V] += u.w * xv;
             }
         } else {
+            // single columns (a row length that is no multiple of four): sixteen rows in flight, then eight
+            for (; r + 15 * (size_t)ry < r1; r += 16 * (size_t)ry) {
+                float u[16], xs[16];
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    u[k] = ab[(r + (size_t)k * ry) * n];
+                    xs[k] = x[r + (size_t)k * ry];
+                }
+#pragma unroll
+                for (int k = 0; k < 16; k++) acc[0] += u[k] * xs[k];
+            }
             for (; r + 7 * (size_t)ry < r1; r += 8 * (size_t)ry) {
                 float u[8], xs[8];
 #pragma unroll
@@ -2406,11 +2417,13 @@ ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float*
         int log2_cx = 0;
         // 16 row-threads (and 16 column-threads) where a row-thread gets four rows or more, fewer for shorter matrices
         // (7 x 1048576: 11.5 us with 16 row-threads, 5.7 us with 4; 64 x 1048576: 50.5 us with 4, 39.1 us with 16)
-        const int cx_max = m >= 64 ? 4 : m >= 32 ? 5 : 6;
+        // single columns (V = 1): 64 column-threads, so that a wave still reads 256 adjacent bytes of a row (16 of them,
+        // 64 bytes: [8192, 32001] at 33 % of 8 TB/s)
+        const int cx_max = V == 1 ? 6 : m >= 64 ? 4 : m >= 32 ? 5 : 6;
         while (((size_t)1 << log2_cx) < colv && log2_cx < cx_max) log2_cx++;
         // narrower column groups (down to 16 column-threads) while they are fewer than two per compute unit: a wide matrix
         // of few rows then needs no row chunks at all
-        while (log2_cx > 4 && ceil_div_sz(colv, (size_t)1 << log2_cx) < 2 * n_cu) log2_cx--;
+        while (V == 4 && log2_cx > 4 && ceil_div_sz(colv, (size_t)1 << log2_cx) < 2 * n_cu) log2_cx--;
         const size_t gx = ceil_div_sz(colv, (size_t)1 << log2_cx);
         const size_t ry = (size_t)256 >> log2_cx;
         // row chunks: about two workgroups per compute unit, at least 64 rows and eight trips of ry rows each, at most 1024

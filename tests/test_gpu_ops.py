@@ -215,7 +215,9 @@ AXIS_SHAPES = [([64, 10], 1), ([64, 10], 0), ([64, 2], 1), ([2708, 16], 0), ([10
                # rows whose last trip of loads is partial
                ([700, 1000], 1), ([300, 1028], 1), ([900, 260], 1), ([50, 2044], 1),
                # tall matrices of one column group: 128 chunks of rows from 64 MiB, 256 from 256 MiB
-               ([262149, 64], 0), ([65541, 256], 0), ([1048581, 68], 0)]
+               ([262149, 64], 0), ([65541, 256], 0), ([1048581, 68], 0),
+               # rows that start off a 16-byte boundary and are read in 16-byte pieces between a head and a tail
+               ([600, 2051], 1), ([50, 4099], 1), ([9, 33001], 1), ([700, 513], 1), ([5, 300001], 1), ([2, 1000003], 1)]
 
 
 @pytest.mark.parametrize("shape,dim", AXIS_SHAPES)

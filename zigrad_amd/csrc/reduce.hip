@@ -154,17 +154,24 @@ __global__ __launch_bounds__(kBlock) void row_segments_kernel(const float* x, ty
     const size_t c_begin = s * seg, c_end = c_begin + seg < cols ? c_begin + seg : cols;
     const float* xr = x + row * cols;
     typename P::Acc acc = P::init();
-    const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15u) == 0) && (cols % 4 == 0);
-    if (vec) {
-        const float4* x4 = reinterpret_cast<const float4*>(xr);
-        const size_t j_end = c_end >> 2;
-        size_t j = (c_begin >> 2) + threadIdx.x;
+    // the segment's values before its first 16-byte boundary and after its last whole 16-byte piece (at most three each,
+    // none where rows start on 16-byte boundaries) go to the first threads, the pieces between are read 16 bytes at a time
+    const float* sp = xr + c_begin;
+    const size_t len = c_end - c_begin;
+    size_t h = (size_t)((0 - (reinterpret_cast<uintptr_t>(sp) >> 2)) & 3);
+    if (h > len) h = len;
+    if (threadIdx.x < h) acc = P::combine(acc, A::term(sp[threadIdx.x], (uint32_t)(c_begin + threadIdx.x)));
+    {
+        const float4* x4 = reinterpret_cast<const float4*>(sp + h);
+        const size_t j_end = (len - h) >> 2;
+        const uint32_t c0 = (uint32_t)(c_begin + h);
+        size_t j = threadIdx.x;
         for (; j + 3 * kBlock < j_end; j += 4 * kBlock) {
             const float4 vs[4] = {nt_load(x4 + j), nt_load(x4 + j + kBlock), nt_load(x4 + j + 2 * kBlock),
                                   nt_load(x4 + j + 3 * kBlock)};
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                const uint32_t c = (uint32_t)(4 * (j + (size_t)u * kBlock));
+                const uint32_t c = c0 + (uint32_t)(4 * (j + (size_t)u * kBlock));
                 acc = P::combine(acc, A::term(vs[u].x, c + 0));
                 acc = P::combine(acc, A::term(vs[u].y, c + 1));
                 acc = P::combine(acc, A::term(vs[u].z, c + 2));
@@ -173,14 +180,14 @@ __global__ __launch_bounds__(kBlock) void row_segments_kernel(const float* x, ty
         }
         for (; j < j_end; j += kBlock) {
             const float4 v = x4[j];
-            const uint32_t c = (uint32_t)(4 * j);
+            const uint32_t c = c0 + (uint32_t)(4 * j);
             acc = P::combine(acc, A::term(v.x, c + 0));
             acc = P::combine(acc, A::term(v.y, c + 1));
             acc = P::combine(acc, A::term(v.z, c + 2));
             acc = P::combine(acc, A::term(v.w, c + 3));
         }
-    } else {
-        for (size_t j = c_begin + threadIdx.x; j < c_end; j += kBlock) acc = P::combine(acc, A::term(xr[j], (uint32_t)j));
+        const size_t tail = h + (j_end << 2) + threadIdx.x;
+        if (tail < len) acc = P::combine(acc, A::term(sp[tail], (uint32_t)(c_begin + tail)));
     }
     acc = block_reduce<P>(acc, smem);
     if (threadIdx.x == 0) partials[s * rows + row] = acc;

@@ -32,7 +32,11 @@ def rng(seed):
 # ----------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 @pytest.mark.parametrize("xl,yl", [(1, 1), (1, 777), (777, 1), (4096, 4096), (1001, 1001), (128, 128 * 64), (128 * 64, 128),
-                                   (10, 640), (640, 10), (4096, 4096 * 33), (12, 12 * 1000), (300000, 300000)])
+                                   (10, 640), (640, 10), (4096, 4096 * 33), (12, 12 * 1000), (300000, 300000),
+                                   # periods that are no multiple of four: short and long ones, results that end in a
+                                   # partial 16-byte piece, a period of two and of three values
+                                   (7, 7 * 1001), (7 * 1001, 7), (3, 3 * 70000), (2, 2 * 5001), (10001, 10001 * 50),
+                                   (5, 15), (3, 6), (8193, 8193 * 9)])
 def test_binary_ops_bit_exact(oracle, hip, op, xl, yl):
     r = rng(xl * 7919 + yl)
     x = r.standard_normal(xl).astype(np.float32)

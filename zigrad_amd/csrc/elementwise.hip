@@ -211,6 +211,56 @@ __global__ __launch_bounds__(kBlock) void bin_modulo_kernel(float* out, const fl
     }
 }
 
+// The same for a long operand and a result on 16-byte boundaries, whatever the period: the long operand is walked as one
+// flat array of 16-byte pieces, four per thread in flight; a workgroup divides once (where its chunk starts in the short
+// operand), a piece finds its place from there and its four values step through the short operand, wrapping at its
+// end.  ([8192, 32001] + [32001]: 701 us with a 64-bit remainder per value, 37 % of 8 TB/s.)
+constexpr int kPeriodU = 4;
+template <class B, bool SHORT_LHS>
+__global__ __launch_bounds__(kBlock) void bin_period_kernel(float* out, const float* lng, const float* sht, size_t n,
+                                                             size_t p) {
+    constexpr size_t kChunk = (size_t)kBlock * kPeriodU;
+    const float4* l4 = reinterpret_cast<const float4*>(lng);
+    float4* o4 = reinterpret_cast<float4*>(out);
+    const size_t n4 = n >> 2;
+    for (size_t c0 = (size_t)blockIdx.x * kChunk; c0 < n4; c0 += (size_t)gridDim.x * kChunk) {
+        const size_t e0 = c0 << 2, cq = e0 / p, cs = e0 - cq * p;
+        float4 v[kPeriodU];
+        float sv[kPeriodU][4];
+#pragma unroll
+        for (int u = 0; u < kPeriodU; u++) {
+            const size_t j = c0 + threadIdx.x + (size_t)u * kBlock;
+            if (j < n4) {
+                v[u] = nt_load(l4 + j);
+                size_t q, s;
+                flat_divmod(0, cs, 4 * (threadIdx.x + (size_t)u * kBlock), p, q, s);
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    sv[u][k] = sht[s];
+                    if (++s == p) s = 0;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kPeriodU; u++) {
+            const size_t j = c0 + threadIdx.x + (size_t)u * kBlock;
+            if (j < n4) {
+                float4 o;
+                o.x = SHORT_LHS ? B::f(sv[u][0], v[u].x) : B::f(v[u].x, sv[u][0]);
+                o.y = SHORT_LHS ? B::f(sv[u][1], v[u].y) : B::f(v[u].y, sv[u][1]);
+                o.z = SHORT_LHS ? B::f(sv[u][2], v[u].z) : B::f(v[u].z, sv[u][2]);
+                o.w = SHORT_LHS ? B::f(sv[u][3], v[u].w) : B::f(v[u].w, sv[u][3]);
+                nt_store(o, o4 + j);
+            }
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const size_t i = (n4 << 2) + threadIdx.x;
+        const float s = sht[i % p];
+        out[i] = SHORT_LHS ? B::f(s, lng[i]) : B::f(lng[i], s);
+    }
+}
+
 __global__ void broadcast_modulo_kernel(float* y, const float* x, size_t xl, size_t yl, float alpha, float beta) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -252,7 +302,10 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
     const bool short_lhs = xl < yl;
     const float* lng = short_lhs ? y : x;
     const float* sht = short_lhs ? x : y;
-    if (mn % 4 == 0 && aligned16(lng) && aligned16(sht) && aligned16(z)) {
+    // rows of whole 16-byte pieces: a workgroup per group of rows keeps its pieces of the short operand in registers.  Not
+    // for rows of fewer than 64 values (a workgroup then has a few lanes at work: [1048576, 4 ... 32] took 66 us
+    // whatever the row length, 6 to 47 us as a flat walk) nor from 256 MiB up, where the flat walk is 4 to 14 % faster
+    if (mn % 4 == 0 && mn >= 64 && zl < ((size_t)1 << 26) && aligned16(lng) && aligned16(sht) && aligned16(z)) {
         size_t p4 = mn / 4, rows = mx / mn;
         unsigned gx = (unsigned)ceil_div_sz(p4, kRbX);
         // a workgroup per group of rows, up to the grid's limit (65536 rows of 4096: 466 -> 370 us against 16 workgroups
@@ -265,6 +318,15 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
             hipLaunchKernelGGL((bin_rowbcast_kernel<B, true>), grid, block, 0, ctx->stream, z, lng, sht, rows, p4);
         else
             hipLaunchKernelGGL((bin_rowbcast_kernel<B, false>), grid, block, 0, ctx->stream, z, lng, sht, rows, p4);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
+    if (aligned16(lng) && aligned16(z) && zl >= 4) {
+        int grid = map_grid(ctx, zl >> 2, kBlock * kPeriodU);
+        if (short_lhs)
+            hipLaunchKernelGGL((bin_period_kernel<B, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, lng, sht, zl, mn);
+        else
+            hipLaunchKernelGGL((bin_period_kernel<B, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, lng, sht, zl, mn);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }

@@ -15,6 +15,24 @@ __device__ __forceinline__ void nt_store(float4 v, float4* p) {
     __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t*>(p));
 }
 
+// Quotient and remainder by p of (cq * p + cs + add), for cs < p and add < 8192, without a 64-bit division: a flat walk
+// over a matrix divides once per chunk and places each of its pieces with this.
+__device__ __forceinline__ void flat_divmod(size_t cq, size_t cs, size_t add, size_t p, size_t& q, size_t& s) {
+    size_t off = cs + add;
+    if (p >= 8192) {
+        q = cq;
+        if (off >= p) {
+            off -= p;
+            q++;
+        }
+        s = off;
+    } else {
+        const uint32_t qq = (uint32_t)off / (uint32_t)p;
+        q = cq + qq;
+        s = off - (size_t)qq * p;
+    }
+}
+
 
 // ---- accumulator policies -------------------------------------------------------------------
 // combine(a, b) must give the same result for (a, b) and (b, a): the butterfly shuffles below apply

@@ -338,7 +338,10 @@ def test_scatter_add_heavy_hitter_is_deterministic(hip):
     np.testing.assert_array_equal(outs[0], want)
 
 
-@pytest.mark.parametrize("rows,stride,n_idx", [(100, 16, 37), (2708, 7, 5000), (50, 300, 200), (10, 1, 10)])
+@pytest.mark.parametrize("rows,stride,n_idx", [(100, 16, 37), (2708, 7, 5000), (50, 300, 200), (10, 1, 10),
+                                               # long rows, cut into spans of columns: whole spans, a partial last one,
+                                               # a row length that is no multiple of four
+                                               (9, 8192, 20), (7, 9220, 11), (5, 70000, 8), (6, 8195, 9)])
 def test_index_select(oracle, hip, rows, stride, n_idx):
     r = rng(rows + stride)
     src = r.standard_normal(rows * stride).astype(np.float32)

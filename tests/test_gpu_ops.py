@@ -311,6 +311,13 @@ def test_broadcast_op(oracle, hip):
         y = r.standard_normal(n).astype(np.float32)
         a, b = both(oracle, hip, "broadcast", {"x": x, "y": y, "alpha": 0.5, "beta": 2.0}, ["y"])
         np.testing.assert_array_equal(a["y"], b["y"])
+    # short operands of any length against results that end in a partial 16-byte piece or not
+    for xl, reps in ((7, 1001), (3, 70000), (2, 5001), (10001, 50), (5, 3), (16, 4096), (1, 4097)):
+        x = r.standard_normal(xl).astype(np.float32)
+        y = r.standard_normal(xl * reps).astype(np.float32)
+        for alpha, beta in ((0.5, 2.0), (1.0, 0.0)):
+            a, b = both(oracle, hip, "broadcast", {"x": x, "y": y, "alpha": alpha, "beta": beta}, ["y"])
+            np.testing.assert_array_equal(a["y"], b["y"])
 
 
 # ----------------------------------------------------------------------------------------------

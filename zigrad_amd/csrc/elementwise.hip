@@ -217,7 +217,17 @@ __global__ __launch_bounds__(kBlock) void bin_modulo_kernel(float* out, const fl
 // end.  ([8192, 32001] + [32001]: 701 us with a 64-bit remainder per value, 37 % of 8 TB/s.)
 constexpr int kPeriodU = 4;
 template <class B, bool SHORT_LHS>
-__global__ __launch_bounds__(kBlock) void bin_period_kernel(float* out, const float* lng, const float* sht, size_t n,
+struct BinPeriod {
+    __device__ __forceinline__ float operator()(float l, float s) const { return SHORT_LHS ? B::f(s, l) : B::f(l, s); }
+};
+struct AxpbyPeriod {  // the broadcast op: alpha * short + beta * long
+    float alpha, beta;
+    __device__ __forceinline__ float operator()(float l, float s) const {
+        return __fadd_rn(__fmul_rn(alpha, s), __fmul_rn(beta, l));
+    }
+};
+template <class F>
+__global__ __launch_bounds__(kBlock) void bin_period_kernel(F f, float* out, const float* lng, const float* sht, size_t n,
                                                              size_t p) {
     constexpr size_t kChunk = (size_t)kBlock * kPeriodU;
     const float4* l4 = reinterpret_cast<const float4*>(lng);
@@ -246,18 +256,17 @@ __global__ __launch_bounds__(kBlock) void bin_period_kernel(float* out, const fl
             const size_t j = c0 + threadIdx.x + (size_t)u * kBlock;
             if (j < n4) {
                 float4 o;
-                o.x = SHORT_LHS ? B::f(sv[u][0], v[u].x) : B::f(v[u].x, sv[u][0]);
-                o.y = SHORT_LHS ? B::f(sv[u][1], v[u].y) : B::f(v[u].y, sv[u][1]);
-                o.z = SHORT_LHS ? B::f(sv[u][2], v[u].z) : B::f(v[u].z, sv[u][2]);
-                o.w = SHORT_LHS ? B::f(sv[u][3], v[u].w) : B::f(v[u].w, sv[u][3]);
+                o.x = f(v[u].x, sv[u][0]);
+                o.y = f(v[u].y, sv[u][1]);
+                o.z = f(v[u].z, sv[u][2]);
+                o.w = f(v[u].w, sv[u][3]);
                 nt_store(o, o4 + j);
             }
         }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const size_t i = (n4 << 2) + threadIdx.x;
-        const float s = sht[i % p];
-        out[i] = SHORT_LHS ? B::f(s, lng[i]) : B::f(lng[i], s);
+        out[i] = f(lng[i], sht[i % p]);
     }
 }
 
@@ -324,9 +333,11 @@ static int binary_op(zg_hip_ctx* ctx, const char* name, const float* x, size_t x
     if (aligned16(lng) && aligned16(z) && zl >= 4) {
         int grid = map_grid(ctx, zl >> 2, kBlock * kPeriodU);
         if (short_lhs)
-            hipLaunchKernelGGL((bin_period_kernel<B, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, lng, sht, zl, mn);
+            hipLaunchKernelGGL((bin_period_kernel<BinPeriod<B, true>>), dim3(grid), dim3(kBlock), 0, ctx->stream,
+                               BinPeriod<B, true>{}, z, lng, sht, zl, mn);
         else
-            hipLaunchKernelGGL((bin_period_kernel<B, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, z, lng, sht, zl, mn);
+            hipLaunchKernelGGL((bin_period_kernel<BinPeriod<B, false>>), dim3(grid), dim3(kBlock), 0, ctx->stream,
+                               BinPeriod<B, false>{}, z, lng, sht, zl, mn);
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
@@ -693,6 +704,13 @@ ZG_API int zg_hip_broadcast(zg_hip_ctx* ctx, const float* x, size_t xl, float* y
         int rc = launch_map<ScaledCopy, 2>(ctx, y, x, y, nullptr, yl, alpha, beta);
         if (rc) return rc;
         return launch_map<ScaledCopy, 2>(ctx, y, x, y, nullptr, yl, alpha, beta);
+    }
+    if (aligned16(y) && yl >= 4) {  // the flat walk in 16-byte pieces of the binary ops (33554432 values from 16: 60 -> 48 us)
+        int grid = map_grid(ctx, yl >> 2, kBlock * kPeriodU);
+        hipLaunchKernelGGL((bin_period_kernel<AxpbyPeriod>), dim3(grid), dim3(kBlock), 0, ctx->stream,
+                           AxpbyPeriod{alpha, beta}, y, y, x, yl, xl);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
     }
     int grid = map_grid(ctx, yl, kBlock);
     hipLaunchKernelGGL(broadcast_modulo_kernel, dim3(grid), dim3(kBlock), 0, ctx->stream, y, x, xl, yl, alpha, beta);

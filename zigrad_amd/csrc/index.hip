@@ -1286,14 +1286,16 @@ __global__ __launch_bounds__(kScatterSmallMax) void scatter_add_small_kernel(con
 template <int G>
 __global__ __launch_bounds__(256) void row_scatter_apply_kernel(const float* src, const uint32_t* row_ptr,
                                                                  const uint32_t* perm, float* dst, size_t nb,
-                                                                 size_t stride) {
+                                                                 size_t stride, size_t span) {
     const size_t b = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     if (b >= nb) return;
     const int lane = threadIdx.x % G;
     const uint32_t s = row_ptr[b], e = row_ptr[b + 1];
     if (s == e) return;
     if (e - s > kLongBucket) return;  // long_bucket_kernel's, a wave per column
-    for (size_t j = lane; j < stride; j += G) {
+    // long rows are cut into spans of columns (blockIdx.y): 32 rows of a million values on 32 lane groups took 15 ms
+    const size_t j_begin = (size_t)blockIdx.y * span, j_end = j_begin + span < stride ? j_begin + span : stride;
+    for (size_t j = j_begin + lane; j < j_end; j += G) {
         float acc = dst[b * stride + j];
         // eight entries' loads at a time (positions, then row elements: two round trips), the additions still in input
         // order (one entry at a time, a destination of ten thousand entries took 440 ns an entry)
@@ -1685,9 +1687,11 @@ __global__ void index_select_fwd_kernel(const float* src, size_t src_len, const 
 // group in flight (two or eight measured no better: a gather of random 1 KiB rows runs at the rate DRAM opens pages) (their indices are loaded first, then their pieces), one piece per lane and trip along the row.
 template <int G>
 __global__ __launch_bounds__(256) void index_select_fwd_vec4_kernel(const float4* src, size_t src_rows, const uint64_t* indices,
-                                                                     size_t n_idx, size_t s4, float4* dst) {
+                                                                     size_t n_idx, size_t s4, float4* dst, size_t span) {
     constexpr int kRows = 4;
     const int lane = threadIdx.x % G;
+    // long rows are cut into spans of pieces (blockIdx.y), so that a few rows of a million values still fill the machine
+    const size_t j_begin = (size_t)blockIdx.y * span, j_end = j_begin + span < s4 ? j_begin + span : s4;
     const size_t slot = (size_t)blockIdx.x * (256 / G) + threadIdx.x / G, n_slots = (size_t)gridDim.x * (256 / G);
     for (size_t d0 = slot; d0 < n_idx; d0 += kRows * n_slots) {
         uint64_t r[kRows];
@@ -1696,7 +1700,7 @@ __global__ __launch_bounds__(256) void index_select_fwd_vec4_kernel(const float4
             const size_t d = d0 + (size_t)u * n_slots;
             r[u] = d < n_idx ? indices[d] : ~(uint64_t)0;
         }
-        for (size_t j = lane; j < s4; j += G) {
+        for (size_t j = j_begin + lane; j < j_end; j += G) {
             float4 v[kRows];
 #pragma unroll
             for (int u = 0; u < kRows; u++)
@@ -1871,9 +1875,13 @@ ZG_API int zg_hip_index_select_fwd(zg_hip_ctx* ctx, const float* src, size_t src
         // a workgroup per 16 to 64 rows at any count (a million rows of 1 KiB: 355 -> 339 us against a grid capped at 16
         // workgroups per compute unit)
         if (vblocks > 0x7fffffffull) vblocks = 0x7fffffffull;
-        ZG_G_DISPATCH(g, hipLaunchKernelGGL((index_select_fwd_vec4_kernel<G>), dim3((unsigned)vblocks), dim3(256), 0,
-                                            ctx->stream, (const float4*)src, src_len / stride, indices, n_idx, s4,
-                                            (float4*)dst));
+        // rows of more than 32 KiB in spans of 16 KiB (1024 rows of 32768 values: 18 % of 8 TB/s as whole rows)
+        const size_t span = s4 > 2048 ? 1024 : s4;
+        const size_t gy = ceil_div_sz(s4, span);
+        ZG_REQUIRE(gy <= 65535, "index_select_fwd: rows of %zu values are too long", stride);
+        ZG_G_DISPATCH(g, hipLaunchKernelGGL((index_select_fwd_vec4_kernel<G>), dim3((unsigned)vblocks, (unsigned)gy), dim3(256),
+                                            0, ctx->stream, (const float4*)src, src_len / stride, indices, n_idx, s4,
+                                            (float4*)dst, span));
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
@@ -1905,8 +1913,11 @@ ZG_API int zg_hip_index_select_bwd(zg_hip_ctx* ctx, const float* y_grad, const u
     const Plan& pl = pr.plan;
     const int g = group_for(stride);
     const unsigned grid = (unsigned)ceil_div_sz(nb, 256 / g);
-    ZG_G_DISPATCH(g, hipLaunchKernelGGL((row_scatter_apply_kernel<G>), dim3(grid), dim3(256), 0, ctx->stream, y_grad,
-                                        pl.row_ptr, pl.perm, x_grad, nb, stride));
+    const size_t span = stride > 2048 ? 1024 : stride;
+    const size_t gy = ceil_div_sz(stride, span);
+    ZG_REQUIRE(gy <= 65535, "index_select_bwd: rows of %zu values are too long", stride);
+    ZG_G_DISPATCH(g, hipLaunchKernelGGL((row_scatter_apply_kernel<G>), dim3(grid, (unsigned)gy), dim3(256), 0, ctx->stream,
+                                        y_grad, pl.row_ptr, pl.perm, x_grad, nb, stride, span));
     ZG_LAUNCH_CHECK();
     // rows that more than kLongBucket entries select: a wave per column, 64 entries' loads in flight (a row selected
     // ten thousand times: 4.6 ms a thread group walking its entries one by one, 0.2 ms this way)

@@ -502,87 +502,113 @@ __global__ __launch_bounds__(kLongRowThreads) void softmax_long_rows_kernel(cons
 // columns, a whole wave beyond) hold the row in registers (at most 4 float4 per lane), so the logits are read once and
 // the row's reductions stay inside the wave: three passes of the matrix instead of four, no LDS, no barrier.
 constexpr int kWaveRowVec = 4;
-template <int TPR, int MODE, int GRAD = 0>
+// RPG rows per lane group (1, 2 or 4): a row of at most TPR * 4 / RPG pieces leaves a lane's other registers to further
+// rows, RPG of them loaded before the first is used.  With one piece per lane a workgroup of 16-lane groups moved 4 KiB
+// per trip and the softmax of [4194304, 64] ran at 57 % of 8 TB/s.  The arithmetic of a row does not depend on RPG: the
+// pieces a row does not have added exp(-inf) = 0 to its sum.
+template <int TPR, int MODE, int GRAD = 0, int RPG = 1>
 __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* logits, const float* target, float* probs,
                                                                     float* row_loss, size_t rows, size_t cols,
                                                                     float* grad = nullptr, float denom = 1.f) {
+    constexpr int PPL = kWaveRowVec / RPG;  // pieces per lane and row
+    constexpr int kGroups = kBlock / TPR;
     const int lane = threadIdx.x & (TPR - 1);
-    const size_t row = (size_t)blockIdx.x * (kBlock / TPR) + threadIdx.x / TPR;
-    if (row >= rows) return;  // the lanes of a row leave together: no barrier follows, and shuffles stay inside the row
+    const size_t row0 = (size_t)blockIdx.x * (kGroups * RPG) + threadIdx.x / TPR;  // this group's rows: row0 + r * kGroups
+    if (row0 >= rows) return;  // the lanes of a group leave together: no barrier follows, and shuffles stay inside it
     const size_t c4 = cols >> 2;
-    const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
-    const float4* t4 = reinterpret_cast<const float4*>(MODE ? target + row * cols : logits);
-    float4* p4 = reinterpret_cast<float4*>(probs + row * cols);
-    float4* g4 = reinterpret_cast<float4*>(GRAD ? grad + row * cols : probs);
     const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     float4 v[kWaveRowVec], t[kWaveRowVec];
 #pragma unroll
-    for (int u = 0; u < kWaveRowVec; u++) {
-        const size_t j = lane + (size_t)u * TPR;
-        v[u] = (j < c4) ? nt_load(x4 + j) : ninf;
+    for (int r = 0; r < RPG; r++) {
+        const size_t row = row0 + (size_t)r * kGroups;
+        const float4* x4 = reinterpret_cast<const float4*>(logits + row * cols);
+#pragma unroll
+        for (int u = 0; u < PPL; u++) {
+            const size_t j = lane + (size_t)u * TPR;
+            v[r * PPL + u] = (row < rows && j < c4) ? nt_load(x4 + j) : ninf;
+        }
     }
     if (MODE) {
 #pragma unroll
-        for (int u = 0; u < kWaveRowVec; u++) {
-            const size_t j = lane + (size_t)u * TPR;
-            t[u] = (j < c4) ? nt_load(t4 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-    }
-    OnlineAccT acc = OnlineAcc::init();
-    float mx = -INFINITY;
+        for (int r = 0; r < RPG; r++) {
+            const size_t row = row0 + (size_t)r * kGroups;
+            const float4* t4 = reinterpret_cast<const float4*>(target + row * cols);
 #pragma unroll
-    for (int u = 0; u < kWaveRowVec; u++) mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
-    if (mx != -INFINITY) {
-        float sum = 0.f;
-#pragma unroll
-        for (int u = 0; u < kWaveRowVec; u++)
-            sum += fexp(v[u].x - mx) + fexp(v[u].y - mx) + fexp(v[u].z - mx) + fexp(v[u].w - mx);
-        acc.m = mx;
-        acc.s = sum;
-    }
-    acc = group_reduce<OnlineAcc, TPR>(acc);
-    const float l = __fadd_rn(acc.m, logf(acc.s));
-    float part = 0.f;
-#pragma unroll
-    for (int u = 0; u < kWaveRowVec; u++) {
-        const size_t j = lane + (size_t)u * TPR;
-        if (j < c4) {
-            float4 p;
-            p.x = fexp(__fsub_rn(v[u].x, l));
-            p.y = fexp(__fsub_rn(v[u].y, l));
-            p.z = fexp(__fsub_rn(v[u].z, l));
-            p.w = fexp(__fsub_rn(v[u].w, l));
-            nt_store(p, p4 + j);
-            if (MODE) {
-                const float pv[4] = {p.x, p.y, p.z, p.w}, tv[4] = {t[u].x, t[u].y, t[u].z, t[u].w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    if (tv[e] != 0.f) {
-                        const float safe = fminf(fmaxf(pv[e], 1e-7f), 1.0f - 1e-7f);
-                        part = __fsub_rn(part, __fmul_rn(tv[e], logf(safe)));
-                    }
-                }
-                if (GRAD) {
-                    float4 d;
-                    d.x = __fdiv_rn(__fsub_rn(p.x, t[u].x), denom);
-                    d.y = __fdiv_rn(__fsub_rn(p.y, t[u].y), denom);
-                    d.z = __fdiv_rn(__fsub_rn(p.z, t[u].z), denom);
-                    d.w = __fdiv_rn(__fsub_rn(p.w, t[u].w), denom);
-                    if (GRAD == 2) {
-                        const float4 g = nt_load(g4 + j);
-                        d.x = __fadd_rn(g.x, d.x);
-                        d.y = __fadd_rn(g.y, d.y);
-                        d.z = __fadd_rn(g.z, d.z);
-                        d.w = __fadd_rn(g.w, d.w);
-                    }
-                    nt_store(d, g4 + j);
-                }
+            for (int u = 0; u < PPL; u++) {
+                const size_t j = lane + (size_t)u * TPR;
+                t[r * PPL + u] = (row < rows && j < c4) ? nt_load(t4 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }
     }
-    if (MODE) {
-        part = group_reduce<SumAcc, TPR>(part);
-        if (lane == 0) row_loss[row] = part;
+#pragma unroll
+    for (int r = 0; r < RPG; r++) {
+        const size_t row = row0 + (size_t)r * kGroups;
+        const bool live = row < rows;  // the same for every lane of the group
+        float4* p4 = reinterpret_cast<float4*>(probs + row * cols);
+        float4* g4 = reinterpret_cast<float4*>(GRAD ? grad + row * cols : probs);
+        OnlineAccT acc = OnlineAcc::init();
+        float mx = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < PPL; u++) {
+            const float4 a = v[r * PPL + u];
+            mx = fmaxf(mx, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)));
+        }
+        if (mx != -INFINITY) {
+            float sum = 0.f;
+#pragma unroll
+            for (int u = 0; u < PPL; u++) {
+                const float4 a = v[r * PPL + u];
+                sum += fexp(a.x - mx) + fexp(a.y - mx) + fexp(a.z - mx) + fexp(a.w - mx);
+            }
+            acc.m = mx;
+            acc.s = sum;
+        }
+        acc = group_reduce<OnlineAcc, TPR>(acc);
+        const float l = __fadd_rn(acc.m, logf(acc.s));
+        float part = 0.f;
+#pragma unroll
+        for (int u = 0; u < PPL; u++) {
+            const size_t j = lane + (size_t)u * TPR;
+            if (live && j < c4) {
+                const float4 a = v[r * PPL + u];
+                float4 p;
+                p.x = fexp(__fsub_rn(a.x, l));
+                p.y = fexp(__fsub_rn(a.y, l));
+                p.z = fexp(__fsub_rn(a.z, l));
+                p.w = fexp(__fsub_rn(a.w, l));
+                nt_store(p, p4 + j);
+                if (MODE) {
+                    const float4 tt = t[r * PPL + u];
+                    const float pv[4] = {p.x, p.y, p.z, p.w}, tv[4] = {tt.x, tt.y, tt.z, tt.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (tv[e] != 0.f) {
+                            const float safe = fminf(fmaxf(pv[e], 1e-7f), 1.0f - 1e-7f);
+                            part = __fsub_rn(part, __fmul_rn(tv[e], logf(safe)));
+                        }
+                    }
+                    if (GRAD) {
+                        float4 dd;
+                        dd.x = __fdiv_rn(__fsub_rn(p.x, tt.x), denom);
+                        dd.y = __fdiv_rn(__fsub_rn(p.y, tt.y), denom);
+                        dd.z = __fdiv_rn(__fsub_rn(p.z, tt.z), denom);
+                        dd.w = __fdiv_rn(__fsub_rn(p.w, tt.w), denom);
+                        if (GRAD == 2) {
+                            const float4 g = nt_load(g4 + j);
+                            dd.x = __fadd_rn(g.x, dd.x);
+                            dd.y = __fadd_rn(g.y, dd.y);
+                            dd.z = __fadd_rn(g.z, dd.z);
+                            dd.w = __fadd_rn(g.w, dd.w);
+                        }
+                        nt_store(dd, g4 + j);
+                    }
+                }
+            }
+        }
+        if (MODE) {
+            part = group_reduce<SumAcc, TPR>(part);
+            if (live && lane == 0) row_loss[row] = part;
+        }
     }
 }
 
@@ -598,17 +624,20 @@ static bool long_row_ok(const float* a, const float* b, const float* c, size_t r
 }
 
 // Launches softmax_wave_rows_kernel<.., MODE, GRAD> with the lanes per row that fit the row length (wave_row_ok holds).
+#define ZG_WAVE_ROWS_AS(TPR_, RPG_, MODE, GRAD, ...)                                                                  \
+    hipLaunchKernelGGL((softmax_wave_rows_kernel<TPR_, MODE, GRAD, RPG_>),                                             \
+                       dim3((unsigned)ceil_div_sz(rows, (size_t)(kBlock / TPR_) * RPG_)), dim3(kBlock), 0, ctx->stream, \
+                       __VA_ARGS__)
 #define ZG_WAVE_ROWS(MODE, GRAD, ...)                                                                                  \
-    do {                                                                                                               \
-        if (cols <= 32) /* the lanes per row of pick_tpr, which the one-workgroup kernel for small batches follows */   \
-            hipLaunchKernelGGL((softmax_wave_rows_kernel<4, MODE, GRAD>), dim3((unsigned)ceil_div_sz(rows, kBlock / 4)), \
-                               dim3(kBlock), 0, ctx->stream, __VA_ARGS__);                                             \
-        else if (cols <= 16 * kWaveRowVec * 4)                                                                         \
-            hipLaunchKernelGGL((softmax_wave_rows_kernel<16, MODE, GRAD>), dim3((unsigned)ceil_div_sz(rows, kBlock / 16)), \
-                               dim3(kBlock), 0, ctx->stream, __VA_ARGS__);                                             \
-        else                                                                                                           \
-            hipLaunchKernelGGL((softmax_wave_rows_kernel<kWave, MODE, GRAD>),                                          \
-                               dim3((unsigned)ceil_div_sz(rows, kBlock / kWave)), dim3(kBlock), 0, ctx->stream, __VA_ARGS__); \
+    do { /* the lanes per row of pick_tpr, which the one-workgroup kernel for small batches follows; rows that leave */ \
+        /* registers free share a lane group two or four at a time */                                                  \
+        if (cols <= 16) ZG_WAVE_ROWS_AS(4, 4, MODE, GRAD, __VA_ARGS__);                                                \
+        else if (cols <= 32) ZG_WAVE_ROWS_AS(4, 2, MODE, GRAD, __VA_ARGS__);                                           \
+        else if (cols <= 64) ZG_WAVE_ROWS_AS(16, 4, MODE, GRAD, __VA_ARGS__);                                          \
+        else if (cols <= 128) ZG_WAVE_ROWS_AS(16, 2, MODE, GRAD, __VA_ARGS__);                                         \
+        else if (cols <= 16 * kWaveRowVec * 4) ZG_WAVE_ROWS_AS(16, 1, MODE, GRAD, __VA_ARGS__);                        \
+        else if (cols <= 512) ZG_WAVE_ROWS_AS(kWave, 2, MODE, GRAD, __VA_ARGS__);                                      \
+        else ZG_WAVE_ROWS_AS(kWave, 1, MODE, GRAD, __VA_ARGS__);                                                       \
     } while (0)
 
 // Launches softmax_long_rows_kernel<.., MODE, GRAD> in the shape that fits the row length (long_row_ok holds).

@@ -221,7 +221,10 @@ AXIS_SHAPES = [([64, 10], 1), ([64, 10], 0), ([64, 2], 1), ([2708, 16], 0), ([10
                # tall matrices of one column group: 128 chunks of rows from 64 MiB, 256 from 256 MiB
                ([262149, 64], 0), ([65541, 256], 0), ([1048581, 68], 0),
                # rows that start off a 16-byte boundary and are read in 16-byte pieces between a head and a tail
-               ([600, 2051], 1), ([50, 4099], 1), ([9, 33001], 1), ([700, 513], 1), ([5, 300001], 1), ([2, 1000003], 1)]
+               ([600, 2051], 1), ([50, 4099], 1), ([9, 33001], 1), ([700, 513], 1), ([5, 300001], 1), ([2, 1000003], 1),
+               # short rows on one, two, four and eight lanes, with and without heads and tails
+               ([5000, 1], 1), ([5000, 3], 1), ([3000, 9], 1), ([3000, 11], 1), ([3000, 12], 1), ([2000, 17], 1),
+               ([2000, 30], 1), ([1500, 35], 1), ([1500, 61], 1), ([1000, 70], 1), ([1000, 130], 1), ([700, 255], 1)]
 
 
 @pytest.mark.parametrize("shape,dim", AXIS_SHAPES)

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
     if (row < rows) {
         const float* xr = x + row * cols;
         // A row starts wherever row * cols puts it: its values before the first 16-byte boundary and after the last whole
-        // 16-byte piece (at most three each) go to the first lanes, the pieces between are read 16 bytes at a time
+        // 16-byte piece (at most three each) are dealt to the lanes one by one, the pieces between are read 16 bytes at a time
         // (sums over the rows of [8192, 32001] value by value: 47 % of 8 TB/s against 84 % for 32000 columns).  Rows of
         // fewer than eight pieces per lane that are not whole pieces stay value by value.
         size_t h = (size_t)((0 - (reinterpret_cast<uintptr_t>(xr) >> 2)) & 3);
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
             const float4* x4 = reinterpret_cast<const float4*>(xr + h);
             const size_t c4 = (cols - h) >> 2;
             const uint32_t h32 = (uint32_t)h;
-            if ((size_t)lane < h) acc = P::combine(acc, A::term(xr[lane], (uint32_t)lane));
+            for (size_t i = lane; i < h; i += TPR) acc = P::combine(acc, A::term(xr[i], (uint32_t)i));
             // whole trips of four loads per lane, then one partial trip whose loads are in flight together as well, the
             // ones past the row's end left out: the trip count is the same for every lane, so a row of 1000 columns takes
             // one memory round trip like a row of 1024 (lanes that finish one by one cost a quarter more)
@@ -127,8 +127,7 @@ __global__ __launch_bounds__(kBlock) void row_reduce_kernel(const float* x, type
                     }
                 }
             }
-            const size_t tail = h + (c4 << 2) + (size_t)lane;
-            if (tail < cols) acc = P::combine(acc, A::term(xr[tail], (uint32_t)tail));
+            for (size_t i = h + (c4 << 2) + (size_t)lane; i < cols; i += TPR) acc = P::combine(acc, A::term(xr[i], (uint32_t)i));
         } else {
             for (size_t j = lane; j < cols; j += TPR) acc = P::combine(acc, A::term(xr[j], (uint32_t)j));
         }
@@ -287,7 +286,13 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
 #define ZG_ROW(TPR)                                                                                          \
     hipLaunchKernelGGL((row_reduce_kernel<A, TPR>), dim3((unsigned)ceil_div_sz(rows, kBlock / TPR)), dim3(kBlock), 0, \
                        ctx->stream, x, y, rows, cols, alpha, beta)
-        if (cols <= 32) ZG_ROW(4);
+        // lanes per row so that a lane has 8 to 16 values of a short row: with four lanes on a row of 4 to 12 values
+        // and sixteen on one of 64 to 128 most lanes had one load or none (sums over the rows of [8388608, 4]: 70 -> 27 us,
+        // [2097152, 16]: 25.6 -> 21.2 us, [524288, 64]: 25.1 -> 20.8 us, 82 to 86 % of 8 TB/s)
+        if (cols < 16) ZG_ROW(1);
+        else if (cols < 32) ZG_ROW(2);
+        else if (cols < 64) ZG_ROW(4);
+        else if (cols < 256) ZG_ROW(8);
         else if (cols <= 256) ZG_ROW(16);
         else if (cols <= 16384 || rows >= (size_t)ctx->n_cu * 8) ZG_ROW(64);
         else ZG_ROW(256);

@@ -61,7 +61,6 @@ __device__ __forceinline__ bool row_in_pieces(size_t h, size_t cols) {
 }
 template <int TPR, bool KEEP = false>
 __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, int lane) {
-    static_assert(TPR >= 4, "the first lanes take the head and the tail of a row");
     OnlineAccT acc = OnlineAcc::init();
     const size_t h = row_head(xr, cols);
     auto load = [](const float4* p) { return KEEP ? *p : nt_load(p); };
@@ -69,7 +68,8 @@ __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, i
         for (size_t j = lane; j < cols; j += TPR)
             if (xr[j] != -INFINITY) online_push(acc, xr[j]);
     } else {
-        if ((size_t)lane < h && xr[lane] != -INFINITY) online_push(acc, xr[lane]);
+        for (size_t i = lane; i < h; i += TPR)
+            if (xr[i] != -INFINITY) online_push(acc, xr[i]);
         const float4* x4 = reinterpret_cast<const float4*>(xr + h);
         const size_t c4 = (cols - h) >> 2;
         // four 16-byte loads in flight per thread; past the end of the row they are replaced by -inf, which adds
@@ -95,8 +95,8 @@ __device__ __forceinline__ OnlineAccT row_online(const float* xr, size_t cols, i
             s += fexp(v3.x - acc.m) + fexp(v3.y - acc.m) + fexp(v3.z - acc.m) + fexp(v3.w - acc.m);
             acc.s += s;
         }
-        const size_t tail = h + (c4 << 2) + (size_t)lane;
-        if (tail < cols && xr[tail] != -INFINITY) online_push(acc, xr[tail]);
+        for (size_t i = h + (c4 << 2) + (size_t)lane; i < cols; i += TPR)
+            if (xr[i] != -INFINITY) online_push(acc, xr[i]);
     }
     return acc;
 }
@@ -137,7 +137,7 @@ __device__ __forceinline__ float row_probs(const float* xr, const float* tr, flo
         return part;
     }
     const size_t h = row_head(xr, cols);
-    if ((size_t)lane < h) scalar(lane);
+    for (size_t i = lane; i < h; i += TPR) scalar(i);
     const size_t c4 = (cols - h) >> 2;
     const float4* x4 = reinterpret_cast<const float4*>(xr + h);
     const float4* t4 = reinterpret_cast<const float4*>(MODE ? tr + h : xr + h);
@@ -170,8 +170,7 @@ __device__ __forceinline__ float row_probs(const float* xr, const float* tr, flo
             }
         }
     }
-    const size_t tail = h + (c4 << 2) + (size_t)lane;
-    if (tail < cols) scalar(tail);
+    for (size_t i = h + (c4 << 2) + (size_t)lane; i < cols; i += TPR) scalar(i);
     return part;
 }
 
@@ -782,7 +781,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
         auto dot4 = [](float4 a, float4 b) {
             return __fadd_rn(__fadd_rn(__fmul_rn(a.x, b.x), __fmul_rn(a.y, b.y)), __fadd_rn(__fmul_rn(a.z, b.z), __fmul_rn(a.w, b.w)));
         };
-        if ((size_t)lane < h) part = __fmul_rn(yr[lane], gr[lane]);
+        for (size_t i = lane; i < h; i += TPR) part = __fadd_rn(part, __fmul_rn(yr[i], gr[i]));
         const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
         float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
         for (size_t j = lane; j < c4; j += 4 * TPR) {
@@ -798,7 +797,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
             s3 = __fadd_rn(s3, dot4(a3, b3));
         }
         part = __fadd_rn(part, __fadd_rn(__fadd_rn(s0, s1), __fadd_rn(s2, s3)));
-        if (tail < cols) part = __fadd_rn(part, __fmul_rn(yr[tail], gr[tail]));
+        for (size_t i = tail; i < cols; i += TPR) part = __fadd_rn(part, __fmul_rn(yr[i], gr[i]));
     } else if (live) {
         for (size_t j = lane; j < cols; j += TPR) part = __fadd_rn(part, __fmul_rn(yr[j], gr[j]));
     }
@@ -812,7 +811,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
         part = bcast;
     }
     if (pieces) {
-        if ((size_t)lane < h) xr[lane] = __fadd_rn(xr[lane], __fmul_rn(yr[lane], __fsub_rn(gr[lane], part)));
+        for (size_t i = lane; i < h; i += TPR) xr[i] = __fadd_rn(xr[i], __fmul_rn(yr[i], __fsub_rn(gr[i], part)));
         for (size_t j0 = lane; j0 < c4; j0 += 2 * TPR) {
             const size_t j1 = j0 + TPR;
             const bool in1 = j1 < c4;
@@ -834,7 +833,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
             nt_store(upd(a0, b0, x0), x4 + j0);
             if (in1) nt_store(upd(a1, b1, x1), x4 + j1);
         }
-        if (tail < cols) xr[tail] = __fadd_rn(xr[tail], __fmul_rn(yr[tail], __fsub_rn(gr[tail], part)));
+        for (size_t i = tail; i < cols; i += TPR) xr[i] = __fadd_rn(xr[i], __fmul_rn(yr[i], __fsub_rn(gr[i], part)));
     } else if (live) {
         for (size_t j = lane; j < cols; j += TPR) xr[j] = __fadd_rn(xr[j], __fmul_rn(yr[j], __fsub_rn(gr[j], part)));
     }
@@ -904,8 +903,23 @@ static int pick_tpr(size_t cols) {
     return 256;
 }
 
+// The integer-label forward has no other kernel whose rows its own must equal, so short rows get fewer lanes: the
+// combining of running maxima and sums across lanes (two exponentials a step) is most of a short row's work.
+static int label_tpr(size_t cols) {
+    // ([3355443, 10]: 96 -> 51 us, [524288, 64]: 75 -> 39 us, [262144, 128]: 43 -> 31 us, [32768, 1000]: 31 -> 28 us)
+    if (cols < 16) return 1;
+    if (cols < 32) return 2;
+    if (cols < 96) return 4;
+    if (cols < 512) return 8;
+    if (cols <= 1024) return 16;
+    return pick_tpr(cols);
+}
+
 #define ZG_TPR_DISPATCH(tpr, CALL) \
     switch (tpr) {                 \
+        case 1: { constexpr int T = 1; CALL; } break;     \
+        case 2: { constexpr int T = 2; CALL; } break;     \
+        case 8: { constexpr int T = 8; CALL; } break;     \
         case 4: { constexpr int T = 4; CALL; } break;     \
         case 16: { constexpr int T = 16; CALL; } break;   \
         case 64: { constexpr int T = 64; CALL; } break;   \
@@ -953,7 +967,7 @@ ZG_API int zg_hip_smce_label_fwd(zg_hip_ctx* ctx, const float* logits, const uin
     if (int rc = check_rows("smce_label_fwd", rows, cols)) return rc;
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
-    const int tpr = pick_tpr(cols);
+    const int tpr = label_tpr(cols);
     const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
                                             labels, lse, row_loss, rows, cols));
@@ -980,7 +994,7 @@ ZG_API int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx* ctx, const float* logits, c
     ZG_REQUIRE(ctx->noalloc_scratch != nullptr, "smce_label_fwd_noalloc: the context has no scratch address");
     float* row_loss = (float*)ctx->noalloc_scratch;
     void* partials = (char*)ctx->noalloc_scratch + kNoAllocRowBytes;
-    const int tpr = pick_tpr(cols);
+    const int tpr = label_tpr(cols);
     const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
                                             labels, lse, row_loss, rows, cols));

@@ -65,7 +65,10 @@ SMCE_SHAPES = [(1, 4), (64, 10), (140, 7), (64, 2), (4096, 1024), (33, 1001), (1
                (7, 5000), (6, 8192), (5, 8196), (3, 20000), (2, 32768),
                # rows that start off a 16-byte boundary: heads and tails of one to three values, pieces that hold the end
                # of one row and the start of the next, rows too long for the registers
-               (1000, 5), (999, 6), (501, 11), (40, 4099), (7, 33001), (3, 70002), (2, 131072), (2000, 3), (5000, 1)]
+               (1000, 5), (999, 6), (501, 11), (40, 4099), (7, 33001), (3, 70002), (2, 131072), (2000, 3), (5000, 1),
+               # a handful of very long rows, cut into segments: whole segments, a short last one, segments that start
+               # off the 16-byte grid, a single row
+               (40, 65536), (3, 200003), (1, 1000001), (255, 65540)]
 
 
 @pytest.mark.parametrize("rows,cols", SMCE_SHAPES)
@@ -86,8 +89,8 @@ def test_smce_onehot_and_label(oracle, hip, rows, cols):
     # The host loop adds the exponentials of a row one after the other in fp32; for rows of tens of thousands
     # of columns that alone drifts past 1e-5 from the exact value.  The device result is held to 1e-5 against
     # fp64; the oracle is held to 1e-5 where its own summation error allows it, to 2e-4 up to rows of 70002 columns
-    # and to 1e-3 beyond (3.3e-4 measured on rows of 131072).
-    oracle_tol = TOL if cols <= 4096 else 2e-4 if cols <= 70002 else 1e-3
+    # to 1e-3 up to 200003 (3.3e-4 measured on rows of 131072) and to 5e-3 beyond (1.7e-3 on a row of 1000001).
+    oracle_tol = TOL if cols <= 4096 else 2e-4 if cols <= 70002 else 1e-3 if cols <= 200003 else 5e-3
     assert rel_fro(b["probs"], sm) <= TOL and rel_fro(a["probs"], sm) <= oracle_tol
     assert rel_fro(b["probs"], a["probs"]) <= max(TOL, 1.1 * rel_fro(a["probs"], sm) + 1e-6)
     assert abs(b["loss"][0] - loss) <= 1e-5 * max(1.0, abs(loss))
@@ -162,7 +165,9 @@ def test_smce_clamp_edge(oracle, hip):
                                        (1000, 4), (700, 32), (300, 36), (1500, 256), (70, 260), (300, 1024), (33, 1028),
                                        (21, 4096), (9, 4100), (5, 8196), (3, 32764), (70, 1030), (500, 30),
                                        # rows that start off a 16-byte boundary, rows too long for the registers
-                                       (999, 6), (501, 11), (40, 4099), (7, 33001), (3, 70002), (2000, 3)])
+                                       (999, 6), (501, 11), (40, 4099), (7, 33001), (3, 70002), (2000, 3),
+                                       # a handful of very long rows, cut into segments
+                                       (40, 65536), (3, 200003), (1, 1000001)])
 def test_softmax_fwd_bwd(oracle, hip, rows, cols):
     r = rng(rows + cols)
     x = r.standard_normal((rows, cols)).astype(np.float32)

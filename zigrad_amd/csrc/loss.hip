@@ -611,6 +611,80 @@ __global__ __launch_bounds__(kBlock) void softmax_wave_rows_kernel(const float* 
     }
 }
 
+// A handful of very long rows (fewer than two per compute unit, rows of 65536 columns and more): a workgroup per row would
+// leave most of the machine idle (32 rows of 1048576 columns: 7 % of 8 TB/s), so a row is cut into segments.  First
+// launch: workgroup (s, r) forms the running maximum and sum of segment s of row r (row_online, which places its
+// 16-byte pieces by the segment's own address) and leaves it at acc[r * n_seg + s].
+__global__ __launch_bounds__(kBlock) void softmax_seg_online_kernel(const float* logits, OnlineAccT* acc_out, size_t cols,
+                                                                     size_t seg, int n_seg) {
+    __shared__ OnlineAccT smem[kBlock / kWave];
+    const size_t s = blockIdx.x, row = blockIdx.y;
+    const size_t c0 = s * seg, c1 = c0 + seg < cols ? c0 + seg : cols;
+    OnlineAccT acc = row_online<kBlock, true>(logits + row * cols + c0, c1 - c0, threadIdx.x);
+    acc = block_reduce<OnlineAcc>(acc, smem);
+    if (threadIdx.x == 0) acc_out[row * n_seg + s] = acc;
+}
+
+// A row's segments (at most one per thread) combined by the workgroup in the fixed order of its reduction tree: log of
+// the sum of the row's exponentials, in every thread.
+__device__ __forceinline__ float seg_row_lse(const OnlineAccT* acc, size_t row, int n_seg, OnlineAccT* smem) {
+    OnlineAccT a = (int)threadIdx.x < n_seg ? acc[row * n_seg + threadIdx.x] : OnlineAcc::init();
+    a = row_group_reduce<kBlock>(a, smem);
+    return __fadd_rn(a.m, logf(a.s));
+}
+
+// Second launch: workgroup (s, r) writes the probabilities of its segment (row_probs) and, MODE 1, leaves the segment's
+// part of the row's loss term at seg_loss[r * n_seg + s].
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void softmax_seg_probs_kernel(const float* logits, const float* target, float* probs,
+                                                                    const OnlineAccT* acc, float* seg_loss, size_t cols,
+                                                                    size_t seg, int n_seg) {
+    __shared__ float lsum[kBlock / kWave];
+    __shared__ OnlineAccT smem[kBlock / kWave];
+    const size_t s = blockIdx.x, row = blockIdx.y;
+    const size_t c0 = s * seg, c1 = c0 + seg < cols ? c0 + seg : cols;
+    const float l = seg_row_lse(acc, row, n_seg, smem);
+    const size_t o = row * cols + c0;
+    float part = row_probs<kBlock, MODE, 0>(logits + o, MODE ? target + o : nullptr, probs + o, nullptr, c1 - c0,
+                                            threadIdx.x, l, 1.f, false);
+    if (MODE) {
+        part = block_reduce<SumAcc>(part, lsum);
+        if (threadIdx.x == 0) seg_loss[row * n_seg + s] = part;
+    }
+}
+
+// Integer labels: lse[row] and the row's loss term from the row's segments, a workgroup per row.
+__global__ __launch_bounds__(kBlock) void label_seg_final_kernel(const float* logits, const uint64_t* labels,
+                                                                  const OnlineAccT* acc, float* lse, float* row_loss,
+                                                                  size_t rows, size_t cols, int n_seg) {
+    __shared__ OnlineAccT smem[kBlock / kWave];
+    const size_t row = blockIdx.x;
+    const float l = seg_row_lse(acc, row, n_seg, smem);
+    if (threadIdx.x != 0) return;
+    lse[row] = l;
+    const uint64_t lab = labels[row];
+    float term = 0.f;
+    if (lab < cols) {
+        const float p = expf(__fsub_rn(logits[row * cols + lab], l));
+        const float safe = fminf(fmaxf(p, 1e-7f), 1.0f - 1e-7f);
+        term = -logf(safe);
+    }
+    row_loss[row] = term;
+}
+
+// Segments for `rows` long rows: about two workgroups per compute unit, segments of at least 16384 columns (a multiple of
+// 1024), at most one per thread of a workgroup.  0: the rows are not cut.
+static int row_segments_for(const zg_hip_ctx* ctx, size_t rows, size_t cols, size_t* seg_out) {
+    if (rows >= 2 * (size_t)ctx->n_cu || cols < 65536) return 0;
+    size_t n_seg = ceil_div_sz(2 * (size_t)ctx->n_cu, rows);
+    if (n_seg > (size_t)kBlock) n_seg = kBlock;
+    size_t seg = ceil_div_sz(ceil_div_sz(cols, n_seg), 1024) * 1024;
+    if (seg < 16384) seg = 16384;
+    n_seg = ceil_div_sz(cols, seg);
+    *seg_out = seg;
+    return n_seg >= 2 ? (int)n_seg : 0;
+}
+
 static bool wave_row_ok(const float* a, const float* b, const float* c, size_t rows, size_t cols) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
     return cols <= (size_t)kWave * kWaveRowVec * 4 && cols % 4 == 0 && (bits & 15u) == 0 && rows <= 0x7fffffffull;
@@ -965,6 +1039,20 @@ ZG_API int zg_hip_smce_label_fwd(zg_hip_ctx* ctx, const float* logits, const uin
     ZG_CTX(ctx);
     ZG_REQUIRE(logits && labels && lse && loss, "smce_label_fwd: null pointer");
     if (int rc = check_rows("smce_label_fwd", rows, cols)) return rc;
+    size_t seg = 0;
+    if (const int n_seg = row_segments_for(ctx, rows, cols, &seg)) {
+        char* mem = (char*)workspace(ctx, rows * sizeof(float) + rows * n_seg * sizeof(OnlineAccT));
+        if (!mem) return ZG_HIP_EOOM;
+        OnlineAccT* acc = (OnlineAccT*)mem;
+        float* row_loss = (float*)(mem + rows * n_seg * sizeof(OnlineAccT));
+        hipLaunchKernelGGL(softmax_seg_online_kernel, dim3((unsigned)n_seg, (unsigned)rows), dim3(kBlock), 0, ctx->stream,
+                           logits, acc, cols, seg, n_seg);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(label_seg_final_kernel, dim3((unsigned)rows), dim3(kBlock), 0, ctx->stream,
+                           logits, labels, acc, lse, row_loss, rows, cols, n_seg);
+        ZG_LAUNCH_CHECK();
+        return flat_reduce<TermId, 1>(ctx, row_loss, nullptr, rows, 0.f, FinDivN{loss, (float)rows});
+    }
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
     const int tpr = label_tpr(cols);
@@ -1061,6 +1149,20 @@ ZG_API int zg_hip_smce_fwd(zg_hip_ctx* ctx, const float* logits, const float* ta
             ZG_LAUNCH_CHECK();
             return ZG_HIP_OK;
         }
+    }
+    size_t seg = 0;
+    if (const int n_seg = row_segments_for(ctx, rows, cols, &seg)) {
+        char* mem = (char*)workspace(ctx, rows * n_seg * (sizeof(float) + sizeof(OnlineAccT)));
+        if (!mem) return ZG_HIP_EOOM;
+        OnlineAccT* acc = (OnlineAccT*)mem;
+        float* seg_loss = (float*)(mem + rows * n_seg * sizeof(OnlineAccT));
+        const dim3 grid((unsigned)n_seg, (unsigned)rows);
+        hipLaunchKernelGGL(softmax_seg_online_kernel, grid, dim3(kBlock), 0, ctx->stream, logits, acc, cols, seg, n_seg);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(softmax_seg_probs_kernel<1>, grid, dim3(kBlock), 0, ctx->stream, logits, target, probs, acc,
+                           seg_loss, cols, seg, n_seg);
+        ZG_LAUNCH_CHECK();
+        return flat_reduce<TermId, 1>(ctx, seg_loss, nullptr, rows * n_seg, 0.f, FinDivN{loss, (float)rows});
     }
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
@@ -1166,6 +1268,18 @@ ZG_API int zg_hip_softmax_fwd(zg_hip_ctx* ctx, const float* x, float* y, size_t 
     if (rows == 0 || cols == 0) return ZG_HIP_OK;
     ZG_REQUIRE(x && y, "softmax_fwd: null pointer");
     if (int rc = check_rows("softmax_fwd", rows, cols)) return rc;
+    size_t seg = 0;
+    if (const int n_seg = row_segments_for(ctx, rows, cols, &seg)) {
+        OnlineAccT* acc = (OnlineAccT*)workspace(ctx, rows * n_seg * sizeof(OnlineAccT));
+        if (!acc) return ZG_HIP_EOOM;
+        const dim3 grid((unsigned)n_seg, (unsigned)rows);
+        hipLaunchKernelGGL(softmax_seg_online_kernel, grid, dim3(kBlock), 0, ctx->stream, x, acc, cols, seg, n_seg);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(softmax_seg_probs_kernel<0>, grid, dim3(kBlock), 0, ctx->stream, x, (const float*)nullptr, y, acc,
+                           (float*)nullptr, cols, seg, n_seg);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     if (long_row_ok(x, x, y, rows, cols)) {
         ZG_LONG_ROWS(0, 0, x, (const float*)nullptr, y, (float*)nullptr, cols, (float*)nullptr, 1.f);
     } else if (wave_row_ok(x, x, y, rows, cols)) {

@@ -827,6 +827,87 @@ __global__ __launch_bounds__(kFlatSingle) void smce_small_kernel(const float* lo
     if (threadIdx.x == 0) FinDivN{loss, denom}(s);
 }
 
+// The two passes of the softmax backward over one row (or one segment of a row) of `cols` values, TPR lanes on it.
+// Rows of the three operands that start at the same offset from a 16-byte boundary are walked in 16-byte pieces, the
+// values before the first boundary and after the last whole piece dealt to the lanes one by one (rows of 32001 columns
+// value by value: 31 % of 8 TB/s); rows of fewer than eight pieces per lane and rows at different offsets go value by
+// value.
+template <int TPR>
+__device__ __forceinline__ bool bwd_row_in_pieces(const float* yr, const float* gr, const float* xr, size_t cols) {
+    return cols >= (size_t)8 * TPR && (((reinterpret_cast<uintptr_t>(yr) ^ reinterpret_cast<uintptr_t>(gr)) |
+                                        (reinterpret_cast<uintptr_t>(yr) ^ reinterpret_cast<uintptr_t>(xr))) & 15u) == 0;
+}
+// this lane's part of sum_j y_j * y_g_j
+template <int TPR>
+__device__ __forceinline__ float bwd_row_dot(const float* yr, const float* gr, size_t cols, int lane, bool pieces) {
+    float part = 0.f;
+    if (!pieces) {
+        for (size_t j = lane; j < cols; j += TPR) part = __fadd_rn(part, __fmul_rn(yr[j], gr[j]));
+        return part;
+    }
+    const size_t h = row_head(yr, cols), c4 = (cols - h) >> 2;
+    const float4* y4 = reinterpret_cast<const float4*>(yr + h);
+    const float4* q4 = reinterpret_cast<const float4*>(gr + h);
+    auto dot4 = [](float4 a, float4 b) {
+        return __fadd_rn(__fadd_rn(__fmul_rn(a.x, b.x), __fmul_rn(a.y, b.y)), __fadd_rn(__fmul_rn(a.z, b.z), __fmul_rn(a.w, b.w)));
+    };
+    for (size_t i = lane; i < h; i += TPR) part = __fadd_rn(part, __fmul_rn(yr[i], gr[i]));
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (size_t j = lane; j < c4; j += 4 * TPR) {
+        const bool in1 = j + TPR < c4, in2 = j + 2 * TPR < c4, in3 = j + 3 * TPR < c4;
+        // plain loads: the second pass reads both rows again
+        const float4 a0 = y4[j], b0 = q4[j];
+        const float4 a1 = in1 ? y4[j + TPR] : zero, b1 = in1 ? q4[j + TPR] : zero;
+        const float4 a2 = in2 ? y4[j + 2 * TPR] : zero, b2 = in2 ? q4[j + 2 * TPR] : zero;
+        const float4 a3 = in3 ? y4[j + 3 * TPR] : zero, b3 = in3 ? q4[j + 3 * TPR] : zero;
+        s0 = __fadd_rn(s0, dot4(a0, b0));
+        s1 = __fadd_rn(s1, dot4(a1, b1));
+        s2 = __fadd_rn(s2, dot4(a2, b2));
+        s3 = __fadd_rn(s3, dot4(a3, b3));
+    }
+    part = __fadd_rn(part, __fadd_rn(__fadd_rn(s0, s1), __fadd_rn(s2, s3)));
+    for (size_t i = h + (c4 << 2) + (size_t)lane; i < cols; i += TPR) part = __fadd_rn(part, __fmul_rn(yr[i], gr[i]));
+    return part;
+}
+// x_g += y * (y_g - dot) over the row
+template <int TPR>
+__device__ __forceinline__ void bwd_row_apply(const float* yr, const float* gr, float* xr, size_t cols, int lane, float dot,
+                                              bool pieces) {
+    if (!pieces) {
+        for (size_t j = lane; j < cols; j += TPR) xr[j] = __fadd_rn(xr[j], __fmul_rn(yr[j], __fsub_rn(gr[j], dot)));
+        return;
+    }
+    const size_t h = row_head(yr, cols), c4 = (cols - h) >> 2;
+    const float4* y4 = reinterpret_cast<const float4*>(yr + h);
+    const float4* q4 = reinterpret_cast<const float4*>(gr + h);
+    float4* x4 = reinterpret_cast<float4*>(xr + h);
+    for (size_t i = lane; i < h; i += TPR) xr[i] = __fadd_rn(xr[i], __fmul_rn(yr[i], __fsub_rn(gr[i], dot)));
+    for (size_t j0 = lane; j0 < c4; j0 += 2 * TPR) {
+        const size_t j1 = j0 + TPR;
+        const bool in1 = j1 < c4;
+        const float4 a0 = nt_load(y4 + j0), b0 = nt_load(q4 + j0), x0 = nt_load(x4 + j0);
+        float4 a1 = a0, b1 = b0, x1 = x0;
+        if (in1) {
+            a1 = nt_load(y4 + j1);
+            b1 = nt_load(q4 + j1);
+            x1 = nt_load(x4 + j1);
+        }
+        auto upd = [&](float4 a, float4 b, float4 x) {
+            float4 o;
+            o.x = __fadd_rn(x.x, __fmul_rn(a.x, __fsub_rn(b.x, dot)));
+            o.y = __fadd_rn(x.y, __fmul_rn(a.y, __fsub_rn(b.y, dot)));
+            o.z = __fadd_rn(x.z, __fmul_rn(a.z, __fsub_rn(b.z, dot)));
+            o.w = __fadd_rn(x.w, __fmul_rn(a.w, __fsub_rn(b.w, dot)));
+            return o;
+        };
+        nt_store(upd(a0, b0, x0), x4 + j0);
+        if (in1) nt_store(upd(a1, b1, x1), x4 + j1);
+    }
+    for (size_t i = h + (c4 << 2) + (size_t)lane; i < cols; i += TPR)
+        xr[i] = __fadd_rn(xr[i], __fmul_rn(yr[i], __fsub_rn(gr[i], dot)));
+}
+
 // src/nn/loss.zig:232-245: x_g += y * (y_g - sum_j y_j * y_g_j) per row
 template <int TPR>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, const float* y_g, float* x_g, size_t rows,
@@ -837,44 +918,11 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
     const int lane = threadIdx.x % TPR;
     const size_t row = (size_t)blockIdx.x * kRows + threadIdx.x / TPR;
     const bool live = row < rows;
-    float part = 0.f;
     const float* yr = y + row * cols;
     const float* gr = y_g + row * cols;
     float* xr = x_g + row * cols;
-    // rows of the three operands that start at the same offset from a 16-byte boundary are walked in 16-byte pieces, the
-    // values before the first boundary and after the last whole piece by the first lanes (rows of 32001 columns value
-    // by value: 31 % of 8 TB/s)
-    const bool pieces = live && cols >= (size_t)8 * TPR &&
-                        (((reinterpret_cast<uintptr_t>(yr) ^ reinterpret_cast<uintptr_t>(gr)) |
-                          (reinterpret_cast<uintptr_t>(yr) ^ reinterpret_cast<uintptr_t>(xr))) & 15u) == 0;
-    const size_t h = live ? row_head(yr, cols) : 0, c4 = (cols - h) >> 2, tail = h + (c4 << 2) + (size_t)lane;
-    const float4* y4 = reinterpret_cast<const float4*>(yr + h);
-    const float4* q4 = reinterpret_cast<const float4*>(gr + h);
-    float4* x4 = reinterpret_cast<float4*>(xr + h);
-    if (pieces) {
-        auto dot4 = [](float4 a, float4 b) {
-            return __fadd_rn(__fadd_rn(__fmul_rn(a.x, b.x), __fmul_rn(a.y, b.y)), __fadd_rn(__fmul_rn(a.z, b.z), __fmul_rn(a.w, b.w)));
-        };
-        for (size_t i = lane; i < h; i += TPR) part = __fadd_rn(part, __fmul_rn(yr[i], gr[i]));
-        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-        for (size_t j = lane; j < c4; j += 4 * TPR) {
-            const bool in1 = j + TPR < c4, in2 = j + 2 * TPR < c4, in3 = j + 3 * TPR < c4;
-            // plain loads: the second pass reads both rows again
-            const float4 a0 = y4[j], b0 = q4[j];
-            const float4 a1 = in1 ? y4[j + TPR] : zero, b1 = in1 ? q4[j + TPR] : zero;
-            const float4 a2 = in2 ? y4[j + 2 * TPR] : zero, b2 = in2 ? q4[j + 2 * TPR] : zero;
-            const float4 a3 = in3 ? y4[j + 3 * TPR] : zero, b3 = in3 ? q4[j + 3 * TPR] : zero;
-            s0 = __fadd_rn(s0, dot4(a0, b0));
-            s1 = __fadd_rn(s1, dot4(a1, b1));
-            s2 = __fadd_rn(s2, dot4(a2, b2));
-            s3 = __fadd_rn(s3, dot4(a3, b3));
-        }
-        part = __fadd_rn(part, __fadd_rn(__fadd_rn(s0, s1), __fadd_rn(s2, s3)));
-        for (size_t i = tail; i < cols; i += TPR) part = __fadd_rn(part, __fmul_rn(yr[i], gr[i]));
-    } else if (live) {
-        for (size_t j = lane; j < cols; j += TPR) part = __fadd_rn(part, __fmul_rn(yr[j], gr[j]));
-    }
+    const bool pieces = live && bwd_row_in_pieces<TPR>(yr, gr, xr, cols);
+    float part = live ? bwd_row_dot<TPR>(yr, gr, cols, lane, pieces) : 0.f;
     if (TPR <= kWave) {
         part = group_reduce<SumAcc, (TPR <= kWave ? TPR : kWave)>(part);
     } else {
@@ -884,33 +932,37 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_kernel(const float* y, con
         __syncthreads();
         part = bcast;
     }
-    if (pieces) {
-        for (size_t i = lane; i < h; i += TPR) xr[i] = __fadd_rn(xr[i], __fmul_rn(yr[i], __fsub_rn(gr[i], part)));
-        for (size_t j0 = lane; j0 < c4; j0 += 2 * TPR) {
-            const size_t j1 = j0 + TPR;
-            const bool in1 = j1 < c4;
-            const float4 a0 = nt_load(y4 + j0), b0 = nt_load(q4 + j0), x0 = nt_load(x4 + j0);
-            float4 a1 = a0, b1 = b0, x1 = x0;
-            if (in1) {
-                a1 = nt_load(y4 + j1);
-                b1 = nt_load(q4 + j1);
-                x1 = nt_load(x4 + j1);
-            }
-            auto upd = [&](float4 a, float4 b, float4 x) {
-                float4 o;
-                o.x = __fadd_rn(x.x, __fmul_rn(a.x, __fsub_rn(b.x, part)));
-                o.y = __fadd_rn(x.y, __fmul_rn(a.y, __fsub_rn(b.y, part)));
-                o.z = __fadd_rn(x.z, __fmul_rn(a.z, __fsub_rn(b.z, part)));
-                o.w = __fadd_rn(x.w, __fmul_rn(a.w, __fsub_rn(b.w, part)));
-                return o;
-            };
-            nt_store(upd(a0, b0, x0), x4 + j0);
-            if (in1) nt_store(upd(a1, b1, x1), x4 + j1);
-        }
-        for (size_t i = tail; i < cols; i += TPR) xr[i] = __fadd_rn(xr[i], __fmul_rn(yr[i], __fsub_rn(gr[i], part)));
-    } else if (live) {
-        for (size_t j = lane; j < cols; j += TPR) xr[j] = __fadd_rn(xr[j], __fmul_rn(yr[j], __fsub_rn(gr[j], part)));
-    }
+    if (live) bwd_row_apply<TPR>(yr, gr, xr, cols, lane, part, pieces);
+}
+
+// A handful of very long rows, cut into segments like the forward kernels cut them: the first launch leaves each
+// segment's part of the row's sum at dots[r * n_seg + s], the second adds a row's parts up in a workgroup (the fixed order
+// of its reduction tree) and updates its segment.
+__global__ __launch_bounds__(kBlock) void softmax_bwd_seg_dot_kernel(const float* y, const float* y_g, const float* x_g,
+                                                                      float* dots, size_t cols, size_t seg, int n_seg) {
+    __shared__ float smem[kBlock / kWave];
+    const size_t s = blockIdx.x, row = blockIdx.y;
+    const size_t c0 = s * seg, c1 = c0 + seg < cols ? c0 + seg : cols, o = row * cols + c0;
+    const bool pieces = bwd_row_in_pieces<kBlock>(y + o, y_g + o, x_g + o, c1 - c0);
+    float part = bwd_row_dot<kBlock>(y + o, y_g + o, c1 - c0, threadIdx.x, pieces);
+    part = block_reduce<SumAcc>(part, smem);
+    if (threadIdx.x == 0) dots[row * n_seg + s] = part;
+}
+__global__ __launch_bounds__(kBlock) void softmax_bwd_seg_apply_kernel(const float* y, const float* y_g, float* x_g,
+                                                                        const float* dots, size_t cols, size_t seg,
+                                                                        int n_seg) {
+    __shared__ float smem[kBlock / kWave];
+    __shared__ float bcast;
+    const size_t s = blockIdx.x, row = blockIdx.y;
+    const size_t c0 = s * seg, c1 = c0 + seg < cols ? c0 + seg : cols, o = row * cols + c0;
+    float dot = (int)threadIdx.x < n_seg ? dots[row * n_seg + threadIdx.x] : 0.f;
+    dot = block_reduce<SumAcc>(dot, smem);
+    __syncthreads();
+    if (threadIdx.x == 0) bcast = dot;
+    __syncthreads();
+    dot = bcast;
+    const bool pieces = bwd_row_in_pieces<kBlock>(y + o, y_g + o, x_g + o, c1 - c0);
+    bwd_row_apply<kBlock>(y + o, y_g + o, x_g + o, c1 - c0, threadIdx.x, dot, pieces);
 }
 
 // The same with the rows of y and y_g held in registers (16-byte aligned rows of up to 32768 columns): NT threads per row
@@ -1299,6 +1351,18 @@ ZG_API int zg_hip_softmax_bwd(zg_hip_ctx* ctx, const float* y, const float* y_g,
     if (rows == 0 || cols == 0) return ZG_HIP_OK;
     ZG_REQUIRE(y && y_g && x_g, "softmax_bwd: null pointer");
     if (int rc = check_rows("softmax_bwd", rows, cols)) return rc;
+    size_t seg = 0;
+    if (const int n_seg = row_segments_for(ctx, rows, cols, &seg)) {
+        float* dots = (float*)workspace(ctx, rows * n_seg * sizeof(float));
+        if (!dots) return ZG_HIP_EOOM;
+        const dim3 grid((unsigned)n_seg, (unsigned)rows);
+        hipLaunchKernelGGL(softmax_bwd_seg_dot_kernel, grid, dim3(kBlock), 0, ctx->stream, y, y_g, x_g, dots, cols, seg, n_seg);
+        ZG_LAUNCH_CHECK();
+        hipLaunchKernelGGL(softmax_bwd_seg_apply_kernel, grid, dim3(kBlock), 0, ctx->stream, y, y_g, x_g, dots, cols, seg,
+                           n_seg);
+        ZG_LAUNCH_CHECK();
+        return ZG_HIP_OK;
+    }
     const uintptr_t bits = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(y_g) | reinterpret_cast<uintptr_t>(x_g);
     if (cols % 4 == 0 && (bits & 15u) == 0 && cols <= 32768 && rows <= 0x7fffffffull) {
 #define ZG_BWD_ROWS(NT, VEC, ROWS_PER_WG)                                                                              \

@@ -292,7 +292,7 @@ static int axis_reduce(zg_hip_ctx* ctx, const float* x, typename A::Out* y, size
         if (cols < 16) ZG_ROW(1);
         else if (cols < 32) ZG_ROW(2);
         else if (cols < 64) ZG_ROW(4);
-        else if (cols < 256) ZG_ROW(8);
+        else if (cols < 192) ZG_ROW(8);
         else if (cols <= 256) ZG_ROW(16);
         else if (cols <= 16384 || rows >= (size_t)ctx->n_cu * 8) ZG_ROW(64);
         else ZG_ROW(256);

@@ -1377,7 +1377,9 @@ ZG_API int zg_hip_softmax_bwd(zg_hip_ctx* ctx, const float* y, const float* y_g,
         ZG_LAUNCH_CHECK();
         return ZG_HIP_OK;
     }
-    const int tpr = pick_tpr(cols);
+    // rows the register kernel does not take (off the 16-byte grid, or longer than 32768 columns); sixteen lanes from 13
+    // columns on (four lanes on 31 columns, eight values each one after the other: 16 % of 8 TB/s)
+    const int tpr = (cols > 12 && cols <= 32) ? 16 : pick_tpr(cols);
     const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((softmax_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, y, y_g,
                                             x_g, rows, cols));

@@ -110,11 +110,13 @@ static Plan carve_plan(void* mem, size_t n, size_t nb) {
     return pl;
 }
 
-__global__ void zero_u32_kernel(uint32_t* a, size_t na, uint32_t* b, size_t nb, uint32_t* one = nullptr) {
+__global__ void zero_u32_kernel(uint32_t* a, size_t na, uint32_t* b, size_t nb, uint32_t* one = nullptr,
+                                uint32_t* other = nullptr) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nt = (size_t)gridDim.x * blockDim.x;
     for (size_t k = i; k < na; k += nt) a[k] = 0;
     for (size_t k = i; k < nb; k += nt) b[k] = 0;
     if (i == 0 && one) one[0] = 0;
+    if (i == 0 && other) other[0] = 0;
 }
 
 // key = idx[e] / divisor (divisor 1 for plain indices)
@@ -126,15 +128,25 @@ __global__ void histogram_kernel(const uint64_t* keys, size_t n, size_t nb, uint
     }
 }
 
-// exclusive scan, three launches: per-tile scan + tile sums, scan of tile sums (one workgroup), add back
+// exclusive scan, three launches: per-tile scan + tile sums, scan of tile sums (scan_single_kernel), add back
 __global__ __launch_bounds__(256) void scan_tiles_kernel(uint32_t* data, size_t n, uint32_t* tile_sums) {
     __shared__ uint32_t wave_tot[4];
     const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * 8;
     uint32_t v[8], s = 0;
+    // a thread's eight values as two 16-byte pieces where they are all there (value by value, a load touched 64 lanes x 4
+    // bytes spread over 2 KiB: 16.7 M buckets took 68 us)
+    const bool whole = base + 8 <= n && (reinterpret_cast<uintptr_t>(data) & 15u) == 0;
+    if (whole) {
+        const uint4 a = *reinterpret_cast<const uint4*>(data + base), b = *reinterpret_cast<const uint4*>(data + base + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 #pragma unroll
-    for (int k = 0; k < 8; k++) {
-        v[k] = (base + k < n) ? data[base + k] : 0;
-        s += v[k];
+        for (int k = 0; k < 8; k++) s += v[k];
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = (base + k < n) ? data[base + k] : 0;
+            s += v[k];
+        }
     }
     // inclusive scan of s across the workgroup
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -149,10 +161,21 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(uint32_t* data, size_t 
     uint32_t wave_off = 0;
     for (int w = 0; w < wave; w++) wave_off += wave_tot[w];
     uint32_t run = wave_off + inc - s;  // exclusive prefix of this thread's first element
+    if (whole) {
+        uint32_t o[8];
 #pragma unroll
-    for (int k = 0; k < 8; k++) {
-        if (base + k < n) data[base + k] = run;
-        run += v[k];
+        for (int k = 0; k < 8; k++) {
+            o[k] = run;
+            run += v[k];
+        }
+        *reinterpret_cast<uint4*>(data + base) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4*>(data + base + 4) = make_uint4(o[4], o[5], o[6], o[7]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            if (base + k < n) data[base + k] = run;
+            run += v[k];
+        }
     }
     if (threadIdx.x == 255) tile_sums[blockIdx.x] = wave_off + inc;
 }
@@ -191,33 +214,6 @@ __global__ __launch_bounds__(256) void scan_single_kernel(uint32_t* data, size_t
     }
 }
 
-__global__ __launch_bounds__(256) void scan_sums_kernel(uint32_t* tile_sums, size_t tiles) {
-    // one workgroup walks the tile sums in chunks of 256, carrying the running total
-    __shared__ uint32_t wave_tot[4];
-    __shared__ uint32_t carry_s;
-    if (threadIdx.x == 0) carry_s = 0;
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (size_t c = 0; c < tiles; c += 256) {
-        size_t i = c + threadIdx.x;
-        uint32_t s = (i < tiles) ? tile_sums[i] : 0;
-        uint32_t inc = s;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            uint32_t t = __shfl_up(inc, d, 64);
-            if (lane >= d) inc += t;
-        }
-        if (lane == 63) wave_tot[wave] = inc;
-        __syncthreads();
-        uint32_t off = carry_s;
-        for (int w = 0; w < wave; w++) off += wave_tot[w];
-        if (i < tiles) tile_sums[i] = off + inc - s;
-        __syncthreads();
-        if (threadIdx.x == 255) carry_s = off + inc;
-        __syncthreads();
-    }
-}
-
 __global__ __launch_bounds__(256) void scan_add_kernel(uint32_t* data, size_t n, const uint32_t* tile_sums) {
     const uint32_t off = tile_sums[blockIdx.x];
     const size_t base = (size_t)blockIdx.x * kScanTile;
@@ -250,17 +246,21 @@ __global__ void place_kernel(const uint64_t* keys, size_t n, size_t nb, const ui
 // With `peer_tmp` the payload is laid out in the same order, so that the apply kernels read it next to perm.
 // Buckets of more than kLongBucket entries are listed in `long_list`; those of more than kRankMax entries are left
 // to order_long_segments_kernel.
+// With `list` (and its length at list_count[0]) the waves take the buckets listed there instead of all buckets, and
+// the long ones among them have been listed already (order_sparse_kernel).
 __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
                                                               uint32_t* perm, const uint32_t* peer_tmp, uint32_t* peer,
-                                                              uint32_t* long_list) {
+                                                              uint32_t* long_list, const uint32_t* list = nullptr,
+                                                              const uint32_t* list_count = nullptr) {
     __shared__ __align__(16) uint32_t ids[4][kRankMax];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const size_t b = (size_t)blockIdx.x * 4 + wave;
+    size_t b = (size_t)blockIdx.x * 4 + wave;
+    if (list) b = b < list_count[0] ? list[b] : nb;
     uint32_t s = 0, len = 0;
     if (b < nb) {
         s = row_ptr[b];
         len = row_ptr[b + 1] - s;
-        if (len > kLongBucket && lane == 0) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)b;
+        if (!list && len > kLongBucket && lane == 0) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)b;
     }
     const bool here = b < nb && len <= kRankMax;
     const uint32_t len4 = (len + 3) & ~3u;
@@ -277,6 +277,42 @@ __global__ __launch_bounds__(256) void order_segments_kernel(const uint32_t* row
         }
         perm[s + rank] = id;
         if (peer_tmp) peer[s + rank] = peer_tmp[s + i];
+    }
+}
+
+// Many destinations for few entries (four destinations per entry and more): a wave per bucket would spend its launch
+// on empty buckets (65536 entries into 16.7 M destinations: 1.07 ms).  Here a thread looks at one bucket: nothing to do
+// for an empty one, a copy for a single entry, a rank by counting for up to kSparseSerial entries; longer buckets go to
+// `mid_list` (count at mid_count[0]) for order_segments_kernel, a wave each, and those of more than kLongBucket entries
+// to `long_list` as order_segments_kernel lists them.
+constexpr uint32_t kSparseSerial = 16;
+__global__ __launch_bounds__(256) void order_sparse_kernel(const uint32_t* row_ptr, size_t nb, const uint32_t* perm_tmp,
+                                                            uint32_t* perm, const uint32_t* peer_tmp, uint32_t* peer,
+                                                            uint32_t* long_list, uint32_t* mid_count, uint32_t* mid_list) {
+    const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= nb) return;
+    const uint32_t s = row_ptr[b], len = row_ptr[b + 1] - s;
+    if (len == 0) return;
+    if (len > kLongBucket) long_list[1 + atomicAdd(&long_list[0], 1u)] = (uint32_t)b;
+    if (len == 1) {
+        perm[s] = perm_tmp[s];
+        if (peer_tmp) peer[s] = peer_tmp[s];
+    } else if (len <= kSparseSerial) {
+        uint32_t ids[kSparseSerial];
+#pragma unroll
+        for (uint32_t i = 0; i < kSparseSerial; i++) ids[i] = i < len ? perm_tmp[s + i] : 0xffffffffu;
+#pragma unroll
+        for (uint32_t i = 0; i < kSparseSerial; i++) {
+            if (i < len) {
+                uint32_t rank = 0;
+#pragma unroll
+                for (uint32_t j = 0; j < kSparseSerial; j++) rank += ids[j] < ids[i] ? 1u : 0u;
+                perm[s + rank] = ids[i];
+                if (peer_tmp) peer[s + rank] = peer_tmp[s + i];
+            }
+        }
+    } else if (len <= kRankMax) {
+        mid_list[atomicAdd(mid_count, 1u)] = (uint32_t)b;
     }
 }
 
@@ -711,7 +747,9 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
     const size_t n = pl.n, nb = pl.nb;
     const int g_n = (int)(ceil_div_sz(n ? n : 1, 256) > 4096 ? 4096 : ceil_div_sz(n ? n : 1, 256));
     const int g_b = (int)(ceil_div_sz(nb + 1, 256) > 4096 ? 4096 : ceil_div_sz(nb + 1, 256));
-    hipLaunchKernelGGL(zero_u32_kernel, dim3(g_b), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.cursor, nb, pl.long_list);
+    // the last word of long_list is spare (at most n / (kLongBucket + 1) buckets are long): the sparse build's second count
+    uint32_t* mid_count = pl.long_list + n / kLongBucket + 1;
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(g_b), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.cursor, nb, pl.long_list, mid_count);
     ZG_LAUNCH_CHECK();
     if (n) {
         hipLaunchKernelGGL(histogram_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr);
@@ -724,7 +762,7 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
     } else {
         hipLaunchKernelGGL(scan_tiles_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
         ZG_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, pl.tile_sums, tiles);
+        hipLaunchKernelGGL(scan_single_kernel, dim3(1), dim3(256), 0, st, pl.tile_sums, tiles);  // 2048 sums a round
         ZG_LAUNCH_CHECK();
         hipLaunchKernelGGL(scan_add_kernel, dim3((unsigned)tiles), dim3(256), 0, st, pl.row_ptr, nb + 1, pl.tile_sums);
         ZG_LAUNCH_CHECK();
@@ -733,9 +771,24 @@ static int build_plan(zg_hip_ctx* ctx, const uint64_t* keys, const Plan& pl, con
         hipLaunchKernelGGL(place_kernel, dim3(g_n), dim3(256), 0, st, keys, n, nb, pl.row_ptr, pl.cursor, pl.perm_tmp, payload,
                            pl.peer_tmp);
         ZG_LAUNCH_CHECK();
-        hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(nb, 4)), dim3(256), 0, st, pl.row_ptr, nb,
-                           pl.perm_tmp, pl.perm, payload ? pl.peer_tmp : (const uint32_t*)nullptr, pl.peer, pl.long_list);
-        ZG_LAUNCH_CHECK();
+        const uint32_t* peer_tmp = payload ? pl.peer_tmp : (const uint32_t*)nullptr;
+        if (nb / 4 >= n) {
+            // the cursors are done with once the entries are placed: their array holds the list of mid-length buckets
+            // (at most n / (kSparseSerial + 1) of them, and nb >= 4 n)
+            hipLaunchKernelGGL(order_sparse_kernel, dim3((unsigned)ceil_div_sz(nb, 256)), dim3(256), 0, st, pl.row_ptr, nb,
+                               pl.perm_tmp, pl.perm, peer_tmp, pl.peer, pl.long_list, mid_count, pl.cursor);
+            ZG_LAUNCH_CHECK();
+            if (n > kSparseSerial) {
+                hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(n / (kSparseSerial + 1) + 1, 4)), dim3(256),
+                                   0, st, pl.row_ptr, nb, pl.perm_tmp, pl.perm, peer_tmp, pl.peer, pl.long_list, pl.cursor,
+                                   mid_count);
+                ZG_LAUNCH_CHECK();
+            }
+        } else {
+            hipLaunchKernelGGL(order_segments_kernel, dim3((unsigned)ceil_div_sz(nb, 4)), dim3(256), 0, st, pl.row_ptr, nb,
+                               pl.perm_tmp, pl.perm, peer_tmp, pl.peer, pl.long_list);
+            ZG_LAUNCH_CHECK();
+        }
         if (n > kRankMax) {  // only then can a bucket be too long to rank; the workgroups exit at once when none is
             size_t grid = n / kRankMax;
             if (grid > 1024) grid = 1024;

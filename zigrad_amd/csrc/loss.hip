@@ -703,13 +703,16 @@ static bool long_row_ok(const float* a, const float* b, const float* c, size_t r
                        __VA_ARGS__)
 #define ZG_WAVE_ROWS(MODE, GRAD, ...)                                                                                  \
     do { /* the lanes per row of pick_tpr, which the one-workgroup kernel for small batches follows; rows that leave */ \
-        /* registers free share a lane group two or four at a time */                                                  \
-        if (cols <= 16) ZG_WAVE_ROWS_AS(4, 4, MODE, GRAD, __VA_ARGS__);                                                \
-        else if (cols <= 32) ZG_WAVE_ROWS_AS(4, 2, MODE, GRAD, __VA_ARGS__);                                           \
-        else if (cols <= 64) ZG_WAVE_ROWS_AS(16, 4, MODE, GRAD, __VA_ARGS__);                                          \
-        else if (cols <= 128) ZG_WAVE_ROWS_AS(16, 2, MODE, GRAD, __VA_ARGS__);                                         \
+        /* registers free share a lane group two or four at a time where that still leaves a thousand workgroups */     \
+        /* ([4096, 64] on 64 workgroups instead of 256: 6.9 -> 8.8 us) */                                              \
+        const bool many = rows >= 65536;                                                                               \
+        if (cols <= 16 && rows >= 4 * 65536) ZG_WAVE_ROWS_AS(4, 4, MODE, GRAD, __VA_ARGS__);                           \
+        else if (cols <= 32 && rows >= 2 * 65536) ZG_WAVE_ROWS_AS(4, 2, MODE, GRAD, __VA_ARGS__);                      \
+        else if (cols <= 32) ZG_WAVE_ROWS_AS(4, 1, MODE, GRAD, __VA_ARGS__);                                           \
+        else if (cols <= 64 && many) ZG_WAVE_ROWS_AS(16, 4, MODE, GRAD, __VA_ARGS__);                                  \
+        else if (cols <= 128 && many) ZG_WAVE_ROWS_AS(16, 2, MODE, GRAD, __VA_ARGS__);                                 \
         else if (cols <= 16 * kWaveRowVec * 4) ZG_WAVE_ROWS_AS(16, 1, MODE, GRAD, __VA_ARGS__);                        \
-        else if (cols <= 512) ZG_WAVE_ROWS_AS(kWave, 2, MODE, GRAD, __VA_ARGS__);                                      \
+        else if (cols <= 512 && rows >= 8192) ZG_WAVE_ROWS_AS(kWave, 2, MODE, GRAD, __VA_ARGS__);                      \
         else ZG_WAVE_ROWS_AS(kWave, 1, MODE, GRAD, __VA_ARGS__);                                                       \
     } while (0)
 
@@ -1031,14 +1034,12 @@ static int pick_tpr(size_t cols) {
 
 // The integer-label forward has no other kernel whose rows its own must equal, so short rows get fewer lanes: the
 // combining of running maxima and sums across lanes (two exponentials a step) is most of a short row's work.
-static int label_tpr(size_t cols) {
-    // ([3355443, 10]: 96 -> 51 us, [524288, 64]: 75 -> 39 us, [262144, 128]: 43 -> 31 us, [32768, 1000]: 31 -> 28 us)
-    if (cols < 16) return 1;
-    if (cols < 32) return 2;
-    if (cols < 96) return 4;
-    if (cols < 512) return 8;
-    if (cols <= 1024) return 16;
-    return pick_tpr(cols);
+static int label_tpr(size_t rows, size_t cols) {
+    // ([3355443, 10]: 96 -> 51 us, [524288, 64]: 75 -> 39 us, [262144, 128]: 43 -> 31 us, [32768, 1000]: 31 -> 28 us);
+    // only where that still leaves a thousand workgroups ([1000, 1000] on 63 instead of 250: 7.0 -> 8.6 us)
+    const int few = cols < 16 ? 1 : cols < 32 ? 2 : cols < 96 ? 4 : cols < 512 ? 8 : cols <= 1024 ? 16 : pick_tpr(cols);
+    const int usual = pick_tpr(cols);
+    return (few < usual && rows / (size_t)(kBlock / few) >= 1024) ? few : usual;
 }
 
 #define ZG_TPR_DISPATCH(tpr, CALL) \
@@ -1107,7 +1108,7 @@ ZG_API int zg_hip_smce_label_fwd(zg_hip_ctx* ctx, const float* logits, const uin
     }
     float* row_loss = (float*)workspace(ctx, rows * sizeof(float));
     if (!row_loss) return ZG_HIP_EOOM;
-    const int tpr = label_tpr(cols);
+    const int tpr = label_tpr(rows, cols);
     const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
                                             labels, lse, row_loss, rows, cols));
@@ -1134,7 +1135,7 @@ ZG_API int zg_hip_smce_label_fwd_noalloc(zg_hip_ctx* ctx, const float* logits, c
     ZG_REQUIRE(ctx->noalloc_scratch != nullptr, "smce_label_fwd_noalloc: the context has no scratch address");
     float* row_loss = (float*)ctx->noalloc_scratch;
     void* partials = (char*)ctx->noalloc_scratch + kNoAllocRowBytes;
-    const int tpr = label_tpr(cols);
+    const int tpr = label_tpr(rows, cols);
     const unsigned grid = (unsigned)ceil_div_sz(rows, kBlock / tpr);
     ZG_TPR_DISPATCH(tpr, hipLaunchKernelGGL((smce_label_fwd_kernel<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, logits,
                                             labels, lse, row_loss, rows, cols));

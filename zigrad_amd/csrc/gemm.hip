@@ -2463,8 +2463,10 @@ ZG_API int zg_hip_outer(zg_hip_ctx* ctx, const float* x, size_t xl, const float*
     ZG_REQUIRE(x && y && A, "outer: null pointer");
     const bool vec = aligned16(A) && aligned16(y) && yl % 4 == 0;
     size_t blocks = ceil_div_sz(xl * yl, vec ? 256 * 16 : 256);
-    // a workgroup per 16 KiB of A at any size (16384 x 16384: 446 -> 363 us against a grid capped at 16 per compute unit)
-    if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
+    // a workgroup per 16 KiB of A at any size (16384 x 16384: 446 -> 363 us against a grid capped at 16 per compute unit);
+    // the value-by-value form keeps the cap, its threads walking the rest (1048576 x 7: 12.2 us capped, 16.8 us not)
+    const size_t cap = vec ? 0x7fffffffull : (size_t)ctx->n_cu * 16;
+    if (blocks > cap) blocks = cap;
     if (vec) hipLaunchKernelGGL(ger_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, x, xl, y, yl, A, alpha);
     else hipLaunchKernelGGL(ger_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, x, xl, y, yl, A, alpha);
     ZG_LAUNCH_CHECK();

@@ -210,6 +210,28 @@ def test_products_on_few_tiles_cut_into_ranges_of_k(hip, shape, ta, tb):
     assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
 
 
+@pytest.mark.parametrize("shape,ta,tb", [
+    # a small layer's weight gradient over a very long batch: up to 256 ranges of k and the reduction that adds many
+    # partial products (64 x 64 tiles in every layout, the 32-wide blocks of the skinny products in the k-strided one)
+    ((64, 64, 65536), False, False), ((64, 64, 65536 + 40), True, False), ((128, 70, 40000), False, True),
+    ((16, 16, 300000), True, False), ((10, 64, 100000), True, False), ((64, 10, 70001), True, False),
+    ((100, 30, 50000), True, True),
+    # leading dimensions of 2^21 values and more: rows of millions of columns
+    ((32, 32, (1 << 21) + 40), False, False), ((24, 40, (1 << 21) + 8), False, True), ((16, 8, 1 << 21), True, True)])
+def test_products_over_a_very_long_k(hip, shape, ta, tb):
+    m, n, k = shape
+    r = np.random.default_rng(m + 3 * n + 7 * k)
+    A = r.standard_normal((k, m) if ta else (m, k), dtype=np.float32)
+    B = r.standard_normal((n, k) if tb else (k, n), dtype=np.float32)
+    C0 = r.standard_normal((m, n), dtype=np.float32)
+    prod = (A.T if ta else A).astype(np.float64) @ (B.T if tb else B).astype(np.float64)
+    got = _matmul(hip, A, B, np.full((m, n), np.nan, np.float32), m, n, k, ta, tb, 1.0, 0.0)
+    assert np.linalg.norm(got - prod) <= TOL * np.linalg.norm(prod)
+    got = _matmul(hip, A, B, C0, m, n, k, ta, tb, -0.5, 1.0)
+    want = C0 - 0.5 * prod
+    assert np.linalg.norm(got - want) <= TOL * np.linalg.norm(want)
+
+
 @pytest.mark.parametrize("m,n", [(5000, 300), (70000, 33), (64, 64), (63, 1), (1, 700), (4096, 4096), (130, 257)])
 def test_transposed_matvec_over_many_rows(oracle, hip, m, n):
     """y = alpha A^T x + beta y with the rows split over workgroups (src/device/host_device.zig:232-240)."""

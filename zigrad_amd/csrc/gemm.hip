@@ -924,6 +924,48 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* P, floa
     }
 }
 
+// The same sum for many partial products (more than 16: a very long k): a workgroup takes 64 adjacent elements, wave w adds
+// partial products w, w + 4, ... in that order with sixteen loads in flight, and the four wave sums are added in wave
+// order.  (A thread walking 256 partial products eight at a time took 38 us for a 64 x 64 block.)
+__global__ __launch_bounds__(256) void splitk_reduce_many_kernel(const float* P, float* C, size_t M, size_t N, size_t ldc,
+                                                                 int splits, float alpha, float beta, size_t c_chunk,
+                                                                 const float* bias, const float* gate, int relu) {
+    __shared__ float smem[4][64];
+    const size_t z = blockIdx.z;
+    const float* p = P + z * (size_t)splits * M * N;
+    float* c = C + z * c_chunk;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const size_t i = (size_t)blockIdx.x * 64 + lane;
+    float acc = 0.f;
+    if (i < M * N) {
+        bool first = true;
+        for (int s0 = w; s0 < splits; s0 += 4 * 16) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                if (s0 + 4 * u < splits) v[u] = p[(size_t)(s0 + 4 * u) * M * N + i];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                if (s0 + 4 * u < splits) {
+                    acc = first ? v[u] : acc + v[u];
+                    first = false;
+                }
+            }
+        }
+    }
+    smem[w][lane] = acc;
+    __syncthreads();
+    if (w == 0 && i < M * N) {
+        const float sum = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
+        const size_t r = i / N, col = i % N;
+        float v = alpha * sum;
+        if (beta != 0.f) v += beta * c[r * ldc + col];
+        v = gemm_extras(v, bias != nullptr, bias ? bias[col] : 0.f, relu != 0);
+        if (gate && gate[z * c_chunk + r * ldc + col] <= 0.f) v = 0.f;
+        c[r * ldc + col] = v;
+    }
+}
+
 // C *= beta (or 0) when k == 0 or alpha == 0: BLAS leaves beta*C
 __global__ void scale_c_kernel(float* C, size_t M, size_t N, size_t ldc, float beta, size_t c_chunk) {
     float* c = C + (size_t)blockIdx.z * c_chunk;
@@ -1138,9 +1180,15 @@ static GemmPlan gemm_plan_single(size_t m, size_t n, size_t k, size_t batches, s
             // a range of k per CU for up to 32 tiles, two per CU beyond (500 x 256 x 2048, 32 tiles: 15.5 us in 16 ranges,
             // 12.9 us in 8), and at most 16 ranges: shorter ones are mostly prologue and the reduction reads them all
             // (256 x 256 x 4096: 17.0 us in 64 ranges of 64 values of k, 13.1 us in 16 of 256)
+            // A very long k (a small layer's weight gradient over a batch of 65536 rows and more) keeps ranges of at least
+            // 512 values of k and takes up to 256 of them: sixteen workgroups stream 30 GB/s each, whatever is left to
+            // read (64 x 64 x 65536: 88 us in 16 ranges, 4.8 % of 8 TB/s).
             size_t splits = ceil_div_sz((t64 <= 32 ? 1 : 2) * n_cu, t64);
             if (splits > kt_total / 4) splits = kt_total / 4;
-            if (splits > 16) splits = 16;
+            size_t cap = kt_total / 16;
+            if (cap < 16) cap = 16;
+            if (cap > 256) cap = 256;
+            if (splits > cap) splits = cap;
             size_t per = ceil_div_sz(kt_total, splits);
             per += per & 1;
             splits = ceil_div_sz(kt_total, per);
@@ -1354,6 +1402,22 @@ static bool gemm_is_tiny(size_t m, size_t n, size_t k, size_t batches, size_t ld
     return small_ld && ((k <= 256 && blocks <= n_cu) || (k <= 512 && blocks <= 16));
 }
 
+// Ranges of k for the skinny weight-gradient products (see gemm_dispatch_body): groups of 8 values of k, a round of 32
+// groups per workgroup at least; at most 32 ranges, or two workgroups per compute unit where k is long enough for
+// ranges of 2048 values and more (16 x 16 over a million rows: 413 us in 32 ranges).  `per`: groups per range.
+static size_t gemm_skinny_splits(size_t m, size_t n, size_t k, size_t n_cu, size_t* per_out) {
+    const size_t groups = ceil_div_sz(k, 8);
+    size_t splits = ceil_div_sz(groups, 32);
+    size_t cap = 2 * n_cu / (ceil_div_sz(m, 32) * ceil_div_sz(n, 32));
+    if (cap > groups / 256) cap = groups / 256;
+    if (cap < 32) cap = 32;
+    if (splits > cap) splits = cap;
+    size_t per = ceil_div_sz(groups, splits);
+    per = (per + 3) & ~(size_t)3;  // whole turns of the four waves
+    *per_out = per;
+    return ceil_div_sz(groups, per);
+}
+
 // One unbatched product of k-contiguous operands with a long k on at most a CU's worth of 16 x 16 blocks: gemm_deep_kernel.
 // It goes before the unstaged kernel where both apply (k of 384 to 512 on up to 16 blocks of 32 x 32: 64 x 64 x 512
 // 8.1 -> 5.6 us, 128 x 64 x 512 8.2 -> 4.8 us).
@@ -1499,8 +1563,13 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     g.split_tiles = kt_total;
     g.split_stride = 0;
 
-    if (!small_ld) return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
-    const bool deep = gemm_is_deep(m, n, k, batches, a_kmajor, b_kmajor, n_cu);
+    // leading dimensions of 2^21 values and more (a few rows of millions of columns): 64 x 64 tiles with 64-bit row
+    // offsets, whole, or with k in ranges where the plan for 64 x 64 tiles cuts it (32 x 32 over 2097152 values of k on
+    // one workgroup: 78 ms)
+    const GemmPlan far_plan = small_ld ? GemmPlan() : gemm_plan_single(m, n, k, batches, n_cu);
+    if (!small_ld && !(far_plan.kind == GemmPlan::kSplit && far_plan.tile == 2))
+        return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
+    const bool deep = small_ld && gemm_is_deep(m, n, k, batches, a_kmajor, b_kmajor, n_cu);
     if (!deep && gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
     if (deep) {
         g.tiles_m = (unsigned)ceil_div_sz(m, 16);
@@ -1514,13 +1583,9 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     // unstaged kernel takes ranges of k (one round of 256 per workgroup, at most 32 ranges) and the split-k reduction
     // adds the partial blocks: 11.9 us against 15.3 us.  With a k-contiguous operand the unstaged kernel's loads are
     // 16 bytes per row and lane, which costs more than the padding (2708 x 16 x 1433: 17.8 us against 14.1 us).
-    if (!a_kmajor && !b_kmajor && (m <= 32 || n <= 32) && k > 512 && tiles(32, 32) <= n_cu) {
-        const size_t groups = ceil_div_sz(k, 8);
-        size_t splits = ceil_div_sz(groups, 32);
-        if (splits > 32) splits = 32;
-        size_t per = ceil_div_sz(groups, splits);
-        per = (per + 3) & ~(size_t)3;  // whole turns of the four waves
-        splits = ceil_div_sz(groups, per);
+    if (small_ld && !a_kmajor && !b_kmajor && (m <= 32 || n <= 32) && k > 512 && tiles(32, 32) <= n_cu) {
+        size_t per = 0;
+        const size_t splits = gemm_skinny_splits(m, n, k, n_cu, &per);
         float* part = (float*)workspace(ctx, batches * splits * m * n * sizeof(float));
         if (!part) return ZG_HIP_EOOM;
         GemmArgs gs = g;
@@ -1535,6 +1600,12 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
         gs.gate = nullptr;
         gs.relu = 0;
         if (int rc = launch_gemm_tiny(ctx, gs, a_kmajor, b_kmajor, batches, splits)) return rc;
+        if (splits > 16) {
+            hipLaunchKernelGGL(splitk_reduce_many_kernel, dim3((unsigned)ceil_div_sz(m * n, 64), 1, (unsigned)batches), dim3(256), 0,
+                               ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk, g.bias, g.gate, g.relu);
+            ZG_LAUNCH_CHECK();
+            return ZG_HIP_OK;
+        }
         size_t blocks = ceil_div_sz(m * n, 256);
         if (blocks > 2048) blocks = 2048;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks, 1, (unsigned)batches), dim3(256), 0, ctx->stream,
@@ -1544,7 +1615,7 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     }
 
     // ---- plan: which tile, whether k is cut, whether C is cut into a block of whole rounds plus strips ----
-    const GemmPlan plan = gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth);
+    const GemmPlan plan = small_ld ? gemm_plan(ctx, m, n, k, batches, a_kmajor, b_kmajor, depth) : far_plan;
     if (plan.kind == GemmPlan::kParts) {
         // C = [ main | right ] over [ bottom ]: main is rm x rn whole large tiles (a whole number of rounds, or nearly),
         // the strips are products of their own and go through this function again (they may cut k, not C).
@@ -1595,6 +1666,12 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
                  : tile == 1 ? launch_gemm<128, 128>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches)
                              : launch_gemm<64, 64>(ctx, gs, a_kmajor, b_kmajor, split_mode, batches);
         if (rc) return rc;
+        if (splits > 16) {
+            hipLaunchKernelGGL(splitk_reduce_many_kernel, dim3((unsigned)ceil_div_sz(m * n, 64), 1, (unsigned)batches), dim3(256), 0,
+                               ctx->stream, part, C, m, n, ldc, (int)splits, alpha, beta, c_chunk, g.bias, g.gate, g.relu);
+            ZG_LAUNCH_CHECK();
+            return ZG_HIP_OK;
+        }
         const bool vec4 = gs.c_vec && c_vec && !g.gate;
         size_t blocks = ceil_div_sz(vec4 ? m * n / 4 : m * n, 256);
         if (blocks > 4096) blocks = 4096;
@@ -1640,16 +1717,15 @@ static size_t gemm_workspace_need(zg_hip_ctx* ctx, size_t m, size_t n, size_t k,
     const bool a_kmajor = !trans_a, b_kmajor = trans_b != 0;
     const size_t n_cu = (size_t)ctx->n_cu;
     const bool small_ld = lda < ((size_t)1 << 21) && ldb < ((size_t)1 << 21);
-    if (!small_ld || gemm_is_tiny(m, n, k, 1, lda, ldb, n_cu)) return 0;
+    if (!small_ld) {
+        const GemmPlan far_plan = gemm_plan_single(m, n, k, 1, n_cu);
+        return (far_plan.kind == GemmPlan::kSplit && far_plan.tile == 2) ? far_plan.splits * m * n * sizeof(float) : 0;
+    }
+    if (gemm_is_tiny(m, n, k, 1, lda, ldb, n_cu)) return 0;
     if (gemm_is_deep(m, n, k, 1, a_kmajor, b_kmajor, n_cu)) return 0;
     if (!a_kmajor && !b_kmajor && (m <= 32 || n <= 32) && k > 512 && ceil_div_sz(m, 32) * ceil_div_sz(n, 32) <= n_cu) {
-        const size_t groups = ceil_div_sz(k, 8);
-        size_t splits = ceil_div_sz(groups, 32);
-        if (splits > 32) splits = 32;
-        size_t per = ceil_div_sz(groups, splits);
-        per = (per + 3) & ~(size_t)3;
-        splits = ceil_div_sz(groups, per);
-        return splits * m * n * sizeof(float);
+        size_t per = 0;
+        return gemm_skinny_splits(m, n, k, n_cu, &per) * m * n * sizeof(float);
     }
     const GemmPlan plan = gemm_plan(ctx, m, n, k, 1, a_kmajor, b_kmajor, depth);
     if (plan.kind == GemmPlan::kTail) {

@@ -233,7 +233,9 @@ def test_bmm_32x512_cubed(oracle, hip):
                                  (130, 5000), (64, 64), (256, 1000), (1000, 1024), (68, 132), (1, 70000), (70000, 1),
                                  # transposes whose tiles are numbered down the diagonals (wide, both sides multiples of 1024)
                                  # and the tall counterpart that is not
-                                 (1024, 1024), (1024, 3072), (2048, 1024)])
+                                 (1024, 1024), (1024, 3072), (2048, 1024),
+                                 # rows short enough for two lanes each
+                                 (3000, 20), (3000, 17)])
 def test_matvec_outer_transpose(oracle, hip, m, n):
     r = rng(m + n)
     A = r.standard_normal((m, n)).astype(np.float32)

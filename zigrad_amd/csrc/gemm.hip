@@ -2448,7 +2448,8 @@ ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float*
     if (!trans_a) {
         const bool vec = aligned16(A) && aligned16(x) && n % 4 == 0;
         // lanes per row by row length; a whole workgroup for rows of more than 4096 columns
-        const int tpr = n <= 64 ? 4 : n <= 256 ? 16 : n <= 4096 ? 64 : 256;
+        // (one lane per row below 16 columns, two below 32: four lanes on a row of 4 values left three of them idle)
+        const int tpr = n < 16 ? 1 : n < 32 ? 2 : n <= 64 ? 4 : n <= 256 ? 16 : n <= 4096 ? 64 : 256;
         const size_t wgs = ceil_div_sz(m, (size_t)(256 / tpr));
         ZG_REQUIRE(wgs <= 0x7fffffffull, "matvec: too many rows");
         // few long rows: segments of at least 4096 columns, about eight workgroups per compute unit
@@ -2476,7 +2477,9 @@ ZG_API int zg_hip_matvec(zg_hip_ctx* ctx, const float* A, const float* x, float*
         else hipLaunchKernelGGL((gemv_rows_kernel<T, false>), grid, dim3(256), 0, ctx->stream, A, x, y, part, m, n, seg, \
                                 alpha, beta);                                                                          \
     } while (0)
-        if (tpr == 4) ZG_GEMV(4);
+        if (tpr == 1) ZG_GEMV(1);
+        else if (tpr == 2) ZG_GEMV(2);
+        else if (tpr == 4) ZG_GEMV(4);
         else if (tpr == 16) ZG_GEMV(16);
         else if (tpr == 64) ZG_GEMV(64);
         else ZG_GEMV(256);

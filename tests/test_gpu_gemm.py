@@ -171,6 +171,32 @@ def test_bmm_acc_batches(oracle, hip, nba, nbb, nbc):
     assert rel_fro(res[1], truth) <= TOL
 
 
+@pytest.mark.parametrize("nb,m,n,k,nba,nbb,ta,tb", [(5000, 8, 8, 8, 5000, 5000, False, False), (4096, 8, 8, 64, 4096, 1, False, True),
+                                                    (70000, 4, 4, 4, 70000, 70000, True, False), (4100, 3, 5, 7, 1, 4100, True, True),
+                                                    (6000, 1, 8, 33, 6000, 6000, False, False),
+                                                    # just outside: 16 x 16 blocks go a workgroup per product
+                                                    (4096, 16, 16, 16, 4096, 1, False, True)])
+def test_thousands_of_very_small_products(hip, nb, m, n, k, nba, nbb, ta, tb):
+    """Batches of at least 4096 products of at most 8 x 8 x 64 take a thread per element of C: every layout, an operand
+    shared by all products, alpha and beta."""
+    r = rng(nb + m * 7 + n * 11 + k)
+    A = r.standard_normal((nba, k, m) if ta else (nba, m, k)).astype(np.float32)
+    B = r.standard_normal((nbb, n, k) if tb else (nbb, k, n)).astype(np.float32)
+    C0 = r.standard_normal((nb, m, n)).astype(np.float32)
+    a, b, c = hip.from_numpy(A), hip.from_numpy(B), hip.from_numpy(C0)
+    hip.dispatch("bmm_acc", A=a, B=b, C=c, A_shape=[nba, m, k], B_shape=[nbb, k, n], C_shape=[nb, m, n], trans_a=ta,
+                 trans_b=tb, lda=(m if ta else k), ldb=(k if tb else n), ldc=n, alpha=0.5, beta=-1.0)
+    hip.sync()
+    got = hip.to_numpy(c).reshape(nb, m, n)
+    A64 = (A.transpose(0, 2, 1) if ta else A).astype(np.float64)
+    B64 = (B.transpose(0, 2, 1) if tb else B).astype(np.float64)
+    ia, ib = np.arange(nb) % nba, np.arange(nb) % nbb
+    truth = 0.5 * np.einsum("bik,bkj->bij", A64[ia], B64[ib]) - C0
+    assert rel_fro(got, truth) <= TOL
+    for x in (a, b, c):
+        hip.mem_free(x)
+
+
 def test_bmm_acc_split_k_batches(oracle, hip):
     """Batched products with few C tiles and a deep k take the split-k path: partial products per batch and split."""
     nb, m, n, k = 3, 64, 48, 1536

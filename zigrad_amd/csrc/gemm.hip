@@ -807,6 +807,45 @@ __global__ __launch_bounds__(kGemmThreads) void linear_bwd_small_kernel(LinearBw
                                      1, &part[0][0][0]);
 }
 
+// Thousands of very small products (m, n <= 8, k <= 64: per-sample transforms): a workgroup per product spends its
+// launch on a block that is 1/16 full (65536 products of 8 x 8 x 8: 280 us, 2 % of 8 TB/s), so here a thread owns one
+// element of one product and walks k; the threads of a product read the same few cache lines.  No epilogue extras.
+template <bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(256) void gemm_micro_kernel(GemmArgs g, size_t batches) {
+    const size_t mn = g.M * g.N, total = batches * mn;
+    const size_t nt = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += nt) {
+        const size_t z = i / mn, e = i - z * mn, r = e / g.N, c = e - r * g.N;
+        const float* a = g.A + (z % g.nba) * g.a_chunk;
+        const float* b = g.B + (z % g.nbb) * g.b_chunk;
+        float acc = 0.f;
+        for (size_t kk = 0; kk < g.K; kk++) {
+            const float av = A_KMAJOR ? a[r * g.lda + kk] : a[kk * g.lda + r];
+            const float bv = B_KMAJOR ? b[c * g.ldb + kk] : b[kk * g.ldb + c];
+            acc = fmaf(av, bv, acc);
+        }
+        float* cp = g.C + z * g.c_chunk + r * g.ldc + c;
+        float v = g.alpha * acc;
+        if (g.beta != 0.f) v += g.beta * *cp;
+        *cp = v;
+    }
+}
+static bool gemm_is_micro(size_t m, size_t n, size_t k, size_t batches, const GemmArgs& g) {
+    // up to 8 x 8 (16 x 16 x 16 with a k-contiguous B: 250 us a workgroup per product, 481 us this way)
+    return batches >= 4096 && m <= 8 && n <= 8 && k <= 64 && !g.bias && !g.gate && !g.relu;
+}
+static int launch_gemm_micro(zg_hip_ctx* ctx, const GemmArgs& g, bool a_kmajor, bool b_kmajor, size_t batches) {
+    size_t blocks = ceil_div_sz(batches * g.M * g.N, 256);
+    if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
+    const dim3 grid((unsigned)blocks), block(256);
+    if (a_kmajor && b_kmajor) hipLaunchKernelGGL((gemm_micro_kernel<true, true>), grid, block, 0, ctx->stream, g, batches);
+    else if (a_kmajor) hipLaunchKernelGGL((gemm_micro_kernel<true, false>), grid, block, 0, ctx->stream, g, batches);
+    else if (b_kmajor) hipLaunchKernelGGL((gemm_micro_kernel<false, true>), grid, block, 0, ctx->stream, g, batches);
+    else hipLaunchKernelGGL((gemm_micro_kernel<false, false>), grid, block, 0, ctx->stream, g, batches);
+    ZG_LAUNCH_CHECK();
+    return ZG_HIP_OK;
+}
+
 static int launch_gemm_tiny(zg_hip_ctx* ctx, GemmArgs& g, bool a_kmajor, bool b_kmajor, size_t batches,
                             size_t splits = 1) {
     g.tiles_m = (unsigned)ceil_div_sz(g.M, 32);
@@ -1569,6 +1608,7 @@ static int gemm_dispatch_body(zg_hip_ctx* ctx, const char* name, const float* A,
     const GemmPlan far_plan = small_ld ? GemmPlan() : gemm_plan_single(m, n, k, batches, n_cu);
     if (!small_ld && !(far_plan.kind == GemmPlan::kSplit && far_plan.tile == 2))
         return launch_gemm<64, 64>(ctx, g, a_kmajor, b_kmajor, 2, batches);
+    if (small_ld && gemm_is_micro(m, n, k, batches, g)) return launch_gemm_micro(ctx, g, a_kmajor, b_kmajor, batches);
     const bool deep = small_ld && gemm_is_deep(m, n, k, batches, a_kmajor, b_kmajor, n_cu);
     if (!deep && gemm_is_tiny(m, n, k, batches, lda, ldb, n_cu)) return launch_gemm_tiny(ctx, g, a_kmajor, b_kmajor, batches);
     if (deep) {
